@@ -1,0 +1,144 @@
+/*
+ * turbine_mi355.h -- C ABI of the MI355X (gfx950) dense-kernel library.
+ *
+ * One shared object, libturbine_mi355.so, exports the functions below.  Every
+ * function takes raw device pointers, plain integer sizes and the HIP stream
+ * to launch on (a hipStream_t passed as void*; NULL = the legacy default
+ * stream).  Nothing here allocates, synchronises or keeps state between calls:
+ * the caller owns all memory, including split-K scratch.
+ *
+ * Return value: 0 on success; a negative MI355_E_* code when the arguments
+ * violate the kernel's contract (nothing was launched); a positive value is
+ * the hipError_t reported by the launch.  mi355_last_error() returns a
+ * thread-local text describing the most recent failure on this thread.
+ *
+ * Reference interfaces these entry points stand behind (paths relative to the
+ * iree-turbine checkout):
+ *   - the eager custom-op hook CustomOp.eager_execute,
+ *     iree/turbine/runtime/op_reg/base.py:221-232 and the dispatcher
+ *     trampoline at base.py:1061-1072;
+ *   - the callable-kernel protocol Launchable.__call__,
+ *     iree/turbine/runtime/launch.py:203-272 (contiguous tensors, one device,
+ *     launch ordered on torch's current stream, runtime/device.py:336-361);
+ *   - the reference itself reaches HIP through ctypes on libamdhip64
+ *     (iree/turbine/runtime/device.py:86-150); this header is the same kind
+ *     of boundary one level up.
+ */
+#ifndef TURBINE_MI355_H_
+#define TURBINE_MI355_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355_ABI_VERSION 1
+
+/* contract-violation codes (returned negated: e.g. -MI355_E_SHAPE) */
+#define MI355_E_NULL 1      /* a required pointer is NULL */
+#define MI355_E_SHAPE 2     /* a size is non-positive or not supported by any kernel variant */
+#define MI355_E_ALIGN 3     /* a pointer is not aligned as the kernel requires (16 bytes) */
+#define MI355_E_DTYPE 4     /* unknown out_dtype / variant selector */
+#define MI355_E_SCRATCH 5   /* split-K scratch missing or too small */
+
+/* output element types */
+#define MI355_F32 0
+#define MI355_F16 1
+#define MI355_BF16 2
+
+int mi355_abi_version(void);
+const char* mi355_last_error(void);
+
+/* Number of kernel variants of a family and the name of variant i
+ * (family: "gemm_f16_nt", "flash_attn_fwd", "paged_decode", "mxfp4_gemm"). */
+int mi355_variant_count(const char* family);
+const char* mi355_variant_name(const char* family, int i);
+
+/*
+ * fp16 NT GEMM:  C[M,N] = A[M,K] . B[N,K]^T, fp32 accumulation.
+ * A, B: fp16 row-major (K contiguous).  C: row-major, out_dtype MI355_F32 or
+ * MI355_F16.  variant < 0 selects by shape; otherwise a variant index.
+ * Replaces: BOO GEMMForward with transpose_b (torch.mm(a, b.t())),
+ * iree/turbine/kernel/boo/op_exports/gemm.py:217-230, and the TK tiled GEMM
+ * of tests/kernel/vector_codegen_test.py:71-100.
+ */
+int mi355_gemm_f16_nt(const void* a, const void* b, void* c,
+                      int64_t M, int64_t N, int64_t K,
+                      int out_dtype, int variant, void* stream);
+
+/*
+ * Flash-attention forward (prefill): O = softmax(scale . Q K^T [+ causal mask]) V.
+ * q, o: [B, H, Sq, D]; k, v: [B, H, Sk, D]; all fp16 contiguous; D == 128.
+ * fp32 online softmax, fp16 output.  is_causal: query i attends keys
+ * j <= i + (Sk - Sq) (lower-right aligned; equals lower-triangular when Sq == Sk).
+ * Replaces: aten::scaled_dot_product_attention as canonicalised by
+ * iree/turbine/kernel/boo/fusion/replacement.py:275-284, and the TK fused
+ * attention of tests/kernel/fused_attention_test.py:25-77.
+ */
+int mi355_flash_attn_fwd(const void* q, const void* k, const void* v, void* o,
+                         int64_t B, int64_t H, int64_t Sq, int64_t Sk, int64_t D,
+                         float scale, int is_causal, int variant, void* stream);
+
+/*
+ * Paged GQA decode attention, one query token per sequence.
+ * q:           [num_seqs, num_q_heads, D]                 fp16
+ * k_cache,
+ * v_cache:     [num_pages, page_size, num_kv_heads, D]    fp16
+ * block_table: [num_seqs, max_pages_per_seq]              int32 page ids; entries at or
+ *              beyond ceil(seq_len/page_size) are never read
+ * seq_lens:    [num_seqs]                                 int32, >= 0
+ * out:         [num_seqs, num_q_heads, D]                 fp16
+ * Requirements: D == 128, page_size == 16, num_q_heads == 4 * num_kv_heads or
+ * any ratio in {1, 2, 4, 8, 16}.
+ *
+ * Split-K: phase 0 writes, for every (seq, q head, split), an unnormalised
+ * fp32 partial output and its (running max in log2 units, running sum);
+ * phase 1 merges the splits.  part_acc: [num_seqs, num_q_heads, num_splits, D]
+ * fp32; part_ml: [num_seqs, num_q_heads, num_splits, 2] fp32.
+ * mi355_paged_decode_attn runs both phases (num_splits == 1 needs no scratch).
+ * No reference counterpart survives in the checkout; semantics follow the GQA
+ * KV-cache attention of tests/dynamo/llama_test.py:82-91,160-181.
+ */
+int mi355_paged_decode_phase0(const void* q, const void* k_cache, const void* v_cache,
+                              const int32_t* block_table, const int32_t* seq_lens,
+                              float* part_acc, float* part_ml,
+                              int64_t num_seqs, int64_t num_q_heads, int64_t num_kv_heads,
+                              int64_t D, int64_t page_size, int64_t max_pages_per_seq,
+                              int64_t num_pages, int64_t num_splits, float scale, void* stream);
+int mi355_paged_decode_phase1(const float* part_acc, const float* part_ml, void* out,
+                              int64_t num_seqs, int64_t num_q_heads, int64_t D,
+                              int64_t num_splits, void* stream);
+int mi355_paged_decode_attn(const void* q, const void* k_cache, const void* v_cache,
+                            const int32_t* block_table, const int32_t* seq_lens, void* out,
+                            float* part_acc, float* part_ml,
+                            int64_t num_seqs, int64_t num_q_heads, int64_t num_kv_heads,
+                            int64_t D, int64_t page_size, int64_t max_pages_per_seq,
+                            int64_t num_pages, int64_t num_splits, float scale, void* stream);
+
+/*
+ * Block-scaled MXFP4 GEMM: C[M,N] = dq(A) . dq(B)^T, fp32 accumulation, bf16 out.
+ * a: uint8 [M, K/2], b: uint8 [N, K/2]  -- two E2M1 codes per byte, element 2i
+ *    in the low nibble, element 2i+1 in the high nibble;
+ * a_scale: uint8 [M, K/32], b_scale: uint8 [N, K/32] -- E8M0 (value 2^(byte-127)),
+ *    one per 32 consecutive K elements.
+ * dq(x)[r,k] = E2M1(code[r,k]) * 2^(scale[r,k/32] - 127).  K % 32 == 0.
+ * Format names: iree/turbine/kernel/_support/dtype.py:117,119 (f8e8m0fnu,
+ * f4e2m1fn); scale symbols iree/turbine/kernel/lang/global_symbols.py:33-35.
+ */
+int mi355_mxfp4_gemm(const void* a, const void* a_scale, const void* b, const void* b_scale,
+                     void* c, int64_t M, int64_t N, int64_t K,
+                     int out_dtype, int variant, void* stream);
+
+/*
+ * MXFP4 dequantisation on the device (used to show that the device decodes
+ * the format bit-exactly): out[r,k] = E2M1(code) * 2^(scale-127) as fp32.
+ * codes: uint8 [rows, K/2]; scales: uint8 [rows, K/32]; out: fp32 [rows, K].
+ */
+int mi355_mxfp4_dequant(const void* codes, const void* scales, float* out,
+                        int64_t rows, int64_t K, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TURBINE_MI355_H_ */

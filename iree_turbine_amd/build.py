@@ -1,0 +1,74 @@
+"""Builds libturbine_mi355.so (the gfx950 kernels + C ABI) in-tree with hipcc.
+
+Usage: ``python -m iree_turbine_amd.build``.  hipcc cross-compiles for gfx950 without a GPU.
+"""
+
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+CSRC = Path(__file__).resolve().parent / "csrc"
+LIB_NAME = "libturbine_mi355.so"
+LIB_PATH = CSRC / LIB_NAME
+SOURCES = ["capi.hip", "gemm_f16_nt.hip", "flash_attn_fwd.hip", "paged_decode.hip", "gemm_mxfp4.hip"]
+
+# -packed-fp32-ops: keep the compiler from forming v_pk_{add,mul,fma}_f32.
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+    "-Wno-unknown-warning-option",
+]
+
+
+def _hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; cannot build the gfx950 kernel library")
+    return exe
+
+
+def _run(cmd: list[str]) -> None:
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"command failed ({proc.returncode}): {' '.join(cmd)}\n{proc.stdout}\n{proc.stderr}")
+    # the host pass warns that it does not know the packed-fp32 feature; that is expected
+    noise = ("packed-fp32-ops", "is not a recognized feature")
+    for line in proc.stderr.splitlines():
+        if line.strip() and not any(n in line for n in noise):
+            print(line, file=sys.stderr)
+
+
+def build_library(verbose: bool = True, save_temps: bool = False) -> Path:
+    """Compiles every kernel source and links the shared library.  Always recompiles."""
+    hipcc = _hipcc()
+    obj_dir = CSRC / "build"
+    obj_dir.mkdir(exist_ok=True)
+    objs = [obj_dir / (Path(s).stem + ".o") for s in SOURCES]
+
+    def compile_one(pair):
+        src, obj = pair
+        cmd = [hipcc, *HIPCC_FLAGS, "-c", str(CSRC / src), "-o", str(obj)]
+        if save_temps:
+            cmd += ["-save-temps=obj"]
+        _run(cmd)
+        return obj
+
+    with ThreadPoolExecutor(max_workers=min(len(SOURCES), os.cpu_count() or 4)) as pool:
+        list(pool.map(compile_one, zip(SOURCES, objs)))
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB_PATH), *map(str, objs)])
+    if verbose:
+        print(f"built {LIB_PATH} ({LIB_PATH.stat().st_size} bytes)")
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build_library(save_temps="--save-temps" in sys.argv)

@@ -1,0 +1,64 @@
+// Error plumbing and introspection entry points of the C ABI.
+#include "common.hpp"
+#include <string.h>
+
+namespace mi355 {
+
+static thread_local char g_error[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_launch(const char* kernel, dim3 grid, dim3 block, size_t lds) {
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess) return 0;
+  set_error("%s: launch failed, grid=(%u,%u,%u) block=(%u,%u,%u) lds=%zu: %s", kernel, grid.x, grid.y, grid.z, block.x,
+            block.y, block.z, lds, hipGetErrorString(e));
+  return (int)e;
+}
+
+int gemm_variant_count();
+const char* gemm_variant_name(int i);
+int fa_variant_count();
+const char* fa_variant_name(int i);
+int decode_variant_count();
+const char* decode_variant_name(int i);
+int mxfp4_variant_count();
+const char* mxfp4_variant_name(int i);
+
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" int mi355_abi_version(void) { return MI355_ABI_VERSION; }
+extern "C" const char* mi355_last_error(void) { return g_error; }
+
+extern "C" int mi355_variant_count(const char* family) {
+  if (!family) return 0;
+  if (!strcmp(family, "gemm_f16_nt")) return gemm_variant_count();
+  if (!strcmp(family, "flash_attn_fwd")) return fa_variant_count();
+  if (!strcmp(family, "paged_decode")) return decode_variant_count();
+  if (!strcmp(family, "mxfp4_gemm")) return mxfp4_variant_count();
+  return 0;
+}
+
+extern "C" const char* mi355_variant_name(const char* family, int i) {
+  if (!family) return nullptr;
+  if (!strcmp(family, "gemm_f16_nt")) return gemm_variant_name(i);
+  if (!strcmp(family, "flash_attn_fwd")) return fa_variant_name(i);
+  if (!strcmp(family, "paged_decode")) return decode_variant_name(i);
+  if (!strcmp(family, "mxfp4_gemm")) return mxfp4_variant_name(i);
+  return nullptr;
+}

@@ -1,0 +1,71 @@
+// Shared device/host helpers for the gfx950 kernels: vector types, MFMA wrappers,
+// LDS address-space casts, direct-to-LDS loads and the error plumbing of the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include "../../include/turbine_mi355.h"
+
+namespace mi355 {
+
+typedef _Float16 half_t;
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef __attribute__((__vector_size__(4 * sizeof(__fp16)))) __fp16 fp16x4_t;
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef int intx2 __attribute__((ext_vector_type(2)));
+typedef int intx4 __attribute__((ext_vector_type(4)));
+typedef int intx8 __attribute__((ext_vector_type(8)));
+typedef unsigned short ushortx4 __attribute__((ext_vector_type(4)));
+
+#define MI355_LDS(T, p) ((__attribute__((address_space(3))) T*)(p))
+#define MI355_GLOBAL(p) ((const __attribute__((address_space(1))) void*)(p))
+
+// One wave copies 64 x 16 bytes from global memory straight into LDS.  Lane l's
+// 16 bytes land at lds_wave_base + 16*l: the LDS side is fixed by the lane id,
+// so any swizzle is applied by choosing which global address each lane reads.
+__device__ __forceinline__ void load_lds_16B(const void* gptr, void* lds_wave_base) {
+  __builtin_amdgcn_global_load_lds(MI355_GLOBAL(gptr), MI355_LDS(void, lds_wave_base), 16, 0, 0);
+}
+
+__device__ __forceinline__ void wait_vmcnt0() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// D(32x32) += A(32x16) * B(16x32).  Lane l supplies A[l%32][8*(l/32) .. +7] and
+// B[8*(l/32) .. +7][l%32]; it receives D[8*(r/4) + 4*(l/32) + r%4][l%32] in register r.
+__device__ __forceinline__ floatx16 mfma_32x32x16(half8 a, half8 b, floatx16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+// D(16x16) += A(16x32) * B(32x16).  Lane l supplies A[l%16][8*(l/16) .. +7] and
+// B[8*(l/16) .. +7][l%16]; it receives D[4*(l/16) + r][l%16] in register r.
+__device__ __forceinline__ floatx4 mfma_16x16x32(half8 a, half8 b, floatx4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+
+// LDS transpose read.  Within each group of 16 lanes, lane i passes the address
+// of 4 consecutive halfs; seen as a 4x16 matrix M[k][n] where lane i supplied
+// M[i/4][4*(i%4) .. +3], lane i receives the column M[0..3][i].
+__device__ __forceinline__ half4 lds_read_tr16(const void* lds_ptr) {
+  fp16x4_t t = __builtin_amdgcn_ds_read_tr16_b64_v4f16(MI355_LDS(fp16x4_t, lds_ptr));
+  return *(half4*)&t;
+}
+
+__device__ __forceinline__ unsigned short f32_to_bf16_rne(float f) {
+  unsigned int u = __builtin_bit_cast(unsigned int, f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40);  // NaN stays NaN
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (unsigned short)(u >> 16);
+}
+
+// ---- host side ---------------------------------------------------------------------------
+
+void set_error(const char* fmt, ...);
+int fail(int code, const char* fmt, ...);
+int check_launch(const char* kernel, dim3 grid, dim3 block, size_t lds);
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace mi355

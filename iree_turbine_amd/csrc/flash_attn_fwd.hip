@@ -1,0 +1,254 @@
+// Flash-attention forward (prefill) for gfx950, head dim 128, fp16 in/out, fp32 softmax.
+//
+// One workgroup = 4 waves = 128 queries of one (batch, head); each wave owns 32 queries and
+// keeps, in registers, its Q fragments (32 VGPRs), the running max / sum of every query, and
+// the 32 x 128 fp32 output accumulator (64 VGPRs).  K and V are streamed in 64-key tiles
+// through a two-stage LDS ring filled by direct-to-LDS loads.
+//
+// Both contractions are computed transposed so that the softmax never leaves registers:
+//   S^T[key][query]  = K . Q^T     (MFMA A operand = K rows from LDS, B operand = Q in registers)
+//   O^T[d][query]   += V^T . P^T   (A operand = V^T via LDS transpose reads, B operand = P)
+// With v_mfma_f32_32x32x16_f16 a lane owns one query column of S^T (16 keys per 32-key tile,
+// the other 16 sit in lane^32), so row max / sum are in-lane reductions plus one cross-lane
+// exchange, and the exponentiated scores are already laid out as the B operand of the second
+// MFMA.  The order in which keys are fed to that MFMA is whatever the S^T register order
+// dictates; V^T is fetched with the matching order by ds_read_b64_tr_b16.
+//
+// LDS swizzles (16-byte chunks, 256-byte rows): K chunk c of row r -> slot c ^ (r & 15);
+// V chunk c of row r -> slot c ^ (2 * (r & 7)).  As in the GEMM, the swizzle is applied on the
+// global side of the direct-to-LDS loads.
+#include "common.hpp"
+#include <math.h>
+
+namespace mi355 {
+
+constexpr int FA_BLOCK_M = 128;
+constexpr int FA_BLOCK_N = 64;
+constexpr int FA_STAGE = 2 * FA_BLOCK_N * 256;  // K tile + V tile, bytes
+
+template <bool CAUSAL>
+__global__ __launch_bounds__(256) void fa_fwd_d128(const half_t* __restrict__ Q, const half_t* __restrict__ K,
+                                                   const half_t* __restrict__ V, half_t* __restrict__ O, int BH, int Sq,
+                                                   int Sk, float scale_log2e, int q_blocks) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r32 = lane & 31, h = lane >> 5;
+
+  // workgroup -> (batch*head, query block).  Consecutive ids land on different XCDs; keep all
+  // query blocks of one head on one XCD so its K/V stay in that XCD's L2.
+  int bh, qb;
+  {
+    const int pid = blockIdx.x;
+    if ((BH & 7) == 0) {
+      const int xcd = pid & 7, loc = pid >> 3;
+      bh = (loc / q_blocks) * 8 + xcd;
+      qb = loc % q_blocks;
+    } else {
+      bh = pid / q_blocks;
+      qb = pid % q_blocks;
+    }
+    if (CAUSAL) qb = q_blocks - 1 - qb;  // longest rows first
+  }
+  const int causal_off = Sk - Sq;  // query i sees keys <= i + causal_off
+  const int q0 = qb * FA_BLOCK_M;
+  const int wq0 = q0 + wave * 32;  // first query of this wave
+  const int q_row = wq0 + r32;
+  const bool q_ok = q_row < Sq;
+
+  const half_t* Qb = Q + (size_t)bh * Sq * 128;
+  const half_t* Kb = K + (size_t)bh * Sk * 128;
+  const half_t* Vb = V + (size_t)bh * Sk * 128;
+  half_t* Ob = O + (size_t)bh * Sq * 128;
+
+  // number of key tiles this workgroup walks
+  int k_end = Sk;
+  if (CAUSAL) {
+    int last_q = q0 + FA_BLOCK_M - 1;
+    if (last_q > Sq - 1) last_q = Sq - 1;
+    int lim = last_q + causal_off + 1;
+    if (lim < k_end) k_end = lim;
+  }
+  const int n_tiles = k_end > 0 ? (k_end + FA_BLOCK_N - 1) / FA_BLOCK_N : 0;
+
+  // ---- Q fragments (MFMA B operand): lane (query r32, half h) holds d = 16*ks + 8*h .. +7 ----
+  half8 qf[8];
+#pragma unroll
+  for (int ks = 0; ks < 8; ks++) {
+    if (q_ok) {
+      qf[ks] = *reinterpret_cast<const half8*>(Qb + (size_t)q_row * 128 + ks * 16 + h * 8);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; e++) qf[ks][e] = (half_t)0;
+    }
+  }
+
+  // ---- global -> LDS: a wave-load moves 4 rows of 256 bytes; lane l: row l/16, slot l%16 ----
+  const int lrow = lane >> 4, lslot = lane & 15;
+  const int k_chunk = lslot ^ (wave * 4 + lrow);           // group g = wave + 4*i, so (row & 15) = 4*wave + lrow
+  const int v_chunk = lslot ^ (2 * ((wave & 1) * 4 + lrow));  // (row & 7) = 4*(wave&1) + lrow
+  auto issue_loads = [&](int tile, int stage) {
+    char* dst = lds + stage * FA_STAGE + wave * 1024;
+    const int key0 = tile * FA_BLOCK_N;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      int row = key0 + (wave + 4 * i) * 4 + lrow;
+      if (row > Sk - 1) row = Sk - 1;  // clamp: the tail rows are masked out of the softmax
+      load_lds_16B(Kb + (size_t)row * 128 + k_chunk * 8, dst + i * 4096);
+      load_lds_16B(Vb + (size_t)row * 128 + v_chunk * 8, dst + FA_BLOCK_N * 256 + i * 4096);
+    }
+  };
+
+  // ---- LDS read addresses ----
+  const int k_base = r32 * 256 + ((h ^ (lane & 15)) * 16);  // ^ (ks*32), + t*8192
+  const int i16 = lane & 15, g16 = lane >> 4;
+  const int v_row = 4 * (g16 >> 1) + (i16 >> 2);
+  const int v_cl = 2 * (g16 & 1) + ((i16 & 3) >> 1);
+  const int v_base = FA_BLOCK_N * 256 + v_row * 256 + ((v_cl ^ (2 * (v_row & 7))) * 16) + (i16 & 1) * 8;  // ^ (dt*64), + t16*4096, + {0,2048}
+
+  floatx16 oacc[4];
+#pragma unroll
+  for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) oacc[dt][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+
+  if (n_tiles > 0) {
+    issue_loads(0, 0);
+    wait_vmcnt0();
+    __syncthreads();
+  }
+
+  for (int j = 0; j < n_tiles; j++) {
+    if (j + 1 < n_tiles) issue_loads(j + 1, (j + 1) & 1);
+    const char* st = lds + (j & 1) * FA_STAGE;
+    const int key0 = j * FA_BLOCK_N;
+    // a wave whose every query is before this tile has nothing to do here (causal only)
+    const bool active = !CAUSAL || (key0 <= wq0 + 31 + causal_off);
+    if (active) {
+      floatx16 s[2];
+#pragma unroll
+      for (int t = 0; t < 2; t++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[t][r] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < 8; ks++) {
+          half8 kf = *reinterpret_cast<const half8*>(st + ((k_base ^ (ks * 32)) + t * 8192));
+          s[t] = mfma_32x32x16(kf, qf[ks], s[t]);
+        }
+      }
+      const bool need_mask = (CAUSAL && (key0 + FA_BLOCK_N - 1 > wq0 + causal_off)) || (key0 + FA_BLOCK_N > Sk);
+      if (need_mask) {
+        const int lim = CAUSAL ? (q_row + causal_off < Sk - 1 ? q_row + causal_off : Sk - 1) : Sk - 1;  // last visible key
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int key = key0 + 32 * t + 8 * (r >> 2) + 4 * h + (r & 3);
+            if (key > lim) s[t][r] = -INFINITY;
+          }
+      }
+      float mx = s[0][0];
+#pragma unroll
+      for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[t][r]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      const float m_new = fmaxf(m_run, mx);
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = exp2f((m_run - m_use) * scale_log2e);
+      const float mc = m_use * scale_log2e;
+      m_run = m_new;
+      float psum = 0.f;
+      half8 pf[4];
+#pragma unroll
+      for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const float p = exp2f(s[t][r] * scale_log2e - mc);
+          psum += p;
+          pf[t * 2 + (r >> 3)][r & 7] = (half_t)p;
+        }
+      l_run = l_run * alpha + psum;
+#pragma unroll
+      for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) oacc[dt][r] *= alpha;
+      // O^T += V^T P^T
+#pragma unroll
+      for (int t16 = 0; t16 < 4; t16++) {
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) {
+          const char* va = st + ((v_base ^ (dt * 64)) + t16 * 4096);
+          half4 lo = lds_read_tr16(va);
+          half4 hi = lds_read_tr16(va + 2048);
+          half8 vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          oacc[dt] = mfma_32x32x16(vf, pf[t16], oacc[dt]);
+        }
+      }
+    }
+    wait_vmcnt0();
+    __syncthreads();
+  }
+
+  // ---- epilogue ----
+  const float l_tot = l_run + __shfl_xor(l_run, 32);
+  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  if (q_ok) {
+    half_t* orow = Ob + (size_t)q_row * 128 + 4 * h;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        half4 v = {(half_t)(oacc[dt][4 * q] * inv), (half_t)(oacc[dt][4 * q + 1] * inv), (half_t)(oacc[dt][4 * q + 2] * inv),
+                   (half_t)(oacc[dt][4 * q + 3] * inv)};
+        *reinterpret_cast<half4*>(orow + dt * 32 + q * 8) = v;
+      }
+  }
+}
+
+static const char* kFaVariants[] = {"d128_bm128_bn64_w4"};
+int fa_variant_count() { return 1; }
+const char* fa_variant_name(int i) { return i == 0 ? kFaVariants[0] : nullptr; }
+
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" int mi355_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, int64_t B, int64_t H, int64_t Sq,
+                                    int64_t Sk, int64_t D, float scale, int is_causal, int variant, void* stream) {
+  if (!q || !k || !v || !o) return fail(-MI355_E_NULL, "flash_attn_fwd: null pointer");
+  if (D != 128) return fail(-MI355_E_SHAPE, "flash_attn_fwd: head dim %lld not supported (only 128)", (long long)D);
+  if (B <= 0 || H <= 0 || Sq <= 0 || Sk <= 0 || B * H > (1 << 24) || Sq > (1 << 24) || Sk > (1 << 24))
+    return fail(-MI355_E_SHAPE, "flash_attn_fwd: bad shape B=%lld H=%lld Sq=%lld Sk=%lld", (long long)B, (long long)H,
+                (long long)Sq, (long long)Sk);
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o))
+    return fail(-MI355_E_ALIGN, "flash_attn_fwd: q, k, v, o must be 16-byte aligned");
+  if (variant > 0) return fail(-MI355_E_DTYPE, "flash_attn_fwd: variant %d out of range", variant);
+  if (!(scale > 0.f) || !isfinite(scale)) return fail(-MI355_E_SHAPE, "flash_attn_fwd: scale must be positive and finite");
+  const int BH = (int)(B * H);
+  const int q_blocks = (int)((Sq + FA_BLOCK_M - 1) / FA_BLOCK_M);
+  const int lds_bytes = 2 * FA_STAGE;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(fa_fwd_d128<true>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(fa_fwd_d128<false>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e1 != hipSuccess || e2 != hipSuccess) {
+      set_error("hipFuncSetAttribute(fa_fwd_d128): %s", hipGetErrorString(e1 != hipSuccess ? e1 : e2));
+      return (int)(e1 != hipSuccess ? e1 : e2);
+    }
+    attr_set = true;
+  }
+  const float scale_log2e = scale * 1.4426950408889634f;
+  dim3 grid(BH * q_blocks), block(256);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (is_causal)
+    hipLaunchKernelGGL(fa_fwd_d128<true>, grid, block, lds_bytes, s, (const half_t*)q, (const half_t*)k, (const half_t*)v,
+                       (half_t*)o, BH, (int)Sq, (int)Sk, scale_log2e, q_blocks);
+  else
+    hipLaunchKernelGGL(fa_fwd_d128<false>, grid, block, lds_bytes, s, (const half_t*)q, (const half_t*)k, (const half_t*)v,
+                       (half_t*)o, BH, (int)Sq, (int)Sk, scale_log2e, q_blocks);
+  return check_launch("fa_fwd_d128", grid, block, lds_bytes);
+}

@@ -1,0 +1,288 @@
+// fp16 NT GEMM for gfx950:  C[M,N] = A[M,K] . B[N,K]^T with fp32 accumulation.
+//
+// Main kernel (gemm_f16_nt_tiled): a BM x BN output tile per workgroup, K walked in slabs
+// of 64 halfs.  A slab row is 128 bytes = 8 chunks of 16 bytes; both operands are
+// K-contiguous, so the same row format serves A and B.  Slabs are copied global -> LDS with
+// direct-to-LDS loads (no VGPR staging) into a two-stage ring: while the MFMAs consume
+// stage s the loads for the next slab fill stage s^1, and one barrier per slab closes the
+// iteration.  LDS rows are XOR-swizzled at chunk granularity (chunk c of row r lives in
+// slot c ^ (r & 7)) so that the 32-row x 16-byte fragment reads of v_mfma_f32_32x32x16_f16
+// are free of bank conflicts; because a direct-to-LDS load fixes the LDS slot by lane id,
+// the swizzle is applied on the global side (lane -> which chunk it fetches).
+//
+// The MFMA roles are swapped (B rows feed the "A" operand, A rows feed the "B" operand) so a
+// lane ends up owning 4 consecutive n for one m, which turns the epilogue into 8/16-byte
+// row-contiguous stores.
+//
+// Workgroup -> tile mapping is XCD aware: hardware deals consecutive workgroup ids
+// round-robin to the 8 XCDs (each with a private L2), so ids are first regrouped into 8
+// contiguous ranges and then walked in GROUP_M-tall column-major panels to keep the A/B
+// slabs that one XCD touches small.
+#include "common.hpp"
+
+namespace mi355 {
+
+template <typename OutT> struct OutPack;
+template <> struct OutPack<float> {
+  static __device__ __forceinline__ void store4(float* p, float a, float b, float c, float d) {
+    floatx4 v = {a, b, c, d};
+    *reinterpret_cast<floatx4*>(p) = v;
+  }
+  static __device__ __forceinline__ void store1(float* p, float a) { *p = a; }
+};
+template <> struct OutPack<half_t> {
+  static __device__ __forceinline__ void store4(half_t* p, float a, float b, float c, float d) {
+    half4 v = {(half_t)a, (half_t)b, (half_t)c, (half_t)d};
+    *reinterpret_cast<half4*>(p) = v;
+  }
+  static __device__ __forceinline__ void store1(half_t* p, float a) { *p = (half_t)a; }
+};
+
+__device__ __forceinline__ void map_tile(int pid, int tiles_m, int tiles_n, int group_m, int& tm, int& tn) {
+  const int T = tiles_m * tiles_n;
+  const int xcd = pid & 7, loc = pid >> 3;
+  const int per = T >> 3, rem = T & 7;
+  const int id = xcd * per + (xcd < rem ? xcd : rem) + loc;
+  const int width = group_m * tiles_n;
+  const int grp = id / width, within = id - grp * width;
+  const int first_m = grp * group_m;
+  const int gsz = (tiles_m - first_m) < group_m ? (tiles_m - first_m) : group_m;
+  tm = first_m + within % gsz;
+  tn = within / gsz;
+}
+
+template <int BM, int BN, int WM, int WN, typename OutT>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_tiled(const half_t* __restrict__ A,
+                                                                 const half_t* __restrict__ B,
+                                                                 OutT* __restrict__ C, int M, int N, int K,
+                                                                 int tiles_m, int tiles_n, int group_m) {
+  constexpr int NW = WM * WN;
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
+  constexpr int A_GROUPS = BM / 8, B_GROUPS = BN / 8;  // 8 rows = 1 KiB = one wave-wide load
+  static_assert(A_GROUPS % NW == 0 && B_GROUPS % NW == 0, "loads must split evenly over waves");
+  constexpr int LA = A_GROUPS / NW, LB = B_GROUPS / NW;
+
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  int tile_m, tile_n;
+  map_tile(blockIdx.x, tiles_m, tiles_n, group_m, tile_m, tile_n);
+
+  // ---- global -> LDS: lane l of a wave-load covers row (l/8) of an 8-row group, slot l%8 ----
+  const int lrow = lane >> 3;
+  const int lchunk = (lane & 7) ^ lrow;  // the chunk that belongs in this lane's slot
+  const half_t* a_src = A + (size_t)(tile_m * BM + wave * 8 + lrow) * K + lchunk * 8;
+  const half_t* b_src = B + (size_t)(tile_n * BN + wave * 8 + lrow) * K + lchunk * 8;
+  const size_t row_step = (size_t)NW * 8 * K;  // halfs between this wave's consecutive groups
+
+  auto issue_loads = [&](int stage) {
+    char* dst = lds + stage * STAGE + wave * 1024;
+#pragma unroll
+    for (int i = 0; i < LA; i++) load_lds_16B(a_src + i * row_step, dst + i * NW * 1024);
+#pragma unroll
+    for (int i = 0; i < LB; i++) load_lds_16B(b_src + i * row_step, dst + A_BYTES + i * NW * 1024);
+    a_src += 64;
+    b_src += 64;
+  };
+
+  // ---- LDS -> MFMA fragments ----
+  const int r32 = lane & 31, h = lane >> 5;
+  const int sw = (h ^ (lane & 7)) * 16;
+  const int a_base = (wm * WTM + r32) * 128 + sw;            // rows of A (m): feeds the MFMA "B" operand
+  const int b_base = A_BYTES + (wn * WTN + r32) * 128 + sw;  // rows of B (n): feeds the MFMA "A" operand
+
+  floatx16 acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; i++)
+#pragma unroll
+    for (int j = 0; j < TM; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+  const int KT = K / 64;
+  issue_loads(0);
+  wait_vmcnt0();
+  __syncthreads();
+
+  for (int kt = 0; kt < KT; kt++) {
+    if (kt + 1 < KT) issue_loads((kt + 1) & 1);
+    const char* st = lds + (kt & 1) * STAGE;
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+      half8 fm[TM], fn[TN];
+#pragma unroll
+      for (int j = 0; j < TM; j++) fm[j] = *reinterpret_cast<const half8*>(st + ((a_base ^ (ks * 32)) + j * 4096));
+#pragma unroll
+      for (int i = 0; i < TN; i++) fn[i] = *reinterpret_cast<const half8*>(st + ((b_base ^ (ks * 32)) + i * 4096));
+#pragma unroll
+      for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int j = 0; j < TM; j++) acc[i][j] = mfma_32x32x16(fn[i], fm[j], acc[i][j]);
+    }
+    wait_vmcnt0();
+    __syncthreads();
+  }
+
+  // ---- epilogue: lane owns m = r32 and, per register quad q, n = 8q + 4h .. +3 ----
+  const int m0 = tile_m * BM + wm * WTM + r32;
+  const int n0 = tile_n * BN + wn * WTN + 4 * h;
+#pragma unroll
+  for (int j = 0; j < TM; j++) {
+    OutT* crow = C + (size_t)(m0 + j * 32) * N + n0;
+#pragma unroll
+    for (int i = 0; i < TN; i++)
+#pragma unroll
+      for (int q = 0; q < 4; q++)
+        OutPack<OutT>::store4(crow + i * 32 + q * 8, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                              acc[i][j][4 * q + 3]);
+  }
+}
+
+// Any-shape kernel: 64x64 tile, 4 waves, bounds-checked staging through registers.  Used for
+// shapes the tiled kernel does not divide (and as an independent implementation in tests).
+template <typename OutT>
+__global__ __launch_bounds__(256) void gemm_f16_nt_generic(const half_t* __restrict__ A, const half_t* __restrict__ B,
+                                                           OutT* __restrict__ C, int M, int N, int K) {
+  constexpr int PITCH = 40;  // halfs per LDS row: 32 data + 8 pad keeps 16-byte alignment, spreads banks
+  __shared__ __attribute__((aligned(16))) half_t sA[64 * PITCH];
+  __shared__ __attribute__((aligned(16))) half_t sB[64 * PITCH];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int row0_m = blockIdx.y * 64, row0_n = blockIdx.x * 64;
+  const int lr = tid >> 2, lk = (tid & 3) * 8;
+  const bool vec_ok = (K % 8) == 0;
+  floatx16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; r++) acc[r] = 0.f;
+  const int r32 = lane & 31, h = lane >> 5;
+
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    half8 va, vb;
+    {
+      const int gm = row0_m + lr, gn = row0_n + lr, gk = k0 + lk;
+      if (gm < M && vec_ok && gk + 8 <= K) {
+        va = *reinterpret_cast<const half8*>(A + (size_t)gm * K + gk);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++) va[e] = (gm < M && gk + e < K) ? A[(size_t)gm * K + gk + e] : (half_t)0;
+      }
+      if (gn < N && vec_ok && gk + 8 <= K) {
+        vb = *reinterpret_cast<const half8*>(B + (size_t)gn * K + gk);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++) vb[e] = (gn < N && gk + e < K) ? B[(size_t)gn * K + gk + e] : (half_t)0;
+      }
+    }
+    __syncthreads();  // previous slab fully consumed
+    *reinterpret_cast<half8*>(sA + lr * PITCH + lk) = va;
+    *reinterpret_cast<half8*>(sB + lr * PITCH + lk) = vb;
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+      half8 fm = *reinterpret_cast<const half8*>(sA + (wm * 32 + r32) * PITCH + ks * 16 + h * 8);
+      half8 fn = *reinterpret_cast<const half8*>(sB + (wn * 32 + r32) * PITCH + ks * 16 + h * 8);
+      acc = mfma_32x32x16(fn, fm, acc);
+    }
+  }
+  const int m = row0_m + wm * 32 + r32;
+  if (m < M) {
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int n = row0_n + wn * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+      if (n < N) OutPack<OutT>::store1(C + (size_t)m * N + n, acc[r]);
+    }
+  }
+}
+
+// ---- host side ----------------------------------------------------------------------------
+
+struct GemmVariant {
+  const char* name;
+  int bm, bn, threads;
+};
+static const GemmVariant kGemmVariants[] = {
+    {"tiled_256x256x64_w2x4", 256, 256, 512},
+    {"tiled_256x256x64_w2x2", 256, 256, 256},
+    {"tiled_128x128x64_w2x2", 128, 128, 256},
+    {"generic_64x64x32", 64, 64, 256},
+};
+constexpr int kNumGemmVariants = sizeof(kGemmVariants) / sizeof(kGemmVariants[0]);
+
+int gemm_variant_count() { return kNumGemmVariants; }
+const char* gemm_variant_name(int i) { return (i >= 0 && i < kNumGemmVariants) ? kGemmVariants[i].name : nullptr; }
+
+template <int BM, int BN, int WM, int WN, typename OutT>
+static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int K, hipStream_t stream) {
+  auto kern = gemm_f16_nt_tiled<BM, BN, WM, WN, OutT>;
+  constexpr int lds_bytes = 2 * (BM + BN) * 128;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       lds_bytes);
+    if (e != hipSuccess) {
+      set_error("hipFuncSetAttribute(gemm_f16_nt_tiled, %d bytes LDS): %s", lds_bytes, hipGetErrorString(e));
+      return (int)e;
+    }
+    attr_set = true;
+  }
+  const int tiles_m = M / BM, tiles_n = N / BN;
+  int group_m = 4;
+  dim3 grid(tiles_m * tiles_n), block(WM * WN * 64);
+  hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, M, N, K, tiles_m,
+                     tiles_n, group_m);
+  return check_launch("gemm_f16_nt_tiled", grid, block, lds_bytes);
+}
+
+template <typename OutT>
+static int launch_variant(int variant, const void* a, const void* b, void* c, int M, int N, int K, hipStream_t stream) {
+  switch (variant) {
+    case 0: return launch_tiled<256, 256, 2, 4, OutT>(a, b, c, M, N, K, stream);
+    case 1: return launch_tiled<256, 256, 2, 2, OutT>(a, b, c, M, N, K, stream);
+    case 2: return launch_tiled<128, 128, 2, 2, OutT>(a, b, c, M, N, K, stream);
+    default: {
+      dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
+      hipLaunchKernelGGL(gemm_f16_nt_generic<OutT>, grid, block, 0, stream, (const half_t*)a, (const half_t*)b, (OutT*)c,
+                         M, N, K);
+      return check_launch("gemm_f16_nt_generic", grid, block, 0);
+    }
+  }
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" int mi355_gemm_f16_nt(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int out_dtype,
+                                 int variant, void* stream) {
+  if (!a || !b || !c) return fail(-MI355_E_NULL, "gemm_f16_nt: null pointer (a=%p b=%p c=%p)", a, b, c);
+  if (M <= 0 || N <= 0 || K <= 0 || M > (1 << 30) || N > (1 << 30) || K > (1 << 30))
+    return fail(-MI355_E_SHAPE, "gemm_f16_nt: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+  if (out_dtype != MI355_F32 && out_dtype != MI355_F16)
+    return fail(-MI355_E_DTYPE, "gemm_f16_nt: out_dtype %d (want MI355_F32 or MI355_F16)", out_dtype);
+  if (variant >= kNumGemmVariants) return fail(-MI355_E_DTYPE, "gemm_f16_nt: variant %d out of range", variant);
+  const bool al = aligned16(a) && aligned16(b) && aligned16(c);
+  auto fits = [&](int v) {
+    if (v == kNumGemmVariants - 1) return true;
+    return al && M % kGemmVariants[v].bm == 0 && N % kGemmVariants[v].bn == 0 && K % 64 == 0;
+  };
+  if (variant < 0) {
+    // Large problems take the 256x256 tile; when that leaves most of the 256 CUs idle the
+    // 128x128 tile (4x the workgroups) wins; everything else goes to the bounds-checked kernel.
+    if (fits(0) && (M / 256) * (N / 256) >= 128) variant = 0;
+    else if (fits(2)) variant = 2;
+    else variant = kNumGemmVariants - 1;
+  } else if (!fits(variant)) {
+    return fail(-MI355_E_SHAPE, "gemm_f16_nt: variant %s needs M%%%d==0, N%%%d==0, K%%64==0 and 16-byte aligned pointers",
+                kGemmVariants[variant].name, kGemmVariants[variant].bm, kGemmVariants[variant].bn);
+  }
+  if (variant == kNumGemmVariants - 1 && ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15u) && K % 8 == 0) {
+    return fail(-MI355_E_ALIGN, "gemm_f16_nt: a and b must be 16-byte aligned when K %% 8 == 0");
+  }
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (out_dtype == MI355_F32) return launch_variant<float>(variant, a, b, c, (int)M, (int)N, (int)K, s);
+  return launch_variant<half_t>(variant, a, b, c, (int)M, (int)N, (int)K, s);
+}

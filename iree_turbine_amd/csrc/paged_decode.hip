@@ -1,0 +1,355 @@
+// Paged GQA decode attention for gfx950 (one query token per sequence, head dim 128,
+// 16-token pages, fp16 KV cache laid out [page][token][kv_head][128]).
+//
+// The op is HBM bound: every K and V byte is read exactly once, so the kernel is organised
+// around keeping many page reads in flight and doing the arithmetic on the side.
+//
+// Phase 0: one workgroup (4 waves) per (sequence, kv head, kv split).  The waves take the
+// split's pages round-robin, two pages (32 tokens) per step, and never synchronise with each
+// other until the end: every wave owns a private LDS ring.
+//   - K pages go global -> registers, already in MFMA A-operand layout (lane = token, 16-byte
+//     chunks of the head row), and S^T[token][q head] = K . Q^T is one v_mfma_f32_16x16x32_f16
+//     chain per page with all q heads of the group in the MFMA N dimension.
+//   - V pages go global -> LDS by direct-to-LDS loads (fully coalesced 256-byte rows), and
+//     O^T[d][q head] += V^T . P^T fetches V^T with LDS transpose reads.  The token order inside
+//     that contraction is the order S^T leaves the scores in registers.
+//   - The next step's K and V are requested before the current step is computed; the wait is
+//     on the loads of the current step only (vmcnt counts loads in order).
+//   The four waves' (max, sum, acc) are merged through LDS and written as one fp32 partial per
+//   (seq, q head, split) -- or, with a single split, normalised and written as fp16 directly.
+// Phase 1: merges the splits of every (seq, q head).
+#include "common.hpp"
+#include <math.h>
+
+namespace mi355 {
+
+constexpr int PD_WAVES = 4;
+constexpr int PD_WAVE_LDS = 2 * 8192;  // two stages of two 4 KiB V pages
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+template <int G>  // q heads per kv head (<= 16)
+__global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
+    const half_t* __restrict__ Q, const half_t* __restrict__ Kc, const half_t* __restrict__ Vc,
+    const int* __restrict__ block_table, const int* __restrict__ seq_lens, float* __restrict__ part_acc,
+    float* __restrict__ part_ml, half_t* __restrict__ out, int num_kv_heads, int max_pages_per_seq, int num_splits,
+    float scale_log2e) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int split = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
+  const int num_q_heads = num_kv_heads * G;
+  const int L = seq_lens[seq];
+  const int pages_total = (L + 15) >> 4;
+  const int pps = (pages_total + num_splits - 1) / num_splits;
+  const int p_begin = split * pps;
+  const int p_end = (p_begin + pps < pages_total) ? p_begin + pps : pages_total;
+  const int n_steps = p_end > p_begin ? (p_end - p_begin + 1) >> 1 : 0;
+  const int* bt = block_table + (size_t)seq * max_pages_per_seq;
+
+  const int i16 = lane & 15, g = lane >> 4;
+  // Q^T fragments (MFMA B operand): lane (head i16, chunk g) holds d = 32*ks + 8*g .. +7
+  half8 qf[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ks++) {
+    if (i16 < G) {
+      qf[ks] = *reinterpret_cast<const half8*>(Q + ((size_t)seq * num_q_heads + kvh * G + i16) * 128 + ks * 32 + g * 8);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; e++) qf[ks][e] = (half_t)0;
+    }
+  }
+
+  char* my_lds = lds + wave * PD_WAVE_LDS;
+  const size_t tok_stride = (size_t)num_kv_heads * 128;  // halfs between consecutive tokens of a page
+  const half_t* k_lane = Kc + (size_t)kvh * 128 + i16 * tok_stride + g * 8;
+  // V direct-to-LDS: wave-load i moves rows 4i .. 4i+3; lane: row 4i + lane/16, slot lane%16
+  const int vl_row = lane >> 4, vl_slot = lane & 15;
+  const half_t* v_lane = Vc + (size_t)kvh * 128 + vl_row * tok_stride;
+  // V transpose reads: lane (i16, g) reads row 4g + i16/4, bytes 32*dt + 8*(i16%4) of the row
+  const int vr_row = 4 * g + (i16 >> 2);
+  const int vr_base = vr_row * 256 + ((((i16 & 3) >> 1) ^ (2 * (vr_row & 7))) * 16) + (i16 & 1) * 8;  // ^ (dt*32)
+
+  half8 kf[2][2][4];  // [buffer][page][ks]
+  auto issue = [&](int step, int buf) {
+    const int pa = p_begin + 2 * (wave + PD_WAVES * step);
+    const int pg0 = bt[pa];
+    const int pg1 = (pa + 1 < p_end) ? bt[pa + 1] : pg0;
+    char* dst = my_lds + buf * 8192;
+#pragma unroll
+    for (int x = 0; x < 2; x++) {
+      const size_t page_off = (size_t)(x ? pg1 : pg0) * 16 * tok_stride;
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const int chunk = vl_slot ^ (2 * ((4 * (i & 1) + vl_row) & 7));
+        load_lds_16B(v_lane + page_off + (size_t)(4 * i) * tok_stride + chunk * 8, dst + x * 4096 + i * 1024);
+      }
+    }
+#pragma unroll
+    for (int x = 0; x < 2; x++) {
+      const size_t page_off = (size_t)(x ? pg1 : pg0) * 16 * tok_stride;
+#pragma unroll
+      for (int ks = 0; ks < 4; ks++) kf[buf][x][ks] = *reinterpret_cast<const half8*>(k_lane + page_off + ks * 32);
+    }
+  };
+
+  floatx4 oacc[8];
+#pragma unroll
+  for (int dt = 0; dt < 8; dt++) oacc[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;
+
+  const int my_steps = n_steps > wave ? (n_steps - wave + PD_WAVES - 1) / PD_WAVES : 0;
+  if (my_steps > 0) issue(0, 0);
+#pragma unroll 1
+  for (int u = 0; u < my_steps; u += 2) {
+    // two steps per trip so that the register buffers are indexed statically
+#pragma unroll
+    for (int b = 0; b < 2; b++) {
+      const int step = u + b;
+      if (step < my_steps) {
+        if (step + 1 < my_steps) {
+          issue(step + 1, b ^ 1);
+          asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+        } else {
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        const int pa = p_begin + 2 * (wave + PD_WAVES * step);
+        const bool has1 = pa + 1 < p_end;
+        floatx4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) s0 = mfma_16x16x32(kf[b][0][ks], qf[ks], s0);
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) s1 = mfma_16x16x32(kf[b][1][ks], qf[ks], s1);
+        // lane (head i16, g) holds tokens 4g + r of each page
+        const int tok0 = pa * 16 + 4 * g;
+        const bool ragged = pa * 16 + 32 > L;  // wave-uniform: this step reaches past the sequence end
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          if (tok0 + r >= L) s0[r] = -INFINITY;
+          if (!has1 || tok0 + 16 + r >= L) s1[r] = -INFINITY;
+        }
+        float mx = fmaxf(fmaxf(fmaxf(s0[0], s0[1]), fmaxf(s0[2], s0[3])), fmaxf(fmaxf(s1[0], s1[1]), fmaxf(s1[2], s1[3])));
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_run, mx);  // finite: the first token of page pa is always valid
+        const float alpha = fast_exp2((m_run - m_new) * scale_log2e);
+        const float mc = m_new * scale_log2e;
+        m_run = m_new;
+        half8 pf;
+        float psum = 0.f;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const float p0 = fast_exp2(s0[r] * scale_log2e - mc);
+          const float p1 = fast_exp2(s1[r] * scale_log2e - mc);
+          psum += p0 + p1;
+          pf[r] = (half_t)p0;
+          pf[4 + r] = (half_t)p1;
+        }
+        l_run = l_run * alpha + psum;
+        const char* vst = my_lds + b * 8192;
+#pragma unroll
+        for (int dt = 0; dt < 8; dt++) {
+          half4 lo = lds_read_tr16(vst + (vr_base ^ (dt * 32)));
+          half4 hi = lds_read_tr16(vst + 4096 + (vr_base ^ (dt * 32)));
+          if (ragged) {  // tokens at or beyond L may hold anything (NaN included): 0 * garbage must stay 0
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              if (tok0 + e >= L) lo[e] = (half_t)0;
+              if (!has1 || tok0 + 16 + e >= L) hi[e] = (half_t)0;
+            }
+          }
+          half8 vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          oacc[dt] = oacc[dt] * alpha;
+          oacc[dt] = mfma_16x16x32(vf, pf, oacc[dt]);
+        }
+      }
+    }
+  }
+
+  // ---- merge the four waves through LDS ----
+  l_run += __shfl_xor(l_run, 16);
+  l_run += __shfl_xor(l_run, 32);
+  __syncthreads();  // every wave is done with its V ring
+  float* sm = reinterpret_cast<float*>(lds);              // [wave][G]
+  float* sl = sm + PD_WAVES * 16;                         // [wave][G]
+  float* sacc = sl + PD_WAVES * 16;                       // [wave][G][128]
+  if (i16 < G) {
+    if (g == 0) {
+      sm[wave * 16 + i16] = m_run;
+      sl[wave * 16 + i16] = l_run;
+    }
+#pragma unroll
+    for (int dt = 0; dt < 8; dt++)
+      *reinterpret_cast<floatx4*>(sacc + ((wave * G + i16) * 128 + dt * 16 + 4 * g)) = oacc[dt];
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < G * 128; idx += PD_WAVES * 64) {
+    const int hd = idx >> 7, d = idx & 127;
+    float m_tot = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < PD_WAVES; w++) m_tot = fmaxf(m_tot, sm[w * 16 + hd]);
+    float acc = 0.f, l = 0.f;
+    if (m_tot > -INFINITY) {
+#pragma unroll
+      for (int w = 0; w < PD_WAVES; w++) {
+        const float mw = sm[w * 16 + hd];
+        const float wgt = mw > -INFINITY ? fast_exp2((mw - m_tot) * scale_log2e) : 0.f;
+        acc += wgt * sacc[(w * G + hd) * 128 + d];
+        l += wgt * sl[w * 16 + hd];
+      }
+    }
+    const int qh = kvh * G + hd;
+    if (out) {
+      out[((size_t)seq * num_q_heads + qh) * 128 + d] = (half_t)(l > 0.f ? acc / l : 0.f);
+    } else {
+      const size_t pidx = ((size_t)seq * num_q_heads + qh) * num_splits + split;
+      part_acc[pidx * 128 + d] = acc;
+      if (d == 0) {
+        part_ml[pidx * 2] = m_tot * scale_log2e;
+        part_ml[pidx * 2 + 1] = l;
+      }
+    }
+  }
+}
+
+// Phase 1: one wave per (seq, q head); lane handles d = 2*lane, 2*lane + 1.
+__global__ __launch_bounds__(64) void paged_decode_phase1(const float* __restrict__ part_acc,
+                                                          const float* __restrict__ part_ml, half_t* __restrict__ out,
+                                                          int num_splits) {
+  const size_t row = blockIdx.x;
+  const int lane = threadIdx.x;
+  const float* ml = part_ml + row * num_splits * 2;
+  float m_tot = -INFINITY;
+  for (int s = 0; s < num_splits; s++) m_tot = fmaxf(m_tot, ml[2 * s]);
+  floatx2 acc = {0.f, 0.f};
+  float l = 0.f;
+  if (m_tot > -INFINITY) {
+    for (int s = 0; s < num_splits; s++) {
+      const float ms = ml[2 * s];
+      if (ms > -INFINITY) {
+        const float w = fast_exp2(ms - m_tot);
+        const floatx2 a = *reinterpret_cast<const floatx2*>(part_acc + (row * num_splits + s) * 128 + 2 * lane);
+        acc += w * a;
+        l += w * ml[2 * s + 1];
+      }
+    }
+  }
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  half2v o = {(half_t)(acc[0] * inv), (half_t)(acc[1] * inv)};
+  *reinterpret_cast<half2v*>(out + row * 128 + 2 * lane) = o;
+}
+
+static const char* kDecodeVariants[] = {"d128_p16_w4_2pages"};
+int decode_variant_count() { return 1; }
+const char* decode_variant_name(int i) { return i == 0 ? kDecodeVariants[0] : nullptr; }
+
+template <int G>
+static int launch_phase0(const void* q, const void* kc, const void* vc, const int32_t* bt, const int32_t* sl, float* pacc,
+                         float* pml, void* out, int num_seqs, int num_kv_heads, int max_pages, int num_splits, float scale,
+                         hipStream_t stream) {
+  auto kern = paged_decode_phase0<G>;
+  constexpr int lds_bytes = PD_WAVES * PD_WAVE_LDS;
+  static_assert(lds_bytes >= (int)((2 * PD_WAVES * 16 + PD_WAVES * G * 128) * sizeof(float)), "merge area must fit");
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       lds_bytes);
+    if (e != hipSuccess) {
+      set_error("hipFuncSetAttribute(paged_decode_phase0): %s", hipGetErrorString(e));
+      return (int)e;
+    }
+    attr_set = true;
+  }
+  dim3 grid(num_splits, num_kv_heads, num_seqs), block(PD_WAVES * 64);
+  hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)q, (const half_t*)kc, (const half_t*)vc, bt, sl,
+                     pacc, pml, (half_t*)out, num_kv_heads, max_pages, num_splits, scale * 1.4426950408889634f);
+  return check_launch("paged_decode_phase0", grid, block, lds_bytes);
+}
+
+static int check_decode_args(const char* fn, int64_t num_seqs, int64_t hq, int64_t hkv, int64_t D, int64_t page_size,
+                             int64_t max_pages, int64_t num_pages, int64_t num_splits, float scale) {
+  if (D != 128) return fail(-MI355_E_SHAPE, "%s: head dim %lld not supported (only 128)", fn, (long long)D);
+  if (page_size != 16) return fail(-MI355_E_SHAPE, "%s: page size %lld not supported (only 16)", fn, (long long)page_size);
+  if (num_seqs <= 0 || hq <= 0 || hkv <= 0 || max_pages <= 0 || num_pages <= 0 || num_seqs > 65535 || hkv > 65535)
+    return fail(-MI355_E_SHAPE, "%s: bad sizes seqs=%lld hq=%lld hkv=%lld max_pages=%lld num_pages=%lld", fn,
+                (long long)num_seqs, (long long)hq, (long long)hkv, (long long)max_pages, (long long)num_pages);
+  if (hq % hkv != 0) return fail(-MI355_E_SHAPE, "%s: q heads %lld not a multiple of kv heads %lld", fn, (long long)hq, (long long)hkv);
+  const int64_t G = hq / hkv;
+  if (G != 1 && G != 2 && G != 4 && G != 8 && G != 16)
+    return fail(-MI355_E_SHAPE, "%s: q heads per kv head = %lld, supported: 1, 2, 4, 8, 16", fn, (long long)G);
+  if (num_splits < 1 || num_splits > 1024) return fail(-MI355_E_SHAPE, "%s: num_splits %lld out of range [1, 1024]", fn, (long long)num_splits);
+  if (!(scale > 0.f) || !isfinite(scale)) return fail(-MI355_E_SHAPE, "%s: scale must be positive and finite", fn);
+  return 0;
+}
+
+static int run_phase0(const void* q, const void* kc, const void* vc, const int32_t* bt, const int32_t* sl, float* pacc,
+                      float* pml, void* out, int64_t num_seqs, int64_t hq, int64_t hkv, int64_t max_pages,
+                      int64_t num_splits, float scale, hipStream_t stream) {
+  const int G = (int)(hq / hkv);
+#define MI355_PD_CASE(GG) \
+  case GG: return launch_phase0<GG>(q, kc, vc, bt, sl, pacc, pml, out, (int)num_seqs, (int)hkv, (int)max_pages, (int)num_splits, scale, stream)
+  switch (G) {
+    MI355_PD_CASE(1);
+    MI355_PD_CASE(2);
+    MI355_PD_CASE(4);
+    MI355_PD_CASE(8);
+    MI355_PD_CASE(16);
+  }
+#undef MI355_PD_CASE
+  return fail(-MI355_E_SHAPE, "paged_decode: unsupported group size %d", G);
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" int mi355_paged_decode_phase0(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
+                                         const int32_t* seq_lens, float* part_acc, float* part_ml, int64_t num_seqs,
+                                         int64_t num_q_heads, int64_t num_kv_heads, int64_t D, int64_t page_size,
+                                         int64_t max_pages_per_seq, int64_t num_pages, int64_t num_splits, float scale,
+                                         void* stream) {
+  if (!q || !k_cache || !v_cache || !block_table || !seq_lens) return fail(-MI355_E_NULL, "paged_decode_phase0: null pointer");
+  if (int rc = check_decode_args("paged_decode_phase0", num_seqs, num_q_heads, num_kv_heads, D, page_size, max_pages_per_seq,
+                                 num_pages, num_splits, scale))
+    return rc;
+  if (!part_acc || !part_ml) return fail(-MI355_E_SCRATCH, "paged_decode_phase0: part_acc / part_ml scratch is required");
+  if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(part_acc))
+    return fail(-MI355_E_ALIGN, "paged_decode_phase0: q, k_cache, v_cache, part_acc must be 16-byte aligned");
+  return run_phase0(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, nullptr, num_seqs, num_q_heads,
+                    num_kv_heads, max_pages_per_seq, num_splits, scale, reinterpret_cast<hipStream_t>(stream));
+}
+
+extern "C" int mi355_paged_decode_phase1(const float* part_acc, const float* part_ml, void* out, int64_t num_seqs,
+                                         int64_t num_q_heads, int64_t D, int64_t num_splits, void* stream) {
+  if (!part_acc || !part_ml || !out) return fail(-MI355_E_NULL, "paged_decode_phase1: null pointer");
+  if (D != 128) return fail(-MI355_E_SHAPE, "paged_decode_phase1: head dim %lld not supported (only 128)", (long long)D);
+  if (num_seqs <= 0 || num_q_heads <= 0 || num_splits < 1 || num_splits > 1024 || num_seqs * num_q_heads > (1ll << 30))
+    return fail(-MI355_E_SHAPE, "paged_decode_phase1: bad sizes");
+  dim3 grid((unsigned)(num_seqs * num_q_heads)), block(64);
+  hipLaunchKernelGGL(paged_decode_phase1, grid, block, 0, reinterpret_cast<hipStream_t>(stream), part_acc, part_ml,
+                     (half_t*)out, (int)num_splits);
+  return check_launch("paged_decode_phase1", grid, block, 0);
+}
+
+extern "C" int mi355_paged_decode_attn(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
+                                       const int32_t* seq_lens, void* out, float* part_acc, float* part_ml, int64_t num_seqs,
+                                       int64_t num_q_heads, int64_t num_kv_heads, int64_t D, int64_t page_size,
+                                       int64_t max_pages_per_seq, int64_t num_pages, int64_t num_splits, float scale,
+                                       void* stream) {
+  if (!q || !k_cache || !v_cache || !block_table || !seq_lens || !out) return fail(-MI355_E_NULL, "paged_decode_attn: null pointer");
+  if (int rc = check_decode_args("paged_decode_attn", num_seqs, num_q_heads, num_kv_heads, D, page_size, max_pages_per_seq,
+                                 num_pages, num_splits, scale))
+    return rc;
+  if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out))
+    return fail(-MI355_E_ALIGN, "paged_decode_attn: q, k_cache, v_cache, out must be 16-byte aligned");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (num_splits == 1)
+    return run_phase0(q, k_cache, v_cache, block_table, seq_lens, nullptr, nullptr, out, num_seqs, num_q_heads, num_kv_heads,
+                      max_pages_per_seq, 1, scale, s);
+  if (!part_acc || !part_ml) return fail(-MI355_E_SCRATCH, "paged_decode_attn: num_splits > 1 needs part_acc / part_ml scratch");
+  if (!aligned16(part_acc)) return fail(-MI355_E_ALIGN, "paged_decode_attn: part_acc must be 16-byte aligned");
+  if (int rc = run_phase0(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, nullptr, num_seqs, num_q_heads,
+                          num_kv_heads, max_pages_per_seq, num_splits, scale, s))
+    return rc;
+  return mi355_paged_decode_phase1(part_acc, part_ml, out, num_seqs, num_q_heads, D, num_splits, stream);
+}

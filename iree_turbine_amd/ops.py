@@ -1,0 +1,313 @@
+"""`torch.ops.mi355.*`: the dense kernels as PyTorch custom ops.
+
+Each op is a `CustomOp` (see op_reg.py): `select` is the shape/dtype contract (and the Meta
+kernel), `eager_execute` hands raw device pointers to the C ABI on torch's current stream.
+Tensor layouts are the contiguous layouts the reference's launch path enforces
+(iree/turbine/runtime/op_reg/eager.py:119-132 makes every input `.contiguous()`).
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+from torch import Tensor
+
+from . import _lib
+from .op_reg import CustomOp, KernelSelection
+
+__all__ = [
+    "gemm_nt",
+    "flash_attn_fwd",
+    "paged_decode_attn",
+    "paged_decode_phase0",
+    "paged_decode_phase1",
+    "mxfp4_gemm",
+    "mxfp4_dequant",
+]
+
+_OUT_DTYPES = {"float32": torch.float32, "float16": torch.float16, "bfloat16": torch.bfloat16}
+
+
+def _require(cond: bool, msg: str) -> None:
+    if not cond:
+        raise ValueError(msg)
+
+
+def _ptr(t: Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def _same_device(*tensors: Tensor) -> torch.device:
+    dev = tensors[0].device
+    for t in tensors[1:]:
+        if t.device != dev:
+            raise RuntimeError(f"Cannot launch with tensors from multiple devices: {t.device} vs {dev}")
+    return dev
+
+
+@CustomOp.register
+class gemm_nt(CustomOp):
+    """C[M,N] = A[M,K] . B[N,K]^T, fp16 inputs, fp32 accumulation; out_dtype "float32" | "float16".
+
+    The NT form is what `gemmfp16 ... --transB 1` computes in the reference
+    (iree/turbine/kernel/boo/op_exports/gemm.py:84-86,228-230) and what `nn.Linear` hands to a
+    kernel (tests/kernel/boo/fusion/subgraph_fusion_test.py:100-116)."""
+
+    signature = "gemm_nt(Tensor a, Tensor b, str out_dtype, int variant) -> Tensor"
+
+    def select(self, sel: KernelSelection):
+        a, b = sel.arg_tensor(0), sel.arg_tensor(1)
+        od = sel.attr_str(2).v
+        sel.attr_int(3)
+        _require(a.t.dim() == 2 and b.t.dim() == 2, "gemm_nt: a and b must be rank 2")
+        _require(a.t.dtype == torch.float16 and b.t.dtype == torch.float16, "gemm_nt: a and b must be float16")
+        _require(a.t.size(1) == b.t.size(1), f"gemm_nt: K mismatch, a is {tuple(a.t.shape)}, b is {tuple(b.t.shape)} (b is [N, K])")
+        _require(od in ("float32", "float16"), f"gemm_nt: out_dtype must be 'float32' or 'float16', got {od!r}")
+        _require(a.t.size(0) > 0 and b.t.size(0) > 0 and a.t.size(1) > 0, "gemm_nt: empty operand")
+        a.specialize_all_dims()
+        b.specialize_all_dims()
+        sel.return_new_tensor([a.t.size(0), b.t.size(0)], _OUT_DTYPES[od]).specialize_all_dims()
+
+    def eager_execute(self, a, b, out_dtype, variant):
+        dev = _same_device(a, b)
+        a, b = a.contiguous(), b.contiguous()
+        M, K = a.shape
+        N = b.shape[0]
+        c = torch.empty((M, N), dtype=_OUT_DTYPES[out_dtype], device=dev)
+        with torch.cuda.device(dev):
+            rc = _lib.load().mi355_gemm_f16_nt(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K,
+                                               _lib.dtype_code(c.dtype), variant, _lib.current_stream_ptr(dev))
+        _lib.check(rc, f"gemm_nt M={M} N={N} K={K} out={out_dtype} variant={variant}")
+        return c
+
+
+@CustomOp.register
+class flash_attn_fwd(CustomOp):
+    """softmax(scale . Q K^T [+ causal mask]) V for q [B,H,Sq,128], k/v [B,H,Sk,128] fp16.
+
+    Same argument meaning as aten.scaled_dot_product_attention(q, k, v, None, 0.0, is_causal,
+    scale=) -- the canonical form the reference rewrites SDPA variants to
+    (iree/turbine/kernel/boo/fusion/replacement.py:275-284).  scale <= 0 selects 1/sqrt(D)."""
+
+    signature = "flash_attn_fwd(Tensor q, Tensor k, Tensor v, bool is_causal, float scale) -> Tensor"
+
+    def select(self, sel: KernelSelection):
+        q, k, v = sel.arg_tensor(0), sel.arg_tensor(1), sel.arg_tensor(2)
+        sel.attr_bool(3)
+        sel.attr_float(4)
+        for name, t in (("q", q.t), ("k", k.t), ("v", v.t)):
+            _require(t.dim() == 4, f"flash_attn_fwd: {name} must be [B, H, S, D]")
+            _require(t.dtype == torch.float16, f"flash_attn_fwd: {name} must be float16")
+        _require(q.t.size(3) == 128, f"flash_attn_fwd: head dim {q.t.size(3)} not supported (only 128)")
+        _require(k.t.shape == v.t.shape, "flash_attn_fwd: k and v shapes differ")
+        _require(q.t.shape[:2] == k.t.shape[:2] and q.t.size(3) == k.t.size(3), "flash_attn_fwd: q and k disagree on B, H or D")
+        _require(q.t.size(2) > 0 and k.t.size(2) > 0, "flash_attn_fwd: empty sequence")
+        for d in (q, k, v):
+            d.specialize_dims(1, 3)
+        sel.return_new_tensor(list(q.t.shape), torch.float16)
+
+    def eager_execute(self, q, k, v, is_causal, scale):
+        dev = _same_device(q, k, v)
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        B, H, Sq, D = q.shape
+        Sk = k.shape[2]
+        if scale <= 0:
+            scale = 1.0 / math.sqrt(D)
+        o = torch.empty_like(q)
+        with torch.cuda.device(dev):
+            rc = _lib.load().mi355_flash_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), B, H, Sq, Sk, D,
+                                                  scale, int(is_causal), -1, _lib.current_stream_ptr(dev))
+        _lib.check(rc, f"flash_attn_fwd B={B} H={H} Sq={Sq} Sk={Sk} D={D} causal={is_causal}")
+        return o
+
+
+def _check_paged_args(op: str, q: Tensor, k_cache: Tensor, v_cache: Tensor, block_table: Tensor, seq_lens: Tensor):
+    _require(q.dim() == 3, f"{op}: q must be [num_seqs, num_q_heads, D]")
+    _require(k_cache.dim() == 4 and v_cache.shape == k_cache.shape, f"{op}: k_cache / v_cache must both be [num_pages, page_size, num_kv_heads, D]")
+    _require(q.dtype == torch.float16 and k_cache.dtype == torch.float16 and v_cache.dtype == torch.float16, f"{op}: q, k_cache, v_cache must be float16")
+    _require(block_table.dim() == 2 and block_table.dtype == torch.int32, f"{op}: block_table must be int32 [num_seqs, max_pages_per_seq]")
+    _require(seq_lens.dim() == 1 and seq_lens.dtype == torch.int32, f"{op}: seq_lens must be int32 [num_seqs]")
+    _require(block_table.size(0) == q.size(0) and seq_lens.size(0) == q.size(0), f"{op}: block_table / seq_lens rows must equal num_seqs")
+    _require(q.size(2) == 128 and k_cache.size(3) == 128, f"{op}: head dim must be 128")
+    _require(k_cache.size(1) == 16, f"{op}: page size {k_cache.size(1)} not supported (only 16)")
+    hq, hkv = q.size(1), k_cache.size(2)
+    _require(hkv > 0 and hq % hkv == 0 and hq // hkv in (1, 2, 4, 8, 16), f"{op}: {hq} q heads over {hkv} kv heads is not supported (ratio 1, 2, 4, 8 or 16)")
+    _require(q.size(0) > 0 and block_table.size(1) > 0, f"{op}: empty batch")
+
+
+def default_num_kv_splits(seq_lens_max: int, num_seqs: int, num_kv_heads: int) -> int:
+    """Splits so that there are a few thousand workgroups of at least ~16 pages each."""
+    pages = max(1, (seq_lens_max + 15) // 16)
+    want = max(1, 2048 // max(1, num_seqs * num_kv_heads))
+    return int(max(1, min(want, pages // 16 if pages >= 16 else 1, 64)))
+
+
+@CustomOp.register
+class paged_decode_attn(CustomOp):
+    """One-token-per-sequence GQA attention over a paged fp16 KV cache (both phases).
+
+    q [S, Hq, 128]; k_cache, v_cache [P, 16, Hkv, 128]; block_table int32 [S, max_pages];
+    seq_lens int32 [S]; returns [S, Hq, 128] fp16.  num_kv_splits <= 0 picks a default from
+    the table width.  scale <= 0 selects 1/sqrt(D).  GQA semantics (q head h reads kv head
+    h // (Hq/Hkv)) follow repeat_kv in tests/dynamo/llama_test.py:82-91."""
+
+    signature = "paged_decode_attn(Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_table, Tensor seq_lens, float scale, int num_kv_splits) -> Tensor"
+
+    def select(self, sel: KernelSelection):
+        q, kc, vc, bt, sl = (sel.arg_tensor(i) for i in range(5))
+        sel.attr_float(5)
+        sel.attr_int(6)
+        _check_paged_args("paged_decode_attn", q.t, kc.t, vc.t, bt.t, sl.t)
+        q.specialize_dims(1, 2)
+        kc.specialize_dims(1, 2, 3)
+        vc.specialize_dims(1, 2, 3)
+        sel.return_new_tensor(list(q.t.shape), torch.float16)
+
+    def eager_execute(self, q, k_cache, v_cache, block_table, seq_lens, scale, num_kv_splits):
+        dev = _same_device(q, k_cache, v_cache, block_table, seq_lens)
+        q, k_cache, v_cache = q.contiguous(), k_cache.contiguous(), v_cache.contiguous()
+        block_table, seq_lens = block_table.contiguous(), seq_lens.contiguous()
+        S, Hq, D = q.shape
+        P, page, Hkv, _ = k_cache.shape
+        max_pages = block_table.shape[1]
+        if scale <= 0:
+            scale = 1.0 / math.sqrt(D)
+        if num_kv_splits <= 0:
+            num_kv_splits = default_num_kv_splits(max_pages * page, S, Hkv)
+        out = torch.empty_like(q)
+        pacc = pml = None
+        if num_kv_splits > 1:
+            pacc = torch.empty((S, Hq, num_kv_splits, D), dtype=torch.float32, device=dev)
+            pml = torch.empty((S, Hq, num_kv_splits, 2), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            rc = _lib.load().mi355_paged_decode_attn(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                                                     block_table.data_ptr(), seq_lens.data_ptr(), out.data_ptr(),
+                                                     _ptr(pacc), _ptr(pml), S, Hq, Hkv, D, page, max_pages, P,
+                                                     num_kv_splits, scale, _lib.current_stream_ptr(dev))
+        _lib.check(rc, f"paged_decode_attn seqs={S} hq={Hq} hkv={Hkv} pages={P} splits={num_kv_splits}")
+        return out
+
+
+@CustomOp.register
+class paged_decode_phase0(CustomOp):
+    """Phase 0 of the split-K decode: per (seq, q head, split) an unnormalised fp32 partial
+    output [S, Hq, splits, 128] and its (max in log2 units, sum) [S, Hq, splits, 2]."""
+
+    signature = "paged_decode_phase0(Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_table, Tensor seq_lens, float scale, int num_kv_splits) -> (Tensor, Tensor)"
+
+    def select(self, sel: KernelSelection):
+        q, kc, vc, bt, sl = (sel.arg_tensor(i) for i in range(5))
+        sel.attr_float(5)
+        ns = sel.attr_int(6).v
+        _check_paged_args("paged_decode_phase0", q.t, kc.t, vc.t, bt.t, sl.t)
+        _require(1 <= ns <= 1024, "paged_decode_phase0: num_kv_splits must be in [1, 1024]")
+        S, Hq, D = q.t.shape
+        sel.return_new_tensor([S, Hq, ns, D], torch.float32)
+        sel.return_new_tensor([S, Hq, ns, 2], torch.float32)
+
+    def eager_execute(self, q, k_cache, v_cache, block_table, seq_lens, scale, num_kv_splits):
+        dev = _same_device(q, k_cache, v_cache, block_table, seq_lens)
+        q, k_cache, v_cache = q.contiguous(), k_cache.contiguous(), v_cache.contiguous()
+        block_table, seq_lens = block_table.contiguous(), seq_lens.contiguous()
+        S, Hq, D = q.shape
+        P, page, Hkv, _ = k_cache.shape
+        if scale <= 0:
+            scale = 1.0 / math.sqrt(D)
+        pacc = torch.empty((S, Hq, num_kv_splits, D), dtype=torch.float32, device=dev)
+        pml = torch.empty((S, Hq, num_kv_splits, 2), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            rc = _lib.load().mi355_paged_decode_phase0(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                                                       block_table.data_ptr(), seq_lens.data_ptr(), pacc.data_ptr(),
+                                                       pml.data_ptr(), S, Hq, Hkv, D, page, block_table.shape[1], P,
+                                                       num_kv_splits, scale, _lib.current_stream_ptr(dev))
+        _lib.check(rc, f"paged_decode_phase0 seqs={S} hq={Hq} hkv={Hkv} splits={num_kv_splits}")
+        return pacc, pml
+
+
+@CustomOp.register
+class paged_decode_phase1(CustomOp):
+    """Phase 1 of the split-K decode: merges the partials of phase 0 into [S, Hq, 128] fp16."""
+
+    signature = "paged_decode_phase1(Tensor part_acc, Tensor part_ml) -> Tensor"
+
+    def select(self, sel: KernelSelection):
+        pa, pm = sel.arg_tensor(0), sel.arg_tensor(1)
+        _require(pa.t.dim() == 4 and pa.t.dtype == torch.float32 and pa.t.size(3) == 128, "paged_decode_phase1: part_acc must be fp32 [S, Hq, splits, 128]")
+        _require(pm.t.dtype == torch.float32 and tuple(pm.t.shape) == (*pa.t.shape[:3], 2), "paged_decode_phase1: part_ml must be fp32 [S, Hq, splits, 2]")
+        sel.return_new_tensor([pa.t.size(0), pa.t.size(1), 128], torch.float16)
+
+    def eager_execute(self, part_acc, part_ml):
+        dev = _same_device(part_acc, part_ml)
+        part_acc, part_ml = part_acc.contiguous(), part_ml.contiguous()
+        S, Hq, ns, D = part_acc.shape
+        out = torch.empty((S, Hq, D), dtype=torch.float16, device=dev)
+        with torch.cuda.device(dev):
+            rc = _lib.load().mi355_paged_decode_phase1(part_acc.data_ptr(), part_ml.data_ptr(), out.data_ptr(), S, Hq, D, ns,
+                                                       _lib.current_stream_ptr(dev))
+        _lib.check(rc, f"paged_decode_phase1 seqs={S} hq={Hq} splits={ns}")
+        return out
+
+
+def _check_mx_operand(op: str, name: str, codes: Tensor, scales: Tensor):
+    _require(codes.dim() == 2 and codes.dtype == torch.uint8, f"{op}: {name} must be uint8 [rows, K/2] (two E2M1 codes per byte)")
+    _require(scales.dim() == 2 and scales.dtype == torch.uint8, f"{op}: {name}_scale must be uint8 [rows, K/32] (E8M0)")
+    K = codes.size(1) * 2
+    _require(K > 0 and K % 32 == 0, f"{op}: K={K} must be a positive multiple of 32")
+    _require(scales.size(0) == codes.size(0) and scales.size(1) == K // 32, f"{op}: {name}_scale shape {tuple(scales.shape)} does not match {name} {tuple(codes.shape)}")
+
+
+@CustomOp.register
+class mxfp4_gemm(CustomOp):
+    """C[M,N] = dq(A) . dq(B)^T for OCP MXFP4 operands (see include/turbine_mi355.h for the format);
+    out_dtype "bfloat16" | "float32"."""
+
+    signature = "mxfp4_gemm(Tensor a, Tensor a_scale, Tensor b, Tensor b_scale, str out_dtype, int variant) -> Tensor"
+
+    def select(self, sel: KernelSelection):
+        a, asc, b, bsc = (sel.arg_tensor(i) for i in range(4))
+        od = sel.attr_str(4).v
+        sel.attr_int(5)
+        _check_mx_operand("mxfp4_gemm", "a", a.t, asc.t)
+        _check_mx_operand("mxfp4_gemm", "b", b.t, bsc.t)
+        _require(a.t.size(1) == b.t.size(1), "mxfp4_gemm: a and b disagree on K")
+        _require(od in ("bfloat16", "float32"), f"mxfp4_gemm: out_dtype must be 'bfloat16' or 'float32', got {od!r}")
+        _require(a.t.size(0) > 0 and b.t.size(0) > 0, "mxfp4_gemm: empty operand")
+        for d in (a, asc, b, bsc):
+            d.specialize_all_dims()
+        sel.return_new_tensor([a.t.size(0), b.t.size(0)], _OUT_DTYPES[od]).specialize_all_dims()
+
+    def eager_execute(self, a, a_scale, b, b_scale, out_dtype, variant):
+        dev = _same_device(a, a_scale, b, b_scale)
+        a, a_scale, b, b_scale = a.contiguous(), a_scale.contiguous(), b.contiguous(), b_scale.contiguous()
+        M, N, K = a.shape[0], b.shape[0], a.shape[1] * 2
+        c = torch.empty((M, N), dtype=_OUT_DTYPES[out_dtype], device=dev)
+        with torch.cuda.device(dev):
+            rc = _lib.load().mi355_mxfp4_gemm(a.data_ptr(), a_scale.data_ptr(), b.data_ptr(), b_scale.data_ptr(), c.data_ptr(),
+                                              M, N, K, _lib.dtype_code(c.dtype), variant, _lib.current_stream_ptr(dev))
+        _lib.check(rc, f"mxfp4_gemm M={M} N={N} K={K} out={out_dtype} variant={variant}")
+        return c
+
+
+@CustomOp.register
+class mxfp4_dequant(CustomOp):
+    """fp32 [rows, K] = E2M1(code) * 2^(scale - 127), computed on the device."""
+
+    signature = "mxfp4_dequant(Tensor codes, Tensor scales) -> Tensor"
+
+    def select(self, sel: KernelSelection):
+        c, s = sel.arg_tensor(0), sel.arg_tensor(1)
+        _check_mx_operand("mxfp4_dequant", "codes", c.t, s.t)
+        _require(c.t.size(0) > 0, "mxfp4_dequant: empty operand")
+        sel.return_new_tensor([c.t.size(0), c.t.size(1) * 2], torch.float32)
+
+    def eager_execute(self, codes, scales):
+        dev = _same_device(codes, scales)
+        codes, scales = codes.contiguous(), scales.contiguous()
+        rows, K = codes.shape[0], codes.shape[1] * 2
+        out = torch.empty((rows, K), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            rc = _lib.load().mi355_mxfp4_dequant(codes.data_ptr(), scales.data_ptr(), out.data_ptr(), rows, K,
+                                                 _lib.current_stream_ptr(dev))
+        _lib.check(rc, f"mxfp4_dequant rows={rows} K={K}")
+        return out

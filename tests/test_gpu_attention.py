@@ -1,0 +1,101 @@
+"""GPU parity: flash-attention prefill through the C ABI vs the CPU oracle (fp32 SDPA), atol 2e-3."""
+
+import math
+
+import pytest
+import torch
+
+from conftest import announce
+
+pytestmark = pytest.mark.gpu
+
+ATOL = 2e-3  # the tolerance BASELINE states for fp16 attention outputs
+RTOL = 1e-2
+
+
+def _run(dev, B, H, Sq, D, causal, seed=10, Sk=None):
+    import iree_turbine_amd  # noqa: F401
+    from oracle import attention as oa, inputs
+
+    announce(f"flash_attn_fwd B={B} H={H} Sq={Sq} Sk={Sk} D={D} causal={causal} seed={seed}")
+    q, k, v = inputs.attention_inputs(B, H, Sq, D, seed=seed, Sk=Sk)
+    o = torch.ops.mi355.flash_attn_fwd(q.to(dev), k.to(dev), v.to(dev), causal, 0.0)
+    torch.cuda.synchronize()
+    return o.float().cpu(), oa.sdpa_ref(q, k, v, is_causal=causal), (q, k, v)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("S", [128, 256, 1024])
+def test_attention_aligned(dev, S, causal):
+    o, ref, _ = _run(dev, 2, 4, S, 128, causal)
+    torch.testing.assert_close(o, ref, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("S", [1, 17, 64, 100, 129, 333])
+def test_attention_ragged(dev, S, causal):
+    o, ref, _ = _run(dev, 1, 3, S, 128, causal)
+    torch.testing.assert_close(o, ref, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_cross_lengths(dev, causal):
+    o, ref, _ = _run(dev, 1, 2, 96, 128, causal, Sk=320)
+    torch.testing.assert_close(o, ref, rtol=RTOL, atol=ATOL)
+
+
+def test_attention_invariants(dev):
+    import iree_turbine_amd  # noqa: F401
+
+    announce("attention invariants")
+    B, H, S, D = 1, 2, 512, 128
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(B, H, S, D, generator=g).half().to(dev)
+    k = torch.randn(B, H, S, D, generator=g).half().to(dev)
+    v = torch.randn(B, H, S, D, generator=g).half().to(dev)
+    # rows of P sum to one: V = 1 => O = 1
+    o = torch.ops.mi355.flash_attn_fwd(q, k, torch.ones_like(v), False, 0.0)
+    assert (o.float() - 1).abs().max().item() <= 1e-3
+    # causal row 0 sees only key 0
+    oc = torch.ops.mi355.flash_attn_fwd(q, k, v, True, 0.0)
+    assert torch.equal(oc[:, :, 0], v[:, :, 0])
+    # Q = 0: uniform weights => prefix means (causal) / the mean (non-causal) of V
+    z = torch.zeros_like(q)
+    om = torch.ops.mi355.flash_attn_fwd(z, k, v, False, 0.0).float()
+    torch.testing.assert_close(om, v.float().mean(dim=2, keepdim=True).expand_as(om), rtol=1e-2, atol=2e-3)
+    op = torch.ops.mi355.flash_attn_fwd(z, k, v, True, 0.0).float()
+    pref = v.float().cumsum(dim=2) / torch.arange(1, S + 1, device=dev).view(1, 1, S, 1)
+    torch.testing.assert_close(op, pref, rtol=1e-2, atol=2e-3)
+    # permuting the keys (with their values) does not change non-causal attention
+    perm = torch.randperm(S, generator=g).to(dev)
+    o1 = torch.ops.mi355.flash_attn_fwd(q, k, v, False, 0.0).float()
+    o2 = torch.ops.mi355.flash_attn_fwd(q, k[:, :, perm], v[:, :, perm], False, 0.0).float()
+    torch.testing.assert_close(o1, o2, rtol=1e-2, atol=2e-3)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_full_size(dev, causal):
+    """B=2 H=32 S=4096 D=128: two full heads against the oracle, every head against torch's GPU SDPA."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import attention as oa, inputs
+
+    announce(f"attention full size causal={causal}")
+    q, k, v = inputs.attention_inputs(2, 32, 4096, 128)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    o = torch.ops.mi355.flash_attn_fwd(qd, kd, vd, causal, 0.0)
+    for (b, h) in [(0, 0), (1, 31)]:
+        ref = oa.sdpa_ref(q[b, h], k[b, h], v[b, h], is_causal=causal)
+        torch.testing.assert_close(o[b, h].float().cpu(), ref, rtol=RTOL, atol=ATOL)
+    lib = torch.nn.functional.scaled_dot_product_attention(qd.float(), kd.float(), vd.float(), is_causal=causal)
+    torch.testing.assert_close(o.float(), lib, rtol=RTOL, atol=ATOL)
+
+
+def test_attention_contract_errors(dev):
+    import iree_turbine_amd  # noqa: F401
+
+    q = torch.zeros(1, 1, 16, 64, dtype=torch.float16, device=dev)
+    with pytest.raises(ValueError):
+        torch.ops.mi355.flash_attn_fwd(q, q, q, False, 0.0)  # D = 64
+    q = torch.zeros(1, 1, 16, 128, dtype=torch.float32, device=dev)
+    with pytest.raises(ValueError):
+        torch.ops.mi355.flash_attn_fwd(q, q, q, False, 0.0)

@@ -1,0 +1,124 @@
+"""GPU parity: fp16 NT GEMM through the C ABI vs the CPU oracle (torch fp32 matmul), rtol = atol = 1e-2."""
+
+import pytest
+import torch
+
+from conftest import announce
+
+pytestmark = pytest.mark.gpu
+
+RTOL = ATOL = 1e-2  # the tolerance BASELINE states for the fp16 GEMM
+
+
+def _run(dev, M, N, K, out_dtype, variant=-1, seed=10):
+    import iree_turbine_amd as ita
+    from oracle import gemm as og, inputs
+
+    announce(f"gemm_nt M={M} N={N} K={K} out={out_dtype} variant={variant} seed={seed}")
+    a, b = inputs.gemm_inputs(M, N, K, seed=seed)
+    c = torch.ops.mi355.gemm_nt(a.to(dev), b.to(dev), out_dtype, variant)
+    torch.cuda.synchronize()
+    ref = og.gemm_nt_ref(a, b)
+    return c.float().cpu(), ref
+
+
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 3])
+def test_gemm_1024_f32_all_variants(dev, variant):
+    c, ref = _run(dev, 1024, 1024, 1024, "float32", variant)
+    torch.testing.assert_close(c, ref, rtol=RTOL, atol=ATOL)
+    # fp32 output of an fp32-accumulating kernel should be much closer than the stated tolerance
+    assert (c - ref).abs().max().item() < 1e-3
+
+
+@pytest.mark.parametrize("shape", [(256, 256, 64), (512, 768, 192), (2048, 1024, 4096), (128, 384, 640)])
+@pytest.mark.parametrize("out_dtype", ["float32", "float16"])
+def test_gemm_tiled_shapes(dev, shape, out_dtype):
+    c, ref = _run(dev, *shape, out_dtype)
+    torch.testing.assert_close(c, ref, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("shape", [(16, 16, 16), (32, 32, 32), (1, 1, 1), (65, 33, 17), (100, 200, 72), (3, 129, 257), (64, 64, 8)])
+def test_gemm_ragged_shapes(dev, shape):
+    # the reference's own smoke sizes are 16^3 / 32^3 (tests/kernel/boo/driver/numerics_smoke_test.py:473-520)
+    c, ref = _run(dev, *shape, "float32")
+    torch.testing.assert_close(c, ref, rtol=RTOL, atol=ATOL)
+    c16, _ = _run(dev, *shape, "float16")
+    torch.testing.assert_close(c16, ref, rtol=RTOL, atol=ATOL)
+
+
+def test_gemm_identity_and_ones(dev):
+    import iree_turbine_amd  # noqa: F401
+
+    announce("gemm identity / block of ones")
+    M = K = 512
+    N = 256
+    b = (torch.randn(N, K) * 0.5).half()
+    eye = torch.eye(M, K).half()
+    c = torch.ops.mi355.gemm_nt(eye.to(dev), b.to(dev), "float16", -1).cpu()
+    assert torch.equal(c, b.t().contiguous())  # A = I  =>  C = B^T exactly
+    # structured block-of-ones (the idea of numerics.py:319-338): integer sums are exact
+    a1 = torch.zeros(256, 1024).half()
+    a1[32:96, 100:612] = 1
+    b1 = torch.zeros(256, 1024).half()
+    b1[:, 300:900] = 1
+    c1 = torch.ops.mi355.gemm_nt(a1.to(dev), b1.to(dev), "float32", -1).cpu()
+    exp = torch.zeros(256, 256)
+    exp[32:96, :] = 612 - 300
+    assert torch.equal(c1, exp)
+
+
+def test_gemm_error_statistics(dev):
+    """The reference's three-way criteria (numerics.py:266-316): no drift, and an error spread no worse
+    than 1.2x torch's own GPU GEMM, both measured against an fp64 CPU result."""
+    from oracle import gemm as og, inputs, numerics as on
+
+    announce("gemm error statistics 1024x1024x2048")
+    a, b = inputs.gemm_inputs(1024, 1024, 2048, seed=3)
+    ref64 = og.gemm_nt_f64(a, b)
+    ours = torch.ops.mi355.gemm_nt(a.to(dev), b.to(dev), "float16", -1).cpu()
+    theirs = torch.mm(a.to(dev), b.to(dev).t()).cpu()
+    e_ours, nan1 = on.element_errors(ours, ref64)
+    e_theirs, nan2 = on.element_errors(theirs, ref64)
+    s_ours, s_theirs = on.error_statistics(e_ours), on.error_statistics(e_theirs)
+    assert not nan1 and not nan2
+    assert on.mean_near_zero(s_ours), s_ours
+    assert on.stddev_ratio_ok(s_ours, s_theirs), (s_ours, s_theirs)
+
+
+def test_gemm_contract_errors(dev):
+    import iree_turbine_amd  # noqa: F401
+
+    a = torch.zeros(64, 64, dtype=torch.float16, device=dev)
+    with pytest.raises(ValueError):
+        torch.ops.mi355.gemm_nt(a, torch.zeros(64, 32, dtype=torch.float16, device=dev), "float32", -1)
+    with pytest.raises(ValueError):
+        torch.ops.mi355.gemm_nt(a.float(), a.float(), "float32", -1)
+    with pytest.raises(ValueError):
+        torch.ops.mi355.gemm_nt(a, a, "float32", 0)  # 256x256 tile does not divide 64x64
+    with pytest.raises(ValueError):
+        torch.ops.mi355.gemm_nt(a, a, "int8", -1)
+
+
+@pytest.mark.parametrize("shape", [(8192, 8192, 8192), (4096, 4096, 4096), (2048, 10240, 8192)])
+def test_gemm_full_size_properties(dev, shape):
+    """At benchmark sizes: sampled rows/columns against the fp32 oracle, plus linearity in A."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs
+
+    M, N, K = shape
+    announce(f"gemm full size {shape}")
+    a, b = inputs.gemm_inputs(M, N, K)
+    ad, bd = a.to(dev), b.to(dev)
+    c = torch.ops.mi355.gemm_nt(ad, bd, "float16", -1)
+    rows = torch.tensor([0, 1, 255, 256, M // 2 + 7, M - 1])
+    cols = torch.tensor([0, 31, 32, 257, N // 2 + 3, N - 1])
+    ref_rows = a[rows].float() @ b.float().t()
+    torch.testing.assert_close(c[rows.to(dev)].float().cpu(), ref_rows, rtol=RTOL, atol=ATOL)
+    ref_cols = a.float() @ b[cols].float().t()
+    torch.testing.assert_close(c[:, cols.to(dev)].float().cpu(), ref_cols, rtol=RTOL, atol=ATOL)
+    # linearity: (2A) B^T == 2 (A B^T) bit for bit with fp32 output (doubling is exact in every
+    # product and partial sum; fp16 output would differ where results round into subnormals)
+    c32 = torch.ops.mi355.gemm_nt(ad, bd, "float32", -1)
+    c2 = torch.ops.mi355.gemm_nt(ad * 2, bd, "float32", -1)
+    assert torch.equal(c2, c32 * 2)
+    assert torch.equal(c32.half(), c)  # the fp16 epilogue is round-to-nearest-even of the fp32 result

@@ -1,0 +1,146 @@
+"""GPU parity: MXFP4 dequantisation (bit-exact) and block-scaled GEMM (<= 1e-2 relative) through the C ABI."""
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import announce
+
+pytestmark = pytest.mark.gpu
+
+REL = 1e-2  # BASELINE: GEMM within 1e-2 relative of an fp32 matmul on the dequantised operands
+
+
+def _rel_err(c: torch.Tensor, ref: torch.Tensor) -> float:
+    return ((c.double() - ref.double()).norm() / ref.double().norm()).item()
+
+
+def test_dequant_exhaustive_bit_exact(dev):
+    """All 16 codes x all 256 scale bytes, in both nibble positions, bit for bit (NaN for 0xFF)."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import mxfp4 as om
+
+    announce("mxfp4 dequant exhaustive")
+    rows, K = 256, 64
+    k = np.arange(K)
+    elem_codes = np.where(k < 32, k % 16, (k + 1) % 16).astype(np.uint8)  # every code in both nibble positions
+    packed = torch.from_numpy(np.ascontiguousarray(np.broadcast_to(om.pack_codes(elem_codes[None, :]), (rows, K // 2))))
+    scales = torch.arange(256, dtype=torch.int32).to(torch.uint8).reshape(rows, 1).repeat(1, 2)
+    out = torch.ops.mi355.mxfp4_dequant(packed.to(dev), scales.to(dev)).cpu().numpy()
+    ref = om.mxfp4_dequant_ref(packed, scales)
+    assert out.dtype == np.float32 and out.shape == ref.shape
+    assert np.array_equal(out.view(np.uint32)[:255], ref.view(np.uint32)[:255])
+    assert np.isnan(out[255]).all() and np.isnan(ref[255]).all()
+
+
+def test_dequant_random_bit_exact(dev):
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs, mxfp4 as om
+
+    announce("mxfp4 dequant random")
+    a, asc, _, _ = inputs.mxfp4_inputs(96, 8, 1024, seed=2)
+    out = torch.ops.mi355.mxfp4_dequant(a.to(dev), asc.to(dev)).cpu().numpy()
+    assert np.array_equal(out.view(np.uint32), om.mxfp4_dequant_ref(a, asc).view(np.uint32))
+
+
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2])
+def test_mxfp4_gemm_variants(dev, variant):
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs, mxfp4 as om
+
+    M, N, K = 512, 768, 1024
+    announce(f"mxfp4_gemm M={M} N={N} K={K} variant={variant}")
+    a, asc, b, bsc = inputs.mxfp4_inputs(M, N, K, seed=7)
+    ref = om.mxfp4_gemm_ref(a, asc, b, bsc)
+    c32 = torch.ops.mi355.mxfp4_gemm(a.to(dev), asc.to(dev), b.to(dev), bsc.to(dev), "float32", variant).cpu()
+    assert _rel_err(c32, ref) < 1e-5
+    c16 = torch.ops.mi355.mxfp4_gemm(a.to(dev), asc.to(dev), b.to(dev), bsc.to(dev), "bfloat16", variant).cpu()
+    assert _rel_err(c16, ref) < REL
+    torch.testing.assert_close(c16.float(), ref, rtol=REL, atol=REL * ref.abs().max().item())
+    assert torch.equal(c16, c32.bfloat16())  # the bf16 epilogue is round-to-nearest-even of the fp32 result
+
+
+@pytest.mark.parametrize("shape", [(32, 256, 512), (1, 1, 32), (33, 65, 96), (32, 8192, 2048), (100, 40, 1056)])
+def test_mxfp4_gemm_ragged(dev, shape):
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs, mxfp4 as om
+
+    M, N, K = shape
+    announce(f"mxfp4_gemm ragged {shape}")
+    a, asc, b, bsc = inputs.mxfp4_inputs(M, N, K, seed=13)
+    ref = om.mxfp4_gemm_ref(a, asc, b, bsc)
+    c = torch.ops.mi355.mxfp4_gemm(a.to(dev), asc.to(dev), b.to(dev), bsc.to(dev), "float32", -1).cpu()
+    assert _rel_err(c, ref) < 1e-5
+
+
+def test_mxfp4_one_hot_nibble_order_and_scale_block(dev):
+    """A single non-zero code at element k of A picks out B[:, k]: pins the nibble order (even k = low
+    nibble) and which 32-element block a scale byte belongs to."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs, mxfp4 as om
+
+    announce("mxfp4 one-hot")
+    M, N, K = 32, 64, 256
+    _, _, b, bsc = inputs.mxfp4_inputs(M, N, K, seed=5)
+    db = om.mxfp4_dequant_ref(b, bsc)
+    for k in (0, 1, 31, 32, 63, 130, 255):
+        a = torch.zeros(M, K // 2, dtype=torch.uint8)
+        a[3, k // 2] = 0x2 << (4 * (k % 2))  # code 2 = 1.0
+        asc = torch.full((M, K // 32), 127, dtype=torch.uint8)
+        asc[3, k // 32] = 130  # x8 on that block only
+        c = torch.ops.mi355.mxfp4_gemm(a.to(dev), asc.to(dev), b.to(dev), bsc.to(dev), "float32", -1).cpu().numpy()
+        assert np.array_equal(c[3], 8.0 * db[:, k]), k
+        assert not c[np.arange(M) != 3].any()
+
+
+def test_mxfp4_exact_cases(dev):
+    """Unit scales and codes in {0, 1, 2, 4}: small-integer sums, exact.  Then +1 on every A scale byte
+    doubles the result exactly."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import mxfp4 as om
+
+    announce("mxfp4 exact cases")
+    M, N, K = 256, 256, 512
+    g = torch.Generator().manual_seed(3)
+    pick = torch.tensor([0, 2, 4, 6], dtype=torch.uint8)  # codes of 0, 1, 2, 4
+    ca = pick[torch.randint(0, 4, (M, K), generator=g)]
+    cb = pick[torch.randint(0, 4, (N, K), generator=g)]
+    a = torch.from_numpy(om.pack_codes(ca.numpy()))
+    b = torch.from_numpy(om.pack_codes(cb.numpy()))
+    one = torch.full((M, K // 32), 127, dtype=torch.uint8)
+    ref = om.mxfp4_gemm_ref(a, one, b, one)
+    c = torch.ops.mi355.mxfp4_gemm(a.to(dev), one.to(dev), b.to(dev), one.to(dev), "float32", -1).cpu()
+    assert torch.equal(c, ref)
+    c2 = torch.ops.mi355.mxfp4_gemm(a.to(dev), (one + 1).to(dev), b.to(dev), one.to(dev), "float32", -1).cpu()
+    assert torch.equal(c2, 2 * c)
+
+
+@pytest.mark.parametrize("shape", [(4096, 8192, 8192), (32, 8192, 8192)])
+def test_mxfp4_full_size(dev, shape):
+    """Benchmark shapes: sampled rows and columns against the oracle."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs, mxfp4 as om
+
+    M, N, K = shape
+    announce(f"mxfp4 full size {shape}")
+    a, asc, b, bsc = inputs.mxfp4_inputs(M, N, K)
+    c = torch.ops.mi355.mxfp4_gemm(a.to(dev), asc.to(dev), b.to(dev), bsc.to(dev), "bfloat16", -1)
+    rows = torch.tensor(sorted({0, 1, 31, M // 2, M - 1}))
+    cols = torch.tensor([0, 255, 256, N // 2 + 5, N - 1])
+    ref_r = om.mxfp4_gemm_ref(a[rows], asc[rows], b, bsc)
+    assert _rel_err(c[rows.to(dev)].float().cpu(), ref_r) < REL
+    ref_c = om.mxfp4_gemm_ref(a, asc, b[cols], bsc[cols])
+    assert _rel_err(c[:, cols.to(dev)].float().cpu(), ref_c) < REL
+
+
+def test_mxfp4_contract_errors(dev):
+    import iree_turbine_amd  # noqa: F401
+
+    a = torch.zeros(32, 16, dtype=torch.uint8, device=dev)
+    s = torch.full((32, 1), 127, dtype=torch.uint8, device=dev)
+    with pytest.raises(ValueError):
+        torch.ops.mi355.mxfp4_gemm(a, s, a[:, :8], s, "bfloat16", -1)
+    with pytest.raises(ValueError):
+        torch.ops.mi355.mxfp4_gemm(a, s[:, :0], a, s, "bfloat16", -1)
+    with pytest.raises(ValueError):
+        torch.ops.mi355.mxfp4_gemm(a, s, a, s, "float16", -1)

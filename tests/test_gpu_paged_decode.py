@@ -1,0 +1,127 @@
+"""GPU parity: paged GQA decode attention through the C ABI vs the CPU oracle (gather + dense fp32)."""
+
+import pytest
+import torch
+
+from conftest import announce
+
+pytestmark = pytest.mark.gpu
+
+ATOL = 2e-3
+RTOL = 1e-2
+
+
+def _to(dev, *ts):
+    return [t.to(dev) for t in ts]
+
+
+@pytest.mark.parametrize("splits", [1, 2, 4, 7, 0])
+def test_decode_small(dev, splits):
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs, paged_decode as op
+
+    announce(f"paged decode small splits={splits}")
+    q, kc, vc, bt, sl = inputs.paged_decode_inputs(num_seqs=6, min_len=1, max_len=700, seed=4)
+    out = torch.ops.mi355.paged_decode_attn(*_to(dev, q, kc, vc, bt, sl), 0.0, splits)
+    ref = op.paged_decode_ref(q, kc, vc, bt, sl)
+    torch.testing.assert_close(out.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("hq,hkv", [(8, 8), (8, 4), (32, 8), (16, 2), (16, 1)])
+def test_decode_gqa_ratios(dev, hq, hkv):
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs, paged_decode as op
+
+    announce(f"paged decode hq={hq} hkv={hkv}")
+    q, kc, vc, bt, sl = inputs.paged_decode_inputs(num_seqs=3, num_q_heads=hq, num_kv_heads=hkv, min_len=5, max_len=300, seed=9)
+    out = torch.ops.mi355.paged_decode_attn(*_to(dev, q, kc, vc, bt, sl), 0.0, 2)
+    ref = op.paged_decode_ref(q, kc, vc, bt, sl)
+    torch.testing.assert_close(out.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+
+
+def test_decode_edge_lengths_and_poison(dev):
+    """Lengths around page boundaries; tail tokens of the last page and unused pages hold NaN, padded
+    block-table entries hold an out-of-range id: none of them may influence (or be read into) the result."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import paged_decode as op
+
+    announce("paged decode edge lengths + poison")
+    lens = torch.tensor([1, 15, 16, 17, 31, 32, 33, 160, 161, 0], dtype=torch.int32)
+    S, Hq, Hkv, D, page = lens.numel(), 8, 2, 128, 16
+    n_pg = (lens + page - 1) // page
+    P = int(n_pg.sum()) + 3
+    g = torch.Generator().manual_seed(11)
+    perm = torch.randperm(P, generator=g)
+    bt = torch.full((S, int(n_pg.max()) + 2), 2**30, dtype=torch.int32)
+    kc = torch.full((P, page, Hkv, D), float("nan")).half()
+    vc = torch.full((P, page, Hkv, D), float("nan")).half()
+    off = 0
+    for s in range(S):
+        n = int(n_pg[s])
+        bt[s, :n] = perm[off:off + n].int()
+        for i in range(n):
+            valid = min(page, int(lens[s]) - i * page)
+            pg = int(perm[off + i])
+            kc[pg, :valid] = torch.randn(valid, Hkv, D, generator=g).half()
+            vc[pg, :valid] = torch.randn(valid, Hkv, D, generator=g).half()
+        off += n
+    q = torch.randn(S, Hq, D, generator=g).half()
+    kz, vz = torch.nan_to_num(kc, nan=0.0), torch.nan_to_num(vc, nan=0.0)
+    bt_ref = bt.clone()
+    bt_ref[bt_ref == 2**30] = 0
+    ref = op.paged_decode_ref(q, kz, vz, bt_ref, lens)
+    for splits in (1, 3):
+        out = torch.ops.mi355.paged_decode_attn(*_to(dev, q, kc, vc, bt, lens), 0.0, splits).float().cpu()
+        assert not torch.isnan(out).any()
+        torch.testing.assert_close(out, ref, rtol=RTOL, atol=ATOL)
+        assert torch.equal(out[-1], torch.zeros(Hq, D))  # an empty sequence yields zeros
+
+
+def test_decode_invariances(dev):
+    """Independent of the physical page placement and of the number of splits; phase0 + phase1 == fused."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs
+
+    announce("paged decode invariances")
+    q, kc, vc, bt, sl = inputs.paged_decode_inputs(num_seqs=5, min_len=100, max_len=1500, seed=21)
+    args = _to(dev, q, kc, vc, bt, sl)
+    base = torch.ops.mi355.paged_decode_attn(*args, 0.0, 4)
+    P = kc.shape[0]
+    perm = torch.randperm(P, generator=torch.Generator().manual_seed(1))
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(P)
+    kc2, vc2 = kc[perm], vc[perm]  # page that was at perm[i] is now at i
+    bt2 = torch.where(bt >= 0, inv[bt.clamp(min=0).long()].int(), bt)
+    moved = torch.ops.mi355.paged_decode_attn(*_to(dev, q, kc2, vc2, bt2, sl), 0.0, 4)
+    assert torch.equal(base, moved)
+    for splits in (1, 2, 8, 16):
+        o = torch.ops.mi355.paged_decode_attn(*args, 0.0, splits)
+        torch.testing.assert_close(o.float(), base.float(), rtol=1e-2, atol=1e-3)
+    pacc, pml = torch.ops.mi355.paged_decode_phase0(*args, 0.0, 4)
+    two = torch.ops.mi355.paged_decode_phase1(pacc, pml)
+    assert torch.equal(two, base)
+
+
+def test_decode_full_size(dev):
+    """The benchmark configuration (64 seqs, 32/8 heads, ctx in [512, 8192]) against the oracle."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs, paged_decode as op
+
+    announce("paged decode full size")
+    q, kc, vc, bt, sl = inputs.paged_decode_inputs()
+    out = torch.ops.mi355.paged_decode_attn(*_to(dev, q, kc, vc, bt, sl), 0.0, 0)
+    ref = op.paged_decode_ref(q, kc, vc, bt, sl)
+    torch.testing.assert_close(out.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+
+
+def test_decode_contract_errors(dev):
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs
+
+    q, kc, vc, bt, sl = _to(dev, *inputs.paged_decode_inputs(num_seqs=2, min_len=5, max_len=40))
+    with pytest.raises(ValueError):
+        torch.ops.mi355.paged_decode_attn(q, kc, vc, bt.long(), sl, 0.0, 1)
+    with pytest.raises(ValueError):
+        torch.ops.mi355.paged_decode_attn(q, kc[:, :8], vc[:, :8], bt, sl, 0.0, 1)  # page size 8
+    with pytest.raises(ValueError):
+        torch.ops.mi355.paged_decode_attn(q[:, :3], kc, vc, bt, sl, 0.0, 1)  # 3 q heads over 8 kv heads
