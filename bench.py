@@ -1,0 +1,286 @@
+#!/usr/bin/env python3
+"""Benchmark of the dense-kernel hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--no-others]
+
+A "step" is one launch of the hot-path kernel over one batch of seeded synthetic input that is
+already resident in HBM.  The headline workload is the fp16 NT GEMM 8192^3 with fp16 output
+(the configuration the TFLOP/s / %-of-MFMA-peak metric is quoted on); the other kernels of the
+path (flash-attention prefill, paged decode, MXFP4 GEMM, remaining GEMM shapes) are measured in
+the same run and reported under "others".  Prints exactly one JSON line.
+
+Timing: W untimed warm-up steps, then K steps bracketed by torch.cuda.synchronize() on both sides
+(wall clock -> value / ms_per_step) and, inside the same region, a HIP event pair on the launch
+stream around every step (-> the kernel's average duration used for the roofline figure).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import platform
+import sys
+import time
+
+import torch
+
+PEAK_F16_TFLOPS = 2500.0   # MI355X dense fp16 MFMA
+PEAK_FP4_TFLOPS = 10100.0  # MI355X dense fp4 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+METRIC = "TFLOP/s & %MFMA peak (f16 GEMM, causal FA, MXFP4 GEMM); decode HBM GB/s"
+
+# HBM bytes per launch measured with `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` (KiB per
+# dispatch, scaled by what the same counters read for a copy kernel of known size); filled in from
+# the summaries kept under profiles/.  None = not measured.
+MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {}
+
+
+def _events(n):
+    return [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+
+
+def time_steps(fn, steps: int, warmup: int):
+    """Returns (wall ms per step, mean device ms per launch, min device ms)."""
+    for _ in range(warmup):
+        fn()
+    ev = _events(steps)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for s, e in ev:
+        s.record()
+        fn()
+        e.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    dev = [s.elapsed_time(e) for s, e in ev]
+    return wall_ms, sum(dev) / len(dev), min(dev)
+
+
+# ---- workloads --------------------------------------------------------------------------------
+
+def wl_gemm(M, N, K, out_dtype="float16"):
+    from oracle import inputs
+
+    def build(dev):
+        a, b = inputs.gemm_inputs(M, N, K)
+        ad, bd = a.to(dev), b.to(dev)
+        flops = 2.0 * M * N * K
+        out_b = 2 if out_dtype == "float16" else 4
+        nbytes = 2.0 * (M * K + N * K) + out_b * M * N
+        return {
+            "fn": lambda: torch.ops.mi355.gemm_nt(ad, bd, out_dtype, -1),
+            "work": flops, "bytes": nbytes, "bound": "mfma", "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
+            "dtype": "f16", "cpu": lambda: cpu_gemm(a, b, M, N, K),
+            "config": {"workload": f"gemm_f16_nt_{M}x{N}x{K}_{'f16' if out_dtype == 'float16' else 'f32'}out",
+                       "M": M, "N": N, "K": K, "layout": "NT", "accumulate": "f32", "out": out_dtype, "seed": 10},
+        }
+    return build
+
+
+def wl_attention(causal, B=2, H=32, S=4096, D=128):
+    from oracle import inputs
+
+    def build(dev):
+        q, k, v = inputs.attention_inputs(B, H, S, D)
+        qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+        flops = 4.0 * B * H * S * S * D * (0.5 if causal else 1.0)
+        return {
+            "fn": lambda: torch.ops.mi355.flash_attn_fwd(qd, kd, vd, causal, 0.0),
+            "work": flops, "bytes": 4 * 2.0 * B * H * S * D, "bound": "mfma", "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
+            "dtype": "f16", "cpu": lambda: cpu_attention(q, k, v, causal),
+            "config": {"workload": f"flash_attn_fwd_{'causal' if causal else 'noncausal'}_B{B}_H{H}_S{S}_D{D}",
+                       "B": B, "H": H, "S": S, "D": D, "causal": causal, "seed": 10},
+        }
+    return build
+
+
+def wl_decode():
+    from oracle import inputs
+
+    def build(dev):
+        q, kc, vc, bt, sl = inputs.paged_decode_inputs()
+        args = [t.to(dev) for t in (q, kc, vc, bt, sl)]
+        total = int(sl.sum())
+        kv_bytes = 4096.0 * total  # 2 (K,V) * 8 kv heads * 128 * 2 B per cached token, read once
+        return {
+            "fn": lambda: torch.ops.mi355.paged_decode_attn(*args, 0.0, 0),
+            "work": kv_bytes, "bytes": kv_bytes, "bound": "hbm", "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "dtype": "f16", "cpu": lambda: cpu_decode(q, kc, vc, bt, sl),
+            "config": {"workload": "paged_decode_64seq_32q8kv_D128_page16_ctx512-8192", "num_seqs": 64, "q_heads": 32,
+                       "kv_heads": 8, "D": 128, "page": 16, "total_tokens": total, "seed": 10},
+        }
+    return build
+
+
+def wl_mxfp4(M, N, K):
+    from oracle import inputs
+
+    def build(dev):
+        a, asc, b, bsc = inputs.mxfp4_inputs(M, N, K)
+        args = [t.to(dev) for t in (a, asc, b, bsc)]
+        flops = 2.0 * M * N * K
+        nbytes = (M + N) * K / 2 + (M + N) * K / 32 + 2.0 * M * N
+        hbm_bound = flops / nbytes < 1250
+        return {
+            "fn": lambda: torch.ops.mi355.mxfp4_gemm(*args, "bfloat16", -1),
+            "work": nbytes if hbm_bound else flops, "bytes": nbytes, "flops": flops,
+            "bound": "hbm" if hbm_bound else "mfma", "peak": PEAK_HBM_GBS if hbm_bound else PEAK_FP4_TFLOPS,
+            "unit": "GB/s" if hbm_bound else "TFLOP/s", "dtype": "fp4(e2m1)+e8m0",
+            "cpu": lambda: cpu_mxfp4(a, asc, b, bsc, M, N, K),
+            "config": {"workload": f"mxfp4_gemm_{M}x{N}x{K}_bf16out", "M": M, "N": N, "K": K, "seed": 10},
+        }
+    return build
+
+
+WORKLOADS = {
+    "gemm_8192": wl_gemm(8192, 8192, 8192),
+    "gemm_4096": wl_gemm(4096, 4096, 4096),
+    "gemm_2048x10240x8192": wl_gemm(2048, 10240, 8192),
+    "gemm_2048x57344x8192": wl_gemm(2048, 57344, 8192),
+    "gemm_1024_f32out": wl_gemm(1024, 1024, 1024, "float32"),
+    "fa_causal": wl_attention(True),
+    "fa_noncausal": wl_attention(False),
+    "decode": wl_decode(),
+    "mxfp4_4096x8192x8192": wl_mxfp4(4096, 8192, 8192),
+    "mxfp4_32x8192x8192": wl_mxfp4(32, 8192, 8192),
+}
+HEADLINE = "gemm_8192"
+
+
+# ---- CPU baselines: the oracle, timed on the host cores on a bounded sample ------------------
+
+def _time_cpu(fn, reps=3):
+    fn()
+    ts = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    return min(ts)
+
+
+def cpu_gemm(a, b, M, N, K):
+    from oracle import gemm as og
+    rows = min(M, 1024)
+    t = _time_cpu(lambda: og.gemm_nt_ref(a[:rows], b))
+    return {"value": 2.0 * rows * N * K / t / 1e12, "unit": "TFLOP/s",
+            "sample": f"torch fp32 matmul of A[0:{rows}] . B^T ({rows}x{N}x{K}), best of 3 after 1 warm-up"}
+
+
+def cpu_attention(q, k, v, causal):
+    from oracle import attention as oa
+    qs, ks, vs = q[:1, :2], k[:1, :2], v[:1, :2]
+    S, D = q.shape[2], q.shape[3]
+    t = _time_cpu(lambda: oa.sdpa_torch(qs, ks, vs, is_causal=causal))
+    flops = 4.0 * 2 * S * S * D * (0.5 if causal else 1.0)
+    return {"value": flops / t / 1e12, "unit": "TFLOP/s",
+            "sample": f"torch fp32 scaled_dot_product_attention on 2 of the {q.shape[0] * q.shape[1]} heads, best of 3 after 1 warm-up"}
+
+
+def cpu_decode(q, kc, vc, bt, sl):
+    from oracle import paged_decode as op
+    n = 4
+    t = _time_cpu(lambda: op.paged_decode_ref(q[:n], kc, vc, bt[:n], sl[:n]), reps=2)
+    return {"value": 4096.0 * int(sl[:n].sum()) / t / 1e9, "unit": "GB/s",
+            "sample": f"gather + dense fp32 attention for {n} of the {q.shape[0]} sequences, best of 2 after 1 warm-up"}
+
+
+def cpu_mxfp4(a, asc, b, bsc, M, N, K):
+    from oracle import mxfp4 as om
+    rows, cols = min(M, 256), min(N, 2048)
+    t = _time_cpu(lambda: om.mxfp4_gemm_ref(a[:rows], asc[:rows], b[:cols], bsc[:cols]))
+    flops = 2.0 * rows * cols * K
+    return {"value": flops / t / 1e12, "unit": "TFLOP/s",
+            "sample": f"table dequantise + torch fp32 matmul of a {rows}x{cols}x{K} corner, best of 3 after 1 warm-up"}
+
+
+# ---- driver -------------------------------------------------------------------------------------
+
+def measure(name: str, dev, steps: int, warmup: int, with_cpu: bool):
+    wl = WORKLOADS[name](dev)
+    wall_ms, dev_ms, dev_min_ms = time_steps(wl["fn"], steps, warmup)
+    scale = 1e9 if wl["unit"] == "GB/s" else 1e12
+    achieved = wl["work"] / (dev_ms * 1e-3) / scale
+    rec = {
+        "workload": wl["config"]["workload"],
+        "value": wl["work"] / (wall_ms * 1e-3) / scale,
+        "unit": wl["unit"],
+        "ms_per_step": wall_ms,
+        "kernel_ms_avg": dev_ms,
+        "kernel_ms_min": dev_min_ms,
+        "dtype": wl["dtype"],
+        "config": wl["config"],
+        "roofline": {"bound": wl["bound"], "achieved": achieved, "peak": wl["peak"], "unit": wl["unit"],
+                     "frac": achieved / wl["peak"], "traffic": MEASURED_TRAFFIC_BYTES.get(name)},
+    }
+    if "flops" in wl and wl["bound"] == "hbm":
+        rec["tflops"] = wl["flops"] / (dev_ms * 1e-3) / 1e12
+    if with_cpu:
+        cpu = wl["cpu"]()
+        cpu.update({"cores": torch.get_num_threads(), "kind": "port"})
+        rec["cpu_baseline"] = cpu
+    return rec
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-others", action="store_true", help="measure only --workload")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); --gpus must be 1", file=sys.stderr)
+        return 2
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the kernels have no CPU fallback", file=sys.stderr)
+        return 3
+
+    import iree_turbine_amd  # noqa: F401  (registers torch.ops.mi355.*; raises if the library is missing)
+
+    dev = torch.device("cuda:0")
+    head = measure(args.workload, dev, args.steps, args.warmup, with_cpu=not args.no_cpu)
+    others = []
+    if not args.no_others:
+        for name in WORKLOADS:
+            if name == args.workload:
+                continue
+            torch.cuda.empty_cache()
+            steps = max(5, min(args.steps, 20))
+            rec = measure(name, dev, steps, min(args.warmup, 3), with_cpu=False)
+            rec.pop("config")
+            others.append(rec)
+
+    line = {
+        "metric": METRIC,
+        "value": head["value"],
+        "unit": head["unit"],
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": head["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": head["dtype"],
+        "data": "synthetic (seeded torch CPU generator, seed 10; random-normal * 0.1 fp16 operands)",
+        "config": head["config"],
+        "kernel_ms_avg": head["kernel_ms_avg"],
+        "kernel_ms_min": head["kernel_ms_min"],
+        "roofline": head["roofline"],
+        "cpu_baseline": head.get("cpu_baseline"),
+        "host": {"cpu": platform.processor() or platform.machine(), "os_cpu_count": os.cpu_count(),
+                 "torch_threads": torch.get_num_threads(), "gpu": torch.cuda.get_device_name(0)},
+        "others": others,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

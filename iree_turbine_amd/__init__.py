@@ -5,7 +5,8 @@ Importing the package registers `torch.ops.mi355.*`.  The kernels live in
 csrc/libturbine_mi355.so (hand-written HIP for gfx950); there is no other implementation.
 """
 
-from . import _lib, op_reg, ops  # noqa: F401
+from . import _lib, lang, launch, launchable, op_reg, ops, templates  # noqa: F401
+from .launchable import Launchable, WaveCompileOptions, wave_compile  # noqa: F401
 from .ops import *  # noqa: F401,F403
 
 __version__ = "0.1.0"

@@ -1,0 +1,149 @@
+"""Out-variant launchers: checked tensors in, C-ABI call on torch's current stream, output tensors
+written in place.  Both the custom ops (ops.py) and the template kernels (templates/) go through
+these functions; they are the only callers of the C ABI."""
+
+from __future__ import annotations
+
+import math
+
+import torch
+from torch import Tensor
+
+from . import _lib
+
+
+def _dev(*tensors: Tensor) -> torch.device:
+    dev = tensors[0].device
+    for t in tensors[1:]:
+        if t.device != dev:
+            # same rule and wording as Launchable.__call__, iree/turbine/runtime/launch.py:220-225
+            raise RuntimeError(f"Cannot launch with tensors from multiple devices: {t.device} vs {dev}")
+    if dev.type != "cuda":
+        raise RuntimeError(f"the kernels run on an MI355X only; got tensors on {dev} (there is no CPU fallback)")
+    return dev
+
+
+def _contig_out(t: Tensor, name: str) -> None:
+    if not t.is_contiguous():
+        raise ValueError(f"{name}: output tensors must be contiguous")  # runtime/launch.py:246
+
+
+def gemm_nt_out(a: Tensor, b: Tensor, c: Tensor, variant: int = -1) -> Tensor:
+    dev = _dev(a, b, c)
+    a, b = a.contiguous(), b.contiguous()
+    _contig_out(c, "gemm_nt")
+    M, K = a.shape
+    N = b.shape[0]
+    if tuple(c.shape) != (M, N):
+        raise ValueError(f"gemm_nt: c is {tuple(c.shape)}, expected {(M, N)}")
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_gemm_f16_nt(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, _lib.dtype_code(c.dtype),
+                                           variant, _lib.current_stream_ptr(dev))
+    _lib.check(rc, f"gemm_nt M={M} N={N} K={K} out={c.dtype} variant={variant}")
+    return c
+
+
+def flash_attn_fwd_out(q: Tensor, k: Tensor, v: Tensor, o: Tensor, is_causal: bool, scale: float) -> Tensor:
+    dev = _dev(q, k, v, o)
+    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+    _contig_out(o, "flash_attn_fwd")
+    B, H, Sq, D = q.shape
+    Sk = k.shape[2]
+    if o.shape != q.shape or o.dtype != torch.float16:
+        raise ValueError("flash_attn_fwd: o must be float16 with q's shape")
+    if scale is None or scale <= 0:
+        scale = 1.0 / math.sqrt(D)
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_flash_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), B, H, Sq, Sk, D, scale,
+                                              int(bool(is_causal)), -1, _lib.current_stream_ptr(dev))
+    _lib.check(rc, f"flash_attn_fwd B={B} H={H} Sq={Sq} Sk={Sk} D={D} causal={is_causal}")
+    return o
+
+
+def paged_decode_phase0_out(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, scale: float) -> None:
+    dev = _dev(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml)
+    q, k_cache, v_cache = q.contiguous(), k_cache.contiguous(), v_cache.contiguous()
+    block_table, seq_lens = block_table.contiguous(), seq_lens.contiguous()
+    _contig_out(part_acc, "paged_decode_phase0")
+    _contig_out(part_ml, "paged_decode_phase0")
+    S, Hq, D = q.shape
+    P, page, Hkv, _ = k_cache.shape
+    ns = part_acc.shape[2]
+    if tuple(part_acc.shape) != (S, Hq, ns, D) or tuple(part_ml.shape) != (S, Hq, ns, 2) or part_acc.dtype != torch.float32 or part_ml.dtype != torch.float32:
+        raise ValueError("paged_decode_phase0: part_acc must be fp32 [S, Hq, splits, D], part_ml fp32 [S, Hq, splits, 2]")
+    if scale is None or scale <= 0:
+        scale = 1.0 / math.sqrt(D)
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_paged_decode_phase0(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
+                                                   seq_lens.data_ptr(), part_acc.data_ptr(), part_ml.data_ptr(), S, Hq, Hkv, D,
+                                                   page, block_table.shape[1], P, ns, scale, _lib.current_stream_ptr(dev))
+    _lib.check(rc, f"paged_decode_phase0 seqs={S} hq={Hq} hkv={Hkv} splits={ns}")
+
+
+def paged_decode_phase1_out(part_acc: Tensor, part_ml: Tensor, out: Tensor) -> Tensor:
+    dev = _dev(part_acc, part_ml, out)
+    part_acc, part_ml = part_acc.contiguous(), part_ml.contiguous()
+    _contig_out(out, "paged_decode_phase1")
+    S, Hq, ns, D = part_acc.shape
+    if tuple(out.shape) != (S, Hq, D) or out.dtype != torch.float16:
+        raise ValueError("paged_decode_phase1: out must be float16 [S, Hq, D]")
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_paged_decode_phase1(part_acc.data_ptr(), part_ml.data_ptr(), out.data_ptr(), S, Hq, D, ns,
+                                                   _lib.current_stream_ptr(dev))
+    _lib.check(rc, f"paged_decode_phase1 seqs={S} hq={Hq} splits={ns}")
+    return out
+
+
+def paged_decode_attn_out(q, k_cache, v_cache, block_table, seq_lens, out, scale: float, num_kv_splits: int,
+                          part_acc: Tensor | None = None, part_ml: Tensor | None = None) -> Tensor:
+    dev = _dev(q, k_cache, v_cache, block_table, seq_lens, out)
+    q, k_cache, v_cache = q.contiguous(), k_cache.contiguous(), v_cache.contiguous()
+    block_table, seq_lens = block_table.contiguous(), seq_lens.contiguous()
+    _contig_out(out, "paged_decode_attn")
+    S, Hq, D = q.shape
+    P, page, Hkv, _ = k_cache.shape
+    if out.shape != q.shape or out.dtype != torch.float16:
+        raise ValueError("paged_decode_attn: out must be float16 with q's shape")
+    if scale is None or scale <= 0:
+        scale = 1.0 / math.sqrt(D)
+    if num_kv_splits > 1:
+        if part_acc is None:
+            part_acc = torch.empty((S, Hq, num_kv_splits, D), dtype=torch.float32, device=dev)
+        if part_ml is None:
+            part_ml = torch.empty((S, Hq, num_kv_splits, 2), dtype=torch.float32, device=dev)
+    pa = part_acc.data_ptr() if part_acc is not None else None
+    pm = part_ml.data_ptr() if part_ml is not None else None
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_paged_decode_attn(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
+                                                 seq_lens.data_ptr(), out.data_ptr(), pa, pm, S, Hq, Hkv, D, page,
+                                                 block_table.shape[1], P, num_kv_splits, scale, _lib.current_stream_ptr(dev))
+    _lib.check(rc, f"paged_decode_attn seqs={S} hq={Hq} hkv={Hkv} pages={P} splits={num_kv_splits}")
+    return out
+
+
+def mxfp4_gemm_out(a, a_scale, b, b_scale, c: Tensor, variant: int = -1) -> Tensor:
+    dev = _dev(a, a_scale, b, b_scale, c)
+    a, a_scale, b, b_scale = a.contiguous(), a_scale.contiguous(), b.contiguous(), b_scale.contiguous()
+    _contig_out(c, "mxfp4_gemm")
+    M, N, K = a.shape[0], b.shape[0], a.shape[1] * 2
+    if tuple(c.shape) != (M, N):
+        raise ValueError(f"mxfp4_gemm: c is {tuple(c.shape)}, expected {(M, N)}")
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_mxfp4_gemm(a.data_ptr(), a_scale.data_ptr(), b.data_ptr(), b_scale.data_ptr(), c.data_ptr(), M, N,
+                                          K, _lib.dtype_code(c.dtype), variant, _lib.current_stream_ptr(dev))
+    _lib.check(rc, f"mxfp4_gemm M={M} N={N} K={K} out={c.dtype} variant={variant}")
+    return c
+
+
+def mxfp4_dequant_out(codes: Tensor, scales: Tensor, out: Tensor) -> Tensor:
+    dev = _dev(codes, scales, out)
+    codes, scales = codes.contiguous(), scales.contiguous()
+    _contig_out(out, "mxfp4_dequant")
+    rows, K = codes.shape[0], codes.shape[1] * 2
+    if tuple(out.shape) != (rows, K) or out.dtype != torch.float32:
+        raise ValueError("mxfp4_dequant: out must be float32 [rows, K]")
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_mxfp4_dequant(codes.data_ptr(), scales.data_ptr(), out.data_ptr(), rows, K,
+                                             _lib.current_stream_ptr(dev))
+    _lib.check(rc, f"mxfp4_dequant rows={rows} K={K}")
+    return out

@@ -13,7 +13,7 @@ import math
 import torch
 from torch import Tensor
 
-from . import _lib
+from . import launch
 from .op_reg import CustomOp, KernelSelection
 
 __all__ = [
@@ -32,18 +32,6 @@ _OUT_DTYPES = {"float32": torch.float32, "float16": torch.float16, "bfloat16": t
 def _require(cond: bool, msg: str) -> None:
     if not cond:
         raise ValueError(msg)
-
-
-def _ptr(t: Tensor | None) -> int | None:
-    return None if t is None else t.data_ptr()
-
-
-def _same_device(*tensors: Tensor) -> torch.device:
-    dev = tensors[0].device
-    for t in tensors[1:]:
-        if t.device != dev:
-            raise RuntimeError(f"Cannot launch with tensors from multiple devices: {t.device} vs {dev}")
-    return dev
 
 
 @CustomOp.register
@@ -70,16 +58,8 @@ class gemm_nt(CustomOp):
         sel.return_new_tensor([a.t.size(0), b.t.size(0)], _OUT_DTYPES[od]).specialize_all_dims()
 
     def eager_execute(self, a, b, out_dtype, variant):
-        dev = _same_device(a, b)
-        a, b = a.contiguous(), b.contiguous()
-        M, K = a.shape
-        N = b.shape[0]
-        c = torch.empty((M, N), dtype=_OUT_DTYPES[out_dtype], device=dev)
-        with torch.cuda.device(dev):
-            rc = _lib.load().mi355_gemm_f16_nt(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K,
-                                               _lib.dtype_code(c.dtype), variant, _lib.current_stream_ptr(dev))
-        _lib.check(rc, f"gemm_nt M={M} N={N} K={K} out={out_dtype} variant={variant}")
-        return c
+        c = torch.empty((a.shape[0], b.shape[0]), dtype=_OUT_DTYPES[out_dtype], device=a.device)
+        return launch.gemm_nt_out(a, b, c, variant)
 
 
 @CustomOp.register
@@ -108,18 +88,8 @@ class flash_attn_fwd(CustomOp):
         sel.return_new_tensor(list(q.t.shape), torch.float16)
 
     def eager_execute(self, q, k, v, is_causal, scale):
-        dev = _same_device(q, k, v)
-        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-        B, H, Sq, D = q.shape
-        Sk = k.shape[2]
-        if scale <= 0:
-            scale = 1.0 / math.sqrt(D)
-        o = torch.empty_like(q)
-        with torch.cuda.device(dev):
-            rc = _lib.load().mi355_flash_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), B, H, Sq, Sk, D,
-                                                  scale, int(is_causal), -1, _lib.current_stream_ptr(dev))
-        _lib.check(rc, f"flash_attn_fwd B={B} H={H} Sq={Sq} Sk={Sk} D={D} causal={is_causal}")
-        return o
+        o = torch.empty(q.shape, dtype=torch.float16, device=q.device)
+        return launch.flash_attn_fwd_out(q, k, v, o, is_causal, scale)
 
 
 def _check_paged_args(op: str, q: Tensor, k_cache: Tensor, v_cache: Tensor, block_table: Tensor, seq_lens: Tensor):
@@ -165,28 +135,10 @@ class paged_decode_attn(CustomOp):
         sel.return_new_tensor(list(q.t.shape), torch.float16)
 
     def eager_execute(self, q, k_cache, v_cache, block_table, seq_lens, scale, num_kv_splits):
-        dev = _same_device(q, k_cache, v_cache, block_table, seq_lens)
-        q, k_cache, v_cache = q.contiguous(), k_cache.contiguous(), v_cache.contiguous()
-        block_table, seq_lens = block_table.contiguous(), seq_lens.contiguous()
-        S, Hq, D = q.shape
-        P, page, Hkv, _ = k_cache.shape
-        max_pages = block_table.shape[1]
-        if scale <= 0:
-            scale = 1.0 / math.sqrt(D)
         if num_kv_splits <= 0:
-            num_kv_splits = default_num_kv_splits(max_pages * page, S, Hkv)
-        out = torch.empty_like(q)
-        pacc = pml = None
-        if num_kv_splits > 1:
-            pacc = torch.empty((S, Hq, num_kv_splits, D), dtype=torch.float32, device=dev)
-            pml = torch.empty((S, Hq, num_kv_splits, 2), dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev):
-            rc = _lib.load().mi355_paged_decode_attn(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
-                                                     block_table.data_ptr(), seq_lens.data_ptr(), out.data_ptr(),
-                                                     _ptr(pacc), _ptr(pml), S, Hq, Hkv, D, page, max_pages, P,
-                                                     num_kv_splits, scale, _lib.current_stream_ptr(dev))
-        _lib.check(rc, f"paged_decode_attn seqs={S} hq={Hq} hkv={Hkv} pages={P} splits={num_kv_splits}")
-        return out
+            num_kv_splits = default_num_kv_splits(block_table.shape[1] * k_cache.shape[1], q.shape[0], k_cache.shape[2])
+        out = torch.empty(q.shape, dtype=torch.float16, device=q.device)
+        return launch.paged_decode_attn_out(q, k_cache, v_cache, block_table, seq_lens, out, scale, num_kv_splits)
 
 
 @CustomOp.register
@@ -207,21 +159,10 @@ class paged_decode_phase0(CustomOp):
         sel.return_new_tensor([S, Hq, ns, 2], torch.float32)
 
     def eager_execute(self, q, k_cache, v_cache, block_table, seq_lens, scale, num_kv_splits):
-        dev = _same_device(q, k_cache, v_cache, block_table, seq_lens)
-        q, k_cache, v_cache = q.contiguous(), k_cache.contiguous(), v_cache.contiguous()
-        block_table, seq_lens = block_table.contiguous(), seq_lens.contiguous()
         S, Hq, D = q.shape
-        P, page, Hkv, _ = k_cache.shape
-        if scale <= 0:
-            scale = 1.0 / math.sqrt(D)
-        pacc = torch.empty((S, Hq, num_kv_splits, D), dtype=torch.float32, device=dev)
-        pml = torch.empty((S, Hq, num_kv_splits, 2), dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev):
-            rc = _lib.load().mi355_paged_decode_phase0(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
-                                                       block_table.data_ptr(), seq_lens.data_ptr(), pacc.data_ptr(),
-                                                       pml.data_ptr(), S, Hq, Hkv, D, page, block_table.shape[1], P,
-                                                       num_kv_splits, scale, _lib.current_stream_ptr(dev))
-        _lib.check(rc, f"paged_decode_phase0 seqs={S} hq={Hq} hkv={Hkv} splits={num_kv_splits}")
+        pacc = torch.empty((S, Hq, num_kv_splits, D), dtype=torch.float32, device=q.device)
+        pml = torch.empty((S, Hq, num_kv_splits, 2), dtype=torch.float32, device=q.device)
+        launch.paged_decode_phase0_out(q, k_cache, v_cache, block_table, seq_lens, pacc, pml, scale)
         return pacc, pml
 
 
@@ -238,15 +179,9 @@ class paged_decode_phase1(CustomOp):
         sel.return_new_tensor([pa.t.size(0), pa.t.size(1), 128], torch.float16)
 
     def eager_execute(self, part_acc, part_ml):
-        dev = _same_device(part_acc, part_ml)
-        part_acc, part_ml = part_acc.contiguous(), part_ml.contiguous()
-        S, Hq, ns, D = part_acc.shape
-        out = torch.empty((S, Hq, D), dtype=torch.float16, device=dev)
-        with torch.cuda.device(dev):
-            rc = _lib.load().mi355_paged_decode_phase1(part_acc.data_ptr(), part_ml.data_ptr(), out.data_ptr(), S, Hq, D, ns,
-                                                       _lib.current_stream_ptr(dev))
-        _lib.check(rc, f"paged_decode_phase1 seqs={S} hq={Hq} splits={ns}")
-        return out
+        S, Hq, _, D = part_acc.shape
+        out = torch.empty((S, Hq, D), dtype=torch.float16, device=part_acc.device)
+        return launch.paged_decode_phase1_out(part_acc, part_ml, out)
 
 
 def _check_mx_operand(op: str, name: str, codes: Tensor, scales: Tensor):
@@ -278,15 +213,8 @@ class mxfp4_gemm(CustomOp):
         sel.return_new_tensor([a.t.size(0), b.t.size(0)], _OUT_DTYPES[od]).specialize_all_dims()
 
     def eager_execute(self, a, a_scale, b, b_scale, out_dtype, variant):
-        dev = _same_device(a, a_scale, b, b_scale)
-        a, a_scale, b, b_scale = a.contiguous(), a_scale.contiguous(), b.contiguous(), b_scale.contiguous()
-        M, N, K = a.shape[0], b.shape[0], a.shape[1] * 2
-        c = torch.empty((M, N), dtype=_OUT_DTYPES[out_dtype], device=dev)
-        with torch.cuda.device(dev):
-            rc = _lib.load().mi355_mxfp4_gemm(a.data_ptr(), a_scale.data_ptr(), b.data_ptr(), b_scale.data_ptr(), c.data_ptr(),
-                                              M, N, K, _lib.dtype_code(c.dtype), variant, _lib.current_stream_ptr(dev))
-        _lib.check(rc, f"mxfp4_gemm M={M} N={N} K={K} out={out_dtype} variant={variant}")
-        return c
+        c = torch.empty((a.shape[0], b.shape[0]), dtype=_OUT_DTYPES[out_dtype], device=a.device)
+        return launch.mxfp4_gemm_out(a, a_scale, b, b_scale, c, variant)
 
 
 @CustomOp.register
@@ -302,12 +230,5 @@ class mxfp4_dequant(CustomOp):
         sel.return_new_tensor([c.t.size(0), c.t.size(1) * 2], torch.float32)
 
     def eager_execute(self, codes, scales):
-        dev = _same_device(codes, scales)
-        codes, scales = codes.contiguous(), scales.contiguous()
-        rows, K = codes.shape[0], codes.shape[1] * 2
-        out = torch.empty((rows, K), dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev):
-            rc = _lib.load().mi355_mxfp4_dequant(codes.data_ptr(), scales.data_ptr(), out.data_ptr(), rows, K,
-                                                 _lib.current_stream_ptr(dev))
-        _lib.check(rc, f"mxfp4_dequant rows={rows} K={K}")
-        return out
+        out = torch.empty((codes.shape[0], codes.shape[1] * 2), dtype=torch.float32, device=codes.device)
+        return launch.mxfp4_dequant_out(codes, scales, out)

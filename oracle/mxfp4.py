@@ -20,7 +20,7 @@ def e2m1_closed_form(code: int) -> float:
 def e8m0_decode(b: np.ndarray) -> np.ndarray:
     """2^(b - 127) as fp32; 0xFF is NaN."""
     b = np.asarray(b, dtype=np.uint8)
-    out = np.ldexp(np.float32(1.0), b.astype(np.int32) - 127).astype(np.float32)
+    out = np.ldexp(np.float32(1.0), np.minimum(b, 254).astype(np.int32) - 127).astype(np.float32)
     out[b == 255] = np.nan
     return out
 
@@ -45,7 +45,8 @@ def mxfp4_dequant_ref(packed, scales) -> np.ndarray:
     scales = scales.detach().cpu().numpy() if isinstance(scales, torch.Tensor) else np.asarray(scales)
     vals = np.asarray(E2M1_VALUES, dtype=np.float32)[unpack_codes(packed)]
     sc = np.repeat(e8m0_decode(scales), BLOCK, axis=1)
-    return (vals * sc).astype(np.float32)
+    with np.errstate(over="ignore", invalid="ignore"):
+        return (vals * sc).astype(np.float32)
 
 
 def mxfp4_gemm_ref(a, a_scale, b, b_scale) -> torch.Tensor:

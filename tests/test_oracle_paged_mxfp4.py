@@ -1,0 +1,139 @@
+"""Pins the paged-decode and MXFP4 oracles (closed forms, library decode of the scale format, brute
+force, the C restatement, invariants)."""
+
+import ctypes
+import math
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import attention as oa, inputs, mxfp4 as om, paged_decode as op
+
+
+def test_paged_decode_equals_dense_attention_on_contiguous_cache():
+    S, Hq, Hkv, D, page = 3, 8, 2, 16, 16
+    g = torch.Generator().manual_seed(1)
+    lens = torch.tensor([16, 40, 7], dtype=torch.int32)
+    n_pg = (lens + page - 1) // page
+    P = int(n_pg.sum())
+    kc = torch.randn(P, page, Hkv, D, generator=g).half()
+    vc = torch.randn(P, page, Hkv, D, generator=g).half()
+    q = torch.randn(S, Hq, D, generator=g).half()
+    bt = torch.full((S, int(n_pg.max())), -1, dtype=torch.int32)
+    off = 0
+    for s in range(S):
+        bt[s, :n_pg[s]] = torch.arange(off, off + int(n_pg[s]), dtype=torch.int32)
+        off += int(n_pg[s])
+    out = op.paged_decode_ref(q, kc, vc, bt, lens)
+    off = 0
+    for s in range(S):
+        ln = int(lens[s])
+        ks = kc[off:off + int(n_pg[s])].reshape(-1, Hkv, D)[:ln]
+        vs = vc[off:off + int(n_pg[s])].reshape(-1, Hkv, D)[:ln]
+        off += int(n_pg[s])
+        for h in range(Hq):
+            kv = h // (Hq // Hkv)  # the GQA rule: q head h reads kv head h // n_rep
+            ref = oa.sdpa_ref(q[s, h][None], ks[:, kv], vs[:, kv])[0]
+            torch.testing.assert_close(out[s, h], ref, rtol=1e-5, atol=1e-6)
+
+
+def test_paged_decode_invariances_and_poison():
+    q, kc, vc, bt, sl = inputs.paged_decode_inputs(num_seqs=4, num_q_heads=4, num_kv_heads=2, D=16, min_len=1, max_len=90, seed=3)
+    base = op.paged_decode_ref(q, kc, vc, bt, sl)
+    P = kc.shape[0]
+    perm = torch.randperm(P, generator=torch.Generator().manual_seed(2))
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(P)
+    bt2 = torch.where(bt >= 0, inv[bt.clamp(min=0).long()].int(), bt)
+    assert torch.equal(op.paged_decode_ref(q, kc[perm], vc[perm], bt2, sl), base)  # physical placement is irrelevant
+    # tokens past the length never matter
+    kp, vp = kc.clone(), vc.clone()
+    for s in range(4):
+        ln = int(sl[s])
+        last = int(bt[s, (ln - 1) // 16])
+        if ln % 16:
+            kp[last, ln % 16:] = float("nan")
+            vp[last, ln % 16:] = float("nan")
+    assert torch.equal(op.paged_decode_ref(q, kp, vp, bt, sl), base)
+    assert inputs.paged_decode_inputs(num_seqs=2, min_len=5, max_len=5, D=16)[3].shape[1] == 1
+    # repeat_kv ordering
+    x = torch.arange(2 * 3 * 1).float().view(2, 3, 1)
+    assert op.repeat_kv(x, 2)[:, :, 0].tolist() == [[0, 0, 1, 1, 2, 2], [3, 3, 4, 4, 5, 5]]
+
+
+def test_e2m1_table_closed_form_and_spec_values():
+    assert [om.e2m1_closed_form(c) for c in range(16)] == list(om.E2M1_VALUES)
+    # OCP MX v1.0 table 5: magnitudes 0, 0.5, 1, 1.5, 2, 3, 4, 6; code 0x8 is negative zero
+    assert om.E2M1_VALUES[:8] == (0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0)
+    assert math.copysign(1.0, om.E2M1_VALUES[8]) == -1.0 and om.E2M1_VALUES[8] == 0.0
+    assert all(om.E2M1_VALUES[c + 8] == -om.E2M1_VALUES[c] for c in range(8))
+
+
+def test_e8m0_decode_vs_torch_library():
+    b = np.arange(256, dtype=np.uint8)
+    ours = om.e8m0_decode(b)
+    lib = torch.from_numpy(b.copy()).view(torch.float8_e8m0fnu).to(torch.float32).numpy()
+    assert np.array_equal(ours[:255].view(np.uint32), lib[:255].view(np.uint32))
+    assert np.isnan(ours[255]) and np.isnan(lib[255])
+    assert ours[127] == 1.0 and ours[119] == 2.0**-8 and ours[135] == 256.0 and ours[0] == 2.0**-127
+
+
+def test_dequant_exhaustive_products_exact_in_bf16():
+    packed = om.pack_codes(np.tile(np.arange(16, dtype=np.uint8), 2)[None, :].repeat(17, 0))
+    scales = (119 + np.arange(17, dtype=np.uint8))[:, None]
+    dq = om.mxfp4_dequant_ref(packed, scales)
+    for r in range(17):
+        for k in range(32):
+            assert dq[r, k] == om.E2M1_VALUES[k % 16] * 2.0 ** (int(scales[r, 0]) - 127)
+    t = torch.from_numpy(dq)
+    assert torch.equal(t.bfloat16().float(), t)  # every value is bf16-representable
+
+
+def test_pack_unpack_nibble_order():
+    codes = np.array([[1, 2, 3, 4]], dtype=np.uint8)
+    packed = om.pack_codes(codes)
+    assert packed.tolist() == [[0x21, 0x43]]  # element 0 in the low nibble
+    assert np.array_equal(om.unpack_codes(packed), codes)
+
+
+def _c_oracle():
+    so = Path(__file__).resolve().parent.parent / "oracle" / "_build" / "libmxfp4_ref.so"
+    if not so.exists():
+        from oracle.build_oracle import build_oracle
+        build_oracle()
+    lib = ctypes.CDLL(str(so))
+    return lib
+
+
+def test_python_oracle_vs_c_restatement():
+    lib = _c_oracle()
+    a, asc, b, bsc = inputs.mxfp4_inputs(9, 7, 96, seed=5)
+    out = np.empty((9, 96), dtype=np.float32)
+    lib.mxfp4_dequant_c(a.numpy().ctypes.data_as(ctypes.c_void_p), asc.numpy().ctypes.data_as(ctypes.c_void_p),
+                        out.ctypes.data_as(ctypes.c_void_p), ctypes.c_int64(9), ctypes.c_int64(96))
+    assert np.array_equal(out.view(np.uint32), om.mxfp4_dequant_ref(a, asc).view(np.uint32))
+    c = np.empty((9, 7), dtype=np.float32)
+    lib.mxfp4_gemm_c(*(t.numpy().ctypes.data_as(ctypes.c_void_p) for t in (a, asc, b, bsc)), c.ctypes.data_as(ctypes.c_void_p),
+                     ctypes.c_int64(9), ctypes.c_int64(7), ctypes.c_int64(96))
+    np.testing.assert_allclose(c, om.mxfp4_gemm_f64(a, asc, b, bsc).numpy(), rtol=1e-6, atol=0)
+    np.testing.assert_allclose(om.mxfp4_gemm_ref(a, asc, b, bsc).numpy(), c, rtol=1e-5, atol=1e-4)
+
+
+def test_mxfp4_gemm_exact_cases_and_scaling_law():
+    g = torch.Generator().manual_seed(3)
+    pick = np.array([0, 2, 4, 6], dtype=np.uint8)
+    ca = pick[torch.randint(0, 4, (8, 64), generator=g).numpy()]
+    cb = pick[torch.randint(0, 4, (6, 64), generator=g).numpy()]
+    a, b = om.pack_codes(ca), om.pack_codes(cb)
+    one_a, one_b = np.full((8, 2), 127, np.uint8), np.full((6, 2), 127, np.uint8)
+    vals = np.array([0, 1, 2, 4])
+    exp = vals[ca // 2].astype(np.int64) @ vals[cb // 2].astype(np.int64).T
+    assert np.array_equal(om.mxfp4_gemm_ref(a, one_a, b, one_b).numpy(), exp.astype(np.float32))
+    assert np.array_equal(om.mxfp4_gemm_ref(a, one_a + 1, b, one_b).numpy(), 2 * exp.astype(np.float32))
+    # a scale byte covers exactly 32 consecutive k
+    sc = one_a.copy()
+    sc[:, 1] = 128
+    exp2 = vals[ca // 2][:, :32] @ vals[cb // 2][:, :32].T + 2 * (vals[ca // 2][:, 32:] @ vals[cb // 2][:, 32:].T)
+    assert np.array_equal(om.mxfp4_gemm_ref(a, sc, b, one_b).numpy(), exp2.astype(np.float32))
