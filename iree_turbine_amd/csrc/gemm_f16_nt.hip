@@ -5,10 +5,12 @@
 // K-contiguous, so the same row format serves A and B.  Slabs are copied global -> LDS with
 // direct-to-LDS loads (no VGPR staging) into a two-stage ring: while the MFMAs consume
 // stage s the loads for the next slab fill stage s^1, and one barrier per slab closes the
-// iteration.  LDS rows are XOR-swizzled at chunk granularity (chunk c of row r lives in
-// slot c ^ (r & 7)) so that the 32-row x 16-byte fragment reads of v_mfma_f32_32x32x16_f16
-// are free of bank conflicts; because a direct-to-LDS load fixes the LDS slot by lane id,
-// the swizzle is applied on the global side (lane -> which chunk it fetches).
+// iteration.  LDS rows are XOR-swizzled at chunk granularity: chunk c of row r lives in slot
+// c ^ ((r >> 1) & 7).  LDS has 64 banks of 4 bytes, so two 128-byte rows span the banks once and a
+// 16-lane phase of a ds_read_b128 (16 consecutive rows, one chunk each) is conflict-free exactly
+// when (r & 1, slot) is distinct over those rows; measured 247 B/clk/CU against 128 for the
+// c ^ (r & 7) swizzle and 32 unswizzled.  Because a direct-to-LDS load fixes the LDS slot by lane
+// id, the swizzle is applied on the global side (lane -> which chunk it fetches).
 //
 // The MFMA roles are swapped (B rows feed the "A" operand, A rows feed the "B" operand) so a
 // lane ends up owning 4 consecutive n for one m, which turns the epilogue into 8/16-byte
@@ -61,7 +63,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_tiled(const half_t* _
   constexpr int TM = WTM / 32, TN = WTN / 32;
   constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
   constexpr int A_GROUPS = BM / 8, B_GROUPS = BN / 8;  // 8 rows = 1 KiB = one wave-wide load
-  static_assert(A_GROUPS % NW == 0 && B_GROUPS % NW == 0, "loads must split evenly over waves");
+  static_assert(A_GROUPS % NW == 0 && B_GROUPS % NW == 0 && NW % 2 == 0, "loads must split evenly over an even number of waves");
   constexpr int LA = A_GROUPS / NW, LB = B_GROUPS / NW;
 
   extern __shared__ __attribute__((aligned(1024))) char lds[];
@@ -74,7 +76,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_tiled(const half_t* _
 
   // ---- global -> LDS: lane l of a wave-load covers row (l/8) of an 8-row group, slot l%8 ----
   const int lrow = lane >> 3;
-  const int lchunk = (lane & 7) ^ lrow;  // the chunk that belongs in this lane's slot
+  const int lchunk = (lane & 7) ^ (((wave & 1) << 2) | (lrow >> 1));  // the chunk that belongs in this lane's slot
   const half_t* a_src = A + (size_t)(tile_m * BM + wave * 8 + lrow) * K + lchunk * 8;
   const half_t* b_src = B + (size_t)(tile_n * BN + wave * 8 + lrow) * K + lchunk * 8;
   const size_t row_step = (size_t)NW * 8 * K;  // halfs between this wave's consecutive groups
@@ -91,7 +93,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_tiled(const half_t* _
 
   // ---- LDS -> MFMA fragments ----
   const int r32 = lane & 31, h = lane >> 5;
-  const int sw = (h ^ (lane & 7)) * 16;
+  const int sw = (h ^ ((r32 >> 1) & 7)) * 16;
   const int a_base = (wm * WTM + r32) * 128 + sw;            // rows of A (m): feeds the MFMA "B" operand
   const int b_base = A_BYTES + (wn * WTN + r32) * 128 + sw;  // rows of B (n): feeds the MFMA "A" operand
 
@@ -128,17 +130,227 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_tiled(const half_t* _
   }
 
   // ---- epilogue: lane owns m = r32 and, per register quad q, n = 8q + 4h .. +3 ----
-  const int m0 = tile_m * BM + wm * WTM + r32;
-  const int n0 = tile_n * BN + wn * WTN + 4 * h;
+  if constexpr (sizeof(OutT) == 2) {
+    // fp16 epilogue through LDS (free after the last barrier): each wave transposes its own
+    // WTM x WTN tile in a private region (ds_write_b64 of 4 consecutive n, chunk slot c ^ ((m>>1)&7)),
+    // then reads whole rows back 16 bytes per lane and stores full 128-byte lines.
+    constexpr int ROW_B = WTN * 2, CH = WTN / 8;
+    char* ep = lds + wave * (WTM * ROW_B);
 #pragma unroll
-  for (int j = 0; j < TM; j++) {
-    OutT* crow = C + (size_t)(m0 + j * 32) * N + n0;
+    for (int j = 0; j < TM; j++) {
+      const int ml = j * 32 + r32;
+#pragma unroll
+      for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const int c = i * 4 + q;
+          half4 v = {(half_t)acc[i][j][4 * q], (half_t)acc[i][j][4 * q + 1], (half_t)acc[i][j][4 * q + 2],
+                     (half_t)acc[i][j][4 * q + 3]};
+          *reinterpret_cast<half4*>(ep + ml * ROW_B + ((c ^ ((ml >> 1) & 7)) * 16) + 8 * h) = v;
+        }
+    }
+    constexpr int ROWS_PER_IT = 64 / CH;
+    const int er = lane / CH, ec = lane % CH;
+    OutT* cbase = C + (size_t)(tile_m * BM + wm * WTM) * N + tile_n * BN + wn * WTN + ec * 8;
+#pragma unroll
+    for (int it = 0; it < WTM / ROWS_PER_IT; it++) {
+      const int row = it * ROWS_PER_IT + er;
+      half8 v = *reinterpret_cast<const half8*>(ep + row * ROW_B + ((ec ^ ((row >> 1) & 7)) * 16));
+      *reinterpret_cast<half8*>(cbase + (size_t)row * N) = v;
+    }
+  } else {
+    const int m0 = tile_m * BM + wm * WTM + r32;
+    const int n0 = tile_n * BN + wn * WTN + 4 * h;
+#pragma unroll
+    for (int j = 0; j < TM; j++) {
+      OutT* crow = C + (size_t)(m0 + j * 32) * N + n0;
+#pragma unroll
+      for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+          OutPack<OutT>::store4(crow + i * 32 + q * 8, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                                acc[i][j][4 * q + 3]);
+    }
+  }
+}
+
+// Software-pipelined form of the tiled kernel.  Same tiling, LDS format and swizzle; the k-loop is
+// rotated so that (a) the fragments of k-step s+1 are requested from LDS before the MFMAs of
+// k-step s issue, (b) the barrier that retires a slab sits in front of the last k-step's MFMAs,
+// which then overlap the first fragment reads of the next slab, and (c) the global -> LDS loads
+// for slab k+2 are issued right after that barrier into the stage that was just retired.
+template <int BM, int BN, int WM, int WN, typename OutT>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_t* __restrict__ A,
+                                                                     const half_t* __restrict__ B,
+                                                                     OutT* __restrict__ C, int M, int N, int K,
+                                                                     int tiles_m, int tiles_n, int group_m) {
+  constexpr int NW = WM * WN;
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
+  constexpr int A_GROUPS = BM / 8, B_GROUPS = BN / 8;
+  static_assert(A_GROUPS % NW == 0 && B_GROUPS % NW == 0 && NW % 2 == 0, "loads must split evenly over an even number of waves");
+  constexpr int LA = A_GROUPS / NW, LB = B_GROUPS / NW;
+
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  int tile_m, tile_n;
+  map_tile(blockIdx.x, tiles_m, tiles_n, group_m, tile_m, tile_n);
+
+  const int lrow = lane >> 3;
+  const int lchunk = (lane & 7) ^ (((wave & 1) << 2) | (lrow >> 1));
+  const half_t* a_src = A + (size_t)(tile_m * BM + wave * 8 + lrow) * K + lchunk * 8;
+  const half_t* b_src = B + (size_t)(tile_n * BN + wave * 8 + lrow) * K + lchunk * 8;
+  const size_t row_step = (size_t)NW * 8 * K;
+
+  auto issue_loads = [&](int stage, int slab) {
+    char* dst = lds + stage * STAGE + wave * 1024;
+    const half_t* ap = a_src + slab * 64;
+    const half_t* bp = b_src + slab * 64;
+#pragma unroll
+    for (int i = 0; i < LA; i++) load_lds_16B(ap + i * row_step, dst + i * NW * 1024);
+#pragma unroll
+    for (int i = 0; i < LB; i++) load_lds_16B(bp + i * row_step, dst + A_BYTES + i * NW * 1024);
+  };
+
+  const int r32 = lane & 31, h = lane >> 5;
+  const int sw = (h ^ ((r32 >> 1) & 7)) * 16;
+  const int a_base = (wm * WTM + r32) * 128 + sw;
+  const int b_base = A_BYTES + (wn * WTN + r32) * 128 + sw;
+  auto read_frags = [&](const char* st, int ks, half8* fm, half8* fn) {
+#pragma unroll
+    for (int j = 0; j < TM; j++) fm[j] = *reinterpret_cast<const half8*>(st + ((a_base ^ (ks * 32)) + j * 4096));
+#pragma unroll
+    for (int i = 0; i < TN; i++) fn[i] = *reinterpret_cast<const half8*>(st + ((b_base ^ (ks * 32)) + i * 4096));
+  };
+
+  floatx16 acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; i++)
+#pragma unroll
+    for (int j = 0; j < TM; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+  auto mfmas = [&](const half8* fm, const half8* fn) {
 #pragma unroll
     for (int i = 0; i < TN; i++)
 #pragma unroll
-      for (int q = 0; q < 4; q++)
-        OutPack<OutT>::store4(crow + i * 32 + q * 8, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
-                              acc[i][j][4 * q + 3]);
+      for (int j = 0; j < TM; j++) acc[i][j] = mfma_32x32x16(fn[i], fm[j], acc[i][j]);
+  };
+
+  const int KT = K / 64;
+  half8 fm0[TM], fn0[TN], fm1[TM], fn1[TN];
+
+  issue_loads(0, 0);
+  wait_vmcnt0();
+  __syncthreads();
+  issue_loads(1, KT > 1 ? 1 : 0);
+  read_frags(lds, 0, fm0, fn0);
+
+  // One k-step region: the MFMAs of the current fragments with the LDS reads of the next fragments
+  // slotted in between them (first instruction is an MFMA, so the wait in front of it only covers
+  // reads issued a whole k-step earlier).
+  auto interleave = [&]() {
+#pragma unroll
+    for (int i = 0; i < TM + TN; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
+  };
+
+  for (int kt = 0; kt < KT; kt++) {
+    const char* st = lds + (kt & 1) * STAGE;
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(st, 1, fm1, fn1);
+    mfmas(fm0, fn0);
+    interleave();
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(st, 2, fm0, fn0);
+    mfmas(fm1, fn1);
+    interleave();
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(st, 3, fm1, fn1);
+    mfmas(fm0, fn0);
+    interleave();
+    __builtin_amdgcn_sched_barrier(0);
+    // retire the slab: every wave's LDS reads of this stage have returned, next slab has landed
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    // The MFMAs of the last k-step need nothing new, so they lead; the loads for slab kt+2 (into the
+    // stage just retired) and the first fragment reads of slab kt+1 are slotted in between them.
+    // Past the end the loads re-fetch the last slab and the reads see stale bytes; neither is used.
+    issue_loads(kt & 1, kt + 2 < KT ? kt + 2 : KT - 1);
+    read_frags(lds + ((kt + 1) & 1) * STAGE, 0, fm0, fn0);
+    mfmas(fm1, fn1);
+    {
+      constexpr int NL = LA + LB, NR = TM + TN, NM = TM * TN;
+      constexpr int M_FOR_LOADS = NM / 2, L_PER_M = (NL + M_FOR_LOADS - 1) / M_FOR_LOADS;
+#pragma unroll
+      for (int i = 0; i < M_FOR_LOADS; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x010, L_PER_M, 0);  // VMEM (direct-to-LDS loads)
+      }
+      constexpr int M_FOR_READS = NM - M_FOR_LOADS - 1, R_PER_M = (NR + M_FOR_READS - 1) / M_FOR_READS;
+#pragma unroll
+      for (int i = 0; i < M_FOR_READS; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, R_PER_M, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  // the speculative loads of the last iterations target LDS: drain them before the epilogue reuses it
+  wait_vmcnt0();
+  __syncthreads();
+
+  if constexpr (sizeof(OutT) == 2) {
+    // fp16 epilogue through LDS (free after the last barrier): each wave transposes its own
+    // WTM x WTN tile in a private region (ds_write_b64 of 4 consecutive n, chunk slot c ^ ((m>>1)&7)),
+    // then reads whole rows back 16 bytes per lane and stores full 128-byte lines.
+    constexpr int ROW_B = WTN * 2, CH = WTN / 8;
+    char* ep = lds + wave * (WTM * ROW_B);
+#pragma unroll
+    for (int j = 0; j < TM; j++) {
+      const int ml = j * 32 + r32;
+#pragma unroll
+      for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const int c = i * 4 + q;
+          half4 v = {(half_t)acc[i][j][4 * q], (half_t)acc[i][j][4 * q + 1], (half_t)acc[i][j][4 * q + 2],
+                     (half_t)acc[i][j][4 * q + 3]};
+          *reinterpret_cast<half4*>(ep + ml * ROW_B + ((c ^ ((ml >> 1) & 7)) * 16) + 8 * h) = v;
+        }
+    }
+    constexpr int ROWS_PER_IT = 64 / CH;
+    const int er = lane / CH, ec = lane % CH;
+    OutT* cbase = C + (size_t)(tile_m * BM + wm * WTM) * N + tile_n * BN + wn * WTN + ec * 8;
+#pragma unroll
+    for (int it = 0; it < WTM / ROWS_PER_IT; it++) {
+      const int row = it * ROWS_PER_IT + er;
+      half8 v = *reinterpret_cast<const half8*>(ep + row * ROW_B + ((ec ^ ((row >> 1) & 7)) * 16));
+      *reinterpret_cast<half8*>(cbase + (size_t)row * N) = v;
+    }
+  } else {
+    const int m0 = tile_m * BM + wm * WTM + r32;
+    const int n0 = tile_n * BN + wn * WTN + 4 * h;
+#pragma unroll
+    for (int j = 0; j < TM; j++) {
+      OutT* crow = C + (size_t)(m0 + j * 32) * N + n0;
+#pragma unroll
+      for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+          OutPack<OutT>::store4(crow + i * 32 + q * 8, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                                acc[i][j][4 * q + 3]);
+    }
   }
 }
 
@@ -205,8 +417,10 @@ struct GemmVariant {
   int bm, bn, threads;
 };
 static const GemmVariant kGemmVariants[] = {
+    {"pipelined_256x256x64_w2x4", 256, 256, 512},
+    {"pipelined_256x256x64_w2x2", 256, 256, 256},
+    {"pipelined_128x128x64_w2x2", 128, 128, 256},
     {"tiled_256x256x64_w2x4", 256, 256, 512},
-    {"tiled_256x256x64_w2x2", 256, 256, 256},
     {"tiled_128x128x64_w2x2", 128, 128, 256},
     {"generic_64x64x32", 64, 64, 256},
 };
@@ -215,16 +429,18 @@ constexpr int kNumGemmVariants = sizeof(kGemmVariants) / sizeof(kGemmVariants[0]
 int gemm_variant_count() { return kNumGemmVariants; }
 const char* gemm_variant_name(int i) { return (i >= 0 && i < kNumGemmVariants) ? kGemmVariants[i].name : nullptr; }
 
-template <int BM, int BN, int WM, int WN, typename OutT>
+template <int BM, int BN, int WM, int WN, typename OutT, bool PIPELINED>
 static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int K, hipStream_t stream) {
-  auto kern = gemm_f16_nt_tiled<BM, BN, WM, WN, OutT>;
+  void (*kern)(const half_t*, const half_t*, OutT*, int, int, int, int, int, int);
+  if constexpr (PIPELINED) kern = gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT>;
+  else kern = gemm_f16_nt_tiled<BM, BN, WM, WN, OutT>;
   constexpr int lds_bytes = 2 * (BM + BN) * 128;
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        lds_bytes);
     if (e != hipSuccess) {
-      set_error("hipFuncSetAttribute(gemm_f16_nt_tiled, %d bytes LDS): %s", lds_bytes, hipGetErrorString(e));
+      set_error("hipFuncSetAttribute(gemm_f16_nt, %d bytes LDS): %s", lds_bytes, hipGetErrorString(e));
       return (int)e;
     }
     attr_set = true;
@@ -234,15 +450,17 @@ static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int
   dim3 grid(tiles_m * tiles_n), block(WM * WN * 64);
   hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, M, N, K, tiles_m,
                      tiles_n, group_m);
-  return check_launch("gemm_f16_nt_tiled", grid, block, lds_bytes);
+  return check_launch(PIPELINED ? "gemm_f16_nt_pipelined" : "gemm_f16_nt_tiled", grid, block, lds_bytes);
 }
 
 template <typename OutT>
 static int launch_variant(int variant, const void* a, const void* b, void* c, int M, int N, int K, hipStream_t stream) {
   switch (variant) {
-    case 0: return launch_tiled<256, 256, 2, 4, OutT>(a, b, c, M, N, K, stream);
-    case 1: return launch_tiled<256, 256, 2, 2, OutT>(a, b, c, M, N, K, stream);
-    case 2: return launch_tiled<128, 128, 2, 2, OutT>(a, b, c, M, N, K, stream);
+    case 0: return launch_tiled<256, 256, 2, 4, OutT, true>(a, b, c, M, N, K, stream);
+    case 1: return launch_tiled<256, 256, 2, 2, OutT, true>(a, b, c, M, N, K, stream);
+    case 2: return launch_tiled<128, 128, 2, 2, OutT, true>(a, b, c, M, N, K, stream);
+    case 3: return launch_tiled<256, 256, 2, 4, OutT, false>(a, b, c, M, N, K, stream);
+    case 4: return launch_tiled<128, 128, 2, 2, OutT, false>(a, b, c, M, N, K, stream);
     default: {
       dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
       hipLaunchKernelGGL(gemm_f16_nt_generic<OutT>, grid, block, 0, stream, (const half_t*)a, (const half_t*)b, (OutT*)c,
@@ -272,7 +490,9 @@ extern "C" int mi355_gemm_f16_nt(const void* a, const void* b, void* c, int64_t 
   if (variant < 0) {
     // Large problems take the 256x256 tile; when that leaves most of the 256 CUs idle the
     // 128x128 tile (4x the workgroups) wins; everything else goes to the bounds-checked kernel.
-    if (fits(0) && (M / 256) * (N / 256) >= 128) variant = 0;
+    const long long t256 = (M / 256) * (N / 256);
+    const long long rounds = (t256 + 255) / 256;  // 256 CUs, one 256x256 workgroup each
+    if (fits(0) && t256 >= 128 && t256 * 100 >= rounds * 256 * 85) variant = 0;  // >= 85% of the last round busy
     else if (fits(2)) variant = 2;
     else variant = kNumGemmVariants - 1;
   } else if (!fits(variant)) {

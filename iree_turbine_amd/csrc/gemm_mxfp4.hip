@@ -75,7 +75,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
   const int Kb = K >> 1;   // bytes per row of codes
   const int Ksc = K >> 5;  // scale bytes per row
   const int lrow = lane >> 3;
-  const int lchunk = (lane & 7) ^ lrow;
+  const int lchunk = (lane & 7) ^ (((wave & 1) << 2) | (lrow >> 1));
   const uint8_t* a_src = A + (size_t)(tile_m * BM + wave * 8 + lrow) * Kb + lchunk * 16;
   const uint8_t* b_src = B + (size_t)(tile_n * BN + wave * 8 + lrow) * Kb + lchunk * 16;
   const size_t row_step = (size_t)NW * 8 * Kb;
@@ -91,7 +91,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
   };
 
   const int r32 = lane & 31, h = lane >> 5;
-  const int sw = (h ^ (lane & 7)) * 16;
+  const int sw = (h ^ ((r32 >> 1) & 7)) * 16;
   const int a_base = (wm * WTM + r32) * 128 + sw;
   const int b_base = A_BYTES + (wn * WTN + r32) * 128 + sw;
 

@@ -10,7 +10,7 @@ M, N, K = sym.M, sym.N, sym.K
 BLOCK_M, BLOCK_N, BLOCK_K = sym.BLOCK_M, sym.BLOCK_N, sym.BLOCK_K
 
 # (BLOCK_M, BLOCK_N) -> kernel variant index of mi355_gemm_f16_nt
-_VARIANT_BY_TILE = {(256, 256): 0, (128, 128): 2, (64, 64): 3}
+_VARIANT_BY_TILE = {(256, 256): 0, (128, 128): 2, (64, 64): 5}
 
 
 def _entry(hp, a, b, c):

@@ -22,7 +22,7 @@ def _run(dev, M, N, K, out_dtype, variant=-1, seed=10):
     return c.float().cpu(), ref
 
 
-@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 3])
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 3, 4, 5])
 def test_gemm_1024_f32_all_variants(dev, variant):
     c, ref = _run(dev, 1024, 1024, 1024, "float32", variant)
     torch.testing.assert_close(c, ref, rtol=RTOL, atol=ATOL)
@@ -95,6 +95,8 @@ def test_gemm_contract_errors(dev):
         torch.ops.mi355.gemm_nt(a.float(), a.float(), "float32", -1)
     with pytest.raises(ValueError):
         torch.ops.mi355.gemm_nt(a, a, "float32", 0)  # 256x256 tile does not divide 64x64
+    with pytest.raises(ValueError):
+        torch.ops.mi355.gemm_nt(a, a, "float32", 99)  # no such variant
     with pytest.raises(ValueError):
         torch.ops.mi355.gemm_nt(a, a, "int8", -1)
 
