@@ -202,8 +202,10 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
 
   const int lrow = lane >> 3;
   const int lchunk = (lane & 7) ^ (((wave & 1) << 2) | (lrow >> 1));
-  const half_t* a_src = A + (size_t)(tile_m * BM + wave * 8 + lrow) * K + lchunk * 8;
-  const half_t* b_src = B + (size_t)(tile_n * BN + wave * 8 + lrow) * K + lchunk * 8;
+  // wave-uniform base pointer + one 32-bit per-lane offset (in halfs) shared by every load of the wave
+  const half_t* a_src = A + (size_t)(tile_m * BM + wave * 8) * K;
+  const half_t* b_src = B + (size_t)(tile_n * BN + wave * 8) * K;
+  const unsigned lane_off = (unsigned)lrow * (unsigned)K + (unsigned)lchunk * 8u;
   const size_t row_step = (size_t)NW * 8 * K;
 
   auto issue_loads = [&](int stage, int slab) {
@@ -211,9 +213,9 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
     const half_t* ap = a_src + slab * 64;
     const half_t* bp = b_src + slab * 64;
 #pragma unroll
-    for (int i = 0; i < LA; i++) load_lds_16B(ap + i * row_step, dst + i * NW * 1024);
+    for (int i = 0; i < LA; i++) load_lds_16B(ap + i * row_step + lane_off, dst + i * NW * 1024);
 #pragma unroll
-    for (int i = 0; i < LB; i++) load_lds_16B(bp + i * row_step, dst + A_BYTES + i * NW * 1024);
+    for (int i = 0; i < LB; i++) load_lds_16B(bp + i * row_step + lane_off, dst + A_BYTES + i * NW * 1024);
   };
 
   const int r32 = lane & 31, h = lane >> 5;
@@ -477,7 +479,7 @@ using namespace mi355;
 extern "C" int mi355_gemm_f16_nt(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int out_dtype,
                                  int variant, void* stream) {
   if (!a || !b || !c) return fail(-MI355_E_NULL, "gemm_f16_nt: null pointer (a=%p b=%p c=%p)", a, b, c);
-  if (M <= 0 || N <= 0 || K <= 0 || M > (1 << 30) || N > (1 << 30) || K > (1 << 30))
+  if (M <= 0 || N <= 0 || K <= 0 || M > (1 << 30) || N > (1 << 30) || K > (1 << 27))
     return fail(-MI355_E_SHAPE, "gemm_f16_nt: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
   if (out_dtype != MI355_F32 && out_dtype != MI355_F16)
     return fail(-MI355_E_DTYPE, "gemm_f16_nt: out_dtype %d (want MI355_F32 or MI355_F16)", out_dtype);

@@ -7,7 +7,8 @@
 //
 // Tiling is the fp16 GEMM's with k measured in bytes: a K slab is 256 fp4 values = 128 bytes
 // per row = 8 chunks of 16 bytes (one chunk = one 32-element scale block), copied with
-// direct-to-LDS loads into a two-stage ring with the same XOR swizzle.  A lane's 16-byte
+// direct-to-LDS loads into a two-stage ring with the same XOR swizzle and the same rotated,
+// software-pipelined k-loop.  A lane's 16-byte
 // fragment is exactly one scale block, so the lane's scale byte is scale[row][slab*8 + 2*ks + h]
 // (h = lane / 32); each lane fetches the 8 scale bytes of its row for a slab with one 8-byte
 // global load one slab ahead, lanes with h = 1 pre-shift by one byte, and the op_sel field of
@@ -52,7 +53,10 @@ __device__ __forceinline__ floatx16 mfma_fp4_32x32x64(intx4 a, int sa, intx4 b, 
   return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, 4, 4, 0, sa, 0, sb);
 }
 
-template <int BM, int BN, int WM, int WN, typename OutT>
+// SCALES_LDS: scale bytes travel through LDS in groups of 4 slabs (32 bytes per row, two buffers behind
+// the data stages) instead of one strided 8-byte global load per lane, row tile and slab.  Needs
+// K % 1024 == 0.
+template <int BM, int BN, int WM, int WN, typename OutT, bool SCALES_LDS>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* __restrict__ A, const uint8_t* __restrict__ As,
                                                                 const uint8_t* __restrict__ B, const uint8_t* __restrict__ Bs,
                                                                 OutT* __restrict__ C, int M, int N, int K, int tiles_m,
@@ -62,7 +66,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
   constexpr int TM = WTM / 32, TN = WTN / 32;
   constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
   constexpr int A_GROUPS = BM / 8, B_GROUPS = BN / 8;
-  static_assert(A_GROUPS % NW == 0 && B_GROUPS % NW == 0, "loads must split evenly over waves");
+  static_assert(A_GROUPS % NW == 0 && B_GROUPS % NW == 0 && NW % 2 == 0, "loads must split evenly over an even number of waves");
   constexpr int LA = A_GROUPS / NW, LB = B_GROUPS / NW;
 
   extern __shared__ __attribute__((aligned(1024))) char lds[];
@@ -75,19 +79,22 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
   const int Kb = K >> 1;   // bytes per row of codes
   const int Ksc = K >> 5;  // scale bytes per row
   const int lrow = lane >> 3;
+  // chunk c of row r lives in slot c ^ ((r >> 1) & 7): conflict-free fragment reads on 64 LDS banks
   const int lchunk = (lane & 7) ^ (((wave & 1) << 2) | (lrow >> 1));
-  const uint8_t* a_src = A + (size_t)(tile_m * BM + wave * 8 + lrow) * Kb + lchunk * 16;
-  const uint8_t* b_src = B + (size_t)(tile_n * BN + wave * 8 + lrow) * Kb + lchunk * 16;
+  // wave-uniform base pointer + one 32-bit per-lane offset shared by every load of the wave
+  const uint8_t* a_src = A + (size_t)(tile_m * BM + wave * 8) * Kb;
+  const uint8_t* b_src = B + (size_t)(tile_n * BN + wave * 8) * Kb;
+  const unsigned lane_off = (unsigned)lrow * (unsigned)Kb + (unsigned)lchunk * 16u;
   const size_t row_step = (size_t)NW * 8 * Kb;
 
-  auto issue_loads = [&](int stage) {
+  auto issue_loads = [&](int stage, int slab) {
     char* dst = lds + stage * STAGE + wave * 1024;
+    const uint8_t* ap = a_src + slab * 128;
+    const uint8_t* bp = b_src + slab * 128;
 #pragma unroll
-    for (int i = 0; i < LA; i++) load_lds_16B(a_src + i * row_step, dst + i * NW * 1024);
+    for (int i = 0; i < LA; i++) load_lds_16B(ap + i * row_step + lane_off, dst + i * NW * 1024);
 #pragma unroll
-    for (int i = 0; i < LB; i++) load_lds_16B(b_src + i * row_step, dst + A_BYTES + i * NW * 1024);
-    a_src += 128;
-    b_src += 128;
+    for (int i = 0; i < LB; i++) load_lds_16B(bp + i * row_step + lane_off, dst + A_BYTES + i * NW * 1024);
   };
 
   const int r32 = lane & 31, h = lane >> 5;
@@ -95,17 +102,68 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
   const int a_base = (wm * WTM + r32) * 128 + sw;
   const int b_base = A_BYTES + (wn * WTN + r32) * 128 + sw;
 
-  // scale bytes: 8 per row per slab
+  // scale bytes: 8 per row per slab, fetched one slab ahead; lanes with h = 1 drop one byte so that
+  // op_sel 0 / 2 address blocks 2*ks + h of the slab for every lane
   const uint8_t* as_src = As + (size_t)(tile_m * BM + wm * WTM + r32) * Ksc;
   const uint8_t* bs_src = Bs + (size_t)(tile_n * BN + wn * WTN + r32) * Ksc;
+  const int shift = 8 * h;
   intx2 sa_cur[TM], sb_cur[TN], sa_nxt[TM], sb_nxt[TN];
-  auto load_scales = [&](intx2* sa, intx2* sb) {
+  // LDS scale buffers: [buffer][A rows then B rows][32 bytes = 4 slabs x 8 blocks]
+  constexpr int SC_BUF = (BM + BN) * 32;
+  char* sc_lds = lds + 2 * STAGE;
+  static_assert(((BM + BN) / 32) % NW == 0, "scale rows must split evenly over waves");
+  constexpr int LS = (BM + BN) / 32 / NW;  // wave-loads (32 rows x 32 bytes) per wave per group
+  const unsigned sc_lane_off = (unsigned)(lane >> 1) * (unsigned)Ksc + (unsigned)(lane & 1) * 16u;
+  auto issue_scale_loads = [&](int group) {
+    char* dst = sc_lds + (group & 1) * SC_BUF;
 #pragma unroll
-    for (int j = 0; j < TM; j++) sa[j] = *reinterpret_cast<const intx2*>(as_src + (size_t)j * 32 * Ksc);
+    for (int i = 0; i < LS; i++) {
+      const int r0 = (wave * LS + i) * 32;  // first of 32 consecutive rows (all in A or all in B: BM % 32 == 0)
+      const uint8_t* src = r0 < BM ? As + (size_t)(tile_m * BM + r0) * Ksc : Bs + (size_t)(tile_n * BN + r0 - BM) * Ksc;
+      load_lds_16B(src + group * 32 + sc_lane_off, dst + r0 * 32);
+    }
+  };
+  const int sa_off = (wm * WTM + r32) * 32, sb_off = (BM + wn * WTN + r32) * 32;
+  auto load_scales = [&](intx2* sa, intx2* sb, int slab) {
+    if constexpr (SCALES_LDS) {
+      const char* buf = sc_lds + ((slab >> 2) & 1) * SC_BUF + (slab & 3) * 8;
 #pragma unroll
-    for (int i = 0; i < TN; i++) sb[i] = *reinterpret_cast<const intx2*>(bs_src + (size_t)i * 32 * Ksc);
-    as_src += 8;
-    bs_src += 8;
+      for (int j = 0; j < TM; j++) sa[j] = *reinterpret_cast<const intx2*>(buf + sa_off + j * 1024);
+#pragma unroll
+      for (int i = 0; i < TN; i++) sb[i] = *reinterpret_cast<const intx2*>(buf + sb_off + i * 1024);
+    } else {
+#pragma unroll
+      for (int j = 0; j < TM; j++) sa[j] = *reinterpret_cast<const intx2*>(as_src + (size_t)j * 32 * Ksc + slab * 8);
+#pragma unroll
+      for (int i = 0; i < TN; i++) sb[i] = *reinterpret_cast<const intx2*>(bs_src + (size_t)i * 32 * Ksc + slab * 8);
+    }
+  };
+  // SCALES_LDS: one dword (4 blocks = 2 k-steps) per row tile straight into the live scale registers
+  auto lds_scales = [&](int slab, int d) {
+    const char* buf = sc_lds + ((slab >> 2) & 1) * SC_BUF + (slab & 3) * 8 + d * 4;
+#pragma unroll
+    for (int j = 0; j < TM; j++) sa_cur[j][d] = (int)(*reinterpret_cast<const unsigned*>(buf + sa_off + j * 1024) >> shift);
+#pragma unroll
+    for (int i = 0; i < TN; i++) sb_cur[i][d] = (int)(*reinterpret_cast<const unsigned*>(buf + sb_off + i * 1024) >> shift);
+  };
+  auto shift_scales = [&](intx2* sa, intx2* sb) {
+#pragma unroll
+    for (int j = 0; j < TM; j++) {
+      sa[j][0] = (int)((unsigned)sa[j][0] >> shift);
+      sa[j][1] = (int)((unsigned)sa[j][1] >> shift);
+    }
+#pragma unroll
+    for (int i = 0; i < TN; i++) {
+      sb[i][0] = (int)((unsigned)sb[i][0] >> shift);
+      sb[i][1] = (int)((unsigned)sb[i][1] >> shift);
+    }
+  };
+
+  auto read_frags = [&](const char* st, int ks, intx4* fm, intx4* fn) {
+#pragma unroll
+    for (int j = 0; j < TM; j++) fm[j] = *reinterpret_cast<const intx4*>(st + ((a_base ^ (ks * 32)) + j * 4096));
+#pragma unroll
+    for (int i = 0; i < TN; i++) fn[i] = *reinterpret_cast<const intx4*>(st + ((b_base ^ (ks * 32)) + i * 4096));
   };
 
   floatx16 acc[TN][TM];
@@ -116,57 +174,154 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-  const int KT = K / 256;
-  load_scales(sa_cur, sb_cur);
-  issue_loads(0);
-  wait_vmcnt0();
-  __syncthreads();
-
-  const int shift = 8 * h;
-  for (int kt = 0; kt < KT; kt++) {
-    if (kt + 1 < KT) {
-      issue_loads((kt + 1) & 1);
-      load_scales(sa_nxt, sb_nxt);
-    }
-    const char* st = lds + (kt & 1) * STAGE;
-#pragma unroll
-    for (int ks = 0; ks < 4; ks++) {
-      intx4 fm[TM], fn[TN];
-      int sm[TM], sn[TN];
-#pragma unroll
-      for (int j = 0; j < TM; j++) {
-        fm[j] = *reinterpret_cast<const intx4*>(st + ((a_base ^ (ks * 32)) + j * 4096));
-        sm[j] = (int)((unsigned)sa_cur[j][ks >> 1] >> shift);
-      }
-#pragma unroll
-      for (int i = 0; i < TN; i++) {
-        fn[i] = *reinterpret_cast<const intx4*>(st + ((b_base ^ (ks * 32)) + i * 4096));
-        sn[i] = (int)((unsigned)sb_cur[i][ks >> 1] >> shift);
-      }
-#pragma unroll
-      for (int i = 0; i < TN; i++)
-#pragma unroll
-        for (int j = 0; j < TM; j++) acc[i][j] = mfma_fp4_32x32x64(fn[i], sn[i], fm[j], sm[j], acc[i][j], ks & 1);
-    }
-    wait_vmcnt0();
-    __syncthreads();
-#pragma unroll
-    for (int j = 0; j < TM; j++) sa_cur[j] = sa_nxt[j];
-#pragma unroll
-    for (int i = 0; i < TN; i++) sb_cur[i] = sb_nxt[i];
-  }
-
-  const int m0 = tile_m * BM + wm * WTM + r32;
-  const int n0 = tile_n * BN + wn * WTN + 4 * h;
-#pragma unroll
-  for (int j = 0; j < TM; j++) {
-    OutT* crow = C + (size_t)(m0 + j * 32) * N + n0;
+  auto mfmas = [&](const intx4* fm, const intx4* fn, int ks) {
 #pragma unroll
     for (int i = 0; i < TN; i++)
 #pragma unroll
-      for (int q = 0; q < 4; q++)
-        MxOut<OutT>::store4(crow + i * 32 + q * 8, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
-                            acc[i][j][4 * q + 3]);
+      for (int j = 0; j < TM; j++)
+        acc[i][j] = mfma_fp4_32x32x64(fn[i], sb_cur[i][ks >> 1], fm[j], sa_cur[j][ks >> 1], acc[i][j], ks & 1);
+  };
+  auto interleave = [&]() {
+#pragma unroll
+    for (int i = 0; i < TM + TN; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
+  };
+
+  // k-step region that also fetches TM + TN scale dwords from LDS: two LDS reads per slot
+  auto interleave_with_scales = [&]() {
+#pragma unroll
+    for (int i = 0; i < TM + TN; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
+  };
+
+  const int KT = K / 256;
+  intx4 fm0[TM], fn0[TN], fm1[TM], fn1[TN];
+
+  const int KG = (KT + 3) >> 2;  // scale groups
+  if constexpr (SCALES_LDS) issue_scale_loads(0);
+  issue_loads(0, 0);
+  wait_vmcnt0();
+  __syncthreads();
+  if constexpr (SCALES_LDS) {
+    lds_scales(0, 0);
+    issue_scale_loads(KG > 1 ? 1 : 0);
+    issue_loads(1, KT > 1 ? 1 : 0);
+  } else {
+    load_scales(sa_cur, sb_cur, 0);
+    issue_loads(1, KT > 1 ? 1 : 0);
+    wait_vmcnt0();
+    shift_scales(sa_cur, sb_cur);
+  }
+  read_frags(lds, 0, fm0, fn0);
+
+  // Rotated k-loop (see gemm_f16_nt_pipelined): fragment reads for k-step s+1 ride between the MFMAs
+  // of k-step s; the slab-retiring barrier sits in front of the last k-step's MFMAs, which overlap the
+  // global -> LDS loads of slab kt+2 and the first fragment reads of slab kt+1.
+  for (int kt = 0; kt < KT; kt++) {
+    const char* st = lds + (kt & 1) * STAGE;
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (SCALES_LDS) lds_scales(kt, 1);  // blocks 4..7 of this slab (their registers went idle after the last k-step)
+    else load_scales(sa_nxt, sb_nxt, kt + 1 < KT ? kt + 1 : KT - 1);
+    read_frags(st, 1, fm1, fn1);
+    mfmas(fm0, fn0, 0);
+    if constexpr (SCALES_LDS) interleave_with_scales(); else interleave();
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(st, 2, fm0, fn0);
+    mfmas(fm1, fn1, 1);
+    interleave();
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(st, 3, fm1, fn1);
+    if constexpr (SCALES_LDS) lds_scales(kt + 1 < KT ? kt + 1 : KT - 1, 0);  // blocks 0..3 of the next slab
+    mfmas(fm0, fn0, 2);
+    if constexpr (SCALES_LDS) interleave_with_scales(); else interleave();
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    issue_loads(kt & 1, kt + 2 < KT ? kt + 2 : KT - 1);
+    if constexpr (SCALES_LDS) {
+      // Group g+1 replaces group g-1 in its buffer once the last slab of g-1 has had its scales read
+      // into registers: that happens during slab 4g-2, i.e. before the barrier of slab 4g-1 = kt.
+      if ((kt & 3) == 3) {
+        const int g = (kt >> 2) + 2;
+        issue_scale_loads(g < KG ? g : KG - 1);
+      }
+    }
+    read_frags(lds + ((kt + 1) & 1) * STAGE, 0, fm0, fn0);
+    mfmas(fm1, fn1, 3);
+    {
+      constexpr int NL = LA + LB, NR = TM + TN, NM = TM * TN;
+      constexpr int M_FOR_LOADS = NM / 2, L_PER_M = (NL + M_FOR_LOADS - 1) / M_FOR_LOADS;
+#pragma unroll
+      for (int i = 0; i < M_FOR_LOADS; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x010, L_PER_M, 0);
+      }
+      constexpr int M_FOR_READS = NM - M_FOR_LOADS - 1, R_PER_M = (NR + M_FOR_READS - 1) / M_FOR_READS;
+#pragma unroll
+      for (int i = 0; i < M_FOR_READS; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, R_PER_M, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (!SCALES_LDS) {
+#pragma unroll
+      for (int j = 0; j < TM; j++) sa_cur[j] = sa_nxt[j];
+#pragma unroll
+      for (int i = 0; i < TN; i++) sb_cur[i] = sb_nxt[i];
+      shift_scales(sa_cur, sb_cur);
+    }
+  }
+  wait_vmcnt0();
+  __syncthreads();
+
+  if constexpr (sizeof(OutT) == 2) {
+    // bf16 epilogue through LDS: each wave transposes its tile privately, then stores full rows
+    constexpr int ROW_B = WTN * 2, CH = WTN / 8;
+    char* ep = lds + wave * (WTM * ROW_B);
+#pragma unroll
+    for (int j = 0; j < TM; j++) {
+      const int ml = j * 32 + r32;
+#pragma unroll
+      for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const int c = i * 4 + q;
+          ushortx4 v = {f32_to_bf16_rne(acc[i][j][4 * q]), f32_to_bf16_rne(acc[i][j][4 * q + 1]),
+                        f32_to_bf16_rne(acc[i][j][4 * q + 2]), f32_to_bf16_rne(acc[i][j][4 * q + 3])};
+          *reinterpret_cast<ushortx4*>(ep + ml * ROW_B + ((c ^ ((ml >> 1) & 7)) * 16) + 8 * h) = v;
+        }
+    }
+    constexpr int ROWS_PER_IT = 64 / CH;
+    const int er = lane / CH, ec = lane % CH;
+    OutT* cbase = C + (size_t)(tile_m * BM + wm * WTM) * N + tile_n * BN + wn * WTN + ec * 8;
+#pragma unroll
+    for (int it = 0; it < WTM / ROWS_PER_IT; it++) {
+      const int row = it * ROWS_PER_IT + er;
+      intx4 v = *reinterpret_cast<const intx4*>(ep + row * ROW_B + ((ec ^ ((row >> 1) & 7)) * 16));
+      *reinterpret_cast<intx4*>(cbase + (size_t)row * N) = v;
+    }
+  } else {
+    const int m0 = tile_m * BM + wm * WTM + r32;
+    const int n0 = tile_n * BN + wn * WTN + 4 * h;
+#pragma unroll
+    for (int j = 0; j < TM; j++) {
+      OutT* crow = C + (size_t)(m0 + j * 32) * N + n0;
+#pragma unroll
+      for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+          MxOut<OutT>::store4(crow + i * 32 + q * 8, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                              acc[i][j][4 * q + 3]);
+    }
   }
 }
 
@@ -210,6 +365,98 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_generic(const uint8_t* __restr
   }
 }
 
+// Skinny-M kernel (M <= 32): weight streaming, HBM bound.  One workgroup (8 waves) per 32 rows of B;
+// wave w owns 128-byte K segments w, w+8, ... of those rows (at most 4 per pass = 16 KiB of LDS per
+// wave).  Everything a wave needs for a pass is requested up front -- B codes by direct-to-LDS loads
+// (8 rows x 128 bytes per instruction, fully coalesced), A fragments and both scale sets straight into
+// registers -- so that the whole 34 MB problem is in flight at once; then 16 MFMAs per wave, a reduction
+// of the 8 partial 32x32 tiles through LDS, and one bf16 store.  Inside a 128-byte segment lane half h
+// takes chunks 4h..4h+3 (k-step s' -> chunk 4h+s'): any chunk order is valid as long as A, B and the
+// scale bytes agree, and this one makes a lane's scale bytes one aligned dword selected by op_sel.
+template <typename OutT>
+__global__ __launch_bounds__(512) void gemm_mxfp4_skinny(const uint8_t* __restrict__ A, const uint8_t* __restrict__ As,
+                                                         const uint8_t* __restrict__ B, const uint8_t* __restrict__ Bs,
+                                                         OutT* __restrict__ C, int M, int N, int K) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r32 = lane & 31, h = lane >> 5;
+  const int n0 = blockIdx.x * 32;
+  const int Kb = K >> 1, Ksc = K >> 5;
+  const int nseg = Kb >> 7;  // 128-byte segments per row
+  char* my = lds + wave * 16384;
+
+  floatx16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; r++) acc[r] = 0.f;
+
+  const int lrow = lane >> 3;
+  const bool m_ok = r32 < M;
+  for (int seg0 = 0; seg0 < nseg; seg0 += 32) {  // a pass covers 32 segments (4 per wave)
+    intx4 fa[4][4];
+    int sa[4], sb[4];
+    int cnt = 0;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      const int seg = seg0 + wave + 8 * q;
+      if (seg < nseg) {
+        cnt = q + 1;
+        // B codes: 32 rows x 128 bytes -> 4 wave-loads of 8 rows; chunk c of row r in slot c ^ ((r >> 1) & 7)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const int row = i * 8 + lrow;
+          const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+          load_lds_16B(B + (size_t)(n0 + row) * Kb + seg * 128 + chunk * 16, my + q * 4096 + i * 1024);
+        }
+        sb[q] = *reinterpret_cast<const int*>(Bs + (size_t)(n0 + r32) * Ksc + seg * 8 + 4 * h);
+        if (m_ok) {
+          sa[q] = *reinterpret_cast<const int*>(As + (size_t)r32 * Ksc + seg * 8 + 4 * h);
+#pragma unroll
+          for (int sp = 0; sp < 4; sp++)
+            fa[q][sp] = *reinterpret_cast<const intx4*>(A + (size_t)r32 * Kb + seg * 128 + (4 * h + sp) * 16);
+        } else {
+          sa[q] = 0x7f7f7f7f;
+#pragma unroll
+          for (int sp = 0; sp < 4; sp++) fa[q][sp] = intx4{0, 0, 0, 0};
+        }
+      }
+    }
+    wait_vmcnt0();
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      if (q < cnt) {
+#pragma unroll
+        for (int sp = 0; sp < 4; sp++) {
+          const int c = 4 * h + sp;
+          intx4 fb = *reinterpret_cast<const intx4*>(my + q * 4096 + r32 * 128 + ((c ^ ((r32 >> 1) & 7)) * 16));
+          intx8 av = {fb[0], fb[1], fb[2], fb[3], 0, 0, 0, 0};
+          intx8 bv = {fa[q][sp][0], fa[q][sp][1], fa[q][sp][2], fa[q][sp][3], 0, 0, 0, 0};
+          // MFMA "A" operand = B rows (n), "B" operand = A rows (m): acc[n][m]
+          if (sp == 0) acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc, 4, 4, 0, sb[q], 0, sa[q]);
+          if (sp == 1) acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc, 4, 4, 1, sb[q], 1, sa[q]);
+          if (sp == 2) acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc, 4, 4, 2, sb[q], 2, sa[q]);
+          if (sp == 3) acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc, 4, 4, 3, sb[q], 3, sa[q]);
+        }
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's LDS reads are done before the next pass overwrites
+  }
+
+  // reduce the 8 partial tiles: lane (m = r32, h) register r holds n = 8*(r/4) + 4h + r%4
+  __syncthreads();
+  float* red = reinterpret_cast<float*>(lds);  // [wave][n 32][m 32]
+#pragma unroll
+  for (int r = 0; r < 16; r++) red[(wave * 32 + 8 * (r >> 2) + 4 * h + (r & 3)) * 32 + r32] = acc[r];
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < 1024; idx += 512) {
+    const int m = idx >> 5, n = idx & 31;
+    float v = 0.f;
+#pragma unroll
+    for (int w = 0; w < 8; w++) v += red[(w * 32 + n) * 32 + m];
+    if (m < M) MxOut<OutT>::store1(C + (size_t)m * N + n0 + n, v);
+  }
+}
+
 // Exact software decode of the format, for checking the device against the closed form.
 __global__ __launch_bounds__(256) void mxfp4_dequant_kernel(const uint8_t* __restrict__ codes, const uint8_t* __restrict__ scales,
                                                             float* __restrict__ out, long long rows, int K) {
@@ -241,17 +488,18 @@ struct MxVariant {
 static const MxVariant kMxVariants[] = {
     {"tiled_256x256x256_w2x4", 256, 256},
     {"tiled_128x128x256_w2x2", 128, 128},
+    {"skinny_m32_n32_w8", 32, 32},
     {"generic_32x128", 32, 128},
 };
 constexpr int kNumMxVariants = sizeof(kMxVariants) / sizeof(kMxVariants[0]);
 int mxfp4_variant_count() { return kNumMxVariants; }
 const char* mxfp4_variant_name(int i) { return (i >= 0 && i < kNumMxVariants) ? kMxVariants[i].name : nullptr; }
 
-template <int BM, int BN, int WM, int WN, typename OutT>
+template <int BM, int BN, int WM, int WN, typename OutT, bool SCALES_LDS>
 static int launch_mx_tiled(const void* a, const void* as, const void* b, const void* bs, void* c, int M, int N, int K,
                            hipStream_t stream) {
-  auto kern = gemm_mxfp4_tiled<BM, BN, WM, WN, OutT>;
-  constexpr int lds_bytes = 2 * (BM + BN) * 128;
+  auto kern = gemm_mxfp4_tiled<BM, BN, WM, WN, OutT, SCALES_LDS>;
+  constexpr int lds_bytes = 2 * (BM + BN) * 128 + (SCALES_LDS ? 2 * (BM + BN) * 32 : 0);
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -273,8 +521,29 @@ template <typename OutT>
 static int launch_mx(int variant, const void* a, const void* as, const void* b, const void* bs, void* c, int M, int N, int K,
                      hipStream_t stream) {
   switch (variant) {
-    case 0: return launch_mx_tiled<256, 256, 2, 4, OutT>(a, as, b, bs, c, M, N, K, stream);
-    case 1: return launch_mx_tiled<128, 128, 2, 2, OutT>(a, as, b, bs, c, M, N, K, stream);
+    case 0:
+      if (K % 1024 == 0) return launch_mx_tiled<256, 256, 2, 4, OutT, true>(a, as, b, bs, c, M, N, K, stream);
+      return launch_mx_tiled<256, 256, 2, 4, OutT, false>(a, as, b, bs, c, M, N, K, stream);
+    case 1:
+      if (K % 1024 == 0) return launch_mx_tiled<128, 128, 2, 2, OutT, true>(a, as, b, bs, c, M, N, K, stream);
+      return launch_mx_tiled<128, 128, 2, 2, OutT, false>(a, as, b, bs, c, M, N, K, stream);
+    case 2: {
+      auto kern = gemm_mxfp4_skinny<OutT>;
+      constexpr int lds_bytes = 8 * 16384;
+      static bool attr_set = false;
+      if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+        if (e != hipSuccess) {
+          set_error("hipFuncSetAttribute(gemm_mxfp4_skinny): %s", hipGetErrorString(e));
+          return (int)e;
+        }
+        attr_set = true;
+      }
+      dim3 grid(N / 32), block(512);
+      hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const uint8_t*)a, (const uint8_t*)as, (const uint8_t*)b,
+                         (const uint8_t*)bs, (OutT*)c, M, N, K);
+      return check_launch("gemm_mxfp4_skinny", grid, block, lds_bytes);
+    }
     default: {
       dim3 grid((N + 127) / 128, (M + 31) / 32), block(256);
       hipLaunchKernelGGL(gemm_mxfp4_generic<OutT>, grid, block, 0, stream, (const uint8_t*)a, (const uint8_t*)as,
@@ -291,7 +560,7 @@ using namespace mi355;
 extern "C" int mi355_mxfp4_gemm(const void* a, const void* a_scale, const void* b, const void* b_scale, void* c, int64_t M,
                                 int64_t N, int64_t K, int out_dtype, int variant, void* stream) {
   if (!a || !a_scale || !b || !b_scale || !c) return fail(-MI355_E_NULL, "mxfp4_gemm: null pointer");
-  if (M <= 0 || N <= 0 || K <= 0 || M > (1 << 30) || N > (1 << 30) || K > (1 << 30))
+  if (M <= 0 || N <= 0 || K <= 0 || M > (1 << 30) || N > (1 << 30) || K > (1 << 28))
     return fail(-MI355_E_SHAPE, "mxfp4_gemm: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
   if (K % 32 != 0) return fail(-MI355_E_SHAPE, "mxfp4_gemm: K=%lld must be a multiple of the 32-element scale block", (long long)K);
   if (out_dtype != MI355_BF16 && out_dtype != MI355_F32)
@@ -300,17 +569,22 @@ extern "C" int mi355_mxfp4_gemm(const void* a, const void* a_scale, const void* 
   if (!aligned16(a) || !aligned16(b) || !aligned16(c))
     return fail(-MI355_E_ALIGN, "mxfp4_gemm: a, b, c must be 16-byte aligned");
   const bool sc_al = ((reinterpret_cast<uintptr_t>(a_scale) | reinterpret_cast<uintptr_t>(b_scale)) & 7u) == 0;
+  const bool sc_al4 = ((reinterpret_cast<uintptr_t>(a_scale) | reinterpret_cast<uintptr_t>(b_scale)) & 3u) == 0;
   auto fits = [&](int v) {
     if (v == kNumMxVariants - 1) return true;
+    if (v == 2) return sc_al4 && M <= 32 && N % 32 == 0 && K % 256 == 0;  // skinny: whole 128-byte segments
     return sc_al && M % kMxVariants[v].bm == 0 && N % kMxVariants[v].bn == 0 && K % 256 == 0;
   };
   if (variant < 0) {
-    if (fits(0) && (M / 256) * (N / 256) >= 128) variant = 0;
+    // The 256x256 tile pays off only with a long K loop (its prologue/epilogue is amortised over
+    // K/256 slabs); M <= 32 is weight streaming and has its own kernel.
+    if (fits(2)) variant = 2;
+    else if (fits(0) && (M / 256) * (N / 256) >= 256 && K >= 16384) variant = 0;
     else if (fits(1)) variant = 1;
     else variant = kNumMxVariants - 1;
   } else if (!fits(variant)) {
-    return fail(-MI355_E_SHAPE, "mxfp4_gemm: variant %s needs M%%%d==0, N%%%d==0, K%%256==0 and 8-byte aligned scales",
-                kMxVariants[variant].name, kMxVariants[variant].bm, kMxVariants[variant].bn);
+    return fail(-MI355_E_SHAPE, "mxfp4_gemm: variant %s does not fit M=%lld N=%lld K=%lld (tile %dx%d, K%%256==0, aligned scales)",
+                kMxVariants[variant].name, (long long)M, (long long)N, (long long)K, kMxVariants[variant].bm, kMxVariants[variant].bn);
   }
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (out_dtype == MI355_F32) return launch_mx<float>(variant, a, a_scale, b, b_scale, c, (int)M, (int)N, (int)K, s);

@@ -43,7 +43,7 @@ def test_dequant_random_bit_exact(dev):
     assert np.array_equal(out.view(np.uint32), om.mxfp4_dequant_ref(a, asc).view(np.uint32))
 
 
-@pytest.mark.parametrize("variant", [-1, 0, 1, 2])
+@pytest.mark.parametrize("variant", [-1, 0, 1, 3])
 def test_mxfp4_gemm_variants(dev, variant):
     import iree_turbine_amd  # noqa: F401
     from oracle import inputs, mxfp4 as om
@@ -71,6 +71,23 @@ def test_mxfp4_gemm_ragged(dev, shape):
     ref = om.mxfp4_gemm_ref(a, asc, b, bsc)
     c = torch.ops.mi355.mxfp4_gemm(a.to(dev), asc.to(dev), b.to(dev), bsc.to(dev), "float32", -1).cpu()
     assert _rel_err(c, ref) < 1e-5
+
+
+@pytest.mark.parametrize("shape", [(32, 256, 512), (1, 64, 256), (7, 96, 2048), (32, 8192, 8192), (20, 160, 16384), (32, 64, 8192 + 256)])
+@pytest.mark.parametrize("variant", [2, 3])
+def test_mxfp4_skinny_vs_generic(dev, shape, variant):
+    """The weight-streaming kernel (variant 2) and the any-shape kernel (variant 3) on skinny shapes."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs, mxfp4 as om
+
+    M, N, K = shape
+    announce(f"mxfp4_gemm skinny {shape} variant={variant}")
+    a, asc, b, bsc = inputs.mxfp4_inputs(M, N, K, seed=17)
+    ref = om.mxfp4_gemm_ref(a, asc, b, bsc)
+    c = torch.ops.mi355.mxfp4_gemm(a.to(dev), asc.to(dev), b.to(dev), bsc.to(dev), "float32", variant).cpu()
+    assert _rel_err(c, ref) < 1e-5
+    c16 = torch.ops.mi355.mxfp4_gemm(a.to(dev), asc.to(dev), b.to(dev), bsc.to(dev), "bfloat16", variant).cpu()
+    assert torch.equal(c16, c.bfloat16())
 
 
 def test_mxfp4_one_hot_nibble_order_and_scale_block(dev):
