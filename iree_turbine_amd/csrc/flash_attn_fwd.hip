@@ -19,6 +19,7 @@
 // global side of the direct-to-LDS loads.
 #include "common.hpp"
 #include <math.h>
+#include <type_traits>
 
 namespace mi355 {
 
@@ -207,9 +208,218 @@ __global__ __launch_bounds__(256) void fa_fwd_d128(const half_t* __restrict__ Q,
   }
 }
 
-static const char* kFaVariants[] = {"d128_bm128_bn64_w4"};
-int fa_variant_count() { return 1; }
-const char* fa_variant_name(int i) { return i == 0 ? kFaVariants[0] : nullptr; }
+// Software-pipelined form.  Same tiling and register layout, but the score MFMAs run one key tile
+// ahead of the softmax: in trip j a wave issues S^T(j+1) = K(j+1) . Q^T, exponentiates the scores of
+// tile j on the VALU while those MFMAs execute, then issues O^T += V(j)^T . P(j)^T.  K and V sit in
+// separate two-deep LDS rings, K one tile ahead of V; the trip is written twice (scores ping-pong
+// between two register sets, ring slots become compile-time constants) so nothing is copied.
+// The running maximum is only raised -- and O rescaled -- when some query's maximum grew by more than
+// 2^8; until then exponentials are taken against the stale maximum (they stay below 2^8, and O / l is
+// the same quotient), which keeps the 64-register rescale off the common path.
+// V swizzle: chunk c of row r -> slot c ^ (4 * (r & 3)), which keeps the four 64-byte row pieces that a
+// half-wave transpose read touches on distinct banks (measured conflict-free; c ^ 2(r & 7) is not).
+template <bool CAUSAL>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void fa_fwd_d128_pipe(
+    const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V, half_t* __restrict__ O, int BH,
+    int Sq, int Sk, float scale_log2e, int q_blocks) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  constexpr int TILE_B = FA_BLOCK_N * 256;  // bytes of one K or V tile
+  constexpr int VBUF = 2 * TILE_B;          // K ring at 0, V ring behind it
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r32 = lane & 31, h = lane >> 5;
+
+  int bh, qb;
+  {
+    const int pid = blockIdx.x;
+    if ((BH & 7) == 0) {
+      const int xcd = pid & 7, loc = pid >> 3;
+      bh = (loc / q_blocks) * 8 + xcd;
+      qb = loc % q_blocks;
+    } else {
+      bh = pid / q_blocks;
+      qb = pid % q_blocks;
+    }
+    if (CAUSAL) qb = q_blocks - 1 - qb;
+  }
+  const int causal_off = Sk - Sq;
+  const int q0 = qb * FA_BLOCK_M;
+  const int wq0 = q0 + wave * 32;
+  const int q_row = wq0 + r32;
+  const bool q_ok = q_row < Sq;
+
+  const half_t* Qb = Q + (size_t)bh * Sq * 128;
+  const half_t* Kb = K + (size_t)bh * Sk * 128;
+  const half_t* Vb = V + (size_t)bh * Sk * 128;
+  half_t* Ob = O + (size_t)bh * Sq * 128;
+
+  int k_end = Sk;
+  if (CAUSAL) {
+    int last_q = q0 + FA_BLOCK_M - 1;
+    if (last_q > Sq - 1) last_q = Sq - 1;
+    int lim = last_q + causal_off + 1;
+    if (lim < k_end) k_end = lim;
+  }
+  const int n_tiles = k_end > 0 ? (k_end + FA_BLOCK_N - 1) / FA_BLOCK_N : 0;
+
+  half8 qf[8];
+#pragma unroll
+  for (int ks = 0; ks < 8; ks++) {
+    if (q_ok) {
+      qf[ks] = *reinterpret_cast<const half8*>(Qb + (size_t)q_row * 128 + ks * 16 + h * 8);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; e++) qf[ks][e] = (half_t)0;
+    }
+  }
+
+  const int lrow = lane >> 4, lslot = lane & 15;
+  const int k_chunk = lslot ^ (wave * 4 + lrow);
+  const int v_chunk = lslot ^ (4 * lrow);
+  auto issue_kv = [&](const half_t* base, int chunk, int tile, int lds_off) {
+    char* dst = lds + lds_off + wave * 1024;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      int row = tile * FA_BLOCK_N + (wave + 4 * i) * 4 + lrow;
+      if (row > Sk - 1) row = Sk - 1;  // clamp: tail rows are masked out of the softmax
+      load_lds_16B(base + (size_t)row * 128 + chunk * 8, dst + i * 4096);
+    }
+  };
+
+  const int k_base = r32 * 256 + ((h ^ (lane & 15)) * 16);
+  const int i16 = lane & 15, g16 = lane >> 4;
+  const int v_row = 4 * (g16 >> 1) + (i16 >> 2);
+  const int v_base = VBUF + v_row * 256 + (i16 >> 2) * 64 + (2 * (g16 & 1) + ((i16 & 3) >> 1)) * 16 + (i16 & 1) * 8;
+
+  floatx16 oacc[4];
+#pragma unroll
+  for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) oacc[dt][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+  constexpr float kRescaleThreshold = 8.f;  // log2 units of the final exponent
+
+  auto wave_active = [&](int tile) { return !CAUSAL || (tile * FA_BLOCK_N <= wq0 + 31 + causal_off); };
+
+  // S^T = K(slot) . Q^T, 16 MFMAs
+  auto scores = [&](int koff, floatx16* s) {
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) s[t][r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < 8; ks++) {
+        half8 kf = *reinterpret_cast<const half8*>(lds + koff + t * 8192 + (k_base ^ (ks * 32)));
+        s[t] = mfma_32x32x16(kf, qf[ks], s[t]);
+      }
+    }
+  };
+
+  // softmax of tile `tile` (scores in s) and O^T += V(slot)^T . P^T
+  auto softmax_pv = [&](auto masked_tag, int tile, int voff, floatx16* s) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
+    if (MASKED) {
+      const int key0 = tile * FA_BLOCK_N;
+      const bool need_mask = (CAUSAL && (key0 + FA_BLOCK_N - 1 > wq0 + causal_off)) || (key0 + FA_BLOCK_N > Sk);
+      if (need_mask) {
+        const int lim = CAUSAL ? (q_row + causal_off < Sk - 1 ? q_row + causal_off : Sk - 1) : Sk - 1;
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int key = key0 + 32 * t + 8 * (r >> 2) + 4 * h + (r & 3);
+            if (key > lim) s[t][r] = -INFINITY;
+          }
+      }
+    }
+    float mx = s[0][0];
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[t][r]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    // raise the running maximum only when it is stale by more than the threshold for some query
+    const float grow = (mx - m_run) * scale_log2e;  // +inf the first time, NaN only for -inf - -inf
+    if (__builtin_amdgcn_ballot_w64(grow > kRescaleThreshold) != 0) {
+      const float m_new = fmaxf(m_run, mx);
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * scale_log2e);
+      l_run *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) oacc[dt][r] *= alpha;
+      m_run = m_new;
+    }
+    const float mc = (m_run == -INFINITY ? 0.f : m_run) * scale_log2e;
+    half8 pf[4];
+    float psum = 0.f;
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const float p = __builtin_amdgcn_exp2f(s[t][r] * scale_log2e - mc);
+        psum += p;
+        pf[t * 2 + (r >> 3)][r & 7] = (half_t)p;
+      }
+    l_run += psum;
+#pragma unroll
+    for (int t16 = 0; t16 < 4; t16++) {
+#pragma unroll
+      for (int dt = 0; dt < 4; dt++) {
+        const char* va = lds + voff + t16 * 4096 + (v_base ^ (dt * 64));
+        half4 lo = lds_read_tr16(va);
+        half4 hi = lds_read_tr16(va + 2048);
+        half8 vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        oacc[dt] = mfma_32x32x16(vf, pf[t16], oacc[dt]);
+      }
+    }
+  };
+
+  floatx16 sa[2], sb[2];
+  if (n_tiles > 0) {
+    issue_kv(Kb, k_chunk, 0, 0);
+    issue_kv(Vb, v_chunk, 0, VBUF);
+    if (n_tiles > 1) issue_kv(Kb, k_chunk, 1, TILE_B);
+    wait_vmcnt0();
+    __syncthreads();
+    if (wave_active(0)) scores(0, sa);
+  }
+
+  // trip j (PAR = j & 1): loads for K(j+2) and V(j+1); scores of tile j+1; softmax + PV of tile j
+  auto trip = [&](auto par_tag, int j, floatx16* s_cur, floatx16* s_next) {
+    constexpr int PAR = decltype(par_tag)::value;
+    constexpr int K_CUR = PAR * TILE_B, K_NEXT = (1 - PAR) * TILE_B, V_CUR = PAR * TILE_B, V_NEXT = VBUF + (1 - PAR) * TILE_B;
+    if (j + 2 < n_tiles) issue_kv(Kb, k_chunk, j + 2, K_CUR);
+    if (j + 1 < n_tiles) issue_kv(Vb, v_chunk, j + 1, V_NEXT);
+    if (j + 1 < n_tiles && wave_active(j + 1)) scores(K_NEXT, s_next);
+    if (wave_active(j)) softmax_pv(std::true_type{}, j, V_CUR, s_cur);
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+  };
+  for (int j = 0; j < n_tiles; j += 2) {
+    trip(std::integral_constant<int, 0>{}, j, sa, sb);
+    if (j + 1 < n_tiles) trip(std::integral_constant<int, 1>{}, j + 1, sb, sa);
+  }
+
+  const float l_tot = l_run + __shfl_xor(l_run, 32);
+  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  if (q_ok) {
+    half_t* orow = Ob + (size_t)q_row * 128 + 4 * h;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        half4 v = {(half_t)(oacc[dt][4 * q] * inv), (half_t)(oacc[dt][4 * q + 1] * inv), (half_t)(oacc[dt][4 * q + 2] * inv),
+                   (half_t)(oacc[dt][4 * q + 3] * inv)};
+        *reinterpret_cast<half4*>(orow + dt * 32 + q * 8) = v;
+      }
+  }
+}
+
+static const char* kFaVariants[] = {"d128_bm128_bn64_w4_pipelined", "d128_bm128_bn64_w4"};
+int fa_variant_count() { return 2; }
+const char* fa_variant_name(int i) { return (i >= 0 && i < 2) ? kFaVariants[i] : nullptr; }
 
 }  // namespace mi355
 
@@ -224,31 +434,31 @@ extern "C" int mi355_flash_attn_fwd(const void* q, const void* k, const void* v,
                 (long long)Sq, (long long)Sk);
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o))
     return fail(-MI355_E_ALIGN, "flash_attn_fwd: q, k, v, o must be 16-byte aligned");
-  if (variant > 0) return fail(-MI355_E_DTYPE, "flash_attn_fwd: variant %d out of range", variant);
+  if (variant > 1) return fail(-MI355_E_DTYPE, "flash_attn_fwd: variant %d out of range", variant);
   if (!(scale > 0.f) || !isfinite(scale)) return fail(-MI355_E_SHAPE, "flash_attn_fwd: scale must be positive and finite");
   const int BH = (int)(B * H);
   const int q_blocks = (int)((Sq + FA_BLOCK_M - 1) / FA_BLOCK_M);
   const int lds_bytes = 2 * FA_STAGE;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(fa_fwd_d128<true>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(fa_fwd_d128<false>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e1 != hipSuccess || e2 != hipSuccess) {
-      set_error("hipFuncSetAttribute(fa_fwd_d128): %s", hipGetErrorString(e1 != hipSuccess ? e1 : e2));
-      return (int)(e1 != hipSuccess ? e1 : e2);
+    const void* kernels[4] = {reinterpret_cast<const void*>(fa_fwd_d128<true>), reinterpret_cast<const void*>(fa_fwd_d128<false>),
+                              reinterpret_cast<const void*>(fa_fwd_d128_pipe<true>),
+                              reinterpret_cast<const void*>(fa_fwd_d128_pipe<false>)};
+    for (const void* kp : kernels) {
+      hipError_t e = hipFuncSetAttribute(kp, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+      if (e != hipSuccess) {
+        set_error("hipFuncSetAttribute(fa_fwd_d128): %s", hipGetErrorString(e));
+        return (int)e;
+      }
     }
     attr_set = true;
   }
   const float scale_log2e = scale * 1.4426950408889634f;
   dim3 grid(BH * q_blocks), block(256);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  if (is_causal)
-    hipLaunchKernelGGL(fa_fwd_d128<true>, grid, block, lds_bytes, s, (const half_t*)q, (const half_t*)k, (const half_t*)v,
-                       (half_t*)o, BH, (int)Sq, (int)Sk, scale_log2e, q_blocks);
-  else
-    hipLaunchKernelGGL(fa_fwd_d128<false>, grid, block, lds_bytes, s, (const half_t*)q, (const half_t*)k, (const half_t*)v,
-                       (half_t*)o, BH, (int)Sq, (int)Sk, scale_log2e, q_blocks);
-  return check_launch("fa_fwd_d128", grid, block, lds_bytes);
+  auto kern = variant == 1 ? (is_causal ? fa_fwd_d128<true> : fa_fwd_d128<false>)
+                           : (is_causal ? fa_fwd_d128_pipe<true> : fa_fwd_d128_pipe<false>);
+  hipLaunchKernelGGL(kern, grid, block, lds_bytes, s, (const half_t*)q, (const half_t*)k, (const half_t*)v, (half_t*)o, BH,
+                     (int)Sq, (int)Sk, scale_log2e, q_blocks);
+  return check_launch(variant == 1 ? "fa_fwd_d128" : "fa_fwd_d128_pipe", grid, block, lds_bytes);
 }

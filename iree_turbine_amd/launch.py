@@ -43,7 +43,7 @@ def gemm_nt_out(a: Tensor, b: Tensor, c: Tensor, variant: int = -1) -> Tensor:
     return c
 
 
-def flash_attn_fwd_out(q: Tensor, k: Tensor, v: Tensor, o: Tensor, is_causal: bool, scale: float) -> Tensor:
+def flash_attn_fwd_out(q: Tensor, k: Tensor, v: Tensor, o: Tensor, is_causal: bool, scale: float, variant: int = -1) -> Tensor:
     dev = _dev(q, k, v, o)
     q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
     _contig_out(o, "flash_attn_fwd")
@@ -55,7 +55,7 @@ def flash_attn_fwd_out(q: Tensor, k: Tensor, v: Tensor, o: Tensor, is_causal: bo
         scale = 1.0 / math.sqrt(D)
     with torch.cuda.device(dev):
         rc = _lib.load().mi355_flash_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), B, H, Sq, Sk, D, scale,
-                                              int(bool(is_causal)), -1, _lib.current_stream_ptr(dev))
+                                              int(bool(is_causal)), variant, _lib.current_stream_ptr(dev))
     _lib.check(rc, f"flash_attn_fwd B={B} H={H} Sq={Sq} Sk={Sk} D={D} causal={is_causal}")
     return o
 
