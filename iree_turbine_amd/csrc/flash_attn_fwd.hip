@@ -316,7 +316,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   };
 
   // softmax of tile `tile` (scores in s) and O^T += V(slot)^T . P^T
-  auto softmax_pv = [&](auto masked_tag, int tile, int voff, floatx16* s) {
+  auto softmax_pv = [&](auto masked_tag, int tile, int voff, floatx16* s, int koff_next, floatx16* s_next) {
     constexpr bool MASKED = decltype(masked_tag)::value;
     if (MASKED) {
       const int key0 = tile * FA_BLOCK_N;
@@ -354,6 +354,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const float mc = (m_run == -INFINITY ? 0.f : m_run) * scale_log2e;
     half8 pf[4];
     float psum = 0.f;
+    // Scores of the next tile and exponentials of this one in one straight-line block: a wave issues in
+    // order, so only VALU work placed between two MFMAs runs while the first occupies the matrix pipe.
+    // (Past the last tile the scores are computed from stale LDS bytes and never used.)
+    __builtin_amdgcn_sched_barrier(0);
+    scores(koff_next, s_next);
 #pragma unroll
     for (int t = 0; t < 2; t++)
 #pragma unroll
@@ -362,17 +367,39 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         psum += p;
         pf[t * 2 + (r >> 3)][r & 7] = (half_t)p;
       }
+    // order: 3 K fragment reads up front, then per score MFMA one more read and the VALU work of two
+    // scores (fma, exp, add, half a cvt_pk each) -- a fragment is requested two MFMAs before its use
+    __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+#pragma unroll
+    for (int i = 0; i < 13; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 3; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
     l_run += psum;
+    // O^T += V^T P^T: 16 MFMAs, each V^T fragment (two transpose reads) requested two MFMAs ahead.
+    // The order is pinned step by step (scheduling groups are not used here: hoisting the transpose
+    // reads with sched_group_barrier produced wrong results).
+    auto vr = [&](int i) {  // i = t16*4 + dt
+      const char* va = lds + voff + (i >> 2) * 4096 + (v_base ^ ((i & 3) * 64));
+      half4 lo = lds_read_tr16(va);
+      half4 hi = lds_read_tr16(va + 2048);
+      return half8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    };
+    half8 vf[3];
+    vf[0] = vr(0);
+    vf[1] = vr(1);
 #pragma unroll
-    for (int t16 = 0; t16 < 4; t16++) {
-#pragma unroll
-      for (int dt = 0; dt < 4; dt++) {
-        const char* va = lds + voff + t16 * 4096 + (v_base ^ (dt * 64));
-        half4 lo = lds_read_tr16(va);
-        half4 hi = lds_read_tr16(va + 2048);
-        half8 vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        oacc[dt] = mfma_32x32x16(vf, pf[t16], oacc[dt]);
-      }
+    for (int i = 0; i < 16; i++) {
+      if (i + 2 < 16) vf[(i + 2) % 3] = vr(i + 2);
+      oacc[i & 3] = mfma_32x32x16(vf[i % 3], pf[i >> 2], oacc[i & 3]);
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
 
@@ -384,6 +411,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     wait_vmcnt0();
     __syncthreads();
     if (wave_active(0)) scores(0, sa);
+    // trip 0 overwrites the K(0) slot with K(2): every wave must have read its K(0) fragments first
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __syncthreads();
   }
 
   // trip j (PAR = j & 1): loads for K(j+2) and V(j+1); scores of tile j+1; softmax + PV of tile j
@@ -392,8 +422,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     constexpr int K_CUR = PAR * TILE_B, K_NEXT = (1 - PAR) * TILE_B, V_CUR = PAR * TILE_B, V_NEXT = VBUF + (1 - PAR) * TILE_B;
     if (j + 2 < n_tiles) issue_kv(Kb, k_chunk, j + 2, K_CUR);
     if (j + 1 < n_tiles) issue_kv(Vb, v_chunk, j + 1, V_NEXT);
-    if (j + 1 < n_tiles && wave_active(j + 1)) scores(K_NEXT, s_next);
-    if (wave_active(j)) softmax_pv(std::true_type{}, j, V_CUR, s_cur);
+    if (wave_active(j)) softmax_pv(std::true_type{}, j, V_CUR, s_cur, K_NEXT, s_next);  // idle from here on otherwise
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
   };

@@ -90,6 +90,28 @@ def test_attention_full_size(dev, causal):
     torch.testing.assert_close(o.float(), lib, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_full_size_repeatable(dev, causal):
+    """Every kernel variant gives bit-identical output on repeated launches at full size, and the variants
+    agree with each other: an unsynchronised LDS slot reuse shows up here as run-to-run differences."""
+    import iree_turbine_amd as ita
+    from oracle import inputs
+
+    announce(f"attention repeatability causal={causal}")
+    q, k, v = [t.to(dev) for t in inputs.attention_inputs(2, 32, 4096, 128)]
+    outs = []
+    for variant in range(len(ita._lib.variants("flash_attn_fwd"))):
+        first = torch.empty_like(q)
+        ita.launch.flash_attn_fwd_out(q, k, v, first, causal, 0.0, variant)
+        for _ in range(3):
+            again = torch.empty_like(q)
+            ita.launch.flash_attn_fwd_out(q, k, v, again, causal, 0.0, variant)
+            assert torch.equal(first, again), f"variant {variant} differs between launches"
+        outs.append(first.float())
+    for other in outs[1:]:
+        torch.testing.assert_close(outs[0], other, rtol=RTOL, atol=ATOL)
+
+
 def test_attention_contract_errors(dev):
     import iree_turbine_amd  # noqa: F401
 

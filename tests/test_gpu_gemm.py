@@ -124,3 +124,22 @@ def test_gemm_full_size_properties(dev, shape):
     c2 = torch.ops.mi355.gemm_nt(ad * 2, bd, "float32", -1)
     assert torch.equal(c2, c32 * 2)
     assert torch.equal(c32.half(), c)  # the fp16 epilogue is round-to-nearest-even of the fp32 result
+
+
+@pytest.mark.parametrize("shape", [(8192, 8192, 8192), (2048, 10240, 8192)])
+def test_gemm_full_size_repeatable(dev, shape):
+    """Whole-matrix checks at benchmark sizes: every tiled variant is bit-identical across launches (an
+    unsynchronised LDS stage reuse would differ from run to run) and agrees with the simple generic kernel."""
+    import iree_turbine_amd as ita
+    from oracle import inputs
+
+    M, N, K = shape
+    announce(f"gemm repeatability {shape}")
+    a, b = [t.to(dev) for t in inputs.gemm_inputs(M, N, K)]
+    names = ita._lib.variants("gemm_f16_nt")
+    generic = torch.ops.mi355.gemm_nt(a, b, "float32", len(names) - 1)
+    for variant in range(len(names) - 1):
+        first = torch.ops.mi355.gemm_nt(a, b, "float32", variant)
+        for _ in range(2):
+            assert torch.equal(first, torch.ops.mi355.gemm_nt(a, b, "float32", variant)), names[variant]
+        torch.testing.assert_close(first, generic, rtol=1e-3, atol=1e-3)

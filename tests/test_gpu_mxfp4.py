@@ -150,6 +150,31 @@ def test_mxfp4_full_size(dev, shape):
     assert _rel_err(c[:, cols.to(dev)].float().cpu(), ref_c) < REL
 
 
+@pytest.mark.parametrize("shape", [(4096, 8192, 8192), (32, 8192, 8192)])
+def test_mxfp4_full_size_repeatable(dev, shape):
+    """Whole-matrix checks at benchmark sizes: each variant that accepts the shape is bit-identical across
+    launches and agrees with the simple generic kernel."""
+    import iree_turbine_amd as ita
+    from oracle import inputs
+
+    M, N, K = shape
+    announce(f"mxfp4 repeatability {shape}")
+    a, asc, b, bsc = [t.to(dev) for t in inputs.mxfp4_inputs(M, N, K)]
+    names = ita._lib.variants("mxfp4_gemm")
+    generic = torch.ops.mi355.mxfp4_gemm(a, asc, b, bsc, "float32", len(names) - 1)
+    ran = 0
+    for variant in range(len(names) - 1):
+        try:
+            first = torch.ops.mi355.mxfp4_gemm(a, asc, b, bsc, "float32", variant)
+        except ValueError:
+            continue  # the variant's tile does not divide this shape
+        ran += 1
+        for _ in range(2):
+            assert torch.equal(first, torch.ops.mi355.mxfp4_gemm(a, asc, b, bsc, "float32", variant)), names[variant]
+        assert _rel_err(first, generic) < 1e-5, names[variant]
+    assert ran >= 1
+
+
 def test_mxfp4_contract_errors(dev):
     import iree_turbine_amd  # noqa: F401
 
