@@ -9,9 +9,10 @@ already resident in HBM.  The headline workload is the fp16 NT GEMM 8192^3 with 
 path (flash-attention prefill, paged decode, MXFP4 GEMM, remaining GEMM shapes) are measured in
 the same run and reported under "others".  Prints exactly one JSON line.
 
-Timing: W untimed warm-up steps, then K steps bracketed by torch.cuda.synchronize() on both sides
-(wall clock -> value / ms_per_step) and, inside the same region, a HIP event pair on the launch
-stream around every step (-> the kernel's average duration used for the roofline figure).
+Timing: W untimed warm-up steps, then exactly K steps, replayed as one HIP graph, bracketed by
+torch.cuda.synchronize() on both sides (wall clock -> value / ms_per_step) and, inside the same
+region, by a HIP event pair on the launch stream (-> the average device time per launch used for the
+roofline figure).
 """
 
 from __future__ import annotations
@@ -35,18 +36,54 @@ METRIC = "TFLOP/s & %MFMA peak (f16 GEMM, causal FA, MXFP4 GEMM); decode HBM GB/
 # HBM bytes per launch measured with `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` (KiB per
 # dispatch, scaled by what the same counters read for a copy kernel of known size); filled in from
 # the summaries kept under profiles/.  None = not measured.
-MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {}
-
-
-def _events(n):
-    return [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
+    "gemm_8192": 1.747e9,              # 1538 MiB read + 128 MiB written: each of the 8 XCD L2s fetches its own copy of
+                                       # the panels its 4x8 block of output tiles needs (12 panels x 4 MiB x 4 rounds x 8)
+    "gemm_4096": 2.350e8,
+    "gemm_2048x10240x8192": 1.027e9,
+    "gemm_2048x57344x8192": 3.056e9,
+    "fa_causal": 2.700e8,
+    "fa_noncausal": 2.686e8,
+    "decode": 1.178e9,
+    "mxfp4_4096x8192x8192": 4.429e8,
+    "mxfp4_32x8192x8192": 3.748e7,
+}
 
 
 def time_steps(fn, steps: int, warmup: int):
-    """Returns (wall ms per step, mean device ms per launch, min device ms)."""
+    """Returns (wall ms per step, device ms per launch, how the steps were launched).
+
+    The K timed steps are captured once into a HIP graph and replayed, so that launches shorter than the
+    host's per-call cost (a 15 us kernel behind a 40 us Python dispatch) are timed back to back on the
+    device; the replay is bracketed by synchronize() for the wall clock and by one HIP event pair on the
+    launch stream for the device time.  If capture fails the same K steps run eagerly, one event pair each.
+    """
     for _ in range(warmup):
         fn()
-    ev = _events(steps)
+    torch.cuda.synchronize()
+    graph = None
+    try:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(steps):
+                fn()
+        graph.replay()  # untimed: first replay uploads the graph
+        torch.cuda.synchronize()
+    except Exception as exc:  # capture unsupported for this op: time eager launches
+        print(f"bench.py: graph capture failed ({type(exc).__name__}: {exc}); timing eager launches", file=sys.stderr)
+        graph = None
+        torch.cuda.synchronize()
+    if graph is not None:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record()
+        graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+        return wall_ms, e0.elapsed_time(e1) / steps, "hip_graph"
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for s, e in ev:
@@ -55,8 +92,7 @@ def time_steps(fn, steps: int, warmup: int):
         e.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    dev = [s.elapsed_time(e) for s, e in ev]
-    return wall_ms, sum(dev) / len(dev), min(dev)
+    return wall_ms, sum(s.elapsed_time(e) for s, e in ev) / steps, "eager"
 
 
 # ---- workloads --------------------------------------------------------------------------------
@@ -135,6 +171,20 @@ def wl_mxfp4(M, N, K):
     return build
 
 
+def wl_copy(nbytes=1 << 30):
+    """Plain device copy of a known size: the calibration point for the HBM traffic counters."""
+    def build(dev):
+        src = torch.full((nbytes // 2,), 1.0, dtype=torch.float16, device=dev)
+        dst = torch.empty_like(src)
+        return {
+            "fn": lambda: dst.copy_(src),
+            "work": 2.0 * nbytes, "bytes": 2.0 * nbytes, "bound": "hbm", "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "dtype": "f16", "cpu": lambda: cpu_copy(nbytes),
+            "config": {"workload": f"copy_{nbytes >> 20}MiB", "bytes_read": nbytes, "bytes_written": nbytes},
+        }
+    return build
+
+
 WORKLOADS = {
     "gemm_8192": wl_gemm(8192, 8192, 8192),
     "gemm_4096": wl_gemm(4096, 4096, 4096),
@@ -147,6 +197,8 @@ WORKLOADS = {
     "mxfp4_4096x8192x8192": wl_mxfp4(4096, 8192, 8192),
     "mxfp4_32x8192x8192": wl_mxfp4(32, 8192, 8192),
 }
+CALIBRATION = {"copy_1GiB": wl_copy()}  # not part of the path: run only when named with --workload
+WORKLOADS_ALL = {**WORKLOADS, **CALIBRATION}
 HEADLINE = "gemm_8192"
 
 
@@ -160,6 +212,13 @@ def _time_cpu(fn, reps=3):
         fn()
         ts.append(time.perf_counter() - t0)
     return min(ts)
+
+
+def cpu_copy(nbytes):
+    src = torch.ones(nbytes // 8, dtype=torch.float16)
+    dst = torch.empty_like(src)
+    t = _time_cpu(lambda: dst.copy_(src))
+    return {"value": 2.0 * (nbytes // 4) / t / 1e9, "unit": "GB/s", "sample": f"torch CPU copy of {nbytes >> 22} MiB"}
 
 
 def cpu_gemm(a, b, M, N, K):
@@ -200,8 +259,8 @@ def cpu_mxfp4(a, asc, b, bsc, M, N, K):
 # ---- driver -------------------------------------------------------------------------------------
 
 def measure(name: str, dev, steps: int, warmup: int, with_cpu: bool):
-    wl = WORKLOADS[name](dev)
-    wall_ms, dev_ms, dev_min_ms = time_steps(wl["fn"], steps, warmup)
+    wl = WORKLOADS_ALL[name](dev)
+    wall_ms, dev_ms, launch_mode = time_steps(wl["fn"], steps, warmup)
     scale = 1e9 if wl["unit"] == "GB/s" else 1e12
     achieved = wl["work"] / (dev_ms * 1e-3) / scale
     rec = {
@@ -210,7 +269,7 @@ def measure(name: str, dev, steps: int, warmup: int, with_cpu: bool):
         "unit": wl["unit"],
         "ms_per_step": wall_ms,
         "kernel_ms_avg": dev_ms,
-        "kernel_ms_min": dev_min_ms,
+        "launch": launch_mode,
         "dtype": wl["dtype"],
         "config": wl["config"],
         "roofline": {"bound": wl["bound"], "achieved": achieved, "peak": wl["peak"], "unit": wl["unit"],
@@ -230,7 +289,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS_ALL))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-others", action="store_true", help="measure only --workload")
     args = ap.parse_args()
@@ -271,7 +330,7 @@ def main() -> int:
         "data": "synthetic (seeded torch CPU generator, seed 10; random-normal * 0.1 fp16 operands)",
         "config": head["config"],
         "kernel_ms_avg": head["kernel_ms_avg"],
-        "kernel_ms_min": head["kernel_ms_min"],
+        "launch": head["launch"],
         "roofline": head["roofline"],
         "cpu_baseline": head.get("cpu_baseline"),
         "host": {"cpu": platform.processor() or platform.machine(), "os_cpu_count": os.cpu_count(),
