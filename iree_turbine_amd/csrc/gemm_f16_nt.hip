@@ -356,6 +356,206 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
   }
 }
 
+// Persistent form of gemm_f16_nt_pipelined: one workgroup per CU walks its share of the output tiles
+// (tile ids pid, pid + grid, ...) as ONE continuous sequence of K slabs.  The loads issued during the last
+// two slabs of a tile already fetch the first two slabs of the next tile, the fragment reads at the end of
+// the last slab already belong to the next tile, and the epilogue runs out of its own LDS region (one
+// 32-row pass at a time), so its global stores drain while the next tile computes.  Without this every
+// round of tiles pays a pipeline fill and a burst of output stores with the matrix cores idle.
+template <int BM, int BN, int WM, int WN, typename OutT>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_persistent(const half_t* __restrict__ A,
+                                                                      const half_t* __restrict__ B,
+                                                                      OutT* __restrict__ C, int M, int N, int K,
+                                                                      int tiles_m, int tiles_n, int group_m) {
+  constexpr int NW = WM * WN;
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
+  constexpr int A_GROUPS = BM / 8, B_GROUPS = BN / 8;
+  static_assert(A_GROUPS % NW == 0 && B_GROUPS % NW == 0 && NW % 2 == 0, "loads must split evenly over an even number of waves");
+  static_assert(WTN == 64, "the fp16 epilogue pass is 32 rows of 128 bytes");
+  constexpr int LA = A_GROUPS / NW, LB = B_GROUPS / NW;
+  constexpr int EP_WAVE = 32 * WTN * 2;  // one epilogue pass of a wave: 32 rows of its tile in fp16
+
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  const int T = tiles_m * tiles_n;
+  const int G = gridDim.x;
+  const int KT = K / 64;  // >= 2 (checked by the host)
+
+  const int lrow = lane >> 3;
+  const int lchunk = (lane & 7) ^ (((wave & 1) << 2) | (lrow >> 1));
+  const unsigned lane_off = (unsigned)lrow * (unsigned)K + (unsigned)lchunk * 8u;
+  const size_t row_step = (size_t)NW * 8 * K;
+
+  // wave-uniform source pointers of a tile's rows
+  auto tile_src = [&](int pid, const half_t*& a_src, const half_t*& b_src, int& tile_m, int& tile_n) {
+    map_tile(pid, tiles_m, tiles_n, group_m, tile_m, tile_n);
+    a_src = A + (size_t)(tile_m * BM + wave * 8) * K;
+    b_src = B + (size_t)(tile_n * BN + wave * 8) * K;
+  };
+  auto issue_loads = [&](int stage, const half_t* ap, const half_t* bp) {
+    char* dst = lds + stage * STAGE + wave * 1024;
+#pragma unroll
+    for (int i = 0; i < LA; i++) load_lds_16B(ap + i * row_step + lane_off, dst + i * NW * 1024);
+#pragma unroll
+    for (int i = 0; i < LB; i++) load_lds_16B(bp + i * row_step + lane_off, dst + A_BYTES + i * NW * 1024);
+  };
+
+  const int r32 = lane & 31, h = lane >> 5;
+  const int sw = (h ^ ((r32 >> 1) & 7)) * 16;
+  const int a_base = (wm * WTM + r32) * 128 + sw;
+  const int b_base = A_BYTES + (wn * WTN + r32) * 128 + sw;
+  auto read_frags = [&](const char* st, int ks, half8* fm, half8* fn) {
+#pragma unroll
+    for (int j = 0; j < TM; j++) fm[j] = *reinterpret_cast<const half8*>(st + ((a_base ^ (ks * 32)) + j * 4096));
+#pragma unroll
+    for (int i = 0; i < TN; i++) fn[i] = *reinterpret_cast<const half8*>(st + ((b_base ^ (ks * 32)) + i * 4096));
+  };
+
+  floatx16 acc[TN][TM];
+  auto zero_acc = [&]() {
+#pragma unroll
+    for (int i = 0; i < TN; i++)
+#pragma unroll
+      for (int j = 0; j < TM; j++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+  };
+  zero_acc();
+  auto mfmas = [&](const half8* fm, const half8* fn) {
+#pragma unroll
+    for (int i = 0; i < TN; i++)
+#pragma unroll
+      for (int j = 0; j < TM; j++) acc[i][j] = mfma_32x32x16(fn[i], fm[j], acc[i][j]);
+  };
+  auto interleave = [&]() {
+#pragma unroll
+    for (int i = 0; i < TM + TN; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
+  };
+
+  half8 fm0[TM], fn0[TN], fm1[TM], fn1[TN];
+
+  int pid = blockIdx.x;
+  if (pid >= T) return;
+  const half_t *a_src, *b_src, *a_nxt, *b_nxt;
+  int tile_m, tile_n, nxt_m, nxt_n;
+  tile_src(pid, a_src, b_src, tile_m, tile_n);
+  issue_loads(0, a_src, b_src);
+  wait_vmcnt0();
+  __syncthreads();
+  issue_loads(1, a_src + 64, b_src + 64);
+  read_frags(lds, 0, fm0, fn0);
+  int v = 0;  // slabs retired so far: selects the LDS stage across tile boundaries
+
+  for (; pid < T; pid += G) {
+    // the tile after this one (the last tile "continues" into itself: its first slabs are fetched again
+    // and never used, like the clamped loads of the non-persistent kernel)
+    const int npid = pid + G < T ? pid + G : pid;
+    tile_src(npid, a_nxt, b_nxt, nxt_m, nxt_n);
+
+    for (int kt = 0; kt < KT; kt++, v++) {
+      const char* st = lds + (v & 1) * STAGE;
+      __builtin_amdgcn_sched_barrier(0);
+      read_frags(st, 1, fm1, fn1);
+      mfmas(fm0, fn0);
+      interleave();
+      __builtin_amdgcn_sched_barrier(0);
+      read_frags(st, 2, fm0, fn0);
+      mfmas(fm1, fn1);
+      interleave();
+      __builtin_amdgcn_sched_barrier(0);
+      read_frags(st, 3, fm1, fn1);
+      mfmas(fm0, fn0);
+      interleave();
+      __builtin_amdgcn_sched_barrier(0);
+      // retire the slab: every wave's LDS reads of this stage have returned, next slab has landed
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+      __syncthreads();
+      __builtin_amdgcn_sched_barrier(0);
+      // loads of the slab after next (branch-free: past the end of this tile they are the next tile's
+      // slabs 0 and 1) and the first fragment reads of the next slab ride between the last MFMAs
+      const bool wrap = kt + 2 >= KT;
+      const int ls = wrap ? kt + 2 - KT : kt + 2;
+      issue_loads(v & 1, (wrap ? a_nxt : a_src) + ls * 64, (wrap ? b_nxt : b_src) + ls * 64);
+      read_frags(lds + ((v + 1) & 1) * STAGE, 0, fm0, fn0);
+      mfmas(fm1, fn1);
+      {
+        constexpr int NL = LA + LB, NR = TM + TN, NM = TM * TN;
+        constexpr int M_FOR_LOADS = NM / 2, L_PER_M = (NL + M_FOR_LOADS - 1) / M_FOR_LOADS;
+#pragma unroll
+        for (int i = 0; i < M_FOR_LOADS; i++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x010, L_PER_M, 0);  // VMEM (direct-to-LDS loads)
+        }
+        constexpr int M_FOR_READS = NM - M_FOR_LOADS - 1, R_PER_M = (NR + M_FOR_READS - 1) / M_FOR_READS;
+#pragma unroll
+        for (int i = 0; i < M_FOR_READS; i++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, R_PER_M, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // ---- epilogue of this tile; the next tile's first two slabs are already in flight ----
+    if constexpr (sizeof(OutT) == 2) {
+      // 32 rows per pass through a private 4 KiB region behind the two stages: ds_write_b64 of 4
+      // consecutive n (chunk slot c ^ ((m>>1)&7)), whole rows read back 16 bytes per lane, stored as
+      // full 128-byte lines.  LDS operations of a wave execute in order, so passes need no waits between them.
+      char* ep = lds + 2 * STAGE + wave * EP_WAVE;
+      const int er = lane >> 3, ec = lane & 7;
+      OutT* cbase = C + (size_t)(tile_m * BM + wm * WTM) * N + tile_n * BN + wn * WTN + ec * 8;
+#pragma unroll
+      for (int j = 0; j < TM; j++) {
+#pragma unroll
+        for (int i = 0; i < TN; i++)
+#pragma unroll
+          for (int q = 0; q < 4; q++) {
+            const int c = i * 4 + q;
+            half4 hv = {(half_t)acc[i][j][4 * q], (half_t)acc[i][j][4 * q + 1], (half_t)acc[i][j][4 * q + 2],
+                        (half_t)acc[i][j][4 * q + 3]};
+            *reinterpret_cast<half4*>(ep + r32 * 128 + ((c ^ ((r32 >> 1) & 7)) * 16) + 8 * h) = hv;
+          }
+#pragma unroll
+        for (int it = 0; it < 4; it++) {
+          const int row = it * 8 + er;
+          half8 ov = *reinterpret_cast<const half8*>(ep + row * 128 + ((ec ^ ((row >> 1) & 7)) * 16));
+          *reinterpret_cast<half8*>(cbase + (size_t)(j * 32 + row) * N) = ov;
+        }
+      }
+    } else {
+      const int m0 = tile_m * BM + wm * WTM + r32;
+      const int n0 = tile_n * BN + wn * WTN + 4 * h;
+#pragma unroll
+      for (int j = 0; j < TM; j++) {
+        OutT* crow = C + (size_t)(m0 + j * 32) * N + n0;
+#pragma unroll
+        for (int i = 0; i < TN; i++)
+#pragma unroll
+          for (int q = 0; q < 4; q++)
+            OutPack<OutT>::store4(crow + i * 32 + q * 8, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                                  acc[i][j][4 * q + 3]);
+      }
+    }
+    zero_acc();
+    a_src = a_nxt;
+    b_src = b_nxt;
+    tile_m = nxt_m;
+    tile_n = nxt_n;
+  }
+  // the loads issued for a tile that does not exist still target LDS: let them land before the block ends
+  wait_vmcnt0();
+}
+
 // Any-shape kernel: 64x64 tile, 4 waves, bounds-checked staging through registers.  Used for
 // shapes the tiled kernel does not divide (and as an independent implementation in tests).
 template <typename OutT>
@@ -419,6 +619,7 @@ struct GemmVariant {
   int bm, bn, threads;
 };
 static const GemmVariant kGemmVariants[] = {
+    {"persistent_256x256x64_w2x4", 256, 256, 512},
     {"pipelined_256x256x64_w2x4", 256, 256, 512},
     {"pipelined_256x256x64_w2x2", 256, 256, 256},
     {"pipelined_128x128x64_w2x2", 128, 128, 256},
@@ -455,14 +656,54 @@ static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int
   return check_launch(PIPELINED ? "gemm_f16_nt_pipelined" : "gemm_f16_nt_tiled", grid, block, lds_bytes);
 }
 
+// number of CUs of the device the stream's context is on (cached per device)
+static int cu_count() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
+template <int BM, int BN, int WM, int WN, typename OutT>
+static int launch_persistent(const void* a, const void* b, void* c, int M, int N, int K, hipStream_t stream) {
+  auto kern = gemm_f16_nt_persistent<BM, BN, WM, WN, OutT>;
+  constexpr int lds_bytes = 2 * (BM + BN) * 128 + WM * WN * 32 * (BN / WN) * 2;  // two stages + one epilogue pass per wave
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       lds_bytes);
+    if (e != hipSuccess) {
+      set_error("hipFuncSetAttribute(gemm_f16_nt_persistent, %d bytes LDS): %s", lds_bytes, hipGetErrorString(e));
+      return (int)e;
+    }
+    attr_set = true;
+  }
+  const int tiles_m = M / BM, tiles_n = N / BN;
+  const int T = tiles_m * tiles_n;
+  // one workgroup per CU (the LDS footprint allows no more), in multiples of 8 so that a workgroup's tile
+  // ids pid + k * grid all fall on the XCD the hardware placed it on
+  int g = cu_count() & ~7;
+  if (g < 8) g = 8;
+  dim3 grid(T < g ? T : g), block(WM * WN * 64);
+  hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, M, N, K, tiles_m,
+                     tiles_n, 4);
+  return check_launch("gemm_f16_nt_persistent", grid, block, lds_bytes);
+}
+
 template <typename OutT>
 static int launch_variant(int variant, const void* a, const void* b, void* c, int M, int N, int K, hipStream_t stream) {
   switch (variant) {
-    case 0: return launch_tiled<256, 256, 2, 4, OutT, true>(a, b, c, M, N, K, stream);
-    case 1: return launch_tiled<256, 256, 2, 2, OutT, true>(a, b, c, M, N, K, stream);
-    case 2: return launch_tiled<128, 128, 2, 2, OutT, true>(a, b, c, M, N, K, stream);
-    case 3: return launch_tiled<256, 256, 2, 4, OutT, false>(a, b, c, M, N, K, stream);
-    case 4: return launch_tiled<128, 128, 2, 2, OutT, false>(a, b, c, M, N, K, stream);
+    case 0: return launch_persistent<256, 256, 2, 4, OutT>(a, b, c, M, N, K, stream);
+    case 1: return launch_tiled<256, 256, 2, 4, OutT, true>(a, b, c, M, N, K, stream);
+    case 2: return launch_tiled<256, 256, 2, 2, OutT, true>(a, b, c, M, N, K, stream);
+    case 3: return launch_tiled<128, 128, 2, 2, OutT, true>(a, b, c, M, N, K, stream);
+    case 4: return launch_tiled<256, 256, 2, 4, OutT, false>(a, b, c, M, N, K, stream);
+    case 5: return launch_tiled<128, 128, 2, 2, OutT, false>(a, b, c, M, N, K, stream);
     default: {
       dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
       hipLaunchKernelGGL(gemm_f16_nt_generic<OutT>, grid, block, 0, stream, (const half_t*)a, (const half_t*)b, (OutT*)c,
@@ -487,6 +728,7 @@ extern "C" int mi355_gemm_f16_nt(const void* a, const void* b, void* c, int64_t 
   const bool al = aligned16(a) && aligned16(b) && aligned16(c);
   auto fits = [&](int v) {
     if (v == kNumGemmVariants - 1) return true;
+    if (v == 0 && K < 128) return false;  // the persistent kernel prefetches two slabs ahead
     return al && M % kGemmVariants[v].bm == 0 && N % kGemmVariants[v].bn == 0 && K % 64 == 0;
   };
   if (variant < 0) {
@@ -495,7 +737,7 @@ extern "C" int mi355_gemm_f16_nt(const void* a, const void* b, void* c, int64_t 
     const long long t256 = (M / 256) * (N / 256);
     const long long rounds = (t256 + 255) / 256;  // 256 CUs, one 256x256 workgroup each
     if (fits(0) && t256 >= 128 && t256 * 100 >= rounds * 256 * 85) variant = 0;  // >= 85% of the last round busy
-    else if (fits(2)) variant = 2;
+    else if (fits(3)) variant = 3;
     else variant = kNumGemmVariants - 1;
   } else if (!fits(variant)) {
     return fail(-MI355_E_SHAPE, "gemm_f16_nt: variant %s needs M%%%d==0, N%%%d==0, K%%64==0 and 16-byte aligned pointers",

@@ -8,11 +8,15 @@
 // Tiling is the fp16 GEMM's with k measured in bytes: a K slab is 256 fp4 values = 128 bytes
 // per row = 8 chunks of 16 bytes (one chunk = one 32-element scale block), copied with
 // direct-to-LDS loads into a two-stage ring with the same XOR swizzle and the same rotated,
-// software-pipelined k-loop.  A lane's 16-byte
-// fragment is exactly one scale block, so the lane's scale byte is scale[row][slab*8 + 2*ks + h]
-// (h = lane / 32); each lane fetches the 8 scale bytes of its row for a slab with one 8-byte
-// global load one slab ahead, lanes with h = 1 pre-shift by one byte, and the op_sel field of
-// the MFMA picks byte 0 or 2.
+// software-pipelined k-loop.
+//
+// A lane's 16-byte fragment is exactly one scale block.  Which two blocks of a slab form a 64-wide
+// k-step is free as long as A and B agree, so k-step ks (0..3) pairs block ks (lanes 0..31) with
+// block 4+ks (lanes 32..63): a lane then needs bytes ks = 0..3 of ONE dword per row and slab
+// (dword h = lane / 32 of the row's 8 scale bytes), fetched one slab ahead, and the op_sel field
+// of the MFMA picks the byte: no shifts or permutes in the loop.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace mi355 {
@@ -46,11 +50,12 @@ template <> struct MxOut<unsigned short> {  // bf16 bits
   static __device__ __forceinline__ void store1(unsigned short* p, float a) { *p = f32_to_bf16_rne(a); }
 };
 
-__device__ __forceinline__ floatx16 mfma_fp4_32x32x64(intx4 a, int sa, intx4 b, int sb, floatx16 c, bool odd) {
+// byte SEL of sa / sb scales the lane's block of a / b
+template <int SEL>
+__device__ __forceinline__ floatx16 mfma_fp4_32x32x64(intx4 a, int sa, intx4 b, int sb, floatx16 c) {
   intx8 av = {a[0], a[1], a[2], a[3], 0, 0, 0, 0};
   intx8 bv = {b[0], b[1], b[2], b[3], 0, 0, 0, 0};
-  if (odd) return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, 4, 4, 2, sa, 2, sb);
-  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, 4, 4, 0, sa, 0, sb);
+  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, c, 4, 4, SEL, sa, SEL, sb);
 }
 
 // SCALES_LDS: scale bytes travel through LDS in groups of 4 slabs (32 bytes per row, two buffers behind
@@ -98,16 +103,15 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
   };
 
   const int r32 = lane & 31, h = lane >> 5;
-  const int sw = (h ^ ((r32 >> 1) & 7)) * 16;
+  const int sw = ((4 * h) ^ ((r32 >> 1) & 7)) * 16;  // chunk ks + 4h of the row, swizzled
   const int a_base = (wm * WTM + r32) * 128 + sw;
   const int b_base = A_BYTES + (wn * WTN + r32) * 128 + sw;
 
-  // scale bytes: 8 per row per slab, fetched one slab ahead; lanes with h = 1 drop one byte so that
-  // op_sel 0 / 2 address blocks 2*ks + h of the slab for every lane
-  const uint8_t* as_src = As + (size_t)(tile_m * BM + wm * WTM + r32) * Ksc;
-  const uint8_t* bs_src = Bs + (size_t)(tile_n * BN + wn * WTN + r32) * Ksc;
-  const int shift = 8 * h;
-  intx2 sa_cur[TM], sb_cur[TN], sa_nxt[TM], sb_nxt[TN];
+  // scale dwords: bytes 4h..4h+3 of the row's 8 scale bytes of a slab, fetched one slab ahead into the
+  // register set the slab after next will not touch
+  const uint8_t* as_src = As + (size_t)(tile_m * BM + wm * WTM + r32) * Ksc + 4 * h;
+  const uint8_t* bs_src = Bs + (size_t)(tile_n * BN + wn * WTN + r32) * Ksc + 4 * h;
+  int sa[2][TM], sb[2][TN];
   // LDS scale buffers: [buffer][A rows then B rows][32 bytes = 4 slabs x 8 blocks]
   constexpr int SC_BUF = (BM + BN) * 32;
   char* sc_lds = lds + 2 * STAGE;
@@ -123,47 +127,27 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
       load_lds_16B(src + group * 32 + sc_lane_off, dst + r0 * 32);
     }
   };
-  const int sa_off = (wm * WTM + r32) * 32, sb_off = (BM + wn * WTN + r32) * 32;
-  auto load_scales = [&](intx2* sa, intx2* sb, int slab) {
+  const int sa_off = (wm * WTM + r32) * 32 + 4 * h, sb_off = (BM + wn * WTN + r32) * 32 + 4 * h;
+  auto fetch_scales = [&](int* da, int* db, int slab) {
     if constexpr (SCALES_LDS) {
       const char* buf = sc_lds + ((slab >> 2) & 1) * SC_BUF + (slab & 3) * 8;
 #pragma unroll
-      for (int j = 0; j < TM; j++) sa[j] = *reinterpret_cast<const intx2*>(buf + sa_off + j * 1024);
+      for (int j = 0; j < TM; j++) da[j] = *reinterpret_cast<const int*>(buf + sa_off + j * 1024);
 #pragma unroll
-      for (int i = 0; i < TN; i++) sb[i] = *reinterpret_cast<const intx2*>(buf + sb_off + i * 1024);
+      for (int i = 0; i < TN; i++) db[i] = *reinterpret_cast<const int*>(buf + sb_off + i * 1024);
     } else {
 #pragma unroll
-      for (int j = 0; j < TM; j++) sa[j] = *reinterpret_cast<const intx2*>(as_src + (size_t)j * 32 * Ksc + slab * 8);
+      for (int j = 0; j < TM; j++) da[j] = *reinterpret_cast<const int*>(as_src + (size_t)j * 32 * Ksc + slab * 8);
 #pragma unroll
-      for (int i = 0; i < TN; i++) sb[i] = *reinterpret_cast<const intx2*>(bs_src + (size_t)i * 32 * Ksc + slab * 8);
-    }
-  };
-  // SCALES_LDS: one dword (4 blocks = 2 k-steps) per row tile straight into the live scale registers
-  auto lds_scales = [&](int slab, int d) {
-    const char* buf = sc_lds + ((slab >> 2) & 1) * SC_BUF + (slab & 3) * 8 + d * 4;
-#pragma unroll
-    for (int j = 0; j < TM; j++) sa_cur[j][d] = (int)(*reinterpret_cast<const unsigned*>(buf + sa_off + j * 1024) >> shift);
-#pragma unroll
-    for (int i = 0; i < TN; i++) sb_cur[i][d] = (int)(*reinterpret_cast<const unsigned*>(buf + sb_off + i * 1024) >> shift);
-  };
-  auto shift_scales = [&](intx2* sa, intx2* sb) {
-#pragma unroll
-    for (int j = 0; j < TM; j++) {
-      sa[j][0] = (int)((unsigned)sa[j][0] >> shift);
-      sa[j][1] = (int)((unsigned)sa[j][1] >> shift);
-    }
-#pragma unroll
-    for (int i = 0; i < TN; i++) {
-      sb[i][0] = (int)((unsigned)sb[i][0] >> shift);
-      sb[i][1] = (int)((unsigned)sb[i][1] >> shift);
+      for (int i = 0; i < TN; i++) db[i] = *reinterpret_cast<const int*>(bs_src + (size_t)i * 32 * Ksc + slab * 8);
     }
   };
 
   auto read_frags = [&](const char* st, int ks, intx4* fm, intx4* fn) {
 #pragma unroll
-    for (int j = 0; j < TM; j++) fm[j] = *reinterpret_cast<const intx4*>(st + ((a_base ^ (ks * 32)) + j * 4096));
+    for (int j = 0; j < TM; j++) fm[j] = *reinterpret_cast<const intx4*>(st + ((a_base ^ (ks * 16)) + j * 4096));
 #pragma unroll
-    for (int i = 0; i < TN; i++) fn[i] = *reinterpret_cast<const intx4*>(st + ((b_base ^ (ks * 32)) + i * 4096));
+    for (int i = 0; i < TN; i++) fn[i] = *reinterpret_cast<const intx4*>(st + ((b_base ^ (ks * 16)) + i * 4096));
   };
 
   floatx16 acc[TN][TM];
@@ -174,12 +158,12 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-  auto mfmas = [&](const intx4* fm, const intx4* fn, int ks) {
+  auto mfmas = [&](auto ks_tag, const intx4* fm, const intx4* fn, const int* ca, const int* cb) __attribute__((always_inline)) {
+    constexpr int KS = decltype(ks_tag)::value;
 #pragma unroll
     for (int i = 0; i < TN; i++)
 #pragma unroll
-      for (int j = 0; j < TM; j++)
-        acc[i][j] = mfma_fp4_32x32x64(fn[i], sb_cur[i][ks >> 1], fm[j], sa_cur[j][ks >> 1], acc[i][j], ks & 1);
+      for (int j = 0; j < TM; j++) acc[i][j] = mfma_fp4_32x32x64<KS>(fn[i], cb[i], fm[j], ca[j], acc[i][j]);
   };
   auto interleave = [&]() {
 #pragma unroll
@@ -190,73 +174,70 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
     __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
   };
 
-  // k-step region that also fetches TM + TN scale dwords from LDS: two LDS reads per slot
-  auto interleave_with_scales = [&]() {
-#pragma unroll
-    for (int i = 0; i < TM + TN; i++) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
-  };
-
   const int KT = K / 256;
   intx4 fm0[TM], fn0[TN], fm1[TM], fn1[TN];
-
   const int KG = (KT + 3) >> 2;  // scale groups
   if constexpr (SCALES_LDS) issue_scale_loads(0);
   issue_loads(0, 0);
   wait_vmcnt0();
   __syncthreads();
-  if constexpr (SCALES_LDS) {
-    lds_scales(0, 0);
-    issue_scale_loads(KG > 1 ? 1 : 0);
-    issue_loads(1, KT > 1 ? 1 : 0);
-  } else {
-    load_scales(sa_cur, sb_cur, 0);
-    issue_loads(1, KT > 1 ? 1 : 0);
-    wait_vmcnt0();
-    shift_scales(sa_cur, sb_cur);
-  }
+  fetch_scales(sa[0], sb[0], 0);
+  if constexpr (SCALES_LDS) issue_scale_loads(KG > 1 ? 1 : 0);
+  issue_loads(1, KT > 1 ? 1 : 0);
   read_frags(lds, 0, fm0, fn0);
+  if constexpr (!SCALES_LDS) wait_vmcnt0();
 
-  // Rotated k-loop (see gemm_f16_nt_pipelined): fragment reads for k-step s+1 ride between the MFMAs
-  // of k-step s; the slab-retiring barrier sits in front of the last k-step's MFMAs, which overlap the
-  // global -> LDS loads of slab kt+2 and the first fragment reads of slab kt+1.
-  for (int kt = 0; kt < KT; kt++) {
+  using K0 = std::integral_constant<int, 0>;
+  using K1 = std::integral_constant<int, 1>;
+  using K2 = std::integral_constant<int, 2>;
+  using K3 = std::integral_constant<int, 3>;
+  // One slab (rotated k-loop, see gemm_f16_nt_pipelined): fragment reads for k-step s+1 ride between the
+  // MFMAs of k-step s; the slab-retiring barrier sits in front of the last k-step's MFMAs, which overlap
+  // the global -> LDS loads of slab kt+2 and the first fragment reads of slab kt+1.  With LDS-staged
+  // scales the loop is unrolled by the scale-group period (4 slabs, KK = kt & 3 static) so that the body
+  // stays one basic block: a branch inside it would end the scheduling region and the fixed
+  // MFMA / LDS-read interleave with it.
+  auto slab = [&](auto kk_tag, int kt) __attribute__((always_inline)) {
+    constexpr int KK = decltype(kk_tag)::value;
+    constexpr int CUR = KK & 1, NXT = CUR ^ 1;
     const char* st = lds + (kt & 1) * STAGE;
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (SCALES_LDS) lds_scales(kt, 1);  // blocks 4..7 of this slab (their registers went idle after the last k-step)
-    else load_scales(sa_nxt, sb_nxt, kt + 1 < KT ? kt + 1 : KT - 1);
+    fetch_scales(sa[NXT], sb[NXT], kt + 1 < KT ? kt + 1 : KT - 1);
     read_frags(st, 1, fm1, fn1);
-    mfmas(fm0, fn0, 0);
-    if constexpr (SCALES_LDS) interleave_with_scales(); else interleave();
+    mfmas(K0{}, fm0, fn0, sa[CUR], sb[CUR]);
+    if constexpr (SCALES_LDS) {
+#pragma unroll
+      for (int i = 0; i < TM + TN; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // one fragment, one scale dword
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
+    } else {
+      interleave();
+    }
     __builtin_amdgcn_sched_barrier(0);
     read_frags(st, 2, fm0, fn0);
-    mfmas(fm1, fn1, 1);
+    mfmas(K1{}, fm1, fn1, sa[CUR], sb[CUR]);
     interleave();
     __builtin_amdgcn_sched_barrier(0);
     read_frags(st, 3, fm1, fn1);
-    if constexpr (SCALES_LDS) lds_scales(kt + 1 < KT ? kt + 1 : KT - 1, 0);  // blocks 0..3 of the next slab
-    mfmas(fm0, fn0, 2);
-    if constexpr (SCALES_LDS) interleave_with_scales(); else interleave();
+    mfmas(K2{}, fm0, fn0, sa[CUR], sb[CUR]);
+    interleave();
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
     issue_loads(kt & 1, kt + 2 < KT ? kt + 2 : KT - 1);
-    if constexpr (SCALES_LDS) {
-      // Group g+1 replaces group g-1 in its buffer once the last slab of g-1 has had its scales read
-      // into registers: that happens during slab 4g-2, i.e. before the barrier of slab 4g-1 = kt.
-      if ((kt & 3) == 3) {
-        const int g = (kt >> 2) + 2;
-        issue_scale_loads(g < KG ? g : KG - 1);
-      }
+    if constexpr (SCALES_LDS && KK == 3) {
+      // Group g replaces group g-2 in its buffer; the last slab of g-2 is this one, and its scale dwords
+      // went into registers during the previous slab, before the barrier above.
+      const int g = (kt >> 2) + 2;
+      issue_scale_loads(g < KG ? g : KG - 1);
     }
     read_frags(lds + ((kt + 1) & 1) * STAGE, 0, fm0, fn0);
-    mfmas(fm1, fn1, 3);
+    mfmas(K3{}, fm1, fn1, sa[CUR], sb[CUR]);
     {
-      constexpr int NL = LA + LB, NR = TM + TN, NM = TM * TN;
+      constexpr int NL = LA + LB + (SCALES_LDS && KK == 3 ? LS : 0), NR = TM + TN, NM = TM * TN;
       constexpr int M_FOR_LOADS = NM / 2, L_PER_M = (NL + M_FOR_LOADS - 1) / M_FOR_LOADS;
 #pragma unroll
       for (int i = 0; i < M_FOR_LOADS; i++) {
@@ -272,13 +253,23 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
-    if constexpr (!SCALES_LDS) {
-#pragma unroll
-      for (int j = 0; j < TM; j++) sa_cur[j] = sa_nxt[j];
-#pragma unroll
-      for (int i = 0; i < TN; i++) sb_cur[i] = sb_nxt[i];
-      shift_scales(sa_cur, sb_cur);
+  };
+  if constexpr (SCALES_LDS) {
+    for (int kt = 0; kt < KT; kt += 4) {  // K % 1024 == 0 on this path
+      slab(K0{}, kt);
+      slab(K1{}, kt + 1);
+      slab(K2{}, kt + 2);
+      slab(K3{}, kt + 3);
     }
+  } else {
+    // scale dwords come straight from global memory (waited for with the slab's loads); two slabs per
+    // trip keep the register-set indices static
+    int kt = 0;
+    for (; kt + 1 < KT; kt += 2) {
+      slab(K0{}, kt);
+      slab(K1{}, kt + 1);
+    }
+    if (kt < KT) slab(K0{}, kt);
   }
   wait_vmcnt0();
   __syncthreads();
@@ -353,7 +344,7 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_generic(const uint8_t* __restr
       fb = *reinterpret_cast<const intx4*>(B + (size_t)n * Kb + blk * 16);
       sb = Bs[(size_t)n * Ksc + blk];
     }
-    acc = mfma_fp4_32x32x64(fb, sb, fa, sa, acc, false);
+    acc = mfma_fp4_32x32x64<0>(fb, sb, fa, sa, acc);
   }
   if (m < M) {
     const int nb = (blockIdx.x * 4 + wave) * 32;
@@ -576,10 +567,13 @@ extern "C" int mi355_mxfp4_gemm(const void* a, const void* a_scale, const void* 
     return sc_al && M % kMxVariants[v].bm == 0 && N % kMxVariants[v].bn == 0 && K % 256 == 0;
   };
   if (variant < 0) {
-    // The 256x256 tile pays off only with a long K loop (its prologue/epilogue is amortised over
-    // K/256 slabs); M <= 32 is weight streaming and has its own kernel.
+    // M <= 32 is weight streaming and has its own kernel.  The 256x256 tile halves the L2 -> LDS bytes per
+    // flop; it is used when there are enough tiles to fill the 256 CUs and the last round of workgroups
+    // is at least 85 % full.
+    const long long t256 = (M / 256) * (N / 256);
+    const long long rounds = (t256 + 255) / 256;
     if (fits(2)) variant = 2;
-    else if (fits(0) && (M / 256) * (N / 256) >= 256 && K >= 16384) variant = 0;
+    else if (fits(0) && t256 >= 128 && t256 * 100 >= rounds * 256 * 85) variant = 0;
     else if (fits(1)) variant = 1;
     else variant = kNumMxVariants - 1;
   } else if (!fits(variant)) {

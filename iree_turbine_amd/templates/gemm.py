@@ -2,20 +2,27 @@ from __future__ import annotations
 
 import torch
 
-from .. import launch
+from .. import _lib, launch
 from ..lang import sym
 from ..launchable import Launchable
 
 M, N, K = sym.M, sym.N, sym.K
 BLOCK_M, BLOCK_N, BLOCK_K = sym.BLOCK_M, sym.BLOCK_N, sym.BLOCK_K
 
-# (BLOCK_M, BLOCK_N) -> kernel variant index of mi355_gemm_f16_nt
-_VARIANT_BY_TILE = {(256, 256): 0, (128, 128): 2, (64, 64): 5}
+def _variant_for_tile(bm, bn) -> int:
+    """First (= preferred) kernel variant of mi355_gemm_f16_nt whose tile is bm x bn; -1 (library's choice) if none."""
+    if bm is None or bn is None:
+        return -1
+    for i, name in enumerate(_lib.variants("gemm_f16_nt")):
+        if f"_{bm}x{bn}x" in name:
+            return i
+    return -1
 
 
 def _entry(hp, a, b, c):
-    tile = (hp.get(BLOCK_M), hp.get(BLOCK_N))
-    variant = hp.get(sym.VARIANT, _VARIANT_BY_TILE.get(tile, -1))
+    variant = hp.get(sym.VARIANT)
+    if variant is None:
+        variant = _variant_for_tile(hp.get(BLOCK_M), hp.get(BLOCK_N))
     for s, dim, t in ((M, 0, a), (K, 1, a), (N, 0, b)):
         if s in hp and hp[s] != t.shape[dim]:
             raise ValueError(f"gemm kernel was specialised for {s}={hp[s]} but got {t.shape[dim]}")

@@ -22,7 +22,7 @@ def _run(dev, M, N, K, out_dtype, variant=-1, seed=10):
     return c.float().cpu(), ref
 
 
-@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 3, 4, 5, 6])
 def test_gemm_1024_f32_all_variants(dev, variant):
     c, ref = _run(dev, 1024, 1024, 1024, "float32", variant)
     torch.testing.assert_close(c, ref, rtol=RTOL, atol=ATOL)
@@ -143,3 +143,26 @@ def test_gemm_full_size_repeatable(dev, shape):
         for _ in range(2):
             assert torch.equal(first, torch.ops.mi355.gemm_nt(a, b, "float32", variant)), names[variant]
         torch.testing.assert_close(first, generic, rtol=1e-3, atol=1e-3)
+
+
+@pytest.mark.parametrize("shape", [(4096, 4608, 192), (4352, 4352, 128), (8192, 8704, 320), (512, 256, 4096)])
+@pytest.mark.parametrize("out_dtype", ["float16", "float32"])
+def test_gemm_persistent_tile_walk(dev, shape, out_dtype):
+    """The persistent kernel walks several tiles per workgroup as one slab sequence: more tiles than CUs,
+    tile counts that are not multiples of 8 or of the grid, odd slab counts (the LDS stage parity flips
+    between tiles), the minimum of two slabs, and fewer tiles than CUs -- whole matrix against the
+    independent generic kernel."""
+    import iree_turbine_amd as ita
+    from oracle import inputs
+
+    M, N, K = shape
+    announce(f"gemm persistent walk {shape} {out_dtype}")
+    names = ita._lib.variants("gemm_f16_nt")
+    assert names[0].startswith("persistent")
+    a, b = [t.to(dev) for t in inputs.gemm_inputs(M, N, K)]
+    got = torch.ops.mi355.gemm_nt(a, b, out_dtype, 0)
+    ref = torch.ops.mi355.gemm_nt(a, b, out_dtype, len(names) - 1)
+    torch.testing.assert_close(got.float(), ref.float(), rtol=1e-3, atol=1e-3)
+    rows = torch.tensor([0, 255, 256, M - 1])
+    exact = a[rows.to(dev)].float() @ b.float().t()
+    torch.testing.assert_close(got[rows.to(dev)].float(), exact, rtol=RTOL, atol=ATOL)

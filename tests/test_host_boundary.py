@@ -26,7 +26,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert getattr(lib, name) is not None
     assert lib.mi355_abi_version() == 1
-    assert _lib.variants("gemm_f16_nt")[0].startswith("pipelined_256x256")
+    assert _lib.variants("gemm_f16_nt")[0].startswith("persistent_256x256")
     assert _lib.variants("no_such_family") == []
 
 
