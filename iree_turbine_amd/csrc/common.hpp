@@ -32,6 +32,17 @@ __device__ __forceinline__ void load_lds_16B(const void* gptr, void* lds_wave_ba
   __builtin_amdgcn_global_load_lds(MI355_GLOBAL(gptr), MI355_LDS(void, lds_wave_base), 16, 0, 0);
 }
 
+// Same copy through a buffer descriptor: address = descriptor base + voffset (per lane) + soffset
+// (wave-uniform), all in bytes, so a load costs no 64-bit vector address arithmetic.  Offsets at or
+// beyond the descriptor's size read zeros instead of faulting.
+typedef __amdgpu_buffer_rsrc_t buffer_rsrc_t;
+__device__ __forceinline__ buffer_rsrc_t make_buffer(const void* base, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ void buffer_load_lds_16B(buffer_rsrc_t rsrc, unsigned voffset, unsigned soffset, void* lds_wave_base) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, MI355_LDS(void, lds_wave_base), 16, (int)voffset, (int)soffset, 0, 0);
+}
+
 __device__ __forceinline__ void wait_vmcnt0() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // D(32x32) += A(32x16) * B(16x32).  Lane l supplies A[l%32][8*(l/32) .. +7] and

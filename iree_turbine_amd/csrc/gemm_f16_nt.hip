@@ -20,6 +20,8 @@
 // round-robin to the 8 XCDs (each with a private L2), so ids are first regrouped into 8
 // contiguous ranges and then walked in GROUP_M-tall column-major panels to keep the A/B
 // slabs that one XCD touches small.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace mi355 {
@@ -356,12 +358,21 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
   }
 }
 
-// Persistent form of gemm_f16_nt_pipelined: one workgroup per CU walks its share of the output tiles
-// (tile ids pid, pid + grid, ...) as ONE continuous sequence of K slabs.  The loads issued during the last
-// two slabs of a tile already fetch the first two slabs of the next tile, the fragment reads at the end of
-// the last slab already belong to the next tile, and the epilogue runs out of its own LDS region (one
-// 32-row pass at a time), so its global stores drain while the next tile computes.  Without this every
-// round of tiles pays a pipeline fill and a burst of output stores with the matrix cores idle.
+// Persistent kernel: one workgroup per CU walks its share of the output tiles (tile ids pid, pid + grid,
+// ...) as ONE continuous sequence of K slabs.  The loads issued during the last two slabs of a tile
+// already fetch the first two slabs of the next tile, the fragment reads at the end of the last slab
+// already belong to the next tile, and the epilogue runs out of its own LDS region (one 32-row pass at a
+// time), so its global stores drain while the next tile computes.
+//
+// Slab schedule (four k-steps of 16, one fragment register set each):
+//   k-step 0: MFMAs of set 0   | LDS reads of sets 1 and 2
+//   k-step 1: MFMAs of set 1   | LDS reads of set 3 (front-loaded)
+//   wait + barrier: every wave has read the whole stage, the next slab has landed
+//   k-step 2: MFMAs of set 2   | most global -> LDS loads of the slab after next (into the stage just read)
+//   k-step 3: MFMAs of set 3   | LDS reads of set 0 of the next slab, remaining loads
+// Reading a slab's last fragments one k-step early frees its stage half a slab sooner, so the loads
+// spread over two k-steps instead of bunching behind the barrier, and they use buffer addressing
+// (descriptor + per-lane offset + scalar offset): no vector address arithmetic in the loop.
 template <int BM, int BN, int WM, int WN, typename OutT>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_persistent(const half_t* __restrict__ A,
                                                                       const half_t* __restrict__ B,
@@ -373,9 +384,11 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_persistent(const half
   constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
   constexpr int A_GROUPS = BM / 8, B_GROUPS = BN / 8;
   static_assert(A_GROUPS % NW == 0 && B_GROUPS % NW == 0 && NW % 2 == 0, "loads must split evenly over an even number of waves");
-  static_assert(WTN == 64, "the fp16 epilogue pass is 32 rows of 128 bytes");
   constexpr int LA = A_GROUPS / NW, LB = B_GROUPS / NW;
-  constexpr int EP_WAVE = 32 * WTN * 2;  // one epilogue pass of a wave: 32 rows of its tile in fp16
+  constexpr int EP_ROW = WTN * 2;        // bytes of one fp16 output row of a wave's tile
+  constexpr int EP_WAVE = 32 * EP_ROW;   // one epilogue pass of a wave: 32 rows
+  constexpr int EP_CH = EP_ROW / 16;     // 16-byte chunks per row
+  constexpr int EP_RPB = EP_ROW >= 256 ? 1 : 256 / EP_ROW;  // rows per 256 bytes (= per sweep of the 64 banks)
 
   extern __shared__ __attribute__((aligned(1024))) char lds[];
 
@@ -388,21 +401,29 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_persistent(const half
 
   const int lrow = lane >> 3;
   const int lchunk = (lane & 7) ^ (((wave & 1) << 2) | (lrow >> 1));
-  const unsigned lane_off = (unsigned)lrow * (unsigned)K + (unsigned)lchunk * 8u;
-  const size_t row_step = (size_t)NW * 8 * K;
+  // byte offsets inside a tile's row panel: per lane (row of the 8-row group, swizzled chunk) and per
+  // wave-load (8 * NW rows further down); the host keeps BM * K * 2 below 2^31
+  const unsigned lane_off = ((unsigned)lrow * (unsigned)K + (unsigned)lchunk * 8u) * 2u;
+  const unsigned row_step = (unsigned)NW * 8u * (unsigned)K * 2u;
+  const unsigned panel_a = (unsigned)(BM - wave * 8) * (unsigned)K * 2u, panel_b = (unsigned)(BN - wave * 8) * (unsigned)K * 2u;
 
-  // wave-uniform source pointers of a tile's rows
-  auto tile_src = [&](int pid, const half_t*& a_src, const half_t*& b_src, int& tile_m, int& tile_n) {
+  // buffer descriptors over the rows of a tile that this wave copies (its first row onwards)
+  auto tile_src = [&](int pid, buffer_rsrc_t& a_src, buffer_rsrc_t& b_src, int& tile_m, int& tile_n) {
     map_tile(pid, tiles_m, tiles_n, group_m, tile_m, tile_n);
-    a_src = A + (size_t)(tile_m * BM + wave * 8) * K;
-    b_src = B + (size_t)(tile_n * BN + wave * 8) * K;
+    a_src = make_buffer(A + (size_t)(tile_m * BM + wave * 8) * K, panel_a);
+    b_src = make_buffer(B + (size_t)(tile_n * BN + wave * 8) * K, panel_b);
   };
-  auto issue_loads = [&](int stage, const half_t* ap, const half_t* bp) {
+  // wave-loads FIRST .. LAST-1 of a slab (A groups first, then B groups)
+  auto issue_loads = [&](auto first_tag, auto last_tag, int stage, buffer_rsrc_t ap, buffer_rsrc_t bp, int slab) __attribute__((always_inline)) {
+    constexpr int FIRST = decltype(first_tag)::value, LAST = decltype(last_tag)::value;
     char* dst = lds + stage * STAGE + wave * 1024;
+    const unsigned k_off = (unsigned)slab * 128u;
 #pragma unroll
-    for (int i = 0; i < LA; i++) load_lds_16B(ap + i * row_step + lane_off, dst + i * NW * 1024);
+    for (int i = 0; i < LA; i++)
+      if (i >= FIRST && i < LAST) buffer_load_lds_16B(ap, lane_off, k_off + i * row_step, dst + i * NW * 1024);
 #pragma unroll
-    for (int i = 0; i < LB; i++) load_lds_16B(bp + i * row_step + lane_off, dst + A_BYTES + i * NW * 1024);
+    for (int i = 0; i < LB; i++)
+      if (LA + i >= FIRST && LA + i < LAST) buffer_load_lds_16B(bp, lane_off, k_off + i * row_step, dst + A_BYTES + i * NW * 1024);
   };
 
   const int r32 = lane & 31, h = lane >> 5;
@@ -432,32 +453,33 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_persistent(const half
 #pragma unroll
       for (int j = 0; j < TM; j++) acc[i][j] = mfma_32x32x16(fn[i], fm[j], acc[i][j]);
   };
-  auto interleave = [&]() {
-#pragma unroll
-    for (int i = 0; i < TM + TN; i++) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
-  };
 
-  half8 fm0[TM], fn0[TN], fm1[TM], fn1[TN];
+  constexpr int NM = TM * TN;       // MFMAs per k-step
+  constexpr int NR = TM + TN;       // fragment reads per k-step
+  constexpr int NL = LA + LB;       // wave-loads per slab
+  constexpr int NL2 = NL < NM ? (3 * NL) / 4 : NM - 2;  // loads issued in k-step 2
+  static_assert(2 * NR <= 2 * NM && NR / 2 + 1 <= NM && NL - NL2 + (NR + 1) / 2 < NM, "k-step regions too small for their memory work");
+  using I0 = std::integral_constant<int, 0>;
+  using IL2 = std::integral_constant<int, NL2>;
+  using IL = std::integral_constant<int, NL>;
+
+  half8 fm0[TM], fn0[TN], fm1[TM], fn1[TN], fm2[TM], fn2[TN], fm3[TM], fn3[TN];
 
   int pid = blockIdx.x;
   if (pid >= T) return;
-  const half_t *a_src, *b_src, *a_nxt, *b_nxt;
+  buffer_rsrc_t a_src, b_src, a_nxt, b_nxt;
   int tile_m, tile_n, nxt_m, nxt_n;
   tile_src(pid, a_src, b_src, tile_m, tile_n);
-  issue_loads(0, a_src, b_src);
+  issue_loads(I0{}, IL{}, 0, a_src, b_src, 0);
   wait_vmcnt0();
   __syncthreads();
-  issue_loads(1, a_src + 64, b_src + 64);
+  issue_loads(I0{}, IL{}, 1, a_src, b_src, 1);
   read_frags(lds, 0, fm0, fn0);
   int v = 0;  // slabs retired so far: selects the LDS stage across tile boundaries
 
   for (; pid < T; pid += G) {
     // the tile after this one (the last tile "continues" into itself: its first slabs are fetched again
-    // and never used, like the clamped loads of the non-persistent kernel)
+    // and never used)
     const int npid = pid + G < T ? pid + G : pid;
     tile_src(npid, a_nxt, b_nxt, nxt_m, nxt_n);
 
@@ -465,54 +487,71 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_persistent(const half
       const char* st = lds + (v & 1) * STAGE;
       __builtin_amdgcn_sched_barrier(0);
       read_frags(st, 1, fm1, fn1);
+      read_frags(st, 2, fm2, fn2);
       mfmas(fm0, fn0);
-      interleave();
+#pragma unroll
+      for (int i = 0; i < (2 * NR) % NM; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, (2 * NR) / NM + 1, 0);
+      }
+#pragma unroll
+      for (int i = (2 * NR) % NM; i < NM; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, (2 * NR) / NM, 0);
+      }
       __builtin_amdgcn_sched_barrier(0);
-      read_frags(st, 2, fm0, fn0);
+      read_frags(st, 3, fm3, fn3);
       mfmas(fm1, fn1);
-      interleave();
+#pragma unroll
+      for (int i = 0; i < (NR + 1) / 2; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, NM - (NR + 1) / 2, 0);
       __builtin_amdgcn_sched_barrier(0);
-      read_frags(st, 3, fm1, fn1);
-      mfmas(fm0, fn0);
-      interleave();
-      __builtin_amdgcn_sched_barrier(0);
-      // retire the slab: every wave's LDS reads of this stage have returned, next slab has landed
+      // retire the slab: every wave's LDS reads of this stage have returned, the next slab has landed
       asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
       __syncthreads();
       __builtin_amdgcn_sched_barrier(0);
       // loads of the slab after next (branch-free: past the end of this tile they are the next tile's
-      // slabs 0 and 1) and the first fragment reads of the next slab ride between the last MFMAs
+      // slabs 0 and 1)
       const bool wrap = kt + 2 >= KT;
       const int ls = wrap ? kt + 2 - KT : kt + 2;
-      issue_loads(v & 1, (wrap ? a_nxt : a_src) + ls * 64, (wrap ? b_nxt : b_src) + ls * 64);
-      read_frags(lds + ((v + 1) & 1) * STAGE, 0, fm0, fn0);
-      mfmas(fm1, fn1);
-      {
-        constexpr int NL = LA + LB, NR = TM + TN, NM = TM * TN;
-        constexpr int M_FOR_LOADS = NM / 2, L_PER_M = (NL + M_FOR_LOADS - 1) / M_FOR_LOADS;
+      const buffer_rsrc_t la = wrap ? a_nxt : a_src, lb = wrap ? b_nxt : b_src;
+      issue_loads(I0{}, IL2{}, v & 1, la, lb, ls);
+      mfmas(fm2, fn2);
 #pragma unroll
-        for (int i = 0; i < M_FOR_LOADS; i++) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x010, L_PER_M, 0);  // VMEM (direct-to-LDS loads)
-        }
-        constexpr int M_FOR_READS = NM - M_FOR_LOADS - 1, R_PER_M = (NR + M_FOR_READS - 1) / M_FOR_READS;
-#pragma unroll
-        for (int i = 0; i < M_FOR_READS; i++) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, R_PER_M, 0);
-        }
+      for (int i = 0; i < NL2; i++) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);  // VMEM (direct-to-LDS load)
       }
+      __builtin_amdgcn_sched_group_barrier(0x008, NM - NL2, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      read_frags(lds + ((v + 1) & 1) * STAGE, 0, fm0, fn0);
+      issue_loads(IL2{}, IL{}, v & 1, la, lb, ls);
+      mfmas(fm3, fn3);
+#pragma unroll
+      for (int i = 0; i < (NR + 1) / 2; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < NL - NL2; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, NM - (NR + 1) / 2 - (NL - NL2), 0);
       __builtin_amdgcn_sched_barrier(0);
     }
 
     // ---- epilogue of this tile; the next tile's first two slabs are already in flight ----
     if constexpr (sizeof(OutT) == 2) {
-      // 32 rows per pass through a private 4 KiB region behind the two stages: ds_write_b64 of 4
-      // consecutive n (chunk slot c ^ ((m>>1)&7)), whole rows read back 16 bytes per lane, stored as
-      // full 128-byte lines.  LDS operations of a wave execute in order, so passes need no waits between them.
+      // 32 rows per pass through a private region behind the two stages: ds_write_b64 of 4 consecutive n
+      // (swizzled 16-byte chunk slots), whole rows read back 16 bytes per lane and stored as full lines.
+      // LDS operations of a wave execute in order, so passes need no waits between them.
       char* ep = lds + 2 * STAGE + wave * EP_WAVE;
-      const int er = lane >> 3, ec = lane & 7;
+      constexpr int ROWS_PER_IT = 64 / EP_CH;
+      const int er = lane / EP_CH, ec = lane % EP_CH;
       OutT* cbase = C + (size_t)(tile_m * BM + wm * WTM) * N + tile_n * BN + wn * WTN + ec * 8;
 #pragma unroll
       for (int j = 0; j < TM; j++) {
@@ -523,14 +562,15 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_persistent(const half
             const int c = i * 4 + q;
             half4 hv = {(half_t)acc[i][j][4 * q], (half_t)acc[i][j][4 * q + 1], (half_t)acc[i][j][4 * q + 2],
                         (half_t)acc[i][j][4 * q + 3]};
-            *reinterpret_cast<half4*>(ep + r32 * 128 + ((c ^ ((r32 >> 1) & 7)) * 16) + 8 * h) = hv;
+            *reinterpret_cast<half4*>(ep + r32 * EP_ROW + ((c ^ ((r32 / EP_RPB) & (EP_CH - 1))) * 16) + 8 * h) = hv;
           }
 #pragma unroll
-        for (int it = 0; it < 4; it++) {
-          const int row = it * 8 + er;
-          half8 ov = *reinterpret_cast<const half8*>(ep + row * 128 + ((ec ^ ((row >> 1) & 7)) * 16));
+        for (int it = 0; it < 32 / ROWS_PER_IT; it++) {
+          const int row = it * ROWS_PER_IT + er;
+          half8 ov = *reinterpret_cast<const half8*>(ep + row * EP_ROW + ((ec ^ ((row / EP_RPB) & (EP_CH - 1))) * 16));
           *reinterpret_cast<half8*>(cbase + (size_t)(j * 32 + row) * N) = ov;
         }
+        __builtin_amdgcn_sched_barrier(0);  // one pass at a time: keeps the converted values of later passes out of registers
       }
     } else {
       const int m0 = tile_m * BM + wm * WTM + r32;
@@ -620,6 +660,7 @@ struct GemmVariant {
 };
 static const GemmVariant kGemmVariants[] = {
     {"persistent_256x256x64_w2x4", 256, 256, 512},
+    {"persistent_256x256x64_w2x2", 256, 256, 256},
     {"pipelined_256x256x64_w2x4", 256, 256, 512},
     {"pipelined_256x256x64_w2x2", 256, 256, 256},
     {"pipelined_128x128x64_w2x2", 128, 128, 256},
@@ -699,11 +740,12 @@ template <typename OutT>
 static int launch_variant(int variant, const void* a, const void* b, void* c, int M, int N, int K, hipStream_t stream) {
   switch (variant) {
     case 0: return launch_persistent<256, 256, 2, 4, OutT>(a, b, c, M, N, K, stream);
-    case 1: return launch_tiled<256, 256, 2, 4, OutT, true>(a, b, c, M, N, K, stream);
-    case 2: return launch_tiled<256, 256, 2, 2, OutT, true>(a, b, c, M, N, K, stream);
-    case 3: return launch_tiled<128, 128, 2, 2, OutT, true>(a, b, c, M, N, K, stream);
-    case 4: return launch_tiled<256, 256, 2, 4, OutT, false>(a, b, c, M, N, K, stream);
-    case 5: return launch_tiled<128, 128, 2, 2, OutT, false>(a, b, c, M, N, K, stream);
+    case 1: return launch_persistent<256, 256, 2, 2, OutT>(a, b, c, M, N, K, stream);
+    case 2: return launch_tiled<256, 256, 2, 4, OutT, true>(a, b, c, M, N, K, stream);
+    case 3: return launch_tiled<256, 256, 2, 2, OutT, true>(a, b, c, M, N, K, stream);
+    case 4: return launch_tiled<128, 128, 2, 2, OutT, true>(a, b, c, M, N, K, stream);
+    case 5: return launch_tiled<256, 256, 2, 4, OutT, false>(a, b, c, M, N, K, stream);
+    case 6: return launch_tiled<128, 128, 2, 2, OutT, false>(a, b, c, M, N, K, stream);
     default: {
       dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
       hipLaunchKernelGGL(gemm_f16_nt_generic<OutT>, grid, block, 0, stream, (const half_t*)a, (const half_t*)b, (OutT*)c,
@@ -728,7 +770,7 @@ extern "C" int mi355_gemm_f16_nt(const void* a, const void* b, void* c, int64_t 
   const bool al = aligned16(a) && aligned16(b) && aligned16(c);
   auto fits = [&](int v) {
     if (v == kNumGemmVariants - 1) return true;
-    if (v == 0 && K < 128) return false;  // the persistent kernel prefetches two slabs ahead
+    if (v <= 1 && (K < 128 || K > (1 << 21))) return false;  // prefetches two slabs ahead; 32-bit byte offsets inside a 256-row panel
     return al && M % kGemmVariants[v].bm == 0 && N % kGemmVariants[v].bn == 0 && K % 64 == 0;
   };
   if (variant < 0) {
@@ -737,7 +779,7 @@ extern "C" int mi355_gemm_f16_nt(const void* a, const void* b, void* c, int64_t 
     const long long t256 = (M / 256) * (N / 256);
     const long long rounds = (t256 + 255) / 256;  // 256 CUs, one 256x256 workgroup each
     if (fits(0) && t256 >= 128 && t256 * 100 >= rounds * 256 * 85) variant = 0;  // >= 85% of the last round busy
-    else if (fits(3)) variant = 3;
+    else if (fits(4)) variant = 4;
     else variant = kNumGemmVariants - 1;
   } else if (!fits(variant)) {
     return fail(-MI355_E_SHAPE, "gemm_f16_nt: variant %s needs M%%%d==0, N%%%d==0, K%%64==0 and 16-byte aligned pointers",

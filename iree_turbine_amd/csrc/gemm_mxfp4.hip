@@ -316,6 +316,268 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
   }
 }
 
+// Persistent kernel: one workgroup per CU walks its output tiles (ids pid, pid + grid, ...) as one
+// continuous sequence of K slabs, so the first slabs and scale groups of the next tile are already in
+// flight while a tile finishes, and the epilogue (through its own small LDS region) overlaps them.
+// Slab schedule, fragment register sets X, Y, Z rotating with period two slabs:
+//   k-step 0: MFMAs | LDS reads of the fragments of k-steps 1 and 2 and of the next slab's scale dwords
+//   k-step 1: MFMAs | LDS reads of k-step 3 (into the set k-step 0 just released)
+//   wait + barrier: the stage is fully read, the next slab has landed
+//   k-step 2: MFMAs | most global -> LDS loads of the slab after next (into the stage just read)
+//   k-step 3: MFMAs | LDS reads of k-step 0 of the next slab, remaining loads, every second slab the next
+//             group of scale bytes
+// Scale bytes are staged in groups of 2 slabs (16 bytes per row, one lane per row, two buffers).  The loop
+// body is unrolled by that period so it contains no branch.  Needs K % 512 == 0 and K >= 1024.
+template <int BM, int BN, int WM, int WN, typename OutT>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_persistent(const uint8_t* __restrict__ A, const uint8_t* __restrict__ As,
+                                                                     const uint8_t* __restrict__ B, const uint8_t* __restrict__ Bs,
+                                                                     OutT* __restrict__ C, int M, int N, int K, int tiles_m,
+                                                                     int tiles_n, int group_m) {
+  constexpr int NW = WM * WN;
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
+  constexpr int A_GROUPS = BM / 8, B_GROUPS = BN / 8;
+  static_assert(A_GROUPS % NW == 0 && B_GROUPS % NW == 0 && NW % 2 == 0, "loads must split evenly over an even number of waves");
+  static_assert((BM + BN) == 64 * NW && BM % 64 == 0, "one scale wave-load (64 rows x 16 bytes) per wave and group");
+  constexpr int LA = A_GROUPS / NW, LB = B_GROUPS / NW;
+  constexpr int SC_BUF = (BM + BN) * 16;  // one scale group: 16 bytes (2 slabs x 8 blocks) per row
+  constexpr int SC_BASE = 2 * STAGE, EP_BASE = SC_BASE + 2 * SC_BUF;
+  constexpr int EP_WAVE = 32 * 64;  // one epilogue pass of a wave: a 32 x 32 bf16 tile, 64-byte rows
+
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  const int T = tiles_m * tiles_n;
+  const int G = gridDim.x;
+  const int Kb = K >> 1;   // bytes per row of codes
+  const int Ksc = K >> 5;  // scale bytes per row
+  const int KT = K / 256;  // even, >= 4 (checked by the host)
+
+  const int lrow = lane >> 3;
+  const int lchunk = (lane & 7) ^ (((wave & 1) << 2) | (lrow >> 1));
+  const unsigned lane_off = (unsigned)lrow * (unsigned)Kb + (unsigned)lchunk * 16u;
+  const unsigned row_step = (unsigned)NW * 8u * (unsigned)Kb;
+  const unsigned panel_a = (unsigned)(BM - wave * 8) * (unsigned)Kb, panel_b = (unsigned)(BN - wave * 8) * (unsigned)Kb;
+  // scale rows: wave w stages rows 64w .. 64w+63 of the tile's BM A rows followed by its BN B rows
+  const bool sc_is_a = wave * 64 < BM;
+  const unsigned sc_lane_off = (unsigned)lane * (unsigned)Ksc;
+
+  auto tile_src = [&](int pid, buffer_rsrc_t& a_src, buffer_rsrc_t& b_src, buffer_rsrc_t& sc_src, int& tile_m, int& tile_n) {
+    map_tile_mx(pid, tiles_m, tiles_n, group_m, tile_m, tile_n);
+    a_src = make_buffer(A + (size_t)(tile_m * BM + wave * 8) * Kb, panel_a);
+    b_src = make_buffer(B + (size_t)(tile_n * BN + wave * 8) * Kb, panel_b);
+    const uint8_t* sp = sc_is_a ? As + (size_t)(tile_m * BM + wave * 64) * Ksc : Bs + (size_t)(tile_n * BN + wave * 64 - BM) * Ksc;
+    sc_src = make_buffer(sp, 64u * (unsigned)Ksc);
+  };
+  auto issue_loads = [&](auto first_tag, auto last_tag, int stage, buffer_rsrc_t ap, buffer_rsrc_t bp, int slab) __attribute__((always_inline)) {
+    constexpr int FIRST = decltype(first_tag)::value, LAST = decltype(last_tag)::value;
+    char* dst = lds + stage * STAGE + wave * 1024;
+    const unsigned k_off = (unsigned)slab * 128u;
+#pragma unroll
+    for (int i = 0; i < LA; i++)
+      if (i >= FIRST && i < LAST) buffer_load_lds_16B(ap, lane_off, k_off + i * row_step, dst + i * NW * 1024);
+#pragma unroll
+    for (int i = 0; i < LB; i++)
+      if (LA + i >= FIRST && LA + i < LAST) buffer_load_lds_16B(bp, lane_off, k_off + i * row_step, dst + A_BYTES + i * NW * 1024);
+  };
+  auto issue_scale_loads = [&](int buf, buffer_rsrc_t sp, int group) {
+    buffer_load_lds_16B(sp, sc_lane_off, (unsigned)group * 16u, lds + SC_BASE + buf * SC_BUF + wave * 1024);
+  };
+
+  const int r32 = lane & 31, h = lane >> 5;
+  const int sw = ((4 * h) ^ ((r32 >> 1) & 7)) * 16;  // chunk ks + 4h of the row, swizzled
+  const int a_base = (wm * WTM + r32) * 128 + sw;
+  const int b_base = A_BYTES + (wn * WTN + r32) * 128 + sw;
+  auto read_frags = [&](const char* st, int ks, intx4* fm, intx4* fn) {
+#pragma unroll
+    for (int j = 0; j < TM; j++) fm[j] = *reinterpret_cast<const intx4*>(st + ((a_base ^ (ks * 16)) + j * 4096));
+#pragma unroll
+    for (int i = 0; i < TN; i++) fn[i] = *reinterpret_cast<const intx4*>(st + ((b_base ^ (ks * 16)) + i * 4096));
+  };
+  // scale dword (bytes 4h .. 4h+3 of the row's 8 bytes of a slab) of virtual slab v
+  const int sa_off = (wm * WTM + r32) * 16 + 4 * h, sb_off = (BM + wn * WTN + r32) * 16 + 4 * h;
+  auto fetch_scales = [&](int* da, int* db, int v) {
+    const char* buf = lds + SC_BASE + ((v >> 1) & 1) * SC_BUF + (v & 1) * 8;
+#pragma unroll
+    for (int j = 0; j < TM; j++) da[j] = *reinterpret_cast<const int*>(buf + sa_off + j * 512);
+#pragma unroll
+    for (int i = 0; i < TN; i++) db[i] = *reinterpret_cast<const int*>(buf + sb_off + i * 512);
+  };
+
+  floatx16 acc[TN][TM];
+  auto zero_acc = [&]() {
+#pragma unroll
+    for (int i = 0; i < TN; i++)
+#pragma unroll
+      for (int j = 0; j < TM; j++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+  };
+  zero_acc();
+  auto mfmas = [&](auto ks_tag, const intx4* fm, const intx4* fn, const int* ca, const int* cb) __attribute__((always_inline)) {
+    constexpr int KS = decltype(ks_tag)::value;
+#pragma unroll
+    for (int i = 0; i < TN; i++)
+#pragma unroll
+      for (int j = 0; j < TM; j++) acc[i][j] = mfma_fp4_32x32x64<KS>(fn[i], cb[i], fm[j], ca[j], acc[i][j]);
+  };
+
+  constexpr int NM = TM * TN, NR = TM + TN, NL = LA + LB;
+  constexpr int NL2 = NL < NM ? (3 * NL) / 4 : NM - 2;  // loads issued in k-step 2
+  static_assert(3 * NR <= 2 * NM + 2 && NL - NL2 + 1 + (NR + 1) / 2 < NM, "k-step regions too small for their memory work");
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+  using I2 = std::integral_constant<int, 2>;
+  using I3 = std::integral_constant<int, 3>;
+  using IL2 = std::integral_constant<int, NL2>;
+  using IL = std::integral_constant<int, NL>;
+
+  intx4 fmx[TM], fnx[TN], fmy[TM], fny[TN], fmz[TM], fnz[TN];
+  int sa[2][TM], sb[2][TN];
+
+  int pid = blockIdx.x;
+  if (pid >= T) return;
+  buffer_rsrc_t a_src, b_src, s_src, a_nxt, b_nxt, s_nxt;
+  int tile_m, tile_n, nxt_m, nxt_n;
+  tile_src(pid, a_src, b_src, s_src, tile_m, tile_n);
+  issue_scale_loads(0, s_src, 0);
+  issue_scale_loads(1, s_src, 1);
+  issue_loads(I0{}, IL{}, 0, a_src, b_src, 0);
+  wait_vmcnt0();
+  __syncthreads();
+  issue_loads(I0{}, IL{}, 1, a_src, b_src, 1);
+  fetch_scales(sa[0], sb[0], 0);
+  read_frags(lds, 0, fmx, fnx);
+  int v = 0;  // slabs retired so far (even at every tile start: KT is even)
+
+  // One slab; PAR = its parity.  Even slabs run k-steps 0..3 on sets X, Y, Z, X and leave the next
+  // slab's first fragments in Y; odd slabs run on Y, Z, X, Y and leave them in X.
+  auto slab = [&](auto par_tag, int kt, intx4* f0m, intx4* f0n, intx4* f1m, intx4* f1n, intx4* f2m, intx4* f2n) __attribute__((always_inline)) {
+    constexpr int PAR = decltype(par_tag)::value;
+    const char* st = lds + PAR * STAGE;
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(st, 1, f1m, f1n);
+    read_frags(st, 2, f2m, f2n);
+    fetch_scales(sa[PAR ^ 1], sb[PAR ^ 1], v + 1);
+    mfmas(I0{}, f0m, f0n, sa[PAR], sb[PAR]);
+#pragma unroll
+    for (int i = 0; i < NM; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, (3 * NR + NM - 1) / NM, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(st, 3, f0m, f0n);  // k-step 0's set is free again
+    mfmas(I1{}, f1m, f1n, sa[PAR], sb[PAR]);
+#pragma unroll
+    for (int i = 0; i < (NR + 1) / 2; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, NM - (NR + 1) / 2, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    // retire the slab: every wave's LDS reads of this stage have returned, the next slab has landed
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    // loads of the slab after next (branch-free: past the end of this tile they belong to the next tile)
+    const bool wrap = kt + 2 >= KT;
+    const int ls = wrap ? kt + 2 - KT : kt + 2;
+    const buffer_rsrc_t la = wrap ? a_nxt : a_src, lb = wrap ? b_nxt : b_src;
+    issue_loads(I0{}, IL2{}, PAR, la, lb, ls);
+    mfmas(I2{}, f2m, f2n, sa[PAR], sb[PAR]);
+#pragma unroll
+    for (int i = 0; i < NL2; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, NM - NL2, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    // next slab's first fragments: into Y after an even slab (k-step 1's set), into X after an odd one
+    // (k-step 2's set) -- both idle by now
+    if constexpr (PAR == 0) read_frags(lds + STAGE, 0, f1m, f1n);
+    else read_frags(lds, 0, f2m, f2n);
+    issue_loads(IL2{}, IL{}, PAR, la, lb, ls);
+    if constexpr (PAR == 1) {
+      // The group two ahead replaces the group of this slab pair: its dwords went into registers during
+      // the previous slab, before the barrier above.
+      const int g = (kt >> 1) + 2, KG = KT >> 1;
+      const bool gwrap = g >= KG;
+      issue_scale_loads((v >> 1) & 1, gwrap ? s_nxt : s_src, gwrap ? g - KG : g);
+    }
+    mfmas(I3{}, f0m, f0n, sa[PAR], sb[PAR]);
+#pragma unroll
+    for (int i = 0; i < (NR + 1) / 2; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < NL - NL2 + PAR; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, NM - (NR + 1) / 2 - (NL - NL2 + PAR), 0);
+    __builtin_amdgcn_sched_barrier(0);
+    v++;
+  };
+
+  for (; pid < T; pid += G) {
+    const int npid = pid + G < T ? pid + G : pid;  // the last tile "continues" into itself; those loads are never used
+    tile_src(npid, a_nxt, b_nxt, s_nxt, nxt_m, nxt_n);
+    for (int kt = 0; kt < KT; kt += 2) {
+      slab(I0{}, kt, fmx, fnx, fmy, fny, fmz, fnz);
+      slab(I1{}, kt + 1, fmy, fny, fmz, fnz, fmx, fnx);
+    }
+
+    // ---- epilogue of this tile; the next tile's first slabs and scale groups are already in flight ----
+    const int m0 = tile_m * BM + wm * WTM, n0 = tile_n * BN + wn * WTN;
+    if constexpr (sizeof(OutT) == 2) {
+      // one 32 x 32 MFMA tile per pass through a private 2 KiB region: 8-byte writes of 4 consecutive n
+      // (chunk slot q ^ ((m>>2)&3)), whole 64-byte rows read back 16 bytes per lane.  LDS operations of a
+      // wave execute in order, so passes need no waits between them.
+      char* ep = lds + EP_BASE + wave * EP_WAVE;
+      const int er = lane >> 2, ec = lane & 3;
+#pragma unroll
+      for (int j = 0; j < TM; j++)
+#pragma unroll
+        for (int i = 0; i < TN; i++) {
+#pragma unroll
+          for (int q = 0; q < 4; q++) {
+            ushortx4 pv = {f32_to_bf16_rne(acc[i][j][4 * q]), f32_to_bf16_rne(acc[i][j][4 * q + 1]),
+                           f32_to_bf16_rne(acc[i][j][4 * q + 2]), f32_to_bf16_rne(acc[i][j][4 * q + 3])};
+            *reinterpret_cast<ushortx4*>(ep + r32 * 64 + ((q ^ ((r32 >> 2) & 3)) * 16) + 8 * h) = pv;
+          }
+#pragma unroll
+          for (int it = 0; it < 2; it++) {
+            const int row = it * 16 + er;
+            intx4 ov = *reinterpret_cast<const intx4*>(ep + row * 64 + ((ec ^ ((row >> 2) & 3)) * 16));
+            *reinterpret_cast<intx4*>(C + (size_t)(m0 + j * 32 + row) * N + n0 + i * 32 + ec * 8) = ov;
+          }
+          __builtin_amdgcn_sched_barrier(0);  // one pass at a time
+        }
+    } else {
+#pragma unroll
+      for (int j = 0; j < TM; j++) {
+        OutT* crow = C + (size_t)(m0 + r32 + j * 32) * N + n0 + 4 * h;
+#pragma unroll
+        for (int i = 0; i < TN; i++)
+#pragma unroll
+          for (int q = 0; q < 4; q++)
+            MxOut<OutT>::store4(crow + i * 32 + q * 8, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                                acc[i][j][4 * q + 3]);
+      }
+    }
+    zero_acc();
+    a_src = a_nxt;
+    b_src = b_nxt;
+    s_src = s_nxt;
+    tile_m = nxt_m;
+    tile_n = nxt_n;
+  }
+  wait_vmcnt0();  // loads issued past the last tile still target LDS: let them land before the block ends
+}
+
 // Any-shape kernel (K % 32 == 0): 32x32 output tile per wave, 4 waves per workgroup along N,
 // operands fetched straight from global memory in fragment layout with bounds checks.
 template <typename OutT>
@@ -477,6 +739,7 @@ struct MxVariant {
   int bm, bn;
 };
 static const MxVariant kMxVariants[] = {
+    {"persistent_256x256x256_w2x4", 256, 256},
     {"tiled_256x256x256_w2x4", 256, 256},
     {"tiled_128x128x256_w2x2", 128, 128},
     {"skinny_m32_n32_w8", 32, 32},
@@ -508,17 +771,56 @@ static int launch_mx_tiled(const void* a, const void* as, const void* b, const v
   return check_launch("gemm_mxfp4_tiled", grid, block, lds_bytes);
 }
 
+static int mx_cu_count() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
+template <int BM, int BN, int WM, int WN, typename OutT>
+static int launch_mx_persistent(const void* a, const void* as, const void* b, const void* bs, void* c, int M, int N, int K,
+                                hipStream_t stream) {
+  auto kern = gemm_mxfp4_persistent<BM, BN, WM, WN, OutT>;
+  // two data stages, two scale groups of 16 bytes per row, one 2 KiB epilogue pass per wave
+  constexpr int lds_bytes = 2 * (BM + BN) * 128 + 2 * (BM + BN) * 16 + WM * WN * 2048;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       lds_bytes);
+    if (e != hipSuccess) {
+      set_error("hipFuncSetAttribute(gemm_mxfp4_persistent, %d bytes LDS): %s", lds_bytes, hipGetErrorString(e));
+      return (int)e;
+    }
+    attr_set = true;
+  }
+  const int tiles_m = M / BM, tiles_n = N / BN;
+  const int T = tiles_m * tiles_n;
+  int g = mx_cu_count() & ~7;  // multiples of 8 keep a workgroup's tiles on the XCD it runs on
+  if (g < 8) g = 8;
+  dim3 grid(T < g ? T : g), block(WM * WN * 64);
+  hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const uint8_t*)a, (const uint8_t*)as, (const uint8_t*)b,
+                     (const uint8_t*)bs, (OutT*)c, M, N, K, tiles_m, tiles_n, 4);
+  return check_launch("gemm_mxfp4_persistent", grid, block, lds_bytes);
+}
+
 template <typename OutT>
 static int launch_mx(int variant, const void* a, const void* as, const void* b, const void* bs, void* c, int M, int N, int K,
                      hipStream_t stream) {
   switch (variant) {
-    case 0:
+    case 0: return launch_mx_persistent<256, 256, 2, 4, OutT>(a, as, b, bs, c, M, N, K, stream);
+    case 1:
       if (K % 1024 == 0) return launch_mx_tiled<256, 256, 2, 4, OutT, true>(a, as, b, bs, c, M, N, K, stream);
       return launch_mx_tiled<256, 256, 2, 4, OutT, false>(a, as, b, bs, c, M, N, K, stream);
-    case 1:
+    case 2:
       if (K % 1024 == 0) return launch_mx_tiled<128, 128, 2, 2, OutT, true>(a, as, b, bs, c, M, N, K, stream);
       return launch_mx_tiled<128, 128, 2, 2, OutT, false>(a, as, b, bs, c, M, N, K, stream);
-    case 2: {
+    case 3: {
       auto kern = gemm_mxfp4_skinny<OutT>;
       constexpr int lds_bytes = 8 * 16384;
       static bool attr_set = false;
@@ -561,9 +863,11 @@ extern "C" int mi355_mxfp4_gemm(const void* a, const void* a_scale, const void* 
     return fail(-MI355_E_ALIGN, "mxfp4_gemm: a, b, c must be 16-byte aligned");
   const bool sc_al = ((reinterpret_cast<uintptr_t>(a_scale) | reinterpret_cast<uintptr_t>(b_scale)) & 7u) == 0;
   const bool sc_al4 = ((reinterpret_cast<uintptr_t>(a_scale) | reinterpret_cast<uintptr_t>(b_scale)) & 3u) == 0;
+  const bool sc_al16 = ((reinterpret_cast<uintptr_t>(a_scale) | reinterpret_cast<uintptr_t>(b_scale)) & 15u) == 0;
   auto fits = [&](int v) {
     if (v == kNumMxVariants - 1) return true;
-    if (v == 2) return sc_al4 && M <= 32 && N % 32 == 0 && K % 256 == 0;  // skinny: whole 128-byte segments
+    if (v == 3) return sc_al4 && M <= 32 && N % 32 == 0 && K % 256 == 0;  // skinny: whole 128-byte segments
+    if (v == 0 && !(sc_al16 && K % 512 == 0 && K >= 1024 && K <= (1 << 22))) return false;  // persistent: 2-slab scale groups
     return sc_al && M % kMxVariants[v].bm == 0 && N % kMxVariants[v].bn == 0 && K % 256 == 0;
   };
   if (variant < 0) {
@@ -572,9 +876,11 @@ extern "C" int mi355_mxfp4_gemm(const void* a, const void* a_scale, const void* 
     // is at least 85 % full.
     const long long t256 = (M / 256) * (N / 256);
     const long long rounds = (t256 + 255) / 256;
-    if (fits(2)) variant = 2;
-    else if (fits(0) && t256 >= 128 && t256 * 100 >= rounds * 256 * 85) variant = 0;
-    else if (fits(1)) variant = 1;
+    const bool big = t256 >= 128 && t256 * 100 >= rounds * 256 * 85;
+    if (fits(3)) variant = 3;
+    else if (big && fits(0)) variant = 0;
+    else if (big && fits(1)) variant = 1;
+    else if (fits(2)) variant = 2;
     else variant = kNumMxVariants - 1;
   } else if (!fits(variant)) {
     return fail(-MI355_E_SHAPE, "mxfp4_gemm: variant %s does not fit M=%lld N=%lld K=%lld (tile %dx%d, K%%256==0, aligned scales)",

@@ -43,7 +43,7 @@ def test_dequant_random_bit_exact(dev):
     assert np.array_equal(out.view(np.uint32), om.mxfp4_dequant_ref(a, asc).view(np.uint32))
 
 
-@pytest.mark.parametrize("variant", [-1, 0, 1, 3])
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 4])
 def test_mxfp4_gemm_variants(dev, variant):
     import iree_turbine_amd  # noqa: F401
     from oracle import inputs, mxfp4 as om
@@ -74,9 +74,9 @@ def test_mxfp4_gemm_ragged(dev, shape):
 
 
 @pytest.mark.parametrize("shape", [(32, 256, 512), (1, 64, 256), (7, 96, 2048), (32, 8192, 8192), (20, 160, 16384), (32, 64, 8192 + 256)])
-@pytest.mark.parametrize("variant", [2, 3])
+@pytest.mark.parametrize("variant", [3, 4])
 def test_mxfp4_skinny_vs_generic(dev, shape, variant):
-    """The weight-streaming kernel (variant 2) and the any-shape kernel (variant 3) on skinny shapes."""
+    """The weight-streaming kernel (variant 3) and the any-shape kernel (variant 4) on skinny shapes."""
     import iree_turbine_amd  # noqa: F401
     from oracle import inputs, mxfp4 as om
 
@@ -173,6 +173,33 @@ def test_mxfp4_full_size_repeatable(dev, shape):
             assert torch.equal(first, torch.ops.mi355.mxfp4_gemm(a, asc, b, bsc, "float32", variant)), names[variant]
         assert _rel_err(first, generic) < 1e-5, names[variant]
     assert ran >= 1
+
+
+@pytest.mark.parametrize("shape", [(4352, 4352, 1024), (4096, 4608, 1536), (512, 256, 8192)])
+@pytest.mark.parametrize("out_dtype", ["bfloat16", "float32"])
+def test_mxfp4_persistent_tile_walk(dev, shape, out_dtype):
+    """The persistent kernel walks several tiles per workgroup as one slab sequence: more tiles than CUs,
+    tile counts that are not multiples of 8 or of the grid, an odd number of scale groups per tile (the
+    scale buffer parity flips between tiles), the minimum K, fewer tiles than CUs -- whole matrix against
+    the independent generic kernel."""
+    import iree_turbine_amd as ita
+    from oracle import inputs
+
+    M, N, K = shape
+    announce(f"mxfp4 persistent walk {shape} {out_dtype}")
+    names = ita._lib.variants("mxfp4_gemm")
+    assert names[0].startswith("persistent")
+    a, asc, b, bsc = [t.to(dev) for t in inputs.mxfp4_inputs(M, N, K)]
+    got = torch.ops.mi355.mxfp4_gemm(a, asc, b, bsc, out_dtype, 0)
+    ref = torch.ops.mi355.mxfp4_gemm(a, asc, b, bsc, out_dtype, len(names) - 1)
+    if out_dtype == "float32":
+        assert _rel_err(got, ref) < 1e-5
+    else:
+        # both round the same fp32 sums (up to summation order) to bf16: at most one bf16 step apart,
+        # plus the summation-order noise of sums that cancel to nearly nothing
+        g32, r32 = got.float(), ref.float()
+        assert _rel_err(g32, r32) < 1e-3
+        assert ((g32 - r32).abs() <= r32.abs() * 2 ** -7 + 1e-5 * r32.abs().max()).all()
 
 
 def test_mxfp4_contract_errors(dev):
