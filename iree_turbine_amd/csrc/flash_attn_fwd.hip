@@ -384,8 +384,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     __builtin_amdgcn_sched_barrier(0);
     l_run += psum;
     // O^T += V^T P^T: 16 MFMAs, each V^T fragment (two transpose reads) requested two MFMAs ahead.
-    // The order is pinned step by step (scheduling groups are not used here: hoisting the transpose
-    // reads with sched_group_barrier produced wrong results).
+    // The order is pinned step by step.
     auto vr = [&](int i) {  // i = t16*4 + dt
       const char* va = lds + voff + (i >> 2) * 4096 + (v_base ^ ((i & 3) * 64));
       half4 lo = lds_read_tr16(va);
