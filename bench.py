@@ -171,6 +171,21 @@ def wl_mxfp4(M, N, K):
     return build
 
 
+def wl_quantize(rows, K):
+    def build(dev):
+        g = torch.Generator().manual_seed(10)
+        x = (torch.randn(rows, K, generator=g) * 0.1).half()
+        xd = x.to(dev)
+        nbytes = rows * K * (2 + 0.5 + 1 / 32)
+        return {
+            "fn": lambda: torch.ops.mi355.mxfp4_quantize(xd),
+            "work": nbytes, "bytes": nbytes, "bound": "hbm", "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "dtype": "f16 -> fp4(e2m1)+e8m0", "cpu": lambda: cpu_quantize(x),
+            "config": {"workload": f"mxfp4_quantize_{rows}x{K}_f16in", "rows": rows, "K": K, "seed": 10},
+        }
+    return build
+
+
 def wl_copy(nbytes=1 << 30):
     """Plain device copy of a known size: the calibration point for the HBM traffic counters."""
     def build(dev):
@@ -196,6 +211,7 @@ WORKLOADS = {
     "decode": wl_decode(),
     "mxfp4_4096x8192x8192": wl_mxfp4(4096, 8192, 8192),
     "mxfp4_32x8192x8192": wl_mxfp4(32, 8192, 8192),
+    "mxfp4_quantize_16384x16384": wl_quantize(16384, 16384),
 }
 CALIBRATION = {"copy_1GiB": wl_copy()}  # not part of the path: run only when named with --workload
 WORKLOADS_ALL = {**WORKLOADS, **CALIBRATION}
@@ -219,6 +235,14 @@ def cpu_copy(nbytes):
     dst = torch.empty_like(src)
     t = _time_cpu(lambda: dst.copy_(src))
     return {"value": 2.0 * (nbytes // 4) / t / 1e9, "unit": "GB/s", "sample": f"torch CPU copy of {nbytes >> 22} MiB"}
+
+
+def cpu_quantize(x):
+    from oracle import mxfp4 as om
+    rows = 512
+    t = _time_cpu(lambda: om.mxfp4_quantize_ref(x[:rows]), reps=2)
+    return {"value": rows * x.shape[1] * (2 + 0.5 + 1 / 32) / t / 1e9, "unit": "GB/s",
+            "sample": f"numpy quantiser on {rows} of the {x.shape[0]} rows, best of 2 after 1 warm-up"}
 
 
 def cpu_gemm(a, b, M, N, K):

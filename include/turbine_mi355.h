@@ -138,6 +138,19 @@ int mi355_mxfp4_gemm(const void* a, const void* a_scale, const void* b, const vo
 int mi355_mxfp4_dequant(const void* codes, const void* scales, float* out,
                         int64_t rows, int64_t K, void* stream);
 
+/*
+ * MXFP4 quantisation, the producer of mi355_mxfp4_gemm's operands: x [rows, K] in
+ * fp16 / bf16 / fp32 (in_dtype MI355_F16 / MI355_BF16 / MI355_F32) ->
+ * codes uint8 [rows, K/2] and scales uint8 [rows, K/32] in the layout above.
+ * Per block of 32: scale exponent floor(log2(max|x|)) - 2 clamped to [-127, 127]
+ * (all-zero block: -127; a NaN or infinity in the block: scale 0xFF), elements
+ * rounded to the nearest E2M1 value, ties to the even code, saturating at 6
+ * (OCP Microscaling Formats v1.0).  K % 32 == 0.  The reference has no producer
+ * for these dtypes; it only declares them (iree/turbine/kernel/_support/dtype.py:117,119).
+ */
+int mi355_mxfp4_quantize(const void* x, int in_dtype, int64_t rows, int64_t K,
+                         void* codes, void* scales, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

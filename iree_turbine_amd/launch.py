@@ -147,3 +147,19 @@ def mxfp4_dequant_out(codes: Tensor, scales: Tensor, out: Tensor) -> Tensor:
                                              _lib.current_stream_ptr(dev))
     _lib.check(rc, f"mxfp4_dequant rows={rows} K={K}")
     return out
+
+
+def mxfp4_quantize_out(x: Tensor, codes: Tensor, scales: Tensor) -> tuple[Tensor, Tensor]:
+    dev = _dev(x, codes, scales)
+    x = x.contiguous()
+    _contig_out(codes, "mxfp4_quantize")
+    _contig_out(scales, "mxfp4_quantize")
+    rows, K = x.shape
+    if tuple(codes.shape) != (rows, K // 2) or tuple(scales.shape) != (rows, K // 32) or codes.dtype != torch.uint8 \
+            or scales.dtype != torch.uint8:
+        raise ValueError("mxfp4_quantize: codes must be uint8 [rows, K/2] and scales uint8 [rows, K/32]")
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_mxfp4_quantize(x.data_ptr(), _lib.dtype_code(x.dtype), rows, K, codes.data_ptr(),
+                                              scales.data_ptr(), _lib.current_stream_ptr(dev))
+    _lib.check(rc, f"mxfp4_quantize rows={rows} K={K} in={x.dtype}")
+    return codes, scales

@@ -24,6 +24,7 @@ __all__ = [
     "paged_decode_phase1",
     "mxfp4_gemm",
     "mxfp4_dequant",
+    "mxfp4_quantize",
 ]
 
 _OUT_DTYPES = {"float32": torch.float32, "float16": torch.float16, "bfloat16": torch.bfloat16}
@@ -232,3 +233,24 @@ class mxfp4_dequant(CustomOp):
     def eager_execute(self, codes, scales):
         out = torch.empty((codes.shape[0], codes.shape[1] * 2), dtype=torch.float32, device=codes.device)
         return launch.mxfp4_dequant_out(codes, scales, out)
+
+
+@CustomOp.register
+class mxfp4_quantize(CustomOp):
+    """(codes uint8 [rows, K/2], scales uint8 [rows, K/32]) of x [rows, K] (fp16, bf16 or fp32): the OCP MX
+    conversion -- block exponent floor(log2(max|x|)) - 2, round to nearest E2M1, ties to the even code."""
+
+    signature = "mxfp4_quantize(Tensor x) -> (Tensor, Tensor)"
+
+    def select(self, sel: KernelSelection):
+        x = sel.arg_tensor(0)
+        _require(x.t.dim() == 2, "mxfp4_quantize: x must be [rows, K]")
+        _require(x.t.dtype in (torch.float16, torch.bfloat16, torch.float32), f"mxfp4_quantize: dtype {x.t.dtype} not supported")
+        _require(x.t.size(0) > 0 and x.t.size(1) > 0 and x.t.size(1) % 32 == 0, "mxfp4_quantize: K must be a positive multiple of 32")
+        sel.return_new_tensor([x.t.size(0), x.t.size(1) // 2], torch.uint8)
+        sel.return_new_tensor([x.t.size(0), x.t.size(1) // 32], torch.uint8)
+
+    def eager_execute(self, x):
+        codes = torch.empty((x.shape[0], x.shape[1] // 2), dtype=torch.uint8, device=x.device)
+        scales = torch.empty((x.shape[0], x.shape[1] // 32), dtype=torch.uint8, device=x.device)
+        return launch.mxfp4_quantize_out(x, codes, scales)
