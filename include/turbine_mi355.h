@@ -117,6 +117,37 @@ int mi355_paged_decode_attn(const void* q, const void* k_cache, const void* v_ca
                             int64_t num_pages, int64_t num_splits, float scale, void* stream);
 
 /*
+ * Paged decode with a sliding window: as mi355_paged_decode_attn, but a query
+ * attends only to the last `window` cached tokens of its sequence (window == 0:
+ * all of them).  Pages wholly in front of the window are not read.  Same masking
+ * convention as the causal mask of tests/dynamo/llama_test.py:160-181 restricted
+ * to a band; the reference has no paged form.
+ */
+int mi355_paged_decode_attn_window(const void* q, const void* k_cache, const void* v_cache,
+                                   const int32_t* block_table, const int32_t* seq_lens, void* out,
+                                   float* part_acc, float* part_ml,
+                                   int64_t num_seqs, int64_t num_q_heads, int64_t num_kv_heads,
+                                   int64_t D, int64_t page_size, int64_t max_pages_per_seq,
+                                   int64_t num_pages, int64_t num_splits, float scale,
+                                   int64_t window, void* stream);
+
+/*
+ * KV-cache append, the step in front of decode: the paged form of
+ *   cache_k[:bsz, start_pos : start_pos + seqlen] = xk   (tests/dynamo/llama_test.py:165-166)
+ * with a start position per sequence.
+ * k_new, v_new: [num_seqs, n_new, num_kv_heads, D] fp16; token t of sequence s is
+ * written at position start_pos[s] + t, i.e. page block_table[s][pos / page_size],
+ * slot pos % page_size of k_cache / v_cache ([num_pages, page_size, num_kv_heads, D]).
+ * Positions without a table entry (pos / page_size >= max_pages_per_seq) or whose
+ * entry is outside [0, num_pages) are skipped.  D == 128, page_size == 16.
+ */
+int mi355_kv_cache_append(const void* k_new, const void* v_new, void* k_cache, void* v_cache,
+                          const int32_t* block_table, const int32_t* start_pos,
+                          int64_t num_seqs, int64_t n_new, int64_t num_kv_heads, int64_t D,
+                          int64_t page_size, int64_t max_pages_per_seq, int64_t num_pages,
+                          void* stream);
+
+/*
  * Block-scaled MXFP4 GEMM: C[M,N] = dq(A) . dq(B)^T, fp32 accumulation, bf16 out.
  * a: uint8 [M, K/2], b: uint8 [N, K/2]  -- two E2M1 codes per byte, element 2i
  *    in the low nibble, element 2i+1 in the high nibble;

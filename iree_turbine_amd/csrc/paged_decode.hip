@@ -33,17 +33,21 @@ __global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
     const half_t* __restrict__ Q, const half_t* __restrict__ Kc, const half_t* __restrict__ Vc,
     const int* __restrict__ block_table, const int* __restrict__ seq_lens, float* __restrict__ part_acc,
     float* __restrict__ part_ml, half_t* __restrict__ out, int num_kv_heads, int max_pages_per_seq, int num_splits,
-    float scale_log2e) {
+    float scale_log2e, int window) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int split = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
   const int num_q_heads = num_kv_heads * G;
   const int L = seq_lens[seq];
-  const int pages_total = (L + 15) >> 4;
-  const int pps = (pages_total + num_splits - 1) / num_splits;
-  const int p_begin = split * pps;
-  const int p_end = (p_begin + pps < pages_total) ? p_begin + pps : pages_total;
+  // sliding window: only the last `window` tokens take part (window <= 0: all of them); pages wholly in
+  // front of the window are never touched and the splits divide the pages that remain
+  const int lo = (window > 0 && L > window) ? L - window : 0;
+  const int p_lo = lo >> 4;
+  const int p_hi = (L + 15) >> 4;
+  const int pps = (p_hi - p_lo + num_splits - 1) / num_splits;
+  const int p_begin = p_lo + split * pps;
+  const int p_end = (p_begin + pps < p_hi) ? p_begin + pps : p_hi;
   const int n_steps = p_end > p_begin ? (p_end - p_begin + 1) >> 1 : 0;
   const int* bt = block_table + (size_t)seq * max_pages_per_seq;
 
@@ -125,13 +129,13 @@ __global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
         const bool ragged = pa * 16 + 32 > L;  // wave-uniform: this step reaches past the sequence end
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-          if (tok0 + r >= L) s0[r] = -INFINITY;
-          if (!has1 || tok0 + 16 + r >= L) s1[r] = -INFINITY;
+          if (tok0 + r >= L || tok0 + r < lo) s0[r] = -INFINITY;
+          if (!has1 || tok0 + 16 + r >= L) s1[r] = -INFINITY;  // the second page of a step lies behind `lo`
         }
         float mx = fmaxf(fmaxf(fmaxf(s0[0], s0[1]), fmaxf(s0[2], s0[3])), fmaxf(fmaxf(s1[0], s1[1]), fmaxf(s1[2], s1[3])));
         mx = fmaxf(mx, __shfl_xor(mx, 16));
         mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_run, mx);  // finite: the first token of page pa is always valid
+        const float m_new = fmaxf(m_run, mx);  // finite: page pa always holds a valid token (the window's first or its own first)
         const float alpha = fast_exp2((m_run - m_new) * scale_log2e);
         const float mc = m_new * scale_log2e;
         m_run = m_new;
@@ -246,7 +250,7 @@ const char* decode_variant_name(int i) { return i == 0 ? kDecodeVariants[0] : nu
 template <int G>
 static int launch_phase0(const void* q, const void* kc, const void* vc, const int32_t* bt, const int32_t* sl, float* pacc,
                          float* pml, void* out, int num_seqs, int num_kv_heads, int max_pages, int num_splits, float scale,
-                         hipStream_t stream) {
+                         int window, hipStream_t stream) {
   auto kern = paged_decode_phase0<G>;
   constexpr int lds_bytes = PD_WAVES * PD_WAVE_LDS;
   static_assert(lds_bytes >= (int)((2 * PD_WAVES * 16 + PD_WAVES * G * 128) * sizeof(float)), "merge area must fit");
@@ -262,7 +266,7 @@ static int launch_phase0(const void* q, const void* kc, const void* vc, const in
   }
   dim3 grid(num_splits, num_kv_heads, num_seqs), block(PD_WAVES * 64);
   hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)q, (const half_t*)kc, (const half_t*)vc, bt, sl,
-                     pacc, pml, (half_t*)out, num_kv_heads, max_pages, num_splits, scale * 1.4426950408889634f);
+                     pacc, pml, (half_t*)out, num_kv_heads, max_pages, num_splits, scale * 1.4426950408889634f, window);
   return check_launch("paged_decode_phase0", grid, block, lds_bytes);
 }
 
@@ -284,10 +288,10 @@ static int check_decode_args(const char* fn, int64_t num_seqs, int64_t hq, int64
 
 static int run_phase0(const void* q, const void* kc, const void* vc, const int32_t* bt, const int32_t* sl, float* pacc,
                       float* pml, void* out, int64_t num_seqs, int64_t hq, int64_t hkv, int64_t max_pages,
-                      int64_t num_splits, float scale, hipStream_t stream) {
+                      int64_t num_splits, float scale, int window, hipStream_t stream) {
   const int G = (int)(hq / hkv);
 #define MI355_PD_CASE(GG) \
-  case GG: return launch_phase0<GG>(q, kc, vc, bt, sl, pacc, pml, out, (int)num_seqs, (int)hkv, (int)max_pages, (int)num_splits, scale, stream)
+  case GG: return launch_phase0<GG>(q, kc, vc, bt, sl, pacc, pml, out, (int)num_seqs, (int)hkv, (int)max_pages, (int)num_splits, scale, window, stream)
   switch (G) {
     MI355_PD_CASE(1);
     MI355_PD_CASE(2);
@@ -316,7 +320,7 @@ extern "C" int mi355_paged_decode_phase0(const void* q, const void* k_cache, con
   if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(part_acc))
     return fail(-MI355_E_ALIGN, "paged_decode_phase0: q, k_cache, v_cache, part_acc must be 16-byte aligned");
   return run_phase0(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, nullptr, num_seqs, num_q_heads,
-                    num_kv_heads, max_pages_per_seq, num_splits, scale, reinterpret_cast<hipStream_t>(stream));
+                    num_kv_heads, max_pages_per_seq, num_splits, scale, 0, reinterpret_cast<hipStream_t>(stream));
 }
 
 extern "C" int mi355_paged_decode_phase1(const float* part_acc, const float* part_ml, void* out, int64_t num_seqs,
@@ -331,25 +335,92 @@ extern "C" int mi355_paged_decode_phase1(const float* part_acc, const float* par
   return check_launch("paged_decode_phase1", grid, block, 0);
 }
 
+static int decode_attn(const char* fn, const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
+                       const int32_t* seq_lens, void* out, float* part_acc, float* part_ml, int64_t num_seqs,
+                       int64_t num_q_heads, int64_t num_kv_heads, int64_t D, int64_t page_size, int64_t max_pages_per_seq,
+                       int64_t num_pages, int64_t num_splits, float scale, int64_t window, void* stream) {
+  if (!q || !k_cache || !v_cache || !block_table || !seq_lens || !out) return fail(-MI355_E_NULL, "%s: null pointer", fn);
+  if (int rc = check_decode_args(fn, num_seqs, num_q_heads, num_kv_heads, D, page_size, max_pages_per_seq, num_pages,
+                                 num_splits, scale))
+    return rc;
+  if (window < 0 || window > (1ll << 30)) return fail(-MI355_E_SHAPE, "%s: window %lld out of range [0, 2^30]", fn, (long long)window);
+  if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out))
+    return fail(-MI355_E_ALIGN, "%s: q, k_cache, v_cache, out must be 16-byte aligned", fn);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (num_splits == 1)
+    return run_phase0(q, k_cache, v_cache, block_table, seq_lens, nullptr, nullptr, out, num_seqs, num_q_heads, num_kv_heads,
+                      max_pages_per_seq, 1, scale, (int)window, s);
+  if (!part_acc || !part_ml) return fail(-MI355_E_SCRATCH, "%s: num_splits > 1 needs part_acc / part_ml scratch", fn);
+  if (!aligned16(part_acc)) return fail(-MI355_E_ALIGN, "%s: part_acc must be 16-byte aligned", fn);
+  if (int rc = run_phase0(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, nullptr, num_seqs, num_q_heads,
+                          num_kv_heads, max_pages_per_seq, num_splits, scale, (int)window, s))
+    return rc;
+  return mi355_paged_decode_phase1(part_acc, part_ml, out, num_seqs, num_q_heads, D, num_splits, stream);
+}
+
 extern "C" int mi355_paged_decode_attn(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
                                        const int32_t* seq_lens, void* out, float* part_acc, float* part_ml, int64_t num_seqs,
                                        int64_t num_q_heads, int64_t num_kv_heads, int64_t D, int64_t page_size,
                                        int64_t max_pages_per_seq, int64_t num_pages, int64_t num_splits, float scale,
                                        void* stream) {
-  if (!q || !k_cache || !v_cache || !block_table || !seq_lens || !out) return fail(-MI355_E_NULL, "paged_decode_attn: null pointer");
-  if (int rc = check_decode_args("paged_decode_attn", num_seqs, num_q_heads, num_kv_heads, D, page_size, max_pages_per_seq,
-                                 num_pages, num_splits, scale))
-    return rc;
-  if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out))
-    return fail(-MI355_E_ALIGN, "paged_decode_attn: q, k_cache, v_cache, out must be 16-byte aligned");
-  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  if (num_splits == 1)
-    return run_phase0(q, k_cache, v_cache, block_table, seq_lens, nullptr, nullptr, out, num_seqs, num_q_heads, num_kv_heads,
-                      max_pages_per_seq, 1, scale, s);
-  if (!part_acc || !part_ml) return fail(-MI355_E_SCRATCH, "paged_decode_attn: num_splits > 1 needs part_acc / part_ml scratch");
-  if (!aligned16(part_acc)) return fail(-MI355_E_ALIGN, "paged_decode_attn: part_acc must be 16-byte aligned");
-  if (int rc = run_phase0(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, nullptr, num_seqs, num_q_heads,
-                          num_kv_heads, max_pages_per_seq, num_splits, scale, s))
-    return rc;
-  return mi355_paged_decode_phase1(part_acc, part_ml, out, num_seqs, num_q_heads, D, num_splits, stream);
+  return decode_attn("paged_decode_attn", q, k_cache, v_cache, block_table, seq_lens, out, part_acc, part_ml, num_seqs,
+                     num_q_heads, num_kv_heads, D, page_size, max_pages_per_seq, num_pages, num_splits, scale, 0, stream);
+}
+
+extern "C" int mi355_paged_decode_attn_window(const void* q, const void* k_cache, const void* v_cache,
+                                              const int32_t* block_table, const int32_t* seq_lens, void* out, float* part_acc,
+                                              float* part_ml, int64_t num_seqs, int64_t num_q_heads, int64_t num_kv_heads,
+                                              int64_t D, int64_t page_size, int64_t max_pages_per_seq, int64_t num_pages,
+                                              int64_t num_splits, float scale, int64_t window, void* stream) {
+  return decode_attn("paged_decode_attn_window", q, k_cache, v_cache, block_table, seq_lens, out, part_acc, part_ml, num_seqs,
+                     num_q_heads, num_kv_heads, D, page_size, max_pages_per_seq, num_pages, num_splits, scale, window, stream);
+}
+
+// ---- KV-cache append: the step in front of decode -------------------------------------------------------
+// Writes tokens start_pos[s] .. start_pos[s] + n_new - 1 of every sequence into its pages.  A token's kv
+// heads are contiguous both in the source ([seq][token][head][128]) and in a page slot, so one token is one
+// contiguous run of num_kv_heads * 256 bytes: one wave per token, 16 bytes per lane and pass.
+__global__ __launch_bounds__(256) void kv_cache_append_kernel(const half_t* __restrict__ k_new, const half_t* __restrict__ v_new,
+                                                              half_t* __restrict__ k_cache, half_t* __restrict__ v_cache,
+                                                              const int* __restrict__ block_table,
+                                                              const int* __restrict__ start_pos, int n_new, int num_kv_heads,
+                                                              int max_pages_per_seq, int num_pages, long long n_tokens) {
+  const int lane = threadIdx.x & 63;
+  const long long tok = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);  // flat (seq, new token) index
+  if (tok >= n_tokens) return;
+  const int seq = (int)(tok / n_new), t = (int)(tok - (long long)seq * n_new);
+  const int pos = start_pos[seq] + t;
+  if (pos < 0) return;
+  const int pidx = pos >> 4;
+  if (pidx >= max_pages_per_seq) return;  // no table entry for this position: nothing is written
+  const int page = block_table[(size_t)seq * max_pages_per_seq + pidx];
+  if (page < 0 || page >= num_pages) return;  // padded entry
+  const int row_halfs = num_kv_heads * 128;
+  const size_t src = (size_t)tok * row_halfs;
+  const size_t dst = ((size_t)page * 16 + (pos & 15)) * row_halfs;
+  for (int c = lane * 8; c < row_halfs; c += 512) {
+    *reinterpret_cast<half8*>(k_cache + dst + c) = *reinterpret_cast<const half8*>(k_new + src + c);
+    *reinterpret_cast<half8*>(v_cache + dst + c) = *reinterpret_cast<const half8*>(v_new + src + c);
+  }
+}
+
+extern "C" int mi355_kv_cache_append(const void* k_new, const void* v_new, void* k_cache, void* v_cache,
+                                     const int32_t* block_table, const int32_t* start_pos, int64_t num_seqs, int64_t n_new,
+                                     int64_t num_kv_heads, int64_t D, int64_t page_size, int64_t max_pages_per_seq,
+                                     int64_t num_pages, void* stream) {
+  if (!k_new || !v_new || !k_cache || !v_cache || !block_table || !start_pos) return fail(-MI355_E_NULL, "kv_cache_append: null pointer");
+  if (D != 128) return fail(-MI355_E_SHAPE, "kv_cache_append: head dim %lld not supported (only 128)", (long long)D);
+  if (page_size != 16) return fail(-MI355_E_SHAPE, "kv_cache_append: page size %lld not supported (only 16)", (long long)page_size);
+  if (num_seqs <= 0 || n_new <= 0 || num_kv_heads <= 0 || max_pages_per_seq <= 0 || num_pages <= 0 || n_new > (1 << 24) ||
+      num_kv_heads > 65535 || num_seqs * n_new > (1ll << 40))
+    return fail(-MI355_E_SHAPE, "kv_cache_append: bad sizes seqs=%lld n_new=%lld hkv=%lld max_pages=%lld num_pages=%lld",
+                (long long)num_seqs, (long long)n_new, (long long)num_kv_heads, (long long)max_pages_per_seq, (long long)num_pages);
+  if (!aligned16(k_new) || !aligned16(v_new) || !aligned16(k_cache) || !aligned16(v_cache))
+    return fail(-MI355_E_ALIGN, "kv_cache_append: k_new, v_new, k_cache, v_cache must be 16-byte aligned");
+  const long long n_tokens = num_seqs * n_new;
+  dim3 grid((unsigned)((n_tokens + 3) / 4)), block(256);
+  hipLaunchKernelGGL(kv_cache_append_kernel, grid, block, 0, reinterpret_cast<hipStream_t>(stream), (const half_t*)k_new,
+                     (const half_t*)v_new, (half_t*)k_cache, (half_t*)v_cache, block_table, start_pos, (int)n_new,
+                     (int)num_kv_heads, (int)max_pages_per_seq, (int)num_pages, n_tokens);
+  return check_launch("kv_cache_append_kernel", grid, block, 0);
 }

@@ -95,7 +95,7 @@ def paged_decode_phase1_out(part_acc: Tensor, part_ml: Tensor, out: Tensor) -> T
 
 
 def paged_decode_attn_out(q, k_cache, v_cache, block_table, seq_lens, out, scale: float, num_kv_splits: int,
-                          part_acc: Tensor | None = None, part_ml: Tensor | None = None) -> Tensor:
+                          part_acc: Tensor | None = None, part_ml: Tensor | None = None, window: int = 0) -> Tensor:
     dev = _dev(q, k_cache, v_cache, block_table, seq_lens, out)
     q, k_cache, v_cache = q.contiguous(), k_cache.contiguous(), v_cache.contiguous()
     block_table, seq_lens = block_table.contiguous(), seq_lens.contiguous()
@@ -113,12 +113,36 @@ def paged_decode_attn_out(q, k_cache, v_cache, block_table, seq_lens, out, scale
             part_ml = torch.empty((S, Hq, num_kv_splits, 2), dtype=torch.float32, device=dev)
     pa = part_acc.data_ptr() if part_acc is not None else None
     pm = part_ml.data_ptr() if part_ml is not None else None
+    if window < 0:
+        raise ValueError(f"paged_decode_attn: window must be >= 0, got {window}")
     with torch.cuda.device(dev):
-        rc = _lib.load().mi355_paged_decode_attn(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
-                                                 seq_lens.data_ptr(), out.data_ptr(), pa, pm, S, Hq, Hkv, D, page,
-                                                 block_table.shape[1], P, num_kv_splits, scale, _lib.current_stream_ptr(dev))
-    _lib.check(rc, f"paged_decode_attn seqs={S} hq={Hq} hkv={Hkv} pages={P} splits={num_kv_splits}")
+        if window == 0:
+            rc = _lib.load().mi355_paged_decode_attn(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
+                                                     seq_lens.data_ptr(), out.data_ptr(), pa, pm, S, Hq, Hkv, D, page,
+                                                     block_table.shape[1], P, num_kv_splits, scale, _lib.current_stream_ptr(dev))
+        else:
+            rc = _lib.load().mi355_paged_decode_attn_window(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                                                            block_table.data_ptr(), seq_lens.data_ptr(), out.data_ptr(), pa, pm, S,
+                                                            Hq, Hkv, D, page, block_table.shape[1], P, num_kv_splits, scale, window,
+                                                            _lib.current_stream_ptr(dev))
+    _lib.check(rc, f"paged_decode_attn seqs={S} hq={Hq} hkv={Hkv} pages={P} splits={num_kv_splits} window={window}")
     return out
+
+
+def kv_cache_append(k_new, v_new, k_cache, v_cache, block_table, start_pos) -> None:
+    """Writes k_new / v_new [S, n_new, Hkv, 128] into the paged caches in place (see mi355_kv_cache_append)."""
+    dev = _dev(k_new, v_new, k_cache, v_cache, block_table, start_pos)
+    k_new, v_new = k_new.contiguous(), v_new.contiguous()
+    block_table, start_pos = block_table.contiguous(), start_pos.contiguous()
+    _contig_out(k_cache, "kv_cache_append")
+    _contig_out(v_cache, "kv_cache_append")
+    S, n_new, Hkv, D = k_new.shape
+    P, page = k_cache.shape[0], k_cache.shape[1]
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_kv_cache_append(k_new.data_ptr(), v_new.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                                               block_table.data_ptr(), start_pos.data_ptr(), S, n_new, Hkv, D, page,
+                                               block_table.shape[1], P, _lib.current_stream_ptr(dev))
+    _lib.check(rc, f"kv_cache_append seqs={S} n_new={n_new} hkv={Hkv} pages={P}")
 
 
 def mxfp4_gemm_out(a, a_scale, b, b_scale, c: Tensor, variant: int = -1) -> Tensor:

@@ -20,6 +20,8 @@ __all__ = [
     "gemm_nt",
     "flash_attn_fwd",
     "paged_decode_attn",
+    "paged_decode_attn_window",
+    "kv_cache_append",
     "paged_decode_phase0",
     "paged_decode_phase1",
     "mxfp4_gemm",
@@ -140,6 +142,58 @@ class paged_decode_attn(CustomOp):
             num_kv_splits = default_num_kv_splits(block_table.shape[1] * k_cache.shape[1], q.shape[0], k_cache.shape[2])
         out = torch.empty(q.shape, dtype=torch.float16, device=q.device)
         return launch.paged_decode_attn_out(q, k_cache, v_cache, block_table, seq_lens, out, scale, num_kv_splits)
+
+
+@CustomOp.register
+class paged_decode_attn_window(CustomOp):
+    """paged_decode_attn restricted to the last `window` cached tokens of every sequence (window == 0: all)."""
+
+    signature = "paged_decode_attn_window(Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_table, Tensor seq_lens, float scale, int num_kv_splits, int window) -> Tensor"
+
+    def select(self, sel: KernelSelection):
+        q, kc, vc, bt, sl = (sel.arg_tensor(i) for i in range(5))
+        sel.attr_float(5)
+        sel.attr_int(6)
+        w = sel.attr_int(7).v
+        _check_paged_args("paged_decode_attn_window", q.t, kc.t, vc.t, bt.t, sl.t)
+        _require(w >= 0, "paged_decode_attn_window: window must be >= 0")
+        q.specialize_dims(1, 2)
+        kc.specialize_dims(1, 2, 3)
+        vc.specialize_dims(1, 2, 3)
+        sel.return_new_tensor(list(q.t.shape), torch.float16)
+
+    def eager_execute(self, q, k_cache, v_cache, block_table, seq_lens, scale, num_kv_splits, window):
+        if num_kv_splits <= 0:
+            span = window if window > 0 else block_table.shape[1] * k_cache.shape[1]
+            num_kv_splits = default_num_kv_splits(span, q.shape[0], k_cache.shape[2])
+        out = torch.empty(q.shape, dtype=torch.float16, device=q.device)
+        return launch.paged_decode_attn_out(q, k_cache, v_cache, block_table, seq_lens, out, scale, num_kv_splits, window=window)
+
+
+@CustomOp.register
+class kv_cache_append(CustomOp):
+    """In-place paged form of `cache[:bsz, start_pos : start_pos + n_new] = x` (tests/dynamo/llama_test.py:165-166)
+    with one start position per sequence: k_new, v_new [S, n_new, Hkv, 128] fp16 go to positions
+    start_pos[s] .. start_pos[s] + n_new - 1 of k_cache, v_cache [P, 16, Hkv, 128] through block_table [S, max_pages]."""
+
+    signature = "kv_cache_append(Tensor k_new, Tensor v_new, Tensor(a!) k_cache, Tensor(b!) v_cache, Tensor block_table, Tensor start_pos) -> ()"
+
+    def select(self, sel: KernelSelection):
+        kn, vn, kc, vc, bt, sp = (sel.arg_tensor(i) for i in range(6))
+        fn = "kv_cache_append"
+        _require(kn.t.dim() == 4 and kn.t.shape == vn.t.shape, f"{fn}: k_new and v_new must both be [S, n_new, Hkv, D]")
+        _require(kc.t.dim() == 4 and kc.t.shape == vc.t.shape, f"{fn}: k_cache and v_cache must both be [P, page, Hkv, D]")
+        _require(all(t.t.dtype == torch.float16 for t in (kn, vn, kc, vc)), f"{fn}: tensors must be float16")
+        _require(kn.t.size(3) == 128 and kc.t.size(3) == 128, f"{fn}: head dim must be 128")
+        _require(kc.t.size(1) == 16, f"{fn}: page size must be 16")
+        _require(kn.t.size(2) == kc.t.size(2), f"{fn}: k_new and k_cache disagree on the number of kv heads")
+        _require(kn.t.size(0) > 0 and kn.t.size(1) > 0, f"{fn}: empty k_new")
+        _require(bt.t.dim() == 2 and bt.t.dtype == torch.int32 and bt.t.size(0) == kn.t.size(0), f"{fn}: block_table must be int32 [S, max_pages]")
+        _require(sp.t.dim() == 1 and sp.t.dtype == torch.int32 and sp.t.size(0) == kn.t.size(0), f"{fn}: start_pos must be int32 [S]")
+
+    def eager_execute(self, k_new, v_new, k_cache, v_cache, block_table, start_pos):
+        launch.kv_cache_append(k_new, v_new, k_cache, v_cache, block_table, start_pos)
+        return None
 
 
 @CustomOp.register

@@ -125,3 +125,84 @@ def test_decode_contract_errors(dev):
         torch.ops.mi355.paged_decode_attn(q, kc[:, :8], vc[:, :8], bt, sl, 0.0, 1)  # page size 8
     with pytest.raises(ValueError):
         torch.ops.mi355.paged_decode_attn(q[:, :3], kc, vc, bt, sl, 0.0, 1)  # 3 q heads over 8 kv heads
+
+
+@pytest.mark.parametrize("window", [1, 5, 16, 17, 100, 1000, 100000])
+@pytest.mark.parametrize("splits", [1, 3])
+def test_decode_sliding_window(dev, window, splits):
+    """Windows smaller than a page, straddling pages, larger than every sequence; single and split-K."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs, paged_decode as op
+
+    announce(f"paged decode window={window} splits={splits}")
+    q, kc, vc, bt, sl = inputs.paged_decode_inputs(num_seqs=6, num_q_heads=16, num_kv_heads=4, min_len=1, max_len=700, seed=21)
+    out = torch.ops.mi355.paged_decode_attn_window(*_to(dev, q, kc, vc, bt, sl), 0.0, splits, window)
+    ref = op.paged_decode_ref(q, kc, vc, bt, sl, window=window)
+    torch.testing.assert_close(out.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+    if window >= 700:  # the window covers everything: identical to the plain op
+        assert torch.equal(out, torch.ops.mi355.paged_decode_attn(*_to(dev, q, kc, vc, bt, sl), 0.0, splits))
+
+
+def test_decode_window_ignores_tokens_in_front(dev):
+    """Tokens in front of the window may hold anything finite: the result does not move."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs
+
+    announce("paged decode window isolation")
+    q, kc, vc, bt, sl = inputs.paged_decode_inputs(num_seqs=3, num_q_heads=8, num_kv_heads=8, min_len=200, max_len=300, seed=5)
+    W = 40
+    base = torch.ops.mi355.paged_decode_attn_window(*_to(dev, q, kc, vc, bt, sl), 0.0, 2, W)
+    kc2, vc2 = kc.clone(), vc.clone()
+    for s in range(3):
+        lo = int(sl[s]) - W
+        for t in range(lo):  # overwrite everything in front of the window
+            kc2[int(bt[s, t // 16]), t % 16] = 7.0
+            vc2[int(bt[s, t // 16]), t % 16] = -9.0
+    again = torch.ops.mi355.paged_decode_attn_window(*_to(dev, q, kc2, vc2, bt, sl), 0.0, 2, W)
+    assert torch.equal(base, again)
+
+
+@pytest.mark.parametrize("n_new", [1, 5, 40])
+def test_kv_cache_append(dev, n_new):
+    """Bit-exact against slice assignment through the table; then decode over the appended cache."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs, paged_decode as op
+
+    announce(f"kv_cache_append n_new={n_new}")
+    S, Hq, Hkv = 7, 16, 4
+    q, kc, vc, bt, sl = inputs.paged_decode_inputs(num_seqs=S, num_q_heads=Hq, num_kv_heads=Hkv, min_len=64, max_len=400, seed=8)
+    g = torch.Generator().manual_seed(n_new)
+    # the new tokens fill the tail of every sequence (one of them from position 0)
+    start = (sl - n_new).clamp(min=0).int()
+    start[0] = 0
+    kn = torch.randn(S, n_new, Hkv, 128, generator=g).half()
+    vn = torch.randn(S, n_new, Hkv, 128, generator=g).half()
+    kd, vd = kc.to(dev), vc.to(dev)
+    torch.ops.mi355.kv_cache_append(kn.to(dev), vn.to(dev), kd, vd, bt.to(dev), start.to(dev))
+    kr, vr = op.kv_cache_append_ref(kn, vn, kc, vc, bt, start)
+    assert torch.equal(kd.cpu(), kr) and torch.equal(vd.cpu(), vr)
+    assert not torch.equal(kr, kc)
+    out = torch.ops.mi355.paged_decode_attn(q.to(dev), kd, vd, bt.to(dev), sl.to(dev), 0.0, 0)
+    torch.testing.assert_close(out.float().cpu(), op.paged_decode_ref(q, kr, vr, bt, sl), rtol=RTOL, atol=ATOL)
+
+
+def test_kv_cache_append_skips_positions_without_a_page(dev):
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs, paged_decode as op
+
+    announce("kv_cache_append bounds")
+    q, kc, vc, bt, sl = inputs.paged_decode_inputs(num_seqs=4, num_q_heads=8, num_kv_heads=2, min_len=20, max_len=60, seed=2)
+    kn = torch.ones(4, 3, 2, 128).half()
+    # beyond the table width, into a padded (-1) entry, negative
+    start = torch.tensor([16 * bt.shape[1] - 1, int(sl[1] + 15) // 16 * 16, -2, 0], dtype=torch.int32)
+    bt2 = bt.clone()
+    if int((sl[1] + 15) // 16) < bt.shape[1]:
+        assert bt2[1, int((sl[1] + 15) // 16)] == -1
+    kd, vd = kc.to(dev), vc.to(dev)
+    torch.ops.mi355.kv_cache_append(kn.to(dev), kn.to(dev), kd, vd, bt2.to(dev), start.to(dev))
+    kr, vr = op.kv_cache_append_ref(kn, kn, kc, vc, bt2, start)
+    assert torch.equal(kd.cpu(), kr) and torch.equal(vd.cpu(), vr)
+    with pytest.raises(ValueError):
+        torch.ops.mi355.kv_cache_append(kn.to(dev), kn.to(dev), kd, vd, bt2.to(dev), start.long().to(dev))
+    with pytest.raises(ValueError):
+        torch.ops.mi355.paged_decode_attn_window(*_to(dev, q, kc, vc, bt, sl), 0.0, 1, -1)

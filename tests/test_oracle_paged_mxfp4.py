@@ -137,3 +137,42 @@ def test_mxfp4_gemm_exact_cases_and_scaling_law():
     sc[:, 1] = 128
     exp2 = vals[ca // 2][:, :32] @ vals[cb // 2][:, :32].T + 2 * (vals[ca // 2][:, 32:] @ vals[cb // 2][:, 32:].T)
     assert np.array_equal(om.mxfp4_gemm_ref(a, sc, b, one_b).numpy(), exp2.astype(np.float32))
+
+
+def test_window_and_append_oracles():
+    """Sliding window = dense attention over the last W tokens; append = slice assignment of a dense cache."""
+    from oracle import inputs, paged_decode as op
+
+    q, kc, vc, bt, sl = inputs.paged_decode_inputs(num_seqs=5, num_q_heads=8, num_kv_heads=2, min_len=3, max_len=90, seed=4)
+    W = 20
+    out = op.paged_decode_ref(q, kc, vc, bt, sl, window=W)
+    assert torch.equal(op.paged_decode_ref(q, kc, vc, bt, sl, window=0), op.paged_decode_ref(q, kc, vc, bt, sl))
+    for s in range(5):
+        ln = int(sl[s])
+        k = op.gather_kv(kc.float(), bt[s], ln)[max(0, ln - W):]            # [w, Hkv, D]
+        v = op.gather_kv(vc.float(), bt[s], ln)[max(0, ln - W):]
+        for h in range(8):
+            p = torch.softmax((k[:, h // 4] @ q[s, h].float()) / 128 ** 0.5, dim=0)
+            torch.testing.assert_close(out[s, h], p @ v[:, h // 4], rtol=1e-5, atol=1e-6)
+    # append: a dense [S, max_len] cache gathered back through the table equals slice assignment
+    S, n_new = 5, 7
+    g = torch.Generator().manual_seed(1)
+    start = torch.tensor([0, 3, 16, 25, int(sl[4]) - n_new], dtype=torch.int32)
+    kn = torch.randn(S, n_new, 2, 128, generator=g).half()
+    vn = torch.randn(S, n_new, 2, 128, generator=g).half()
+    need = (start + n_new + 15) // 16
+    bt2 = bt.clone()
+    free = [p for p in range(kc.shape[0]) if p not in set(bt[bt >= 0].tolist())]
+    assert not free  # every page is owned; give short sequences room by re-using their own table only
+    ok = [s for s in range(S) if int(need[s]) <= int((sl[s] + 15) // 16)]
+    k2, v2 = op.kv_cache_append_ref(kn, vn, kc, vc, bt2, start)
+    for s in ok:
+        ln = int(start[s]) + n_new
+        dense = op.gather_kv(kc, bt[s], ln).clone()
+        dense[int(start[s]):ln] = kn[s]
+        assert torch.equal(op.gather_kv(k2, bt[s], ln), dense)
+    assert len(ok) >= 2
+    # a position beyond the table is skipped, not written elsewhere
+    far = torch.full((S,), 16 * bt.shape[1], dtype=torch.int32)
+    k3, v3 = op.kv_cache_append_ref(kn, vn, kc, vc, bt, far)
+    assert torch.equal(k3, kc) and torch.equal(v3, vc)
