@@ -81,6 +81,25 @@ int mi355_flash_attn_fwd(const void* q, const void* k, const void* v, void* o,
                          float scale, int is_causal, int variant, void* stream);
 
 /*
+ * The same computation on strided operands and with grouped K/V heads, so that
+ * a caller holding [B, S, H, D] projections (the `x.view(B, S, H, D).transpose(1, 2)`
+ * views a model hands to scaled_dot_product_attention) needs no copies.
+ * q, o: logical [B, H, Sq, D]; k, v: logical [B, Hkv, Sk, D] with H % Hkv == 0:
+ * query head h reads K/V head h / (H / Hkv)  (enable_gqa semantics).
+ * *_strides: {batch, head, row} strides in ELEMENTS; the D elements of a row are
+ * contiguous.  Every stride is a non-negative multiple of 8 (16-byte rows), row
+ * strides lie in [128, 2^31); a 0 batch or head stride on q, k or v broadcasts.
+ * Replaces: the same SDPA root as above for the non-contiguous operands that the
+ * reference makes contiguous before every launch
+ * (iree/turbine/runtime/op_reg/eager.py:119-132).
+ */
+int mi355_flash_attn_fwd_strided(const void* q, const void* k, const void* v, void* o,
+                                 int64_t B, int64_t H, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D,
+                                 const int64_t* q_strides, const int64_t* k_strides,
+                                 const int64_t* v_strides, const int64_t* o_strides,
+                                 float scale, int is_causal, int variant, void* stream);
+
+/*
  * Paged GQA decode attention, one query token per sequence.
  * q:           [num_seqs, num_q_heads, D]                 fp16
  * k_cache,

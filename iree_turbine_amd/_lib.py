@@ -34,6 +34,10 @@ _PROTOS = {
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_float, c_int, c_int, c_void_p],
     ),
+    "mi355_flash_attn_fwd_strided": (
+        c_int,
+        [c_void_p] * 4 + [c_int64] * 6 + [ctypes.POINTER(c_int64)] * 4 + [c_float, c_int, c_int, c_void_p],
+    ),
     "mi355_paged_decode_phase0": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]

@@ -27,10 +27,18 @@ constexpr int FA_BLOCK_M = 128;
 constexpr int FA_BLOCK_N = 64;
 constexpr int FA_STAGE = 2 * FA_BLOCK_N * 256;  // K tile + V tile, bytes
 
+// Where each operand's (batch, head, row) lives, in elements; the 128 elements of a row are contiguous.
+// `group` query heads share one K/V head (1 = plain multi-head attention).
+struct FaLayout {
+  int64_t q_b, q_h, k_b, k_h, v_b, v_h, o_b, o_h;
+  unsigned q_r, k_r, v_r, o_r;
+  int H, group;
+};
+
 template <bool CAUSAL>
 __global__ __launch_bounds__(256) void fa_fwd_d128(const half_t* __restrict__ Q, const half_t* __restrict__ K,
                                                    const half_t* __restrict__ V, half_t* __restrict__ O, int BH, int Sq,
-                                                   int Sk, float scale_log2e, int q_blocks) {
+                                                   int Sk, float scale_log2e, int q_blocks, FaLayout lay) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -41,10 +49,12 @@ __global__ __launch_bounds__(256) void fa_fwd_d128(const half_t* __restrict__ Q,
   int bh, qb;
   {
     const int pid = blockIdx.x;
-    if ((BH & 7) == 0) {
-      const int xcd = pid & 7, loc = pid >> 3;
-      bh = (loc / q_blocks) * 8 + xcd;
-      qb = loc % q_blocks;
+    if (((BH / lay.group) & 7) == 0) {
+      // all query blocks of the `group` query heads that share one K/V head sit on one XCD
+      const int xcd = pid & 7, loc = pid >> 3, per_kv = q_blocks * lay.group;
+      const int w = loc % per_kv;
+      bh = ((loc / per_kv) * 8 + xcd) * lay.group + w / q_blocks;
+      qb = w % q_blocks;
     } else {
       bh = pid / q_blocks;
       qb = pid % q_blocks;
@@ -57,10 +67,11 @@ __global__ __launch_bounds__(256) void fa_fwd_d128(const half_t* __restrict__ Q,
   const int q_row = wq0 + r32;
   const bool q_ok = q_row < Sq;
 
-  const half_t* Qb = Q + (size_t)bh * Sq * 128;
-  const half_t* Kb = K + (size_t)bh * Sk * 128;
-  const half_t* Vb = V + (size_t)bh * Sk * 128;
-  half_t* Ob = O + (size_t)bh * Sq * 128;
+  const int b_idx = bh / lay.H, h_idx = bh - b_idx * lay.H, hk_idx = h_idx / lay.group;
+  const half_t* Qb = Q + b_idx * lay.q_b + h_idx * lay.q_h;
+  const half_t* Kb = K + b_idx * lay.k_b + hk_idx * lay.k_h;
+  const half_t* Vb = V + b_idx * lay.v_b + hk_idx * lay.v_h;
+  half_t* Ob = O + b_idx * lay.o_b + h_idx * lay.o_h;
 
   // number of key tiles this workgroup walks
   int k_end = Sk;
@@ -77,7 +88,7 @@ __global__ __launch_bounds__(256) void fa_fwd_d128(const half_t* __restrict__ Q,
 #pragma unroll
   for (int ks = 0; ks < 8; ks++) {
     if (q_ok) {
-      qf[ks] = *reinterpret_cast<const half8*>(Qb + (size_t)q_row * 128 + ks * 16 + h * 8);
+      qf[ks] = *reinterpret_cast<const half8*>(Qb + (size_t)q_row * lay.q_r + ks * 16 + h * 8);
     } else {
 #pragma unroll
       for (int e = 0; e < 8; e++) qf[ks][e] = (half_t)0;
@@ -95,8 +106,8 @@ __global__ __launch_bounds__(256) void fa_fwd_d128(const half_t* __restrict__ Q,
     for (int i = 0; i < 4; i++) {
       int row = key0 + (wave + 4 * i) * 4 + lrow;
       if (row > Sk - 1) row = Sk - 1;  // clamp: the tail rows are masked out of the softmax
-      load_lds_16B(Kb + (size_t)row * 128 + k_chunk * 8, dst + i * 4096);
-      load_lds_16B(Vb + (size_t)row * 128 + v_chunk * 8, dst + FA_BLOCK_N * 256 + i * 4096);
+      load_lds_16B(Kb + (size_t)row * lay.k_r + k_chunk * 8, dst + i * 4096);
+      load_lds_16B(Vb + (size_t)row * lay.v_r + v_chunk * 8, dst + FA_BLOCK_N * 256 + i * 4096);
     }
   };
 
@@ -196,7 +207,7 @@ __global__ __launch_bounds__(256) void fa_fwd_d128(const half_t* __restrict__ Q,
   const float l_tot = l_run + __shfl_xor(l_run, 32);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   if (q_ok) {
-    half_t* orow = Ob + (size_t)q_row * 128 + 4 * h;
+    half_t* orow = Ob + (size_t)q_row * lay.o_r + 4 * h;
 #pragma unroll
     for (int dt = 0; dt < 4; dt++)
 #pragma unroll
@@ -221,7 +232,7 @@ __global__ __launch_bounds__(256) void fa_fwd_d128(const half_t* __restrict__ Q,
 template <bool CAUSAL>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void fa_fwd_d128_pipe(
     const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V, half_t* __restrict__ O, int BH,
-    int Sq, int Sk, float scale_log2e, int q_blocks) {
+    int Sq, int Sk, float scale_log2e, int q_blocks, FaLayout lay) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   constexpr int TILE_B = FA_BLOCK_N * 256;  // bytes of one K or V tile
   constexpr int VBUF = 2 * TILE_B;          // K ring at 0, V ring behind it
@@ -232,10 +243,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   int bh, qb;
   {
     const int pid = blockIdx.x;
-    if ((BH & 7) == 0) {
-      const int xcd = pid & 7, loc = pid >> 3;
-      bh = (loc / q_blocks) * 8 + xcd;
-      qb = loc % q_blocks;
+    if (((BH / lay.group) & 7) == 0) {
+      // all query blocks of the `group` query heads that share one K/V head sit on one XCD
+      const int xcd = pid & 7, loc = pid >> 3, per_kv = q_blocks * lay.group;
+      const int w = loc % per_kv;
+      bh = ((loc / per_kv) * 8 + xcd) * lay.group + w / q_blocks;
+      qb = w % q_blocks;
     } else {
       bh = pid / q_blocks;
       qb = pid % q_blocks;
@@ -248,10 +261,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int q_row = wq0 + r32;
   const bool q_ok = q_row < Sq;
 
-  const half_t* Qb = Q + (size_t)bh * Sq * 128;
-  const half_t* Kb = K + (size_t)bh * Sk * 128;
-  const half_t* Vb = V + (size_t)bh * Sk * 128;
-  half_t* Ob = O + (size_t)bh * Sq * 128;
+  const int b_idx = bh / lay.H, h_idx = bh - b_idx * lay.H, hk_idx = h_idx / lay.group;
+  const half_t* Qb = Q + b_idx * lay.q_b + h_idx * lay.q_h;
+  const half_t* Kb = K + b_idx * lay.k_b + hk_idx * lay.k_h;
+  const half_t* Vb = V + b_idx * lay.v_b + hk_idx * lay.v_h;
+  half_t* Ob = O + b_idx * lay.o_b + h_idx * lay.o_h;
 
   int k_end = Sk;
   if (CAUSAL) {
@@ -266,7 +280,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
   for (int ks = 0; ks < 8; ks++) {
     if (q_ok) {
-      qf[ks] = *reinterpret_cast<const half8*>(Qb + (size_t)q_row * 128 + ks * 16 + h * 8);
+      qf[ks] = *reinterpret_cast<const half8*>(Qb + (size_t)q_row * lay.q_r + ks * 16 + h * 8);
     } else {
 #pragma unroll
       for (int e = 0; e < 8; e++) qf[ks][e] = (half_t)0;
@@ -276,13 +290,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int lrow = lane >> 4, lslot = lane & 15;
   const int k_chunk = lslot ^ (wave * 4 + lrow);
   const int v_chunk = lslot ^ (4 * lrow);
-  auto issue_kv = [&](const half_t* base, int chunk, int tile, int lds_off) {
+  auto issue_kv = [&](const half_t* base, unsigned row_stride, int chunk, int tile, int lds_off) {
     char* dst = lds + lds_off + wave * 1024;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       int row = tile * FA_BLOCK_N + (wave + 4 * i) * 4 + lrow;
       if (row > Sk - 1) row = Sk - 1;  // clamp: tail rows are masked out of the softmax
-      load_lds_16B(base + (size_t)row * 128 + chunk * 8, dst + i * 4096);
+      load_lds_16B(base + (size_t)row * row_stride + chunk * 8, dst + i * 4096);
     }
   };
 
@@ -404,9 +418,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
   floatx16 sa[2], sb[2];
   if (n_tiles > 0) {
-    issue_kv(Kb, k_chunk, 0, 0);
-    issue_kv(Vb, v_chunk, 0, VBUF);
-    if (n_tiles > 1) issue_kv(Kb, k_chunk, 1, TILE_B);
+    issue_kv(Kb, lay.k_r, k_chunk, 0, 0);
+    issue_kv(Vb, lay.v_r, v_chunk, 0, VBUF);
+    if (n_tiles > 1) issue_kv(Kb, lay.k_r, k_chunk, 1, TILE_B);
     wait_vmcnt0();
     __syncthreads();
     if (wave_active(0)) scores(0, sa);
@@ -419,8 +433,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   auto trip = [&](auto par_tag, int j, floatx16* s_cur, floatx16* s_next) {
     constexpr int PAR = decltype(par_tag)::value;
     constexpr int K_CUR = PAR * TILE_B, K_NEXT = (1 - PAR) * TILE_B, V_CUR = PAR * TILE_B, V_NEXT = VBUF + (1 - PAR) * TILE_B;
-    if (j + 2 < n_tiles) issue_kv(Kb, k_chunk, j + 2, K_CUR);
-    if (j + 1 < n_tiles) issue_kv(Vb, v_chunk, j + 1, V_NEXT);
+    if (j + 2 < n_tiles) issue_kv(Kb, lay.k_r, k_chunk, j + 2, K_CUR);
+    if (j + 1 < n_tiles) issue_kv(Vb, lay.v_r, v_chunk, j + 1, V_NEXT);
     if (wave_active(j)) softmax_pv(std::true_type{}, j, V_CUR, s_cur, K_NEXT, s_next);  // idle from here on otherwise
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
@@ -433,7 +447,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const float l_tot = l_run + __shfl_xor(l_run, 32);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   if (q_ok) {
-    half_t* orow = Ob + (size_t)q_row * 128 + 4 * h;
+    half_t* orow = Ob + (size_t)q_row * lay.o_r + 4 * h;
 #pragma unroll
     for (int dt = 0; dt < 4; dt++)
 #pragma unroll
@@ -453,17 +467,20 @@ const char* fa_variant_name(int i) { return (i >= 0 && i < 2) ? kFaVariants[i] :
 
 using namespace mi355;
 
-extern "C" int mi355_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, int64_t B, int64_t H, int64_t Sq,
-                                    int64_t Sk, int64_t D, float scale, int is_causal, int variant, void* stream) {
-  if (!q || !k || !v || !o) return fail(-MI355_E_NULL, "flash_attn_fwd: null pointer");
-  if (D != 128) return fail(-MI355_E_SHAPE, "flash_attn_fwd: head dim %lld not supported (only 128)", (long long)D);
+static int fa_launch(const void* q, const void* k, const void* v, void* o, int64_t B, int64_t H, int64_t Hkv, int64_t Sq,
+                     int64_t Sk, int64_t D, const FaLayout& lay, float scale, int is_causal, int variant, void* stream,
+                     const char* who) {
+  if (!q || !k || !v || !o) return fail(-MI355_E_NULL, "%s: null pointer", who);
+  if (D != 128) return fail(-MI355_E_SHAPE, "%s: head dim %lld not supported (only 128)", who, (long long)D);
   if (B <= 0 || H <= 0 || Sq <= 0 || Sk <= 0 || B * H > (1 << 24) || Sq > (1 << 24) || Sk > (1 << 24))
-    return fail(-MI355_E_SHAPE, "flash_attn_fwd: bad shape B=%lld H=%lld Sq=%lld Sk=%lld", (long long)B, (long long)H,
-                (long long)Sq, (long long)Sk);
+    return fail(-MI355_E_SHAPE, "%s: bad shape B=%lld H=%lld Sq=%lld Sk=%lld", who, (long long)B, (long long)H, (long long)Sq,
+                (long long)Sk);
+  if (Hkv <= 0 || H % Hkv != 0)
+    return fail(-MI355_E_SHAPE, "%s: %lld query heads over %lld key/value heads", who, (long long)H, (long long)Hkv);
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o))
-    return fail(-MI355_E_ALIGN, "flash_attn_fwd: q, k, v, o must be 16-byte aligned");
-  if (variant > 1) return fail(-MI355_E_DTYPE, "flash_attn_fwd: variant %d out of range", variant);
-  if (!(scale > 0.f) || !isfinite(scale)) return fail(-MI355_E_SHAPE, "flash_attn_fwd: scale must be positive and finite");
+    return fail(-MI355_E_ALIGN, "%s: q, k, v, o must be 16-byte aligned", who);
+  if (variant > 1) return fail(-MI355_E_DTYPE, "%s: variant %d out of range", who, variant);
+  if (!(scale > 0.f) || !isfinite(scale)) return fail(-MI355_E_SHAPE, "%s: scale must be positive and finite", who);
   const int BH = (int)(B * H);
   const int q_blocks = (int)((Sq + FA_BLOCK_M - 1) / FA_BLOCK_M);
   const int lds_bytes = 2 * FA_STAGE;
@@ -487,6 +504,39 @@ extern "C" int mi355_flash_attn_fwd(const void* q, const void* k, const void* v,
   auto kern = variant == 1 ? (is_causal ? fa_fwd_d128<true> : fa_fwd_d128<false>)
                            : (is_causal ? fa_fwd_d128_pipe<true> : fa_fwd_d128_pipe<false>);
   hipLaunchKernelGGL(kern, grid, block, lds_bytes, s, (const half_t*)q, (const half_t*)k, (const half_t*)v, (half_t*)o, BH,
-                     (int)Sq, (int)Sk, scale_log2e, q_blocks);
+                     (int)Sq, (int)Sk, scale_log2e, q_blocks, lay);
   return check_launch(variant == 1 ? "fa_fwd_d128" : "fa_fwd_d128_pipe", grid, block, lds_bytes);
+}
+
+extern "C" int mi355_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, int64_t B, int64_t H, int64_t Sq,
+                                    int64_t Sk, int64_t D, float scale, int is_causal, int variant, void* stream) {
+  FaLayout lay;
+  lay.q_b = H * Sq * 128, lay.q_h = Sq * 128, lay.q_r = 128;
+  lay.o_b = lay.q_b, lay.o_h = lay.q_h, lay.o_r = 128;
+  lay.k_b = lay.v_b = H * Sk * 128, lay.k_h = lay.v_h = Sk * 128, lay.k_r = lay.v_r = 128;
+  lay.H = (int)H, lay.group = 1;
+  return fa_launch(q, k, v, o, B, H, H, Sq, Sk, D, lay, scale, is_causal, variant, stream, "flash_attn_fwd");
+}
+
+extern "C" int mi355_flash_attn_fwd_strided(const void* q, const void* k, const void* v, void* o, int64_t B, int64_t H,
+                                            int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, const int64_t* q_strides,
+                                            const int64_t* k_strides, const int64_t* v_strides, const int64_t* o_strides,
+                                            float scale, int is_causal, int variant, void* stream) {
+  const char* who = "flash_attn_fwd_strided";
+  if (!q_strides || !k_strides || !v_strides || !o_strides) return fail(-MI355_E_NULL, "%s: null stride array", who);
+  const int64_t* all[4] = {q_strides, k_strides, v_strides, o_strides};
+  for (const int64_t* st : all) {
+    for (int i = 0; i < 3; i++)
+      if (st[i] < 0 || (st[i] & 7)) return fail(-MI355_E_ALIGN, "%s: strides must be non-negative multiples of 8 elements", who);
+    if (st[2] < 128 || st[2] >= (1ll << 31))
+      return fail(-MI355_E_SHAPE, "%s: row stride %lld outside [128, 2^31)", who, (long long)st[2]);
+  }
+  if ((B > 1 && o_strides[0] == 0) || (H > 1 && o_strides[1] == 0)) return fail(-MI355_E_SHAPE, "%s: output batch / head strides must not be 0", who);
+  FaLayout lay;
+  lay.q_b = q_strides[0], lay.q_h = q_strides[1], lay.q_r = (unsigned)q_strides[2];
+  lay.k_b = k_strides[0], lay.k_h = k_strides[1], lay.k_r = (unsigned)k_strides[2];
+  lay.v_b = v_strides[0], lay.v_h = v_strides[1], lay.v_r = (unsigned)v_strides[2];
+  lay.o_b = o_strides[0], lay.o_h = o_strides[1], lay.o_r = (unsigned)o_strides[2];
+  lay.H = (int)H, lay.group = Hkv > 0 ? (int)(H / Hkv) : 1;
+  return fa_launch(q, k, v, o, B, H, Hkv, Sq, Sk, D, lay, scale, is_causal, variant, stream, who);
 }

@@ -4,6 +4,7 @@ these functions; they are the only callers of the C ABI."""
 
 from __future__ import annotations
 
+import ctypes
 import math
 
 import torch
@@ -43,20 +44,49 @@ def gemm_nt_out(a: Tensor, b: Tensor, c: Tensor, variant: int = -1) -> Tensor:
     return c
 
 
+def _fa_strides(t: Tensor):
+    """{batch, head, row} element strides if the kernel can read `t` in place, else None."""
+    sb, sh, sr, sd = t.stride()
+    if t.size(3) != 1 and sd != 1:
+        return None
+    if t.size(0) == 1:
+        sb = 0
+    if t.size(1) == 1:
+        sh = 0
+    if t.size(2) == 1:
+        sr = 128
+    if min(sb, sh) < 0 or sr < 128 or sr >= 2**31 or (sb | sh | sr) & 7 or t.data_ptr() & 15:
+        return None
+    return (sb, sh, sr)
+
+
 def flash_attn_fwd_out(q: Tensor, k: Tensor, v: Tensor, o: Tensor, is_causal: bool, scale: float, variant: int = -1) -> Tensor:
+    """q, o: [B, H, Sq, 128]; k, v: [B, Hkv, Sk, 128] with H % Hkv == 0.  Operands whose rows are contiguous and
+    16-byte aligned (any batch / head / row strides, e.g. transposed [B, S, H, D] views) are read in place; others
+    are copied first.  `o` must be such a tensor."""
     dev = _dev(q, k, v, o)
-    q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-    _contig_out(o, "flash_attn_fwd")
     B, H, Sq, D = q.shape
-    Sk = k.shape[2]
+    Hkv, Sk = k.shape[1], k.shape[2]
     if o.shape != q.shape or o.dtype != torch.float16:
         raise ValueError("flash_attn_fwd: o must be float16 with q's shape")
     if scale is None or scale <= 0:
         scale = 1.0 / math.sqrt(D)
+    ins = []
+    for t in (q, k, v):
+        st = _fa_strides(t)
+        if st is None:
+            t = t.contiguous()
+            st = _fa_strides(t)
+        ins.append((t, st))
+    o_st = _fa_strides(o)
+    if o_st is None or (B > 1 and o_st[0] == 0) or (H > 1 and o_st[1] == 0):
+        raise ValueError("flash_attn_fwd: output rows must be contiguous, 16-byte aligned and not overlapping")  # runtime/launch.py:246
+    arr = lambda st: (ctypes.c_int64 * 3)(*st)
     with torch.cuda.device(dev):
-        rc = _lib.load().mi355_flash_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), B, H, Sq, Sk, D, scale,
-                                              int(bool(is_causal)), variant, _lib.current_stream_ptr(dev))
-    _lib.check(rc, f"flash_attn_fwd B={B} H={H} Sq={Sq} Sk={Sk} D={D} causal={is_causal}")
+        rc = _lib.load().mi355_flash_attn_fwd_strided(ins[0][0].data_ptr(), ins[1][0].data_ptr(), ins[2][0].data_ptr(), o.data_ptr(),
+                                                      B, H, Hkv, Sq, Sk, D, arr(ins[0][1]), arr(ins[1][1]), arr(ins[2][1]), arr(o_st),
+                                                      scale, int(bool(is_causal)), variant, _lib.current_stream_ptr(dev))
+    _lib.check(rc, f"flash_attn_fwd B={B} H={H} Hkv={Hkv} Sq={Sq} Sk={Sk} D={D} causal={is_causal}")
     return o
 
 

@@ -67,11 +67,13 @@ class gemm_nt(CustomOp):
 
 @CustomOp.register
 class flash_attn_fwd(CustomOp):
-    """softmax(scale . Q K^T [+ causal mask]) V for q [B,H,Sq,128], k/v [B,H,Sk,128] fp16.
+    """softmax(scale . Q K^T [+ causal mask]) V for q [B,H,Sq,128], k/v [B,Hkv,Sk,128] fp16, H % Hkv == 0
+    (query head h reads K/V head h // (H // Hkv), as `enable_gqa=True` does).
 
     Same argument meaning as aten.scaled_dot_product_attention(q, k, v, None, 0.0, is_causal,
     scale=) -- the canonical form the reference rewrites SDPA variants to
-    (iree/turbine/kernel/boo/fusion/replacement.py:275-284).  scale <= 0 selects 1/sqrt(D)."""
+    (iree/turbine/kernel/boo/fusion/replacement.py:275-284).  scale <= 0 selects 1/sqrt(D).
+    The result is laid out like `torch.empty_like(q)`: a transposed [B, S, H, D] view in gives one out."""
 
     signature = "flash_attn_fwd(Tensor q, Tensor k, Tensor v, bool is_causal, float scale) -> Tensor"
 
@@ -84,15 +86,25 @@ class flash_attn_fwd(CustomOp):
             _require(t.dtype == torch.float16, f"flash_attn_fwd: {name} must be float16")
         _require(q.t.size(3) == 128, f"flash_attn_fwd: head dim {q.t.size(3)} not supported (only 128)")
         _require(k.t.shape == v.t.shape, "flash_attn_fwd: k and v shapes differ")
-        _require(q.t.shape[:2] == k.t.shape[:2] and q.t.size(3) == k.t.size(3), "flash_attn_fwd: q and k disagree on B, H or D")
+        _require(q.t.size(0) == k.t.size(0) and q.t.size(3) == k.t.size(3), "flash_attn_fwd: q and k disagree on B or D")
+        _require(k.t.size(1) > 0 and q.t.size(1) % k.t.size(1) == 0,
+                 f"flash_attn_fwd: {q.t.size(1)} query heads over {k.t.size(1)} key/value heads")
         _require(q.t.size(2) > 0 and k.t.size(2) > 0, "flash_attn_fwd: empty sequence")
         for d in (q, k, v):
             d.specialize_dims(1, 3)
-        sel.return_new_tensor(list(q.t.shape), torch.float16)
+        sel.return_tensor(_like_q(q.t, "meta"))
 
     def eager_execute(self, q, k, v, is_causal, scale):
-        o = torch.empty(q.shape, dtype=torch.float16, device=q.device)
-        return launch.flash_attn_fwd_out(q, k, v, o, is_causal, scale)
+        return launch.flash_attn_fwd_out(q, k, v, _like_q(q, q.device), is_causal, scale)
+
+
+def _like_q(q: Tensor, device) -> Tensor:
+    """An output with q's dimension order in memory, densely packed (what `empty_like` gives a dense q)."""
+    order = sorted(range(4), key=lambda i: (q.stride(i), -i), reverse=True) if q.size(3) > 1 and q.stride(3) == 1 else [0, 1, 2, 3]
+    if order[-1] != 3 or any(q.stride(i) == 0 and q.size(i) > 1 for i in range(4)):
+        order = [0, 1, 2, 3]
+    inv = [order.index(i) for i in range(4)]
+    return torch.empty([q.size(i) for i in order], dtype=torch.float16, device=device).permute(inv)
 
 
 def _check_paged_args(op: str, q: Tensor, k_cache: Tensor, v_cache: Tensor, block_table: Tensor, seq_lens: Tensor):

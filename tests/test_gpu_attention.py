@@ -112,6 +112,80 @@ def test_attention_full_size_repeatable(dev, causal):
         torch.testing.assert_close(outs[0], other, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("layout", ["bshd", "packed_qkv", "head_slice"])
+def test_attention_strided_operands(dev, layout, causal):
+    """Transposed [B, S, H, D] views, slices of one packed QKV projection and head slices are read in place
+    (no copies) and give what the contiguous tensors give."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import attention as oa, inputs
+
+    B, H, S, D = 2, 4, 200, 128
+    announce(f"flash_attn_fwd strided layout={layout} causal={causal}")
+    q, k, v = inputs.attention_inputs(B, H, S, D, seed=21)
+    if layout == "bshd":
+        dq, dk, dv = (t.to(dev).transpose(1, 2).contiguous().transpose(1, 2) for t in (q, k, v))
+    elif layout == "packed_qkv":
+        packed = torch.stack([t.transpose(1, 2) for t in (q, k, v)], dim=2).contiguous().to(dev)  # [B, S, 3, H, D]
+        dq, dk, dv = (packed[:, :, i].transpose(1, 2) for i in range(3))
+    else:
+        wide = [torch.randn(B, H + 3, S, D, dtype=torch.float16, device=dev) for _ in range(3)]
+        for w, t in zip(wide, (q, k, v)):
+            w[:, 2:2 + H] = t.to(dev)
+        dq, dk, dv = (w[:, 2:2 + H] for w in wide)
+    assert not dq.is_contiguous()
+    o = torch.ops.mi355.flash_attn_fwd(dq, dk, dv, causal, 0.0)
+    torch.cuda.synchronize()
+    if layout != "head_slice":
+        assert o.transpose(1, 2).is_contiguous()  # laid out like q: [B, S, H, D] in memory
+    ref = oa.sdpa_ref(q, k, v, is_causal=causal)
+    torch.testing.assert_close(o.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+    # bit-identical to the contiguous call: the layout changes addresses only
+    oc = torch.ops.mi355.flash_attn_fwd(q.to(dev), k.to(dev), v.to(dev), causal, 0.0)
+    assert torch.equal(o.contiguous(), oc)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("H,Hkv", [(8, 2), (8, 1), (16, 8), (6, 3)])
+def test_attention_grouped_kv_heads(dev, H, Hkv, causal):
+    """Query head h reads K/V head h // (H // Hkv): equal to attention over K/V repeated per group."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import attention as oa, inputs
+
+    B, S, D = 2, 160, 128
+    announce(f"flash_attn_fwd gqa H={H} Hkv={Hkv} causal={causal}")
+    q, _, _ = inputs.attention_inputs(B, H, S, D, seed=31)
+    _, k, v = inputs.attention_inputs(B, Hkv, S, D, seed=32)
+    o = torch.ops.mi355.flash_attn_fwd(q.to(dev), k.to(dev), v.to(dev), causal, 0.0)
+    torch.cuda.synchronize()
+    kr, vr = (t.repeat_interleave(H // Hkv, dim=1) for t in (k, v))
+    torch.testing.assert_close(o.float().cpu(), oa.sdpa_ref(q, kr, vr, is_causal=causal), rtol=RTOL, atol=ATOL)
+    if Hkv == 1:  # a broadcast (head stride 0) view of the single K/V head is the same computation
+        o2 = torch.ops.mi355.flash_attn_fwd(q.to(dev), k.to(dev).expand(B, H, S, D), v.to(dev).expand(B, H, S, D), causal, 0.0)
+    else:
+        o2 = torch.ops.mi355.flash_attn_fwd(q.to(dev), kr.to(dev), vr.to(dev), causal, 0.0)
+    assert torch.equal(o, o2)
+
+
+def test_attention_strided_c_abi_errors(dev):
+    """The strided entry point rejects what the kernel cannot address."""
+    import ctypes
+    from iree_turbine_amd import _lib
+
+    lib = _lib.load()
+    t = torch.zeros(1, 1, 16, 128, dtype=torch.float16, device=dev)
+    arr = lambda *s: (ctypes.c_int64 * 3)(*s)
+    good = arr(2048, 2048, 128)
+    call = lambda qs, os_, hkv=1, h=1, b=1: lib.mi355_flash_attn_fwd_strided(
+        t.data_ptr(), t.data_ptr(), t.data_ptr(), t.data_ptr(), b, h, hkv, 16, 16, 128, qs, good, good, os_, 0.1, 0, -1, None)
+    assert call(arr(2048, 2048, 100), good) < 0   # row stride not a multiple of 8 and < 128
+    assert call(arr(2048, 2048, 64), good) < 0    # rows would overlap
+    assert call(arr(2048, -8, 128), good) < 0     # negative stride
+    assert call(good, arr(0, 2048, 128), b=2) < 0  # output batch stride 0 with two batches
+    assert call(good, good, hkv=2, h=3) < 0       # heads not divisible
+    assert b"flash_attn_fwd_strided" in lib.mi355_last_error()
+
+
 def test_attention_contract_errors(dev):
     import iree_turbine_amd  # noqa: F401
 
