@@ -88,7 +88,7 @@ int mi355_flash_attn_fwd(const void* q, const void* k, const void* v, void* o,
  * query head h reads K/V head h / (H / Hkv)  (enable_gqa semantics).
  * *_strides: {batch, head, row} strides in ELEMENTS; the D elements of a row are
  * contiguous.  Every stride is a non-negative multiple of 8 (16-byte rows), row
- * strides lie in [128, 2^31); a 0 batch or head stride on q, k or v broadcasts.
+ * strides lie in [128, 2^24); a 0 batch or head stride on q, k or v broadcasts.
  * Replaces: the same SDPA root as above for the non-contiguous operands that the
  * reference makes contiguous before every launch
  * (iree/turbine/runtime/op_reg/eager.py:119-132).

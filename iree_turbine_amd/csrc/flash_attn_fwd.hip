@@ -280,7 +280,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
   for (int ks = 0; ks < 8; ks++) {
     if (q_ok) {
-      qf[ks] = *reinterpret_cast<const half8*>(Qb + (size_t)q_row * lay.q_r + ks * 16 + h * 8);
+      // scale . log2(e) is folded into Q (rounded to fp16 again: a relative error of 2^-11 per element, the
+      // same size as the rounding of P to fp16), so the MFMA delivers exponents of 2 directly
+      const half8 raw = *reinterpret_cast<const half8*>(Qb + (size_t)q_row * lay.q_r + ks * 16 + h * 8);
+#pragma unroll
+      for (int e = 0; e < 8; e++) qf[ks][e] = (half_t)((float)raw[e] * scale_log2e);
     } else {
 #pragma unroll
       for (int e = 0; e < 8; e++) qf[ks][e] = (half_t)0;
@@ -290,14 +294,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int lrow = lane >> 4, lslot = lane & 15;
   const int k_chunk = lslot ^ (wave * 4 + lrow);
   const int v_chunk = lslot ^ (4 * lrow);
-  auto issue_kv = [&](const half_t* base, unsigned row_stride, int chunk, int tile, int lds_off) {
+  // Global -> LDS through a buffer descriptor rebuilt per tile on the scalar unit (base = first row of the tile,
+  // size = up to the end of the tile's last valid row): the per-lane byte offset is loop-invariant, rows at or
+  // beyond Sk read zeros (they are masked out of the softmax), and no 64-bit vector address arithmetic is left.
+  const unsigned k_rb = lay.k_r * 2, v_rb = lay.v_r * 2;  // row strides in bytes
+  const unsigned k_voff = (wave * 4 + lrow) * k_rb + k_chunk * 16;
+  const unsigned v_voff = (wave * 4 + lrow) * v_rb + v_chunk * 16;
+  auto issue_kv = [&](const half_t* base, unsigned rb, unsigned voff, int tile, int lds_off) {
     char* dst = lds + lds_off + wave * 1024;
+    const int row0 = tile * FA_BLOCK_N;
+    int rem = Sk - row0;
+    rem = rem > FA_BLOCK_N ? FA_BLOCK_N : rem;
+    const buffer_rsrc_t rs = make_buffer(reinterpret_cast<const char*>(base) + (size_t)row0 * rb, (unsigned)(rem - 1) * rb + 256u);
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-      int row = tile * FA_BLOCK_N + (wave + 4 * i) * 4 + lrow;
-      if (row > Sk - 1) row = Sk - 1;  // clamp: tail rows are masked out of the softmax
-      load_lds_16B(base + (size_t)row * row_stride + chunk * 8, dst + i * 4096);
-    }
+    for (int i = 0; i < 4; i++) buffer_load_lds_16B(rs, voff + (unsigned)i * 16u * rb, 0, dst + i * 4096);
   };
 
   const int k_base = r32 * 256 + ((h ^ (lane & 15)) * 16);
@@ -310,8 +320,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   for (int dt = 0; dt < 4; dt++)
 #pragma unroll
     for (int r = 0; r < 16; r++) oacc[dt][r] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
-  constexpr float kRescaleThreshold = 8.f;  // log2 units of the final exponent
+  // The running maximum m of a query lives negated in all 16 registers of `negm`, which every score MFMA chain
+  // starts from: the accumulators then hold log2-domain scores relative to m and feed v_exp_f32 unchanged.
+  // (A lane owns one query column of S^T, so the 16 values of a lane are equal.)
+  floatx16 negm;
+#pragma unroll
+  for (int r = 0; r < 16; r++) negm[r] = 0.f;
+  float l_run = 0.f;
+  // m is raised -- and O rescaled -- only when a score exceeds it by more than 2^8; -inf until the query has
+  // seen its first unmasked key, so that the first one always sets m
+  float grow_thr = -INFINITY;
+  constexpr float kRescaleThreshold = 8.f;
 
   auto wave_active = [&](int tile) { return !CAUSAL || (tile * FA_BLOCK_N <= wq0 + 31 + causal_off); };
 
@@ -320,11 +339,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int t = 0; t < 2; t++) {
 #pragma unroll
-      for (int r = 0; r < 16; r++) s[t][r] = 0.f;
-#pragma unroll
       for (int ks = 0; ks < 8; ks++) {
         half8 kf = *reinterpret_cast<const half8*>(lds + koff + t * 8192 + (k_base ^ (ks * 32)));
-        s[t] = mfma_32x32x16(kf, qf[ks], s[t]);
+        s[t] = mfma_32x32x16(kf, qf[ks], ks == 0 ? negm : s[t]);
       }
     }
   };
@@ -351,21 +368,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int t = 0; t < 2; t++)
 #pragma unroll
       for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[t][r]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    // raise the running maximum only when it is stale by more than the threshold for some query
-    const float grow = (mx - m_run) * scale_log2e;  // +inf the first time, NaN only for -inf - -inf
-    if (__builtin_amdgcn_ballot_w64(grow > kRescaleThreshold) != 0) {
-      const float m_new = fmaxf(m_run, mx);
-      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-      const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * scale_log2e);
+    if (__builtin_amdgcn_ballot_w64(mx > grow_thr) != 0) {
+      // rare: some query's scores outgrew its maximum (or it saw its first key).  The other half of a query's
+      // keys sits in lane ^ 32; both lanes take the same decision.
+      const float mxx = fmaxf(mx, __shfl_xor(mx, 32));
+      const bool fresh = grow_thr == -INFINITY;
+      const float delta = fresh ? (mxx == -INFINITY ? 0.f : mxx) : fmaxf(mxx, 0.f);
+      const float alpha = fresh ? 1.f : __builtin_amdgcn_exp2f(-delta);
+      if (mxx != -INFINITY) grow_thr = kRescaleThreshold;
       l_run *= alpha;
 #pragma unroll
       for (int dt = 0; dt < 4; dt++)
 #pragma unroll
         for (int r = 0; r < 16; r++) oacc[dt][r] *= alpha;
-      m_run = m_new;
+#pragma unroll
+      for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[t][r] -= delta;
+#pragma unroll
+      for (int r = 0; r < 16; r++) negm[r] -= delta;
     }
-    const float mc = (m_run == -INFINITY ? 0.f : m_run) * scale_log2e;
     half8 pf[4];
     float psum = 0.f;
     // Scores of the next tile and exponentials of this one in one straight-line block: a wave issues in
@@ -373,27 +395,31 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // (Past the last tile the scores are computed from stale LDS bytes and never used.)
     __builtin_amdgcn_sched_barrier(0);
     scores(koff_next, s_next);
+    const half2v ones = {(half_t)1.f, (half_t)1.f};
 #pragma unroll
     for (int t = 0; t < 2; t++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const float p = __builtin_amdgcn_exp2f(s[t][r] * scale_log2e - mc);
-        psum += p;
-        pf[t * 2 + (r >> 3)][r & 7] = (half_t)p;
+      for (int r = 0; r < 16; r += 2) {
+        const half2v pp = {(half_t)__builtin_amdgcn_exp2f(s[t][r]), (half_t)__builtin_amdgcn_exp2f(s[t][r + 1])};
+        psum = __builtin_amdgcn_fdot2(pp, ones, psum, false);  // sums what the second MFMA multiplies
+        pf[t * 2 + (r >> 3)][r & 7] = pp[0];
+        pf[t * 2 + (r >> 3)][(r & 7) + 1] = pp[1];
       }
-    // order: 3 K fragment reads up front, then per score MFMA one more read and the VALU work of two
-    // scores (fma, exp, add, half a cvt_pk each) -- a fragment is requested two MFMAs before its use
+    // order: 3 K fragment reads up front, then per score MFMA one more read and the work of two scores
+    // (two exp, one cvt_pk, one dot2) -- a fragment is requested two MFMAs before its use
     __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
 #pragma unroll
     for (int i = 0; i < 13; i++) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
+      __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
     }
 #pragma unroll
     for (int i = 0; i < 3; i++) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
+      __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
     l_run += psum;
@@ -418,9 +444,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
   floatx16 sa[2], sb[2];
   if (n_tiles > 0) {
-    issue_kv(Kb, lay.k_r, k_chunk, 0, 0);
-    issue_kv(Vb, lay.v_r, v_chunk, 0, VBUF);
-    if (n_tiles > 1) issue_kv(Kb, lay.k_r, k_chunk, 1, TILE_B);
+    issue_kv(Kb, k_rb, k_voff, 0, 0);
+    issue_kv(Vb, v_rb, v_voff, 0, VBUF);
+    if (n_tiles > 1) issue_kv(Kb, k_rb, k_voff, 1, TILE_B);
     wait_vmcnt0();
     __syncthreads();
     if (wave_active(0)) scores(0, sa);
@@ -433,8 +459,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   auto trip = [&](auto par_tag, int j, floatx16* s_cur, floatx16* s_next) {
     constexpr int PAR = decltype(par_tag)::value;
     constexpr int K_CUR = PAR * TILE_B, K_NEXT = (1 - PAR) * TILE_B, V_CUR = PAR * TILE_B, V_NEXT = VBUF + (1 - PAR) * TILE_B;
-    if (j + 2 < n_tiles) issue_kv(Kb, lay.k_r, k_chunk, j + 2, K_CUR);
-    if (j + 1 < n_tiles) issue_kv(Vb, lay.v_r, v_chunk, j + 1, V_NEXT);
+    if (j + 2 < n_tiles) issue_kv(Kb, k_rb, k_voff, j + 2, K_CUR);
+    if (j + 1 < n_tiles) issue_kv(Vb, v_rb, v_voff, j + 1, V_NEXT);
     if (wave_active(j)) softmax_pv(std::true_type{}, j, V_CUR, s_cur, K_NEXT, s_next);  // idle from here on otherwise
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
@@ -528,8 +554,8 @@ extern "C" int mi355_flash_attn_fwd_strided(const void* q, const void* k, const 
   for (const int64_t* st : all) {
     for (int i = 0; i < 3; i++)
       if (st[i] < 0 || (st[i] & 7)) return fail(-MI355_E_ALIGN, "%s: strides must be non-negative multiples of 8 elements", who);
-    if (st[2] < 128 || st[2] >= (1ll << 31))
-      return fail(-MI355_E_SHAPE, "%s: row stride %lld outside [128, 2^31)", who, (long long)st[2]);
+    if (st[2] < 128 || st[2] >= (1ll << 24))
+      return fail(-MI355_E_SHAPE, "%s: row stride %lld outside [128, 2^24)", who, (long long)st[2]);
   }
   if ((B > 1 && o_strides[0] == 0) || (H > 1 && o_strides[1] == 0)) return fail(-MI355_E_SHAPE, "%s: output batch / head strides must not be 0", who);
   FaLayout lay;

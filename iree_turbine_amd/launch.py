@@ -55,7 +55,7 @@ def _fa_strides(t: Tensor):
         sh = 0
     if t.size(2) == 1:
         sr = 128
-    if min(sb, sh) < 0 or sr < 128 or sr >= 2**31 or (sb | sh | sr) & 7 or t.data_ptr() & 15:
+    if min(sb, sh) < 0 or sr < 128 or sr >= 2**24 or (sb | sh | sr) & 7 or t.data_ptr() & 15:
         return None
     return (sb, sh, sr)
 
