@@ -240,32 +240,38 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r32 = lane & 31, h = lane >> 5;
 
-  int bh, qb;
+  // Workgroup -> (batch * head, unit).  A unit is one 128-query block; with the causal mask it is a pair of
+  // blocks, the i-th from the end and the i-th from the start, processed one after the other, so that every
+  // workgroup walks the same number of key tiles (q_blocks + 1) and the grid has no long tail.
+  const int units = CAUSAL ? (q_blocks + 1) / 2 : q_blocks;
+  int bh, unit;
   {
     const int pid = blockIdx.x;
     if (((BH / lay.group) & 7) == 0) {
-      // all query blocks of the `group` query heads that share one K/V head sit on one XCD
-      const int xcd = pid & 7, loc = pid >> 3, per_kv = q_blocks * lay.group;
+      // all units of the `group` query heads that share one K/V head sit on one XCD
+      const int xcd = pid & 7, loc = pid >> 3, per_kv = units * lay.group;
       const int w = loc % per_kv;
-      bh = ((loc / per_kv) * 8 + xcd) * lay.group + w / q_blocks;
-      qb = w % q_blocks;
+      bh = ((loc / per_kv) * 8 + xcd) * lay.group + w / units;
+      unit = w % units;
     } else {
-      bh = pid / q_blocks;
-      qb = pid % q_blocks;
+      bh = pid / units;
+      unit = pid % units;
     }
-    if (CAUSAL) qb = q_blocks - 1 - qb;
   }
   const int causal_off = Sk - Sq;
-  const int q0 = qb * FA_BLOCK_M;
-  const int wq0 = q0 + wave * 32;
-  const int q_row = wq0 + r32;
-  const bool q_ok = q_row < Sq;
-
   const int b_idx = bh / lay.H, h_idx = bh - b_idx * lay.H, hk_idx = h_idx / lay.group;
   const half_t* Qb = Q + b_idx * lay.q_b + h_idx * lay.q_h;
   const half_t* Kb = K + b_idx * lay.k_b + hk_idx * lay.k_h;
   const half_t* Vb = V + b_idx * lay.v_b + hk_idx * lay.v_h;
   half_t* Ob = O + b_idx * lay.o_b + h_idx * lay.o_h;
+
+  for (int pass = 0; pass < (CAUSAL ? 2 : 1); pass++) {
+  const int qb = CAUSAL ? (pass == 0 ? q_blocks - 1 - unit : unit) : unit;
+  if (CAUSAL && pass == 1 && 2 * unit == q_blocks - 1) break;  // the middle block of an odd count has no partner
+  const int q0 = qb * FA_BLOCK_M;
+  const int wq0 = q0 + wave * 32;
+  const int q_row = wq0 + r32;
+  const bool q_ok = q_row < Sq;
 
   int k_end = Sk;
   if (CAUSAL) {
@@ -483,6 +489,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         *reinterpret_cast<half4*>(orow + dt * 32 + q * 8) = v;
       }
   }
+  }  // pass
 }
 
 static const char* kFaVariants[] = {"d128_bm128_bn64_w4_pipelined", "d128_bm128_bn64_w4"};
@@ -525,7 +532,9 @@ static int fa_launch(const void* q, const void* k, const void* v, void* o, int64
     attr_set = true;
   }
   const float scale_log2e = scale * 1.4426950408889634f;
-  dim3 grid(BH * q_blocks), block(256);
+  // the pipelined causal kernel takes a pair of query blocks per workgroup
+  const int units = (variant != 1 && is_causal) ? (q_blocks + 1) / 2 : q_blocks;
+  dim3 grid(BH * units), block(256);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   auto kern = variant == 1 ? (is_causal ? fa_fwd_d128<true> : fa_fwd_d128<false>)
                            : (is_causal ? fa_fwd_d128_pipe<true> : fa_fwd_d128_pipe<false>);
