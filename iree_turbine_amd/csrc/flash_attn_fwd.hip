@@ -360,12 +360,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       const bool need_mask = (CAUSAL && (key0 + FA_BLOCK_N - 1 > wq0 + causal_off)) || (key0 + FA_BLOCK_N > Sk);
       if (need_mask) {
         const int lim = CAUSAL ? (q_row + causal_off < Sk - 1 ? q_row + causal_off : Sk - 1) : Sk - 1;
+        const int rel = lim - key0 - 4 * h;  // last visible key, relative to the tile and to this lane's rows
 #pragma unroll
         for (int t = 0; t < 2; t++)
 #pragma unroll
-          for (int r = 0; r < 16; r++) {
-            const int key = key0 + 32 * t + 8 * (r >> 2) + 4 * h + (r & 3);
-            if (key > lim) s[t][r] = -INFINITY;
+          for (int r = 0; r < 16; r++)
+          {
+            // -inf where the key is beyond `rel`, by bit selection: a compare-and-select per score would hold
+            // a scalar register pair per score and push loop-invariant scalars out of the register file
+            const unsigned hide = (unsigned)((rel - (32 * t + 8 * (r >> 2) + (r & 3))) >> 31);
+            const float sv = s[t][r];  // (bit_cast straight from a vector element miscompiles)
+            s[t][r] = __builtin_bit_cast(float, (hide & 0xFF800000u) | (~hide & __builtin_bit_cast(unsigned, sv)));
           }
       }
     }
