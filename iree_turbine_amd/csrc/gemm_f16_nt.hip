@@ -358,6 +358,239 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
   }
 }
 
+// Register-staged form: the slab after next waits in VGPRs instead of LDS.  160 KiB of LDS hold only two
+// 64 KiB stages, so a direct-to-LDS load of slab s+2 cannot start before every wave has read slab s: the 16
+// loads of a wave then issue in one burst in the last k-step, and a wave that is alone on its SIMD stands
+// still while the texture path drains them (measured on the pipelined 4-wave kernel: 30 % of the time).
+// Here four waves (512 registers each: 256 accumulators, two fragment sets, two staging sets of 16 x 16
+// bytes) load slab s+3 into registers while slab s computes and copy slab s+1 from registers into the LDS
+// stage that slab s-1 left, one load and about one ds_write per four MFMAs, evenly over the slab.  A load
+// has two slab times to land, and there is still one barrier per slab:
+//   k-steps 0..2: MFMAs | fragment reads of the next k-step | ds_write of slab s+1 | loads of slab s+3
+//   wait + barrier: slab s+1 is complete in LDS, every wave has read slab s
+//   k-step 3:     MFMAs | fragment reads of k-step 0 of slab s+1 | the last loads of slab s+3
+// The loads are inline assembly so that the waits for them can be placed by hand (the compiler's vmcnt
+// placement merges the loop's entry and back edge pessimistically).  Same LDS format as the other tiled
+// kernels; the swizzle is applied by the ds_write address.
+template <int BM, int BN, int WM, int WN, typename OutT>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_staged(const half_t* __restrict__ A, const half_t* __restrict__ B,
+                                                                  OutT* __restrict__ C, int M, int N, int K, int tiles_m,
+                                                                  int tiles_n, int group_m) {
+  constexpr int NW = WM * WN;
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
+  constexpr int LA = BM / 8 / NW, LB = BN / 8 / NW;
+  static_assert(NW == 4 && TM == 4 && TN == 4 && LA == 8 && LB == 8, "the slab schedule below is written out for a 2x2 grid of 128x128 wave tiles");
+  static_assert(A_BYTES + (LB - 1) * NW * 1024 < 65536, "ds_write immediate offsets");
+  typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+  typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  int tile_m, tile_n;
+  map_tile(blockIdx.x, tiles_m, tiles_n, group_m, tile_m, tile_n);
+
+  // global side: wave-load i covers rows (i * NW + wave) * 8 .. + 7 of the tile, 8 lanes per 128-byte row piece
+  const int lrow = lane >> 3, lc = lane & 7;
+  const unsigned row_bytes = (unsigned)K * 2u;
+  // buffer descriptors by hand: base, stride 0, size, raw dword format
+  auto make_desc = [&](const half_t* base, unsigned bytes) {
+    const unsigned long long p = reinterpret_cast<unsigned long long>(base);
+    i32x4 d;
+    d[0] = __builtin_amdgcn_readfirstlane((int)(unsigned)p);
+    d[1] = __builtin_amdgcn_readfirstlane((int)(unsigned)((p >> 32) & 0xFFFFu));
+    d[2] = __builtin_amdgcn_readfirstlane((int)bytes);
+    d[3] = 0x00020000;
+    return d;
+  };
+  const i32x4 a_src = make_desc(A + (size_t)(tile_m * BM + wave * 8) * K, (unsigned)(BM - wave * 8) * row_bytes);
+  const i32x4 b_src = make_desc(B + (size_t)(tile_n * BN + wave * 8) * K, (unsigned)(BN - wave * 8) * row_bytes);
+  const unsigned g_off = (unsigned)lrow * row_bytes + (unsigned)lc * 16u;
+  const unsigned row_step = (unsigned)NW * 8u * row_bytes;
+  // LDS side: row r = (i * NW + wave) * 8 + lrow, chunk lc in slot lc ^ ((r >> 1) & 7); NW is even, so the
+  // swizzle term does not depend on i
+  const int w_off = wave * 1024 + lrow * 128 + ((lc ^ (((wave & 1) << 2) | (lrow >> 1))) * 16);
+
+  // staging registers: r[set][n], n < 8 the A row groups, n >= 8 the B row groups
+  u32x4 r[2][16];
+  // (macros: inline assembly inside a generic lambda cannot name the enclosing function's arrays)
+#define MI355_ST_LOAD(S, n, k_off_)                                                                  \
+  asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"                                            \
+               : "=v"(r[S][n])                                                                       \
+               : "v"(g_off), "s"((n) < 8 ? a_src : b_src), "s"((k_off_) + (unsigned)((n)&7) * row_step) \
+               : "memory")
+  // `newer` = loads issued after the one that filled r[S][n]; they may still be in flight
+#define MI355_ST_WRITE(S, n, newer, st_)                                                                                   \
+  do {                                                                                                                     \
+    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(r[S][n]) : "n"(newer) : "memory");                                           \
+    *reinterpret_cast<u32x4*>((st_) + w_off + ((n) < 8 ? (n)*NW * 1024 : A_BYTES + ((n)-8) * NW * 1024)) = r[S][n];        \
+  } while (0)
+
+  const int r32 = lane & 31, h = lane >> 5;
+  const int sw = (h ^ ((r32 >> 1) & 7)) * 16;
+  const int a_base = (wm * WTM + r32) * 128 + sw;
+  const int b_base = A_BYTES + (wn * WTN + r32) * 128 + sw;
+  auto read_frags = [&](const char* st, int ks, half8* fm, half8* fn) {
+#pragma unroll
+    for (int j = 0; j < TM; j++) fm[j] = *reinterpret_cast<const half8*>(st + ((a_base ^ (ks * 32)) + j * 4096));
+#pragma unroll
+    for (int i = 0; i < TN; i++) fn[i] = *reinterpret_cast<const half8*>(st + ((b_base ^ (ks * 32)) + i * 4096));
+  };
+
+  floatx16 acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; i++)
+#pragma unroll
+    for (int j = 0; j < TM; j++)
+#pragma unroll
+      for (int q = 0; q < 16; q++) acc[i][j][q] = 0.f;
+
+  const int KT = K / 64;  // even, >= 4 (checked on the host)
+  half8 fm0[TM], fn0[TN], fm1[TM], fn1[TN];
+
+  // prologue: slab 0 -> set 0 -> stage 0; slab 1 -> set 1; slab 2 -> set 0
+#define MI355_ST_LOAD_ALL(S, slab_)                                       \
+  do {                                                                    \
+    const unsigned ko_ = (unsigned)(slab_)*128u;                          \
+    MI355_ST_LOAD(S, 0, ko_); MI355_ST_LOAD(S, 1, ko_); MI355_ST_LOAD(S, 2, ko_); MI355_ST_LOAD(S, 3, ko_);     \
+    MI355_ST_LOAD(S, 4, ko_); MI355_ST_LOAD(S, 5, ko_); MI355_ST_LOAD(S, 6, ko_); MI355_ST_LOAD(S, 7, ko_);     \
+    MI355_ST_LOAD(S, 8, ko_); MI355_ST_LOAD(S, 9, ko_); MI355_ST_LOAD(S, 10, ko_); MI355_ST_LOAD(S, 11, ko_);   \
+    MI355_ST_LOAD(S, 12, ko_); MI355_ST_LOAD(S, 13, ko_); MI355_ST_LOAD(S, 14, ko_); MI355_ST_LOAD(S, 15, ko_); \
+  } while (0)
+  MI355_ST_LOAD_ALL(0, 0);
+  MI355_ST_LOAD_ALL(1, 1);
+  MI355_ST_WRITE(0, 0, 16, lds); MI355_ST_WRITE(0, 1, 16, lds); MI355_ST_WRITE(0, 2, 16, lds); MI355_ST_WRITE(0, 3, 16, lds);
+  MI355_ST_WRITE(0, 4, 16, lds); MI355_ST_WRITE(0, 5, 16, lds); MI355_ST_WRITE(0, 6, 16, lds); MI355_ST_WRITE(0, 7, 16, lds);
+  MI355_ST_WRITE(0, 8, 16, lds); MI355_ST_WRITE(0, 9, 16, lds); MI355_ST_WRITE(0, 10, 16, lds); MI355_ST_WRITE(0, 11, 16, lds);
+  MI355_ST_WRITE(0, 12, 16, lds); MI355_ST_WRITE(0, 13, 16, lds); MI355_ST_WRITE(0, 14, 16, lds); MI355_ST_WRITE(0, 15, 16, lds);
+  MI355_ST_LOAD_ALL(0, 2);
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __syncthreads();
+  read_frags(lds, 0, fm0, fn0);
+
+  // One group = the four MFMAs of accumulator row g, each followed by one piece of memory work, so that no
+  // MFMA waits behind more than one long-issuing instruction (a 1 KiB ds_write takes about 20 cycles to
+  // issue, an MFMA keeps the pipe busy for 32): up to two ds_writes, the load, and two fragment reads of the
+  // next k-step.  The A fragments (all four are needed by the next k-step's first group) are read in groups
+  // 0 and 1, the B fragments in groups 2 and 3: every fragment is requested two groups or more before its use.
+  auto frag_reads = [&](int g, const char* rst, int rks, half8* fm_n, half8* fn_n) {
+    if (g < 2) {
+      fm_n[2 * g] = *reinterpret_cast<const half8*>(rst + ((a_base ^ (rks * 32)) + (2 * g) * 4096));
+      fm_n[2 * g + 1] = *reinterpret_cast<const half8*>(rst + ((a_base ^ (rks * 32)) + (2 * g + 1) * 4096));
+    } else {
+      fn_n[2 * g - 4] = *reinterpret_cast<const half8*>(rst + ((b_base ^ (rks * 32)) + (2 * g - 4) * 4096));
+      fn_n[2 * g - 3] = *reinterpret_cast<const half8*>(rst + ((b_base ^ (rks * 32)) + (2 * g - 3) * 4096));
+    }
+  };
+#define MI355_ST_GROUP(g, fm, fn, rst, rks, fm_n, fn_n, W1, W2, LD) \
+  do {                                                              \
+    acc[g][0] = mfma_32x32x16(fn[g], fm[0], acc[g][0]);             \
+    W1;                                                             \
+    __builtin_amdgcn_sched_barrier(0);                              \
+    acc[g][1] = mfma_32x32x16(fn[g], fm[1], acc[g][1]);             \
+    W2;                                                             \
+    __builtin_amdgcn_sched_barrier(0);                              \
+    acc[g][2] = mfma_32x32x16(fn[g], fm[2], acc[g][2]);             \
+    LD;                                                             \
+    __builtin_amdgcn_sched_barrier(0);                              \
+    acc[g][3] = mfma_32x32x16(fn[g], fm[3], acc[g][3]);             \
+    frag_reads(g, rst, rks, fm_n, fn_n);                            \
+    __builtin_amdgcn_sched_barrier(0);                              \
+  } while (0)
+#define MI355_NOP ((void)0)
+
+  // Slab kt sits in stage P.  Set Q = 1 - P holds slab kt+1 (loaded during slab kt-2) and is copied to stage Q
+  // register by register, each register reloaded with slab kt+3 once it is written out; set P is receiving
+  // slab kt+2.  Loads in flight when register n is written: the rest of its own round (15 - n), the 16 of the
+  // other set, and the G loads of this slab issued so far.
+#define MI355_ST_SLAB(P, Q, kt_)                                                                                           \
+  do {                                                                                                                     \
+    const char* st = lds + P * STAGE;                                                                                      \
+    char* nst = lds + Q * STAGE;                                                                                           \
+    const int nxt_ = (kt_) + 3 < KT ? (kt_) + 3 : KT - 1; /* past the end: re-fetch, never used */                         \
+    const unsigned ko = (unsigned)nxt_ * 128u;                                                                             \
+    __builtin_amdgcn_sched_barrier(0);                                                                                     \
+    MI355_ST_GROUP(0, fm0, fn0, st, 1, fm1, fn1, MI355_ST_WRITE(Q, 0, 31, nst), MI355_ST_WRITE(Q, 1, 30, nst), MI355_ST_LOAD(Q, 0, ko));   \
+    MI355_ST_GROUP(1, fm0, fn0, st, 1, fm1, fn1, MI355_ST_WRITE(Q, 2, 30, nst), MI355_NOP, MI355_ST_LOAD(Q, 1, ko));                       \
+    MI355_ST_GROUP(2, fm0, fn0, st, 1, fm1, fn1, MI355_ST_WRITE(Q, 3, 30, nst), MI355_ST_WRITE(Q, 4, 29, nst), MI355_ST_LOAD(Q, 2, ko));   \
+    MI355_ST_GROUP(3, fm0, fn0, st, 1, fm1, fn1, MI355_ST_WRITE(Q, 5, 29, nst), MI355_NOP, MI355_ST_LOAD(Q, 3, ko));                       \
+    MI355_ST_GROUP(0, fm1, fn1, st, 2, fm0, fn0, MI355_ST_WRITE(Q, 6, 29, nst), MI355_ST_WRITE(Q, 7, 28, nst), MI355_ST_LOAD(Q, 4, ko));   \
+    MI355_ST_GROUP(1, fm1, fn1, st, 2, fm0, fn0, MI355_ST_WRITE(Q, 8, 28, nst), MI355_NOP, MI355_ST_LOAD(Q, 5, ko));                       \
+    MI355_ST_GROUP(2, fm1, fn1, st, 2, fm0, fn0, MI355_ST_WRITE(Q, 9, 28, nst), MI355_ST_WRITE(Q, 10, 27, nst), MI355_ST_LOAD(Q, 6, ko));  \
+    MI355_ST_GROUP(3, fm1, fn1, st, 2, fm0, fn0, MI355_ST_WRITE(Q, 11, 27, nst), MI355_NOP, MI355_ST_LOAD(Q, 7, ko));                      \
+    MI355_ST_GROUP(0, fm0, fn0, st, 3, fm1, fn1, MI355_ST_WRITE(Q, 12, 27, nst), MI355_NOP, MI355_ST_LOAD(Q, 8, ko));                      \
+    MI355_ST_GROUP(1, fm0, fn0, st, 3, fm1, fn1, MI355_ST_WRITE(Q, 13, 27, nst), MI355_NOP, MI355_ST_LOAD(Q, 9, ko));                      \
+    MI355_ST_GROUP(2, fm0, fn0, st, 3, fm1, fn1, MI355_ST_WRITE(Q, 14, 27, nst), MI355_NOP, MI355_ST_LOAD(Q, 10, ko));                     \
+    MI355_ST_GROUP(3, fm0, fn0, st, 3, fm1, fn1, MI355_ST_WRITE(Q, 15, 27, nst), MI355_NOP, MI355_ST_LOAD(Q, 11, ko));                     \
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                                                     \
+    __syncthreads();                                                                                                       \
+    __builtin_amdgcn_sched_barrier(0);                                                                                     \
+    MI355_ST_GROUP(0, fm1, fn1, nst, 0, fm0, fn0, MI355_NOP, MI355_NOP, MI355_ST_LOAD(Q, 12, ko));                         \
+    MI355_ST_GROUP(1, fm1, fn1, nst, 0, fm0, fn0, MI355_NOP, MI355_NOP, MI355_ST_LOAD(Q, 13, ko));                         \
+    MI355_ST_GROUP(2, fm1, fn1, nst, 0, fm0, fn0, MI355_NOP, MI355_NOP, MI355_ST_LOAD(Q, 14, ko));                         \
+    MI355_ST_GROUP(3, fm1, fn1, nst, 0, fm0, fn0, MI355_NOP, MI355_NOP, MI355_ST_LOAD(Q, 15, ko));                         \
+  } while (0)
+
+  for (int kt = 0; kt < KT; kt += 2) {
+    MI355_ST_SLAB(0, 1, kt);
+    MI355_ST_SLAB(1, 0, kt + 1);
+  }
+#undef MI355_ST_SLAB
+#undef MI355_ST_GROUP
+#undef MI355_NOP
+#undef MI355_ST_LOAD_ALL
+#undef MI355_ST_WRITE
+#undef MI355_ST_LOAD
+  // drain the speculative loads; every wave is past its last fragment read before the epilogue reuses LDS
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  if constexpr (sizeof(OutT) == 2) {
+    // fp16 epilogue through LDS, one wave-private region each, 32 rows per pass (see the tiled kernel)
+    constexpr int ROW_B = WTN * 2, CH = WTN / 8;
+    char* ep = lds + wave * (32 * ROW_B);
+    constexpr int ROWS_PER_IT = 64 / CH;
+    const int er = lane / CH, ec = lane % CH;
+#pragma unroll
+    for (int j = 0; j < TM; j++) {
+#pragma unroll
+      for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const int c = i * 4 + q;
+          half4 v = {(half_t)acc[i][j][4 * q], (half_t)acc[i][j][4 * q + 1], (half_t)acc[i][j][4 * q + 2],
+                     (half_t)acc[i][j][4 * q + 3]};
+          *reinterpret_cast<half4*>(ep + r32 * ROW_B + ((c ^ ((r32 >> 1) & 7)) * 16) + 8 * h) = v;
+        }
+      OutT* cbase = C + (size_t)(tile_m * BM + wm * WTM + j * 32) * N + tile_n * BN + wn * WTN + ec * 8;
+#pragma unroll
+      for (int it = 0; it < 32 / ROWS_PER_IT; it++) {
+        const int row = it * ROWS_PER_IT + er;
+        half8 v = *reinterpret_cast<const half8*>(ep + row * ROW_B + ((ec ^ ((row >> 1) & 7)) * 16));
+        *reinterpret_cast<half8*>(cbase + (size_t)row * N) = v;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  } else {
+    const int m0 = tile_m * BM + wm * WTM + r32;
+    const int n0 = tile_n * BN + wn * WTN + 4 * h;
+#pragma unroll
+    for (int j = 0; j < TM; j++) {
+      OutT* crow = C + (size_t)(m0 + j * 32) * N + n0;
+#pragma unroll
+      for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+          OutPack<OutT>::store4(crow + i * 32 + q * 8, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                                acc[i][j][4 * q + 3]);
+    }
+  }
+}
+
 // Persistent kernel: one workgroup per CU walks its share of the output tiles (tile ids pid, pid + grid,
 // ...) as ONE continuous sequence of K slabs.  The loads issued during the last two slabs of a tile
 // already fetch the first two slabs of the next tile, the fragment reads at the end of the last slab
@@ -666,6 +899,7 @@ static const GemmVariant kGemmVariants[] = {
     {"pipelined_128x128x64_w2x2", 128, 128, 256},
     {"tiled_256x256x64_w2x4", 256, 256, 512},
     {"tiled_128x128x64_w2x2", 128, 128, 256},
+    {"staged_256x256x64_w2x2", 256, 256, 256},
     {"generic_64x64x32", 64, 64, 256},
 };
 constexpr int kNumGemmVariants = sizeof(kGemmVariants) / sizeof(kGemmVariants[0]);
@@ -673,10 +907,12 @@ constexpr int kNumGemmVariants = sizeof(kGemmVariants) / sizeof(kGemmVariants[0]
 int gemm_variant_count() { return kNumGemmVariants; }
 const char* gemm_variant_name(int i) { return (i >= 0 && i < kNumGemmVariants) ? kGemmVariants[i].name : nullptr; }
 
-template <int BM, int BN, int WM, int WN, typename OutT, bool PIPELINED>
+template <int BM, int BN, int WM, int WN, typename OutT, int KIND>  // 0 tiled, 1 pipelined, 2 register-staged
 static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int K, hipStream_t stream) {
+  constexpr bool PIPELINED = KIND == 1;
   void (*kern)(const half_t*, const half_t*, OutT*, int, int, int, int, int, int);
-  if constexpr (PIPELINED) kern = gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT>;
+  if constexpr (KIND == 2) kern = gemm_f16_nt_staged<BM, BN, WM, WN, OutT>;
+  else if constexpr (PIPELINED) kern = gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT>;
   else kern = gemm_f16_nt_tiled<BM, BN, WM, WN, OutT>;
   constexpr int lds_bytes = 2 * (BM + BN) * 128;
   static bool attr_set = false;
@@ -694,7 +930,7 @@ static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int
   dim3 grid(tiles_m * tiles_n), block(WM * WN * 64);
   hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, M, N, K, tiles_m,
                      tiles_n, group_m);
-  return check_launch(PIPELINED ? "gemm_f16_nt_pipelined" : "gemm_f16_nt_tiled", grid, block, lds_bytes);
+  return check_launch(KIND == 2 ? "gemm_f16_nt_staged" : PIPELINED ? "gemm_f16_nt_pipelined" : "gemm_f16_nt_tiled", grid, block, lds_bytes);
 }
 
 // number of CUs of the device the stream's context is on (cached per device)
@@ -741,11 +977,12 @@ static int launch_variant(int variant, const void* a, const void* b, void* c, in
   switch (variant) {
     case 0: return launch_persistent<256, 256, 2, 4, OutT>(a, b, c, M, N, K, stream);
     case 1: return launch_persistent<256, 256, 2, 2, OutT>(a, b, c, M, N, K, stream);
-    case 2: return launch_tiled<256, 256, 2, 4, OutT, true>(a, b, c, M, N, K, stream);
-    case 3: return launch_tiled<256, 256, 2, 2, OutT, true>(a, b, c, M, N, K, stream);
-    case 4: return launch_tiled<128, 128, 2, 2, OutT, true>(a, b, c, M, N, K, stream);
-    case 5: return launch_tiled<256, 256, 2, 4, OutT, false>(a, b, c, M, N, K, stream);
-    case 6: return launch_tiled<128, 128, 2, 2, OutT, false>(a, b, c, M, N, K, stream);
+    case 2: return launch_tiled<256, 256, 2, 4, OutT, 1>(a, b, c, M, N, K, stream);
+    case 3: return launch_tiled<256, 256, 2, 2, OutT, 1>(a, b, c, M, N, K, stream);
+    case 4: return launch_tiled<128, 128, 2, 2, OutT, 1>(a, b, c, M, N, K, stream);
+    case 5: return launch_tiled<256, 256, 2, 4, OutT, 0>(a, b, c, M, N, K, stream);
+    case 6: return launch_tiled<128, 128, 2, 2, OutT, 0>(a, b, c, M, N, K, stream);
+    case 7: return launch_tiled<256, 256, 2, 2, OutT, 2>(a, b, c, M, N, K, stream);
     default: {
       dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
       hipLaunchKernelGGL(gemm_f16_nt_generic<OutT>, grid, block, 0, stream, (const half_t*)a, (const half_t*)b, (OutT*)c,
@@ -771,6 +1008,7 @@ extern "C" int mi355_gemm_f16_nt(const void* a, const void* b, void* c, int64_t 
   auto fits = [&](int v) {
     if (v == kNumGemmVariants - 1) return true;
     if (v <= 1 && (K < 128 || K > (1 << 21))) return false;  // prefetches two slabs ahead; 32-bit byte offsets inside a 256-row panel
+    if (v == 7 && (K < 256 || K % 128 != 0 || K > (1 << 21))) return false;  // slabs in pairs, three in flight
     return al && M % kGemmVariants[v].bm == 0 && N % kGemmVariants[v].bn == 0 && K % 64 == 0;
   };
   if (variant < 0) {
