@@ -1016,7 +1016,8 @@ extern "C" int mi355_gemm_f16_nt(const void* a, const void* b, void* c, int64_t 
     // 128x128 tile (4x the workgroups) wins; everything else goes to the bounds-checked kernel.
     const long long t256 = (M / 256) * (N / 256);
     const long long rounds = (t256 + 255) / 256;  // 256 CUs, one 256x256 workgroup each
-    if (fits(0) && t256 >= 128 && t256 * 100 >= rounds * 256 * 85) variant = 0;  // >= 85% of the last round busy
+    if (fits(7) && t256 >= 128) variant = 7;  // measured best on every large shape, also with a ragged last round
+    else if (fits(0) && t256 >= 128 && t256 * 100 >= rounds * 256 * 85) variant = 0;  // >= 85% of the last round busy
     else if (fits(4)) variant = 4;
     else variant = kNumGemmVariants - 1;
   } else if (!fits(variant)) {

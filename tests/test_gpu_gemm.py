@@ -166,3 +166,39 @@ def test_gemm_persistent_tile_walk(dev, shape, out_dtype):
     rows = torch.tensor([0, 255, 256, M - 1])
     exact = a[rows.to(dev)].float() @ b.float().t()
     torch.testing.assert_close(got[rows.to(dev)].float(), exact, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("out_dtype", ["float16", "float32"])
+@pytest.mark.parametrize("shape", [(256, 256, 256), (512, 768, 384), (1024, 512, 1152), (2048, 10240, 512)])
+def test_gemm_staged_slab_rotation(dev, shape, out_dtype):
+    """The register-staged kernel keeps three slabs in flight in two alternating register sets: the minimum of
+    four slabs, slab counts that are 2 and 0 mod 4 (the loop is written for pairs), a ragged tile grid and a
+    grid larger than the chip -- whole matrix against the independent generic kernel, rows against fp32."""
+    import iree_turbine_amd as ita
+    from oracle import inputs
+
+    M, N, K = shape
+    announce(f"gemm staged {shape} {out_dtype}")
+    names = ita._lib.variants("gemm_f16_nt")
+    v = next(i for i, n in enumerate(names) if n.startswith("staged"))
+    a, b = [t.to(dev) for t in inputs.gemm_inputs(M, N, K)]
+    got = torch.ops.mi355.gemm_nt(a, b, out_dtype, v)
+    ref = torch.ops.mi355.gemm_nt(a, b, out_dtype, len(names) - 1)
+    torch.testing.assert_close(got.float(), ref.float(), rtol=1e-3, atol=1e-3)
+    rows = torch.tensor([0, 127, 128, M - 1])
+    exact = a[rows.to(dev)].float() @ b.float().t()
+    torch.testing.assert_close(got[rows.to(dev)].float(), exact, rtol=RTOL, atol=ATOL)
+    assert torch.equal(got, torch.ops.mi355.gemm_nt(a, b, out_dtype, v))
+
+
+def test_gemm_staged_contract(dev):
+    import iree_turbine_amd as ita
+
+    names = ita._lib.variants("gemm_f16_nt")
+    v = next(i for i, n in enumerate(names) if n.startswith("staged"))
+    a = torch.zeros(256, 192, dtype=torch.float16, device=dev)
+    with pytest.raises(ValueError):
+        torch.ops.mi355.gemm_nt(a, a, "float16", v)  # K = 192 is not a whole number of slab pairs
+    a = torch.zeros(256, 128, dtype=torch.float16, device=dev)
+    with pytest.raises(ValueError):
+        torch.ops.mi355.gemm_nt(a, a, "float16", v)  # fewer than four slabs
