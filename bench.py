@@ -37,16 +37,17 @@ METRIC = "TFLOP/s & %MFMA peak (f16 GEMM, causal FA, MXFP4 GEMM); decode HBM GB/
 # dispatch, scaled by what the same counters read for a copy kernel of known size); filled in from
 # the summaries kept under profiles/.  None = not measured.
 MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
-    "gemm_8192": 1.764e9,              # 1555 MiB read + 128 MiB written: each of the 8 XCD L2s fetches its own copy of
+    "gemm_8192": 1.745e9,              # 1536 MiB read + 128 MiB written: each of the 8 XCD L2s fetches its own copy of
                                        # the panels its 4x8 block of output tiles needs (12 panels x 4 MiB x 4 rounds x 8)
-    "gemm_4096": 2.458e8,
-    "gemm_2048x10240x8192": 1.026e9,
-    "gemm_2048x57344x8192": 3.080e9,
-    "fa_causal": 2.701e8,
+    "gemm_4096": 2.351e8,
+    "gemm_2048x10240x8192": 6.461e8,
+    "gemm_2048x57344x8192": 3.054e9,
+    "fa_causal": 3.428e8,
     "fa_noncausal": 2.686e8,
     "decode": 1.178e9,
-    "mxfp4_4096x8192x8192": 2.950e8,
-    "mxfp4_32x8192x8192": 3.747e7,
+    "mxfp4_4096x8192x8192": 2.947e8,
+    "mxfp4_32x8192x8192": 3.748e7,
+    "mxfp4_quantize_16384x16384": 6.795e8,
 }
 
 
