@@ -28,7 +28,7 @@ def sdpa_ref(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, is_causal: bool 
 
 
 def sdpa_torch(q, k, v, is_causal=False, scale=None) -> torch.Tensor:
-    """torch's own SDPA in fp32 (the library routine BASELINE names as the oracle)."""
+    """torch's own SDPA in fp32 (the library routine the numerical contract names as the oracle)."""
     qf, kf, vf = (t.detach().cpu().float() for t in (q, k, v))
     return torch.nn.functional.scaled_dot_product_attention(qf, kf, vf, is_causal=is_causal, scale=scale)
 

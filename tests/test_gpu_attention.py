@@ -9,7 +9,7 @@ from conftest import announce
 
 pytestmark = pytest.mark.gpu
 
-ATOL = 2e-3  # the tolerance BASELINE states for fp16 attention outputs
+ATOL = 2e-3  # the contract tolerance for fp16 attention outputs
 RTOL = 1e-2
 
 

@@ -7,7 +7,7 @@ from conftest import announce
 
 pytestmark = pytest.mark.gpu
 
-RTOL = ATOL = 1e-2  # the tolerance BASELINE states for the fp16 GEMM
+RTOL = ATOL = 1e-2  # the contract tolerance for the fp16 GEMM
 
 
 def _run(dev, M, N, K, out_dtype, variant=-1, seed=10):

@@ -8,7 +8,7 @@ from conftest import announce
 
 pytestmark = pytest.mark.gpu
 
-REL = 1e-2  # BASELINE: GEMM within 1e-2 relative of an fp32 matmul on the dequantised operands
+REL = 1e-2  # the contract: GEMM within 1e-2 relative of an fp32 matmul on the dequantised operands
 
 
 def _rel_err(c: torch.Tensor, ref: torch.Tensor) -> float:
