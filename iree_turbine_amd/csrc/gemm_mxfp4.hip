@@ -734,6 +734,269 @@ __global__ __launch_bounds__(256) void mxfp4_dequant_kernel(const uint8_t* __res
   *reinterpret_cast<floatx2*>(out + 2 * idx) = floatx2{v[0], v[1]};
 }
 
+// Register-staged form (see gemm_f16_nt_staged for the reasoning): four waves with 128x128 wave tiles, the
+// codes of slab s+3 loaded into VGPRs while slab s computes, slab s+1 copied from registers into the LDS
+// stage that slab s-1 left, every memory instruction alone between two MFMAs, one barrier per slab.
+// Scales ride along as a 17th staging register: a lane owns one row of the tile and fetches the 16 scale
+// bytes of two slabs, A rows with the even slabs (their own group), B rows with the odd slabs (the group that
+// starts one slab later); they pass through four 4 KiB LDS buffers (A / B, group parity) from which every
+// lane reads one dword per row tile and slab -- bytes 4h..4h+3, picked by op_sel -- one slab ahead.
+template <typename OutT>
+__global__ __launch_bounds__(256) void gemm_mxfp4_staged(const uint8_t* __restrict__ A, const uint8_t* __restrict__ As,
+                                                         const uint8_t* __restrict__ B, const uint8_t* __restrict__ Bs,
+                                                         OutT* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n,
+                                                         int group_m) {
+  constexpr int BM = 256, BN = 256, WN = 2, NW = 4;
+  constexpr int WTM = 128, WTN = 128, TM = 4, TN = 4;
+  constexpr int A_BYTES = BM * 128, STAGE = (BM + BN) * 128;
+  constexpr int SC_OFF = 2 * STAGE;  // scale buffers: A parity 0, A parity 1, B parity 0, B parity 1, 4 KiB each
+  typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+  typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  int tile_m, tile_n;
+  map_tile_mx(blockIdx.x, tiles_m, tiles_n, group_m, tile_m, tile_n);
+
+  const unsigned row_bytes = (unsigned)K >> 1;  // codes
+  const unsigned sc_bytes = (unsigned)K >> 5;   // scale bytes per row
+  auto make_desc = [&](const uint8_t* base, unsigned bytes) {
+    const unsigned long long p = reinterpret_cast<unsigned long long>(base);
+    i32x4 d;
+    d[0] = __builtin_amdgcn_readfirstlane((int)(unsigned)p);
+    d[1] = __builtin_amdgcn_readfirstlane((int)(unsigned)((p >> 32) & 0xFFFFu));
+    d[2] = __builtin_amdgcn_readfirstlane((int)bytes);
+    d[3] = 0x00020000;
+    return d;
+  };
+  // codes: wave-load i covers rows (i * NW + wave) * 8 .. + 7 of the tile, 8 lanes per 128-byte row piece
+  const int lrow = lane >> 3, lc = lane & 7;
+  const i32x4 a_src = make_desc(A + (size_t)(tile_m * BM + wave * 8) * row_bytes, (unsigned)(BM - wave * 8) * row_bytes);
+  const i32x4 b_src = make_desc(B + (size_t)(tile_n * BN + wave * 8) * row_bytes, (unsigned)(BN - wave * 8) * row_bytes);
+  const unsigned g_off = (unsigned)lrow * row_bytes + (unsigned)lc * 16u;
+  const unsigned row_step = (unsigned)NW * 8u * row_bytes;
+  const int w_off = wave * 1024 + lrow * 128 + ((lc ^ (((wave & 1) << 2) | (lrow >> 1))) * 16);
+  // scales: lane l of wave w owns row 64 w + l of the tile
+  const i32x4 as_src = make_desc(As + (size_t)(tile_m * BM + wave * 64) * sc_bytes, (unsigned)(BM - wave * 64) * sc_bytes);
+  const i32x4 bs_src = make_desc(Bs + (size_t)(tile_n * BN + wave * 64) * sc_bytes, (unsigned)(BN - wave * 64) * sc_bytes);
+  const unsigned s_off = (unsigned)lane * sc_bytes;
+  int sc_wr = SC_OFF + 4096 + (wave * 64 + lane) * 16;  // where the NEXT group's A scales go (B: + 8192); flips per group
+
+  // staging registers: r[set][n], n < 8 the A row groups, 8..15 the B row groups, 16 the scale row
+  u32x4 r[2][17];
+#define MI355_MX_LOAD(S, n, k_off_)                                                                  \
+  asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"                                            \
+               : "=v"(r[S][n])                                                                       \
+               : "v"(g_off), "s"((n) < 8 ? a_src : b_src), "s"((k_off_) + (unsigned)((n)&7) * row_step) \
+               : "memory")
+#define MI355_MX_LOAD_SC(S, desc, group_)                                                            \
+  asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen" : "=v"(r[S][16]) : "v"(s_off), "s"(desc), "s"((unsigned)(group_)*16u) : "memory")
+  // `newer` = loads issued after the one that filled the register; they may still be in flight
+#define MI355_MX_WRITE(S, n, newer, st_)                                                                                   \
+  do {                                                                                                                     \
+    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(r[S][n]) : "n"(newer) : "memory");                                           \
+    *reinterpret_cast<u32x4*>((st_) + w_off + ((n) < 8 ? (n)*NW * 1024 : A_BYTES + ((n)-8) * NW * 1024)) = r[S][n];        \
+  } while (0)
+#define MI355_MX_WRITE_SC(S, newer, addr_)                                                   \
+  do {                                                                                       \
+    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(r[S][16]) : "n"(newer) : "memory");            \
+    *reinterpret_cast<u32x4*>(lds + (addr_)) = r[S][16];                                     \
+  } while (0)
+
+  const int r32 = lane & 31, h = lane >> 5;
+  const int sw = ((4 * h) ^ ((r32 >> 1) & 7)) * 16;  // chunk ks + 4h of the row, swizzled
+  const int a_base = (wm * WTM + r32) * 128 + sw;
+  const int b_base = A_BYTES + (wn * WTN + r32) * 128 + sw;
+  // scale dwords of the CURRENT group (parity flips per group); + 8 for the group's second slab
+  int sc_rd_a = SC_OFF + (wm * WTM + r32) * 16 + 4 * h;
+  int sc_rd_b = SC_OFF + 8192 + (wn * WTN + r32) * 16 + 4 * h;
+
+  floatx16 acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; i++)
+#pragma unroll
+    for (int j = 0; j < TM; j++)
+#pragma unroll
+      for (int q = 0; q < 16; q++) acc[i][j][q] = 0.f;
+
+  const int KT = K / 256;  // even, >= 4 (checked on the host)
+  intx4 fm0[TM], fn0[TN], fm1[TM], fn1[TN];
+  int ca0[TM], cb0[TN], ca1[TM], cb1[TN];
+
+#define MI355_MX_LOAD_ALL(S, slab_)                                                                              \
+  do {                                                                                                           \
+    const unsigned ko_ = (unsigned)(slab_)*128u;                                                                 \
+    MI355_MX_LOAD(S, 0, ko_); MI355_MX_LOAD(S, 1, ko_); MI355_MX_LOAD(S, 2, ko_); MI355_MX_LOAD(S, 3, ko_);      \
+    MI355_MX_LOAD(S, 4, ko_); MI355_MX_LOAD(S, 5, ko_); MI355_MX_LOAD(S, 6, ko_); MI355_MX_LOAD(S, 7, ko_);      \
+    MI355_MX_LOAD(S, 8, ko_); MI355_MX_LOAD(S, 9, ko_); MI355_MX_LOAD(S, 10, ko_); MI355_MX_LOAD(S, 11, ko_);    \
+    MI355_MX_LOAD(S, 12, ko_); MI355_MX_LOAD(S, 13, ko_); MI355_MX_LOAD(S, 14, ko_); MI355_MX_LOAD(S, 15, ko_);  \
+  } while (0)
+  // prologue: slab 0 (+ A scales of group 0) -> set 0 -> stage 0; B scales of group 0 through a spare
+  // register; slab 1 (+ B scales of group 1) -> set 1; then slab 2 (+ A scales of group 1) -> set 0
+  const int KG = KT / 2;  // scale groups
+  u32x4 rs;
+  MI355_MX_LOAD_ALL(0, 0);
+  MI355_MX_LOAD_SC(0, as_src, 0);
+  asm volatile("buffer_load_dwordx4 %0, %1, %2, 0 offen" : "=v"(rs) : "v"(s_off), "s"(bs_src) : "memory");
+  MI355_MX_LOAD_ALL(1, 1);
+  MI355_MX_LOAD_SC(1, bs_src, KG > 1 ? 1 : 0);
+  MI355_MX_WRITE(0, 0, 17, lds); MI355_MX_WRITE(0, 1, 17, lds); MI355_MX_WRITE(0, 2, 17, lds); MI355_MX_WRITE(0, 3, 17, lds);
+  MI355_MX_WRITE(0, 4, 17, lds); MI355_MX_WRITE(0, 5, 17, lds); MI355_MX_WRITE(0, 6, 17, lds); MI355_MX_WRITE(0, 7, 17, lds);
+  MI355_MX_WRITE(0, 8, 17, lds); MI355_MX_WRITE(0, 9, 17, lds); MI355_MX_WRITE(0, 10, 17, lds); MI355_MX_WRITE(0, 11, 17, lds);
+  MI355_MX_WRITE(0, 12, 17, lds); MI355_MX_WRITE(0, 13, 17, lds); MI355_MX_WRITE(0, 14, 17, lds); MI355_MX_WRITE(0, 15, 17, lds);
+  MI355_MX_WRITE_SC(0, 17, sc_wr - 4096);
+  asm volatile("s_waitcnt vmcnt(17)" : "+v"(rs) : : "memory");
+  *reinterpret_cast<u32x4*>(lds + sc_wr - 4096 + 8192) = rs;
+  MI355_MX_LOAD_ALL(0, 2);
+  MI355_MX_LOAD_SC(0, as_src, KG > 1 ? 1 : 0);
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < TM; j++) {
+    fm0[j] = *reinterpret_cast<const intx4*>(lds + (a_base + j * 4096));
+    fn0[j] = *reinterpret_cast<const intx4*>(lds + (b_base + j * 4096));
+    ca0[j] = *reinterpret_cast<const int*>(lds + sc_rd_a + j * 512);
+    cb0[j] = *reinterpret_cast<const int*>(lds + sc_rd_b + j * 512);
+  }
+
+  // fragment reads of the next k-step: A fragments in groups 0 and 1, B fragments in groups 2 and 3
+  auto frag_reads = [&](int g, const char* rst, int rks, intx4* fm_n, intx4* fn_n) {
+    if (g < 2) {
+      fm_n[2 * g] = *reinterpret_cast<const intx4*>(rst + ((a_base ^ (rks * 16)) + (2 * g) * 4096));
+      fm_n[2 * g + 1] = *reinterpret_cast<const intx4*>(rst + ((a_base ^ (rks * 16)) + (2 * g + 1) * 4096));
+    } else {
+      fn_n[2 * g - 4] = *reinterpret_cast<const intx4*>(rst + ((b_base ^ (rks * 16)) + (2 * g - 4) * 4096));
+      fn_n[2 * g - 3] = *reinterpret_cast<const intx4*>(rst + ((b_base ^ (rks * 16)) + (2 * g - 3) * 4096));
+    }
+  };
+  // scale dwords of the next slab (two per group of four MFMAs), `half` = 0 / 8 for the slab within its group
+  auto scale_reads = [&](int g, int half, int* ca_n, int* cb_n) {
+    if (g < 2) {
+      ca_n[2 * g] = *reinterpret_cast<const int*>(lds + sc_rd_a + half + (2 * g) * 512);
+      ca_n[2 * g + 1] = *reinterpret_cast<const int*>(lds + sc_rd_a + half + (2 * g + 1) * 512);
+    } else {
+      cb_n[2 * g - 4] = *reinterpret_cast<const int*>(lds + sc_rd_b + half + (2 * g - 4) * 512);
+      cb_n[2 * g - 3] = *reinterpret_cast<const int*>(lds + sc_rd_b + half + (2 * g - 3) * 512);
+    }
+  };
+#define MI355_MX_GROUP(KS, g, fm, fn, ca, cb, READS, W1, W2, LD)                        \
+  do {                                                                                  \
+    acc[g][0] = mfma_fp4_32x32x64<KS>(fn[g], cb[g], fm[0], ca[0], acc[g][0]);           \
+    W1;                                                                                 \
+    __builtin_amdgcn_sched_barrier(0);                                                  \
+    acc[g][1] = mfma_fp4_32x32x64<KS>(fn[g], cb[g], fm[1], ca[1], acc[g][1]);           \
+    W2;                                                                                 \
+    __builtin_amdgcn_sched_barrier(0);                                                  \
+    acc[g][2] = mfma_fp4_32x32x64<KS>(fn[g], cb[g], fm[2], ca[2], acc[g][2]);           \
+    LD;                                                                                 \
+    __builtin_amdgcn_sched_barrier(0);                                                  \
+    acc[g][3] = mfma_fp4_32x32x64<KS>(fn[g], cb[g], fm[3], ca[3], acc[g][3]);           \
+    READS;                                                                              \
+    __builtin_amdgcn_sched_barrier(0);                                                  \
+  } while (0)
+#define MI355_NOP ((void)0)
+
+  // Slab kt (scales in ca/cb) sits in stage P; set Q = 1 - P holds slab kt+1 and the scale row SCD travels
+  // with (written to SCW), and is reloaded register by register with slab kt+3 and the scales of group GN.
+  // In flight when register n is written: the rest of its own round (16 - n), the 17 loads of the other
+  // set, and the loads of this slab issued so far.  HALF = 8 if slab kt+1 is the second slab of its group.
+#define MI355_MX_SLAB(P, Q, kt_, ca, cb, ca_n, cb_n, SCD, SCW, GN, HALF)                                                    \
+  do {                                                                                                                     \
+    const char* st = lds + P * STAGE;                                                                                      \
+    char* nst = lds + Q * STAGE;                                                                                           \
+    const int nxt_ = (kt_) + 3 < KT ? (kt_) + 3 : KT - 1; /* past the end: re-fetch, never used */                         \
+    const unsigned ko = (unsigned)nxt_ * 128u;                                                                             \
+    const int gn_ = (GN) < KG ? (GN) : KG - 1;                                                                             \
+    __builtin_amdgcn_sched_barrier(0);                                                                                     \
+    MI355_MX_GROUP(0, 0, fm0, fn0, ca, cb, frag_reads(0, st, 1, fm1, fn1), MI355_MX_WRITE(Q, 0, 33, nst), MI355_MX_WRITE(Q, 1, 32, nst), MI355_MX_LOAD(Q, 0, ko));   \
+    MI355_MX_GROUP(0, 1, fm0, fn0, ca, cb, frag_reads(1, st, 1, fm1, fn1), MI355_MX_WRITE(Q, 2, 32, nst), MI355_NOP, MI355_MX_LOAD(Q, 1, ko));                       \
+    MI355_MX_GROUP(0, 2, fm0, fn0, ca, cb, frag_reads(2, st, 1, fm1, fn1), MI355_MX_WRITE(Q, 3, 32, nst), MI355_MX_WRITE(Q, 4, 31, nst), MI355_MX_LOAD(Q, 2, ko));   \
+    MI355_MX_GROUP(0, 3, fm0, fn0, ca, cb, frag_reads(3, st, 1, fm1, fn1), MI355_MX_WRITE(Q, 5, 31, nst), MI355_NOP, MI355_MX_LOAD(Q, 3, ko));                       \
+    MI355_MX_GROUP(1, 0, fm1, fn1, ca, cb, frag_reads(0, st, 2, fm0, fn0), MI355_MX_WRITE(Q, 6, 31, nst), MI355_MX_WRITE(Q, 7, 30, nst), MI355_MX_LOAD(Q, 4, ko));   \
+    MI355_MX_GROUP(1, 1, fm1, fn1, ca, cb, frag_reads(1, st, 2, fm0, fn0), MI355_MX_WRITE(Q, 8, 30, nst), MI355_NOP, MI355_MX_LOAD(Q, 5, ko));                       \
+    MI355_MX_GROUP(1, 2, fm1, fn1, ca, cb, frag_reads(2, st, 2, fm0, fn0), MI355_MX_WRITE(Q, 9, 30, nst), MI355_MX_WRITE(Q, 10, 29, nst), MI355_MX_LOAD(Q, 6, ko));  \
+    MI355_MX_GROUP(1, 3, fm1, fn1, ca, cb, frag_reads(3, st, 2, fm0, fn0), MI355_MX_WRITE(Q, 11, 29, nst), MI355_NOP, MI355_MX_LOAD(Q, 7, ko));                      \
+    MI355_MX_GROUP(2, 0, fm0, fn0, ca, cb, frag_reads(0, st, 3, fm1, fn1), MI355_MX_WRITE(Q, 12, 29, nst), MI355_NOP, MI355_MX_LOAD(Q, 8, ko));                      \
+    MI355_MX_GROUP(2, 1, fm0, fn0, ca, cb, frag_reads(1, st, 3, fm1, fn1), MI355_MX_WRITE(Q, 13, 29, nst), MI355_NOP, MI355_MX_LOAD(Q, 9, ko));                      \
+    MI355_MX_GROUP(2, 2, fm0, fn0, ca, cb, frag_reads(2, st, 3, fm1, fn1), MI355_MX_WRITE(Q, 14, 29, nst), MI355_NOP, MI355_MX_LOAD(Q, 10, ko));                     \
+    MI355_MX_GROUP(2, 3, fm0, fn0, ca, cb, frag_reads(3, st, 3, fm1, fn1), MI355_MX_WRITE(Q, 15, 29, nst), MI355_MX_WRITE_SC(Q, 28, SCW), MI355_MX_LOAD(Q, 11, ko)); \
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                                                     \
+    __syncthreads();                                                                                                       \
+    __builtin_amdgcn_sched_barrier(0);                                                                                     \
+    if (HALF == 0) { sc_rd_a ^= 4096; sc_rd_b ^= 4096; }                                                                   \
+    MI355_MX_GROUP(3, 0, fm1, fn1, ca, cb, frag_reads(0, nst, 0, fm0, fn0); scale_reads(0, HALF, ca_n, cb_n), MI355_NOP, MI355_NOP, MI355_MX_LOAD(Q, 12, ko)); \
+    MI355_MX_GROUP(3, 1, fm1, fn1, ca, cb, frag_reads(1, nst, 0, fm0, fn0); scale_reads(1, HALF, ca_n, cb_n), MI355_NOP, MI355_NOP, MI355_MX_LOAD(Q, 13, ko)); \
+    MI355_MX_GROUP(3, 2, fm1, fn1, ca, cb, frag_reads(2, nst, 0, fm0, fn0); scale_reads(2, HALF, ca_n, cb_n), MI355_NOP, MI355_NOP, MI355_MX_LOAD(Q, 14, ko)); \
+    MI355_MX_GROUP(3, 3, fm1, fn1, ca, cb, frag_reads(3, nst, 0, fm0, fn0); scale_reads(3, HALF, ca_n, cb_n), MI355_NOP, MI355_NOP,                            \
+                   MI355_MX_LOAD(Q, 15, ko); MI355_MX_LOAD_SC(Q, SCD, gn_));                                             \
+  } while (0)
+
+  for (int kt = 0; kt < KT; kt += 2) {
+    const int g0 = kt >> 1;
+    // even slab: set 1 carries slab kt+1 and the B scales of group g0+1; reloaded with slab kt+3 and the B scales of g0+2
+    MI355_MX_SLAB(0, 1, kt, ca0, cb0, ca1, cb1, bs_src, sc_wr + 8192, g0 + 2, 8);
+    // odd slab: set 0 carries slab kt+2 and the A scales of group g0+1; reloaded with slab kt+4 and the A scales of g0+2
+    MI355_MX_SLAB(1, 0, kt + 1, ca1, cb1, ca0, cb0, as_src, sc_wr, g0 + 2, 0);
+    sc_wr ^= 4096;
+  }
+#undef MI355_MX_SLAB
+#undef MI355_MX_GROUP
+#undef MI355_NOP
+#undef MI355_MX_LOAD_ALL
+#undef MI355_MX_WRITE_SC
+#undef MI355_MX_WRITE
+#undef MI355_MX_LOAD_SC
+#undef MI355_MX_LOAD
+  // drain the speculative loads; every wave is past its last fragment read before the epilogue reuses LDS
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  if constexpr (sizeof(OutT) == 2) {
+    // bf16 epilogue through LDS, one wave-private region each, 32 rows per pass: ds_write_b64 of 4 consecutive n
+    // (chunk slot c ^ ((m >> 1) & 7)), whole 256-byte rows read back 16 bytes per lane
+    constexpr int ROW_B = WTN * 2, CH = WTN / 8;
+    char* ep = lds + wave * (32 * ROW_B);
+    constexpr int ROWS_PER_IT = 64 / CH;
+    const int er = lane / CH, ec = lane % CH;
+#pragma unroll
+    for (int j = 0; j < TM; j++) {
+#pragma unroll
+      for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const int c = i * 4 + q;
+          ushortx4 v = {f32_to_bf16_rne(acc[i][j][4 * q]), f32_to_bf16_rne(acc[i][j][4 * q + 1]),
+                        f32_to_bf16_rne(acc[i][j][4 * q + 2]), f32_to_bf16_rne(acc[i][j][4 * q + 3])};
+          *reinterpret_cast<ushortx4*>(ep + r32 * ROW_B + ((c ^ ((r32 >> 1) & 7)) * 16) + 8 * h) = v;
+        }
+      OutT* cbase = C + (size_t)(tile_m * BM + wm * WTM + j * 32) * N + tile_n * BN + wn * WTN + ec * 8;
+#pragma unroll
+      for (int it = 0; it < 32 / ROWS_PER_IT; it++) {
+        const int row = it * ROWS_PER_IT + er;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(ep + row * ROW_B + ((ec ^ ((row >> 1) & 7)) * 16));
+        *reinterpret_cast<u32x4*>(cbase + (size_t)row * N) = v;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  } else {
+    const int m0 = tile_m * BM + wm * WTM + r32;
+    const int n0 = tile_n * BN + wn * WTN + 4 * h;
+#pragma unroll
+    for (int j = 0; j < TM; j++) {
+      OutT* crow = C + (size_t)(m0 + j * 32) * N + n0;
+#pragma unroll
+      for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+          MxOut<OutT>::store4(crow + i * 32 + q * 8, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                              acc[i][j][4 * q + 3]);
+    }
+  }
+}
+
 struct MxVariant {
   const char* name;
   int bm, bn;
@@ -743,6 +1006,7 @@ static const MxVariant kMxVariants[] = {
     {"tiled_256x256x256_w2x4", 256, 256},
     {"tiled_128x128x256_w2x2", 128, 128},
     {"skinny_m32_n32_w8", 32, 32},
+    {"staged_256x256x256_w2x2", 256, 256},
     {"generic_32x128", 32, 128},
 };
 constexpr int kNumMxVariants = sizeof(kMxVariants) / sizeof(kMxVariants[0]);
@@ -810,6 +1074,28 @@ static int launch_mx_persistent(const void* a, const void* as, const void* b, co
 }
 
 template <typename OutT>
+static int launch_mx_staged(const void* a, const void* as, const void* b, const void* bs, void* c, int M, int N, int K,
+                            hipStream_t stream) {
+  auto kern = gemm_mxfp4_staged<OutT>;
+  constexpr int lds_bytes = 2 * 512 * 128 + 4 * 4096;  // two data stages, four scale buffers
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       lds_bytes);
+    if (e != hipSuccess) {
+      set_error("hipFuncSetAttribute(gemm_mxfp4_staged, %d bytes LDS): %s", lds_bytes, hipGetErrorString(e));
+      return (int)e;
+    }
+    attr_set = true;
+  }
+  const int tiles_m = M / 256, tiles_n = N / 256;
+  dim3 grid(tiles_m * tiles_n), block(256);
+  hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const uint8_t*)a, (const uint8_t*)as, (const uint8_t*)b,
+                     (const uint8_t*)bs, (OutT*)c, M, N, K, tiles_m, tiles_n, 4);
+  return check_launch("gemm_mxfp4_staged", grid, block, lds_bytes);
+}
+
+template <typename OutT>
 static int launch_mx(int variant, const void* a, const void* as, const void* b, const void* bs, void* c, int M, int N, int K,
                      hipStream_t stream) {
   switch (variant) {
@@ -837,6 +1123,7 @@ static int launch_mx(int variant, const void* a, const void* as, const void* b, 
                          (const uint8_t*)bs, (OutT*)c, M, N, K);
       return check_launch("gemm_mxfp4_skinny", grid, block, lds_bytes);
     }
+    case 4: return launch_mx_staged<OutT>(a, as, b, bs, c, M, N, K, stream);
     default: {
       dim3 grid((N + 127) / 128, (M + 31) / 32), block(256);
       hipLaunchKernelGGL(gemm_mxfp4_generic<OutT>, grid, block, 0, stream, (const uint8_t*)a, (const uint8_t*)as,
@@ -867,7 +1154,7 @@ extern "C" int mi355_mxfp4_gemm(const void* a, const void* a_scale, const void* 
   auto fits = [&](int v) {
     if (v == kNumMxVariants - 1) return true;
     if (v == 3) return sc_al4 && M <= 32 && N % 32 == 0 && K % 256 == 0;  // skinny: whole 128-byte segments
-    if (v == 0 && !(sc_al16 && K % 512 == 0 && K >= 1024 && K <= (1 << 22))) return false;  // persistent: 2-slab scale groups
+    if ((v == 0 || v == 4) && !(sc_al16 && K % 512 == 0 && K >= 1024 && K <= (1 << 22))) return false;  // 2-slab scale groups
     return sc_al && M % kMxVariants[v].bm == 0 && N % kMxVariants[v].bn == 0 && K % 256 == 0;
   };
   if (variant < 0) {
@@ -878,6 +1165,7 @@ extern "C" int mi355_mxfp4_gemm(const void* a, const void* a_scale, const void* 
     const long long rounds = (t256 + 255) / 256;
     const bool big = t256 >= 128 && t256 * 100 >= rounds * 256 * 85;
     if (fits(3)) variant = 3;
+    else if (big && K >= 32768 && fits(4)) variant = 4;  // its epilogue is not overlapped: ahead only from 128 slabs per tile
     else if (big && fits(0)) variant = 0;
     else if (big && fits(1)) variant = 1;
     else if (fits(2)) variant = 2;

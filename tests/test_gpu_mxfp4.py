@@ -43,7 +43,7 @@ def test_dequant_random_bit_exact(dev):
     assert np.array_equal(out.view(np.uint32), om.mxfp4_dequant_ref(a, asc).view(np.uint32))
 
 
-@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 4])
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 4, 5])
 def test_mxfp4_gemm_variants(dev, variant):
     import iree_turbine_amd  # noqa: F401
     from oracle import inputs, mxfp4 as om
@@ -74,7 +74,7 @@ def test_mxfp4_gemm_ragged(dev, shape):
 
 
 @pytest.mark.parametrize("shape", [(32, 256, 512), (1, 64, 256), (7, 96, 2048), (32, 8192, 8192), (20, 160, 16384), (32, 64, 8192 + 256)])
-@pytest.mark.parametrize("variant", [3, 4])
+@pytest.mark.parametrize("variant", [3, 5])
 def test_mxfp4_skinny_vs_generic(dev, shape, variant):
     """The weight-streaming kernel (variant 3) and the any-shape kernel (variant 4) on skinny shapes."""
     import iree_turbine_amd  # noqa: F401
@@ -213,3 +213,28 @@ def test_mxfp4_contract_errors(dev):
         torch.ops.mi355.mxfp4_gemm(a, s[:, :0], a, s, "bfloat16", -1)
     with pytest.raises(ValueError):
         torch.ops.mi355.mxfp4_gemm(a, s, a, s, "float16", -1)
+
+
+@pytest.mark.parametrize("shape", [(256, 256, 1024), (512, 768, 1536), (4352, 4352, 1024), (256, 512, 8192)])
+@pytest.mark.parametrize("out_dtype", ["bfloat16", "float32"])
+def test_mxfp4_staged_slab_rotation(dev, shape, out_dtype):
+    """The register-staged kernel keeps three slabs and two scale groups in flight: the minimum of four slabs,
+    odd and even numbers of scale groups (the scale buffer parity), a ragged tile grid larger than the chip
+    and a long K -- whole matrix against the independent generic kernel."""
+    import iree_turbine_amd as ita
+    from oracle import inputs
+
+    M, N, K = shape
+    announce(f"mxfp4 staged {shape} {out_dtype}")
+    names = ita._lib.variants("mxfp4_gemm")
+    v = next(i for i, n in enumerate(names) if n.startswith("staged"))
+    a, asc, b, bsc = [t.to(dev) for t in inputs.mxfp4_inputs(M, N, K)]
+    got = torch.ops.mi355.mxfp4_gemm(a, asc, b, bsc, out_dtype, v)
+    ref = torch.ops.mi355.mxfp4_gemm(a, asc, b, bsc, out_dtype, len(names) - 1)
+    if out_dtype == "float32":
+        assert _rel_err(got, ref) < 1e-5
+    else:
+        g32, r32 = got.float(), ref.float()
+        assert _rel_err(g32, r32) < 1e-3
+        assert ((g32 - r32).abs() <= r32.abs() * 2 ** -7 + 1e-5 * r32.abs().max()).all()
+    assert torch.equal(got, torch.ops.mi355.mxfp4_gemm(a, asc, b, bsc, out_dtype, v))
