@@ -44,6 +44,23 @@ def test_attention_cross_lengths(dev, causal):
     torch.testing.assert_close(o, ref, rtol=RTOL, atol=ATOL)
 
 
+def test_attention_causal_more_queries_than_keys(dev):
+    """Lower-right aligned causal mask with Sq > Sk: query i sees keys j <= i - (Sq - Sk), so the first
+    Sq - Sk queries see no key at all.  Those rows are defined as zero (the sum of an empty softmax); every
+    other row matches the oracle."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import attention as oa, inputs
+
+    B, H, Sq, Sk, D = 1, 2, 300, 100, 128  # the boundary falls inside a wave: rows with and without keys side by side
+    announce(f"flash_attn_fwd causal Sq={Sq} > Sk={Sk}")
+    q, k, v = inputs.attention_inputs(B, H, Sq, D, seed=11, Sk=Sk)
+    o = torch.ops.mi355.flash_attn_fwd(q.to(dev), k.to(dev), v.to(dev), True, 0.0).float().cpu()
+    empty = Sq - Sk
+    assert torch.equal(o[:, :, :empty], torch.zeros_like(o[:, :, :empty]))
+    ref = oa.sdpa_ref(q[:, :, empty:], k, v, is_causal=True)  # the remaining Sk queries against Sk keys: square mask
+    torch.testing.assert_close(o[:, :, empty:], ref, rtol=RTOL, atol=ATOL)
+
+
 def test_attention_invariants(dev):
     import iree_turbine_amd  # noqa: F401
 
