@@ -152,6 +152,27 @@ def wl_decode():
     return build
 
 
+def wl_paged_prefill(num_seqs=16, n_new=512, min_len=1024, max_len=8192):
+    from oracle import inputs
+
+    def build(dev):
+        _, kc, vc, bt, sl = inputs.paged_decode_inputs(num_seqs=num_seqs, min_len=min_len, max_len=max_len)
+        q = torch.randn((num_seqs, n_new, 32, 128), generator=torch.Generator().manual_seed(10)).half()
+        args = [t.to(dev) for t in (q, kc, vc, bt, sl)]
+        # query t of a sequence of length L sees L - n_new + t + 1 cached positions
+        visible = sum(n_new * (int(L) - n_new) + n_new * (n_new + 1) // 2 for L in sl.tolist())
+        flops = 4.0 * visible * 32 * 128
+        return {
+            "fn": lambda: torch.ops.mi355.paged_prefill_attn(*args, 0.0),
+            "work": flops, "bytes": 4096.0 * int(sl.sum()) + 2 * q.numel() * 2.0, "bound": "mfma", "peak": PEAK_F16_TFLOPS,
+            "unit": "TFLOP/s", "dtype": "f16", "cpu": lambda: cpu_paged_prefill(q, kc, vc, bt, sl),
+            "config": {"workload": f"paged_prefill_{num_seqs}seq_{n_new}new_32q8kv_D128_page16_ctx{min_len}-{max_len}",
+                       "num_seqs": num_seqs, "n_new": n_new, "q_heads": 32, "kv_heads": 8, "D": 128, "page": 16,
+                       "total_tokens": int(sl.sum()), "seed": 10},
+        }
+    return build
+
+
 def wl_mxfp4(M, N, K):
     from oracle import inputs
 
@@ -210,6 +231,7 @@ WORKLOADS = {
     "fa_causal": wl_attention(True),
     "fa_noncausal": wl_attention(False),
     "decode": wl_decode(),
+    "paged_prefill": wl_paged_prefill(),
     "mxfp4_4096x8192x8192": wl_mxfp4(4096, 8192, 8192),
     "mxfp4_32x8192x8192": wl_mxfp4(32, 8192, 8192),
     "mxfp4_quantize_16384x16384": wl_quantize(16384, 16384),
@@ -270,6 +292,16 @@ def cpu_decode(q, kc, vc, bt, sl):
     t = _time_cpu(lambda: op.paged_decode_ref(q[:n], kc, vc, bt[:n], sl[:n]), reps=2)
     return {"value": 4096.0 * int(sl[:n].sum()) / t / 1e9, "unit": "GB/s",
             "sample": f"gather + dense fp32 attention for {n} of the {q.shape[0]} sequences, best of 2 after 1 warm-up"}
+
+
+def cpu_paged_prefill(q, kc, vc, bt, sl):
+    from oracle import paged_decode as op
+    n, t_new = 1, 64
+    t = _time_cpu(lambda: op.paged_prefill_ref(q[:n, :t_new], kc, vc, bt[:n], sl[:n]), reps=2)
+    L = int(sl[0])
+    flops = 4.0 * (t_new * (L - t_new) + t_new * (t_new + 1) // 2) * q.shape[2] * q.shape[3]
+    return {"value": flops / t / 1e12, "unit": "TFLOP/s",
+            "sample": f"gather + dense fp32 causal attention for the last {t_new} tokens of 1 of the {q.shape[0]} sequences, best of 2 after 1 warm-up"}
 
 
 def cpu_mxfp4(a, asc, b, bsc, M, N, K):

@@ -167,6 +167,31 @@ int mi355_kv_cache_append(const void* k_new, const void* v_new, void* k_cache, v
                           void* stream);
 
 /*
+ * Prefill over a paged KV cache (chunked / prefix prefill, the step between append and decode):
+ * the num_new latest tokens of every sequence attend to that sequence's cached keys and values,
+ * causally -- query t (0-based among the new tokens) of sequence s sees cache positions
+ * j <= seq_lens[s] - num_new + t, the mask of tests/dynamo/llama_test.py:285-290 shifted by the
+ * cached prefix.  The new tokens' own K/V are expected in the cache already
+ * (mi355_kv_cache_append), so seq_lens counts them.
+ * q, out:      [num_seqs, num_new, num_q_heads, D]        fp16
+ * k_cache,
+ * v_cache:     [num_pages, page_size, num_kv_heads, D]    fp16
+ * block_table: [num_seqs, max_pages_per_seq] int32; entries at or beyond
+ *              ceil(seq_len/page_size) are never read, ids outside [0, num_pages) read as zeros
+ * seq_lens:    [num_seqs] int32 (clamped to [0, max_pages_per_seq * page_size]); queries with
+ *              no visible key produce zeros
+ * D == 128, page_size == 16, num_q_heads % num_kv_heads == 0.  Same kernel as
+ * mi355_flash_attn_fwd (fp32 online softmax, fp16 output), K/V tiles fetched page by page.
+ * Replaces: the prefill call of the attention in tests/dynamo/llama_test.py:144-182 when the
+ * cache is paged (no surviving paged counterpart in the reference).
+ */
+int mi355_paged_prefill_attn(const void* q, const void* k_cache, const void* v_cache,
+                             const void* block_table, const void* seq_lens, void* out,
+                             int64_t num_seqs, int64_t num_new, int64_t num_q_heads,
+                             int64_t num_kv_heads, int64_t D, int64_t page_size,
+                             int64_t max_pages_per_seq, int64_t num_pages, float scale, void* stream);
+
+/*
  * Block-scaled MXFP4 GEMM: C[M,N] = dq(A) . dq(B)^T, fp32 accumulation, bf16 out.
  * a: uint8 [M, K/2], b: uint8 [N, K/2]  -- two E2M1 codes per byte, element 2i
  *    in the low nibble, element 2i+1 in the high nibble;

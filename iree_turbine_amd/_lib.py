@@ -58,6 +58,7 @@ _PROTOS = {
         + [c_float, c_int64, c_void_p],
     ),
     "mi355_kv_cache_append": (c_int, [c_void_p] * 6 + [c_int64] * 7 + [c_void_p]),
+    "mi355_paged_prefill_attn": (c_int, [c_void_p] * 6 + [c_int64] * 8 + [c_float, c_void_p]),
     "mi355_mxfp4_gemm": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_void_p],

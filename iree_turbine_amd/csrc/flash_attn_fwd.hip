@@ -219,6 +219,14 @@ __global__ __launch_bounds__(256) void fa_fwd_d128(const half_t* __restrict__ Q,
   }
 }
 
+// Paged K/V (PAGED kernels): the keys and values of sequence b are the first seq_lens[b] token rows of the
+// pages block_table[b][0..], 16 tokens per page, laid out [page][token][kv head][128].
+struct FaPaged {
+  const int* block_table;  // [batch][max_pages]
+  const int* seq_lens;     // [batch]
+  int max_pages, num_pages;
+};
+
 // Software-pipelined form.  Same tiling and register layout, but the score MFMAs run one key tile
 // ahead of the softmax: in trip j a wave issues S^T(j+1) = K(j+1) . Q^T, exponentiates the scores of
 // tile j on the VALU while those MFMAs execute, then issues O^T += V(j)^T . P(j)^T.  K and V sit in
@@ -229,10 +237,10 @@ __global__ __launch_bounds__(256) void fa_fwd_d128(const half_t* __restrict__ Q,
 // the same quotient), which keeps the 64-register rescale off the common path.
 // V swizzle: chunk c of row r -> slot c ^ (4 * (r & 3)), which keeps the four 64-byte row pieces that a
 // half-wave transpose read touches on distinct banks (measured conflict-free; c ^ 2(r & 7) is not).
-template <bool CAUSAL>
+template <bool CAUSAL, bool PAGED = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void fa_fwd_d128_pipe(
     const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V, half_t* __restrict__ O, int BH,
-    int Sq, int Sk, float scale_log2e, int q_blocks, FaLayout lay) {
+    int Sq, int Sk_arg, float scale_log2e, int q_blocks, FaLayout lay, FaPaged pg) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   constexpr int TILE_B = FA_BLOCK_N * 256;  // bytes of one K or V tile
   constexpr int VBUF = 2 * TILE_B;          // K ring at 0, V ring behind it
@@ -258,11 +266,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       unit = pid % units;
     }
   }
-  const int causal_off = Sk - Sq;
   const int b_idx = bh / lay.H, h_idx = bh - b_idx * lay.H, hk_idx = h_idx / lay.group;
+  int Sk = Sk_arg;
+  if constexpr (PAGED) {
+    Sk = __builtin_amdgcn_readfirstlane(pg.seq_lens[b_idx]);
+    Sk = Sk < 0 ? 0 : (Sk > pg.max_pages * 16 ? pg.max_pages * 16 : Sk);
+  }
+  const int causal_off = Sk - Sq;
   const half_t* Qb = Q + b_idx * lay.q_b + h_idx * lay.q_h;
-  const half_t* Kb = K + b_idx * lay.k_b + hk_idx * lay.k_h;
-  const half_t* Vb = V + b_idx * lay.v_b + hk_idx * lay.v_h;
+  const half_t* Kb = K + (PAGED ? 0 : b_idx * lay.k_b) + hk_idx * lay.k_h;
+  const half_t* Vb = V + (PAGED ? 0 : b_idx * lay.v_b) + hk_idx * lay.v_h;
   half_t* Ob = O + b_idx * lay.o_b + h_idx * lay.o_h;
 
   for (int pass = 0; pass < (CAUSAL ? 2 : 1); pass++) {
@@ -306,14 +319,40 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const unsigned k_rb = lay.k_r * 2, v_rb = lay.v_r * 2;  // row strides in bytes
   const unsigned k_voff = (wave * 4 + lrow) * k_rb + k_chunk * 16;
   const unsigned v_voff = (wave * 4 + lrow) * v_rb + v_chunk * 16;
-  auto issue_kv = [&](const half_t* base, unsigned rb, unsigned voff, int tile, int lds_off) {
+  // page ids come through the scalar cache (constant address space: the table is not written while the kernel
+  // runs), one tile ahead of their use, so that no K/V load waits for a table read
+  typedef const int __attribute__((address_space(4)))* table_ptr_t;
+  const table_ptr_t table_row =
+      PAGED ? (table_ptr_t)(unsigned long long)(pg.block_table + (size_t)b_idx * pg.max_pages) : (table_ptr_t)0;
+  auto load_ids = [&](int tile, int* ids) {
+    if constexpr (PAGED) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) ids[i] = (tile * 4 + i < pg.max_pages) ? table_row[tile * 4 + i] : -1;
+    }
+  };
+  auto issue_kv = [&](const half_t* base, unsigned rb, unsigned voff, int tile, int lds_off, const int* ids) {
     char* dst = lds + lds_off + wave * 1024;
     const int row0 = tile * FA_BLOCK_N;
     int rem = Sk - row0;
     rem = rem > FA_BLOCK_N ? FA_BLOCK_N : rem;
-    const buffer_rsrc_t rs = make_buffer(reinterpret_cast<const char*>(base) + (size_t)row0 * rb, (unsigned)(rem - 1) * rb + 256u);
+    if constexpr (PAGED) {
+      // wave-load i covers rows 16 i .. 16 i + 15 of the tile = page 4 tile + i of the sequence: one descriptor
+      // per page, sized to the page's valid rows (none for a page beyond the sequence or an id outside the cache)
 #pragma unroll
-    for (int i = 0; i < 4; i++) buffer_load_lds_16B(rs, voff + (unsigned)i * 16u * rb, 0, dst + i * 4096);
+      for (int i = 0; i < 4; i++) {
+        const int id = ids[i];
+        int rows = rem - 16 * i;
+        rows = rows > 16 ? 16 : rows;
+        const bool ok = rows > 0 && id >= 0 && id < pg.num_pages;
+        const buffer_rsrc_t rs = make_buffer(reinterpret_cast<const char*>(base) + (size_t)(ok ? id : 0) * 16u * rb,
+                                             ok ? (unsigned)(rows - 1) * rb + 256u : 0u);
+        buffer_load_lds_16B(rs, voff, 0, dst + i * 4096);
+      }
+    } else {
+      const buffer_rsrc_t rs = make_buffer(reinterpret_cast<const char*>(base) + (size_t)row0 * rb, (unsigned)(rem - 1) * rb + 256u);
+#pragma unroll
+      for (int i = 0; i < 4; i++) buffer_load_lds_16B(rs, voff + (unsigned)i * 16u * rb, 0, dst + i * 4096);
+    }
   };
 
   const int k_base = r32 * 256 + ((h ^ (lane & 15)) * 16);
@@ -454,10 +493,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   };
 
   floatx16 sa[2], sb[2];
+  int k_ids[4] = {-1, -1, -1, -1}, v_ids[4] = {-1, -1, -1, -1};  // page ids of the next K tile and the next V tile to fetch
   if (n_tiles > 0) {
-    issue_kv(Kb, k_rb, k_voff, 0, 0);
-    issue_kv(Vb, v_rb, v_voff, 0, VBUF);
-    if (n_tiles > 1) issue_kv(Kb, k_rb, k_voff, 1, TILE_B);
+    load_ids(0, k_ids);
+    issue_kv(Kb, k_rb, k_voff, 0, 0, k_ids);
+    issue_kv(Vb, v_rb, v_voff, 0, VBUF, k_ids);
+    load_ids(1, v_ids);
+    if (n_tiles > 1) issue_kv(Kb, k_rb, k_voff, 1, TILE_B, v_ids);
+    load_ids(2, k_ids);  // what trip 0 issues: K(2) and V(1)
     wait_vmcnt0();
     __syncthreads();
     if (wave_active(0)) scores(0, sa);
@@ -470,8 +513,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   auto trip = [&](auto par_tag, int j, floatx16* s_cur, floatx16* s_next) {
     constexpr int PAR = decltype(par_tag)::value;
     constexpr int K_CUR = PAR * TILE_B, K_NEXT = (1 - PAR) * TILE_B, V_CUR = PAR * TILE_B, V_NEXT = VBUF + (1 - PAR) * TILE_B;
-    if (j + 2 < n_tiles) issue_kv(Kb, k_rb, k_voff, j + 2, K_CUR);
-    if (j + 1 < n_tiles) issue_kv(Vb, v_rb, v_voff, j + 1, V_NEXT);
+    if (j + 2 < n_tiles) issue_kv(Kb, k_rb, k_voff, j + 2, K_CUR, k_ids);
+    if (j + 1 < n_tiles) issue_kv(Vb, v_rb, v_voff, j + 1, V_NEXT, v_ids);
+    if constexpr (PAGED) {
+      // the next trip fetches V(j+2) -- the tile whose ids K just used -- and K(j+3)
+#pragma unroll
+      for (int i = 0; i < 4; i++) v_ids[i] = k_ids[i];
+      load_ids(j + 3, k_ids);
+    }
     if (wave_active(j)) softmax_pv(std::true_type{}, j, V_CUR, s_cur, K_NEXT, s_next);  // idle from here on otherwise
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
@@ -525,8 +574,8 @@ static int fa_launch(const void* q, const void* k, const void* v, void* o, int64
   static bool attr_set = false;
   if (!attr_set) {
     const void* kernels[4] = {reinterpret_cast<const void*>(fa_fwd_d128<true>), reinterpret_cast<const void*>(fa_fwd_d128<false>),
-                              reinterpret_cast<const void*>(fa_fwd_d128_pipe<true>),
-                              reinterpret_cast<const void*>(fa_fwd_d128_pipe<false>)};
+                              reinterpret_cast<const void*>(fa_fwd_d128_pipe<true, false>),
+                              reinterpret_cast<const void*>(fa_fwd_d128_pipe<false, false>)};
     for (const void* kp : kernels) {
       hipError_t e = hipFuncSetAttribute(kp, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
       if (e != hipSuccess) {
@@ -541,10 +590,15 @@ static int fa_launch(const void* q, const void* k, const void* v, void* o, int64
   const int units = (variant != 1 && is_causal) ? (q_blocks + 1) / 2 : q_blocks;
   dim3 grid(BH * units), block(256);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  auto kern = variant == 1 ? (is_causal ? fa_fwd_d128<true> : fa_fwd_d128<false>)
-                           : (is_causal ? fa_fwd_d128_pipe<true> : fa_fwd_d128_pipe<false>);
-  hipLaunchKernelGGL(kern, grid, block, lds_bytes, s, (const half_t*)q, (const half_t*)k, (const half_t*)v, (half_t*)o, BH,
-                     (int)Sq, (int)Sk, scale_log2e, q_blocks, lay);
+  if (variant == 1) {
+    auto kern = is_causal ? fa_fwd_d128<true> : fa_fwd_d128<false>;
+    hipLaunchKernelGGL(kern, grid, block, lds_bytes, s, (const half_t*)q, (const half_t*)k, (const half_t*)v, (half_t*)o, BH,
+                       (int)Sq, (int)Sk, scale_log2e, q_blocks, lay);
+  } else {
+    auto kern = is_causal ? fa_fwd_d128_pipe<true, false> : fa_fwd_d128_pipe<false, false>;
+    hipLaunchKernelGGL(kern, grid, block, lds_bytes, s, (const half_t*)q, (const half_t*)k, (const half_t*)v, (half_t*)o, BH,
+                       (int)Sq, (int)Sk, scale_log2e, q_blocks, lay, FaPaged{nullptr, nullptr, 0, 0});
+  }
   return check_launch(variant == 1 ? "fa_fwd_d128" : "fa_fwd_d128_pipe", grid, block, lds_bytes);
 }
 
@@ -579,4 +633,48 @@ extern "C" int mi355_flash_attn_fwd_strided(const void* q, const void* k, const 
   lay.o_b = o_strides[0], lay.o_h = o_strides[1], lay.o_r = (unsigned)o_strides[2];
   lay.H = (int)H, lay.group = Hkv > 0 ? (int)(H / Hkv) : 1;
   return fa_launch(q, k, v, o, B, H, Hkv, Sq, Sk, D, lay, scale, is_causal, variant, stream, who);
+}
+
+extern "C" int mi355_paged_prefill_attn(const void* q, const void* k_cache, const void* v_cache, const void* block_table,
+                                        const void* seq_lens, void* out, int64_t num_seqs, int64_t num_new, int64_t num_q_heads,
+                                        int64_t num_kv_heads, int64_t D, int64_t page_size, int64_t max_pages_per_seq,
+                                        int64_t num_pages, float scale, void* stream) {
+  const char* who = "paged_prefill_attn";
+  if (!q || !k_cache || !v_cache || !block_table || !seq_lens || !out) return fail(-MI355_E_NULL, "%s: null pointer", who);
+  if (D != 128) return fail(-MI355_E_SHAPE, "%s: head dim %lld not supported (only 128)", who, (long long)D);
+  if (page_size != 16) return fail(-MI355_E_SHAPE, "%s: page size %lld not supported (only 16)", who, (long long)page_size);
+  if (num_seqs <= 0 || num_new <= 0 || num_q_heads <= 0 || num_kv_heads <= 0 || max_pages_per_seq <= 0 || num_pages <= 0 ||
+      num_seqs * num_q_heads > (1 << 24) || num_new > (1 << 20) || max_pages_per_seq > (1 << 20) || num_pages > (1 << 24))
+    return fail(-MI355_E_SHAPE, "%s: bad shape seqs=%lld new=%lld q_heads=%lld kv_heads=%lld max_pages=%lld pages=%lld", who,
+                (long long)num_seqs, (long long)num_new, (long long)num_q_heads, (long long)num_kv_heads,
+                (long long)max_pages_per_seq, (long long)num_pages);
+  if (num_q_heads % num_kv_heads != 0)
+    return fail(-MI355_E_SHAPE, "%s: %lld query heads over %lld key/value heads", who, (long long)num_q_heads, (long long)num_kv_heads);
+  if (num_kv_heads * 128 >= (1 << 24)) return fail(-MI355_E_SHAPE, "%s: too many key/value heads", who);
+  if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(out))
+    return fail(-MI355_E_ALIGN, "%s: q, k_cache, v_cache, out must be 16-byte aligned", who);
+  if (!(scale > 0.f) || !isfinite(scale)) return fail(-MI355_E_SHAPE, "%s: scale must be positive and finite", who);
+  FaLayout lay;
+  lay.q_b = num_new * num_q_heads * 128, lay.q_h = 128, lay.q_r = (unsigned)(num_q_heads * 128);
+  lay.o_b = lay.q_b, lay.o_h = 128, lay.o_r = lay.q_r;
+  lay.k_b = lay.v_b = 0, lay.k_h = lay.v_h = 128, lay.k_r = lay.v_r = (unsigned)(num_kv_heads * 128);
+  lay.H = (int)num_q_heads, lay.group = (int)(num_q_heads / num_kv_heads);
+  const int BH = (int)(num_seqs * num_q_heads);
+  const int q_blocks = (int)((num_new + FA_BLOCK_M - 1) / FA_BLOCK_M);
+  const int lds_bytes = 2 * FA_STAGE;
+  auto kern = fa_fwd_d128_pipe<true, true>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e != hipSuccess) {
+      set_error("hipFuncSetAttribute(fa_fwd_d128_pipe paged): %s", hipGetErrorString(e));
+      return (int)e;
+    }
+    attr_set = true;
+  }
+  dim3 grid(BH * ((q_blocks + 1) / 2)), block(256);
+  const FaPaged pg{static_cast<const int*>(block_table), static_cast<const int*>(seq_lens), (int)max_pages_per_seq, (int)num_pages};
+  hipLaunchKernelGGL(kern, grid, block, lds_bytes, reinterpret_cast<hipStream_t>(stream), (const half_t*)q, (const half_t*)k_cache,
+                     (const half_t*)v_cache, (half_t*)out, BH, (int)num_new, 0, scale * 1.4426950408889634f, q_blocks, lay, pg);
+  return check_launch("fa_fwd_d128_pipe<paged>", grid, block, lds_bytes);
 }

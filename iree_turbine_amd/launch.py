@@ -175,6 +175,27 @@ def kv_cache_append(k_new, v_new, k_cache, v_cache, block_table, start_pos) -> N
     _lib.check(rc, f"kv_cache_append seqs={S} n_new={n_new} hkv={Hkv} pages={P}")
 
 
+def paged_prefill_attn_out(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_table: Tensor, seq_lens: Tensor, out: Tensor,
+                           scale: float) -> Tensor:
+    """q, out [S, n_new, Hq, 128]; caches [P, 16, Hkv, 128]; seq_lens counts the new tokens (see mi355_paged_prefill_attn)."""
+    dev = _dev(q, k_cache, v_cache, block_table, seq_lens, out)
+    q, k_cache, v_cache = q.contiguous(), k_cache.contiguous(), v_cache.contiguous()
+    block_table, seq_lens = block_table.contiguous(), seq_lens.contiguous()
+    _contig_out(out, "paged_prefill_attn")
+    S, n_new, Hq, D = q.shape
+    P, page, Hkv = k_cache.shape[0], k_cache.shape[1], k_cache.shape[2]
+    if out.shape != q.shape or out.dtype != torch.float16:
+        raise ValueError("paged_prefill_attn: out must be float16 with q's shape")
+    if scale is None or scale <= 0:
+        scale = 1.0 / math.sqrt(D)
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_paged_prefill_attn(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
+                                                  seq_lens.data_ptr(), out.data_ptr(), S, n_new, Hq, Hkv, D, page,
+                                                  block_table.shape[1], P, scale, _lib.current_stream_ptr(dev))
+    _lib.check(rc, f"paged_prefill_attn seqs={S} n_new={n_new} hq={Hq} hkv={Hkv} pages={P}")
+    return out
+
+
 def mxfp4_gemm_out(a, a_scale, b, b_scale, c: Tensor, variant: int = -1) -> Tensor:
     dev = _dev(a, a_scale, b, b_scale, c)
     a, a_scale, b, b_scale = a.contiguous(), a_scale.contiguous(), b.contiguous(), b_scale.contiguous()

@@ -209,6 +209,36 @@ class kv_cache_append(CustomOp):
 
 
 @CustomOp.register
+class paged_prefill_attn(CustomOp):
+    """Causal attention of the n_new latest tokens of every sequence over its paged KV cache (chunked / prefix
+    prefill): q [S, n_new, Hq, 128], caches [P, 16, Hkv, 128], block_table int32 [S, max_pages], seq_lens int32 [S]
+    counting the new tokens, whose K/V are in the cache already (kv_cache_append).  Query t sees positions
+    j <= seq_lens[s] - n_new + t: the mask of tests/dynamo/llama_test.py:285-290 shifted by the cached prefix."""
+
+    signature = "paged_prefill_attn(Tensor q, Tensor k_cache, Tensor v_cache, Tensor block_table, Tensor seq_lens, float scale) -> Tensor"
+
+    def select(self, sel: KernelSelection):
+        q, kc, vc, bt, sl = (sel.arg_tensor(i) for i in range(5))
+        sel.attr_float(5)
+        fn = "paged_prefill_attn"
+        _require(q.t.dim() == 4, f"{fn}: q must be [num_seqs, n_new, num_q_heads, D]")
+        _require(kc.t.dim() == 4 and kc.t.shape == vc.t.shape, f"{fn}: k_cache / v_cache must both be [num_pages, page_size, num_kv_heads, D]")
+        _require(all(t.t.dtype == torch.float16 for t in (q, kc, vc)), f"{fn}: q, k_cache, v_cache must be float16")
+        _require(q.t.size(3) == 128 and kc.t.size(3) == 128, f"{fn}: head dim must be 128")
+        _require(kc.t.size(1) == 16, f"{fn}: page size {kc.t.size(1)} not supported (only 16)")
+        _require(kc.t.size(2) > 0 and q.t.size(2) % kc.t.size(2) == 0, f"{fn}: {q.t.size(2)} q heads over {kc.t.size(2)} kv heads")
+        _require(bt.t.dim() == 2 and bt.t.dtype == torch.int32 and bt.t.size(0) == q.t.size(0), f"{fn}: block_table must be int32 [num_seqs, max_pages]")
+        _require(sl.t.dim() == 1 and sl.t.dtype == torch.int32 and sl.t.size(0) == q.t.size(0), f"{fn}: seq_lens must be int32 [num_seqs]")
+        _require(q.t.size(0) > 0 and q.t.size(1) > 0 and bt.t.size(1) > 0, f"{fn}: empty batch")
+        q.specialize_dims(2, 3)
+        sel.return_new_tensor(list(q.t.shape), torch.float16)
+
+    def eager_execute(self, q, k_cache, v_cache, block_table, seq_lens, scale):
+        out = torch.empty(q.shape, dtype=torch.float16, device=q.device)
+        return launch.paged_prefill_attn_out(q, k_cache, v_cache, block_table, seq_lens, out, scale)
+
+
+@CustomOp.register
 class paged_decode_phase0(CustomOp):
     """Phase 0 of the split-K decode: per (seq, q head, split) an unnormalised fp32 partial
     output [S, Hq, splits, 128] and its (max in log2 units, sum) [S, Hq, splits, 2]."""

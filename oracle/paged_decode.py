@@ -66,3 +66,33 @@ def kv_cache_append_ref(k_new, v_new, k_cache, v_cache, block_table, start_pos):
             kc[pg, pos % page] = k_new[s, t].cpu()
             vc[pg, pos % page] = v_new[s, t].cpu()
     return kc, vc
+
+
+def paged_prefill_ref(q, k_cache, v_cache, block_table, seq_lens, scale: float | None = None) -> torch.Tensor:
+    """out[s, t, h] = softmax over the cached positions j <= seq_lens[s] - n_new + t of q[s, t, h] . K_s[j] * scale,
+    times V_s: the attention of tests/dynamo/llama_test.py:160-181 with the mask of :285-290 (query t of the
+    new chunk sees the cached prefix and the chunk up to itself), K/V gathered through the block table.
+    q [S, n_new, Hq, D]; a query with no visible position gives zeros."""
+    qf = q.detach().cpu().float()
+    kc, vc = k_cache.detach().cpu().float(), v_cache.detach().cpu().float()
+    bt, sl = block_table.detach().cpu(), seq_lens.detach().cpu()
+    S, T, Hq, D = qf.shape
+    n_rep = Hq // kc.shape[2]
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    out = torch.zeros((S, T, Hq, D), dtype=torch.float32)
+    for s in range(S):
+        ln = max(0, min(int(sl[s]), bt.shape[1] * kc.shape[1]))
+        if ln == 0:
+            continue
+        ks = repeat_kv(gather_kv(kc, bt[s], ln), n_rep)  # [ln, Hq, D]
+        vs = repeat_kv(gather_kv(vc, bt[s], ln), n_rep)
+        scores = torch.einsum("thd,lhd->thl", qf[s], ks) * scale
+        pos = torch.arange(ln)[None, :]
+        last = (ln - T + torch.arange(T))[:, None]  # last visible position of query t
+        visible = pos <= last  # [T, ln]
+        scores = scores.masked_fill(~visible[:, None, :], float("-inf"))
+        p = torch.softmax(scores, dim=-1)
+        p = torch.where(visible.any(dim=1)[:, None, None], p, torch.zeros_like(p))  # rows with nothing visible
+        out[s] = torch.einsum("thl,lhd->thd", p, vs)
+    return out

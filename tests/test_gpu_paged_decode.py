@@ -206,3 +206,69 @@ def test_kv_cache_append_skips_positions_without_a_page(dev):
         torch.ops.mi355.kv_cache_append(kn.to(dev), kn.to(dev), kd, vd, bt2.to(dev), start.long().to(dev))
     with pytest.raises(ValueError):
         torch.ops.mi355.paged_decode_attn_window(*_to(dev, q, kc, vc, bt, sl), 0.0, 1, -1)
+
+
+@pytest.mark.parametrize("n_new", [1, 16, 100, 200])
+@pytest.mark.parametrize("hq,hkv", [(8, 2), (4, 4)])
+def test_paged_prefill_vs_oracle(dev, n_new, hq, hkv):
+    """Chunked prefill over the paged cache: chunks shorter and longer than a query block, prefixes that end
+    inside a page, sequences shorter than the chunk (their first queries see nothing: zeros)."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs, paged_decode as op
+
+    announce(f"paged prefill n_new={n_new} hq={hq} hkv={hkv}")
+    _, kc, vc, bt, sl = inputs.paged_decode_inputs(num_seqs=5, num_q_heads=hq, num_kv_heads=hkv, min_len=40, max_len=600, seed=6)
+    g = torch.Generator().manual_seed(n_new)
+    q = torch.randn(5, n_new, hq, 128, generator=g).half()
+    out = torch.ops.mi355.paged_prefill_attn(*_to(dev, q, kc, vc, bt, sl), 0.0)
+    torch.cuda.synchronize()
+    ref = op.paged_prefill_ref(q, kc, vc, bt, sl)
+    torch.testing.assert_close(out.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+
+
+def test_paged_prefill_matches_decode_and_dense_attention(dev):
+    """One new token is the decode kernel's problem; a chunk covering the whole sequence on an in-order block
+    table is plain causal attention over the same rows."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs
+
+    announce("paged prefill vs decode kernel and dense kernel")
+    q1, kc, vc, bt, sl = inputs.paged_decode_inputs(num_seqs=6, num_q_heads=16, num_kv_heads=4, min_len=1, max_len=900, seed=8)
+    dq, dkc, dvc, dbt, dsl = _to(dev, q1, kc, vc, bt, sl)
+    a = torch.ops.mi355.paged_prefill_attn(dq[:, None].contiguous(), dkc, dvc, dbt, dsl, 0.0)[:, 0]
+    b = torch.ops.mi355.paged_decode_attn(dq, dkc, dvc, dbt, dsl, 0.0, 1)
+    torch.testing.assert_close(a.float(), b.float(), rtol=RTOL, atol=ATOL)
+    # dense: sequence of 320 tokens in pages 0..19, queries for all of them
+    S, L, Hq, Hkv = 2, 320, 8, 2
+    g = torch.Generator().manual_seed(3)
+    k = torch.randn(S, L, Hkv, 128, generator=g).half().to(dev)
+    v = torch.randn(S, L, Hkv, 128, generator=g).half().to(dev)
+    q = torch.randn(S, L, Hq, 128, generator=g).half().to(dev)
+    kcache, vcache = k.reshape(S * L // 16, 16, Hkv, 128), v.reshape(S * L // 16, 16, Hkv, 128)
+    table = torch.arange(S * L // 16, dtype=torch.int32, device=dev).reshape(S, L // 16)
+    lens = torch.full((S,), L, dtype=torch.int32, device=dev)
+    paged = torch.ops.mi355.paged_prefill_attn(q, kcache, vcache, table, lens, 0.0)
+    dense = torch.ops.mi355.flash_attn_fwd(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), True, 0.0).transpose(1, 2)
+    assert torch.equal(paged, dense.contiguous())  # same kernel, same tiles, pages in order: bit-identical
+
+
+def test_paged_prefill_guards(dev):
+    """Page ids outside the cache and table entries beyond the sequence are never dereferenced: poisoned
+    entries change nothing; contract violations raise."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs
+
+    announce("paged prefill guards")
+    _, kc, vc, bt, sl = inputs.paged_decode_inputs(num_seqs=4, num_q_heads=8, num_kv_heads=2, min_len=20, max_len=300, seed=12)
+    q = torch.randn(4, 24, 8, 128, generator=torch.Generator().manual_seed(1)).half()
+    dq, dkc, dvc, dbt, dsl = _to(dev, q, kc, vc, bt, sl)
+    want = torch.ops.mi355.paged_prefill_attn(dq, dkc, dvc, dbt, dsl, 0.0)
+    poisoned = dbt.clone()
+    for s in range(4):
+        used = (int(sl[s]) + 15) // 16
+        poisoned[s, used:] = 2 ** 30
+    assert torch.equal(torch.ops.mi355.paged_prefill_attn(dq, dkc, dvc, poisoned, dsl, 0.0), want)
+    with pytest.raises(ValueError):
+        torch.ops.mi355.paged_prefill_attn(dq[..., :64].contiguous(), dkc, dvc, dbt, dsl, 0.0)
+    with pytest.raises(ValueError):
+        torch.ops.mi355.paged_prefill_attn(dq, dkc, dvc, dbt.long(), dsl, 0.0)

@@ -176,3 +176,33 @@ def test_window_and_append_oracles():
     far = torch.full((S,), 16 * bt.shape[1], dtype=torch.int32)
     k3, v3 = op.kv_cache_append_ref(kn, vn, kc, vc, bt, far)
     assert torch.equal(k3, kc) and torch.equal(v3, vc)
+
+
+def test_paged_prefill_oracle_reduces_to_known_cases():
+    """One new token = the decode oracle; a chunk that is the whole sequence = causal SDPA over the gathered
+    dense tensors; a chunk after a prefix = the last rows of causal SDPA over the whole sequence; a chunk longer
+    than the sequence leaves its first queries (nothing visible) at zero."""
+    from oracle import attention as oa, inputs, paged_decode as op
+
+    q1, kc, vc, bt, sl = inputs.paged_decode_inputs(num_seqs=4, num_q_heads=8, num_kv_heads=2, min_len=5, max_len=70, seed=9)
+    torch.testing.assert_close(op.paged_prefill_ref(q1[:, None], kc, vc, bt, sl)[:, 0], op.paged_decode_ref(q1, kc, vc, bt, sl),
+                               rtol=1e-5, atol=1e-6)
+    g = torch.Generator().manual_seed(2)
+    T = 12
+    q = torch.randn(4, T, 8, 128, generator=g).half()
+    out = op.paged_prefill_ref(q, kc, vc, bt, sl)
+    for s in range(4):
+        ln = int(sl[s])
+        k = op.repeat_kv(op.gather_kv(kc, bt[s], ln), 4).transpose(0, 1)[None]  # [1, Hq, ln, D]
+        v = op.repeat_kv(op.gather_kv(vc, bt[s], ln), 4).transpose(0, 1)[None]
+        if ln >= T:
+            # queries for all ln positions, of which the chunk is the last T: plain square causal attention
+            q_all = torch.zeros(1, 8, ln, 128, dtype=torch.float16)
+            q_all[0, :, ln - T:] = q[s].transpose(0, 1)
+            ref = oa.sdpa_ref(q_all, k, v, is_causal=True)[0, :, ln - T:].transpose(0, 1)
+            torch.testing.assert_close(out[s], ref, rtol=1e-5, atol=1e-6)
+        else:
+            assert torch.equal(out[s, :T - ln], torch.zeros(T - ln, 8, 128))
+            ref = oa.sdpa_ref(q[s, T - ln:].transpose(0, 1)[None], k, v, is_causal=True)[0].transpose(0, 1)
+            torch.testing.assert_close(out[s, T - ln:], ref, rtol=1e-5, atol=1e-6)
+    assert (sl < T).any() and (sl >= T).any()
