@@ -206,6 +206,19 @@ int mi355_mxfp4_gemm(const void* a, const void* a_scale, const void* b, const vo
                      int out_dtype, int variant, void* stream);
 
 /*
+ * Block-scaled MXFP8 GEMM: C[M,N] = dq(A) . dq(B)^T, fp32 accumulation, bf16 or fp32 out.
+ * a: uint8 [M, K], b: uint8 [N, K] -- OCP FP8 E4M3 codes (sign, 4 exponent bits of bias 7,
+ *    3 mantissa bits, no infinities, NaN = S.1111.111), one per element;
+ * a_scale: uint8 [M, K/32], b_scale: uint8 [N, K/32] -- E8M0, one per 32 consecutive K elements.
+ * dq(x)[r,k] = E4M3(code[r,k]) * 2^(scale[r,k/32] - 127).  K % 32 == 0.
+ * The wider element format at the boundary of mi355_mxfp4_gemm: same scales, same layout, one byte per
+ * element.  Format names: iree/turbine/kernel/_support/dtype.py:115,117 (f8e4m3fn, f8e8m0fnu).
+ */
+int mi355_mxfp8_gemm(const void* a, const void* a_scale, const void* b, const void* b_scale,
+                     void* c, int64_t M, int64_t N, int64_t K,
+                     int out_dtype, int variant, void* stream);
+
+/*
  * MXFP4 dequantisation on the device (used to show that the device decodes
  * the format bit-exactly): out[r,k] = E2M1(code) * 2^(scale-127) as fp32.
  * codes: uint8 [rows, K/2]; scales: uint8 [rows, K/32]; out: fp32 [rows, K].

@@ -37,6 +37,8 @@ int decode_variant_count();
 const char* decode_variant_name(int i);
 int mxfp4_variant_count();
 const char* mxfp4_variant_name(int i);
+int mxfp8_variant_count();
+const char* mxfp8_variant_name(int i);
 
 }  // namespace mi355
 
@@ -51,6 +53,7 @@ extern "C" int mi355_variant_count(const char* family) {
   if (!strcmp(family, "flash_attn_fwd")) return fa_variant_count();
   if (!strcmp(family, "paged_decode")) return decode_variant_count();
   if (!strcmp(family, "mxfp4_gemm")) return mxfp4_variant_count();
+  if (!strcmp(family, "mxfp8_gemm")) return mxfp8_variant_count();
   return 0;
 }
 
@@ -60,5 +63,6 @@ extern "C" const char* mi355_variant_name(const char* family, int i) {
   if (!strcmp(family, "flash_attn_fwd")) return fa_variant_name(i);
   if (!strcmp(family, "paged_decode")) return decode_variant_name(i);
   if (!strcmp(family, "mxfp4_gemm")) return mxfp4_variant_name(i);
+  if (!strcmp(family, "mxfp8_gemm")) return mxfp8_variant_name(i);
   return nullptr;
 }

@@ -210,6 +210,20 @@ def mxfp4_gemm_out(a, a_scale, b, b_scale, c: Tensor, variant: int = -1) -> Tens
     return c
 
 
+def mxfp8_gemm_out(a, a_scale, b, b_scale, c: Tensor, variant: int = -1) -> Tensor:
+    dev = _dev(a, a_scale, b, b_scale, c)
+    a, a_scale, b, b_scale = a.contiguous(), a_scale.contiguous(), b.contiguous(), b_scale.contiguous()
+    _contig_out(c, "mxfp8_gemm")
+    M, N, K = a.shape[0], b.shape[0], a.shape[1]
+    if tuple(c.shape) != (M, N):
+        raise ValueError(f"mxfp8_gemm: c is {tuple(c.shape)}, expected {(M, N)}")
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_mxfp8_gemm(a.data_ptr(), a_scale.data_ptr(), b.data_ptr(), b_scale.data_ptr(), c.data_ptr(), M, N,
+                                          K, _lib.dtype_code(c.dtype), variant, _lib.current_stream_ptr(dev))
+    _lib.check(rc, f"mxfp8_gemm M={M} N={N} K={K} out={c.dtype} variant={variant}")
+    return c
+
+
 def mxfp4_dequant_out(codes: Tensor, scales: Tensor, out: Tensor) -> Tensor:
     dev = _dev(codes, scales, out)
     codes, scales = codes.contiguous(), scales.contiguous()

@@ -281,10 +281,11 @@ class paged_decode_phase1(CustomOp):
         return launch.paged_decode_phase1_out(part_acc, part_ml, out)
 
 
-def _check_mx_operand(op: str, name: str, codes: Tensor, scales: Tensor):
-    _require(codes.dim() == 2 and codes.dtype == torch.uint8, f"{op}: {name} must be uint8 [rows, K/2] (two E2M1 codes per byte)")
+def _check_mx_operand(op: str, name: str, codes: Tensor, scales: Tensor, per_byte: int = 2):
+    what = "[rows, K/2] (two E2M1 codes per byte)" if per_byte == 2 else "[rows, K] (one E4M3 code per byte)"
+    _require(codes.dim() == 2 and codes.dtype == torch.uint8, f"{op}: {name} must be uint8 {what}")
     _require(scales.dim() == 2 and scales.dtype == torch.uint8, f"{op}: {name}_scale must be uint8 [rows, K/32] (E8M0)")
-    K = codes.size(1) * 2
+    K = codes.size(1) * per_byte
     _require(K > 0 and K % 32 == 0, f"{op}: K={K} must be a positive multiple of 32")
     _require(scales.size(0) == codes.size(0) and scales.size(1) == K // 32, f"{op}: {name}_scale shape {tuple(scales.shape)} does not match {name} {tuple(codes.shape)}")
 
@@ -312,6 +313,31 @@ class mxfp4_gemm(CustomOp):
     def eager_execute(self, a, a_scale, b, b_scale, out_dtype, variant):
         c = torch.empty((a.shape[0], b.shape[0]), dtype=_OUT_DTYPES[out_dtype], device=a.device)
         return launch.mxfp4_gemm_out(a, a_scale, b, b_scale, c, variant)
+
+
+@CustomOp.register
+class mxfp8_gemm(CustomOp):
+    """C[M,N] = dq(A) . dq(B)^T for OCP MXFP8 operands: E4M3 codes uint8 [rows, K] (torch.float8_e4m3fn viewed as
+    uint8), E8M0 scales uint8 [rows, K/32]; out_dtype "bfloat16" | "float32"."""
+
+    signature = "mxfp8_gemm(Tensor a, Tensor a_scale, Tensor b, Tensor b_scale, str out_dtype, int variant) -> Tensor"
+
+    def select(self, sel: KernelSelection):
+        a, asc, b, bsc = (sel.arg_tensor(i) for i in range(4))
+        od = sel.attr_str(4).v
+        sel.attr_int(5)
+        _check_mx_operand("mxfp8_gemm", "a", a.t, asc.t, per_byte=1)
+        _check_mx_operand("mxfp8_gemm", "b", b.t, bsc.t, per_byte=1)
+        _require(a.t.size(1) == b.t.size(1), "mxfp8_gemm: a and b disagree on K")
+        _require(od in ("bfloat16", "float32"), f"mxfp8_gemm: out_dtype must be 'bfloat16' or 'float32', got {od!r}")
+        _require(a.t.size(0) > 0 and b.t.size(0) > 0, "mxfp8_gemm: empty operand")
+        for d in (a, asc, b, bsc):
+            d.specialize_all_dims()
+        sel.return_new_tensor([a.t.size(0), b.t.size(0)], _OUT_DTYPES[od]).specialize_all_dims()
+
+    def eager_execute(self, a, a_scale, b, b_scale, out_dtype, variant):
+        c = torch.empty((a.shape[0], b.shape[0]), dtype=_OUT_DTYPES[out_dtype], device=a.device)
+        return launch.mxfp8_gemm_out(a, a_scale, b, b_scale, c, variant)
 
 
 @CustomOp.register

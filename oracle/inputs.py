@@ -64,3 +64,19 @@ def mxfp4_inputs(M: int, N: int, K: int, seed: int = DEFAULT_SEED, exp_range: in
     b = torch.randint(0, 256, (N, K // 2), generator=g).to(torch.uint8)
     b_scale = (127 + torch.randint(-exp_range, exp_range + 1, (N, K // 32), generator=g)).to(torch.uint8)
     return a, a_scale, b, b_scale
+
+
+def mxfp8_inputs(M: int, N: int, K: int, seed: int = DEFAULT_SEED, exp_range: int = 8):
+    """E4M3 codes uniform over the 254 finite values (the two NaN patterns 0x7F / 0xFF are redrawn as their
+    neighbours 0x7E / 0xFE), E8M0 scale bytes 127 + U[-exp_range, exp_range]."""
+    g = _gen(seed)
+
+    def codes(rows):
+        c = torch.randint(0, 256, (rows, K), generator=g).to(torch.uint8)
+        return torch.where((c & 0x7F) == 0x7F, c - 1, c)
+
+    a = codes(M)
+    a_scale = (127 + torch.randint(-exp_range, exp_range + 1, (M, K // 32), generator=g)).to(torch.uint8)
+    b = codes(N)
+    b_scale = (127 + torch.randint(-exp_range, exp_range + 1, (N, K // 32), generator=g)).to(torch.uint8)
+    return a, a_scale, b, b_scale

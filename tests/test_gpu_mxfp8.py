@@ -1,0 +1,133 @@
+"""GPU parity: block-scaled MXFP8 GEMM through the C ABI vs the CPU oracle (table dequantise + fp32 matmul).
+Contract as for MXFP4: the decode is exact (every product of two fp8 values and two power-of-two scales is exact
+in fp32), the GEMM within 1e-2 relative of the fp32 matmul on the dequantised operands."""
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import announce
+
+pytestmark = pytest.mark.gpu
+
+REL = 1e-2
+# The matrix unit adds the products of one 16-element lane group in fixed point, aligned to the largest of them
+# with 13 bits below it (measured: 2^16 + 2^3 is kept, 2^16 + 2^2 is not); sums across groups and with the
+# accumulator are full fp32.  With E4M3's 2^17 range of magnitudes that shows as ~1e-4 of the largest output;
+# a single product per group is exact.
+HW_SUM = 5e-4
+
+
+def _rel_err(got, ref):
+    return ((got.double() - ref.double()).abs().max() / ref.double().abs().max()).item()
+
+
+def test_mxfp8_decode_exhaustive(dev):
+    """Every finite E4M3 code against the scale bytes 20..234, through the GEMM with a one-hot partner: the
+    single product of each output cell is exact, so the result must equal the table bit for bit."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import mxfp8 as o8
+
+    announce("mxfp8 decode exhaustive")
+    K = 32
+    codes = torch.arange(256, dtype=torch.uint8)
+    finite = codes[(codes & 0x7F) != 0x7F]
+    a = torch.zeros(len(finite), K, dtype=torch.uint8)
+    a[:, 0] = finite
+    b = torch.zeros(32, K, dtype=torch.uint8)
+    b[:, 0] = 0x38  # 1.0
+    bsc = torch.full((32, 1), 127, dtype=torch.uint8)
+    # scale bytes 20..234: every product stays a normal fp32 number (the matrix unit's treatment of fp32
+    # denormals is not part of the contract)
+    for sc in range(20, 235):
+        asc = torch.full((len(finite), 1), sc, dtype=torch.uint8)
+        c = torch.ops.mi355.mxfp8_gemm(a.to(dev), asc.to(dev), b.to(dev), bsc.to(dev), "float32", -1).cpu()
+        want = o8.mxfp8_dequant_ref(a, asc)[:, 0]
+        assert np.array_equal(c[:, 0].numpy().view(np.uint32) & 0x7FFFFFFF, want.view(np.uint32) & 0x7FFFFFFF), sc
+        nz = want != 0
+        assert np.array_equal(np.signbit(c[:, 0].numpy())[nz], np.signbit(want)[nz]), sc
+
+
+@pytest.mark.parametrize("variant", [-1, 0, 1])
+def test_mxfp8_gemm_variants(dev, variant):
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs, mxfp8 as o8
+
+    M, N, K = 512, 768, 1024
+    announce(f"mxfp8_gemm M={M} N={N} K={K} variant={variant}")
+    a, asc, b, bsc = inputs.mxfp8_inputs(M, N, K, seed=7)
+    ref = o8.mxfp8_gemm_ref(a, asc, b, bsc)
+    c32 = torch.ops.mi355.mxfp8_gemm(a.to(dev), asc.to(dev), b.to(dev), bsc.to(dev), "float32", variant).cpu()
+    assert _rel_err(c32, ref) < HW_SUM
+    c16 = torch.ops.mi355.mxfp8_gemm(a.to(dev), asc.to(dev), b.to(dev), bsc.to(dev), "bfloat16", variant).cpu()
+    assert _rel_err(c16, ref) < REL
+    assert torch.equal(c16, c32.bfloat16())  # the bf16 epilogue is round-to-nearest-even of the fp32 result
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 32), (33, 70, 96), (100, 260, 160), (257, 255, 2048), (256, 256, 256), (512, 256, 768)])
+def test_mxfp8_gemm_shapes(dev, shape):
+    """Ragged shapes (generic kernel: odd numbers of scale blocks, partial tiles) and the smallest / odd slab
+    counts of the tiled kernel."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs, mxfp8 as o8
+
+    M, N, K = shape
+    announce(f"mxfp8_gemm shape {shape}")
+    a, asc, b, bsc = inputs.mxfp8_inputs(M, N, K, seed=5)
+    ref = o8.mxfp8_gemm_ref(a, asc, b, bsc)
+    c = torch.ops.mi355.mxfp8_gemm(a.to(dev), asc.to(dev), b.to(dev), bsc.to(dev), "float32", -1).cpu()
+    assert _rel_err(c, ref) < HW_SUM
+
+
+def test_mxfp8_one_hot_layout(dev):
+    """A single non-zero element at every k position of a 256-wide row pair: pins which byte of a lane's 32
+    belongs to which k and which scale byte goes with which block (a swapped half or block shows up here)."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import mxfp8 as o8
+
+    announce("mxfp8 one-hot layout")
+    K = 256
+    a = torch.zeros(K, K, dtype=torch.uint8)
+    a[torch.arange(K), torch.arange(K)] = 0x38  # row i has 1.0 at k = i
+    g = torch.Generator().manual_seed(1)
+    asc = (120 + torch.randint(0, 15, (K, K // 32), generator=g)).to(torch.uint8)
+    b = torch.randint(0, 256, (256, K), generator=g).to(torch.uint8)
+    b = torch.where((b & 0x7F) == 0x7F, b - 1, b)
+    bsc = (120 + torch.randint(0, 15, (256, K // 32), generator=g)).to(torch.uint8)
+    for variant in (0, 1):
+        c = torch.ops.mi355.mxfp8_gemm(a.to(dev), asc.to(dev), b.to(dev), bsc.to(dev), "float32", variant).cpu()
+        # C[i, n] = 2^(asc[i, i/32] - 127) * dq(B)[n, i]
+        db = torch.from_numpy(o8.mxfp8_dequant_ref(b, bsc))
+        sa = torch.from_numpy(o8.mxfp8_dequant_ref(a, asc))[torch.arange(K), torch.arange(K)]
+        assert torch.equal(c, sa[:, None] * db.t()), variant
+
+
+def test_mxfp8_full_size_cross_variant(dev):
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs, mxfp8 as o8
+
+    M, N, K = 2048, 4096, 4096
+    announce(f"mxfp8 full size {M}x{N}x{K}")
+    a, asc, b, bsc = [t.to(dev) for t in inputs.mxfp8_inputs(M, N, K)]
+    tiled = torch.ops.mi355.mxfp8_gemm(a, asc, b, bsc, "float32", 0)
+    assert torch.equal(tiled, torch.ops.mi355.mxfp8_gemm(a, asc, b, bsc, "float32", 0))
+    generic = torch.ops.mi355.mxfp8_gemm(a, asc, b, bsc, "float32", 1)
+    assert _rel_err(tiled, generic) < HW_SUM  # the two kernels pair blocks differently
+    rows = torch.tensor([0, 255, 256, 1023, M - 1])
+    ref = o8.mxfp8_gemm_ref(a[rows.to(dev)].cpu(), asc[rows.to(dev)].cpu(), b.cpu(), bsc.cpu())
+    assert _rel_err(tiled[rows.to(dev)].cpu(), ref) < HW_SUM
+
+
+def test_mxfp8_contract_errors(dev):
+    import iree_turbine_amd  # noqa: F401
+
+    a = torch.zeros(256, 48, dtype=torch.uint8, device=dev)
+    s = torch.zeros(256, 1, dtype=torch.uint8, device=dev)
+    with pytest.raises(ValueError):
+        torch.ops.mi355.mxfp8_gemm(a, s, a, s, "bfloat16", -1)  # K = 48
+    a = torch.zeros(256, 128, dtype=torch.uint8, device=dev)
+    s = torch.zeros(256, 4, dtype=torch.uint8, device=dev)
+    with pytest.raises(ValueError):
+        torch.ops.mi355.mxfp8_gemm(a, s, a, s, "bfloat16", 0)  # tiled kernel needs K % 256 == 0
+    with pytest.raises(ValueError):
+        torch.ops.mi355.mxfp8_gemm(a, s, a, s, "float16", -1)
