@@ -108,7 +108,7 @@ int mi355_flash_attn_fwd_strided(const void* q, const void* k, const void* v, vo
  *              beyond ceil(seq_len/page_size) are never read
  * seq_lens:    [num_seqs]                                 int32, >= 0
  * out:         [num_seqs, num_q_heads, D]                 fp16
- * Requirements: D == 128, page_size == 16, num_q_heads == 4 * num_kv_heads or
+ * Requirements: D == 128, page_size 16, 32, 64, 128 or 256, num_q_heads == 4 * num_kv_heads or
  * any ratio in {1, 2, 4, 8, 16}.
  *
  * Split-K: phase 0 writes, for every (seq, q head, split), an unnormalised
@@ -158,7 +158,7 @@ int mi355_paged_decode_attn_window(const void* q, const void* k_cache, const voi
  * written at position start_pos[s] + t, i.e. page block_table[s][pos / page_size],
  * slot pos % page_size of k_cache / v_cache ([num_pages, page_size, num_kv_heads, D]).
  * Positions without a table entry (pos / page_size >= max_pages_per_seq) or whose
- * entry is outside [0, num_pages) are skipped.  D == 128, page_size == 16.
+ * entry is outside [0, num_pages) are skipped.  D == 128, page_size 16, 32, 64, 128 or 256.
  */
 int mi355_kv_cache_append(const void* k_new, const void* v_new, void* k_cache, void* v_cache,
                           const int32_t* block_table, const int32_t* start_pos,
@@ -180,7 +180,7 @@ int mi355_kv_cache_append(const void* k_new, const void* v_new, void* k_cache, v
  *              ceil(seq_len/page_size) are never read, ids outside [0, num_pages) read as zeros
  * seq_lens:    [num_seqs] int32 (clamped to [0, max_pages_per_seq * page_size]); queries with
  *              no visible key produce zeros
- * D == 128, page_size == 16, num_q_heads % num_kv_heads == 0.  Same kernel as
+ * D == 128, page_size 16, 32, 64, 128 or 256, num_q_heads % num_kv_heads == 0.  Same kernel as
  * mi355_flash_attn_fwd (fp32 online softmax, fp16 output), K/V tiles fetched page by page.
  * Replaces: the prefill call of the attention in tests/dynamo/llama_test.py:144-182 when the
  * cache is paged (no surviving paged counterpart in the reference).

@@ -220,11 +220,12 @@ __global__ __launch_bounds__(256) void fa_fwd_d128(const half_t* __restrict__ Q,
 }
 
 // Paged K/V (PAGED kernels): the keys and values of sequence b are the first seq_lens[b] token rows of the
-// pages block_table[b][0..], 16 tokens per page, laid out [page][token][kv head][128].
+// pages block_table[b][0..], 16 << page_shift tokens per page, laid out [page][token][kv head][128].  The kernel
+// walks 16-token blocks; a page is 1 << page_shift consecutive blocks.
 struct FaPaged {
   const int* block_table;  // [batch][max_pages]
   const int* seq_lens;     // [batch]
-  int max_pages, num_pages;
+  int max_pages, num_pages, page_shift;
 };
 
 // Software-pipelined form.  Same tiling and register layout, but the score MFMAs run one key tile
@@ -270,7 +271,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   int Sk = Sk_arg;
   if constexpr (PAGED) {
     Sk = __builtin_amdgcn_readfirstlane(pg.seq_lens[b_idx]);
-    Sk = Sk < 0 ? 0 : (Sk > pg.max_pages * 16 ? pg.max_pages * 16 : Sk);
+    const int cap = (pg.max_pages * 16) << pg.page_shift;
+    Sk = Sk < 0 ? 0 : (Sk > cap ? cap : Sk);
   }
   const int causal_off = Sk - Sq;
   const half_t* Qb = Q + b_idx * lay.q_b + h_idx * lay.q_h;
@@ -327,7 +329,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   auto load_ids = [&](int tile, int* ids) {
     if constexpr (PAGED) {
 #pragma unroll
-      for (int i = 0; i < 4; i++) ids[i] = (tile * 4 + i < pg.max_pages) ? table_row[tile * 4 + i] : -1;
+      for (int i = 0; i < 4; i++) {
+        const int blk = tile * 4 + i, page = blk >> pg.page_shift;  // 16-token block -> its page and place in it
+        const int e = page < pg.max_pages ? table_row[page] : -1;
+        ids[i] = (e >= 0 && e < pg.num_pages) ? (e << pg.page_shift) + (blk & ((1 << pg.page_shift) - 1)) : -1;
+      }
     }
   };
   auto issue_kv = [&](const half_t* base, unsigned rb, unsigned voff, int tile, int lds_off, const int* ids) {
@@ -343,7 +349,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         const int id = ids[i];
         int rows = rem - 16 * i;
         rows = rows > 16 ? 16 : rows;
-        const bool ok = rows > 0 && id >= 0 && id < pg.num_pages;
+        const bool ok = rows > 0 && id >= 0;
         const buffer_rsrc_t rs = make_buffer(reinterpret_cast<const char*>(base) + (size_t)(ok ? id : 0) * 16u * rb,
                                              ok ? (unsigned)(rows - 1) * rb + 256u : 0u);
         buffer_load_lds_16B(rs, voff, 0, dst + i * 4096);
@@ -597,7 +603,7 @@ static int fa_launch(const void* q, const void* k, const void* v, void* o, int64
   } else {
     auto kern = is_causal ? fa_fwd_d128_pipe<true, false> : fa_fwd_d128_pipe<false, false>;
     hipLaunchKernelGGL(kern, grid, block, lds_bytes, s, (const half_t*)q, (const half_t*)k, (const half_t*)v, (half_t*)o, BH,
-                       (int)Sq, (int)Sk, scale_log2e, q_blocks, lay, FaPaged{nullptr, nullptr, 0, 0});
+                       (int)Sq, (int)Sk, scale_log2e, q_blocks, lay, FaPaged{nullptr, nullptr, 0, 0, 0});
   }
   return check_launch(variant == 1 ? "fa_fwd_d128" : "fa_fwd_d128_pipe", grid, block, lds_bytes);
 }
@@ -642,9 +648,13 @@ extern "C" int mi355_paged_prefill_attn(const void* q, const void* k_cache, cons
   const char* who = "paged_prefill_attn";
   if (!q || !k_cache || !v_cache || !block_table || !seq_lens || !out) return fail(-MI355_E_NULL, "%s: null pointer", who);
   if (D != 128) return fail(-MI355_E_SHAPE, "%s: head dim %lld not supported (only 128)", who, (long long)D);
-  if (page_size != 16) return fail(-MI355_E_SHAPE, "%s: page size %lld not supported (only 16)", who, (long long)page_size);
+  int page_shift = -1;
+  for (int sh = 0; sh <= 4; sh++)
+    if (page_size == (16ll << sh)) page_shift = sh;
+  if (page_shift < 0) return fail(-MI355_E_SHAPE, "%s: page size %lld not supported (16, 32, 64, 128 or 256)", who, (long long)page_size);
   if (num_seqs <= 0 || num_new <= 0 || num_q_heads <= 0 || num_kv_heads <= 0 || max_pages_per_seq <= 0 || num_pages <= 0 ||
-      num_seqs * num_q_heads > (1 << 24) || num_new > (1 << 20) || max_pages_per_seq > (1 << 20) || num_pages > (1 << 24))
+      num_seqs * num_q_heads > (1 << 24) || num_new > (1 << 20) || max_pages_per_seq > (1 << 20) || num_pages > (1 << 24) ||
+      (max_pages_per_seq * page_size) > (1 << 24))
     return fail(-MI355_E_SHAPE, "%s: bad shape seqs=%lld new=%lld q_heads=%lld kv_heads=%lld max_pages=%lld pages=%lld", who,
                 (long long)num_seqs, (long long)num_new, (long long)num_q_heads, (long long)num_kv_heads,
                 (long long)max_pages_per_seq, (long long)num_pages);
@@ -673,7 +683,8 @@ extern "C" int mi355_paged_prefill_attn(const void* q, const void* k_cache, cons
     attr_set = true;
   }
   dim3 grid(BH * ((q_blocks + 1) / 2)), block(256);
-  const FaPaged pg{static_cast<const int*>(block_table), static_cast<const int*>(seq_lens), (int)max_pages_per_seq, (int)num_pages};
+  const FaPaged pg{static_cast<const int*>(block_table), static_cast<const int*>(seq_lens), (int)max_pages_per_seq, (int)num_pages,
+                   page_shift};
   hipLaunchKernelGGL(kern, grid, block, lds_bytes, reinterpret_cast<hipStream_t>(stream), (const half_t*)q, (const half_t*)k_cache,
                      (const half_t*)v_cache, (half_t*)out, BH, (int)num_new, 0, scale * 1.4426950408889634f, q_blocks, lay, pg);
   return check_launch("fa_fwd_d128_pipe<paged>", grid, block, lds_bytes);

@@ -33,7 +33,7 @@ __global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
     const half_t* __restrict__ Q, const half_t* __restrict__ Kc, const half_t* __restrict__ Vc,
     const int* __restrict__ block_table, const int* __restrict__ seq_lens, float* __restrict__ part_acc,
     float* __restrict__ part_ml, half_t* __restrict__ out, int num_kv_heads, int max_pages_per_seq, int num_splits,
-    float scale_log2e, int window) {
+    float scale_log2e, int window, int page_shift) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -77,8 +77,10 @@ __global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
   half8 kf[2][2][4];  // [buffer][page][ks]
   auto issue = [&](int step, int buf) {
     const int pa = p_begin + 2 * (wave + PD_WAVES * step);
-    const int pg0 = bt[pa];
-    const int pg1 = (pa + 1 < p_end) ? bt[pa + 1] : pg0;
+    // the kernel walks 16-token blocks; a page of 16 << page_shift tokens is that many consecutive blocks
+    const int sub = (1 << page_shift) - 1;
+    const int pg0 = (bt[pa >> page_shift] << page_shift) + (pa & sub);
+    const int pg1 = (pa + 1 < p_end) ? (bt[(pa + 1) >> page_shift] << page_shift) + ((pa + 1) & sub) : pg0;
     char* dst = my_lds + buf * 8192;
 #pragma unroll
     for (int x = 0; x < 2; x++) {
@@ -250,7 +252,7 @@ const char* decode_variant_name(int i) { return i == 0 ? kDecodeVariants[0] : nu
 template <int G>
 static int launch_phase0(const void* q, const void* kc, const void* vc, const int32_t* bt, const int32_t* sl, float* pacc,
                          float* pml, void* out, int num_seqs, int num_kv_heads, int max_pages, int num_splits, float scale,
-                         int window, hipStream_t stream) {
+                         int window, int page_shift, hipStream_t stream) {
   auto kern = paged_decode_phase0<G>;
   constexpr int lds_bytes = PD_WAVES * PD_WAVE_LDS;
   static_assert(lds_bytes >= (int)((2 * PD_WAVES * 16 + PD_WAVES * G * 128) * sizeof(float)), "merge area must fit");
@@ -266,14 +268,23 @@ static int launch_phase0(const void* q, const void* kc, const void* vc, const in
   }
   dim3 grid(num_splits, num_kv_heads, num_seqs), block(PD_WAVES * 64);
   hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)q, (const half_t*)kc, (const half_t*)vc, bt, sl,
-                     pacc, pml, (half_t*)out, num_kv_heads, max_pages, num_splits, scale * 1.4426950408889634f, window);
+                     pacc, pml, (half_t*)out, num_kv_heads, max_pages, num_splits, scale * 1.4426950408889634f, window, page_shift);
   return check_launch("paged_decode_phase0", grid, block, lds_bytes);
+}
+
+// 16 << shift tokens per page, shift 0..4; -1 for any other size
+static int page_shift_of(int64_t page_size) {
+  for (int sh = 0; sh <= 4; sh++)
+    if (page_size == (16ll << sh)) return sh;
+  return -1;
 }
 
 static int check_decode_args(const char* fn, int64_t num_seqs, int64_t hq, int64_t hkv, int64_t D, int64_t page_size,
                              int64_t max_pages, int64_t num_pages, int64_t num_splits, float scale) {
   if (D != 128) return fail(-MI355_E_SHAPE, "%s: head dim %lld not supported (only 128)", fn, (long long)D);
-  if (page_size != 16) return fail(-MI355_E_SHAPE, "%s: page size %lld not supported (only 16)", fn, (long long)page_size);
+  if (page_shift_of(page_size) < 0)
+    return fail(-MI355_E_SHAPE, "%s: page size %lld not supported (16, 32, 64, 128 or 256)", fn, (long long)page_size);
+  if (num_pages > (1 << 26)) return fail(-MI355_E_SHAPE, "%s: too many pages", fn);
   if (num_seqs <= 0 || hq <= 0 || hkv <= 0 || max_pages <= 0 || num_pages <= 0 || num_seqs > 65535 || hkv > 65535)
     return fail(-MI355_E_SHAPE, "%s: bad sizes seqs=%lld hq=%lld hkv=%lld max_pages=%lld num_pages=%lld", fn,
                 (long long)num_seqs, (long long)hq, (long long)hkv, (long long)max_pages, (long long)num_pages);
@@ -288,10 +299,10 @@ static int check_decode_args(const char* fn, int64_t num_seqs, int64_t hq, int64
 
 static int run_phase0(const void* q, const void* kc, const void* vc, const int32_t* bt, const int32_t* sl, float* pacc,
                       float* pml, void* out, int64_t num_seqs, int64_t hq, int64_t hkv, int64_t max_pages,
-                      int64_t num_splits, float scale, int window, hipStream_t stream) {
+                      int64_t num_splits, float scale, int window, int page_shift, hipStream_t stream) {
   const int G = (int)(hq / hkv);
 #define MI355_PD_CASE(GG) \
-  case GG: return launch_phase0<GG>(q, kc, vc, bt, sl, pacc, pml, out, (int)num_seqs, (int)hkv, (int)max_pages, (int)num_splits, scale, window, stream)
+  case GG: return launch_phase0<GG>(q, kc, vc, bt, sl, pacc, pml, out, (int)num_seqs, (int)hkv, (int)max_pages, (int)num_splits, scale, window, page_shift, stream)
   switch (G) {
     MI355_PD_CASE(1);
     MI355_PD_CASE(2);
@@ -320,7 +331,7 @@ extern "C" int mi355_paged_decode_phase0(const void* q, const void* k_cache, con
   if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(part_acc))
     return fail(-MI355_E_ALIGN, "paged_decode_phase0: q, k_cache, v_cache, part_acc must be 16-byte aligned");
   return run_phase0(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, nullptr, num_seqs, num_q_heads,
-                    num_kv_heads, max_pages_per_seq, num_splits, scale, 0, reinterpret_cast<hipStream_t>(stream));
+                    num_kv_heads, max_pages_per_seq, num_splits, scale, 0, page_shift_of(page_size), reinterpret_cast<hipStream_t>(stream));
 }
 
 extern "C" int mi355_paged_decode_phase1(const float* part_acc, const float* part_ml, void* out, int64_t num_seqs,
@@ -349,11 +360,11 @@ static int decode_attn(const char* fn, const void* q, const void* k_cache, const
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (num_splits == 1)
     return run_phase0(q, k_cache, v_cache, block_table, seq_lens, nullptr, nullptr, out, num_seqs, num_q_heads, num_kv_heads,
-                      max_pages_per_seq, 1, scale, (int)window, s);
+                      max_pages_per_seq, 1, scale, (int)window, page_shift_of(page_size), s);
   if (!part_acc || !part_ml) return fail(-MI355_E_SCRATCH, "%s: num_splits > 1 needs part_acc / part_ml scratch", fn);
   if (!aligned16(part_acc)) return fail(-MI355_E_ALIGN, "%s: part_acc must be 16-byte aligned", fn);
   if (int rc = run_phase0(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, nullptr, num_seqs, num_q_heads,
-                          num_kv_heads, max_pages_per_seq, num_splits, scale, (int)window, s))
+                          num_kv_heads, max_pages_per_seq, num_splits, scale, (int)window, page_shift_of(page_size), s))
     return rc;
   return mi355_paged_decode_phase1(part_acc, part_ml, out, num_seqs, num_q_heads, D, num_splits, stream);
 }
@@ -384,20 +395,21 @@ __global__ __launch_bounds__(256) void kv_cache_append_kernel(const half_t* __re
                                                               half_t* __restrict__ k_cache, half_t* __restrict__ v_cache,
                                                               const int* __restrict__ block_table,
                                                               const int* __restrict__ start_pos, int n_new, int num_kv_heads,
-                                                              int max_pages_per_seq, int num_pages, long long n_tokens) {
+                                                              int max_pages_per_seq, int num_pages, long long n_tokens,
+                                                              int page_bits) {
   const int lane = threadIdx.x & 63;
   const long long tok = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);  // flat (seq, new token) index
   if (tok >= n_tokens) return;
   const int seq = (int)(tok / n_new), t = (int)(tok - (long long)seq * n_new);
   const int pos = start_pos[seq] + t;
   if (pos < 0) return;
-  const int pidx = pos >> 4;
+  const int pidx = pos >> page_bits;  // page_bits = log2(tokens per page)
   if (pidx >= max_pages_per_seq) return;  // no table entry for this position: nothing is written
   const int page = block_table[(size_t)seq * max_pages_per_seq + pidx];
   if (page < 0 || page >= num_pages) return;  // padded entry
   const int row_halfs = num_kv_heads * 128;
   const size_t src = (size_t)tok * row_halfs;
-  const size_t dst = ((size_t)page * 16 + (pos & 15)) * row_halfs;
+  const size_t dst = (((size_t)page << page_bits) + (pos & ((1 << page_bits) - 1))) * row_halfs;
   for (int c = lane * 8; c < row_halfs; c += 512) {
     *reinterpret_cast<half8*>(k_cache + dst + c) = *reinterpret_cast<const half8*>(k_new + src + c);
     *reinterpret_cast<half8*>(v_cache + dst + c) = *reinterpret_cast<const half8*>(v_new + src + c);
@@ -410,7 +422,8 @@ extern "C" int mi355_kv_cache_append(const void* k_new, const void* v_new, void*
                                      int64_t num_pages, void* stream) {
   if (!k_new || !v_new || !k_cache || !v_cache || !block_table || !start_pos) return fail(-MI355_E_NULL, "kv_cache_append: null pointer");
   if (D != 128) return fail(-MI355_E_SHAPE, "kv_cache_append: head dim %lld not supported (only 128)", (long long)D);
-  if (page_size != 16) return fail(-MI355_E_SHAPE, "kv_cache_append: page size %lld not supported (only 16)", (long long)page_size);
+  if (page_shift_of(page_size) < 0)
+    return fail(-MI355_E_SHAPE, "kv_cache_append: page size %lld not supported (16, 32, 64, 128 or 256)", (long long)page_size);
   if (num_seqs <= 0 || n_new <= 0 || num_kv_heads <= 0 || max_pages_per_seq <= 0 || num_pages <= 0 || n_new > (1 << 24) ||
       num_kv_heads > 65535 || num_seqs * n_new > (1ll << 40))
     return fail(-MI355_E_SHAPE, "kv_cache_append: bad sizes seqs=%lld n_new=%lld hkv=%lld max_pages=%lld num_pages=%lld",
@@ -421,6 +434,6 @@ extern "C" int mi355_kv_cache_append(const void* k_new, const void* v_new, void*
   dim3 grid((unsigned)((n_tokens + 3) / 4)), block(256);
   hipLaunchKernelGGL(kv_cache_append_kernel, grid, block, 0, reinterpret_cast<hipStream_t>(stream), (const half_t*)k_new,
                      (const half_t*)v_new, (half_t*)k_cache, (half_t*)v_cache, block_table, start_pos, (int)n_new,
-                     (int)num_kv_heads, (int)max_pages_per_seq, (int)num_pages, n_tokens);
+                     (int)num_kv_heads, (int)max_pages_per_seq, (int)num_pages, n_tokens, 4 + page_shift_of(page_size));
   return check_launch("kv_cache_append_kernel", grid, block, 0);
 }

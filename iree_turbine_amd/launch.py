@@ -177,7 +177,7 @@ def kv_cache_append(k_new, v_new, k_cache, v_cache, block_table, start_pos) -> N
 
 def paged_prefill_attn_out(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_table: Tensor, seq_lens: Tensor, out: Tensor,
                            scale: float) -> Tensor:
-    """q, out [S, n_new, Hq, 128]; caches [P, 16, Hkv, 128]; seq_lens counts the new tokens (see mi355_paged_prefill_attn)."""
+    """q, out [S, n_new, Hq, 128]; caches [P, page, Hkv, 128]; seq_lens counts the new tokens (see mi355_paged_prefill_attn)."""
     dev = _dev(q, k_cache, v_cache, block_table, seq_lens, out)
     q, k_cache, v_cache = q.contiguous(), k_cache.contiguous(), v_cache.contiguous()
     block_table, seq_lens = block_table.contiguous(), seq_lens.contiguous()

@@ -107,6 +107,9 @@ def _like_q(q: Tensor, device) -> Tensor:
     return torch.empty([q.size(i) for i in order], dtype=torch.float16, device=device).permute(inv)
 
 
+PAGE_SIZES = (16, 32, 64, 128, 256)  # tokens per KV-cache page
+
+
 def _check_paged_args(op: str, q: Tensor, k_cache: Tensor, v_cache: Tensor, block_table: Tensor, seq_lens: Tensor):
     _require(q.dim() == 3, f"{op}: q must be [num_seqs, num_q_heads, D]")
     _require(k_cache.dim() == 4 and v_cache.shape == k_cache.shape, f"{op}: k_cache / v_cache must both be [num_pages, page_size, num_kv_heads, D]")
@@ -115,7 +118,7 @@ def _check_paged_args(op: str, q: Tensor, k_cache: Tensor, v_cache: Tensor, bloc
     _require(seq_lens.dim() == 1 and seq_lens.dtype == torch.int32, f"{op}: seq_lens must be int32 [num_seqs]")
     _require(block_table.size(0) == q.size(0) and seq_lens.size(0) == q.size(0), f"{op}: block_table / seq_lens rows must equal num_seqs")
     _require(q.size(2) == 128 and k_cache.size(3) == 128, f"{op}: head dim must be 128")
-    _require(k_cache.size(1) == 16, f"{op}: page size {k_cache.size(1)} not supported (only 16)")
+    _require(k_cache.size(1) in PAGE_SIZES, f"{op}: page size {k_cache.size(1)} not supported {PAGE_SIZES}")
     hq, hkv = q.size(1), k_cache.size(2)
     _require(hkv > 0 and hq % hkv == 0 and hq // hkv in (1, 2, 4, 8, 16), f"{op}: {hq} q heads over {hkv} kv heads is not supported (ratio 1, 2, 4, 8 or 16)")
     _require(q.size(0) > 0 and block_table.size(1) > 0, f"{op}: empty batch")
@@ -132,7 +135,7 @@ def default_num_kv_splits(seq_lens_max: int, num_seqs: int, num_kv_heads: int) -
 class paged_decode_attn(CustomOp):
     """One-token-per-sequence GQA attention over a paged fp16 KV cache (both phases).
 
-    q [S, Hq, 128]; k_cache, v_cache [P, 16, Hkv, 128]; block_table int32 [S, max_pages];
+    q [S, Hq, 128]; k_cache, v_cache [P, page, Hkv, 128]; block_table int32 [S, max_pages];
     seq_lens int32 [S]; returns [S, Hq, 128] fp16.  num_kv_splits <= 0 picks a default from
     the table width.  scale <= 0 selects 1/sqrt(D).  GQA semantics (q head h reads kv head
     h // (Hq/Hkv)) follow repeat_kv in tests/dynamo/llama_test.py:82-91."""
@@ -186,7 +189,7 @@ class paged_decode_attn_window(CustomOp):
 class kv_cache_append(CustomOp):
     """In-place paged form of `cache[:bsz, start_pos : start_pos + n_new] = x` (tests/dynamo/llama_test.py:165-166)
     with one start position per sequence: k_new, v_new [S, n_new, Hkv, 128] fp16 go to positions
-    start_pos[s] .. start_pos[s] + n_new - 1 of k_cache, v_cache [P, 16, Hkv, 128] through block_table [S, max_pages]."""
+    start_pos[s] .. start_pos[s] + n_new - 1 of k_cache, v_cache [P, page, Hkv, 128] through block_table [S, max_pages]."""
 
     signature = "kv_cache_append(Tensor k_new, Tensor v_new, Tensor(a!) k_cache, Tensor(b!) v_cache, Tensor block_table, Tensor start_pos) -> ()"
 
@@ -197,7 +200,7 @@ class kv_cache_append(CustomOp):
         _require(kc.t.dim() == 4 and kc.t.shape == vc.t.shape, f"{fn}: k_cache and v_cache must both be [P, page, Hkv, D]")
         _require(all(t.t.dtype == torch.float16 for t in (kn, vn, kc, vc)), f"{fn}: tensors must be float16")
         _require(kn.t.size(3) == 128 and kc.t.size(3) == 128, f"{fn}: head dim must be 128")
-        _require(kc.t.size(1) == 16, f"{fn}: page size must be 16")
+        _require(kc.t.size(1) in PAGE_SIZES, f"{fn}: page size {kc.t.size(1)} not supported {PAGE_SIZES}")
         _require(kn.t.size(2) == kc.t.size(2), f"{fn}: k_new and k_cache disagree on the number of kv heads")
         _require(kn.t.size(0) > 0 and kn.t.size(1) > 0, f"{fn}: empty k_new")
         _require(bt.t.dim() == 2 and bt.t.dtype == torch.int32 and bt.t.size(0) == kn.t.size(0), f"{fn}: block_table must be int32 [S, max_pages]")
@@ -211,7 +214,7 @@ class kv_cache_append(CustomOp):
 @CustomOp.register
 class paged_prefill_attn(CustomOp):
     """Causal attention of the n_new latest tokens of every sequence over its paged KV cache (chunked / prefix
-    prefill): q [S, n_new, Hq, 128], caches [P, 16, Hkv, 128], block_table int32 [S, max_pages], seq_lens int32 [S]
+    prefill): q [S, n_new, Hq, 128], caches [P, page, Hkv, 128], block_table int32 [S, max_pages], seq_lens int32 [S]
     counting the new tokens, whose K/V are in the cache already (kv_cache_append).  Query t sees positions
     j <= seq_lens[s] - n_new + t: the mask of tests/dynamo/llama_test.py:285-290 shifted by the cached prefix."""
 
@@ -225,7 +228,7 @@ class paged_prefill_attn(CustomOp):
         _require(kc.t.dim() == 4 and kc.t.shape == vc.t.shape, f"{fn}: k_cache / v_cache must both be [num_pages, page_size, num_kv_heads, D]")
         _require(all(t.t.dtype == torch.float16 for t in (q, kc, vc)), f"{fn}: q, k_cache, v_cache must be float16")
         _require(q.t.size(3) == 128 and kc.t.size(3) == 128, f"{fn}: head dim must be 128")
-        _require(kc.t.size(1) == 16, f"{fn}: page size {kc.t.size(1)} not supported (only 16)")
+        _require(kc.t.size(1) in PAGE_SIZES, f"{fn}: page size {kc.t.size(1)} not supported {PAGE_SIZES}")
         _require(kc.t.size(2) > 0 and q.t.size(2) % kc.t.size(2) == 0, f"{fn}: {q.t.size(2)} q heads over {kc.t.size(2)} kv heads")
         _require(bt.t.dim() == 2 and bt.t.dtype == torch.int32 and bt.t.size(0) == q.t.size(0), f"{fn}: block_table must be int32 [num_seqs, max_pages]")
         _require(sl.t.dim() == 1 and sl.t.dtype == torch.int32 and sl.t.size(0) == q.t.size(0), f"{fn}: seq_lens must be int32 [num_seqs]")

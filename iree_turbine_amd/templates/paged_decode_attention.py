@@ -22,7 +22,7 @@ def get_paged_decode_attention_kernels(shape: AttentionShape, mfma_variant=None,
     """Two-phase paged GQA decode attention.
 
     phase 0: kernel(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml)
-             q [S, Hq, 128] f16; caches [P, 16, Hkv, 128] f16; block_table i32 [S, max_pages];
+             q [S, Hq, 128] f16; caches [P, page, Hkv, 128] f16; block_table i32 [S, max_pages];
              seq_lens i32 [S]; part_acc f32 [S, Hq, U, 128]; part_ml f32 [S, Hq, U, 2] (outputs)
     phase 1: kernel(part_acc, part_ml, out) with out [S, Hq, 128] f16 (output)
     Returns (phase_0, phase_1, hyperparams_0, hyperparams_1).  GQA semantics as repeat_kv,

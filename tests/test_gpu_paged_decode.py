@@ -272,3 +272,38 @@ def test_paged_prefill_guards(dev):
         torch.ops.mi355.paged_prefill_attn(dq[..., :64].contiguous(), dkc, dvc, dbt, dsl, 0.0)
     with pytest.raises(ValueError):
         torch.ops.mi355.paged_prefill_attn(dq, dkc, dvc, dbt.long(), dsl, 0.0)
+
+
+@pytest.mark.parametrize("page", [32, 64, 128, 256])
+def test_larger_pages_decode_append_prefill(dev, page):
+    """Pages of 32..256 tokens: the kernels walk 16-token blocks inside them.  Decode (with and without split
+    and window), append and chunked prefill against the oracles, which gather whole pages."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs, paged_decode as op
+
+    announce(f"paged kernels with page size {page}")
+    q, kc, vc, bt, sl = inputs.paged_decode_inputs(num_seqs=5, num_q_heads=8, num_kv_heads=2, page=page, min_len=1, max_len=900, seed=13)
+    dq, dkc, dvc, dbt, dsl = _to(dev, q, kc, vc, bt, sl)
+    for splits in (1, 3):
+        out = torch.ops.mi355.paged_decode_attn(dq, dkc, dvc, dbt, dsl, 0.0, splits)
+        torch.testing.assert_close(out.float().cpu(), op.paged_decode_ref(q, kc, vc, bt, sl), rtol=RTOL, atol=ATOL)
+    out = torch.ops.mi355.paged_decode_attn_window(dq, dkc, dvc, dbt, dsl, 0.0, 2, 100)
+    torch.testing.assert_close(out.float().cpu(), op.paged_decode_ref(q, kc, vc, bt, sl, window=100), rtol=RTOL, atol=ATOL)
+    # append 40 tokens at the end of every sequence that has room for them in its own pages
+    n_new = 40
+    g = torch.Generator().manual_seed(page)
+    kn = torch.randn(5, n_new, 2, 128, generator=g).half()
+    vn = torch.randn(5, n_new, 2, 128, generator=g).half()
+    start = (sl - n_new).clamp(min=0).int()
+    k2, v2 = dkc.clone(), dvc.clone()
+    torch.ops.mi355.kv_cache_append(kn.to(dev), vn.to(dev), k2, v2, dbt, start.to(dev))
+    kr, vr = op.kv_cache_append_ref(kn, vn, kc, vc, bt, start)
+    assert torch.equal(k2.cpu(), kr) and torch.equal(v2.cpu(), vr)
+    # chunked prefill of those 40 tokens over the updated caches
+    qn = torch.randn(5, n_new, 8, 128, generator=g).half()
+    lens2 = torch.maximum(sl, torch.full_like(sl, n_new)).int()  # sequences shorter than the chunk grew to its length
+    ok = [s for s in range(5) if int(lens2[s]) <= int((sl[s] + page - 1) // page) * page]  # ... if their pages hold it
+    got = torch.ops.mi355.paged_prefill_attn(qn.to(dev), k2, v2, dbt, lens2.to(dev), 0.0).float().cpu()
+    ref = op.paged_prefill_ref(qn, kr, vr, bt, lens2)
+    assert len(ok) >= 3
+    torch.testing.assert_close(got[ok], ref[ok], rtol=RTOL, atol=ATOL)

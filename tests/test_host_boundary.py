@@ -75,7 +75,7 @@ def test_op_contract_errors_on_meta():
     bt = torch.empty(2, 4, dtype=torch.int32, device="meta")
     sl = torch.empty(2, dtype=torch.int32, device="meta")
     with pytest.raises(ValueError, match="page size"):
-        torch.ops.mi355.paged_decode_attn(h(2, 8, 128), h(9, 32, 2, 128), h(9, 32, 2, 128), bt, sl, 0.0, 1)
+        torch.ops.mi355.paged_decode_attn(h(2, 8, 128), h(9, 48, 2, 128), h(9, 48, 2, 128), bt, sl, 0.0, 1)  # 48 is not 16 * 2^n
     with pytest.raises(ValueError, match="q heads"):
         torch.ops.mi355.paged_decode_attn(h(2, 6, 128), h(9, 16, 4, 128), h(9, 16, 4, 128), bt, sl, 0.0, 1)
 
