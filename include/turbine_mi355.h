@@ -219,6 +219,16 @@ int mi355_mxfp8_gemm(const void* a, const void* a_scale, const void* b, const vo
                      int out_dtype, int variant, void* stream);
 
 /*
+ * Plain fp8 GEMM (no block scales): C[M,N] = alpha . A . B^T with A [M, K], B [N, K] OCP FP8 E4M3 codes,
+ * fp32 accumulation, bf16 or fp32 out; alpha carries the product of the per-tensor scales a caller
+ * quantised with.  The kernels of mi355_mxfp8_gemm with every block scale fixed at 2^0.  K % 32 == 0.
+ * Replaces: GEMMForward (iree/turbine/kernel/boo/op_exports/gemm.py:217-230) for fp8 operands
+ * (dtype iree/turbine/kernel/_support/dtype.py:115, f8e4m3fn).
+ */
+int mi355_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K,
+                   float alpha, int out_dtype, int variant, void* stream);
+
+/*
  * MXFP4 dequantisation on the device (used to show that the device decodes
  * the format bit-exactly): out[r,k] = E2M1(code) * 2^(scale-127) as fp32.
  * codes: uint8 [rows, K/2]; scales: uint8 [rows, K/32]; out: fp32 [rows, K].

@@ -15,6 +15,7 @@
 // (its half of block ks) and chunk 4+2ks+h (its half of block 2+ks), and supplies byte ks (h = 0) or 2+ks
 // (h = 1) of the ONE scale dword a row has per slab; lanes of the upper half shift their dword right by 16
 // once, so that op_sel = ks picks the byte for both halves.
+#include <math.h>
 #include <type_traits>
 
 #include "common.hpp"
@@ -60,11 +61,12 @@ __device__ __forceinline__ floatx16 mfma_fp8_32x32x64(intx8 a, int sa, intx8 b, 
 
 }  // namespace
 
-template <int BM, int BN, int WM, int WN, typename OutT>
+// SCALED = false: plain fp8 GEMM, C = alpha . A . B^T (every block scale is 2^0, no scale traffic).
+template <int BM, int BN, int WM, int WN, typename OutT, bool SCALED>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp8_tiled(const uint8_t* __restrict__ A, const uint8_t* __restrict__ As,
                                                                 const uint8_t* __restrict__ B, const uint8_t* __restrict__ Bs,
                                                                 OutT* __restrict__ C, int M, int N, int K, int tiles_m,
-                                                                int tiles_n, int group_m) {
+                                                                int tiles_n, int group_m, float alpha) {
   constexpr int NW = WM * WN;
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -122,12 +124,19 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp8_tiled(const uint8_t* _
   const uint8_t* as_src = As + (size_t)(tile_m * BM + wm * WTM + r32) * Ksc;
   const uint8_t* bs_src = Bs + (size_t)(tile_n * BN + wn * WTN + r32) * Ksc;
   auto fetch_scales = [&](int* da, int* db, int slab) {
+    if constexpr (SCALED) {
 #pragma unroll
-    for (int j = 0; j < TM; j++)
-      da[j] = (int)(*reinterpret_cast<const unsigned*>(as_src + (size_t)j * 32 * Ksc + slab * 4) >> (16 * h));
+      for (int j = 0; j < TM; j++)
+        da[j] = (int)(*reinterpret_cast<const unsigned*>(as_src + (size_t)j * 32 * Ksc + slab * 4) >> (16 * h));
 #pragma unroll
-    for (int i = 0; i < TN; i++)
-      db[i] = (int)(*reinterpret_cast<const unsigned*>(bs_src + (size_t)i * 32 * Ksc + slab * 4) >> (16 * h));
+      for (int i = 0; i < TN; i++)
+        db[i] = (int)(*reinterpret_cast<const unsigned*>(bs_src + (size_t)i * 32 * Ksc + slab * 4) >> (16 * h));
+    } else {
+#pragma unroll
+      for (int j = 0; j < TM; j++) da[j] = 0x7f7f7f7f;
+#pragma unroll
+      for (int i = 0; i < TN; i++) db[i] = 0x7f7f7f7f;
+    }
   };
 
   floatx16 acc[TN][TM];
@@ -178,7 +187,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp8_tiled(const uint8_t* _
     mfmas(K0{}, fm0, fn0, sa[CUR], sb[CUR]);
     interleave();
     __builtin_amdgcn_sched_barrier(0);
-    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(TM + TN) : "memory");
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(SCALED ? TM + TN : 0) : "memory");
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
     issue_loads(CUR, kt + 2 < KT ? kt + 2 : KT - 1);
@@ -207,15 +216,16 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp8_tiled(const uint8_t* _
     for (int i = 0; i < TN; i++)
 #pragma unroll
       for (int q = 0; q < 4; q++)
-        Out8<OutT>::store4(crow + i * 32 + q * 8, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+        Out8<OutT>::store4(crow + i * 32 + q * 8, alpha * acc[i][j][4 * q], alpha * acc[i][j][4 * q + 1], alpha * acc[i][j][4 * q + 2],
+                           alpha * acc[i][j][4 * q + 3]);
   }
 }
 
 // Any shape with K % 32 == 0: one wave per 32x32 output tile, operands straight from global memory.
-template <typename OutT>
+template <typename OutT, bool SCALED>
 __global__ __launch_bounds__(256) void gemm_mxfp8_generic(const uint8_t* __restrict__ A, const uint8_t* __restrict__ As,
                                                           const uint8_t* __restrict__ B, const uint8_t* __restrict__ Bs,
-                                                          OutT* __restrict__ C, int M, int N, int K) {
+                                                          OutT* __restrict__ C, int M, int N, int K, float alpha) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r32 = lane & 31, h = lane >> 5;
   const int m = blockIdx.y * 32 + r32;
@@ -236,14 +246,14 @@ __global__ __launch_bounds__(256) void gemm_mxfp8_generic(const uint8_t* __restr
       const intx4 lo = *reinterpret_cast<const intx4*>(row);
       const intx4 hi = k1_ok ? *reinterpret_cast<const intx4*>(row + 32) : intx4{0, 0, 0, 0};
       fa = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      if (k_ok) sa = As[(size_t)m * Ksc + blk];
+      if (SCALED && k_ok) sa = As[(size_t)m * Ksc + blk];
     }
     if (n < N) {
       const uint8_t* row = B + (size_t)n * K + kb * 32 + 16 * h;
       const intx4 lo = *reinterpret_cast<const intx4*>(row);
       const intx4 hi = k1_ok ? *reinterpret_cast<const intx4*>(row + 32) : intx4{0, 0, 0, 0};
       fb = intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      if (k_ok) sb = Bs[(size_t)n * Ksc + blk];
+      if (SCALED && k_ok) sb = Bs[(size_t)n * Ksc + blk];
     }
     acc = mfma_fp8_32x32x64<0>(fb, sb, fa, sa, acc);
   }
@@ -252,7 +262,7 @@ __global__ __launch_bounds__(256) void gemm_mxfp8_generic(const uint8_t* __restr
 #pragma unroll
     for (int r = 0; r < 16; r++) {
       const int nn = nb + 8 * (r >> 2) + 4 * h + (r & 3);
-      if (nn < N) Out8<OutT>::store1(C + (size_t)m * N + nn, acc[r]);
+      if (nn < N) Out8<OutT>::store1(C + (size_t)m * N + nn, alpha * acc[r]);
     }
   }
 }
@@ -261,11 +271,11 @@ static const char* kMx8Variants[] = {"tiled_256x256x128_w2x2", "generic_32x128"}
 int mxfp8_variant_count() { return 2; }
 const char* mxfp8_variant_name(int i) { return (i >= 0 && i < 2) ? kMx8Variants[i] : nullptr; }
 
-template <typename OutT>
+template <typename OutT, bool SCALED>
 static int launch_mx8(int variant, const void* a, const void* as, const void* b, const void* bs, void* c, int M, int N, int K,
-                      hipStream_t stream) {
+                      float alpha, hipStream_t stream) {
   if (variant == 0) {
-    auto kern = gemm_mxfp8_tiled<256, 256, 2, 2, OutT>;
+    auto kern = gemm_mxfp8_tiled<256, 256, 2, 2, OutT, SCALED>;
     constexpr int lds_bytes = 2 * 512 * 128;
     static bool attr_set = false;
     if (!attr_set) {
@@ -279,12 +289,12 @@ static int launch_mx8(int variant, const void* a, const void* as, const void* b,
     const int tiles_m = M / 256, tiles_n = N / 256;
     dim3 grid(tiles_m * tiles_n), block(256);
     hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const uint8_t*)a, (const uint8_t*)as, (const uint8_t*)b,
-                       (const uint8_t*)bs, (OutT*)c, M, N, K, tiles_m, tiles_n, 4);
+                       (const uint8_t*)bs, (OutT*)c, M, N, K, tiles_m, tiles_n, 4, alpha);
     return check_launch("gemm_mxfp8_tiled", grid, block, lds_bytes);
   }
   dim3 grid((N + 127) / 128, (M + 31) / 32), block(256);
-  hipLaunchKernelGGL(gemm_mxfp8_generic<OutT>, grid, block, 0, stream, (const uint8_t*)a, (const uint8_t*)as, (const uint8_t*)b,
-                     (const uint8_t*)bs, (OutT*)c, M, N, K);
+  hipLaunchKernelGGL((gemm_mxfp8_generic<OutT, SCALED>), grid, block, 0, stream, (const uint8_t*)a, (const uint8_t*)as,
+                     (const uint8_t*)b, (const uint8_t*)bs, (OutT*)c, M, N, K, alpha);
   return check_launch("gemm_mxfp8_generic", grid, block, 0);
 }
 
@@ -308,6 +318,26 @@ extern "C" int mi355_mxfp8_gemm(const void* a, const void* a_scale, const void* 
   else if (variant == 0 && !fits0)
     return fail(-MI355_E_SHAPE, "mxfp8_gemm: variant %s needs M%%256==0, N%%256==0, K%%256==0 and 4-byte aligned scales", kMx8Variants[0]);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  if (out_dtype == MI355_F32) return launch_mx8<float>(variant, a, a_scale, b, b_scale, c, (int)M, (int)N, (int)K, s);
-  return launch_mx8<unsigned short>(variant, a, a_scale, b, b_scale, c, (int)M, (int)N, (int)K, s);
+  if (out_dtype == MI355_F32) return launch_mx8<float, true>(variant, a, a_scale, b, b_scale, c, (int)M, (int)N, (int)K, 1.f, s);
+  return launch_mx8<unsigned short, true>(variant, a, a_scale, b, b_scale, c, (int)M, (int)N, (int)K, 1.f, s);
+}
+
+extern "C" int mi355_fp8_gemm(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, float alpha, int out_dtype,
+                              int variant, void* stream) {
+  if (!a || !b || !c) return fail(-MI355_E_NULL, "fp8_gemm: null pointer");
+  if (M <= 0 || N <= 0 || K <= 0 || M > (1 << 30) || N > (1 << 30) || K > (1 << 27))
+    return fail(-MI355_E_SHAPE, "fp8_gemm: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+  if (K % 32 != 0) return fail(-MI355_E_SHAPE, "fp8_gemm: K=%lld must be a multiple of 32", (long long)K);
+  if (out_dtype != MI355_BF16 && out_dtype != MI355_F32)
+    return fail(-MI355_E_DTYPE, "fp8_gemm: out_dtype %d (want MI355_BF16 or MI355_F32)", out_dtype);
+  if (variant > 1) return fail(-MI355_E_DTYPE, "fp8_gemm: variant %d out of range", variant);
+  if (!isfinite(alpha)) return fail(-MI355_E_SHAPE, "fp8_gemm: alpha must be finite");
+  if (!aligned16(a) || !aligned16(b) || !aligned16(c)) return fail(-MI355_E_ALIGN, "fp8_gemm: a, b, c must be 16-byte aligned");
+  const bool fits0 = M % 256 == 0 && N % 256 == 0 && K % 256 == 0 && K >= 256;
+  if (variant < 0) variant = fits0 ? 0 : 1;
+  else if (variant == 0 && !fits0)
+    return fail(-MI355_E_SHAPE, "fp8_gemm: variant %s needs M%%256==0, N%%256==0, K%%256==0", kMx8Variants[0]);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (out_dtype == MI355_F32) return launch_mx8<float, false>(variant, a, nullptr, b, nullptr, c, (int)M, (int)N, (int)K, alpha, s);
+  return launch_mx8<unsigned short, false>(variant, a, nullptr, b, nullptr, c, (int)M, (int)N, (int)K, alpha, s);
 }

@@ -224,6 +224,20 @@ def mxfp8_gemm_out(a, a_scale, b, b_scale, c: Tensor, variant: int = -1) -> Tens
     return c
 
 
+def fp8_gemm_out(a, b, c: Tensor, alpha: float = 1.0, variant: int = -1) -> Tensor:
+    dev = _dev(a, b, c)
+    a, b = a.contiguous(), b.contiguous()
+    _contig_out(c, "fp8_gemm")
+    M, N, K = a.shape[0], b.shape[0], a.shape[1]
+    if tuple(c.shape) != (M, N):
+        raise ValueError(f"fp8_gemm: c is {tuple(c.shape)}, expected {(M, N)}")
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_fp8_gemm(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, float(alpha), _lib.dtype_code(c.dtype),
+                                        variant, _lib.current_stream_ptr(dev))
+    _lib.check(rc, f"fp8_gemm M={M} N={N} K={K} out={c.dtype} variant={variant}")
+    return c
+
+
 def mxfp4_dequant_out(codes: Tensor, scales: Tensor, out: Tensor) -> Tensor:
     dev = _dev(codes, scales, out)
     codes, scales = codes.contiguous(), scales.contiguous()

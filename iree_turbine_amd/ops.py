@@ -344,6 +344,34 @@ class mxfp8_gemm(CustomOp):
 
 
 @CustomOp.register
+class fp8_gemm(CustomOp):
+    """C[M,N] = alpha . A . B^T for E4M3 operands: a [M, K], b [N, K] as torch.float8_e4m3fn or the same bytes as
+    uint8; out_dtype "bfloat16" | "float32".  alpha = the product of the per-tensor scales used when quantising."""
+
+    signature = "fp8_gemm(Tensor a, Tensor b, float alpha, str out_dtype, int variant) -> Tensor"
+
+    def select(self, sel: KernelSelection):
+        a, b = sel.arg_tensor(0), sel.arg_tensor(1)
+        sel.attr_float(2)
+        od = sel.attr_str(3).v
+        sel.attr_int(4)
+        ok = (torch.uint8, torch.float8_e4m3fn)
+        _require(a.t.dim() == 2 and b.t.dim() == 2, "fp8_gemm: a and b must be rank 2")
+        _require(a.t.dtype in ok and b.t.dtype in ok, "fp8_gemm: a and b must be float8_e4m3fn (or its bytes as uint8)")
+        _require(a.t.size(1) == b.t.size(1), f"fp8_gemm: K mismatch, a is {tuple(a.t.shape)}, b is {tuple(b.t.shape)} (b is [N, K])")
+        _require(a.t.size(1) > 0 and a.t.size(1) % 32 == 0, f"fp8_gemm: K={a.t.size(1)} must be a positive multiple of 32")
+        _require(od in ("bfloat16", "float32"), f"fp8_gemm: out_dtype must be 'bfloat16' or 'float32', got {od!r}")
+        _require(a.t.size(0) > 0 and b.t.size(0) > 0, "fp8_gemm: empty operand")
+        a.specialize_all_dims()
+        b.specialize_all_dims()
+        sel.return_new_tensor([a.t.size(0), b.t.size(0)], _OUT_DTYPES[od]).specialize_all_dims()
+
+    def eager_execute(self, a, b, alpha, out_dtype, variant):
+        c = torch.empty((a.shape[0], b.shape[0]), dtype=_OUT_DTYPES[out_dtype], device=a.device)
+        return launch.fp8_gemm_out(a, b, c, alpha, variant)
+
+
+@CustomOp.register
 class mxfp4_dequant(CustomOp):
     """fp32 [rows, K] = E2M1(code) * 2^(scale - 127), computed on the device."""
 

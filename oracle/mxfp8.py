@@ -46,3 +46,12 @@ def mxfp8_gemm_f64(a, a_scale, b, b_scale) -> torch.Tensor:
     da = torch.from_numpy(mxfp8_dequant_ref(a, a_scale)).double()
     db = torch.from_numpy(mxfp8_dequant_ref(b, b_scale)).double()
     return torch.mm(da, db.t())
+
+
+def fp8_gemm_ref(a, b, alpha: float = 1.0) -> torch.Tensor:
+    """alpha . E4M3(a) . E4M3(b)^T in fp32 (no block scales).  a, b: uint8 codes or torch.float8_e4m3fn."""
+    def dec(t):
+        t = t.detach().cpu()
+        t = t.view(torch.uint8) if t.dtype != torch.uint8 else t
+        return torch.from_numpy(E4M3_VALUES[t.numpy()])
+    return alpha * torch.mm(dec(a), dec(b).t())

@@ -131,3 +131,28 @@ def test_mxfp8_contract_errors(dev):
         torch.ops.mi355.mxfp8_gemm(a, s, a, s, "bfloat16", 0)  # tiled kernel needs K % 256 == 0
     with pytest.raises(ValueError):
         torch.ops.mi355.mxfp8_gemm(a, s, a, s, "float16", -1)
+
+
+@pytest.mark.parametrize("shape", [(256, 512, 1024), (100, 70, 96), (1, 1, 32)])
+def test_fp8_gemm_plain(dev, shape):
+    """The GEMM without block scales: torch.float8_e4m3fn operands in, alpha applied to the fp32 sums; equal to
+    the block-scaled kernel with every scale byte 127."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs, mxfp8 as o8
+
+    M, N, K = shape
+    announce(f"fp8_gemm {shape}")
+    a, _, b, _ = inputs.mxfp8_inputs(M, N, K, seed=9)
+    alpha = 0.0625 * 3
+    ref = o8.fp8_gemm_ref(a, b, alpha)
+    got = torch.ops.mi355.fp8_gemm(a.to(dev).view(torch.float8_e4m3fn), b.to(dev).view(torch.float8_e4m3fn), alpha, "float32", -1)
+    assert _rel_err(got.cpu(), ref) < HW_SUM
+    ones_a = torch.full((M, K // 32), 127, dtype=torch.uint8, device=dev)
+    ones_b = torch.full((N, K // 32), 127, dtype=torch.uint8, device=dev)
+    scaled = torch.ops.mi355.mxfp8_gemm(a.to(dev), ones_a, b.to(dev), ones_b, "float32", -1)
+    assert torch.equal(got, alpha * scaled)
+    bf = torch.ops.mi355.fp8_gemm(a.to(dev), b.to(dev), alpha, "bfloat16", -1)
+    assert torch.equal(bf, got.bfloat16())
+    # against torch's own decode of the same bytes
+    lib = alpha * (a.view(torch.float8_e4m3fn).float() @ b.view(torch.float8_e4m3fn).float().t())
+    assert _rel_err(got.cpu(), lib) < HW_SUM

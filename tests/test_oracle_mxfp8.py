@@ -54,3 +54,11 @@ def test_gemm_oracle_exact_and_vs_float64():
     assert torch.equal(c2, 2 * c32)
     # inputs never hold a NaN code
     assert not (((A & 0x7F) == 0x7F).any() or ((B & 0x7F) == 0x7F).any())
+
+
+def test_plain_fp8_gemm_oracle_vs_torch_decode():
+    A, _, B, _ = inputs.mxfp8_inputs(20, 24, 96, seed=4)
+    ref = o8.fp8_gemm_ref(A, B, 0.5)
+    lib = 0.5 * (A.view(torch.float8_e4m3fn).float() @ B.view(torch.float8_e4m3fn).float().t())
+    assert torch.equal(ref, lib)
+    assert torch.equal(o8.fp8_gemm_ref(A.view(torch.float8_e4m3fn), B, 0.5), ref)
