@@ -49,6 +49,8 @@ MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
     "mxfp4_4096x8192x8192": 2.947e8,
     "mxfp4_32x8192x8192": 3.748e7,
     "mxfp4_quantize_16384x16384": 6.795e8,
+    "paged_prefill": 6.966e8,
+    "mxfp8_4096x8192x8192": 4.834e8,
 }
 
 
