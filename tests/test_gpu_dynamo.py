@@ -83,3 +83,27 @@ def test_compiled_training_step_keeps_attention_in_pytorch(dev):
     for (n, p), (_, r) in zip(model.named_parameters(), ref.named_parameters()):
         scale = r.grad.float().abs().max().item() + 1e-6
         assert (p.grad.float() - r.grad.float()).abs().max().item() <= 2e-2 * scale, n
+
+
+def test_compiled_block_with_inductor_as_nested_backend(dev):
+    """`mi355_inductor`: the same substitution, everything else (norms, activations, residuals) compiled by
+    inductor; the custom ops pass through it as opaque calls."""
+    import iree_turbine_amd.dynamo as mdyn
+
+    announce("torch.compile backend=mi355_inductor")
+    torch.manual_seed(3)
+    torch._dynamo.reset()
+    model = Block().to(dev).half().eval()
+    x = torch.randn(2, 192, 512, device=dev).half()
+    with torch.no_grad():
+        want = model(x)
+        mdyn.LAST_SUBSTITUTIONS.clear()
+        try:
+            got = torch.compile(model, backend="mi355_inductor")(x)
+        except Exception as e:  # no code generator for inductor on this installation
+            if "triton" in str(e).lower():
+                pytest.skip(f"inductor cannot generate code here: {str(e)[:100]}")
+            raise
+    torch.cuda.synchronize()
+    assert mdyn.LAST_SUBSTITUTIONS["mm"] == 7 and mdyn.LAST_SUBSTITUTIONS["sdpa"] == 1
+    torch.testing.assert_close(got.float(), want.float(), rtol=1e-2, atol=1e-2)
