@@ -36,13 +36,39 @@ def _hipcc() -> str:
     return exe
 
 
+# Kernels that load into registers with hand-placed waits ("staged") must not spill: the compiler does not know
+# that such a register is still being filled, and a spill would store it before its data has arrived.
+NO_SPILL_KERNELS = ("staged",)
+_USAGE_FLAG = "-Rpass-analysis=kernel-resource-usage"
+
+
+def _check_resource_remarks(stderr: str) -> list[str]:
+    """Returns the remark-free stderr lines; raises if a kernel named in NO_SPILL_KERNELS uses scratch."""
+    rest, name = [], None
+    for line in stderr.splitlines():
+        if _USAGE_FLAG not in line and "remark:" not in line:
+            # the source excerpt and caret lines that follow a remark
+            if name is not None and (line.lstrip().startswith("|") or line.strip()[:1].isdigit() or line.strip() in ("^", "")):
+                continue
+            rest.append(line)
+            continue
+        text = line.split("remark:", 1)[1]
+        if "Function Name:" in text:
+            name = text.split("Function Name:", 1)[1].split("[")[0].strip()
+        elif "ScratchSize" in text and name is not None:
+            scratch = int(text.split(":", 1)[1].split("[")[0].strip())
+            if scratch and any(k in name for k in NO_SPILL_KERNELS):
+                raise RuntimeError(f"kernel {name} spills ({scratch} bytes of scratch per lane); it must fit its registers")
+    return rest
+
+
 def _run(cmd: list[str]) -> None:
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"command failed ({proc.returncode}): {' '.join(cmd)}\n{proc.stdout}\n{proc.stderr}")
     # the host pass warns that it does not know the packed-fp32 feature; that is expected
     noise = ("packed-fp32-ops", "is not a recognized feature")
-    for line in proc.stderr.splitlines():
+    for line in _check_resource_remarks(proc.stderr):
         if line.strip() and not any(n in line for n in noise):
             print(line, file=sys.stderr)
 
@@ -56,7 +82,7 @@ def build_library(verbose: bool = True, save_temps: bool = False) -> Path:
 
     def compile_one(pair):
         src, obj = pair
-        cmd = [hipcc, *HIPCC_FLAGS, "-c", str(CSRC / src), "-o", str(obj)]
+        cmd = [hipcc, *HIPCC_FLAGS, _USAGE_FLAG, "-c", str(CSRC / src), "-o", str(obj)]
         if save_temps:
             cmd += ["-save-temps=obj"]
         _run(cmd)

@@ -538,6 +538,9 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_staged(const half_t* 
   for (int kt = 0; kt < KT; kt += 2) {
     MI355_ST_SLAB(0, 1, kt);
     MI355_ST_SLAB(1, 0, kt + 1);
+    // The loads of the last slabs fetch nothing that is used, and behind the loop the compiler hands their
+    // registers to the epilogue: let them land while the registers still belong to them.
+    if (kt + 2 >= KT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }
 #undef MI355_ST_SLAB
 #undef MI355_ST_GROUP

@@ -941,6 +941,9 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_staged(const uint8_t* __restri
     // odd slab: set 0 carries slab kt+2 and the A scales of group g0+1; reloaded with slab kt+4 and the A scales of g0+2
     MI355_MX_SLAB(1, 0, kt + 1, ca1, cb1, ca0, cb0, as_src, sc_wr, g0 + 2, 0);
     sc_wr ^= 4096;
+    // The loads of the last slabs fetch nothing that is used, and behind the loop the compiler hands their
+    // registers to the epilogue: let them land while the registers still belong to them.
+    if (kt + 2 >= KT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   }
 #undef MI355_MX_SLAB
 #undef MI355_MX_GROUP

@@ -267,9 +267,311 @@ __global__ __launch_bounds__(256) void gemm_mxfp8_generic(const uint8_t* __restr
   }
 }
 
-static const char* kMx8Variants[] = {"tiled_256x256x128_w2x2", "generic_32x128"};
-int mxfp8_variant_count() { return 2; }
-const char* mxfp8_variant_name(int i) { return (i >= 0 && i < 2) ? kMx8Variants[i] : nullptr; }
+// Register-staged form: the two-stage direct-to-LDS ring above has only one slab of loads in flight, and a slab's
+// 32 MFMAs (about 0.85 us) are shorter than a loaded memory system's round trip, so it runs at the speed of
+// the loads.  Here slab s+3 is loaded into VGPRs while slab s computes, slab s+1 is copied from registers into the
+// LDS stage that slab s-1 left, and a slab has one barrier, late in its second k-step.  An 8-bit fragment is 8
+// registers, so fragments are not double buffered: the four B fragments stay for a k-step and each is re-read
+// right behind its last MFMA, the A fragments stream through two registers one row tile ahead.  With 64-cycle
+// MFMAs that leaves every read about three MFMAs of latency.  Scales travel as in the staged MXFP4 kernel: a
+// lane owns one row and fetches the 8 scale bytes of two slabs, A rows with the even slabs, B rows with the odd
+// ones, through four 4 KiB LDS buffers (A / B, group parity) that hold every slab's scale dword twice, plain
+// and rotated by 16 bits, so that both lane halves find their two bytes where op_sel looks for them.
+// Loads into registers are inline assembly with hand-placed waits, which the compiler cannot see through: the
+// kernel must not spill (a register would be stored before its data has arrived; the build checks that).
+template <typename OutT, bool SCALED>
+__global__ __launch_bounds__(256) void gemm_mxfp8_staged(const uint8_t* __restrict__ A, const uint8_t* __restrict__ As,
+                                                         const uint8_t* __restrict__ B, const uint8_t* __restrict__ Bs,
+                                                         OutT* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n,
+                                                         int group_m, float alpha) {
+  constexpr int BM = 256, BN = 256, WN = 2, NW = 4;
+  constexpr int WTM = 128, WTN = 128, TM = 4, TN = 4;
+  // LDS, per operand and stage: eight planes, one per 16-byte chunk of the slab's 128-byte rows, each 256 rows x 16
+  // bytes plus 32 bytes of padding.  A fragment read is 16 consecutive rows of one plane (conflict free), the
+  // chunk a lane wants is a constant plane offset, and the padding spreads the 8 chunks x 2 rows that 16 lanes
+  // of a staging write carry over all banks.  Order: A stage 0, A stage 1, B stage 0, B stage 1, so that one
+  // address register per operand reaches both stages through the 16-bit instruction offset; then the scale
+  // buffers A parity 0, A parity 1, B parity 0, B parity 1, 4 KiB each.
+  constexpr int PL = 256 * 16 + 32, OP_BYTES = 8 * PL, B_OFF = 2 * OP_BYTES;
+  constexpr int SC_OFF = 17 * 8192;
+  static_assert(SC_OFF >= 4 * OP_BYTES && SC_OFF % 8192 == 0, "scale buffers behind the data stages; parity is address bit 12");
+  constexpr int NL = SCALED ? 17 : 16;  // loads per slab and lane
+  typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+  typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+  typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  int tile_m, tile_n;
+  map_tile8(blockIdx.x, tiles_m, tiles_n, group_m, tile_m, tile_n);
+
+  const unsigned row_bytes = (unsigned)K;
+  const unsigned sc_bytes = (unsigned)K >> 5;
+  auto make_desc = [&](const uint8_t* base, unsigned bytes) {
+    const unsigned long long p = reinterpret_cast<unsigned long long>(base);
+    i32x4 d;
+    d[0] = __builtin_amdgcn_readfirstlane((int)(unsigned)p);
+    d[1] = __builtin_amdgcn_readfirstlane((int)(unsigned)((p >> 32) & 0xFFFFu));
+    d[2] = __builtin_amdgcn_readfirstlane((int)bytes);
+    d[3] = 0x00020000;
+    return d;
+  };
+  // codes: wave-load i covers rows (i * NW + wave) * 8 .. + 7 of the tile, 8 lanes per 128-byte row piece
+  const int lrow = lane >> 3, lc = lane & 7;
+  const i32x4 a_src = make_desc(A + (size_t)(tile_m * BM + wave * 8) * row_bytes, (unsigned)(BM - wave * 8) * row_bytes);
+  const i32x4 b_src = make_desc(B + (size_t)(tile_n * BN + wave * 8) * row_bytes, (unsigned)(BN - wave * 8) * row_bytes);
+  const unsigned g_off = (unsigned)lrow * row_bytes + (unsigned)lc * 16u;
+  const unsigned row_step = (unsigned)NW * 8u * row_bytes;
+  const int w_off_a = lc * PL + (wave * 8 + lrow) * 16;
+  const int w_off_b = w_off_a + B_OFF;
+  // scales: lane l of wave w owns row 64 w + l of the tile
+  i32x4 as_src = {0, 0, 0, 0}, bs_src = {0, 0, 0, 0};
+  if constexpr (SCALED) {
+    as_src = make_desc(As + (size_t)(tile_m * BM + wave * 64) * sc_bytes, (unsigned)(BM - wave * 64) * sc_bytes);
+    bs_src = make_desc(Bs + (size_t)(tile_n * BN + wave * 64) * sc_bytes, (unsigned)(BN - wave * 64) * sc_bytes);
+  }
+  const unsigned s_off = (unsigned)lane * sc_bytes;
+  int sc_wr = SC_OFF + 4096 + (wave * 64 + lane) * 16;  // where the NEXT group's A scales go (B: + 8192); flips per group
+
+  // staging registers: r[set][n], n < 8 the A row groups, 8..15 the B row groups; rsc[set] the scale row
+  u32x4 r[2][16];
+  u32x2 rsc[2];
+#define MI355_M8_LOAD(S, n, k_off_)                                                                  \
+  asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"                                            \
+               : "=v"(r[S][n])                                                                       \
+               : "v"(g_off), "s"((n) < 8 ? a_src : b_src), "s"((k_off_) + (unsigned)((n)&7) * row_step) \
+               : "memory")
+#define MI355_M8_LOAD_SC(S, desc, group_)                                                                                          \
+  do {                                                                                                                             \
+    if constexpr (SCALED)                                                                                                          \
+      asm volatile("buffer_load_dwordx2 %0, %1, %2, %3 offen" : "=v"(rsc[S]) : "v"(s_off), "s"(desc), "s"((unsigned)(group_)*8u) : "memory"); \
+  } while (0)
+  // `newer` = loads issued after the one that filled the register; they may still be in flight
+#define MI355_M8_WRITE(S, n, newer, st_)                                                                                   \
+  do {                                                                                                                     \
+    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(r[S][n]) : "n"(newer) : "memory");                                           \
+    *reinterpret_cast<u32x4*>(lds + ((n) < 8 ? w_off_a : w_off_b) + ((st_)*OP_BYTES + ((n)&7) * NW * 128)) = r[S][n];        \
+  } while (0)
+#define MI355_M8_WRITE_SC(S, newer, addr_)                                                 \
+  do {                                                                                     \
+    if constexpr (SCALED) {                                                                \
+      asm volatile("s_waitcnt vmcnt(%1)" : "+v"(rsc[S]) : "n"(newer) : "memory");          \
+      *reinterpret_cast<u32x4*>(lds + (addr_)) = both_halves(rsc[S]);                      \
+    }                                                                                      \
+  } while (0)
+
+  // a row's two slab dwords, each followed by itself rotated by 16 bits (what lane half 1 reads)
+  auto both_halves = [](u32x2 d) { return u32x4{d[0], (d[0] >> 16) | (d[0] << 16), d[1], (d[1] >> 16) | (d[1] << 16)}; };
+
+  const int r32 = lane & 31, h = lane >> 5;
+  // lane half h reads chunks 2 ks + h (its half of block ks) and 4 + 2 ks + h (its half of block 2 + ks)
+  const int a_rd = (wm * WTM + r32) * 16 + h * PL;
+  const int b_rd = B_OFF + (wn * WTN + r32) * 16 + h * PL;
+  // scale dwords of the CURRENT group (parity flips per group); + 8 for the group's second slab.  Lane half h takes
+  // the copy whose bytes 0, 1 are blocks 2h, 2h + 1 of the slab: op_sel = ks picks block 2h + ks.
+  int sc_rd_a = SC_OFF + (wm * WTM + r32) * 16 + 4 * h;
+  int sc_rd_b = SC_OFF + 8192 + (wn * WTN + r32) * 16 + 4 * h;
+
+  floatx16 acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; i++)
+#pragma unroll
+    for (int j = 0; j < TM; j++)
+#pragma unroll
+      for (int q = 0; q < 16; q++) acc[i][j][q] = 0.f;
+
+  const int KT = K / 128;  // even, >= 4 (checked on the host)
+  // B fragments stay for a k-step; A fragments stream through two registers sets, one row tile ahead
+  intx8 fa0, fa1, fn[TN];
+  int ca[TM], cb[TN];  // one scale dword per row tile: replaced, like the fragments, right after its last use
+
+  // fragment of k-step ks at constant offset `imm` (stage and row tile) from the operand's address register
+  auto frag = [&](int at, int ks, int imm) {
+    const intx4 lo = *reinterpret_cast<const intx4*>(lds + at + (2 * ks * PL + imm));
+    const intx4 hi = *reinterpret_cast<const intx4*>(lds + at + ((4 + 2 * ks) * PL + imm));
+    return intx8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  };
+  auto scale_dword = [&](int addr) {
+    if constexpr (SCALED) return *reinterpret_cast<const int*>(lds + addr);
+    else return 0x7f7f7f7f;
+  };
+
+#define MI355_M8_LOAD_ALL(S, slab_)                                                                              \
+  do {                                                                                                           \
+    const unsigned ko_ = (unsigned)(slab_)*128u;                                                                 \
+    MI355_M8_LOAD(S, 0, ko_); MI355_M8_LOAD(S, 1, ko_); MI355_M8_LOAD(S, 2, ko_); MI355_M8_LOAD(S, 3, ko_);      \
+    MI355_M8_LOAD(S, 4, ko_); MI355_M8_LOAD(S, 5, ko_); MI355_M8_LOAD(S, 6, ko_); MI355_M8_LOAD(S, 7, ko_);      \
+    MI355_M8_LOAD(S, 8, ko_); MI355_M8_LOAD(S, 9, ko_); MI355_M8_LOAD(S, 10, ko_); MI355_M8_LOAD(S, 11, ko_);    \
+    MI355_M8_LOAD(S, 12, ko_); MI355_M8_LOAD(S, 13, ko_); MI355_M8_LOAD(S, 14, ko_); MI355_M8_LOAD(S, 15, ko_);  \
+  } while (0)
+  // prologue: slab 0 (+ A scales of group 0) -> set 0 -> stage 0; B scales of group 0 through a spare
+  // register; slab 1 (+ B scales of group 1) -> set 1; then slab 2 (+ A scales of group 1) -> set 0
+  const int KG = KT / 2;  // scale groups
+  u32x2 rs;
+  MI355_M8_LOAD_ALL(0, 0);
+  MI355_M8_LOAD_SC(0, as_src, 0);
+  if constexpr (SCALED) asm volatile("buffer_load_dwordx2 %0, %1, %2, 0 offen" : "=v"(rs) : "v"(s_off), "s"(bs_src) : "memory");
+  MI355_M8_LOAD_ALL(1, 1);
+  MI355_M8_LOAD_SC(1, bs_src, KG > 1 ? 1 : 0);
+  // everything older than set 1's loads has landed once at most NL are outstanding
+  MI355_M8_WRITE(0, 0, NL, 0); MI355_M8_WRITE(0, 1, NL, 0); MI355_M8_WRITE(0, 2, NL, 0); MI355_M8_WRITE(0, 3, NL, 0);
+  MI355_M8_WRITE(0, 4, NL, 0); MI355_M8_WRITE(0, 5, NL, 0); MI355_M8_WRITE(0, 6, NL, 0); MI355_M8_WRITE(0, 7, NL, 0);
+  MI355_M8_WRITE(0, 8, NL, 0); MI355_M8_WRITE(0, 9, NL, 0); MI355_M8_WRITE(0, 10, NL, 0); MI355_M8_WRITE(0, 11, NL, 0);
+  MI355_M8_WRITE(0, 12, NL, 0); MI355_M8_WRITE(0, 13, NL, 0); MI355_M8_WRITE(0, 14, NL, 0); MI355_M8_WRITE(0, 15, NL, 0);
+  MI355_M8_WRITE_SC(0, NL, sc_wr - 4096);
+  if constexpr (SCALED) {
+    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(rs) : "n"(NL) : "memory");
+    *reinterpret_cast<u32x4*>(lds + sc_wr - 4096 + 8192) = both_halves(rs);
+  }
+  MI355_M8_LOAD_ALL(0, 2);
+  MI355_M8_LOAD_SC(0, as_src, KG > 1 ? 1 : 0);
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __syncthreads();
+  fa0 = frag(a_rd, 0, 0);
+#pragma unroll
+  for (int j = 0; j < TM; j++) {
+    fn[j] = frag(b_rd, 0, j * 512);
+    ca[j] = scale_dword(sc_rd_a + j * 512);
+    cb[j] = scale_dword(sc_rd_b + j * 512);
+  }
+
+  // Four MFMAs of A row tile j (fragment FA) against the four B fragments; X0..X3 are what follows each of them:
+  // one or two memory instructions, or the re-read of the B fragment just used.
+#define MI355_M8_GROUP(KS, j, FA, X0, X1, X2, X3)                                      \
+  do {                                                                                 \
+    acc[0][j] = mfma_fp8_32x32x64<KS>(fn[0], cb[0], FA, ca[j], acc[0][j]);             \
+    X0;                                                                                \
+    __builtin_amdgcn_sched_barrier(0);                                                 \
+    acc[1][j] = mfma_fp8_32x32x64<KS>(fn[1], cb[1], FA, ca[j], acc[1][j]);             \
+    X1;                                                                                \
+    __builtin_amdgcn_sched_barrier(0);                                                 \
+    acc[2][j] = mfma_fp8_32x32x64<KS>(fn[2], cb[2], FA, ca[j], acc[2][j]);             \
+    X2;                                                                                \
+    __builtin_amdgcn_sched_barrier(0);                                                 \
+    acc[3][j] = mfma_fp8_32x32x64<KS>(fn[3], cb[3], FA, ca[j], acc[3][j]);             \
+    X3;                                                                                \
+    __builtin_amdgcn_sched_barrier(0);                                                 \
+  } while (0)
+#define MI355_NOP ((void)0)
+
+  // Slab kt (scales in ca/cb) sits in stage P; set Q = 1 - P holds slab kt+1 and the scale row SCD travels with
+  // (written to SCW); each register is reloaded with slab kt+3 (the scale row with group GN) soon after it is
+  // written or later in the slab.  In flight when register n is written: the rest of its own round (NL - 1 - n),
+  // the NL loads of the other set and the loads of this slab issued so far.
+  // The one barrier of the slab stands behind the last read of stage P and before the first read of stage Q, in
+  // the last group of k-step 1; the MFMAs around it cover the latency of the reads on both sides.
+  // HALF = 8 if slab kt+1 is the second slab of its group.
+#define MI355_M8_W(Q, n, issued) MI355_M8_WRITE(Q, n, 2 * NL - 1 - (n) + (issued), Q)
+#define MI355_M8_SLAB(P, Q, kt_, SCD, SCW, GN, HALF)                                                                       \
+  do {                                                                                                                     \
+    constexpr int st = P * OP_BYTES, nst = Q * OP_BYTES;                                                                   \
+    const int nxt_ = (kt_) + 3 < KT ? (kt_) + 3 : KT - 1; /* past the end: re-fetch, never used */                         \
+    const unsigned ko = (unsigned)nxt_ * 128u;                                                                             \
+    const int gn_ = (GN) < KG ? (GN) : KG - 1;                                                                             \
+    __builtin_amdgcn_sched_barrier(0);                                                                                     \
+    MI355_M8_GROUP(0, 0, fa0, MI355_M8_W(Q, 0, 0); MI355_M8_W(Q, 1, 0), MI355_M8_W(Q, 2, 0); fa1 = frag(a_rd, 0, st + 512),      \
+                   MI355_M8_W(Q, 3, 0); MI355_M8_W(Q, 4, 0), MI355_M8_W(Q, 5, 0); MI355_M8_LOAD(Q, 0, ko));                 \
+    MI355_M8_GROUP(0, 1, fa1, MI355_M8_W(Q, 6, 1); MI355_M8_W(Q, 7, 1), MI355_M8_W(Q, 8, 1); fa0 = frag(a_rd, 0, st + 2 * 512),  \
+                   MI355_M8_W(Q, 9, 1); MI355_M8_W(Q, 10, 1), MI355_M8_W(Q, 11, 1); MI355_M8_LOAD(Q, 1, ko));               \
+    MI355_M8_GROUP(0, 2, fa0, MI355_M8_W(Q, 12, 2); MI355_M8_W(Q, 13, 2), MI355_M8_W(Q, 14, 2); fa1 = frag(a_rd, 0, st + 3 * 512), \
+                   MI355_M8_W(Q, 15, 2); MI355_M8_WRITE_SC(Q, NL + 2, SCW), MI355_M8_LOAD(Q, 2, ko));                      \
+    MI355_M8_GROUP(0, 3, fa1, fn[0] = frag(b_rd, 1, st); fa0 = frag(a_rd, 1, st),                                          \
+                   MI355_M8_LOAD(Q, 3, ko); fn[1] = frag(b_rd, 1, st + 512), fn[2] = frag(b_rd, 1, st + 2 * 512),          \
+                   fn[3] = frag(b_rd, 1, st + 3 * 512));                                                                   \
+    MI355_M8_GROUP(1, 0, fa0, MI355_M8_LOAD(Q, 4, ko), fa1 = frag(a_rd, 1, st + 512), MI355_M8_LOAD(Q, 5, ko),             \
+                   MI355_M8_LOAD(Q, 6, ko));                                                                               \
+    MI355_M8_GROUP(1, 1, fa1, MI355_M8_LOAD(Q, 7, ko), fa0 = frag(a_rd, 1, st + 2 * 512), MI355_M8_LOAD(Q, 8, ko),         \
+                   MI355_M8_LOAD(Q, 9, ko));                                                                               \
+    MI355_M8_GROUP(1, 2, fa0, MI355_M8_LOAD(Q, 10, ko), fa1 = frag(a_rd, 1, st + 3 * 512), MI355_M8_LOAD(Q, 11, ko),       \
+                   MI355_M8_LOAD(Q, 12, ko));                                                                              \
+    if (HALF == 0) { sc_rd_a ^= 4096; sc_rd_b ^= 4096; }                                                                   \
+    /* the slab's one barrier: behind the last read of stage P, before the first read of stage Q and of new scales */    \
+    MI355_M8_GROUP(1, 3, fa1,                                                                                              \
+                   asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); __builtin_amdgcn_s_barrier();                       \
+                   fa0 = frag(a_rd, 0, nst); fn[0] = frag(b_rd, 0, nst); cb[0] = scale_dword(sc_rd_b + HALF);              \
+                   ca[0] = scale_dword(sc_rd_a + HALF),                                                                    \
+                   MI355_M8_LOAD(Q, 13, ko); fn[1] = frag(b_rd, 0, nst + 512); cb[1] = scale_dword(sc_rd_b + HALF + 512);  \
+                   ca[1] = scale_dword(sc_rd_a + HALF + 512),                                                              \
+                   MI355_M8_LOAD(Q, 14, ko); fn[2] = frag(b_rd, 0, nst + 2 * 512); cb[2] = scale_dword(sc_rd_b + HALF + 1024); \
+                   ca[2] = scale_dword(sc_rd_a + HALF + 1024),                                                             \
+                   MI355_M8_LOAD(Q, 15, ko); MI355_M8_LOAD_SC(Q, SCD, gn_); fn[3] = frag(b_rd, 0, nst + 3 * 512);          \
+                   cb[3] = scale_dword(sc_rd_b + HALF + 1536); ca[3] = scale_dword(sc_rd_a + HALF + 1536));                \
+  } while (0)
+
+  for (int kt = 0; kt < KT; kt += 2) {
+    const int g0 = kt >> 1;
+    // even slab: set 1 carries slab kt+1 and the B scales of group g0+1; reloaded with slab kt+3 and the B scales of g0+2
+    MI355_M8_SLAB(0, 1, kt, bs_src, sc_wr + 8192, g0 + 2, 8);
+    // odd slab: set 0 carries slab kt+2 and the A scales of group g0+1; reloaded with slab kt+4 and the A scales of g0+2
+    MI355_M8_SLAB(1, 0, kt + 1, as_src, sc_wr, g0 + 2, 0);
+    sc_wr ^= 4096;
+    // The loads of the last slabs fetch nothing that is used, and behind the loop the compiler hands their
+    // registers to the epilogue: let them land while the registers still belong to them.
+    if (kt + 2 >= KT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
+#undef MI355_M8_SLAB
+#undef MI355_M8_W
+#undef MI355_M8_GROUP
+#undef MI355_NOP
+#undef MI355_M8_LOAD_ALL
+#undef MI355_M8_WRITE_SC
+#undef MI355_M8_WRITE
+#undef MI355_M8_LOAD_SC
+#undef MI355_M8_LOAD
+  // drain the speculative loads; every wave is past its last fragment read before the epilogue reuses LDS
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  if constexpr (sizeof(OutT) == 2) {
+    // bf16 epilogue through LDS, one wave-private region each, 32 rows per pass: ds_write_b64 of 4 consecutive n
+    // (chunk slot c ^ ((m >> 1) & 7)), whole 256-byte rows read back 16 bytes per lane
+    constexpr int ROW_B = WTN * 2, CH = WTN / 8;
+    char* ep = lds + wave * (32 * ROW_B);
+    constexpr int ROWS_PER_IT = 64 / CH;
+    const int er = lane / CH, ec = lane % CH;
+#pragma unroll
+    for (int j = 0; j < TM; j++) {
+#pragma unroll
+      for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          const int c = i * 4 + q;
+          ushortx4 v = {f32_to_bf16_rne(alpha * acc[i][j][4 * q]), f32_to_bf16_rne(alpha * acc[i][j][4 * q + 1]),
+                        f32_to_bf16_rne(alpha * acc[i][j][4 * q + 2]), f32_to_bf16_rne(alpha * acc[i][j][4 * q + 3])};
+          *reinterpret_cast<ushortx4*>(ep + r32 * ROW_B + ((c ^ ((r32 >> 1) & 7)) * 16) + 8 * h) = v;
+        }
+      OutT* cbase = C + (size_t)(tile_m * BM + wm * WTM + j * 32) * N + tile_n * BN + wn * WTN + ec * 8;
+#pragma unroll
+      for (int it = 0; it < 32 / ROWS_PER_IT; it++) {
+        const int row = it * ROWS_PER_IT + er;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(ep + row * ROW_B + ((ec ^ ((row >> 1) & 7)) * 16));
+        *reinterpret_cast<u32x4*>(cbase + (size_t)row * N) = v;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  } else {
+    const int m0 = tile_m * BM + wm * WTM + r32;
+    const int n0 = tile_n * BN + wn * WTN + 4 * h;
+#pragma unroll
+    for (int j = 0; j < TM; j++) {
+      OutT* crow = C + (size_t)(m0 + j * 32) * N + n0;
+#pragma unroll
+      for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+          Out8<OutT>::store4(crow + i * 32 + q * 8, alpha * acc[i][j][4 * q], alpha * acc[i][j][4 * q + 1], alpha * acc[i][j][4 * q + 2],
+                             alpha * acc[i][j][4 * q + 3]);
+    }
+  }
+}
+
+static const char* kMx8Variants[] = {"tiled_256x256x128_w2x2", "generic_32x128", "staged_256x256x128_w2x2"};
+constexpr int kNumMx8Variants = 3;
+int mxfp8_variant_count() { return kNumMx8Variants; }
+const char* mxfp8_variant_name(int i) { return (i >= 0 && i < kNumMx8Variants) ? kMx8Variants[i] : nullptr; }
 
 template <typename OutT, bool SCALED>
 static int launch_mx8(int variant, const void* a, const void* as, const void* b, const void* bs, void* c, int M, int N, int K,
@@ -292,6 +594,24 @@ static int launch_mx8(int variant, const void* a, const void* as, const void* b,
                        (const uint8_t*)bs, (OutT*)c, M, N, K, tiles_m, tiles_n, 4, alpha);
     return check_launch("gemm_mxfp8_tiled", grid, block, lds_bytes);
   }
+  if (variant == 2) {
+    auto kern = gemm_mxfp8_staged<OutT, SCALED>;
+    constexpr int lds_bytes = 17 * 8192 + 4 * 4096;  // two padded stages per operand, four scale buffers
+    static bool attr_set = false;
+    if (!attr_set) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+      if (e != hipSuccess) {
+        set_error("hipFuncSetAttribute(gemm_mxfp8_staged, %d bytes LDS): %s", lds_bytes, hipGetErrorString(e));
+        return (int)e;
+      }
+      attr_set = true;
+    }
+    const int tiles_m = M / 256, tiles_n = N / 256;
+    dim3 grid(tiles_m * tiles_n), block(256);
+    hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const uint8_t*)a, (const uint8_t*)as, (const uint8_t*)b,
+                       (const uint8_t*)bs, (OutT*)c, M, N, K, tiles_m, tiles_n, 4, alpha);
+    return check_launch("gemm_mxfp8_staged", grid, block, lds_bytes);
+  }
   dim3 grid((N + 127) / 128, (M + 31) / 32), block(256);
   hipLaunchKernelGGL((gemm_mxfp8_generic<OutT, SCALED>), grid, block, 0, stream, (const uint8_t*)a, (const uint8_t*)as,
                      (const uint8_t*)b, (const uint8_t*)bs, (OutT*)c, M, N, K, alpha);
@@ -310,13 +630,17 @@ extern "C" int mi355_mxfp8_gemm(const void* a, const void* a_scale, const void* 
   if (K % 32 != 0) return fail(-MI355_E_SHAPE, "mxfp8_gemm: K=%lld must be a multiple of the 32-element scale block", (long long)K);
   if (out_dtype != MI355_BF16 && out_dtype != MI355_F32)
     return fail(-MI355_E_DTYPE, "mxfp8_gemm: out_dtype %d (want MI355_BF16 or MI355_F32)", out_dtype);
-  if (variant > 1) return fail(-MI355_E_DTYPE, "mxfp8_gemm: variant %d out of range", variant);
+  if (variant >= kNumMx8Variants) return fail(-MI355_E_DTYPE, "mxfp8_gemm: variant %d out of range", variant);
   if (!aligned16(a) || !aligned16(b) || !aligned16(c)) return fail(-MI355_E_ALIGN, "mxfp8_gemm: a, b, c must be 16-byte aligned");
   const bool sc_al4 = ((reinterpret_cast<uintptr_t>(a_scale) | reinterpret_cast<uintptr_t>(b_scale)) & 3u) == 0;
   const bool fits0 = sc_al4 && M % 256 == 0 && N % 256 == 0 && K % 256 == 0 && K >= 256;  // slabs in pairs, one scale dword per slab
-  if (variant < 0) variant = fits0 ? 0 : 1;
+  const bool fits2 = fits0 && K >= 512 && K <= (1 << 23);  // four slabs in flight; 32-bit buffer offsets
+  if (variant < 0) variant = fits2 ? 2 : fits0 ? 0 : 1;
   else if (variant == 0 && !fits0)
     return fail(-MI355_E_SHAPE, "mxfp8_gemm: variant %s needs M%%256==0, N%%256==0, K%%256==0 and 4-byte aligned scales", kMx8Variants[0]);
+  else if (variant == 2 && !fits2)
+    return fail(-MI355_E_SHAPE, "mxfp8_gemm: variant %s needs M%%256==0, N%%256==0, K%%256==0, 512 <= K <= 2^23 and 4-byte aligned scales",
+                kMx8Variants[2]);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (out_dtype == MI355_F32) return launch_mx8<float, true>(variant, a, a_scale, b, b_scale, c, (int)M, (int)N, (int)K, 1.f, s);
   return launch_mx8<unsigned short, true>(variant, a, a_scale, b, b_scale, c, (int)M, (int)N, (int)K, 1.f, s);
@@ -330,13 +654,16 @@ extern "C" int mi355_fp8_gemm(const void* a, const void* b, void* c, int64_t M, 
   if (K % 32 != 0) return fail(-MI355_E_SHAPE, "fp8_gemm: K=%lld must be a multiple of 32", (long long)K);
   if (out_dtype != MI355_BF16 && out_dtype != MI355_F32)
     return fail(-MI355_E_DTYPE, "fp8_gemm: out_dtype %d (want MI355_BF16 or MI355_F32)", out_dtype);
-  if (variant > 1) return fail(-MI355_E_DTYPE, "fp8_gemm: variant %d out of range", variant);
+  if (variant >= kNumMx8Variants) return fail(-MI355_E_DTYPE, "fp8_gemm: variant %d out of range", variant);
   if (!isfinite(alpha)) return fail(-MI355_E_SHAPE, "fp8_gemm: alpha must be finite");
   if (!aligned16(a) || !aligned16(b) || !aligned16(c)) return fail(-MI355_E_ALIGN, "fp8_gemm: a, b, c must be 16-byte aligned");
   const bool fits0 = M % 256 == 0 && N % 256 == 0 && K % 256 == 0 && K >= 256;
-  if (variant < 0) variant = fits0 ? 0 : 1;
+  const bool fits2 = fits0 && K >= 512 && K <= (1 << 23);
+  if (variant < 0) variant = fits2 ? 2 : fits0 ? 0 : 1;
   else if (variant == 0 && !fits0)
     return fail(-MI355_E_SHAPE, "fp8_gemm: variant %s needs M%%256==0, N%%256==0, K%%256==0", kMx8Variants[0]);
+  else if (variant == 2 && !fits2)
+    return fail(-MI355_E_SHAPE, "fp8_gemm: variant %s needs M%%256==0, N%%256==0, K%%256==0 and 512 <= K <= 2^23", kMx8Variants[2]);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (out_dtype == MI355_F32) return launch_mx8<float, false>(variant, a, nullptr, b, nullptr, c, (int)M, (int)N, (int)K, alpha, s);
   return launch_mx8<unsigned short, false>(variant, a, nullptr, b, nullptr, c, (int)M, (int)N, (int)K, alpha, s);

@@ -48,7 +48,7 @@ def test_mxfp8_decode_exhaustive(dev):
         assert np.array_equal(np.signbit(c[:, 0].numpy())[nz], np.signbit(want)[nz]), sc
 
 
-@pytest.mark.parametrize("variant", [-1, 0, 1])
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2])
 def test_mxfp8_gemm_variants(dev, variant):
     import iree_turbine_amd  # noqa: F401
     from oracle import inputs, mxfp8 as o8
@@ -80,13 +80,13 @@ def test_mxfp8_gemm_shapes(dev, shape):
 
 
 def test_mxfp8_one_hot_layout(dev):
-    """A single non-zero element at every k position of a 256-wide row pair: pins which byte of a lane's 32
+    """A single non-zero element at every k position of a 512-wide row: pins which byte of a lane's 32
     belongs to which k and which scale byte goes with which block (a swapped half or block shows up here)."""
     import iree_turbine_amd  # noqa: F401
     from oracle import mxfp8 as o8
 
     announce("mxfp8 one-hot layout")
-    K = 256
+    K = 512
     a = torch.zeros(K, K, dtype=torch.uint8)
     a[torch.arange(K), torch.arange(K)] = 0x38  # row i has 1.0 at k = i
     g = torch.Generator().manual_seed(1)
@@ -94,7 +94,7 @@ def test_mxfp8_one_hot_layout(dev):
     b = torch.randint(0, 256, (256, K), generator=g).to(torch.uint8)
     b = torch.where((b & 0x7F) == 0x7F, b - 1, b)
     bsc = (120 + torch.randint(0, 15, (256, K // 32), generator=g)).to(torch.uint8)
-    for variant in (0, 1):
+    for variant in (0, 1, 2):
         c = torch.ops.mi355.mxfp8_gemm(a.to(dev), asc.to(dev), b.to(dev), bsc.to(dev), "float32", variant).cpu()
         # C[i, n] = 2^(asc[i, i/32] - 127) * dq(B)[n, i]
         db = torch.from_numpy(o8.mxfp8_dequant_ref(b, bsc))
@@ -116,6 +116,32 @@ def test_mxfp8_full_size_cross_variant(dev):
     rows = torch.tensor([0, 255, 256, 1023, M - 1])
     ref = o8.mxfp8_gemm_ref(a[rows.to(dev)].cpu(), asc[rows.to(dev)].cpu(), b.cpu(), bsc.cpu())
     assert _rel_err(tiled[rows.to(dev)].cpu(), ref) < HW_SUM
+    # the register-staged kernel feeds the same block pairs to the same instruction in the same order
+    staged = torch.ops.mi355.mxfp8_gemm(a, asc, b, bsc, "float32", 2)
+    assert torch.equal(staged, tiled)
+    assert torch.equal(staged, torch.ops.mi355.mxfp8_gemm(a, asc, b, bsc, "float32", 2))
+
+
+@pytest.mark.parametrize("out_dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape", [(256, 256, 512), (512, 768, 768), (1024, 512, 1280), (2048, 10240, 512), (256, 512, 8192)])
+def test_mxfp8_staged_slab_rotation(dev, shape, out_dtype):
+    """The register-staged kernel keeps three slabs in flight in two register sets and passes scales through
+    parity buffers per pair of slabs: the minimum of four slabs, slab-pair counts that are odd and even, a grid
+    larger than the chip, a long K -- whole matrix bit-identical to the two-stage kernel, rows against fp32."""
+    import iree_turbine_amd as ita
+    from oracle import inputs, mxfp8 as o8
+
+    M, N, K = shape
+    announce(f"mxfp8 staged {shape} {out_dtype}")
+    names = ita._lib.variants("mxfp8_gemm")
+    v = next(i for i, n in enumerate(names) if n.startswith("staged"))
+    a, asc, b, bsc = [t.to(dev) for t in inputs.mxfp8_inputs(M, N, K, seed=3)]
+    got = torch.ops.mi355.mxfp8_gemm(a, asc, b, bsc, out_dtype, v)
+    assert torch.equal(got, torch.ops.mi355.mxfp8_gemm(a, asc, b, bsc, out_dtype, 0))
+    assert torch.equal(got, torch.ops.mi355.mxfp8_gemm(a, asc, b, bsc, out_dtype, v))
+    rows = torch.tensor([0, 127, 128, M - 1])
+    ref = o8.mxfp8_gemm_ref(a[rows.to(dev)].cpu(), asc[rows.to(dev)].cpu(), b.cpu(), bsc.cpu())
+    assert _rel_err(got[rows.to(dev)].float().cpu(), ref) < (HW_SUM if out_dtype == "float32" else REL)
 
 
 def test_mxfp8_contract_errors(dev):
@@ -131,6 +157,12 @@ def test_mxfp8_contract_errors(dev):
         torch.ops.mi355.mxfp8_gemm(a, s, a, s, "bfloat16", 0)  # tiled kernel needs K % 256 == 0
     with pytest.raises(ValueError):
         torch.ops.mi355.mxfp8_gemm(a, s, a, s, "float16", -1)
+    a = torch.zeros(256, 256, dtype=torch.uint8, device=dev)
+    s = torch.zeros(256, 8, dtype=torch.uint8, device=dev)
+    with pytest.raises(ValueError):
+        torch.ops.mi355.mxfp8_gemm(a, s, a, s, "bfloat16", 2)  # the staged kernel needs four slabs
+    with pytest.raises(ValueError):
+        torch.ops.mi355.mxfp8_gemm(a, s, a, s, "bfloat16", 3)  # no such variant
 
 
 @pytest.mark.parametrize("shape", [(256, 512, 1024), (100, 70, 96), (1, 1, 32)])
@@ -153,6 +185,9 @@ def test_fp8_gemm_plain(dev, shape):
     assert torch.equal(got, alpha * scaled)
     bf = torch.ops.mi355.fp8_gemm(a.to(dev), b.to(dev), alpha, "bfloat16", -1)
     assert torch.equal(bf, got.bfloat16())
+    if M % 256 == 0:  # both tiled kernels, chosen explicitly
+        for variant in (0, 2):
+            assert torch.equal(got, torch.ops.mi355.fp8_gemm(a.to(dev), b.to(dev), alpha, "float32", variant)), variant
     # against torch's own decode of the same bytes
     lib = alpha * (a.view(torch.float8_e4m3fn).float() @ b.view(torch.float8_e4m3fn).float().t())
     assert _rel_err(got.cpu(), lib) < HW_SUM
