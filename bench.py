@@ -49,6 +49,7 @@ MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
     "mxfp4_4096x8192x8192": 2.947e8,
     "mxfp4_32x8192x8192": 3.748e7,
     "mxfp4_quantize_16384x16384": 6.795e8,
+    "mxfp8_quantize_16384x16384": 8.137e8,
     "paged_prefill": 6.966e8,
     "mxfp8_4096x8192x8192": 4.834e8,
 }
@@ -228,6 +229,21 @@ def wl_quantize(rows, K):
     return build
 
 
+def wl_quantize8(rows, K):
+    def build(dev):
+        g = torch.Generator().manual_seed(10)
+        x = (torch.randn(rows, K, generator=g) * 0.1).half()
+        xd = x.to(dev)
+        nbytes = rows * K * (2 + 1 + 1 / 32)
+        return {
+            "fn": lambda: torch.ops.mi355.mxfp8_quantize(xd),
+            "work": nbytes, "bytes": nbytes, "bound": "hbm", "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "dtype": "f16 -> fp8(e4m3)+e8m0", "cpu": lambda: cpu_quantize8(x),
+            "config": {"workload": f"mxfp8_quantize_{rows}x{K}_f16in", "rows": rows, "K": K, "seed": 10},
+        }
+    return build
+
+
 def wl_copy(nbytes=1 << 30):
     """Plain device copy of a known size: the calibration point for the HBM traffic counters."""
     def build(dev):
@@ -255,6 +271,7 @@ WORKLOADS = {
     "mxfp4_4096x8192x8192": wl_mxfp4(4096, 8192, 8192),
     "mxfp4_32x8192x8192": wl_mxfp4(32, 8192, 8192),
     "mxfp4_quantize_16384x16384": wl_quantize(16384, 16384),
+    "mxfp8_quantize_16384x16384": wl_quantize8(16384, 16384),
     "mxfp8_4096x8192x8192": wl_mxfp8(4096, 8192, 8192),
 }
 CALIBRATION = {"copy_1GiB": wl_copy()}  # not part of the path: run only when named with --workload
@@ -286,6 +303,14 @@ def cpu_quantize(x):
     rows = 512
     t = _time_cpu(lambda: om.mxfp4_quantize_ref(x[:rows]), reps=2)
     return {"value": rows * x.shape[1] * (2 + 0.5 + 1 / 32) / t / 1e9, "unit": "GB/s",
+            "sample": f"numpy quantiser on {rows} of the {x.shape[0]} rows, best of 2 after 1 warm-up"}
+
+
+def cpu_quantize8(x):
+    from oracle import mxfp8 as o8
+    rows = 512
+    t = _time_cpu(lambda: o8.mxfp8_quantize_ref(x[:rows]), reps=2)
+    return {"value": rows * x.shape[1] * (2 + 1 + 1 / 32) / t / 1e9, "unit": "GB/s",
             "sample": f"numpy quantiser on {rows} of the {x.shape[0]} rows, best of 2 after 1 warm-up"}
 
 

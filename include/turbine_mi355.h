@@ -249,6 +249,19 @@ int mi355_mxfp4_dequant(const void* codes, const void* scales, float* out,
 int mi355_mxfp4_quantize(const void* x, int in_dtype, int64_t rows, int64_t K,
                          void* codes, void* scales, void* stream);
 
+/*
+ * MXFP8 quantisation, the producer of mi355_mxfp8_gemm's operands: x [rows, K] in
+ * fp16 / bf16 / fp32 -> codes uint8 [rows, K] (OCP E4M3, 8-byte aligned) and
+ * scales uint8 [rows, K/32].  Per block of 32: scale exponent
+ * floor(log2(max|x|)) - 8 clamped to [-127, 127] (all-zero block: -127; a NaN or
+ * infinity in the block: scale 0xFF and signed-zero codes), elements rounded to
+ * the nearest E4M3 value, ties to the even code, saturating at 448 (OCP
+ * Microscaling Formats v1.0).  K % 32 == 0.  As for MXFP4 the reference only
+ * declares the element dtype (iree/turbine/kernel/_support/dtype.py:115,117).
+ */
+int mi355_mxfp8_quantize(const void* x, int in_dtype, int64_t rows, int64_t K,
+                         void* codes, void* scales, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,4 +1,4 @@
-// MXFP4 quantisation for gfx950: x[rows, K] (fp16 / bf16 / fp32) -> E2M1 codes (two per byte, even k in the
+// MXFP4 and MXFP8 quantisation for gfx950 (the fp8 kernel is at the end of the file).  MXFP4: x[rows, K] (fp16 / bf16 / fp32) -> E2M1 codes (two per byte, even k in the
 // low nibble) + one E8M0 scale byte per 32 consecutive k.  This is the producer of the block-scaled GEMM's
 // operands.  OCP Microscaling Formats v1.0 conversion: shared exponent = floor(log2(max |x|)) - 2 per block
 // (clamped to [-127, 127]; an all-zero block takes -127, a block with a NaN or infinity the NaN scale 0xFF),
@@ -176,6 +176,59 @@ __global__ __launch_bounds__(256) void mxfp4_quantize_kernel(const T* __restrict
   }
 }
 
+// MXFP8 (E4M3 codes, one byte per element): the same block walk with the element format's emax of 8 -- shared
+// exponent floor(log2(max |x|)) - 8 -- and values beyond the largest finite code (448) saturating to it.  The
+// scaling by 2^-shared is exact (v_ldexp_f32), the clamp makes every value representable in range, and
+// v_cvt_pk_fp8_f32 rounds to the nearest code, ties to even, subnormal codes included (checked against the
+// brute-force nearest-code search over every fp16 value).
+template <typename T>
+__global__ __launch_bounds__(256) void mxfp8_quantize_kernel(const T* __restrict__ x, uint8_t* __restrict__ codes,
+                                                             uint8_t* __restrict__ scales, long long n_elems) {
+  const int lane = threadIdx.x & 63;
+  const long long wave_id = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const long long e0 = wave_id * 512 + lane * 8;
+  const bool live = e0 < n_elems;
+  QIn<T> in;
+  if (live) in.load(x + e0);
+  else in.zero();
+  unsigned mb = in.amax_bits();
+  unsigned o = __shfl_xor(mb, 1);
+  mb = o > mb ? o : mb;
+  o = __shfl_xor(mb, 2);
+  mb = o > mb ? o : mb;
+  const bool poisoned = mb >= QIn<T>::kInf;
+  const float amax = QIn<T>::bits_to_float(mb);
+  int shared = mb == 0 ? -127 : __builtin_amdgcn_frexp_expf(amax) - 1 - 8;
+  shared = shared < -127 ? -127 : (shared > 127 ? 127 : shared);
+  float v[8];
+  in.to_float(v);
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const float y = __builtin_amdgcn_ldexpf(v[i], -shared);
+    v[i] = poisoned ? __builtin_copysignf(0.f, v[i]) : __builtin_fminf(__builtin_fmaxf(y, -448.f), 448.f);
+  }
+  int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
+  w0 = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], w0, true);
+  int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(v[4], v[5], 0, false);
+  w1 = __builtin_amdgcn_cvt_pk_fp8_f32(v[6], v[7], w1, true);
+  if (live) *reinterpret_cast<intx2*>(codes + e0) = intx2{w0, w1};
+  const int sbyte = poisoned ? 255 : shared + 127;
+  unsigned sw = 0;
+#pragma unroll
+  for (int j = 0; j < 4; j++) sw |= (unsigned)__shfl(sbyte, 16 * (lane & 3) + 4 * j) << (8 * j);
+  if (lane < 4) {
+    const long long b0 = wave_id * 16 + lane * 4;
+    const long long n_blocks = n_elems >> 5;
+    if (b0 + 4 <= n_blocks && ((reinterpret_cast<uintptr_t>(scales) + b0) & 3) == 0) {
+      *reinterpret_cast<unsigned*>(scales + b0) = sw;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        if (b0 + j < n_blocks) scales[b0 + j] = (uint8_t)(sw >> (8 * j));
+    }
+  }
+}
+
 }  // namespace mi355
 
 using namespace mi355;
@@ -202,4 +255,28 @@ extern "C" int mi355_mxfp4_quantize(const void* x, int in_dtype, int64_t rows, i
   else
     hipLaunchKernelGGL(mxfp4_quantize_kernel<float>, grid, block, 0, s, (const float*)x, (uint8_t*)codes, (uint8_t*)scales, n);
   return check_launch("mxfp4_quantize_kernel", grid, block, 0);
+}
+
+extern "C" int mi355_mxfp8_quantize(const void* x, int in_dtype, int64_t rows, int64_t K, void* codes, void* scales,
+                                    void* stream) {
+  if (!x || !codes || !scales) return fail(-MI355_E_NULL, "mxfp8_quantize: null pointer");
+  if (rows <= 0 || K <= 0 || K % 32 != 0 || rows > (1ll << 40) / K)
+    return fail(-MI355_E_SHAPE, "mxfp8_quantize: bad shape rows=%lld K=%lld (K must be a multiple of 32)", (long long)rows,
+                (long long)K);
+  if (in_dtype != MI355_F32 && in_dtype != MI355_F16 && in_dtype != MI355_BF16)
+    return fail(-MI355_E_DTYPE, "mxfp8_quantize: in_dtype %d (want MI355_F32, MI355_F16 or MI355_BF16)", in_dtype);
+  if (!aligned16(x) || (reinterpret_cast<uintptr_t>(codes) & 7u))
+    return fail(-MI355_E_ALIGN, "mxfp8_quantize: x must be 16-byte aligned and codes 8-byte aligned");
+  const long long n = rows * K;
+  const long long waves = (n + 511) / 512;
+  dim3 grid((unsigned)((waves + 3) / 4)), block(256);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (in_dtype == MI355_F16)
+    hipLaunchKernelGGL(mxfp8_quantize_kernel<half_t>, grid, block, 0, s, (const half_t*)x, (uint8_t*)codes, (uint8_t*)scales, n);
+  else if (in_dtype == MI355_BF16)
+    hipLaunchKernelGGL(mxfp8_quantize_kernel<unsigned short>, grid, block, 0, s, (const unsigned short*)x, (uint8_t*)codes,
+                       (uint8_t*)scales, n);
+  else
+    hipLaunchKernelGGL(mxfp8_quantize_kernel<float>, grid, block, 0, s, (const float*)x, (uint8_t*)codes, (uint8_t*)scales, n);
+  return check_launch("mxfp8_quantize_kernel", grid, block, 0);
 }

@@ -266,3 +266,19 @@ def mxfp4_quantize_out(x: Tensor, codes: Tensor, scales: Tensor) -> tuple[Tensor
                                               scales.data_ptr(), _lib.current_stream_ptr(dev))
     _lib.check(rc, f"mxfp4_quantize rows={rows} K={K} in={x.dtype}")
     return codes, scales
+
+
+def mxfp8_quantize_out(x: Tensor, codes: Tensor, scales: Tensor) -> tuple[Tensor, Tensor]:
+    dev = _dev(x, codes, scales)
+    x = x.contiguous()
+    _contig_out(codes, "mxfp8_quantize")
+    _contig_out(scales, "mxfp8_quantize")
+    rows, K = x.shape
+    if tuple(codes.shape) != (rows, K) or tuple(scales.shape) != (rows, K // 32) or codes.dtype != torch.uint8 \
+            or scales.dtype != torch.uint8:
+        raise ValueError("mxfp8_quantize: codes must be uint8 [rows, K] and scales uint8 [rows, K/32]")
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_mxfp8_quantize(x.data_ptr(), _lib.dtype_code(x.dtype), rows, K, codes.data_ptr(),
+                                              scales.data_ptr(), _lib.current_stream_ptr(dev))
+    _lib.check(rc, f"mxfp8_quantize rows={rows} K={K} in={x.dtype}")
+    return codes, scales

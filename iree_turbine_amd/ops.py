@@ -27,6 +27,7 @@ __all__ = [
     "mxfp4_gemm",
     "mxfp4_dequant",
     "mxfp4_quantize",
+    "mxfp8_quantize",
 ]
 
 _OUT_DTYPES = {"float32": torch.float32, "float16": torch.float16, "bfloat16": torch.bfloat16}
@@ -407,3 +408,25 @@ class mxfp4_quantize(CustomOp):
         codes = torch.empty((x.shape[0], x.shape[1] // 2), dtype=torch.uint8, device=x.device)
         scales = torch.empty((x.shape[0], x.shape[1] // 32), dtype=torch.uint8, device=x.device)
         return launch.mxfp4_quantize_out(x, codes, scales)
+
+
+@CustomOp.register
+class mxfp8_quantize(CustomOp):
+    """(codes uint8 [rows, K], scales uint8 [rows, K/32]) of x [rows, K] (fp16, bf16 or fp32): the OCP MX
+    conversion to E4M3 elements -- block exponent floor(log2(max|x|)) - 8, round to nearest, ties to the even
+    code, saturating at 448.  The codes view as torch.float8_e4m3fn."""
+
+    signature = "mxfp8_quantize(Tensor x) -> (Tensor, Tensor)"
+
+    def select(self, sel: KernelSelection):
+        x = sel.arg_tensor(0)
+        _require(x.t.dim() == 2, "mxfp8_quantize: x must be [rows, K]")
+        _require(x.t.dtype in (torch.float16, torch.bfloat16, torch.float32), f"mxfp8_quantize: dtype {x.t.dtype} not supported")
+        _require(x.t.size(0) > 0 and x.t.size(1) > 0 and x.t.size(1) % 32 == 0, "mxfp8_quantize: K must be a positive multiple of 32")
+        sel.return_new_tensor([x.t.size(0), x.t.size(1)], torch.uint8)
+        sel.return_new_tensor([x.t.size(0), x.t.size(1) // 32], torch.uint8)
+
+    def eager_execute(self, x):
+        codes = torch.empty((x.shape[0], x.shape[1]), dtype=torch.uint8, device=x.device)
+        scales = torch.empty((x.shape[0], x.shape[1] // 32), dtype=torch.uint8, device=x.device)
+        return launch.mxfp8_quantize_out(x, codes, scales)

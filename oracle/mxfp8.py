@@ -55,3 +55,37 @@ def fp8_gemm_ref(a, b, alpha: float = 1.0) -> torch.Tensor:
         t = t.view(torch.uint8) if t.dtype != torch.uint8 else t
         return torch.from_numpy(E4M3_VALUES[t.numpy()])
     return alpha * torch.mm(dec(a), dec(b).t())
+
+
+E4M3_EMAX = 8  # exponent of the largest finite E4M3 value, 448 = 1.75 * 2^8
+_POS = E4M3_VALUES[:127].astype(np.float64)  # codes 0x00..0x7E ascend in value; 0x7F is NaN
+
+
+def e4m3_round(y: np.ndarray) -> np.ndarray:
+    """Code (0..0x7E) of the E4M3 value nearest to each non-negative y, by search over the value table: a tie
+    goes to the even code, anything beyond 448 to 448."""
+    y = np.minimum(np.asarray(y, dtype=np.float64), _POS[-1])
+    hi = np.clip(np.searchsorted(_POS, y, side="left"), 1, len(_POS) - 1)
+    lo = hi - 1
+    d_lo, d_hi = y - _POS[lo], _POS[hi] - y
+    pick_hi = (d_hi < d_lo) | ((d_hi == d_lo) & (hi % 2 == 0))
+    return np.where(pick_hi, hi, lo).astype(np.uint8)
+
+
+def mxfp8_quantize_ref(x) -> tuple[np.ndarray, np.ndarray]:
+    """(codes uint8 [rows, K], scales uint8 [rows, K/32]) of a [rows, K] array: OCP MX v1.0 conversion with E4M3
+    elements -- shared exponent floor(log2(max|x|)) - 8 clamped to [-127, 127] (zero block: -127; NaN / infinity
+    in the block: scale 0xFF, signed-zero codes); arithmetic exact in float64."""
+    x = x.detach().cpu().to(torch.float64).numpy() if isinstance(x, torch.Tensor) else np.asarray(x, dtype=np.float64)
+    rows, K = x.shape
+    assert K % BLOCK == 0
+    xb = x.reshape(rows, K // BLOCK, BLOCK)
+    amax = np.abs(xb).max(axis=2)
+    bad = ~np.isfinite(amax)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        _, exp = np.frexp(np.where(bad | (amax == 0), 1.0, amax))
+    shared = np.where(amax == 0, -127, np.clip(exp - 1 - E4M3_EMAX, -127, 127)).astype(np.int64)
+    scales = np.where(bad, 255, shared + 127).astype(np.uint8)
+    y = np.abs(np.ldexp(np.where(bad[:, :, None], 0.0, xb), -shared[:, :, None]))
+    code = e4m3_round(y) | (np.signbit(xb).astype(np.uint8) << 7)
+    return code.reshape(rows, K), scales

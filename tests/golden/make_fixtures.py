@@ -27,6 +27,7 @@ CASES = {
     "mxfp4_gemm": dict(M=64, N=96, K=256, seed=6),
     "mxfp8_gemm": dict(M=64, N=96, K=256, seed=6),
     "mxfp4_quantize": dict(rows=8, K=64, seed=7),
+    "mxfp8_quantize": dict(rows=8, K=64, seed=7),
 }
 
 
@@ -58,6 +59,10 @@ def compute(name: str) -> dict:
     if name == "mxfp4_quantize":
         x = (torch.randn(c["rows"], c["K"], generator=torch.Generator().manual_seed(c["seed"])) * 3).half()
         codes, scales = o4.mxfp4_quantize_ref(x)
+        return {"codes": np.asarray(codes).astype(int).tolist(), "scales": np.asarray(scales).astype(int).tolist()}
+    if name == "mxfp8_quantize":
+        x = (torch.randn(c["rows"], c["K"], generator=torch.Generator().manual_seed(c["seed"])) * 3).half()
+        codes, scales = o8.mxfp8_quantize_ref(x)
         return {"codes": np.asarray(codes).astype(int).tolist(), "scales": np.asarray(scales).astype(int).tolist()}
     raise KeyError(name)
 

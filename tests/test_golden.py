@@ -91,3 +91,8 @@ def test_kernels_match_fixtures(dev):
     x = (torch.randn(c["rows"], c["K"], generator=torch.Generator().manual_seed(c["seed"])) * 3).half().to(dev)
     codes, scales = torch.ops.mi355.mxfp4_quantize(x)
     assert codes.cpu().tolist() == e["codes"] and scales.cpu().tolist() == e["scales"]
+
+    c, e = case("mxfp8_quantize")
+    x = (torch.randn(c["rows"], c["K"], generator=torch.Generator().manual_seed(c["seed"])) * 3).half().to(dev)
+    codes, scales = torch.ops.mi355.mxfp8_quantize(x)
+    assert codes.cpu().tolist() == e["codes"] and scales.cpu().tolist() == e["scales"]

@@ -62,3 +62,42 @@ def test_plain_fp8_gemm_oracle_vs_torch_decode():
     lib = 0.5 * (A.view(torch.float8_e4m3fn).float() @ B.view(torch.float8_e4m3fn).float().t())
     assert torch.equal(ref, lib)
     assert torch.equal(o8.fp8_gemm_ref(A.view(torch.float8_e4m3fn), B, 0.5), ref)
+
+
+def test_quantize_oracle_rounding_vs_torch_library_and_spec_cases():
+    """The nearest-code search against torch's own float -> float8_e4m3fn conversion on every midpoint, every
+    representable value and random magnitudes up to the largest finite value; block exponents by hand."""
+    from oracle import mxfp8 as o8
+
+    g = torch.Generator().manual_seed(0)
+    pos = o8.E4M3_VALUES[:127].astype(np.float64)
+    mids = (pos[:-1] + pos[1:]) / 2
+    y = np.concatenate([pos, mids, np.nextafter(mids.astype(np.float32), 0).astype(np.float64),
+                        np.nextafter(mids.astype(np.float32), 1e9).astype(np.float64),
+                        (torch.rand(50000, generator=g, dtype=torch.float64) * 448).numpy(),
+                        (torch.rand(5000, generator=g, dtype=torch.float64) * 0.04).numpy()])
+    lib = torch.from_numpy(y).float().to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(o8.e4m3_round(y), lib)
+    assert o8.e4m3_round(np.array([449.0, 464.0, 1e6]))[...].tolist() == [0x7E, 0x7E, 0x7E]  # saturation at 448
+    # ties go to the even code: 0.5 * 2^-9 -> 0, 1.5 * 2^-9 -> 2, 17 (between 16 and 18) -> 16 (code 0x58)
+    assert o8.e4m3_round(np.array([2.0 ** -10, 3 * 2.0 ** -10, 17.0])).tolist() == [0, 2, 0x58]
+
+    # block exponent: amax 1.0 -> shared -8 -> 1.0 becomes 256 = 0x78, scale byte 119
+    x = torch.zeros(4, 32)
+    x[0, 0], x[0, 1] = 1.0, -0.5
+    x[1, :] = 0.0
+    x[2, 3] = float("nan")
+    x[2, 4] = -3.0
+    x[3, 0], x[3, 1] = 7.9, 3.0  # 7.9 * 2^6 = 505.6 saturates to 448; 3 * 64 = 192 = 0x74
+    codes, scales = o8.mxfp8_quantize_ref(x)
+    assert scales[:, 0].tolist() == [119, 0, 255, 121]
+    assert codes[0, :2].tolist() == [0x78, 0xF0] and not codes[1].any()
+    assert codes[2, 4] == 0x80 and codes[2, 0] == 0
+    assert codes[3, :2].tolist() == [0x7E, 0x74]
+    # a representable tensor survives the round trip exactly
+    g2 = torch.Generator().manual_seed(4)
+    c0 = torch.randint(0, 256, (16, 64), generator=g2).to(torch.uint8)
+    c0 = torch.where((c0 & 0x7F) == 0x7F, c0 - 1, c0)
+    s0 = (127 + torch.randint(-20, 20, (16, 2), generator=g2)).to(torch.uint8)
+    back = o8.mxfp8_dequant_ref(*o8.mxfp8_quantize_ref(torch.from_numpy(o8.mxfp8_dequant_ref(c0, s0))))
+    assert np.array_equal(back, o8.mxfp8_dequant_ref(c0, s0))
