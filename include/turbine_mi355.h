@@ -219,6 +219,22 @@ int mi355_mxfp8_gemm(const void* a, const void* a_scale, const void* b, const vo
                      int out_dtype, int variant, void* stream);
 
 /*
+ * Block-scaled MXFP6 GEMM: C[M,N] = dq(A) . dq(B)^T, fp32 accumulation, bf16 or fp32 out.
+ * a: uint8 [M, K*3/4], b: uint8 [N, K*3/4] -- OCP 6-bit codes packed as a little-endian bit stream per row:
+ *    element k occupies bits [6k, 6k+6) of the row, a scale block of 32 elements is 24 bytes.
+ *    element_format MI355_FP6_E2M3: sign, 2 exponent bits (bias 1), 3 mantissa bits, values up to 7.5
+ *    (the reference's f6E2M3FN, iree/turbine/kernel/_support/dtype.py:118);
+ *    MI355_FP6_E3M2: sign, 3 exponent bits (bias 3), 2 mantissa bits, values up to 28.  No NaN or infinity codes.
+ * a_scale: uint8 [M, K/32], b_scale: uint8 [N, K/32] -- E8M0, one per 32 consecutive K elements.
+ * dq(x)[r,k] = FP6(code[r,k]) * 2^(scale[r,k/32] - 127).  K % 32 == 0.
+ */
+#define MI355_FP6_E2M3 0
+#define MI355_FP6_E3M2 1
+int mi355_mxfp6_gemm(const void* a, const void* a_scale, const void* b, const void* b_scale,
+                     void* c, int64_t M, int64_t N, int64_t K, int element_format,
+                     int out_dtype, int variant, void* stream);
+
+/*
  * Plain fp8 GEMM (no block scales): C[M,N] = alpha . A . B^T with A [M, K], B [N, K] OCP FP8 E4M3 codes,
  * fp32 accumulation, bf16 or fp32 out; alpha carries the product of the per-tensor scales a caller
  * quantised with.  The kernels of mi355_mxfp8_gemm with every block scale fixed at 2^0.  K % 32 == 0.

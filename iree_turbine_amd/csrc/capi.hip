@@ -39,6 +39,8 @@ int mxfp4_variant_count();
 const char* mxfp4_variant_name(int i);
 int mxfp8_variant_count();
 const char* mxfp8_variant_name(int i);
+int mxfp6_variant_count();
+const char* mxfp6_variant_name(int i);
 
 }  // namespace mi355
 
@@ -54,6 +56,7 @@ extern "C" int mi355_variant_count(const char* family) {
   if (!strcmp(family, "paged_decode")) return decode_variant_count();
   if (!strcmp(family, "mxfp4_gemm")) return mxfp4_variant_count();
   if (!strcmp(family, "mxfp8_gemm")) return mxfp8_variant_count();
+  if (!strcmp(family, "mxfp6_gemm")) return mxfp6_variant_count();
   return 0;
 }
 
@@ -64,5 +67,6 @@ extern "C" const char* mi355_variant_name(const char* family, int i) {
   if (!strcmp(family, "paged_decode")) return decode_variant_name(i);
   if (!strcmp(family, "mxfp4_gemm")) return mxfp4_variant_name(i);
   if (!strcmp(family, "mxfp8_gemm")) return mxfp8_variant_name(i);
+  if (!strcmp(family, "mxfp6_gemm")) return mxfp6_variant_name(i);
   return nullptr;
 }

@@ -224,6 +224,29 @@ def mxfp8_gemm_out(a, a_scale, b, b_scale, c: Tensor, variant: int = -1) -> Tens
     return c
 
 
+FP6_FORMATS = {"e2m3": 0, "e3m2": 1}  # MI355_FP6_E2M3, MI355_FP6_E3M2
+
+
+def mxfp6_gemm_out(a, a_scale, b, b_scale, c: Tensor, element_format: str = "e2m3", variant: int = -1) -> Tensor:
+    dev = _dev(a, a_scale, b, b_scale, c)
+    if element_format not in FP6_FORMATS:
+        raise ValueError(f"mxfp6_gemm: element_format must be one of {sorted(FP6_FORMATS)}, got {element_format!r}")
+    a, a_scale, b, b_scale = a.contiguous(), a_scale.contiguous(), b.contiguous(), b_scale.contiguous()
+    _contig_out(c, "mxfp6_gemm")
+    M, N, K = a.shape[0], b.shape[0], a_scale.shape[1] * 32
+    if tuple(c.shape) != (M, N):
+        raise ValueError(f"mxfp6_gemm: c is {tuple(c.shape)}, expected {(M, N)}")
+    if a.shape[1] * 4 != K * 3 or b.shape[1] * 4 != K * 3 or b_scale.shape[1] * 32 != K:
+        raise ValueError(f"mxfp6_gemm: operands must be uint8 [rows, K*3/4] with scales [rows, K/32]; got a {tuple(a.shape)}, "
+                         f"a_scale {tuple(a_scale.shape)}, b {tuple(b.shape)}, b_scale {tuple(b_scale.shape)}")
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_mxfp6_gemm(a.data_ptr(), a_scale.data_ptr(), b.data_ptr(), b_scale.data_ptr(), c.data_ptr(), M, N,
+                                          K, FP6_FORMATS[element_format], _lib.dtype_code(c.dtype), variant,
+                                          _lib.current_stream_ptr(dev))
+    _lib.check(rc, f"mxfp6_gemm M={M} N={N} K={K} format={element_format} out={c.dtype} variant={variant}")
+    return c
+
+
 def fp8_gemm_out(a, b, c: Tensor, alpha: float = 1.0, variant: int = -1) -> Tensor:
     dev = _dev(a, b, c)
     a, b = a.contiguous(), b.contiguous()

@@ -28,6 +28,7 @@ __all__ = [
     "mxfp4_dequant",
     "mxfp4_quantize",
     "mxfp8_quantize",
+    "mxfp6_gemm",
 ]
 
 _OUT_DTYPES = {"float32": torch.float32, "float16": torch.float16, "bfloat16": torch.bfloat16}
@@ -342,6 +343,38 @@ class mxfp8_gemm(CustomOp):
     def eager_execute(self, a, a_scale, b, b_scale, out_dtype, variant):
         c = torch.empty((a.shape[0], b.shape[0]), dtype=_OUT_DTYPES[out_dtype], device=a.device)
         return launch.mxfp8_gemm_out(a, a_scale, b, b_scale, c, variant)
+
+
+@CustomOp.register
+class mxfp6_gemm(CustomOp):
+    """C[M,N] = dq(A) . dq(B)^T for OCP MXFP6 operands: 6-bit codes packed as a little-endian bit stream, uint8
+    [rows, K*3/4] (element k at bits [6k, 6k+6) of its row), E8M0 scales uint8 [rows, K/32]; element_format
+    "e2m3" (the reference's f6E2M3FN, iree/turbine/kernel/_support/dtype.py:118) | "e3m2"; out_dtype "bfloat16" |
+    "float32"."""
+
+    signature = "mxfp6_gemm(Tensor a, Tensor a_scale, Tensor b, Tensor b_scale, str element_format, str out_dtype, int variant) -> Tensor"
+
+    def select(self, sel: KernelSelection):
+        a, asc, b, bsc = (sel.arg_tensor(i) for i in range(4))
+        fmt = sel.attr_str(4).v
+        od = sel.attr_str(5).v
+        sel.attr_int(6)
+        for name, codes, scales in (("a", a.t, asc.t), ("b", b.t, bsc.t)):
+            _require(codes.dim() == 2 and codes.dtype == torch.uint8, f"mxfp6_gemm: {name} must be uint8 [rows, K*3/4] (packed 6-bit codes)")
+            _require(scales.dim() == 2 and scales.dtype == torch.uint8, f"mxfp6_gemm: {name}_scale must be uint8 [rows, K/32] (E8M0)")
+            _require(scales.size(1) > 0 and codes.size(1) == scales.size(1) * 24 and scales.size(0) == codes.size(0),
+                     f"mxfp6_gemm: {name} {tuple(codes.shape)} and {name}_scale {tuple(scales.shape)} disagree (24 code bytes per scale byte)")
+        _require(a.t.size(1) == b.t.size(1), "mxfp6_gemm: a and b disagree on K")
+        _require(fmt in launch.FP6_FORMATS, f"mxfp6_gemm: element_format must be 'e2m3' or 'e3m2', got {fmt!r}")
+        _require(od in ("bfloat16", "float32"), f"mxfp6_gemm: out_dtype must be 'bfloat16' or 'float32', got {od!r}")
+        _require(a.t.size(0) > 0 and b.t.size(0) > 0, "mxfp6_gemm: empty operand")
+        for d in (a, asc, b, bsc):
+            d.specialize_all_dims()
+        sel.return_new_tensor([a.t.size(0), b.t.size(0)], _OUT_DTYPES[od]).specialize_all_dims()
+
+    def eager_execute(self, a, a_scale, b, b_scale, element_format, out_dtype, variant):
+        c = torch.empty((a.shape[0], b.shape[0]), dtype=_OUT_DTYPES[out_dtype], device=a.device)
+        return launch.mxfp6_gemm_out(a, a_scale, b, b_scale, c, element_format, variant)
 
 
 @CustomOp.register

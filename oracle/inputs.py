@@ -80,3 +80,16 @@ def mxfp8_inputs(M: int, N: int, K: int, seed: int = DEFAULT_SEED, exp_range: in
     b = codes(N)
     b_scale = (127 + torch.randint(-exp_range, exp_range + 1, (N, K // 32), generator=g)).to(torch.uint8)
     return a, a_scale, b, b_scale
+
+
+def mxfp6_inputs(M: int, N: int, K: int, seed: int = DEFAULT_SEED, exp_range: int = 8):
+    """6-bit codes uniform over all 64 (every code is a finite value in both formats), packed four to three
+    bytes, E8M0 scale bytes 127 + U[-exp_range, exp_range].  Draw order: A codes, A scales, B codes, B scales."""
+    from .mxfp6 import pack_fp6
+
+    g = _gen(seed)
+    a = torch.from_numpy(pack_fp6(torch.randint(0, 64, (M, K), generator=g)))
+    a_scale = (127 + torch.randint(-exp_range, exp_range + 1, (M, K // 32), generator=g)).to(torch.uint8)
+    b = torch.from_numpy(pack_fp6(torch.randint(0, 64, (N, K), generator=g)))
+    b_scale = (127 + torch.randint(-exp_range, exp_range + 1, (N, K // 32), generator=g)).to(torch.uint8)
+    return a, a_scale, b, b_scale
