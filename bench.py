@@ -30,6 +30,7 @@ import torch
 PEAK_F16_TFLOPS = 2500.0   # MI355X dense fp16 MFMA
 PEAK_FP4_TFLOPS = 10100.0  # MI355X dense fp4 MFMA
 PEAK_FP8_TFLOPS = 5000.0   # MI355X dense fp8 MFMA
+PEAK_FP6_TFLOPS = 10100.0  # MI355X dense fp6 MFMA (the fp4 rate)
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 
 METRIC = "TFLOP/s & %MFMA peak (f16 GEMM, causal FA, MXFP4 GEMM); decode HBM GB/s"
@@ -52,6 +53,7 @@ MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
     "mxfp8_quantize_16384x16384": 8.137e8,
     "paged_prefill": 6.966e8,
     "mxfp8_4096x8192x8192": 4.834e8,
+    "mxfp6_4096x8192x8192": 3.822e8,
 }
 
 
@@ -214,6 +216,23 @@ def wl_mxfp8(M, N, K):
     return build
 
 
+def wl_mxfp6(M, N, K):
+    from oracle import inputs
+
+    def build(dev):
+        a, asc, b, bsc = inputs.mxfp6_inputs(M, N, K)
+        args = [t.to(dev) for t in (a, asc, b, bsc)]
+        flops = 2.0 * M * N * K
+        nbytes = (M + N) * K * 0.75 + (M + N) * K / 32 + 2.0 * M * N
+        return {
+            "fn": lambda: torch.ops.mi355.mxfp6_gemm(*args, "e2m3", "bfloat16", -1),
+            "work": flops, "bytes": nbytes, "flops": flops, "bound": "mfma", "peak": PEAK_FP6_TFLOPS, "unit": "TFLOP/s",
+            "dtype": "fp6(e2m3)+e8m0", "cpu": lambda: cpu_mxfp6(a, asc, b, bsc, M, N, K),
+            "config": {"workload": f"mxfp6_gemm_{M}x{N}x{K}_bf16out", "M": M, "N": N, "K": K, "seed": 10},
+        }
+    return build
+
+
 def wl_quantize(rows, K):
     def build(dev):
         g = torch.Generator().manual_seed(10)
@@ -273,6 +292,7 @@ WORKLOADS = {
     "mxfp4_quantize_16384x16384": wl_quantize(16384, 16384),
     "mxfp8_quantize_16384x16384": wl_quantize8(16384, 16384),
     "mxfp8_4096x8192x8192": wl_mxfp8(4096, 8192, 8192),
+    "mxfp6_4096x8192x8192": wl_mxfp6(4096, 8192, 8192),
 }
 CALIBRATION = {"copy_1GiB": wl_copy()}  # not part of the path: run only when named with --workload
 WORKLOADS_ALL = {**WORKLOADS, **CALIBRATION}
@@ -357,6 +377,15 @@ def cpu_mxfp4(a, asc, b, bsc, M, N, K):
     flops = 2.0 * rows * cols * K
     return {"value": flops / t / 1e12, "unit": "TFLOP/s",
             "sample": f"table dequantise + torch fp32 matmul of a {rows}x{cols}x{K} corner, best of 3 after 1 warm-up"}
+
+
+def cpu_mxfp6(a, asc, b, bsc, M, N, K):
+    from oracle import mxfp6 as o6
+    rows, cols = min(M, 256), min(N, 2048)
+    t = _time_cpu(lambda: o6.mxfp6_gemm_ref(a[:rows], asc[:rows], b[:cols], bsc[:cols], "e2m3"))
+    flops = 2.0 * rows * cols * K
+    return {"value": flops / t / 1e12, "unit": "TFLOP/s",
+            "sample": f"bit-unpack + table dequantise + torch fp32 matmul of a {rows}x{cols}x{K} corner, best of 3 after 1 warm-up"}
 
 
 def cpu_mxfp8(a, asc, b, bsc, M, N, K):

@@ -71,6 +71,52 @@ def test_mxfp6_gemm_shapes(dev, shape, fmt):
     assert torch.equal(c16, c32.bfloat16())
 
 
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("out_dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape", [(256, 256, 512), (512, 768, 768), (1024, 512, 1280), (2048, 10240, 512), (256, 512, 8192)])
+def test_mxfp6_staged_slab_rotation(dev, shape, out_dtype, fmt):
+    """The register-staged kernel: the minimum of four slabs, odd and even numbers of slab pairs, a grid larger
+    than the chip, a long K -- whole matrix against the any-shape kernel (which pairs blocks differently, so sums
+    agree to the unit's summation error), rows against the fp32 oracle, and bit-identical from launch to launch."""
+    import iree_turbine_amd as ita
+    from oracle import inputs, mxfp6 as o6
+
+    M, N, K = shape
+    announce(f"mxfp6 staged {fmt} {shape} {out_dtype}")
+    names = ita._lib.variants("mxfp6_gemm")
+    v = next(i for i, n in enumerate(names) if n.startswith("staged"))
+    g = next(i for i, n in enumerate(names) if n.startswith("generic"))
+    a, asc, b, bsc = [t.to(dev) for t in inputs.mxfp6_inputs(M, N, K, seed=3)]
+    got = torch.ops.mi355.mxfp6_gemm(a, asc, b, bsc, fmt, out_dtype, v)
+    assert torch.equal(got, torch.ops.mi355.mxfp6_gemm(a, asc, b, bsc, fmt, out_dtype, v))
+    tol = HW_SUM[fmt] if out_dtype == "float32" else REL
+    assert _rel_err(got.float(), torch.ops.mi355.mxfp6_gemm(a, asc, b, bsc, fmt, out_dtype, g).float()) < tol
+    rows = torch.tensor([0, 127, 128, M - 1])
+    ref = o6.mxfp6_gemm_ref(a[rows.to(dev)].cpu(), asc[rows.to(dev)].cpu(), b.cpu(), bsc.cpu(), fmt)
+    assert _rel_err(got[rows.to(dev)].float().cpu(), ref) < tol
+
+
+def test_mxfp6_staged_one_hot(dev):
+    """One-hot rows through the staged kernel: every element position of a slab pair, and the scale byte that goes
+    with it (the kernel pairs blocks 0 / 2 and 1 / 3 of a slab and reads rotated copies of the scale dword)."""
+    import iree_turbine_amd as ita
+    from oracle import inputs, mxfp6 as o6
+
+    announce("mxfp6 staged one-hot")
+    K = 512
+    g = torch.Generator().manual_seed(1)
+    codes = np.zeros((K, K), dtype=np.uint8)
+    codes[np.arange(K), np.arange(K)] = 8
+    asc = (120 + torch.randint(0, 15, (K, K // 32), generator=g)).to(torch.uint8)
+    _, _, b, bsc = inputs.mxfp6_inputs(8, 256, K, seed=2)
+    a = torch.from_numpy(o6.pack_fp6(codes))
+    v = next(i for i, n in enumerate(ita._lib.variants("mxfp6_gemm")) if n.startswith("staged"))
+    c = torch.ops.mi355.mxfp6_gemm(a.to(dev), asc.to(dev), b.to(dev), bsc.to(dev), "e2m3", "float32", v).cpu()
+    db = torch.from_numpy(o6.mxfp6_dequant_ref(b, bsc, "e2m3"))
+    sa = torch.from_numpy(o6.mxfp6_dequant_ref(a, asc, "e2m3"))[torch.arange(K), torch.arange(K)]
+    assert torch.equal(c, sa[:, None] * db.t())
+
+
 def test_mxfp6_one_hot_layout_and_scaling_law(dev):
     """A single non-zero element at every k of a row pins the bit-stream position of every element and the scale
     byte that goes with it; +1 on every A scale byte doubles the result exactly."""
@@ -85,7 +131,7 @@ def test_mxfp6_one_hot_layout_and_scaling_law(dev):
     asc = (120 + torch.randint(0, 15, (K, K // 32), generator=g)).to(torch.uint8)
     _, _, b, bsc = inputs.mxfp6_inputs(8, 96, K, seed=2)
     a = torch.from_numpy(o6.pack_fp6(codes))
-    c = torch.ops.mi355.mxfp6_gemm(a.to(dev), asc.to(dev), b.to(dev), bsc.to(dev), "e2m3", "float32", -1).cpu()
+    c = torch.ops.mi355.mxfp6_gemm(a.to(dev), asc.to(dev), b.to(dev), bsc.to(dev), "e2m3", "float32", 0).cpu()
     db = torch.from_numpy(o6.mxfp6_dequant_ref(b, bsc, "e2m3"))
     sa = torch.from_numpy(o6.mxfp6_dequant_ref(a, asc, "e2m3"))[torch.arange(K), torch.arange(K)]
     assert torch.equal(c, sa[:, None] * db.t())
@@ -109,3 +155,5 @@ def test_mxfp6_contract_errors(dev):
         torch.ops.mi355.mxfp6_gemm(a[:, :16].contiguous(), s, a, s, "e2m3", "bfloat16", -1)  # 16 code bytes for one scale byte
     with pytest.raises(ValueError):
         torch.ops.mi355.mxfp6_gemm(a, s, a, s, "e2m3", "bfloat16", 7)           # no such variant
+    with pytest.raises(ValueError):
+        torch.ops.mi355.mxfp6_gemm(a, s, a, s, "e2m3", "bfloat16", 1)           # the staged kernel needs 256-multiples
