@@ -51,6 +51,7 @@ MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
     "mxfp4_32x8192x8192": 3.748e7,
     "mxfp4_quantize_16384x16384": 6.795e8,
     "mxfp8_quantize_16384x16384": 8.137e8,
+    "mxfp6_quantize_16384x16384": 7.466e8,
     "paged_prefill": 6.966e8,
     "mxfp8_4096x8192x8192": 4.834e8,
     "mxfp6_4096x8192x8192": 3.822e8,
@@ -263,6 +264,21 @@ def wl_quantize8(rows, K):
     return build
 
 
+def wl_quantize6(rows, K):
+    def build(dev):
+        g = torch.Generator().manual_seed(10)
+        x = (torch.randn(rows, K, generator=g) * 0.1).half()
+        xd = x.to(dev)
+        nbytes = rows * K * (2 + 0.75 + 1 / 32)
+        return {
+            "fn": lambda: torch.ops.mi355.mxfp6_quantize(xd, "e2m3"),
+            "work": nbytes, "bytes": nbytes, "bound": "hbm", "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "dtype": "f16 -> fp6(e2m3)+e8m0", "cpu": lambda: cpu_quantize6(x),
+            "config": {"workload": f"mxfp6_quantize_{rows}x{K}_f16in", "rows": rows, "K": K, "seed": 10},
+        }
+    return build
+
+
 def wl_copy(nbytes=1 << 30):
     """Plain device copy of a known size: the calibration point for the HBM traffic counters."""
     def build(dev):
@@ -291,6 +307,7 @@ WORKLOADS = {
     "mxfp4_32x8192x8192": wl_mxfp4(32, 8192, 8192),
     "mxfp4_quantize_16384x16384": wl_quantize(16384, 16384),
     "mxfp8_quantize_16384x16384": wl_quantize8(16384, 16384),
+    "mxfp6_quantize_16384x16384": wl_quantize6(16384, 16384),
     "mxfp8_4096x8192x8192": wl_mxfp8(4096, 8192, 8192),
     "mxfp6_4096x8192x8192": wl_mxfp6(4096, 8192, 8192),
 }
@@ -323,6 +340,14 @@ def cpu_quantize(x):
     rows = 512
     t = _time_cpu(lambda: om.mxfp4_quantize_ref(x[:rows]), reps=2)
     return {"value": rows * x.shape[1] * (2 + 0.5 + 1 / 32) / t / 1e9, "unit": "GB/s",
+            "sample": f"numpy quantiser on {rows} of the {x.shape[0]} rows, best of 2 after 1 warm-up"}
+
+
+def cpu_quantize6(x):
+    from oracle import mxfp6 as o6
+    rows = 512
+    t = _time_cpu(lambda: o6.mxfp6_quantize_ref(x[:rows], "e2m3"), reps=2)
+    return {"value": rows * x.shape[1] * (2 + 0.75 + 1 / 32) / t / 1e9, "unit": "GB/s",
             "sample": f"numpy quantiser on {rows} of the {x.shape[0]} rows, best of 2 after 1 warm-up"}
 
 
@@ -428,8 +453,9 @@ def measure(name: str, dev, steps: int, warmup: int, with_cpu: bool):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=100,
+                    help="untimed launches first; the clocks of an idle GPU take some tens of milliseconds of work to settle")
     ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS_ALL))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-others", action="store_true", help="measure only --workload")

@@ -235,6 +235,17 @@ int mi355_mxfp6_gemm(const void* a, const void* a_scale, const void* b, const vo
                      int out_dtype, int variant, void* stream);
 
 /*
+ * MXFP6 quantisation, the producer of mi355_mxfp6_gemm's operands: x [rows, K] in fp16 / bf16 / fp32 ->
+ * codes uint8 [rows, K*3/4] (8-byte aligned, the bit-stream layout above) and scales uint8 [rows, K/32].
+ * Per block of 32: scale exponent floor(log2(max|x|)) - emax (emax 2 for E2M3, 4 for E3M2) clamped to
+ * [-127, 127] (all-zero block: -127; a NaN or infinity in the block: scale 0xFF and signed-zero codes),
+ * elements rounded to the nearest value, ties to the even code, saturating at the largest value (7.5 / 28)
+ * (OCP Microscaling Formats v1.0).  K % 32 == 0.
+ */
+int mi355_mxfp6_quantize(const void* x, int in_dtype, int64_t rows, int64_t K, int element_format,
+                         void* codes, void* scales, void* stream);
+
+/*
  * Plain fp8 GEMM (no block scales): C[M,N] = alpha . A . B^T with A [M, K], B [N, K] OCP FP8 E4M3 codes,
  * fp32 accumulation, bf16 or fp32 out; alpha carries the product of the per-tensor scales a caller
  * quantised with.  The kernels of mi355_mxfp8_gemm with every block scale fixed at 2^0.  K % 32 == 0.

@@ -39,7 +39,10 @@ __global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int split = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
   const int num_q_heads = num_kv_heads * G;
-  const int L = seq_lens[seq];
+  // a length beyond what the block table can address is cut to the table's reach
+  const int max_tokens = (max_pages_per_seq << page_shift) * 16;
+  const int L_in = seq_lens[seq];
+  const int L = L_in < 0 ? 0 : (L_in > max_tokens ? max_tokens : L_in);
   // sliding window: only the last `window` tokens take part (window <= 0: all of them); pages wholly in
   // front of the window are never touched and the splits divide the pages that remain
   const int lo = (window > 0 && L > window) ? L - window : 0;
@@ -293,6 +296,7 @@ static int check_decode_args(const char* fn, int64_t num_seqs, int64_t hq, int64
   if (G != 1 && G != 2 && G != 4 && G != 8 && G != 16)
     return fail(-MI355_E_SHAPE, "%s: q heads per kv head = %lld, supported: 1, 2, 4, 8, 16", fn, (long long)G);
   if (num_splits < 1 || num_splits > 1024) return fail(-MI355_E_SHAPE, "%s: num_splits %lld out of range [1, 1024]", fn, (long long)num_splits);
+  if (max_pages > (1 << 22)) return fail(-MI355_E_SHAPE, "%s: block table too wide (%lld pages per sequence)", fn, (long long)max_pages);
   if (!(scale > 0.f) || !isfinite(scale)) return fail(-MI355_E_SHAPE, "%s: scale must be positive and finite", fn);
   return 0;
 }

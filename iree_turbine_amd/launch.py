@@ -291,6 +291,24 @@ def mxfp4_quantize_out(x: Tensor, codes: Tensor, scales: Tensor) -> tuple[Tensor
     return codes, scales
 
 
+def mxfp6_quantize_out(x: Tensor, codes: Tensor, scales: Tensor, element_format: str = "e2m3") -> tuple[Tensor, Tensor]:
+    dev = _dev(x, codes, scales)
+    if element_format not in FP6_FORMATS:
+        raise ValueError(f"mxfp6_quantize: element_format must be one of {sorted(FP6_FORMATS)}, got {element_format!r}")
+    x = x.contiguous()
+    _contig_out(codes, "mxfp6_quantize")
+    _contig_out(scales, "mxfp6_quantize")
+    rows, K = x.shape
+    if tuple(codes.shape) != (rows, K // 4 * 3) or tuple(scales.shape) != (rows, K // 32) or codes.dtype != torch.uint8 \
+            or scales.dtype != torch.uint8:
+        raise ValueError("mxfp6_quantize: codes must be uint8 [rows, K*3/4] and scales uint8 [rows, K/32]")
+    with torch.cuda.device(dev):
+        rc = _lib.load().mi355_mxfp6_quantize(x.data_ptr(), _lib.dtype_code(x.dtype), rows, K, FP6_FORMATS[element_format],
+                                              codes.data_ptr(), scales.data_ptr(), _lib.current_stream_ptr(dev))
+    _lib.check(rc, f"mxfp6_quantize rows={rows} K={K} in={x.dtype} format={element_format}")
+    return codes, scales
+
+
 def mxfp8_quantize_out(x: Tensor, codes: Tensor, scales: Tensor) -> tuple[Tensor, Tensor]:
     dev = _dev(x, codes, scales)
     x = x.contiguous()

@@ -29,6 +29,7 @@ __all__ = [
     "mxfp4_quantize",
     "mxfp8_quantize",
     "mxfp6_gemm",
+    "mxfp6_quantize",
 ]
 
 _OUT_DTYPES = {"float32": torch.float32, "float16": torch.float16, "bfloat16": torch.bfloat16}
@@ -441,6 +442,30 @@ class mxfp4_quantize(CustomOp):
         codes = torch.empty((x.shape[0], x.shape[1] // 2), dtype=torch.uint8, device=x.device)
         scales = torch.empty((x.shape[0], x.shape[1] // 32), dtype=torch.uint8, device=x.device)
         return launch.mxfp4_quantize_out(x, codes, scales)
+
+
+@CustomOp.register
+class mxfp6_quantize(CustomOp):
+    """(codes uint8 [rows, K*3/4], scales uint8 [rows, K/32]) of x [rows, K] (fp16, bf16 or fp32): the OCP MX
+    conversion to 6-bit elements, element_format "e2m3" | "e3m2" -- block exponent floor(log2(max|x|)) - emax
+    (2 / 4), round to nearest, ties to the even code, saturating at 7.5 / 28; codes packed as mxfp6_gemm reads them."""
+
+    signature = "mxfp6_quantize(Tensor x, str element_format) -> (Tensor, Tensor)"
+
+    def select(self, sel: KernelSelection):
+        x = sel.arg_tensor(0)
+        fmt = sel.attr_str(1).v
+        _require(x.t.dim() == 2, "mxfp6_quantize: x must be [rows, K]")
+        _require(x.t.dtype in (torch.float16, torch.bfloat16, torch.float32), f"mxfp6_quantize: dtype {x.t.dtype} not supported")
+        _require(x.t.size(0) > 0 and x.t.size(1) > 0 and x.t.size(1) % 32 == 0, "mxfp6_quantize: K must be a positive multiple of 32")
+        _require(fmt in launch.FP6_FORMATS, f"mxfp6_quantize: element_format must be 'e2m3' or 'e3m2', got {fmt!r}")
+        sel.return_new_tensor([x.t.size(0), x.t.size(1) // 4 * 3], torch.uint8)
+        sel.return_new_tensor([x.t.size(0), x.t.size(1) // 32], torch.uint8)
+
+    def eager_execute(self, x, element_format):
+        codes = torch.empty((x.shape[0], x.shape[1] // 4 * 3), dtype=torch.uint8, device=x.device)
+        scales = torch.empty((x.shape[0], x.shape[1] // 32), dtype=torch.uint8, device=x.device)
+        return launch.mxfp6_quantize_out(x, codes, scales, element_format)
 
 
 @CustomOp.register

@@ -68,3 +68,37 @@ def mxfp6_gemm_f64(a, a_scale, b, b_scale, fmt: str = "e2m3") -> torch.Tensor:
     da = torch.from_numpy(mxfp6_dequant_ref(a, a_scale, fmt)).double()
     db = torch.from_numpy(mxfp6_dequant_ref(b, b_scale, fmt)).double()
     return torch.mm(da, db.t())
+
+
+EMAX = {"e2m3": 2, "e3m2": 4}  # exponent of the largest value: 7.5 = 1.875 * 2^2, 28 = 1.75 * 2^4
+
+
+def fp6_round(y: np.ndarray, fmt: str) -> np.ndarray:
+    """Magnitude code (0..31) of the value nearest to each non-negative y, by search over the value table: a tie
+    goes to the even code, anything beyond the largest value to the largest value."""
+    pos = FP6_VALUES[fmt][:32].astype(np.float64)
+    y = np.minimum(np.asarray(y, dtype=np.float64), pos[-1])
+    hi = np.clip(np.searchsorted(pos, y, side="left"), 1, 31)
+    lo = hi - 1
+    d_lo, d_hi = y - pos[lo], pos[hi] - y
+    pick_hi = (d_hi < d_lo) | ((d_hi == d_lo) & (hi % 2 == 0))
+    return np.where(pick_hi, hi, lo).astype(np.uint8)
+
+
+def mxfp6_quantize_ref(x, fmt: str = "e2m3") -> tuple[np.ndarray, np.ndarray]:
+    """(packed codes uint8 [rows, K*3/4], scales uint8 [rows, K/32]) of a [rows, K] array: OCP MX v1.0 conversion
+    -- shared exponent floor(log2(max|x|)) - emax clamped to [-127, 127] (zero block: -127; NaN / infinity in the
+    block: scale 0xFF, signed-zero codes); arithmetic exact in float64."""
+    x = x.detach().cpu().to(torch.float64).numpy() if isinstance(x, torch.Tensor) else np.asarray(x, dtype=np.float64)
+    rows, K = x.shape
+    assert K % BLOCK == 0
+    xb = x.reshape(rows, K // BLOCK, BLOCK)
+    amax = np.abs(xb).max(axis=2)
+    bad = ~np.isfinite(amax)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        _, exp = np.frexp(np.where(bad | (amax == 0), 1.0, amax))
+    shared = np.where(amax == 0, -127, np.clip(exp - 1 - EMAX[fmt], -127, 127)).astype(np.int64)
+    scales = np.where(bad, 255, shared + 127).astype(np.uint8)
+    y = np.abs(np.ldexp(np.where(bad[:, :, None], 0.0, xb), -shared[:, :, None]))
+    code = fp6_round(y, fmt) | (np.signbit(xb).astype(np.uint8) << 5)
+    return pack_fp6(code.reshape(rows, K)), scales

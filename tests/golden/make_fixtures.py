@@ -17,7 +17,7 @@ import torch
 ROOT = Path(__file__).resolve().parents[2]
 sys.path.insert(0, str(ROOT))
 
-from oracle import attention as oa, inputs, mxfp4 as o4, mxfp8 as o8, paged_decode as op  # noqa: E402
+from oracle import attention as oa, inputs, mxfp4 as o4, mxfp6 as o6, mxfp8 as o8, paged_decode as op  # noqa: E402
 
 CASES = {
     "gemm_nt": dict(M=96, N=80, K=160, seed=3),
@@ -28,6 +28,8 @@ CASES = {
     "mxfp8_gemm": dict(M=64, N=96, K=256, seed=6),
     "mxfp4_quantize": dict(rows=8, K=64, seed=7),
     "mxfp8_quantize": dict(rows=8, K=64, seed=7),
+    "mxfp6_gemm": dict(M=64, N=96, K=256, seed=6),
+    "mxfp6_quantize": dict(rows=8, K=64, seed=7),
 }
 
 
@@ -64,6 +66,17 @@ def compute(name: str) -> dict:
         x = (torch.randn(c["rows"], c["K"], generator=torch.Generator().manual_seed(c["seed"])) * 3).half()
         codes, scales = o8.mxfp8_quantize_ref(x)
         return {"codes": np.asarray(codes).astype(int).tolist(), "scales": np.asarray(scales).astype(int).tolist()}
+    if name == "mxfp6_gemm":
+        args = inputs.mxfp6_inputs(c["M"], c["N"], c["K"], seed=c["seed"])
+        return {"e2m3": summarise(o6.mxfp6_gemm_ref(*args, "e2m3")), "e3m2": summarise(o6.mxfp6_gemm_ref(*args, "e3m2"))}
+    if name == "mxfp6_quantize":
+        x = (torch.randn(c["rows"], c["K"], generator=torch.Generator().manual_seed(c["seed"])) * 3).half()
+        out = {}
+        for fmt in ("e2m3", "e3m2"):
+            codes, scales = o6.mxfp6_quantize_ref(x, fmt)
+            out[fmt + "_codes"] = np.asarray(codes).astype(int).tolist()
+            out[fmt + "_scales"] = np.asarray(scales).astype(int).tolist()
+        return out
     raise KeyError(name)
 
 

@@ -43,7 +43,9 @@ def test_oracle_reproduces_fixtures(name):
     for key in want:
         if isinstance(want[key], dict):
             assert now[key]["shape"] == want[key]["shape"]
-            np.testing.assert_allclose(np.asarray(now[key]["corner"]), np.asarray(want[key]["corner"]), rtol=1e-6, atol=1e-7)
+            # fp32 matmuls add in an order that depends on the host's core count: allow that much
+            corner = np.asarray(want[key]["corner"])
+            np.testing.assert_allclose(np.asarray(now[key]["corner"]), corner, rtol=1e-5, atol=1e-6 * np.abs(corner).max())
             assert abs(now[key]["sum"] - want[key]["sum"]) <= 1e-6 * want[key]["abs_sum"]
         else:
             assert now[key] == want[key]
@@ -96,3 +98,15 @@ def test_kernels_match_fixtures(dev):
     x = (torch.randn(c["rows"], c["K"], generator=torch.Generator().manual_seed(c["seed"])) * 3).half().to(dev)
     codes, scales = torch.ops.mi355.mxfp8_quantize(x)
     assert codes.cpu().tolist() == e["codes"] and scales.cpu().tolist() == e["scales"]
+
+    c, e = case("mxfp6_gemm")
+    args = [t.to(dev) for t in inputs.mxfp6_inputs(c["M"], c["N"], c["K"], seed=c["seed"])]
+    for fmt in ("e2m3", "e3m2"):
+        scale = e[fmt]["abs_sum"] / (c["M"] * c["N"])
+        _check(torch.ops.mi355.mxfp6_gemm(*args, fmt, "float32", -1), e[fmt], 5e-4, 5e-3 * scale)
+
+    c, e = case("mxfp6_quantize")
+    x = (torch.randn(c["rows"], c["K"], generator=torch.Generator().manual_seed(c["seed"])) * 3).half().to(dev)
+    for fmt in ("e2m3", "e3m2"):
+        codes, scales = torch.ops.mi355.mxfp6_quantize(x, fmt)
+        assert codes.cpu().tolist() == e[fmt + "_codes"] and scales.cpu().tolist() == e[fmt + "_scales"]

@@ -77,6 +77,28 @@ def test_decode_edge_lengths_and_poison(dev):
         assert torch.equal(out[-1], torch.zeros(Hq, D))  # an empty sequence yields zeros
 
 
+@pytest.mark.parametrize("splits", [1, 3])
+def test_decode_lengths_outside_the_table(dev, splits):
+    """A length beyond what the block table addresses is cut to the table's reach, a negative one counts as
+    empty: the table is never read past its end."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs
+
+    announce(f"paged decode out-of-range lengths splits={splits}")
+    q, kc, vc, bt, sl = inputs.paged_decode_inputs(num_seqs=4, num_q_heads=8, num_kv_heads=2, min_len=100, max_len=300, seed=8)
+    width = bt.shape[1]
+    longest = int(sl.argmax())
+    wild, tame = sl.clone(), sl.clone()
+    wild[longest], tame[longest] = 10 ** 6, int((sl[longest] + 15) // 16 * 16)  # its row of the table is full
+    other = (longest + 1) % 4
+    wild[other], tame[other] = -7, 0
+    assert (int(sl[longest]) + 15) // 16 == width
+    got = torch.ops.mi355.paged_decode_attn(*_to(dev, q, kc, vc, bt, wild), 0.0, splits)
+    want = torch.ops.mi355.paged_decode_attn(*_to(dev, q, kc, vc, bt, tame), 0.0, splits)
+    assert torch.equal(got, want)
+    assert torch.equal(got[other].cpu(), torch.zeros(8, 128, dtype=torch.float16))
+
+
 def test_decode_invariances(dev):
     """Independent of the physical page placement and of the number of splits; phase0 + phase1 == fused."""
     import iree_turbine_amd  # noqa: F401

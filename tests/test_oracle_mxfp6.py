@@ -61,3 +61,30 @@ def test_mxfp6_dequant_and_gemm_hand_cases():
         c1 = o6.mxfp6_gemm_f64(a_, as_, b_, bs_, fmt)
         c2 = o6.mxfp6_gemm_f64(a_, as_ + 1, b_, bs_, fmt)
         assert torch.equal(c2, 2 * c1)
+
+
+def test_mxfp6_quantize_oracle_hand_cases():
+    from oracle import mxfp6 as o6
+
+    # rounding: ties to the even code, saturation, subnormal steps (E2M3 step 1/8 below 1, E3M2 step 1/16 below 1/4)
+    assert o6.fp6_round(np.array([0.0, 0.0625, 0.1875, 1.0625, 1.1875, 7.5, 7.75, 100.0, 3.875]), "e2m3").tolist() == [0, 0, 2, 8, 10, 31, 31, 31, 24]
+    assert o6.fp6_round(np.array([0.03125, 0.09375, 0.25, 1.125, 1.375, 28.0, 30.0, 26.0]), "e3m2").tolist() == [0, 2, 4, 12, 14, 31, 31, 30]
+    x = torch.zeros(4, 32)
+    x[0, 0], x[0, 1] = 1.0, -0.5       # amax 1 -> E2M3 shared -2: 1.0 -> 4.0 (code 24), -0.5 -> -2.0 (code 32 + 16)
+    x[2, 3], x[2, 4] = float("inf"), -3.0
+    x[3, 0], x[3, 1] = 7.9, 3.0        # E2M3: shared 0 -> 7.9 saturates to 7.5 (31), 3.0 (code 20)
+    packed, scales = o6.mxfp6_quantize_ref(x, "e2m3")
+    codes = o6.unpack_fp6(packed)
+    assert scales[:, 0].tolist() == [125, 0, 255, 127]
+    assert codes[0, :2].tolist() == [24, 48] and not codes[1].any()
+    assert codes[2, 4] == 32 and codes[2, 3] == 0
+    assert codes[3, :2].tolist() == [31, 20]
+    packed, scales = o6.mxfp6_quantize_ref(x, "e3m2")  # emax 4: amax 1 -> shared -4: 1.0 -> 16 (code 28)
+    assert scales[:, 0].tolist() == [123, 0, 255, 125] and o6.unpack_fp6(packed)[0, 0] == 28
+    # representable tensors survive the round trip exactly
+    g = torch.Generator().manual_seed(4)
+    for fmt in ("e2m3", "e3m2"):
+        c0 = o6.pack_fp6(torch.randint(0, 64, (16, 64), generator=g))
+        s0 = (127 + torch.randint(-20, 20, (16, 2), generator=g)).to(torch.uint8)
+        dq = o6.mxfp6_dequant_ref(c0, s0, fmt)
+        assert np.array_equal(o6.mxfp6_dequant_ref(*o6.mxfp6_quantize_ref(torch.from_numpy(dq), fmt), fmt), dq)
