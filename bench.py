@@ -46,7 +46,7 @@ MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
     "gemm_2048x57344x8192": 3.054e9,
     "fa_causal": 3.428e8,
     "fa_noncausal": 2.686e8,
-    "decode": 1.178e9,
+    "decode": 1.177e9,
     "mxfp4_4096x8192x8192": 2.947e8,
     "mxfp4_32x8192x8192": 3.748e7,
     "mxfp4_quantize_16384x16384": 6.795e8,

@@ -37,7 +37,29 @@ __global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int split = blockIdx.x, kvh = blockIdx.y, seq = blockIdx.z;
+  const int split = blockIdx.x, kvh = blockIdx.y;
+  // Workgroups are dispatched in grid order and a ragged batch ends with whatever is dispatched last: walking
+  // the sequences longest first leaves the short ones for the tail.  Each workgroup finds "the sequence with
+  // rank blockIdx.z" itself -- thread t counts the sequences that come before sequence t -- which costs a
+  // few hundred cached loads for the batch sizes where the tail matters; larger batches keep their order.
+  int seq = blockIdx.z;
+  const int num_seqs = (int)gridDim.z;
+  if (num_seqs > 1 && num_seqs <= PD_WAVES * 64) {
+    int* pick = reinterpret_cast<int*>(lds);
+    const int t = threadIdx.x;
+    if (t < num_seqs) {
+      const int mine = seq_lens[t];
+      int rank = 0;
+      for (int j = 0; j < num_seqs; j++) {
+        const int other = seq_lens[j];
+        rank += (other > mine) || (other == mine && j < t);
+      }
+      if (rank == (int)blockIdx.z) *pick = t;
+    }
+    __syncthreads();
+    seq = *pick;
+    __syncthreads();  // the slot is part of the V ring
+  }
   const int num_q_heads = num_kv_heads * G;
   // a length beyond what the block table can address is cut to the table's reach
   const int max_tokens = (max_pages_per_seq << page_shift) * 16;

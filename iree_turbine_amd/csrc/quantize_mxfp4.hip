@@ -128,44 +128,16 @@ template <> struct QIn<float> {
   }
 };
 
-template <typename T>
-__global__ __launch_bounds__(256) void mxfp4_quantize_kernel(const T* __restrict__ x, uint8_t* __restrict__ codes,
-                                                             uint8_t* __restrict__ scales, long long n_elems) {
-  const int lane = threadIdx.x & 63;
-  const long long wave_id = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
-  const long long e0 = wave_id * 512 + lane * 8;  // first of this lane's 8 elements
-  const bool live = e0 < n_elems;                 // n_elems is a multiple of 32, so a lane is all in or all out
-  QIn<T> in;
-  if (live) in.load(x + e0);
-  else in.zero();
-  // block maximum of |x| over 4 lanes, as a bit pattern: anything at or above infinity poisons the block
-  unsigned mb = in.amax_bits();
-  unsigned o = __shfl_xor(mb, 1);
-  mb = o > mb ? o : mb;
-  o = __shfl_xor(mb, 2);
-  mb = o > mb ? o : mb;
-  const bool poisoned = mb >= QIn<T>::kInf;
-  const float amax = QIn<T>::bits_to_float(mb);
-  // floor(log2(amax)) = frexp exponent - 1 (also right for subnormal inputs)
-  int shared = mb == 0 ? -127 : __builtin_amdgcn_frexp_expf(amax) - 1 - 2;
-  shared = shared < -127 ? -127 : (shared > 127 ? 127 : shared);
-  unsigned packed;
-  if (__builtin_amdgcn_ballot_w64(live && (poisoned || shared < -126)) != 0) {
-    float v[8];
-    in.to_float(v);
-    packed = quantize8_sw(v, shared, poisoned);
-  } else {
-    packed = in.convert(__builtin_amdgcn_ldexpf(1.0f, shared));
-  }
-  if (live) *reinterpret_cast<unsigned*>(codes + (e0 >> 1)) = packed;
-  // scale bytes: block b of the wave lives in lanes 4b..4b+3; lanes 0..3 each gather four of them
-  const int sbyte = poisoned ? 255 : shared + 127;
+// A wave covers QU chunks of 512 elements; all of a lane's loads are issued before any is used, which is what
+// keeps enough bytes in flight to stream at the memory system's rate.
+constexpr int QU = 4;
+
+// scale bytes of one 512-element chunk: block b lives in lanes 4b..4b+3; lanes 0..3 each gather four of them
+__device__ __forceinline__ void store_scales(uint8_t* scales, int sbyte, int lane, long long b0, long long n_blocks) {
   unsigned sw = 0;
 #pragma unroll
   for (int j = 0; j < 4; j++) sw |= (unsigned)__shfl(sbyte, 16 * (lane & 3) + 4 * j) << (8 * j);
   if (lane < 4) {
-    const long long b0 = wave_id * 16 + lane * 4;  // first of this lane's four blocks
-    const long long n_blocks = n_elems >> 5;
     if (b0 + 4 <= n_blocks && ((reinterpret_cast<uintptr_t>(scales) + b0) & 3) == 0) {
       *reinterpret_cast<unsigned*>(scales + b0) = sw;
     } else {
@@ -173,6 +145,46 @@ __global__ __launch_bounds__(256) void mxfp4_quantize_kernel(const T* __restrict
       for (int j = 0; j < 4; j++)
         if (b0 + j < n_blocks) scales[b0 + j] = (uint8_t)(sw >> (8 * j));
     }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void mxfp4_quantize_kernel(const T* __restrict__ x, uint8_t* __restrict__ codes,
+                                                             uint8_t* __restrict__ scales, long long n_elems) {
+  const int lane = threadIdx.x & 63;
+  const long long wave_id = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  QIn<T> in[QU];
+#pragma unroll
+  for (int u = 0; u < QU; u++) {
+    const long long e0 = (wave_id * QU + u) * 512 + lane * 8;  // first of this lane's 8 elements of chunk u
+    if (e0 < n_elems) in[u].load(x + e0);  // n_elems is a multiple of 32, so a lane is all in or all out
+    else in[u].zero();
+  }
+#pragma unroll
+  for (int u = 0; u < QU; u++) {
+    const long long e0 = (wave_id * QU + u) * 512 + lane * 8;
+    const bool live = e0 < n_elems;
+    // block maximum of |x| over 4 lanes, as a bit pattern: anything at or above infinity poisons the block
+    unsigned mb = in[u].amax_bits();
+    unsigned o = __shfl_xor(mb, 1);
+    mb = o > mb ? o : mb;
+    o = __shfl_xor(mb, 2);
+    mb = o > mb ? o : mb;
+    const bool poisoned = mb >= QIn<T>::kInf;
+    const float amax = QIn<T>::bits_to_float(mb);
+    // floor(log2(amax)) = frexp exponent - 1 (also right for subnormal inputs)
+    int shared = mb == 0 ? -127 : __builtin_amdgcn_frexp_expf(amax) - 1 - 2;
+    shared = shared < -127 ? -127 : (shared > 127 ? 127 : shared);
+    unsigned packed;
+    if (__builtin_amdgcn_ballot_w64(live && (poisoned || shared < -126)) != 0) {
+      float v[8];
+      in[u].to_float(v);
+      packed = quantize8_sw(v, shared, poisoned);
+    } else {
+      packed = in[u].convert(__builtin_amdgcn_ldexpf(1.0f, shared));
+    }
+    if (live) *reinterpret_cast<unsigned*>(codes + (e0 >> 1)) = packed;
+    store_scales(scales, poisoned ? 255 : shared + 127, lane, (wave_id * QU + u) * 16 + lane * 4, n_elems >> 5);
   }
 }
 
@@ -186,46 +198,39 @@ __global__ __launch_bounds__(256) void mxfp8_quantize_kernel(const T* __restrict
                                                              uint8_t* __restrict__ scales, long long n_elems) {
   const int lane = threadIdx.x & 63;
   const long long wave_id = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
-  const long long e0 = wave_id * 512 + lane * 8;
-  const bool live = e0 < n_elems;
-  QIn<T> in;
-  if (live) in.load(x + e0);
-  else in.zero();
-  unsigned mb = in.amax_bits();
-  unsigned o = __shfl_xor(mb, 1);
-  mb = o > mb ? o : mb;
-  o = __shfl_xor(mb, 2);
-  mb = o > mb ? o : mb;
-  const bool poisoned = mb >= QIn<T>::kInf;
-  const float amax = QIn<T>::bits_to_float(mb);
-  int shared = mb == 0 ? -127 : __builtin_amdgcn_frexp_expf(amax) - 1 - 8;
-  shared = shared < -127 ? -127 : (shared > 127 ? 127 : shared);
-  float v[8];
-  in.to_float(v);
+  QIn<T> in[QU];
 #pragma unroll
-  for (int i = 0; i < 8; i++) {
-    const float y = __builtin_amdgcn_ldexpf(v[i], -shared);
-    v[i] = poisoned ? __builtin_copysignf(0.f, v[i]) : __builtin_fminf(__builtin_fmaxf(y, -448.f), 448.f);
+  for (int u = 0; u < QU; u++) {
+    const long long e0 = (wave_id * QU + u) * 512 + lane * 8;
+    if (e0 < n_elems) in[u].load(x + e0);
+    else in[u].zero();
   }
-  int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
-  w0 = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], w0, true);
-  int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(v[4], v[5], 0, false);
-  w1 = __builtin_amdgcn_cvt_pk_fp8_f32(v[6], v[7], w1, true);
-  if (live) *reinterpret_cast<intx2*>(codes + e0) = intx2{w0, w1};
-  const int sbyte = poisoned ? 255 : shared + 127;
-  unsigned sw = 0;
 #pragma unroll
-  for (int j = 0; j < 4; j++) sw |= (unsigned)__shfl(sbyte, 16 * (lane & 3) + 4 * j) << (8 * j);
-  if (lane < 4) {
-    const long long b0 = wave_id * 16 + lane * 4;
-    const long long n_blocks = n_elems >> 5;
-    if (b0 + 4 <= n_blocks && ((reinterpret_cast<uintptr_t>(scales) + b0) & 3) == 0) {
-      *reinterpret_cast<unsigned*>(scales + b0) = sw;
-    } else {
+  for (int u = 0; u < QU; u++) {
+    const long long e0 = (wave_id * QU + u) * 512 + lane * 8;
+    const bool live = e0 < n_elems;
+    unsigned mb = in[u].amax_bits();
+    unsigned o = __shfl_xor(mb, 1);
+    mb = o > mb ? o : mb;
+    o = __shfl_xor(mb, 2);
+    mb = o > mb ? o : mb;
+    const bool poisoned = mb >= QIn<T>::kInf;
+    const float amax = QIn<T>::bits_to_float(mb);
+    int shared = mb == 0 ? -127 : __builtin_amdgcn_frexp_expf(amax) - 1 - 8;
+    shared = shared < -127 ? -127 : (shared > 127 ? 127 : shared);
+    float v[8];
+    in[u].to_float(v);
 #pragma unroll
-      for (int j = 0; j < 4; j++)
-        if (b0 + j < n_blocks) scales[b0 + j] = (uint8_t)(sw >> (8 * j));
+    for (int i = 0; i < 8; i++) {
+      const float y = __builtin_amdgcn_ldexpf(v[i], -shared);
+      v[i] = poisoned ? __builtin_copysignf(0.f, v[i]) : __builtin_fminf(__builtin_fmaxf(y, -448.f), 448.f);
     }
+    int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], 0, false);
+    w0 = __builtin_amdgcn_cvt_pk_fp8_f32(v[2], v[3], w0, true);
+    int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(v[4], v[5], 0, false);
+    w1 = __builtin_amdgcn_cvt_pk_fp8_f32(v[6], v[7], w1, true);
+    if (live) *reinterpret_cast<intx2*>(codes + e0) = intx2{w0, w1};
+    store_scales(scales, poisoned ? 255 : shared + 127, lane, (wave_id * QU + u) * 16 + lane * 4, n_elems >> 5);
   }
 }
 
@@ -244,7 +249,7 @@ extern "C" int mi355_mxfp4_quantize(const void* x, int in_dtype, int64_t rows, i
   if (!aligned16(x) || (reinterpret_cast<uintptr_t>(codes) & 3u))
     return fail(-MI355_E_ALIGN, "mxfp4_quantize: x must be 16-byte aligned and codes 4-byte aligned");
   const long long n = rows * K;
-  const long long waves = (n + 511) / 512;
+  const long long waves = (n + 512 * QU - 1) / (512 * QU);
   dim3 grid((unsigned)((waves + 3) / 4)), block(256);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (in_dtype == MI355_F16)
@@ -268,7 +273,7 @@ extern "C" int mi355_mxfp8_quantize(const void* x, int in_dtype, int64_t rows, i
   if (!aligned16(x) || (reinterpret_cast<uintptr_t>(codes) & 7u))
     return fail(-MI355_E_ALIGN, "mxfp8_quantize: x must be 16-byte aligned and codes 8-byte aligned");
   const long long n = rows * K;
-  const long long waves = (n + 511) / 512;
+  const long long waves = (n + 512 * QU - 1) / (512 * QU);
   dim3 grid((unsigned)((waves + 3) / 4)), block(256);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (in_dtype == MI355_F16)
