@@ -267,9 +267,29 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       unit = pid % units;
     }
   }
-  const int b_idx = bh / lay.H, h_idx = bh - b_idx * lay.H, hk_idx = h_idx / lay.group;
+  int b_idx = bh / lay.H;
+  const int h_idx = bh - b_idx * lay.H, hk_idx = h_idx / lay.group;
   int Sk = Sk_arg;
   if constexpr (PAGED) {
+    // Sequences differ in length and workgroups are dispatched in grid order: take the sequences longest first,
+    // so that the short ones make up the tail.  Thread t counts the sequences that come before sequence t.
+    const int num_seqs = BH / lay.H;
+    if (num_seqs > 1 && num_seqs <= 256) {
+      int* pick = reinterpret_cast<int*>(lds);
+      const int t = threadIdx.x;
+      if (t < num_seqs) {
+        const int mine = pg.seq_lens[t];
+        int rank = 0;
+        for (int j = 0; j < num_seqs; j++) {
+          const int other = pg.seq_lens[j];
+          rank += (other > mine) || (other == mine && j < t);
+        }
+        if (rank == b_idx) *pick = t;
+      }
+      __syncthreads();
+      b_idx = __builtin_amdgcn_readfirstlane(*pick);
+      __syncthreads();  // the slot is part of the K ring
+    }
     Sk = __builtin_amdgcn_readfirstlane(pg.seq_lens[b_idx]);
     const int cap = (pg.max_pages * 16) << pg.page_shift;
     Sk = Sk < 0 ? 0 : (Sk > cap ? cap : Sk);
