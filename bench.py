@@ -44,16 +44,17 @@ MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
     "gemm_4096": 2.351e8,
     "gemm_2048x10240x8192": 6.461e8,
     "gemm_2048x57344x8192": 3.054e9,
-    "fa_causal": 3.428e8,
+    "gemm_1024_f32out": 1.684e7,
+    "fa_causal": 3.425e8,
     "fa_noncausal": 2.686e8,
     "decode": 1.177e9,
     "mxfp4_4096x8192x8192": 2.947e8,
     "mxfp4_32x8192x8192": 3.748e7,
-    "mxfp4_quantize_16384x16384": 6.795e8,
-    "mxfp8_quantize_16384x16384": 8.137e8,
+    "mxfp4_quantize_16384x16384": 6.796e8,
+    "mxfp8_quantize_16384x16384": 8.138e8,
     "mxfp6_quantize_16384x16384": 7.466e8,
-    "paged_prefill": 6.966e8,
-    "mxfp8_4096x8192x8192": 4.834e8,
+    "paged_prefill": 6.959e8,
+    "mxfp8_4096x8192x8192": 4.832e8,
     "mxfp6_4096x8192x8192": 3.822e8,
 }
 
@@ -477,8 +478,7 @@ def main() -> int:
             if name == args.workload:
                 continue
             torch.cuda.empty_cache()
-            steps = max(5, min(args.steps, 20))
-            rec = measure(name, dev, steps, min(args.warmup, 3), with_cpu=False)
+            rec = measure(name, dev, args.steps, args.warmup, with_cpu=False)
             rec.pop("config")
             others.append(rec)
 
