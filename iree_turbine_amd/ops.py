@@ -68,6 +68,28 @@ class gemm_nt(CustomOp):
         return launch.gemm_nt_out(a, b, c, variant)
 
 
+def _gemm_nt_setup_context(ctx, inputs, output):
+    a, b, _, _ = inputs
+    ctx.save_for_backward(a, b)
+
+
+def _gemm_nt_backward(ctx, grad):
+    """For C = A . B^T: dA = dC . B and dB = dC^T . A (the formulas of GEMMBackwardA / GEMMBackwardB,
+    iree/turbine/kernel/boo/op_exports/gemm.py:232-269, for the NT layout), each one launch of the same kernel
+    on operands re-laid K-contiguous; gradients come back in fp16 like the operands."""
+    a, b = ctx.saved_tensors
+    g = grad.to(torch.float16)
+    grad_a = grad_b = None
+    if ctx.needs_input_grad[0]:
+        grad_a = torch.ops.mi355.gemm_nt(g.contiguous(), b.t().contiguous(), "float16", -1)      # [M,N] . [K,N]^T
+    if ctx.needs_input_grad[1]:
+        grad_b = torch.ops.mi355.gemm_nt(g.t().contiguous(), a.t().contiguous(), "float16", -1)  # [N,M] . [K,M]^T
+    return grad_a, grad_b, None, None
+
+
+torch.library.register_autograd("mi355::gemm_nt", _gemm_nt_backward, setup_context=_gemm_nt_setup_context)
+
+
 @CustomOp.register
 class flash_attn_fwd(CustomOp):
     """softmax(scale . Q K^T [+ causal mask]) V for q [B,H,Sq,128], k/v [B,Hkv,Sk,128] fp16, H % Hkv == 0

@@ -202,3 +202,29 @@ def test_gemm_staged_contract(dev):
     a = torch.zeros(256, 128, dtype=torch.float16, device=dev)
     with pytest.raises(ValueError):
         torch.ops.mi355.gemm_nt(a, a, "float16", v)  # fewer than four slabs
+
+
+@pytest.mark.parametrize("shape", [(32, 12, 64), (256, 512, 384), (100, 70, 72)])
+@pytest.mark.parametrize("out_dtype", ["float16", "float32"])
+def test_gemm_autograd(dev, shape, out_dtype):
+    """Gradients of the op against torch's own for C = A . B^T (the reference checks its GEMM backward formulas the
+    same way, tests/kernel/boo/op_exports/gemm_backward_test.py:17-83), fp32 reference on the CPU."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs
+
+    M, N, K = shape
+    announce(f"gemm autograd {shape} {out_dtype}")
+    a, b = inputs.gemm_inputs(M, N, K, seed=1)
+    w = torch.randn(M, N, generator=torch.Generator().manual_seed(2)) * 0.1
+    ar, br = a.float().requires_grad_(True), b.float().requires_grad_(True)
+    ((ar @ br.t()) * w).sum().backward()
+    ad, bd = a.to(dev).requires_grad_(True), b.to(dev).requires_grad_(True)
+    c = torch.ops.mi355.gemm_nt(ad, bd, out_dtype, -1)
+    (c.float() * w.to(dev)).sum().backward()
+    assert ad.grad.dtype == torch.float16 and bd.grad.dtype == torch.float16
+    torch.testing.assert_close(ad.grad.float().cpu(), ar.grad, rtol=RTOL, atol=ATOL)
+    torch.testing.assert_close(bd.grad.float().cpu(), br.grad, rtol=RTOL, atol=ATOL)
+    # only one operand needs a gradient
+    ad2 = a.to(dev).requires_grad_(True)
+    torch.ops.mi355.gemm_nt(ad2, b.to(dev), out_dtype, -1).float().sum().backward()
+    torch.testing.assert_close(ad2.grad.float().cpu(), b.float().sum(dim=0).expand(M, K), rtol=RTOL, atol=ATOL)
