@@ -903,6 +903,7 @@ static const GemmVariant kGemmVariants[] = {
     {"tiled_256x256x64_w2x4", 256, 256, 512},
     {"tiled_128x128x64_w2x2", 128, 128, 256},
     {"staged_256x256x64_w2x2", 256, 256, 256},
+    {"staged_256x256_tail_128x128", 256, 256, 256},
     {"generic_64x64x32", 64, 64, 256},
 };
 constexpr int kNumGemmVariants = sizeof(kGemmVariants) / sizeof(kGemmVariants[0]);
@@ -911,7 +912,9 @@ int gemm_variant_count() { return kNumGemmVariants; }
 const char* gemm_variant_name(int i) { return (i >= 0 && i < kNumGemmVariants) ? kGemmVariants[i].name : nullptr; }
 
 template <int BM, int BN, int WM, int WN, typename OutT, int KIND>  // 0 tiled, 1 pipelined, 2 register-staged
-static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int K, hipStream_t stream) {
+static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int K, int ldc, hipStream_t stream) {
+  // the kernels use their N argument only as the row stride of C, so a column range of a wider C is the
+  // same launch with ldc in its place
   constexpr bool PIPELINED = KIND == 1;
   void (*kern)(const half_t*, const half_t*, OutT*, int, int, int, int, int, int);
   if constexpr (KIND == 2) kern = gemm_f16_nt_staged<BM, BN, WM, WN, OutT>;
@@ -931,7 +934,7 @@ static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int
   const int tiles_m = M / BM, tiles_n = N / BN;
   int group_m = 4;
   dim3 grid(tiles_m * tiles_n), block(WM * WN * 64);
-  hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, M, N, K, tiles_m,
+  hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, M, ldc, K, tiles_m,
                      tiles_n, group_m);
   return check_launch(KIND == 2 ? "gemm_f16_nt_staged" : PIPELINED ? "gemm_f16_nt_pipelined" : "gemm_f16_nt_tiled", grid, block, lds_bytes);
 }
@@ -975,17 +978,49 @@ static int launch_persistent(const void* a, const void* b, void* c, int M, int N
   return check_launch("gemm_f16_nt_persistent", grid, block, lds_bytes);
 }
 
+// Register-staged kernel with a finer-grained last round.  256x256 tiles go to the 256 CUs in rounds; when the
+// last round would leave most CUs idle and its tiles form whole tile columns (or rows) of the grid, that
+// strip is computed by the 128x128 kernel instead (four times the workgroups, so the strip spreads over the
+// whole chip) in a second launch on the same stream.  Shapes that do not split this way run the staged
+// kernel alone.
+static bool tail_split(int M, int N, int& main_m, int& main_n) {
+  const int tm = M / 256, tn = N / 256;
+  const long long t = (long long)tm * tn;
+  const int rem = (int)(t % 256);
+  main_m = M;
+  main_n = N;
+  if (t <= 256 || rem == 0 || rem > 96) return false;  // one round, a full last round, or one that is busy enough
+  if (rem % tm == 0) main_n = N - (rem / tm) * 256;
+  else if (rem % tn == 0) main_m = M - (rem / tn) * 256;
+  else return false;
+  return true;
+}
+
+template <typename OutT>
+static int launch_split(const void* a, const void* b, void* c, int M, int N, int K, hipStream_t stream) {
+  int mm, mn;
+  if (!tail_split(M, N, mm, mn)) return launch_tiled<256, 256, 2, 2, OutT, 2>(a, b, c, M, N, K, N, stream);
+  int rc = launch_tiled<256, 256, 2, 2, OutT, 2>(a, b, c, mm, mn, K, N, stream);
+  if (rc) return rc;
+  const half_t* ah = (const half_t*)a;
+  const half_t* bh = (const half_t*)b;
+  OutT* ch = (OutT*)c;
+  if (mn < N) return launch_tiled<128, 128, 2, 2, OutT, 1>(ah, bh + (size_t)mn * K, ch + mn, M, N - mn, K, N, stream);
+  return launch_tiled<128, 128, 2, 2, OutT, 1>(ah + (size_t)mm * K, bh, ch + (size_t)mm * N, M - mm, N, K, N, stream);
+}
+
 template <typename OutT>
 static int launch_variant(int variant, const void* a, const void* b, void* c, int M, int N, int K, hipStream_t stream) {
   switch (variant) {
     case 0: return launch_persistent<256, 256, 2, 4, OutT>(a, b, c, M, N, K, stream);
     case 1: return launch_persistent<256, 256, 2, 2, OutT>(a, b, c, M, N, K, stream);
-    case 2: return launch_tiled<256, 256, 2, 4, OutT, 1>(a, b, c, M, N, K, stream);
-    case 3: return launch_tiled<256, 256, 2, 2, OutT, 1>(a, b, c, M, N, K, stream);
-    case 4: return launch_tiled<128, 128, 2, 2, OutT, 1>(a, b, c, M, N, K, stream);
-    case 5: return launch_tiled<256, 256, 2, 4, OutT, 0>(a, b, c, M, N, K, stream);
-    case 6: return launch_tiled<128, 128, 2, 2, OutT, 0>(a, b, c, M, N, K, stream);
-    case 7: return launch_tiled<256, 256, 2, 2, OutT, 2>(a, b, c, M, N, K, stream);
+    case 2: return launch_tiled<256, 256, 2, 4, OutT, 1>(a, b, c, M, N, K, N, stream);
+    case 3: return launch_tiled<256, 256, 2, 2, OutT, 1>(a, b, c, M, N, K, N, stream);
+    case 4: return launch_tiled<128, 128, 2, 2, OutT, 1>(a, b, c, M, N, K, N, stream);
+    case 5: return launch_tiled<256, 256, 2, 4, OutT, 0>(a, b, c, M, N, K, N, stream);
+    case 6: return launch_tiled<128, 128, 2, 2, OutT, 0>(a, b, c, M, N, K, N, stream);
+    case 7: return launch_tiled<256, 256, 2, 2, OutT, 2>(a, b, c, M, N, K, N, stream);
+    case 8: return launch_split<OutT>(a, b, c, M, N, K, stream);
     default: {
       dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
       hipLaunchKernelGGL(gemm_f16_nt_generic<OutT>, grid, block, 0, stream, (const half_t*)a, (const half_t*)b, (OutT*)c,
@@ -1011,7 +1046,7 @@ extern "C" int mi355_gemm_f16_nt(const void* a, const void* b, void* c, int64_t 
   auto fits = [&](int v) {
     if (v == kNumGemmVariants - 1) return true;
     if (v <= 1 && (K < 128 || K > (1 << 21))) return false;  // prefetches two slabs ahead; 32-bit byte offsets inside a 256-row panel
-    if (v == 7 && (K < 256 || K % 128 != 0 || K > (1 << 21))) return false;  // slabs in pairs, three in flight
+    if ((v == 7 || v == 8) && (K < 256 || K % 128 != 0 || K > (1 << 21))) return false;  // slabs in pairs, three in flight
     return al && M % kGemmVariants[v].bm == 0 && N % kGemmVariants[v].bn == 0 && K % 64 == 0;
   };
   if (variant < 0) {
@@ -1019,7 +1054,9 @@ extern "C" int mi355_gemm_f16_nt(const void* a, const void* b, void* c, int64_t 
     // 128x128 tile (4x the workgroups) wins; everything else goes to the bounds-checked kernel.
     const long long t256 = (M / 256) * (N / 256);
     const long long rounds = (t256 + 255) / 256;  // 256 CUs, one 256x256 workgroup each
-    if (fits(7) && t256 >= 128) variant = 7;  // measured best on every large shape, also with a ragged last round
+    // the register-staged kernel measured best on every large shape; a sparse last round of 256x256 tiles goes
+    // to the 128x128 kernel when it can be cut off as whole tile columns or rows (+13% at 2048x10240x8192)
+    if (fits(8) && t256 >= 128) variant = 8;
     else if (fits(0) && t256 >= 128 && t256 * 100 >= rounds * 256 * 85) variant = 0;  // >= 85% of the last round busy
     else if (fits(4)) variant = 4;
     else variant = kNumGemmVariants - 1;

@@ -22,7 +22,7 @@ def _run(dev, M, N, K, out_dtype, variant=-1, seed=10):
     return c.float().cpu(), ref
 
 
-@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 3, 4, 5, 6, 7, 8])
 def test_gemm_1024_f32_all_variants(dev, variant):
     c, ref = _run(dev, 1024, 1024, 1024, "float32", variant)
     torch.testing.assert_close(c, ref, rtol=RTOL, atol=ATOL)
@@ -189,6 +189,32 @@ def test_gemm_staged_slab_rotation(dev, shape, out_dtype):
     exact = a[rows.to(dev)].float() @ b.float().t()
     torch.testing.assert_close(got[rows.to(dev)].float(), exact, rtol=RTOL, atol=ATOL)
     assert torch.equal(got, torch.ops.mi355.gemm_nt(a, b, out_dtype, v))
+
+
+@pytest.mark.parametrize("out_dtype", ["float16", "float32"])
+@pytest.mark.parametrize("shape", [(2048, 10240, 512), (10240, 2048, 256), (768, 23296, 256), (2048, 8448, 256)])
+def test_gemm_tail_split(dev, shape, out_dtype):
+    """The staged kernel with its sparse last round handed to the 128x128 kernel: a strip of tile columns
+    (2048 x 10240: 64 of 320 tiles), a strip of tile rows (10240 x 2048), a remainder that is neither (runs
+    unsplit) and the smallest strip (one tile column after a full round of 8 x 32) -- bit-identical to the
+    unsplit staged kernel (both accumulate K in the same order), whole matrix against the generic kernel."""
+    import iree_turbine_amd as ita
+    from oracle import inputs
+
+    M, N, K = shape
+    announce(f"gemm tail split {shape} {out_dtype}")
+    names = ita._lib.variants("gemm_f16_nt")
+    v = next(i for i, n in enumerate(names) if "tail" in n)
+    staged = next(i for i, n in enumerate(names) if n.startswith("staged") and "tail" not in n)
+    a, b = [t.to(dev) for t in inputs.gemm_inputs(M, N, K)]
+    got = torch.ops.mi355.gemm_nt(a, b, out_dtype, v)
+    assert torch.equal(got, torch.ops.mi355.gemm_nt(a, b, out_dtype, staged))
+    assert torch.equal(got, torch.ops.mi355.gemm_nt(a, b, out_dtype, -1))
+    ref = torch.ops.mi355.gemm_nt(a, b, out_dtype, len(names) - 1)
+    torch.testing.assert_close(got.float(), ref.float(), rtol=1e-3, atol=1e-3)
+    rows = torch.tensor([0, 255, M - 256, M - 1])
+    exact = a[rows.to(dev)].float() @ b.float().t()
+    torch.testing.assert_close(got[rows.to(dev)].float(), exact, rtol=RTOL, atol=ATOL)
 
 
 def test_gemm_staged_contract(dev):
