@@ -5,6 +5,7 @@
 #include <stdint.h>
 #include <stdarg.h>
 #include <stdio.h>
+#include <atomic>
 #include "../../include/turbine_mi355.h"
 
 namespace mi355 {
@@ -78,5 +79,21 @@ int fail(int code, const char* fmt, ...);
 int check_launch(const char* kernel, dim3 grid, dim3 block, size_t lds);
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Raises a kernel's dynamic-LDS limit, once per device.  The attribute belongs to the (kernel, device) pair
+// and a process may drive several devices, so `done` -- the call site's own record -- holds one bit per device
+// ordinal; ordinals past 63 set the attribute on every launch.
+inline int allow_lds(const void* kernel, int bytes, std::atomic<uint64_t>& done, const char* name) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev > 63) dev = -1;
+  if (dev >= 0 && ((done.load(std::memory_order_relaxed) >> dev) & 1u)) return 0;
+  hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) {
+    set_error("hipFuncSetAttribute(%s, %d bytes of LDS): %s", name, bytes, hipGetErrorString(e));
+    return (int)e;
+  }
+  if (dev >= 0) done.fetch_or(uint64_t(1) << dev, std::memory_order_relaxed);
+  return 0;
+}
 
 }  // namespace mi355

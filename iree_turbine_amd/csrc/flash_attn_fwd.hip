@@ -597,20 +597,12 @@ static int fa_launch(const void* q, const void* k, const void* v, void* o, int64
   const int BH = (int)(B * H);
   const int q_blocks = (int)((Sq + FA_BLOCK_M - 1) / FA_BLOCK_M);
   const int lds_bytes = 2 * FA_STAGE;
-  static bool attr_set = false;
-  if (!attr_set) {
-    const void* kernels[4] = {reinterpret_cast<const void*>(fa_fwd_d128<true>), reinterpret_cast<const void*>(fa_fwd_d128<false>),
-                              reinterpret_cast<const void*>(fa_fwd_d128_pipe<true, false>),
-                              reinterpret_cast<const void*>(fa_fwd_d128_pipe<false, false>)};
-    for (const void* kp : kernels) {
-      hipError_t e = hipFuncSetAttribute(kp, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-      if (e != hipSuccess) {
-        set_error("hipFuncSetAttribute(fa_fwd_d128): %s", hipGetErrorString(e));
-        return (int)e;
-      }
-    }
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_ok[4] = {};
+  const void* kernels[4] = {reinterpret_cast<const void*>(fa_fwd_d128<true>), reinterpret_cast<const void*>(fa_fwd_d128<false>),
+                            reinterpret_cast<const void*>(fa_fwd_d128_pipe<true, false>),
+                            reinterpret_cast<const void*>(fa_fwd_d128_pipe<false, false>)};
+  for (int i = 0; i < 4; i++)
+    if (int rc = allow_lds(kernels[i], lds_bytes, lds_ok[i], "fa_fwd_d128")) return rc;
   const float scale_log2e = scale * 1.4426950408889634f;
   // the pipelined causal kernel takes a pair of query blocks per workgroup
   const int units = (variant != 1 && is_causal) ? (q_blocks + 1) / 2 : q_blocks;
@@ -693,15 +685,8 @@ extern "C" int mi355_paged_prefill_attn(const void* q, const void* k_cache, cons
   const int q_blocks = (int)((num_new + FA_BLOCK_M - 1) / FA_BLOCK_M);
   const int lds_bytes = 2 * FA_STAGE;
   auto kern = fa_fwd_d128_pipe<true, true>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) {
-      set_error("hipFuncSetAttribute(fa_fwd_d128_pipe paged): %s", hipGetErrorString(e));
-      return (int)e;
-    }
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_ok{0};
+  if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "fa_fwd_d128_pipe")) return rc;
   dim3 grid(BH * ((q_blocks + 1) / 2)), block(256);
   const FaPaged pg{static_cast<const int*>(block_table), static_cast<const int*>(seq_lens), (int)max_pages_per_seq, (int)num_pages,
                    page_shift};

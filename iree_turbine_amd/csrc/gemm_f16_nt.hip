@@ -921,16 +921,8 @@ static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int
   else if constexpr (PIPELINED) kern = gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT>;
   else kern = gemm_f16_nt_tiled<BM, BN, WM, WN, OutT>;
   constexpr int lds_bytes = 2 * (BM + BN) * 128;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       lds_bytes);
-    if (e != hipSuccess) {
-      set_error("hipFuncSetAttribute(gemm_f16_nt, %d bytes LDS): %s", lds_bytes, hipGetErrorString(e));
-      return (int)e;
-    }
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_ok{0};
+  if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt")) return rc;
   const int tiles_m = M / BM, tiles_n = N / BN;
   int group_m = 4;
   dim3 grid(tiles_m * tiles_n), block(WM * WN * 64);
@@ -956,16 +948,8 @@ template <int BM, int BN, int WM, int WN, typename OutT>
 static int launch_persistent(const void* a, const void* b, void* c, int M, int N, int K, hipStream_t stream) {
   auto kern = gemm_f16_nt_persistent<BM, BN, WM, WN, OutT>;
   constexpr int lds_bytes = 2 * (BM + BN) * 128 + WM * WN * 32 * (BN / WN) * 2;  // two stages + one epilogue pass per wave
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       lds_bytes);
-    if (e != hipSuccess) {
-      set_error("hipFuncSetAttribute(gemm_f16_nt_persistent, %d bytes LDS): %s", lds_bytes, hipGetErrorString(e));
-      return (int)e;
-    }
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_ok{0};
+  if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt_persistent")) return rc;
   const int tiles_m = M / BM, tiles_n = N / BN;
   const int T = tiles_m * tiles_n;
   // one workgroup per CU (the LDS footprint allows no more), in multiples of 8 so that a workgroup's tile

@@ -1021,16 +1021,8 @@ static int launch_mx_tiled(const void* a, const void* as, const void* b, const v
                            hipStream_t stream) {
   auto kern = gemm_mxfp4_tiled<BM, BN, WM, WN, OutT, SCALES_LDS>;
   constexpr int lds_bytes = 2 * (BM + BN) * 128 + (SCALES_LDS ? 2 * (BM + BN) * 32 : 0);
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       lds_bytes);
-    if (e != hipSuccess) {
-      set_error("hipFuncSetAttribute(gemm_mxfp4_tiled, %d bytes LDS): %s", lds_bytes, hipGetErrorString(e));
-      return (int)e;
-    }
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_ok{0};
+  if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_mxfp4_tiled")) return rc;
   const int tiles_m = M / BM, tiles_n = N / BN;
   dim3 grid(tiles_m * tiles_n), block(WM * WN * 64);
   hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const uint8_t*)a, (const uint8_t*)as, (const uint8_t*)b,
@@ -1056,16 +1048,8 @@ static int launch_mx_persistent(const void* a, const void* as, const void* b, co
   auto kern = gemm_mxfp4_persistent<BM, BN, WM, WN, OutT>;
   // two data stages, two scale groups of 16 bytes per row, one 2 KiB epilogue pass per wave
   constexpr int lds_bytes = 2 * (BM + BN) * 128 + 2 * (BM + BN) * 16 + WM * WN * 2048;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       lds_bytes);
-    if (e != hipSuccess) {
-      set_error("hipFuncSetAttribute(gemm_mxfp4_persistent, %d bytes LDS): %s", lds_bytes, hipGetErrorString(e));
-      return (int)e;
-    }
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_ok{0};
+  if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_mxfp4_persistent")) return rc;
   const int tiles_m = M / BM, tiles_n = N / BN;
   const int T = tiles_m * tiles_n;
   int g = mx_cu_count() & ~7;  // multiples of 8 keep a workgroup's tiles on the XCD it runs on
@@ -1081,16 +1065,8 @@ static int launch_mx_staged(const void* a, const void* as, const void* b, const 
                             hipStream_t stream) {
   auto kern = gemm_mxfp4_staged<OutT>;
   constexpr int lds_bytes = 2 * 512 * 128 + 4 * 4096;  // two data stages, four scale buffers
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       lds_bytes);
-    if (e != hipSuccess) {
-      set_error("hipFuncSetAttribute(gemm_mxfp4_staged, %d bytes LDS): %s", lds_bytes, hipGetErrorString(e));
-      return (int)e;
-    }
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_ok{0};
+  if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_mxfp4_staged")) return rc;
   const int tiles_m = M / 256, tiles_n = N / 256;
   dim3 grid(tiles_m * tiles_n), block(256);
   hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const uint8_t*)a, (const uint8_t*)as, (const uint8_t*)b,
@@ -1112,15 +1088,8 @@ static int launch_mx(int variant, const void* a, const void* as, const void* b, 
     case 3: {
       auto kern = gemm_mxfp4_skinny<OutT>;
       constexpr int lds_bytes = 8 * 16384;
-      static bool attr_set = false;
-      if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-        if (e != hipSuccess) {
-          set_error("hipFuncSetAttribute(gemm_mxfp4_skinny): %s", hipGetErrorString(e));
-          return (int)e;
-        }
-        attr_set = true;
-      }
+      static std::atomic<uint64_t> lds_ok{0};
+      if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_mxfp4_skinny")) return rc;
       dim3 grid(N / 32), block(512);
       hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const uint8_t*)a, (const uint8_t*)as, (const uint8_t*)b,
                          (const uint8_t*)bs, (OutT*)c, M, N, K);

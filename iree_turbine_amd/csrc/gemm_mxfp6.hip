@@ -399,15 +399,8 @@ static int launch_mx6(int variant, const void* a, const void* as, const void* b,
     {
       auto kern = gemm_mxfp6_staged<OutT, FMT>;
       constexpr int lds_bytes = 13 * 8192 + 4 * 4096;  // two padded stages per operand, four scale buffers
-      static bool attr_set = false;
-      if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-        if (e != hipSuccess) {
-          set_error("hipFuncSetAttribute(gemm_mxfp6_staged, %d bytes LDS): %s", lds_bytes, hipGetErrorString(e));
-          return (int)e;
-        }
-        attr_set = true;
-      }
+      static std::atomic<uint64_t> lds_ok{0};
+      if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_mxfp6_staged")) return rc;
       const int tiles_m = M / 256, tiles_n = N / 256;
       dim3 grid(tiles_m * tiles_n), block(256);
       hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const uint8_t*)a, (const uint8_t*)as, (const uint8_t*)b,

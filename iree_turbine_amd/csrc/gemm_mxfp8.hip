@@ -579,15 +579,8 @@ static int launch_mx8(int variant, const void* a, const void* as, const void* b,
   if (variant == 0) {
     auto kern = gemm_mxfp8_tiled<256, 256, 2, 2, OutT, SCALED>;
     constexpr int lds_bytes = 2 * 512 * 128;
-    static bool attr_set = false;
-    if (!attr_set) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-      if (e != hipSuccess) {
-        set_error("hipFuncSetAttribute(gemm_mxfp8_tiled, %d bytes LDS): %s", lds_bytes, hipGetErrorString(e));
-        return (int)e;
-      }
-      attr_set = true;
-    }
+    static std::atomic<uint64_t> lds_ok{0};
+    if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_mxfp8_tiled")) return rc;
     const int tiles_m = M / 256, tiles_n = N / 256;
     dim3 grid(tiles_m * tiles_n), block(256);
     hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const uint8_t*)a, (const uint8_t*)as, (const uint8_t*)b,
@@ -597,15 +590,8 @@ static int launch_mx8(int variant, const void* a, const void* as, const void* b,
   if (variant == 2) {
     auto kern = gemm_mxfp8_staged<OutT, SCALED>;
     constexpr int lds_bytes = 17 * 8192 + 4 * 4096;  // two padded stages per operand, four scale buffers
-    static bool attr_set = false;
-    if (!attr_set) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-      if (e != hipSuccess) {
-        set_error("hipFuncSetAttribute(gemm_mxfp8_staged, %d bytes LDS): %s", lds_bytes, hipGetErrorString(e));
-        return (int)e;
-      }
-      attr_set = true;
-    }
+    static std::atomic<uint64_t> lds_ok{0};
+    if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_mxfp8_staged")) return rc;
     const int tiles_m = M / 256, tiles_n = N / 256;
     dim3 grid(tiles_m * tiles_n), block(256);
     hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const uint8_t*)a, (const uint8_t*)as, (const uint8_t*)b,

@@ -281,16 +281,8 @@ static int launch_phase0(const void* q, const void* kc, const void* vc, const in
   auto kern = paged_decode_phase0<G>;
   constexpr int lds_bytes = PD_WAVES * PD_WAVE_LDS;
   static_assert(lds_bytes >= (int)((2 * PD_WAVES * 16 + PD_WAVES * G * 128) * sizeof(float)), "merge area must fit");
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       lds_bytes);
-    if (e != hipSuccess) {
-      set_error("hipFuncSetAttribute(paged_decode_phase0): %s", hipGetErrorString(e));
-      return (int)e;
-    }
-    attr_set = true;
-  }
+  static std::atomic<uint64_t> lds_ok{0};
+  if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "paged_decode_phase0")) return rc;
   dim3 grid(num_splits, num_kv_heads, num_seqs), block(PD_WAVES * 64);
   hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)q, (const half_t*)kc, (const half_t*)vc, bt, sl,
                      pacc, pml, (half_t*)out, num_kv_heads, max_pages, num_splits, scale * 1.4426950408889634f, window, page_shift);
