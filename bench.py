@@ -41,7 +41,7 @@ METRIC = "TFLOP/s & %MFMA peak (f16 GEMM, causal FA, MXFP4 GEMM); decode HBM GB/
 MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
     "gemm_8192": 1.745e9,              # 1536 MiB read + 128 MiB written: each of the 8 XCD L2s fetches its own copy of
                                        # the panels its 4x8 block of output tiles needs (12 panels x 4 MiB x 4 rounds x 8)
-    "gemm_4096": 2.351e8,
+    "gemm_4096": 2.458e8,
     "gemm_2048x10240x8192": 6.472e8,
     "gemm_2048x57344x8192": 3.054e9,
     "gemm_1024_f32out": 1.684e7,

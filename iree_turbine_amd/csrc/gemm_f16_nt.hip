@@ -1038,10 +1038,15 @@ extern "C" int mi355_gemm_f16_nt(const void* a, const void* b, void* c, int64_t 
     // 128x128 tile (4x the workgroups) wins; everything else goes to the bounds-checked kernel.
     const long long t256 = (M / 256) * (N / 256);
     const long long rounds = (t256 + 255) / 256;  // 256 CUs, one 256x256 workgroup each
-    // the register-staged kernel measured best on every large shape; a sparse last round of 256x256 tiles goes
-    // to the 128x128 kernel when it can be cut off as whole tile columns or rows (+13% at 2048x10240x8192)
-    if (fits(8) && t256 >= 128) variant = 8;
-    else if (fits(0) && t256 >= 128 && t256 * 100 >= rounds * 256 * 85) variant = 0;  // >= 85% of the last round busy
+    // Long K: the register-staged kernel (measured best from K = 6144 up, and at any K once there are thousands
+    // of tiles); a sparse last round of its 256x256 tiles goes to the 128x128 kernel when it can be cut off as
+    // whole tile columns or rows (+13% at 2048x10240x8192).  Short K: the persistent kernel, which hides each
+    // tile's prologue and epilogue under its neighbours (8192x8192x512: +30%, x1024: +14%, x4096: +2%), as
+    // long as its last round is >= 85% busy.
+    const bool full_rounds = t256 * 100 >= rounds * 256 * 85;
+    if (K <= 4096 && t256 <= 2048 && fits(0) && t256 >= 128 && full_rounds) variant = 0;
+    else if (fits(8) && t256 >= 128) variant = 8;
+    else if (fits(0) && t256 >= 128 && full_rounds) variant = 0;
     else if (fits(4)) variant = 4;
     else variant = kNumGemmVariants - 1;
   } else if (!fits(variant)) {
