@@ -49,7 +49,7 @@ MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
     "fa_noncausal": 2.686e8,
     "decode": 1.177e9,
     "mxfp4_4096x8192x8192": 2.947e8,
-    "mxfp4_32x8192x8192": 3.748e7,
+    "mxfp4_32x8192x8192": 3.739e7,
     "mxfp4_quantize_16384x16384": 6.796e8,
     "mxfp8_quantize_16384x16384": 8.138e8,
     "mxfp6_quantize_16384x16384": 7.466e8,

@@ -38,7 +38,7 @@ def _hipcc() -> str:
 
 # Kernels that load into registers with hand-placed waits ("staged") must not spill: the compiler does not know
 # that such a register is still being filled, and a spill would store it before its data has arrived.
-NO_SPILL_KERNELS = ("staged",)
+NO_SPILL_KERNELS = ("staged", "skinny")
 _USAGE_FLAG = "-Rpass-analysis=kernel-resource-usage"
 
 

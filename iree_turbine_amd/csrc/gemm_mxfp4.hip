@@ -645,10 +645,78 @@ __global__ __launch_bounds__(512) void gemm_mxfp4_skinny(const uint8_t* __restri
 
   const int lrow = lane >> 3;
   const bool m_ok = r32 < M;
+  char* tr = lds + 8 * 16384 + wave * 4096;  // one A segment (32 rows x 128 bytes) per wave, for the transposition below
+  const int m_cl = r32 < M ? r32 : M - 1;    // rows past M repeat the last one: their output columns are never stored
   for (int seg0 = 0; seg0 < nseg; seg0 += 32) {  // a pass covers 32 segments (4 per wave)
     intx4 fa[4][4];
     int sa[4], sb[4];
     int cnt = 0;
+    if (seg0 + 32 <= nseg) {
+      // Full pass, straight-line.  A is the same 128 KiB for every workgroup and comes out of L2 -- as many bytes
+      // per workgroup as its share of B, and what they cost is L2 bandwidth (32x8192x8192: 8.7 us without the A
+      // loads, 12.6 with them in the MFMA's own layout, where a lane = one row and every load instruction
+      // touches 32 cache lines).  A is fetched like B -- 8 rows x 128 bytes per instruction, lane = (row, chunk)
+      // -- FIRST, and while the B loads issued behind it are still in flight it is turned into the MFMA layout
+      // through a 4 KiB LDS region (same swizzle as B): 12.2 us; with the B loads first 12.4.
+      // The A loads, the wait for them and the LDS instructions of the transposition are inline assembly: the
+      // compiler waits for EVERY load in flight before the first use of a loaded register once direct-to-LDS
+      // loads are among them, and before any LDS access it can see.  Loads return in order, so "at most the 16 B
+      // loads outstanding" means A has landed; a scale load that the compiler places behind the A loads only
+      // makes that wait longer.  LDS executes a wave's instructions in order, so the reads see the writes and
+      // the next segment's writes come after this one's reads.
+      // Workgroups start together and walk K in the same order, and rows are a multiple of 4 KiB apart: without
+      // the rotation every workgroup of an XCD would ask for the same A lines at the same time (11.8 us with
+      // it).  Ids 8 apart share an XCD, so the step is taken from the id's bits above those.
+      const int rot = (blockIdx.x >> 3) & 3;
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const int seg = seg0 + wave + 8 * ((q + rot) & 3);
+        sa[q] = *reinterpret_cast<const int*>(As + (size_t)m_cl * Ksc + seg * 8 + 4 * h);
+        sb[q] = *reinterpret_cast<const int*>(Bs + (size_t)(n0 + r32) * Ksc + seg * 8 + 4 * h);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const int seg = seg0 + wave + 8 * ((q + rot) & 3);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const int row = i * 8 + lrow;
+          const uint8_t* ap = A + (size_t)(row < M ? row : M - 1) * Kb + seg * 128 + (lane & 7) * 16;
+          asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(fa[q][i]) : "v"(ap) : "memory");
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const int seg = seg0 + wave + 8 * ((q + rot) & 3);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const int row = i * 8 + lrow;
+          const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+          load_lds_16B(B + (size_t)(n0 + row) * Kb + seg * 128 + chunk * 16, my + q * 4096 + i * 1024);
+        }
+      }
+      cnt = 4;
+      __builtin_amdgcn_sched_barrier(0);
+      asm volatile("s_waitcnt vmcnt(16)"
+                   : "+v"(fa[0][0]), "+v"(fa[0][1]), "+v"(fa[0][2]), "+v"(fa[0][3]), "+v"(fa[1][0]), "+v"(fa[1][1]),
+                     "+v"(fa[1][2]), "+v"(fa[1][3]), "+v"(fa[2][0]), "+v"(fa[2][1]), "+v"(fa[2][2]), "+v"(fa[2][3]),
+                     "+v"(fa[3][0]), "+v"(fa[3][1]), "+v"(fa[3][2]), "+v"(fa[3][3]));
+      const unsigned tr_base = (unsigned)(uintptr_t)MI355_LDS(char, tr);
+      unsigned wa[4], ra[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const int row = i * 8 + lrow;
+        wa[i] = tr_base + row * 128 + (((lane & 7) ^ ((row >> 1) & 7)) * 16);
+        ra[i] = tr_base + r32 * 128 + (((4 * h + i) ^ ((r32 >> 1) & 7)) * 16);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) asm volatile("ds_write_b128 %0, %1" ::"v"(wa[i]), "v"(fa[q][i]));
+#pragma unroll
+        for (int sp = 0; sp < 4; sp++) asm volatile("ds_read_b128 %0, %1" : "=v"(fa[q][sp]) : "v"(ra[sp]));
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    } else {
 #pragma unroll
     for (int q = 0; q < 4; q++) {
       const int seg = seg0 + wave + 8 * q;
@@ -673,6 +741,7 @@ __global__ __launch_bounds__(512) void gemm_mxfp4_skinny(const uint8_t* __restri
           for (int sp = 0; sp < 4; sp++) fa[q][sp] = intx4{0, 0, 0, 0};
         }
       }
+    }
     }
     wait_vmcnt0();
 #pragma unroll
@@ -1087,7 +1156,7 @@ static int launch_mx(int variant, const void* a, const void* as, const void* b, 
       return launch_mx_tiled<128, 128, 2, 2, OutT, false>(a, as, b, bs, c, M, N, K, stream);
     case 3: {
       auto kern = gemm_mxfp4_skinny<OutT>;
-      constexpr int lds_bytes = 8 * 16384;
+      constexpr int lds_bytes = 8 * 16384 + 8 * 4096;  // B segments + one A transposition region per wave
       static std::atomic<uint64_t> lds_ok{0};
       if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_mxfp4_skinny")) return rc;
       dim3 grid(N / 32), block(512);
