@@ -254,3 +254,25 @@ def test_gemm_autograd(dev, shape, out_dtype):
     ad2 = a.to(dev).requires_grad_(True)
     torch.ops.mi355.gemm_nt(ad2, b.to(dev), out_dtype, -1).float().sum().backward()
     torch.testing.assert_close(ad2.grad.float().cpu(), b.float().sum(dim=0).expand(M, K), rtol=RTOL, atol=ATOL)
+
+
+def test_gemm_output_beyond_4_gib(dev):
+    """A 49152 x 49152 fp16 result is 4.5 GiB: row offsets into C pass 2^32 bytes.  Sampled rows (the first, two
+    either side of the 4 GiB line, the last tile's) against an fp32 product, for the kernels the automatic choice
+    can reach and the any-shape kernel."""
+    import iree_turbine_amd as ita
+
+    M = N = 49152
+    K = 256
+    names = ita._lib.variants("gemm_f16_nt")
+    gen = torch.Generator(device="cpu").manual_seed(5)
+    a = (torch.randn(M, K, generator=gen) * 0.1).half().to(dev)
+    b = (torch.randn(N, K, generator=gen) * 0.1).half().to(dev)
+    rows = torch.tensor([0, 1000, 43690, 43691, M - 257, M - 1], device=dev)
+    ref = a[rows].float() @ b.float().t()
+    tail = next(i for i, n in enumerate(names) if "tail" in n)
+    for variant in (-1, tail, 0, 4, len(names) - 1):
+        announce(f"gemm {M}x{N}x{K} float16 variant={variant} (C beyond 4 GiB)")
+        c = torch.ops.mi355.gemm_nt(a, b, "float16", variant)
+        torch.testing.assert_close(c[rows].float(), ref, rtol=RTOL, atol=ATOL)
+        del c
