@@ -45,6 +45,7 @@ MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
     "gemm_2048x10240x8192": 6.472e8,
     "gemm_2048x57344x8192": 3.054e9,
     "gemm_1024_f32out": 1.684e7,
+    "gemm_bf16_8192": 1.746e9,
     "fa_causal": 3.425e8,
     "fa_noncausal": 2.686e8,
     "decode": 1.177e9,
@@ -106,20 +107,22 @@ def time_steps(fn, steps: int, warmup: int):
 
 # ---- workloads --------------------------------------------------------------------------------
 
-def wl_gemm(M, N, K, out_dtype="float16"):
+def wl_gemm(M, N, K, out_dtype="float16", in_dtype=torch.float16):
     from oracle import inputs
 
+    tag = "bf16" if in_dtype == torch.bfloat16 else "f16"
+
     def build(dev):
-        a, b = inputs.gemm_inputs(M, N, K)
+        a, b = inputs.gemm_inputs(M, N, K, dtype=in_dtype)
         ad, bd = a.to(dev), b.to(dev)
         flops = 2.0 * M * N * K
-        out_b = 2 if out_dtype == "float16" else 4
+        out_b = 4 if out_dtype == "float32" else 2
         nbytes = 2.0 * (M * K + N * K) + out_b * M * N
         return {
             "fn": lambda: torch.ops.mi355.gemm_nt(ad, bd, out_dtype, -1),
             "work": flops, "bytes": nbytes, "bound": "mfma", "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
-            "dtype": "f16", "cpu": lambda: cpu_gemm(a, b, M, N, K),
-            "config": {"workload": f"gemm_f16_nt_{M}x{N}x{K}_{'f16' if out_dtype == 'float16' else 'f32'}out",
+            "dtype": tag, "cpu": lambda: cpu_gemm(a, b, M, N, K),
+            "config": {"workload": f"gemm_{tag}_nt_{M}x{N}x{K}_{'f32' if out_dtype == 'float32' else tag}out",
                        "M": M, "N": N, "K": K, "layout": "NT", "accumulate": "f32", "out": out_dtype, "seed": 10},
         }
     return build
@@ -300,6 +303,7 @@ WORKLOADS = {
     "gemm_2048x10240x8192": wl_gemm(2048, 10240, 8192),
     "gemm_2048x57344x8192": wl_gemm(2048, 57344, 8192),
     "gemm_1024_f32out": wl_gemm(1024, 1024, 1024, "float32"),
+    "gemm_bf16_8192": wl_gemm(8192, 8192, 8192, "bfloat16", torch.bfloat16),
     "fa_causal": wl_attention(True),
     "fa_noncausal": wl_attention(False),
     "decode": wl_decode(),

@@ -68,6 +68,19 @@ int mi355_gemm_f16_nt(const void* a, const void* b, void* c,
                       int out_dtype, int variant, void* stream);
 
 /*
+ * The same GEMM with bf16 operands: A, B bf16 row-major (K contiguous), fp32
+ * accumulation, C out_dtype MI355_F32 or MI355_BF16 (round to nearest even).
+ * Same kernels, variants and shape rules as mi355_gemm_f16_nt.
+ * Replaces: aten::mm / aten::addmm signatures with bf16 operands
+ * (iree/turbine/kernel/boo/op_exports/aten.py:44-49, dtype names parsed at
+ * iree/turbine/kernel/boo/op_exports/aten.py:101-144) and nn.Linear in bf16
+ * under the BOO backend (iree/turbine/kernel/boo/ops/graph.py:171-182).
+ */
+int mi355_gemm_bf16_nt(const void* a, const void* b, void* c,
+                       int64_t M, int64_t N, int64_t K,
+                       int out_dtype, int variant, void* stream);
+
+/*
  * Flash-attention forward (prefill): O = softmax(scale . Q K^T [+ causal mask]) V.
  * q, o: [B, H, Sq, D]; k, v: [B, H, Sk, D]; all fp16 contiguous; D == 128.
  * fp32 online softmax, fp16 output.  is_causal: query i attends keys

@@ -26,20 +26,38 @@
 
 namespace mi355 {
 
-template <typename OutT> struct OutPack;
-template <> struct OutPack<float> {
+// BF selects the 16-bit input format: false = fp16, true = bf16.  Both travel through the kernels as opaque
+// 16-bit lanes of half8 / half4 vectors (same tiles, same LDS format, same fragment layout); only the MFMA
+// instruction and the conversion of the fp32 sums in the epilogue differ.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+template <bool BF>
+__device__ __forceinline__ floatx16 mfma16(half8 a, half8 b, floatx16 c) {
+  if constexpr (BF)
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  else
+    return mfma_32x32x16(a, b, c);
+}
+// fp32 -> the 16-bit output format (round to nearest even), returned in a half_t-sized container
+template <bool BF>
+__device__ __forceinline__ half_t cvt16(float f) {
+  if constexpr (BF) return __builtin_bit_cast(half_t, f32_to_bf16_rne(f));
+  else return (half_t)f;
+}
+
+template <typename OutT, bool BF> struct OutPack;
+template <bool BF> struct OutPack<float, BF> {
   static __device__ __forceinline__ void store4(float* p, float a, float b, float c, float d) {
     floatx4 v = {a, b, c, d};
     *reinterpret_cast<floatx4*>(p) = v;
   }
   static __device__ __forceinline__ void store1(float* p, float a) { *p = a; }
 };
-template <> struct OutPack<half_t> {
+template <bool BF> struct OutPack<half_t, BF> {
   static __device__ __forceinline__ void store4(half_t* p, float a, float b, float c, float d) {
-    half4 v = {(half_t)a, (half_t)b, (half_t)c, (half_t)d};
+    half4 v = {cvt16<BF>(a), cvt16<BF>(b), cvt16<BF>(c), cvt16<BF>(d)};
     *reinterpret_cast<half4*>(p) = v;
   }
-  static __device__ __forceinline__ void store1(half_t* p, float a) { *p = (half_t)a; }
+  static __device__ __forceinline__ void store1(half_t* p, float a) { *p = cvt16<BF>(a); }
 };
 
 __device__ __forceinline__ void map_tile(int pid, int tiles_m, int tiles_n, int group_m, int& tm, int& tn) {
@@ -55,7 +73,7 @@ __device__ __forceinline__ void map_tile(int pid, int tiles_m, int tiles_n, int 
   tn = within / gsz;
 }
 
-template <int BM, int BN, int WM, int WN, typename OutT>
+template <int BM, int BN, int WM, int WN, typename OutT, bool BF>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_tiled(const half_t* __restrict__ A,
                                                                  const half_t* __restrict__ B,
                                                                  OutT* __restrict__ C, int M, int N, int K,
@@ -125,7 +143,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_tiled(const half_t* _
 #pragma unroll
       for (int i = 0; i < TN; i++)
 #pragma unroll
-        for (int j = 0; j < TM; j++) acc[i][j] = mfma_32x32x16(fn[i], fm[j], acc[i][j]);
+        for (int j = 0; j < TM; j++) acc[i][j] = mfma16<BF>(fn[i], fm[j], acc[i][j]);
     }
     wait_vmcnt0();
     __syncthreads();
@@ -146,8 +164,8 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_tiled(const half_t* _
 #pragma unroll
         for (int q = 0; q < 4; q++) {
           const int c = i * 4 + q;
-          half4 v = {(half_t)acc[i][j][4 * q], (half_t)acc[i][j][4 * q + 1], (half_t)acc[i][j][4 * q + 2],
-                     (half_t)acc[i][j][4 * q + 3]};
+          half4 v = {cvt16<BF>(acc[i][j][4 * q]), cvt16<BF>(acc[i][j][4 * q + 1]), cvt16<BF>(acc[i][j][4 * q + 2]),
+                     cvt16<BF>(acc[i][j][4 * q + 3])};
           *reinterpret_cast<half4*>(ep + ml * ROW_B + ((c ^ ((ml >> 1) & 7)) * 16) + 8 * h) = v;
         }
     }
@@ -170,7 +188,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_tiled(const half_t* _
       for (int i = 0; i < TN; i++)
 #pragma unroll
         for (int q = 0; q < 4; q++)
-          OutPack<OutT>::store4(crow + i * 32 + q * 8, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+          OutPack<OutT, BF>::store4(crow + i * 32 + q * 8, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
                                 acc[i][j][4 * q + 3]);
     }
   }
@@ -181,7 +199,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_tiled(const half_t* _
 // k-step s issue, (b) the barrier that retires a slab sits in front of the last k-step's MFMAs,
 // which then overlap the first fragment reads of the next slab, and (c) the global -> LDS loads
 // for slab k+2 are issued right after that barrier into the stage that was just retired.
-template <int BM, int BN, int WM, int WN, typename OutT>
+template <int BM, int BN, int WM, int WN, typename OutT, bool BF>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_t* __restrict__ A,
                                                                      const half_t* __restrict__ B,
                                                                      OutT* __restrict__ C, int M, int N, int K,
@@ -243,7 +261,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
 #pragma unroll
     for (int i = 0; i < TN; i++)
 #pragma unroll
-      for (int j = 0; j < TM; j++) acc[i][j] = mfma_32x32x16(fn[i], fm[j], acc[i][j]);
+      for (int j = 0; j < TM; j++) acc[i][j] = mfma16<BF>(fn[i], fm[j], acc[i][j]);
   };
 
   const int KT = K / 64;
@@ -328,8 +346,8 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
 #pragma unroll
         for (int q = 0; q < 4; q++) {
           const int c = i * 4 + q;
-          half4 v = {(half_t)acc[i][j][4 * q], (half_t)acc[i][j][4 * q + 1], (half_t)acc[i][j][4 * q + 2],
-                     (half_t)acc[i][j][4 * q + 3]};
+          half4 v = {cvt16<BF>(acc[i][j][4 * q]), cvt16<BF>(acc[i][j][4 * q + 1]), cvt16<BF>(acc[i][j][4 * q + 2]),
+                     cvt16<BF>(acc[i][j][4 * q + 3])};
           *reinterpret_cast<half4*>(ep + ml * ROW_B + ((c ^ ((ml >> 1) & 7)) * 16) + 8 * h) = v;
         }
     }
@@ -352,7 +370,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
       for (int i = 0; i < TN; i++)
 #pragma unroll
         for (int q = 0; q < 4; q++)
-          OutPack<OutT>::store4(crow + i * 32 + q * 8, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+          OutPack<OutT, BF>::store4(crow + i * 32 + q * 8, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
                                 acc[i][j][4 * q + 3]);
     }
   }
@@ -372,7 +390,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
 // The loads are inline assembly so that the waits for them can be placed by hand (the compiler's vmcnt
 // placement merges the loop's entry and back edge pessimistically).  Same LDS format as the other tiled
 // kernels; the swizzle is applied by the ds_write address.
-template <int BM, int BN, int WM, int WN, typename OutT>
+template <int BM, int BN, int WM, int WN, typename OutT, bool BF>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_staged(const half_t* __restrict__ A, const half_t* __restrict__ B,
                                                                   OutT* __restrict__ C, int M, int N, int K, int tiles_m,
                                                                   int tiles_n, int group_m) {
@@ -488,16 +506,16 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_staged(const half_t* 
   };
 #define MI355_ST_GROUP(g, fm, fn, rst, rks, fm_n, fn_n, W1, W2, LD) \
   do {                                                              \
-    acc[g][0] = mfma_32x32x16(fn[g], fm[0], acc[g][0]);             \
+    acc[g][0] = mfma16<BF>(fn[g], fm[0], acc[g][0]);             \
     W1;                                                             \
     __builtin_amdgcn_sched_barrier(0);                              \
-    acc[g][1] = mfma_32x32x16(fn[g], fm[1], acc[g][1]);             \
+    acc[g][1] = mfma16<BF>(fn[g], fm[1], acc[g][1]);             \
     W2;                                                             \
     __builtin_amdgcn_sched_barrier(0);                              \
-    acc[g][2] = mfma_32x32x16(fn[g], fm[2], acc[g][2]);             \
+    acc[g][2] = mfma16<BF>(fn[g], fm[2], acc[g][2]);             \
     LD;                                                             \
     __builtin_amdgcn_sched_barrier(0);                              \
-    acc[g][3] = mfma_32x32x16(fn[g], fm[3], acc[g][3]);             \
+    acc[g][3] = mfma16<BF>(fn[g], fm[3], acc[g][3]);             \
     frag_reads(g, rst, rks, fm_n, fn_n);                            \
     __builtin_amdgcn_sched_barrier(0);                              \
   } while (0)
@@ -565,8 +583,8 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_staged(const half_t* 
 #pragma unroll
         for (int q = 0; q < 4; q++) {
           const int c = i * 4 + q;
-          half4 v = {(half_t)acc[i][j][4 * q], (half_t)acc[i][j][4 * q + 1], (half_t)acc[i][j][4 * q + 2],
-                     (half_t)acc[i][j][4 * q + 3]};
+          half4 v = {cvt16<BF>(acc[i][j][4 * q]), cvt16<BF>(acc[i][j][4 * q + 1]), cvt16<BF>(acc[i][j][4 * q + 2]),
+                     cvt16<BF>(acc[i][j][4 * q + 3])};
           *reinterpret_cast<half4*>(ep + r32 * ROW_B + ((c ^ ((r32 >> 1) & 7)) * 16) + 8 * h) = v;
         }
       OutT* cbase = C + (size_t)(tile_m * BM + wm * WTM + j * 32) * N + tile_n * BN + wn * WTN + ec * 8;
@@ -588,7 +606,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_staged(const half_t* 
       for (int i = 0; i < TN; i++)
 #pragma unroll
         for (int q = 0; q < 4; q++)
-          OutPack<OutT>::store4(crow + i * 32 + q * 8, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+          OutPack<OutT, BF>::store4(crow + i * 32 + q * 8, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
                                 acc[i][j][4 * q + 3]);
     }
   }
@@ -609,7 +627,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_staged(const half_t* 
 // Reading a slab's last fragments one k-step early frees its stage half a slab sooner, so the loads
 // spread over two k-steps instead of bunching behind the barrier, and they use buffer addressing
 // (descriptor + per-lane offset + scalar offset): no vector address arithmetic in the loop.
-template <int BM, int BN, int WM, int WN, typename OutT>
+template <int BM, int BN, int WM, int WN, typename OutT, bool BF>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_persistent(const half_t* __restrict__ A,
                                                                       const half_t* __restrict__ B,
                                                                       OutT* __restrict__ C, int M, int N, int K,
@@ -687,7 +705,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_persistent(const half
 #pragma unroll
     for (int i = 0; i < TN; i++)
 #pragma unroll
-      for (int j = 0; j < TM; j++) acc[i][j] = mfma_32x32x16(fn[i], fm[j], acc[i][j]);
+      for (int j = 0; j < TM; j++) acc[i][j] = mfma16<BF>(fn[i], fm[j], acc[i][j]);
   };
 
   constexpr int NM = TM * TN;       // MFMAs per k-step
@@ -796,8 +814,8 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_persistent(const half
 #pragma unroll
           for (int q = 0; q < 4; q++) {
             const int c = i * 4 + q;
-            half4 hv = {(half_t)acc[i][j][4 * q], (half_t)acc[i][j][4 * q + 1], (half_t)acc[i][j][4 * q + 2],
-                        (half_t)acc[i][j][4 * q + 3]};
+            half4 hv = {cvt16<BF>(acc[i][j][4 * q]), cvt16<BF>(acc[i][j][4 * q + 1]), cvt16<BF>(acc[i][j][4 * q + 2]),
+                        cvt16<BF>(acc[i][j][4 * q + 3])};
             *reinterpret_cast<half4*>(ep + r32 * EP_ROW + ((c ^ ((r32 / EP_RPB) & (EP_CH - 1))) * 16) + 8 * h) = hv;
           }
 #pragma unroll
@@ -818,7 +836,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_persistent(const half
         for (int i = 0; i < TN; i++)
 #pragma unroll
           for (int q = 0; q < 4; q++)
-            OutPack<OutT>::store4(crow + i * 32 + q * 8, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+            OutPack<OutT, BF>::store4(crow + i * 32 + q * 8, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
                                   acc[i][j][4 * q + 3]);
       }
     }
@@ -834,7 +852,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_persistent(const half
 
 // Any-shape kernel: 64x64 tile, 4 waves, bounds-checked staging through registers.  Used for
 // shapes the tiled kernel does not divide (and as an independent implementation in tests).
-template <typename OutT>
+template <typename OutT, bool BF>
 __global__ __launch_bounds__(256) void gemm_f16_nt_generic(const half_t* __restrict__ A, const half_t* __restrict__ B,
                                                            OutT* __restrict__ C, int M, int N, int K) {
   constexpr int PITCH = 40;  // halfs per LDS row: 32 data + 8 pad keeps 16-byte alignment, spreads banks
@@ -875,7 +893,7 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_generic(const half_t* __restr
     for (int ks = 0; ks < 2; ks++) {
       half8 fm = *reinterpret_cast<const half8*>(sA + (wm * 32 + r32) * PITCH + ks * 16 + h * 8);
       half8 fn = *reinterpret_cast<const half8*>(sB + (wn * 32 + r32) * PITCH + ks * 16 + h * 8);
-      acc = mfma_32x32x16(fn, fm, acc);
+      acc = mfma16<BF>(fn, fm, acc);
     }
   }
   const int m = row0_m + wm * 32 + r32;
@@ -883,7 +901,7 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_generic(const half_t* __restr
 #pragma unroll
     for (int r = 0; r < 16; r++) {
       const int n = row0_n + wn * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-      if (n < N) OutPack<OutT>::store1(C + (size_t)m * N + n, acc[r]);
+      if (n < N) OutPack<OutT, BF>::store1(C + (size_t)m * N + n, acc[r]);
     }
   }
 }
@@ -911,15 +929,15 @@ constexpr int kNumGemmVariants = sizeof(kGemmVariants) / sizeof(kGemmVariants[0]
 int gemm_variant_count() { return kNumGemmVariants; }
 const char* gemm_variant_name(int i) { return (i >= 0 && i < kNumGemmVariants) ? kGemmVariants[i].name : nullptr; }
 
-template <int BM, int BN, int WM, int WN, typename OutT, int KIND>  // 0 tiled, 1 pipelined, 2 register-staged
+template <int BM, int BN, int WM, int WN, typename OutT, int KIND, bool BF>  // KIND: 0 tiled, 1 pipelined, 2 register-staged
 static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int K, int ldc, hipStream_t stream) {
   // the kernels use their N argument only as the row stride of C, so a column range of a wider C is the
   // same launch with ldc in its place
   constexpr bool PIPELINED = KIND == 1;
   void (*kern)(const half_t*, const half_t*, OutT*, int, int, int, int, int, int);
-  if constexpr (KIND == 2) kern = gemm_f16_nt_staged<BM, BN, WM, WN, OutT>;
-  else if constexpr (PIPELINED) kern = gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT>;
-  else kern = gemm_f16_nt_tiled<BM, BN, WM, WN, OutT>;
+  if constexpr (KIND == 2) kern = gemm_f16_nt_staged<BM, BN, WM, WN, OutT, BF>;
+  else if constexpr (PIPELINED) kern = gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT, BF>;
+  else kern = gemm_f16_nt_tiled<BM, BN, WM, WN, OutT, BF>;
   constexpr int lds_bytes = 2 * (BM + BN) * 128;
   static std::atomic<uint64_t> lds_ok{0};
   if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt")) return rc;
@@ -944,9 +962,9 @@ static int cu_count() {
   return cached[dev];
 }
 
-template <int BM, int BN, int WM, int WN, typename OutT>
+template <int BM, int BN, int WM, int WN, typename OutT, bool BF>
 static int launch_persistent(const void* a, const void* b, void* c, int M, int N, int K, hipStream_t stream) {
-  auto kern = gemm_f16_nt_persistent<BM, BN, WM, WN, OutT>;
+  auto kern = gemm_f16_nt_persistent<BM, BN, WM, WN, OutT, BF>;
   constexpr int lds_bytes = 2 * (BM + BN) * 128 + WM * WN * 32 * (BN / WN) * 2;  // two stages + one epilogue pass per wave
   static std::atomic<uint64_t> lds_ok{0};
   if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt_persistent")) return rc;
@@ -980,34 +998,34 @@ static bool tail_split(int M, int N, int& main_m, int& main_n) {
   return true;
 }
 
-template <typename OutT>
+template <typename OutT, bool BF>
 static int launch_split(const void* a, const void* b, void* c, int M, int N, int K, hipStream_t stream) {
   int mm, mn;
-  if (!tail_split(M, N, mm, mn)) return launch_tiled<256, 256, 2, 2, OutT, 2>(a, b, c, M, N, K, N, stream);
-  int rc = launch_tiled<256, 256, 2, 2, OutT, 2>(a, b, c, mm, mn, K, N, stream);
+  if (!tail_split(M, N, mm, mn)) return launch_tiled<256, 256, 2, 2, OutT, 2, BF>(a, b, c, M, N, K, N, stream);
+  int rc = launch_tiled<256, 256, 2, 2, OutT, 2, BF>(a, b, c, mm, mn, K, N, stream);
   if (rc) return rc;
   const half_t* ah = (const half_t*)a;
   const half_t* bh = (const half_t*)b;
   OutT* ch = (OutT*)c;
-  if (mn < N) return launch_tiled<128, 128, 2, 2, OutT, 1>(ah, bh + (size_t)mn * K, ch + mn, M, N - mn, K, N, stream);
-  return launch_tiled<128, 128, 2, 2, OutT, 1>(ah + (size_t)mm * K, bh, ch + (size_t)mm * N, M - mm, N, K, N, stream);
+  if (mn < N) return launch_tiled<128, 128, 2, 2, OutT, 1, BF>(ah, bh + (size_t)mn * K, ch + mn, M, N - mn, K, N, stream);
+  return launch_tiled<128, 128, 2, 2, OutT, 1, BF>(ah + (size_t)mm * K, bh, ch + (size_t)mm * N, M - mm, N, K, N, stream);
 }
 
-template <typename OutT>
+template <typename OutT, bool BF>
 static int launch_variant(int variant, const void* a, const void* b, void* c, int M, int N, int K, hipStream_t stream) {
   switch (variant) {
-    case 0: return launch_persistent<256, 256, 2, 4, OutT>(a, b, c, M, N, K, stream);
-    case 1: return launch_persistent<256, 256, 2, 2, OutT>(a, b, c, M, N, K, stream);
-    case 2: return launch_tiled<256, 256, 2, 4, OutT, 1>(a, b, c, M, N, K, N, stream);
-    case 3: return launch_tiled<256, 256, 2, 2, OutT, 1>(a, b, c, M, N, K, N, stream);
-    case 4: return launch_tiled<128, 128, 2, 2, OutT, 1>(a, b, c, M, N, K, N, stream);
-    case 5: return launch_tiled<256, 256, 2, 4, OutT, 0>(a, b, c, M, N, K, N, stream);
-    case 6: return launch_tiled<128, 128, 2, 2, OutT, 0>(a, b, c, M, N, K, N, stream);
-    case 7: return launch_tiled<256, 256, 2, 2, OutT, 2>(a, b, c, M, N, K, N, stream);
-    case 8: return launch_split<OutT>(a, b, c, M, N, K, stream);
+    case 0: return launch_persistent<256, 256, 2, 4, OutT, BF>(a, b, c, M, N, K, stream);
+    case 1: return launch_persistent<256, 256, 2, 2, OutT, BF>(a, b, c, M, N, K, stream);
+    case 2: return launch_tiled<256, 256, 2, 4, OutT, 1, BF>(a, b, c, M, N, K, N, stream);
+    case 3: return launch_tiled<256, 256, 2, 2, OutT, 1, BF>(a, b, c, M, N, K, N, stream);
+    case 4: return launch_tiled<128, 128, 2, 2, OutT, 1, BF>(a, b, c, M, N, K, N, stream);
+    case 5: return launch_tiled<256, 256, 2, 4, OutT, 0, BF>(a, b, c, M, N, K, N, stream);
+    case 6: return launch_tiled<128, 128, 2, 2, OutT, 0, BF>(a, b, c, M, N, K, N, stream);
+    case 7: return launch_tiled<256, 256, 2, 2, OutT, 2, BF>(a, b, c, M, N, K, N, stream);
+    case 8: return launch_split<OutT, BF>(a, b, c, M, N, K, stream);
     default: {
       dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
-      hipLaunchKernelGGL(gemm_f16_nt_generic<OutT>, grid, block, 0, stream, (const half_t*)a, (const half_t*)b, (OutT*)c,
+      hipLaunchKernelGGL((gemm_f16_nt_generic<OutT, BF>), grid, block, 0, stream, (const half_t*)a, (const half_t*)b, (OutT*)c,
                          M, N, K);
       return check_launch("gemm_f16_nt_generic", grid, block, 0);
     }
@@ -1018,13 +1036,14 @@ static int launch_variant(int variant, const void* a, const void* b, void* c, in
 
 using namespace mi355;
 
-extern "C" int mi355_gemm_f16_nt(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int out_dtype,
-                                 int variant, void* stream) {
+// fp16 and bf16 share everything but the kernel instantiation; `bf` also names the 16-bit output format
+static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int out_dtype, int variant,
+                         void* stream) {
   if (!a || !b || !c) return fail(-MI355_E_NULL, "gemm_f16_nt: null pointer (a=%p b=%p c=%p)", a, b, c);
   if (M <= 0 || N <= 0 || K <= 0 || M > (1 << 30) || N > (1 << 30) || K > (1 << 27))
     return fail(-MI355_E_SHAPE, "gemm_f16_nt: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
-  if (out_dtype != MI355_F32 && out_dtype != MI355_F16)
-    return fail(-MI355_E_DTYPE, "gemm_f16_nt: out_dtype %d (want MI355_F32 or MI355_F16)", out_dtype);
+  if (out_dtype != MI355_F32 && out_dtype != (bf ? MI355_BF16 : MI355_F16))
+    return fail(-MI355_E_DTYPE, "gemm_f16_nt: out_dtype %d (want MI355_F32 or %s)", out_dtype, bf ? "MI355_BF16" : "MI355_F16");
   if (variant >= kNumGemmVariants) return fail(-MI355_E_DTYPE, "gemm_f16_nt: variant %d out of range", variant);
   const bool al = aligned16(a) && aligned16(b) && aligned16(c);
   auto fits = [&](int v) {
@@ -1057,6 +1076,20 @@ extern "C" int mi355_gemm_f16_nt(const void* a, const void* b, void* c, int64_t 
     return fail(-MI355_E_ALIGN, "gemm_f16_nt: a and b must be 16-byte aligned when K %% 8 == 0");
   }
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  if (out_dtype == MI355_F32) return launch_variant<float>(variant, a, b, c, (int)M, (int)N, (int)K, s);
-  return launch_variant<half_t>(variant, a, b, c, (int)M, (int)N, (int)K, s);
+  if (bf) {
+    if (out_dtype == MI355_F32) return launch_variant<float, true>(variant, a, b, c, (int)M, (int)N, (int)K, s);
+    return launch_variant<half_t, true>(variant, a, b, c, (int)M, (int)N, (int)K, s);
+  }
+  if (out_dtype == MI355_F32) return launch_variant<float, false>(variant, a, b, c, (int)M, (int)N, (int)K, s);
+  return launch_variant<half_t, false>(variant, a, b, c, (int)M, (int)N, (int)K, s);
+}
+
+extern "C" int mi355_gemm_f16_nt(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int out_dtype,
+                                 int variant, void* stream) {
+  return gemm_nt_entry(false, a, b, c, M, N, K, out_dtype, variant, stream);
+}
+
+extern "C" int mi355_gemm_bf16_nt(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int out_dtype,
+                                  int variant, void* stream) {
+  return gemm_nt_entry(true, a, b, c, M, N, K, out_dtype, variant, stream);
 }

@@ -15,8 +15,8 @@ substitution is a direct FX rewrite of the ATen graph that AOT-autograd produces
   aten._scaled_dot_product_{flash,efficient,flash_for_cpu}_attention(q, k, v, ...)[0]
                               -> mi355.flash_attn_fwd(q, k, v, is_causal, scale)
 
-A node is rewritten only when the kernels cover it (fp16 tensors on a CUDA device, head dim 128, no mask, no
-dropout, auxiliary outputs unused -- so training graphs keep PyTorch's attention); everything else is left
+A node is rewritten only when the kernels cover it (fp16 -- for mm / addmm also bf16 -- tensors on a CUDA device,
+head dim 128, no mask, no dropout, auxiliary outputs unused -- so training graphs keep PyTorch's attention); everything else is left
 for the nested backend.  Layouts: the ops make their operands contiguous themselves, so transposed views
 (`q.transpose(1, 2)`) need no graph surgery.
 """
@@ -43,9 +43,14 @@ def _val(node):
     return node.meta.get("val") if isinstance(node, fx.Node) else None
 
 
-def _is_half_matrix(node, device_ok) -> bool:
+_GEMM_DTYPES = (torch.float16, torch.bfloat16)
+
+
+def _is_half_matrix(node, device_ok, dtype=None) -> bool:
+    """A non-empty rank-2 fp16 / bf16 tensor on a device the backend serves (of exactly `dtype` if given)."""
     v = _val(node)
-    return isinstance(v, torch.Tensor) and v.dim() == 2 and v.dtype == torch.float16 and device_ok(v.device) and v.numel() > 0
+    return (isinstance(v, torch.Tensor) and v.dim() == 2 and v.dtype in _GEMM_DTYPES and (dtype is None or v.dtype == dtype)
+            and device_ok(v.device) and v.numel() > 0)
 
 
 def _transposed_source(node):
@@ -69,12 +74,16 @@ def _gemm_nt_node(graph: fx.Graph, a, b):
         b_nk = src
     else:
         b_nk = graph.call_function(aten.t.default, (b,))
-    return graph.call_function(torch.ops.mi355.gemm_nt.default, (a, b_nk, "float16", -1))
+    own = str(_val(a).dtype).removeprefix("torch.")
+    return graph.call_function(torch.ops.mi355.gemm_nt.default, (a, b_nk, own, -1))
 
 
 def _rewrite_mm(node: fx.Node, device_ok) -> bool:
     a, b = node.args[:2]
-    if not (_is_half_matrix(a, device_ok) and _is_half_matrix(b, device_ok) and _is_half_matrix(node, device_ok)):
+    if not _is_half_matrix(a, device_ok):
+        return False
+    dt = _val(a).dtype
+    if not (_is_half_matrix(b, device_ok, dt) and _is_half_matrix(node, device_ok, dt)):
         return False
     with node.graph.inserting_before(node):
         new = _gemm_nt_node(node.graph, a, b)
@@ -89,9 +98,12 @@ def _rewrite_addmm(node: fx.Node, device_ok) -> bool:
     if node.kwargs.get("beta", 1) != 1 or node.kwargs.get("alpha", 1) != 1:
         return False
     bv = _val(bias)
-    if not (_is_half_matrix(a, device_ok) and _is_half_matrix(b, device_ok) and _is_half_matrix(node, device_ok)):
+    if not _is_half_matrix(a, device_ok):
         return False
-    if not (isinstance(bv, torch.Tensor) and bv.dtype == torch.float16 and bv.dim() in (1, 2)):
+    dt = _val(a).dtype
+    if not (_is_half_matrix(b, device_ok, dt) and _is_half_matrix(node, device_ok, dt)):
+        return False
+    if not (isinstance(bv, torch.Tensor) and bv.dtype == dt and bv.dim() in (1, 2)):
         return False
     with node.graph.inserting_before(node):
         mm = _gemm_nt_node(node.graph, a, b)

@@ -37,10 +37,16 @@ def gemm_nt_out(a: Tensor, b: Tensor, c: Tensor, variant: int = -1) -> Tensor:
     N = b.shape[0]
     if tuple(c.shape) != (M, N):
         raise ValueError(f"gemm_nt: c is {tuple(c.shape)}, expected {(M, N)}")
+    if a.dtype != b.dtype or a.dtype not in (torch.float16, torch.bfloat16):
+        raise ValueError(f"gemm_nt: a and b must both be float16 or both bfloat16, got {a.dtype} and {b.dtype}")
+    if c.dtype not in (torch.float32, a.dtype):
+        raise ValueError(f"gemm_nt: c must be float32 or {a.dtype}, got {c.dtype}")
+    lib = _lib.load()
+    entry = lib.mi355_gemm_bf16_nt if a.dtype == torch.bfloat16 else lib.mi355_gemm_f16_nt
     with torch.cuda.device(dev):
-        rc = _lib.load().mi355_gemm_f16_nt(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, _lib.dtype_code(c.dtype),
-                                           variant, _lib.current_stream_ptr(dev))
-    _lib.check(rc, f"gemm_nt M={M} N={N} K={K} out={c.dtype} variant={variant}")
+        rc = entry(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, _lib.dtype_code(c.dtype), variant,
+                   _lib.current_stream_ptr(dev))
+    _lib.check(rc, f"gemm_nt M={M} N={N} K={K} in={a.dtype} out={c.dtype} variant={variant}")
     return c
 
 

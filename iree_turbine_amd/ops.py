@@ -42,7 +42,8 @@ def _require(cond: bool, msg: str) -> None:
 
 @CustomOp.register
 class gemm_nt(CustomOp):
-    """C[M,N] = A[M,K] . B[N,K]^T, fp16 inputs, fp32 accumulation; out_dtype "float32" | "float16".
+    """C[M,N] = A[M,K] . B[N,K]^T, fp16 or bf16 inputs, fp32 accumulation; out_dtype "float32" or the inputs' own
+    ("float16" | "bfloat16").
 
     The NT form is what `gemmfp16 ... --transB 1` computes in the reference
     (iree/turbine/kernel/boo/op_exports/gemm.py:84-86,228-230) and what `nn.Linear` hands to a
@@ -55,9 +56,11 @@ class gemm_nt(CustomOp):
         od = sel.attr_str(2).v
         sel.attr_int(3)
         _require(a.t.dim() == 2 and b.t.dim() == 2, "gemm_nt: a and b must be rank 2")
-        _require(a.t.dtype == torch.float16 and b.t.dtype == torch.float16, "gemm_nt: a and b must be float16")
+        _require(a.t.dtype == b.t.dtype and a.t.dtype in (torch.float16, torch.bfloat16),
+                 "gemm_nt: a and b must both be float16 or both bfloat16")
         _require(a.t.size(1) == b.t.size(1), f"gemm_nt: K mismatch, a is {tuple(a.t.shape)}, b is {tuple(b.t.shape)} (b is [N, K])")
-        _require(od in ("float32", "float16"), f"gemm_nt: out_dtype must be 'float32' or 'float16', got {od!r}")
+        own = str(a.t.dtype).removeprefix("torch.")
+        _require(od in ("float32", own), f"gemm_nt: out_dtype must be 'float32' or '{own}' for {own} operands, got {od!r}")
         _require(a.t.size(0) > 0 and b.t.size(0) > 0 and a.t.size(1) > 0, "gemm_nt: empty operand")
         a.specialize_all_dims()
         b.specialize_all_dims()
@@ -76,14 +79,15 @@ def _gemm_nt_setup_context(ctx, inputs, output):
 def _gemm_nt_backward(ctx, grad):
     """For C = A . B^T: dA = dC . B and dB = dC^T . A (the formulas of GEMMBackwardA / GEMMBackwardB,
     iree/turbine/kernel/boo/op_exports/gemm.py:232-269, for the NT layout), each one launch of the same kernel
-    on operands re-laid K-contiguous; gradients come back in fp16 like the operands."""
+    on operands re-laid K-contiguous; gradients come back in the operands' dtype."""
     a, b = ctx.saved_tensors
-    g = grad.to(torch.float16)
+    g = grad.to(a.dtype)
+    own = str(a.dtype).removeprefix("torch.")
     grad_a = grad_b = None
     if ctx.needs_input_grad[0]:
-        grad_a = torch.ops.mi355.gemm_nt(g.contiguous(), b.t().contiguous(), "float16", -1)      # [M,N] . [K,N]^T
+        grad_a = torch.ops.mi355.gemm_nt(g.contiguous(), b.t().contiguous(), own, -1)      # [M,N] . [K,N]^T
     if ctx.needs_input_grad[1]:
-        grad_b = torch.ops.mi355.gemm_nt(g.t().contiguous(), a.t().contiguous(), "float16", -1)  # [N,M] . [K,M]^T
+        grad_b = torch.ops.mi355.gemm_nt(g.t().contiguous(), a.t().contiguous(), own, -1)  # [N,M] . [K,M]^T
     return grad_a, grad_b, None, None
 
 

@@ -31,15 +31,15 @@ def _entry(hp, a, b, c):
 
 def get_gemm_kernel(shape: tuple[int, int, int], dynamic_dims: bool = False, mfma_variant=None,
                     dtype: torch.dtype = torch.float16):
-    """C[M, N] = A[M, K] . B[N, K]^T with fp32 accumulation.  Call as kernel(a, b, c): a [M, K] f16,
-    b [N, K] f16, c [M, N] f32 or f16 (written in place).
+    """C[M, N] = A[M, K] . B[N, K]^T with fp32 accumulation.  Call as kernel(a, b, c): a [M, K] and b [N, K] of
+    `dtype` (float16 or bfloat16), c [M, N] f32 or `dtype` (written in place).
 
     Returns (kernel, hyperparams).  With dynamic_dims the sizes are read from the tensors at call
     time; otherwise M, N, K are bound and checked.  `mfma_variant` is accepted for call-site
-    compatibility; the pre-built kernels use v_mfma_f32_32x32x16_f16.
+    compatibility; the pre-built kernels use v_mfma_f32_32x32x16_f16 / _bf16.
     The loop nest this stands for is the TK tiled GEMM, tests/kernel/vector_codegen_test.py:71-100."""
-    if dtype != torch.float16:
-        raise ValueError(f"get_gemm_kernel: only float16 operands are built, got {dtype}")
+    if dtype not in (torch.float16, torch.bfloat16):
+        raise ValueError(f"get_gemm_kernel: float16 and bfloat16 operands are built, got {dtype}")
     m, n, k = shape
     if m % 256 == 0 and n % 256 == 0 and k % 64 == 0 and (m // 256) * (n // 256) >= 128:
         bm = bn = 256
@@ -50,6 +50,7 @@ def get_gemm_kernel(shape: tuple[int, int, int], dynamic_dims: bool = False, mfm
     hyperparams = {BLOCK_M: bm, BLOCK_N: bn, BLOCK_K: 64 if bm > 64 else 32}
     if not dynamic_dims:
         hyperparams.update({M: m, N: n, K: k})
-    kernel = Launchable("gemm_f16_nt", _entry, num_outputs=1,
-                        description="fp16 NT GEMM, fp32 accumulate (hand-written gfx950 MFMA kernel)")
+    name = "gemm_bf16_nt" if dtype == torch.bfloat16 else "gemm_f16_nt"
+    kernel = Launchable(name, _entry, num_outputs=1,
+                        description="16-bit NT GEMM, fp32 accumulate (hand-written gfx950 MFMA kernel)")
     return kernel, hyperparams

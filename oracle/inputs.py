@@ -16,11 +16,11 @@ def _gen(seed: int) -> torch.Generator:
     return torch.Generator(device="cpu").manual_seed(seed)
 
 
-def gemm_inputs(M: int, N: int, K: int, seed: int = DEFAULT_SEED, std: float = 0.1):
-    """A [M, K], B [N, K] ~ N(0, 1) * std, fp16."""
+def gemm_inputs(M: int, N: int, K: int, seed: int = DEFAULT_SEED, std: float = 0.1, dtype: torch.dtype = torch.float16):
+    """A [M, K], B [N, K] ~ N(0, 1) * std, fp16 (or `dtype`; the fp32 draws are the same either way)."""
     g = _gen(seed)
-    a = (torch.randn((M, K), generator=g) * std).half()
-    b = (torch.randn((N, K), generator=g) * std).half()
+    a = (torch.randn((M, K), generator=g) * std).to(dtype)
+    b = (torch.randn((N, K), generator=g) * std).to(dtype)
     return a, b
 
 

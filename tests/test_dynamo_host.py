@@ -54,14 +54,24 @@ def test_mm_with_untransposed_rhs_gets_a_transpose():
     assert g.args[1].target is torch.ops.aten.t.default  # b^T is [N, K]; the launcher packs it
 
 
-@pytest.mark.parametrize("what", ["fp32", "bf16", "addmm_beta", "empty"])
+def test_bf16_linear_layers_keep_their_dtype():
+    from iree_turbine_amd import dynamo
+
+    x, w, b = _h(64, 256).bfloat16(), _h(512, 256).bfloat16(), _h(512).bfloat16()
+    gm = _trace(lambda x, w, b: F.linear(x, w, b) + x @ w.t(), x, w, b)
+    assert dynamo.substitute_kernels(gm, device_ok=ANY) == {"mm": 1, "addmm": 1, "sdpa": 0}
+    gemms = [n for n in gm.graph.nodes if n.target is torch.ops.mi355.gemm_nt.default]
+    assert len(gemms) == 2 and all(g.args[2] == "bfloat16" for g in gemms)
+
+
+@pytest.mark.parametrize("what", ["fp32", "fp64", "addmm_beta", "empty"])
 def test_unsupported_matmuls_are_left_alone(what):
     from iree_turbine_amd import dynamo
 
     if what == "fp32":
         gm = _trace(lambda a, b: a @ b, torch.randn(8, 8), torch.randn(8, 8))
-    elif what == "bf16":
-        gm = _trace(lambda a, b: a @ b, torch.randn(8, 8).bfloat16(), torch.randn(8, 8).bfloat16())
+    elif what == "fp64":
+        gm = _trace(lambda a, b: a @ b, torch.randn(8, 8).double(), torch.randn(8, 8).double())
     elif what == "addmm_beta":
         gm = _trace(lambda c, a, b: torch.addmm(c, a, b, beta=0.5), _h(8, 8), _h(8, 8), _h(8, 8))
     else:

@@ -63,6 +63,27 @@ def test_compiled_block_matches_eager(dev, bias, hkv):
     assert torch.equal(got, again)
 
 
+def test_compiled_bf16_block_routes_its_linear_layers(dev):
+    """In bf16 the seven linear layers go to the bf16 GEMM; attention stays with PyTorch (the attention kernel is
+    fp16 only) and the result is what eager gives, to bf16's 8 bits."""
+    import iree_turbine_amd.dynamo as mdyn
+
+    announce("torch.compile backend=mi355 bf16")
+    torch.manual_seed(4)
+    torch._dynamo.reset()
+    model = Block(bias=True).to(dev).bfloat16().eval()
+    x = torch.randn(2, 192, 512, device=dev).bfloat16()
+    with torch.no_grad():
+        want = model(x)
+        mdyn.LAST_SUBSTITUTIONS.clear()
+        got = torch.compile(model, backend="mi355")(x)
+    torch.cuda.synchronize()
+    counts = dict(mdyn.LAST_SUBSTITUTIONS)
+    assert counts["addmm"] == 7 and counts["sdpa"] == 0, counts
+    assert got.dtype == torch.bfloat16
+    torch.testing.assert_close(got.float(), want.float(), rtol=5e-2, atol=5e-2)
+
+
 def test_compiled_training_step_keeps_attention_in_pytorch(dev):
     """With gradients the log-sum-exp of the attention is consumed by the backward graph, so the attention stays
     with PyTorch; the matrix products of both the forward and the backward graph still go to the kernels."""

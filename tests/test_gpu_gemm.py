@@ -231,7 +231,7 @@ def test_gemm_staged_contract(dev):
 
 
 @pytest.mark.parametrize("shape", [(32, 12, 64), (256, 512, 384), (100, 70, 72)])
-@pytest.mark.parametrize("out_dtype", ["float16", "float32"])
+@pytest.mark.parametrize("out_dtype", ["float16", "float32", "bfloat16"])
 def test_gemm_autograd(dev, shape, out_dtype):
     """Gradients of the op against torch's own for C = A . B^T (the reference checks its GEMM backward formulas the
     same way, tests/kernel/boo/op_exports/gemm_backward_test.py:17-83), fp32 reference on the CPU."""
@@ -240,20 +240,22 @@ def test_gemm_autograd(dev, shape, out_dtype):
 
     M, N, K = shape
     announce(f"gemm autograd {shape} {out_dtype}")
-    a, b = inputs.gemm_inputs(M, N, K, seed=1)
+    in_dtype = torch.bfloat16 if out_dtype == "bfloat16" else torch.float16
+    a, b = inputs.gemm_inputs(M, N, K, seed=1, dtype=in_dtype)
     w = torch.randn(M, N, generator=torch.Generator().manual_seed(2)) * 0.1
     ar, br = a.float().requires_grad_(True), b.float().requires_grad_(True)
     ((ar @ br.t()) * w).sum().backward()
     ad, bd = a.to(dev).requires_grad_(True), b.to(dev).requires_grad_(True)
     c = torch.ops.mi355.gemm_nt(ad, bd, out_dtype, -1)
     (c.float() * w.to(dev)).sum().backward()
-    assert ad.grad.dtype == torch.float16 and bd.grad.dtype == torch.float16
-    torch.testing.assert_close(ad.grad.float().cpu(), ar.grad, rtol=RTOL, atol=ATOL)
-    torch.testing.assert_close(bd.grad.float().cpu(), br.grad, rtol=RTOL, atol=ATOL)
+    assert ad.grad.dtype == in_dtype and bd.grad.dtype == in_dtype
+    tol = 3e-2 if in_dtype == torch.bfloat16 else RTOL  # bf16 keeps 8 bits: the upstream gradient and the result are rounded to it
+    torch.testing.assert_close(ad.grad.float().cpu(), ar.grad, rtol=tol, atol=tol)
+    torch.testing.assert_close(bd.grad.float().cpu(), br.grad, rtol=tol, atol=tol)
     # only one operand needs a gradient
     ad2 = a.to(dev).requires_grad_(True)
     torch.ops.mi355.gemm_nt(ad2, b.to(dev), out_dtype, -1).float().sum().backward()
-    torch.testing.assert_close(ad2.grad.float().cpu(), b.float().sum(dim=0).expand(M, K), rtol=RTOL, atol=ATOL)
+    torch.testing.assert_close(ad2.grad.float().cpu(), b.float().sum(dim=0).expand(M, K), rtol=tol, atol=tol)
 
 
 def test_gemm_output_beyond_4_gib(dev):
@@ -276,3 +278,63 @@ def test_gemm_output_beyond_4_gib(dev):
         c = torch.ops.mi355.gemm_nt(a, b, "float16", variant)
         torch.testing.assert_close(c[rows].float(), ref, rtol=RTOL, atol=ATOL)
         del c
+
+
+BF16_SHAPES = [(1024, 1024, 1024), (256, 256, 256), (512, 768, 384), (2048, 10240, 512), (100, 70, 72), (33, 129, 40)]
+
+
+@pytest.mark.parametrize("out_dtype", ["bfloat16", "float32"])
+@pytest.mark.parametrize("shape", BF16_SHAPES)
+def test_gemm_bf16_every_variant(dev, shape, out_dtype):
+    """bf16 operands through every kernel variant that accepts the shape (same tiles, other MFMA instruction and
+    epilogue conversion): whole matrix against the fp32 product of the same bf16 values.  fp32 results to 1e-3 of
+    the largest entry (accumulation order only); bf16 results must be the fp32 result of the same variant rounded
+    to nearest even."""
+    import iree_turbine_amd as ita
+    from oracle import inputs
+
+    M, N, K = shape
+    a, b = inputs.gemm_inputs(M, N, K, seed=21, dtype=torch.bfloat16)
+    ref = a.float() @ b.float().t()
+    a, b = a.to(dev), b.to(dev)
+    names = ita._lib.variants("gemm_f16_nt")
+    ran = 0
+    for variant in [-1] + list(range(len(names))):
+        announce(f"gemm_nt bf16 {shape} out={out_dtype} variant={variant}")
+        try:
+            c = torch.ops.mi355.gemm_nt(a, b, out_dtype, variant)
+        except ValueError:
+            continue  # the variant's tile does not divide this shape
+        ran += 1
+        assert c.dtype == getattr(torch, out_dtype)
+        if out_dtype == "float32":
+            torch.testing.assert_close(c.cpu(), ref, rtol=1e-3, atol=1e-3 * ref.abs().max().item())
+        else:
+            c32 = torch.ops.mi355.gemm_nt(a, b, "float32", variant)
+            assert torch.equal(c, c32.bfloat16()), names[variant]
+            torch.testing.assert_close(c.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+    assert ran >= 2  # at least the automatic choice and the any-shape kernel
+
+
+def test_gemm_bf16_full_size(dev):
+    """8192^3 in bf16: sampled rows against the fp32 product, and the same launch twice is bit-identical."""
+    from oracle import inputs
+
+    M = N = K = 8192
+    announce("gemm_nt bf16 8192^3")
+    a, b = [t.to(dev) for t in inputs.gemm_inputs(M, N, K, dtype=torch.bfloat16)]
+    c = torch.ops.mi355.gemm_nt(a, b, "bfloat16", -1)
+    rows = torch.tensor([0, 255, 4097, M - 1], device=dev)
+    torch.testing.assert_close(c[rows].float(), a[rows].float() @ b.float().t(), rtol=RTOL, atol=ATOL)
+    assert torch.equal(c, torch.ops.mi355.gemm_nt(a, b, "bfloat16", -1))
+
+
+def test_gemm_dtype_contract(dev):
+    a16 = torch.zeros(64, 64, dtype=torch.float16, device=dev)
+    abf = torch.zeros(64, 64, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(ValueError):
+        torch.ops.mi355.gemm_nt(a16, abf, "float32", -1)  # mixed operand formats
+    with pytest.raises(ValueError):
+        torch.ops.mi355.gemm_nt(abf, abf, "float16", -1)  # 16-bit output is the operands' own format
+    with pytest.raises(ValueError):
+        torch.ops.mi355.gemm_nt(a16, a16, "bfloat16", -1)
