@@ -41,8 +41,9 @@ def _nt_operand(t: torch.Tensor, stored_transposed: bool, counter: list[int]) ->
 
 
 def _mi355_gemm(sig: GEMMSignature) -> Callable:
-    if sig.dtype != torch.float16:
-        raise UnsupportedSignature(f"{sig.func_name}: the MFMA GEMM takes fp16 operands, not {sig.dtype}")
+    if sig.dtype not in (torch.float16, torch.bfloat16):
+        raise UnsupportedSignature(f"{sig.func_name}: the MFMA GEMM takes fp16 or bf16 operands, not {sig.dtype}")
+    own = str(sig.dtype).removeprefix("torch.")
 
     def run(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
         n = [1]
@@ -53,7 +54,7 @@ def _mi355_gemm(sig: GEMMSignature) -> Callable:
             n[0] += 1
             a_mk = a_mk.contiguous()
         b_nk = _nt_operand(b, sig.transpose_b, n)
-        out = torch.ops.mi355.gemm_nt(a_mk, b_nk, "float16", -1)
+        out = torch.ops.mi355.gemm_nt(a_mk, b_nk, own, -1)
         run.dispatches = n[0]
         return out
 
@@ -63,18 +64,21 @@ def _mi355_gemm(sig: GEMMSignature) -> Callable:
 def _mi355_aten(sig: AtenSignature) -> Callable:
     kwargs = sig.concrete_kwargs()
     types = [t for (_, t, _) in sig.get_non_concrete_args()]
-    if any(t != "c10::Half" for t in types):
-        raise UnsupportedSignature(f"{sig.name}: the kernels take fp16 tensors, got {types}")
-    if sig.name == "aten::mm":
+    half_like = {"c10::Half": "float16", "c10::BFloat16": "bfloat16"}
+    if sig.name == "aten::mm" and len(set(types)) == 1 and types[0] in half_like:
+        own = half_like[types[0]]
+
         def run(a, b):
             n = [1]
             if not a.is_contiguous():
                 n[0] += 1
                 a = a.contiguous()
-            out = torch.ops.mi355.gemm_nt(a, _nt_operand(b, False, n), "float16", -1)
+            out = torch.ops.mi355.gemm_nt(a, _nt_operand(b, False, n), own, -1)
             run.dispatches = n[0]
             return out
         return run
+    if any(t != "c10::Half" for t in types):
+        raise UnsupportedSignature(f"{sig.name}: the kernels take fp16 tensors (aten::mm also bf16), got {types}")
     if sig.name == "aten::scaled_dot_product_attention":
         if kwargs.get("attn_mask") is not None or float(kwargs.get("dropout_p", 0.0) or 0.0) != 0.0:
             raise UnsupportedSignature(f"{sig.name}: attention masks and dropout are not covered")

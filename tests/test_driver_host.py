@@ -86,8 +86,12 @@ def test_aten_parser_sdpa_and_strides():
 def test_backend_rejects_what_the_kernels_do_not_cover():
     with pytest.raises(UnsupportedSignature):
         mi355_backend(parse_command(["gemm", "--a_w", "64"]))  # fp32 operands
+    # bf16 products are covered, mixed or fp32 operands are not
+    mi355_backend(parse_command(["aten::mm", "[[8, 8], [8, 8]]", "['c10::BFloat16', 'c10::BFloat16']", "[[8, 1], [8, 1]]", "['', '']"]))
     with pytest.raises(UnsupportedSignature):
-        mi355_backend(parse_command(["aten::mm", "[[8, 8], [8, 8]]", "['c10::BFloat16', 'c10::BFloat16']", "[[8, 1], [8, 1]]", "['', '']"]))
+        mi355_backend(parse_command(["aten::mm", "[[8, 8], [8, 8]]", "['c10::BFloat16', 'c10::Half']", "[[8, 1], [8, 1]]", "['', '']"]))
+    with pytest.raises(UnsupportedSignature):
+        mi355_backend(parse_command(["aten::mm", "[[8, 8], [8, 8]]", "['float', 'float']", "[[8, 1], [8, 1]]", "['', '']"]))
     with pytest.raises(UnsupportedSignature):  # head dim 64
         mi355_backend(parse_command(["aten::scaled_dot_product_attention",
                                      "[[2, 2, 16, 64], [2, 2, 16, 64], [2, 2, 16, 64], [], [], [], [], []]",

@@ -12,6 +12,7 @@ from conftest import announce
 
 pytestmark = pytest.mark.gpu
 
+MM_BF16 = ["aten::mm", "[[256, 512], [512, 384]]", "['c10::BFloat16', 'c10::BFloat16']", "[[512, 1], [384, 1]]", "['', '']"]
 SDPA_128 = ["aten::scaled_dot_product_attention",
             "[[2, 4, 256, 128], [2, 4, 256, 128], [2, 4, 256, 128], [], [], [], [], []]",
             "['c10::Half', 'c10::Half', 'c10::Half', '', 'Scalar', 'Scalar', '', 'Scalar']",
@@ -65,7 +66,7 @@ def test_commands_file_two_backends_and_layout_copy(dev, tmp_path):
 
 @pytest.mark.parametrize("cmd", [["gemmfp16", "--a_w", "512", "--a_h", "1024", "--b_w", "256", "--transB", "1"],
                                  ["gemmfp16", "--a_w", "96", "--a_h", "40", "--b_w", "72", "--transA", "1"],
-                                 MM_HALF, SDPA_128])
+                                 MM_HALF, MM_BF16, SDPA_128])
 def test_numerics_verdict_passes(dev, cmd):
     from iree_turbine_amd.driver.numerics import format_verdict_verbose, verify_numerics
 
