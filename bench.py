@@ -49,6 +49,8 @@ MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
     "fa_causal": 3.425e8,
     "fa_noncausal": 2.686e8,
     "decode": 1.177e9,
+    "fa_causal_bf16": 3.482e8,
+    "decode_bf16": 1.177e9,
     "mxfp4_4096x8192x8192": 2.947e8,
     "mxfp4_32x8192x8192": 3.739e7,
     "mxfp4_quantize_16384x16384": 6.796e8,
@@ -128,36 +130,40 @@ def wl_gemm(M, N, K, out_dtype="float16", in_dtype=torch.float16):
     return build
 
 
-def wl_attention(causal, B=2, H=32, S=4096, D=128):
+def wl_attention(causal, B=2, H=32, S=4096, D=128, bf16=False):
     from oracle import inputs
 
     def build(dev):
         q, k, v = inputs.attention_inputs(B, H, S, D)
+        if bf16:
+            q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
         qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
         flops = 4.0 * B * H * S * S * D * (0.5 if causal else 1.0)
         return {
             "fn": lambda: torch.ops.mi355.flash_attn_fwd(qd, kd, vd, causal, 0.0),
             "work": flops, "bytes": 4 * 2.0 * B * H * S * D, "bound": "mfma", "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
-            "dtype": "f16", "cpu": lambda: cpu_attention(q, k, v, causal),
-            "config": {"workload": f"flash_attn_fwd_{'causal' if causal else 'noncausal'}_B{B}_H{H}_S{S}_D{D}",
+            "dtype": "bf16" if bf16 else "f16", "cpu": lambda: cpu_attention(q, k, v, causal),
+            "config": {"workload": f"flash_attn_fwd_{'bf16_' if bf16 else ''}{'causal' if causal else 'noncausal'}_B{B}_H{H}_S{S}_D{D}",
                        "B": B, "H": H, "S": S, "D": D, "causal": causal, "seed": 10},
         }
     return build
 
 
-def wl_decode():
+def wl_decode(bf16=False):
     from oracle import inputs
 
     def build(dev):
         q, kc, vc, bt, sl = inputs.paged_decode_inputs()
+        if bf16:
+            q, kc, vc = q.bfloat16(), kc.bfloat16(), vc.bfloat16()
         args = [t.to(dev) for t in (q, kc, vc, bt, sl)]
         total = int(sl.sum())
         kv_bytes = 4096.0 * total  # 2 (K,V) * 8 kv heads * 128 * 2 B per cached token, read once
         return {
             "fn": lambda: torch.ops.mi355.paged_decode_attn(*args, 0.0, 0),
             "work": kv_bytes, "bytes": kv_bytes, "bound": "hbm", "peak": PEAK_HBM_GBS, "unit": "GB/s",
-            "dtype": "f16", "cpu": lambda: cpu_decode(q, kc, vc, bt, sl),
-            "config": {"workload": "paged_decode_64seq_32q8kv_D128_page16_ctx512-8192", "num_seqs": 64, "q_heads": 32,
+            "dtype": "bf16" if bf16 else "f16", "cpu": lambda: cpu_decode(q, kc, vc, bt, sl),
+            "config": {"workload": f"paged_decode_{'bf16_' if bf16 else ''}64seq_32q8kv_D128_page16_ctx512-8192", "num_seqs": 64, "q_heads": 32,
                        "kv_heads": 8, "D": 128, "page": 16, "total_tokens": total, "seed": 10},
         }
     return build
@@ -307,6 +313,8 @@ WORKLOADS = {
     "fa_causal": wl_attention(True),
     "fa_noncausal": wl_attention(False),
     "decode": wl_decode(),
+    "fa_causal_bf16": wl_attention(True, bf16=True),
+    "decode_bf16": wl_decode(bf16=True),
     "paged_prefill": wl_paged_prefill(),
     "mxfp4_4096x8192x8192": wl_mxfp4(4096, 8192, 8192),
     "mxfp4_32x8192x8192": wl_mxfp4(32, 8192, 8192),

@@ -113,6 +113,23 @@ int mi355_flash_attn_fwd_strided(const void* q, const void* k, const void* v, vo
                                  float scale, int is_causal, int variant, void* stream);
 
 /*
+ * bf16 forms of the two entries above: q, k, v, o bf16, fp32 online softmax, the
+ * probabilities rounded to bf16 for the second product, bf16 output.  Same kernels
+ * (instantiated with the bf16 MFMA), shapes, strides and variants.
+ * Replaces: the same SDPA root for bf16 operands -- the reference's signature
+ * parser takes the dtype from the tensor type names,
+ * iree/turbine/kernel/boo/op_exports/aten.py:101-144.
+ */
+int mi355_flash_attn_fwd_bf16(const void* q, const void* k, const void* v, void* o,
+                              int64_t B, int64_t H, int64_t Sq, int64_t Sk, int64_t D,
+                              float scale, int is_causal, int variant, void* stream);
+int mi355_flash_attn_fwd_strided_bf16(const void* q, const void* k, const void* v, void* o,
+                                      int64_t B, int64_t H, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D,
+                                      const int64_t* q_strides, const int64_t* k_strides,
+                                      const int64_t* v_strides, const int64_t* o_strides,
+                                      float scale, int is_causal, int variant, void* stream);
+
+/*
  * Paged GQA decode attention, one query token per sequence.
  * q:           [num_seqs, num_q_heads, D]                 fp16
  * k_cache,
@@ -164,10 +181,24 @@ int mi355_paged_decode_attn_window(const void* q, const void* k_cache, const voi
                                    int64_t window, void* stream);
 
 /*
+ * The same with q, k_cache, v_cache and out in bf16 (window == 0: plain paged
+ * decode).  The fp32 split-K scratch has the same layout.  For the bf16 KV cache
+ * of a bf16 model (the llama of tests/dynamo/llama_test.py runs in the dtype of
+ * its weights); mi355_kv_cache_append moves 16-bit elements and serves both.
+ */
+int mi355_paged_decode_attn_window_bf16(const void* q, const void* k_cache, const void* v_cache,
+                                        const int32_t* block_table, const int32_t* seq_lens, void* out,
+                                        float* part_acc, float* part_ml,
+                                        int64_t num_seqs, int64_t num_q_heads, int64_t num_kv_heads,
+                                        int64_t D, int64_t page_size, int64_t max_pages_per_seq,
+                                        int64_t num_pages, int64_t num_splits, float scale,
+                                        int64_t window, void* stream);
+
+/*
  * KV-cache append, the step in front of decode: the paged form of
  *   cache_k[:bsz, start_pos : start_pos + seqlen] = xk   (tests/dynamo/llama_test.py:165-166)
  * with a start position per sequence.
- * k_new, v_new: [num_seqs, n_new, num_kv_heads, D] fp16; token t of sequence s is
+ * k_new, v_new: [num_seqs, n_new, num_kv_heads, D] fp16 or bf16 (16-bit elements are moved as they are); token t of sequence s is
  * written at position start_pos[s] + t, i.e. page block_table[s][pos / page_size],
  * slot pos % page_size of k_cache / v_cache ([num_pages, page_size, num_kv_heads, D]).
  * Positions without a table entry (pos / page_size >= max_pages_per_seq) or whose
@@ -203,6 +234,13 @@ int mi355_paged_prefill_attn(const void* q, const void* k_cache, const void* v_c
                              int64_t num_seqs, int64_t num_new, int64_t num_q_heads,
                              int64_t num_kv_heads, int64_t D, int64_t page_size,
                              int64_t max_pages_per_seq, int64_t num_pages, float scale, void* stream);
+
+/* The same with q, k_cache, v_cache and out in bf16. */
+int mi355_paged_prefill_attn_bf16(const void* q, const void* k_cache, const void* v_cache,
+                                  const void* block_table, const void* seq_lens, void* out,
+                                  int64_t num_seqs, int64_t num_new, int64_t num_q_heads,
+                                  int64_t num_kv_heads, int64_t D, int64_t page_size,
+                                  int64_t max_pages_per_seq, int64_t num_pages, float scale, void* stream);
 
 /*
  * Block-scaled MXFP4 GEMM: C[M,N] = dq(A) . dq(B)^T, fp32 accumulation, bf16 out.

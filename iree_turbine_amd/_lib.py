@@ -39,6 +39,14 @@ _PROTOS = {
         c_int,
         [c_void_p] * 4 + [c_int64] * 6 + [ctypes.POINTER(c_int64)] * 4 + [c_float, c_int, c_int, c_void_p],
     ),
+    "mi355_flash_attn_fwd_bf16": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_float, c_int, c_int, c_void_p],
+    ),
+    "mi355_flash_attn_fwd_strided_bf16": (
+        c_int,
+        [c_void_p] * 4 + [c_int64] * 6 + [ctypes.POINTER(c_int64)] * 4 + [c_float, c_int, c_int, c_void_p],
+    ),
     "mi355_paged_decode_phase0": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
@@ -58,8 +66,15 @@ _PROTOS = {
         + [c_int64] * 8
         + [c_float, c_int64, c_void_p],
     ),
+    "mi355_paged_decode_attn_window_bf16": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+        + [c_int64] * 8
+        + [c_float, c_int64, c_void_p],
+    ),
     "mi355_kv_cache_append": (c_int, [c_void_p] * 6 + [c_int64] * 7 + [c_void_p]),
     "mi355_paged_prefill_attn": (c_int, [c_void_p] * 6 + [c_int64] * 8 + [c_float, c_void_p]),
+    "mi355_paged_prefill_attn_bf16": (c_int, [c_void_p] * 6 + [c_int64] * 8 + [c_float, c_void_p]),
     "mi355_mxfp4_gemm": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_void_p],

@@ -72,6 +72,58 @@ __device__ __forceinline__ unsigned short f32_to_bf16_rne(float f) {
   return (unsigned short)(u >> 16);
 }
 
+// ---- fp16 / bf16 as a template switch ----------------------------------------------------
+// Kernels that serve both 16-bit formats carry the data as opaque 16-bit lanes of half_t vectors and take a
+// `bool BF` (false = fp16, true = bf16) for the few places where the format matters: the MFMA instruction, the
+// conversions from and to fp32, the packed dot product.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+template <bool BF>
+__device__ __forceinline__ floatx16 mfma16(half8 a, half8 b, floatx16 c) {
+  if constexpr (BF)
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  else
+    return mfma_32x32x16(a, b, c);
+}
+template <bool BF>
+__device__ __forceinline__ floatx4 mfma16_16x16x32(half8 a, half8 b, floatx4 c) {
+  if constexpr (BF)
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  else
+    return mfma_16x16x32(a, b, c);
+}
+// fp32 -> the 16-bit format (round to nearest even), returned in a half_t-sized container
+template <bool BF>
+__device__ __forceinline__ half_t cvt16(float f) {
+  if constexpr (BF) return __builtin_bit_cast(half_t, (__bf16)f);
+  else return (half_t)f;
+}
+template <bool BF>
+__device__ __forceinline__ float to_f32(half_t v) {
+  if constexpr (BF) return __builtin_bit_cast(float, (unsigned)__builtin_bit_cast(unsigned short, v) << 16);
+  else return (float)v;
+}
+// two fp32 values rounded to the 16-bit format and packed; dot2_ones adds the two ROUNDED values to acc in fp32
+template <bool BF>
+__device__ __forceinline__ half2v cvt16x2(float a, float b) {
+  if constexpr (BF) {
+    bf16x2_t p = {(__bf16)a, (__bf16)b};
+    return __builtin_bit_cast(half2v, p);
+  } else {
+    return half2v{(half_t)a, (half_t)b};
+  }
+}
+template <bool BF>
+__device__ __forceinline__ float dot2_ones(half2v p, float acc) {
+  if constexpr (BF) {
+    const bf16x2_t ones = {(__bf16)1.f, (__bf16)1.f};
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, p), ones, acc, false);
+  } else {
+    const half2v ones = {(half_t)1.f, (half_t)1.f};
+    return __builtin_amdgcn_fdot2(p, ones, acc, false);
+  }
+}
+
 // ---- host side ---------------------------------------------------------------------------
 
 void set_error(const char* fmt, ...);

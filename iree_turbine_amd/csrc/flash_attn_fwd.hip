@@ -35,7 +35,7 @@ struct FaLayout {
   int H, group;
 };
 
-template <bool CAUSAL>
+template <bool CAUSAL, bool BF>
 __global__ __launch_bounds__(256) void fa_fwd_d128(const half_t* __restrict__ Q, const half_t* __restrict__ K,
                                                    const half_t* __restrict__ V, half_t* __restrict__ O, int BH, int Sq,
                                                    int Sk, float scale_log2e, int q_blocks, FaLayout lay) {
@@ -146,7 +146,7 @@ __global__ __launch_bounds__(256) void fa_fwd_d128(const half_t* __restrict__ Q,
 #pragma unroll
         for (int ks = 0; ks < 8; ks++) {
           half8 kf = *reinterpret_cast<const half8*>(st + ((k_base ^ (ks * 32)) + t * 8192));
-          s[t] = mfma_32x32x16(kf, qf[ks], s[t]);
+          s[t] = mfma16<BF>(kf, qf[ks], s[t]);
         }
       }
       const bool need_mask = (CAUSAL && (key0 + FA_BLOCK_N - 1 > wq0 + causal_off)) || (key0 + FA_BLOCK_N > Sk);
@@ -179,7 +179,7 @@ __global__ __launch_bounds__(256) void fa_fwd_d128(const half_t* __restrict__ Q,
         for (int r = 0; r < 16; r++) {
           const float p = exp2f(s[t][r] * scale_log2e - mc);
           psum += p;
-          pf[t * 2 + (r >> 3)][r & 7] = (half_t)p;
+          pf[t * 2 + (r >> 3)][r & 7] = cvt16<BF>(p);
         }
       l_run = l_run * alpha + psum;
 #pragma unroll
@@ -195,7 +195,7 @@ __global__ __launch_bounds__(256) void fa_fwd_d128(const half_t* __restrict__ Q,
           half4 lo = lds_read_tr16(va);
           half4 hi = lds_read_tr16(va + 2048);
           half8 vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-          oacc[dt] = mfma_32x32x16(vf, pf[t16], oacc[dt]);
+          oacc[dt] = mfma16<BF>(vf, pf[t16], oacc[dt]);
         }
       }
     }
@@ -212,8 +212,8 @@ __global__ __launch_bounds__(256) void fa_fwd_d128(const half_t* __restrict__ Q,
     for (int dt = 0; dt < 4; dt++)
 #pragma unroll
       for (int q = 0; q < 4; q++) {
-        half4 v = {(half_t)(oacc[dt][4 * q] * inv), (half_t)(oacc[dt][4 * q + 1] * inv), (half_t)(oacc[dt][4 * q + 2] * inv),
-                   (half_t)(oacc[dt][4 * q + 3] * inv)};
+        half4 v = {cvt16<BF>(oacc[dt][4 * q] * inv), cvt16<BF>(oacc[dt][4 * q + 1] * inv), cvt16<BF>(oacc[dt][4 * q + 2] * inv),
+                   cvt16<BF>(oacc[dt][4 * q + 3] * inv)};
         *reinterpret_cast<half4*>(orow + dt * 32 + q * 8) = v;
       }
   }
@@ -238,7 +238,7 @@ struct FaPaged {
 // the same quotient), which keeps the 64-register rescale off the common path.
 // V swizzle: chunk c of row r -> slot c ^ (4 * (r & 3)), which keeps the four 64-byte row pieces that a
 // half-wave transpose read touches on distinct banks (measured conflict-free; c ^ 2(r & 7) is not).
-template <bool CAUSAL, bool PAGED = false>
+template <bool CAUSAL, bool PAGED, bool BF>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void fa_fwd_d128_pipe(
     const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V, half_t* __restrict__ O, int BH,
     int Sq, int Sk_arg, float scale_log2e, int q_blocks, FaLayout lay, FaPaged pg) {
@@ -321,11 +321,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
   for (int ks = 0; ks < 8; ks++) {
     if (q_ok) {
-      // scale . log2(e) is folded into Q (rounded to fp16 again: a relative error of 2^-11 per element, the
-      // same size as the rounding of P to fp16), so the MFMA delivers exponents of 2 directly
+      // scale . log2(e) is folded into Q (rounded to the 16-bit format again: a relative error of 2^-11 per
+      // element for fp16, 2^-8 for bf16 -- the same size as the rounding of P), so the MFMA delivers exponents of
+      // 2 directly
       const half8 raw = *reinterpret_cast<const half8*>(Qb + (size_t)q_row * lay.q_r + ks * 16 + h * 8);
 #pragma unroll
-      for (int e = 0; e < 8; e++) qf[ks][e] = (half_t)((float)raw[e] * scale_log2e);
+      for (int e = 0; e < 8; e++) qf[ks][e] = cvt16<BF>(to_f32<BF>(raw[e]) * scale_log2e);
     } else {
 #pragma unroll
       for (int e = 0; e < 8; e++) qf[ks][e] = (half_t)0;
@@ -412,7 +413,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
       for (int ks = 0; ks < 8; ks++) {
         half8 kf = *reinterpret_cast<const half8*>(lds + koff + t * 8192 + (k_base ^ (ks * 32)));
-        s[t] = mfma_32x32x16(kf, qf[ks], ks == 0 ? negm : s[t]);
+        s[t] = mfma16<BF>(kf, qf[ks], ks == 0 ? negm : s[t]);
       }
     }
   };
@@ -471,13 +472,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // (Past the last tile the scores are computed from stale LDS bytes and never used.)
     __builtin_amdgcn_sched_barrier(0);
     scores(koff_next, s_next);
-    const half2v ones = {(half_t)1.f, (half_t)1.f};
 #pragma unroll
     for (int t = 0; t < 2; t++)
 #pragma unroll
       for (int r = 0; r < 16; r += 2) {
-        const half2v pp = {(half_t)__builtin_amdgcn_exp2f(s[t][r]), (half_t)__builtin_amdgcn_exp2f(s[t][r + 1])};
-        psum = __builtin_amdgcn_fdot2(pp, ones, psum, false);  // sums what the second MFMA multiplies
+        const half2v pp = cvt16x2<BF>(__builtin_amdgcn_exp2f(s[t][r]), __builtin_amdgcn_exp2f(s[t][r + 1]));
+        psum = dot2_ones<BF>(pp, psum);  // sums what the second MFMA multiplies
         pf[t * 2 + (r >> 3)][r & 7] = pp[0];
         pf[t * 2 + (r >> 3)][(r & 7) + 1] = pp[1];
       }
@@ -513,7 +513,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int i = 0; i < 16; i++) {
       if (i + 2 < 16) vf[(i + 2) % 3] = vr(i + 2);
-      oacc[i & 3] = mfma_32x32x16(vf[i % 3], pf[i >> 2], oacc[i & 3]);
+      oacc[i & 3] = mfma16<BF>(vf[i % 3], pf[i >> 2], oacc[i & 3]);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -564,8 +564,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int dt = 0; dt < 4; dt++)
 #pragma unroll
       for (int q = 0; q < 4; q++) {
-        half4 v = {(half_t)(oacc[dt][4 * q] * inv), (half_t)(oacc[dt][4 * q + 1] * inv), (half_t)(oacc[dt][4 * q + 2] * inv),
-                   (half_t)(oacc[dt][4 * q + 3] * inv)};
+        half4 v = {cvt16<BF>(oacc[dt][4 * q] * inv), cvt16<BF>(oacc[dt][4 * q + 1] * inv), cvt16<BF>(oacc[dt][4 * q + 2] * inv),
+                   cvt16<BF>(oacc[dt][4 * q + 3] * inv)};
         *reinterpret_cast<half4*>(orow + dt * 32 + q * 8) = v;
       }
   }
@@ -580,6 +580,7 @@ const char* fa_variant_name(int i) { return (i >= 0 && i < 2) ? kFaVariants[i] :
 
 using namespace mi355;
 
+template <bool BF>
 static int fa_launch(const void* q, const void* k, const void* v, void* o, int64_t B, int64_t H, int64_t Hkv, int64_t Sq,
                      int64_t Sk, int64_t D, const FaLayout& lay, float scale, int is_causal, int variant, void* stream,
                      const char* who) {
@@ -598,9 +599,9 @@ static int fa_launch(const void* q, const void* k, const void* v, void* o, int64
   const int q_blocks = (int)((Sq + FA_BLOCK_M - 1) / FA_BLOCK_M);
   const int lds_bytes = 2 * FA_STAGE;
   static std::atomic<uint64_t> lds_ok[4] = {};
-  const void* kernels[4] = {reinterpret_cast<const void*>(fa_fwd_d128<true>), reinterpret_cast<const void*>(fa_fwd_d128<false>),
-                            reinterpret_cast<const void*>(fa_fwd_d128_pipe<true, false>),
-                            reinterpret_cast<const void*>(fa_fwd_d128_pipe<false, false>)};
+  const void* kernels[4] = {reinterpret_cast<const void*>(fa_fwd_d128<true, BF>), reinterpret_cast<const void*>(fa_fwd_d128<false, BF>),
+                            reinterpret_cast<const void*>(fa_fwd_d128_pipe<true, false, BF>),
+                            reinterpret_cast<const void*>(fa_fwd_d128_pipe<false, false, BF>)};
   for (int i = 0; i < 4; i++)
     if (int rc = allow_lds(kernels[i], lds_bytes, lds_ok[i], "fa_fwd_d128")) return rc;
   const float scale_log2e = scale * 1.4426950408889634f;
@@ -609,32 +610,44 @@ static int fa_launch(const void* q, const void* k, const void* v, void* o, int64
   dim3 grid(BH * units), block(256);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (variant == 1) {
-    auto kern = is_causal ? fa_fwd_d128<true> : fa_fwd_d128<false>;
+    auto kern = is_causal ? fa_fwd_d128<true, BF> : fa_fwd_d128<false, BF>;
     hipLaunchKernelGGL(kern, grid, block, lds_bytes, s, (const half_t*)q, (const half_t*)k, (const half_t*)v, (half_t*)o, BH,
                        (int)Sq, (int)Sk, scale_log2e, q_blocks, lay);
   } else {
-    auto kern = is_causal ? fa_fwd_d128_pipe<true, false> : fa_fwd_d128_pipe<false, false>;
+    auto kern = is_causal ? fa_fwd_d128_pipe<true, false, BF> : fa_fwd_d128_pipe<false, false, BF>;
     hipLaunchKernelGGL(kern, grid, block, lds_bytes, s, (const half_t*)q, (const half_t*)k, (const half_t*)v, (half_t*)o, BH,
                        (int)Sq, (int)Sk, scale_log2e, q_blocks, lay, FaPaged{nullptr, nullptr, 0, 0, 0});
   }
   return check_launch(variant == 1 ? "fa_fwd_d128" : "fa_fwd_d128_pipe", grid, block, lds_bytes);
 }
 
-extern "C" int mi355_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, int64_t B, int64_t H, int64_t Sq,
-                                    int64_t Sk, int64_t D, float scale, int is_causal, int variant, void* stream) {
+template <bool BF>
+static int fa_contiguous(const void* q, const void* k, const void* v, void* o, int64_t B, int64_t H, int64_t Sq, int64_t Sk,
+                         int64_t D, float scale, int is_causal, int variant, void* stream) {
   FaLayout lay;
   lay.q_b = H * Sq * 128, lay.q_h = Sq * 128, lay.q_r = 128;
   lay.o_b = lay.q_b, lay.o_h = lay.q_h, lay.o_r = 128;
   lay.k_b = lay.v_b = H * Sk * 128, lay.k_h = lay.v_h = Sk * 128, lay.k_r = lay.v_r = 128;
   lay.H = (int)H, lay.group = 1;
-  return fa_launch(q, k, v, o, B, H, H, Sq, Sk, D, lay, scale, is_causal, variant, stream, "flash_attn_fwd");
+  return fa_launch<BF>(q, k, v, o, B, H, H, Sq, Sk, D, lay, scale, is_causal, variant, stream,
+                       BF ? "flash_attn_fwd_bf16" : "flash_attn_fwd");
 }
 
-extern "C" int mi355_flash_attn_fwd_strided(const void* q, const void* k, const void* v, void* o, int64_t B, int64_t H,
-                                            int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, const int64_t* q_strides,
-                                            const int64_t* k_strides, const int64_t* v_strides, const int64_t* o_strides,
-                                            float scale, int is_causal, int variant, void* stream) {
-  const char* who = "flash_attn_fwd_strided";
+extern "C" int mi355_flash_attn_fwd(const void* q, const void* k, const void* v, void* o, int64_t B, int64_t H, int64_t Sq,
+                                    int64_t Sk, int64_t D, float scale, int is_causal, int variant, void* stream) {
+  return fa_contiguous<false>(q, k, v, o, B, H, Sq, Sk, D, scale, is_causal, variant, stream);
+}
+
+extern "C" int mi355_flash_attn_fwd_bf16(const void* q, const void* k, const void* v, void* o, int64_t B, int64_t H, int64_t Sq,
+                                         int64_t Sk, int64_t D, float scale, int is_causal, int variant, void* stream) {
+  return fa_contiguous<true>(q, k, v, o, B, H, Sq, Sk, D, scale, is_causal, variant, stream);
+}
+
+template <bool BF>
+static int fa_strided(const void* q, const void* k, const void* v, void* o, int64_t B, int64_t H, int64_t Hkv, int64_t Sq,
+                      int64_t Sk, int64_t D, const int64_t* q_strides, const int64_t* k_strides, const int64_t* v_strides,
+                      const int64_t* o_strides, float scale, int is_causal, int variant, void* stream) {
+  const char* who = BF ? "flash_attn_fwd_strided_bf16" : "flash_attn_fwd_strided";
   if (!q_strides || !k_strides || !v_strides || !o_strides) return fail(-MI355_E_NULL, "%s: null stride array", who);
   const int64_t* all[4] = {q_strides, k_strides, v_strides, o_strides};
   for (const int64_t* st : all) {
@@ -650,14 +663,30 @@ extern "C" int mi355_flash_attn_fwd_strided(const void* q, const void* k, const 
   lay.v_b = v_strides[0], lay.v_h = v_strides[1], lay.v_r = (unsigned)v_strides[2];
   lay.o_b = o_strides[0], lay.o_h = o_strides[1], lay.o_r = (unsigned)o_strides[2];
   lay.H = (int)H, lay.group = Hkv > 0 ? (int)(H / Hkv) : 1;
-  return fa_launch(q, k, v, o, B, H, Hkv, Sq, Sk, D, lay, scale, is_causal, variant, stream, who);
+  return fa_launch<BF>(q, k, v, o, B, H, Hkv, Sq, Sk, D, lay, scale, is_causal, variant, stream, who);
 }
 
-extern "C" int mi355_paged_prefill_attn(const void* q, const void* k_cache, const void* v_cache, const void* block_table,
-                                        const void* seq_lens, void* out, int64_t num_seqs, int64_t num_new, int64_t num_q_heads,
-                                        int64_t num_kv_heads, int64_t D, int64_t page_size, int64_t max_pages_per_seq,
-                                        int64_t num_pages, float scale, void* stream) {
-  const char* who = "paged_prefill_attn";
+extern "C" int mi355_flash_attn_fwd_strided(const void* q, const void* k, const void* v, void* o, int64_t B, int64_t H,
+                                            int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, const int64_t* q_strides,
+                                            const int64_t* k_strides, const int64_t* v_strides, const int64_t* o_strides,
+                                            float scale, int is_causal, int variant, void* stream) {
+  return fa_strided<false>(q, k, v, o, B, H, Hkv, Sq, Sk, D, q_strides, k_strides, v_strides, o_strides, scale, is_causal, variant,
+                           stream);
+}
+
+extern "C" int mi355_flash_attn_fwd_strided_bf16(const void* q, const void* k, const void* v, void* o, int64_t B, int64_t H,
+                                                 int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, const int64_t* q_strides,
+                                                 const int64_t* k_strides, const int64_t* v_strides, const int64_t* o_strides,
+                                                 float scale, int is_causal, int variant, void* stream) {
+  return fa_strided<true>(q, k, v, o, B, H, Hkv, Sq, Sk, D, q_strides, k_strides, v_strides, o_strides, scale, is_causal, variant,
+                          stream);
+}
+
+template <bool BF>
+static int fa_paged_prefill(const void* q, const void* k_cache, const void* v_cache, const void* block_table, const void* seq_lens,
+                            void* out, int64_t num_seqs, int64_t num_new, int64_t num_q_heads, int64_t num_kv_heads, int64_t D,
+                            int64_t page_size, int64_t max_pages_per_seq, int64_t num_pages, float scale, void* stream) {
+  const char* who = BF ? "paged_prefill_attn_bf16" : "paged_prefill_attn";
   if (!q || !k_cache || !v_cache || !block_table || !seq_lens || !out) return fail(-MI355_E_NULL, "%s: null pointer", who);
   if (D != 128) return fail(-MI355_E_SHAPE, "%s: head dim %lld not supported (only 128)", who, (long long)D);
   int page_shift = -1;
@@ -684,7 +713,7 @@ extern "C" int mi355_paged_prefill_attn(const void* q, const void* k_cache, cons
   const int BH = (int)(num_seqs * num_q_heads);
   const int q_blocks = (int)((num_new + FA_BLOCK_M - 1) / FA_BLOCK_M);
   const int lds_bytes = 2 * FA_STAGE;
-  auto kern = fa_fwd_d128_pipe<true, true>;
+  auto kern = fa_fwd_d128_pipe<true, true, BF>;
   static std::atomic<uint64_t> lds_ok{0};
   if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "fa_fwd_d128_pipe")) return rc;
   dim3 grid(BH * ((q_blocks + 1) / 2)), block(256);
@@ -693,4 +722,20 @@ extern "C" int mi355_paged_prefill_attn(const void* q, const void* k_cache, cons
   hipLaunchKernelGGL(kern, grid, block, lds_bytes, reinterpret_cast<hipStream_t>(stream), (const half_t*)q, (const half_t*)k_cache,
                      (const half_t*)v_cache, (half_t*)out, BH, (int)num_new, 0, scale * 1.4426950408889634f, q_blocks, lay, pg);
   return check_launch("fa_fwd_d128_pipe<paged>", grid, block, lds_bytes);
+}
+
+extern "C" int mi355_paged_prefill_attn(const void* q, const void* k_cache, const void* v_cache, const void* block_table,
+                                        const void* seq_lens, void* out, int64_t num_seqs, int64_t num_new, int64_t num_q_heads,
+                                        int64_t num_kv_heads, int64_t D, int64_t page_size, int64_t max_pages_per_seq,
+                                        int64_t num_pages, float scale, void* stream) {
+  return fa_paged_prefill<false>(q, k_cache, v_cache, block_table, seq_lens, out, num_seqs, num_new, num_q_heads, num_kv_heads, D,
+                                 page_size, max_pages_per_seq, num_pages, scale, stream);
+}
+
+extern "C" int mi355_paged_prefill_attn_bf16(const void* q, const void* k_cache, const void* v_cache, const void* block_table,
+                                             const void* seq_lens, void* out, int64_t num_seqs, int64_t num_new,
+                                             int64_t num_q_heads, int64_t num_kv_heads, int64_t D, int64_t page_size,
+                                             int64_t max_pages_per_seq, int64_t num_pages, float scale, void* stream) {
+  return fa_paged_prefill<true>(q, k_cache, v_cache, block_table, seq_lens, out, num_seqs, num_new, num_q_heads, num_kv_heads, D,
+                                page_size, max_pages_per_seq, num_pages, scale, stream);
 }

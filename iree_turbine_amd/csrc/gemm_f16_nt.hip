@@ -26,24 +26,9 @@
 
 namespace mi355 {
 
-// BF selects the 16-bit input format: false = fp16, true = bf16.  Both travel through the kernels as opaque
-// 16-bit lanes of half8 / half4 vectors (same tiles, same LDS format, same fragment layout); only the MFMA
-// instruction and the conversion of the fp32 sums in the epilogue differ.
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-template <bool BF>
-__device__ __forceinline__ floatx16 mfma16(half8 a, half8 b, floatx16 c) {
-  if constexpr (BF)
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
-  else
-    return mfma_32x32x16(a, b, c);
-}
-// fp32 -> the 16-bit output format (round to nearest even), returned in a half_t-sized container
-template <bool BF>
-__device__ __forceinline__ half_t cvt16(float f) {
-  if constexpr (BF) return __builtin_bit_cast(half_t, f32_to_bf16_rne(f));
-  else return (half_t)f;
-}
-
+// BF selects the 16-bit input format (false = fp16, true = bf16; mfma16 / cvt16 of the shared header).  Both travel
+// through the kernels as opaque 16-bit lanes of half8 / half4 vectors (same tiles, same LDS format, same fragment
+// layout); only the MFMA instruction and the conversion of the fp32 sums in the epilogue differ.
 template <typename OutT, bool BF> struct OutPack;
 template <bool BF> struct OutPack<float, BF> {
   static __device__ __forceinline__ void store4(float* p, float a, float b, float c, float d) {

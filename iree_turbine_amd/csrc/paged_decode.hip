@@ -28,7 +28,7 @@ constexpr int PD_WAVE_LDS = 2 * 8192;  // two stages of two 4 KiB V pages
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-template <int G>  // q heads per kv head (<= 16)
+template <int G, bool BF>  // G = q heads per kv head (<= 16); BF = bf16 instead of fp16 operands and output
 __global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
     const half_t* __restrict__ Q, const half_t* __restrict__ Kc, const half_t* __restrict__ Vc,
     const int* __restrict__ block_table, const int* __restrict__ seq_lens, float* __restrict__ part_acc,
@@ -148,9 +148,9 @@ __global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
         const bool has1 = pa + 1 < p_end;
         floatx4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int ks = 0; ks < 4; ks++) s0 = mfma_16x16x32(kf[b][0][ks], qf[ks], s0);
+        for (int ks = 0; ks < 4; ks++) s0 = mfma16_16x16x32<BF>(kf[b][0][ks], qf[ks], s0);
 #pragma unroll
-        for (int ks = 0; ks < 4; ks++) s1 = mfma_16x16x32(kf[b][1][ks], qf[ks], s1);
+        for (int ks = 0; ks < 4; ks++) s1 = mfma16_16x16x32<BF>(kf[b][1][ks], qf[ks], s1);
         // lane (head i16, g) holds tokens 4g + r of each page
         const int tok0 = pa * 16 + 4 * g;
         const bool ragged = pa * 16 + 32 > L;  // wave-uniform: this step reaches past the sequence end
@@ -173,8 +173,8 @@ __global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
           const float p0 = fast_exp2(s0[r] * scale_log2e - mc);
           const float p1 = fast_exp2(s1[r] * scale_log2e - mc);
           psum += p0 + p1;
-          pf[r] = (half_t)p0;
-          pf[4 + r] = (half_t)p1;
+          pf[r] = cvt16<BF>(p0);
+          pf[4 + r] = cvt16<BF>(p1);
         }
         l_run = l_run * alpha + psum;
         const char* vst = my_lds + b * 8192;
@@ -191,7 +191,7 @@ __global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
           }
           half8 vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
           oacc[dt] = oacc[dt] * alpha;
-          oacc[dt] = mfma_16x16x32(vf, pf, oacc[dt]);
+          oacc[dt] = mfma16_16x16x32<BF>(vf, pf, oacc[dt]);
         }
       }
     }
@@ -231,7 +231,7 @@ __global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
     }
     const int qh = kvh * G + hd;
     if (out) {
-      out[((size_t)seq * num_q_heads + qh) * 128 + d] = (half_t)(l > 0.f ? acc / l : 0.f);
+      out[((size_t)seq * num_q_heads + qh) * 128 + d] = cvt16<BF>(l > 0.f ? acc / l : 0.f);
     } else {
       const size_t pidx = ((size_t)seq * num_q_heads + qh) * num_splits + split;
       part_acc[pidx * 128 + d] = acc;
@@ -244,6 +244,7 @@ __global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
 }
 
 // Phase 1: one wave per (seq, q head); lane handles d = 2*lane, 2*lane + 1.
+template <bool BF>
 __global__ __launch_bounds__(64) void paged_decode_phase1(const float* __restrict__ part_acc,
                                                           const float* __restrict__ part_ml, half_t* __restrict__ out,
                                                           int num_splits) {
@@ -266,7 +267,7 @@ __global__ __launch_bounds__(64) void paged_decode_phase1(const float* __restric
     }
   }
   const float inv = l > 0.f ? 1.f / l : 0.f;
-  half2v o = {(half_t)(acc[0] * inv), (half_t)(acc[1] * inv)};
+  half2v o = {cvt16<BF>(acc[0] * inv), cvt16<BF>(acc[1] * inv)};
   *reinterpret_cast<half2v*>(out + row * 128 + 2 * lane) = o;
 }
 
@@ -274,11 +275,11 @@ static const char* kDecodeVariants[] = {"d128_p16_w4_2pages"};
 int decode_variant_count() { return 1; }
 const char* decode_variant_name(int i) { return i == 0 ? kDecodeVariants[0] : nullptr; }
 
-template <int G>
+template <int G, bool BF>
 static int launch_phase0(const void* q, const void* kc, const void* vc, const int32_t* bt, const int32_t* sl, float* pacc,
                          float* pml, void* out, int num_seqs, int num_kv_heads, int max_pages, int num_splits, float scale,
                          int window, int page_shift, hipStream_t stream) {
-  auto kern = paged_decode_phase0<G>;
+  auto kern = paged_decode_phase0<G, BF>;
   constexpr int lds_bytes = PD_WAVES * PD_WAVE_LDS;
   static_assert(lds_bytes >= (int)((2 * PD_WAVES * 16 + PD_WAVES * G * 128) * sizeof(float)), "merge area must fit");
   static std::atomic<uint64_t> lds_ok{0};
@@ -315,12 +316,13 @@ static int check_decode_args(const char* fn, int64_t num_seqs, int64_t hq, int64
   return 0;
 }
 
+template <bool BF>
 static int run_phase0(const void* q, const void* kc, const void* vc, const int32_t* bt, const int32_t* sl, float* pacc,
                       float* pml, void* out, int64_t num_seqs, int64_t hq, int64_t hkv, int64_t max_pages,
                       int64_t num_splits, float scale, int window, int page_shift, hipStream_t stream) {
   const int G = (int)(hq / hkv);
 #define MI355_PD_CASE(GG) \
-  case GG: return launch_phase0<GG>(q, kc, vc, bt, sl, pacc, pml, out, (int)num_seqs, (int)hkv, (int)max_pages, (int)num_splits, scale, window, page_shift, stream)
+  case GG: return launch_phase0<GG, BF>(q, kc, vc, bt, sl, pacc, pml, out, (int)num_seqs, (int)hkv, (int)max_pages, (int)num_splits, scale, window, page_shift, stream)
   switch (G) {
     MI355_PD_CASE(1);
     MI355_PD_CASE(2);
@@ -348,22 +350,30 @@ extern "C" int mi355_paged_decode_phase0(const void* q, const void* k_cache, con
   if (!part_acc || !part_ml) return fail(-MI355_E_SCRATCH, "paged_decode_phase0: part_acc / part_ml scratch is required");
   if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(part_acc))
     return fail(-MI355_E_ALIGN, "paged_decode_phase0: q, k_cache, v_cache, part_acc must be 16-byte aligned");
-  return run_phase0(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, nullptr, num_seqs, num_q_heads,
-                    num_kv_heads, max_pages_per_seq, num_splits, scale, 0, page_shift_of(page_size), reinterpret_cast<hipStream_t>(stream));
+  return run_phase0<false>(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, nullptr, num_seqs, num_q_heads,
+                           num_kv_heads, max_pages_per_seq, num_splits, scale, 0, page_shift_of(page_size),
+                           reinterpret_cast<hipStream_t>(stream));
 }
 
-extern "C" int mi355_paged_decode_phase1(const float* part_acc, const float* part_ml, void* out, int64_t num_seqs,
-                                         int64_t num_q_heads, int64_t D, int64_t num_splits, void* stream) {
+template <bool BF>
+static int run_phase1(const float* part_acc, const float* part_ml, void* out, int64_t num_seqs, int64_t num_q_heads, int64_t D,
+                      int64_t num_splits, void* stream) {
   if (!part_acc || !part_ml || !out) return fail(-MI355_E_NULL, "paged_decode_phase1: null pointer");
   if (D != 128) return fail(-MI355_E_SHAPE, "paged_decode_phase1: head dim %lld not supported (only 128)", (long long)D);
   if (num_seqs <= 0 || num_q_heads <= 0 || num_splits < 1 || num_splits > 1024 || num_seqs * num_q_heads > (1ll << 30))
     return fail(-MI355_E_SHAPE, "paged_decode_phase1: bad sizes");
   dim3 grid((unsigned)(num_seqs * num_q_heads)), block(64);
-  hipLaunchKernelGGL(paged_decode_phase1, grid, block, 0, reinterpret_cast<hipStream_t>(stream), part_acc, part_ml,
+  hipLaunchKernelGGL(paged_decode_phase1<BF>, grid, block, 0, reinterpret_cast<hipStream_t>(stream), part_acc, part_ml,
                      (half_t*)out, (int)num_splits);
   return check_launch("paged_decode_phase1", grid, block, 0);
 }
 
+extern "C" int mi355_paged_decode_phase1(const float* part_acc, const float* part_ml, void* out, int64_t num_seqs,
+                                         int64_t num_q_heads, int64_t D, int64_t num_splits, void* stream) {
+  return run_phase1<false>(part_acc, part_ml, out, num_seqs, num_q_heads, D, num_splits, stream);
+}
+
+template <bool BF>
 static int decode_attn(const char* fn, const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
                        const int32_t* seq_lens, void* out, float* part_acc, float* part_ml, int64_t num_seqs,
                        int64_t num_q_heads, int64_t num_kv_heads, int64_t D, int64_t page_size, int64_t max_pages_per_seq,
@@ -377,14 +387,14 @@ static int decode_attn(const char* fn, const void* q, const void* k_cache, const
     return fail(-MI355_E_ALIGN, "%s: q, k_cache, v_cache, out must be 16-byte aligned", fn);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (num_splits == 1)
-    return run_phase0(q, k_cache, v_cache, block_table, seq_lens, nullptr, nullptr, out, num_seqs, num_q_heads, num_kv_heads,
-                      max_pages_per_seq, 1, scale, (int)window, page_shift_of(page_size), s);
+    return run_phase0<BF>(q, k_cache, v_cache, block_table, seq_lens, nullptr, nullptr, out, num_seqs, num_q_heads, num_kv_heads,
+                          max_pages_per_seq, 1, scale, (int)window, page_shift_of(page_size), s);
   if (!part_acc || !part_ml) return fail(-MI355_E_SCRATCH, "%s: num_splits > 1 needs part_acc / part_ml scratch", fn);
   if (!aligned16(part_acc)) return fail(-MI355_E_ALIGN, "%s: part_acc must be 16-byte aligned", fn);
-  if (int rc = run_phase0(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, nullptr, num_seqs, num_q_heads,
-                          num_kv_heads, max_pages_per_seq, num_splits, scale, (int)window, page_shift_of(page_size), s))
+  if (int rc = run_phase0<BF>(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, nullptr, num_seqs, num_q_heads,
+                              num_kv_heads, max_pages_per_seq, num_splits, scale, (int)window, page_shift_of(page_size), s))
     return rc;
-  return mi355_paged_decode_phase1(part_acc, part_ml, out, num_seqs, num_q_heads, D, num_splits, stream);
+  return run_phase1<BF>(part_acc, part_ml, out, num_seqs, num_q_heads, D, num_splits, stream);
 }
 
 extern "C" int mi355_paged_decode_attn(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
@@ -392,7 +402,7 @@ extern "C" int mi355_paged_decode_attn(const void* q, const void* k_cache, const
                                        int64_t num_q_heads, int64_t num_kv_heads, int64_t D, int64_t page_size,
                                        int64_t max_pages_per_seq, int64_t num_pages, int64_t num_splits, float scale,
                                        void* stream) {
-  return decode_attn("paged_decode_attn", q, k_cache, v_cache, block_table, seq_lens, out, part_acc, part_ml, num_seqs,
+  return decode_attn<false>("paged_decode_attn", q, k_cache, v_cache, block_table, seq_lens, out, part_acc, part_ml, num_seqs,
                      num_q_heads, num_kv_heads, D, page_size, max_pages_per_seq, num_pages, num_splits, scale, 0, stream);
 }
 
@@ -401,8 +411,20 @@ extern "C" int mi355_paged_decode_attn_window(const void* q, const void* k_cache
                                               float* part_ml, int64_t num_seqs, int64_t num_q_heads, int64_t num_kv_heads,
                                               int64_t D, int64_t page_size, int64_t max_pages_per_seq, int64_t num_pages,
                                               int64_t num_splits, float scale, int64_t window, void* stream) {
-  return decode_attn("paged_decode_attn_window", q, k_cache, v_cache, block_table, seq_lens, out, part_acc, part_ml, num_seqs,
-                     num_q_heads, num_kv_heads, D, page_size, max_pages_per_seq, num_pages, num_splits, scale, window, stream);
+  return decode_attn<false>("paged_decode_attn_window", q, k_cache, v_cache, block_table, seq_lens, out, part_acc, part_ml,
+                            num_seqs, num_q_heads, num_kv_heads, D, page_size, max_pages_per_seq, num_pages, num_splits, scale,
+                            window, stream);
+}
+
+extern "C" int mi355_paged_decode_attn_window_bf16(const void* q, const void* k_cache, const void* v_cache,
+                                                   const int32_t* block_table, const int32_t* seq_lens, void* out,
+                                                   float* part_acc, float* part_ml, int64_t num_seqs, int64_t num_q_heads,
+                                                   int64_t num_kv_heads, int64_t D, int64_t page_size,
+                                                   int64_t max_pages_per_seq, int64_t num_pages, int64_t num_splits,
+                                                   float scale, int64_t window, void* stream) {
+  return decode_attn<true>("paged_decode_attn_window_bf16", q, k_cache, v_cache, block_table, seq_lens, out, part_acc, part_ml,
+                           num_seqs, num_q_heads, num_kv_heads, D, page_size, max_pages_per_seq, num_pages, num_splits, scale,
+                           window, stream);
 }
 
 // ---- KV-cache append: the step in front of decode -------------------------------------------------------

@@ -15,8 +15,7 @@ substitution is a direct FX rewrite of the ATen graph that AOT-autograd produces
   aten._scaled_dot_product_{flash,efficient,flash_for_cpu}_attention(q, k, v, ...)[0]
                               -> mi355.flash_attn_fwd(q, k, v, is_causal, scale)
 
-A node is rewritten only when the kernels cover it (fp16 -- for mm / addmm also bf16 -- tensors on a CUDA device,
-head dim 128, no mask, no dropout, auxiliary outputs unused -- so training graphs keep PyTorch's attention); everything else is left
+A node is rewritten only when the kernels cover it (fp16 or bf16 tensors of one dtype on a CUDA device, head dim 128, no mask, no dropout, auxiliary outputs unused -- so training graphs keep PyTorch's attention); everything else is left
 for the nested backend.  Layouts: the ops make their operands contiguous themselves, so transposed views
 (`q.transpose(1, 2)`) need no graph surgery.
 """
@@ -126,7 +125,9 @@ def _rewrite_sdpa(node: fx.Node, device_ok) -> bool:
     if float(bound.get("dropout_p", 0.0) or 0.0) != 0.0:
         return False
     vals = [_val(t) for t in (q, k, v)]
-    if not all(isinstance(t, torch.Tensor) and t.dim() == 4 and t.dtype == torch.float16 and device_ok(t.device) for t in vals):
+    if not all(isinstance(t, torch.Tensor) and t.dim() == 4 and t.dtype in _GEMM_DTYPES and device_ok(t.device) for t in vals):
+        return False
+    if len({t.dtype for t in vals}) != 1:
         return False
     qv, kv, vv = vals
     if qv.shape[-1] != 128 or kv.shape != vv.shape or qv.shape[0] != kv.shape[0] or kv.shape[-1] != 128:

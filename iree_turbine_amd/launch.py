@@ -24,6 +24,14 @@ def _dev(*tensors: Tensor) -> torch.device:
     return dev
 
 
+def _half_dtype(name: str, *tensors: Tensor) -> torch.dtype:
+    """The one 16-bit float format (fp16 or bf16) that all of `tensors` share; the kernels exist for both."""
+    dt = tensors[0].dtype
+    if dt not in (torch.float16, torch.bfloat16) or any(t.dtype != dt for t in tensors):
+        raise ValueError(f"{name}: tensors must all be float16 or all bfloat16, got {[str(t.dtype) for t in tensors]}")
+    return dt
+
+
 def _contig_out(t: Tensor, name: str) -> None:
     if not t.is_contiguous():
         raise ValueError(f"{name}: output tensors must be contiguous")  # runtime/launch.py:246
@@ -73,8 +81,9 @@ def flash_attn_fwd_out(q: Tensor, k: Tensor, v: Tensor, o: Tensor, is_causal: bo
     dev = _dev(q, k, v, o)
     B, H, Sq, D = q.shape
     Hkv, Sk = k.shape[1], k.shape[2]
-    if o.shape != q.shape or o.dtype != torch.float16:
-        raise ValueError("flash_attn_fwd: o must be float16 with q's shape")
+    dt = _half_dtype("flash_attn_fwd", q, k, v, o)
+    if o.shape != q.shape:
+        raise ValueError("flash_attn_fwd: o must have q's shape")
     if scale is None or scale <= 0:
         scale = 1.0 / math.sqrt(D)
     ins = []
@@ -88,11 +97,13 @@ def flash_attn_fwd_out(q: Tensor, k: Tensor, v: Tensor, o: Tensor, is_causal: bo
     if o_st is None or (B > 1 and o_st[0] == 0) or (H > 1 and o_st[1] == 0):
         raise ValueError("flash_attn_fwd: output rows must be contiguous, 16-byte aligned and not overlapping")  # runtime/launch.py:246
     arr = lambda st: (ctypes.c_int64 * 3)(*st)
+    lib = _lib.load()
+    entry = lib.mi355_flash_attn_fwd_strided_bf16 if dt == torch.bfloat16 else lib.mi355_flash_attn_fwd_strided
     with torch.cuda.device(dev):
-        rc = _lib.load().mi355_flash_attn_fwd_strided(ins[0][0].data_ptr(), ins[1][0].data_ptr(), ins[2][0].data_ptr(), o.data_ptr(),
-                                                      B, H, Hkv, Sq, Sk, D, arr(ins[0][1]), arr(ins[1][1]), arr(ins[2][1]), arr(o_st),
-                                                      scale, int(bool(is_causal)), variant, _lib.current_stream_ptr(dev))
-    _lib.check(rc, f"flash_attn_fwd B={B} H={H} Hkv={Hkv} Sq={Sq} Sk={Sk} D={D} causal={is_causal}")
+        rc = entry(ins[0][0].data_ptr(), ins[1][0].data_ptr(), ins[2][0].data_ptr(), o.data_ptr(), B, H, Hkv, Sq, Sk, D,
+                   arr(ins[0][1]), arr(ins[1][1]), arr(ins[2][1]), arr(o_st), scale, int(bool(is_causal)), variant,
+                   _lib.current_stream_ptr(dev))
+    _lib.check(rc, f"flash_attn_fwd {dt} B={B} H={H} Hkv={Hkv} Sq={Sq} Sk={Sk} D={D} causal={is_causal}")
     return o
 
 
@@ -138,8 +149,9 @@ def paged_decode_attn_out(q, k_cache, v_cache, block_table, seq_lens, out, scale
     _contig_out(out, "paged_decode_attn")
     S, Hq, D = q.shape
     P, page, Hkv, _ = k_cache.shape
-    if out.shape != q.shape or out.dtype != torch.float16:
-        raise ValueError("paged_decode_attn: out must be float16 with q's shape")
+    dt = _half_dtype("paged_decode_attn", q, k_cache, v_cache, out)
+    if out.shape != q.shape:
+        raise ValueError("paged_decode_attn: out must have q's shape")
     if scale is None or scale <= 0:
         scale = 1.0 / math.sqrt(D)
     if num_kv_splits > 1:
@@ -152,7 +164,12 @@ def paged_decode_attn_out(q, k_cache, v_cache, block_table, seq_lens, out, scale
     if window < 0:
         raise ValueError(f"paged_decode_attn: window must be >= 0, got {window}")
     with torch.cuda.device(dev):
-        if window == 0:
+        if dt == torch.bfloat16:
+            rc = _lib.load().mi355_paged_decode_attn_window_bf16(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                                                                 block_table.data_ptr(), seq_lens.data_ptr(), out.data_ptr(), pa,
+                                                                 pm, S, Hq, Hkv, D, page, block_table.shape[1], P, num_kv_splits,
+                                                                 scale, window, _lib.current_stream_ptr(dev))
+        elif window == 0:
             rc = _lib.load().mi355_paged_decode_attn(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
                                                      seq_lens.data_ptr(), out.data_ptr(), pa, pm, S, Hq, Hkv, D, page,
                                                      block_table.shape[1], P, num_kv_splits, scale, _lib.current_stream_ptr(dev))
@@ -161,7 +178,7 @@ def paged_decode_attn_out(q, k_cache, v_cache, block_table, seq_lens, out, scale
                                                             block_table.data_ptr(), seq_lens.data_ptr(), out.data_ptr(), pa, pm, S,
                                                             Hq, Hkv, D, page, block_table.shape[1], P, num_kv_splits, scale, window,
                                                             _lib.current_stream_ptr(dev))
-    _lib.check(rc, f"paged_decode_attn seqs={S} hq={Hq} hkv={Hkv} pages={P} splits={num_kv_splits} window={window}")
+    _lib.check(rc, f"paged_decode_attn {dt} seqs={S} hq={Hq} hkv={Hkv} pages={P} splits={num_kv_splits} window={window}")
     return out
 
 
@@ -172,6 +189,7 @@ def kv_cache_append(k_new, v_new, k_cache, v_cache, block_table, start_pos) -> N
     block_table, start_pos = block_table.contiguous(), start_pos.contiguous()
     _contig_out(k_cache, "kv_cache_append")
     _contig_out(v_cache, "kv_cache_append")
+    _half_dtype("kv_cache_append", k_new, v_new, k_cache, v_cache)  # 16-bit elements are moved as they are
     S, n_new, Hkv, D = k_new.shape
     P, page = k_cache.shape[0], k_cache.shape[1]
     with torch.cuda.device(dev):
@@ -190,14 +208,16 @@ def paged_prefill_attn_out(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_ta
     _contig_out(out, "paged_prefill_attn")
     S, n_new, Hq, D = q.shape
     P, page, Hkv = k_cache.shape[0], k_cache.shape[1], k_cache.shape[2]
-    if out.shape != q.shape or out.dtype != torch.float16:
-        raise ValueError("paged_prefill_attn: out must be float16 with q's shape")
+    dt = _half_dtype("paged_prefill_attn", q, k_cache, v_cache, out)
+    if out.shape != q.shape:
+        raise ValueError("paged_prefill_attn: out must have q's shape")
     if scale is None or scale <= 0:
         scale = 1.0 / math.sqrt(D)
+    lib = _lib.load()
+    entry = lib.mi355_paged_prefill_attn_bf16 if dt == torch.bfloat16 else lib.mi355_paged_prefill_attn
     with torch.cuda.device(dev):
-        rc = _lib.load().mi355_paged_prefill_attn(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
-                                                  seq_lens.data_ptr(), out.data_ptr(), S, n_new, Hq, Hkv, D, page,
-                                                  block_table.shape[1], P, scale, _lib.current_stream_ptr(dev))
+        rc = entry(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), seq_lens.data_ptr(),
+                   out.data_ptr(), S, n_new, Hq, Hkv, D, page, block_table.shape[1], P, scale, _lib.current_stream_ptr(dev))
     _lib.check(rc, f"paged_prefill_attn seqs={S} n_new={n_new} hq={Hq} hkv={Hkv} pages={P}")
     return out
 

@@ -33,6 +33,11 @@ __all__ = [
 ]
 
 _OUT_DTYPES = {"float32": torch.float32, "float16": torch.float16, "bfloat16": torch.bfloat16}
+_HALF_DTYPES = (torch.float16, torch.bfloat16)  # the attention and GEMM kernels are built for both 16-bit formats
+
+
+def _same_half_dtype(tensors) -> bool:
+    return tensors[0].dtype in _HALF_DTYPES and all(t.dtype == tensors[0].dtype for t in tensors)
 
 
 def _require(cond: bool, msg: str) -> None:
@@ -112,7 +117,7 @@ class flash_attn_fwd(CustomOp):
         sel.attr_float(4)
         for name, t in (("q", q.t), ("k", k.t), ("v", v.t)):
             _require(t.dim() == 4, f"flash_attn_fwd: {name} must be [B, H, S, D]")
-            _require(t.dtype == torch.float16, f"flash_attn_fwd: {name} must be float16")
+        _require(_same_half_dtype((q.t, k.t, v.t)), "flash_attn_fwd: q, k, v must all be float16 or all bfloat16")
         _require(q.t.size(3) == 128, f"flash_attn_fwd: head dim {q.t.size(3)} not supported (only 128)")
         _require(k.t.shape == v.t.shape, "flash_attn_fwd: k and v shapes differ")
         _require(q.t.size(0) == k.t.size(0) and q.t.size(3) == k.t.size(3), "flash_attn_fwd: q and k disagree on B or D")
@@ -133,16 +138,20 @@ def _like_q(q: Tensor, device) -> Tensor:
     if order[-1] != 3 or any(q.stride(i) == 0 and q.size(i) > 1 for i in range(4)):
         order = [0, 1, 2, 3]
     inv = [order.index(i) for i in range(4)]
-    return torch.empty([q.size(i) for i in order], dtype=torch.float16, device=device).permute(inv)
+    return torch.empty([q.size(i) for i in order], dtype=q.dtype, device=device).permute(inv)
 
 
 PAGE_SIZES = (16, 32, 64, 128, 256)  # tokens per KV-cache page
 
 
-def _check_paged_args(op: str, q: Tensor, k_cache: Tensor, v_cache: Tensor, block_table: Tensor, seq_lens: Tensor):
+def _check_paged_args(op: str, q: Tensor, k_cache: Tensor, v_cache: Tensor, block_table: Tensor, seq_lens: Tensor,
+                      bf16_ok: bool = False):
     _require(q.dim() == 3, f"{op}: q must be [num_seqs, num_q_heads, D]")
     _require(k_cache.dim() == 4 and v_cache.shape == k_cache.shape, f"{op}: k_cache / v_cache must both be [num_pages, page_size, num_kv_heads, D]")
-    _require(q.dtype == torch.float16 and k_cache.dtype == torch.float16 and v_cache.dtype == torch.float16, f"{op}: q, k_cache, v_cache must be float16")
+    if bf16_ok:
+        _require(_same_half_dtype((q, k_cache, v_cache)), f"{op}: q, k_cache, v_cache must all be float16 or all bfloat16")
+    else:  # the two-phase interface exists in fp16 only
+        _require(q.dtype == torch.float16 and k_cache.dtype == torch.float16 and v_cache.dtype == torch.float16, f"{op}: q, k_cache, v_cache must be float16")
     _require(block_table.dim() == 2 and block_table.dtype == torch.int32, f"{op}: block_table must be int32 [num_seqs, max_pages_per_seq]")
     _require(seq_lens.dim() == 1 and seq_lens.dtype == torch.int32, f"{op}: seq_lens must be int32 [num_seqs]")
     _require(block_table.size(0) == q.size(0) and seq_lens.size(0) == q.size(0), f"{op}: block_table / seq_lens rows must equal num_seqs")
@@ -177,16 +186,16 @@ class paged_decode_attn(CustomOp):
         q, kc, vc, bt, sl = (sel.arg_tensor(i) for i in range(5))
         sel.attr_float(5)
         sel.attr_int(6)
-        _check_paged_args("paged_decode_attn", q.t, kc.t, vc.t, bt.t, sl.t)
+        _check_paged_args("paged_decode_attn", q.t, kc.t, vc.t, bt.t, sl.t, bf16_ok=True)
         q.specialize_dims(1, 2)
         kc.specialize_dims(1, 2, 3)
         vc.specialize_dims(1, 2, 3)
-        sel.return_new_tensor(list(q.t.shape), torch.float16)
+        sel.return_new_tensor(list(q.t.shape), q.t.dtype)
 
     def eager_execute(self, q, k_cache, v_cache, block_table, seq_lens, scale, num_kv_splits):
         if num_kv_splits <= 0:
             num_kv_splits = default_num_kv_splits(block_table.shape[1] * k_cache.shape[1], q.shape[0], k_cache.shape[2])
-        out = torch.empty(q.shape, dtype=torch.float16, device=q.device)
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
         return launch.paged_decode_attn_out(q, k_cache, v_cache, block_table, seq_lens, out, scale, num_kv_splits)
 
 
@@ -201,25 +210,25 @@ class paged_decode_attn_window(CustomOp):
         sel.attr_float(5)
         sel.attr_int(6)
         w = sel.attr_int(7).v
-        _check_paged_args("paged_decode_attn_window", q.t, kc.t, vc.t, bt.t, sl.t)
+        _check_paged_args("paged_decode_attn_window", q.t, kc.t, vc.t, bt.t, sl.t, bf16_ok=True)
         _require(w >= 0, "paged_decode_attn_window: window must be >= 0")
         q.specialize_dims(1, 2)
         kc.specialize_dims(1, 2, 3)
         vc.specialize_dims(1, 2, 3)
-        sel.return_new_tensor(list(q.t.shape), torch.float16)
+        sel.return_new_tensor(list(q.t.shape), q.t.dtype)
 
     def eager_execute(self, q, k_cache, v_cache, block_table, seq_lens, scale, num_kv_splits, window):
         if num_kv_splits <= 0:
             span = window if window > 0 else block_table.shape[1] * k_cache.shape[1]
             num_kv_splits = default_num_kv_splits(span, q.shape[0], k_cache.shape[2])
-        out = torch.empty(q.shape, dtype=torch.float16, device=q.device)
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
         return launch.paged_decode_attn_out(q, k_cache, v_cache, block_table, seq_lens, out, scale, num_kv_splits, window=window)
 
 
 @CustomOp.register
 class kv_cache_append(CustomOp):
     """In-place paged form of `cache[:bsz, start_pos : start_pos + n_new] = x` (tests/dynamo/llama_test.py:165-166)
-    with one start position per sequence: k_new, v_new [S, n_new, Hkv, 128] fp16 go to positions
+    with one start position per sequence: k_new, v_new [S, n_new, Hkv, 128] (fp16 or bf16) go to positions
     start_pos[s] .. start_pos[s] + n_new - 1 of k_cache, v_cache [P, page, Hkv, 128] through block_table [S, max_pages]."""
 
     signature = "kv_cache_append(Tensor k_new, Tensor v_new, Tensor(a!) k_cache, Tensor(b!) v_cache, Tensor block_table, Tensor start_pos) -> ()"
@@ -229,7 +238,7 @@ class kv_cache_append(CustomOp):
         fn = "kv_cache_append"
         _require(kn.t.dim() == 4 and kn.t.shape == vn.t.shape, f"{fn}: k_new and v_new must both be [S, n_new, Hkv, D]")
         _require(kc.t.dim() == 4 and kc.t.shape == vc.t.shape, f"{fn}: k_cache and v_cache must both be [P, page, Hkv, D]")
-        _require(all(t.t.dtype == torch.float16 for t in (kn, vn, kc, vc)), f"{fn}: tensors must be float16")
+        _require(_same_half_dtype((kn.t, vn.t, kc.t, vc.t)), f"{fn}: tensors must all be float16 or all bfloat16")
         _require(kn.t.size(3) == 128 and kc.t.size(3) == 128, f"{fn}: head dim must be 128")
         _require(kc.t.size(1) in PAGE_SIZES, f"{fn}: page size {kc.t.size(1)} not supported {PAGE_SIZES}")
         _require(kn.t.size(2) == kc.t.size(2), f"{fn}: k_new and k_cache disagree on the number of kv heads")
@@ -257,7 +266,7 @@ class paged_prefill_attn(CustomOp):
         fn = "paged_prefill_attn"
         _require(q.t.dim() == 4, f"{fn}: q must be [num_seqs, n_new, num_q_heads, D]")
         _require(kc.t.dim() == 4 and kc.t.shape == vc.t.shape, f"{fn}: k_cache / v_cache must both be [num_pages, page_size, num_kv_heads, D]")
-        _require(all(t.t.dtype == torch.float16 for t in (q, kc, vc)), f"{fn}: q, k_cache, v_cache must be float16")
+        _require(_same_half_dtype((q.t, kc.t, vc.t)), f"{fn}: q, k_cache, v_cache must all be float16 or all bfloat16")
         _require(q.t.size(3) == 128 and kc.t.size(3) == 128, f"{fn}: head dim must be 128")
         _require(kc.t.size(1) in PAGE_SIZES, f"{fn}: page size {kc.t.size(1)} not supported {PAGE_SIZES}")
         _require(kc.t.size(2) > 0 and q.t.size(2) % kc.t.size(2) == 0, f"{fn}: {q.t.size(2)} q heads over {kc.t.size(2)} kv heads")
@@ -265,10 +274,10 @@ class paged_prefill_attn(CustomOp):
         _require(sl.t.dim() == 1 and sl.t.dtype == torch.int32 and sl.t.size(0) == q.t.size(0), f"{fn}: seq_lens must be int32 [num_seqs]")
         _require(q.t.size(0) > 0 and q.t.size(1) > 0 and bt.t.size(1) > 0, f"{fn}: empty batch")
         q.specialize_dims(2, 3)
-        sel.return_new_tensor(list(q.t.shape), torch.float16)
+        sel.return_new_tensor(list(q.t.shape), q.t.dtype)
 
     def eager_execute(self, q, k_cache, v_cache, block_table, seq_lens, scale):
-        out = torch.empty(q.shape, dtype=torch.float16, device=q.device)
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
         return launch.paged_prefill_attn_out(q, k_cache, v_cache, block_table, seq_lens, out, scale)
 
 
