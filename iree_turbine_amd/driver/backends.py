@@ -77,8 +77,8 @@ def _mi355_aten(sig: AtenSignature) -> Callable:
             run.dispatches = n[0]
             return out
         return run
-    if any(t != "c10::Half" for t in types):
-        raise UnsupportedSignature(f"{sig.name}: the kernels take fp16 tensors (aten::mm also bf16), got {types}")
+    if len(set(types)) != 1 or types[0] not in half_like:
+        raise UnsupportedSignature(f"{sig.name}: the kernels take fp16 or bf16 tensors of one dtype, got {types}")
     if sig.name == "aten::scaled_dot_product_attention":
         if kwargs.get("attn_mask") is not None or float(kwargs.get("dropout_p", 0.0) or 0.0) != 0.0:
             raise UnsupportedSignature(f"{sig.name}: attention masks and dropout are not covered")

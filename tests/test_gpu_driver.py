@@ -66,7 +66,7 @@ def test_commands_file_two_backends_and_layout_copy(dev, tmp_path):
 
 @pytest.mark.parametrize("cmd", [["gemmfp16", "--a_w", "512", "--a_h", "1024", "--b_w", "256", "--transB", "1"],
                                  ["gemmfp16", "--a_w", "96", "--a_h", "40", "--b_w", "72", "--transA", "1"],
-                                 MM_HALF, MM_BF16, SDPA_128])
+                                 MM_HALF, MM_BF16, SDPA_128, [a.replace("c10::Half", "c10::BFloat16") for a in SDPA_128]])
 def test_numerics_verdict_passes(dev, cmd):
     from iree_turbine_amd.driver.numerics import format_verdict_verbose, verify_numerics
 
