@@ -113,6 +113,9 @@ def paged_decode_phase0_out(q, k_cache, v_cache, block_table, seq_lens, part_acc
     block_table, seq_lens = block_table.contiguous(), seq_lens.contiguous()
     _contig_out(part_acc, "paged_decode_phase0")
     _contig_out(part_ml, "paged_decode_phase0")
+    if any(t.dtype != torch.float16 for t in (q, k_cache, v_cache)):
+        raise ValueError("paged_decode_phase0: q, k_cache, v_cache must be float16 (the two-phase interface is fp16 only; "
+                         "paged_decode_attn takes bfloat16 as well)")
     S, Hq, D = q.shape
     P, page, Hkv, _ = k_cache.shape
     ns = part_acc.shape[2]
