@@ -25,7 +25,7 @@ def _make_entry(is_causal: bool, scale: float | None):
 def get_vanilla_attention_kernel(shape: AttentionShape, mfma_variant=None, dynamic_dims: bool = False,
                                  is_causal: bool = False, scale: float | None = None):
     """O = softmax(scale . Q K^T [causal]) V, fp32 online softmax.  Call as kernel(q, k, v, o) with
-    q, o [B, H, S_q, D] (or [B*H, S_q, D]) and k, v [B, H, S_kv, D], all f16; o is written in place.
+    q, o [B, H, S_q, D] (or [B*H, S_q, D]) and k, v [B, H, S_kv, D], all f16 (or all bf16); o is written in place.
 
     The recurrence is the fused attention of tests/kernel/fused_attention_test.py:25-77 (running max,
     rescaled running sum and accumulator, P cast to f16 before the second contraction) with the
