@@ -158,6 +158,18 @@ int mi355_paged_decode_phase0(const void* q, const void* k_cache, const void* v_
 int mi355_paged_decode_phase1(const float* part_acc, const float* part_ml, void* out,
                               int64_t num_seqs, int64_t num_q_heads, int64_t D,
                               int64_t num_splits, void* stream);
+
+/* The two phases with q, k_cache, v_cache (phase 0) and out (phase 1) in bf16; the fp32
+ * partial results between them have the same layout and meaning. */
+int mi355_paged_decode_phase0_bf16(const void* q, const void* k_cache, const void* v_cache,
+                                   const int32_t* block_table, const int32_t* seq_lens,
+                                   float* part_acc, float* part_ml,
+                                   int64_t num_seqs, int64_t num_q_heads, int64_t num_kv_heads,
+                                   int64_t D, int64_t page_size, int64_t max_pages_per_seq,
+                                   int64_t num_pages, int64_t num_splits, float scale, void* stream);
+int mi355_paged_decode_phase1_bf16(const float* part_acc, const float* part_ml, void* out,
+                                   int64_t num_seqs, int64_t num_q_heads, int64_t D,
+                                   int64_t num_splits, void* stream);
 int mi355_paged_decode_attn(const void* q, const void* k_cache, const void* v_cache,
                             const int32_t* block_table, const int32_t* seq_lens, void* out,
                             float* part_acc, float* part_ml,

@@ -54,6 +54,13 @@ _PROTOS = {
         + [c_float, c_void_p],
     ),
     "mi355_paged_decode_phase1": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p]),
+    "mi355_paged_decode_phase0_bf16": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+        + [c_int64] * 8
+        + [c_float, c_void_p],
+    ),
+    "mi355_paged_decode_phase1_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p]),
     "mi355_paged_decode_attn": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]

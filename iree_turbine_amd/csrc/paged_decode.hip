@@ -338,11 +338,11 @@ static int run_phase0(const void* q, const void* kc, const void* vc, const int32
 
 using namespace mi355;
 
-extern "C" int mi355_paged_decode_phase0(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
-                                         const int32_t* seq_lens, float* part_acc, float* part_ml, int64_t num_seqs,
-                                         int64_t num_q_heads, int64_t num_kv_heads, int64_t D, int64_t page_size,
-                                         int64_t max_pages_per_seq, int64_t num_pages, int64_t num_splits, float scale,
-                                         void* stream) {
+template <bool BF>
+static int phase0_entry(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
+                        const int32_t* seq_lens, float* part_acc, float* part_ml, int64_t num_seqs, int64_t num_q_heads,
+                        int64_t num_kv_heads, int64_t D, int64_t page_size, int64_t max_pages_per_seq, int64_t num_pages,
+                        int64_t num_splits, float scale, void* stream) {
   if (!q || !k_cache || !v_cache || !block_table || !seq_lens) return fail(-MI355_E_NULL, "paged_decode_phase0: null pointer");
   if (int rc = check_decode_args("paged_decode_phase0", num_seqs, num_q_heads, num_kv_heads, D, page_size, max_pages_per_seq,
                                  num_pages, num_splits, scale))
@@ -350,9 +350,27 @@ extern "C" int mi355_paged_decode_phase0(const void* q, const void* k_cache, con
   if (!part_acc || !part_ml) return fail(-MI355_E_SCRATCH, "paged_decode_phase0: part_acc / part_ml scratch is required");
   if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(part_acc))
     return fail(-MI355_E_ALIGN, "paged_decode_phase0: q, k_cache, v_cache, part_acc must be 16-byte aligned");
-  return run_phase0<false>(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, nullptr, num_seqs, num_q_heads,
+  return run_phase0<BF>(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, nullptr, num_seqs, num_q_heads,
                            num_kv_heads, max_pages_per_seq, num_splits, scale, 0, page_shift_of(page_size),
                            reinterpret_cast<hipStream_t>(stream));
+}
+
+extern "C" int mi355_paged_decode_phase0(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
+                                         const int32_t* seq_lens, float* part_acc, float* part_ml, int64_t num_seqs,
+                                         int64_t num_q_heads, int64_t num_kv_heads, int64_t D, int64_t page_size,
+                                         int64_t max_pages_per_seq, int64_t num_pages, int64_t num_splits, float scale,
+                                         void* stream) {
+  return phase0_entry<false>(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, num_seqs, num_q_heads, num_kv_heads, D,
+                             page_size, max_pages_per_seq, num_pages, num_splits, scale, stream);
+}
+
+extern "C" int mi355_paged_decode_phase0_bf16(const void* q, const void* k_cache, const void* v_cache,
+                                              const int32_t* block_table, const int32_t* seq_lens, float* part_acc,
+                                              float* part_ml, int64_t num_seqs, int64_t num_q_heads, int64_t num_kv_heads,
+                                              int64_t D, int64_t page_size, int64_t max_pages_per_seq, int64_t num_pages,
+                                              int64_t num_splits, float scale, void* stream) {
+  return phase0_entry<true>(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, num_seqs, num_q_heads, num_kv_heads, D,
+                            page_size, max_pages_per_seq, num_pages, num_splits, scale, stream);
 }
 
 template <bool BF>
@@ -371,6 +389,11 @@ static int run_phase1(const float* part_acc, const float* part_ml, void* out, in
 extern "C" int mi355_paged_decode_phase1(const float* part_acc, const float* part_ml, void* out, int64_t num_seqs,
                                          int64_t num_q_heads, int64_t D, int64_t num_splits, void* stream) {
   return run_phase1<false>(part_acc, part_ml, out, num_seqs, num_q_heads, D, num_splits, stream);
+}
+
+extern "C" int mi355_paged_decode_phase1_bf16(const float* part_acc, const float* part_ml, void* out, int64_t num_seqs,
+                                              int64_t num_q_heads, int64_t D, int64_t num_splits, void* stream) {
+  return run_phase1<true>(part_acc, part_ml, out, num_seqs, num_q_heads, D, num_splits, stream);
 }
 
 template <bool BF>

@@ -113,9 +113,7 @@ def paged_decode_phase0_out(q, k_cache, v_cache, block_table, seq_lens, part_acc
     block_table, seq_lens = block_table.contiguous(), seq_lens.contiguous()
     _contig_out(part_acc, "paged_decode_phase0")
     _contig_out(part_ml, "paged_decode_phase0")
-    if any(t.dtype != torch.float16 for t in (q, k_cache, v_cache)):
-        raise ValueError("paged_decode_phase0: q, k_cache, v_cache must be float16 (the two-phase interface is fp16 only; "
-                         "paged_decode_attn takes bfloat16 as well)")
+    dt = _half_dtype("paged_decode_phase0", q, k_cache, v_cache)
     S, Hq, D = q.shape
     P, page, Hkv, _ = k_cache.shape
     ns = part_acc.shape[2]
@@ -123,10 +121,12 @@ def paged_decode_phase0_out(q, k_cache, v_cache, block_table, seq_lens, part_acc
         raise ValueError("paged_decode_phase0: part_acc must be fp32 [S, Hq, splits, D], part_ml fp32 [S, Hq, splits, 2]")
     if scale is None or scale <= 0:
         scale = 1.0 / math.sqrt(D)
+    lib = _lib.load()
+    entry = lib.mi355_paged_decode_phase0_bf16 if dt == torch.bfloat16 else lib.mi355_paged_decode_phase0
     with torch.cuda.device(dev):
-        rc = _lib.load().mi355_paged_decode_phase0(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
-                                                   seq_lens.data_ptr(), part_acc.data_ptr(), part_ml.data_ptr(), S, Hq, Hkv, D,
-                                                   page, block_table.shape[1], P, ns, scale, _lib.current_stream_ptr(dev))
+        rc = entry(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), seq_lens.data_ptr(),
+                   part_acc.data_ptr(), part_ml.data_ptr(), S, Hq, Hkv, D, page, block_table.shape[1], P, ns, scale,
+                   _lib.current_stream_ptr(dev))
     _lib.check(rc, f"paged_decode_phase0 seqs={S} hq={Hq} hkv={Hkv} splits={ns}")
 
 
@@ -135,11 +135,12 @@ def paged_decode_phase1_out(part_acc: Tensor, part_ml: Tensor, out: Tensor) -> T
     part_acc, part_ml = part_acc.contiguous(), part_ml.contiguous()
     _contig_out(out, "paged_decode_phase1")
     S, Hq, ns, D = part_acc.shape
-    if tuple(out.shape) != (S, Hq, D) or out.dtype != torch.float16:
-        raise ValueError("paged_decode_phase1: out must be float16 [S, Hq, D]")
+    if tuple(out.shape) != (S, Hq, D) or out.dtype not in (torch.float16, torch.bfloat16):
+        raise ValueError("paged_decode_phase1: out must be float16 or bfloat16 [S, Hq, D]")
+    lib = _lib.load()
+    entry = lib.mi355_paged_decode_phase1_bf16 if out.dtype == torch.bfloat16 else lib.mi355_paged_decode_phase1
     with torch.cuda.device(dev):
-        rc = _lib.load().mi355_paged_decode_phase1(part_acc.data_ptr(), part_ml.data_ptr(), out.data_ptr(), S, Hq, D, ns,
-                                                   _lib.current_stream_ptr(dev))
+        rc = entry(part_acc.data_ptr(), part_ml.data_ptr(), out.data_ptr(), S, Hq, D, ns, _lib.current_stream_ptr(dev))
     _lib.check(rc, f"paged_decode_phase1 seqs={S} hq={Hq} splits={ns}")
     return out
 

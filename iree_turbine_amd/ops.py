@@ -150,7 +150,7 @@ def _check_paged_args(op: str, q: Tensor, k_cache: Tensor, v_cache: Tensor, bloc
     _require(k_cache.dim() == 4 and v_cache.shape == k_cache.shape, f"{op}: k_cache / v_cache must both be [num_pages, page_size, num_kv_heads, D]")
     if bf16_ok:
         _require(_same_half_dtype((q, k_cache, v_cache)), f"{op}: q, k_cache, v_cache must all be float16 or all bfloat16")
-    else:  # the two-phase interface exists in fp16 only
+    else:
         _require(q.dtype == torch.float16 and k_cache.dtype == torch.float16 and v_cache.dtype == torch.float16, f"{op}: q, k_cache, v_cache must be float16")
     _require(block_table.dim() == 2 and block_table.dtype == torch.int32, f"{op}: block_table must be int32 [num_seqs, max_pages_per_seq]")
     _require(seq_lens.dim() == 1 and seq_lens.dtype == torch.int32, f"{op}: seq_lens must be int32 [num_seqs]")
@@ -292,7 +292,7 @@ class paged_decode_phase0(CustomOp):
         q, kc, vc, bt, sl = (sel.arg_tensor(i) for i in range(5))
         sel.attr_float(5)
         ns = sel.attr_int(6).v
-        _check_paged_args("paged_decode_phase0", q.t, kc.t, vc.t, bt.t, sl.t)
+        _check_paged_args("paged_decode_phase0", q.t, kc.t, vc.t, bt.t, sl.t, bf16_ok=True)
         _require(1 <= ns <= 1024, "paged_decode_phase0: num_kv_splits must be in [1, 1024]")
         S, Hq, D = q.t.shape
         sel.return_new_tensor([S, Hq, ns, D], torch.float32)
@@ -308,7 +308,8 @@ class paged_decode_phase0(CustomOp):
 
 @CustomOp.register
 class paged_decode_phase1(CustomOp):
-    """Phase 1 of the split-K decode: merges the partials of phase 0 into [S, Hq, 128] fp16."""
+    """Phase 1 of the split-K decode: merges the partials of phase 0 into [S, Hq, 128] fp16 (a bf16 result comes
+    from `launch.paged_decode_phase1_out` with a bf16 `out`, or from the one-call `paged_decode_attn`)."""
 
     signature = "paged_decode_phase1(Tensor part_acc, Tensor part_ml) -> Tensor"
 

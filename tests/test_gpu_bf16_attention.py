@@ -168,5 +168,21 @@ def test_mixed_formats_are_rejected(dev):
     sl = torch.ones(1, dtype=torch.int32, device=dev)
     with pytest.raises(ValueError):
         torch.ops.mi355.paged_decode_attn(qbf[0, :, 0], kc16, kc16, bt, sl, 0.0, 1)
-    with pytest.raises(ValueError):  # the two-phase interface is fp16 only
-        torch.ops.mi355.paged_decode_phase0(qbf[0, :, 0], kc16.bfloat16(), kc16.bfloat16(), bt, sl, 0.0, 2)
+    with pytest.raises(ValueError):
+        torch.ops.mi355.paged_decode_phase0(qbf[0, :, 0], kc16, kc16, bt, sl, 0.0, 2)
+
+
+def test_decode_bf16_two_phases(dev):
+    """Phase 0 on bf16 operands, phase 1 into a bf16 result: bit-identical to the one-call form with as many splits."""
+    import iree_turbine_amd as ita
+    from oracle import inputs, paged_decode as op
+
+    announce("paged decode bf16 two phases")
+    q, kc, vc, bt, sl = inputs.paged_decode_inputs(num_seqs=4, min_len=30, max_len=900, seed=2)
+    q, kc, vc = _bf(q, kc, vc)
+    qd, kd, vd, btd, sld = _to(dev, q, kc, vc, bt, sl)
+    pacc, pml = torch.ops.mi355.paged_decode_phase0(qd, kd, vd, btd, sld, 0.0, 4)
+    out = torch.empty_like(qd)
+    ita.launch.paged_decode_phase1_out(pacc, pml, out)
+    assert torch.equal(out, torch.ops.mi355.paged_decode_attn(qd, kd, vd, btd, sld, 0.0, 4))
+    torch.testing.assert_close(out.float().cpu(), op.paged_decode_ref(q, kc, vc, bt, sl), rtol=TOL, atol=TOL)
