@@ -144,8 +144,9 @@ def test_template_getters_and_launchable_rules():
     dshape = paged_decode_attention_shape(32, 8, 128, 128, 16, 64)
     p0, p1, hp0, hp1 = get_paged_decode_attention_kernels(dshape, num_kv_splits=8, k_shape=(100, 16, 8, 128))
     assert p0.num_outputs == 2 and p1.num_outputs == 1 and hp0[lang.sym.U] == 8
-    with pytest.raises(ValueError, match="16-token pages"):
-        get_paged_decode_attention_kernels(paged_decode_attention_shape(32, 8, 128, 128, 32, 64))
+    assert get_paged_decode_attention_kernels(paged_decode_attention_shape(32, 8, 128, 128, 32, 64))[2][lang.sym.BLOCK_SIZE] == 32
+    with pytest.raises(ValueError, match="pages of 16, 32, 64, 128 or 256"):
+        get_paged_decode_attention_kernels(paged_decode_attention_shape(32, 8, 128, 128, 48, 64))
     mk, mhp = get_mxfp4_gemm_kernel((4096, 8192, 8192))
     assert mhp[lang.sym.BLOCK_K] == 256
     with pytest.raises(ValueError, match="multiple of 32"):
