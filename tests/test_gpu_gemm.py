@@ -338,3 +338,28 @@ def test_gemm_dtype_contract(dev):
         torch.ops.mi355.gemm_nt(abf, abf, "float16", -1)  # 16-bit output is the operands' own format
     with pytest.raises(ValueError):
         torch.ops.mi355.gemm_nt(a16, a16, "bfloat16", -1)
+
+
+@pytest.mark.parametrize("shape,dtype,out_dtype", [((3000, 5000, 4104), torch.float16, "float16"),
+                                                   ((1100, 4200, 2056), torch.bfloat16, "float32"),
+                                                   ((2304, 4096, 4100), torch.float16, "float32"),
+                                                   ((2100, 4096, 4096), torch.bfloat16, "bfloat16")])
+def test_gemm_large_ragged_shapes_take_the_padded_path(dev, shape, dtype, out_dtype):
+    """Large products whose sizes are not tile multiples run on the tiled kernels over zero-padded copies (only the
+    ragged operands are copied): the result must be what the bounds-checked kernel gives on the original operands,
+    and the caller's tensors stay untouched."""
+    import iree_turbine_amd as ita
+    from oracle import inputs
+
+    M, N, K = shape
+    announce(f"gemm ragged {shape} {dtype} -> {out_dtype}")
+    a, b = [t.to(dev) for t in inputs.gemm_inputs(M, N, K, seed=31, dtype=dtype)]
+    a0, b0 = a.clone(), b.clone()
+    names = ita._lib.variants("gemm_f16_nt")
+    got = torch.ops.mi355.gemm_nt(a, b, out_dtype, -1)
+    assert got.shape == (M, N) and got.is_contiguous()
+    ref = torch.ops.mi355.gemm_nt(a, b, out_dtype, len(names) - 1)
+    torch.testing.assert_close(got.float(), ref.float(), rtol=1e-3, atol=1e-3)
+    rows = torch.tensor([0, M // 2, M - 1], device=dev)
+    torch.testing.assert_close(got[rows].float(), a[rows].float() @ b.float().t(), rtol=RTOL, atol=ATOL)
+    assert torch.equal(a, a0) and torch.equal(b, b0)
