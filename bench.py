@@ -46,6 +46,7 @@ MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
     "gemm_2048x57344x8192": 3.054e9,
     "gemm_1024_f32out": 1.684e7,
     "gemm_bf16_8192": 1.746e9,
+    "gemm_16x8192x8192": 1.366e8,
     "fa_causal": 3.425e8,
     "fa_noncausal": 2.686e8,
     "decode": 1.177e9,
@@ -120,9 +121,11 @@ def wl_gemm(M, N, K, out_dtype="float16", in_dtype=torch.float16):
         flops = 2.0 * M * N * K
         out_b = 4 if out_dtype == "float32" else 2
         nbytes = 2.0 * (M * K + N * K) + out_b * M * N
+        hbm_bound = M <= 64  # decode-shaped: the weights are streamed once, far below the fp16 ridge point (312 flop/B)
         return {
             "fn": lambda: torch.ops.mi355.gemm_nt(ad, bd, out_dtype, -1),
-            "work": flops, "bytes": nbytes, "bound": "mfma", "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
+            "work": nbytes if hbm_bound else flops, "bytes": nbytes, "flops": flops, "bound": "hbm" if hbm_bound else "mfma",
+            "peak": PEAK_HBM_GBS if hbm_bound else PEAK_F16_TFLOPS, "unit": "GB/s" if hbm_bound else "TFLOP/s",
             "dtype": tag, "cpu": lambda: cpu_gemm(a, b, M, N, K),
             "config": {"workload": f"gemm_{tag}_nt_{M}x{N}x{K}_{'f32' if out_dtype == 'float32' else tag}out",
                        "M": M, "N": N, "K": K, "layout": "NT", "accumulate": "f32", "out": out_dtype, "seed": 10},
@@ -310,6 +313,7 @@ WORKLOADS = {
     "gemm_2048x57344x8192": wl_gemm(2048, 57344, 8192),
     "gemm_1024_f32out": wl_gemm(1024, 1024, 1024, "float32"),
     "gemm_bf16_8192": wl_gemm(8192, 8192, 8192, "bfloat16", torch.bfloat16),
+    "gemm_16x8192x8192": wl_gemm(16, 8192, 8192),
     "fa_causal": wl_attention(True),
     "fa_noncausal": wl_attention(False),
     "decode": wl_decode(),

@@ -835,6 +835,97 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_persistent(const half
   wait_vmcnt0();
 }
 
+// Skinny-M kernel (M <= 32, the decode-shaped product): weight streaming, HBM bound.  One workgroup of 8 waves per
+// 32 rows of B; wave w owns the 64-half K segments w, w + 8, ... of those rows and walks them through a private
+// double buffer in LDS (2 x (4 KiB of B + 4 KiB of A)): the direct-to-LDS loads of segment j + 1 -- 8 rows x 128
+// bytes per instruction for both operands -- are issued before segment j is consumed.  Rows of A past M repeat row
+// M - 1 (same cache lines; their output columns are never stored).  The 8 partial 32 x 32 tiles are summed through
+// LDS at the end.
+// Nothing loaded is carried in registers across iterations, and the waits and the LDS fragment reads are inline
+// assembly: with direct-to-LDS loads in flight the compiler waits for ALL of them before any LDS access it can
+// see, which would serialise the two segments.  Loads return in order, so "at most the 8 loads of the next segment
+// outstanding" means this one has landed.
+template <typename OutT, bool BF>
+__global__ __launch_bounds__(512) void gemm_f16_nt_skinny(const half_t* __restrict__ A, const half_t* __restrict__ B,
+                                                          OutT* __restrict__ C, int M, int N, int K) {
+  extern __shared__ __attribute__((aligned(16384))) char lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r32 = lane & 31, h = lane >> 5;
+  const int n0 = blockIdx.x * 32;
+  const int nseg = K >> 6;
+  const int mine = wave < nseg ? (nseg - wave + 7) >> 3 : 0;  // segments of this wave
+  char* my = lds + wave * 16384;
+  const unsigned my_lds = (unsigned)(uintptr_t)MI355_LDS(char, my);
+
+  floatx16 acc;
+#pragma unroll
+  for (int r = 0; r < 16; r++) acc[r] = 0.f;
+
+  // global side of the loads: instruction i covers rows 8i .. 8i + 7, lane = (row, slot); the chunk it fetches is
+  // slot ^ ((row >> 1) & 7), the swizzle of the tiled kernels
+  const int lrow = lane >> 3;
+  const half_t* b_src[4];
+  const half_t* a_src[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int row = i * 8 + lrow;
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    b_src[i] = B + (size_t)(n0 + row) * K + chunk * 8;
+    a_src[i] = A + (size_t)(row < M ? row : M - 1) * K + chunk * 8;
+  }
+  // fragment reads: row r32, chunk 2 * ks + h
+  unsigned rd[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ks++) rd[ks] = my_lds + r32 * 128 + (((2 * ks + h) ^ ((r32 >> 1) & 7)) * 16);
+
+  auto issue = [&](int j) {
+    const int seg = wave + 8 * j;
+    char* dst = my + (j & 1) * 8192;
+#pragma unroll
+    for (int i = 0; i < 4; i++) load_lds_16B(b_src[i] + seg * 64, dst + i * 1024);
+#pragma unroll
+    for (int i = 0; i < 4; i++) load_lds_16B(a_src[i] + seg * 64, dst + 4096 + i * 1024);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  if (mine > 0) issue(0);
+  for (int j = 0; j < mine; j++) {
+    if (j + 1 < mine) {
+      issue(j + 1);
+      asm volatile("s_waitcnt vmcnt(8)");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)");
+    }
+    const unsigned bo = (unsigned)(j & 1) << 13;
+    half8 fb[4], fa[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+      asm volatile("ds_read_b128 %0, %1" : "=v"(fb[ks]) : "v"(rd[ks] + bo));
+      asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(fa[ks]) : "v"(rd[ks] + bo));
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]), "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]));
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) acc = mfma16<BF>(fb[ks], fa[ks], acc);  // acc[n][m]
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  // reduce the 8 partial tiles: lane (m = r32, h) register r holds n = 8*(r/4) + 4h + r%4
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+  __syncthreads();
+  float* red = reinterpret_cast<float*>(lds);  // [wave][n 32][m 32]
+#pragma unroll
+  for (int r = 0; r < 16; r++) red[(wave * 32 + 8 * (r >> 2) + 4 * h + (r & 3)) * 32 + r32] = acc[r];
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < 1024; idx += 512) {
+    const int m = idx >> 5, n = idx & 31;
+    float v = 0.f;
+#pragma unroll
+    for (int w = 0; w < 8; w++) v += red[(w * 32 + n) * 32 + m];
+    if (m < M) OutPack<OutT, BF>::store1(C + (size_t)m * N + n0 + n, v);
+  }
+}
+
 // Any-shape kernel: 64x64 tile, 4 waves, bounds-checked staging through registers.  Used for
 // shapes the tiled kernel does not divide (and as an independent implementation in tests).
 template <typename OutT, bool BF>
@@ -907,6 +998,7 @@ static const GemmVariant kGemmVariants[] = {
     {"tiled_128x128x64_w2x2", 128, 128, 256},
     {"staged_256x256x64_w2x2", 256, 256, 256},
     {"staged_256x256_tail_128x128", 256, 256, 256},
+    {"skinny_m32_n32_w8", 32, 32, 512},
     {"generic_64x64x32", 64, 64, 256},
 };
 constexpr int kNumGemmVariants = sizeof(kGemmVariants) / sizeof(kGemmVariants[0]);
@@ -1008,6 +1100,15 @@ static int launch_variant(int variant, const void* a, const void* b, void* c, in
     case 6: return launch_tiled<128, 128, 2, 2, OutT, 0, BF>(a, b, c, M, N, K, N, stream);
     case 7: return launch_tiled<256, 256, 2, 2, OutT, 2, BF>(a, b, c, M, N, K, N, stream);
     case 8: return launch_split<OutT, BF>(a, b, c, M, N, K, stream);
+    case 9: {
+      auto kern = gemm_f16_nt_skinny<OutT, BF>;
+      constexpr int lds_bytes = 8 * 16384;
+      static std::atomic<uint64_t> lds_ok{0};
+      if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt_skinny")) return rc;
+      dim3 grid(N / 32), block(512);
+      hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, M, N, K);
+      return check_launch("gemm_f16_nt_skinny", grid, block, lds_bytes);
+    }
     default: {
       dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
       hipLaunchKernelGGL((gemm_f16_nt_generic<OutT, BF>), grid, block, 0, stream, (const half_t*)a, (const half_t*)b, (OutT*)c,
@@ -1035,6 +1136,7 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
     if (v == kNumGemmVariants - 1) return true;
     if (v <= 1 && (K < 128 || K > (1 << 21))) return false;  // prefetches two slabs ahead; 32-bit byte offsets inside a 256-row panel
     if ((v == 7 || v == 8) && (K < 256 || K % 128 != 0 || K > (1 << 21))) return false;  // slabs in pairs, three in flight
+    if (v == 9) return al && M <= 32 && N % 32 == 0 && K % 64 == 0;  // a tile is 32 rows of B; 64-half K segments
     return al && M % kGemmVariants[v].bm == 0 && N % kGemmVariants[v].bn == 0 && K % 64 == 0;
   };
   if (variant < 0) {
@@ -1048,11 +1150,16 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
     // tile's prologue and epilogue under its neighbours (8192x8192x512: +30%, x1024: +14%, x4096: +2%), as
     // long as its last round is >= 85% busy.
     const bool full_rounds = t256 * 100 >= rounds * 256 * 85;
+    if (fits(9) && N >= 2048 && K >= 512) variant = 9;  // decode-shaped: stream the weights once
+    else
     if (K <= 4096 && t256 <= 2048 && fits(0) && t256 >= 128 && full_rounds) variant = 0;
     else if (fits(8) && t256 >= 128) variant = 8;
     else if (fits(0) && t256 >= 128 && full_rounds) variant = 0;
     else if (fits(4)) variant = 4;
     else variant = kNumGemmVariants - 1;
+  } else if (!fits(variant) && variant == 9) {
+    return fail(-MI355_E_SHAPE, "gemm_f16_nt: variant %s needs M<=32, N%%32==0, K%%64==0 and 16-byte aligned pointers",
+                kGemmVariants[variant].name);
   } else if (!fits(variant)) {
     return fail(-MI355_E_SHAPE, "gemm_f16_nt: variant %s needs M%%%d==0, N%%%d==0, K%%64==0 and 16-byte aligned pointers",
                 kGemmVariants[variant].name, kGemmVariants[variant].bm, kGemmVariants[variant].bn);

@@ -139,6 +139,8 @@ def test_gemm_full_size_repeatable(dev, shape):
     names = ita._lib.variants("gemm_f16_nt")
     generic = torch.ops.mi355.gemm_nt(a, b, "float32", len(names) - 1)
     for variant in range(len(names) - 1):
+        if names[variant].startswith("skinny"):
+            continue  # M <= 32 only: covered by test_gemm_skinny_m
         first = torch.ops.mi355.gemm_nt(a, b, "float32", variant)
         for _ in range(2):
             assert torch.equal(first, torch.ops.mi355.gemm_nt(a, b, "float32", variant)), names[variant]
@@ -363,3 +365,46 @@ def test_gemm_large_ragged_shapes_take_the_padded_path(dev, shape, dtype, out_dt
     rows = torch.tensor([0, M // 2, M - 1], device=dev)
     torch.testing.assert_close(got[rows].float(), a[rows].float() @ b.float().t(), rtol=RTOL, atol=ATOL)
     assert torch.equal(a, a0) and torch.equal(b, b0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(16, 8192, 8192), (1, 4096, 4096), (32, 2048, 192), (7, 256, 64), (32, 32, 448), (5, 64, 1088),
+                                   (20, 4096, 14336), (31, 96, 8256)])
+def test_gemm_skinny_m(dev, shape, dtype):
+    """The weight-streaming kernel for M <= 32: one to 32 rows, one K segment per wave and fewer segments than waves,
+    odd segment counts (the double buffer ends on either half), several segments per wave; fp32 result against the
+    fp32 product of the same values, 16-bit result = the fp32 result rounded, launches repeat bit for bit, and
+    decode-shaped products take this kernel by themselves."""
+    import iree_turbine_amd as ita
+    from oracle import inputs
+
+    M, N, K = shape
+    names = ita._lib.variants("gemm_f16_nt")
+    sk = next(i for i, n in enumerate(names) if n.startswith("skinny"))
+    own = str(dtype).removeprefix("torch.")
+    announce(f"gemm skinny {shape} {own} variant={sk}")
+    a, b = inputs.gemm_inputs(M, N, K, seed=13, dtype=dtype)
+    ref = a.float() @ b.float().t()
+    a, b = a.to(dev), b.to(dev)
+    c32 = torch.ops.mi355.gemm_nt(a, b, "float32", sk)
+    torch.testing.assert_close(c32.cpu(), ref, rtol=1e-3, atol=1e-3 * max(1.0, ref.abs().max().item()))
+    c16 = torch.ops.mi355.gemm_nt(a, b, own, sk)
+    assert torch.equal(c16, c32.to(dtype))
+    assert torch.equal(c32, torch.ops.mi355.gemm_nt(a, b, "float32", sk))
+    if N >= 2048 and K >= 512:
+        assert torch.equal(c32, torch.ops.mi355.gemm_nt(a, b, "float32", -1))
+
+
+def test_gemm_skinny_contract(dev):
+    import iree_turbine_amd as ita
+
+    names = ita._lib.variants("gemm_f16_nt")
+    sk = next(i for i, n in enumerate(names) if n.startswith("skinny"))
+    a = torch.zeros(33, 64, dtype=torch.float16, device=dev)
+    b = torch.zeros(64, 64, dtype=torch.float16, device=dev)
+    with pytest.raises(ValueError):
+        torch.ops.mi355.gemm_nt(a, b, "float32", sk)  # 33 rows
+    with pytest.raises(ValueError):
+        torch.ops.mi355.gemm_nt(a[:8], b[:48], "float32", sk)  # N = 48 is not whole 32-row tiles
+    with pytest.raises(ValueError):
+        torch.ops.mi355.gemm_nt(a[:8, :32].contiguous(), b[:, :32].contiguous(), "float32", sk)  # K = 32 < one segment
