@@ -369,9 +369,9 @@ def test_gemm_large_ragged_shapes_take_the_padded_path(dev, shape, dtype, out_dt
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("shape", [(16, 8192, 8192), (1, 4096, 4096), (32, 2048, 192), (7, 256, 64), (32, 32, 448), (5, 64, 1088),
-                                   (20, 4096, 14336), (31, 96, 8256)])
+                                   (20, 4096, 14336), (31, 96, 8256), (64, 4096, 4096), (33, 2048, 1024), (50, 64, 320)])
 def test_gemm_skinny_m(dev, shape, dtype):
-    """The weight-streaming kernel for M <= 32: one to 32 rows, one K segment per wave and fewer segments than waves,
+    """The weight-streaming kernel for M <= 64 (33 rows and more take two launches): one to 64 rows, one K segment per wave and fewer segments than waves,
     odd segment counts (the double buffer ends on either half), several segments per wave; fp32 result against the
     fp32 product of the same values, 16-bit result = the fp32 result rounded, launches repeat bit for bit, and
     decode-shaped products take this kernel by themselves."""
@@ -400,10 +400,10 @@ def test_gemm_skinny_contract(dev):
 
     names = ita._lib.variants("gemm_f16_nt")
     sk = next(i for i, n in enumerate(names) if n.startswith("skinny"))
-    a = torch.zeros(33, 64, dtype=torch.float16, device=dev)
+    a = torch.zeros(65, 64, dtype=torch.float16, device=dev)
     b = torch.zeros(64, 64, dtype=torch.float16, device=dev)
     with pytest.raises(ValueError):
-        torch.ops.mi355.gemm_nt(a, b, "float32", sk)  # 33 rows
+        torch.ops.mi355.gemm_nt(a, b, "float32", sk)  # 65 rows
     with pytest.raises(ValueError):
         torch.ops.mi355.gemm_nt(a[:8], b[:48], "float32", sk)  # N = 48 is not whole 32-row tiles
     with pytest.raises(ValueError):
