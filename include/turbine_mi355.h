@@ -51,7 +51,8 @@ int mi355_abi_version(void);
 const char* mi355_last_error(void);
 
 /* Number of kernel variants of a family and the name of variant i
- * (family: "gemm_f16_nt", "flash_attn_fwd", "paged_decode", "mxfp4_gemm"). */
+ * (family: "gemm_f16_nt" -- shared by the bf16 entry --, "flash_attn_fwd", "paged_decode",
+ * "mxfp4_gemm", "mxfp8_gemm" -- shared by mi355_fp8_gemm --, "mxfp6_gemm"). */
 int mi355_variant_count(const char* family);
 const char* mi355_variant_name(const char* family, int i);
 
