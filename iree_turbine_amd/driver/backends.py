@@ -88,6 +88,10 @@ def _mi355_aten(sig: AtenSignature) -> Callable:
         if len(dims) != 3 or any(len(d) != 4 for d in dims) or dims[0][3] != 128:
             raise UnsupportedSignature(f"{sig.name}: the prefill kernel covers [B, H, S, 128] tensors, got {dims}")
         causal = bool(kwargs.get("is_causal", False))
+        if causal and dims[0][2] != dims[1][2]:
+            # aten's mask is aligned to the upper-left corner, the kernel's to the lower-right one
+            raise UnsupportedSignature(f"{sig.name}: is_causal with Sq={dims[0][2]} != Sk={dims[1][2]} is not covered "
+                                       "(the kernel's causal mask is aligned to the last key)")
         scale = kwargs.get("scale")
         scale = 0.0 if scale is None else float(scale)
 

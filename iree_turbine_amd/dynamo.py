@@ -1,7 +1,7 @@
 """`torch.compile` routing: a backend that substitutes this library's kernels for the ATen ops they cover.
 
     model = torch.compile(model, backend="mi355")            # registered on import
-    model = torch.compile(model, backend=iree_turbine_amd.dynamo.backend(nested_backend="inductor"))
+    model = torch.compile(model, backend=iree_turbine_amd.dynamo.backend(nested_backend=my_compiler_fn))
 
 The role of the reference's `iree_boo_experimental` backend (iree/turbine/dynamo/backends/boo.py:55-126),
 whose schema roots offloading at `aten.mm` / `aten.addmm` and the `_scaled_dot_product_*` variants
@@ -15,7 +15,7 @@ substitution is a direct FX rewrite of the ATen graph that AOT-autograd produces
   aten._scaled_dot_product_{flash,efficient,flash_for_cpu}_attention(q, k, v, ...)[0]
                               -> mi355.flash_attn_fwd(q, k, v, is_causal, scale)
 
-A node is rewritten only when the kernels cover it (fp16 or bf16 tensors of one dtype on a CUDA device, head dim 128, no mask, no dropout, auxiliary outputs unused -- so training graphs keep PyTorch's attention); everything else is left
+A node is rewritten only when the kernels cover it (fp16 or bf16 tensors of one dtype on a CUDA device, head dim 128, no mask, no dropout, a causal mask only with Sq == Sk, auxiliary outputs unused -- so training graphs keep PyTorch's attention); everything else is left
 for the nested backend.  Layouts: the ops make their operands contiguous themselves, so transposed views
 (`q.transpose(1, 2)`) need no graph surgery.
 """
@@ -136,6 +136,10 @@ def _rewrite_sdpa(node: fx.Node, device_ok) -> bool:
         return False
     if min(qv.shape[2], kv.shape[2]) == 0 or qv.numel() == 0:
         return False
+    if bool(bound.get("is_causal", False)) and qv.shape[2] != kv.shape[2]:
+        # aten aligns the causal mask to the upper-left corner (query i sees keys <= i); the kernel aligns it to the
+        # lower-right one (the last query sees every key).  The two agree only for Sq == Sk.
+        return False
     getitems = [u for u in node.users if u.op == "call_function" and u.target is operator.getitem]
     if len(getitems) != len(node.users):
         return False
@@ -214,18 +218,9 @@ def backend(*, nested_backend="eager"):
     from torch._dynamo.backends.common import aot_autograd
 
     if nested_backend == "inductor":
-        from torch._inductor.compile_fx import compile_fx_inner
-        from torch._inductor.decomposition import select_decomp_table
-
-        def fw(gm: fx.GraphModule, example_inputs):
-            LAST_SUBSTITUTIONS.update(substitute_kernels(gm))
-            return compile_fx_inner(gm, example_inputs)
-
-        def bw(gm: fx.GraphModule, example_inputs):
-            return compile_fx_inner(gm, example_inputs, is_backward=True)
-
-        return aot_autograd(fw_compiler=fw, bw_compiler=bw, decompositions=select_decomp_table())
-
+        # inductor compiles the rest of the graph into Triton kernels; this library ships hand-written HIP only
+        raise ValueError("nested_backend='inductor' is not supported: it would generate Triton kernels for the remaining "
+                         "graph; use 'eager' (the default) or a compiler function of your own")
     if nested_backend != "eager" and not callable(nested_backend):
         warnings.warn(f"nested_backend {nested_backend!r} is not known to preserve the substituted ops")
     nested_fn = torch._dynamo.lookup_backend(nested_backend)
@@ -242,7 +237,6 @@ def _register() -> None:
 
     try:
         register_backend(name="mi355", compiler_fn=backend())
-        register_backend(name="mi355_inductor", compiler_fn=backend(nested_backend="inductor"))
     except Exception:  # already registered (module re-import)
         pass
 

@@ -1,6 +1,7 @@
 """Out-variant launchers: checked tensors in, C-ABI call on torch's current stream, output tensors
 written in place.  Both the custom ops (ops.py) and the template kernels (templates/) go through
-these functions; they are the only callers of the C ABI."""
+these functions; they are the only callers of the C ABI, and each one runs the kernel's shape / dtype
+contract (contract.py) on its tensors before it takes a single device pointer."""
 
 from __future__ import annotations
 
@@ -10,7 +11,7 @@ import math
 import torch
 from torch import Tensor
 
-from . import _lib
+from . import _lib, contract
 
 
 def _dev(*tensors: Tensor) -> torch.device:
@@ -40,7 +41,14 @@ def _contig_out(t: Tensor, name: str) -> None:
 _PAD_MIN_FLOPS = 1.5e10  # below this the copies cost what the faster kernel gains (measured break-even 1-2e10)
 
 
+def _skinny_fits(M: int, N: int, K: int) -> bool:
+    """The shapes the library's weight-streaming kernel takes by itself (decode-shaped products: few rows of A
+    against a large B); padding A to a tile would multiply their work by 128 / M."""
+    return M <= 64 and N % 32 == 0 and K % 64 == 0 and N >= 2048 and K >= 512
+
+
 def gemm_nt_out(a: Tensor, b: Tensor, c: Tensor, variant: int = -1) -> Tensor:
+    contract.check_gemm_operands("gemm_nt", a, b)
     dev = _dev(a, b, c)
     a, b = a.contiguous(), b.contiguous()
     _contig_out(c, "gemm_nt")
@@ -48,14 +56,12 @@ def gemm_nt_out(a: Tensor, b: Tensor, c: Tensor, variant: int = -1) -> Tensor:
     N = b.shape[0]
     if tuple(c.shape) != (M, N):
         raise ValueError(f"gemm_nt: c is {tuple(c.shape)}, expected {(M, N)}")
-    if a.dtype != b.dtype or a.dtype not in (torch.float16, torch.bfloat16):
-        raise ValueError(f"gemm_nt: a and b must both be float16 or both bfloat16, got {a.dtype} and {b.dtype}")
     if c.dtype not in (torch.float32, a.dtype):
         raise ValueError(f"gemm_nt: c must be float32 or {a.dtype}, got {c.dtype}")
     lib = _lib.load()
     entry = lib.mi355_gemm_bf16_nt if a.dtype == torch.bfloat16 else lib.mi355_gemm_f16_nt
     a_k, b_k, c_k = a, b, c
-    if variant < 0 and 2.0 * M * N * K >= _PAD_MIN_FLOPS and (M % 128 or N % 128 or K % 64):
+    if variant < 0 and 2.0 * M * N * K >= _PAD_MIN_FLOPS and (M % 128 or N % 128 or K % 64) and not _skinny_fits(M, N, K):
         # Ragged sizes would go to the bounds-checked 64x64 kernel (about a fifth of the tiled kernels' rate).  Zero
         # padding changes no sum, so the ragged operands are copied into tile-aligned buffers and the result cut
         # out again: three extra passes over memory against a 4-5x faster product (3000x5000x4104: 508 -> 190 us).
@@ -98,6 +104,7 @@ def flash_attn_fwd_out(q: Tensor, k: Tensor, v: Tensor, o: Tensor, is_causal: bo
     """q, o: [B, H, Sq, 128]; k, v: [B, Hkv, Sk, 128] with H % Hkv == 0.  Operands whose rows are contiguous and
     16-byte aligned (any batch / head / row strides, e.g. transposed [B, S, H, D] views) are read in place; others
     are copied first.  `o` must be such a tensor."""
+    contract.check_attention_operands("flash_attn_fwd", q, k, v)
     dev = _dev(q, k, v, o)
     B, H, Sq, D = q.shape
     Hkv, Sk = k.shape[1], k.shape[2]
@@ -128,6 +135,8 @@ def flash_attn_fwd_out(q: Tensor, k: Tensor, v: Tensor, o: Tensor, is_causal: bo
 
 
 def paged_decode_phase0_out(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, scale: float) -> None:
+    contract.check_paged_args("paged_decode_phase0", q, k_cache, v_cache, block_table, seq_lens, bf16_ok=True)
+    ns = contract.check_decode_partials("paged_decode_phase0", part_acc, part_ml, q.shape[0], q.shape[1])
     dev = _dev(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml)
     q, k_cache, v_cache = q.contiguous(), k_cache.contiguous(), v_cache.contiguous()
     block_table, seq_lens = block_table.contiguous(), seq_lens.contiguous()
@@ -136,9 +145,6 @@ def paged_decode_phase0_out(q, k_cache, v_cache, block_table, seq_lens, part_acc
     dt = _half_dtype("paged_decode_phase0", q, k_cache, v_cache)
     S, Hq, D = q.shape
     P, page, Hkv, _ = k_cache.shape
-    ns = part_acc.shape[2]
-    if tuple(part_acc.shape) != (S, Hq, ns, D) or tuple(part_ml.shape) != (S, Hq, ns, 2) or part_acc.dtype != torch.float32 or part_ml.dtype != torch.float32:
-        raise ValueError("paged_decode_phase0: part_acc must be fp32 [S, Hq, splits, D], part_ml fp32 [S, Hq, splits, 2]")
     if scale is None or scale <= 0:
         scale = 1.0 / math.sqrt(D)
     lib = _lib.load()
@@ -151,6 +157,8 @@ def paged_decode_phase0_out(q, k_cache, v_cache, block_table, seq_lens, part_acc
 
 
 def paged_decode_phase1_out(part_acc: Tensor, part_ml: Tensor, out: Tensor) -> Tensor:
+    contract.require(part_acc.dim() == 4, "paged_decode_phase1: part_acc must be fp32 [S, Hq, splits, 128]")
+    contract.check_decode_partials("paged_decode_phase1", part_acc, part_ml, part_acc.shape[0], part_acc.shape[1])
     dev = _dev(part_acc, part_ml, out)
     part_acc, part_ml = part_acc.contiguous(), part_ml.contiguous()
     _contig_out(out, "paged_decode_phase1")
@@ -167,6 +175,10 @@ def paged_decode_phase1_out(part_acc: Tensor, part_ml: Tensor, out: Tensor) -> T
 
 def paged_decode_attn_out(q, k_cache, v_cache, block_table, seq_lens, out, scale: float, num_kv_splits: int,
                           part_acc: Tensor | None = None, part_ml: Tensor | None = None, window: int = 0) -> Tensor:
+    contract.check_paged_args("paged_decode_attn", q, k_cache, v_cache, block_table, seq_lens, bf16_ok=True)
+    contract.require(1 <= num_kv_splits <= 1024, f"paged_decode_attn: num_kv_splits must be in [1, 1024], got {num_kv_splits}")
+    if num_kv_splits > 1 and part_acc is not None and part_ml is not None:  # caller-owned scratch
+        contract.check_decode_partials("paged_decode_attn", part_acc, part_ml, q.shape[0], q.shape[1], num_kv_splits)
     dev = _dev(q, k_cache, v_cache, block_table, seq_lens, out)
     q, k_cache, v_cache = q.contiguous(), k_cache.contiguous(), v_cache.contiguous()
     block_table, seq_lens = block_table.contiguous(), seq_lens.contiguous()
@@ -183,8 +195,12 @@ def paged_decode_attn_out(q, k_cache, v_cache, block_table, seq_lens, out, scale
             part_acc = torch.empty((S, Hq, num_kv_splits, D), dtype=torch.float32, device=dev)
         if part_ml is None:
             part_ml = torch.empty((S, Hq, num_kv_splits, 2), dtype=torch.float32, device=dev)
-    pa = part_acc.data_ptr() if part_acc is not None else None
-    pm = part_ml.data_ptr() if part_ml is not None else None
+        _dev(q, part_acc, part_ml)
+        contract.check_decode_partials("paged_decode_attn", part_acc, part_ml, S, Hq, num_kv_splits)
+        _contig_out(part_acc, "paged_decode_attn")
+        _contig_out(part_ml, "paged_decode_attn")
+    pa = part_acc.data_ptr() if num_kv_splits > 1 else None
+    pm = part_ml.data_ptr() if num_kv_splits > 1 else None
     if window < 0:
         raise ValueError(f"paged_decode_attn: window must be >= 0, got {window}")
     with torch.cuda.device(dev):
@@ -208,6 +224,7 @@ def paged_decode_attn_out(q, k_cache, v_cache, block_table, seq_lens, out, scale
 
 def kv_cache_append(k_new, v_new, k_cache, v_cache, block_table, start_pos) -> None:
     """Writes k_new / v_new [S, n_new, Hkv, 128] into the paged caches in place (see mi355_kv_cache_append)."""
+    contract.check_kv_append("kv_cache_append", k_new, v_new, k_cache, v_cache, block_table, start_pos)
     dev = _dev(k_new, v_new, k_cache, v_cache, block_table, start_pos)
     k_new, v_new = k_new.contiguous(), v_new.contiguous()
     block_table, start_pos = block_table.contiguous(), start_pos.contiguous()
@@ -226,6 +243,7 @@ def kv_cache_append(k_new, v_new, k_cache, v_cache, block_table, start_pos) -> N
 def paged_prefill_attn_out(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_table: Tensor, seq_lens: Tensor, out: Tensor,
                            scale: float) -> Tensor:
     """q, out [S, n_new, Hq, 128]; caches [P, page, Hkv, 128]; seq_lens counts the new tokens (see mi355_paged_prefill_attn)."""
+    contract.check_paged_prefill("paged_prefill_attn", q, k_cache, v_cache, block_table, seq_lens)
     dev = _dev(q, k_cache, v_cache, block_table, seq_lens, out)
     q, k_cache, v_cache = q.contiguous(), k_cache.contiguous(), v_cache.contiguous()
     block_table, seq_lens = block_table.contiguous(), seq_lens.contiguous()
@@ -246,7 +264,14 @@ def paged_prefill_attn_out(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_ta
     return out
 
 
+def _check_mx_out(op: str, c: Tensor) -> None:
+    if c.dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError(f"{op}: c must be bfloat16 or float32, got {c.dtype}")
+
+
 def mxfp4_gemm_out(a, a_scale, b, b_scale, c: Tensor, variant: int = -1) -> Tensor:
+    contract.check_mx_pair("mxfp4_gemm", a, a_scale, b, b_scale, per_byte=2)
+    _check_mx_out("mxfp4_gemm", c)
     dev = _dev(a, a_scale, b, b_scale, c)
     a, a_scale, b, b_scale = a.contiguous(), a_scale.contiguous(), b.contiguous(), b_scale.contiguous()
     _contig_out(c, "mxfp4_gemm")
@@ -261,6 +286,8 @@ def mxfp4_gemm_out(a, a_scale, b, b_scale, c: Tensor, variant: int = -1) -> Tens
 
 
 def mxfp8_gemm_out(a, a_scale, b, b_scale, c: Tensor, variant: int = -1) -> Tensor:
+    contract.check_mx_pair("mxfp8_gemm", a, a_scale, b, b_scale, per_byte=1)
+    _check_mx_out("mxfp8_gemm", c)
     dev = _dev(a, a_scale, b, b_scale, c)
     a, a_scale, b, b_scale = a.contiguous(), a_scale.contiguous(), b.contiguous(), b_scale.contiguous()
     _contig_out(c, "mxfp8_gemm")
@@ -281,14 +308,13 @@ def mxfp6_gemm_out(a, a_scale, b, b_scale, c: Tensor, element_format: str = "e2m
     dev = _dev(a, a_scale, b, b_scale, c)
     if element_format not in FP6_FORMATS:
         raise ValueError(f"mxfp6_gemm: element_format must be one of {sorted(FP6_FORMATS)}, got {element_format!r}")
+    contract.check_mxfp6_pair("mxfp6_gemm", a, a_scale, b, b_scale)
+    _check_mx_out("mxfp6_gemm", c)
     a, a_scale, b, b_scale = a.contiguous(), a_scale.contiguous(), b.contiguous(), b_scale.contiguous()
     _contig_out(c, "mxfp6_gemm")
     M, N, K = a.shape[0], b.shape[0], a_scale.shape[1] * 32
     if tuple(c.shape) != (M, N):
         raise ValueError(f"mxfp6_gemm: c is {tuple(c.shape)}, expected {(M, N)}")
-    if a.shape[1] * 4 != K * 3 or b.shape[1] * 4 != K * 3 or b_scale.shape[1] * 32 != K:
-        raise ValueError(f"mxfp6_gemm: operands must be uint8 [rows, K*3/4] with scales [rows, K/32]; got a {tuple(a.shape)}, "
-                         f"a_scale {tuple(a_scale.shape)}, b {tuple(b.shape)}, b_scale {tuple(b_scale.shape)}")
     with torch.cuda.device(dev):
         rc = _lib.load().mi355_mxfp6_gemm(a.data_ptr(), a_scale.data_ptr(), b.data_ptr(), b_scale.data_ptr(), c.data_ptr(), M, N,
                                           K, FP6_FORMATS[element_format], _lib.dtype_code(c.dtype), variant,
@@ -298,6 +324,8 @@ def mxfp6_gemm_out(a, a_scale, b, b_scale, c: Tensor, element_format: str = "e2m
 
 
 def fp8_gemm_out(a, b, c: Tensor, alpha: float = 1.0, variant: int = -1) -> Tensor:
+    contract.check_fp8_operands("fp8_gemm", a, b)
+    _check_mx_out("fp8_gemm", c)
     dev = _dev(a, b, c)
     a, b = a.contiguous(), b.contiguous()
     _contig_out(c, "fp8_gemm")
@@ -312,6 +340,7 @@ def fp8_gemm_out(a, b, c: Tensor, alpha: float = 1.0, variant: int = -1) -> Tens
 
 
 def mxfp4_dequant_out(codes: Tensor, scales: Tensor, out: Tensor) -> Tensor:
+    contract.check_mx_operand("mxfp4_dequant", "codes", codes, scales)
     dev = _dev(codes, scales, out)
     codes, scales = codes.contiguous(), scales.contiguous()
     _contig_out(out, "mxfp4_dequant")
@@ -326,6 +355,7 @@ def mxfp4_dequant_out(codes: Tensor, scales: Tensor, out: Tensor) -> Tensor:
 
 
 def mxfp4_quantize_out(x: Tensor, codes: Tensor, scales: Tensor) -> tuple[Tensor, Tensor]:
+    contract.check_quantize_input("mxfp4_quantize", x)
     dev = _dev(x, codes, scales)
     x = x.contiguous()
     _contig_out(codes, "mxfp4_quantize")
@@ -345,6 +375,7 @@ def mxfp6_quantize_out(x: Tensor, codes: Tensor, scales: Tensor, element_format:
     dev = _dev(x, codes, scales)
     if element_format not in FP6_FORMATS:
         raise ValueError(f"mxfp6_quantize: element_format must be one of {sorted(FP6_FORMATS)}, got {element_format!r}")
+    contract.check_quantize_input("mxfp6_quantize", x)
     x = x.contiguous()
     _contig_out(codes, "mxfp6_quantize")
     _contig_out(scales, "mxfp6_quantize")
@@ -360,6 +391,7 @@ def mxfp6_quantize_out(x: Tensor, codes: Tensor, scales: Tensor, element_format:
 
 
 def mxfp8_quantize_out(x: Tensor, codes: Tensor, scales: Tensor) -> tuple[Tensor, Tensor]:
+    contract.check_quantize_input("mxfp8_quantize", x)
     dev = _dev(x, codes, scales)
     x = x.contiguous()
     _contig_out(codes, "mxfp8_quantize")

@@ -14,6 +14,9 @@ import torch
 from torch import Tensor
 
 from . import launch
+from .contract import PAGE_SIZES, check_mx_operand as _check_mx_operand, check_paged_args as _check_paged_args  # noqa: F401
+from . import contract
+from .contract import require as _require
 from .op_reg import CustomOp, KernelSelection
 
 __all__ = [
@@ -36,15 +39,6 @@ _OUT_DTYPES = {"float32": torch.float32, "float16": torch.float16, "bfloat16": t
 _HALF_DTYPES = (torch.float16, torch.bfloat16)  # the attention and GEMM kernels are built for both 16-bit formats
 
 
-def _same_half_dtype(tensors) -> bool:
-    return tensors[0].dtype in _HALF_DTYPES and all(t.dtype == tensors[0].dtype for t in tensors)
-
-
-def _require(cond: bool, msg: str) -> None:
-    if not cond:
-        raise ValueError(msg)
-
-
 @CustomOp.register
 class gemm_nt(CustomOp):
     """C[M,N] = A[M,K] . B[N,K]^T, fp16 or bf16 inputs, fp32 accumulation; out_dtype "float32" or the inputs' own
@@ -60,13 +54,9 @@ class gemm_nt(CustomOp):
         a, b = sel.arg_tensor(0), sel.arg_tensor(1)
         od = sel.attr_str(2).v
         sel.attr_int(3)
-        _require(a.t.dim() == 2 and b.t.dim() == 2, "gemm_nt: a and b must be rank 2")
-        _require(a.t.dtype == b.t.dtype and a.t.dtype in (torch.float16, torch.bfloat16),
-                 "gemm_nt: a and b must both be float16 or both bfloat16")
-        _require(a.t.size(1) == b.t.size(1), f"gemm_nt: K mismatch, a is {tuple(a.t.shape)}, b is {tuple(b.t.shape)} (b is [N, K])")
+        contract.check_gemm_operands("gemm_nt", a.t, b.t)
         own = str(a.t.dtype).removeprefix("torch.")
         _require(od in ("float32", own), f"gemm_nt: out_dtype must be 'float32' or '{own}' for {own} operands, got {od!r}")
-        _require(a.t.size(0) > 0 and b.t.size(0) > 0 and a.t.size(1) > 0, "gemm_nt: empty operand")
         a.specialize_all_dims()
         b.specialize_all_dims()
         sel.return_new_tensor([a.t.size(0), b.t.size(0)], _OUT_DTYPES[od]).specialize_all_dims()
@@ -104,9 +94,12 @@ class flash_attn_fwd(CustomOp):
     """softmax(scale . Q K^T [+ causal mask]) V for q [B,H,Sq,128], k/v [B,Hkv,Sk,128] fp16, H % Hkv == 0
     (query head h reads K/V head h // (H // Hkv), as `enable_gqa=True` does).
 
-    Same argument meaning as aten.scaled_dot_product_attention(q, k, v, None, 0.0, is_causal,
-    scale=) -- the canonical form the reference rewrites SDPA variants to
-    (iree/turbine/kernel/boo/fusion/replacement.py:275-284).  scale <= 0 selects 1/sqrt(D).
+    Argument order of aten.scaled_dot_product_attention(q, k, v, None, 0.0, is_causal, scale=) -- the
+    canonical form the reference rewrites SDPA variants to (iree/turbine/kernel/boo/fusion/replacement.py:275-284).
+    scale <= 0 selects 1/sqrt(D).  One difference in meaning: with Sq != Sk the causal mask is aligned to the LAST
+    key (query i sees keys <= i + Sk - Sq, the chunked-prefill convention), where aten aligns it to the first
+    (keys <= i); for Sq == Sk the two are the same mask.  The torch.compile pass and the driver backend therefore
+    route a causal call to this op only when Sq == Sk.
     The result is laid out like `torch.empty_like(q)`: a transposed [B, S, H, D] view in gives one out."""
 
     signature = "flash_attn_fwd(Tensor q, Tensor k, Tensor v, bool is_causal, float scale) -> Tensor"
@@ -115,15 +108,7 @@ class flash_attn_fwd(CustomOp):
         q, k, v = sel.arg_tensor(0), sel.arg_tensor(1), sel.arg_tensor(2)
         sel.attr_bool(3)
         sel.attr_float(4)
-        for name, t in (("q", q.t), ("k", k.t), ("v", v.t)):
-            _require(t.dim() == 4, f"flash_attn_fwd: {name} must be [B, H, S, D]")
-        _require(_same_half_dtype((q.t, k.t, v.t)), "flash_attn_fwd: q, k, v must all be float16 or all bfloat16")
-        _require(q.t.size(3) == 128, f"flash_attn_fwd: head dim {q.t.size(3)} not supported (only 128)")
-        _require(k.t.shape == v.t.shape, "flash_attn_fwd: k and v shapes differ")
-        _require(q.t.size(0) == k.t.size(0) and q.t.size(3) == k.t.size(3), "flash_attn_fwd: q and k disagree on B or D")
-        _require(k.t.size(1) > 0 and q.t.size(1) % k.t.size(1) == 0,
-                 f"flash_attn_fwd: {q.t.size(1)} query heads over {k.t.size(1)} key/value heads")
-        _require(q.t.size(2) > 0 and k.t.size(2) > 0, "flash_attn_fwd: empty sequence")
+        contract.check_attention_operands("flash_attn_fwd", q.t, k.t, v.t)
         for d in (q, k, v):
             d.specialize_dims(1, 3)
         sel.return_tensor(_like_q(q.t, "meta"))
@@ -139,27 +124,6 @@ def _like_q(q: Tensor, device) -> Tensor:
         order = [0, 1, 2, 3]
     inv = [order.index(i) for i in range(4)]
     return torch.empty([q.size(i) for i in order], dtype=q.dtype, device=device).permute(inv)
-
-
-PAGE_SIZES = (16, 32, 64, 128, 256)  # tokens per KV-cache page
-
-
-def _check_paged_args(op: str, q: Tensor, k_cache: Tensor, v_cache: Tensor, block_table: Tensor, seq_lens: Tensor,
-                      bf16_ok: bool = False):
-    _require(q.dim() == 3, f"{op}: q must be [num_seqs, num_q_heads, D]")
-    _require(k_cache.dim() == 4 and v_cache.shape == k_cache.shape, f"{op}: k_cache / v_cache must both be [num_pages, page_size, num_kv_heads, D]")
-    if bf16_ok:
-        _require(_same_half_dtype((q, k_cache, v_cache)), f"{op}: q, k_cache, v_cache must all be float16 or all bfloat16")
-    else:
-        _require(q.dtype == torch.float16 and k_cache.dtype == torch.float16 and v_cache.dtype == torch.float16, f"{op}: q, k_cache, v_cache must be float16")
-    _require(block_table.dim() == 2 and block_table.dtype == torch.int32, f"{op}: block_table must be int32 [num_seqs, max_pages_per_seq]")
-    _require(seq_lens.dim() == 1 and seq_lens.dtype == torch.int32, f"{op}: seq_lens must be int32 [num_seqs]")
-    _require(block_table.size(0) == q.size(0) and seq_lens.size(0) == q.size(0), f"{op}: block_table / seq_lens rows must equal num_seqs")
-    _require(q.size(2) == 128 and k_cache.size(3) == 128, f"{op}: head dim must be 128")
-    _require(k_cache.size(1) in PAGE_SIZES, f"{op}: page size {k_cache.size(1)} not supported {PAGE_SIZES}")
-    hq, hkv = q.size(1), k_cache.size(2)
-    _require(hkv > 0 and hq % hkv == 0 and hq // hkv in (1, 2, 4, 8, 16), f"{op}: {hq} q heads over {hkv} kv heads is not supported (ratio 1, 2, 4, 8 or 16)")
-    _require(q.size(0) > 0 and block_table.size(1) > 0, f"{op}: empty batch")
 
 
 def default_num_kv_splits(seq_lens_max: int, num_seqs: int, num_kv_heads: int) -> int:
@@ -237,16 +201,7 @@ class kv_cache_append(CustomOp):
 
     def select(self, sel: KernelSelection):
         kn, vn, kc, vc, bt, sp = (sel.arg_tensor(i) for i in range(6))
-        fn = "kv_cache_append"
-        _require(kn.t.dim() == 4 and kn.t.shape == vn.t.shape, f"{fn}: k_new and v_new must both be [S, n_new, Hkv, D]")
-        _require(kc.t.dim() == 4 and kc.t.shape == vc.t.shape, f"{fn}: k_cache and v_cache must both be [P, page, Hkv, D]")
-        _require(_same_half_dtype((kn.t, vn.t, kc.t, vc.t)), f"{fn}: tensors must all be float16 or all bfloat16")
-        _require(kn.t.size(3) == 128 and kc.t.size(3) == 128, f"{fn}: head dim must be 128")
-        _require(kc.t.size(1) in PAGE_SIZES, f"{fn}: page size {kc.t.size(1)} not supported {PAGE_SIZES}")
-        _require(kn.t.size(2) == kc.t.size(2), f"{fn}: k_new and k_cache disagree on the number of kv heads")
-        _require(kn.t.size(0) > 0 and kn.t.size(1) > 0, f"{fn}: empty k_new")
-        _require(bt.t.dim() == 2 and bt.t.dtype == torch.int32 and bt.t.size(0) == kn.t.size(0), f"{fn}: block_table must be int32 [S, max_pages]")
-        _require(sp.t.dim() == 1 and sp.t.dtype == torch.int32 and sp.t.size(0) == kn.t.size(0), f"{fn}: start_pos must be int32 [S]")
+        contract.check_kv_append("kv_cache_append", kn.t, vn.t, kc.t, vc.t, bt.t, sp.t)
 
     def eager_execute(self, k_new, v_new, k_cache, v_cache, block_table, start_pos):
         launch.kv_cache_append(k_new, v_new, k_cache, v_cache, block_table, start_pos)
@@ -265,16 +220,7 @@ class paged_prefill_attn(CustomOp):
     def select(self, sel: KernelSelection):
         q, kc, vc, bt, sl = (sel.arg_tensor(i) for i in range(5))
         sel.attr_float(5)
-        fn = "paged_prefill_attn"
-        _require(q.t.dim() == 4, f"{fn}: q must be [num_seqs, n_new, num_q_heads, D]")
-        _require(kc.t.dim() == 4 and kc.t.shape == vc.t.shape, f"{fn}: k_cache / v_cache must both be [num_pages, page_size, num_kv_heads, D]")
-        _require(_same_half_dtype((q.t, kc.t, vc.t)), f"{fn}: q, k_cache, v_cache must all be float16 or all bfloat16")
-        _require(q.t.size(3) == 128 and kc.t.size(3) == 128, f"{fn}: head dim must be 128")
-        _require(kc.t.size(1) in PAGE_SIZES, f"{fn}: page size {kc.t.size(1)} not supported {PAGE_SIZES}")
-        _require(kc.t.size(2) > 0 and q.t.size(2) % kc.t.size(2) == 0, f"{fn}: {q.t.size(2)} q heads over {kc.t.size(2)} kv heads")
-        _require(bt.t.dim() == 2 and bt.t.dtype == torch.int32 and bt.t.size(0) == q.t.size(0), f"{fn}: block_table must be int32 [num_seqs, max_pages]")
-        _require(sl.t.dim() == 1 and sl.t.dtype == torch.int32 and sl.t.size(0) == q.t.size(0), f"{fn}: seq_lens must be int32 [num_seqs]")
-        _require(q.t.size(0) > 0 and q.t.size(1) > 0 and bt.t.size(1) > 0, f"{fn}: empty batch")
+        contract.check_paged_prefill("paged_prefill_attn", q.t, kc.t, vc.t, bt.t, sl.t)
         q.specialize_dims(2, 3)
         sel.return_new_tensor(list(q.t.shape), q.t.dtype)
 
@@ -327,15 +273,6 @@ class paged_decode_phase1(CustomOp):
         return launch.paged_decode_phase1_out(part_acc, part_ml, out)
 
 
-def _check_mx_operand(op: str, name: str, codes: Tensor, scales: Tensor, per_byte: int = 2):
-    what = "[rows, K/2] (two E2M1 codes per byte)" if per_byte == 2 else "[rows, K] (one E4M3 code per byte)"
-    _require(codes.dim() == 2 and codes.dtype == torch.uint8, f"{op}: {name} must be uint8 {what}")
-    _require(scales.dim() == 2 and scales.dtype == torch.uint8, f"{op}: {name}_scale must be uint8 [rows, K/32] (E8M0)")
-    K = codes.size(1) * per_byte
-    _require(K > 0 and K % 32 == 0, f"{op}: K={K} must be a positive multiple of 32")
-    _require(scales.size(0) == codes.size(0) and scales.size(1) == K // 32, f"{op}: {name}_scale shape {tuple(scales.shape)} does not match {name} {tuple(codes.shape)}")
-
-
 @CustomOp.register
 class mxfp4_gemm(CustomOp):
     """C[M,N] = dq(A) . dq(B)^T for OCP MXFP4 operands (see include/turbine_mi355.h for the format);
@@ -347,11 +284,8 @@ class mxfp4_gemm(CustomOp):
         a, asc, b, bsc = (sel.arg_tensor(i) for i in range(4))
         od = sel.attr_str(4).v
         sel.attr_int(5)
-        _check_mx_operand("mxfp4_gemm", "a", a.t, asc.t)
-        _check_mx_operand("mxfp4_gemm", "b", b.t, bsc.t)
-        _require(a.t.size(1) == b.t.size(1), "mxfp4_gemm: a and b disagree on K")
+        contract.check_mx_pair("mxfp4_gemm", a.t, asc.t, b.t, bsc.t, per_byte=2)
         _require(od in ("bfloat16", "float32"), f"mxfp4_gemm: out_dtype must be 'bfloat16' or 'float32', got {od!r}")
-        _require(a.t.size(0) > 0 and b.t.size(0) > 0, "mxfp4_gemm: empty operand")
         for d in (a, asc, b, bsc):
             d.specialize_all_dims()
         sel.return_new_tensor([a.t.size(0), b.t.size(0)], _OUT_DTYPES[od]).specialize_all_dims()
@@ -372,11 +306,8 @@ class mxfp8_gemm(CustomOp):
         a, asc, b, bsc = (sel.arg_tensor(i) for i in range(4))
         od = sel.attr_str(4).v
         sel.attr_int(5)
-        _check_mx_operand("mxfp8_gemm", "a", a.t, asc.t, per_byte=1)
-        _check_mx_operand("mxfp8_gemm", "b", b.t, bsc.t, per_byte=1)
-        _require(a.t.size(1) == b.t.size(1), "mxfp8_gemm: a and b disagree on K")
+        contract.check_mx_pair("mxfp8_gemm", a.t, asc.t, b.t, bsc.t, per_byte=1)
         _require(od in ("bfloat16", "float32"), f"mxfp8_gemm: out_dtype must be 'bfloat16' or 'float32', got {od!r}")
-        _require(a.t.size(0) > 0 and b.t.size(0) > 0, "mxfp8_gemm: empty operand")
         for d in (a, asc, b, bsc):
             d.specialize_all_dims()
         sel.return_new_tensor([a.t.size(0), b.t.size(0)], _OUT_DTYPES[od]).specialize_all_dims()
@@ -400,15 +331,9 @@ class mxfp6_gemm(CustomOp):
         fmt = sel.attr_str(4).v
         od = sel.attr_str(5).v
         sel.attr_int(6)
-        for name, codes, scales in (("a", a.t, asc.t), ("b", b.t, bsc.t)):
-            _require(codes.dim() == 2 and codes.dtype == torch.uint8, f"mxfp6_gemm: {name} must be uint8 [rows, K*3/4] (packed 6-bit codes)")
-            _require(scales.dim() == 2 and scales.dtype == torch.uint8, f"mxfp6_gemm: {name}_scale must be uint8 [rows, K/32] (E8M0)")
-            _require(scales.size(1) > 0 and codes.size(1) == scales.size(1) * 24 and scales.size(0) == codes.size(0),
-                     f"mxfp6_gemm: {name} {tuple(codes.shape)} and {name}_scale {tuple(scales.shape)} disagree (24 code bytes per scale byte)")
-        _require(a.t.size(1) == b.t.size(1), "mxfp6_gemm: a and b disagree on K")
+        contract.check_mxfp6_pair("mxfp6_gemm", a.t, asc.t, b.t, bsc.t)
         _require(fmt in launch.FP6_FORMATS, f"mxfp6_gemm: element_format must be 'e2m3' or 'e3m2', got {fmt!r}")
         _require(od in ("bfloat16", "float32"), f"mxfp6_gemm: out_dtype must be 'bfloat16' or 'float32', got {od!r}")
-        _require(a.t.size(0) > 0 and b.t.size(0) > 0, "mxfp6_gemm: empty operand")
         for d in (a, asc, b, bsc):
             d.specialize_all_dims()
         sel.return_new_tensor([a.t.size(0), b.t.size(0)], _OUT_DTYPES[od]).specialize_all_dims()
@@ -430,13 +355,8 @@ class fp8_gemm(CustomOp):
         sel.attr_float(2)
         od = sel.attr_str(3).v
         sel.attr_int(4)
-        ok = (torch.uint8, torch.float8_e4m3fn)
-        _require(a.t.dim() == 2 and b.t.dim() == 2, "fp8_gemm: a and b must be rank 2")
-        _require(a.t.dtype in ok and b.t.dtype in ok, "fp8_gemm: a and b must be float8_e4m3fn (or its bytes as uint8)")
-        _require(a.t.size(1) == b.t.size(1), f"fp8_gemm: K mismatch, a is {tuple(a.t.shape)}, b is {tuple(b.t.shape)} (b is [N, K])")
-        _require(a.t.size(1) > 0 and a.t.size(1) % 32 == 0, f"fp8_gemm: K={a.t.size(1)} must be a positive multiple of 32")
+        contract.check_fp8_operands("fp8_gemm", a.t, b.t)
         _require(od in ("bfloat16", "float32"), f"fp8_gemm: out_dtype must be 'bfloat16' or 'float32', got {od!r}")
-        _require(a.t.size(0) > 0 and b.t.size(0) > 0, "fp8_gemm: empty operand")
         a.specialize_all_dims()
         b.specialize_all_dims()
         sel.return_new_tensor([a.t.size(0), b.t.size(0)], _OUT_DTYPES[od]).specialize_all_dims()
@@ -472,9 +392,7 @@ class mxfp4_quantize(CustomOp):
 
     def select(self, sel: KernelSelection):
         x = sel.arg_tensor(0)
-        _require(x.t.dim() == 2, "mxfp4_quantize: x must be [rows, K]")
-        _require(x.t.dtype in (torch.float16, torch.bfloat16, torch.float32), f"mxfp4_quantize: dtype {x.t.dtype} not supported")
-        _require(x.t.size(0) > 0 and x.t.size(1) > 0 and x.t.size(1) % 32 == 0, "mxfp4_quantize: K must be a positive multiple of 32")
+        contract.check_quantize_input("mxfp4_quantize", x.t)
         sel.return_new_tensor([x.t.size(0), x.t.size(1) // 2], torch.uint8)
         sel.return_new_tensor([x.t.size(0), x.t.size(1) // 32], torch.uint8)
 
@@ -495,9 +413,7 @@ class mxfp6_quantize(CustomOp):
     def select(self, sel: KernelSelection):
         x = sel.arg_tensor(0)
         fmt = sel.attr_str(1).v
-        _require(x.t.dim() == 2, "mxfp6_quantize: x must be [rows, K]")
-        _require(x.t.dtype in (torch.float16, torch.bfloat16, torch.float32), f"mxfp6_quantize: dtype {x.t.dtype} not supported")
-        _require(x.t.size(0) > 0 and x.t.size(1) > 0 and x.t.size(1) % 32 == 0, "mxfp6_quantize: K must be a positive multiple of 32")
+        contract.check_quantize_input("mxfp6_quantize", x.t)
         _require(fmt in launch.FP6_FORMATS, f"mxfp6_quantize: element_format must be 'e2m3' or 'e3m2', got {fmt!r}")
         sel.return_new_tensor([x.t.size(0), x.t.size(1) // 4 * 3], torch.uint8)
         sel.return_new_tensor([x.t.size(0), x.t.size(1) // 32], torch.uint8)
@@ -518,9 +434,7 @@ class mxfp8_quantize(CustomOp):
 
     def select(self, sel: KernelSelection):
         x = sel.arg_tensor(0)
-        _require(x.t.dim() == 2, "mxfp8_quantize: x must be [rows, K]")
-        _require(x.t.dtype in (torch.float16, torch.bfloat16, torch.float32), f"mxfp8_quantize: dtype {x.t.dtype} not supported")
-        _require(x.t.size(0) > 0 and x.t.size(1) > 0 and x.t.size(1) % 32 == 0, "mxfp8_quantize: K must be a positive multiple of 32")
+        contract.check_quantize_input("mxfp8_quantize", x.t)
         sel.return_new_tensor([x.t.size(0), x.t.size(1)], torch.uint8)
         sel.return_new_tensor([x.t.size(0), x.t.size(1) // 32], torch.uint8)
 

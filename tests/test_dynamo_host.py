@@ -115,11 +115,13 @@ def test_sdpa_is_rewritten_to_the_single_output_kernel(causal):
     assert fa.meta["val"].stride() == q.transpose(1, 2).stride()
 
 
-@pytest.mark.parametrize("what", ["mask", "head_dim", "fp32"])
+@pytest.mark.parametrize("what", ["mask", "head_dim", "fp32", "causal_unequal_lengths"])
 def test_unsupported_sdpa_is_left_alone(what):
     from iree_turbine_amd import dynamo
 
-    if what == "mask":
+    if what == "causal_unequal_lengths":  # aten masks keys > i, the kernel keys > i + Sk - Sq
+        gm = _trace(_sdpa_fn(causal=True), _h(1, 32, 2, 128), _h(1, 96, 2, 128), _h(1, 96, 2, 128))
+    elif what == "mask":
         gm = _trace(_sdpa_fn(mask=True), _h(1, 32, 2, 128), _h(1, 32, 2, 128), _h(1, 32, 2, 128), _h(32, 32))
     elif what == "head_dim":
         gm = _trace(_sdpa_fn(), _h(1, 32, 2, 64), _h(1, 32, 2, 64), _h(1, 32, 2, 64))
@@ -172,4 +174,6 @@ def test_backends_are_registered():
     import iree_turbine_amd.dynamo  # noqa: F401
 
     names = torch._dynamo.list_backends(exclude_tags=None)
-    assert "mi355" in names and "mi355_inductor" in names
+    assert "mi355" in names and "mi355_inductor" not in names
+    with pytest.raises(ValueError, match="Triton"):
+        iree_turbine_amd.dynamo.backend(nested_backend="inductor")

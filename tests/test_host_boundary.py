@@ -151,3 +151,86 @@ def test_template_getters_and_launchable_rules():
     assert mhp[lang.sym.BLOCK_K] == 256
     with pytest.raises(ValueError, match="multiple of 32"):
         get_mxfp4_gemm_kernel((32, 32, 48))
+
+
+def test_template_path_runs_the_shape_contract_before_any_device_pointer_is_taken():
+    """The getters call the launchers directly (no op `select` in between): a short operand, a wrong scale shape or
+    64-bit index tensors must be rejected on the host.  CPU tensors suffice: the contract runs before the device check."""
+    run, _ = get_gemm_kernel((64, 64, 64), dynamic_dims=True)
+    h = lambda *s: torch.zeros(*s, dtype=torch.float16)
+    with pytest.raises(ValueError, match="K mismatch"):
+        run(h(64, 64), h(64, 32), torch.zeros(64, 64))
+    with pytest.raises(ValueError, match="rank 2"):
+        run(h(64, 64), h(64), torch.zeros(64, 64))
+    u8 = lambda *s: torch.zeros(*s, dtype=torch.uint8)
+    mk, _ = get_mxfp4_gemm_kernel((32, 32, 64), dynamic_dims=True)
+    with pytest.raises(ValueError, match="a_scale shape"):
+        mk(u8(32, 32), u8(32, 1), u8(32, 32), u8(32, 2), torch.zeros(32, 32))
+    with pytest.raises(ValueError, match="b must be uint8"):
+        mk(u8(32, 32), u8(32, 2), torch.zeros(32, 32, dtype=torch.int8), u8(32, 2), torch.zeros(32, 32))
+    with pytest.raises(ValueError, match="disagree on K"):
+        mk(u8(32, 32), u8(32, 2), u8(32, 64), u8(32, 4), torch.zeros(32, 32))
+    p0, p1, hp0, _ = get_paged_decode_attention_kernels(paged_decode_attention_shape(8, 2, 128, 128, 16, 3), num_kv_splits=2)
+    p0 = ita.wave_compile(ita.WaveCompileOptions(subs=hp0), p0)
+    q, kc = h(3, 8, 128), h(10, 16, 2, 128)
+    bt, sl = torch.zeros(3, 4, dtype=torch.int32), torch.zeros(3, dtype=torch.int32)
+    pa, pm = torch.zeros(3, 8, 2, 128), torch.zeros(3, 8, 2, 2)
+    with pytest.raises(ValueError, match="seq_lens must be int32"):
+        p0(q, kc, kc, bt, sl.long(), pa, pm)
+    with pytest.raises(ValueError, match="block_table must be int32"):
+        p0(q, kc, kc, bt.long(), sl, pa, pm)
+    with pytest.raises(ValueError, match="rows must equal num_seqs"):
+        p0(q, kc, kc, bt[:2], sl, pa, pm)
+    with pytest.raises(ValueError, match="part_ml fp32"):
+        p0(q, kc, kc, bt, sl, pa, torch.zeros(3, 8, 2, 1))
+    from iree_turbine_amd import launch
+
+    with pytest.raises(ValueError, match="part_acc must be fp32"):
+        launch.paged_decode_attn_out(q, kc, kc, bt, sl, torch.zeros(3, 8, 128).half(), 0.0, 2, part_acc=pa[:, :, :1], part_ml=pm)
+    with pytest.raises(ValueError, match="start_pos must be int32"):
+        launch.kv_cache_append(h(3, 1, 2, 128), h(3, 1, 2, 128), kc, kc, bt, sl.long())
+    with pytest.raises(ValueError, match="number of kv heads"):
+        launch.kv_cache_append(h(3, 1, 4, 128), h(3, 1, 4, 128), kc, kc, bt, sl)
+
+
+def test_ragged_decode_shapes_are_not_padded_into_the_tiled_kernels():
+    """A few rows of A against a large B go to the weight-streaming kernel as they are; padding them to a 128-row
+    tile would multiply the work by 128 / M."""
+    from iree_turbine_amd import launch
+
+    assert launch._skinny_fits(16, 128256, 8192) and launch._skinny_fits(32, 32768, 8192) and launch._skinny_fits(1, 8192, 8192)
+    assert not launch._skinny_fits(65, 8192, 8192) and not launch._skinny_fits(16, 8200, 8192) and not launch._skinny_fits(16, 1024, 8192)
+
+
+def test_dtype_registry_and_shape_inference():
+    """Names and bit widths of the reference's registry (iree/turbine/kernel/_support/dtype.py:68-120); dimension
+    binding messages of tests/kernel/indexing_test.py:100-159."""
+    widths = {d.name: d.bitwidth() for d in lang.ALL_DTYPES}
+    assert widths == {"bf16": 16, "bool": 1, "i4": 4, "i8": 8, "i16": 16, "i32": 32, "i64": 64, "f16": 16, "f32": 32, "f64": 64,
+                      "f8E5M2": 8, "f8E5M2FNUZ": 8, "f8E4M3FN": 8, "f8E4M3FNUZ": 8, "f8E8M0FNU": 8, "f6E2M3FN": 6, "f4E2M1FN": 4,
+                      "index": 64}
+    assert repr(lang.f6e2m3fn) == "DataType(f6E2M3FN)" and repr(lang.bool) == "DataType(i1)" and lang.i1 is lang.bool
+    assert lang.f8e4m3fn.is_float_asm() and lang.i4.is_int_asm() and lang.index.is_index_asm() and not lang.index.is_int_asm()
+    M, N = lang.sym.M, lang.sym.N
+    assert repr(lang.KernelBuffer[M, N].of(lang.f32)) == "KernelBuffer[M, N].of(f32)"
+    assert repr(lang.InputBuffer[M].of(lang.f16)) == "InputBuffer[M].of(f16)"
+    c = lang.SymbolBindings()
+    c.bind_shaped(object(), lang.KernelBuffer[M, M, lang.f32], (1, 2))
+    with pytest.raises(ValueError, match=r"KernelBuffer\[M, M\]\.of\(f32\) attempt to bind dim M=2 conflicts with previous 1"):
+        c.finalize()
+    c = lang.SymbolBindings()
+    c.bind_shaped(object(), lang.KernelBuffer[M, N, lang.f32], (4, None))
+    with pytest.raises(ValueError, match=r"KernelBuffer\[M, N\]\.of\(f32\)\[1\]=N did not resolve to a known value"):
+        c.finalize()
+    c = lang.SymbolBindings()
+    c.bind_shaped(object(), lang.KernelBuffer[M, M / 2, lang.f32], (4, 3))
+    with pytest.raises(ValueError, match=r"KernelBuffer\[M, M/2\]\.of\(f32\)\[1\]=2 was initialized with a mismatched runtime value of 3"):
+        c.finalize()
+    c, inst, kb = lang.SymbolBindings(), object(), lang.KernelBuffer[M, M * 4, lang.f32]
+    c.bind_shaped(inst, kb, (4, None))
+    c.finalize()
+    assert c.eval_static_dim(inst, kb, 0) == 4 and c.eval_static_dim(inst, kb, 1) == 16
+    with pytest.raises(ValueError, match="already bound"):
+        c.bind_shaped(inst, kb, (4, 16))
+    with pytest.raises(ValueError, match="dim arity"):
+        c.bind_shaped(object(), kb, (4,))
