@@ -9,10 +9,18 @@ already resident in HBM.  The headline workload is the fp16 NT GEMM 8192^3 with 
 path (flash-attention prefill, paged decode, MXFP4 GEMM, remaining GEMM shapes) are measured in
 the same run and reported under "others".  Prints exactly one JSON line.
 
-Timing: W untimed warm-up steps, then exactly K steps, replayed as one HIP graph, bracketed by
+Timing: W untimed warm-up steps and about 0.3 s more of untimed launches (until the GPU's clocks have settled:
+"settle_ms" in the output), then exactly K steps, replayed as one HIP graph, bracketed by
 torch.cuda.synchronize() on both sides (wall clock -> value / ms_per_step) and, inside the same
 region, by a HIP event pair on the launch stream (-> the average device time per launch used for the
-roofline figure).
+roofline figure).  HBM-bound workloads whose operands would fit the 256 MiB memory-side cache rotate over
+enough copies of them that every timed launch streams from HBM.  The legs of the metric (GEMM, causal and
+non-causal prefill, MXFP4 GEMM, decode) each carry a "cpu_baseline": the CPU restatement of the same
+computation timed on a bounded sample on the host cores in the same run.
+
+Calibration workloads (run only when named): copy_1GiB (what the HBM counters read for a known copy) and
+mfma_{f16,fp4}_regloop_{zeros,benchmark} (what the MFMA unit sustains from registers on all-zero operands
+and on operands drawn like the benchmark's: the measured ceiling beside the datasheet peak).
 """
 
 from __future__ import annotations
@@ -63,6 +71,31 @@ MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
 }
 
 
+SETTLE_MS = 300.0  # untimed launches before the timed region, by device time
+
+
+def settle_clocks(fn, budget_ms: float = SETTLE_MS) -> int:
+    """Keeps launching `fn`, untimed, until about `budget_ms` of device time have passed; returns the launch count.
+    An idle GPU's power management takes tens of milliseconds of sustained work to reach the clocks it will hold, and
+    a kernel of 0.1-0.3 ms measured right after a handful of warm-up launches reads 10-20 % off its sustained rate
+    in either direction.  The W warm-up steps of the command line come first and are not replaced by this."""
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    done, batch = 0, 4
+    torch.cuda.synchronize()
+    e0.record()
+    while True:
+        for _ in range(batch):
+            fn()
+        done += batch
+        e1.record()
+        e1.synchronize()
+        spent = e0.elapsed_time(e1)
+        if spent >= budget_ms or done >= 20000:
+            return done
+        per_launch = max(spent / done, 1e-4)
+        batch = max(4, min(2000, int((budget_ms - spent) / per_launch / 2) + 1))  # halve the remainder: no long overshoot
+
+
 def time_steps(fn, steps: int, warmup: int):
     """Returns (wall ms per step, device ms per launch, how the steps were launched).
 
@@ -74,6 +107,7 @@ def time_steps(fn, steps: int, warmup: int):
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
+    settle_clocks(fn)
     graph = None
     try:
         graph = torch.cuda.CUDAGraph()
@@ -110,6 +144,27 @@ def time_steps(fn, steps: int, warmup: int):
 
 # ---- workloads --------------------------------------------------------------------------------
 
+MEMORY_SIDE_CACHE_BYTES = 256 << 20  # sits behind L2; a buffer set smaller than this is served from it on replays
+
+
+def rotating(call, operand_sets):
+    """A step function that takes the next operand set on every call, round robin.  HBM-bound workloads whose
+    operands fit the memory-side cache are given several copies of them (more than the cache holds in total), so
+    that every launch of the timed region streams from HBM; the launches captured into the replayed graph each
+    bind their own set."""
+    state = [0]
+
+    def fn():
+        k = state[0] % len(operand_sets)
+        state[0] += 1
+        return call(*operand_sets[k])
+    return fn
+
+
+def copies_beyond_cache(nbytes: float) -> int:
+    return max(2, int(math.ceil(1.5 * MEMORY_SIDE_CACHE_BYTES / nbytes)))
+
+
 def wl_gemm(M, N, K, out_dtype="float16", in_dtype=torch.float16):
     from oracle import inputs
 
@@ -122,13 +177,20 @@ def wl_gemm(M, N, K, out_dtype="float16", in_dtype=torch.float16):
         out_b = 4 if out_dtype == "float32" else 2
         nbytes = 2.0 * (M * K + N * K) + out_b * M * N
         hbm_bound = M <= 64  # decode-shaped: the weights are streamed once, far below the fp16 ridge point (312 flop/B)
+        fn = lambda: torch.ops.mi355.gemm_nt(ad, bd, out_dtype, -1)
+        rotate = 1
+        if hbm_bound and nbytes < MEMORY_SIDE_CACHE_BYTES:
+            rotate = copies_beyond_cache(nbytes)
+            sets = [(ad, bd)] + [(ad.clone(), bd.clone()) for _ in range(rotate - 1)]
+            fn = rotating(lambda x, w: torch.ops.mi355.gemm_nt(x, w, out_dtype, -1), sets)
         return {
-            "fn": lambda: torch.ops.mi355.gemm_nt(ad, bd, out_dtype, -1),
+            "fn": fn,
             "work": nbytes if hbm_bound else flops, "bytes": nbytes, "flops": flops, "bound": "hbm" if hbm_bound else "mfma",
             "peak": PEAK_HBM_GBS if hbm_bound else PEAK_F16_TFLOPS, "unit": "GB/s" if hbm_bound else "TFLOP/s",
             "dtype": tag, "cpu": lambda: cpu_gemm(a, b, M, N, K),
             "config": {"workload": f"gemm_{tag}_nt_{M}x{N}x{K}_{'f32' if out_dtype == 'float32' else tag}out",
-                       "M": M, "N": N, "K": K, "layout": "NT", "accumulate": "f32", "out": out_dtype, "seed": 10},
+                       "M": M, "N": N, "K": K, "layout": "NT", "accumulate": "f32", "out": out_dtype, "seed": 10,
+                       "operand_sets_rotated": rotate},
         }
     return build
 
@@ -202,13 +264,20 @@ def wl_mxfp4(M, N, K):
         flops = 2.0 * M * N * K
         nbytes = (M + N) * K / 2 + (M + N) * K / 32 + 2.0 * M * N
         hbm_bound = flops / nbytes < 1250
+        fn = lambda: torch.ops.mi355.mxfp4_gemm(*args, "bfloat16", -1)
+        rotate = 1
+        if hbm_bound and nbytes < MEMORY_SIDE_CACHE_BYTES:
+            rotate = copies_beyond_cache(nbytes)
+            sets = [tuple(args)] + [tuple(t.clone() for t in args) for _ in range(rotate - 1)]
+            fn = rotating(lambda *ops: torch.ops.mi355.mxfp4_gemm(*ops, "bfloat16", -1), sets)
         return {
-            "fn": lambda: torch.ops.mi355.mxfp4_gemm(*args, "bfloat16", -1),
+            "fn": fn,
             "work": nbytes if hbm_bound else flops, "bytes": nbytes, "flops": flops,
             "bound": "hbm" if hbm_bound else "mfma", "peak": PEAK_HBM_GBS if hbm_bound else PEAK_FP4_TFLOPS,
             "unit": "GB/s" if hbm_bound else "TFLOP/s", "dtype": "fp4(e2m1)+e8m0",
             "cpu": lambda: cpu_mxfp4(a, asc, b, bsc, M, N, K),
-            "config": {"workload": f"mxfp4_gemm_{M}x{N}x{K}_bf16out", "M": M, "N": N, "K": K, "seed": 10},
+            "config": {"workload": f"mxfp4_gemm_{M}x{N}x{K}_bf16out", "M": M, "N": N, "K": K, "seed": 10,
+                       "operand_sets_rotated": rotate},
         }
     return build
 
@@ -306,6 +375,46 @@ def wl_copy(nbytes=1 << 30):
     return build
 
 
+def wl_mfma_regloop(kind: str, data: str):
+    """Register-only MFMA loop (mi355_calibrate_mfma): the rate the MFMA unit sustains on `data` with nothing else
+    in the way.  "zeros" reads the issue-rate peak; "benchmark" uses operands drawn like the GEMM benchmarks'
+    (fp16: N(0,1)*0.1; fp4: codes uniform over all 16 values, E8M0 exponents spread over [-8, 7])."""
+    import ctypes
+
+    from iree_turbine_amd import _lib
+
+    def build(dev):
+        g = torch.Generator().manual_seed(10)
+        nbytes = 1 << 20
+        if data == "zeros":
+            ops = torch.zeros(nbytes, dtype=torch.uint8)
+        elif kind == "f16":
+            ops = (torch.randn(nbytes // 2, generator=g) * 0.1).half().view(torch.uint8)
+        else:
+            ops = torch.randint(0, 256, (nbytes,), generator=g, dtype=torch.uint8)
+        opsd = ops.to(dev)
+        workgroups, trips = 512, 2000  # two workgroups of four waves per CU
+        sink = torch.empty(workgroups * 256, dtype=torch.float32, device=dev)
+        code = 0 if kind == "f16" else (1 if data == "zeros" else 2)
+        flop = ctypes.c_double(0.0)
+        lib = _lib.load()
+
+        def fn():
+            rc = lib.mi355_calibrate_mfma(code, opsd.data_ptr(), nbytes, sink.data_ptr(), sink.numel(), workgroups, trips,
+                                          ctypes.byref(flop), _lib.current_stream_ptr(dev))
+            _lib.check(rc, "calibrate_mfma")
+        fn()
+        torch.cuda.synchronize()
+        return {
+            "fn": fn, "work": flop.value, "bytes": 0.0, "flops": flop.value, "bound": "mfma",
+            "peak": PEAK_F16_TFLOPS if kind == "f16" else PEAK_FP4_TFLOPS, "unit": "TFLOP/s",
+            "dtype": "f16" if kind == "f16" else "fp4(e2m1)+e8m0", "cpu": lambda: None,
+            "config": {"workload": f"mfma_{kind}_regloop_{data}", "workgroups": workgroups, "trips": trips,
+                       "instruction": "v_mfma_f32_32x32x16_f16" if kind == "f16" else "v_mfma_scale_f32_32x32x64_f8f6f4 (fp4 x fp4)"},
+        }
+    return build
+
+
 WORKLOADS = {
     "gemm_8192": wl_gemm(8192, 8192, 8192),
     "gemm_4096": wl_gemm(4096, 4096, 4096),
@@ -328,7 +437,13 @@ WORKLOADS = {
     "mxfp8_4096x8192x8192": wl_mxfp8(4096, 8192, 8192),
     "mxfp6_4096x8192x8192": wl_mxfp6(4096, 8192, 8192),
 }
-CALIBRATION = {"copy_1GiB": wl_copy()}  # not part of the path: run only when named with --workload
+CALIBRATION = {  # not part of the path: run only when named with --workload
+    "copy_1GiB": wl_copy(),
+    "mfma_f16_regloop_zeros": wl_mfma_regloop("f16", "zeros"),
+    "mfma_f16_regloop_benchmark": wl_mfma_regloop("f16", "benchmark"),
+    "mfma_fp4_regloop_zeros": wl_mfma_regloop("fp4", "zeros"),
+    "mfma_fp4_regloop_benchmark": wl_mfma_regloop("fp4", "benchmark"),
+}
 WORKLOADS_ALL = {**WORKLOADS, **CALIBRATION}
 HEADLINE = "gemm_8192"
 
@@ -462,9 +577,14 @@ def measure(name: str, dev, steps: int, warmup: int, with_cpu: bool):
         rec["tflops"] = wl["flops"] / (dev_ms * 1e-3) / 1e12
     if with_cpu:
         cpu = wl["cpu"]()
-        cpu.update({"cores": torch.get_num_threads(), "kind": "port"})
-        rec["cpu_baseline"] = cpu
+        if cpu is not None:
+            cpu.update({"cores": torch.get_num_threads(), "kind": "port"})
+            rec["cpu_baseline"] = cpu
     return rec
+
+
+# the legs of the metric (GEMM, causal prefill, MXFP4 GEMM, decode): each gets its CPU baseline in the same run
+CPU_TIMED = ("gemm_8192", "fa_causal", "fa_noncausal", "decode", "mxfp4_4096x8192x8192", "mxfp4_32x8192x8192")
 
 
 def main() -> int:
@@ -494,7 +614,7 @@ def main() -> int:
             if name == args.workload:
                 continue
             torch.cuda.empty_cache()
-            rec = measure(name, dev, args.steps, args.warmup, with_cpu=False)
+            rec = measure(name, dev, args.steps, args.warmup, with_cpu=not args.no_cpu and name in CPU_TIMED)
             rec.pop("config")
             others.append(rec)
 
@@ -514,6 +634,7 @@ def main() -> int:
         "config": head["config"],
         "kernel_ms_avg": head["kernel_ms_avg"],
         "launch": head["launch"],
+        "settle_ms": SETTLE_MS,
         "roofline": head["roofline"],
         "cpu_baseline": head.get("cpu_baseline"),
         "host": {"cpu": platform.processor() or platform.machine(), "os_cpu_count": os.cpu_count(),

@@ -353,6 +353,21 @@ int mi355_mxfp4_quantize(const void* x, int in_dtype, int64_t rows, int64_t K,
 int mi355_mxfp8_quantize(const void* x, int in_dtype, int64_t rows, int64_t K,
                          void* codes, void* scales, void* stream);
 
+/*
+ * Calibration, not part of the path: a register-only MFMA loop (no LDS, no memory traffic inside the
+ * loop) on caller-supplied operand bytes, to measure what the MFMA unit of the board sustains on a
+ * given data distribution -- the ceiling that the roofline fractions of the GEMM and attention
+ * kernels can be read against beside the datasheet peak.  No counterpart in the reference; it plays
+ * the part of the plain-copy workload for the HBM figures.
+ * kind 0: v_mfma_f32_32x32x16_f16; 1: v_mfma_scale_f32_32x32x64_f8f6f4 with fp4 operands and unit
+ * scales; 2: the same with E8M0 scales spread over 2^-8 .. 2^7.  operands: operand_bytes (a power of
+ * two >= 16) of device memory read once before the loop; sink: >= workgroups * 256 floats, written
+ * once after it; *flop_per_launch (optional, host memory) receives the flop count of the launch.
+ */
+int mi355_calibrate_mfma(int kind, const void* operands, int64_t operand_bytes, float* sink,
+                         int64_t sink_floats, int64_t workgroups, int64_t trips,
+                         double* flop_per_launch, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -15,7 +15,7 @@ from pathlib import Path
 CSRC = Path(__file__).resolve().parent / "csrc"
 LIB_NAME = "libturbine_mi355.so"
 LIB_PATH = CSRC / LIB_NAME
-SOURCES = ["capi.hip", "gemm_f16_nt.hip", "flash_attn_fwd.hip", "paged_decode.hip", "gemm_mxfp4.hip", "gemm_mxfp8.hip", "gemm_mxfp6.hip", "quantize_mxfp4.hip", "quantize_mxfp6.hip"]
+SOURCES = ["capi.hip", "gemm_f16_nt.hip", "flash_attn_fwd.hip", "paged_decode.hip", "gemm_mxfp4.hip", "gemm_mxfp8.hip", "gemm_mxfp6.hip", "quantize_mxfp4.hip", "quantize_mxfp6.hip", "calibrate.hip"]
 
 # -packed-fp32-ops: keep the compiler from forming v_pk_{add,mul,fma}_f32.
 HIPCC_FLAGS = [

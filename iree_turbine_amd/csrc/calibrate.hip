@@ -1,0 +1,104 @@
+// Calibration loops: what the MFMA unit of this board sustains when nothing else is in the way.
+//
+// Every wave keeps its operands in registers and issues MFMAs back to back: no LDS, no global traffic inside the
+// loop.  The rate such a loop sustains depends on the DATA (the board's power limit lowers the clock as more bits
+// toggle), so the caller supplies the operand bytes: all zeros reads the issue-rate peak, operands drawn like a
+// benchmark's read the ceiling any kernel can reach on that benchmark's data.  A roofline fraction quoted against
+// the datasheet peak can then be read against the measured ceiling as well.
+#include "common.hpp"
+
+namespace mi355 {
+
+constexpr int CAL_WAVES = 4;      // one wave per SIMD
+constexpr int CAL_CHAINS = 8;     // independent accumulator chains per wave: more than the MFMA pipeline is deep
+
+// 32x32x16 fp16 MFMAs: per wave and trip, CAL_CHAINS MFMAs of 32*32*16*2 flop.
+__global__ __launch_bounds__(CAL_WAVES * 64) void calibrate_mfma_f16_kernel(const half8* __restrict__ operands, unsigned mask,
+                                                                            float* __restrict__ sink, int trips) {
+  const unsigned t = threadIdx.x + blockIdx.x * blockDim.x;
+  half8 a[4], b[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    a[i] = operands[(t * 8 + i) & mask];
+    b[i] = operands[(t * 8 + 4 + i) & mask];
+  }
+  floatx16 c[CAL_CHAINS];
+#pragma unroll
+  for (int i = 0; i < CAL_CHAINS; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) c[i][r] = 0.f;
+#pragma unroll 1
+  for (int it = 0; it < trips; it++) {
+#pragma unroll
+    for (int i = 0; i < CAL_CHAINS; i++) c[i] = mfma_32x32x16(a[i & 3], b[(i >> 1) & 3], c[i]);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < CAL_CHAINS; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) s += c[i][r];
+  sink[t] = s;
+}
+
+// Scaled 32x32x64 MFMAs with fp4 operands (16 bytes per lane; the upper half of the operand registers is unused):
+// per wave and trip, CAL_CHAINS MFMAs of 32*32*64*2 flop.  scale_mode 0: every block scale 2^0; 1: E8M0 bytes
+// 119..134 derived from the operand bits (exponents spread over [-8, 7] like a block-scaled benchmark's).
+__global__ __launch_bounds__(CAL_WAVES * 64) void calibrate_mfma_fp4_kernel(const intx4* __restrict__ operands, unsigned mask,
+                                                                            float* __restrict__ sink, int trips, int scale_mode) {
+  const unsigned t = threadIdx.x + blockIdx.x * blockDim.x;
+  intx8 a[4], b[4];
+  int sa[4], sb[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const intx4 x = operands[(t * 8 + i) & mask], y = operands[(t * 8 + 4 + i) & mask];
+    a[i] = intx8{x[0], x[1], x[2], x[3], 0, 0, 0, 0};
+    b[i] = intx8{y[0], y[1], y[2], y[3], 0, 0, 0, 0};
+    sa[i] = scale_mode ? 119 + ((x[0] >> 3) & 15) : 127;
+    sb[i] = scale_mode ? 119 + ((y[1] >> 5) & 15) : 127;
+  }
+  floatx16 c[CAL_CHAINS];
+#pragma unroll
+  for (int i = 0; i < CAL_CHAINS; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) c[i][r] = 0.f;
+#pragma unroll 1
+  for (int it = 0; it < trips; it++) {
+#pragma unroll
+    for (int i = 0; i < CAL_CHAINS; i++)
+      c[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[i & 3], b[(i >> 1) & 3], c[i], 4, 4, 0, sa[i & 3], 0, sb[(i >> 1) & 3]);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < CAL_CHAINS; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) s += c[i][r];
+  sink[t] = s;
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+// kind 0: fp16 32x32x16; kind 1: fp4 32x32x64 with unit scales; kind 2: fp4 with spread scales.
+extern "C" int mi355_calibrate_mfma(int kind, const void* operands, int64_t operand_bytes, float* sink, int64_t sink_floats,
+                                    int64_t workgroups, int64_t trips, double* flop_per_launch, void* stream) {
+  if (!operands || !sink) return fail(-MI355_E_NULL, "calibrate_mfma: null pointer");
+  if (kind < 0 || kind > 2) return fail(-MI355_E_DTYPE, "calibrate_mfma: kind %d unknown (0 fp16, 1 fp4, 2 fp4 with spread scales)", kind);
+  if (operand_bytes < 16 || (operand_bytes & (operand_bytes - 1)) || operand_bytes > (1ll << 30))
+    return fail(-MI355_E_SHAPE, "calibrate_mfma: operand_bytes %lld must be a power of two in [16, 2^30]", (long long)operand_bytes);
+  if (workgroups <= 0 || workgroups > 65535 || trips <= 0 || trips > (1 << 24))
+    return fail(-MI355_E_SHAPE, "calibrate_mfma: workgroups %lld / trips %lld out of range", (long long)workgroups, (long long)trips);
+  if (sink_floats < workgroups * CAL_WAVES * 64)
+    return fail(-MI355_E_SCRATCH, "calibrate_mfma: sink needs %lld floats", (long long)(workgroups * CAL_WAVES * 64));
+  if (!aligned16(operands)) return fail(-MI355_E_ALIGN, "calibrate_mfma: operands must be 16-byte aligned");
+  const unsigned mask = (unsigned)(operand_bytes / 16 - 1);
+  dim3 grid((unsigned)workgroups), block(CAL_WAVES * 64);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const double per_mfma = kind == 0 ? 2.0 * 32 * 32 * 16 : 2.0 * 32 * 32 * 64;
+  if (flop_per_launch) *flop_per_launch = per_mfma * CAL_CHAINS * (double)trips * CAL_WAVES * (double)workgroups;
+  if (kind == 0)
+    hipLaunchKernelGGL(calibrate_mfma_f16_kernel, grid, block, 0, s, (const half8*)operands, mask, sink, (int)trips);
+  else
+    hipLaunchKernelGGL(calibrate_mfma_fp4_kernel, grid, block, 0, s, (const intx4*)operands, mask, sink, (int)trips, kind == 2);
+  return check_launch("calibrate_mfma", grid, block, 0);
+}

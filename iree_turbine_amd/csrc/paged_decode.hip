@@ -33,7 +33,7 @@ __global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
     const half_t* __restrict__ Q, const half_t* __restrict__ Kc, const half_t* __restrict__ Vc,
     const int* __restrict__ block_table, const int* __restrict__ seq_lens, float* __restrict__ part_acc,
     float* __restrict__ part_ml, half_t* __restrict__ out, int num_kv_heads, int max_pages_per_seq, int num_splits,
-    float scale_log2e, int window, int page_shift) {
+    float scale_log2e, int window, int page_shift, int num_pages) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -100,12 +100,22 @@ __global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
   const int vr_base = vr_row * 256 + ((((i16 & 3) >> 1) ^ (2 * (vr_row & 7))) * 16) + (i16 & 1) * 8;  // ^ (dt*32)
 
   half8 kf[2][2][4];  // [buffer][page][ks]
+  // A table entry outside [0, num_pages) (a stale or padding id inside a sequence's live range) must not become an
+  // address: such a block is fetched from page 0 instead and bad[buffer] remembers to drop it -- its scores become
+  // -inf and its V rows zero, so it contributes nothing.  Wave-uniform, so the flags live in scalar registers.
+  int bad[2] = {0, 0};  // bit x: block x of the step in this buffer is dropped
   auto issue = [&](int step, int buf) {
     const int pa = p_begin + 2 * (wave + PD_WAVES * step);
     // the kernel walks 16-token blocks; a page of 16 << page_shift tokens is that many consecutive blocks
     const int sub = (1 << page_shift) - 1;
-    const int pg0 = (bt[pa >> page_shift] << page_shift) + (pa & sub);
-    const int pg1 = (pa + 1 < p_end) ? (bt[(pa + 1) >> page_shift] << page_shift) + ((pa + 1) & sub) : pg0;
+    int id0 = bt[pa >> page_shift];
+    int id1 = (pa + 1 < p_end) ? bt[(pa + 1) >> page_shift] : id0;
+    const int drop0 = (unsigned)id0 >= (unsigned)num_pages, drop1 = (unsigned)id1 >= (unsigned)num_pages;
+    id0 = drop0 ? 0 : id0;
+    id1 = drop1 ? 0 : id1;
+    bad[buf] = drop0 | (drop1 << 1);
+    const int pg0 = (id0 << page_shift) + (pa & sub);
+    const int pg1 = (pa + 1 < p_end) ? (id1 << page_shift) + ((pa + 1) & sub) : pg0;
     char* dst = my_lds + buf * 8192;
 #pragma unroll
     for (int x = 0; x < 2; x++) {
@@ -145,7 +155,8 @@ __global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
           asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
         const int pa = p_begin + 2 * (wave + PD_WAVES * step);
-        const bool has1 = pa + 1 < p_end;
+        const bool drop0 = bad[b] & 1;
+        const bool has1 = pa + 1 < p_end && !(bad[b] & 2);
         floatx4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) s0 = mfma16_16x16x32<BF>(kf[b][0][ks], qf[ks], s0);
@@ -153,18 +164,21 @@ __global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
         for (int ks = 0; ks < 4; ks++) s1 = mfma16_16x16x32<BF>(kf[b][1][ks], qf[ks], s1);
         // lane (head i16, g) holds tokens 4g + r of each page
         const int tok0 = pa * 16 + 4 * g;
-        const bool ragged = pa * 16 + 32 > L;  // wave-uniform: this step reaches past the sequence end
+        const bool ragged = pa * 16 + 32 > L || bad[b] != 0;  // wave-uniform: this step reaches past the sequence end or drops a block
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-          if (tok0 + r >= L || tok0 + r < lo) s0[r] = -INFINITY;
+          if (drop0 || tok0 + r >= L || tok0 + r < lo) s0[r] = -INFINITY;
           if (!has1 || tok0 + 16 + r >= L) s1[r] = -INFINITY;  // the second page of a step lies behind `lo`
         }
         float mx = fmaxf(fmaxf(fmaxf(s0[0], s0[1]), fmaxf(s0[2], s0[3])), fmaxf(fmaxf(s1[0], s1[1]), fmaxf(s1[2], s1[3])));
         mx = fmaxf(mx, __shfl_xor(mx, 16));
         mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_run, mx);  // finite: page pa always holds a valid token (the window's first or its own first)
-        const float alpha = fast_exp2((m_run - m_new) * scale_log2e);
-        const float mc = m_new * scale_log2e;
+        // block pa holds a valid token (the window's first or its own first) unless it was dropped: m_new may still be
+        // -inf then, and (-inf) - (-inf) must not reach the exponentials
+        const float m_new = fmaxf(m_run, mx);
+        const bool none_yet = m_new == -INFINITY;
+        const float alpha = none_yet ? 1.f : fast_exp2((m_run - m_new) * scale_log2e);
+        const float mc = none_yet ? 0.f : m_new * scale_log2e;
         m_run = m_new;
         half8 pf;
         float psum = 0.f;
@@ -185,7 +199,7 @@ __global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
           if (ragged) {  // tokens at or beyond L may hold anything (NaN included): 0 * garbage must stay 0
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-              if (tok0 + e >= L) lo[e] = (half_t)0;
+              if (drop0 || tok0 + e >= L) lo[e] = (half_t)0;
               if (!has1 || tok0 + 16 + e >= L) hi[e] = (half_t)0;
             }
           }
@@ -278,7 +292,7 @@ const char* decode_variant_name(int i) { return i == 0 ? kDecodeVariants[0] : nu
 template <int G, bool BF>
 static int launch_phase0(const void* q, const void* kc, const void* vc, const int32_t* bt, const int32_t* sl, float* pacc,
                          float* pml, void* out, int num_seqs, int num_kv_heads, int max_pages, int num_splits, float scale,
-                         int window, int page_shift, hipStream_t stream) {
+                         int window, int page_shift, int num_pages, hipStream_t stream) {
   auto kern = paged_decode_phase0<G, BF>;
   constexpr int lds_bytes = PD_WAVES * PD_WAVE_LDS;
   static_assert(lds_bytes >= (int)((2 * PD_WAVES * 16 + PD_WAVES * G * 128) * sizeof(float)), "merge area must fit");
@@ -286,7 +300,7 @@ static int launch_phase0(const void* q, const void* kc, const void* vc, const in
   if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "paged_decode_phase0")) return rc;
   dim3 grid(num_splits, num_kv_heads, num_seqs), block(PD_WAVES * 64);
   hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)q, (const half_t*)kc, (const half_t*)vc, bt, sl,
-                     pacc, pml, (half_t*)out, num_kv_heads, max_pages, num_splits, scale * 1.4426950408889634f, window, page_shift);
+                     pacc, pml, (half_t*)out, num_kv_heads, max_pages, num_splits, scale * 1.4426950408889634f, window, page_shift, num_pages);
   return check_launch("paged_decode_phase0", grid, block, lds_bytes);
 }
 
@@ -319,10 +333,10 @@ static int check_decode_args(const char* fn, int64_t num_seqs, int64_t hq, int64
 template <bool BF>
 static int run_phase0(const void* q, const void* kc, const void* vc, const int32_t* bt, const int32_t* sl, float* pacc,
                       float* pml, void* out, int64_t num_seqs, int64_t hq, int64_t hkv, int64_t max_pages,
-                      int64_t num_splits, float scale, int window, int page_shift, hipStream_t stream) {
+                      int64_t num_splits, float scale, int window, int page_shift, int64_t num_pages, hipStream_t stream) {
   const int G = (int)(hq / hkv);
 #define MI355_PD_CASE(GG) \
-  case GG: return launch_phase0<GG, BF>(q, kc, vc, bt, sl, pacc, pml, out, (int)num_seqs, (int)hkv, (int)max_pages, (int)num_splits, scale, window, page_shift, stream)
+  case GG: return launch_phase0<GG, BF>(q, kc, vc, bt, sl, pacc, pml, out, (int)num_seqs, (int)hkv, (int)max_pages, (int)num_splits, scale, window, page_shift, (int)num_pages, stream)
   switch (G) {
     MI355_PD_CASE(1);
     MI355_PD_CASE(2);
@@ -351,7 +365,7 @@ static int phase0_entry(const void* q, const void* k_cache, const void* v_cache,
   if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(part_acc))
     return fail(-MI355_E_ALIGN, "paged_decode_phase0: q, k_cache, v_cache, part_acc must be 16-byte aligned");
   return run_phase0<BF>(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, nullptr, num_seqs, num_q_heads,
-                           num_kv_heads, max_pages_per_seq, num_splits, scale, 0, page_shift_of(page_size),
+                           num_kv_heads, max_pages_per_seq, num_splits, scale, 0, page_shift_of(page_size), num_pages,
                            reinterpret_cast<hipStream_t>(stream));
 }
 
@@ -411,11 +425,11 @@ static int decode_attn(const char* fn, const void* q, const void* k_cache, const
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (num_splits == 1)
     return run_phase0<BF>(q, k_cache, v_cache, block_table, seq_lens, nullptr, nullptr, out, num_seqs, num_q_heads, num_kv_heads,
-                          max_pages_per_seq, 1, scale, (int)window, page_shift_of(page_size), s);
+                          max_pages_per_seq, 1, scale, (int)window, page_shift_of(page_size), num_pages, s);
   if (!part_acc || !part_ml) return fail(-MI355_E_SCRATCH, "%s: num_splits > 1 needs part_acc / part_ml scratch", fn);
   if (!aligned16(part_acc)) return fail(-MI355_E_ALIGN, "%s: part_acc must be 16-byte aligned", fn);
   if (int rc = run_phase0<BF>(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, nullptr, num_seqs, num_q_heads,
-                              num_kv_heads, max_pages_per_seq, num_splits, scale, (int)window, page_shift_of(page_size), s))
+                              num_kv_heads, max_pages_per_seq, num_splits, scale, (int)window, page_shift_of(page_size), num_pages, s))
     return rc;
   return run_phase1<BF>(part_acc, part_ml, out, num_seqs, num_q_heads, D, num_splits, stream);
 }

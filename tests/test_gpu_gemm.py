@@ -101,7 +101,7 @@ def test_gemm_contract_errors(dev):
         torch.ops.mi355.gemm_nt(a, a, "int8", -1)
 
 
-@pytest.mark.parametrize("shape", [(8192, 8192, 8192), (4096, 4096, 4096), (2048, 10240, 8192)])
+@pytest.mark.parametrize("shape", [(8192, 8192, 8192), (4096, 4096, 4096), (2048, 10240, 8192), (2048, 57344, 8192)])
 def test_gemm_full_size_properties(dev, shape):
     """At benchmark sizes: sampled rows/columns against the fp32 oracle, plus linearity in A."""
     import iree_turbine_amd  # noqa: F401
@@ -126,7 +126,7 @@ def test_gemm_full_size_properties(dev, shape):
     assert torch.equal(c32.half(), c)  # the fp16 epilogue is round-to-nearest-even of the fp32 result
 
 
-@pytest.mark.parametrize("shape", [(8192, 8192, 8192), (2048, 10240, 8192)])
+@pytest.mark.parametrize("shape", [(8192, 8192, 8192), (2048, 10240, 8192), (2048, 57344, 8192)])
 def test_gemm_full_size_repeatable(dev, shape):
     """Whole-matrix checks at benchmark sizes: every tiled variant is bit-identical across launches (an
     unsynchronised LDS stage reuse would differ from run to run) and agrees with the simple generic kernel."""
@@ -138,6 +138,7 @@ def test_gemm_full_size_repeatable(dev, shape):
     a, b = [t.to(dev) for t in inputs.gemm_inputs(M, N, K)]
     names = ita._lib.variants("gemm_f16_nt")
     generic = torch.ops.mi355.gemm_nt(a, b, "float32", len(names) - 1)
+    by_name = {}
     for variant in range(len(names) - 1):
         if names[variant].startswith("skinny"):
             continue  # M <= 32 only: covered by test_gemm_skinny_m
@@ -145,6 +146,13 @@ def test_gemm_full_size_repeatable(dev, shape):
         for _ in range(2):
             assert torch.equal(first, torch.ops.mi355.gemm_nt(a, b, "float32", variant)), names[variant]
         torch.testing.assert_close(first, generic, rtol=1e-3, atol=1e-3)
+        if names[variant].startswith("staged"):
+            by_name[names[variant]] = first
+        del first
+    # the tail split hands the last tile columns to a second kernel that adds K in the same order: the whole
+    # matrix equals the unsplit staged kernel's bit for bit
+    staged = [v for k, v in sorted(by_name.items())]
+    assert len(staged) == 2 and torch.equal(staged[0], staged[1])
 
 
 @pytest.mark.parametrize("shape", [(4096, 4608, 192), (4352, 4352, 128), (8192, 8704, 320), (512, 256, 4096)])

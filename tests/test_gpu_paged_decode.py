@@ -78,6 +78,38 @@ def test_decode_edge_lengths_and_poison(dev):
 
 
 @pytest.mark.parametrize("splits", [1, 3])
+def test_decode_bad_page_ids_inside_a_sequence_are_dropped(dev, splits):
+    """A stale or padding id (-1, or one past the cache) INSIDE a sequence's live range must not become an address:
+    that block contributes nothing, exactly as if its 16 tokens were masked out -- also when it is the first block a
+    wave sees, and when every block of a sequence is bad (zeros out)."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs
+
+    announce(f"paged decode bad page ids splits={splits}")
+    q, kc, vc, bt, sl = inputs.paged_decode_inputs(num_seqs=4, num_q_heads=8, num_kv_heads=2, min_len=200, max_len=400, seed=13)
+    P = kc.shape[0]
+    bad = bt.clone()
+    bad[0, 0], bad[0, 3], bad[1, 1], bad[2, 5] = -1, P, 2**30, -(2**31)
+    n3 = (int(sl[3]) + 15) // 16
+    bad[3, :n3] = -1
+    got = torch.ops.mi355.paged_decode_attn(*_to(dev, q, kc, vc, bad, sl), 0.0, splits).float().cpu()
+    assert torch.isfinite(got).all()
+    assert torch.equal(got[3], torch.zeros(8, 128))
+    # the same attention with the dropped blocks masked out by hand: dense softmax over the remaining tokens
+    for s, dropped in ((0, (0, 3)), (1, (1,)), (2, (5,))):
+        L = int(sl[s])
+        keep = torch.ones(L, dtype=torch.bool)
+        for b in dropped:
+            keep[b * 16:(b + 1) * 16] = False
+        pages = bt[s, :(L + 15) // 16].long()
+        k = kc[pages].reshape(-1, 2, 128)[:L][keep].float()
+        v = vc[pages].reshape(-1, 2, 128)[:L][keep].float()
+        for h in range(8):
+            p = torch.softmax((k[:, h // 4] @ q[s, h].float()) * 128 ** -0.5, dim=0)
+            torch.testing.assert_close(got[s, h], p @ v[:, h // 4], rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("splits", [1, 3])
 def test_decode_lengths_outside_the_table(dev, splits):
     """A length beyond what the block table addresses is cut to the table's reach, a negative one counts as
     empty: the table is never read past its end."""
