@@ -179,6 +179,24 @@ int mi355_paged_decode_attn(const void* q, const void* k_cache, const void* v_ca
                             int64_t num_pages, int64_t num_splits, float scale, void* stream);
 
 /*
+ * mi355_paged_decode_attn for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference,
+ * whose runtime allocates its results itself (iree/turbine/runtime/op_reg/eager.py:195-199).
+ * Same arguments, kernels and results as mi355_paged_decode_attn, fp16, without part_acc / part_ml:
+ * the split-K partials go to a 16.25 MiB array that is part of the library's device image (one copy
+ * per GPU the library is used on, held until the process ends).  The call allocates nothing and
+ * frees nothing.  Limit: num_seqs * num_q_heads * num_splits <= 32768, otherwise -MI355_E_SCRATCH
+ * (nothing launched).  Every call on a GPU uses that GPU's one array: calls that may overlap on
+ * one GPU (different streams or threads) race on it and must be serialised by the caller; calls
+ * on one stream are ordered.  The first call on a device looks up the array's address.
+ */
+int mi355_paged_decode_attn_static(const void* q, const void* k_cache, const void* v_cache,
+                                   const int32_t* block_table, const int32_t* seq_lens, void* out,
+                                   int64_t num_seqs, int64_t num_q_heads, int64_t num_kv_heads,
+                                   int64_t D, int64_t page_size, int64_t max_pages_per_seq,
+                                   int64_t num_pages, int64_t num_splits, float scale, void* stream);
+
+/*
  * Paged decode with a sliding window: as mi355_paged_decode_attn, but a query
  * attends only to the last `window` cached tokens of its sequence (window == 0:
  * all of them).  Pages wholly in front of the window are not read.  Same masking

@@ -464,6 +464,60 @@ extern "C" int mi355_paged_decode_attn_window_bf16(const void* q, const void* k_
                            window, stream);
 }
 
+// ---- decode for callers that cannot allocate --------------------------------------------------------------
+// The split-K partials live in a file-scope device array instead of caller memory.  Every GPU the library runs on
+// holds its own copy of the array (at its own address) until the process ends; the address is looked up once per
+// device, with that device current, and kept.
+constexpr int64_t PD_STATIC_MAX_ROWS = 32768;  // num_seqs * num_q_heads * num_splits
+static __device__ __align__(256) float scratch[PD_STATIC_MAX_ROWS * (128 + 2)];  // 16.25 MiB: part_acc, then part_ml
+
+static std::atomic<float*> g_scratch_ptr[64];  // per device ordinal; host code uses these, never the array's name
+
+static int static_scratch(const char* fn, float** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    set_error("%s: hipGetDevice: %s", fn, hipGetErrorString(e));
+    return (int)e;
+  }
+  if (dev < 0 || dev >= 64) return fail(-MI355_E_SHAPE, "%s: device ordinal %d not supported (0..63)", fn, dev);
+  float* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    e = hipGetSymbolAddress(reinterpret_cast<void**>(&p), HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      set_error("%s: hipGetSymbolAddress(scratch) on device %d: %s", fn, dev, hipGetErrorString(e));
+      return e != hipSuccess ? (int)e : (int)hipErrorInvalidSymbol;
+    }
+    g_scratch_ptr[dev].store(p, std::memory_order_release);  // two threads racing here store the same address
+  }
+  *ptr = p;
+  return 0;
+}
+
+extern "C" int mi355_paged_decode_attn_static(const void* q, const void* k_cache, const void* v_cache,
+                                              const int32_t* block_table, const int32_t* seq_lens, void* out,
+                                              int64_t num_seqs, int64_t num_q_heads, int64_t num_kv_heads, int64_t D,
+                                              int64_t page_size, int64_t max_pages_per_seq, int64_t num_pages,
+                                              int64_t num_splits, float scale, void* stream) {
+  const char* fn = "paged_decode_attn_static";
+  if (num_splits <= 1)  // a single split needs no partials at all
+    return decode_attn<false>(fn, q, k_cache, v_cache, block_table, seq_lens, out, nullptr, nullptr, num_seqs, num_q_heads,
+                              num_kv_heads, D, page_size, max_pages_per_seq, num_pages, num_splits, scale, 0, stream);
+  if (num_seqs <= 0 || num_q_heads <= 0 || num_seqs > PD_STATIC_MAX_ROWS || num_q_heads > PD_STATIC_MAX_ROWS ||
+      num_splits > PD_STATIC_MAX_ROWS || num_seqs * num_q_heads * num_splits > PD_STATIC_MAX_ROWS)
+    return fail(-MI355_E_SCRATCH, "%s: num_seqs * num_q_heads * num_splits = %lld x %lld x %lld exceeds the built-in scratch "
+                "of %lld rows; use mi355_paged_decode_attn with caller-owned scratch", fn, (long long)num_seqs,
+                (long long)num_q_heads, (long long)num_splits, (long long)PD_STATIC_MAX_ROWS);
+  float* base = nullptr;
+  if (int rc = static_scratch(fn, &base)) return rc;
+  // Phase 0 writes every (seq, q head, split) row of both arrays -- an empty split writes (-inf, 0, zeros) -- so
+  // nothing of the previous call's contents is read and nothing needs clearing.
+  float* part_acc = base;
+  float* part_ml = base + num_seqs * num_q_heads * num_splits * 128;
+  return decode_attn<false>(fn, q, k_cache, v_cache, block_table, seq_lens, out, part_acc, part_ml, num_seqs, num_q_heads,
+                            num_kv_heads, D, page_size, max_pages_per_seq, num_pages, num_splits, scale, 0, stream);
+}
+
 // ---- KV-cache append: the step in front of decode -------------------------------------------------------
 // Writes tokens start_pos[s] .. start_pos[s] + n_new - 1 of every sequence into its pages.  A token's kv
 // heads are contiguous both in the source ([seq][token][head][128]) and in a page slot, so one token is one
