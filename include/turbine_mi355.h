@@ -179,6 +179,24 @@ int mi355_paged_decode_attn(const void* q, const void* k_cache, const void* v_ca
                             int64_t num_pages, int64_t num_splits, float scale, void* stream);
 
 /*
+ * Paged decode in ONE launch: as mi355_paged_decode_attn_window (window == 0: all tokens), for fp16
+ * or bf16 tensors (dtype = MI355_F16 | MI355_BF16), with the merge of the kv splits done inside the
+ * phase-0 kernel by whichever workgroup of a (sequence, kv head) finishes last, instead of by a second
+ * launch -- when the whole grid is resident at once (num_seqs * num_kv_heads * num_splits <= 512);
+ * larger grids run the two launches, which is faster there, and leave `arrivals` untouched.  arrivals: int32 [num_seqs * num_kv_heads] of device memory that is all zero when the kernel
+ * starts; the kernel leaves it all zero again, so one buffer zeroed once serves every later call that is
+ * ordered after this one (calls that may overlap need a buffer each).  Not needed (may be NULL) for
+ * num_splits == 1.  No counterpart in the reference (GQA semantics tests/dynamo/llama_test.py:82-91).
+ */
+int mi355_paged_decode_attn_fused(const void* q, const void* k_cache, const void* v_cache,
+                                  const int32_t* block_table, const int32_t* seq_lens, void* out,
+                                  float* part_acc, float* part_ml, int32_t* arrivals,
+                                  int64_t num_seqs, int64_t num_q_heads, int64_t num_kv_heads,
+                                  int64_t D, int64_t page_size, int64_t max_pages_per_seq,
+                                  int64_t num_pages, int64_t num_splits, float scale,
+                                  int64_t window, int dtype, void* stream);
+
+/*
  * mi355_paged_decode_attn for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference,
  * whose runtime allocates its results itself (iree/turbine/runtime/op_reg/eager.py:195-199).

@@ -67,6 +67,7 @@ _PROTOS = {
         + [c_int64] * 8
         + [c_float, c_void_p],
     ),
+    "mi355_paged_decode_attn_fused": (c_int, [c_void_p] * 9 + [c_int64] * 8 + [c_float, c_int64, c_int, c_void_p]),
     "mi355_paged_decode_attn_static": (c_int, [c_void_p] * 6 + [c_int64] * 8 + [c_float, c_void_p]),
     "mi355_paged_decode_attn_window": (
         c_int,

@@ -28,12 +28,44 @@ constexpr int PD_WAVE_LDS = 2 * 8192;  // two stages of two 4 KiB V pages
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Merge of the kv splits of one (sequence, q head) for output element d: the one statement of this arithmetic,
+// used by the merge kernel and by the last-arriving workgroup of the one-launch form, so that both give the same
+// bits.  COHERENT: read with device-scope loads (partials written by other workgroups of the running kernel,
+// possibly through another XCD's L2).
+template <bool COHERENT>
+__device__ __forceinline__ float pd_load(const float* p) {
+  if constexpr (COHERENT) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  else return *p;
+}
+template <bool COHERENT>
+__device__ __forceinline__ float merge_splits(const float* part_acc, const float* part_ml, size_t row, int d, int num_splits) {
+  const float* ml = part_ml + row * num_splits * 2;
+  float m_tot = -INFINITY;
+  for (int s = 0; s < num_splits; s++) m_tot = fmaxf(m_tot, pd_load<COHERENT>(ml + 2 * s));
+  float acc = 0.f, l = 0.f;
+  if (m_tot > -INFINITY) {
+    for (int s = 0; s < num_splits; s++) {
+      const float ms = pd_load<COHERENT>(ml + 2 * s);
+      if (ms > -INFINITY) {
+        const float w = fast_exp2(ms - m_tot);
+        acc = __builtin_fmaf(w, pd_load<COHERENT>(part_acc + (row * num_splits + s) * 128 + d), acc);
+        l = __builtin_fmaf(w, pd_load<COHERENT>(ml + 2 * s + 1), l);
+      }
+    }
+  }
+  float r = acc * (l > 0.f ? 1.f / l : 0.f);
+  // keep the product a rounded fp32 value in both users: left alone, the compiler fuses it with a following
+  // conversion to fp16 into one mixed-precision instruction with a single rounding where it can, and not elsewhere
+  asm volatile("" : "+v"(r));
+  return r;
+}
+
 template <int G, bool BF>  // G = q heads per kv head (<= 16); BF = bf16 instead of fp16 operands and output
 __global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
     const half_t* __restrict__ Q, const half_t* __restrict__ Kc, const half_t* __restrict__ Vc,
     const int* __restrict__ block_table, const int* __restrict__ seq_lens, float* __restrict__ part_acc,
-    float* __restrict__ part_ml, half_t* __restrict__ out, int num_kv_heads, int max_pages_per_seq, int num_splits,
-    float scale_log2e, int window, int page_shift, int num_pages) {
+    float* __restrict__ part_ml, half_t* __restrict__ out, half_t* __restrict__ final_out, int num_kv_heads, int max_pages_per_seq, int num_splits,
+    float scale_log2e, int window, int page_shift, int num_pages, int* __restrict__ arrivals) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -248,12 +280,38 @@ __global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
       out[((size_t)seq * num_q_heads + qh) * 128 + d] = cvt16<BF>(l > 0.f ? acc / l : 0.f);
     } else {
       const size_t pidx = ((size_t)seq * num_q_heads + qh) * num_splits + split;
-      part_acc[pidx * 128 + d] = acc;
+      // device-scope stores: written through to where every XCD sees them, so the merging workgroup needs no
+      // cache-wide write-back or invalidate (one of those per workgroup cost 3x the kernel's time)
+      __hip_atomic_store(part_acc + pidx * 128 + d, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if (d == 0) {
-        part_ml[pidx * 2] = m_tot * scale_log2e;
-        part_ml[pidx * 2 + 1] = l;
+        __hip_atomic_store(part_ml + pidx * 2, m_tot * scale_log2e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(part_ml + pidx * 2 + 1, l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
+  }
+  if (out || !arrivals) return;
+
+  // ---- merge of the splits by whichever workgroup of this (sequence, kv head) finishes last ----
+  // Every workgroup waits until its partials (device-scope stores) are written, then counts itself in with a
+  // device-scope atomic; the one that finds all the others counted merges them (what paged_decode_phase1 does in
+  // a launch of its own) and puts the counter back to zero, so the array is all zero again when the kernel ends.
+  // Partials of other workgroups are read with device-scope loads, past this XCD's L2.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  int* flag = reinterpret_cast<int*>(lds);
+  if (threadIdx.x == 0) {
+    int* ctr = arrivals + (size_t)seq * num_kv_heads + kvh;
+    const int before = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const int last = before == num_splits - 1;
+    if (last) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *flag = last;
+  }
+  __syncthreads();
+  if (!*flag) return;
+  for (int idx = threadIdx.x; idx < G * 128; idx += PD_WAVES * 64) {
+    const int hd = idx >> 7, d = idx & 127;
+    const size_t row = (size_t)seq * num_q_heads + kvh * G + hd;
+    final_out[row * 128 + d] = cvt16<BF>(merge_splits<true>(part_acc, part_ml, row, d, num_splits));
   }
 }
 
@@ -264,24 +322,43 @@ __global__ __launch_bounds__(64) void paged_decode_phase1(const float* __restric
                                                           int num_splits) {
   const size_t row = blockIdx.x;
   const int lane = threadIdx.x;
-  const float* ml = part_ml + row * num_splits * 2;
-  float m_tot = -INFINITY;
-  for (int s = 0; s < num_splits; s++) m_tot = fmaxf(m_tot, ml[2 * s]);
-  floatx2 acc = {0.f, 0.f};
-  float l = 0.f;
-  if (m_tot > -INFINITY) {
-    for (int s = 0; s < num_splits; s++) {
-      const float ms = ml[2 * s];
-      if (ms > -INFINITY) {
-        const float w = fast_exp2(ms - m_tot);
-        const floatx2 a = *reinterpret_cast<const floatx2*>(part_acc + (row * num_splits + s) * 128 + 2 * lane);
-        acc += w * a;
-        l += w * ml[2 * s + 1];
+  half2v o;
+  if (num_splits <= 8) {
+    // the usual case: every load of the row is issued before the first is used (one memory round trip instead of
+    // one per split); the arithmetic is merge_splits' own, operation for operation
+    const float* ml = part_ml + row * num_splits * 2;
+    float m[8], ls[8];
+    floatx2 a[8];
+#pragma unroll
+    for (int s = 0; s < 8; s++) {
+      const bool on = s < num_splits;
+      m[s] = on ? ml[2 * s] : -INFINITY;
+      ls[s] = on ? ml[2 * s + 1] : 0.f;
+      a[s] = on ? *reinterpret_cast<const floatx2*>(part_acc + (row * num_splits + s) * 128 + 2 * lane) : floatx2{0.f, 0.f};
+    }
+    float m_tot = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < 8; s++) m_tot = fmaxf(m_tot, m[s]);
+    float acc0 = 0.f, acc1 = 0.f, l = 0.f;
+    if (m_tot > -INFINITY) {
+#pragma unroll
+      for (int s = 0; s < 8; s++) {
+        if (m[s] > -INFINITY) {
+          const float w = fast_exp2(m[s] - m_tot);
+          acc0 = __builtin_fmaf(w, a[s][0], acc0);
+          acc1 = __builtin_fmaf(w, a[s][1], acc1);
+          l = __builtin_fmaf(w, ls[s], l);
+        }
       }
     }
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    float r0 = acc0 * inv, r1 = acc1 * inv;
+    asm volatile("" : "+v"(r0), "+v"(r1));  // rounded fp32 products, as in merge_splits
+    o = half2v{cvt16<BF>(r0), cvt16<BF>(r1)};
+  } else {
+    o = half2v{cvt16<BF>(merge_splits<false>(part_acc, part_ml, row, 2 * lane, num_splits)),
+               cvt16<BF>(merge_splits<false>(part_acc, part_ml, row, 2 * lane + 1, num_splits))};
   }
-  const float inv = l > 0.f ? 1.f / l : 0.f;
-  half2v o = {cvt16<BF>(acc[0] * inv), cvt16<BF>(acc[1] * inv)};
   *reinterpret_cast<half2v*>(out + row * 128 + 2 * lane) = o;
 }
 
@@ -291,8 +368,8 @@ const char* decode_variant_name(int i) { return i == 0 ? kDecodeVariants[0] : nu
 
 template <int G, bool BF>
 static int launch_phase0(const void* q, const void* kc, const void* vc, const int32_t* bt, const int32_t* sl, float* pacc,
-                         float* pml, void* out, int num_seqs, int num_kv_heads, int max_pages, int num_splits, float scale,
-                         int window, int page_shift, int num_pages, hipStream_t stream) {
+                         float* pml, void* out, void* final_out, int32_t* arrivals, int num_seqs, int num_kv_heads, int max_pages,
+                         int num_splits, float scale, int window, int page_shift, int num_pages, hipStream_t stream) {
   auto kern = paged_decode_phase0<G, BF>;
   constexpr int lds_bytes = PD_WAVES * PD_WAVE_LDS;
   static_assert(lds_bytes >= (int)((2 * PD_WAVES * 16 + PD_WAVES * G * 128) * sizeof(float)), "merge area must fit");
@@ -300,7 +377,8 @@ static int launch_phase0(const void* q, const void* kc, const void* vc, const in
   if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "paged_decode_phase0")) return rc;
   dim3 grid(num_splits, num_kv_heads, num_seqs), block(PD_WAVES * 64);
   hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)q, (const half_t*)kc, (const half_t*)vc, bt, sl,
-                     pacc, pml, (half_t*)out, num_kv_heads, max_pages, num_splits, scale * 1.4426950408889634f, window, page_shift, num_pages);
+                     pacc, pml, (half_t*)out, (half_t*)final_out, num_kv_heads, max_pages, num_splits, scale * 1.4426950408889634f, window,
+                     page_shift, num_pages, arrivals);
   return check_launch("paged_decode_phase0", grid, block, lds_bytes);
 }
 
@@ -332,11 +410,12 @@ static int check_decode_args(const char* fn, int64_t num_seqs, int64_t hq, int64
 
 template <bool BF>
 static int run_phase0(const void* q, const void* kc, const void* vc, const int32_t* bt, const int32_t* sl, float* pacc,
-                      float* pml, void* out, int64_t num_seqs, int64_t hq, int64_t hkv, int64_t max_pages,
+                      float* pml, void* out, void* final_out, int32_t* arrivals, int64_t num_seqs, int64_t hq, int64_t hkv,
+                      int64_t max_pages,
                       int64_t num_splits, float scale, int window, int page_shift, int64_t num_pages, hipStream_t stream) {
   const int G = (int)(hq / hkv);
 #define MI355_PD_CASE(GG) \
-  case GG: return launch_phase0<GG, BF>(q, kc, vc, bt, sl, pacc, pml, out, (int)num_seqs, (int)hkv, (int)max_pages, (int)num_splits, scale, window, page_shift, (int)num_pages, stream)
+  case GG: return launch_phase0<GG, BF>(q, kc, vc, bt, sl, pacc, pml, out, final_out, arrivals, (int)num_seqs, (int)hkv, (int)max_pages, (int)num_splits, scale, window, page_shift, (int)num_pages, stream)
   switch (G) {
     MI355_PD_CASE(1);
     MI355_PD_CASE(2);
@@ -364,8 +443,8 @@ static int phase0_entry(const void* q, const void* k_cache, const void* v_cache,
   if (!part_acc || !part_ml) return fail(-MI355_E_SCRATCH, "paged_decode_phase0: part_acc / part_ml scratch is required");
   if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || !aligned16(part_acc))
     return fail(-MI355_E_ALIGN, "paged_decode_phase0: q, k_cache, v_cache, part_acc must be 16-byte aligned");
-  return run_phase0<BF>(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, nullptr, num_seqs, num_q_heads,
-                           num_kv_heads, max_pages_per_seq, num_splits, scale, 0, page_shift_of(page_size), num_pages,
+  return run_phase0<BF>(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, nullptr, nullptr, nullptr, num_seqs,
+                        num_q_heads, num_kv_heads, max_pages_per_seq, num_splits, scale, 0, page_shift_of(page_size), num_pages,
                            reinterpret_cast<hipStream_t>(stream));
 }
 
@@ -412,7 +491,7 @@ extern "C" int mi355_paged_decode_phase1_bf16(const float* part_acc, const float
 
 template <bool BF>
 static int decode_attn(const char* fn, const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
-                       const int32_t* seq_lens, void* out, float* part_acc, float* part_ml, int64_t num_seqs,
+                       const int32_t* seq_lens, void* out, float* part_acc, float* part_ml, int32_t* arrivals, int64_t num_seqs,
                        int64_t num_q_heads, int64_t num_kv_heads, int64_t D, int64_t page_size, int64_t max_pages_per_seq,
                        int64_t num_pages, int64_t num_splits, float scale, int64_t window, void* stream) {
   if (!q || !k_cache || !v_cache || !block_table || !seq_lens || !out) return fail(-MI355_E_NULL, "%s: null pointer", fn);
@@ -424,14 +503,42 @@ static int decode_attn(const char* fn, const void* q, const void* k_cache, const
     return fail(-MI355_E_ALIGN, "%s: q, k_cache, v_cache, out must be 16-byte aligned", fn);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (num_splits == 1)
-    return run_phase0<BF>(q, k_cache, v_cache, block_table, seq_lens, nullptr, nullptr, out, num_seqs, num_q_heads, num_kv_heads,
-                          max_pages_per_seq, 1, scale, (int)window, page_shift_of(page_size), num_pages, s);
+    return run_phase0<BF>(q, k_cache, v_cache, block_table, seq_lens, nullptr, nullptr, out, nullptr, nullptr, num_seqs, num_q_heads,
+                          num_kv_heads, max_pages_per_seq, 1, scale, (int)window, page_shift_of(page_size), num_pages, s);
   if (!part_acc || !part_ml) return fail(-MI355_E_SCRATCH, "%s: num_splits > 1 needs part_acc / part_ml scratch", fn);
   if (!aligned16(part_acc)) return fail(-MI355_E_ALIGN, "%s: part_acc must be 16-byte aligned", fn);
-  if (int rc = run_phase0<BF>(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, nullptr, num_seqs, num_q_heads,
-                              num_kv_heads, max_pages_per_seq, num_splits, scale, (int)window, page_shift_of(page_size), num_pages, s))
+  // One launch, the last workgroup of every (sequence, kv head) merging, pays a store acknowledgement and an atomic
+  // round trip (about 3 us) at the end of EVERY workgroup, during which its LDS keeps the next workgroup off the CU.
+  // With all workgroups resident at once (two per CU) that wait is hidden behind nothing and still costs less than
+  // a second launch (1 sequence x 32768 tokens: one launch is ahead); with several rounds of workgroups it adds up
+  // to more than the merge kernel's 5 us (the 64-sequence benchmark batch: 216 us against 211), so those grids keep
+  // the two launches.
+  const bool one_launch = arrivals && num_splits * num_kv_heads * num_seqs <= 2 * 256;
+  if (one_launch)
+    return run_phase0<BF>(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, nullptr, out, arrivals, num_seqs,
+                          num_q_heads, num_kv_heads, max_pages_per_seq, num_splits, scale, (int)window, page_shift_of(page_size),
+                          num_pages, s);
+  if (int rc = run_phase0<BF>(q, k_cache, v_cache, block_table, seq_lens, part_acc, part_ml, nullptr, nullptr, nullptr, num_seqs,
+                              num_q_heads, num_kv_heads, max_pages_per_seq, num_splits, scale, (int)window,
+                              page_shift_of(page_size), num_pages, s))
     return rc;
   return run_phase1<BF>(part_acc, part_ml, out, num_seqs, num_q_heads, D, num_splits, stream);
+}
+
+extern "C" int mi355_paged_decode_attn_fused(const void* q, const void* k_cache, const void* v_cache,
+                                             const int32_t* block_table, const int32_t* seq_lens, void* out, float* part_acc,
+                                             float* part_ml, int32_t* arrivals, int64_t num_seqs, int64_t num_q_heads,
+                                             int64_t num_kv_heads, int64_t D, int64_t page_size, int64_t max_pages_per_seq,
+                                             int64_t num_pages, int64_t num_splits, float scale, int64_t window, int dtype,
+                                             void* stream) {
+  const char* fn = "paged_decode_attn_fused";
+  if (dtype != MI355_F16 && dtype != MI355_BF16) return fail(-MI355_E_DTYPE, "%s: dtype %d (MI355_F16 or MI355_BF16)", fn, dtype);
+  if (num_splits > 1 && !arrivals) return fail(-MI355_E_SCRATCH, "%s: num_splits > 1 needs the arrivals counters", fn);
+  if (dtype == MI355_BF16)
+    return decode_attn<true>(fn, q, k_cache, v_cache, block_table, seq_lens, out, part_acc, part_ml, arrivals, num_seqs, num_q_heads,
+                             num_kv_heads, D, page_size, max_pages_per_seq, num_pages, num_splits, scale, window, stream);
+  return decode_attn<false>(fn, q, k_cache, v_cache, block_table, seq_lens, out, part_acc, part_ml, arrivals, num_seqs, num_q_heads,
+                            num_kv_heads, D, page_size, max_pages_per_seq, num_pages, num_splits, scale, window, stream);
 }
 
 extern "C" int mi355_paged_decode_attn(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
@@ -439,7 +546,7 @@ extern "C" int mi355_paged_decode_attn(const void* q, const void* k_cache, const
                                        int64_t num_q_heads, int64_t num_kv_heads, int64_t D, int64_t page_size,
                                        int64_t max_pages_per_seq, int64_t num_pages, int64_t num_splits, float scale,
                                        void* stream) {
-  return decode_attn<false>("paged_decode_attn", q, k_cache, v_cache, block_table, seq_lens, out, part_acc, part_ml, num_seqs,
+  return decode_attn<false>("paged_decode_attn", q, k_cache, v_cache, block_table, seq_lens, out, part_acc, part_ml, nullptr, num_seqs,
                      num_q_heads, num_kv_heads, D, page_size, max_pages_per_seq, num_pages, num_splits, scale, 0, stream);
 }
 
@@ -448,7 +555,7 @@ extern "C" int mi355_paged_decode_attn_window(const void* q, const void* k_cache
                                               float* part_ml, int64_t num_seqs, int64_t num_q_heads, int64_t num_kv_heads,
                                               int64_t D, int64_t page_size, int64_t max_pages_per_seq, int64_t num_pages,
                                               int64_t num_splits, float scale, int64_t window, void* stream) {
-  return decode_attn<false>("paged_decode_attn_window", q, k_cache, v_cache, block_table, seq_lens, out, part_acc, part_ml,
+  return decode_attn<false>("paged_decode_attn_window", q, k_cache, v_cache, block_table, seq_lens, out, part_acc, part_ml, nullptr,
                             num_seqs, num_q_heads, num_kv_heads, D, page_size, max_pages_per_seq, num_pages, num_splits, scale,
                             window, stream);
 }
@@ -459,7 +566,7 @@ extern "C" int mi355_paged_decode_attn_window_bf16(const void* q, const void* k_
                                                    int64_t num_kv_heads, int64_t D, int64_t page_size,
                                                    int64_t max_pages_per_seq, int64_t num_pages, int64_t num_splits,
                                                    float scale, int64_t window, void* stream) {
-  return decode_attn<true>("paged_decode_attn_window_bf16", q, k_cache, v_cache, block_table, seq_lens, out, part_acc, part_ml,
+  return decode_attn<true>("paged_decode_attn_window_bf16", q, k_cache, v_cache, block_table, seq_lens, out, part_acc, part_ml, nullptr,
                            num_seqs, num_q_heads, num_kv_heads, D, page_size, max_pages_per_seq, num_pages, num_splits, scale,
                            window, stream);
 }
@@ -501,7 +608,7 @@ extern "C" int mi355_paged_decode_attn_static(const void* q, const void* k_cache
                                               int64_t num_splits, float scale, void* stream) {
   const char* fn = "paged_decode_attn_static";
   if (num_splits <= 1)  // a single split needs no partials at all
-    return decode_attn<false>(fn, q, k_cache, v_cache, block_table, seq_lens, out, nullptr, nullptr, num_seqs, num_q_heads,
+    return decode_attn<false>(fn, q, k_cache, v_cache, block_table, seq_lens, out, nullptr, nullptr, nullptr, num_seqs, num_q_heads,
                               num_kv_heads, D, page_size, max_pages_per_seq, num_pages, num_splits, scale, 0, stream);
   if (num_seqs <= 0 || num_q_heads <= 0 || num_seqs > PD_STATIC_MAX_ROWS || num_q_heads > PD_STATIC_MAX_ROWS ||
       num_splits > PD_STATIC_MAX_ROWS || num_seqs * num_q_heads * num_splits > PD_STATIC_MAX_ROWS)
@@ -514,7 +621,7 @@ extern "C" int mi355_paged_decode_attn_static(const void* q, const void* k_cache
   // nothing of the previous call's contents is read and nothing needs clearing.
   float* part_acc = base;
   float* part_ml = base + num_seqs * num_q_heads * num_splits * 128;
-  return decode_attn<false>(fn, q, k_cache, v_cache, block_table, seq_lens, out, part_acc, part_ml, num_seqs, num_q_heads,
+  return decode_attn<false>(fn, q, k_cache, v_cache, block_table, seq_lens, out, part_acc, part_ml, nullptr, num_seqs, num_q_heads,
                             num_kv_heads, D, page_size, max_pages_per_seq, num_pages, num_splits, scale, 0, stream);
 }
 

@@ -173,10 +173,26 @@ def paged_decode_phase1_out(part_acc: Tensor, part_ml: Tensor, out: Tensor) -> T
     return out
 
 
+_ARRIVALS: dict[tuple[int, int], Tensor] = {}  # (device index, stream) -> zeroed int32 counters, grown on demand
+
+
+def _arrival_counters(dev: torch.device, n: int) -> Tensor:
+    """The per-(sequence, kv head) arrival counters of the one-launch decode.  The kernel needs them zero when it
+    starts and leaves them zero, so one buffer per stream, zeroed when it is created, serves every call on that
+    stream (launches on one stream are ordered; two streams never share a buffer)."""
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(dev).cuda_stream)
+    buf = _ARRIVALS.get(key)
+    if buf is None or buf.numel() < n:
+        buf = torch.zeros(max(n, 4096), dtype=torch.int32, device=dev)
+        _ARRIVALS[key] = buf
+    return buf
+
+
 def paged_decode_attn_out(q, k_cache, v_cache, block_table, seq_lens, out, scale: float, num_kv_splits: int,
                           part_acc: Tensor | None = None, part_ml: Tensor | None = None, window: int = 0) -> Tensor:
     contract.check_paged_args("paged_decode_attn", q, k_cache, v_cache, block_table, seq_lens, bf16_ok=True)
     contract.require(1 <= num_kv_splits <= 1024, f"paged_decode_attn: num_kv_splits must be in [1, 1024], got {num_kv_splits}")
+    contract.require(window >= 0, f"paged_decode_attn: window must be >= 0, got {window}")
     if num_kv_splits > 1 and part_acc is not None and part_ml is not None:  # caller-owned scratch
         contract.check_decode_partials("paged_decode_attn", part_acc, part_ml, q.shape[0], q.shape[1], num_kv_splits)
     dev = _dev(q, k_cache, v_cache, block_table, seq_lens, out)
@@ -201,23 +217,12 @@ def paged_decode_attn_out(q, k_cache, v_cache, block_table, seq_lens, out, scale
         _contig_out(part_ml, "paged_decode_attn")
     pa = part_acc.data_ptr() if num_kv_splits > 1 else None
     pm = part_ml.data_ptr() if num_kv_splits > 1 else None
-    if window < 0:
-        raise ValueError(f"paged_decode_attn: window must be >= 0, got {window}")
+    arrivals = _arrival_counters(dev, S * Hkv).data_ptr() if num_kv_splits > 1 else None
     with torch.cuda.device(dev):
-        if dt == torch.bfloat16:
-            rc = _lib.load().mi355_paged_decode_attn_window_bf16(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
-                                                                 block_table.data_ptr(), seq_lens.data_ptr(), out.data_ptr(), pa,
-                                                                 pm, S, Hq, Hkv, D, page, block_table.shape[1], P, num_kv_splits,
-                                                                 scale, window, _lib.current_stream_ptr(dev))
-        elif window == 0:
-            rc = _lib.load().mi355_paged_decode_attn(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
-                                                     seq_lens.data_ptr(), out.data_ptr(), pa, pm, S, Hq, Hkv, D, page,
-                                                     block_table.shape[1], P, num_kv_splits, scale, _lib.current_stream_ptr(dev))
-        else:
-            rc = _lib.load().mi355_paged_decode_attn_window(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
-                                                            block_table.data_ptr(), seq_lens.data_ptr(), out.data_ptr(), pa, pm, S,
-                                                            Hq, Hkv, D, page, block_table.shape[1], P, num_kv_splits, scale, window,
-                                                            _lib.current_stream_ptr(dev))
+        rc = _lib.load().mi355_paged_decode_attn_fused(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
+                                                       seq_lens.data_ptr(), out.data_ptr(), pa, pm, arrivals, S, Hq, Hkv, D, page,
+                                                       block_table.shape[1], P, num_kv_splits, scale, window, _lib.dtype_code(dt),
+                                                       _lib.current_stream_ptr(dev))
     _lib.check(rc, f"paged_decode_attn {dt} seqs={S} hq={Hq} hkv={Hkv} pages={P} splits={num_kv_splits} window={window}")
     return out
 

@@ -156,6 +156,42 @@ def test_decode_invariances(dev):
     assert torch.equal(two, base)
 
 
+def test_decode_one_launch_merge_equals_two_phase(dev):
+    """The op merges the kv splits inside the phase-0 kernel (the last workgroup of a (sequence, kv head) to finish
+    does it); the C entry with caller scratch runs phase 0 and phase 1 as two launches.  Same arithmetic: bit-equal,
+    over calls in a row with different split counts, batch shapes and dtypes (the arrival counters must come back
+    to zero every time), with a window, and for the full benchmark batch."""
+    import iree_turbine_amd  # noqa: F401
+    from iree_turbine_amd import _lib, launch
+    from oracle import inputs
+
+    lib = _lib.load()
+
+    def two_phase(q, kc, vc, bt, sl, splits):
+        S, Hq, D = q.shape
+        P, page, Hkv, _ = kc.shape
+        out = torch.empty_like(q)
+        pacc = torch.empty((S, Hq, splits, D), dtype=torch.float32, device=dev)
+        pml = torch.empty((S, Hq, splits, 2), dtype=torch.float32, device=dev)
+        entry = lib.mi355_paged_decode_attn_window_bf16 if q.dtype == torch.bfloat16 else lib.mi355_paged_decode_attn_window
+        rc = entry(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), bt.data_ptr(), sl.data_ptr(), out.data_ptr(), pacc.data_ptr(),
+                   pml.data_ptr(), S, Hq, Hkv, D, page, bt.shape[1], P, splits, 128 ** -0.5, 0, _lib.current_stream_ptr(dev))
+        _lib.check(rc, "two-phase decode")
+        return out
+
+    cases = [(dict(num_seqs=7, min_len=1, max_len=900, seed=41), 4, False), (dict(num_seqs=3, min_len=300, max_len=2000, seed=42), 9, False),
+             (dict(num_seqs=7, min_len=1, max_len=900, seed=43), 2, True), (dict(), 3, False), (dict(num_seqs=2, min_len=50, max_len=60, seed=44), 16, False)]
+    for kw, splits, bf in cases:
+        announce(f"decode one-launch merge {kw} splits={splits} bf16={bf}")
+        q, kc, vc, bt, sl = _to(dev, *inputs.paged_decode_inputs(**kw))
+        if bf:
+            q, kc, vc = q.bfloat16(), kc.bfloat16(), vc.bfloat16()
+        got = torch.ops.mi355.paged_decode_attn(q, kc, vc, bt, sl, 0.0, splits)
+        assert torch.equal(got, two_phase(q, kc, vc, bt, sl, splits))
+    torch.cuda.synchronize()
+    assert launch._ARRIVALS and all(int(buf.abs().sum()) == 0 for buf in launch._ARRIVALS.values())
+
+
 def test_decode_full_size(dev):
     """The benchmark configuration (64 seqs, 32/8 heads, ctx in [512, 8192]) against the oracle."""
     import iree_turbine_amd  # noqa: F401
