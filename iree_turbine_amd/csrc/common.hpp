@@ -44,6 +44,14 @@ __device__ __forceinline__ void buffer_load_lds_16B(buffer_rsrc_t rsrc, unsigned
   __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, MI355_LDS(void, lds_wave_base), 16, (int)voffset, (int)soffset, 0, 0);
 }
 
+// The lane id (0..63) recomputed on the spot, opaque to the compiler: what is derived from it is neither hoisted out
+// of a loop nor kept in a register across code that has none to spare.
+__device__ __forceinline__ int opaque_lane_id() {
+  int l;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+  return l;
+}
+
 __device__ __forceinline__ void wait_vmcnt0() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // D(32x32) += A(32x16) * B(16x32).  Lane l supplies A[l%32][8*(l/32) .. +7] and

@@ -394,11 +394,16 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_staged(const half_t* 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm = wave / WN, wn = wave % WN;
+  // The workgroup walks tiles blockIdx.x, blockIdx.x + gridDim.x, ... as ONE slab sequence: launched with one
+  // workgroup per tile it is the plain kernel; launched with one workgroup per CU, the loads of a tile's last
+  // three slabs fetch the next tile's first three, so only the first tile of a workgroup pays the pipeline fill,
+  // and a tile's stores drain under the next tile's MFMAs.
+  const int T = tiles_m * tiles_n;
+  int pid = blockIdx.x;
   int tile_m, tile_n;
-  map_tile(blockIdx.x, tiles_m, tiles_n, group_m, tile_m, tile_n);
+  map_tile(pid, tiles_m, tiles_n, group_m, tile_m, tile_n);
 
   // global side: wave-load i covers rows (i * NW + wave) * 8 .. + 7 of the tile, 8 lanes per 128-byte row piece
-  const int lrow = lane >> 3, lc = lane & 7;
   const unsigned row_bytes = (unsigned)K * 2u;
   // buffer descriptors by hand: base, stride 0, size, raw dword format
   auto make_desc = [&](const half_t* base, unsigned bytes) {
@@ -410,21 +415,36 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_staged(const half_t* 
     d[3] = 0x00020000;
     return d;
   };
-  const i32x4 a_src = make_desc(A + (size_t)(tile_m * BM + wave * 8) * K, (unsigned)(BM - wave * 8) * row_bytes);
-  const i32x4 b_src = make_desc(B + (size_t)(tile_n * BN + wave * 8) * K, (unsigned)(BN - wave * 8) * row_bytes);
-  const unsigned g_off = (unsigned)lrow * row_bytes + (unsigned)lc * 16u;
+  i32x4 a_src = make_desc(A + (size_t)(tile_m * BM + wave * 8) * K, (unsigned)(BM - wave * 8) * row_bytes);
+  i32x4 b_src = make_desc(B + (size_t)(tile_n * BN + wave * 8) * K, (unsigned)(BN - wave * 8) * row_bytes);
+  i32x4 a_nxt = a_src, b_nxt = b_src;  // the tile after this one (the last tile: itself; those loads are never used)
   const unsigned row_step = (unsigned)NW * 8u * row_bytes;
-  // LDS side: row r = (i * NW + wave) * 8 + lrow, chunk lc in slot lc ^ ((r >> 1) & 7); NW is even, so the
-  // swizzle term does not depend on i
-  const int w_off = wave * 1024 + lrow * 128 + ((lc ^ (((wave & 1) << 2) | (lrow >> 1))) * 16);
+  // Per-lane offsets of the K loop.  They are set at the start of every tile from a lane id the compiler cannot see
+  // through: as plain loop invariants they would stay live across the epilogue, which has no registers to spare
+  // beside the staging sets, and would be spilled to scratch around it.
+  unsigned g_off;
+  int w_off, a_base, b_base;
+  auto lane_offsets = [&]() {
+    const int lk = opaque_lane_id();
+    const int lrow = lk >> 3, lc = lk & 7;
+    g_off = (unsigned)lrow * row_bytes + (unsigned)lc * 16u;
+    // LDS side of the staging writes: row r = (i * NW + wave) * 8 + lrow, chunk lc in slot lc ^ ((r >> 1) & 7); NW is
+    // even, so the swizzle term does not depend on i
+    w_off = wave * 1024 + lrow * 128 + ((lc ^ (((wave & 1) << 2) | (lrow >> 1))) * 16);
+    const int r32k = lk & 31, hk = lk >> 5;
+    const int sw = (hk ^ ((r32k >> 1) & 7)) * 16;
+    a_base = (wm * WTM + r32k) * 128 + sw;
+    b_base = A_BYTES + (wn * WTN + r32k) * 128 + sw;
+  };
+  lane_offsets();
 
   // staging registers: r[set][n], n < 8 the A row groups, n >= 8 the B row groups
   u32x4 r[2][16];
   // (macros: inline assembly inside a generic lambda cannot name the enclosing function's arrays)
-#define MI355_ST_LOAD(S, n, k_off_)                                                                  \
+#define MI355_ST_LOAD(S, n, k_off_, da_, db_)                                                        \
   asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"                                            \
                : "=v"(r[S][n])                                                                       \
-               : "v"(g_off), "s"((n) < 8 ? a_src : b_src), "s"((k_off_) + (unsigned)((n)&7) * row_step) \
+               : "v"(g_off), "s"((n) < 8 ? da_ : db_), "s"((k_off_) + (unsigned)((n)&7) * row_step)   \
                : "memory")
   // `newer` = loads issued after the one that filled r[S][n]; they may still be in flight
 #define MI355_ST_WRITE(S, n, newer, st_)                                                                                   \
@@ -433,10 +453,6 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_staged(const half_t* 
     *reinterpret_cast<u32x4*>((st_) + w_off + ((n) < 8 ? (n)*NW * 1024 : A_BYTES + ((n)-8) * NW * 1024)) = r[S][n];        \
   } while (0)
 
-  const int r32 = lane & 31, h = lane >> 5;
-  const int sw = (h ^ ((r32 >> 1) & 7)) * 16;
-  const int a_base = (wm * WTM + r32) * 128 + sw;
-  const int b_base = A_BYTES + (wn * WTN + r32) * 128 + sw;
   auto read_frags = [&](const char* st, int ks, half8* fm, half8* fn) {
 #pragma unroll
     for (int j = 0; j < TM; j++) fm[j] = *reinterpret_cast<const half8*>(st + ((a_base ^ (ks * 32)) + j * 4096));
@@ -459,10 +475,12 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_staged(const half_t* 
 #define MI355_ST_LOAD_ALL(S, slab_)                                       \
   do {                                                                    \
     const unsigned ko_ = (unsigned)(slab_)*128u;                          \
-    MI355_ST_LOAD(S, 0, ko_); MI355_ST_LOAD(S, 1, ko_); MI355_ST_LOAD(S, 2, ko_); MI355_ST_LOAD(S, 3, ko_);     \
-    MI355_ST_LOAD(S, 4, ko_); MI355_ST_LOAD(S, 5, ko_); MI355_ST_LOAD(S, 6, ko_); MI355_ST_LOAD(S, 7, ko_);     \
-    MI355_ST_LOAD(S, 8, ko_); MI355_ST_LOAD(S, 9, ko_); MI355_ST_LOAD(S, 10, ko_); MI355_ST_LOAD(S, 11, ko_);   \
-    MI355_ST_LOAD(S, 12, ko_); MI355_ST_LOAD(S, 13, ko_); MI355_ST_LOAD(S, 14, ko_); MI355_ST_LOAD(S, 15, ko_); \
+    MI355_ST_LOAD(S, 0, ko_, a_src, b_src); MI355_ST_LOAD(S, 1, ko_, a_src, b_src); MI355_ST_LOAD(S, 2, ko_, a_src, b_src);     \
+    MI355_ST_LOAD(S, 3, ko_, a_src, b_src); MI355_ST_LOAD(S, 4, ko_, a_src, b_src); MI355_ST_LOAD(S, 5, ko_, a_src, b_src);     \
+    MI355_ST_LOAD(S, 6, ko_, a_src, b_src); MI355_ST_LOAD(S, 7, ko_, a_src, b_src); MI355_ST_LOAD(S, 8, ko_, a_src, b_src);     \
+    MI355_ST_LOAD(S, 9, ko_, a_src, b_src); MI355_ST_LOAD(S, 10, ko_, a_src, b_src); MI355_ST_LOAD(S, 11, ko_, a_src, b_src);   \
+    MI355_ST_LOAD(S, 12, ko_, a_src, b_src); MI355_ST_LOAD(S, 13, ko_, a_src, b_src); MI355_ST_LOAD(S, 14, ko_, a_src, b_src);  \
+    MI355_ST_LOAD(S, 15, ko_, a_src, b_src);                                                                                    \
   } while (0)
   MI355_ST_LOAD_ALL(0, 0);
   MI355_ST_LOAD_ALL(1, 1);
@@ -471,7 +489,9 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_staged(const half_t* 
   MI355_ST_WRITE(0, 8, 16, lds); MI355_ST_WRITE(0, 9, 16, lds); MI355_ST_WRITE(0, 10, 16, lds); MI355_ST_WRITE(0, 11, 16, lds);
   MI355_ST_WRITE(0, 12, 16, lds); MI355_ST_WRITE(0, 13, 16, lds); MI355_ST_WRITE(0, 14, 16, lds); MI355_ST_WRITE(0, 15, 16, lds);
   MI355_ST_LOAD_ALL(0, 2);
-  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  // every tile starts with all three slabs landed (later tiles: the K loop ends that way), so the first two slabs
+  // of a tile never wait for a load
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
   __syncthreads();
   read_frags(lds, 0, fm0, fn0);
 
@@ -510,40 +530,127 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_staged(const half_t* 
   // register by register, each register reloaded with slab kt+3 once it is written out; set P is receiving
   // slab kt+2.  Loads in flight when register n is written: the rest of its own round (15 - n), the 16 of the
   // other set, and the G loads of this slab issued so far.
-#define MI355_ST_SLAB(P, Q, kt_)                                                                                           \
+  // Past the end of the tile the loads belong to the next tile (branch-free: descriptors and slab index are selected).
+  // W: 0 = exact waits; 1 = none -- used for the first two slabs behind an epilogue, where every staging register has
+  // landed (the K loop ends with vmcnt(0)) and the only operations in flight are the epilogue's stores, which an
+  // exact count would wait for.
+#define MI355_ST_SLAB(P, Q, kt_, W)                                                                                        \
   do {                                                                                                                     \
     const char* st = lds + P * STAGE;                                                                                      \
     char* nst = lds + Q * STAGE;                                                                                           \
-    const int nxt_ = (kt_) + 3 < KT ? (kt_) + 3 : KT - 1; /* past the end: re-fetch, never used */                         \
-    const unsigned ko = (unsigned)nxt_ * 128u;                                                                             \
+    const bool wrap_ = (kt_) + 3 >= KT;                                                                                    \
+    const unsigned ko = (unsigned)(wrap_ ? (kt_) + 3 - KT : (kt_) + 3) * 128u;                                             \
+    const i32x4 la = wrap_ ? a_nxt : a_src, lb = wrap_ ? b_nxt : b_src;                                                    \
     __builtin_amdgcn_sched_barrier(0);                                                                                     \
-    MI355_ST_GROUP(0, fm0, fn0, st, 1, fm1, fn1, MI355_ST_WRITE(Q, 0, 31, nst), MI355_ST_WRITE(Q, 1, 30, nst), MI355_ST_LOAD(Q, 0, ko));   \
-    MI355_ST_GROUP(1, fm0, fn0, st, 1, fm1, fn1, MI355_ST_WRITE(Q, 2, 30, nst), MI355_NOP, MI355_ST_LOAD(Q, 1, ko));                       \
-    MI355_ST_GROUP(2, fm0, fn0, st, 1, fm1, fn1, MI355_ST_WRITE(Q, 3, 30, nst), MI355_ST_WRITE(Q, 4, 29, nst), MI355_ST_LOAD(Q, 2, ko));   \
-    MI355_ST_GROUP(3, fm0, fn0, st, 1, fm1, fn1, MI355_ST_WRITE(Q, 5, 29, nst), MI355_NOP, MI355_ST_LOAD(Q, 3, ko));                       \
-    MI355_ST_GROUP(0, fm1, fn1, st, 2, fm0, fn0, MI355_ST_WRITE(Q, 6, 29, nst), MI355_ST_WRITE(Q, 7, 28, nst), MI355_ST_LOAD(Q, 4, ko));   \
-    MI355_ST_GROUP(1, fm1, fn1, st, 2, fm0, fn0, MI355_ST_WRITE(Q, 8, 28, nst), MI355_NOP, MI355_ST_LOAD(Q, 5, ko));                       \
-    MI355_ST_GROUP(2, fm1, fn1, st, 2, fm0, fn0, MI355_ST_WRITE(Q, 9, 28, nst), MI355_ST_WRITE(Q, 10, 27, nst), MI355_ST_LOAD(Q, 6, ko));  \
-    MI355_ST_GROUP(3, fm1, fn1, st, 2, fm0, fn0, MI355_ST_WRITE(Q, 11, 27, nst), MI355_NOP, MI355_ST_LOAD(Q, 7, ko));                      \
-    MI355_ST_GROUP(0, fm0, fn0, st, 3, fm1, fn1, MI355_ST_WRITE(Q, 12, 27, nst), MI355_NOP, MI355_ST_LOAD(Q, 8, ko));                      \
-    MI355_ST_GROUP(1, fm0, fn0, st, 3, fm1, fn1, MI355_ST_WRITE(Q, 13, 27, nst), MI355_NOP, MI355_ST_LOAD(Q, 9, ko));                      \
-    MI355_ST_GROUP(2, fm0, fn0, st, 3, fm1, fn1, MI355_ST_WRITE(Q, 14, 27, nst), MI355_NOP, MI355_ST_LOAD(Q, 10, ko));                     \
-    MI355_ST_GROUP(3, fm0, fn0, st, 3, fm1, fn1, MI355_ST_WRITE(Q, 15, 27, nst), MI355_NOP, MI355_ST_LOAD(Q, 11, ko));                     \
+    MI355_ST_GROUP(0, fm0, fn0, st, 1, fm1, fn1, MI355_ST_WRITE(Q, 0, (W) ? 63 : 31, nst), MI355_ST_WRITE(Q, 1, (W) ? 63 : 30, nst), MI355_ST_LOAD(Q, 0, ko, la, lb));   \
+    MI355_ST_GROUP(1, fm0, fn0, st, 1, fm1, fn1, MI355_ST_WRITE(Q, 2, (W) ? 63 : 30, nst), MI355_NOP, MI355_ST_LOAD(Q, 1, ko, la, lb));                                  \
+    MI355_ST_GROUP(2, fm0, fn0, st, 1, fm1, fn1, MI355_ST_WRITE(Q, 3, (W) ? 63 : 30, nst), MI355_ST_WRITE(Q, 4, (W) ? 63 : 29, nst), MI355_ST_LOAD(Q, 2, ko, la, lb));   \
+    MI355_ST_GROUP(3, fm0, fn0, st, 1, fm1, fn1, MI355_ST_WRITE(Q, 5, (W) ? 63 : 29, nst), MI355_NOP, MI355_ST_LOAD(Q, 3, ko, la, lb));                                  \
+    MI355_ST_GROUP(0, fm1, fn1, st, 2, fm0, fn0, MI355_ST_WRITE(Q, 6, (W) ? 63 : 29, nst), MI355_ST_WRITE(Q, 7, (W) ? 63 : 28, nst), MI355_ST_LOAD(Q, 4, ko, la, lb));   \
+    MI355_ST_GROUP(1, fm1, fn1, st, 2, fm0, fn0, MI355_ST_WRITE(Q, 8, (W) ? 63 : 28, nst), MI355_NOP, MI355_ST_LOAD(Q, 5, ko, la, lb));                                  \
+    MI355_ST_GROUP(2, fm1, fn1, st, 2, fm0, fn0, MI355_ST_WRITE(Q, 9, (W) ? 63 : 28, nst), MI355_ST_WRITE(Q, 10, (W) ? 63 : 27, nst), MI355_ST_LOAD(Q, 6, ko, la, lb));  \
+    MI355_ST_GROUP(3, fm1, fn1, st, 2, fm0, fn0, MI355_ST_WRITE(Q, 11, (W) ? 63 : 27, nst), MI355_NOP, MI355_ST_LOAD(Q, 7, ko, la, lb));                                 \
+    MI355_ST_GROUP(0, fm0, fn0, st, 3, fm1, fn1, MI355_ST_WRITE(Q, 12, (W) ? 63 : 27, nst), MI355_NOP, MI355_ST_LOAD(Q, 8, ko, la, lb));                                 \
+    MI355_ST_GROUP(1, fm0, fn0, st, 3, fm1, fn1, MI355_ST_WRITE(Q, 13, (W) ? 63 : 27, nst), MI355_NOP, MI355_ST_LOAD(Q, 9, ko, la, lb));                                 \
+    MI355_ST_GROUP(2, fm0, fn0, st, 3, fm1, fn1, MI355_ST_WRITE(Q, 14, (W) ? 63 : 27, nst), MI355_NOP, MI355_ST_LOAD(Q, 10, ko, la, lb));                                \
+    MI355_ST_GROUP(3, fm0, fn0, st, 3, fm1, fn1, MI355_ST_WRITE(Q, 15, (W) ? 63 : 27, nst), MI355_NOP, MI355_ST_LOAD(Q, 11, ko, la, lb));                                \
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                                                     \
     __syncthreads();                                                                                                       \
     __builtin_amdgcn_sched_barrier(0);                                                                                     \
-    MI355_ST_GROUP(0, fm1, fn1, nst, 0, fm0, fn0, MI355_NOP, MI355_NOP, MI355_ST_LOAD(Q, 12, ko));                         \
-    MI355_ST_GROUP(1, fm1, fn1, nst, 0, fm0, fn0, MI355_NOP, MI355_NOP, MI355_ST_LOAD(Q, 13, ko));                         \
-    MI355_ST_GROUP(2, fm1, fn1, nst, 0, fm0, fn0, MI355_NOP, MI355_NOP, MI355_ST_LOAD(Q, 14, ko));                         \
-    MI355_ST_GROUP(3, fm1, fn1, nst, 0, fm0, fn0, MI355_NOP, MI355_NOP, MI355_ST_LOAD(Q, 15, ko));                         \
+    MI355_ST_GROUP(0, fm1, fn1, nst, 0, fm0, fn0, MI355_NOP, MI355_NOP, MI355_ST_LOAD(Q, 12, ko, la, lb));                 \
+    MI355_ST_GROUP(1, fm1, fn1, nst, 0, fm0, fn0, MI355_NOP, MI355_NOP, MI355_ST_LOAD(Q, 13, ko, la, lb));                 \
+    MI355_ST_GROUP(2, fm1, fn1, nst, 0, fm0, fn0, MI355_NOP, MI355_NOP, MI355_ST_LOAD(Q, 14, ko, la, lb));                 \
+    MI355_ST_GROUP(3, fm1, fn1, nst, 0, fm0, fn0, MI355_NOP, MI355_NOP, MI355_ST_LOAD(Q, 15, ko, la, lb));                 \
   } while (0)
 
-  for (int kt = 0; kt < KT; kt += 2) {
-    MI355_ST_SLAB(0, 1, kt);
-    MI355_ST_SLAB(1, 0, kt + 1);
-    // The loads of the last slabs fetch nothing that is used, and behind the loop the compiler hands their
-    // registers to the epilogue: let them land while the registers still belong to them.
-    if (kt + 2 >= KT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  const int G = (int)gridDim.x;
+  for (; pid < T; pid += G) {
+    int nxt_m = tile_m, nxt_n = tile_n;
+    if (pid + G < T) {
+      map_tile(pid + G, tiles_m, tiles_n, group_m, nxt_m, nxt_n);
+      a_nxt = make_desc(A + (size_t)(nxt_m * BM + wave * 8) * K, (unsigned)(BM - wave * 8) * row_bytes);
+      b_nxt = make_desc(B + (size_t)(nxt_n * BN + wave * 8) * K, (unsigned)(BN - wave * 8) * row_bytes);
+    }
+    MI355_ST_SLAB(0, 1, 0, 1);
+    MI355_ST_SLAB(1, 0, 1, 1);
+    for (int kt = 2; kt < KT; kt += 2) {
+      MI355_ST_SLAB(0, 1, kt, 0);
+      MI355_ST_SLAB(1, 0, kt + 1, 0);
+    }
+    // The staging registers now hold the next tile's slabs 1 and 2 (for the last tile: loads that are never used).
+    // The code from here to the next slab is scheduled by the compiler, which does not know that such a register may
+    // still be receiving its load: let every load land while nothing but the loads owns these registers.
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+
+    // ---- epilogue of this tile, out of LDS that no stage uses (stage 0 already holds the next tile's slab 0) ----
+    // Its addresses are derived from a lane id the compiler cannot see through, or it would compute all of them
+    // ahead of the tile loop and keep them in registers that the K loop needs (it then spills to scratch).
+    const int le = opaque_lane_id();
+    const int r32e = le & 31, he = le >> 5;
+    if constexpr (sizeof(OutT) == 2) {
+      // 16-bit epilogue through a wave-private LDS region, one 32-row x 64-column piece (two accumulator tiles) per
+      // pass: 8-byte writes of 4 consecutive n (chunk slot c ^ ((m >> 1) & 7) of the 128-byte row), whole rows read
+      // back 16 bytes per lane and stored as full cache lines.  LDS operations of a wave execute in order, so the
+      // passes need no waits between them.  Two tiles per pass, not four: the staging registers stay live across the
+      // epilogue (they hold the next tile's slabs) and a wider pass would not fit the remaining registers.
+      constexpr int ROW_B = 128;
+      char* ep = lds + 2 * STAGE + wave * (32 * ROW_B);
+      const int er = le >> 3, ec = le & 7;
+      const buffer_rsrc_t c_dst = make_buffer(C + (size_t)(tile_m * BM + wm * WTM) * N + tile_n * BN + wn * WTN,
+                                              (unsigned)(((WTM - 1) * (size_t)N + WTN) * 2));
+      const int c_lane_off = (er * N + ec * 8) * 2;
+#pragma unroll
+      for (int j = 0; j < TM; j++) {
+#pragma unroll
+        for (int ip = 0; ip < TN / 2; ip++) {
+#pragma unroll
+          for (int ii = 0; ii < 2; ii++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+              const int c = ii * 4 + q, i = 2 * ip + ii;
+              half4 v = {cvt16<BF>(acc[i][j][4 * q]), cvt16<BF>(acc[i][j][4 * q + 1]), cvt16<BF>(acc[i][j][4 * q + 2]),
+                         cvt16<BF>(acc[i][j][4 * q + 3])};
+              *reinterpret_cast<half4*>(ep + r32e * ROW_B + ((c ^ ((r32e >> 1) & 7)) * 16) + 8 * he) = v;
+            }
+#pragma unroll
+          for (int it = 0; it < 4; it++) {
+            const int row = it * 8 + er;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(ep + row * ROW_B + ((ec ^ ((row >> 1) & 7)) * 16));
+            // row j * 32 + it * 8 + er of the wave's 128 x 128 block, columns ip * 64 + ec * 8 .. + 7: one per-lane
+            // offset for the whole epilogue, the rest in the scalar offset
+            __builtin_amdgcn_raw_buffer_store_b128(v, c_dst, c_lane_off, ((j * 32 + it * 8) * N + ip * 64) * 2, 0);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    } else {
+      const int m0 = tile_m * BM + wm * WTM + r32e;
+      const int n0 = tile_n * BN + wn * WTN + 4 * he;
+#pragma unroll
+      for (int j = 0; j < TM; j++) {
+        OutT* crow = C + (size_t)(m0 + j * 32) * N + n0;
+#pragma unroll
+        for (int i = 0; i < TN; i++)
+#pragma unroll
+          for (int q = 0; q < 4; q++)
+            OutPack<OutT, BF>::store4(crow + i * 32 + q * 8, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                                      acc[i][j][4 * q + 3]);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < TN; i++)
+#pragma unroll
+      for (int j = 0; j < TM; j++)
+#pragma unroll
+        for (int q = 0; q < 16; q++) acc[i][j][q] = 0.f;
+    a_src = a_nxt;
+    b_src = b_nxt;
+    tile_m = nxt_m;
+    tile_n = nxt_n;
+    lane_offsets();
+    // the next tile's first fragments, read again (stage 0 holds its slab 0): not carrying them across the epilogue
+    // leaves the epilogue 32 more registers
+    read_frags(lds, 0, fm0, fn0);
   }
 #undef MI355_ST_SLAB
 #undef MI355_ST_GROUP
@@ -551,50 +658,6 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_staged(const half_t* 
 #undef MI355_ST_LOAD_ALL
 #undef MI355_ST_WRITE
 #undef MI355_ST_LOAD
-  // drain the speculative loads; every wave is past its last fragment read before the epilogue reuses LDS
-  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-  __syncthreads();
-
-  if constexpr (sizeof(OutT) == 2) {
-    // fp16 epilogue through LDS, one wave-private region each, 32 rows per pass (see the tiled kernel)
-    constexpr int ROW_B = WTN * 2, CH = WTN / 8;
-    char* ep = lds + wave * (32 * ROW_B);
-    constexpr int ROWS_PER_IT = 64 / CH;
-    const int er = lane / CH, ec = lane % CH;
-#pragma unroll
-    for (int j = 0; j < TM; j++) {
-#pragma unroll
-      for (int i = 0; i < TN; i++)
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-          const int c = i * 4 + q;
-          half4 v = {cvt16<BF>(acc[i][j][4 * q]), cvt16<BF>(acc[i][j][4 * q + 1]), cvt16<BF>(acc[i][j][4 * q + 2]),
-                     cvt16<BF>(acc[i][j][4 * q + 3])};
-          *reinterpret_cast<half4*>(ep + r32 * ROW_B + ((c ^ ((r32 >> 1) & 7)) * 16) + 8 * h) = v;
-        }
-      OutT* cbase = C + (size_t)(tile_m * BM + wm * WTM + j * 32) * N + tile_n * BN + wn * WTN + ec * 8;
-#pragma unroll
-      for (int it = 0; it < 32 / ROWS_PER_IT; it++) {
-        const int row = it * ROWS_PER_IT + er;
-        half8 v = *reinterpret_cast<const half8*>(ep + row * ROW_B + ((ec ^ ((row >> 1) & 7)) * 16));
-        *reinterpret_cast<half8*>(cbase + (size_t)row * N) = v;
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  } else {
-    const int m0 = tile_m * BM + wm * WTM + r32;
-    const int n0 = tile_n * BN + wn * WTN + 4 * h;
-#pragma unroll
-    for (int j = 0; j < TM; j++) {
-      OutT* crow = C + (size_t)(m0 + j * 32) * N + n0;
-#pragma unroll
-      for (int i = 0; i < TN; i++)
-#pragma unroll
-        for (int q = 0; q < 4; q++)
-          OutPack<OutT, BF>::store4(crow + i * 32 + q * 8, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
-                                acc[i][j][4 * q + 3]);
-    }
-  }
 }
 
 // Persistent kernel: one workgroup per CU walks its share of the output tiles (tile ids pid, pid + grid,
@@ -999,32 +1062,13 @@ static const GemmVariant kGemmVariants[] = {
     {"staged_256x256x64_w2x2", 256, 256, 256},
     {"staged_256x256_tail_128x128", 256, 256, 256},
     {"skinny_m32_n32_w8", 32, 32, 512},
+    {"staged_256x256x64_w2x2_walk", 256, 256, 256},
     {"generic_64x64x32", 64, 64, 256},
 };
 constexpr int kNumGemmVariants = sizeof(kGemmVariants) / sizeof(kGemmVariants[0]);
 
 int gemm_variant_count() { return kNumGemmVariants; }
 const char* gemm_variant_name(int i) { return (i >= 0 && i < kNumGemmVariants) ? kGemmVariants[i].name : nullptr; }
-
-template <int BM, int BN, int WM, int WN, typename OutT, int KIND, bool BF>  // KIND: 0 tiled, 1 pipelined, 2 register-staged
-static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int K, int ldc, hipStream_t stream) {
-  // the kernels use their N argument only as the row stride of C, so a column range of a wider C is the
-  // same launch with ldc in its place
-  constexpr bool PIPELINED = KIND == 1;
-  void (*kern)(const half_t*, const half_t*, OutT*, int, int, int, int, int, int);
-  if constexpr (KIND == 2) kern = gemm_f16_nt_staged<BM, BN, WM, WN, OutT, BF>;
-  else if constexpr (PIPELINED) kern = gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT, BF>;
-  else kern = gemm_f16_nt_tiled<BM, BN, WM, WN, OutT, BF>;
-  constexpr int lds_bytes = 2 * (BM + BN) * 128;
-  static std::atomic<uint64_t> lds_ok{0};
-  if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt")) return rc;
-  const int tiles_m = M / BM, tiles_n = N / BN;
-  int group_m = 4;
-  dim3 grid(tiles_m * tiles_n), block(WM * WN * 64);
-  hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, M, ldc, K, tiles_m,
-                     tiles_n, group_m);
-  return check_launch(KIND == 2 ? "gemm_f16_nt_staged" : PIPELINED ? "gemm_f16_nt_pipelined" : "gemm_f16_nt_tiled", grid, block, lds_bytes);
-}
 
 // number of CUs of the device the stream's context is on (cached per device)
 static int cu_count() {
@@ -1037,6 +1081,35 @@ static int cu_count() {
     cached[dev] = n;
   }
   return cached[dev];
+}
+
+template <int BM, int BN, int WM, int WN, typename OutT, int KIND, bool BF>  // KIND: 0 tiled, 1 pipelined, 2 register-staged
+static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int K, int ldc, hipStream_t stream,
+                        bool one_per_cu = false) {
+  // the kernels use their N argument only as the row stride of C, so a column range of a wider C is the
+  // same launch with ldc in its place
+  constexpr bool PIPELINED = KIND == 1;
+  void (*kern)(const half_t*, const half_t*, OutT*, int, int, int, int, int, int);
+  if constexpr (KIND == 2) kern = gemm_f16_nt_staged<BM, BN, WM, WN, OutT, BF>;
+  else if constexpr (PIPELINED) kern = gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT, BF>;
+  else kern = gemm_f16_nt_tiled<BM, BN, WM, WN, OutT, BF>;
+  // the register-staged kernel keeps its epilogue out of the stages: 32 rows x 128 bytes per wave
+  constexpr int lds_bytes = 2 * (BM + BN) * 128 + (KIND == 2 ? WM * WN * 32 * 128 : 0);
+  static std::atomic<uint64_t> lds_ok{0};
+  if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt")) return rc;
+  const int tiles_m = M / BM, tiles_n = N / BN;
+  int group_m = 4;
+  int wgs = tiles_m * tiles_n;
+  if (KIND == 2 && one_per_cu) {
+    // one workgroup per CU walking tiles pid, pid + grid, ...; a multiple of 8 keeps a workgroup's tiles on its XCD
+    int g = cu_count() & ~7;
+    if (g < 8) g = 8;
+    if (wgs > g) wgs = g;
+  }
+  dim3 grid(wgs), block(WM * WN * 64);
+  hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, M, ldc, K, tiles_m,
+                     tiles_n, group_m);
+  return check_launch(KIND == 2 ? "gemm_f16_nt_staged" : PIPELINED ? "gemm_f16_nt_pipelined" : "gemm_f16_nt_tiled", grid, block, lds_bytes);
 }
 
 template <int BM, int BN, int WM, int WN, typename OutT, bool BF>
@@ -1116,6 +1189,7 @@ static int launch_variant(int variant, const void* a, const void* b, void* c, in
       }
       return 0;
     }
+    case 10: return launch_tiled<256, 256, 2, 2, OutT, 2, BF>(a, b, c, M, N, K, N, stream, true);
     default: {
       dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
       hipLaunchKernelGGL((gemm_f16_nt_generic<OutT, BF>), grid, block, 0, stream, (const half_t*)a, (const half_t*)b, (OutT*)c,
@@ -1142,7 +1216,8 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
   auto fits = [&](int v) {
     if (v == kNumGemmVariants - 1) return true;
     if (v <= 1 && (K < 128 || K > (1 << 21))) return false;  // prefetches two slabs ahead; 32-bit byte offsets inside a 256-row panel
-    if ((v == 7 || v == 8) && (K < 256 || K % 128 != 0 || K > (1 << 21))) return false;  // slabs in pairs, three in flight
+    if ((v == 7 || v == 8 || v == 10) && N > (1 << 22)) return false;  // 32-bit byte offsets inside a wave's 128 rows of C
+    if ((v == 7 || v == 8 || v == 10) && (K < 256 || K % 128 != 0 || K > (1 << 21))) return false;  // slabs in pairs, three in flight
     if (v == 9) return al && M <= 64 && N % 32 == 0 && K % 64 == 0;  // a tile is 32 rows of B; 64-half K segments
     return al && M % kGemmVariants[v].bm == 0 && N % kGemmVariants[v].bn == 0 && K % 64 == 0;
   };
