@@ -36,14 +36,23 @@ def _hipcc() -> str:
     return exe
 
 
-# Kernels that load into registers with hand-placed waits ("staged") must not spill: the compiler does not know
-# that such a register is still being filled, and a spill would store it before its data has arrived.
+# Kernels that load into registers by inline assembly with hand-placed waits ("staged", "skinny"): the compiler does
+# not know that such a register may still be receiving its load, so it must never move one -- no spill to scratch,
+# no spill of any other kind, and no change of the register budget that a different occupancy would bring.  The
+# expected occupancy (waves per SIMD) is pinned per kernel family; a compiler that allocates differently fails the
+# build instead of producing a kernel that stores a register before its data has arrived.
 NO_SPILL_KERNELS = ("staged", "skinny")
+EXPECTED_OCCUPANCY = {"staged": 1, "gemm_f16_nt_skinny": 7, "gemm_mxfp4_skinny": 2}
 _USAGE_FLAG = "-Rpass-analysis=kernel-resource-usage"
 
 
+def _remark_int(text: str) -> int:
+    return int(text.split(":", 1)[1].split("[")[0].strip())
+
+
 def _check_resource_remarks(stderr: str) -> list[str]:
-    """Returns the remark-free stderr lines; raises if a kernel named in NO_SPILL_KERNELS uses scratch."""
+    """Returns the remark-free stderr lines; raises if a kernel named in NO_SPILL_KERNELS uses scratch, spills a
+    vector register, or is built for another occupancy than EXPECTED_OCCUPANCY pins for it."""
     rest, name = [], None
     for line in stderr.splitlines():
         if _USAGE_FLAG not in line and "remark:" not in line:
@@ -55,10 +64,18 @@ def _check_resource_remarks(stderr: str) -> list[str]:
         text = line.split("remark:", 1)[1]
         if "Function Name:" in text:
             name = text.split("Function Name:", 1)[1].split("[")[0].strip()
-        elif "ScratchSize" in text and name is not None:
-            scratch = int(text.split(":", 1)[1].split("[")[0].strip())
-            if scratch and any(k in name for k in NO_SPILL_KERNELS):
-                raise RuntimeError(f"kernel {name} spills ({scratch} bytes of scratch per lane); it must fit its registers")
+            continue
+        if name is None or not any(k in name for k in NO_SPILL_KERNELS):
+            continue
+        if "ScratchSize" in text and _remark_int(text):
+            raise RuntimeError(f"kernel {name} spills ({_remark_int(text)} bytes of scratch per lane); it must fit its registers")
+        if "VGPRs Spill" in text and _remark_int(text):
+            raise RuntimeError(f"kernel {name} spills {_remark_int(text)} vector registers; it must fit its registers")
+        if "Occupancy" in text:
+            for family, want in EXPECTED_OCCUPANCY.items():
+                if family in name and _remark_int(text) != want:
+                    raise RuntimeError(f"kernel {name} is built for {_remark_int(text)} waves per SIMD, expected {want}: its "
+                                       "register allocation changed; check the hand-placed waits against the new code")
     return rest
 
 

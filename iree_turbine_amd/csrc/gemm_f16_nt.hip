@@ -580,7 +580,11 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_staged(const half_t* 
     // The staging registers now hold the next tile's slabs 1 and 2 (for the last tile: loads that are never used).
     // The code from here to the next slab is scheduled by the compiler, which does not know that such a register may
     // still be receiving its load: let every load land while nothing but the loads owns these registers.
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    // The wait names every staging register as an input: the compiler has to keep them allocated to the loads up
+    // to this point and cannot hand one to other code while its load (a speculative one past the last slab included)
+    // is still in flight.
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::"v"(r[0][0]), "v"(r[0][1]), "v"(r[0][2]), "v"(r[0][3]), "v"(r[0][4]), "v"(r[0][5]), "v"(r[0][6]), "v"(r[0][7]), "v"(r[0][8]), "v"(r[0][9]), "v"(r[0][10]), "v"(r[0][11]), "v"(r[0][12]), "v"(r[0][13]), "v"(r[0][14]), "v"(r[0][15]) : "memory");
+    asm volatile("" ::"v"(r[1][0]), "v"(r[1][1]), "v"(r[1][2]), "v"(r[1][3]), "v"(r[1][4]), "v"(r[1][5]), "v"(r[1][6]), "v"(r[1][7]), "v"(r[1][8]), "v"(r[1][9]), "v"(r[1][10]), "v"(r[1][11]), "v"(r[1][12]), "v"(r[1][13]), "v"(r[1][14]), "v"(r[1][15]) : "memory");
 
     // ---- epilogue of this tile, out of LDS that no stage uses (stage 0 already holds the next tile's slab 0) ----
     // Its addresses are derived from a lane id the compiler cannot see through, or it would compute all of them

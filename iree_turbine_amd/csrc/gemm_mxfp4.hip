@@ -1012,7 +1012,12 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_staged(const uint8_t* __restri
     sc_wr ^= 4096;
     // The loads of the last slabs fetch nothing that is used, and behind the loop the compiler hands their
     // registers to the epilogue: let them land while the registers still belong to them.
-    if (kt + 2 >= KT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // The wait names every staging register as an input, so that the registers stay allocated to the loads up to it
+    // however the compiler restructures the last iteration.
+    if (kt + 2 >= KT) {
+      asm volatile("s_waitcnt vmcnt(0)" ::"v"(r[0][0]), "v"(r[0][1]), "v"(r[0][2]), "v"(r[0][3]), "v"(r[0][4]), "v"(r[0][5]), "v"(r[0][6]), "v"(r[0][7]), "v"(r[0][8]), "v"(r[0][9]), "v"(r[0][10]), "v"(r[0][11]), "v"(r[0][12]), "v"(r[0][13]), "v"(r[0][14]), "v"(r[0][15]), "v"(r[0][16]) : "memory");
+      asm volatile("" ::"v"(r[1][0]), "v"(r[1][1]), "v"(r[1][2]), "v"(r[1][3]), "v"(r[1][4]), "v"(r[1][5]), "v"(r[1][6]), "v"(r[1][7]), "v"(r[1][8]), "v"(r[1][9]), "v"(r[1][10]), "v"(r[1][11]), "v"(r[1][12]), "v"(r[1][13]), "v"(r[1][14]), "v"(r[1][15]), "v"(r[1][16]) : "memory");
+    }
   }
 #undef MI355_MX_SLAB
 #undef MI355_MX_GROUP
@@ -1026,13 +1031,17 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_staged(const uint8_t* __restri
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
   __syncthreads();
 
+  // epilogue addresses from a lane id taken behind the drain: derived from `lane` they would be computed ahead of it,
+  // in registers that are not free while the staging sets are live
+  const int le = opaque_lane_id();
+  const int r32e = le & 31, he = le >> 5;
   if constexpr (sizeof(OutT) == 2) {
     // bf16 epilogue through LDS, one wave-private region each, 32 rows per pass: ds_write_b64 of 4 consecutive n
     // (chunk slot c ^ ((m >> 1) & 7)), whole 256-byte rows read back 16 bytes per lane
     constexpr int ROW_B = WTN * 2, CH = WTN / 8;
     char* ep = lds + wave * (32 * ROW_B);
     constexpr int ROWS_PER_IT = 64 / CH;
-    const int er = lane / CH, ec = lane % CH;
+    const int er = le / CH, ec = le % CH;
 #pragma unroll
     for (int j = 0; j < TM; j++) {
 #pragma unroll
@@ -1042,7 +1051,7 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_staged(const uint8_t* __restri
           const int c = i * 4 + q;
           ushortx4 v = {f32_to_bf16_rne(acc[i][j][4 * q]), f32_to_bf16_rne(acc[i][j][4 * q + 1]),
                         f32_to_bf16_rne(acc[i][j][4 * q + 2]), f32_to_bf16_rne(acc[i][j][4 * q + 3])};
-          *reinterpret_cast<ushortx4*>(ep + r32 * ROW_B + ((c ^ ((r32 >> 1) & 7)) * 16) + 8 * h) = v;
+          *reinterpret_cast<ushortx4*>(ep + r32e * ROW_B + ((c ^ ((r32e >> 1) & 7)) * 16) + 8 * he) = v;
         }
       OutT* cbase = C + (size_t)(tile_m * BM + wm * WTM + j * 32) * N + tile_n * BN + wn * WTN + ec * 8;
 #pragma unroll
@@ -1054,8 +1063,8 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_staged(const uint8_t* __restri
       __builtin_amdgcn_sched_barrier(0);
     }
   } else {
-    const int m0 = tile_m * BM + wm * WTM + r32;
-    const int n0 = tile_n * BN + wn * WTN + 4 * h;
+    const int m0 = tile_m * BM + wm * WTM + r32e;
+    const int n0 = tile_n * BN + wn * WTN + 4 * he;
 #pragma unroll
     for (int j = 0; j < TM; j++) {
       OutT* crow = C + (size_t)(m0 + j * 32) * N + n0;

@@ -329,7 +329,12 @@ __global__ __launch_bounds__(256) void gemm_mxfp6_staged(const uint8_t* __restri
     sc_wr ^= 4096;
     // The loads of the last slabs fetch nothing that is used, and behind the loop the compiler hands their
     // registers to the epilogue: let them land while the registers still belong to them.
-    if (kt + 2 >= KT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // The wait names every staging register as an input, so that the registers stay allocated to the loads up to it
+    // however the compiler restructures the last iteration.
+    if (kt + 2 >= KT) {
+      asm volatile("s_waitcnt vmcnt(0)" ::"v"(r[0][0]), "v"(r[0][1]), "v"(r[0][2]), "v"(r[0][3]), "v"(r[0][4]), "v"(r[0][5]), "v"(r[0][6]), "v"(r[0][7]), "v"(r[0][8]), "v"(r[0][9]), "v"(r[0][10]), "v"(r[0][11]) : "memory");
+      asm volatile("" ::"v"(r[1][0]), "v"(r[1][1]), "v"(r[1][2]), "v"(r[1][3]), "v"(r[1][4]), "v"(r[1][5]), "v"(r[1][6]), "v"(r[1][7]), "v"(r[1][8]), "v"(r[1][9]), "v"(r[1][10]), "v"(r[1][11]) : "memory");
+    }
   }
 #undef MI355_M6_SLAB
 #undef MI355_M6_W
@@ -340,7 +345,7 @@ __global__ __launch_bounds__(256) void gemm_mxfp6_staged(const uint8_t* __restri
 #undef MI355_M6_WRITE
 #undef MI355_M6_LOAD_SC
 #undef MI355_M6_LOAD
-  // every wave is past its last fragment read before the epilogue reuses LDS
+  // drain the speculative loads; every wave is past its last fragment read before the epilogue reuses LDS
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
   __syncthreads();
 

@@ -8,14 +8,16 @@ from iree_turbine_amd import build
 REMARK = "x.hip:1:1: remark: {} [-Rpass-analysis=kernel-resource-usage]"
 
 
-def _remarks(name, scratch):
+def _remarks(name, scratch, vgpr_spill=0, occupancy=1):
     return "\n".join([
         REMARK.format(f"Function Name: {name}"),
         "    1 | void k() {",
         "      | ^",
         REMARK.format("    VGPRs: 256"),
         REMARK.format(f"    ScratchSize [bytes/lane]: {scratch}"),
-        REMARK.format("    VGPRs Spill: 3"),
+        REMARK.format(f"    Occupancy [waves/SIMD]: {occupancy}"),
+        REMARK.format("    SGPRs Spill: 2"),
+        REMARK.format(f"    VGPRs Spill: {vgpr_spill}"),
         "x.hip:7:3: warning: something else",
     ])
 
@@ -25,8 +27,18 @@ def test_staged_kernel_with_scratch_is_refused():
         build._check_resource_remarks(_remarks("_ZN5mi35517gemm_mxfp8_stagedItLb1EEEv", 36))
 
 
+def test_staged_kernel_with_a_register_spill_or_another_occupancy_is_refused():
+    with pytest.raises(RuntimeError, match="spills 3 vector registers"):
+        build._check_resource_remarks(_remarks("_ZN5mi35517gemm_mxfp8_stagedItLb1EEEv", 0, vgpr_spill=3))
+    with pytest.raises(RuntimeError, match="2 waves per SIMD, expected 1"):
+        build._check_resource_remarks(_remarks("_ZN5mi35517gemm_mxfp8_stagedItLb1EEEv", 0, occupancy=2))
+    with pytest.raises(RuntimeError, match="expected 7"):
+        build._check_resource_remarks(_remarks("_ZN5mi35518gemm_f16_nt_skinnyIfLb1EEEv", 0, occupancy=8))
+    build._check_resource_remarks(_remarks("_ZN5mi35517gemm_mxfp4_skinnyIfEEv", 0, occupancy=2))
+
+
 def test_other_kernels_may_use_scratch_and_warnings_pass_through():
-    rest = build._check_resource_remarks(_remarks("_ZN5mi35517gemm_mxfp8_genericItLb1EEEv", 36))
+    rest = build._check_resource_remarks(_remarks("_ZN5mi35517gemm_mxfp8_genericItLb1EEEv", 36, vgpr_spill=3, occupancy=4))
     assert rest == ["x.hip:7:3: warning: something else"]
     rest = build._check_resource_remarks(_remarks("_ZN5mi35517gemm_mxfp8_stagedItLb1EEEv", 0))
     assert rest == ["x.hip:7:3: warning: something else"]
