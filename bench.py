@@ -18,7 +18,7 @@ enough copies of them that every timed launch streams from HBM.  The legs of the
 non-causal prefill, MXFP4 GEMM, decode) each carry a "cpu_baseline": the CPU restatement of the same
 computation timed on a bounded sample on the host cores in the same run.
 
-Calibration workloads (run only when named): copy_1GiB (what the HBM counters read for a known copy) and
+Calibration workloads (run only when named): library_gemm_8192 (torch.mm, the vendor library, on the headline shape), copy_1GiB (what the HBM counters read for a known copy) and
 mfma_{f16,fp4}_regloop_{zeros,benchmark} (what the MFMA unit sustains from registers on all-zero operands
 and on operands drawn like the benchmark's: the measured ceiling beside the datasheet peak).
 """
@@ -437,7 +437,24 @@ WORKLOADS = {
     "mxfp8_4096x8192x8192": wl_mxfp8(4096, 8192, 8192),
     "mxfp6_4096x8192x8192": wl_mxfp6(4096, 8192, 8192),
 }
+def wl_library_gemm(M, N, K):
+    """The same NT product through torch.mm (hipBLASLt / rocBLAS): the vendor library's time beside this path's."""
+    from oracle import inputs
+
+    def build(dev):
+        a, b = inputs.gemm_inputs(M, N, K)
+        ad, bd = a.to(dev), b.to(dev)
+        flops = 2.0 * M * N * K
+        return {
+            "fn": lambda: torch.mm(ad, bd.t()), "work": flops, "bytes": 2.0 * (M * K + N * K + M * N), "flops": flops,
+            "bound": "mfma", "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s", "dtype": "f16", "cpu": lambda: None,
+            "config": {"workload": f"library_torch_mm_f16_nt_{M}x{N}x{K}_f16out", "M": M, "N": N, "K": K, "seed": 10},
+        }
+    return build
+
+
 CALIBRATION = {  # not part of the path: run only when named with --workload
+    "library_gemm_8192": wl_library_gemm(8192, 8192, 8192),
     "copy_1GiB": wl_copy(),
     "mfma_f16_regloop_zeros": wl_mfma_regloop("f16", "zeros"),
     "mfma_f16_regloop_benchmark": wl_mfma_regloop("f16", "benchmark"),
