@@ -238,12 +238,21 @@ struct FaPaged {
 // the same quotient), which keeps the 64-register rescale off the common path.
 // V swizzle: chunk c of row r -> slot c ^ (4 * (r & 3)), which keeps the four 64-byte row pieces that a
 // half-wave transpose read touches on distinct banks (measured conflict-free; c ^ 2(r & 7) is not).
-template <bool CAUSAL, bool PAGED, bool BF>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void fa_fwd_d128_pipe(
+// NW = waves per workgroup: 4 (128 queries, two workgroups per CU) or 8 (256 queries, one workgroup per CU: the two
+// wave quartets of a CU then share ONE copy of every K / V tile instead of loading one each -- half the LDS writes
+// and half the L2 reads for the same fragment reads).
+template <bool CAUSAL, bool PAGED, bool BF, int NW = 4>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void fa_fwd_d128_pipe(
     const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V, half_t* __restrict__ O, int BH,
     int Sq, int Sk_arg, float scale_log2e, int q_blocks, FaLayout lay, FaPaged pg) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
+  static_assert(NW == 4 || (NW == 8 && !PAGED), "the paged form maps one page to one wave-load of a 4-wave workgroup");
+  constexpr int BLOCK_M = NW * 32;          // queries per workgroup
+  constexpr int NI = 16 / NW;               // wave-loads per wave and tile (a wave-load = 4 rows of 256 bytes)
   constexpr int TILE_B = FA_BLOCK_N * 256;  // bytes of one K or V tile
+  // (A three-slot ring for the 8-wave form -- tiles loaded two trips ahead, a trip waiting only for the loads of the
+  // trip before -- measured 5 % slower than two slots: load latency is not what the trips wait for, and ring slots
+  // that are not compile-time constants cost address arithmetic.)
   constexpr int VBUF = 2 * TILE_B;          // K ring at 0, V ring behind it
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -303,14 +312,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   for (int pass = 0; pass < (CAUSAL ? 2 : 1); pass++) {
   const int qb = CAUSAL ? (pass == 0 ? q_blocks - 1 - unit : unit) : unit;
   if (CAUSAL && pass == 1 && 2 * unit == q_blocks - 1) break;  // the middle block of an odd count has no partner
-  const int q0 = qb * FA_BLOCK_M;
+  const int q0 = qb * BLOCK_M;
   const int wq0 = q0 + wave * 32;
   const int q_row = wq0 + r32;
   const bool q_ok = q_row < Sq;
 
   int k_end = Sk;
   if (CAUSAL) {
-    int last_q = q0 + FA_BLOCK_M - 1;
+    int last_q = q0 + BLOCK_M - 1;
     if (last_q > Sq - 1) last_q = Sq - 1;
     int lim = last_q + causal_off + 1;
     if (lim < k_end) k_end = lim;
@@ -334,7 +343,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   }
 
   const int lrow = lane >> 4, lslot = lane & 15;
-  const int k_chunk = lslot ^ (wave * 4 + lrow);
+  const int k_chunk = lslot ^ ((wave * 4 + lrow) & 15);
   const int v_chunk = lslot ^ (4 * lrow);
   // Global -> LDS through a buffer descriptor rebuilt per tile on the scalar unit (base = first row of the tile,
   // size = up to the end of the tile's last valid row): the per-lane byte offset is loop-invariant, rows at or
@@ -378,7 +387,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     } else {
       const buffer_rsrc_t rs = make_buffer(reinterpret_cast<const char*>(base) + (size_t)row0 * rb, (unsigned)(rem - 1) * rb + 256u);
 #pragma unroll
-      for (int i = 0; i < 4; i++) buffer_load_lds_16B(rs, voff + (unsigned)i * 16u * rb, 0, dst + i * 4096);
+      for (int i = 0; i < NI; i++) buffer_load_lds_16B(rs, voff + (unsigned)(i * NW * 4) * rb, 0, dst + i * NW * 1024);
     }
   };
 
@@ -572,9 +581,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   }  // pass
 }
 
-static const char* kFaVariants[] = {"d128_bm128_bn64_w4_pipelined", "d128_bm128_bn64_w4"};
-int fa_variant_count() { return 2; }
-const char* fa_variant_name(int i) { return (i >= 0 && i < 2) ? kFaVariants[i] : nullptr; }
+static const char* kFaVariants[] = {"d128_bm128_bn64_w4_pipelined", "d128_bm128_bn64_w4", "d128_bm256_bn64_w8_pipelined"};
+int fa_variant_count() { return 3; }
+const char* fa_variant_name(int i) { return (i >= 0 && i < 3) ? kFaVariants[i] : nullptr; }
 
 }  // namespace mi355
 
@@ -593,7 +602,7 @@ static int fa_launch(const void* q, const void* k, const void* v, void* o, int64
     return fail(-MI355_E_SHAPE, "%s: %lld query heads over %lld key/value heads", who, (long long)H, (long long)Hkv);
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o))
     return fail(-MI355_E_ALIGN, "%s: q, k, v, o must be 16-byte aligned", who);
-  if (variant > 1) return fail(-MI355_E_DTYPE, "%s: variant %d out of range", who, variant);
+  if (variant > 2) return fail(-MI355_E_DTYPE, "%s: variant %d out of range", who, variant);
   if (!(scale > 0.f) || !isfinite(scale)) return fail(-MI355_E_SHAPE, "%s: scale must be positive and finite", who);
   const int BH = (int)(B * H);
   const int q_blocks = (int)((Sq + FA_BLOCK_M - 1) / FA_BLOCK_M);
@@ -605,6 +614,21 @@ static int fa_launch(const void* q, const void* k, const void* v, void* o, int64
   for (int i = 0; i < 4; i++)
     if (int rc = allow_lds(kernels[i], lds_bytes, lds_ok[i], "fa_fwd_d128")) return rc;
   const float scale_log2e = scale * 1.4426950408889634f;
+  // Without a mask, and with enough 256-query blocks for every CU, the 8-wave form is ahead (2 x 32 x 4096: 503 against
+  // 514 us); with the causal mask the two are level and the 4-wave form has the finer-grained tail.
+  if (variant < 0 && !is_causal && (int64_t)BH * ((Sq + 255) / 256) >= 512) variant = 2;
+  if (variant == 2) {
+    // eight waves: 256-query blocks, one workgroup per CU
+    auto kern = is_causal ? fa_fwd_d128_pipe<true, false, BF, 8> : fa_fwd_d128_pipe<false, false, BF, 8>;
+    static std::atomic<uint64_t> ok8[2] = {};
+    const int lds8 = lds_bytes;
+    if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds8, ok8[is_causal ? 1 : 0], "fa_fwd_d128_pipe<8>")) return rc;
+    const int qb8 = (int)((Sq + 255) / 256);
+    dim3 grid(BH * (is_causal ? (qb8 + 1) / 2 : qb8)), block(512);
+    hipLaunchKernelGGL(kern, grid, block, lds8, reinterpret_cast<hipStream_t>(stream), (const half_t*)q, (const half_t*)k,
+                       (const half_t*)v, (half_t*)o, BH, (int)Sq, (int)Sk, scale_log2e, qb8, lay, FaPaged{nullptr, nullptr, 0, 0, 0});
+    return check_launch("fa_fwd_d128_pipe<8 waves>", grid, block, lds8);
+  }
   // the pipelined causal kernel takes a pair of query blocks per workgroup
   const int units = (variant != 1 && is_causal) ? (q_blocks + 1) / 2 : q_blocks;
   dim3 grid(BH * units), block(256);

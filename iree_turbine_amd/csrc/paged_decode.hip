@@ -60,6 +60,30 @@ __device__ __forceinline__ float merge_splits(const float* part_acc, const float
   return r;
 }
 
+// Exclusive prefix sum of one int per thread over the 256 threads of the workgroup (wave scans by shuffles, the
+// four wave totals through `tmp`, 4 ints of LDS); every thread also gets the grand total.
+__device__ __forceinline__ int block_exclusive_scan(int v, int* tmp, int& total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int incl = v;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int n = __shfl_up(incl, d);
+    if (lane >= d) incl += n;
+  }
+  if (lane == 63) tmp[wave] = incl;
+  __syncthreads();
+  int base = 0;
+  total = 0;
+#pragma unroll
+  for (int w = 0; w < PD_WAVES; w++) {
+    const int tw = tmp[w];
+    base += w < wave ? tw : 0;
+    total += tw;
+  }
+  __syncthreads();
+  return base + incl - v;
+}
+
 template <int G, bool BF>  // G = q heads per kv head (<= 16); BF = bf16 instead of fp16 operands and output
 __global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
     const half_t* __restrict__ Q, const half_t* __restrict__ Kc, const half_t* __restrict__ Vc,
@@ -91,6 +115,46 @@ __global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
     __syncthreads();
     seq = *pick;
     __syncthreads();  // the slot is part of the V ring
+  } else if (num_seqs > PD_WAVES * 64 && num_seqs <= 16384) {
+    // Larger batches: an exact rank would cost num_seqs^2 / 256 loads per thread.  Sequences are instead put into 256
+    // buckets by length (longest first) with a counting pass, the workgroup finds the bucket that holds rank
+    // blockIdx.z, and takes the sequence at that offset inside the bucket in thread-major order -- a bijection from
+    // ranks to sequences that is ordered by length down to 1/256 of the longest possible length, for a few loads
+    // per thread and two block scans.
+    int* hist = reinterpret_cast<int*>(lds);  // [256] sequences per bucket
+    int* tmp = hist + 256;                    // [4] scan scratch
+    int* res = tmp + 4;                       // bucket, offset inside it, chosen sequence
+    const int t = threadIdx.x;
+    const int reach = (max_pages_per_seq << page_shift) * 16;
+    auto bucket_of = [&](int len) {
+      len = len < 0 ? 0 : (len > reach ? reach : len);
+      return 255 - (int)(((long long)len * 255) / (reach > 0 ? reach : 1));
+    };
+    hist[t] = 0;
+    __syncthreads();
+    for (int j = t; j < num_seqs; j += PD_WAVES * 64) atomicAdd(&hist[bucket_of(seq_lens[j])], 1);
+    __syncthreads();
+    int total;
+    const int mine = hist[t];
+    const int first = block_exclusive_scan(mine, tmp, total);
+    const int z = (int)blockIdx.z;
+    if (first <= z && z < first + mine) {
+      res[0] = t;
+      res[1] = z - first;
+    }
+    __syncthreads();
+    const int bkt = res[0], off = res[1];
+    int hits = 0;
+    for (int j = t; j < num_seqs; j += PD_WAVES * 64) hits += bucket_of(seq_lens[j]) == bkt;
+    const int before = block_exclusive_scan(hits, tmp, total);
+    if (before <= off && off < before + hits) {
+      int k = off - before;
+      for (int j = t; j < num_seqs; j += PD_WAVES * 64)
+        if (bucket_of(seq_lens[j]) == bkt && k-- == 0) res[2] = j;
+    }
+    __syncthreads();
+    seq = res[2];
+    __syncthreads();  // the area is part of the V ring
   }
   const int num_q_heads = num_kv_heads * G;
   // a length beyond what the block table can address is cut to the table's reach

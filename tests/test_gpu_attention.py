@@ -44,6 +44,30 @@ def test_attention_cross_lengths(dev, causal):
     torch.testing.assert_close(o, ref, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("Sq,Sk", [(1, 1), (64, 64), (255, 255), (257, 257), (300, 777), (1024, 1024), (700, 100)])
+def test_attention_eight_wave_form(dev, Sq, Sk, causal):
+    """The 8-wave form (256 queries per workgroup, both wave quartets sharing one copy of every K / V tile): ragged
+    and cross lengths, query counts around the 256-query block, Sq > Sk -- against the oracle, and bit-identical to
+    the 4-wave form (same per-wave arithmetic, only the tile loads are split differently)."""
+    import iree_turbine_amd as ita
+    from oracle import attention as oa, inputs
+
+    announce(f"flash_attn_fwd 8 waves Sq={Sq} Sk={Sk} causal={causal}")
+    names = ita._lib.variants("flash_attn_fwd")
+    v8 = names.index("d128_bm256_bn64_w8_pipelined")
+    q, k, v = inputs.attention_inputs(2, 3, Sq, 128, seed=12, Sk=Sk)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    o8, o4 = torch.empty_like(qd), torch.empty_like(qd)
+    ita.launch.flash_attn_fwd_out(qd, kd, vd, o8, causal, 0.0, v8)
+    ita.launch.flash_attn_fwd_out(qd, kd, vd, o4, causal, 0.0, 0)
+    assert torch.equal(o8, o4)
+    got = o8.float().cpu()
+    if causal and Sq > Sk:
+        got, q = got[:, :, Sq - Sk:], q[:, :, Sq - Sk:]  # the first Sq - Sk queries see no key (zeros, checked elsewhere)
+    torch.testing.assert_close(got, oa.sdpa_ref(q, k, v, is_causal=causal), rtol=RTOL, atol=ATOL)
+
+
 def test_attention_causal_more_queries_than_keys(dev):
     """Lower-right aligned causal mask with Sq > Sk: query i sees keys j <= i - (Sq - Sk), so the first
     Sq - Sk queries see no key at all.  Those rows are defined as zero (the sum of an empty softmax); every

@@ -24,7 +24,7 @@ def _to(dev, *ts):
     return [t.to(dev) for t in ts]
 
 
-@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("variant", [0, 1, 2])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("Sq,Sk", [(128, 128), (1024, 1024), (100, 100), (333, 333), (96, 320), (1, 77)])
 def test_prefill_bf16(dev, Sq, Sk, causal, variant):

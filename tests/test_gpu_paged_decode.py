@@ -156,6 +156,23 @@ def test_decode_invariances(dev):
     assert torch.equal(two, base)
 
 
+@pytest.mark.parametrize("num_seqs,splits", [(257, 1), (300, 2), (1000, 1)])
+def test_decode_large_batches_walk_sequences_by_length_bucket(dev, num_seqs, splits):
+    """Beyond 256 sequences the kernel orders its workgroups by length bucket (a counting pass and two block scans)
+    instead of by exact rank: every sequence must still be computed exactly once -- equal lengths, empty sequences
+    and one very long sequence among short ones included."""
+    import iree_turbine_amd  # noqa: F401
+    from oracle import inputs, paged_decode as op
+
+    announce(f"paged decode {num_seqs} sequences splits={splits}")
+    q, kc, vc, bt, sl = inputs.paged_decode_inputs(num_seqs=num_seqs, num_q_heads=8, num_kv_heads=2, min_len=1, max_len=90, seed=17)
+    sl[5] = 0  # equal lengths are plentiful: up to 1000 draws from 90 values
+    out = torch.ops.mi355.paged_decode_attn(*_to(dev, q, kc, vc, bt, sl), 0.0, splits)
+    ref = op.paged_decode_ref(q, kc, vc, bt, sl)
+    torch.testing.assert_close(out.float().cpu(), ref, rtol=RTOL, atol=ATOL)
+    assert torch.equal(out[5].cpu(), torch.zeros(8, 128, dtype=torch.float16))
+
+
 def test_decode_one_launch_merge_equals_two_phase(dev):
     """The op merges the kv splits inside the phase-0 kernel (the last workgroup of a (sequence, kv head) to finish
     does it); the C entry with caller scratch runs phase 0 and phase 1 as two launches.  Same arithmetic: bit-equal,
