@@ -19,7 +19,7 @@ non-causal prefill, MXFP4 GEMM, decode) each carry a "cpu_baseline": the CPU res
 computation timed on a bounded sample on the host cores in the same run.
 
 Calibration workloads (run only when named): library_gemm_8192 (torch.mm, the vendor library, on the headline shape), copy_1GiB (what the HBM counters read for a known copy) and
-mfma_{f16,fp4}_regloop_{zeros,benchmark} (what the MFMA unit sustains from registers on all-zero operands
+mfma_{f16,f16x16,fp4}_regloop_{zeros,benchmark} (what the MFMA unit sustains from registers on all-zero operands
 and on operands drawn like the benchmark's: the measured ceiling beside the datasheet peak).
 """
 
@@ -47,27 +47,27 @@ METRIC = "TFLOP/s & %MFMA peak (f16 GEMM, causal FA, MXFP4 GEMM); decode HBM GB/
 # dispatch, scaled by what the same counters read for a copy kernel of known size); filled in from
 # the summaries kept under profiles/.  None = not measured.
 MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
-    "gemm_8192": 1.745e9,              # 1536 MiB read + 128 MiB written: each of the 8 XCD L2s fetches its own copy of
+    "gemm_8192": 1.783e9,              # 1572 MiB read + 128 MiB written: each of the 8 XCD L2s fetches its own copy of
                                        # the panels its 4x8 block of output tiles needs (12 panels x 4 MiB x 4 rounds x 8)
-    "gemm_4096": 2.458e8,
-    "gemm_2048x10240x8192": 6.472e8,
-    "gemm_2048x57344x8192": 3.054e9,
+    "gemm_4096": 2.464e8,
+    "gemm_2048x10240x8192": 6.570e8,
+    "gemm_2048x57344x8192": 3.120e9,
     "gemm_1024_f32out": 1.684e7,
-    "gemm_bf16_8192": 1.746e9,
+    "gemm_bf16_8192": 1.783e9,
     "gemm_16x8192x8192": 1.366e8,
     "fa_causal": 3.425e8,
     "fa_noncausal": 2.686e8,
     "decode": 1.177e9,
-    "fa_causal_bf16": 3.482e8,
+    "fa_causal_bf16": 3.481e8,
     "decode_bf16": 1.177e9,
-    "mxfp4_4096x8192x8192": 2.947e8,
+    "mxfp4_4096x8192x8192": 3.011e8,
     "mxfp4_32x8192x8192": 3.739e7,
     "mxfp4_quantize_16384x16384": 6.796e8,
     "mxfp8_quantize_16384x16384": 8.138e8,
     "mxfp6_quantize_16384x16384": 7.466e8,
-    "paged_prefill": 6.959e8,
-    "mxfp8_4096x8192x8192": 4.832e8,
-    "mxfp6_4096x8192x8192": 3.822e8,
+    "paged_prefill": 6.948e8,
+    "mxfp8_4096x8192x8192": 4.828e8,
+    "mxfp6_4096x8192x8192": 3.819e8,
 }
 
 
@@ -388,14 +388,14 @@ def wl_mfma_regloop(kind: str, data: str):
         nbytes = 1 << 20
         if data == "zeros":
             ops = torch.zeros(nbytes, dtype=torch.uint8)
-        elif kind == "f16":
+        elif kind in ("f16", "f16x16"):
             ops = (torch.randn(nbytes // 2, generator=g) * 0.1).half().view(torch.uint8)
         else:
             ops = torch.randint(0, 256, (nbytes,), generator=g, dtype=torch.uint8)
         opsd = ops.to(dev)
         workgroups, trips = 512, 2000  # two workgroups of four waves per CU
         sink = torch.empty(workgroups * 256, dtype=torch.float32, device=dev)
-        code = 0 if kind == "f16" else (1 if data == "zeros" else 2)
+        code = {"f16": 0, "f16x16": 3}.get(kind, 1 if data == "zeros" else 2)
         flop = ctypes.c_double(0.0)
         lib = _lib.load()
 
@@ -407,10 +407,11 @@ def wl_mfma_regloop(kind: str, data: str):
         torch.cuda.synchronize()
         return {
             "fn": fn, "work": flop.value, "bytes": 0.0, "flops": flop.value, "bound": "mfma",
-            "peak": PEAK_F16_TFLOPS if kind == "f16" else PEAK_FP4_TFLOPS, "unit": "TFLOP/s",
-            "dtype": "f16" if kind == "f16" else "fp4(e2m1)+e8m0", "cpu": lambda: None,
+            "peak": PEAK_F16_TFLOPS if kind != "fp4" else PEAK_FP4_TFLOPS, "unit": "TFLOP/s",
+            "dtype": "f16" if kind != "fp4" else "fp4(e2m1)+e8m0", "cpu": lambda: None,
             "config": {"workload": f"mfma_{kind}_regloop_{data}", "workgroups": workgroups, "trips": trips,
-                       "instruction": "v_mfma_f32_32x32x16_f16" if kind == "f16" else "v_mfma_scale_f32_32x32x64_f8f6f4 (fp4 x fp4)"},
+                       "instruction": {"f16": "v_mfma_f32_32x32x16_f16", "f16x16": "v_mfma_f32_16x16x32_f16"}.get(
+                           kind, "v_mfma_scale_f32_32x32x64_f8f6f4 (fp4 x fp4)")},
         }
     return build
 
@@ -458,6 +459,8 @@ CALIBRATION = {  # not part of the path: run only when named with --workload
     "copy_1GiB": wl_copy(),
     "mfma_f16_regloop_zeros": wl_mfma_regloop("f16", "zeros"),
     "mfma_f16_regloop_benchmark": wl_mfma_regloop("f16", "benchmark"),
+    "mfma_f16x16_regloop_zeros": wl_mfma_regloop("f16x16", "zeros"),
+    "mfma_f16x16_regloop_benchmark": wl_mfma_regloop("f16x16", "benchmark"),
     "mfma_fp4_regloop_zeros": wl_mfma_regloop("fp4", "zeros"),
     "mfma_fp4_regloop_benchmark": wl_mfma_regloop("fp4", "benchmark"),
 }

@@ -396,7 +396,8 @@ int mi355_mxfp8_quantize(const void* x, int in_dtype, int64_t rows, int64_t K,
  * kernels can be read against beside the datasheet peak.  No counterpart in the reference; it plays
  * the part of the plain-copy workload for the HBM figures.
  * kind 0: v_mfma_f32_32x32x16_f16; 1: v_mfma_scale_f32_32x32x64_f8f6f4 with fp4 operands and unit
- * scales; 2: the same with E8M0 scales spread over 2^-8 .. 2^7.  operands: operand_bytes (a power of
+ * scales; 2: the same with E8M0 scales spread over 2^-8 .. 2^7; 3: v_mfma_f32_16x16x32_f16 (two per
+ * 32x32x16's worth of flop).  operands: operand_bytes (a power of
  * two >= 16) of device memory read once before the loop; sink: >= workgroups * 256 floats, written
  * once after it; *flop_per_launch (optional, host memory) receives the flop count of the launch.
  */

@@ -40,6 +40,33 @@ __global__ __launch_bounds__(CAL_WAVES * 64) void calibrate_mfma_f16_kernel(cons
   sink[t] = s;
 }
 
+// 16x16x32 fp16 MFMAs (half the output block, twice the depth per instruction): per wave and trip, 2 * CAL_CHAINS
+// MFMAs of 16*16*32*2 flop, the same flop per trip as the 32x32x16 loop.
+__global__ __launch_bounds__(CAL_WAVES * 64) void calibrate_mfma_f16_16x16x32_kernel(const half8* __restrict__ operands, unsigned mask,
+                                                                                     float* __restrict__ sink, int trips) {
+  const unsigned t = threadIdx.x + blockIdx.x * blockDim.x;
+  half8 a[4], b[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    a[i] = operands[(t * 8 + i) & mask];
+    b[i] = operands[(t * 8 + 4 + i) & mask];
+  }
+  floatx4 c[2 * CAL_CHAINS];
+#pragma unroll
+  for (int i = 0; i < 2 * CAL_CHAINS; i++) c[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 1
+  for (int it = 0; it < trips; it++) {
+#pragma unroll
+    for (int i = 0; i < 2 * CAL_CHAINS; i++) c[i] = mfma_16x16x32(a[i & 3], b[(i >> 2) & 3], c[i]);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 2 * CAL_CHAINS; i++)
+#pragma unroll
+    for (int r = 0; r < 4; r++) s += c[i][r];
+  sink[t] = s;
+}
+
 // Scaled 32x32x64 MFMAs with fp4 operands (16 bytes per lane; the upper half of the operand registers is unused):
 // per wave and trip, CAL_CHAINS MFMAs of 32*32*64*2 flop.  scale_mode 0: every block scale 2^0; 1: E8M0 bytes
 // 119..134 derived from the operand bits (exponents spread over [-8, 7] like a block-scaled benchmark's).
@@ -79,11 +106,11 @@ __global__ __launch_bounds__(CAL_WAVES * 64) void calibrate_mfma_fp4_kernel(cons
 
 using namespace mi355;
 
-// kind 0: fp16 32x32x16; kind 1: fp4 32x32x64 with unit scales; kind 2: fp4 with spread scales.
+// kind 0: fp16 32x32x16; kind 1: fp4 32x32x64 with unit scales; kind 2: fp4 with spread scales; kind 3: fp16 16x16x32.
 extern "C" int mi355_calibrate_mfma(int kind, const void* operands, int64_t operand_bytes, float* sink, int64_t sink_floats,
                                     int64_t workgroups, int64_t trips, double* flop_per_launch, void* stream) {
   if (!operands || !sink) return fail(-MI355_E_NULL, "calibrate_mfma: null pointer");
-  if (kind < 0 || kind > 2) return fail(-MI355_E_DTYPE, "calibrate_mfma: kind %d unknown (0 fp16, 1 fp4, 2 fp4 with spread scales)", kind);
+  if (kind < 0 || kind > 3) return fail(-MI355_E_DTYPE, "calibrate_mfma: kind %d unknown (0 fp16 32x32x16, 1 fp4, 2 fp4 with spread scales, 3 fp16 16x16x32)", kind);
   if (operand_bytes < 16 || (operand_bytes & (operand_bytes - 1)) || operand_bytes > (1ll << 30))
     return fail(-MI355_E_SHAPE, "calibrate_mfma: operand_bytes %lld must be a power of two in [16, 2^30]", (long long)operand_bytes);
   if (workgroups <= 0 || workgroups > 65535 || trips <= 0 || trips > (1 << 24))
@@ -94,9 +121,11 @@ extern "C" int mi355_calibrate_mfma(int kind, const void* operands, int64_t oper
   const unsigned mask = (unsigned)(operand_bytes / 16 - 1);
   dim3 grid((unsigned)workgroups), block(CAL_WAVES * 64);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  const double per_mfma = kind == 0 ? 2.0 * 32 * 32 * 16 : 2.0 * 32 * 32 * 64;
+  const double per_mfma = (kind == 0 || kind == 3) ? 2.0 * 32 * 32 * 16 : 2.0 * 32 * 32 * 64;  // kind 3: per pair of MFMAs
   if (flop_per_launch) *flop_per_launch = per_mfma * CAL_CHAINS * (double)trips * CAL_WAVES * (double)workgroups;
-  if (kind == 0)
+  if (kind == 3)
+    hipLaunchKernelGGL(calibrate_mfma_f16_16x16x32_kernel, grid, block, 0, s, (const half8*)operands, mask, sink, (int)trips);
+  else if (kind == 0)
     hipLaunchKernelGGL(calibrate_mfma_f16_kernel, grid, block, 0, s, (const half8*)operands, mask, sink, (int)trips);
   else
     hipLaunchKernelGGL(calibrate_mfma_fp4_kernel, grid, block, 0, s, (const intx4*)operands, mask, sink, (int)trips, kind == 2);
