@@ -5,6 +5,8 @@
 // toggle), so the caller supplies the operand bytes: all zeros reads the issue-rate peak, operands drawn like a
 // benchmark's read the ceiling any kernel can reach on that benchmark's data.  A roofline fraction quoted against
 // the datasheet peak can then be read against the measured ceiling as well.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace mi355 {
@@ -67,6 +69,57 @@ __global__ __launch_bounds__(CAL_WAVES * 64) void calibrate_mfma_f16_16x16x32_ke
   sink[t] = s;
 }
 
+// GEMM-like register loops: 256 accumulators per lane (a 128 x 128 block per wave, as the GEMM kernels hold), eight A
+// and eight B operand registers rotated over the trips, and every product subtracted again eight trips later (a negated
+// copy of the A operands), so the accumulators wander around zero like the partial sums of a product of zero-mean
+// data instead of growing without bound -- the accumulate path sees operands of comparable exponents, as in a real
+// GEMM.  WIDE = false: 16 MFMAs 32x32x16 per trip; true: 64 MFMAs 16x16x32 per trip (twice the flop).
+template <bool WIDE>
+__global__ __launch_bounds__(CAL_WAVES * 64) void calibrate_mfma_f16_walk_kernel(const half8* __restrict__ operands, unsigned mask,
+                                                                                 float* __restrict__ sink, int trips) {
+  const unsigned t = threadIdx.x + blockIdx.x * blockDim.x;
+  half8 a[16], b[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    a[i] = operands[(t * 16 + i) & mask];
+    a[8 + i] = -a[i];
+    b[i] = operands[(t * 16 + 8 + i) & mask];
+  }
+#pragma unroll
+  for (int i = 0; i < 8; i++) asm volatile("" : "+v"(a[8 + i]));  // kept in registers, not recomputed inside the loop
+  constexpr int R = WIDE ? 8 : 4;
+  typedef typename std::conditional<WIDE, floatx4, floatx16>::type acc_t;
+  acc_t c[R][R];
+#pragma unroll
+  for (int i = 0; i < R; i++)
+#pragma unroll
+    for (int j = 0; j < R; j++)
+#pragma unroll
+      for (int r = 0; r < (WIDE ? 4 : 16); r++) c[i][j][r] = 0.f;
+#pragma unroll 1
+  for (int it = 0; it < trips; it += 16) {
+#pragma unroll
+    for (int tt = 0; tt < 16; tt++) {
+#pragma unroll
+      for (int i = 0; i < R; i++)
+#pragma unroll
+        for (int j = 0; j < R; j++) {
+          const half8 av = a[((j + tt) & 7) + (tt >= 8 ? 8 : 0)], bv = b[(i + 3 * tt) & 7];
+          if constexpr (WIDE) c[i][j] = mfma_16x16x32(bv, av, c[i][j]);
+          else c[i][j] = mfma_32x32x16(bv, av, c[i][j]);
+        }
+    }
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < R; i++)
+#pragma unroll
+    for (int j = 0; j < R; j++)
+#pragma unroll
+      for (int r = 0; r < (WIDE ? 4 : 16); r++) s += c[i][j][r];
+  sink[t] = s;
+}
+
 // Scaled 32x32x64 MFMAs with fp4 operands (16 bytes per lane; the upper half of the operand registers is unused):
 // per wave and trip, CAL_CHAINS MFMAs of 32*32*64*2 flop.  scale_mode 0: every block scale 2^0; 1: E8M0 bytes
 // 119..134 derived from the operand bits (exponents spread over [-8, 7] like a block-scaled benchmark's).
@@ -106,11 +159,12 @@ __global__ __launch_bounds__(CAL_WAVES * 64) void calibrate_mfma_fp4_kernel(cons
 
 using namespace mi355;
 
-// kind 0: fp16 32x32x16; kind 1: fp4 32x32x64 with unit scales; kind 2: fp4 with spread scales; kind 3: fp16 16x16x32.
+// kind 0: fp16 32x32x16; kind 1: fp4 32x32x64 with unit scales; kind 2: fp4 with spread scales; kind 3: fp16 16x16x32;
+// kinds 4 / 5: the GEMM-like loops with 32x32x16 / 16x16x32 (trips rounded down to a multiple of 16).
 extern "C" int mi355_calibrate_mfma(int kind, const void* operands, int64_t operand_bytes, float* sink, int64_t sink_floats,
                                     int64_t workgroups, int64_t trips, double* flop_per_launch, void* stream) {
   if (!operands || !sink) return fail(-MI355_E_NULL, "calibrate_mfma: null pointer");
-  if (kind < 0 || kind > 3) return fail(-MI355_E_DTYPE, "calibrate_mfma: kind %d unknown (0 fp16 32x32x16, 1 fp4, 2 fp4 with spread scales, 3 fp16 16x16x32)", kind);
+  if (kind < 0 || kind > 5) return fail(-MI355_E_DTYPE, "calibrate_mfma: kind %d unknown (0 fp16 32x32x16, 1 fp4, 2 fp4 with spread scales, 3 fp16 16x16x32, 4 / 5 GEMM-like 32x32x16 / 16x16x32)", kind);
   if (operand_bytes < 16 || (operand_bytes & (operand_bytes - 1)) || operand_bytes > (1ll << 30))
     return fail(-MI355_E_SHAPE, "calibrate_mfma: operand_bytes %lld must be a power of two in [16, 2^30]", (long long)operand_bytes);
   if (workgroups <= 0 || workgroups > 65535 || trips <= 0 || trips > (1 << 24))
@@ -122,6 +176,16 @@ extern "C" int mi355_calibrate_mfma(int kind, const void* operands, int64_t oper
   dim3 grid((unsigned)workgroups), block(CAL_WAVES * 64);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const double per_mfma = (kind == 0 || kind == 3) ? 2.0 * 32 * 32 * 16 : 2.0 * 32 * 32 * 64;  // kind 3: per pair of MFMAs
+  if (kind >= 4) {
+    trips &= ~15ll;
+    if (trips <= 0) return fail(-MI355_E_SHAPE, "calibrate_mfma: the GEMM-like loops need trips >= 16");
+    if (flop_per_launch) *flop_per_launch = 2.0 * 32 * 32 * 16 * (kind == 4 ? 16 : 32) * (double)trips * CAL_WAVES * (double)workgroups;
+    if (kind == 4)
+      hipLaunchKernelGGL(calibrate_mfma_f16_walk_kernel<false>, grid, block, 0, s, (const half8*)operands, mask, sink, (int)trips);
+    else
+      hipLaunchKernelGGL(calibrate_mfma_f16_walk_kernel<true>, grid, block, 0, s, (const half8*)operands, mask, sink, (int)trips);
+    return check_launch("calibrate_mfma", grid, block, 0);
+  }
   if (flop_per_launch) *flop_per_launch = per_mfma * CAL_CHAINS * (double)trips * CAL_WAVES * (double)workgroups;
   if (kind == 3)
     hipLaunchKernelGGL(calibrate_mfma_f16_16x16x32_kernel, grid, block, 0, s, (const half8*)operands, mask, sink, (int)trips);

@@ -664,6 +664,252 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_staged(const half_t* 
 #undef MI355_ST_LOAD
 }
 
+// Streamed form: whole 128-byte rows of a 64-half slab go global -> LDS directly (8 rows per wave-load), and LDS is
+// freed in pieces WITHIN a slab, so that loads run two slabs ahead in 160 KiB with no staging registers and no ds_write:
+//  * the B fragments of a slab (128 rows x 64 halfs per wave = 16 registers of 8 halfs) are held in registers for the
+//    whole slab and fetched from LDS during the first half of the slab before, so a B buffer is free half a slab after
+//    its reads begin; three 32 KiB B buffers;
+//  * the A rows are streamed: fragment (16 rows, 32 halfs) by fragment, each feeding 8 MFMAs 16x16x32 against the held
+//    B fragments, read from LDS four steps (one interval) ahead; a block of 32 A rows per half is free one interval
+//    after it was read; two 32 KiB A buffers, the loads of slab t + 2 follow the reads of slab t block by block.
+// One step = 8 MFMAs (m block j = step / 2, k half = step % 2) + one A read + (first half of the slab) two B reads + one
+// load; 16 steps per slab, a barrier every 4 steps (an interval).  At a barrier every wave has waited for its loads older
+// than one slab and for its LDS reads older than one interval, which is what the reuse below relies on:
+//   interval q of slab t loads   A: block q - 1 of slab t + 2 (q = 0: block 3 of slab t + 1)
+//                                B: part q + 1 of slab t + 3 (q = 3: part 0 of slab t + 4)
+// Reads and waits are inline assembly (with direct-to-LDS loads in flight the compiler would wait for all of them before
+// any LDS read it can see); every read's destination is tied to the wait that covers it.
+template <typename OutT, bool BF>
+__global__ __launch_bounds__(256) void gemm_f16_nt_stream(const half_t* __restrict__ A, const half_t* __restrict__ B,
+                                                          OutT* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n,
+                                                          int group_m) {
+  constexpr int BM = 256, BN = 256, WN = 2, WTM = 128, WTN = 128;
+  constexpr int BUF = 256 * 128;                 // one operand, one slab
+  constexpr int B_AT = 0, A_AT = 3 * BUF;        // three B buffers, then two A buffers
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  int tile_m, tile_n;
+  map_tile(blockIdx.x, tiles_m, tiles_n, group_m, tile_m, tile_n);
+
+  // global side: a wave-load covers 8 rows x 128 bytes; wave w loads rows 128 h + 32 blk + 8 w .. + 7 of either operand.
+  // lane = (row l >> 3, slot l & 7) fetches chunk slot ^ ((row >> 1) & 7): the row's 8-row group index 16 h + 4 blk + w
+  // has the parity of w
+  const unsigned row_bytes = (unsigned)K * 2u;
+  const buffer_rsrc_t a_src = make_buffer(A + (size_t)(tile_m * BM + wave * 8) * K, (unsigned)(BM - wave * 8) * row_bytes);
+  const buffer_rsrc_t b_src = make_buffer(B + (size_t)(tile_n * BN + wave * 8) * K, (unsigned)(BN - wave * 8) * row_bytes);
+  const int lrow = lane >> 3;
+  const unsigned g_off = (unsigned)lrow * row_bytes + (unsigned)((lane & 7) ^ (((wave & 1) << 2) | (lrow >> 1))) * 16u;
+  const int KT = K / 64;  // even, >= 4 (checked on the host)
+  // rows 128 h + 32 blk (+ 8 wave) of slab `slab` of operand X into the buffer at byte offset buf_at
+  auto load = [&](bool is_a, int buf_at, int h, int blk, int slab) {
+    const unsigned so = (unsigned)(h * 128 + blk * 32) * row_bytes + (unsigned)(slab < KT ? slab : KT - 1) * 128u;
+    buffer_load_lds_16B(is_a ? a_src : b_src, g_off, so, lds + buf_at + (h * 16 + blk * 4 + wave) * 1024);
+  };
+
+  // fragment reads: lane l takes row l & 15 of a 16-row block, chunk 4 kh + (l >> 4) of the 128-byte row
+  const int r16 = lane & 15, cq = lane >> 4;
+  const unsigned lds0 = (unsigned)(uintptr_t)MI355_LDS(char, lds);
+  const unsigned lane_rd = (unsigned)(r16 * 128 + ((cq ^ (r16 >> 1)) & 7) * 16);  // k half 1: ^ 64
+  unsigned aaddr[2][2];  // [A buffer][k half]
+#pragma unroll
+  for (int bf = 0; bf < 2; bf++)
+#pragma unroll
+    for (int kh = 0; kh < 2; kh++) aaddr[bf][kh] = lds0 + A_AT + bf * BUF + wm * (WTM * 128) + (lane_rd ^ (kh * 64));
+  const unsigned b_lane = lds0 + B_AT + wn * (WTN * 128) + lane_rd;
+  unsigned baddr[2];  // [k half], of the B buffer being read in this slab
+
+  floatx4 acc[8][8];  // [n block][m block]
+#pragma unroll
+  for (int i = 0; i < 8; i++)
+#pragma unroll
+    for (int j = 0; j < 8; j++) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+  half8 fb0[2][8], fb1[2][8], fa[8];
+
+  // MFMAs as inline assembly with the accumulators pinned to AGPRs: with 64 four-register accumulators the compiler's
+  // own allocation keeps moving some of them between the two register classes inside the loop.  No MFMA here reads an
+  // accumulator written fewer than 8 MFMAs earlier, and nothing else touches the accumulators before the loop ends.
+#define MI355_SM_MFMA(c, x, y)                                                                                  \
+  do {                                                                                                          \
+    if constexpr (BF) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(x), "v"(y));       \
+    else asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(x), "v"(y));                     \
+  } while (0)
+#define MI355_SM_READ(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off))
+#define MI355_SM_TIE8(X) "+v"(X[0]), "+v"(X[1]), "+v"(X[2]), "+v"(X[3]), "+v"(X[4]), "+v"(X[5]), "+v"(X[6]), "+v"(X[7])
+
+  // ---- prologue: B0, A0, B1, A1 blocks 0..2, B2 ----
+#pragma unroll
+  for (int x = 0; x < 8; x++) load(false, B_AT, x & 1, x >> 1, 0);
+#pragma unroll
+  for (int x = 0; x < 8; x++) load(true, A_AT, x & 1, x >> 1, 0);
+#pragma unroll
+  for (int x = 0; x < 8; x++) load(false, B_AT + BUF, x & 1, x >> 1, 1);
+#pragma unroll
+  for (int x = 0; x < 6; x++) load(true, A_AT + BUF, x & 1, x >> 1, 1);
+#pragma unroll
+  for (int x = 0; x < 8; x++) load(false, B_AT + 2 * BUF, x & 1, x >> 1, 2);
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_waitcnt vmcnt(14)" ::: "memory");  // B0, A0, B1 have landed
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+  baddr[0] = b_lane;
+  baddr[1] = b_lane ^ 64;
+  MI355_SM_READ(fb0[0][0], baddr[0], 0 * 2048); MI355_SM_READ(fb0[0][1], baddr[0], 1 * 2048);
+  MI355_SM_READ(fb0[0][2], baddr[0], 2 * 2048); MI355_SM_READ(fb0[0][3], baddr[0], 3 * 2048);
+  MI355_SM_READ(fb0[0][4], baddr[0], 4 * 2048); MI355_SM_READ(fb0[0][5], baddr[0], 5 * 2048);
+  MI355_SM_READ(fb0[0][6], baddr[0], 6 * 2048); MI355_SM_READ(fb0[0][7], baddr[0], 7 * 2048);
+  MI355_SM_READ(fb0[1][0], baddr[1], 0 * 2048); MI355_SM_READ(fb0[1][1], baddr[1], 1 * 2048);
+  MI355_SM_READ(fb0[1][2], baddr[1], 2 * 2048); MI355_SM_READ(fb0[1][3], baddr[1], 3 * 2048);
+  MI355_SM_READ(fb0[1][4], baddr[1], 4 * 2048); MI355_SM_READ(fb0[1][5], baddr[1], 5 * 2048);
+  MI355_SM_READ(fb0[1][6], baddr[1], 6 * 2048); MI355_SM_READ(fb0[1][7], baddr[1], 7 * 2048);
+  MI355_SM_READ(fa[0], aaddr[0][0], 0); MI355_SM_READ(fa[1], aaddr[0][1], 0);
+  MI355_SM_READ(fa[2], aaddr[0][0], 2048); MI355_SM_READ(fa[3], aaddr[0][1], 2048);
+  asm volatile("s_waitcnt lgkmcnt(0)" : MI355_SM_TIE8(fb0[0]), MI355_SM_TIE8(fb0[1]), "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]));
+  __builtin_amdgcn_s_barrier();  // every wave has read B0: its buffer may receive slab 3
+  __builtin_amdgcn_sched_barrier(0);
+  load(false, B_AT, 0, 0, 3);
+  load(false, B_AT, 1, 0, 3);
+  __builtin_amdgcn_sched_barrier(0);
+
+  // B buffer rotation: slab t lives in buffer t % 3
+  int b_rd = BUF;       // byte offset of the buffer read during this slab (slab t + 1)
+  int b_ld012 = 0;      // buffer loaded in intervals 0..2 (slab t + 3)
+
+  // Step s of a slab whose A buffer is PAR: MFMAs of (m block s / 2, k half s % 2) on fa[s % 8] against FB[s % 2][0..7].
+  // LGKM = LDS reads issued after the read that filled fa[s % 8] (they may still be in flight).
+#define MI355_SM_STEP(s, PAR, FB, FBN, LGKM)                                                                               \
+  do {                                                                                                                     \
+    constexpr int s4 = (s) + 4, nb = s4 >= 16 ? 1 - (PAR) : (PAR), ns = s4 & 15;                                           \
+    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(fa[(s)&7]) : "n"(LGKM));                                                   \
+    __builtin_amdgcn_sched_barrier(0);                                                                                     \
+    MI355_SM_MFMA(acc[0][(s) >> 1], FB[(s)&1][0], fa[(s)&7]);                                      \
+    MI355_SM_READ(fa[s4 & 7], aaddr[nb][ns & 1], (ns >> 1) * 2048);                                                        \
+    __builtin_amdgcn_sched_barrier(0);                                                                                     \
+    MI355_SM_MFMA(acc[1][(s) >> 1], FB[(s)&1][1], fa[(s)&7]);                                      \
+    if constexpr ((s) < 8) MI355_SM_READ(FBN[(s) >> 2][(2 * (s)) & 7], baddr[(s) >> 2], ((2 * (s)) & 7) * 2048);           \
+    __builtin_amdgcn_sched_barrier(0);                                                                                     \
+    MI355_SM_MFMA(acc[2][(s) >> 1], FB[(s)&1][2], fa[(s)&7]);                                      \
+    MI355_SM_MFMA(acc[3][(s) >> 1], FB[(s)&1][3], fa[(s)&7]);                                      \
+    if constexpr ((s) < 8) MI355_SM_READ(FBN[(s) >> 2][(2 * (s) + 1) & 7], baddr[(s) >> 2], ((2 * (s) + 1) & 7) * 2048);   \
+    __builtin_amdgcn_sched_barrier(0);                                                                                     \
+    MI355_SM_MFMA(acc[4][(s) >> 1], FB[(s)&1][4], fa[(s)&7]);                                      \
+    MI355_SM_MFMA(acc[5][(s) >> 1], FB[(s)&1][5], fa[(s)&7]);                                      \
+    {                                                                                                                      \
+      constexpr int q = (s) >> 2, x = (s)&3;                                                                               \
+      if constexpr (x < 2) {                                                                                               \
+        if constexpr (q == 0) load(true, A_AT + (1 - (PAR)) * BUF, x, 3, kt + 1);                                          \
+        else load(true, A_AT + (PAR) * BUF, x, q - 1, kt + 2);                                                             \
+      } else {                                                                                                             \
+        if constexpr (q == 3) load(false, B_AT + b_rd, x - 2, 0, kt + 4);                                                  \
+        else load(false, B_AT + b_ld012, x - 2, q + 1, kt + 3);                                                            \
+      }                                                                                                                    \
+    }                                                                                                                      \
+    __builtin_amdgcn_sched_barrier(0);                                                                                     \
+    MI355_SM_MFMA(acc[6][(s) >> 1], FB[(s)&1][6], fa[(s)&7]);                                      \
+    MI355_SM_MFMA(acc[7][(s) >> 1], FB[(s)&1][7], fa[(s)&7]);                                      \
+    __builtin_amdgcn_sched_barrier(0);                                                                                     \
+  } while (0)
+  // End of an interval: loads older than one slab and LDS reads older than this interval are complete in every wave.
+#define MI355_SM_SYNC(RD)                                                        \
+  do {                                                                           \
+    asm volatile("s_waitcnt vmcnt(16) lgkmcnt(%0)" ::"n"(RD) : "memory");        \
+    __builtin_amdgcn_s_barrier();                                                \
+    __builtin_amdgcn_sched_barrier(0);                                           \
+  } while (0)
+  // Reads issued in one step: 3 in the first half of a slab (A, B, B), 1 in the second.  The read that fills fa for
+  // step s was the first read of step s - 4.
+#define MI355_SM_SLAB(PAR, FB, FBN)                                                                             \
+  do {                                                                                                          \
+    baddr[0] = b_lane + (unsigned)b_rd;                                                                         \
+    baddr[1] = baddr[0] ^ 64;                                                                                   \
+    MI355_SM_STEP(0, PAR, FB, FBN, 3);  /* steps 12..15 of the slab before: one read each */                    \
+    MI355_SM_STEP(1, PAR, FB, FBN, 5);                                                                          \
+    MI355_SM_STEP(2, PAR, FB, FBN, 7);                                                                          \
+    MI355_SM_STEP(3, PAR, FB, FBN, 9);                                                                          \
+    MI355_SM_SYNC(12);                                                                                          \
+    MI355_SM_STEP(4, PAR, FB, FBN, 11);                                                                         \
+    MI355_SM_STEP(5, PAR, FB, FBN, 11);                                                                         \
+    MI355_SM_STEP(6, PAR, FB, FBN, 11);                                                                         \
+    MI355_SM_STEP(7, PAR, FB, FBN, 11);                                                                         \
+    MI355_SM_SYNC(12);                                                                                          \
+    MI355_SM_STEP(8, PAR, FB, FBN, 11);                                                                         \
+    MI355_SM_STEP(9, PAR, FB, FBN, 9);                                                                          \
+    MI355_SM_STEP(10, PAR, FB, FBN, 7);                                                                         \
+    MI355_SM_STEP(11, PAR, FB, FBN, 5);                                                                         \
+    MI355_SM_SYNC(4);                                                                                           \
+    MI355_SM_STEP(12, PAR, FB, FBN, 3);                                                                         \
+    MI355_SM_STEP(13, PAR, FB, FBN, 3);                                                                         \
+    MI355_SM_STEP(14, PAR, FB, FBN, 3);                                                                         \
+    MI355_SM_STEP(15, PAR, FB, FBN, 3);                                                                         \
+    /* the B fragments of the next slab were all requested in steps 0..7: they have landed; tie them to this point */ \
+    asm volatile("s_waitcnt vmcnt(16) lgkmcnt(4)" : MI355_SM_TIE8(FBN[0]), MI355_SM_TIE8(FBN[1])::"memory");    \
+    __builtin_amdgcn_s_barrier();                                                                               \
+    __builtin_amdgcn_sched_barrier(0);                                                                          \
+    b_ld012 = b_rd;                                                                                             \
+    b_rd = b_rd == 2 * BUF ? 0 : b_rd + BUF;                                                                    \
+  } while (0)
+
+  for (int kt = 0; kt < KT; kt += 2) {
+    MI355_SM_SLAB(0, fb0, fb1);
+    kt++;
+    MI355_SM_SLAB(1, fb1, fb0);
+    kt--;
+  }
+  // reads and loads issued for slabs past the end are never used, but they target registers and LDS the epilogue reuses
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : MI355_SM_TIE8(fa));
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+#undef MI355_SM_SLAB
+#undef MI355_SM_SYNC
+#undef MI355_SM_STEP
+#undef MI355_SM_TIE8
+#undef MI355_SM_READ
+#undef MI355_SM_MFMA
+
+  // lane holds, for m = 16 j + (l & 15): n = 16 i + 4 (l >> 4) + r, r < 4.  The epilogue's addresses come from a lane id
+  // the compiler cannot see through, so that none of them is computed ahead of the K loop and kept across it.
+  const int le = opaque_lane_id();
+  const int r16e = le & 15, cqe = le >> 4;
+  if constexpr (sizeof(OutT) == 2) {
+    // 16-bit epilogue through LDS (every buffer is free now), one m block (16 rows x 128 columns) per pass in a
+    // wave-private region: 8-byte writes of 4 consecutive n (chunk slot c ^ ((m >> 1) & 7) within each 128-byte half
+    // row), whole rows read back 16 bytes per lane and stored as full cache lines.  LDS operations of a wave execute in
+    // order, so the passes need no waits between them.
+    constexpr int ROW_B = WTN * 2;
+    char* ep = lds + wave * (WTM * ROW_B);
+    const int er = le >> 4, ec = le & 15;
+    OutT* cbase = C + (size_t)(tile_m * BM + wm * WTM) * N + tile_n * BN + wn * WTN + ec * 8;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const int ml = j * 16 + r16e;
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        const int c = 2 * i + (cqe >> 1);
+        half4 v = {cvt16<BF>(acc[i][j][0]), cvt16<BF>(acc[i][j][1]), cvt16<BF>(acc[i][j][2]), cvt16<BF>(acc[i][j][3])};
+        *reinterpret_cast<half4*>(ep + ml * ROW_B + ((c ^ ((ml >> 1) & 7)) * 16) + 8 * (cqe & 1)) = v;
+      }
+#pragma unroll
+      for (int it = 0; it < 4; it++) {
+        const int row = j * 16 + it * 4 + er;
+        half8 v = *reinterpret_cast<const half8*>(ep + row * ROW_B + ((ec ^ ((row >> 1) & 7)) * 16));
+        *reinterpret_cast<half8*>(cbase + (size_t)row * N) = v;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  } else {
+    const int m0 = tile_m * BM + wm * WTM + r16e;
+    const int n0 = tile_n * BN + wn * WTN + 4 * cqe;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      OutT* crow = C + (size_t)(m0 + j * 16) * N + n0;
+#pragma unroll
+      for (int i = 0; i < 8; i++)
+        OutPack<OutT, BF>::store4(crow + i * 16, acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
+    }
+  }
+}
+
 // Persistent kernel: one workgroup per CU walks its share of the output tiles (tile ids pid, pid + grid,
 // ...) as ONE continuous sequence of K slabs.  The loads issued during the last two slabs of a tile
 // already fetch the first two slabs of the next tile, the fragment reads at the end of the last slab
@@ -1067,6 +1313,8 @@ static const GemmVariant kGemmVariants[] = {
     {"staged_256x256_tail_128x128", 256, 256, 256},
     {"skinny_m32_n32_w8", 32, 32, 512},
     {"staged_256x256x64_w2x2_walk", 256, 256, 256},
+    {"stream_256x256x64_w2x2", 256, 256, 256},
+    {"stream_256x256_tail_128x128", 256, 256, 256},
     {"generic_64x64x32", 64, 64, 256},
 };
 constexpr int kNumGemmVariants = sizeof(kGemmVariants) / sizeof(kGemmVariants[0]);
@@ -1134,6 +1382,19 @@ static int launch_persistent(const void* a, const void* b, void* c, int M, int N
   return check_launch("gemm_f16_nt_persistent", grid, block, lds_bytes);
 }
 
+template <typename OutT, bool BF>
+static int launch_stream(const void* a, const void* b, void* c, int M, int N, int K, int ldc, hipStream_t stream) {
+  auto kern = gemm_f16_nt_stream<OutT, BF>;
+  constexpr int lds_bytes = 5 * 256 * 128;  // three B buffers and two A buffers of 32 KiB
+  static std::atomic<uint64_t> lds_ok{0};
+  if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt_stream")) return rc;
+  const int tiles_m = M / 256, tiles_n = N / 256;
+  dim3 grid(tiles_m * tiles_n), block(256);
+  hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, M, ldc, K, tiles_m,
+                     tiles_n, 4);
+  return check_launch("gemm_f16_nt_stream", grid, block, lds_bytes);
+}
+
 // Register-staged kernel with a finer-grained last round.  256x256 tiles go to the 256 CUs in rounds; when the
 // last round would leave most CUs idle and its tiles form whole tile columns (or rows) of the grid, that
 // strip is computed by the 128x128 kernel instead (four times the workgroups, so the strip spreads over the
@@ -1152,11 +1413,15 @@ static bool tail_split(int M, int N, int& main_m, int& main_n) {
   return true;
 }
 
-template <typename OutT, bool BF>
+template <typename OutT, bool BF, bool STREAMED>
 static int launch_split(const void* a, const void* b, void* c, int M, int N, int K, hipStream_t stream) {
+  auto main_part = [&](int m, int n) {
+    if constexpr (STREAMED) return launch_stream<OutT, BF>(a, b, c, m, n, K, N, stream);
+    else return launch_tiled<256, 256, 2, 2, OutT, 2, BF>(a, b, c, m, n, K, N, stream);
+  };
   int mm, mn;
-  if (!tail_split(M, N, mm, mn)) return launch_tiled<256, 256, 2, 2, OutT, 2, BF>(a, b, c, M, N, K, N, stream);
-  int rc = launch_tiled<256, 256, 2, 2, OutT, 2, BF>(a, b, c, mm, mn, K, N, stream);
+  if (!tail_split(M, N, mm, mn)) return main_part(M, N);
+  int rc = main_part(mm, mn);
   if (rc) return rc;
   const half_t* ah = (const half_t*)a;
   const half_t* bh = (const half_t*)b;
@@ -1176,7 +1441,7 @@ static int launch_variant(int variant, const void* a, const void* b, void* c, in
     case 5: return launch_tiled<256, 256, 2, 4, OutT, 0, BF>(a, b, c, M, N, K, N, stream);
     case 6: return launch_tiled<128, 128, 2, 2, OutT, 0, BF>(a, b, c, M, N, K, N, stream);
     case 7: return launch_tiled<256, 256, 2, 2, OutT, 2, BF>(a, b, c, M, N, K, N, stream);
-    case 8: return launch_split<OutT, BF>(a, b, c, M, N, K, stream);
+    case 8: return launch_split<OutT, BF, false>(a, b, c, M, N, K, stream);
     case 9: {
       auto kern = gemm_f16_nt_skinny<OutT, BF>;
       constexpr int lds_bytes = 8 * 16384;
@@ -1194,6 +1459,8 @@ static int launch_variant(int variant, const void* a, const void* b, void* c, in
       return 0;
     }
     case 10: return launch_tiled<256, 256, 2, 2, OutT, 2, BF>(a, b, c, M, N, K, N, stream, true);
+    case 11: return launch_stream<OutT, BF>(a, b, c, M, N, K, N, stream);
+    case 12: return launch_split<OutT, BF, true>(a, b, c, M, N, K, stream);
     default: {
       dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
       hipLaunchKernelGGL((gemm_f16_nt_generic<OutT, BF>), grid, block, 0, stream, (const half_t*)a, (const half_t*)b, (OutT*)c,
@@ -1222,6 +1489,7 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
     if (v <= 1 && (K < 128 || K > (1 << 21))) return false;  // prefetches two slabs ahead; 32-bit byte offsets inside a 256-row panel
     if ((v == 7 || v == 8 || v == 10) && N > (1 << 22)) return false;  // 32-bit byte offsets inside a wave's 128 rows of C
     if ((v == 7 || v == 8 || v == 10) && (K < 256 || K % 128 != 0 || K > (1 << 21))) return false;  // slabs in pairs, three in flight
+    if ((v == 11 || v == 12) && (K < 256 || K % 128 != 0 || K > (1 << 21))) return false;  // slabs in pairs; 32-bit byte offsets inside a 256-row panel
     if (v == 9) return al && M <= 64 && N % 32 == 0 && K % 64 == 0;  // a tile is 32 rows of B; 64-half K segments
     return al && M % kGemmVariants[v].bm == 0 && N % kGemmVariants[v].bn == 0 && K % 64 == 0;
   };
@@ -1230,16 +1498,16 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
     // 128x128 tile (4x the workgroups) wins; everything else goes to the bounds-checked kernel.
     const long long t256 = (M / 256) * (N / 256);
     const long long rounds = (t256 + 255) / 256;  // 256 CUs, one 256x256 workgroup each
-    // Long K: the register-staged kernel (measured best from K = 6144 up, and at any K once there are thousands
-    // of tiles); a sparse last round of its 256x256 tiles goes to the 128x128 kernel when it can be cut off as
-    // whole tile columns or rows (+13% at 2048x10240x8192).  Short K: the persistent kernel, which hides each
-    // tile's prologue and epilogue under its neighbours (8192x8192x512: +30%, x1024: +14%, x4096: +2%), as
-    // long as its last round is >= 85% busy.
+    // The streamed kernel with its sparse last round cut off (variant 12) from K = 1024 up: 8192^3 1460 against 1295
+    // TFLOP/s for the register-staged kernel and 1285 for the persistent one, 4096^3 1405 / 1240 / 1244,
+    // 2048x10240x8192 1285 / 1180 / 1044, 8192x8192x1024 1174 / 1064 / 1167.  Shorter K: the persistent kernel, which
+    // hides each tile's prologue and epilogue under its neighbours (8192x8192x512: 978 against 854), as long as its
+    // last round is >= 85% busy.
     const bool full_rounds = t256 * 100 >= rounds * 256 * 85;
     if (fits(9) && N >= 2048 && K >= 512) variant = 9;  // decode-shaped: stream the weights once
     else
-    if (K <= 4096 && t256 <= 2048 && fits(0) && t256 >= 128 && full_rounds) variant = 0;
-    else if (fits(8) && t256 >= 128) variant = 8;
+    if (K < 1024 && t256 <= 2048 && fits(0) && t256 >= 128 && full_rounds) variant = 0;
+    else if (fits(12) && t256 >= 128) variant = 12;
     else if (fits(0) && t256 >= 128 && full_rounds) variant = 0;
     else if (fits(4)) variant = 4;
     else variant = kNumGemmVariants - 1;

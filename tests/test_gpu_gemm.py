@@ -22,7 +22,7 @@ def _run(dev, M, N, K, out_dtype, variant=-1, seed=10):
     return c.float().cpu(), ref
 
 
-@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 3, 4, 5, 6, 7, 8, 10])
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 3, 4, 5, 6, 7, 8, 10, 11, 12])
 def test_gemm_1024_f32_all_variants(dev, variant):
     c, ref = _run(dev, 1024, 1024, 1024, "float32", variant)
     torch.testing.assert_close(c, ref, rtol=RTOL, atol=ATOL)
@@ -146,14 +146,17 @@ def test_gemm_full_size_repeatable(dev, shape):
         for _ in range(2):
             assert torch.equal(first, torch.ops.mi355.gemm_nt(a, b, "float32", variant)), names[variant]
         torch.testing.assert_close(first, generic, rtol=1e-3, atol=1e-3)
-        if names[variant].startswith("staged"):
+        if names[variant].startswith(("staged", "stream")):
             by_name[names[variant]] = first
         del first
     # the tail split hands the last tile columns to a second kernel that adds K in the same order: the whole
     # matrix equals the unsplit staged kernel's bit for bit
     # and so does the same kernel launched with one workgroup per CU, walking its tiles as one slab sequence
-    staged = [v for k, v in sorted(by_name.items())]
+    staged = [v for k, v in sorted(by_name.items()) if k.startswith("staged")]
     assert len(staged) == 3 and torch.equal(staged[0], staged[1]) and torch.equal(staged[0], staged[2])
+    # likewise the streamed kernel and its tail-split launch
+    streamed = [v for k, v in sorted(by_name.items()) if k.startswith("stream")]
+    assert len(streamed) == 2 and torch.equal(streamed[0], streamed[1])
 
 
 @pytest.mark.parametrize("shape", [(4096, 4608, 192), (4352, 4352, 128), (8192, 8704, 320), (512, 256, 4096)])
@@ -227,24 +230,58 @@ def test_gemm_staged_slab_rotation(dev, shape, out_dtype):
 
 
 @pytest.mark.parametrize("out_dtype", ["float16", "float32"])
-@pytest.mark.parametrize("shape", [(2048, 10240, 512), (10240, 2048, 256), (768, 23296, 256), (2048, 8448, 256)])
-def test_gemm_tail_split(dev, shape, out_dtype):
-    """The staged kernel with its sparse last round handed to the 128x128 kernel: a strip of tile columns
-    (2048 x 10240: 64 of 320 tiles), a strip of tile rows (10240 x 2048), a remainder that is neither (runs
-    unsplit) and the smallest strip (one tile column after a full round of 8 x 32) -- bit-identical to the
-    unsplit staged kernel (both accumulate K in the same order), whole matrix against the generic kernel."""
+@pytest.mark.parametrize("shape", [(256, 256, 256), (512, 768, 384), (1024, 512, 1152), (2048, 10240, 512), (4352, 4352, 640)])
+def test_gemm_stream_slab_rotation(dev, shape, out_dtype):
+    """The streamed kernel keeps B in three rotating LDS buffers and A in two, with loads two slabs ahead of the reads:
+    the minimum of four slabs, slab counts that are 2 and 0 mod 4 and 0, 1 and 2 mod 3 (4, 6, 18, 8, 10: the loop is
+    written for pairs, the B buffers rotate in threes), a ragged tile grid and grids larger than the chip -- whole
+    matrix against the independent generic kernel, rows against fp32, launches repeat bit for bit."""
     import iree_turbine_amd as ita
     from oracle import inputs
 
     M, N, K = shape
-    announce(f"gemm tail split {shape} {out_dtype}")
+    announce(f"gemm streamed {shape} {out_dtype}")
     names = ita._lib.variants("gemm_f16_nt")
-    v = next(i for i, n in enumerate(names) if "tail" in n)
-    staged = next(i for i, n in enumerate(names) if n.startswith("staged") and "tail" not in n)
+    v = names.index("stream_256x256x64_w2x2")
+    a, b = [t.to(dev) for t in inputs.gemm_inputs(M, N, K)]
+    got = torch.ops.mi355.gemm_nt(a, b, out_dtype, v)
+    ref = torch.ops.mi355.gemm_nt(a, b, out_dtype, len(names) - 1)
+    torch.testing.assert_close(got.float(), ref.float(), rtol=1e-3, atol=1e-3)
+    rows = torch.tensor([0, 127, 128, M - 1])
+    exact = a[rows.to(dev)].float() @ b.float().t()
+    torch.testing.assert_close(got[rows.to(dev)].float(), exact, rtol=RTOL, atol=ATOL)
+    assert torch.equal(got, torch.ops.mi355.gemm_nt(a, b, out_dtype, v))
+
+
+def test_gemm_stream_contract(dev):
+    import iree_turbine_amd as ita
+
+    names = ita._lib.variants("gemm_f16_nt")
+    v = names.index("stream_256x256x64_w2x2")
+    a = torch.zeros(256, 192, dtype=torch.float16, device=dev)
+    with pytest.raises(ValueError):
+        torch.ops.mi355.gemm_nt(a, a, "float16", v)  # K = 192 is not a whole number of slab pairs
+
+
+@pytest.mark.parametrize("out_dtype", ["float16", "float32"])
+@pytest.mark.parametrize("shape", [(2048, 10240, 512), (10240, 2048, 256), (768, 23296, 256), (2048, 8448, 256)])
+@pytest.mark.parametrize("family", ["staged", "stream"])
+def test_gemm_tail_split(dev, shape, out_dtype, family):
+    """The staged / streamed kernel with its sparse last round handed to the 128x128 kernel: a strip of tile columns
+    (2048 x 10240: 64 of 320 tiles), a strip of tile rows (10240 x 2048), a remainder that is neither (runs
+    unsplit) and the smallest strip (one tile column after a full round of 8 x 32) -- bit-identical to the
+    unsplit kernel (both accumulate K in the same order), whole matrix against the generic kernel."""
+    import iree_turbine_amd as ita
+    from oracle import inputs
+
+    M, N, K = shape
+    announce(f"gemm tail split {family} {shape} {out_dtype}")
+    names = ita._lib.variants("gemm_f16_nt")
+    v = next(i for i, n in enumerate(names) if n.startswith(family) and "tail" in n)
+    staged = next(i for i, n in enumerate(names) if n.startswith(family) and "tail" not in n)
     a, b = [t.to(dev) for t in inputs.gemm_inputs(M, N, K)]
     got = torch.ops.mi355.gemm_nt(a, b, out_dtype, v)
     assert torch.equal(got, torch.ops.mi355.gemm_nt(a, b, out_dtype, staged))
-    assert torch.equal(got, torch.ops.mi355.gemm_nt(a, b, out_dtype, -1))
     ref = torch.ops.mi355.gemm_nt(a, b, out_dtype, len(names) - 1)
     torch.testing.assert_close(got.float(), ref.float(), rtol=1e-3, atol=1e-3)
     rows = torch.tensor([0, 255, M - 256, M - 1])
@@ -307,8 +344,8 @@ def test_gemm_output_beyond_4_gib(dev):
     b = (torch.randn(N, K, generator=gen) * 0.1).half().to(dev)
     rows = torch.tensor([0, 1000, 43690, 43691, M - 257, M - 1], device=dev)
     ref = a[rows].float() @ b.float().t()
-    tail = next(i for i, n in enumerate(names) if "tail" in n)
-    for variant in (-1, tail, 0, 4, len(names) - 1):
+    tails = [i for i, n in enumerate(names) if "tail" in n]
+    for variant in (-1, *tails, 0, 4, len(names) - 1):
         announce(f"gemm {M}x{N}x{K} float16 variant={variant} (C beyond 4 GiB)")
         c = torch.ops.mi355.gemm_nt(a, b, "float16", variant)
         torch.testing.assert_close(c[rows].float(), ref, rtol=RTOL, atol=ATOL)
