@@ -395,7 +395,7 @@ def wl_mfma_regloop(kind: str, data: str):
         opsd = ops.to(dev)
         workgroups, trips = (256, 1024) if kind.endswith("walk") else (512, 2000)  # one (512 registers per wave) or two workgroups of four waves per CU
         sink = torch.empty(workgroups * 256, dtype=torch.float32, device=dev)
-        code = {"f16": 0, "f16x16": 3, "f16walk": 4, "f16x16walk": 5}.get(kind, 1 if data == "zeros" else 2)
+        code = {"f16": 0, "f16x16": 3, "f16walk": 4, "f16x16walk": 5, "fp4walk": 6, "fp4x16walk": 7}.get(kind, 1 if data == "zeros" else 2)
         flop = ctypes.c_double(0.0)
         lib = _lib.load()
 
@@ -407,12 +407,14 @@ def wl_mfma_regloop(kind: str, data: str):
         torch.cuda.synchronize()
         return {
             "fn": fn, "work": flop.value, "bytes": 0.0, "flops": flop.value, "bound": "mfma",
-            "peak": PEAK_F16_TFLOPS if kind != "fp4" else PEAK_FP4_TFLOPS, "unit": "TFLOP/s",
-            "dtype": "f16" if kind != "fp4" else "fp4(e2m1)+e8m0", "cpu": lambda: None,
+            "peak": PEAK_F16_TFLOPS if not kind.startswith("fp4") else PEAK_FP4_TFLOPS, "unit": "TFLOP/s",
+            "dtype": "f16" if not kind.startswith("fp4") else "fp4(e2m1)+e8m0", "cpu": lambda: None,
             "config": {"workload": f"mfma_{kind}_regloop_{data}", "workgroups": workgroups, "trips": trips,
                        "instruction": {"f16": "v_mfma_f32_32x32x16_f16", "f16x16": "v_mfma_f32_16x16x32_f16",
                                        "f16walk": "v_mfma_f32_32x32x16_f16, 256 accumulators wandering around zero",
-                                       "f16x16walk": "v_mfma_f32_16x16x32_f16, 256 accumulators wandering around zero"}.get(
+                                       "f16x16walk": "v_mfma_f32_16x16x32_f16, 256 accumulators wandering around zero",
+                                       "fp4walk": "v_mfma_scale_f32_32x32x64_f8f6f4 (fp4 x fp4), 256 accumulators wandering around zero",
+                                       "fp4x16walk": "v_mfma_scale_f32_16x16x128_f8f6f4 (fp4 x fp4), 256 accumulators wandering around zero"}.get(
                            kind, "v_mfma_scale_f32_32x32x64_f8f6f4 (fp4 x fp4)")},
         }
     return build
@@ -467,6 +469,10 @@ CALIBRATION = {  # not part of the path: run only when named with --workload
     "mfma_f16walk_regloop_benchmark": wl_mfma_regloop("f16walk", "benchmark"),
     "mfma_f16x16walk_regloop_zeros": wl_mfma_regloop("f16x16walk", "zeros"),
     "mfma_f16x16walk_regloop_benchmark": wl_mfma_regloop("f16x16walk", "benchmark"),
+    "mfma_fp4walk_regloop_zeros": wl_mfma_regloop("fp4walk", "zeros"),
+    "mfma_fp4walk_regloop_benchmark": wl_mfma_regloop("fp4walk", "benchmark"),
+    "mfma_fp4x16walk_regloop_zeros": wl_mfma_regloop("fp4x16walk", "zeros"),
+    "mfma_fp4x16walk_regloop_benchmark": wl_mfma_regloop("fp4x16walk", "benchmark"),
     "mfma_fp4_regloop_zeros": wl_mfma_regloop("fp4", "zeros"),
     "mfma_fp4_regloop_benchmark": wl_mfma_regloop("fp4", "benchmark"),
 }

@@ -155,16 +155,72 @@ __global__ __launch_bounds__(CAL_WAVES * 64) void calibrate_mfma_fp4_kernel(cons
   sink[t] = s;
 }
 
+// The GEMM-like loop for the scaled fp4 MFMAs: 256 accumulators, eight A and eight B operand registers (16 bytes of
+// codes per lane) with E8M0 scales spread over 2^-8 .. 2^7, rotated over the trips.  fp4 has no exact negation by
+// sign flip of a register here (the codes are sign-magnitude nibbles: XOR 0x88888888 flips every sign), so the
+// negated A operands are that XOR.  WIDE = false: 16 MFMAs 32x32x64 per trip; true: 64 MFMAs 16x16x128.
+template <bool WIDE>
+__global__ __launch_bounds__(CAL_WAVES * 64) void calibrate_mfma_fp4_walk_kernel(const intx4* __restrict__ operands, unsigned mask,
+                                                                                 float* __restrict__ sink, int trips) {
+  const unsigned t = threadIdx.x + blockIdx.x * blockDim.x;
+  intx8 a[16], b[8];
+  int sa[8], sb[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const intx4 x = operands[(t * 16 + i) & mask], y = operands[(t * 16 + 8 + i) & mask];
+    a[i] = intx8{x[0], x[1], x[2], x[3], 0, 0, 0, 0};
+    a[8 + i] = intx8{x[0] ^ (int)0x88888888, x[1] ^ (int)0x88888888, x[2] ^ (int)0x88888888, x[3] ^ (int)0x88888888, 0, 0, 0, 0};
+    b[i] = intx8{y[0], y[1], y[2], y[3], 0, 0, 0, 0};
+    sa[i] = 119 + ((x[0] >> 3) & 15);
+    sb[i] = 119 + ((y[1] >> 5) & 15);
+  }
+#pragma unroll
+  for (int i = 0; i < 8; i++) asm volatile("" : "+v"(a[8 + i]));
+  constexpr int R = WIDE ? 8 : 4;
+  typedef typename std::conditional<WIDE, floatx4, floatx16>::type acc_t;
+  acc_t c[R][R];
+#pragma unroll
+  for (int i = 0; i < R; i++)
+#pragma unroll
+    for (int j = 0; j < R; j++)
+#pragma unroll
+      for (int r = 0; r < (WIDE ? 4 : 16); r++) c[i][j][r] = 0.f;
+#pragma unroll 1
+  for (int it = 0; it < trips; it += 16) {
+#pragma unroll
+    for (int tt = 0; tt < 16; tt++) {
+#pragma unroll
+      for (int i = 0; i < R; i++)
+#pragma unroll
+        for (int j = 0; j < R; j++) {
+          const int ai = (j + tt) & 7, bi = (i + 3 * tt) & 7;
+          const intx8 av = a[ai + (tt >= 8 ? 8 : 0)], bv = b[bi];
+          if constexpr (WIDE) c[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bv, av, c[i][j], 4, 4, 0, sb[bi], 0, sa[ai]);
+          else c[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bv, av, c[i][j], 4, 4, 0, sb[bi], 0, sa[ai]);
+        }
+    }
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < R; i++)
+#pragma unroll
+    for (int j = 0; j < R; j++)
+#pragma unroll
+      for (int r = 0; r < (WIDE ? 4 : 16); r++) s += c[i][j][r];
+  sink[t] = s;
+}
+
 }  // namespace mi355
 
 using namespace mi355;
 
 // kind 0: fp16 32x32x16; kind 1: fp4 32x32x64 with unit scales; kind 2: fp4 with spread scales; kind 3: fp16 16x16x32;
-// kinds 4 / 5: the GEMM-like loops with 32x32x16 / 16x16x32 (trips rounded down to a multiple of 16).
+// kinds 4 / 5: the GEMM-like loops with 32x32x16 / 16x16x32 (trips rounded down to a multiple of 16); kinds 6 / 7: the
+// GEMM-like loops with fp4 32x32x64 / 16x16x128.
 extern "C" int mi355_calibrate_mfma(int kind, const void* operands, int64_t operand_bytes, float* sink, int64_t sink_floats,
                                     int64_t workgroups, int64_t trips, double* flop_per_launch, void* stream) {
   if (!operands || !sink) return fail(-MI355_E_NULL, "calibrate_mfma: null pointer");
-  if (kind < 0 || kind > 5) return fail(-MI355_E_DTYPE, "calibrate_mfma: kind %d unknown (0 fp16 32x32x16, 1 fp4, 2 fp4 with spread scales, 3 fp16 16x16x32, 4 / 5 GEMM-like 32x32x16 / 16x16x32)", kind);
+  if (kind < 0 || kind > 7) return fail(-MI355_E_DTYPE, "calibrate_mfma: kind %d unknown (0 fp16 32x32x16, 1 fp4, 2 fp4 with spread scales, 3 fp16 16x16x32, 4 / 5 GEMM-like 32x32x16 / 16x16x32, 6 / 7 GEMM-like fp4 32x32x64 / 16x16x128)", kind);
   if (operand_bytes < 16 || (operand_bytes & (operand_bytes - 1)) || operand_bytes > (1ll << 30))
     return fail(-MI355_E_SHAPE, "calibrate_mfma: operand_bytes %lld must be a power of two in [16, 2^30]", (long long)operand_bytes);
   if (workgroups <= 0 || workgroups > 65535 || trips <= 0 || trips > (1 << 24))
@@ -179,8 +235,13 @@ extern "C" int mi355_calibrate_mfma(int kind, const void* operands, int64_t oper
   if (kind >= 4) {
     trips &= ~15ll;
     if (trips <= 0) return fail(-MI355_E_SHAPE, "calibrate_mfma: the GEMM-like loops need trips >= 16");
-    if (flop_per_launch) *flop_per_launch = 2.0 * 32 * 32 * 16 * (kind == 4 ? 16 : 32) * (double)trips * CAL_WAVES * (double)workgroups;
-    if (kind == 4)
+    if (flop_per_launch) *flop_per_launch = 2.0 * 32 * 32 * 16 * ((kind & 1) ? 32 : 16) * (double)trips * CAL_WAVES * (double)workgroups;
+    if (kind >= 6 && flop_per_launch) *flop_per_launch *= 4.0;  // four times the depth per MFMA
+    if (kind == 6)
+      hipLaunchKernelGGL(calibrate_mfma_fp4_walk_kernel<false>, grid, block, 0, s, (const intx4*)operands, mask, sink, (int)trips);
+    else if (kind == 7)
+      hipLaunchKernelGGL(calibrate_mfma_fp4_walk_kernel<true>, grid, block, 0, s, (const intx4*)operands, mask, sink, (int)trips);
+    else if (kind == 4)
       hipLaunchKernelGGL(calibrate_mfma_f16_walk_kernel<false>, grid, block, 0, s, (const half8*)operands, mask, sink, (int)trips);
     else
       hipLaunchKernelGGL(calibrate_mfma_f16_walk_kernel<true>, grid, block, 0, s, (const half8*)operands, mask, sink, (int)trips);

@@ -690,21 +690,36 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_stream(const half_t* __restri
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm = wave / WN, wn = wave % WN;
+  // The workgroup walks tiles blockIdx.x, blockIdx.x + gridDim.x, ... as ONE slab sequence (launched with one workgroup
+  // per tile it runs just that tile): loads for slabs past a tile's end fetch the next tile's first slabs, so only a
+  // workgroup's first tile pays the pipeline fill, and a tile's stores drain under the next tile's MFMAs.
+  const int T = tiles_m * tiles_n, G = (int)gridDim.x;
+  int pid = blockIdx.x;
   int tile_m, tile_n;
-  map_tile(blockIdx.x, tiles_m, tiles_n, group_m, tile_m, tile_n);
+  map_tile(pid, tiles_m, tiles_n, group_m, tile_m, tile_n);
 
   // global side: a wave-load covers 8 rows x 128 bytes; wave w loads rows 128 h + 32 blk + 8 w .. + 7 of either operand.
   // lane = (row l >> 3, slot l & 7) fetches chunk slot ^ ((row >> 1) & 7): the row's 8-row group index 16 h + 4 blk + w
   // has the parity of w
+  // One descriptor per operand covers all of it (under 4 GiB, checked on the host); the tile, the slab and the row block
+  // go into the scalar offset, so that moving on to the next tile changes one scalar.
   const unsigned row_bytes = (unsigned)K * 2u;
-  const buffer_rsrc_t a_src = make_buffer(A + (size_t)(tile_m * BM + wave * 8) * K, (unsigned)(BM - wave * 8) * row_bytes);
-  const buffer_rsrc_t b_src = make_buffer(B + (size_t)(tile_n * BN + wave * 8) * K, (unsigned)(BN - wave * 8) * row_bytes);
+  const buffer_rsrc_t a_src = make_buffer(A, (unsigned)(tiles_m * BM) * row_bytes);
+  const buffer_rsrc_t b_src = make_buffer(B, (unsigned)(tiles_n * BN) * row_bytes);
   const int lrow = lane >> 3;
-  const unsigned g_off = (unsigned)lrow * row_bytes + (unsigned)((lane & 7) ^ (((wave & 1) << 2) | (lrow >> 1))) * 16u;
+  const unsigned g_off = (unsigned)(wave * 8 + lrow) * row_bytes + (unsigned)((lane & 7) ^ (((wave & 1) << 2) | (lrow >> 1))) * 16u;
   const int KT = K / 64;  // even, >= 4 (checked on the host)
-  // rows 128 h + 32 blk (+ 8 wave) of slab `slab` of operand X into the buffer at byte offset buf_at
-  auto load = [&](bool is_a, int buf_at, int h, int blk, int slab) {
-    const unsigned so = (unsigned)(h * 128 + blk * 32) * row_bytes + (unsigned)(slab < KT ? slab : KT - 1) * 128u;
+  unsigned a_cur = (unsigned)(tile_m * BM) * row_bytes, b_cur = (unsigned)(tile_n * BN) * row_bytes;  // this tile's rows
+  unsigned a_nxt = a_cur, b_nxt = b_cur;  // the next tile's (after the last tile: its own again; those loads are never used)
+  // byte offset of slab kt + d of the walk: past this tile's end it is a slab of the next tile
+  auto slab_at = [&](int s, unsigned cur, unsigned nxt) { return s < KT ? cur + (unsigned)s * 128u : nxt + (unsigned)(s - KT) * 128u; };
+  // offsets of the slabs 1, 2 (A) and 3, 4 (B) ahead of the current one; those of the next slab are worked out one per
+  // step in the second half of a slab (scalar instructions bunched at a slab's start would hold up its first MFMAs)
+  unsigned a_off1 = a_cur + 128u, a_off2 = a_cur + 256u, b_off3 = b_cur + 384u, b_off4 = b_cur + 512u;
+  unsigned n_a1 = 0, n_a2 = 0, n_b3 = 0, n_b4 = 0;
+  // rows 128 h + 32 blk (+ 8 wave) of the slab at byte offset `at` of operand X into the buffer at byte offset buf_at
+  auto load = [&](bool is_a, int buf_at, int h, int blk, unsigned at) {
+    const unsigned so = (unsigned)(h * 128 + blk * 32) * row_bytes + at;
     buffer_load_lds_16B(is_a ? a_src : b_src, g_off, so, lds + buf_at + (h * 16 + blk * 4 + wave) * 1024);
   };
 
@@ -720,11 +735,10 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_stream(const half_t* __restri
   const unsigned b_lane = lds0 + B_AT + wn * (WTN * 128) + lane_rd;
   unsigned baddr[2];  // [k half], of the B buffer being read in this slab
 
-  floatx4 acc[8][8];  // [n block][m block]
-#pragma unroll
-  for (int i = 0; i < 8; i++)
-#pragma unroll
-    for (int j = 0; j < 8; j++) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+  // [n block][m block].  Never cleared: the first MFMA of a tile on each accumulator (slab 0, k half 0) takes a zero
+  // addend instead -- a register write in front of an inline-assembly MFMA would need wait states the compiler does not
+  // know to insert.
+  floatx4 acc[8][8];
   half8 fb0[2][8], fb1[2][8], fa[8];
 
   // MFMAs as inline assembly with the accumulators pinned to AGPRs: with 64 four-register accumulators the compiler's
@@ -735,22 +749,34 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_stream(const half_t* __restri
     if constexpr (BF) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(x), "v"(y));       \
     else asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(x), "v"(y));                     \
   } while (0)
+#define MI355_SM_ACC(ZERO, c, x, y)   \
+  do {                                \
+    if constexpr (ZERO) MI355_SM_MFMA0(c, x, y); \
+    else MI355_SM_MFMA(c, x, y);      \
+  } while (0)
+#define MI355_SM_MFMA0(c, x, y)                                                                                 \
+  do {                                                                                                          \
+    if constexpr (BF) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=a"(c) : "v"(x), "v"(y));        \
+    else asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=a"(c) : "v"(x), "v"(y));                      \
+  } while (0)
 #define MI355_SM_READ(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off))
 #define MI355_SM_TIE8(X) "+v"(X[0]), "+v"(X[1]), "+v"(X[2]), "+v"(X[3]), "+v"(X[4]), "+v"(X[5]), "+v"(X[6]), "+v"(X[7])
 
   // ---- prologue: B0, A0, B1, A1 blocks 0..2, B2 ----
 #pragma unroll
-  for (int x = 0; x < 8; x++) load(false, B_AT, x & 1, x >> 1, 0);
+  for (int x = 0; x < 8; x++) load(false, B_AT, x & 1, x >> 1, b_cur);
 #pragma unroll
-  for (int x = 0; x < 8; x++) load(true, A_AT, x & 1, x >> 1, 0);
+  for (int x = 0; x < 8; x++) load(true, A_AT, x & 1, x >> 1, a_cur);
 #pragma unroll
-  for (int x = 0; x < 8; x++) load(false, B_AT + BUF, x & 1, x >> 1, 1);
+  for (int x = 0; x < 8; x++) load(false, B_AT + BUF, x & 1, x >> 1, b_cur + 128u);
 #pragma unroll
-  for (int x = 0; x < 6; x++) load(true, A_AT + BUF, x & 1, x >> 1, 1);
+  for (int x = 0; x < 6; x++) load(true, A_AT + BUF, x & 1, x >> 1, a_cur + 128u);
 #pragma unroll
-  for (int x = 0; x < 8; x++) load(false, B_AT + 2 * BUF, x & 1, x >> 1, 2);
+  for (int x = 0; x < 8; x++) load(false, B_AT + 2 * BUF, x & 1, x >> 1, b_cur + 256u);
   __builtin_amdgcn_sched_barrier(0);
-  asm volatile("s_waitcnt vmcnt(14)" ::: "memory");  // B0, A0, B1 have landed
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // everything has landed: a tile starts with all loads but those of the interval before it complete (later tiles: the
+  // wait in the middle of the epilogue), and its first slab runs without load waits
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_sched_barrier(0);
   baddr[0] = b_lane;
@@ -768,8 +794,8 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_stream(const half_t* __restri
   asm volatile("s_waitcnt lgkmcnt(0)" : MI355_SM_TIE8(fb0[0]), MI355_SM_TIE8(fb0[1]), "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]));
   __builtin_amdgcn_s_barrier();  // every wave has read B0: its buffer may receive slab 3
   __builtin_amdgcn_sched_barrier(0);
-  load(false, B_AT, 0, 0, 3);
-  load(false, B_AT, 1, 0, 3);
+  load(false, B_AT, 0, 0, b_cur + 384u);
+  load(false, B_AT, 1, 0, b_cur + 384u);
   __builtin_amdgcn_sched_barrier(0);
 
   // B buffer rotation: slab t lives in buffer t % 3
@@ -778,136 +804,184 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_stream(const half_t* __restri
 
   // Step s of a slab whose A buffer is PAR: MFMAs of (m block s / 2, k half s % 2) on fa[s % 8] against FB[s % 2][0..7].
   // LGKM = LDS reads issued after the read that filled fa[s % 8] (they may still be in flight).
-#define MI355_SM_STEP(s, PAR, FB, FBN, LGKM)                                                                               \
+#define MI355_SM_STEP(s, PAR, FB, FBN, LGKM, FIRST)                                                                              \
   do {                                                                                                                     \
     constexpr int s4 = (s) + 4, nb = s4 >= 16 ? 1 - (PAR) : (PAR), ns = s4 & 15;                                           \
     asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(fa[(s)&7]) : "n"(LGKM));                                                   \
     __builtin_amdgcn_sched_barrier(0);                                                                                     \
-    MI355_SM_MFMA(acc[0][(s) >> 1], FB[(s)&1][0], fa[(s)&7]);                                      \
+    MI355_SM_ACC(FIRST && !((s)&1), acc[0][(s) >> 1], FB[(s)&1][0], fa[(s)&7]);                                      \
     MI355_SM_READ(fa[s4 & 7], aaddr[nb][ns & 1], (ns >> 1) * 2048);                                                        \
     __builtin_amdgcn_sched_barrier(0);                                                                                     \
-    MI355_SM_MFMA(acc[1][(s) >> 1], FB[(s)&1][1], fa[(s)&7]);                                      \
+    MI355_SM_ACC(FIRST && !((s)&1), acc[1][(s) >> 1], FB[(s)&1][1], fa[(s)&7]);                                      \
     if constexpr ((s) < 8) MI355_SM_READ(FBN[(s) >> 2][(2 * (s)) & 7], baddr[(s) >> 2], ((2 * (s)) & 7) * 2048);           \
     __builtin_amdgcn_sched_barrier(0);                                                                                     \
-    MI355_SM_MFMA(acc[2][(s) >> 1], FB[(s)&1][2], fa[(s)&7]);                                      \
-    MI355_SM_MFMA(acc[3][(s) >> 1], FB[(s)&1][3], fa[(s)&7]);                                      \
+    MI355_SM_ACC(FIRST && !((s)&1), acc[2][(s) >> 1], FB[(s)&1][2], fa[(s)&7]);                                      \
+    MI355_SM_ACC(FIRST && !((s)&1), acc[3][(s) >> 1], FB[(s)&1][3], fa[(s)&7]);                                      \
     if constexpr ((s) < 8) MI355_SM_READ(FBN[(s) >> 2][(2 * (s) + 1) & 7], baddr[(s) >> 2], ((2 * (s) + 1) & 7) * 2048);   \
     __builtin_amdgcn_sched_barrier(0);                                                                                     \
-    MI355_SM_MFMA(acc[4][(s) >> 1], FB[(s)&1][4], fa[(s)&7]);                                      \
-    MI355_SM_MFMA(acc[5][(s) >> 1], FB[(s)&1][5], fa[(s)&7]);                                      \
+    MI355_SM_ACC(FIRST && !((s)&1), acc[4][(s) >> 1], FB[(s)&1][4], fa[(s)&7]);                                      \
+    MI355_SM_ACC(FIRST && !((s)&1), acc[5][(s) >> 1], FB[(s)&1][5], fa[(s)&7]);                                      \
     {                                                                                                                      \
       constexpr int q = (s) >> 2, x = (s)&3;                                                                               \
       if constexpr (x < 2) {                                                                                               \
-        if constexpr (q == 0) load(true, A_AT + (1 - (PAR)) * BUF, x, 3, kt + 1);                                          \
-        else load(true, A_AT + (PAR) * BUF, x, q - 1, kt + 2);                                                             \
+        if constexpr (q == 0) load(true, A_AT + (1 - (PAR)) * BUF, x, 3, a_off1);                                          \
+        else load(true, A_AT + (PAR) * BUF, x, q - 1, a_off2);                                                             \
       } else {                                                                                                             \
-        if constexpr (q == 3) load(false, B_AT + b_rd, x - 2, 0, kt + 4);                                                  \
-        else load(false, B_AT + b_ld012, x - 2, q + 1, kt + 3);                                                            \
+        if constexpr (q == 3) load(false, B_AT + b_rd, x - 2, 0, b_off4);                                                  \
+        else load(false, B_AT + b_ld012, x - 2, q + 1, b_off3);                                                            \
       }                                                                                                                    \
     }                                                                                                                      \
     __builtin_amdgcn_sched_barrier(0);                                                                                     \
-    MI355_SM_MFMA(acc[6][(s) >> 1], FB[(s)&1][6], fa[(s)&7]);                                      \
-    MI355_SM_MFMA(acc[7][(s) >> 1], FB[(s)&1][7], fa[(s)&7]);                                      \
+    if constexpr ((s) == 8) n_a1 = slab_at(kt + 2, a_cur, a_nxt);                                                          \
+    if constexpr ((s) == 9) n_a2 = slab_at(kt + 3, a_cur, a_nxt);                                                          \
+    if constexpr ((s) == 10) n_b3 = slab_at(kt + 4, b_cur, b_nxt);                                                         \
+    if constexpr ((s) == 11) n_b4 = slab_at(kt + 5, b_cur, b_nxt);                                                         \
+    MI355_SM_ACC(FIRST && !((s)&1), acc[6][(s) >> 1], FB[(s)&1][6], fa[(s)&7]);                                      \
+    MI355_SM_ACC(FIRST && !((s)&1), acc[7][(s) >> 1], FB[(s)&1][7], fa[(s)&7]);                                      \
     __builtin_amdgcn_sched_barrier(0);                                                                                     \
   } while (0)
   // End of an interval: loads older than one slab and LDS reads older than this interval are complete in every wave.
-#define MI355_SM_SYNC(RD)                                                        \
+#define MI355_SM_SYNC(RD, VM)                                                    \
   do {                                                                           \
-    asm volatile("s_waitcnt vmcnt(16) lgkmcnt(%0)" ::"n"(RD) : "memory");        \
+    if constexpr (VM) asm volatile("s_waitcnt vmcnt(16) lgkmcnt(%0)" ::"n"(RD) : "memory"); \
+    else asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(RD) : "memory");             \
     __builtin_amdgcn_s_barrier();                                                \
     __builtin_amdgcn_sched_barrier(0);                                           \
   } while (0)
   // Reads issued in one step: 3 in the first half of a slab (A, B, B), 1 in the second.  The read that fills fa for
   // step s was the first read of step s - 4.
-#define MI355_SM_SLAB(PAR, FB, FBN)                                                                             \
+#define MI355_SM_SLAB(PAR, FB, FBN, VM, FIRST)                                                                            \
   do {                                                                                                          \
     baddr[0] = b_lane + (unsigned)b_rd;                                                                         \
     baddr[1] = baddr[0] ^ 64;                                                                                   \
-    MI355_SM_STEP(0, PAR, FB, FBN, 3);  /* steps 12..15 of the slab before: one read each */                    \
-    MI355_SM_STEP(1, PAR, FB, FBN, 5);                                                                          \
-    MI355_SM_STEP(2, PAR, FB, FBN, 7);                                                                          \
-    MI355_SM_STEP(3, PAR, FB, FBN, 9);                                                                          \
-    MI355_SM_SYNC(12);                                                                                          \
-    MI355_SM_STEP(4, PAR, FB, FBN, 11);                                                                         \
-    MI355_SM_STEP(5, PAR, FB, FBN, 11);                                                                         \
-    MI355_SM_STEP(6, PAR, FB, FBN, 11);                                                                         \
-    MI355_SM_STEP(7, PAR, FB, FBN, 11);                                                                         \
-    MI355_SM_SYNC(12);                                                                                          \
-    MI355_SM_STEP(8, PAR, FB, FBN, 11);                                                                         \
-    MI355_SM_STEP(9, PAR, FB, FBN, 9);                                                                          \
-    MI355_SM_STEP(10, PAR, FB, FBN, 7);                                                                         \
-    MI355_SM_STEP(11, PAR, FB, FBN, 5);                                                                         \
-    MI355_SM_SYNC(4);                                                                                           \
-    MI355_SM_STEP(12, PAR, FB, FBN, 3);                                                                         \
-    MI355_SM_STEP(13, PAR, FB, FBN, 3);                                                                         \
-    MI355_SM_STEP(14, PAR, FB, FBN, 3);                                                                         \
-    MI355_SM_STEP(15, PAR, FB, FBN, 3);                                                                         \
+    MI355_SM_STEP(0, PAR, FB, FBN, 3, FIRST);  /* steps 12..15 of the slab before: one read each */                    \
+    MI355_SM_STEP(1, PAR, FB, FBN, 5, FIRST);                                                                          \
+    MI355_SM_STEP(2, PAR, FB, FBN, 7, FIRST);                                                                          \
+    MI355_SM_STEP(3, PAR, FB, FBN, 9, FIRST);                                                                          \
+    MI355_SM_SYNC(12, VM);                                                                                        \
+    MI355_SM_STEP(4, PAR, FB, FBN, 11, FIRST);                                                                         \
+    MI355_SM_STEP(5, PAR, FB, FBN, 11, FIRST);                                                                         \
+    MI355_SM_STEP(6, PAR, FB, FBN, 11, FIRST);                                                                         \
+    MI355_SM_STEP(7, PAR, FB, FBN, 11, FIRST);                                                                         \
+    MI355_SM_SYNC(12, VM);                                                                                        \
+    MI355_SM_STEP(8, PAR, FB, FBN, 11, FIRST);                                                                         \
+    MI355_SM_STEP(9, PAR, FB, FBN, 9, FIRST);                                                                          \
+    MI355_SM_STEP(10, PAR, FB, FBN, 7, FIRST);                                                                         \
+    MI355_SM_STEP(11, PAR, FB, FBN, 5, FIRST);                                                                         \
+    MI355_SM_SYNC(4, VM);                                                                                        \
+    MI355_SM_STEP(12, PAR, FB, FBN, 3, FIRST);                                                                         \
+    MI355_SM_STEP(13, PAR, FB, FBN, 3, FIRST);                                                                         \
+    MI355_SM_STEP(14, PAR, FB, FBN, 3, FIRST);                                                                         \
+    MI355_SM_STEP(15, PAR, FB, FBN, 3, FIRST);                                                                         \
     /* the B fragments of the next slab were all requested in steps 0..7: they have landed; tie them to this point */ \
-    asm volatile("s_waitcnt vmcnt(16) lgkmcnt(4)" : MI355_SM_TIE8(FBN[0]), MI355_SM_TIE8(FBN[1])::"memory");    \
+    if constexpr (VM) asm volatile("s_waitcnt vmcnt(16) lgkmcnt(4)" : MI355_SM_TIE8(FBN[0]), MI355_SM_TIE8(FBN[1])::"memory"); \
+    else asm volatile("s_waitcnt lgkmcnt(4)" : MI355_SM_TIE8(FBN[0]), MI355_SM_TIE8(FBN[1])::"memory");         \
     __builtin_amdgcn_s_barrier();                                                                               \
     __builtin_amdgcn_sched_barrier(0);                                                                          \
+    a_off1 = n_a1;                                                                                              \
+    a_off2 = n_a2;                                                                                              \
+    b_off3 = n_b3;                                                                                              \
+    b_off4 = n_b4;                                                                                              \
     b_ld012 = b_rd;                                                                                             \
     b_rd = b_rd == 2 * BUF ? 0 : b_rd + BUF;                                                                    \
   } while (0)
 
-  for (int kt = 0; kt < KT; kt += 2) {
-    MI355_SM_SLAB(0, fb0, fb1);
-    kt++;
-    MI355_SM_SLAB(1, fb1, fb0);
-    kt--;
+  for (; pid < T; pid += G) {
+    int nxt_m = tile_m, nxt_n = tile_n;
+    if (pid + G < T) map_tile(pid + G, tiles_m, tiles_n, group_m, nxt_m, nxt_n);
+    a_nxt = (unsigned)(nxt_m * BM) * row_bytes;
+    b_nxt = (unsigned)(nxt_n * BN) * row_bytes;
+    int kt = 0;
+    MI355_SM_SLAB(0, fb0, fb1, false, true);  // everything its reads need landed before the tile began
+    kt = 1;
+    MI355_SM_SLAB(1, fb1, fb0, true, false);
+    for (kt = 2; kt < KT; kt += 2) {
+      MI355_SM_SLAB(0, fb0, fb1, true, false);
+      kt++;
+      MI355_SM_SLAB(1, fb1, fb0, true, false);
+      kt--;
+    }
+    // ---- epilogue ----
+    // The MFMAs are inline assembly, so the compiler does not know that the accumulators were written just now: the
+    // wait states an MFMA result needs before another instruction may read it are spelled out, and every accumulator is
+    // tied to a statement behind them so that no read of it can be scheduled earlier.
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+      asm volatile("" : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]), "+a"(acc[i][4]), "+a"(acc[i][5]),
+                        "+a"(acc[i][6]), "+a"(acc[i][7]));
+    // lane holds, for m = 16 j + (l & 15): n = 16 i + 4 (l >> 4) + r, r < 4.  The addresses come from a lane id the
+    // compiler cannot see through, so that none of them is computed ahead of the K loop and kept across it.
+    const int le = opaque_lane_id();
+    const int r16e = le & 15, cqe = le >> 4;
+    if constexpr (sizeof(OutT) == 2) {
+      // 16-bit results go through LDS, one m block (16 rows x 128 columns = 4 KiB) per pass in a wave-private region:
+      // 8-byte writes of 4 consecutive n (chunk slot c ^ ((m >> 1) & 7) within each 128-byte half row), whole rows read
+      // back 16 bytes per lane and stored as full cache lines.  LDS operations of a wave execute in order, so the passes
+      // need no waits between them.  The next tile's slabs are landing in LDS meanwhile; free at this point are parts
+      // 1..3 of the B buffer whose part 0 was loaded in the interval before (rows 32..127 of either half: twice 12 KiB),
+      // which the next loads reach only after the barrier below.
+      // These LDS accesses are inline assembly like the K loop's: a direct-to-LDS load is in flight at this point, and
+      // the compiler would wait for all of them in front of an LDS access it can see.
+      const unsigned ep = lds0 + (unsigned)(B_AT + b_ld012 + (wave < 3 ? 4096 + wave * 4096 : 16 * 1024 + 4096));
+      const int er = le >> 4, ec = le & 15, sw = (r16e >> 1) & 7;
+      // write: row r16e, chunk (2 i + (cqe >> 1)) ^ sw, 8-byte half cqe & 1; the chunk's i term is an XOR of the address
+      const unsigned wa = ep + (unsigned)(r16e * 256 + ((((cqe >> 1) ^ (sw & 1)) | (sw & 6)) * 16) + 8 * (cqe & 1));
+      // read: row 4 it + er, chunk ec ^ ((row >> 1) & 7) = (ec ^ (er >> 1)) ^ 2 it
+      const unsigned ra = ep + (unsigned)(er * 256 + ((ec ^ (er >> 1)) * 16));
+      OutT* cbase = C + (size_t)(tile_m * BM + wm * WTM + er) * N + tile_n * BN + wn * WTN + ec * 8;
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+          half4 v = {cvt16<BF>(acc[i][j][0]), cvt16<BF>(acc[i][j][1]), cvt16<BF>(acc[i][j][2]), cvt16<BF>(acc[i][j][3])};
+          asm volatile("ds_write_b64 %0, %1" ::"v"(wa ^ (unsigned)(32 * i)), "v"(v) : "memory");
+        }
+        half8 rv[4];
+        asm volatile("ds_read_b128 %0, %1" : "=v"(rv[0]) : "v"(ra));
+        asm volatile("ds_read_b128 %0, %1 offset:1024" : "=v"(rv[1]) : "v"(ra ^ 32u));
+        asm volatile("ds_read_b128 %0, %1 offset:2048" : "=v"(rv[2]) : "v"(ra ^ 64u));
+        asm volatile("ds_read_b128 %0, %1 offset:3072" : "=v"(rv[3]) : "v"(ra ^ 96u));
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(rv[0]), "+v"(rv[1]), "+v"(rv[2]), "+v"(rv[3]));
+#pragma unroll
+        for (int it = 0; it < 4; it++) *reinterpret_cast<half8*>(cbase + (size_t)(j * 16 + it * 4) * N) = rv[it];
+        if (j == 3) {
+          // Half of the stores are out.  The next tile's first slab runs without load waits: everything it and the
+          // first interval after it read was loaded before this tile's last interval, i.e. all but the 4 loads
+          // issued since -- which are followed in the queue by the 16 stores above.
+          asm volatile("s_waitcnt vmcnt(20)" ::: "memory");
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else {
+      OutT* crow = C + (size_t)(tile_m * BM + wm * WTM + r16e) * N + tile_n * BN + wn * WTN + 4 * cqe;
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+          OutPack<OutT, BF>::store4(crow + (size_t)(j * 16) * N + i * 16, acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
+        if (j == 3) asm volatile("s_waitcnt vmcnt(36)" ::: "memory");  // as above, behind 32 stores
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    a_cur = a_nxt;
+    b_cur = b_nxt;
+    tile_m = nxt_m;
+    tile_n = nxt_n;
+    // the waves leave the epilogue together: the first slab's reads rely on the wait above having been made by all
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
   }
-  // reads and loads issued for slabs past the end are never used, but they target registers and LDS the epilogue reuses
+  // the loads issued for a tile that does not exist still target LDS: let them land before the workgroup ends
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : MI355_SM_TIE8(fa));
-  __builtin_amdgcn_s_barrier();
-  __builtin_amdgcn_sched_barrier(0);
 #undef MI355_SM_SLAB
 #undef MI355_SM_SYNC
 #undef MI355_SM_STEP
 #undef MI355_SM_TIE8
 #undef MI355_SM_READ
+#undef MI355_SM_ACC
+#undef MI355_SM_MFMA0
 #undef MI355_SM_MFMA
-
-  // lane holds, for m = 16 j + (l & 15): n = 16 i + 4 (l >> 4) + r, r < 4.  The epilogue's addresses come from a lane id
-  // the compiler cannot see through, so that none of them is computed ahead of the K loop and kept across it.
-  const int le = opaque_lane_id();
-  const int r16e = le & 15, cqe = le >> 4;
-  if constexpr (sizeof(OutT) == 2) {
-    // 16-bit epilogue through LDS (every buffer is free now), one m block (16 rows x 128 columns) per pass in a
-    // wave-private region: 8-byte writes of 4 consecutive n (chunk slot c ^ ((m >> 1) & 7) within each 128-byte half
-    // row), whole rows read back 16 bytes per lane and stored as full cache lines.  LDS operations of a wave execute in
-    // order, so the passes need no waits between them.
-    constexpr int ROW_B = WTN * 2;
-    char* ep = lds + wave * (WTM * ROW_B);
-    const int er = le >> 4, ec = le & 15;
-    OutT* cbase = C + (size_t)(tile_m * BM + wm * WTM) * N + tile_n * BN + wn * WTN + ec * 8;
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-      const int ml = j * 16 + r16e;
-#pragma unroll
-      for (int i = 0; i < 8; i++) {
-        const int c = 2 * i + (cqe >> 1);
-        half4 v = {cvt16<BF>(acc[i][j][0]), cvt16<BF>(acc[i][j][1]), cvt16<BF>(acc[i][j][2]), cvt16<BF>(acc[i][j][3])};
-        *reinterpret_cast<half4*>(ep + ml * ROW_B + ((c ^ ((ml >> 1) & 7)) * 16) + 8 * (cqe & 1)) = v;
-      }
-#pragma unroll
-      for (int it = 0; it < 4; it++) {
-        const int row = j * 16 + it * 4 + er;
-        half8 v = *reinterpret_cast<const half8*>(ep + row * ROW_B + ((ec ^ ((row >> 1) & 7)) * 16));
-        *reinterpret_cast<half8*>(cbase + (size_t)row * N) = v;
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  } else {
-    const int m0 = tile_m * BM + wm * WTM + r16e;
-    const int n0 = tile_n * BN + wn * WTN + 4 * cqe;
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-      OutT* crow = C + (size_t)(m0 + j * 16) * N + n0;
-#pragma unroll
-      for (int i = 0; i < 8; i++)
-        OutPack<OutT, BF>::store4(crow + i * 16, acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
-    }
-  }
 }
 
 // Persistent kernel: one workgroup per CU walks its share of the output tiles (tile ids pid, pid + grid,
@@ -1315,6 +1389,7 @@ static const GemmVariant kGemmVariants[] = {
     {"staged_256x256x64_w2x2_walk", 256, 256, 256},
     {"stream_256x256x64_w2x2", 256, 256, 256},
     {"stream_256x256_tail_128x128", 256, 256, 256},
+    {"stream_256x256x64_w2x2_walk", 256, 256, 256},
     {"generic_64x64x32", 64, 64, 256},
 };
 constexpr int kNumGemmVariants = sizeof(kGemmVariants) / sizeof(kGemmVariants[0]);
@@ -1383,13 +1458,22 @@ static int launch_persistent(const void* a, const void* b, void* c, int M, int N
 }
 
 template <typename OutT, bool BF>
-static int launch_stream(const void* a, const void* b, void* c, int M, int N, int K, int ldc, hipStream_t stream) {
+static int launch_stream(const void* a, const void* b, void* c, int M, int N, int K, int ldc, hipStream_t stream,
+                         bool one_per_cu = false) {
   auto kern = gemm_f16_nt_stream<OutT, BF>;
   constexpr int lds_bytes = 5 * 256 * 128;  // three B buffers and two A buffers of 32 KiB
   static std::atomic<uint64_t> lds_ok{0};
   if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt_stream")) return rc;
   const int tiles_m = M / 256, tiles_n = N / 256;
-  dim3 grid(tiles_m * tiles_n), block(256);
+  int wgs = tiles_m * tiles_n;
+  // The walk looks up to five slabs ahead and knows one tile ahead: a tile needs six slabs or more.
+  if (one_per_cu && K >= 384) {
+    // one workgroup per CU walking tiles pid, pid + grid, ...; a multiple of 8 keeps a workgroup's tiles on its XCD
+    int g = cu_count() & ~7;
+    if (g < 8) g = 8;
+    if (wgs > g) wgs = g;
+  }
+  dim3 grid(wgs), block(256);
   hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, M, ldc, K, tiles_m,
                      tiles_n, 4);
   return check_launch("gemm_f16_nt_stream", grid, block, lds_bytes);
@@ -1416,7 +1500,7 @@ static bool tail_split(int M, int N, int& main_m, int& main_n) {
 template <typename OutT, bool BF, bool STREAMED>
 static int launch_split(const void* a, const void* b, void* c, int M, int N, int K, hipStream_t stream) {
   auto main_part = [&](int m, int n) {
-    if constexpr (STREAMED) return launch_stream<OutT, BF>(a, b, c, m, n, K, N, stream);
+    if constexpr (STREAMED) return launch_stream<OutT, BF>(a, b, c, m, n, K, N, stream, true);  // one workgroup per CU
     else return launch_tiled<256, 256, 2, 2, OutT, 2, BF>(a, b, c, m, n, K, N, stream);
   };
   int mm, mn;
@@ -1461,6 +1545,7 @@ static int launch_variant(int variant, const void* a, const void* b, void* c, in
     case 10: return launch_tiled<256, 256, 2, 2, OutT, 2, BF>(a, b, c, M, N, K, N, stream, true);
     case 11: return launch_stream<OutT, BF>(a, b, c, M, N, K, N, stream);
     case 12: return launch_split<OutT, BF, true>(a, b, c, M, N, K, stream);
+    case 13: return launch_stream<OutT, BF>(a, b, c, M, N, K, N, stream, true);
     default: {
       dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
       hipLaunchKernelGGL((gemm_f16_nt_generic<OutT, BF>), grid, block, 0, stream, (const half_t*)a, (const half_t*)b, (OutT*)c,
@@ -1489,7 +1574,9 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
     if (v <= 1 && (K < 128 || K > (1 << 21))) return false;  // prefetches two slabs ahead; 32-bit byte offsets inside a 256-row panel
     if ((v == 7 || v == 8 || v == 10) && N > (1 << 22)) return false;  // 32-bit byte offsets inside a wave's 128 rows of C
     if ((v == 7 || v == 8 || v == 10) && (K < 256 || K % 128 != 0 || K > (1 << 21))) return false;  // slabs in pairs, three in flight
-    if ((v == 11 || v == 12) && (K < 256 || K % 128 != 0 || K > (1 << 21))) return false;  // slabs in pairs; 32-bit byte offsets inside a 256-row panel
+    // the streamed kernel addresses each operand through one buffer descriptor
+    if ((v == 11 || v == 12 || v == 13) && (M * K * 2 >= (1ll << 32) || N * K * 2 >= (1ll << 32))) return false;
+    if ((v == 11 || v == 12 || v == 13) && (K < 256 || K % 128 != 0 || K > (1 << 21))) return false;  // slabs in pairs; 32-bit byte offsets inside a 256-row panel
     if (v == 9) return al && M <= 64 && N % 32 == 0 && K % 64 == 0;  // a tile is 32 rows of B; 64-half K segments
     return al && M % kGemmVariants[v].bm == 0 && N % kGemmVariants[v].bn == 0 && K % 64 == 0;
   };

@@ -22,7 +22,7 @@ def _run(dev, M, N, K, out_dtype, variant=-1, seed=10):
     return c.float().cpu(), ref
 
 
-@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 3, 4, 5, 6, 7, 8, 10, 11, 12])
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 3, 4, 5, 6, 7, 8, 10, 11, 12, 13])
 def test_gemm_1024_f32_all_variants(dev, variant):
     c, ref = _run(dev, 1024, 1024, 1024, "float32", variant)
     torch.testing.assert_close(c, ref, rtol=RTOL, atol=ATOL)
@@ -156,7 +156,7 @@ def test_gemm_full_size_repeatable(dev, shape):
     assert len(staged) == 3 and torch.equal(staged[0], staged[1]) and torch.equal(staged[0], staged[2])
     # likewise the streamed kernel and its tail-split launch
     streamed = [v for k, v in sorted(by_name.items()) if k.startswith("stream")]
-    assert len(streamed) == 2 and torch.equal(streamed[0], streamed[1])
+    assert len(streamed) == 3 and torch.equal(streamed[0], streamed[1]) and torch.equal(streamed[0], streamed[2])
 
 
 @pytest.mark.parametrize("shape", [(4096, 4608, 192), (4352, 4352, 128), (8192, 8704, 320), (512, 256, 4096)])
@@ -251,6 +251,30 @@ def test_gemm_stream_slab_rotation(dev, shape, out_dtype):
     exact = a[rows.to(dev)].float() @ b.float().t()
     torch.testing.assert_close(got[rows.to(dev)].float(), exact, rtol=RTOL, atol=ATOL)
     assert torch.equal(got, torch.ops.mi355.gemm_nt(a, b, out_dtype, v))
+
+
+@pytest.mark.parametrize("out_dtype", ["float16", "float32"])
+@pytest.mark.parametrize("shape", [(4096, 4608, 256), (4352, 4352, 384), (8192, 8704, 512), (8192, 16384, 1152), (512, 256, 4096)])
+def test_gemm_stream_tile_walk(dev, shape, out_dtype):
+    """The streamed kernel launched with one workgroup per CU: every workgroup walks several tiles as one slab sequence
+    (loads past a tile's end fetch the next tile's first slabs, a tile's first slab runs without load waits, the
+    epilogue uses the part of LDS the next loads reach last, the first MFMA on each accumulator takes a zero addend).
+    More tiles than CUs with a ragged last round, the minimum of four slabs, slab counts 2 and 0 mod 4 and 0, 1, 2 mod 3,
+    up to nine tiles per workgroup, fewer tiles than CUs -- whole matrix bit-identical to the same kernel launched one
+    workgroup per tile, and against the independent generic kernel."""
+    import iree_turbine_amd as ita
+    from oracle import inputs
+
+    M, N, K = shape
+    announce(f"gemm streamed walk {shape} {out_dtype}")
+    names = ita._lib.variants("gemm_f16_nt")
+    walk, plain = names.index("stream_256x256x64_w2x2_walk"), names.index("stream_256x256x64_w2x2")
+    a, b = [t.to(dev) for t in inputs.gemm_inputs(M, N, K)]
+    got = torch.ops.mi355.gemm_nt(a, b, out_dtype, walk)
+    assert torch.equal(got, torch.ops.mi355.gemm_nt(a, b, out_dtype, plain))
+    assert torch.equal(got, torch.ops.mi355.gemm_nt(a, b, out_dtype, walk))
+    ref = torch.ops.mi355.gemm_nt(a, b, out_dtype, len(names) - 1)
+    torch.testing.assert_close(got.float(), ref.float(), rtol=1e-3, atol=1e-3)
 
 
 def test_gemm_stream_contract(dev):
