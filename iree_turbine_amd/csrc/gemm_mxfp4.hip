@@ -1078,6 +1078,398 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_staged(const uint8_t* __restri
   }
 }
 
+// Streamed form (see gemm_f16_nt_stream for the reasoning; the code bytes are laid out identically: a slab row is 128
+// bytes = 256 codes = 8 scale blocks).  Whole 128-byte rows go global -> LDS directly, about two slabs ahead; the B
+// fragments of a slab are held in registers (read from LDS during the first quarter of the slab before), the A rows
+// are streamed fragment by fragment, each feeding 8 MFMAs 16x16x128 (a lane's 16 bytes are one scale block: lane l
+// supplies row l & 15, block 4 kh + (l >> 4) of the slab).  One workgroup per CU walks its tiles as one slab sequence.
+// LDS (160 KiB): B in a ring of five 16 KiB half buffers (U = rows 0..63, V = rows 64..127 of both 128-row halves; a
+// half is loaded over two intervals, read seven or six intervals later and free one interval after that), A in two 32
+// KiB buffers freed block by block, and 16 KiB for the scales.
+// Scales are staged through LDS in groups of two slabs: 16 bytes per row, one lane per row, 8 KiB per group (A rows,
+// then B rows), two buffers; a group is loaded in the first two steps of an even slab and first read 19 steps later.
+// A lane fetches its scale with a one-byte LDS read, which lands in bits 0..7 of a register as the MFMA wants it: the A
+// scale of a step four steps ahead, next to its fragment; the 16 B scales of the next slab in steps 4..11, into the
+// register set the current slab does not use.
+// One step = 8 MFMAs + LDS reads (A fragment and scale; steps 0..3: four B fragments; steps 4..11: two B scales) + one
+// data load (+ a scale group load); a barrier every 4 steps.  At a barrier every wave has waited for its loads older
+// than the newest 15 (about a slab's worth; the tightest case is B part 3, read 16 loads after its own) and for its LDS
+// reads older than the interval:
+//   interval q of slab t loads   A: block q - 1 of slab t + 2 (q = 0: block 3 of slab t + 1)
+//                                B: part q of slab t + 3 (parts 0, 1 -> its U half, parts 2, 3 -> its V half)
+template <typename OutT>
+__global__ __launch_bounds__(256) void gemm_mxfp4_stream(const uint8_t* __restrict__ A, const uint8_t* __restrict__ As,
+                                                         const uint8_t* __restrict__ B, const uint8_t* __restrict__ Bs,
+                                                         OutT* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n,
+                                                         int group_m) {
+  typedef _Float16 half8 __attribute__((ext_vector_type(8)));  // 16 opaque bytes of codes
+  constexpr int BM = 256, BN = 256, WN = 2, WTM = 128, WTN = 128;
+  constexpr int HALF = 128 * 128, ABUF = 256 * 128, SGRP = 8192;
+  constexpr int B_AT = 0, A_AT = 5 * HALF, S_AT = A_AT + 2 * ABUF;
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  const int T = tiles_m * tiles_n, G = (int)gridDim.x;
+  int pid = blockIdx.x;
+  int tile_m, tile_n;
+  map_tile_mx(pid, tiles_m, tiles_n, group_m, tile_m, tile_n);
+
+  // One descriptor per array (each under 4 GiB, checked on the host); tile, slab and row block go into the scalar offset.
+  const unsigned row_bytes = (unsigned)K / 2u, SK = (unsigned)K / 32u;
+  const buffer_rsrc_t a_src = make_buffer(A, (unsigned)(tiles_m * BM) * row_bytes);
+  const buffer_rsrc_t b_src = make_buffer(B, (unsigned)(tiles_n * BN) * row_bytes);
+  const buffer_rsrc_t sa_src = make_buffer(As, (unsigned)(tiles_m * BM) * SK);
+  const buffer_rsrc_t sb_src = make_buffer(Bs, (unsigned)(tiles_n * BN) * SK);
+  const int lrow = lane >> 3;
+  // codes: a wave-load covers 8 rows x 128 bytes; lane = (row l >> 3, slot l & 7) fetches chunk slot ^ ((row >> 1) & 7)
+  const unsigned g_off = (unsigned)(wave * 8 + lrow) * row_bytes + (unsigned)((lane & 7) ^ (((wave & 1) << 2) | (lrow >> 1))) * 16u;
+  // scales: a wave-load covers rows 64 w .. 64 w + 63 of the tile, 16 bytes (two slabs) per lane
+  const unsigned gs_off = (unsigned)(wave * 64 + lane) * SK;
+  const int KT = K / 256;  // even, >= 4 (checked on the host)
+  unsigned a_cur = (unsigned)(tile_m * BM) * row_bytes, b_cur = (unsigned)(tile_n * BN) * row_bytes;
+  unsigned a_nxt = a_cur, b_nxt = b_cur;  // the next tile (after the last: itself again; those loads are never used)
+  unsigned sa_cur = (unsigned)(tile_m * BM) * SK, sb_cur = (unsigned)(tile_n * BN) * SK, sa_nxt = sa_cur, sb_nxt = sb_cur;
+  auto slab_at = [&](int s, unsigned cur, unsigned nxt) { return s < KT ? cur + (unsigned)s * 128u : nxt + (unsigned)(s - KT) * 128u; };
+  auto grp_at = [&](int s, unsigned cur, unsigned nxt) { return s < KT ? cur + (unsigned)s * 8u : nxt + (unsigned)(s - KT) * 8u; };
+  // offsets of the slabs 1, 2 (A) and 3 (B) ahead and of the scale group after this pair of slabs; those of the next slab
+  // are worked out one per step in the second half of a slab
+  unsigned a_off1 = a_cur + 128u, a_off2 = a_cur + 256u, b_off3 = b_cur + 384u, sa_off = sa_cur + 16u, sb_off = sb_cur + 16u;
+  unsigned n_a1 = 0, n_a2 = 0, n_b3 = 0, n_sa = 0, n_sb = 0;
+  auto load_a = [&](int buf, int h, int blk, unsigned at) {
+    buffer_load_lds_16B(a_src, g_off, (unsigned)(h * 128 + blk * 32) * row_bytes + at,
+                        lds + A_AT + buf * ABUF + (h * 16 + blk * 4 + wave) * 1024);
+  };
+  // part p (rows 32 p .. 32 p + 31 of either 128-row half) into the half buffer at byte offset half_at
+  auto load_b = [&](int half_at, int h, int part, unsigned at) {
+    buffer_load_lds_16B(b_src, g_off, (unsigned)(h * 128 + part * 32) * row_bytes + at,
+                        lds + B_AT + half_at + (h * 8 + (part & 1) * 4 + wave) * 1024);
+  };
+  auto load_scales = [&](bool is_b, int grp_at_lds, unsigned at) {
+    buffer_load_lds_16B(is_b ? sb_src : sa_src, gs_off, at, lds + S_AT + grp_at_lds + (is_b ? 4096 : 0) + wave * 1024);
+  };
+
+  // fragment reads: lane l takes row l & 15 of a 16-row block, chunk 4 kh + (l >> 4) of the 128-byte row
+  const int r16 = lane & 15, cq = lane >> 4;
+  const unsigned lds0 = (unsigned)(uintptr_t)MI355_LDS(char, lds);
+  const unsigned lane_rd = (unsigned)(r16 * 128 + ((cq ^ (r16 >> 1)) & 7) * 16);  // k half 1: ^ 64
+  unsigned aaddr[2][2];  // [A buffer][k half]
+#pragma unroll
+  for (int bf = 0; bf < 2; bf++)
+#pragma unroll
+    for (int kh = 0; kh < 2; kh++) aaddr[bf][kh] = lds0 + A_AT + bf * ABUF + wm * (WTM * 128) + (lane_rd ^ (kh * 64));
+  const unsigned b_lane = lds0 + B_AT + wn * (64 * 128) + lane_rd;  // 64 rows of either half per half buffer
+  unsigned bU[2], bV[2];  // [k half]: the U and V half buffers read in this slab
+  // scale reads: the byte of row (16 rb + r16), slab parity sp, block 4 kh + cq sits at row * 16 + 8 sp + 4 kh + cq
+  const unsigned sa_lane = lds0 + S_AT + (unsigned)((wm * WTM + r16) * 16 + cq);
+  const unsigned sb_lane = lds0 + S_AT + 4096 + (unsigned)((wn * WTN + r16) * 16 + cq);
+  unsigned sa_rd = sa_lane, sa_rdn = sa_lane + 8, sb_rdn = sb_lane + 8;  // this slab's A scales, the next slab's A and B
+
+  // [n block][m block].  Never cleared: the first MFMA of a tile on each accumulator (slab 0, k half 0) takes a zero
+  // addend instead -- a register write in front of an inline-assembly MFMA would need wait states the compiler does not
+  // know to insert.
+  floatx4 acc[8][8];
+  half8 fb0[2][8], fb1[2][8], fa[8];
+  int sb0[2][8], sb1[2][8], sat[8];  // B scales [k half][row block] of the two slab parities; A scales by step
+
+  // MFMAs as inline assembly with the accumulators pinned to AGPRs (64 four-register accumulators: the compiler's own
+  // allocation keeps moving some of them between the two register classes inside the loop).  No MFMA here reads an
+  // accumulator written fewer than 8 MFMAs earlier.  x, sx: B codes and scale (bits 0..7); y, sy: A codes and scale.
+#define MI355_SM_MFMA(c, x, sx, y, sy)                                                                                    \
+  asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0] cbsz:4 blgp:4"                  \
+               : "+a"(c) : "v"(x), "v"(y), "v"(sx), "v"(sy))
+#define MI355_SM_MFMA0(c, x, sx, y, sy)                                                                                   \
+  asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, 0, %3, %4 op_sel_hi:[0,0,0] cbsz:4 blgp:4"                   \
+               : "=a"(c) : "v"(x), "v"(y), "v"(sx), "v"(sy))
+#define MI355_SM_ACC(ZERO, c, x, sx, y, sy)              \
+  do {                                                   \
+    if constexpr (ZERO) MI355_SM_MFMA0(c, x, sx, y, sy); \
+    else MI355_SM_MFMA(c, x, sx, y, sy);                 \
+  } while (0)
+  // The first MFMA of a step together with the wait for the step's A fragment and scale (y, sy: both were requested four
+  // steps earlier; LG = LDS reads issued since).  One statement, with the registers as plain inputs: a separate wait
+  // statement that names them as outputs makes the compiler put a wait state in front of their next use.  All the
+  // statements involved are volatile assembly, which keeps their order.
+#define MI355_SM_ACCW(ZERO, LG, c, x, sx, y, sy)                                                                                  \
+  do {                                                                                                                          \
+    if constexpr (ZERO)                                                                                                         \
+      asm volatile("s_waitcnt lgkmcnt(%5)\n\tv_mfma_scale_f32_16x16x128_f8f6f4 %0, %3, %1, 0, %4, %2 op_sel_hi:[0,0,0] cbsz:4 blgp:4" \
+                   : "=a"(c) : "v"(y), "v"(sy), "v"(x), "v"(sx), "n"(LG));                                                      \
+    else                                                                                                                        \
+      asm volatile("s_waitcnt lgkmcnt(%5)\n\tv_mfma_scale_f32_16x16x128_f8f6f4 %0, %3, %1, %0, %4, %2 op_sel_hi:[0,0,0] cbsz:4 blgp:4" \
+                   : "+a"(c) : "v"(y), "v"(sy), "v"(x), "v"(sx), "n"(LG));                                                      \
+  } while (0)
+#define MI355_SM_READ(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off))
+#define MI355_SM_READ8(dst, addr, off) asm volatile("ds_read_u8 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off))
+#define MI355_SM_TIE8(X) "+v"(X[0]), "+v"(X[1]), "+v"(X[2]), "+v"(X[3]), "+v"(X[4]), "+v"(X[5]), "+v"(X[6]), "+v"(X[7])
+
+  // ---- prologue: B0 (half buffers 0, 1), A0, B1 (2, 3), A1 blocks 0..2, scale group 0 ----
+#pragma unroll
+  for (int x = 0; x < 8; x++) load_b((x >> 2) * HALF, x & 1, x >> 1, b_cur);
+#pragma unroll
+  for (int x = 0; x < 8; x++) load_a(0, x & 1, x >> 1, a_cur);
+#pragma unroll
+  for (int x = 0; x < 8; x++) load_b((2 + (x >> 2)) * HALF, x & 1, x >> 1, b_cur + 128u);
+#pragma unroll
+  for (int x = 0; x < 6; x++) load_a(1, x & 1, x >> 1, a_cur + 128u);
+  load_scales(false, 0, sa_cur);
+  load_scales(true, 0, sb_cur);
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+  bU[0] = b_lane; bU[1] = b_lane ^ 64;
+  bV[0] = b_lane + HALF; bV[1] = bV[0] ^ 64;
+  MI355_SM_READ(fb0[0][0], bU[0], 0 * 2048); MI355_SM_READ(fb0[0][1], bU[0], 1 * 2048);
+  MI355_SM_READ(fb0[0][2], bU[0], 2 * 2048); MI355_SM_READ(fb0[0][3], bU[0], 3 * 2048);
+  MI355_SM_READ(fb0[0][4], bV[0], 0 * 2048); MI355_SM_READ(fb0[0][5], bV[0], 1 * 2048);
+  MI355_SM_READ(fb0[0][6], bV[0], 2 * 2048); MI355_SM_READ(fb0[0][7], bV[0], 3 * 2048);
+  MI355_SM_READ(fb0[1][0], bU[1], 0 * 2048); MI355_SM_READ(fb0[1][1], bU[1], 1 * 2048);
+  MI355_SM_READ(fb0[1][2], bU[1], 2 * 2048); MI355_SM_READ(fb0[1][3], bU[1], 3 * 2048);
+  MI355_SM_READ(fb0[1][4], bV[1], 0 * 2048); MI355_SM_READ(fb0[1][5], bV[1], 1 * 2048);
+  MI355_SM_READ(fb0[1][6], bV[1], 2 * 2048); MI355_SM_READ(fb0[1][7], bV[1], 3 * 2048);
+  MI355_SM_READ(fa[0], aaddr[0][0], 0); MI355_SM_READ(fa[1], aaddr[0][1], 0);
+  MI355_SM_READ(fa[2], aaddr[0][0], 2048); MI355_SM_READ(fa[3], aaddr[0][1], 2048);
+  asm volatile("s_waitcnt lgkmcnt(0)" : MI355_SM_TIE8(fb0[0]), MI355_SM_TIE8(fb0[1]), "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]));
+  MI355_SM_READ8(sb0[0][0], sb_lane, 0 * 256); MI355_SM_READ8(sb0[0][1], sb_lane, 1 * 256);
+  MI355_SM_READ8(sb0[0][2], sb_lane, 2 * 256); MI355_SM_READ8(sb0[0][3], sb_lane, 3 * 256);
+  MI355_SM_READ8(sb0[0][4], sb_lane, 4 * 256); MI355_SM_READ8(sb0[0][5], sb_lane, 5 * 256);
+  MI355_SM_READ8(sb0[0][6], sb_lane, 6 * 256); MI355_SM_READ8(sb0[0][7], sb_lane, 7 * 256);
+  MI355_SM_READ8(sb0[1][0], sb_lane, 0 * 256 + 4); MI355_SM_READ8(sb0[1][1], sb_lane, 1 * 256 + 4);
+  MI355_SM_READ8(sb0[1][2], sb_lane, 2 * 256 + 4); MI355_SM_READ8(sb0[1][3], sb_lane, 3 * 256 + 4);
+  MI355_SM_READ8(sb0[1][4], sb_lane, 4 * 256 + 4); MI355_SM_READ8(sb0[1][5], sb_lane, 5 * 256 + 4);
+  MI355_SM_READ8(sb0[1][6], sb_lane, 6 * 256 + 4); MI355_SM_READ8(sb0[1][7], sb_lane, 7 * 256 + 4);
+  MI355_SM_READ8(sat[0], sa_lane, 0); MI355_SM_READ8(sat[1], sa_lane, 4);
+  MI355_SM_READ8(sat[2], sa_lane, 256); MI355_SM_READ8(sat[3], sa_lane, 256 + 4);
+  asm volatile("s_waitcnt lgkmcnt(0)" : MI355_SM_TIE8(sb0[0]), MI355_SM_TIE8(sb0[1]), "+v"(sat[0]), "+v"(sat[1]), "+v"(sat[2]), "+v"(sat[3]));
+  __builtin_amdgcn_s_barrier();  // every wave has read B0: its half buffers may receive slab 2's V half (0) and slab 3's U half (1)
+  __builtin_amdgcn_sched_barrier(0);
+  // B2: U half -> half buffer 4, V half -> half buffer 0
+#pragma unroll
+  for (int x = 0; x < 8; x++) load_b(((4 + (x >> 2)) % 5) * HALF, x & 1, x >> 1, b_cur + 256u);
+  __builtin_amdgcn_sched_barrier(0);
+
+  // B ring: slab t's halves live in half buffers (2 t) % 5 and (2 t + 1) % 5; pos = (2 t) % 5 for the current slab t
+  int pos = 0;
+  int sg_ld = SGRP;  // LDS offset of the scale group buffer the next group goes to (groups alternate)
+
+  // Step s of a slab whose A buffer is PAR: MFMAs of (m block s / 2, k half s % 2) on fa[s % 8], sat[s % 8] against
+  // FB / SB[s % 2][0..7].  LGKM = LDS reads issued after those of step s - 4 (which filled fa and sat of this step).
+#define MI355_SM_STEP(s, PAR, FB, FBN, SB, SBN, LGKM, FIRST)                                                               \
+  do {                                                                                                                     \
+    constexpr int s4 = (s) + 4, nb = s4 >= 16 ? 1 - (PAR) : (PAR), ns = s4 & 15;                                           \
+    MI355_SM_ACCW(FIRST && !((s)&1), LGKM, acc[0][(s) >> 1], FB[(s)&1][0], SB[(s)&1][0], fa[(s)&7], sat[(s)&7]);            \
+    MI355_SM_READ(fa[s4 & 7], aaddr[nb][ns & 1], (ns >> 1) * 2048);                                                        \
+    __builtin_amdgcn_sched_barrier(0);                                                                                     \
+    MI355_SM_ACC(FIRST && !((s)&1), acc[1][(s) >> 1], FB[(s)&1][1], SB[(s)&1][1], fa[(s)&7], sat[(s)&7]);                   \
+    if constexpr (s4 >= 16) MI355_SM_READ8(sat[s4 & 7], sa_rdn, (ns >> 1) * 256 + (ns & 1) * 4);                           \
+    else MI355_SM_READ8(sat[s4 & 7], sa_rd, (ns >> 1) * 256 + (ns & 1) * 4);                                               \
+    __builtin_amdgcn_sched_barrier(0);                                                                                     \
+    MI355_SM_ACC(FIRST && !((s)&1), acc[2][(s) >> 1], FB[(s)&1][2], SB[(s)&1][2], fa[(s)&7], sat[(s)&7]);                   \
+    if constexpr ((s) < 4) {                                                                                               \
+      MI355_SM_READ(FBN[(s) >> 1][(4 * (s)) & 7], ((s)&1 ? bV : bU)[(s) >> 1], 0 * 2048);                                  \
+      MI355_SM_READ(FBN[(s) >> 1][(4 * (s) + 1) & 7], ((s)&1 ? bV : bU)[(s) >> 1], 1 * 2048);                              \
+    } else if constexpr ((s) < 12) {                                                                                       \
+      MI355_SM_READ8(SBN[((s)-4) >> 2][(2 * ((s)-4)) & 7], sb_rdn, ((2 * ((s)-4)) & 7) * 256 + (((s)-4) >> 2) * 4);        \
+    }                                                                                                                      \
+    __builtin_amdgcn_sched_barrier(0);                                                                                     \
+    MI355_SM_ACC(FIRST && !((s)&1), acc[3][(s) >> 1], FB[(s)&1][3], SB[(s)&1][3], fa[(s)&7], sat[(s)&7]);                   \
+    if constexpr ((s) < 4) {                                                                                               \
+      MI355_SM_READ(FBN[(s) >> 1][(4 * (s) + 2) & 7], ((s)&1 ? bV : bU)[(s) >> 1], 2 * 2048);                              \
+      MI355_SM_READ(FBN[(s) >> 1][(4 * (s) + 3) & 7], ((s)&1 ? bV : bU)[(s) >> 1], 3 * 2048);                              \
+    } else if constexpr ((s) < 12) {                                                                                       \
+      MI355_SM_READ8(SBN[((s)-4) >> 2][(2 * ((s)-4) + 1) & 7], sb_rdn, ((2 * ((s)-4) + 1) & 7) * 256 + (((s)-4) >> 2) * 4); \
+    }                                                                                                                      \
+    __builtin_amdgcn_sched_barrier(0);                                                                                     \
+    MI355_SM_ACC(FIRST && !((s)&1), acc[4][(s) >> 1], FB[(s)&1][4], SB[(s)&1][4], fa[(s)&7], sat[(s)&7]);                   \
+    MI355_SM_ACC(FIRST && !((s)&1), acc[5][(s) >> 1], FB[(s)&1][5], SB[(s)&1][5], fa[(s)&7], sat[(s)&7]);                   \
+    {                                                                                                                      \
+      constexpr int q = (s) >> 2, x = (s)&3;                                                                               \
+      /* the scale group after this pair of slabs: A rows in step 0, B rows in step 1 of an even slab */                  \
+      if constexpr ((PAR) == 0 && (s) == 0) load_scales(false, sg_ld, sa_off);                                             \
+      if constexpr ((PAR) == 0 && (s) == 1) load_scales(true, sg_ld, sb_off);                                              \
+      if constexpr (x < 2) {                                                                                               \
+        if constexpr (q == 0) load_a(1 - (PAR), x, 3, a_off1);                                                             \
+        else load_a(PAR, x, q - 1, a_off2);                                                                                \
+      } else {                                                                                                             \
+        load_b(q < 2 ? ld_u : ld_v, x - 2, q, b_off3);                                                                     \
+      }                                                                                                                    \
+    }                                                                                                                      \
+    __builtin_amdgcn_sched_barrier(0);                                                                                     \
+    if constexpr ((s) == 8) n_a1 = slab_at(kt + 2, a_cur, a_nxt);                                                          \
+    if constexpr ((s) == 9) n_a2 = slab_at(kt + 3, a_cur, a_nxt);                                                          \
+    if constexpr ((s) == 10) n_b3 = slab_at(kt + 4, b_cur, b_nxt);                                                         \
+    if constexpr ((PAR) == 1 && (s) == 11) n_sa = grp_at(kt + 3, sa_cur, sa_nxt);                                          \
+    if constexpr ((PAR) == 1 && (s) == 12) n_sb = grp_at(kt + 3, sb_cur, sb_nxt);                                          \
+    MI355_SM_ACC(FIRST && !((s)&1), acc[6][(s) >> 1], FB[(s)&1][6], SB[(s)&1][6], fa[(s)&7], sat[(s)&7]);                   \
+    MI355_SM_ACC(FIRST && !((s)&1), acc[7][(s) >> 1], FB[(s)&1][7], SB[(s)&1][7], fa[(s)&7], sat[(s)&7]);                   \
+    __builtin_amdgcn_sched_barrier(0);                                                                                     \
+  } while (0)
+  // End of an interval: loads older than the newest VMC and LDS reads older than the interval are complete in every wave.
+#define MI355_SM_SYNC(RD, VMC)                                                        \
+  do {                                                                                \
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(%1)" ::"n"(VMC), "n"(RD) : "memory");   \
+    __builtin_amdgcn_s_barrier();                                                     \
+    __builtin_amdgcn_sched_barrier(0);                                                \
+  } while (0)
+  // LDS reads per step: 2 (A fragment, A scale) + 4 B fragments in steps 0..3 or 2 B scales in steps 4..11.
+#define MI355_SM_SLAB(PAR, FB, FBN, SB, SBN, FIRST, VMC)                                                         \
+  do {                                                                                                          \
+    {                                                                                                           \
+      const int pu = pos + 2 >= 5 ? pos - 3 : pos + 2, pv = pos + 3 >= 5 ? pos - 2 : pos + 3; /* slab t + 1 */   \
+      bU[0] = b_lane + (unsigned)(pu * HALF);                                                                   \
+      bU[1] = bU[0] ^ 64;                                                                                       \
+      bV[0] = b_lane + (unsigned)(pv * HALF);                                                                   \
+      bV[1] = bV[0] ^ 64;                                                                                       \
+    }                                                                                                           \
+    /* slab t + 3: U half -> (2 t + 6) % 5 = pos + 1, V half -> (2 t + 7) % 5 = pos + 2 */                       \
+    const int ld_u = (pos + 1 >= 5 ? pos - 4 : pos + 1) * HALF, ld_v = (pos + 2 >= 5 ? pos - 3 : pos + 2) * HALF; \
+    MI355_SM_STEP(0, PAR, FB, FBN, SB, SBN, 6, FIRST);                                                          \
+    MI355_SM_STEP(1, PAR, FB, FBN, SB, SBN, 10, FIRST);                                                         \
+    MI355_SM_STEP(2, PAR, FB, FBN, SB, SBN, 14, FIRST);                                                         \
+    MI355_SM_STEP(3, PAR, FB, FBN, SB, SBN, 15, FIRST);                                                         \
+    MI355_SM_SYNC(15, VMC);                                                                                     \
+    MI355_SM_STEP(4, PAR, FB, FBN, SB, SBN, 15, FIRST);                                                         \
+    MI355_SM_STEP(5, PAR, FB, FBN, SB, SBN, 15, FIRST);                                                         \
+    MI355_SM_STEP(6, PAR, FB, FBN, SB, SBN, 14, FIRST);                                                         \
+    MI355_SM_STEP(7, PAR, FB, FBN, SB, SBN, 12, FIRST);                                                         \
+    MI355_SM_SYNC(15, VMC);                                                                                     \
+    MI355_SM_STEP(8, PAR, FB, FBN, SB, SBN, 12, FIRST);                                                         \
+    MI355_SM_STEP(9, PAR, FB, FBN, SB, SBN, 12, FIRST);                                                         \
+    MI355_SM_STEP(10, PAR, FB, FBN, SB, SBN, 12, FIRST);                                                        \
+    MI355_SM_STEP(11, PAR, FB, FBN, SB, SBN, 12, FIRST);                                                        \
+    MI355_SM_SYNC(15, VMC);                                                                                     \
+    MI355_SM_STEP(12, PAR, FB, FBN, SB, SBN, 12, FIRST);                                                        \
+    MI355_SM_STEP(13, PAR, FB, FBN, SB, SBN, 10, FIRST);                                                        \
+    MI355_SM_STEP(14, PAR, FB, FBN, SB, SBN, 8, FIRST);                                                         \
+    MI355_SM_STEP(15, PAR, FB, FBN, SB, SBN, 6, FIRST);                                                         \
+    /* the next slab's B fragments and scales were requested in steps 0..11: they have landed; tie them here */ \
+    asm volatile("s_waitcnt vmcnt(%32) lgkmcnt(8)"                                                              \
+                 : MI355_SM_TIE8(FBN[0]), MI355_SM_TIE8(FBN[1]), MI355_SM_TIE8(SBN[0]), MI355_SM_TIE8(SBN[1])   \
+                 : "n"(VMC) : "memory");                                                                        \
+    __builtin_amdgcn_s_barrier();                                                                               \
+    __builtin_amdgcn_sched_barrier(0);                                                                          \
+    a_off1 = n_a1;                                                                                              \
+    a_off2 = n_a2;                                                                                              \
+    b_off3 = n_b3;                                                                                              \
+    pos = pos + 2 >= 5 ? pos - 3 : pos + 2;                                                                     \
+    /* the scale reads of the next slab: its parity's 8 bytes; an odd slab's successor starts the next group */ \
+    if constexpr ((PAR) == 0) {                                                                                 \
+      sa_rd = sa_rdn;                                                                                           \
+      sa_rdn = sa_lane + (unsigned)sg_ld;        /* slab t + 2: the group being loaded, first 8 bytes */        \
+      sb_rdn = sb_lane + (unsigned)sg_ld;                                                                       \
+    } else {                                                                                                    \
+      sa_rd = sa_rdn;                                                                                           \
+      sa_rdn = sa_rd + 8;                                                                                       \
+      sb_rdn = sb_rdn + 8;                                                                                      \
+      sg_ld ^= SGRP;                                                                                            \
+      sa_off = n_sa;                                                                                            \
+      sb_off = n_sb;                                                                                            \
+    }                                                                                                           \
+  } while (0)
+
+  for (; pid < T; pid += G) {
+    int nxt_m = tile_m, nxt_n = tile_n;
+    if (pid + G < T) map_tile_mx(pid + G, tiles_m, tiles_n, group_m, nxt_m, nxt_n);
+    a_nxt = (unsigned)(nxt_m * BM) * row_bytes;
+    b_nxt = (unsigned)(nxt_n * BN) * row_bytes;
+    sa_nxt = (unsigned)(nxt_m * BM) * SK;
+    sb_nxt = (unsigned)(nxt_n * BN) * SK;
+    // In a tile's first slab the 32 stores of the epilogue before it sit in the queue behind the loads the waits are
+    // about (a 32-bit epilogue, 64 stores, drains the queue instead).
+    constexpr int VMC_FIRST = sizeof(OutT) == 2 ? 15 + 32 : 15;
+    int kt = 0;
+    MI355_SM_SLAB(0, fb0, fb1, sb0, sb1, true, VMC_FIRST);
+    kt = 1;
+    MI355_SM_SLAB(1, fb1, fb0, sb1, sb0, false, 15);
+    for (kt = 2; kt < KT; kt += 2) {
+      MI355_SM_SLAB(0, fb0, fb1, sb0, sb1, false, 15);
+      kt++;
+      MI355_SM_SLAB(1, fb1, fb0, sb1, sb0, false, 15);
+      kt--;
+    }
+    // ---- epilogue ----
+    // The MFMAs are inline assembly, so the compiler does not know that the accumulators were written just now: the
+    // wait states an MFMA result needs before another instruction may read it are spelled out, and every accumulator is
+    // tied to a statement behind them so that no read of it can be scheduled earlier.
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+      asm volatile("" : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]), "+a"(acc[i][4]), "+a"(acc[i][5]),
+                        "+a"(acc[i][6]), "+a"(acc[i][7]));
+    // lane holds, for m = 16 j + (l & 15): n = 16 i + 4 (l >> 4) + r, r < 4.  The addresses come from a lane id the
+    // compiler cannot see through, so that none of them is computed ahead of the K loop and kept across it.
+    const int le = opaque_lane_id();
+    const int r16e = le & 15, cqe = le >> 4;
+    if constexpr (sizeof(OutT) == 2) {
+      // bf16 results go through LDS, 16 rows x 64 columns (2 KiB) per pass in a wave-private region: 8-byte writes of 4
+      // consecutive n (chunk slot c ^ ((m >> 1) & 7) of the 128-byte row), whole rows read back 16 bytes per lane and
+      // stored as full cache lines.  LDS operations of a wave execute in order, so the passes need no waits between
+      // them.  The next tile's slabs are landing in LDS meanwhile; free at this point is block 3 of A buffer 1 (rows
+      // 96..127 of either half: twice 4 KiB), which the next loads reach only after the barrier below.  Inline
+      // assembly like the K loop's LDS accesses: direct-to-LDS loads are in flight.
+      const unsigned ep = lds0 + (unsigned)(A_AT + ABUF + (wave < 2 ? 12 * 1024 + wave * 2048 : 28 * 1024 + (wave - 2) * 2048));
+      const int er = le >> 3, ec = le & 7, sw = (r16e >> 1) & 7;
+      // write: row r16e, chunk (2 (i & 3) + (cqe >> 1)) ^ sw, 8-byte half cqe & 1; the i term is an XOR of the address
+      const unsigned wa = ep + (unsigned)(r16e * 128 + ((((cqe >> 1) ^ (sw & 1)) | (sw & 6)) * 16) + 8 * (cqe & 1));
+      // read: row 8 it + er, chunk ec ^ ((row >> 1) & 7) = (ec ^ (er >> 1)) ^ 4 it
+      const unsigned ra = ep + (unsigned)(er * 128 + ((ec ^ (er >> 1)) * 16));
+      OutT* cbase = C + (size_t)(tile_m * BM + wm * WTM + er) * N + tile_n * BN + wn * WTN + ec * 8;
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+#pragma unroll
+        for (int ih = 0; ih < 2; ih++) {
+#pragma unroll
+          for (int ii = 0; ii < 4; ii++) {
+            const int i = ih * 4 + ii;
+            ushortx4 v = {f32_to_bf16_rne(acc[i][j][0]), f32_to_bf16_rne(acc[i][j][1]), f32_to_bf16_rne(acc[i][j][2]),
+                          f32_to_bf16_rne(acc[i][j][3])};
+            asm volatile("ds_write_b64 %0, %1" ::"v"(wa ^ (unsigned)(32 * ii)), "v"(v) : "memory");
+          }
+          half8 rv[2];
+          asm volatile("ds_read_b128 %0, %1" : "=v"(rv[0]) : "v"(ra));
+          asm volatile("ds_read_b128 %0, %1 offset:1024" : "=v"(rv[1]) : "v"(ra ^ 64u));
+          asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(rv[0]), "+v"(rv[1]));
+#pragma unroll
+          for (int it = 0; it < 2; it++) *reinterpret_cast<half8*>(cbase + (size_t)(j * 16 + it * 8) * N + ih * 64) = rv[it];
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    } else {
+      OutT* crow = C + (size_t)(tile_m * BM + wm * WTM + r16e) * N + tile_n * BN + wn * WTN + 4 * cqe;
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+          MxOut<OutT>::store4(crow + (size_t)(j * 16) * N + i * 16, acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // 64 stores: more than a wait can count past
+    }
+    a_cur = a_nxt;
+    b_cur = b_nxt;
+    sa_cur = sa_nxt;
+    sb_cur = sb_nxt;
+    tile_m = nxt_m;
+    tile_n = nxt_n;
+    // the waves leave the epilogue together: the next loads reach the LDS the other waves' epilogues use
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  // the loads issued for a tile that does not exist still target LDS: let them land before the workgroup ends
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : MI355_SM_TIE8(fa), MI355_SM_TIE8(sat));
+#undef MI355_SM_SLAB
+#undef MI355_SM_SYNC
+#undef MI355_SM_STEP
+#undef MI355_SM_TIE8
+#undef MI355_SM_READ8
+#undef MI355_SM_READ
+#undef MI355_SM_ACCW
+#undef MI355_SM_ACC
+#undef MI355_SM_MFMA0
+#undef MI355_SM_MFMA
+}
+
 struct MxVariant {
   const char* name;
   int bm, bn;
@@ -1088,6 +1480,8 @@ static const MxVariant kMxVariants[] = {
     {"tiled_128x128x256_w2x2", 128, 128},
     {"skinny_m32_n32_w8", 32, 32},
     {"staged_256x256x256_w2x2", 256, 256},
+    {"stream_256x256x256_w2x2", 256, 256},
+    {"stream_256x256x256_w2x2_walk", 256, 256},
     {"generic_32x128", 32, 128},
 };
 constexpr int kNumMxVariants = sizeof(kMxVariants) / sizeof(kMxVariants[0]);
@@ -1153,6 +1547,26 @@ static int launch_mx_staged(const void* a, const void* as, const void* b, const 
 }
 
 template <typename OutT>
+static int launch_mx_stream(const void* a, const void* as, const void* b, const void* bs, void* c, int M, int N, int K,
+                            hipStream_t stream, bool one_per_cu) {
+  auto kern = gemm_mxfp4_stream<OutT>;
+  constexpr int lds_bytes = 5 * 256 * 128;  // three B buffers and two A buffers of 32 KiB
+  static std::atomic<uint64_t> lds_ok{0};
+  if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_mxfp4_stream")) return rc;
+  const int tiles_m = M / 256, tiles_n = N / 256;
+  int wgs = tiles_m * tiles_n;
+  if (one_per_cu) {
+    int g = mx_cu_count() & ~7;  // multiples of 8 keep a workgroup's tiles on the XCD it runs on
+    if (g < 8) g = 8;
+    if (wgs > g) wgs = g;
+  }
+  dim3 grid(wgs), block(256);
+  hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const uint8_t*)a, (const uint8_t*)as, (const uint8_t*)b,
+                     (const uint8_t*)bs, (OutT*)c, M, N, K, tiles_m, tiles_n, 4);
+  return check_launch("gemm_mxfp4_stream", grid, block, lds_bytes);
+}
+
+template <typename OutT>
 static int launch_mx(int variant, const void* a, const void* as, const void* b, const void* bs, void* c, int M, int N, int K,
                      hipStream_t stream) {
   switch (variant) {
@@ -1174,6 +1588,8 @@ static int launch_mx(int variant, const void* a, const void* as, const void* b, 
       return check_launch("gemm_mxfp4_skinny", grid, block, lds_bytes);
     }
     case 4: return launch_mx_staged<OutT>(a, as, b, bs, c, M, N, K, stream);
+    case 5: return launch_mx_stream<OutT>(a, as, b, bs, c, M, N, K, stream, false);
+    case 6: return launch_mx_stream<OutT>(a, as, b, bs, c, M, N, K, stream, true);
     default: {
       dim3 grid((N + 127) / 128, (M + 31) / 32), block(256);
       hipLaunchKernelGGL(gemm_mxfp4_generic<OutT>, grid, block, 0, stream, (const uint8_t*)a, (const uint8_t*)as,
@@ -1205,6 +1621,8 @@ extern "C" int mi355_mxfp4_gemm(const void* a, const void* a_scale, const void* 
     if (v == kNumMxVariants - 1) return true;
     if (v == 3) return sc_al4 && M <= 32 && N % 32 == 0 && K % 256 == 0;  // skinny: whole 128-byte segments
     if ((v == 0 || v == 4) && !(sc_al16 && K % 512 == 0 && K >= 1024 && K <= (1 << 22))) return false;  // 2-slab scale groups
+    // streamed: slabs in pairs, four or more; each operand behind one buffer descriptor
+    if ((v == 5 || v == 6) && !(sc_al16 && K % 512 == 0 && K >= 1024 && M * (K / 2) < (1ll << 32) && N * (K / 2) < (1ll << 32))) return false;
     return sc_al && M % kMxVariants[v].bm == 0 && N % kMxVariants[v].bn == 0 && K % 256 == 0;
   };
   if (variant < 0) {
@@ -1215,6 +1633,7 @@ extern "C" int mi355_mxfp4_gemm(const void* a, const void* a_scale, const void* 
     const long long rounds = (t256 + 255) / 256;
     const bool big = t256 >= 128 && t256 * 100 >= rounds * 256 * 85;
     if (fits(3)) variant = 3;
+    else if (big && fits(6)) variant = 6;  // streamed, one workgroup per CU: 4096x8192x8192 124 us against 133 for the persistent kernel
     else if (big && K >= 32768 && fits(4)) variant = 4;  // its epilogue is not overlapped: ahead only from 128 slabs per tile
     else if (big && fits(0)) variant = 0;
     else if (big && fits(1)) variant = 1;

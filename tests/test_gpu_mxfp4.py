@@ -43,7 +43,7 @@ def test_dequant_random_bit_exact(dev):
     assert np.array_equal(out.view(np.uint32), om.mxfp4_dequant_ref(a, asc).view(np.uint32))
 
 
-@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 4, 5])
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 4, 5, 6, 7])
 def test_mxfp4_gemm_variants(dev, variant):
     import iree_turbine_amd  # noqa: F401
     from oracle import inputs, mxfp4 as om
@@ -74,9 +74,9 @@ def test_mxfp4_gemm_ragged(dev, shape):
 
 
 @pytest.mark.parametrize("shape", [(32, 256, 512), (1, 64, 256), (7, 96, 2048), (32, 8192, 8192), (20, 160, 16384), (32, 64, 8192 + 256)])
-@pytest.mark.parametrize("variant", [3, 5])
+@pytest.mark.parametrize("variant", [3, 7])
 def test_mxfp4_skinny_vs_generic(dev, shape, variant):
-    """The weight-streaming kernel (variant 3) and the any-shape kernel (variant 5) on skinny shapes."""
+    """The weight-streaming kernel (variant 3) and the any-shape kernel (variant 7) on skinny shapes."""
     import iree_turbine_amd  # noqa: F401
     from oracle import inputs, mxfp4 as om
 
@@ -203,6 +203,35 @@ def test_mxfp4_persistent_tile_walk(dev, shape, out_dtype):
     else:
         # both round the same fp32 sums (up to summation order) to bf16: at most one bf16 step apart,
         # plus the summation-order noise of sums that cancel to nearly nothing
+        g32, r32 = got.float(), ref.float()
+        assert _rel_err(g32, r32) < 1e-3
+        assert ((g32 - r32).abs() <= r32.abs() * 2 ** -7 + 1e-5 * r32.abs().max()).all()
+
+
+@pytest.mark.parametrize("shape", [(256, 256, 1024), (512, 768, 1536), (4352, 4352, 1024), (4096, 4608, 2560), (8192, 8704, 1024),
+                                   (256, 512, 8192)])
+@pytest.mark.parametrize("out_dtype", ["bfloat16", "float32"])
+def test_mxfp4_stream_tile_walk(dev, shape, out_dtype):
+    """The streamed kernel: B in a ring of five half buffers (slab counts 4, 6, 10, 32: the ring position at a tile's end takes
+    every value), scale groups of two slabs (even and odd numbers of groups per tile: the
+    scale buffer parity flips between tiles), more tiles than CUs with a ragged last round, up to five tiles per
+    workgroup, fewer tiles than CUs -- the walk bit-identical to the same kernel launched one workgroup per tile,
+    whole matrix against the independent generic kernel, launches repeat bit for bit."""
+    import iree_turbine_amd as ita
+    from oracle import inputs
+
+    M, N, K = shape
+    announce(f"mxfp4 streamed walk {shape} {out_dtype}")
+    names = ita._lib.variants("mxfp4_gemm")
+    walk, plain = names.index("stream_256x256x256_w2x2_walk"), names.index("stream_256x256x256_w2x2")
+    a, asc, b, bsc = [t.to(dev) for t in inputs.mxfp4_inputs(M, N, K)]
+    got = torch.ops.mi355.mxfp4_gemm(a, asc, b, bsc, out_dtype, walk)
+    assert torch.equal(got, torch.ops.mi355.mxfp4_gemm(a, asc, b, bsc, out_dtype, plain))
+    assert torch.equal(got, torch.ops.mi355.mxfp4_gemm(a, asc, b, bsc, out_dtype, walk))
+    ref = torch.ops.mi355.mxfp4_gemm(a, asc, b, bsc, out_dtype, len(names) - 1)
+    if out_dtype == "float32":
+        assert _rel_err(got, ref) < 1e-5
+    else:
         g32, r32 = got.float(), ref.float()
         assert _rel_err(g32, r32) < 1e-3
         assert ((g32 - r32).abs() <= r32.abs() * 2 ** -7 + 1e-5 * r32.abs().max()).all()
