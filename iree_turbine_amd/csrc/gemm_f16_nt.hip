@@ -759,6 +759,17 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_stream(const half_t* __restri
     if constexpr (BF) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=a"(c) : "v"(x), "v"(y));        \
     else asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=a"(c) : "v"(x), "v"(y));                      \
   } while (0)
+  // The first MFMA of a step together with the wait for the step's A fragment y (requested four steps earlier; LG = LDS
+  // reads issued since).  One statement, with the fragment as a plain input: a separate wait statement that names it as
+  // an output makes the compiler put a wait state in front of its next use.  All the statements involved are volatile
+  // assembly, which keeps their order.
+#define MI355_SM_ACCW(ZERO, LG, c, x, y)                                                                                         \
+  do {                                                                                                                          \
+    if constexpr (ZERO && BF) asm volatile("s_waitcnt lgkmcnt(%3)\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=a"(c) : "v"(x), "v"(y), "n"(LG)); \
+    else if constexpr (ZERO) asm volatile("s_waitcnt lgkmcnt(%3)\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=a"(c) : "v"(x), "v"(y), "n"(LG)); \
+    else if constexpr (BF) asm volatile("s_waitcnt lgkmcnt(%3)\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(x), "v"(y), "n"(LG)); \
+    else asm volatile("s_waitcnt lgkmcnt(%3)\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(x), "v"(y), "n"(LG)); \
+  } while (0)
 #define MI355_SM_READ(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off))
 #define MI355_SM_TIE8(X) "+v"(X[0]), "+v"(X[1]), "+v"(X[2]), "+v"(X[3]), "+v"(X[4]), "+v"(X[5]), "+v"(X[6]), "+v"(X[7])
 
@@ -807,9 +818,7 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_stream(const half_t* __restri
 #define MI355_SM_STEP(s, PAR, FB, FBN, LGKM, FIRST)                                                                              \
   do {                                                                                                                     \
     constexpr int s4 = (s) + 4, nb = s4 >= 16 ? 1 - (PAR) : (PAR), ns = s4 & 15;                                           \
-    asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(fa[(s)&7]) : "n"(LGKM));                                                   \
-    __builtin_amdgcn_sched_barrier(0);                                                                                     \
-    MI355_SM_ACC(FIRST && !((s)&1), acc[0][(s) >> 1], FB[(s)&1][0], fa[(s)&7]);                                      \
+    MI355_SM_ACCW(FIRST && !((s)&1), LGKM, acc[0][(s) >> 1], FB[(s)&1][0], fa[(s)&7]);                                     \
     MI355_SM_READ(fa[s4 & 7], aaddr[nb][ns & 1], (ns >> 1) * 2048);                                                        \
     __builtin_amdgcn_sched_barrier(0);                                                                                     \
     MI355_SM_ACC(FIRST && !((s)&1), acc[1][(s) >> 1], FB[(s)&1][1], fa[(s)&7]);                                      \
@@ -979,6 +988,7 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_stream(const half_t* __restri
 #undef MI355_SM_STEP
 #undef MI355_SM_TIE8
 #undef MI355_SM_READ
+#undef MI355_SM_ACCW
 #undef MI355_SM_ACC
 #undef MI355_SM_MFMA0
 #undef MI355_SM_MFMA
