@@ -47,20 +47,20 @@ METRIC = "TFLOP/s & %MFMA peak (f16 GEMM, causal FA, MXFP4 GEMM); decode HBM GB/
 # dispatch, scaled by what the same counters read for a copy kernel of known size); filled in from
 # the summaries kept under profiles/.  None = not measured.
 MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
-    "gemm_8192": 1.783e9,              # 1572 MiB read + 128 MiB written: each of the 8 XCD L2s fetches its own copy of
+    "gemm_8192": 1.754e9,              # 1545 MiB read + 128 MiB written: each of the 8 XCD L2s fetches its own copy of
                                        # the panels its 4x8 block of output tiles needs (12 panels x 4 MiB x 4 rounds x 8)
-    "gemm_4096": 2.464e8,
-    "gemm_2048x10240x8192": 6.570e8,
-    "gemm_2048x57344x8192": 3.120e9,
+    "gemm_4096": 2.438e8,
+    "gemm_2048x10240x8192": 6.563e8,
+    "gemm_2048x57344x8192": 3.062e9,
     "gemm_1024_f32out": 1.684e7,
-    "gemm_bf16_8192": 1.783e9,
+    "gemm_bf16_8192": 1.754e9,
     "gemm_16x8192x8192": 1.366e8,
     "fa_causal": 3.425e8,
     "fa_noncausal": 2.686e8,
     "decode": 1.177e9,
     "fa_causal_bf16": 3.481e8,
     "decode_bf16": 1.177e9,
-    "mxfp4_4096x8192x8192": 3.011e8,
+    "mxfp4_4096x8192x8192": 2.958e8,
     "mxfp4_32x8192x8192": 3.739e7,
     "mxfp4_quantize_16384x16384": 6.796e8,
     "mxfp8_quantize_16384x16384": 8.138e8,
