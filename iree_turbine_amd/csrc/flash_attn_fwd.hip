@@ -567,16 +567,28 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 
   const float l_tot = l_run + __shfl_xor(l_run, 32);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-  if (q_ok) {
-    half_t* orow = Ob + (size_t)q_row * lay.o_r + 4 * h;
+  {
+    // Output through LDS (the K / V rings are idle: the last trip ended with a barrier): a lane holds 64 of its query's 128
+    // values in 4-value pieces; each wave assembles its 32 rows x 256 bytes in a private region (chunk c of row r in
+    // slot c ^ (r & 15)), reads whole 16-byte chunks back and stores full rows -- 8 stores of 16 bytes per lane instead
+    // of 16 of 8 bytes that each touch 32 rows.
+    char* ep = lds + wave * 8192;
 #pragma unroll
     for (int dt = 0; dt < 4; dt++)
 #pragma unroll
       for (int q = 0; q < 4; q++) {
         half4 v = {cvt16<BF>(oacc[dt][4 * q] * inv), cvt16<BF>(oacc[dt][4 * q + 1] * inv), cvt16<BF>(oacc[dt][4 * q + 2] * inv),
                    cvt16<BF>(oacc[dt][4 * q + 3] * inv)};
-        *reinterpret_cast<half4*>(orow + dt * 32 + q * 8) = v;
+        *reinterpret_cast<half4*>(ep + r32 * 256 + (((dt * 4 + q) ^ (r32 & 15)) * 16) + 8 * h) = v;
       }
+    const int er = lane >> 4, ec = lane & 15;
+#pragma unroll
+    for (int it = 0; it < 8; it++) {
+      const int row = it * 4 + er;
+      const half8 v = *reinterpret_cast<const half8*>(ep + row * 256 + ((ec ^ (row & 15)) * 16));
+      if (wq0 + row < Sq) *reinterpret_cast<half8*>(Ob + (size_t)(wq0 + row) * lay.o_r + ec * 8) = v;
+    }
+    if (CAUSAL) __syncthreads();  // the next pass loads K / V tiles over these regions
   }
   }  // pass
 }
