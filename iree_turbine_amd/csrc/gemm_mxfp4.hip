@@ -1550,7 +1550,7 @@ template <typename OutT>
 static int launch_mx_stream(const void* a, const void* as, const void* b, const void* bs, void* c, int M, int N, int K,
                             hipStream_t stream, bool one_per_cu) {
   auto kern = gemm_mxfp4_stream<OutT>;
-  constexpr int lds_bytes = 5 * 256 * 128;  // three B buffers and two A buffers of 32 KiB
+  constexpr int lds_bytes = 5 * 16384 + 2 * 32768 + 16384;  // five B half buffers, two A buffers, two scale groups
   static std::atomic<uint64_t> lds_ok{0};
   if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_mxfp4_stream")) return rc;
   const int tiles_m = M / 256, tiles_n = N / 256;

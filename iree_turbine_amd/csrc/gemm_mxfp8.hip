@@ -15,6 +15,10 @@
 // (its half of block ks) and chunk 4+2ks+h (its half of block 2+ks), and supplies byte ks (h = 0) or 2+ks
 // (h = 1) of the ONE scale dword a row has per slab; lanes of the upper half shift their dword right by 16
 // once, so that op_sel = ks picks the byte for both halves.
+//
+// The streamed kernel uses v_mfma_scale_f32_16x16x128_f8f6f4 instead, one instruction per 128-element slab row:
+// lane (r = l % 16, g = l / 16) supplies bytes 16g..16g+15 and 64+16g..64+16g+15 of row r (measured with
+// one-hot operands), and its scale byte is that of block g (k 32g..32g+31) of the slab.
 #include <math.h>
 #include <type_traits>
 
@@ -573,10 +577,437 @@ __global__ __launch_bounds__(256) void gemm_mxfp8_staged(const uint8_t* __restri
   }
 }
 
-static const char* kMx8Variants[] = {"tiled_256x256x128_w2x2", "generic_32x128", "staged_256x256x128_w2x2"};
-constexpr int kNumMx8Variants = 3;
+// Streamed form (see gemm_f16_nt_stream and gemm_mxfp4_stream for the reasoning; the LDS map, the load schedule and the
+// tile walk are those of the MXFP4 kernel).  A slab row is 128 bytes = 128 codes = 4 scale blocks = one k step of the
+// 16x16x128 MFMA: lane l supplies row l & 15 and the 16-byte chunks (l >> 4) and 4 + (l >> 4) of the row as one
+// 32-byte operand, and its scale byte is that of block l >> 4 of the slab.  The B fragments of a slab are held in
+// registers (read from LDS during the first two steps of the slab before), the A rows are streamed one 16-row
+// fragment per step, two steps ahead; a step is 8 MFMAs (one A fragment against the 8 B fragments).
+// LDS (160 KiB): B in a ring of five 16 KiB half buffers (U = rows 0..63, V = rows 64..127 of both 128-row halves), A
+// in two 32 KiB buffers freed block by block, 16 KiB for the scales.
+// Scales are staged through LDS in groups of four slabs: 16 bytes per row, one lane per row, 8 KiB per group (A rows,
+// then B rows), two buffers; a group is loaded in the first two steps of every fourth slab, three slabs before its
+// first read.  A lane fetches a scale with a one-byte LDS read (bits 0..7 of a register, as the MFMA wants it): the A
+// scale of a step next to its fragment, the 8 B scales of the next slab in steps 2..5.
+// One step = 8 MFMAs + LDS reads + two data loads; a barrier every 2 steps (an interval):
+//   interval q of slab t loads   A: block q - 1 of slab t + 2 (q = 0: block 3 of slab t + 1)
+//                                B: part q of slab t + 3 (parts 0, 1 -> its U half, parts 2, 3 -> its V half)
+// At a barrier every wave has waited for its loads older than the newest 15 and for its LDS reads older than the interval.
+// SCALED = false: every scale is 2^0 (no scale traffic) and the result is multiplied by alpha.
+template <typename OutT, bool SCALED>
+__global__ __launch_bounds__(256) void gemm_mxfp8_stream(const uint8_t* __restrict__ A, const uint8_t* __restrict__ As,
+                                                         const uint8_t* __restrict__ B, const uint8_t* __restrict__ Bs,
+                                                         OutT* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n,
+                                                         int group_m, float alpha) {
+  typedef _Float16 half8 __attribute__((ext_vector_type(8)));  // 16 opaque bytes
+  constexpr int BM = 256, BN = 256, WN = 2, WTM = 128, WTN = 128;
+  constexpr int HALF = 128 * 128, ABUF = 256 * 128, SGRP = 8192;
+  constexpr int B_AT = 0, A_AT = 5 * HALF, S_AT = A_AT + 2 * ABUF;
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  const int T = tiles_m * tiles_n, G = (int)gridDim.x;
+  int pid = blockIdx.x;
+  int tile_m, tile_n;
+  map_tile8(pid, tiles_m, tiles_n, group_m, tile_m, tile_n);
+
+  // One descriptor per array (each under 4 GiB, checked on the host); tile, slab and row block go into the scalar offset.
+  const unsigned row_bytes = (unsigned)K, SK = (unsigned)K / 32u;
+  const buffer_rsrc_t a_src = make_buffer(A, (unsigned)(tiles_m * BM) * row_bytes);
+  const buffer_rsrc_t b_src = make_buffer(B, (unsigned)(tiles_n * BN) * row_bytes);
+  const buffer_rsrc_t sa_src = make_buffer(SCALED ? As : A, (unsigned)(tiles_m * BM) * SK);
+  const buffer_rsrc_t sb_src = make_buffer(SCALED ? Bs : B, (unsigned)(tiles_n * BN) * SK);
+  const int lrow = lane >> 3;
+  // codes: a wave-load covers 8 rows x 128 bytes; lane = (row l >> 3, slot l & 7) fetches chunk slot ^ ((row >> 1) & 7)
+  const unsigned g_off = (unsigned)(wave * 8 + lrow) * row_bytes + (unsigned)((lane & 7) ^ (((wave & 1) << 2) | (lrow >> 1))) * 16u;
+  // scales: a wave-load covers rows 64 w .. 64 w + 63 of the tile, 16 bytes (four slabs) per lane
+  const unsigned gs_off = (unsigned)(wave * 64 + lane) * SK;
+  const int KT = K / 128;  // a multiple of 4, >= 8 (checked on the host)
+  unsigned a_cur = (unsigned)(tile_m * BM) * row_bytes, b_cur = (unsigned)(tile_n * BN) * row_bytes;
+  unsigned a_nxt = a_cur, b_nxt = b_cur;  // the next tile (after the last: itself again; those loads are never used)
+  unsigned sa_cur = (unsigned)(tile_m * BM) * SK, sb_cur = (unsigned)(tile_n * BN) * SK, sa_nxt = sa_cur, sb_nxt = sb_cur;
+  auto slab_at = [&](int s, unsigned cur, unsigned nxt) { return s < KT ? cur + (unsigned)s * 128u : nxt + (unsigned)(s - KT) * 128u; };
+  auto grp_at = [&](int s, unsigned cur, unsigned nxt) { return s < KT ? cur + (unsigned)s * 4u : nxt + (unsigned)(s - KT) * 4u; };
+  // offsets of the slabs 1, 2 (A) and 3 (B) ahead and of the scale group after this one; those of the next slab are
+  // worked out one per step in the second half of a slab
+  unsigned a_off1 = a_cur + 128u, a_off2 = a_cur + 256u, b_off3 = b_cur + 384u, sa_off = sa_cur + 16u, sb_off = sb_cur + 16u;
+  unsigned n_a1 = 0, n_a2 = 0, n_b3 = 0, n_sa = 0, n_sb = 0;
+  auto load_a = [&](int buf, int h, int blk, unsigned at) {
+    buffer_load_lds_16B(a_src, g_off, (unsigned)(h * 128 + blk * 32) * row_bytes + at,
+                        lds + A_AT + buf * ABUF + (h * 16 + blk * 4 + wave) * 1024);
+  };
+  // part p (rows 32 p .. 32 p + 31 of either 128-row half) into the half buffer at byte offset half_at
+  auto load_b = [&](int half_at, int h, int part, unsigned at) {
+    buffer_load_lds_16B(b_src, g_off, (unsigned)(h * 128 + part * 32) * row_bytes + at,
+                        lds + B_AT + half_at + (h * 8 + (part & 1) * 4 + wave) * 1024);
+  };
+  auto load_scales = [&](bool is_b, int grp_at_lds, unsigned at) {
+    buffer_load_lds_16B(is_b ? sb_src : sa_src, gs_off, at, lds + S_AT + grp_at_lds + (is_b ? 4096 : 0) + wave * 1024);
+  };
+
+  // fragment reads: lane l takes row l & 15 of a 16-row block, chunks (l >> 4) and 4 + (l >> 4) of the 128-byte row
+  const int r16 = lane & 15, cq = lane >> 4;
+  const unsigned lds0 = (unsigned)(uintptr_t)MI355_LDS(char, lds);
+  const unsigned lane_rd = (unsigned)(r16 * 128 + ((cq ^ (r16 >> 1)) & 7) * 16);  // upper chunk: ^ 64
+  unsigned aaddr[2][2];  // [A buffer][lower / upper chunk]
+#pragma unroll
+  for (int bf = 0; bf < 2; bf++)
+#pragma unroll
+    for (int kh = 0; kh < 2; kh++) aaddr[bf][kh] = lds0 + A_AT + bf * ABUF + wm * (WTM * 128) + (lane_rd ^ (kh * 64));
+  const unsigned b_lane = lds0 + B_AT + wn * (64 * 128) + lane_rd;  // 64 rows of either half per half buffer
+  unsigned bU[2], bV[2];  // [lower / upper chunk]: the U and V half buffers read in this slab
+  // scale reads: the byte of row (16 rb + r16), slab s, block cq sits at row * 16 + 4 (s & 3) + cq of the slab's group
+  const unsigned sa_lane = lds0 + S_AT + (unsigned)((wm * WTM + r16) * 16 + cq);
+  const unsigned sb_lane = lds0 + S_AT + 4096 + (unsigned)((wn * WTN + r16) * 16 + cq);
+  unsigned sa_rd = sa_lane, sa_rdn = sa_lane + 4, sb_rdn = sb_lane + 4;  // this slab's A scales, the next slab's A and B
+
+  // [n block][m block].  Never cleared: the MFMAs of a tile's first slab take a zero addend instead -- a register write
+  // in front of an inline-assembly MFMA would need wait states the compiler does not know to insert.
+  floatx4 acc[8][8];
+  intx4 fbl0[8], fbh0[8], fbl1[8], fbh1[8];  // B fragments as read (lower, upper chunk) for the two slab parities
+  intx8 fb0[8], fb1[8];                       // ... as MFMA operands
+  intx4 fal[4], fah[4];                       // A fragments by step
+  int sb0[8], sb1[8], sat[4];                 // B scales of the two slab parities; A scales by step
+  if constexpr (!SCALED) {
+#pragma unroll
+    for (int i = 0; i < 8; i++) sb0[i] = sb1[i] = 127;
+#pragma unroll
+    for (int i = 0; i < 4; i++) sat[i] = 127;
+  }
+
+#define MI355_S8_CAT(lo, hi) __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7)
+  // MFMAs as inline assembly with the accumulators pinned to AGPRs.  No MFMA here reads an accumulator written fewer
+  // than 64 MFMAs earlier.  x, sx: B codes and scale (bits 0..7); y, sy: A codes and scale.
+#define MI355_S8_ACC(ZERO, c, x, sx, y, sy)                                                               \
+  do {                                                                                                    \
+    if constexpr (ZERO)                                                                                   \
+      asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, 0, %3, %4 op_sel_hi:[0,0,0]"            \
+                   : "=a"(c) : "v"(x), "v"(y), "v"(sx), "v"(sy));                                         \
+    else                                                                                                  \
+      asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0]"           \
+                   : "+a"(c) : "v"(x), "v"(y), "v"(sx), "v"(sy));                                         \
+  } while (0)
+  // The first MFMA of a step together with the wait for the step's A fragment and scale (requested two steps earlier;
+  // LG = LDS reads issued since).  One statement, with the registers as plain inputs: a separate wait statement that
+  // names them as outputs makes the compiler put a wait state in front of their next use.
+#define MI355_S8_ACCW(ZERO, LG, c, x, sx, y, sy)                                                                         \
+  do {                                                                                                                   \
+    if constexpr (ZERO)                                                                                                  \
+      asm volatile("s_waitcnt lgkmcnt(%5)\n\tv_mfma_scale_f32_16x16x128_f8f6f4 %0, %3, %1, 0, %4, %2 op_sel_hi:[0,0,0]"   \
+                   : "=a"(c) : "v"(y), "v"(sy), "v"(x), "v"(sx), "n"(LG));                                               \
+    else                                                                                                                 \
+      asm volatile("s_waitcnt lgkmcnt(%5)\n\tv_mfma_scale_f32_16x16x128_f8f6f4 %0, %3, %1, %0, %4, %2 op_sel_hi:[0,0,0]"  \
+                   : "+a"(c) : "v"(y), "v"(sy), "v"(x), "v"(sx), "n"(LG));                                               \
+  } while (0)
+#define MI355_S8_READ(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off))
+#define MI355_S8_READ8(dst, addr, off) asm volatile("ds_read_u8 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off))
+#define MI355_S8_TIE8(X) "+v"(X[0]), "+v"(X[1]), "+v"(X[2]), "+v"(X[3]), "+v"(X[4]), "+v"(X[5]), "+v"(X[6]), "+v"(X[7])
+#define MI355_S8_TIE4(X) "+v"(X[0]), "+v"(X[1]), "+v"(X[2]), "+v"(X[3])
+
+  // ---- prologue: B0 (half buffers 0, 1), A0, B1 (2, 3), A1 blocks 0..2, scale group 0 ----
+#pragma unroll
+  for (int x = 0; x < 8; x++) load_b((x >> 2) * HALF, x & 1, x >> 1, b_cur);
+#pragma unroll
+  for (int x = 0; x < 8; x++) load_a(0, x & 1, x >> 1, a_cur);
+#pragma unroll
+  for (int x = 0; x < 8; x++) load_b((2 + (x >> 2)) * HALF, x & 1, x >> 1, b_cur + 128u);
+#pragma unroll
+  for (int x = 0; x < 6; x++) load_a(1, x & 1, x >> 1, a_cur + 128u);
+  if constexpr (SCALED) {
+    load_scales(false, 0, sa_cur);
+    load_scales(true, 0, sb_cur);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+  bU[0] = b_lane; bU[1] = b_lane ^ 64;
+  bV[0] = b_lane + HALF; bV[1] = bV[0] ^ 64;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    MI355_S8_READ(fbl0[i], bU[0], i * 2048); MI355_S8_READ(fbh0[i], bU[1], i * 2048);
+    MI355_S8_READ(fbl0[4 + i], bV[0], i * 2048); MI355_S8_READ(fbh0[4 + i], bV[1], i * 2048);
+  }
+  MI355_S8_READ(fal[0], aaddr[0][0], 0); MI355_S8_READ(fah[0], aaddr[0][1], 0);
+  MI355_S8_READ(fal[1], aaddr[0][0], 2048); MI355_S8_READ(fah[1], aaddr[0][1], 2048);
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : MI355_S8_TIE8(fbl0), MI355_S8_TIE8(fbh0), "+v"(fal[0]), "+v"(fah[0]), "+v"(fal[1]), "+v"(fah[1]));
+  if constexpr (SCALED) {
+#pragma unroll
+    for (int i = 0; i < 8; i++) MI355_S8_READ8(sb0[i], sb_lane, i * 256);
+    MI355_S8_READ8(sat[0], sa_lane, 0); MI355_S8_READ8(sat[1], sa_lane, 256);
+    asm volatile("s_waitcnt lgkmcnt(0)" : MI355_S8_TIE8(sb0), "+v"(sat[0]), "+v"(sat[1]));
+  }
+#pragma unroll
+  for (int i = 0; i < 8; i++) fb0[i] = MI355_S8_CAT(fbl0[i], fbh0[i]);
+  __builtin_amdgcn_s_barrier();  // every wave has read B0: its half buffers may receive slab 2's V half (0) and slab 3's U half (1)
+  __builtin_amdgcn_sched_barrier(0);
+  // B2: U half -> half buffer 4, V half -> half buffer 0
+#pragma unroll
+  for (int x = 0; x < 8; x++) load_b(((4 + (x >> 2)) % 5) * HALF, x & 1, x >> 1, b_cur + 256u);
+  __builtin_amdgcn_sched_barrier(0);
+
+  // B ring: slab t's halves live in half buffers (2 t) % 5 and (2 t + 1) % 5; pos = (2 t) % 5 for the current slab t
+  int pos = 0;
+  int sg_ld = SGRP;  // LDS offset of the scale group buffer the next group goes to (groups alternate)
+
+  // Step j of slab phase PH (slab index mod 4; A buffer PH & 1): the MFMAs of m block j on fal/fah[j % 4], sat[j % 4]
+  // against FB / SB[0..7].  LGKM = LDS reads issued after those of step j - 2 (which filled this step's fragment).
+#define MI355_S8_STEP(j, PH, FB, FBNL, FBNH, SB, SBN, LGKM, FIRST)                                                      \
+  do {                                                                                                                 \
+    constexpr int PAR = (PH)&1, j2 = (j) + 2, nb = j2 >= 8 ? 1 - PAR : PAR, nj = j2 & 7;                                \
+    const intx8 ya = MI355_S8_CAT(fal[(j)&3], fah[(j)&3]);                                                             \
+    MI355_S8_ACCW(FIRST, LGKM, acc[0][j], FB[0], SB[0], ya, sat[(j)&3]);                                               \
+    MI355_S8_READ(fal[j2 & 3], aaddr[nb][0], nj * 2048);                                                               \
+    MI355_S8_READ(fah[j2 & 3], aaddr[nb][1], nj * 2048);                                                               \
+    __builtin_amdgcn_sched_barrier(0);                                                                                 \
+    MI355_S8_ACC(FIRST, acc[1][j], FB[1], SB[1], ya, sat[(j)&3]);                                                      \
+    if constexpr (SCALED) {                                                                                            \
+      if constexpr (j2 >= 8) MI355_S8_READ8(sat[j2 & 3], sa_rdn, nj * 256);                                            \
+      else MI355_S8_READ8(sat[j2 & 3], sa_rd, nj * 256);                                                               \
+    }                                                                                                                  \
+    __builtin_amdgcn_sched_barrier(0);                                                                                 \
+    MI355_S8_ACC(FIRST, acc[2][j], FB[2], SB[2], ya, sat[(j)&3]);                                                      \
+    if constexpr ((j) < 2) {                                                                                           \
+      MI355_S8_READ(FBNL[4 * (j)], ((j) ? bV : bU)[0], 0 * 2048);                                                      \
+      MI355_S8_READ(FBNH[4 * (j)], ((j) ? bV : bU)[1], 0 * 2048);                                                      \
+      MI355_S8_READ(FBNL[4 * (j) + 1], ((j) ? bV : bU)[0], 1 * 2048);                                                  \
+      MI355_S8_READ(FBNH[4 * (j) + 1], ((j) ? bV : bU)[1], 1 * 2048);                                                  \
+    } else if constexpr (SCALED && (j) < 6) {                                                                          \
+      MI355_S8_READ8(SBN[2 * ((j)-2)], sb_rdn, (2 * ((j)-2)) * 256);                                                   \
+    }                                                                                                                  \
+    __builtin_amdgcn_sched_barrier(0);                                                                                 \
+    MI355_S8_ACC(FIRST, acc[3][j], FB[3], SB[3], ya, sat[(j)&3]);                                                      \
+    if constexpr ((j) < 2) {                                                                                           \
+      MI355_S8_READ(FBNL[4 * (j) + 2], ((j) ? bV : bU)[0], 2 * 2048);                                                  \
+      MI355_S8_READ(FBNH[4 * (j) + 2], ((j) ? bV : bU)[1], 2 * 2048);                                                  \
+      MI355_S8_READ(FBNL[4 * (j) + 3], ((j) ? bV : bU)[0], 3 * 2048);                                                  \
+      MI355_S8_READ(FBNH[4 * (j) + 3], ((j) ? bV : bU)[1], 3 * 2048);                                                  \
+    } else if constexpr (SCALED && (j) < 6) {                                                                          \
+      MI355_S8_READ8(SBN[2 * ((j)-2) + 1], sb_rdn, (2 * ((j)-2) + 1) * 256);                                           \
+    }                                                                                                                  \
+    __builtin_amdgcn_sched_barrier(0);                                                                                 \
+    MI355_S8_ACC(FIRST, acc[4][j], FB[4], SB[4], ya, sat[(j)&3]);                                                      \
+    {                                                                                                                  \
+      constexpr int q = (j) >> 1;                                                                                      \
+      /* the scale group after this one: A rows in step 0, B rows in step 1 of every fourth slab */                   \
+      if constexpr (SCALED && (PH) == 0 && (j) == 0) load_scales(false, sg_ld, sa_off);                                \
+      if constexpr (SCALED && (PH) == 0 && (j) == 1) load_scales(true, sg_ld, sb_off);                                 \
+      if constexpr (((j)&1) == 0) {                                                                                    \
+        if constexpr (q == 0) load_a(1 - PAR, 0, 3, a_off1);                                                           \
+        else load_a(PAR, 0, q - 1, a_off2);                                                                            \
+      } else {                                                                                                         \
+        load_b(q < 2 ? ld_u : ld_v, 0, q, b_off3);                                                                     \
+      }                                                                                                                \
+    }                                                                                                                  \
+    __builtin_amdgcn_sched_barrier(0);                                                                                 \
+    MI355_S8_ACC(FIRST, acc[5][j], FB[5], SB[5], ya, sat[(j)&3]);                                                      \
+    {                                                                                                                  \
+      constexpr int q = (j) >> 1;                                                                                      \
+      if constexpr (((j)&1) == 0) {                                                                                    \
+        if constexpr (q == 0) load_a(1 - PAR, 1, 3, a_off1);                                                           \
+        else load_a(PAR, 1, q - 1, a_off2);                                                                            \
+      } else {                                                                                                         \
+        load_b(q < 2 ? ld_u : ld_v, 1, q, b_off3);                                                                     \
+      }                                                                                                                \
+    }                                                                                                                  \
+    __builtin_amdgcn_sched_barrier(0);                                                                                 \
+    if constexpr ((j) == 3) n_a1 = slab_at(kt + 2, a_cur, a_nxt);                                                      \
+    if constexpr ((j) == 4) n_a2 = slab_at(kt + 3, a_cur, a_nxt);                                                      \
+    if constexpr ((j) == 5) n_b3 = slab_at(kt + 4, b_cur, b_nxt);                                                      \
+    if constexpr (SCALED && (PH) == 3 && (j) == 6) n_sa = grp_at(kt + 5, sa_cur, sa_nxt);                              \
+    if constexpr (SCALED && (PH) == 3 && (j) == 7) n_sb = grp_at(kt + 5, sb_cur, sb_nxt);                              \
+    MI355_S8_ACC(FIRST, acc[6][j], FB[6], SB[6], ya, sat[(j)&3]);                                                      \
+    MI355_S8_ACC(FIRST, acc[7][j], FB[7], SB[7], ya, sat[(j)&3]);                                                      \
+    __builtin_amdgcn_sched_barrier(0);                                                                                 \
+  } while (0)
+  // End of an interval: loads older than the newest VMC and LDS reads older than the interval are complete in every wave.
+#define MI355_S8_SYNC(RD, VMC)                                                      \
+  do {                                                                              \
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(%1)" ::"n"(VMC), "n"(RD) : "memory"); \
+    __builtin_amdgcn_s_barrier();                                                   \
+    __builtin_amdgcn_sched_barrier(0);                                              \
+  } while (0)
+  // LDS reads per step: A fragment (2) and scale (1) + 8 for four B fragments in steps 0, 1 or 2 B scales in steps 2..5.
+  constexpr int RA = SCALED ? 3 : 2, RB = SCALED ? 2 : 0;
+#define MI355_S8_SLAB(PH, FB, FBNL, FBNH, FBN, SB, SBN, FIRST, VMC)                                              \
+  do {                                                                                                          \
+    {                                                                                                           \
+      const int pu = pos + 2 >= 5 ? pos - 3 : pos + 2, pv = pos + 3 >= 5 ? pos - 2 : pos + 3; /* slab t + 1 */   \
+      bU[0] = b_lane + (unsigned)(pu * HALF);                                                                   \
+      bU[1] = bU[0] ^ 64;                                                                                       \
+      bV[0] = b_lane + (unsigned)(pv * HALF);                                                                   \
+      bV[1] = bV[0] ^ 64;                                                                                       \
+    }                                                                                                           \
+    /* slab t + 3: U half -> (2 t + 6) % 5 = pos + 1, V half -> (2 t + 7) % 5 = pos + 2 */                       \
+    const int ld_u = (pos + 1 >= 5 ? pos - 4 : pos + 1) * HALF, ld_v = (pos + 2 >= 5 ? pos - 3 : pos + 2) * HALF; \
+    MI355_S8_STEP(0, PH, FB, FBNL, FBNH, SB, SBN, RA, FIRST);                                                   \
+    MI355_S8_STEP(1, PH, FB, FBNL, FBNH, SB, SBN, RA + 8, FIRST);                                               \
+    MI355_S8_SYNC(15, VMC);                                                                                     \
+    MI355_S8_STEP(2, PH, FB, FBNL, FBNH, SB, SBN, RA + 8, FIRST);                                               \
+    MI355_S8_STEP(3, PH, FB, FBNL, FBNH, SB, SBN, RA + RB, FIRST);                                              \
+    MI355_S8_SYNC(2 * (RA + RB), VMC);                                                                          \
+    MI355_S8_STEP(4, PH, FB, FBNL, FBNH, SB, SBN, RA + RB, FIRST);                                              \
+    MI355_S8_STEP(5, PH, FB, FBNL, FBNH, SB, SBN, RA + RB, FIRST);                                              \
+    MI355_S8_SYNC(2 * (RA + RB), VMC);                                                                          \
+    MI355_S8_STEP(6, PH, FB, FBNL, FBNH, SB, SBN, RA + RB, FIRST);                                              \
+    MI355_S8_STEP(7, PH, FB, FBNL, FBNH, SB, SBN, RA, FIRST);                                                   \
+    /* the next slab's B fragments and scales were requested in steps 0..5: they have landed; tie them here */  \
+    asm volatile("s_waitcnt vmcnt(%24) lgkmcnt(%25)"                                                            \
+                 : MI355_S8_TIE8(FBNL), MI355_S8_TIE8(FBNH), MI355_S8_TIE8(SBN)                                 \
+                 : "n"(VMC), "n"(2 * RA) : "memory");                                                           \
+    _Pragma("unroll") for (int i_ = 0; i_ < 8; i_++) FBN[i_] = MI355_S8_CAT(FBNL[i_], FBNH[i_]);                \
+    __builtin_amdgcn_s_barrier();                                                                               \
+    __builtin_amdgcn_sched_barrier(0);                                                                          \
+    a_off1 = n_a1;                                                                                              \
+    a_off2 = n_a2;                                                                                              \
+    b_off3 = n_b3;                                                                                              \
+    pos = pos + 2 >= 5 ? pos - 3 : pos + 2;                                                                     \
+    /* the scale reads of the slabs after this one: 4 bytes on per slab; slab 4 g starts group g's buffer */    \
+    sa_rd = sa_rdn;                                                                                             \
+    if constexpr ((PH) == 2) {                                                                                  \
+      sa_rdn = sa_lane + (unsigned)sg_ld;                                                                       \
+      sb_rdn = sb_lane + (unsigned)sg_ld;                                                                       \
+    } else {                                                                                                    \
+      sa_rdn = sa_rdn + 4;                                                                                      \
+      sb_rdn = sb_rdn + 4;                                                                                      \
+    }                                                                                                           \
+    if constexpr ((PH) == 3) {                                                                                  \
+      sg_ld ^= SGRP;                                                                                            \
+      sa_off = n_sa;                                                                                            \
+      sb_off = n_sb;                                                                                            \
+    }                                                                                                           \
+  } while (0)
+
+  for (; pid < T; pid += G) {
+    int nxt_m = tile_m, nxt_n = tile_n;
+    if (pid + G < T) map_tile8(pid + G, tiles_m, tiles_n, group_m, nxt_m, nxt_n);
+    a_nxt = (unsigned)(nxt_m * BM) * row_bytes;
+    b_nxt = (unsigned)(nxt_n * BN) * row_bytes;
+    sa_nxt = (unsigned)(nxt_m * BM) * SK;
+    sb_nxt = (unsigned)(nxt_n * BN) * SK;
+    // In a tile's first slab the 32 stores of the epilogue before it sit in the queue behind the loads the waits are
+    // about (a 32-bit epilogue, 64 stores, drains the queue instead).
+    constexpr int VMC_FIRST = sizeof(OutT) == 2 ? 15 + 32 : 15;
+    int kt = 0;
+    MI355_S8_SLAB(0, fb0, fbl1, fbh1, fb1, sb0, sb1, true, VMC_FIRST);
+    kt = 1;
+    MI355_S8_SLAB(1, fb1, fbl0, fbh0, fb0, sb1, sb0, false, 15);
+    kt = 2;
+    MI355_S8_SLAB(2, fb0, fbl1, fbh1, fb1, sb0, sb1, false, 15);
+    kt = 3;
+    MI355_S8_SLAB(3, fb1, fbl0, fbh0, fb0, sb1, sb0, false, 15);
+    for (kt = 4; kt < KT; kt += 4) {
+      MI355_S8_SLAB(0, fb0, fbl1, fbh1, fb1, sb0, sb1, false, 15);
+      kt++;
+      MI355_S8_SLAB(1, fb1, fbl0, fbh0, fb0, sb1, sb0, false, 15);
+      kt++;
+      MI355_S8_SLAB(2, fb0, fbl1, fbh1, fb1, sb0, sb1, false, 15);
+      kt++;
+      MI355_S8_SLAB(3, fb1, fbl0, fbh0, fb0, sb1, sb0, false, 15);
+      kt -= 3;
+    }
+    // ---- epilogue ----
+    // The MFMAs are inline assembly, so the compiler does not know that the accumulators were written just now: the
+    // wait states an MFMA result needs before another instruction may read it are spelled out, and every accumulator is
+    // tied to a statement behind them so that no read of it can be scheduled earlier.
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+      asm volatile("" : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]), "+a"(acc[i][4]), "+a"(acc[i][5]),
+                        "+a"(acc[i][6]), "+a"(acc[i][7]));
+    // lane holds, for m = 16 j + (l & 15): n = 16 i + 4 (l >> 4) + r, r < 4.  The addresses come from a lane id the
+    // compiler cannot see through, so that none of them is computed ahead of the K loop and kept across it.
+    const int le = opaque_lane_id();
+    const int r16e = le & 15, cqe = le >> 4;
+    if constexpr (sizeof(OutT) == 2) {
+      // bf16 results go through LDS, 16 rows x 64 columns (2 KiB) per pass in a wave-private region: 8-byte writes of 4
+      // consecutive n (chunk slot c ^ ((m >> 1) & 7) of the 128-byte row), whole rows read back 16 bytes per lane and
+      // stored as full cache lines.  LDS operations of a wave execute in order, so the passes need no waits between
+      // them.  The next tile's slabs are landing in LDS meanwhile; free at this point is block 3 of A buffer 1 (rows
+      // 96..127 of either half: twice 4 KiB), which the next loads reach only after the barrier below.  Inline
+      // assembly like the K loop's LDS accesses: direct-to-LDS loads are in flight.
+      const unsigned ep = lds0 + (unsigned)(A_AT + ABUF + (wave < 2 ? 12 * 1024 + wave * 2048 : 28 * 1024 + (wave - 2) * 2048));
+      const int er = le >> 3, ec = le & 7, sw = (r16e >> 1) & 7;
+      // write: row r16e, chunk (2 (i & 3) + (cqe >> 1)) ^ sw, 8-byte half cqe & 1; the i term is an XOR of the address
+      const unsigned wa = ep + (unsigned)(r16e * 128 + ((((cqe >> 1) ^ (sw & 1)) | (sw & 6)) * 16) + 8 * (cqe & 1));
+      // read: row 8 it + er, chunk ec ^ ((row >> 1) & 7) = (ec ^ (er >> 1)) ^ 4 it
+      const unsigned ra = ep + (unsigned)(er * 128 + ((ec ^ (er >> 1)) * 16));
+      OutT* cbase = C + (size_t)(tile_m * BM + wm * WTM + er) * N + tile_n * BN + wn * WTN + ec * 8;
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+#pragma unroll
+        for (int ih = 0; ih < 2; ih++) {
+#pragma unroll
+          for (int ii = 0; ii < 4; ii++) {
+            const int i = ih * 4 + ii;
+            ushortx4 v = {f32_to_bf16_rne(alpha * acc[i][j][0]), f32_to_bf16_rne(alpha * acc[i][j][1]),
+                          f32_to_bf16_rne(alpha * acc[i][j][2]), f32_to_bf16_rne(alpha * acc[i][j][3])};
+            asm volatile("ds_write_b64 %0, %1" ::"v"(wa ^ (unsigned)(32 * ii)), "v"(v) : "memory");
+          }
+          half8 rv[2];
+          asm volatile("ds_read_b128 %0, %1" : "=v"(rv[0]) : "v"(ra));
+          asm volatile("ds_read_b128 %0, %1 offset:1024" : "=v"(rv[1]) : "v"(ra ^ 64u));
+          asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(rv[0]), "+v"(rv[1]));
+#pragma unroll
+          for (int it = 0; it < 2; it++) *reinterpret_cast<half8*>(cbase + (size_t)(j * 16 + it * 8) * N + ih * 64) = rv[it];
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    } else {
+      OutT* crow = C + (size_t)(tile_m * BM + wm * WTM + r16e) * N + tile_n * BN + wn * WTN + 4 * cqe;
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+          Out8<OutT>::store4(crow + (size_t)(j * 16) * N + i * 16, alpha * acc[i][j][0], alpha * acc[i][j][1],
+                             alpha * acc[i][j][2], alpha * acc[i][j][3]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // 64 stores: more than a wait can count past
+    }
+    a_cur = a_nxt;
+    b_cur = b_nxt;
+    sa_cur = sa_nxt;
+    sb_cur = sb_nxt;
+    tile_m = nxt_m;
+    tile_n = nxt_n;
+    // the waves leave the epilogue together: the next loads reach the LDS the other waves' epilogues use
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  // the loads issued for a tile that does not exist still target LDS: let them land before the workgroup ends
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : MI355_S8_TIE4(fal), MI355_S8_TIE4(fah), MI355_S8_TIE4(sat));
+#undef MI355_S8_SLAB
+#undef MI355_S8_SYNC
+#undef MI355_S8_STEP
+#undef MI355_S8_TIE4
+#undef MI355_S8_TIE8
+#undef MI355_S8_READ8
+#undef MI355_S8_READ
+#undef MI355_S8_ACCW
+#undef MI355_S8_ACC
+#undef MI355_S8_CAT
+}
+
+static const char* kMx8Variants[] = {"tiled_256x256x128_w2x2", "generic_32x128", "staged_256x256x128_w2x2",
+                                     "stream_256x256x128_w2x2", "stream_256x256x128_w2x2_walk"};
+constexpr int kNumMx8Variants = 5;
 int mxfp8_variant_count() { return kNumMx8Variants; }
 const char* mxfp8_variant_name(int i) { return (i >= 0 && i < kNumMx8Variants) ? kMx8Variants[i] : nullptr; }
+
+static int mx8_cu_count() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
 
 template <typename OutT, bool SCALED>
 static int launch_mx8(int variant, const void* a, const void* as, const void* b, const void* bs, void* c, int M, int N, int K,
@@ -603,6 +1034,23 @@ static int launch_mx8(int variant, const void* a, const void* as, const void* b,
                        (const uint8_t*)bs, (OutT*)c, M, N, K, tiles_m, tiles_n, 4, alpha);
     return check_launch("gemm_mxfp8_staged", grid, block, lds_bytes);
   }
+  if (variant == 3 || variant == 4) {
+    auto kern = gemm_mxfp8_stream<OutT, SCALED>;
+    constexpr int lds_bytes = 5 * 16384 + 2 * 32768 + 16384;  // five B half buffers, two A buffers, two scale groups
+    static std::atomic<uint64_t> lds_ok{0};
+    if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_mxfp8_stream")) return rc;
+    const int tiles_m = M / 256, tiles_n = N / 256;
+    int wgs = tiles_m * tiles_n;
+    if (variant == 4) {  // one workgroup per CU walks its tiles
+      int g = mx8_cu_count() & ~7;  // multiples of 8 keep a workgroup's tiles on the XCD it runs on
+      if (g < 8) g = 8;
+      if (wgs > g) wgs = g;
+    }
+    dim3 grid(wgs), block(256);
+    hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const uint8_t*)a, (const uint8_t*)as, (const uint8_t*)b,
+                       (const uint8_t*)bs, (OutT*)c, M, N, K, tiles_m, tiles_n, 4, alpha);
+    return check_launch("gemm_mxfp8_stream", grid, block, lds_bytes);
+  }
   dim3 grid((N + 127) / 128, (M + 31) / 32), block(256);
   hipLaunchKernelGGL((gemm_mxfp8_generic<OutT, SCALED>), grid, block, 0, stream, (const uint8_t*)a, (const uint8_t*)as,
                      (const uint8_t*)b, (const uint8_t*)bs, (OutT*)c, M, N, K, alpha);
@@ -626,7 +1074,16 @@ extern "C" int mi355_mxfp8_gemm(const void* a, const void* a_scale, const void* 
   const bool sc_al4 = ((reinterpret_cast<uintptr_t>(a_scale) | reinterpret_cast<uintptr_t>(b_scale)) & 3u) == 0;
   const bool fits0 = sc_al4 && M % 256 == 0 && N % 256 == 0 && K % 256 == 0 && K >= 256;  // slabs in pairs, one scale dword per slab
   const bool fits2 = fits0 && K >= 512 && K <= (1 << 23);  // four slabs in flight; 32-bit buffer offsets
-  if (variant < 0) variant = fits2 ? 2 : fits0 ? 0 : 1;
+  // streamed: scale groups of four slabs (16-byte loads), the look-ahead stays within the next tile, one descriptor per array
+  const bool sc_al16 = ((reinterpret_cast<uintptr_t>(a_scale) | reinterpret_cast<uintptr_t>(b_scale)) & 15u) == 0;
+  const bool fits3 = sc_al16 && M % 256 == 0 && N % 256 == 0 && K % 512 == 0 && K >= 1024 && M * K < (int64_t(1) << 32) &&
+                     N * K < (int64_t(1) << 32);
+  // streamed, one workgroup per CU walking its tiles: 4096x8192x8192 200 us against 233 for the staged kernel
+  if (variant < 0) variant = fits3 ? 4 : fits2 ? 2 : fits0 ? 0 : 1;
+  else if ((variant == 3 || variant == 4) && !fits3)
+    return fail(-MI355_E_SHAPE,
+                "mxfp8_gemm: variant %s needs M%%256==0, N%%256==0, K%%512==0, K >= 1024, 16-byte aligned scales and a, b under 4 GiB",
+                kMx8Variants[variant]);
   else if (variant == 0 && !fits0)
     return fail(-MI355_E_SHAPE, "mxfp8_gemm: variant %s needs M%%256==0, N%%256==0, K%%256==0 and 4-byte aligned scales", kMx8Variants[0]);
   else if (variant == 2 && !fits2)
@@ -650,7 +1107,12 @@ extern "C" int mi355_fp8_gemm(const void* a, const void* b, void* c, int64_t M, 
   if (!aligned16(a) || !aligned16(b) || !aligned16(c)) return fail(-MI355_E_ALIGN, "fp8_gemm: a, b, c must be 16-byte aligned");
   const bool fits0 = M % 256 == 0 && N % 256 == 0 && K % 256 == 0 && K >= 256;
   const bool fits2 = fits0 && K >= 512 && K <= (1 << 23);
-  if (variant < 0) variant = fits2 ? 2 : fits0 ? 0 : 1;
+  const bool fits3 = M % 256 == 0 && N % 256 == 0 && K % 512 == 0 && K >= 1024 && M * K < (int64_t(1) << 32) && N * K < (int64_t(1) << 32);
+  // streamed, one workgroup per CU walking its tiles: 4096x8192x8192 200 us against 233 for the staged kernel
+  if (variant < 0) variant = fits3 ? 4 : fits2 ? 2 : fits0 ? 0 : 1;
+  else if ((variant == 3 || variant == 4) && !fits3)
+    return fail(-MI355_E_SHAPE, "fp8_gemm: variant %s needs M%%256==0, N%%256==0, K%%512==0, K >= 1024 and a, b under 4 GiB",
+                kMx8Variants[variant]);
   else if (variant == 0 && !fits0)
     return fail(-MI355_E_SHAPE, "fp8_gemm: variant %s needs M%%256==0, N%%256==0, K%%256==0", kMx8Variants[0]);
   else if (variant == 2 && !fits2)

@@ -48,7 +48,7 @@ def test_mxfp8_decode_exhaustive(dev):
         assert np.array_equal(np.signbit(c[:, 0].numpy())[nz], np.signbit(want)[nz]), sc
 
 
-@pytest.mark.parametrize("variant", [-1, 0, 1, 2])
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 3, 4])
 def test_mxfp8_gemm_variants(dev, variant):
     import iree_turbine_amd  # noqa: F401
     from oracle import inputs, mxfp8 as o8
@@ -103,7 +103,7 @@ def test_mxfp8_one_hot_layout(dev):
 
 
 def test_mxfp8_full_size_cross_variant(dev):
-    import iree_turbine_amd  # noqa: F401
+    import iree_turbine_amd as ita
     from oracle import inputs, mxfp8 as o8
 
     M, N, K = 2048, 4096, 4096
@@ -120,6 +120,11 @@ def test_mxfp8_full_size_cross_variant(dev):
     staged = torch.ops.mi355.mxfp8_gemm(a, asc, b, bsc, "float32", 2)
     assert torch.equal(staged, tiled)
     assert torch.equal(staged, torch.ops.mi355.mxfp8_gemm(a, asc, b, bsc, "float32", 2))
+    # the streamed kernel takes a whole 128-element slab per instruction
+    names = ita._lib.variants("mxfp8_gemm")
+    stream = torch.ops.mi355.mxfp8_gemm(a, asc, b, bsc, "float32", names.index("stream_256x256x128_w2x2_walk"))
+    assert _rel_err(stream, generic) < HW_SUM
+    assert torch.equal(stream, torch.ops.mi355.mxfp8_gemm(a, asc, b, bsc, "float32", -1))  # the automatic choice at this size
 
 
 @pytest.mark.parametrize("out_dtype", ["float32", "bfloat16"])
@@ -142,6 +147,64 @@ def test_mxfp8_staged_slab_rotation(dev, shape, out_dtype):
     rows = torch.tensor([0, 127, 128, M - 1])
     ref = o8.mxfp8_gemm_ref(a[rows.to(dev)].cpu(), asc[rows.to(dev)].cpu(), b.cpu(), bsc.cpu())
     assert _rel_err(got[rows.to(dev)].float().cpu(), ref) < (HW_SUM if out_dtype == "float32" else REL)
+
+
+@pytest.mark.parametrize("shape", [(256, 256, 1024), (512, 768, 1536), (4352, 4352, 1024), (4096, 4608, 2560), (8192, 8704, 1024),
+                                   (256, 512, 8192)])
+@pytest.mark.parametrize("out_dtype", ["bfloat16", "float32"])
+def test_mxfp8_stream_tile_walk(dev, shape, out_dtype):
+    """The streamed kernel: B in a ring of five half buffers (slab counts 8, 12, 20, 64: the ring position at a tile's
+    end takes every value), scale groups of four slabs (even and odd numbers of groups per tile: the scale buffer
+    parity flips between tiles), more tiles than CUs with a ragged last round, up to five tiles per workgroup, fewer
+    tiles than CUs -- the walk bit-identical to the same kernel launched one workgroup per tile, whole matrix against
+    the independent generic kernel, rows against the fp32 oracle, launches repeat bit for bit."""
+    import iree_turbine_amd as ita
+    from oracle import inputs, mxfp8 as o8
+
+    M, N, K = shape
+    announce(f"mxfp8 streamed walk {shape} {out_dtype}")
+    names = ita._lib.variants("mxfp8_gemm")
+    walk, plain = names.index("stream_256x256x128_w2x2_walk"), names.index("stream_256x256x128_w2x2")
+    a, asc, b, bsc = [t.to(dev) for t in inputs.mxfp8_inputs(M, N, K, seed=11)]
+    got = torch.ops.mi355.mxfp8_gemm(a, asc, b, bsc, out_dtype, walk)
+    assert torch.equal(got, torch.ops.mi355.mxfp8_gemm(a, asc, b, bsc, out_dtype, plain))
+    assert torch.equal(got, torch.ops.mi355.mxfp8_gemm(a, asc, b, bsc, out_dtype, walk))
+    ref = torch.ops.mi355.mxfp8_gemm(a, asc, b, bsc, out_dtype, names.index("generic_32x128"))
+    if out_dtype == "float32":
+        assert _rel_err(got, ref) < HW_SUM
+    else:
+        g32, r32 = got.float(), ref.float()
+        assert _rel_err(g32, r32) < REL
+        assert ((g32 - r32).abs() <= r32.abs() * 2 ** -7 + 1e-5 * r32.abs().max()).all()
+    rows = torch.tensor([0, 127, 128, M - 1])
+    want = o8.mxfp8_gemm_ref(a[rows.to(dev)].cpu(), asc[rows.to(dev)].cpu(), b.cpu(), bsc.cpu())
+    assert _rel_err(got[rows.to(dev)].float().cpu(), want) < (HW_SUM if out_dtype == "float32" else REL)
+
+
+def test_mxfp8_stream_contract(dev):
+    """What the streamed kernels cannot take is refused by name, and the automatic choice falls back."""
+    import iree_turbine_amd as ita
+    from oracle import inputs, mxfp8 as o8
+
+    announce("mxfp8 streamed contract")
+    names = ita._lib.variants("mxfp8_gemm")
+    for (M, N, K) in [(256, 256, 512), (256, 256, 1280), (128, 256, 1024)]:  # K < 1024, K % 512 != 0, M % 256 != 0
+        a, asc, b, bsc = [t.to(dev) for t in inputs.mxfp8_inputs(M, N, K, seed=2)]
+        for vn in ("stream_256x256x128_w2x2", "stream_256x256x128_w2x2_walk"):
+            with pytest.raises(ValueError, match="stream_256x256x128"):
+                torch.ops.mi355.mxfp8_gemm(a, asc, b, bsc, "bfloat16", names.index(vn))
+        got = torch.ops.mi355.mxfp8_gemm(a, asc, b, bsc, "float32", -1)
+        assert _rel_err(got.cpu(), o8.mxfp8_gemm_ref(a.cpu(), asc.cpu(), b.cpu(), bsc.cpu())) < HW_SUM
+    # scale rows that are not 16-byte aligned: the streamed kernel loads scale groups 16 bytes at a time
+    M, N, K = 256, 256, 1024
+    a, asc, b, bsc = [t.to(dev) for t in inputs.mxfp8_inputs(M, N, K, seed=2)]
+    pad = torch.zeros(M * (K // 32) + 4, dtype=torch.uint8, device=dev)
+    asc_off = pad[4:].view(M, K // 32)
+    asc_off.copy_(asc)
+    with pytest.raises(ValueError, match="stream_256x256x128"):
+        torch.ops.mi355.mxfp8_gemm(a, asc_off, b, bsc, "bfloat16", names.index("stream_256x256x128_w2x2"))
+    got = torch.ops.mi355.mxfp8_gemm(a, asc_off, b, bsc, "float32", -1)
+    assert _rel_err(got, torch.ops.mi355.mxfp8_gemm(a, asc, b, bsc, "float32", names.index("generic_32x128"))) < HW_SUM
 
 
 def test_mxfp8_contract_errors(dev):
@@ -185,9 +248,15 @@ def test_fp8_gemm_plain(dev, shape):
     assert torch.equal(got, alpha * scaled)
     bf = torch.ops.mi355.fp8_gemm(a.to(dev), b.to(dev), alpha, "bfloat16", -1)
     assert torch.equal(bf, got.bfloat16())
-    if M % 256 == 0:  # both tiled kernels, chosen explicitly
-        for variant in (0, 2):
-            assert torch.equal(got, torch.ops.mi355.fp8_gemm(a.to(dev), b.to(dev), alpha, "float32", variant)), variant
+    if M % 256 == 0:  # the tiled kernels, chosen explicitly: each pair takes the k blocks in the same order
+        by_variant = [torch.ops.mi355.fp8_gemm(a.to(dev), b.to(dev), alpha, "float32", variant) for variant in range(5)]
+        assert torch.equal(by_variant[0], by_variant[2])
+        assert torch.equal(by_variant[3], by_variant[4])
+        for variant in range(5):
+            assert _rel_err(by_variant[variant].cpu(), ref) < HW_SUM, variant
+        assert torch.equal(got, by_variant[4])  # the automatic choice here
+        bf = torch.ops.mi355.fp8_gemm(a.to(dev), b.to(dev), alpha, "bfloat16", 3)
+        assert torch.equal(bf, by_variant[3].bfloat16())
     # against torch's own decode of the same bytes
     lib = alpha * (a.view(torch.float8_e4m3fn).float() @ b.view(torch.float8_e4m3fn).float().t())
     assert _rel_err(got.cpu(), lib) < HW_SUM
