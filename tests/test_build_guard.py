@@ -42,3 +42,20 @@ def test_other_kernels_may_use_scratch_and_warnings_pass_through():
     assert rest == ["x.hip:7:3: warning: something else"]
     rest = build._check_resource_remarks(_remarks("_ZN5mi35517gemm_mxfp8_stagedItLb1EEEv", 0))
     assert rest == ["x.hip:7:3: warning: something else"]
+
+
+def test_remarks_with_the_location_behind_the_word_remark_are_read_too():
+    """With preprocessed sources (-save-temps) the compiler prints 'remark: file:line:col: Field: N'."""
+    located = "remark: /x/gemm_mxfp8.hip:597:0: {} [-Rpass-analysis=kernel-resource-usage]"
+    text = "\n".join([
+        located.format("Function Name: _ZN5mi35517gemm_mxfp8_streamItLb1EEEvPKhS2_S2_S2_PT_iiiiiif"),
+        located.format("    VGPRs: 199"),
+        located.format("    ScratchSize [bytes/lane]: 0"),
+        located.format("    Occupancy [waves/SIMD]: 1"),
+        located.format("    VGPRs Spill: 0"),
+    ])
+    assert build._check_resource_remarks(text) == []
+    with pytest.raises(RuntimeError, match="spills \\(16 bytes"):
+        build._check_resource_remarks(text.replace("ScratchSize [bytes/lane]: 0", "ScratchSize [bytes/lane]: 16"))
+    with pytest.raises(RuntimeError, match="2 waves per SIMD, expected 1"):
+        build._check_resource_remarks(text.replace("Occupancy [waves/SIMD]: 1", "Occupancy [waves/SIMD]: 2"))
