@@ -309,6 +309,19 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
   const half_t* Vb = V + (PAGED ? 0 : b_idx * lay.v_b) + hk_idx * lay.v_h;
   half_t* Ob = O + b_idx * lay.o_b + h_idx * lay.o_h;
 
+  // LDS addresses of the eight K fragment reads of a 32-key half tile (ks = 0..7), formed once: left to the
+  // compiler inside the pass loop, the offsets are hoisted as integers and each read then adds the LDS base to
+  // one again, vector instructions that upset the pinned MFMA / softmax interleave
+  typedef const __attribute__((address_space(3))) half8* lds_half8_t;
+  unsigned k_frag[8];
+  {
+    const int kb0 = r32 * 256 + ((h ^ (lane & 15)) * 16);
+#pragma unroll
+    for (int ks = 0; ks < 8; ks++) {
+      k_frag[ks] = (unsigned)(uintptr_t)MI355_LDS(char, lds + (kb0 ^ (ks * 32)));
+      asm volatile("" : "+v"(k_frag[ks]));  // one opaque value per read: nothing to re-derive it from
+    }
+  }
   for (int pass = 0; pass < (CAUSAL ? 2 : 1); pass++) {
   const int qb = CAUSAL ? (pass == 0 ? q_blocks - 1 - unit : unit) : unit;
   if (CAUSAL && pass == 1 && 2 * unit == q_blocks - 1) break;  // the middle block of an odd count has no partner
@@ -391,7 +404,6 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     }
   };
 
-  const int k_base = r32 * 256 + ((h ^ (lane & 15)) * 16);
   const int i16 = lane & 15, g16 = lane >> 4;
   const int v_row = 4 * (g16 >> 1) + (i16 >> 2);
   const int v_base = VBUF + v_row * 256 + (i16 >> 2) * 64 + (2 * (g16 & 1) + ((i16 & 3) >> 1)) * 16 + (i16 & 1) * 8;
@@ -421,7 +433,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     for (int t = 0; t < 2; t++) {
 #pragma unroll
       for (int ks = 0; ks < 8; ks++) {
-        half8 kf = *reinterpret_cast<const half8*>(lds + koff + t * 8192 + (k_base ^ (ks * 32)));
+        half8 kf = *(lds_half8_t)(uintptr_t)(k_frag[ks] + (unsigned)(koff + t * 8192));
         s[t] = mfma16<BF>(kf, qf[ks], ks == 0 ? negm : s[t]);
       }
     }
@@ -573,15 +585,19 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     // slot c ^ (r & 15)), reads whole 16-byte chunks back and stores full rows -- 8 stores of 16 bytes per lane instead
     // of 16 of 8 bytes that each touch 32 rows.
     char* ep = lds + wave * 8192;
+    // (the lane id is taken afresh: addresses derived from the kernel's own `lane` are invariant over the passes of a
+    // causal pair, get hoisted in front of the pass loop and then occupy registers all through the key walk)
+    const int el = CAUSAL ? opaque_lane_id() : lane;
+    const int e32 = el & 31, eh = el >> 5;
 #pragma unroll
     for (int dt = 0; dt < 4; dt++)
 #pragma unroll
       for (int q = 0; q < 4; q++) {
         half4 v = {cvt16<BF>(oacc[dt][4 * q] * inv), cvt16<BF>(oacc[dt][4 * q + 1] * inv), cvt16<BF>(oacc[dt][4 * q + 2] * inv),
                    cvt16<BF>(oacc[dt][4 * q + 3] * inv)};
-        *reinterpret_cast<half4*>(ep + r32 * 256 + (((dt * 4 + q) ^ (r32 & 15)) * 16) + 8 * h) = v;
+        *reinterpret_cast<half4*>(ep + e32 * 256 + (((dt * 4 + q) ^ (e32 & 15)) * 16) + 8 * eh) = v;
       }
-    const int er = lane >> 4, ec = lane & 15;
+    const int er = el >> 4, ec = el & 15;
 #pragma unroll
     for (int it = 0; it < 8; it++) {
       const int row = it * 4 + er;
