@@ -420,6 +420,46 @@ def wl_mfma_regloop(kind: str, data: str):
     return build
 
 
+def wl_fa_issue_regloop(mode: str, waves_per_simd: int, data: str = "benchmark"):
+    """The prefill tile's instruction mix out of registers (mi355_calibrate_fa_issue): what instruction issue alone
+    lets the prefill kernel reach, at one or two waves per SIMD, on operands drawn like the attention benchmark's."""
+    import ctypes
+
+    from iree_turbine_amd import _lib
+
+    def build(dev):
+        g = torch.Generator().manual_seed(10)
+        nbytes = 1 << 20
+        if data == "zeros":  # the issue-rate reading: nothing toggles, the clock stays up
+            opsd = torch.zeros(nbytes, dtype=torch.uint8, device=dev)
+        else:
+            opsd = (torch.randn(nbytes // 2, generator=g) * 0.35).half().view(torch.uint8).to(dev)  # scores of a few units
+        workgroups, trips = 256 * waves_per_simd, 4000
+        sink = torch.empty(workgroups * 256, dtype=torch.float32, device=dev)
+        code = {"mix": 0, "nomax": 1, "mfma": 2, "vector": 3, "spread": 4, "stepwise": 5}[mode]
+        flop = ctypes.c_double(0.0)
+        lib = _lib.load()
+
+        def fn():
+            rc = lib.mi355_calibrate_fa_issue(code, opsd.data_ptr(), nbytes, sink.data_ptr(), sink.numel(), workgroups, trips,
+                                              ctypes.byref(flop), _lib.current_stream_ptr(dev))
+            _lib.check(rc, "calibrate_fa_issue")
+        fn()
+        torch.cuda.synchronize()
+        return {
+            "fn": fn, "work": flop.value, "bytes": 0.0, "flops": flop.value, "bound": "mfma", "peak": PEAK_F16_TFLOPS,
+            "unit": "TFLOP/s", "dtype": "f16", "cpu": lambda: None,
+            "config": {"workload": f"fa_issue_regloop_{mode}_w{waves_per_simd}" + ("_zeros" if data == "zeros" else ""), "workgroups": workgroups, "trips": trips,
+                       "waves_per_simd": waves_per_simd,
+                       "per_wave_and_trip": {"mix": "32 MFMA 32x32x16, 32 v_exp_f32, 16 cvt_pk, 16 dot2, 16 v_max3 + test",
+                                             "nomax": "32 MFMA 32x32x16, 32 v_exp_f32, 16 cvt_pk, 16 dot2",
+                                             "mfma": "32 MFMA 32x32x16", "vector": "32 v_exp_f32, 16 cvt_pk, 16 dot2 (flop counted as if the MFMAs ran)",
+                                             "spread": "the whole mix, vector work spread over all 32 MFMAs",
+                                             "stepwise": "the whole mix, vector work behind the 16 score MFMAs, maximum chain behind the last 8 output MFMAs"}[mode]},
+        }
+    return build
+
+
 WORKLOADS = {
     "gemm_8192": wl_gemm(8192, 8192, 8192),
     "gemm_4096": wl_gemm(4096, 4096, 4096),
@@ -473,6 +513,8 @@ CALIBRATION = {  # not part of the path: run only when named with --workload
     "mfma_fp4walk_regloop_benchmark": wl_mfma_regloop("fp4walk", "benchmark"),
     "mfma_fp4x16walk_regloop_zeros": wl_mfma_regloop("fp4x16walk", "zeros"),
     "mfma_fp4x16walk_regloop_benchmark": wl_mfma_regloop("fp4x16walk", "benchmark"),
+    **{f"fa_issue_regloop_{m}_w{w}": wl_fa_issue_regloop(m, w) for m in ("mix", "nomax", "mfma", "vector", "spread", "stepwise") for w in (1, 2)},
+    **{f"fa_issue_regloop_{m}_w{w}_zeros": wl_fa_issue_regloop(m, w, "zeros") for m in ("mix", "mfma", "vector", "spread", "stepwise") for w in (1, 2)},
     "mfma_fp4_regloop_zeros": wl_mfma_regloop("fp4", "zeros"),
     "mfma_fp4_regloop_benchmark": wl_mfma_regloop("fp4", "benchmark"),
 }

@@ -397,13 +397,29 @@ int mi355_mxfp8_quantize(const void* x, int in_dtype, int64_t rows, int64_t K,
  * the part of the plain-copy workload for the HBM figures.
  * kind 0: v_mfma_f32_32x32x16_f16; 1: v_mfma_scale_f32_32x32x64_f8f6f4 with fp4 operands and unit
  * scales; 2: the same with E8M0 scales spread over 2^-8 .. 2^7; 3: v_mfma_f32_16x16x32_f16 (two per
- * 32x32x16's worth of flop).  operands: operand_bytes (a power of
+ * 32x32x16's worth of flop); 4 / 5: loops with a GEMM's register structure (256 accumulators per lane,
+ * eight A and eight B operands rotated, every product subtracted again eight trips later) on
+ * 32x32x16 / 16x16x32 fp16 MFMAs, trips rounded down to a multiple of 16; 6 / 7: the same structure on
+ * scaled fp4 MFMAs 32x32x64 / 16x16x128.  operands: operand_bytes (a power of
  * two >= 16) of device memory read once before the loop; sink: >= workgroups * 256 floats, written
  * once after it; *flop_per_launch (optional, host memory) receives the flop count of the launch.
  */
 int mi355_calibrate_mfma(int kind, const void* operands, int64_t operand_bytes, float* sink,
                          int64_t sink_floats, int64_t workgroups, int64_t trips,
                          double* flop_per_launch, void* stream);
+
+/*
+ * Calibration, not part of the path and without a counterpart in the reference: the instruction mix of one
+ * 64-key tile of the prefill kernel per wave of 32 queries (32 MFMAs 32x32x16, 32 v_exp_f32, 16 packed
+ * conversions, 16 dot2, the v_max3 chain and its wave-wide test), out of registers only -- no LDS reads,
+ * loads or barriers.  What it sustains is the ceiling that instruction issue sets for the prefill kernel.
+ * mode 0: the whole mix; 1: without the maximum chain; 2: the MFMAs alone, same dependences; 3: the vector
+ * work alone.  256 workgroups (of 256 threads) put one wave on every SIMD, 512 two.  operands, sink and
+ * flop_per_launch as for mi355_calibrate_mfma; the flop count is that of the tile's 32 MFMAs.
+ */
+int mi355_calibrate_fa_issue(int mode, const void* operands, int64_t operand_bytes, float* sink,
+                             int64_t sink_floats, int64_t workgroups, int64_t trips,
+                             double* flop_per_launch, void* stream);
 
 #ifdef __cplusplus
 }

@@ -95,6 +95,7 @@ _PROTOS = {
     "mi355_mxfp6_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_void_p]),
     "mi355_fp8_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_float, c_int, c_int, c_void_p]),
     "mi355_calibrate_mfma": (c_int, [c_int, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, ctypes.POINTER(ctypes.c_double), c_void_p]),
+    "mi355_calibrate_fa_issue": (c_int, [c_int, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, ctypes.POINTER(ctypes.c_double), c_void_p]),
     "mi355_mxfp4_dequant": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
     "mi355_mxfp4_quantize": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p]),
     "mi355_mxfp6_quantize": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int, c_void_p, c_void_p, c_void_p]),

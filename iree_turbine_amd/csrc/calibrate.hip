@@ -210,9 +210,229 @@ __global__ __launch_bounds__(CAL_WAVES * 64) void calibrate_mfma_fp4_walk_kernel
   sink[t] = s;
 }
 
+// The instruction mix of one 64-key tile of the prefill kernel, per wave of 32 queries, out of registers only: 16 score
+// MFMAs 32x32x16 (two chains of eight, each starting from one block of addends) with the softmax of the PREVIOUS tile's
+// scores placed between them as the prefill kernel pins it -- per MFMA two v_exp_f32, one packed conversion and one
+// dot2 -- then 16 MFMAs into four output accumulators that take the packed probabilities as their B operand; before
+// them the in-lane v_max3 chain over the 32 scores and its wave-wide test.  No LDS reads, no loads, no barrier: what
+// this loop sustains is the ceiling the instruction mix itself sets for the prefill kernel at one (256 workgroups) or
+// two (512) waves per SIMD.  MODE 0: the whole mix; 1: without the maximum chain; 2: the MFMAs alone, same
+// dependences; 3: the vector work alone.
+template <int MODE>
+__global__ __launch_bounds__(CAL_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void calibrate_fa_issue_kernel(
+    const half8* __restrict__ operands, unsigned mask, float* __restrict__ sink, int trips) {
+  constexpr bool MFMAS = MODE != 3, VECTOR = MODE != 2, MAXIMUM = MODE == 0;
+  const unsigned t = threadIdx.x + blockIdx.x * blockDim.x;
+  half8 kf[4], vf[4], qf[8];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    kf[i] = operands[(t * 16 + i) & mask];
+    vf[i] = operands[(t * 16 + 4 + i) & mask];
+  }
+#pragma unroll
+  for (int i = 0; i < 8; i++) qf[i] = operands[(t * 16 + 8 + i) & mask];
+  floatx16 oacc[4], negm, sa[2], sb[2];
+#pragma unroll
+  for (int r = 0; r < 16; r++) {
+    negm[r] = -1.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) oacc[i][r] = 0.f;
+    sa[0][r] = sa[1][r] = sb[0][r] = sb[1][r] = -2.f;
+  }
+  float l_run = 0.f, grow_thr = 1e30f;
+  auto tile = [&](floatx16* s, floatx16* s_next) {
+    if constexpr (MAXIMUM) {
+      float mx = s[0][0];
+#pragma unroll
+      for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[tt][r]);
+      if (__builtin_amdgcn_ballot_w64(mx > grow_thr) != 0) {  // never taken: the threshold is out of reach
+#pragma unroll
+        for (int r = 0; r < 16; r++) negm[r] -= mx;
+      }
+    }
+    half8 pf[4];
+    float psum = 0.f;
+    asm volatile("" : "+v"(negm));  // opaque: the score MFMAs are not loop-invariant
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (MFMAS) {
+#pragma unroll
+      for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+        for (int ks = 0; ks < 8; ks++) s_next[tt] = mfma_32x32x16(kf[(ks + tt) & 3], qf[ks], ks == 0 ? negm : s_next[tt]);
+    }
+    if constexpr (VECTOR) {
+#pragma unroll
+      for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+          const half2v pp = {(half_t)__builtin_amdgcn_exp2f(s[tt][r]), (half_t)__builtin_amdgcn_exp2f(s[tt][r + 1])};
+          psum = __builtin_amdgcn_fdot2(pp, half2v{(half_t)1.f, (half_t)1.f}, psum, false);
+          pf[tt * 2 + (r >> 3)][r & 7] = pp[0];
+          pf[tt * 2 + (r >> 3)][(r & 7) + 1] = pp[1];
+        }
+    } else {
+      asm volatile("" ::"v"(s[0]), "v"(s[1]));  // the scores count as used
+#pragma unroll
+      for (int i = 0; i < 4; i++) pf[i] = qf[i];
+    }
+    if constexpr (MFMAS && VECTOR) {
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    l_run += psum;
+    if constexpr (MFMAS) {
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        oacc[i & 3] = mfma_32x32x16(vf[(i + (i >> 2)) & 3], pf[i >> 2], oacc[i & 3]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) oacc[i][e] += (float)pf[i][e];
+    }
+    if constexpr (!MFMAS) {  // the next tile's scores: opaque copies, so that their exponentials are computed anew
+#pragma unroll
+      for (int tt = 0; tt < 2; tt++) {
+        s_next[tt] = s[tt];
+        asm volatile("" : "+v"(s_next[tt]));
+      }
+    }
+  };
+#pragma unroll 1
+  for (int it = 0; it < trips; it += 2) {
+    tile(sa, sb);
+    tile(sb, sa);
+  }
+  float acc = l_run;
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc += oacc[i][r];
+  sink[t] = acc;
+}
+
+// The same work per tile with the vector instructions spread over all 32 MFMAs instead of the 16 score MFMAs: one
+// exponential behind every score MFMA (the first 32-key half of the tile), two behind each of the first eight output
+// MFMAs (the second half; those MFMAs multiply the first half's probabilities), and the maximum chain of the NEXT
+// tile's scores behind the last eight.  EXPS_A = exponentials behind each score MFMA (1 or 2: 2 is the order of
+// calibrate_fa_issue_kernel written step by step).
+template <int EXPS_A>
+__global__ __launch_bounds__(CAL_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void calibrate_fa_spread_kernel(
+    const half8* __restrict__ operands, unsigned mask, float* __restrict__ sink, int trips) {
+  const unsigned t = threadIdx.x + blockIdx.x * blockDim.x;
+  half8 kf[4], vf[4], qf[8];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    kf[i] = operands[(t * 16 + i) & mask];
+    vf[i] = operands[(t * 16 + 4 + i) & mask];
+  }
+#pragma unroll
+  for (int i = 0; i < 8; i++) qf[i] = operands[(t * 16 + 8 + i) & mask];
+  floatx16 oacc[4], negm, sa[2], sb[2];
+#pragma unroll
+  for (int r = 0; r < 16; r++) {
+    negm[r] = -1.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) oacc[i][r] = 0.f;
+    sa[0][r] = sa[1][r] = sb[0][r] = sb[1][r] = -2.f;
+  }
+  float l_run = 0.f, grow_thr = 1e30f, mx = -3.f;
+  const half2v ones = {(half_t)1.f, (half_t)1.f};
+  auto tile = [&](floatx16* s, floatx16* s_next) {
+    if (__builtin_amdgcn_ballot_w64(mx > grow_thr) != 0) {  // never taken
+#pragma unroll
+      for (int r = 0; r < 16; r++) negm[r] -= mx;
+    }
+    half8 pf[4];
+    float psum = 0.f;
+    asm volatile("" : "+v"(negm));
+    __builtin_amdgcn_sched_barrier(0);
+    // exponentials of score pair p (0..15) of the current tile -> pf
+    auto softmax_pair = [&](int p) {
+      const int tt = p >> 3, r = (p & 7) * 2;
+      const half2v pp = {(half_t)__builtin_amdgcn_exp2f(s[tt][r]), (half_t)__builtin_amdgcn_exp2f(s[tt][r + 1])};
+      psum = __builtin_amdgcn_fdot2(pp, ones, psum, false);
+      pf[tt * 2 + (r >> 3)][r & 7] = pp[0];
+      pf[tt * 2 + (r >> 3)][(r & 7) + 1] = pp[1];
+    };
+    constexpr int PAIRS_A = EXPS_A * 8;  // pairs finished during the score MFMAs
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      const int tt = i >> 3, ks = i & 7;
+      s_next[tt] = mfma_32x32x16(kf[(ks + tt) & 3], qf[ks], ks == 0 ? negm : s_next[tt]);
+      if (EXPS_A == 2) softmax_pair(i);
+      else if (i & 1) softmax_pair(i >> 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    float mxn = s_next[0][0];
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      oacc[i & 3] = mfma_32x32x16(vf[(i + (i >> 2)) & 3], pf[i >> 2], oacc[i & 3]);
+      if (EXPS_A == 1 && i < 8) softmax_pair(PAIRS_A + i);
+      if (i >= 8) {
+        const int tt = (i - 8) >> 2, r = ((i - 8) & 3) * 4;
+        mxn = fmaxf(fmaxf(mxn, s_next[tt][r]), s_next[tt][r + 1]);
+        mxn = fmaxf(fmaxf(mxn, s_next[tt][r + 2]), s_next[tt][r + 3]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    mx = mxn;
+    l_run += psum;
+  };
+#pragma unroll 1
+  for (int it = 0; it < trips; it += 2) {
+    tile(sa, sb);
+    tile(sb, sa);
+  }
+  float acc = l_run;
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc += oacc[i][r];
+  sink[t] = acc;
+}
+
 }  // namespace mi355
 
 using namespace mi355;
+
+// The prefill tile's instruction mix out of registers (calibrate_fa_issue_kernel).  mode 0..3 as documented there;
+// 256 workgroups put one wave on every SIMD, 512 two.  flop_per_launch counts the 32 MFMAs of a tile (modes 0..2).
+extern "C" int mi355_calibrate_fa_issue(int mode, const void* operands, int64_t operand_bytes, float* sink, int64_t sink_floats,
+                                        int64_t workgroups, int64_t trips, double* flop_per_launch, void* stream) {
+  if (!operands || !sink) return fail(-MI355_E_NULL, "calibrate_fa_issue: null pointer");
+  if (mode < 0 || mode > 5) return fail(-MI355_E_DTYPE, "calibrate_fa_issue: mode %d unknown (0 whole mix, 1 without the maximum chain, 2 MFMAs alone, 3 vector work alone, 4 vector work spread over all 32 MFMAs, 5 the order of mode 0 written step by step)", mode);
+  if (operand_bytes < 16 || (operand_bytes & (operand_bytes - 1)) || operand_bytes > (1ll << 30))
+    return fail(-MI355_E_SHAPE, "calibrate_fa_issue: operand_bytes %lld must be a power of two in [16, 2^30]", (long long)operand_bytes);
+  if (workgroups <= 0 || workgroups > 65535 || trips <= 0 || trips > (1 << 24))
+    return fail(-MI355_E_SHAPE, "calibrate_fa_issue: workgroups %lld / trips %lld out of range", (long long)workgroups, (long long)trips);
+  if (sink_floats < workgroups * CAL_WAVES * 64)
+    return fail(-MI355_E_SCRATCH, "calibrate_fa_issue: sink needs %lld floats", (long long)(workgroups * CAL_WAVES * 64));
+  if (!aligned16(operands)) return fail(-MI355_E_ALIGN, "calibrate_fa_issue: operands must be 16-byte aligned");
+  trips = (trips + 1) & ~1ll;
+  const unsigned mask = (unsigned)(operand_bytes / 16 - 1);
+  dim3 grid((unsigned)workgroups), block(CAL_WAVES * 64);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (flop_per_launch) *flop_per_launch = 32.0 * (2.0 * 32 * 32 * 16) * (double)trips * CAL_WAVES * (double)workgroups;
+  switch (mode) {
+    case 0: hipLaunchKernelGGL(calibrate_fa_issue_kernel<0>, grid, block, 0, s, (const half8*)operands, mask, sink, (int)trips); break;
+    case 1: hipLaunchKernelGGL(calibrate_fa_issue_kernel<1>, grid, block, 0, s, (const half8*)operands, mask, sink, (int)trips); break;
+    case 2: hipLaunchKernelGGL(calibrate_fa_issue_kernel<2>, grid, block, 0, s, (const half8*)operands, mask, sink, (int)trips); break;
+    case 3: hipLaunchKernelGGL(calibrate_fa_issue_kernel<3>, grid, block, 0, s, (const half8*)operands, mask, sink, (int)trips); break;
+    case 4: hipLaunchKernelGGL(calibrate_fa_spread_kernel<1>, grid, block, 0, s, (const half8*)operands, mask, sink, (int)trips); break;
+    default: hipLaunchKernelGGL(calibrate_fa_spread_kernel<2>, grid, block, 0, s, (const half8*)operands, mask, sink, (int)trips); break;
+  }
+  return check_launch("calibrate_fa_issue", grid, block, 0);
+}
 
 // kind 0: fp16 32x32x16; kind 1: fp4 32x32x64 with unit scales; kind 2: fp4 with spread scales; kind 3: fp16 16x16x32;
 // kinds 4 / 5: the GEMM-like loops with 32x32x16 / 16x16x32 (trips rounded down to a multiple of 16); kinds 6 / 7: the

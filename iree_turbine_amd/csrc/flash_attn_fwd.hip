@@ -228,6 +228,16 @@ struct FaPaged {
   int max_pages, num_pages, page_shift;
 };
 
+// body(std::integral_constant<int, 0>{}), ..., body(std::integral_constant<int, N - 1>{}): a loop whose index is a
+// constant expression in the body (instruction immediates of inline assembly need one).
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F&& body) {
+  if constexpr (I < N) {
+    body(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(body);
+  }
+}
+
 // Software-pipelined form.  Same tiling and register layout, but the score MFMAs run one key tile
 // ahead of the softmax: in trip j a wave issues S^T(j+1) = K(j+1) . Q^T, exponentiates the scores of
 // tile j on the VALU while those MFMAs execute, then issues O^T += V(j)^T . P(j)^T.  K and V sit in
@@ -322,6 +332,18 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
       asm volatile("" : "+v"(k_frag[ks]));  // one opaque value per read: nothing to re-derive it from
     }
   }
+  // LDS addresses of the V^T transpose reads (slot 0 of the V ring; dt = 0..3), same treatment
+  unsigned v_frag[4];
+  {
+    const int i16 = lane & 15, g16 = lane >> 4;
+    const int v_row = 4 * (g16 >> 1) + (i16 >> 2);
+    const int vb0 = VBUF + v_row * 256 + (i16 >> 2) * 64 + (2 * (g16 & 1) + ((i16 & 3) >> 1)) * 16 + (i16 & 1) * 8;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++) {
+      v_frag[dt] = (unsigned)(uintptr_t)MI355_LDS(char, lds + (vb0 ^ (dt * 64)));
+      asm volatile("" : "+v"(v_frag[dt]));
+    }
+  }
   for (int pass = 0; pass < (CAUSAL ? 2 : 1); pass++) {
   const int qb = CAUSAL ? (pass == 0 ? q_blocks - 1 - unit : unit) : unit;
   if (CAUSAL && pass == 1 && 2 * unit == q_blocks - 1) break;  // the middle block of an odd count has no partner
@@ -404,10 +426,6 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     }
   };
 
-  const int i16 = lane & 15, g16 = lane >> 4;
-  const int v_row = 4 * (g16 >> 1) + (i16 >> 2);
-  const int v_base = VBUF + v_row * 256 + (i16 >> 2) * 64 + (2 * (g16 & 1) + ((i16 & 3) >> 1)) * 16 + (i16 & 1) * 8;
-
   floatx16 oacc[4];
 #pragma unroll
   for (int dt = 0; dt < 4; dt++)
@@ -440,8 +458,9 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
   };
 
   // softmax of tile `tile` (scores in s) and O^T += V(slot)^T . P^T
-  auto softmax_pv = [&](auto masked_tag, int tile, int voff, floatx16* s, int koff_next, floatx16* s_next) {
+  auto softmax_pv = [&](auto masked_tag, int tile, auto voff_tag, floatx16* s, int koff_next, floatx16* s_next) {
     constexpr bool MASKED = decltype(masked_tag)::value;
+    constexpr int VOFF = decltype(voff_tag)::value;  // byte offset of the V ring slot to read
     if (MASKED) {
       const int key0 = tile * FA_BLOCK_N;
       const bool need_mask = (CAUSAL && (key0 + FA_BLOCK_N - 1 > wq0 + causal_off)) || (key0 + FA_BLOCK_N > Sk);
@@ -488,55 +507,107 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     }
     half8 pf[4];
     float psum = 0.f;
-    // Scores of the next tile and exponentials of this one in one straight-line block: a wave issues in
-    // order, so only VALU work placed between two MFMAs runs while the first occupies the matrix pipe.
-    // (Past the last tile the scores are computed from stale LDS bytes and never used.)
-    __builtin_amdgcn_sched_barrier(0);
-    scores(koff_next, s_next);
+    if constexpr (!PAGED) {
+      // Scores of the next tile and exponentials of this one in one straight-line block: a wave issues in
+      // order, so only VALU work placed between two MFMAs runs while the first occupies the matrix pipe.
+      // (Past the last tile the scores are computed from stale LDS bytes and never used.)
+      __builtin_amdgcn_sched_barrier(0);
+      scores(koff_next, s_next);
 #pragma unroll
-    for (int t = 0; t < 2; t++)
+      for (int t = 0; t < 2; t++)
 #pragma unroll
-      for (int r = 0; r < 16; r += 2) {
-        const half2v pp = cvt16x2<BF>(__builtin_amdgcn_exp2f(s[t][r]), __builtin_amdgcn_exp2f(s[t][r + 1]));
-        psum = dot2_ones<BF>(pp, psum);  // sums what the second MFMA multiplies
-        pf[t * 2 + (r >> 3)][r & 7] = pp[0];
-        pf[t * 2 + (r >> 3)][(r & 7) + 1] = pp[1];
+        for (int r = 0; r < 16; r += 2) {
+          const half2v pp = cvt16x2<BF>(__builtin_amdgcn_exp2f(s[t][r]), __builtin_amdgcn_exp2f(s[t][r + 1]));
+          psum = dot2_ones<BF>(pp, psum);  // sums what the second MFMA multiplies
+          pf[t * 2 + (r >> 3)][r & 7] = pp[0];
+          pf[t * 2 + (r >> 3)][(r & 7) + 1] = pp[1];
+        }
+      // order: 3 K fragment reads up front, then per score MFMA one more read and the work of two scores
+      // (two exp, one cvt_pk, one dot2) -- a fragment is requested two MFMAs before its use
+      __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+#pragma unroll
+      for (int i = 0; i < 13; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
       }
-    // order: 3 K fragment reads up front, then per score MFMA one more read and the work of two scores
-    // (two exp, one cvt_pk, one dot2) -- a fragment is requested two MFMAs before its use
-    __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
 #pragma unroll
-    for (int i = 0; i < 13; i++) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+      for (int i = 0; i < 3; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    } else {
+      // The paged form's page-id bookkeeping keeps the group barriers above from being honoured (the block came out
+      // as sixteen MFMAs, each behind its own fragment read, and the exponentials after them); here the same order is
+      // written step by step.
+      // Scores of the next tile and the softmax of this one, step by step: score MFMA i, the K fragment of MFMA i + 3
+      // requested, and the work of score pair i (two exponentials, one packed conversion, one dot2) behind it.  A
+      // scheduling barrier after every step pins the order (a wave issues in order: only vector work placed between two
+      // MFMAs runs while the first occupies the matrix pipe).
+      __builtin_amdgcn_sched_barrier(0);
+      {
+        half8 kf[4];
+        half2v pp_prev = {(half_t)0, (half_t)0};
+        auto kread = [&](int i) { return *(lds_half8_t)(uintptr_t)(k_frag[i & 7] + (unsigned)(koff_next + (i >> 3) * 8192)); };
+        kf[0] = kread(0);
+        kf[1] = kread(1);
+        kf[2] = kread(2);
+  #pragma unroll
+        for (int i = 0; i < 16; i++) {
+          const int t = i >> 3, ks = i & 7, r = 2 * ks;
+          if (i + 3 < 16) kf[(i + 3) & 3] = kread(i + 3);
+          s_next[t] = mfma16<BF>(kf[i & 3], qf[ks], ks == 0 ? negm : s_next[t]);
+          // (the empty statement ties the pair's arithmetic to this step: without side effects of its own it is placed
+          // wherever instruction selection likes, scheduling barriers or not.  The dot2 of a pair runs one step behind its
+          // conversion, so that neither waits for the instruction in front of it.)
+          float e0 = __builtin_amdgcn_exp2f(s[t][r]), e1 = __builtin_amdgcn_exp2f(s[t][r + 1]);
+          if (i > 0) psum = dot2_ones<BF>(pp_prev, psum);  // sums what the second MFMA multiplies
+          half2v pp = cvt16x2<BF>(e0, e1);
+          asm volatile("" : "+v"(pp), "+v"(psum));
+          pf[t * 2 + (r >> 3)][r & 7] = pp[0];
+          pf[t * 2 + (r >> 3)][(r & 7) + 1] = pp[1];
+          pp_prev = pp;
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        psum = dot2_ones<BF>(pp_prev, psum);
+      }
     }
-#pragma unroll
-    for (int i = 0; i < 3; i++) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
     l_run += psum;
     // O^T += V^T P^T: 16 MFMAs, each V^T fragment (two transpose reads) requested two MFMAs ahead.
-    // The order is pinned step by step.
-    auto vr = [&](int i) {  // i = t16*4 + dt
-      const char* va = lds + voff + (i >> 2) * 4096 + (v_base ^ ((i & 3) * 64));
-      half4 lo = lds_read_tr16(va);
-      half4 hi = lds_read_tr16(va + 2048);
-      return half8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    // The reads and their waits are inline assembly: a transpose read the compiler can see makes it wait for
+    // EVERY direct-to-LDS load in flight first (it cannot tell that the loads fill other ring slots), which put a
+    // vmcnt(0) -- the loads issued at the head of this trip -- in the middle of every trip.  In this block nothing
+    // else counts in lgkmcnt: LDS returns in order, so MFMA i may run once at most the reads of fragments i + 1
+    // and i + 2 (two each) are outstanding.  Each wait names the fragment's registers, so no use moves above it.
+    half4 vlo[3], vhi[3];
+    auto vr = [&](auto itag) {  // i = t16*4 + dt
+      constexpr int i = decltype(itag)::value;
+      constexpr int off = VOFF + (i >> 2) * 4096;
+      half4 &lo = vlo[i % 3], &hi = vhi[i % 3];  // (operands of an assembly statement do not capture by themselves)
+      const unsigned addr = v_frag[i & 3];
+      asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4"
+                   : "=&v"(lo), "=&v"(hi)
+                   : "v"(addr), "n"(off), "n"(off + 2048));
     };
-    half8 vf[3];
-    vf[0] = vr(0);
-    vf[1] = vr(1);
-#pragma unroll
-    for (int i = 0; i < 16; i++) {
-      if (i + 2 < 16) vf[(i + 2) % 3] = vr(i + 2);
-      oacc[i & 3] = mfma16<BF>(vf[i % 3], pf[i >> 2], oacc[i & 3]);
+    vr(std::integral_constant<int, 0>{});
+    vr(std::integral_constant<int, 1>{});
+    static_for<0, 16>([&](auto itag) {
+      constexpr int i = decltype(itag)::value;
+      if constexpr (i + 2 < 16) vr(std::integral_constant<int, i + 2>{});
+      half4 &lo = vlo[i % 3], &hi = vhi[i % 3];
+      if constexpr (i + 2 < 16)
+        asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(lo), "+v"(hi));
+      else if constexpr (i + 1 < 16)
+        asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(lo), "+v"(hi));
+      else
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lo), "+v"(hi));
+      const half8 vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      oacc[i & 3] = mfma16<BF>(vf, pf[i >> 2], oacc[i & 3]);
       __builtin_amdgcn_sched_barrier(0);
-    }
+    });
   };
 
   floatx16 sa[2], sb[2];
@@ -568,7 +639,7 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
       for (int i = 0; i < 4; i++) v_ids[i] = k_ids[i];
       load_ids(j + 3, k_ids);
     }
-    if (wave_active(j)) softmax_pv(std::true_type{}, j, V_CUR, s_cur, K_NEXT, s_next);  // idle from here on otherwise
+    if (wave_active(j)) softmax_pv(std::true_type{}, j, std::integral_constant<int, V_CUR>{}, s_cur, K_NEXT, s_next);  // idle from here on otherwise
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
   };
@@ -609,13 +680,411 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
   }  // pass
 }
 
-static const char* kFaVariants[] = {"d128_bm128_bn64_w4_pipelined", "d128_bm128_bn64_w4", "d128_bm256_bn64_w8_pipelined"};
-int fa_variant_count() { return 3; }
-const char* fa_variant_name(int i) { return (i >= 0 && i < 3) ? kFaVariants[i] : nullptr; }
+
+// Persistent form of fa_fwd_d128_pipe ("walk"): one workgroup per CU slot runs its passes (a pass = one block of
+// NW * 32 queries of one head against its keys) one after the other -- units dealt round-robin (unit = workgroup +
+// i * grid), a causal unit being a pair of blocks as above -- and overlaps what a pass costs beside its key tiles:
+//  * the next pass's Q rows and first tiles (K 0, K 1, V 0) are requested in front of the current pass's LAST tile when
+//    that tile has odd number (a pass of an even tile count): both K slots and V slot 0 are free from there on, the Q
+//    rows land in registers that would hold the scores of a following tile (the last tile computes none), and nothing
+//    waits for any of it before the finished pass has been normalised and staged.  Otherwise they are requested right
+//    after the last trip;
+//  * the output goes through a staging region of its own (the rings are being filled) and is stored behind the barrier
+//    that opens the next pass; the stores are not waited for: they drain under the next pass's first trip, whose
+//    closing wait covers them.
+// A pass has at least two key tiles (the launcher checks Sk >= 128, and Sq == Sk with the mask).  The arithmetic per
+// query is that of fa_fwd_d128_pipe, instruction for instruction: results are bit-identical.
+template <bool CAUSAL, bool BF, int NW>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void fa_fwd_d128_walk(
+    const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V, half_t* __restrict__ O, int BH,
+    int Sq, int Sk, float scale_log2e, int q_blocks, FaLayout lay) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  constexpr int BLOCK_M = NW * 32, NI = 16 / NW;
+  constexpr int TILE_B = FA_BLOCK_N * 256, VBUF = 2 * TILE_B, STG = 4 * TILE_B;  // K ring, V ring, output staging
+  constexpr int STG_ROWS = NW == 8 ? 32 : 8;  // rows a wave stages per round: 8 KiB (one round) or 2 KiB (four) per wave
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r32 = lane & 31, h = lane >> 5;
+  const int causal_off = Sk - Sq;
+  const int units = CAUSAL ? (q_blocks + 1) / 2 : q_blocks;
+  const int total_units = BH * units;
+  const bool xcd_map = ((BH / lay.group) & 7) == 0;  // the launcher makes the grid a multiple of 8 then
+
+  // ---- passes of this workgroup, by ordinal: unit = blockIdx.x + (ord / passes per unit) * gridDim.x ----
+  struct Pass {
+    int ord;  // < 0: there is no such pass
+    int b, hq, hk, qb, n;  // batch, query head, K/V head, query block, key tiles
+  };
+  auto pass_at = [&](int ord) {  // the first existing pass with ordinal >= ord
+    Pass ps;
+    for (;;) {
+      const int pid = (int)blockIdx.x + (CAUSAL ? (ord >> 1) : ord) * (int)gridDim.x;
+      if (pid >= total_units) {
+        ps.ord = -1, ps.b = ps.hq = ps.hk = ps.qb = 0, ps.n = 2;
+        return ps;
+      }
+      int bh, unit;
+      if (xcd_map) {
+        const int xcd = pid & 7, loc = pid >> 3, per_kv = units * lay.group;
+        const int w = loc % per_kv;
+        bh = ((loc / per_kv) * 8 + xcd) * lay.group + w / units;
+        unit = w % units;
+      } else {
+        bh = pid / units;
+        unit = pid % units;
+      }
+      const bool second = CAUSAL && (ord & 1);
+      if (second && 2 * unit == q_blocks - 1) {  // the middle block of an odd count has no partner
+        ord++;
+        continue;
+      }
+      ps.ord = ord;
+      ps.qb = CAUSAL ? (second ? unit : q_blocks - 1 - unit) : unit;
+      ps.b = bh / lay.H;
+      ps.hq = bh - ps.b * lay.H;
+      ps.hk = ps.hq / lay.group;
+      int k_end = Sk;
+      if (CAUSAL) {
+        int last_q = ps.qb * BLOCK_M + BLOCK_M - 1;
+        if (last_q > Sq - 1) last_q = Sq - 1;
+        const int lim = last_q + causal_off + 1;
+        if (lim < k_end) k_end = lim;
+      }
+      ps.n = (k_end + FA_BLOCK_N - 1) / FA_BLOCK_N;
+      // (the divisions run on the vector unit; the fields are wave-uniform and belong in scalar registers)
+      ps.qb = __builtin_amdgcn_readfirstlane(ps.qb), ps.b = __builtin_amdgcn_readfirstlane(ps.b);
+      ps.hq = __builtin_amdgcn_readfirstlane(ps.hq), ps.hk = __builtin_amdgcn_readfirstlane(ps.hk);
+      ps.n = __builtin_amdgcn_readfirstlane(ps.n);
+      return ps;
+    }
+  };
+
+  // ---- per-lane constants ----
+  const int lrow = lane >> 4, lslot = lane & 15;
+  const int k_chunk = lslot ^ ((wave * 4 + lrow) & 15);
+  const int v_chunk = lslot ^ (4 * lrow);
+  const unsigned k_rb = lay.k_r * 2, v_rb = lay.v_r * 2;  // row strides in bytes
+  const unsigned k_voff = (wave * 4 + lrow) * k_rb + k_chunk * 16;
+  const unsigned v_voff = (wave * 4 + lrow) * v_rb + v_chunk * 16;
+  typedef const __attribute__((address_space(3))) half8* lds_half8_t;
+  unsigned k_frag[8], v_frag[4];  // LDS addresses of the fragment reads, opaque (see fa_fwd_d128_pipe)
+  {
+    const int kb0 = r32 * 256 + ((h ^ (lane & 15)) * 16);
+#pragma unroll
+    for (int ks = 0; ks < 8; ks++) {
+      k_frag[ks] = (unsigned)(uintptr_t)MI355_LDS(char, lds + (kb0 ^ (ks * 32)));
+      asm volatile("" : "+v"(k_frag[ks]));
+    }
+    const int i16 = lane & 15, g16 = lane >> 4;
+    const int v_row = 4 * (g16 >> 1) + (i16 >> 2);
+    const int vb0 = VBUF + v_row * 256 + (i16 >> 2) * 64 + (2 * (g16 & 1) + ((i16 & 3) >> 1)) * 16 + (i16 & 1) * 8;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++) {
+      v_frag[dt] = (unsigned)(uintptr_t)MI355_LDS(char, lds + (vb0 ^ (dt * 64)));
+      asm volatile("" : "+v"(v_frag[dt]));
+    }
+  }
+
+  half8 qf[8];
+  // Q rows of pass ps: requested as they lie in memory (rows at or beyond Sq: zeros), later scaled by scale . log2(e),
+  // rounded to the 16-bit format again and kept as the B operands of the score MFMAs
+  auto request_q = [&](const Pass& ps, half8* raw) {
+    const int ql = opaque_lane_id();  // (addresses derived from `lane` would be held in registers through the key walk)
+    const int q_row = ps.qb * BLOCK_M + wave * 32 + (ql & 31);
+    const half_t* qp = Q + ps.b * lay.q_b + ps.hq * lay.q_h + (size_t)q_row * lay.q_r + (ql >> 5) * 8;
+    if (q_row < Sq) {
+#pragma unroll
+      for (int ks = 0; ks < 8; ks++) raw[ks] = *reinterpret_cast<const half8*>(qp + ks * 16);
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < 8; ks++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) raw[ks][e] = (half_t)0;
+    }
+  };
+  auto convert_q = [&](const half8* raw) {
+#pragma unroll
+    for (int ks = 0; ks < 8; ks++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) qf[ks][e] = cvt16<BF>(to_f32<BF>(raw[ks][e]) * scale_log2e);
+  };
+
+  Pass cur = pass_at(0);
+  if (cur.ord < 0) return;  // (the launcher starts no more workgroups than units)
+  bool tiles_requested = false;  // K 0, K 1, V 0 of `cur` already requested (by the pass before)
+
+  for (;;) {  // passes
+  Pass nxt;  // looked up behind trip 0 (its divisions then run beside the other waves' work, not between two passes)
+  nxt.ord = -1, nxt.b = nxt.hq = nxt.hk = nxt.qb = 0, nxt.n = 2;
+  const int q0 = cur.qb * BLOCK_M;
+  const int wq0 = q0 + wave * 32;
+  const int q_row = wq0 + r32;
+  const int n_tiles = cur.n;
+  const half_t* Kb = K + cur.b * lay.k_b + cur.hk * lay.k_h;
+  const half_t* Vb = V + cur.b * lay.v_b + cur.hk * lay.v_h;
+
+  auto issue_kv = [&](const half_t* base, unsigned rb, unsigned voff, int tile, int lds_off) {
+    char* dst = lds + lds_off + wave * 1024;
+    const int row0 = tile * FA_BLOCK_N;
+    int rem = Sk - row0;
+    rem = rem > FA_BLOCK_N ? FA_BLOCK_N : rem;
+    const buffer_rsrc_t rs = make_buffer(reinterpret_cast<const char*>(base) + (size_t)row0 * rb, (unsigned)(rem - 1) * rb + 256u);
+#pragma unroll
+    for (int i = 0; i < NI; i++) buffer_load_lds_16B(rs, voff + (unsigned)(i * NW * 4) * rb, 0, dst + i * NW * 1024);
+  };
+
+  floatx16 oacc[4];
+#pragma unroll
+  for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) oacc[dt][r] = 0.f;
+  floatx16 negm;
+#pragma unroll
+  for (int r = 0; r < 16; r++) negm[r] = 0.f;
+  float l_run = 0.f;
+  float grow_thr = -INFINITY;
+  constexpr float kRescaleThreshold = 8.f;
+
+  auto wave_active = [&](int tile) { return !CAUSAL || (tile * FA_BLOCK_N <= wq0 + 31 + causal_off); };
+
+  auto scores = [&](int koff, floatx16* s) {
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+#pragma unroll
+      for (int ks = 0; ks < 8; ks++) {
+        half8 kf = *(lds_half8_t)(uintptr_t)(k_frag[ks] + (unsigned)(koff + t * 8192));
+        s[t] = mfma16<BF>(kf, qf[ks], ks == 0 ? negm : s[t]);
+      }
+    }
+  };
+
+  // softmax of tile `tile` (scores in s) and O^T += V(slot)^T . P^T, with the scores of the following tile computed between
+  // the exponentials; LAST: there is no following tile
+  auto softmax_pv = [&](int tile, auto voff_tag, auto last_tag, floatx16* s, int koff_next, floatx16* s_next) {
+    constexpr int VOFF = decltype(voff_tag)::value;
+    constexpr bool LAST = decltype(last_tag)::value;
+    {
+      const int key0 = tile * FA_BLOCK_N;
+      const bool need_mask = (CAUSAL && (key0 + FA_BLOCK_N - 1 > wq0 + causal_off)) || (key0 + FA_BLOCK_N > Sk);
+      if (need_mask) {
+        const int lim = CAUSAL ? (q_row + causal_off < Sk - 1 ? q_row + causal_off : Sk - 1) : Sk - 1;
+        const int rel = lim - key0 - 4 * h;
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const unsigned hide = (unsigned)((rel - (32 * t + 8 * (r >> 2) + (r & 3))) >> 31);
+            const float sv = s[t][r];
+            s[t][r] = __builtin_bit_cast(float, (hide & 0xFF800000u) | (~hide & __builtin_bit_cast(unsigned, sv)));
+          }
+      }
+    }
+    float mx = s[0][0];
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[t][r]);
+    if (__builtin_amdgcn_ballot_w64(mx > grow_thr) != 0) {
+      const float mxx = fmaxf(mx, __shfl_xor(mx, 32));
+      const bool first = grow_thr == -INFINITY;
+      const float delta = first ? (mxx == -INFINITY ? 0.f : mxx) : fmaxf(mxx, 0.f);
+      const float alpha = first ? 1.f : __builtin_amdgcn_exp2f(-delta);
+      if (mxx != -INFINITY) grow_thr = kRescaleThreshold;
+      l_run *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) oacc[dt][r] *= alpha;
+#pragma unroll
+      for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[t][r] -= delta;
+#pragma unroll
+      for (int r = 0; r < 16; r++) negm[r] -= delta;
+    }
+    half8 pf[4];
+    float psum = 0.f;
+    // Scores of the next tile and the softmax of this one, step by step: score MFMA i, the K fragment of MFMA i + 3
+    // requested, and the work of score pair i (two exponentials, one packed conversion, one dot2) behind it.  A
+    // scheduling barrier after every step pins the order (a wave issues in order: only vector work placed between two
+    // MFMAs runs while the first occupies the matrix pipe).
+    __builtin_amdgcn_sched_barrier(0);
+    {
+      half8 kf[4];
+      half2v pp_prev = {(half_t)0, (half_t)0};
+      auto kread = [&](int i) { return *(lds_half8_t)(uintptr_t)(k_frag[i & 7] + (unsigned)(koff_next + (i >> 3) * 8192)); };
+      if constexpr (!LAST) {
+        kf[0] = kread(0);
+        kf[1] = kread(1);
+        kf[2] = kread(2);
+      }
+#pragma unroll
+      for (int i = 0; i < 16; i++) {
+        const int t = i >> 3, ks = i & 7, r = 2 * ks;
+        if constexpr (!LAST) {
+          if (i + 3 < 16) kf[(i + 3) & 3] = kread(i + 3);
+          s_next[t] = mfma16<BF>(kf[i & 3], qf[ks], ks == 0 ? negm : s_next[t]);
+        }
+        // (the empty statement ties the pair's arithmetic to this step: without side effects of its own it is placed
+        // wherever instruction selection likes, scheduling barriers or not)
+        float e0 = __builtin_amdgcn_exp2f(s[t][r]), e1 = __builtin_amdgcn_exp2f(s[t][r + 1]);
+        if (i > 0) psum = dot2_ones<BF>(pp_prev, psum);  // (one step behind its conversion, as in fa_fwd_d128_pipe)
+        half2v pp = cvt16x2<BF>(e0, e1);
+        asm volatile("" : "+v"(pp), "+v"(psum));
+        pf[t * 2 + (r >> 3)][r & 7] = pp[0];
+        pf[t * 2 + (r >> 3)][(r & 7) + 1] = pp[1];
+        pp_prev = pp;
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      psum = dot2_ones<BF>(pp_prev, psum);
+    }
+    l_run += psum;
+    half4 vlo[3], vhi[3];  // V^T reads and their waits in assembly, as in fa_fwd_d128_pipe
+    auto vr = [&](auto itag) {
+      constexpr int i = decltype(itag)::value;
+      constexpr int off = VOFF + (i >> 2) * 4096;
+      half4 &lo = vlo[i % 3], &hi = vhi[i % 3];
+      const unsigned addr = v_frag[i & 3];
+      asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4"
+                   : "=&v"(lo), "=&v"(hi)
+                   : "v"(addr), "n"(off), "n"(off + 2048));
+    };
+    vr(std::integral_constant<int, 0>{});
+    vr(std::integral_constant<int, 1>{});
+    static_for<0, 16>([&](auto itag) {
+      constexpr int i = decltype(itag)::value;
+      if constexpr (i + 2 < 16) vr(std::integral_constant<int, i + 2>{});
+      half4 &lo = vlo[i % 3], &hi = vhi[i % 3];
+      if constexpr (i + 2 < 16)
+        asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(lo), "+v"(hi));
+      else if constexpr (i + 1 < 16)
+        asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(lo), "+v"(hi));
+      else
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lo), "+v"(hi));
+      const half8 vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      oacc[i & 3] = mfma16<BF>(vf, pf[i >> 2], oacc[i & 3]);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+
+  floatx16 sa[2], sb[2];
+  if (!tiles_requested) {
+    half8 raw[8];
+    request_q(cur, raw);
+    issue_kv(Kb, k_rb, k_voff, 0, 0);
+    issue_kv(Vb, v_rb, v_voff, 0, VBUF);
+    issue_kv(Kb, k_rb, k_voff, 1, TILE_B);
+    convert_q(raw);
+    wait_vmcnt0();
+    __syncthreads();
+  }
+  scores(0, sa);  // every wave sees keys in a pass's first tile
+  // trip 0 overwrites the K(0) slot with K(2): every wave must have read its K(0) fragments first
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __syncthreads();
+
+  // trip j (PAR = j & 1): loads for K(j+2) and V(j+1); scores of tile j+1; softmax + PV of tile j
+  auto trip = [&](auto par_tag, int j, floatx16* s_cur, floatx16* s_next) {
+    constexpr int PAR = decltype(par_tag)::value;
+    constexpr int K_CUR = PAR * TILE_B, K_NEXT = (1 - PAR) * TILE_B, V_CUR = PAR * TILE_B, V_NEXT = VBUF + (1 - PAR) * TILE_B;
+    if (j + 2 < n_tiles) issue_kv(Kb, k_rb, k_voff, j + 2, K_CUR);
+    if (j + 1 < n_tiles) issue_kv(Vb, v_rb, v_voff, j + 1, V_NEXT);
+    if (wave_active(j)) softmax_pv(j, std::integral_constant<int, V_CUR>{}, std::false_type{}, s_cur, K_NEXT, s_next);  // idle from here on otherwise
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+  };
+  // A pass of an even tile count runs its last tile (an odd trip) apart, behind the requests for the next pass: there are
+  // no loads and no scores left for this pass, neither K slot is read again and V slot 0 was last read by the trip before.
+  // A pass of an odd count ends with an ordinary trip and the requests follow it.
+  const int n_plain = (n_tiles & 1) ? n_tiles : n_tiles - 1;
+  for (int j = 0; j < n_plain; j += 2) {
+    trip(std::integral_constant<int, 0>{}, j, sa, sb);
+    if (j == 0) nxt = pass_at(cur.ord + 1);  // (two tiles at least: trip 0 is never the last)
+    if (j + 1 < n_plain) trip(std::integral_constant<int, 1>{}, j + 1, sb, sa);
+  }
+
+  // ---- between passes ----
+  half8 qraw[8];
+  request_q(nxt.ord >= 0 ? nxt : cur, qraw);  // (unconditional, and converted unconditionally below: the old Q fragments are dead from here on)
+  if (nxt.ord >= 0) {
+    const half_t* Kn = K + nxt.b * lay.k_b + nxt.hk * lay.k_h;
+    const half_t* Vn = V + nxt.b * lay.v_b + nxt.hk * lay.v_h;
+    issue_kv(Kn, k_rb, k_voff, 0, 0);
+    issue_kv(Vn, v_rb, v_voff, 0, VBUF);
+    issue_kv(Kn, k_rb, k_voff, 1, TILE_B);
+  }
+  if (n_plain < n_tiles) {
+    if (wave_active(n_tiles - 1)) softmax_pv(n_tiles - 1, std::integral_constant<int, TILE_B>{}, std::true_type{}, sb, 0, sa);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  }
+  const float l_tot = l_run + __shfl_xor(l_run, 32);
+  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  half8 orow[32 / 4];  // the rows this lane stores: 16-byte chunk ec of rows er, er + 4, ...
+  const int el = opaque_lane_id();
+  const int er = el >> 4, ec = el & 15;
+  {
+    // Output through the wave's staging region, STG_ROWS rows per round (chunk c of row r in slot c ^ (r & 15)): a lane
+    // holds 4-value pieces of one row; whole 16-byte chunks are read back, to be stored as full rows
+    char* ep = lds + STG + wave * (STG_ROWS * 256);
+    const int e32 = el & 31, eh = el >> 5;
+#pragma unroll
+    for (int round = 0; round < 32 / STG_ROWS; round++) {
+      if (STG_ROWS == 32 || (e32 / STG_ROWS) == round) {
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+          for (int q = 0; q < 4; q++) {
+            const half4 v = {cvt16<BF>(oacc[dt][4 * q] * inv), cvt16<BF>(oacc[dt][4 * q + 1] * inv), cvt16<BF>(oacc[dt][4 * q + 2] * inv),
+                             cvt16<BF>(oacc[dt][4 * q + 3] * inv)};
+            *reinterpret_cast<half4*>(ep + (e32 % STG_ROWS) * 256 + (((dt * 4 + q) ^ (e32 & 15)) * 16) + 8 * eh) = v;
+          }
+      }
+#pragma unroll
+      for (int it = 0; it < STG_ROWS / 4; it++) {
+        const int lr = it * 4 + er, row = round * STG_ROWS + lr;
+        orow[round * (STG_ROWS / 4) + it] = *reinterpret_cast<const half8*>(ep + lr * 256 + ((ec ^ (row & 15)) * 16));
+      }
+    }
+  }
+  convert_q(qraw);  // (the oldest of the requests)
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // the next pass's first tiles
+  __syncthreads();
+  {
+    // the stores are left in flight: they drain under the next pass's first trip, whose closing wait covers them
+    half_t* Ob = O + cur.b * lay.o_b + cur.hq * lay.o_h;
+#pragma unroll
+    for (int it = 0; it < 8; it++) {
+      const int row = it * 4 + er;
+      if (wq0 + row < Sq) *reinterpret_cast<half8*>(Ob + (size_t)(wq0 + row) * lay.o_r + ec * 8) = orow[it];
+    }
+  }
+  if (nxt.ord < 0) break;
+  tiles_requested = true;
+  cur = nxt;
+  }  // passes
+}
+
+static const char* kFaVariants[] = {"d128_bm128_bn64_w4_pipelined", "d128_bm128_bn64_w4", "d128_bm256_bn64_w8_pipelined",
+                                    "d128_bm256_bn64_w8_walk", "d128_bm128_bn64_w4_walk"};
+int fa_variant_count() { return 5; }
+const char* fa_variant_name(int i) { return (i >= 0 && i < 5) ? kFaVariants[i] : nullptr; }
 
 }  // namespace mi355
 
 using namespace mi355;
+
+// number of CUs of the current device (cached per device)
+static int fa_cu_count() {
+  static std::atomic<int> cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
 
 template <bool BF>
 static int fa_launch(const void* q, const void* k, const void* v, void* o, int64_t B, int64_t H, int64_t Hkv, int64_t Sq,
@@ -630,7 +1099,7 @@ static int fa_launch(const void* q, const void* k, const void* v, void* o, int64
     return fail(-MI355_E_SHAPE, "%s: %lld query heads over %lld key/value heads", who, (long long)H, (long long)Hkv);
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o))
     return fail(-MI355_E_ALIGN, "%s: q, k, v, o must be 16-byte aligned", who);
-  if (variant > 2) return fail(-MI355_E_DTYPE, "%s: variant %d out of range", who, variant);
+  if (variant > 4) return fail(-MI355_E_DTYPE, "%s: variant %d out of range", who, variant);
   if (!(scale > 0.f) || !isfinite(scale)) return fail(-MI355_E_SHAPE, "%s: scale must be positive and finite", who);
   const int BH = (int)(B * H);
   const int q_blocks = (int)((Sq + FA_BLOCK_M - 1) / FA_BLOCK_M);
@@ -645,6 +1114,36 @@ static int fa_launch(const void* q, const void* k, const void* v, void* o, int64
   // Without a mask, and with enough 256-query blocks for every CU, the 8-wave form is ahead (2 x 32 x 4096: 503 against
   // 514 us); with the causal mask the two are level and the 4-wave form has the finer-grained tail.
   if (variant < 0 && !is_causal && (int64_t)BH * ((Sq + 255) / 256) >= 512) variant = 2;
+  if (variant == 3 || variant == 4) {
+    // the persistent forms: every pass needs two key tiles, and the masked form a square mask (no pass without keys)
+    const bool w8 = variant == 3;
+    const int bm = w8 ? 256 : 128;
+    const int qbw = (int)((Sq + bm - 1) / bm);
+    const int64_t units_w = (int64_t)BH * (is_causal ? (qbw + 1) / 2 : qbw);
+    if (Sk < 128 || (is_causal && Sq != Sk) || units_w >= (1ll << 30))
+      return fail(-MI355_E_SHAPE, "%s: the persistent form needs Sk >= 128%s (Sq=%lld Sk=%lld)", who, is_causal ? " and Sq == Sk" : "",
+                  (long long)Sq, (long long)Sk);
+    const void* kern = w8 ? (is_causal ? (const void*)fa_fwd_d128_walk<true, BF, 8> : (const void*)fa_fwd_d128_walk<false, BF, 8>)
+                          : (is_causal ? (const void*)fa_fwd_d128_walk<true, BF, 4> : (const void*)fa_fwd_d128_walk<false, BF, 4>);
+    static std::atomic<uint64_t> okw[4] = {};
+    const int ldsw = 4 * FA_BLOCK_N * 256 + (w8 ? 8 * 8192 : 4 * 2048);  // K and V rings + output staging
+    if (int rc = allow_lds(kern, ldsw, okw[(w8 ? 2 : 0) + (is_causal ? 1 : 0)], "fa_fwd_d128_walk")) return rc;
+    int g = fa_cu_count() * (w8 ? 1 : 2);  // workgroups resident at once
+    if (((BH / lay.group) & 7) == 0) g &= ~7;  // units of one K/V head stay on the XCD that a workgroup runs on
+    if (g < 1) g = 1;
+    if (units_w < g) g = (int)units_w;
+    dim3 grid(g), block(w8 ? 512 : 256);
+    const half_t *qp = (const half_t*)q, *kp = (const half_t*)k, *vp = (const half_t*)v;
+    half_t* op = (half_t*)o;
+    int bh_i = BH, sq_i = (int)Sq, sk_i = (int)Sk;
+    FaLayout lay_v = lay;
+    float sc = scale_log2e;
+    int qb_i = qbw;
+    void* args[] = {&qp, &kp, &vp, &op, &bh_i, &sq_i, &sk_i, &sc, &qb_i, &lay_v};
+    hipError_t e = hipLaunchKernel(kern, grid, block, args, ldsw, reinterpret_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail((int)e, "%s: launch of fa_fwd_d128_walk failed: %s", who, hipGetErrorString(e));
+    return check_launch("fa_fwd_d128_walk", grid, block, ldsw);
+  }
   if (variant == 2) {
     // eight waves: 256-query blocks, one workgroup per CU
     auto kern = is_causal ? fa_fwd_d128_pipe<true, false, BF, 8> : fa_fwd_d128_pipe<false, false, BF, 8>;

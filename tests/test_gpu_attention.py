@@ -68,6 +68,48 @@ def test_attention_eight_wave_form(dev, Sq, Sk, causal):
     torch.testing.assert_close(got, oa.sdpa_ref(q, k, v, is_causal=causal), rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("form", ["d128_bm256_bn64_w8_walk", "d128_bm128_bn64_w4_walk"])
+@pytest.mark.parametrize("B,H,Sq,Sk", [(2, 3, 128, 128), (1, 2, 255, 255), (1, 2, 257, 257), (2, 3, 320, 320), (1, 5, 777, 777),
+                                       (3, 40, 1024, 1024), (2, 3, 300, 777), (1, 2, 700, 128), (1, 9, 192, 4200)])
+def test_attention_persistent_forms(dev, B, H, Sq, Sk, form, causal):
+    """The persistent forms (one workgroup per CU slot running its passes back to back, the next pass's rows and first
+    tiles requested under the current pass's last tile): passes of even and odd tile counts, ragged lengths, more
+    units than workgroup slots (3 x 40 heads), a single workgroup per head -- against the oracle and bit-identical to
+    the 4-wave form, whose arithmetic per query they repeat.  The masked form only takes square problems."""
+    import iree_turbine_amd as ita
+    from oracle import attention as oa, inputs
+
+    announce(f"flash_attn_fwd {form} B={B} H={H} Sq={Sq} Sk={Sk} causal={causal}")
+    vw = ita._lib.variants("flash_attn_fwd").index(form)
+    q, k, v = inputs.attention_inputs(B, H, Sq, 128, seed=14, Sk=Sk)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    ow, o4 = torch.empty_like(qd), torch.empty_like(qd)
+    if causal and Sq != Sk:
+        with pytest.raises(ValueError, match="persistent form"):
+            ita.launch.flash_attn_fwd_out(qd, kd, vd, ow, causal, 0.0, vw)
+        return
+    ita.launch.flash_attn_fwd_out(qd, kd, vd, ow, causal, 0.0, vw)
+    ita.launch.flash_attn_fwd_out(qd, kd, vd, o4, causal, 0.0, 0)
+    assert torch.equal(ow, o4)
+    if B * H <= 12:
+        torch.testing.assert_close(ow.float().cpu(), oa.sdpa_ref(q, k, v, is_causal=causal), rtol=RTOL, atol=ATOL)
+
+
+def test_attention_persistent_forms_need_two_tiles(dev):
+    """A pass of the persistent forms has at least two key tiles: fewer than 128 keys is refused, nothing is launched."""
+    import iree_turbine_amd as ita
+    from oracle import inputs
+
+    announce("flash_attn_fwd persistent forms, Sk < 128")
+    q, k, v = [t.to(dev) for t in inputs.attention_inputs(1, 2, 100, 128, seed=15)]
+    o = torch.full_like(q, 7.0)
+    for form in ("d128_bm256_bn64_w8_walk", "d128_bm128_bn64_w4_walk"):
+        with pytest.raises(ValueError, match="Sk >= 128"):
+            ita.launch.flash_attn_fwd_out(q, k, v, o, False, 0.0, ita._lib.variants("flash_attn_fwd").index(form))
+    assert bool((o == 7.0).all())
+
+
 def test_attention_causal_more_queries_than_keys(dev):
     """Lower-right aligned causal mask with Sq > Sk: query i sees keys j <= i - (Sq - Sk), so the first
     Sq - Sk queries see no key at all.  Those rows are defined as zero (the sum of an empty softmax); every
