@@ -584,11 +584,22 @@ def cpu_attention(q, k, v, causal):
 
 
 def cpu_decode(q, kc, vc, bt, sl):
+    """The oracle on the first 4 sequences, over a cache that holds only THEIR pages (renumbered): the oracle converts
+    the cache it is handed to fp32 as a whole, and with the full 1.1 GB cache that conversion is what would be timed."""
     from oracle import paged_decode as op
     n = 4
-    t = _time_cpu(lambda: op.paged_decode_ref(q[:n], kc, vc, bt[:n], sl[:n]), reps=2)
+    page = kc.shape[1]
+    used = [int((int(sl[i]) + page - 1) // page) for i in range(n)]
+    ids = torch.cat([bt[i, :used[i]].long() for i in range(n)])
+    kc_s, vc_s = kc[ids].contiguous(), vc[ids].contiguous()
+    bt_s = torch.zeros(n, max(used), dtype=bt.dtype)
+    at = 0
+    for i in range(n):
+        bt_s[i, :used[i]] = torch.arange(at, at + used[i], dtype=bt.dtype)
+        at += used[i]
+    t = _time_cpu(lambda: op.paged_decode_ref(q[:n], kc_s, vc_s, bt_s, sl[:n]), reps=2)
     return {"value": 4096.0 * int(sl[:n].sum()) / t / 1e9, "unit": "GB/s",
-            "sample": f"gather + dense fp32 attention for {n} of the {q.shape[0]} sequences, best of 2 after 1 warm-up"}
+            "sample": f"gather + dense fp32 attention for {n} of the {q.shape[0]} sequences over their own pages, best of 2 after 1 warm-up"}
 
 
 def cpu_paged_prefill(q, kc, vc, bt, sl):
@@ -657,6 +668,14 @@ def measure(name: str, dev, steps: int, warmup: int, with_cpu: bool):
     return rec
 
 
+# Calibration runs that ride along with every default run, so that the line carries the vendor library's figure and the
+# board's ceilings from the SAME box and session as the kernels' (boxes differ by a few per cent): hipBLASLt on the
+# headline shape, the register-only MFMA loops on benchmark-like operands (plain and with a GEMM's register structure),
+# the prefill tile's instruction mix out of registers.  They are not part of the path; `calibration: true` marks them.
+CALIBRATION_IN_DEFAULT_RUN = ("library_gemm_8192", "mfma_f16_regloop_benchmark", "mfma_f16x16walk_regloop_benchmark",
+                              "mfma_fp4_regloop_benchmark", "mfma_fp4x16walk_regloop_benchmark", "fa_issue_regloop_mix_w2",
+                              "fa_issue_regloop_mfma_w2")
+
 # the legs of the metric (GEMM, causal prefill, MXFP4 GEMM, decode): each gets its CPU baseline in the same run
 CPU_TIMED = ("gemm_8192", "fa_causal", "fa_noncausal", "decode", "mxfp4_4096x8192x8192", "mxfp4_32x8192x8192")
 
@@ -690,6 +709,14 @@ def main() -> int:
             torch.cuda.empty_cache()
             rec = measure(name, dev, args.steps, args.warmup, with_cpu=not args.no_cpu and name in CPU_TIMED)
             rec.pop("config")
+            others.append(rec)
+        for name in CALIBRATION_IN_DEFAULT_RUN:
+            if name == args.workload:
+                continue
+            torch.cuda.empty_cache()
+            rec = measure(name, dev, args.steps, args.warmup, with_cpu=False)
+            rec.pop("config")
+            rec["calibration"] = True
             others.append(rec)
 
     line = {

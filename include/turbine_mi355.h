@@ -4,8 +4,12 @@
  * One shared object, libturbine_mi355.so, exports the functions below.  Every
  * function takes raw device pointers, plain integer sizes and the HIP stream
  * to launch on (a hipStream_t passed as void*; NULL = the legacy default
- * stream).  Nothing here allocates, synchronises or keeps state between calls:
- * the caller owns all memory, including split-K scratch.
+ * stream).  Nothing here allocates or synchronises, and the caller owns all
+ * memory, including split-K scratch.  Two entry points keep state of their own
+ * and say so where they are declared: mi355_paged_decode_attn_static (its
+ * scratch is a device array inside the library image, one copy per GPU) and
+ * mi355_paged_decode_attn_fused (arrival counters in caller memory, tagged
+ * with a per-call number the library hands out).
  *
  * Return value: 0 on success; a negative MI355_E_* code when the arguments
  * violate the kernel's contract (nothing was launched); a positive value is
@@ -183,10 +187,17 @@ int mi355_paged_decode_attn(const void* q, const void* k_cache, const void* v_ca
  * or bf16 tensors (dtype = MI355_F16 | MI355_BF16), with the merge of the kv splits done inside the
  * phase-0 kernel by whichever workgroup of a (sequence, kv head) finishes last, instead of by a second
  * launch -- when the whole grid is resident at once (num_seqs * num_kv_heads * num_splits <= 512);
- * larger grids run the two launches, which is faster there, and leave `arrivals` untouched.  arrivals: int32 [num_seqs * num_kv_heads] of device memory that is all zero when the kernel
- * starts; the kernel leaves it all zero again, so one buffer zeroed once serves every later call that is
- * ordered after this one (calls that may overlap need a buffer each).  Not needed (may be NULL) for
- * num_splits == 1.  No counterpart in the reference (GQA semantics tests/dynamo/llama_test.py:82-91).
+ * larger grids run the two launches, which is faster there, and leave `arrivals` untouched.
+ * arrivals: int32 [num_seqs * num_kv_heads] of device memory, the per-(sequence, kv head) arrival
+ * counters.  Every call tags the words it counts in with a number of its own (handed out inside the
+ * library, 1 .. 2^20 - 1, cyclic) and treats a word that carries another tag as zero, so a call does
+ * not depend on the buffer's contents: an earlier call that did not run to its end, or memory that was
+ * never cleared, does no harm (short of a stale word that happens to carry this call's tag).  A call
+ * that completes leaves its words zero.  One buffer serves every call ordered after this one; calls
+ * that may overlap need a buffer each.  A captured graph replays one tag: its replays rely on the words
+ * being left zero by the replay before.  Not needed (may be NULL) for num_splits == 1.
+ * num_splits <= 512 on this path.  No counterpart in the reference (GQA semantics
+ * tests/dynamo/llama_test.py:82-91).
  */
 int mi355_paged_decode_attn_fused(const void* q, const void* k_cache, const void* v_cache,
                                   const int32_t* block_table, const int32_t* seq_lens, void* out,

@@ -54,6 +54,19 @@ __device__ __forceinline__ int opaque_lane_id() {
 
 __device__ __forceinline__ void wait_vmcnt0() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
+// One 16-byte global store per lane as ONE instruction, written out: kernels whose later `s_waitcnt vmcnt(n)` counts
+// past the stores of an epilogue (stores and loads share the counter, in issue order) need the number of store
+// instructions fixed by the source, not left to how the compiler lowers an assignment.
+// The two wait states behind the store are the part's rule for a store of more than 8 bytes followed by a vector
+// instruction that overwrites its data registers (the store reads them late); the compiler inserts them for stores it
+// emits itself and cannot for one inside an assembly statement.  Without them the next conversion into the same
+// registers corrupted one value in sixteen.
+template <typename T>
+__device__ __forceinline__ void store_global_16B(void* p, const T& v) {
+  static_assert(sizeof(T) == 16, "store_global_16B stores exactly 16 bytes per lane");
+  asm volatile("global_store_dwordx4 %0, %1, off\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
+}
+
 // D(32x32) += A(32x16) * B(16x32).  Lane l supplies A[l%32][8*(l/32) .. +7] and
 // B[8*(l/32) .. +7][l%32]; it receives D[8*(r/4) + 4*(l/32) + r%4][l%32] in register r.
 __device__ __forceinline__ floatx16 mfma_32x32x16(half8 a, half8 b, floatx16 c) {

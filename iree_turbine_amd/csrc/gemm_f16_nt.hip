@@ -953,11 +953,11 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_stream(const half_t* __restri
         asm volatile("ds_read_b128 %0, %1 offset:3072" : "=v"(rv[3]) : "v"(ra ^ 96u));
         asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(rv[0]), "+v"(rv[1]), "+v"(rv[2]), "+v"(rv[3]));
 #pragma unroll
-        for (int it = 0; it < 4; it++) *reinterpret_cast<half8*>(cbase + (size_t)(j * 16 + it * 4) * N) = rv[it];
+        for (int it = 0; it < 4; it++) store_global_16B(cbase + (size_t)(j * 16 + it * 4) * N, rv[it]);  // one instruction each
         if (j == 3) {
           // Half of the stores are out.  The next tile's first slab runs without load waits: everything it and the
           // first interval after it read was loaded before this tile's last interval, i.e. all but the 4 loads
-          // issued since -- which are followed in the queue by the 16 stores above.
+          // issued since -- which are followed in the queue by the 16 store instructions above.
           asm volatile("s_waitcnt vmcnt(20)" ::: "memory");
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -967,9 +967,12 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_stream(const half_t* __restri
 #pragma unroll
       for (int j = 0; j < 8; j++) {
 #pragma unroll
-        for (int i = 0; i < 8; i++)
-          OutPack<OutT, BF>::store4(crow + (size_t)(j * 16) * N + i * 16, acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
-        if (j == 3) asm volatile("s_waitcnt vmcnt(36)" ::: "memory");  // as above, behind 32 stores
+        for (int i = 0; i < 8; i++) {
+          static_assert(sizeof(OutT) == 2 || sizeof(OutT) == 4, "16- or 32-bit output");
+          const floatx4 v = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
+          store_global_16B(crow + (size_t)(j * 16) * N + i * 16, v);  // one instruction each
+        }
+        if (j == 3) asm volatile("s_waitcnt vmcnt(36)" ::: "memory");  // as above, behind 32 store instructions
         __builtin_amdgcn_sched_barrier(0);
       }
     }

@@ -1431,7 +1431,8 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_stream(const uint8_t* __restri
           asm volatile("ds_read_b128 %0, %1 offset:1024" : "=v"(rv[1]) : "v"(ra ^ 64u));
           asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(rv[0]), "+v"(rv[1]));
 #pragma unroll
-          for (int it = 0; it < 2; it++) *reinterpret_cast<half8*>(cbase + (size_t)(j * 16 + it * 8) * N + ih * 64) = rv[it];
+          for (int it = 0; it < 2; it++)  // one store instruction each: the next tile's first waits count past these 32
+            store_global_16B(cbase + (size_t)(j * 16 + it * 8) * N + ih * 64, rv[it]);
           __builtin_amdgcn_sched_barrier(0);
         }
       }

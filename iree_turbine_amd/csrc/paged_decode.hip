@@ -89,7 +89,7 @@ __global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
     const half_t* __restrict__ Q, const half_t* __restrict__ Kc, const half_t* __restrict__ Vc,
     const int* __restrict__ block_table, const int* __restrict__ seq_lens, float* __restrict__ part_acc,
     float* __restrict__ part_ml, half_t* __restrict__ out, half_t* __restrict__ final_out, int num_kv_heads, int max_pages_per_seq, int num_splits,
-    float scale_log2e, int window, int page_shift, int num_pages, int* __restrict__ arrivals) {
+    float scale_log2e, int window, int page_shift, int num_pages, int* __restrict__ arrivals, unsigned epoch) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -356,18 +356,33 @@ __global__ __launch_bounds__(PD_WAVES * 64) void paged_decode_phase0(
   if (out || !arrivals) return;
 
   // ---- merge of the splits by whichever workgroup of this (sequence, kv head) finishes last ----
-  // Every workgroup waits until its partials (device-scope stores) are written, then counts itself in with a
-  // device-scope atomic; the one that finds all the others counted merges them (what paged_decode_phase1 does in
-  // a launch of its own) and puts the counter back to zero, so the array is all zero again when the kernel ends.
-  // Partials of other workgroups are read with device-scope loads, past this XCD's L2.
+  // Every workgroup waits until its partials are written, then counts itself in on the (sequence, kv head) counter;
+  // the one that completes the count merges the splits (what paged_decode_phase1 does in a launch of its own) and puts
+  // the counter back to zero.
+  // Ordering.  The partials are written with device-scope stores: they go through to the memory every XCD sees (no
+  // dirty line stays behind in this XCD's L2).  vmcnt(0) returns once all of them are acknowledged there, and only
+  // then is the counter's read-modify-write issued, itself at device scope, so it executes behind the stores in the
+  // one place all workgroups' accesses to that word are ordered.  A workgroup that observes the completed count
+  // therefore runs after every other workgroup's partials are in memory, and reads them with device-scope loads,
+  // which do not hit in a cache that could hold an older copy.  That is release (stores, wait, RMW) and acquire (RMW,
+  // then loads) spelled with a wait and cache-bypassing accesses instead of cache-wide write-back and invalidate
+  // operations: one of those per workgroup tripled the kernel's time.
+  // The counter word is (epoch << 12) | count.  A word that carries another epoch -- whatever an earlier call that
+  // did not run to its end, or memory that was never cleared, left behind -- counts as zero, so a call does not
+  // depend on what it finds; epochs are handed out per call by the launcher (1 .. 2^20 - 1, cyclic).
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   int* flag = reinterpret_cast<int*>(lds);
   if (threadIdx.x == 0) {
-    int* ctr = arrivals + (size_t)seq * num_kv_heads + kvh;
-    const int before = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const int last = before == num_splits - 1;
-    if (last) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    unsigned* ctr = reinterpret_cast<unsigned*>(arrivals) + (size_t)seq * num_kv_heads + kvh;
+    unsigned seen = __hip_atomic_load(ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    unsigned count;
+    do {  // at most num_splits workgroups contend for the word
+      count = ((seen >> 12) == epoch ? (seen & 0xFFFu) : 0u) + 1u;
+    } while (!__hip_atomic_compare_exchange_strong(ctr, &seen, (epoch << 12) | count, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT));
+    const int last = count == (unsigned)num_splits;
+    if (last) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     *flag = last;
   }
   __syncthreads();
@@ -430,6 +445,12 @@ static const char* kDecodeVariants[] = {"d128_p16_w4_2pages"};
 int decode_variant_count() { return 1; }
 const char* decode_variant_name(int i) { return i == 0 ? kDecodeVariants[0] : nullptr; }
 
+// A fresh tag for the arrival counters of the one-launch form, 1 .. 2^20 - 1, per call and process-wide.
+static unsigned next_decode_epoch() {
+  static std::atomic<unsigned> counter{0};
+  return counter.fetch_add(1, std::memory_order_relaxed) % ((1u << 20) - 1u) + 1u;
+}
+
 template <int G, bool BF>
 static int launch_phase0(const void* q, const void* kc, const void* vc, const int32_t* bt, const int32_t* sl, float* pacc,
                          float* pml, void* out, void* final_out, int32_t* arrivals, int num_seqs, int num_kv_heads, int max_pages,
@@ -442,7 +463,7 @@ static int launch_phase0(const void* q, const void* kc, const void* vc, const in
   dim3 grid(num_splits, num_kv_heads, num_seqs), block(PD_WAVES * 64);
   hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)q, (const half_t*)kc, (const half_t*)vc, bt, sl,
                      pacc, pml, (half_t*)out, (half_t*)final_out, num_kv_heads, max_pages, num_splits, scale * 1.4426950408889634f, window,
-                     page_shift, num_pages, arrivals);
+                     page_shift, num_pages, arrivals, arrivals ? next_decode_epoch() : 0u);
   return check_launch("paged_decode_phase0", grid, block, lds_bytes);
 }
 

@@ -250,23 +250,21 @@ def verify_numerics(commands: Sequence[str], *, device: int = 0, **kwargs) -> li
     return verdicts
 
 
+# One line per verdict: the labels of whatever failed, in the order the CSV consumers expect them.
+_FAILURE_LABELS = (
+    ("mean bias", lambda v: not v.mean_near_zero),
+    ("stddev", lambda v: not v.stddev_ratio_ok),
+    ("NaN mismatch", lambda v: bool(v.boo_nan_mismatch)),
+    ("structured test", lambda v: v.structured_test_passed is False),
+    ("error", lambda v: bool(v.error_message)),
+)
+
+
 def format_verdict_simple(verdict: NumericsVerdict) -> str:
     if verdict.passed:
         return "Numerics: PASS"
-    reasons = []
-    if not verdict.mean_near_zero:
-        reasons.append("mean bias")
-    if not verdict.stddev_ratio_ok:
-        reasons.append("stddev")
-    if verdict.boo_nan_mismatch:
-        reasons.append("NaN mismatch")
-    if verdict.structured_test_passed is False:
-        reasons.append("structured test")
-    if verdict.error_message:
-        reasons.append("error")
-    if not reasons:
-        reasons.append("unknown")
-    return f"Numerics: FAIL ({', '.join(reasons)})"
+    labels = [label for label, failed in _FAILURE_LABELS if failed(verdict)] or ["unknown"]
+    return "Numerics: FAIL (" + ", ".join(labels) + ")"
 
 
 def format_verdict_verbose(verdict: NumericsVerdict) -> str:

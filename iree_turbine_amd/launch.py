@@ -173,16 +173,22 @@ def paged_decode_phase1_out(part_acc: Tensor, part_ml: Tensor, out: Tensor) -> T
     return out
 
 
-_ARRIVALS: dict[tuple[int, int], Tensor] = {}  # (device index, stream) -> zeroed int32 counters, grown on demand
+_ARRIVALS: dict[tuple[int, int], Tensor] = {}  # (device index, stream) -> int32 arrival counters, grown on demand
 
 
 def _arrival_counters(dev: torch.device, n: int) -> Tensor:
-    """The per-(sequence, kv head) arrival counters of the one-launch decode.  The kernel needs them zero when it
-    starts and leaves them zero, so one buffer per stream, zeroed when it is created, serves every call on that
-    stream (launches on one stream are ordered; two streams never share a buffer)."""
+    """The per-(sequence, kv head) arrival counters of the one-launch decode: one buffer per stream (launches on one
+    stream are ordered; two streams never share a buffer).  The kernel tags what it counts with a per-call number and
+    ignores words that carry another, so it does not depend on the buffer's contents; the buffer is zeroed all the
+    same when it is created -- eagerly: under stream capture the fill would be recorded instead of run, so the
+    first call on a stream has to happen outside a capture."""
     key = (dev.index if dev.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(dev).cuda_stream)
     buf = _ARRIVALS.get(key)
     if buf is None or buf.numel() < n:
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("paged_decode_attn: the arrival counters of this stream do not exist yet (or are too small "
+                               f"for {n} (sequence, kv head) pairs) and cannot be created while the stream is being "
+                               "captured; run the same call once eagerly first")
         buf = torch.zeros(max(n, 4096), dtype=torch.int32, device=dev)
         _ARRIVALS[key] = buf
     return buf

@@ -209,6 +209,88 @@ def test_decode_one_launch_merge_equals_two_phase(dev):
     assert launch._ARRIVALS and all(int(buf.abs().sum()) == 0 for buf in launch._ARRIVALS.values())
 
 
+def test_decode_one_launch_merge_does_not_depend_on_the_counters(dev):
+    """The arrival counters are tagged per call: words left behind by a call that never finished, or memory that was
+    never cleared, count as zero.  The counters are filled with junk (words whose tag cannot be a live call's: tags
+    are at most 2^20 - 1, the junk carries 0xFFFFF) before each of two calls; the result is the two-launch result bit
+    for bit and the words the call used are zero afterwards."""
+    import iree_turbine_amd  # noqa: F401
+    from iree_turbine_amd import _lib
+    from oracle import inputs
+
+    announce("decode one-launch merge over junk counters")
+    lib = _lib.load()
+    q, kc, vc, bt, sl = _to(dev, *inputs.paged_decode_inputs(num_seqs=5, min_len=100, max_len=1500, seed=47))
+    S, Hq, D = q.shape
+    P, page, Hkv, _ = kc.shape
+    splits = 5
+    pacc = torch.empty((S, Hq, splits, D), dtype=torch.float32, device=dev)
+    pml = torch.empty((S, Hq, splits, 2), dtype=torch.float32, device=dev)
+    ref = torch.empty_like(q)
+    rc = lib.mi355_paged_decode_attn(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), bt.data_ptr(), sl.data_ptr(), ref.data_ptr(),
+                                     pacc.data_ptr(), pml.data_ptr(), S, Hq, Hkv, D, page, bt.shape[1], P, splits, 128 ** -0.5,
+                                     _lib.current_stream_ptr(dev))
+    _lib.check(rc, "two-launch decode")
+    for junk in (0xFFFFF003, 0xFFFFF000 | (splits - 1)):
+        counters = torch.full((S * Hkv,), junk - (1 << 32), dtype=torch.int32, device=dev)
+        out = torch.full_like(q, 9.0)
+        rc = lib.mi355_paged_decode_attn_fused(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), bt.data_ptr(), sl.data_ptr(),
+                                               out.data_ptr(), pacc.data_ptr(), pml.data_ptr(), counters.data_ptr(), S, Hq, Hkv, D,
+                                               page, bt.shape[1], P, splits, 128 ** -0.5, 0, _lib.dtype_code(torch.float16),
+                                               _lib.current_stream_ptr(dev))
+        _lib.check(rc, "one-launch decode")
+        assert torch.equal(out, ref)
+        assert int(counters.abs().sum()) == 0
+
+
+def test_decode_one_launch_merge_under_graph_replay(dev):
+    """The one-launch form captured into a HIP graph (after one eager call, which creates the stream's counters),
+    replayed several times with eager calls of other shapes in between, then called eagerly again: every result is
+    the two-launch result bit for bit.  A replay reuses its call's tag; it relies on the replay before having left
+    its words zero."""
+    import iree_turbine_amd  # noqa: F401
+    from iree_turbine_amd import _lib, launch
+    from oracle import inputs
+
+    announce("decode one-launch merge, graph capture and replays")
+    lib = _lib.load()
+    q, kc, vc, bt, sl = _to(dev, *inputs.paged_decode_inputs(num_seqs=6, min_len=200, max_len=1800, seed=48))
+    q2, kc2, vc2, bt2, sl2 = _to(dev, *inputs.paged_decode_inputs(num_seqs=3, min_len=10, max_len=700, seed=49))
+    S, Hq, D = q.shape
+    P, page, Hkv, _ = kc.shape
+    splits = 4
+    pacc = torch.empty((S, Hq, splits, D), dtype=torch.float32, device=dev)
+    pml = torch.empty((S, Hq, splits, 2), dtype=torch.float32, device=dev)
+    ref = torch.empty_like(q)
+    rc = lib.mi355_paged_decode_attn(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), bt.data_ptr(), sl.data_ptr(), ref.data_ptr(),
+                                     pacc.data_ptr(), pml.data_ptr(), S, Hq, Hkv, D, page, bt.shape[1], P, splits, 128 ** -0.5,
+                                     _lib.current_stream_ptr(dev))
+    _lib.check(rc, "two-launch decode")
+    side = torch.cuda.Stream(device=dev)  # (default priority)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        out = torch.empty_like(q)
+        launch.paged_decode_attn_out(q, kc, vc, bt, sl, out, 0.0, splits)  # eager: creates this stream's counters
+        assert torch.equal(out, ref)
+        graph = torch.cuda.CUDAGraph()
+        out.fill_(3.0)
+        with torch.cuda.graph(graph, stream=side):
+            launch.paged_decode_attn_out(q, kc, vc, bt, sl, out, 0.0, splits)
+        for rep in range(4):
+            out.fill_(float(rep))
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, ref), f"replay {rep}"
+            other = torch.ops.mi355.paged_decode_attn(q2, kc2, vc2, bt2, sl2, 0.0, 3)  # eager work between the replays
+            torch.cuda.synchronize()
+            assert torch.isfinite(other.float()).all()
+        out.fill_(5.0)
+        launch.paged_decode_attn_out(q, kc, vc, bt, sl, out, 0.0, splits)
+        torch.cuda.synchronize()
+        assert torch.equal(out, ref)
+    torch.cuda.current_stream(dev).wait_stream(side)
+
+
 def test_decode_full_size(dev):
     """The benchmark configuration (64 seqs, 32/8 heads, ctx in [512, 8192]) against the oracle."""
     import iree_turbine_amd  # noqa: F401
