@@ -195,7 +195,8 @@ int mi355_paged_decode_attn(const void* q, const void* k_cache, const void* v_ca
  * never cleared, does no harm (short of a stale word that happens to carry this call's tag).  A call
  * that completes leaves its words zero.  One buffer serves every call ordered after this one; calls
  * that may overlap need a buffer each.  A captured graph replays one tag: its replays rely on the words
- * being left zero by the replay before.  Not needed (may be NULL) for num_splits == 1.
+ * being left zero by the replay before.  arrivals == NULL selects the two launches whatever the
+ * grid (for a caller that cannot provide counters, e.g. a first call under stream capture).
  * num_splits <= 512 on this path.  No counterpart in the reference (GQA semantics
  * tests/dynamo/llama_test.py:82-91).
  */

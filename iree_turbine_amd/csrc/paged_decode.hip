@@ -618,7 +618,6 @@ extern "C" int mi355_paged_decode_attn_fused(const void* q, const void* k_cache,
                                              void* stream) {
   const char* fn = "paged_decode_attn_fused";
   if (dtype != MI355_F16 && dtype != MI355_BF16) return fail(-MI355_E_DTYPE, "%s: dtype %d (MI355_F16 or MI355_BF16)", fn, dtype);
-  if (num_splits > 1 && !arrivals) return fail(-MI355_E_SCRATCH, "%s: num_splits > 1 needs the arrivals counters", fn);
   if (dtype == MI355_BF16)
     return decode_attn<true>(fn, q, k_cache, v_cache, block_table, seq_lens, out, part_acc, part_ml, arrivals, num_seqs, num_q_heads,
                              num_kv_heads, D, page_size, max_pages_per_seq, num_pages, num_splits, scale, window, stream);

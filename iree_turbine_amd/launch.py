@@ -176,19 +176,16 @@ def paged_decode_phase1_out(part_acc: Tensor, part_ml: Tensor, out: Tensor) -> T
 _ARRIVALS: dict[tuple[int, int], Tensor] = {}  # (device index, stream) -> int32 arrival counters, grown on demand
 
 
-def _arrival_counters(dev: torch.device, n: int) -> Tensor:
+def _arrival_counters(dev: torch.device, n: int) -> Tensor | None:
     """The per-(sequence, kv head) arrival counters of the one-launch decode: one buffer per stream (launches on one
-    stream are ordered; two streams never share a buffer).  The kernel tags what it counts with a per-call number and
-    ignores words that carry another, so it does not depend on the buffer's contents; the buffer is zeroed all the
-    same when it is created -- eagerly: under stream capture the fill would be recorded instead of run, so the
-    first call on a stream has to happen outside a capture."""
+    stream are ordered; two streams never share a buffer), zeroed when it is created.  Under stream capture a fill
+    would be recorded instead of run, so a stream that meets its first call (or a larger batch than any before) while
+    it is being captured gets no counters: that call takes the two-launch form, which needs none."""
     key = (dev.index if dev.index is not None else torch.cuda.current_device(), torch.cuda.current_stream(dev).cuda_stream)
     buf = _ARRIVALS.get(key)
     if buf is None or buf.numel() < n:
         if torch.cuda.is_current_stream_capturing():
-            raise RuntimeError("paged_decode_attn: the arrival counters of this stream do not exist yet (or are too small "
-                               f"for {n} (sequence, kv head) pairs) and cannot be created while the stream is being "
-                               "captured; run the same call once eagerly first")
+            return None
         buf = torch.zeros(max(n, 4096), dtype=torch.int32, device=dev)
         _ARRIVALS[key] = buf
     return buf
@@ -223,7 +220,8 @@ def paged_decode_attn_out(q, k_cache, v_cache, block_table, seq_lens, out, scale
         _contig_out(part_ml, "paged_decode_attn")
     pa = part_acc.data_ptr() if num_kv_splits > 1 else None
     pm = part_ml.data_ptr() if num_kv_splits > 1 else None
-    arrivals = _arrival_counters(dev, S * Hkv).data_ptr() if num_kv_splits > 1 else None
+    counters = _arrival_counters(dev, S * Hkv) if num_kv_splits > 1 else None
+    arrivals = counters.data_ptr() if counters is not None else None
     with torch.cuda.device(dev):
         rc = _lib.load().mi355_paged_decode_attn_fused(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
                                                        seq_lens.data_ptr(), out.data_ptr(), pa, pm, arrivals, S, Hq, Hkv, D, page,

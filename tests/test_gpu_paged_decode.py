@@ -276,7 +276,7 @@ def test_decode_one_launch_merge_under_graph_replay(dev):
         out.fill_(3.0)
         with torch.cuda.graph(graph, stream=side):
             launch.paged_decode_attn_out(q, kc, vc, bt, sl, out, 0.0, splits)
-        for rep in range(4):
+        for rep in range(4):  # (the capture above ran on a stream with counters: the one-launch form is what replays)
             out.fill_(float(rep))
             graph.replay()
             torch.cuda.synchronize()
