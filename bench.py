@@ -436,7 +436,7 @@ def wl_fa_issue_regloop(mode: str, waves_per_simd: int, data: str = "benchmark")
             opsd = (torch.randn(nbytes // 2, generator=g) * 0.35).half().view(torch.uint8).to(dev)  # scores of a few units
         workgroups, trips = 256 * waves_per_simd, 4000
         sink = torch.empty(workgroups * 256, dtype=torch.float32, device=dev)
-        code = {"mix": 0, "nomax": 1, "mfma": 2, "vector": 3, "spread": 4, "stepwise": 5}[mode]
+        code = {"mix": 0, "nomax": 1, "mfma": 2, "vector": 3, "spread": 4, "stepwise": 5, "mix16": 6, "mfma16": 7}[mode]
         flop = ctypes.c_double(0.0)
         lib = _lib.load()
 
@@ -455,7 +455,9 @@ def wl_fa_issue_regloop(mode: str, waves_per_simd: int, data: str = "benchmark")
                                              "nomax": "32 MFMA 32x32x16, 32 v_exp_f32, 16 cvt_pk, 16 dot2",
                                              "mfma": "32 MFMA 32x32x16", "vector": "32 v_exp_f32, 16 cvt_pk, 16 dot2 (flop counted as if the MFMAs ran)",
                                              "spread": "the whole mix, vector work spread over all 32 MFMAs",
-                                             "stepwise": "the whole mix, vector work behind the 16 score MFMAs, maximum chain behind the last 8 output MFMAs"}[mode]},
+                                             "stepwise": "the whole mix, vector work behind the 16 score MFMAs, maximum chain behind the last 8 output MFMAs",
+                                             "mix16": "64 MFMA 16x16x32 (the same flop), 32 v_exp_f32, 16 cvt_pk, 16 dot2",
+                                             "mfma16": "64 MFMA 16x16x32 (the same flop)"}[mode]},
         }
     return build
 
@@ -513,8 +515,8 @@ CALIBRATION = {  # not part of the path: run only when named with --workload
     "mfma_fp4walk_regloop_benchmark": wl_mfma_regloop("fp4walk", "benchmark"),
     "mfma_fp4x16walk_regloop_zeros": wl_mfma_regloop("fp4x16walk", "zeros"),
     "mfma_fp4x16walk_regloop_benchmark": wl_mfma_regloop("fp4x16walk", "benchmark"),
-    **{f"fa_issue_regloop_{m}_w{w}": wl_fa_issue_regloop(m, w) for m in ("mix", "nomax", "mfma", "vector", "spread", "stepwise") for w in (1, 2)},
-    **{f"fa_issue_regloop_{m}_w{w}_zeros": wl_fa_issue_regloop(m, w, "zeros") for m in ("mix", "mfma", "vector", "spread", "stepwise") for w in (1, 2)},
+    **{f"fa_issue_regloop_{m}_w{w}": wl_fa_issue_regloop(m, w) for m in ("mix", "nomax", "mfma", "vector", "spread", "stepwise", "mix16", "mfma16") for w in (1, 2)},
+    **{f"fa_issue_regloop_{m}_w{w}_zeros": wl_fa_issue_regloop(m, w, "zeros") for m in ("mix", "mfma", "vector", "spread", "stepwise", "mix16", "mfma16") for w in (1, 2)},
     "mfma_fp4_regloop_zeros": wl_mfma_regloop("fp4", "zeros"),
     "mfma_fp4_regloop_benchmark": wl_mfma_regloop("fp4", "benchmark"),
 }

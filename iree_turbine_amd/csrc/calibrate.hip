@@ -401,6 +401,79 @@ __global__ __launch_bounds__(CAL_WAVES * 64) __attribute__((amdgpu_waves_per_eu(
   sink[t] = acc;
 }
 
+// The same tile with v_mfma_f32_16x16x32_f16 in place of 32x32x16: the same flop, registers and operand bytes per tile --
+// 32 score MFMAs (4 key groups x 2 query groups x 4 steps over d; a K fragment serves both query groups) and 32 output
+// MFMAs (8 d groups x 2 query groups x 2 steps over the keys) -- with the vector work behind the score MFMAs (one
+// exponential each).  VECTOR = false: the MFMAs alone.  Whether the narrower MFMA is cheaper on benchmark-like data
+// here as it is in a GEMM's register structure is what this loop answers.
+template <bool VECTOR>
+__global__ __launch_bounds__(CAL_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void calibrate_fa_issue16_kernel(
+    const half8* __restrict__ operands, unsigned mask, float* __restrict__ sink, int trips) {
+  const unsigned t = threadIdx.x + blockIdx.x * blockDim.x;
+  half8 kf[4], vf[4], qf[8];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    kf[i] = operands[(t * 16 + i) & mask];
+    vf[i] = operands[(t * 16 + 4 + i) & mask];
+  }
+#pragma unroll
+  for (int i = 0; i < 8; i++) qf[i] = operands[(t * 16 + 8 + i) & mask];  // [query group][step over d]
+  floatx4 oacc[16], negm, sa[8], sb[8];
+  negm = floatx4{-1.f, -1.f, -1.f, -1.f};
+#pragma unroll
+  for (int i = 0; i < 16; i++) oacc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < 8; i++) sa[i] = sb[i] = floatx4{-2.f, -2.f, -2.f, -2.f};
+  float l_run = 0.f;
+  const half2v ones = {(half_t)1.f, (half_t)1.f};
+  auto tile = [&](floatx4* s, floatx4* s_next) {
+    half8 pf[4];  // [query group][key step]: 8 probabilities
+    float psum = 0.f;
+    asm volatile("" : "+v"(negm));
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < 32; i++) {
+      const int kg = i >> 3, ks = (i >> 1) & 3, qg = i & 1;  // a K fragment (kg, ks) feeds both query groups back to back
+      s_next[kg * 2 + qg] = mfma_16x16x32(kf[(kg + ks) & 3], qf[qg * 4 + ks], ks == 0 ? negm : s_next[kg * 2 + qg]);
+      if constexpr (VECTOR) {
+        // one exponential per score MFMA; every second MFMA packs a pair
+        const int e = i;  // score e of the tile's 32 per lane: accumulator e / 4, element e % 4
+        if (i & 1) {
+          const half2v pp = {(half_t)__builtin_amdgcn_exp2f(s[(e - 1) >> 2][(e - 1) & 3]), (half_t)__builtin_amdgcn_exp2f(s[e >> 2][e & 3])};
+          psum = __builtin_amdgcn_fdot2(pp, ones, psum, false);
+          pf[e >> 3][(e & 7) - 1] = pp[0];
+          pf[e >> 3][e & 7] = pp[1];
+          asm volatile("" : "+v"(psum));
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (!VECTOR) {
+      asm volatile("" ::"v"(s[0]), "v"(s[1]), "v"(s[2]), "v"(s[3]), "v"(s[4]), "v"(s[5]), "v"(s[6]), "v"(s[7]));
+#pragma unroll
+      for (int i = 0; i < 4; i++) pf[i] = qf[i];
+    }
+    l_run += psum;
+#pragma unroll
+    for (int i = 0; i < 32; i++) {
+      const int dg = i & 7, qg = (i >> 3) & 1, st = i >> 4;  // V^T fragment (dg, st); accumulators rotate
+      oacc[dg * 2 + qg] = mfma_16x16x32(vf[(dg + st) & 3], pf[qg * 2 + st], oacc[dg * 2 + qg]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+#pragma unroll 1
+  for (int it = 0; it < trips; it += 2) {
+    tile(sa, sb);
+    tile(sb, sa);
+  }
+  float acc = l_run;
+#pragma unroll
+  for (int i = 0; i < 16; i++)
+#pragma unroll
+    for (int r = 0; r < 4; r++) acc += oacc[i][r];
+  sink[t] = acc;
+}
+
 }  // namespace mi355
 
 using namespace mi355;
@@ -410,7 +483,7 @@ using namespace mi355;
 extern "C" int mi355_calibrate_fa_issue(int mode, const void* operands, int64_t operand_bytes, float* sink, int64_t sink_floats,
                                         int64_t workgroups, int64_t trips, double* flop_per_launch, void* stream) {
   if (!operands || !sink) return fail(-MI355_E_NULL, "calibrate_fa_issue: null pointer");
-  if (mode < 0 || mode > 5) return fail(-MI355_E_DTYPE, "calibrate_fa_issue: mode %d unknown (0 whole mix, 1 without the maximum chain, 2 MFMAs alone, 3 vector work alone, 4 vector work spread over all 32 MFMAs, 5 the order of mode 0 written step by step)", mode);
+  if (mode < 0 || mode > 7) return fail(-MI355_E_DTYPE, "calibrate_fa_issue: mode %d unknown (0 whole mix, 1 without the maximum chain, 2 MFMAs alone, 3 vector work alone, 4 vector work spread over all 32 MFMAs, 5 the order of mode 0 written step by step, 6 / 7 the tile on 16x16x32 MFMAs: whole mix / MFMAs alone)", mode);
   if (operand_bytes < 16 || (operand_bytes & (operand_bytes - 1)) || operand_bytes > (1ll << 30))
     return fail(-MI355_E_SHAPE, "calibrate_fa_issue: operand_bytes %lld must be a power of two in [16, 2^30]", (long long)operand_bytes);
   if (workgroups <= 0 || workgroups > 65535 || trips <= 0 || trips > (1 << 24))
@@ -429,7 +502,9 @@ extern "C" int mi355_calibrate_fa_issue(int mode, const void* operands, int64_t 
     case 2: hipLaunchKernelGGL(calibrate_fa_issue_kernel<2>, grid, block, 0, s, (const half8*)operands, mask, sink, (int)trips); break;
     case 3: hipLaunchKernelGGL(calibrate_fa_issue_kernel<3>, grid, block, 0, s, (const half8*)operands, mask, sink, (int)trips); break;
     case 4: hipLaunchKernelGGL(calibrate_fa_spread_kernel<1>, grid, block, 0, s, (const half8*)operands, mask, sink, (int)trips); break;
-    default: hipLaunchKernelGGL(calibrate_fa_spread_kernel<2>, grid, block, 0, s, (const half8*)operands, mask, sink, (int)trips); break;
+    case 5: hipLaunchKernelGGL(calibrate_fa_spread_kernel<2>, grid, block, 0, s, (const half8*)operands, mask, sink, (int)trips); break;
+    case 6: hipLaunchKernelGGL(calibrate_fa_issue16_kernel<true>, grid, block, 0, s, (const half8*)operands, mask, sink, (int)trips); break;
+    default: hipLaunchKernelGGL(calibrate_fa_issue16_kernel<false>, grid, block, 0, s, (const half8*)operands, mask, sink, (int)trips); break;
   }
   return check_launch("calibrate_fa_issue", grid, block, 0);
 }
