@@ -75,10 +75,11 @@ SETTLE_MS = 300.0  # untimed launches before the timed region, by device time
 
 
 def settle_clocks(fn, budget_ms: float = SETTLE_MS) -> int:
-    """Keeps launching `fn`, untimed, until about `budget_ms` of device time have passed; returns the launch count.
-    An idle GPU's power management takes tens of milliseconds of sustained work to reach the clocks it will hold, and
-    a kernel of 0.1-0.3 ms measured right after a handful of warm-up launches reads 10-20 % off its sustained rate
-    in either direction.  The W warm-up steps of the command line come first and are not replaced by this."""
+    """Keeps calling `fn` (one launch, or one replay of the captured steps), untimed, until about `budget_ms` of device
+    time have passed; returns the call count.  An idle GPU's power management takes tens of milliseconds of sustained
+    work to reach the clocks it will hold, and a kernel of 0.1-0.3 ms measured right after a handful of warm-up launches
+    reads 10-20 % off its sustained rate in either direction.  The W warm-up steps of the command line come first and
+    are not replaced by this."""
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     done, batch = 0, 4
     torch.cuda.synchronize()
@@ -103,11 +104,13 @@ def time_steps(fn, steps: int, warmup: int):
     host's per-call cost (a 15 us kernel behind a 40 us Python dispatch) are timed back to back on the
     device; the replay is bracketed by synchronize() for the wall clock and by one HIP event pair on the
     launch stream for the device time.  If capture fails the same K steps run eagerly, one event pair each.
+    The settling phase comes AFTER the capture, as untimed replays of the same graph that run right up to the timed
+    one: capturing and instantiating a graph leaves the GPU idle for long enough that its clocks fall back, and a
+    kernel that runs at a high clock (few stalls, power to spare) then reads up to 10 % low over a 5 ms timed region.
     """
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    settle_clocks(fn)
     graph = None
     try:
         graph = torch.cuda.CUDAGraph()
@@ -121,6 +124,7 @@ def time_steps(fn, steps: int, warmup: int):
         graph = None
         torch.cuda.synchronize()
     if graph is not None:
+        settle_clocks(graph.replay)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -130,6 +134,7 @@ def time_steps(fn, steps: int, warmup: int):
         torch.cuda.synchronize()
         wall_ms = (time.perf_counter() - t0) * 1e3 / steps
         return wall_ms, e0.elapsed_time(e1) / steps, "hip_graph"
+    settle_clocks(fn)
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()

@@ -681,6 +681,357 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 }
 
 
+// The pipelined form on v_mfma_f32_16x16x32 (variant "..._m16").  Same tiles, rings, loads, passes and barriers as
+// fa_fwd_d128_pipe; what changes is the MFMA shape and with it every fragment layout.  On benchmark-like data a
+// 16x16x32 MFMA costs the board less energy per flop than a 32x32x16 (register-only loops with this tile's structure:
+// 0.75 against 0.66 of the datasheet peak for the MFMAs alone, 0.60 against 0.57 with the softmax), and the prefill
+// kernel runs against the power limit.
+// A wave's 32 queries are two groups of 16 (qg), a 64-key tile four groups of 16 keys (kg), d = 128 four steps of 32 (ks),
+// eight groups of 16 (dg).  With q16 = lane & 15, g = lane >> 4:
+//   S^T(kg, qg) = K(kg) . Q(qg)^T:  A = K rows kg*16 + q16, d = 32 ks + 8 g .. + 7 (one 16-byte chunk from LDS, shared by
+//       both query groups); B = Q row qg*16 + q16, same d (registers); the lane receives keys kg*16 + 4 g + r, r < 4, of
+//       query qg*16 + q16: it owns one query per group and a quarter of the tile's keys.
+//   O^T(dg, qg) += V(dg)^T . P(qg)^T over two steps of 32 keys (key groups 2 st, 2 st + 1): the lane's eight probabilities
+//       (4 of either key group) are the B operand as they stand; A = V^T rows d = dg*16 + q16 for those same keys: two
+//       transpose reads, each a 4 x 16 block (keys 4 g .. 4 g + 3 of one key group, 16 consecutive d) per 16 lanes.
+// LDS: K chunk c of row r in slot c ^ (r & 15) as before; V chunk c of row r in slot c ^ 2 (r & 7): the 8 rows a half
+// wave's transpose read touches (32 bytes each) then fall on 8 distinct 32-byte bank groups.
+// SPREAD: the exponentials of a tile's second key step run behind the first key step's output MFMAs instead of behind
+// the score MFMAs (vector work behind 48 of the trip's 64 MFMAs instead of 32).  Measured on 2 x 32 x 4096: ahead with
+// eight waves (unmasked 475 against 484 us), behind with four (causal 268 against 263); each form is built the way it
+// runs faster.
+template <bool CAUSAL, bool BF, int NW, bool SPREAD>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void fa_fwd_d128_m16(
+    const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V, half_t* __restrict__ O, int BH,
+    int Sq, int Sk, float scale_log2e, int q_blocks, FaLayout lay) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  constexpr int BLOCK_M = NW * 32, NI = 16 / NW;
+  constexpr int TILE_B = FA_BLOCK_N * 256, VBUF = 2 * TILE_B;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int q16 = lane & 15, g = lane >> 4;
+
+  const int units = CAUSAL ? (q_blocks + 1) / 2 : q_blocks;
+  int bh, unit;
+  {
+    const int pid = blockIdx.x;
+    if (((BH / lay.group) & 7) == 0) {
+      const int xcd = pid & 7, loc = pid >> 3, per_kv = units * lay.group;
+      const int w = loc % per_kv;
+      bh = ((loc / per_kv) * 8 + xcd) * lay.group + w / units;
+      unit = w % units;
+    } else {
+      bh = pid / units;
+      unit = pid % units;
+    }
+  }
+  const int b_idx = bh / lay.H;
+  const int h_idx = bh - b_idx * lay.H, hk_idx = h_idx / lay.group;
+  const int causal_off = Sk - Sq;
+  const half_t* Qb = Q + b_idx * lay.q_b + h_idx * lay.q_h;
+  const half_t* Kb = K + b_idx * lay.k_b + hk_idx * lay.k_h;
+  const half_t* Vb = V + b_idx * lay.v_b + hk_idx * lay.v_h;
+  half_t* Ob = O + b_idx * lay.o_b + h_idx * lay.o_h;
+
+  // fragment read addresses, opaque (see fa_fwd_d128_pipe): K by step over d, V by d group
+  typedef const __attribute__((address_space(3))) half8* lds_half8_t;
+  unsigned k_frag[4], v_frag[8];
+  {
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+      k_frag[ks] = (unsigned)(uintptr_t)MI355_LDS(char, lds + q16 * 256 + (((ks * 4 + g) ^ q16) * 16));
+      asm volatile("" : "+v"(k_frag[ks]));
+    }
+    // lane i of a 16-lane group hands in row i / 4, halfs 4 (i % 4) .. + 3 of the 4 x 16 block
+    const int row = 4 * g + (q16 >> 2), rr = row & 7;
+    const int vb0 = VBUF + row * 256 + (rr << 5) + 16 * ((q16 & 3) >> 1) + 8 * (q16 & 1);
+#pragma unroll
+    for (int dg = 0; dg < 8; dg++) {
+      v_frag[dg] = (unsigned)(uintptr_t)MI355_LDS(char, lds + (vb0 ^ (dg << 5)));
+      asm volatile("" : "+v"(v_frag[dg]));
+    }
+  }
+
+  for (int pass = 0; pass < (CAUSAL ? 2 : 1); pass++) {
+  const int qb = CAUSAL ? (pass == 0 ? q_blocks - 1 - unit : unit) : unit;
+  if (CAUSAL && pass == 1 && 2 * unit == q_blocks - 1) break;
+  const int q0 = qb * BLOCK_M;
+  const int wq0 = q0 + wave * 32;
+
+  int k_end = Sk;
+  if (CAUSAL) {
+    int last_q = q0 + BLOCK_M - 1;
+    if (last_q > Sq - 1) last_q = Sq - 1;
+    int lim = last_q + causal_off + 1;
+    if (lim < k_end) k_end = lim;
+  }
+  const int n_tiles = k_end > 0 ? (k_end + FA_BLOCK_N - 1) / FA_BLOCK_N : 0;
+
+  // Q fragments [query group][step over d], scale . log2(e) folded in and rounded to the 16-bit format again
+  half8 qf[2][4];
+#pragma unroll
+  for (int qg = 0; qg < 2; qg++) {
+    const int q_row = wq0 + qg * 16 + q16;
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+      if (q_row < Sq) {
+        const half8 raw = *reinterpret_cast<const half8*>(Qb + (size_t)q_row * lay.q_r + ks * 32 + g * 8);
+#pragma unroll
+        for (int e = 0; e < 8; e++) qf[qg][ks][e] = cvt16<BF>(to_f32<BF>(raw[e]) * scale_log2e);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++) qf[qg][ks][e] = (half_t)0;
+      }
+    }
+  }
+
+  const int lrow = lane >> 4, lslot = lane & 15;
+  const int k_chunk = lslot ^ ((wave * 4 + lrow) & 15);
+  const int v_chunk = lslot ^ (2 * (((wave & 1) << 2) | lrow));
+  const unsigned k_rb = lay.k_r * 2, v_rb = lay.v_r * 2;
+  const unsigned k_voff = (wave * 4 + lrow) * k_rb + k_chunk * 16;
+  const unsigned v_voff = (wave * 4 + lrow) * v_rb + v_chunk * 16;
+  auto issue_kv = [&](const half_t* base, unsigned rb, unsigned voff, int tile, int lds_off) {
+    char* dst = lds + lds_off + wave * 1024;
+    const int row0 = tile * FA_BLOCK_N;
+    int rem = Sk - row0;
+    rem = rem > FA_BLOCK_N ? FA_BLOCK_N : rem;
+    const buffer_rsrc_t rs = make_buffer(reinterpret_cast<const char*>(base) + (size_t)row0 * rb, (unsigned)(rem - 1) * rb + 256u);
+#pragma unroll
+    for (int i = 0; i < NI; i++) buffer_load_lds_16B(rs, voff + (unsigned)(i * NW * 4) * rb, 0, dst + i * NW * 1024);
+  };
+
+  floatx4 oacc[8][2];  // [d group][query group]
+#pragma unroll
+  for (int dg = 0; dg < 8; dg++)
+#pragma unroll
+    for (int qg = 0; qg < 2; qg++) oacc[dg][qg] = floatx4{0.f, 0.f, 0.f, 0.f};
+  // the negated running maximum of the lane's query in either group, four equal values: the addend of every score chain
+  floatx4 negm[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
+  float l_run[2] = {0.f, 0.f};
+  float grow_thr[2] = {-INFINITY, -INFINITY};
+  constexpr float kRescaleThreshold = 8.f;
+
+  auto wave_active = [&](int tile) { return !CAUSAL || (tile * FA_BLOCK_N <= wq0 + 31 + causal_off); };
+  auto kread = [&](int f, int koff) {  // K fragment f = kg * 4 + ks of the slot at koff
+    return *(lds_half8_t)(uintptr_t)(k_frag[f & 3] + (unsigned)(koff + (f >> 2) * 4096));
+  };
+  // S^T of one tile, no softmax beside it (a pass's first tile)
+  auto scores = [&](int koff, floatx4 (*s)[2]) {
+#pragma unroll
+    for (int f = 0; f < 16; f++) {
+      const int kg = f >> 2, ks = f & 3;
+      const half8 kf = kread(f, koff);
+#pragma unroll
+      for (int qg = 0; qg < 2; qg++) s[kg][qg] = mfma16_16x16x32<BF>(kf, qf[qg][ks], ks == 0 ? negm[qg] : s[kg][qg]);
+    }
+  };
+
+  auto softmax_pv = [&](int tile, auto voff_tag, floatx4 (*s)[2], int koff_next, floatx4 (*s_next)[2]) {
+    constexpr int VOFF = decltype(voff_tag)::value;
+    {
+      const int key0 = tile * FA_BLOCK_N;
+      const bool need_mask = (CAUSAL && (key0 + FA_BLOCK_N - 1 > wq0 + causal_off)) || (key0 + FA_BLOCK_N > Sk);
+      if (need_mask) {
+#pragma unroll
+        for (int qg = 0; qg < 2; qg++) {
+          const int q_row = wq0 + qg * 16 + q16;
+          const int lim = CAUSAL ? (q_row + causal_off < Sk - 1 ? q_row + causal_off : Sk - 1) : Sk - 1;  // last visible key
+          const int rel = lim - key0 - 4 * g;
+#pragma unroll
+          for (int kg = 0; kg < 4; kg++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+              const unsigned hide = (unsigned)((rel - (16 * kg + r)) >> 31);
+              const float sv = s[kg][qg][r];
+              s[kg][qg][r] = __builtin_bit_cast(float, (hide & 0xFF800000u) | (~hide & __builtin_bit_cast(unsigned, sv)));
+            }
+        }
+      }
+    }
+    float mx[2];
+#pragma unroll
+    for (int qg = 0; qg < 2; qg++) {
+      mx[qg] = s[0][qg][0];
+#pragma unroll
+      for (int kg = 0; kg < 4; kg++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) mx[qg] = fmaxf(mx[qg], s[kg][qg][r]);
+    }
+    if (__builtin_amdgcn_ballot_w64(mx[0] > grow_thr[0] || mx[1] > grow_thr[1]) != 0) {
+      // rare: some query's scores outgrew its maximum (or it saw its first key).  A query's keys are spread over the
+      // four lanes q16 + 16 g; they take the same decision.
+#pragma unroll
+      for (int qg = 0; qg < 2; qg++) {
+        float mxx = fmaxf(mx[qg], __shfl_xor(mx[qg], 16));
+        mxx = fmaxf(mxx, __shfl_xor(mxx, 32));
+        if (mxx > grow_thr[qg]) {
+          const bool fresh = grow_thr[qg] == -INFINITY;
+          const float delta = fresh ? mxx : fmaxf(mxx, 0.f);  // (mxx > -inf here)
+          const float alpha = fresh ? 1.f : __builtin_amdgcn_exp2f(-delta);
+          grow_thr[qg] = kRescaleThreshold;
+          l_run[qg] *= alpha;
+#pragma unroll
+          for (int dg = 0; dg < 8; dg++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) oacc[dg][qg][r] *= alpha;
+#pragma unroll
+          for (int kg = 0; kg < 4; kg++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) s[kg][qg][r] -= delta;
+#pragma unroll
+          for (int r = 0; r < 4; r++) negm[qg][r] -= delta;
+        }
+      }
+    }
+    // Scores of the next tile and the softmax of this one, step by step.  Step i = MFMA (kg, ks, qg) = (i / 8, (i / 2) % 4,
+    // i % 2) of the next tile -- a K fragment serves both query groups back to back and is requested three fragments
+    // ahead -- and one exponential of this tile, taken in the order the output MFMAs want the probabilities: key step,
+    // query group, key group of the pair, r.  Every second step packs a pair; its dot2 (the row sum of what the second
+    // contraction multiplies) runs one pair behind.  The empty statements tie the vector work to its step.
+    half8 pf[2][2];  // [query group][key step]
+    float psum[2] = {0.f, 0.f};
+    half2v pp_prev = {(half_t)0, (half_t)0};
+    // exponential e of the tile (0..31), in the order the output MFMAs want the probabilities: key step e / 16, query group
+    // (e / 8) % 2, key group of the pair (e / 4) % 2, r = e % 4.  Every second one packs a pair; the pair's dot2 (the row
+    // sum of what the second contraction multiplies) runs one pair behind.  The empty statements tie the work to its step.
+    float e_even = 0.f;
+    auto expo = [&](int e) {
+      const int st = e >> 4, eq = (e >> 3) & 1, ekg = 2 * st + ((e >> 2) & 1), r = e & 3;
+      const float ev = __builtin_amdgcn_exp2f(s[ekg][eq][r]);
+      if (e & 1) {
+        if (e > 1) psum[((e - 2) >> 3) & 1] = dot2_ones<BF>(pp_prev, psum[((e - 2) >> 3) & 1]);
+        half2v pp = cvt16x2<BF>(e_even, ev);
+        asm volatile("" : "+v"(pp), "+v"(psum[0]), "+v"(psum[1]));
+        pf[eq][st][((e >> 2) & 1) * 4 + r - 1] = pp[0];
+        pf[eq][st][((e >> 2) & 1) * 4 + r] = pp[1];
+        pp_prev = pp;
+      } else {
+        e_even = ev;
+        asm volatile("" : "+v"(e_even));
+      }
+    };
+    // Scores of the next tile, step by step: step i = MFMA (kg, ks, qg) = (i / 8, (i / 2) % 4, i % 2) -- a K fragment serves
+    // both query groups back to back and is requested three fragments ahead -- with the exponentials of this tile's
+    // FIRST key step behind every second MFMA; those of the second key step run behind the first key step's output
+    // MFMAs below, so that the vector work is spread over 48 of the trip's 64 MFMAs.
+    __builtin_amdgcn_sched_barrier(0);
+    {
+      half8 kf[4];
+      kf[0] = kread(0, koff_next);
+      kf[1] = kread(1, koff_next);
+      kf[2] = kread(2, koff_next);
+#pragma unroll
+      for (int i = 0; i < 32; i++) {
+        const int f = i >> 1, kg = f >> 2, ks = f & 3, qg = i & 1;
+        if (qg == 0 && f + 3 < 16) kf[(f + 3) & 3] = kread(f + 3, koff_next);
+        s_next[kg][qg] = mfma16_16x16x32<BF>(kf[f & 3], qf[qg][ks], ks == 0 ? negm[qg] : s_next[kg][qg]);
+        if (SPREAD) {
+          if (i & 1) expo(i >> 1);
+        } else {
+          expo(i);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    // O^T += V^T P^T: step f = (key step, d group) = (f / 8, f % 8), two MFMAs (one per query group) on one V^T fragment
+    // (two transpose reads, in assembly with their waits, see fa_fwd_d128_pipe), requested two fragments ahead.
+    half4 vlo[3], vhi[3];
+    auto vr = [&](auto ftag) {  // fragment f = st * 8 + dg
+      constexpr int f = decltype(ftag)::value;
+      constexpr int off = VOFF + (f >> 3) * 8192;  // key groups 2 st and 2 st + 1: 16 rows of 256 bytes apart
+      half4 &lo = vlo[f % 3], &hi = vhi[f % 3];
+      const unsigned addr = v_frag[f & 7];
+      asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4"
+                   : "=&v"(lo), "=&v"(hi)
+                   : "v"(addr), "n"(off), "n"(off + 4096));
+    };
+    vr(std::integral_constant<int, 0>{});
+    vr(std::integral_constant<int, 1>{});
+    static_for<0, 16>([&](auto ftag) {
+      constexpr int f = decltype(ftag)::value;
+      constexpr int st = f >> 3, dg = f & 7;
+      if constexpr (f + 2 < 16) vr(std::integral_constant<int, f + 2>{});
+      half4 &lo = vlo[f % 3], &hi = vhi[f % 3];
+      if constexpr (f + 2 < 16)
+        asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(lo), "+v"(hi));
+      else if constexpr (f + 1 < 16)
+        asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(lo), "+v"(hi));
+      else
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lo), "+v"(hi));
+      const half8 vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      oacc[dg][0] = mfma16_16x16x32<BF>(vf, pf[0][st], oacc[dg][0]);
+      if constexpr (SPREAD && f < 8) expo(16 + 2 * f);
+      __builtin_amdgcn_sched_barrier(0);
+      oacc[dg][1] = mfma16_16x16x32<BF>(vf, pf[1][st], oacc[dg][1]);
+      if constexpr (SPREAD && f < 8) expo(16 + 2 * f + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (f == 7 || (!SPREAD && f == 0)) {  // the last pair's dot2 (it belongs to query group 1)
+        if (SPREAD || f == 0) {
+          psum[1] = dot2_ones<BF>(pp_prev, psum[1]);
+          l_run[0] += psum[0];
+          l_run[1] += psum[1];
+        }
+      }
+    });
+  };
+
+  floatx4 sa[4][2], sb[4][2];  // scores [key group][query group], two tiles
+  if (n_tiles > 0) {
+    issue_kv(Kb, k_rb, k_voff, 0, 0);
+    issue_kv(Vb, v_rb, v_voff, 0, VBUF);
+    if (n_tiles > 1) issue_kv(Kb, k_rb, k_voff, 1, TILE_B);
+    wait_vmcnt0();
+    __syncthreads();
+    if (wave_active(0)) scores(0, sa);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+  }
+  auto trip = [&](auto par_tag, int j, floatx4 (*s_cur)[2], floatx4 (*s_next)[2]) {
+    constexpr int PAR = decltype(par_tag)::value;
+    constexpr int K_CUR = PAR * TILE_B, K_NEXT = (1 - PAR) * TILE_B, V_CUR = VBUF + PAR * TILE_B, V_NEXT = VBUF + (1 - PAR) * TILE_B;
+    if (j + 2 < n_tiles) issue_kv(Kb, k_rb, k_voff, j + 2, K_CUR);
+    if (j + 1 < n_tiles) issue_kv(Vb, v_rb, v_voff, j + 1, V_NEXT);
+    if (wave_active(j)) softmax_pv(j, std::integral_constant<int, V_CUR - VBUF>{}, s_cur, K_NEXT, s_next);
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+  };
+  for (int j = 0; j < n_tiles; j += 2) {
+    trip(std::integral_constant<int, 0>{}, j, sa, sb);
+    if (j + 1 < n_tiles) trip(std::integral_constant<int, 1>{}, j + 1, sb, sa);
+  }
+
+  {
+    // Output through LDS (the rings are idle: the last trip ended with a barrier): each wave assembles its 32 rows x 256
+    // bytes in a private region (chunk c of row r in slot c ^ (r & 15)) from 8-byte pieces -- the lane holds d = 16 dg +
+    // 4 g .. + 3 of its query in either group -- and stores whole rows, 16 bytes per lane.
+    char* ep = lds + wave * 8192;
+    const int el = CAUSAL ? opaque_lane_id() : lane;  // (see fa_fwd_d128_pipe)
+    const int e16 = el & 15, eg = el >> 4;
+#pragma unroll
+    for (int qg = 0; qg < 2; qg++) {
+      float l_tot = l_run[qg] + __shfl_xor(l_run[qg], 16);
+      l_tot += __shfl_xor(l_tot, 32);
+      const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+#pragma unroll
+      for (int dg = 0; dg < 8; dg++) {
+        const half4 v = {cvt16<BF>(oacc[dg][qg][0] * inv), cvt16<BF>(oacc[dg][qg][1] * inv), cvt16<BF>(oacc[dg][qg][2] * inv),
+                         cvt16<BF>(oacc[dg][qg][3] * inv)};
+        *reinterpret_cast<half4*>(ep + (qg * 16 + e16) * 256 + (((dg * 2 + (eg >> 1)) ^ e16) * 16) + 8 * (eg & 1)) = v;
+      }
+    }
+    const int er = el >> 4, ec = el & 15;
+#pragma unroll
+    for (int it = 0; it < 8; it++) {
+      const int row = it * 4 + er;
+      const half8 v = *reinterpret_cast<const half8*>(ep + row * 256 + ((ec ^ (row & 15)) * 16));
+      if (wq0 + row < Sq) *reinterpret_cast<half8*>(Ob + (size_t)(wq0 + row) * lay.o_r + ec * 8) = v;
+    }
+    if (CAUSAL) __syncthreads();  // the next pass loads K / V tiles over these regions
+  }
+  }  // pass
+}
+
 // Persistent form of fa_fwd_d128_pipe ("walk"): one workgroup per CU slot runs its passes (a pass = one block of
 // NW * 32 queries of one head against its keys) one after the other -- units dealt round-robin (unit = workgroup +
 // i * grid), a causal unit being a pair of blocks as above -- and overlaps what a pass costs beside its key tiles:
@@ -1065,9 +1416,10 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 }
 
 static const char* kFaVariants[] = {"d128_bm128_bn64_w4_pipelined", "d128_bm128_bn64_w4", "d128_bm256_bn64_w8_pipelined",
-                                    "d128_bm256_bn64_w8_walk", "d128_bm128_bn64_w4_walk"};
-int fa_variant_count() { return 5; }
-const char* fa_variant_name(int i) { return (i >= 0 && i < 5) ? kFaVariants[i] : nullptr; }
+                                    "d128_bm256_bn64_w8_walk", "d128_bm128_bn64_w4_walk", "d128_bm128_bn64_w4_m16",
+                                    "d128_bm256_bn64_w8_m16"};
+int fa_variant_count() { return 7; }
+const char* fa_variant_name(int i) { return (i >= 0 && i < 7) ? kFaVariants[i] : nullptr; }
 
 }  // namespace mi355
 
@@ -1099,7 +1451,7 @@ static int fa_launch(const void* q, const void* k, const void* v, void* o, int64
     return fail(-MI355_E_SHAPE, "%s: %lld query heads over %lld key/value heads", who, (long long)H, (long long)Hkv);
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o))
     return fail(-MI355_E_ALIGN, "%s: q, k, v, o must be 16-byte aligned", who);
-  if (variant > 4) return fail(-MI355_E_DTYPE, "%s: variant %d out of range", who, variant);
+  if (variant > 6) return fail(-MI355_E_DTYPE, "%s: variant %d out of range", who, variant);
   if (!(scale > 0.f) || !isfinite(scale)) return fail(-MI355_E_SHAPE, "%s: scale must be positive and finite", who);
   const int BH = (int)(B * H);
   const int q_blocks = (int)((Sq + FA_BLOCK_M - 1) / FA_BLOCK_M);
@@ -1113,7 +1465,30 @@ static int fa_launch(const void* q, const void* k, const void* v, void* o, int64
   const float scale_log2e = scale * 1.4426950408889634f;
   // Without a mask, and with enough 256-query blocks for every CU, the 8-wave form is ahead (2 x 32 x 4096: 503 against
   // 514 us); with the causal mask the two are level and the 4-wave form has the finer-grained tail.
-  if (variant < 0 && !is_causal && (int64_t)BH * ((Sq + 255) / 256) >= 512) variant = 2;
+  // The automatic choice is the 16x16x32 form: eight waves (with the exponentials spread into the output MFMAs) for
+  // unmasked shapes with enough 256-query blocks for every CU (2 x 32 x 4096: 475 us against 483 for the 32x32x16 form
+  // on the same box), four waves otherwise (causal 2 x 32 x 4096: 263 against 269; the finer-grained tail).
+  if (variant < 0) variant = (!is_causal && (int64_t)BH * ((Sq + 255) / 256) >= 512) ? 6 : 5;
+  if (variant == 5 || variant == 6) {
+    // the pipelined forms on 16x16x32 MFMAs, 4 waves (128-query blocks) or 8 (256)
+    const bool w8 = variant == 6;
+    const int bm = w8 ? 256 : 128;
+    const int qbm = (int)((Sq + bm - 1) / bm);
+    const void* kern = w8 ? (is_causal ? (const void*)fa_fwd_d128_m16<true, BF, 8, true> : (const void*)fa_fwd_d128_m16<false, BF, 8, true>)
+                          : (is_causal ? (const void*)fa_fwd_d128_m16<true, BF, 4, false> : (const void*)fa_fwd_d128_m16<false, BF, 4, false>);
+    static std::atomic<uint64_t> okm[4] = {};
+    if (int rc = allow_lds(kern, lds_bytes, okm[(w8 ? 2 : 0) + (is_causal ? 1 : 0)], "fa_fwd_d128_m16")) return rc;
+    dim3 grid(BH * (is_causal ? (qbm + 1) / 2 : qbm)), block(w8 ? 512 : 256);
+    const half_t *qp = (const half_t*)q, *kp = (const half_t*)k, *vp = (const half_t*)v;
+    half_t* op = (half_t*)o;
+    int bh_i = BH, sq_i = (int)Sq, sk_i = (int)Sk, qb_i = qbm;
+    FaLayout lay_v = lay;
+    float sc = scale_log2e;
+    void* args[] = {&qp, &kp, &vp, &op, &bh_i, &sq_i, &sk_i, &sc, &qb_i, &lay_v};
+    hipError_t e = hipLaunchKernel(kern, grid, block, args, lds_bytes, reinterpret_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail((int)e, "%s: launch of fa_fwd_d128_m16 failed: %s", who, hipGetErrorString(e));
+    return check_launch("fa_fwd_d128_m16", grid, block, lds_bytes);
+  }
   if (variant == 3 || variant == 4) {
     // the persistent forms: every pass needs two key tiles, and the masked form a square mask (no pass without keys)
     const bool w8 = variant == 3;

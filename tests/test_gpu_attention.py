@@ -69,6 +69,36 @@ def test_attention_eight_wave_form(dev, Sq, Sk, causal):
 
 
 @pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("Sq,Sk", [(1, 1), (17, 17), (64, 64), (100, 100), (255, 255), (257, 257), (300, 777), (1024, 1024), (700, 100),
+                                   (96, 320), (2048, 2048)])
+def test_attention_16x16x32_forms(dev, Sq, Sk, causal):
+    """The forms on 16x16x32 MFMAs (the automatic choice; a lane owns one query of either 16-query group and a quarter of
+    a tile's keys, so masks, row sums and the rare rescale are laid out differently from the 32x32x16 forms): ragged and
+    cross lengths, lengths around the block sizes, Sq > Sk, several tiles -- against the oracle; the 4- and the 8-wave
+    form agree bit for bit (same per-wave arithmetic, only the exponentials sit at other places of the trip), and
+    both agree with the 32x32x16 form to the rounding of the output."""
+    import iree_turbine_amd as ita
+    from oracle import attention as oa, inputs
+
+    announce(f"flash_attn_fwd 16x16x32 forms Sq={Sq} Sk={Sk} causal={causal}")
+    names = ita._lib.variants("flash_attn_fwd")
+    q, k, v = inputs.attention_inputs(2, 3, Sq, 128, seed=16, Sk=Sk)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    o4, o8, o32 = torch.empty_like(qd), torch.empty_like(qd), torch.empty_like(qd)
+    ita.launch.flash_attn_fwd_out(qd, kd, vd, o4, causal, 0.0, names.index("d128_bm128_bn64_w4_m16"))
+    ita.launch.flash_attn_fwd_out(qd, kd, vd, o8, causal, 0.0, names.index("d128_bm256_bn64_w8_m16"))
+    ita.launch.flash_attn_fwd_out(qd, kd, vd, o32, causal, 0.0, 0)
+    assert torch.equal(o4, o8)
+    torch.testing.assert_close(o4.float(), o32.float(), rtol=RTOL, atol=ATOL)
+    assert torch.equal(o4, torch.ops.mi355.flash_attn_fwd(qd, kd, vd, causal, 0.0))  # what the op runs at these sizes
+    got = o4.float().cpu()
+    if causal and Sq > Sk:
+        assert torch.equal(got[:, :, :Sq - Sk], torch.zeros_like(got[:, :, :Sq - Sk]))  # queries that see no key
+        got, q = got[:, :, Sq - Sk:], q[:, :, Sq - Sk:]
+    torch.testing.assert_close(got, oa.sdpa_ref(q, k, v, is_causal=causal), rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("form", ["d128_bm256_bn64_w8_walk", "d128_bm128_bn64_w4_walk"])
 @pytest.mark.parametrize("B,H,Sq,Sk", [(2, 3, 128, 128), (1, 2, 255, 255), (1, 2, 257, 257), (2, 3, 320, 320), (1, 5, 777, 777),
                                        (3, 40, 1024, 1024), (2, 3, 300, 777), (1, 2, 700, 128), (1, 9, 192, 4200)])

@@ -437,8 +437,13 @@ def test_paged_prefill_matches_decode_and_dense_attention(dev):
     table = torch.arange(S * L // 16, dtype=torch.int32, device=dev).reshape(S, L // 16)
     lens = torch.full((S,), L, dtype=torch.int32, device=dev)
     paged = torch.ops.mi355.paged_prefill_attn(q, kcache, vcache, table, lens, 0.0)
-    dense = torch.ops.mi355.flash_attn_fwd(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), True, 0.0).transpose(1, 2)
-    assert torch.equal(paged, dense.contiguous())  # same kernel, same tiles, pages in order: bit-identical
+    from iree_turbine_amd import launch
+    qt = q.transpose(1, 2)
+    dense = torch.empty_like(qt)  # laid out like q
+    launch.flash_attn_fwd_out(qt, k.transpose(1, 2), v.transpose(1, 2), dense, True, 0.0, 0)  # the 32x32x16 form the paged kernel is
+    assert torch.equal(paged, dense.transpose(1, 2).contiguous())  # same kernel, same tiles, pages in order: bit-identical
+    auto = torch.ops.mi355.flash_attn_fwd(qt, k.transpose(1, 2), v.transpose(1, 2), True, 0.0).transpose(1, 2)
+    torch.testing.assert_close(paged.float(), auto.float(), rtol=RTOL, atol=ATOL)  # the op's own choice (16x16x32 MFMAs)
 
 
 def test_paged_prefill_guards(dev):
