@@ -696,6 +696,9 @@ def main() -> int:
     ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS_ALL))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-others", action="store_true", help="measure only --workload")
+    ap.add_argument("--library", default=None,
+                    help="measure another build of the kernel library (python -m iree_turbine_amd.build -D... --out PATH); "
+                         "a build with ablation switches computes wrong results and is named in the record")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); --gpus must be 1", file=sys.stderr)
@@ -704,7 +707,16 @@ def main() -> int:
         print("bench.py: no GPU visible; the kernels have no CPU fallback", file=sys.stderr)
         return 3
 
+    if args.library:
+        from pathlib import Path
+
+        from iree_turbine_amd import _lib as _kernel_lib
+
+        _kernel_lib.LIB_PATH = Path(args.library).resolve()
     import iree_turbine_amd  # noqa: F401  (registers torch.ops.mi355.*; raises if the library is missing)
+    from iree_turbine_amd import _lib as _kernel_lib
+
+    build_flags = _kernel_lib.build_flags()
 
     dev = torch.device("cuda:0")
     head = measure(args.workload, dev, args.steps, args.warmup, with_cpu=not args.no_cpu)
@@ -749,6 +761,8 @@ def main() -> int:
                  "torch_threads": torch.get_num_threads(), "gpu": torch.cuda.get_device_name(0)},
         "others": others,
     }
+    if build_flags:  # not the product library: a timing-only build, its results are wrong on purpose
+        line["library_ablations"] = build_flags
     print(json.dumps(line))
     return 0
 

@@ -53,6 +53,10 @@ extern "C" {
 
 int mi355_abi_version(void);
 const char* mi355_last_error(void);
+/* "" for the product build.  A library built with timing-only ablation switches (-DMI355_ABLATE_..., see
+ * csrc/common.hpp) names them here: such a build computes wrong results on purpose and exists to measure what a part
+ * of a kernel costs.  No counterpart in the reference. */
+const char* mi355_build_flags(void);
 
 /* Number of kernel variants of a family and the name of variant i
  * (family: "gemm_f16_nt" -- shared by the bf16 entry --, "flash_attn_fwd", "paged_decode",

@@ -27,6 +27,7 @@ _lib = None
 _PROTOS = {
     "mi355_abi_version": (c_int, []),
     "mi355_last_error": (c_char_p, []),
+    "mi355_build_flags": (c_char_p, []),
     "mi355_variant_count": (c_int, [c_char_p]),
     "mi355_variant_name": (c_char_p, [c_char_p, c_int]),
     "mi355_gemm_f16_nt": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_void_p]),
@@ -132,6 +133,11 @@ def load():
             raise KernelLibraryError(f"ABI version mismatch: library reports {lib.mi355_abi_version()}, binding expects 1")
         _lib = lib
     return _lib
+
+
+def build_flags() -> str:
+    """The timing-only ablation switches the loaded library was built with ("" for the product build)."""
+    return (load().mi355_build_flags() or b"").decode().strip()
 
 
 def last_error() -> str:

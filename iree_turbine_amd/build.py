@@ -95,16 +95,22 @@ def _run(cmd: list[str]) -> None:
             print(line, file=sys.stderr)
 
 
-def build_library(verbose: bool = True, save_temps: bool = False) -> Path:
-    """Compiles every kernel source and links the shared library.  Always recompiles."""
+def build_library(verbose: bool = True, save_temps: bool = False, defines: tuple[str, ...] = (), out: Path | None = None) -> Path:
+    """Compiles every kernel source and links the shared library.  Always recompiles.
+
+    `defines` (e.g. ("MI355_ABLATE_NO_LOADS",), the timing-only switches of csrc/common.hpp) and `out` build a second
+    library beside the product one, with its own object directory; the product library is the call without them."""
     hipcc = _hipcc()
-    obj_dir = CSRC / "build"
-    obj_dir.mkdir(exist_ok=True)
+    lib_path = Path(out).resolve() if out is not None else LIB_PATH
+    if defines and lib_path == LIB_PATH:
+        raise ValueError("a build with ablation switches needs its own --out path: it must not replace the product library")
+    obj_dir = CSRC / "build" if lib_path == LIB_PATH else lib_path.parent / (lib_path.stem + "_obj")
+    obj_dir.mkdir(parents=True, exist_ok=True)
     objs = [obj_dir / (Path(s).stem + ".o") for s in SOURCES]
 
     def compile_one(pair):
         src, obj = pair
-        cmd = [hipcc, *HIPCC_FLAGS, _USAGE_FLAG, "-c", str(CSRC / src), "-o", str(obj)]
+        cmd = [hipcc, *HIPCC_FLAGS, *(f"-D{d}" for d in defines), _USAGE_FLAG, "-c", str(CSRC / src), "-o", str(obj)]
         if save_temps:
             cmd += ["-save-temps=obj"]
         _run(cmd)
@@ -112,11 +118,43 @@ def build_library(verbose: bool = True, save_temps: bool = False) -> Path:
 
     with ThreadPoolExecutor(max_workers=min(len(SOURCES), os.cpu_count() or 4)) as pool:
         list(pool.map(compile_one, zip(SOURCES, objs)))
-    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(LIB_PATH), *map(str, objs)])
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(lib_path), *map(str, objs)])
     if verbose:
-        print(f"built {LIB_PATH} ({LIB_PATH.stat().st_size} bytes)")
-    return LIB_PATH
+        print(f"built {lib_path} ({lib_path.stat().st_size} bytes)" + (f" with {' '.join(defines)}" if defines else ""))
+    return lib_path
+
+
+PROBES = ["lds_read_patterns.hip", "load_rate.hip", "mfma_load_bubble.hip"]
+
+
+def build_probes(verbose: bool = True) -> list[Path]:
+    """Compiles the stand-alone measurement programs of csrc/probes/ (no Python, no library: each prints a table)."""
+    hipcc = _hipcc()
+    out_dir = CSRC / "probes" / "bin"
+    out_dir.mkdir(exist_ok=True)
+
+    def one(src):
+        exe = out_dir / Path(src).stem
+        _run([hipcc, *[f for f in HIPCC_FLAGS if f != "-fPIC"], str(CSRC / "probes" / src), "-o", str(exe)])
+        return exe
+
+    with ThreadPoolExecutor(max_workers=len(PROBES)) as pool:
+        exes = list(pool.map(one, PROBES))
+    if verbose:
+        print("built " + ", ".join(str(e) for e in exes))
+    return exes
 
 
 if __name__ == "__main__":
-    build_library(save_temps="--save-temps" in sys.argv)
+    import argparse
+
+    ap = argparse.ArgumentParser(description=__doc__)
+    ap.add_argument("--save-temps", action="store_true")
+    ap.add_argument("-D", dest="defines", action="append", default=[], metavar="MI355_ABLATE_...",
+                    help="a timing-only ablation switch (csrc/common.hpp); needs --out")
+    ap.add_argument("--out", default=None, help="path of the library to write (default: the product library in csrc/)")
+    ap.add_argument("--probes", action="store_true", help="also build the measurement programs of csrc/probes/")
+    a = ap.parse_args()
+    if a.probes:
+        build_probes()
+    build_library(save_temps=a.save_temps, defines=tuple(a.defines), out=a.out)

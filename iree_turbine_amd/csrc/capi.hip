@@ -47,6 +47,39 @@ const char* mxfp6_variant_name(int i);
 using namespace mi355;
 
 extern "C" int mi355_abi_version(void) { return MI355_ABI_VERSION; }
+
+// The timing-only ablations this library was built with (common.hpp), "" for the product build.
+extern "C" const char* mi355_build_flags(void) {
+  return ""
+#if defined(MI355_ABLATE_NO_LOADS)
+         " NO_LOADS"
+#endif
+#if defined(MI355_ABLATE_L1_LOADS)
+         " L1_LOADS"
+#endif
+#if defined(MI355_ABLATE_NO_LOAD_WAITS)
+         " NO_LOAD_WAITS"
+#endif
+#if defined(MI355_ABLATE_NO_BARRIERS)
+         " NO_BARRIERS"
+#endif
+#if defined(MI355_ABLATE_NO_SCALE_READS)
+         " NO_SCALE_READS"
+#endif
+#if defined(MI355_ABLATE_NO_SCALE_LOADS)
+         " NO_SCALE_LOADS"
+#endif
+#if defined(MI355_ABLATE_NO_EXP)
+         " NO_EXP"
+#endif
+#if defined(MI355_ABLATE_NO_K_READS)
+         " NO_K_READS"
+#endif
+#if defined(MI355_ABLATE_NO_V_READS)
+         " NO_V_READS"
+#endif
+      ;
+}
 extern "C" const char* mi355_last_error(void) { return g_error; }
 
 extern "C" int mi355_variant_count(const char* family) {

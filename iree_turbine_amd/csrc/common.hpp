@@ -52,6 +52,28 @@ __device__ __forceinline__ int opaque_lane_id() {
   return l;
 }
 
+// Timing-only ablations of the streamed GEMM and prefill kernels, for measuring what a part of a kernel costs: a
+// library built with one of these (python -m iree_turbine_amd.build -DMI355_ABLATE_... --out other.so) computes WRONG
+// results by construction and says so through mi355_build_flags().  The default build defines none of them.
+//   MI355_ABLATE_NO_LOADS       the K loop issues no global -> LDS loads (LDS keeps whatever it held)
+//   MI355_ABLATE_L1_LOADS       every load of the K loop reads the same few KiB (always an L1 hit)
+//   MI355_ABLATE_NO_LOAD_WAITS  the K loop never waits for a load
+//   MI355_ABLATE_NO_BARRIERS    the K loop has no workgroup barriers
+//   MI355_ABLATE_NO_SCALE_READS / MI355_ABLATE_NO_SCALE_LOADS   (block-scaled GEMMs) no LDS reads / no loads of scales
+//   MI355_ABLATE_NO_EXP / MI355_ABLATE_NO_K_READS / MI355_ABLATE_NO_V_READS   (prefill) no exponentials / fragment reads
+#if defined(MI355_ABLATE_NO_BARRIERS)
+#define MI355_KLOOP_BARRIER() do {} while (0)
+#else
+#define MI355_KLOOP_BARRIER() __builtin_amdgcn_s_barrier()
+#endif
+#if defined(MI355_ABLATE_NO_LOAD_WAITS)
+#define MI355_KLOOP_VMCNT(n) 63
+#define MI355_KLOOP_VMCNT_STR(n) "63"
+#else
+#define MI355_KLOOP_VMCNT(n) (n)
+#define MI355_KLOOP_VMCNT_STR(n) #n
+#endif
+
 __device__ __forceinline__ void wait_vmcnt0() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // One 16-byte global store per lane as ONE instruction, written out: kernels whose later `s_waitcnt vmcnt(n)` counts

@@ -798,7 +798,11 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     rem = rem > FA_BLOCK_N ? FA_BLOCK_N : rem;
     const buffer_rsrc_t rs = make_buffer(reinterpret_cast<const char*>(base) + (size_t)row0 * rb, (unsigned)(rem - 1) * rb + 256u);
 #pragma unroll
-    for (int i = 0; i < NI; i++) buffer_load_lds_16B(rs, voff + (unsigned)(i * NW * 4) * rb, 0, dst + i * NW * 1024);
+    for (int i = 0; i < NI; i++) {
+#if !defined(MI355_ABLATE_NO_LOADS)
+      buffer_load_lds_16B(rs, voff + (unsigned)(i * NW * 4) * rb, 0, dst + i * NW * 1024);
+#endif
+    }
   };
 
   floatx4 oacc[8][2];  // [d group][query group]
@@ -814,7 +818,13 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 
   auto wave_active = [&](int tile) { return !CAUSAL || (tile * FA_BLOCK_N <= wq0 + 31 + causal_off); };
   auto kread = [&](int f, int koff) {  // K fragment f = kg * 4 + ks of the slot at koff
+#if defined(MI355_ABLATE_NO_K_READS)
+    half8 stale = qf[0][f & 3];
+    asm volatile("" : "+v"(stale));
+    return stale;
+#else
     return *(lds_half8_t)(uintptr_t)(k_frag[f & 3] + (unsigned)(koff + (f >> 2) * 4096));
+#endif
   };
   // S^T of one tile, no softmax beside it (a pass's first tile)
   auto scores = [&](int koff, floatx4 (*s)[2]) {
@@ -898,7 +908,11 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     float e_even = 0.f;
     auto expo = [&](int e) {
       const int st = e >> 4, eq = (e >> 3) & 1, ekg = 2 * st + ((e >> 2) & 1), r = e & 3;
+#if defined(MI355_ABLATE_NO_EXP)
+      const float ev = s[ekg][eq][r];
+#else
       const float ev = __builtin_amdgcn_exp2f(s[ekg][eq][r]);
+#endif
       if (e & 1) {
         if (e > 1) psum[((e - 2) >> 3) & 1] = dot2_ones<BF>(pp_prev, psum[((e - 2) >> 3) & 1]);
         half2v pp = cvt16x2<BF>(e_even, ev);
@@ -942,9 +956,13 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
       constexpr int off = VOFF + (f >> 3) * 8192;  // key groups 2 st and 2 st + 1: 16 rows of 256 bytes apart
       half4 &lo = vlo[f % 3], &hi = vhi[f % 3];
       const unsigned addr = v_frag[f & 7];
+#if defined(MI355_ABLATE_NO_V_READS)
+      asm volatile("" : "=&v"(lo), "=&v"(hi) : "v"(addr));
+#else
       asm volatile("ds_read_b64_tr_b16 %0, %2 offset:%3\n\tds_read_b64_tr_b16 %1, %2 offset:%4"
                    : "=&v"(lo), "=&v"(hi)
                    : "v"(addr), "n"(off), "n"(off + 4096));
+#endif
     };
     vr(std::integral_constant<int, 0>{});
     vr(std::integral_constant<int, 1>{});
@@ -994,7 +1012,9 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     if (j + 1 < n_tiles) issue_kv(Vb, v_rb, v_voff, j + 1, V_NEXT);
     if (wave_active(j)) softmax_pv(j, std::integral_constant<int, V_CUR - VBUF>{}, s_cur, K_NEXT, s_next);
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+#if !defined(MI355_ABLATE_NO_BARRIERS)
     __syncthreads();
+#endif
   };
   for (int j = 0; j < n_tiles; j += 2) {
     trip(std::integral_constant<int, 0>{}, j, sa, sb);

@@ -720,7 +720,12 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_stream(const half_t* __restri
   // rows 128 h + 32 blk (+ 8 wave) of the slab at byte offset `at` of operand X into the buffer at byte offset buf_at
   auto load = [&](bool is_a, int buf_at, int h, int blk, unsigned at) {
     const unsigned so = (unsigned)(h * 128 + blk * 32) * row_bytes + at;
+#if defined(MI355_ABLATE_L1_LOADS)
+    buffer_load_lds_16B(is_a ? a_src : b_src, (unsigned)lane * 16u, (so & 1024u) + (unsigned)(blockIdx.x & 31) * 4096u,
+                        lds + buf_at + (h * 16 + blk * 4 + wave) * 1024);
+#elif !defined(MI355_ABLATE_NO_LOADS)
     buffer_load_lds_16B(is_a ? a_src : b_src, g_off, so, lds + buf_at + (h * 16 + blk * 4 + wave) * 1024);
+#endif
   };
 
   // fragment reads: lane l takes row l & 15 of a 16-row block, chunk 4 kh + (l >> 4) of the 128-byte row
@@ -852,9 +857,9 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_stream(const half_t* __restri
   // End of an interval: loads older than one slab and LDS reads older than this interval are complete in every wave.
 #define MI355_SM_SYNC(RD, VM)                                                    \
   do {                                                                           \
-    if constexpr (VM) asm volatile("s_waitcnt vmcnt(16) lgkmcnt(%0)" ::"n"(RD) : "memory"); \
+    if constexpr (VM) asm volatile("s_waitcnt vmcnt(" MI355_KLOOP_VMCNT_STR(16) ") lgkmcnt(%0)" ::"n"(RD) : "memory"); \
     else asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(RD) : "memory");             \
-    __builtin_amdgcn_s_barrier();                                                \
+    MI355_KLOOP_BARRIER();                                                          \
     __builtin_amdgcn_sched_barrier(0);                                           \
   } while (0)
   // Reads issued in one step: 3 in the first half of a slab (A, B, B), 1 in the second.  The read that fills fa for
@@ -883,9 +888,9 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_stream(const half_t* __restri
     MI355_SM_STEP(14, PAR, FB, FBN, 3, FIRST);                                                                         \
     MI355_SM_STEP(15, PAR, FB, FBN, 3, FIRST);                                                                         \
     /* the B fragments of the next slab were all requested in steps 0..7: they have landed; tie them to this point */ \
-    if constexpr (VM) asm volatile("s_waitcnt vmcnt(16) lgkmcnt(4)" : MI355_SM_TIE8(FBN[0]), MI355_SM_TIE8(FBN[1])::"memory"); \
+    if constexpr (VM) asm volatile("s_waitcnt vmcnt(" MI355_KLOOP_VMCNT_STR(16) ") lgkmcnt(4)" : MI355_SM_TIE8(FBN[0]), MI355_SM_TIE8(FBN[1])::"memory"); \
     else asm volatile("s_waitcnt lgkmcnt(4)" : MI355_SM_TIE8(FBN[0]), MI355_SM_TIE8(FBN[1])::"memory");         \
-    __builtin_amdgcn_s_barrier();                                                                               \
+    MI355_KLOOP_BARRIER();                                                                                         \
     __builtin_amdgcn_sched_barrier(0);                                                                          \
     a_off1 = n_a1;                                                                                              \
     a_off2 = n_a2;                                                                                              \

@@ -1137,16 +1137,22 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_stream(const uint8_t* __restri
   unsigned a_off1 = a_cur + 128u, a_off2 = a_cur + 256u, b_off3 = b_cur + 384u, sa_off = sa_cur + 16u, sb_off = sb_cur + 16u;
   unsigned n_a1 = 0, n_a2 = 0, n_b3 = 0, n_sa = 0, n_sb = 0;
   auto load_a = [&](int buf, int h, int blk, unsigned at) {
+#if !defined(MI355_ABLATE_NO_LOADS)
     buffer_load_lds_16B(a_src, g_off, (unsigned)(h * 128 + blk * 32) * row_bytes + at,
                         lds + A_AT + buf * ABUF + (h * 16 + blk * 4 + wave) * 1024);
+#endif
   };
   // part p (rows 32 p .. 32 p + 31 of either 128-row half) into the half buffer at byte offset half_at
   auto load_b = [&](int half_at, int h, int part, unsigned at) {
+#if !defined(MI355_ABLATE_NO_LOADS)
     buffer_load_lds_16B(b_src, g_off, (unsigned)(h * 128 + part * 32) * row_bytes + at,
                         lds + B_AT + half_at + (h * 8 + (part & 1) * 4 + wave) * 1024);
+#endif
   };
   auto load_scales = [&](bool is_b, int grp_at_lds, unsigned at) {
+#if !defined(MI355_ABLATE_NO_LOADS) && !defined(MI355_ABLATE_NO_SCALE_LOADS)
     buffer_load_lds_16B(is_b ? sb_src : sa_src, gs_off, at, lds + S_AT + grp_at_lds + (is_b ? 4096 : 0) + wave * 1024);
+#endif
   };
 
   // fragment reads: lane l takes row l & 15 of a 16-row block, chunk 4 kh + (l >> 4) of the 128-byte row
@@ -1171,6 +1177,9 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_stream(const uint8_t* __restri
   floatx4 acc[8][8];
   half8 fb0[2][8], fb1[2][8], fa[8];
   int sb0[2][8], sb1[2][8], sat[8];  // B scales [k half][row block] of the two slab parities; A scales by step
+#if defined(MI355_ABLATE_NO_SCALE_READS)
+  for (int i = 0; i < 8; i++) sat[i] = sb0[0][i] = sb0[1][i] = sb1[0][i] = sb1[1][i] = 127;
+#endif
 
   // MFMAs as inline assembly with the accumulators pinned to AGPRs (64 four-register accumulators: the compiler's own
   // allocation keeps moving some of them between the two register classes inside the loop).  No MFMA here reads an
@@ -1200,7 +1209,15 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_stream(const uint8_t* __restri
                    : "+a"(c) : "v"(y), "v"(sy), "v"(x), "v"(sx), "n"(LG));                                                      \
   } while (0)
 #define MI355_SM_READ(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off))
+#if defined(MI355_ABLATE_NO_SCALE_READS)  // no scale reads: the counted waits shrink by the reads that are gone
+#define MI355_SM_READ8(dst, addr, off) do {} while (0)
+#define MI355_SM_LG(with_scales, without) without
+#define MI355_SM_LG_END "3"
+#else
 #define MI355_SM_READ8(dst, addr, off) asm volatile("ds_read_u8 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off))
+#define MI355_SM_LG(with_scales, without) with_scales
+#define MI355_SM_LG_END "8"
+#endif
 #define MI355_SM_TIE8(X) "+v"(X[0]), "+v"(X[1]), "+v"(X[2]), "+v"(X[3]), "+v"(X[4]), "+v"(X[5]), "+v"(X[6]), "+v"(X[7])
 
   // ---- prologue: B0 (half buffers 0, 1), A0, B1 (2, 3), A1 blocks 0..2, scale group 0 ----
@@ -1308,8 +1325,8 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_stream(const uint8_t* __restri
   // End of an interval: loads older than the newest VMC and LDS reads older than the interval are complete in every wave.
 #define MI355_SM_SYNC(RD, VMC)                                                        \
   do {                                                                                \
-    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(%1)" ::"n"(VMC), "n"(RD) : "memory");   \
-    __builtin_amdgcn_s_barrier();                                                     \
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(%1)" ::"n"(MI355_KLOOP_VMCNT(VMC)), "n"(RD) : "memory");   \
+    MI355_KLOOP_BARRIER();                                                               \
     __builtin_amdgcn_sched_barrier(0);                                                \
   } while (0)
   // LDS reads per step: 2 (A fragment, A scale) + 4 B fragments in steps 0..3 or 2 B scales in steps 4..11.
@@ -1324,30 +1341,30 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_stream(const uint8_t* __restri
     }                                                                                                           \
     /* slab t + 3: U half -> (2 t + 6) % 5 = pos + 1, V half -> (2 t + 7) % 5 = pos + 2 */                       \
     const int ld_u = (pos + 1 >= 5 ? pos - 4 : pos + 1) * HALF, ld_v = (pos + 2 >= 5 ? pos - 3 : pos + 2) * HALF; \
-    MI355_SM_STEP(0, PAR, FB, FBN, SB, SBN, 6, FIRST);                                                          \
-    MI355_SM_STEP(1, PAR, FB, FBN, SB, SBN, 10, FIRST);                                                         \
-    MI355_SM_STEP(2, PAR, FB, FBN, SB, SBN, 14, FIRST);                                                         \
-    MI355_SM_STEP(3, PAR, FB, FBN, SB, SBN, 15, FIRST);                                                         \
+    MI355_SM_STEP(0, PAR, FB, FBN, SB, SBN, MI355_SM_LG(6, 3), FIRST);                                          \
+    MI355_SM_STEP(1, PAR, FB, FBN, SB, SBN, MI355_SM_LG(10, 7), FIRST);                                         \
+    MI355_SM_STEP(2, PAR, FB, FBN, SB, SBN, MI355_SM_LG(14, 11), FIRST);                                        \
+    MI355_SM_STEP(3, PAR, FB, FBN, SB, SBN, MI355_SM_LG(15, 15), FIRST);                                        \
     MI355_SM_SYNC(15, VMC);                                                                                     \
-    MI355_SM_STEP(4, PAR, FB, FBN, SB, SBN, 15, FIRST);                                                         \
-    MI355_SM_STEP(5, PAR, FB, FBN, SB, SBN, 15, FIRST);                                                         \
-    MI355_SM_STEP(6, PAR, FB, FBN, SB, SBN, 14, FIRST);                                                         \
-    MI355_SM_STEP(7, PAR, FB, FBN, SB, SBN, 12, FIRST);                                                         \
+    MI355_SM_STEP(4, PAR, FB, FBN, SB, SBN, MI355_SM_LG(15, 15), FIRST);                                        \
+    MI355_SM_STEP(5, PAR, FB, FBN, SB, SBN, MI355_SM_LG(15, 15), FIRST);                                        \
+    MI355_SM_STEP(6, PAR, FB, FBN, SB, SBN, MI355_SM_LG(14, 11), FIRST);                                        \
+    MI355_SM_STEP(7, PAR, FB, FBN, SB, SBN, MI355_SM_LG(12, 7), FIRST);                                         \
     MI355_SM_SYNC(15, VMC);                                                                                     \
-    MI355_SM_STEP(8, PAR, FB, FBN, SB, SBN, 12, FIRST);                                                         \
-    MI355_SM_STEP(9, PAR, FB, FBN, SB, SBN, 12, FIRST);                                                         \
-    MI355_SM_STEP(10, PAR, FB, FBN, SB, SBN, 12, FIRST);                                                        \
-    MI355_SM_STEP(11, PAR, FB, FBN, SB, SBN, 12, FIRST);                                                        \
+    MI355_SM_STEP(8, PAR, FB, FBN, SB, SBN, MI355_SM_LG(12, 3), FIRST);                                         \
+    MI355_SM_STEP(9, PAR, FB, FBN, SB, SBN, MI355_SM_LG(12, 3), FIRST);                                         \
+    MI355_SM_STEP(10, PAR, FB, FBN, SB, SBN, MI355_SM_LG(12, 3), FIRST);                                        \
+    MI355_SM_STEP(11, PAR, FB, FBN, SB, SBN, MI355_SM_LG(12, 3), FIRST);                                        \
     MI355_SM_SYNC(15, VMC);                                                                                     \
-    MI355_SM_STEP(12, PAR, FB, FBN, SB, SBN, 12, FIRST);                                                        \
-    MI355_SM_STEP(13, PAR, FB, FBN, SB, SBN, 10, FIRST);                                                        \
-    MI355_SM_STEP(14, PAR, FB, FBN, SB, SBN, 8, FIRST);                                                         \
-    MI355_SM_STEP(15, PAR, FB, FBN, SB, SBN, 6, FIRST);                                                         \
+    MI355_SM_STEP(12, PAR, FB, FBN, SB, SBN, MI355_SM_LG(12, 3), FIRST);                                        \
+    MI355_SM_STEP(13, PAR, FB, FBN, SB, SBN, MI355_SM_LG(10, 3), FIRST);                                        \
+    MI355_SM_STEP(14, PAR, FB, FBN, SB, SBN, MI355_SM_LG(8, 3), FIRST);                                         \
+    MI355_SM_STEP(15, PAR, FB, FBN, SB, SBN, MI355_SM_LG(6, 3), FIRST);                                         \
     /* the next slab's B fragments and scales were requested in steps 0..11: they have landed; tie them here */ \
-    asm volatile("s_waitcnt vmcnt(%32) lgkmcnt(8)"                                                              \
+    asm volatile("s_waitcnt vmcnt(%32) lgkmcnt(" MI355_SM_LG_END ")"                                                              \
                  : MI355_SM_TIE8(FBN[0]), MI355_SM_TIE8(FBN[1]), MI355_SM_TIE8(SBN[0]), MI355_SM_TIE8(SBN[1])   \
-                 : "n"(VMC) : "memory");                                                                        \
-    __builtin_amdgcn_s_barrier();                                                                               \
+                 : "n"(MI355_KLOOP_VMCNT(VMC)) : "memory");                                                                        \
+    MI355_KLOOP_BARRIER();                                                                                         \
     __builtin_amdgcn_sched_barrier(0);                                                                          \
     a_off1 = n_a1;                                                                                              \
     a_off2 = n_a2;                                                                                              \
@@ -1464,6 +1481,8 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_stream(const uint8_t* __restri
 #undef MI355_SM_STEP
 #undef MI355_SM_TIE8
 #undef MI355_SM_READ8
+#undef MI355_SM_LG
+#undef MI355_SM_LG_END
 #undef MI355_SM_READ
 #undef MI355_SM_ACCW
 #undef MI355_SM_ACC

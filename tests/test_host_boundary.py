@@ -234,3 +234,10 @@ def test_dtype_registry_and_shape_inference():
         c.bind_shaped(inst, kb, (4, 16))
     with pytest.raises(ValueError, match="dim arity"):
         c.bind_shaped(object(), kb, (4,))
+
+
+def test_product_library_has_no_ablation_switches():
+    """The in-tree library is the product build: timing-only ablation builds live elsewhere (build.py --out)."""
+    from iree_turbine_amd import _lib
+
+    assert _lib.build_flags() == ""
