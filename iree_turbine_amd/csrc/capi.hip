@@ -63,6 +63,9 @@ extern "C" const char* mi355_build_flags(void) {
 #if defined(MI355_ABLATE_NO_BARRIERS)
          " NO_BARRIERS"
 #endif
+#if defined(MI355_ABLATE_PLAIN_LOAD_ORDER)
+         " PLAIN_LOAD_ORDER"
+#endif
 #if defined(MI355_ABLATE_NO_SCALE_READS)
          " NO_SCALE_READS"
 #endif

@@ -58,6 +58,7 @@ __device__ __forceinline__ int opaque_lane_id() {
 //   MI355_ABLATE_NO_LOADS       the K loop issues no global -> LDS loads (LDS keeps whatever it held)
 //   MI355_ABLATE_L1_LOADS       every load of the K loop reads the same few KiB (always an L1 hit)
 //   MI355_ABLATE_NO_LOAD_WAITS  the K loop never waits for a load
+//   MI355_ABLATE_PLAIN_LOAD_ORDER  (fp16 GEMM) the lanes of a row fetch its 16-byte chunks in ascending order
 //   MI355_ABLATE_NO_BARRIERS    the K loop has no workgroup barriers
 //   MI355_ABLATE_NO_SCALE_READS / MI355_ABLATE_NO_SCALE_LOADS   (block-scaled GEMMs) no LDS reads / no loads of scales
 //   MI355_ABLATE_NO_EXP / MI355_ABLATE_NO_K_READS / MI355_ABLATE_NO_V_READS   (prefill) no exponentials / fragment reads

@@ -707,7 +707,11 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_stream(const half_t* __restri
   const buffer_rsrc_t a_src = make_buffer(A, (unsigned)(tiles_m * BM) * row_bytes);
   const buffer_rsrc_t b_src = make_buffer(B, (unsigned)(tiles_n * BN) * row_bytes);
   const int lrow = lane >> 3;
+#if defined(MI355_ABLATE_PLAIN_LOAD_ORDER)   // timing only: the lanes of a row fetch its chunks in ascending order (LDS then holds the wrong layout)
+  const unsigned g_off = (unsigned)(wave * 8 + lrow) * row_bytes + (unsigned)(lane & 7) * 16u;
+#else
   const unsigned g_off = (unsigned)(wave * 8 + lrow) * row_bytes + (unsigned)((lane & 7) ^ (((wave & 1) << 2) | (lrow >> 1))) * 16u;
+#endif
   const int KT = K / 64;  // even, >= 4 (checked on the host)
   unsigned a_cur = (unsigned)(tile_m * BM) * row_bytes, b_cur = (unsigned)(tile_n * BN) * row_bytes;  // this tile's rows
   unsigned a_nxt = a_cur, b_nxt = b_cur;  // the next tile's (after the last tile: its own again; those loads are never used)

@@ -50,6 +50,44 @@ def test_no_alloc_decode_matches_caller_scratch_twice(dev):
     assert torch.equal(got, want)
 
 
+def test_no_alloc_decode_allocates_nothing(dev):
+    """The property in the entry point's name: free device memory (hipMemGetInfo) is the same before and after a
+    call once the first call on the device has looked up the array's address."""
+    from iree_turbine_amd import _lib
+    from oracle import inputs
+
+    lib = _lib.load()
+    q, kc, vc, bt, sl = (t.to(dev).contiguous() for t in inputs.paged_decode_inputs(num_seqs=6, min_len=30, max_len=700, seed=33))
+    S, Hq, D = q.shape
+    P, page, Hkv, _ = kc.shape
+    out = torch.empty((S, Hq, D), dtype=torch.float16, device=dev)
+    stream = _lib.current_stream_ptr(dev)
+
+    def call():
+        rc = lib.mi355_paged_decode_attn_static(q.data_ptr(), kc.data_ptr(), vc.data_ptr(), bt.data_ptr(), sl.data_ptr(),
+                                                out.data_ptr(), S, Hq, Hkv, D, page, bt.shape[1], P, 4, 128 ** -0.5, stream)
+        _lib.check(rc, "paged_decode_attn_static")
+        torch.cuda.synchronize()
+
+    announce("no-alloc decode: free device memory unchanged across calls")
+    call()  # the first call on a device may load the code object and looks up the array
+    free_before, _ = torch.cuda.mem_get_info(dev)
+    for _ in range(3):
+        call()
+    free_after, _ = torch.cuda.mem_get_info(dev)
+    assert free_after == free_before
+
+
+def test_no_alloc_decode_at_the_arrays_last_row(dev):
+    """num_seqs x num_q_heads x num_splits == 32768 exactly: the last partial ends at the array's last float."""
+    from oracle import inputs
+
+    announce("no-alloc decode: 64 seqs x 32 heads x 16 splits = 32768 rows (the limit)")
+    case = inputs.paged_decode_inputs(num_seqs=64, min_len=300, max_len=1200, seed=34)
+    got, want = _both(dev, *case, 16)
+    assert torch.equal(got, want)
+
+
 def test_no_alloc_decode_rejects_sizes_beyond_its_array(dev):
     from iree_turbine_amd import _lib
 
