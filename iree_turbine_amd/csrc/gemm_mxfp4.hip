@@ -1155,20 +1155,22 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_stream(const uint8_t* __restri
 #endif
   };
 
-  // fragment reads: lane l takes row l & 15 of a 16-row block, chunk 4 kh + (l >> 4) of the 128-byte row
+  // fragment reads: lane l takes row l & 15 of a 16-row block, chunk 2 (l >> 4) + kh of the 128-byte row: which scale
+  // blocks of a slab meet in a k half is free as long as A and B agree, and this pairing puts a lane's two scale bytes
+  // of a slab (k halves 0 and 1) side by side, so one two-byte LDS read fetches both and op_sel picks the byte
   const int r16 = lane & 15, cq = lane >> 4;
   const unsigned lds0 = (unsigned)(uintptr_t)MI355_LDS(char, lds);
-  const unsigned lane_rd = (unsigned)(r16 * 128 + ((cq ^ (r16 >> 1)) & 7) * 16);  // k half 1: ^ 64
+  const unsigned lane_rd = (unsigned)(r16 * 128 + (((2 * cq) ^ (r16 >> 1)) & 7) * 16);  // k half 1: ^ 16
   unsigned aaddr[2][2];  // [A buffer][k half]
 #pragma unroll
   for (int bf = 0; bf < 2; bf++)
 #pragma unroll
-    for (int kh = 0; kh < 2; kh++) aaddr[bf][kh] = lds0 + A_AT + bf * ABUF + wm * (WTM * 128) + (lane_rd ^ (kh * 64));
+    for (int kh = 0; kh < 2; kh++) aaddr[bf][kh] = lds0 + A_AT + bf * ABUF + wm * (WTM * 128) + (lane_rd ^ (kh * 16));
   const unsigned b_lane = lds0 + B_AT + wn * (64 * 128) + lane_rd;  // 64 rows of either half per half buffer
   unsigned bU[2], bV[2];  // [k half]: the U and V half buffers read in this slab
-  // scale reads: the byte of row (16 rb + r16), slab parity sp, block 4 kh + cq sits at row * 16 + 8 sp + 4 kh + cq
-  const unsigned sa_lane = lds0 + S_AT + (unsigned)((wm * WTM + r16) * 16 + cq);
-  const unsigned sb_lane = lds0 + S_AT + 4096 + (unsigned)((wn * WTN + r16) * 16 + cq);
+  // scale reads: the bytes of row (16 rb + r16), slab parity sp, blocks 2 cq and 2 cq + 1 sit at row * 16 + 8 sp + 2 cq
+  const unsigned sa_lane = lds0 + S_AT + (unsigned)((wm * WTM + r16) * 16 + 2 * cq);
+  const unsigned sb_lane = lds0 + S_AT + 4096 + (unsigned)((wn * WTN + r16) * 16 + 2 * cq);
   unsigned sa_rd = sa_lane, sa_rdn = sa_lane + 8, sb_rdn = sb_lane + 8;  // this slab's A scales, the next slab's A and B
 
   // [n block][m block].  Never cleared: the first MFMA of a tile on each accumulator (slab 0, k half 0) takes a zero
@@ -1176,47 +1178,50 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_stream(const uint8_t* __restri
   // know to insert.
   floatx4 acc[8][8];
   half8 fb0[2][8], fb1[2][8], fa[8];
-  int sb0[2][8], sb1[2][8], sat[8];  // B scales [k half][row block] of the two slab parities; A scales by step
+  // scale registers hold two bytes: k half 0 in bits 0..7, k half 1 in bits 8..15 (the MFMA's op_sel picks one)
+  int sb0[8], sb1[8], sat[4];  // B scales [row block] of the two slab parities; A scales by m block (a ring of four)
 #if defined(MI355_ABLATE_NO_SCALE_READS)
-  for (int i = 0; i < 8; i++) sat[i] = sb0[0][i] = sb0[1][i] = sb1[0][i] = sb1[1][i] = 127;
+  for (int i = 0; i < 8; i++) sb0[i] = sb1[i] = 127 * 257;
+  for (int i = 0; i < 4; i++) sat[i] = 127 * 257;
 #endif
 
   // MFMAs as inline assembly with the accumulators pinned to AGPRs (64 four-register accumulators: the compiler's own
   // allocation keeps moving some of them between the two register classes inside the loop).  No MFMA here reads an
-  // accumulator written fewer than 8 MFMAs earlier.  x, sx: B codes and scale (bits 0..7); y, sy: A codes and scale.
-#define MI355_SM_MFMA(c, x, sx, y, sy)                                                                                    \
-  asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0] cbsz:4 blgp:4"                  \
-               : "+a"(c) : "v"(x), "v"(y), "v"(sx), "v"(sy))
-#define MI355_SM_MFMA0(c, x, sx, y, sy)                                                                                   \
-  asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, 0, %3, %4 op_sel_hi:[0,0,0] cbsz:4 blgp:4"                   \
-               : "=a"(c) : "v"(x), "v"(y), "v"(sx), "v"(sy))
-#define MI355_SM_ACC(ZERO, c, x, sx, y, sy)              \
-  do {                                                   \
-    if constexpr (ZERO) MI355_SM_MFMA0(c, x, sx, y, sy); \
-    else MI355_SM_MFMA(c, x, sx, y, sy);                 \
+  // accumulator written fewer than 8 MFMAs earlier.  x, sx: B codes and scales; y, sy: A codes and scales; KH (0 / 1): the
+  // k half, which is also the byte of both scale registers that the MFMA applies.
+#define MI355_SM_MFMA(KH, c, x, sx, y, sy)                                                                                \
+  asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[%5,%5,0] op_sel_hi:[0,0,0] cbsz:4 blgp:4" \
+               : "+a"(c) : "v"(x), "v"(y), "v"(sx), "v"(sy), "n"(KH))
+#define MI355_SM_MFMA0(KH, c, x, sx, y, sy)                                                                               \
+  asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, 0, %3, %4 op_sel:[%5,%5,0] op_sel_hi:[0,0,0] cbsz:4 blgp:4"  \
+               : "=a"(c) : "v"(x), "v"(y), "v"(sx), "v"(sy), "n"(KH))
+#define MI355_SM_ACC(ZERO, KH, c, x, sx, y, sy)              \
+  do {                                                       \
+    if constexpr (ZERO) MI355_SM_MFMA0(KH, c, x, sx, y, sy); \
+    else MI355_SM_MFMA(KH, c, x, sx, y, sy);                 \
   } while (0)
   // The first MFMA of a step together with the wait for the step's A fragment and scale (y, sy: both were requested four
   // steps earlier; LG = LDS reads issued since).  One statement, with the registers as plain inputs: a separate wait
   // statement that names them as outputs makes the compiler put a wait state in front of their next use.  All the
   // statements involved are volatile assembly, which keeps their order.
-#define MI355_SM_ACCW(ZERO, LG, c, x, sx, y, sy)                                                                                  \
+#define MI355_SM_ACCW(ZERO, KH, LG, c, x, sx, y, sy)                                                                              \
   do {                                                                                                                          \
     if constexpr (ZERO)                                                                                                         \
-      asm volatile("s_waitcnt lgkmcnt(%5)\n\tv_mfma_scale_f32_16x16x128_f8f6f4 %0, %3, %1, 0, %4, %2 op_sel_hi:[0,0,0] cbsz:4 blgp:4" \
-                   : "=a"(c) : "v"(y), "v"(sy), "v"(x), "v"(sx), "n"(LG));                                                      \
+      asm volatile("s_waitcnt lgkmcnt(%5)\n\tv_mfma_scale_f32_16x16x128_f8f6f4 %0, %3, %1, 0, %4, %2 op_sel:[%6,%6,0] op_sel_hi:[0,0,0] cbsz:4 blgp:4" \
+                   : "=a"(c) : "v"(y), "v"(sy), "v"(x), "v"(sx), "n"(LG), "n"(KH));                                             \
     else                                                                                                                        \
-      asm volatile("s_waitcnt lgkmcnt(%5)\n\tv_mfma_scale_f32_16x16x128_f8f6f4 %0, %3, %1, %0, %4, %2 op_sel_hi:[0,0,0] cbsz:4 blgp:4" \
-                   : "+a"(c) : "v"(y), "v"(sy), "v"(x), "v"(sx), "n"(LG));                                                      \
+      asm volatile("s_waitcnt lgkmcnt(%5)\n\tv_mfma_scale_f32_16x16x128_f8f6f4 %0, %3, %1, %0, %4, %2 op_sel:[%6,%6,0] op_sel_hi:[0,0,0] cbsz:4 blgp:4" \
+                   : "+a"(c) : "v"(y), "v"(sy), "v"(x), "v"(sx), "n"(LG), "n"(KH));                                             \
   } while (0)
 #define MI355_SM_READ(dst, addr, off) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off))
 #if defined(MI355_ABLATE_NO_SCALE_READS)  // no scale reads: the counted waits shrink by the reads that are gone
-#define MI355_SM_READ8(dst, addr, off) do {} while (0)
+#define MI355_SM_READ16(dst, addr, off) do {} while (0)
 #define MI355_SM_LG(with_scales, without) without
 #define MI355_SM_LG_END "3"
 #else
-#define MI355_SM_READ8(dst, addr, off) asm volatile("ds_read_u8 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off))
+#define MI355_SM_READ16(dst, addr, off) asm volatile("ds_read_u16 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off))
 #define MI355_SM_LG(with_scales, without) with_scales
-#define MI355_SM_LG_END "8"
+#define MI355_SM_LG_END "6"
 #endif
 #define MI355_SM_TIE8(X) "+v"(X[0]), "+v"(X[1]), "+v"(X[2]), "+v"(X[3]), "+v"(X[4]), "+v"(X[5]), "+v"(X[6]), "+v"(X[7])
 
@@ -1235,8 +1240,8 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_stream(const uint8_t* __restri
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __builtin_amdgcn_s_barrier();
   __builtin_amdgcn_sched_barrier(0);
-  bU[0] = b_lane; bU[1] = b_lane ^ 64;
-  bV[0] = b_lane + HALF; bV[1] = bV[0] ^ 64;
+  bU[0] = b_lane; bU[1] = b_lane ^ 16;
+  bV[0] = b_lane + HALF; bV[1] = bV[0] ^ 16;
   MI355_SM_READ(fb0[0][0], bU[0], 0 * 2048); MI355_SM_READ(fb0[0][1], bU[0], 1 * 2048);
   MI355_SM_READ(fb0[0][2], bU[0], 2 * 2048); MI355_SM_READ(fb0[0][3], bU[0], 3 * 2048);
   MI355_SM_READ(fb0[0][4], bV[0], 0 * 2048); MI355_SM_READ(fb0[0][5], bV[0], 1 * 2048);
@@ -1248,17 +1253,12 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_stream(const uint8_t* __restri
   MI355_SM_READ(fa[0], aaddr[0][0], 0); MI355_SM_READ(fa[1], aaddr[0][1], 0);
   MI355_SM_READ(fa[2], aaddr[0][0], 2048); MI355_SM_READ(fa[3], aaddr[0][1], 2048);
   asm volatile("s_waitcnt lgkmcnt(0)" : MI355_SM_TIE8(fb0[0]), MI355_SM_TIE8(fb0[1]), "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]));
-  MI355_SM_READ8(sb0[0][0], sb_lane, 0 * 256); MI355_SM_READ8(sb0[0][1], sb_lane, 1 * 256);
-  MI355_SM_READ8(sb0[0][2], sb_lane, 2 * 256); MI355_SM_READ8(sb0[0][3], sb_lane, 3 * 256);
-  MI355_SM_READ8(sb0[0][4], sb_lane, 4 * 256); MI355_SM_READ8(sb0[0][5], sb_lane, 5 * 256);
-  MI355_SM_READ8(sb0[0][6], sb_lane, 6 * 256); MI355_SM_READ8(sb0[0][7], sb_lane, 7 * 256);
-  MI355_SM_READ8(sb0[1][0], sb_lane, 0 * 256 + 4); MI355_SM_READ8(sb0[1][1], sb_lane, 1 * 256 + 4);
-  MI355_SM_READ8(sb0[1][2], sb_lane, 2 * 256 + 4); MI355_SM_READ8(sb0[1][3], sb_lane, 3 * 256 + 4);
-  MI355_SM_READ8(sb0[1][4], sb_lane, 4 * 256 + 4); MI355_SM_READ8(sb0[1][5], sb_lane, 5 * 256 + 4);
-  MI355_SM_READ8(sb0[1][6], sb_lane, 6 * 256 + 4); MI355_SM_READ8(sb0[1][7], sb_lane, 7 * 256 + 4);
-  MI355_SM_READ8(sat[0], sa_lane, 0); MI355_SM_READ8(sat[1], sa_lane, 4);
-  MI355_SM_READ8(sat[2], sa_lane, 256); MI355_SM_READ8(sat[3], sa_lane, 256 + 4);
-  asm volatile("s_waitcnt lgkmcnt(0)" : MI355_SM_TIE8(sb0[0]), MI355_SM_TIE8(sb0[1]), "+v"(sat[0]), "+v"(sat[1]), "+v"(sat[2]), "+v"(sat[3]));
+  MI355_SM_READ16(sb0[0], sb_lane, 0 * 256); MI355_SM_READ16(sb0[1], sb_lane, 1 * 256);
+  MI355_SM_READ16(sb0[2], sb_lane, 2 * 256); MI355_SM_READ16(sb0[3], sb_lane, 3 * 256);
+  MI355_SM_READ16(sb0[4], sb_lane, 4 * 256); MI355_SM_READ16(sb0[5], sb_lane, 5 * 256);
+  MI355_SM_READ16(sb0[6], sb_lane, 6 * 256); MI355_SM_READ16(sb0[7], sb_lane, 7 * 256);
+  MI355_SM_READ16(sat[0], sa_lane, 0); MI355_SM_READ16(sat[1], sa_lane, 256);
+  asm volatile("s_waitcnt lgkmcnt(0)" : MI355_SM_TIE8(sb0), "+v"(sat[0]), "+v"(sat[1]));
   __builtin_amdgcn_s_barrier();  // every wave has read B0: its half buffers may receive slab 2's V half (0) and slab 3's U half (1)
   __builtin_amdgcn_sched_barrier(0);
   // B2: U half -> half buffer 4, V half -> half buffer 0
@@ -1270,36 +1270,37 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_stream(const uint8_t* __restri
   int pos = 0;
   int sg_ld = SGRP;  // LDS offset of the scale group buffer the next group goes to (groups alternate)
 
-  // Step s of a slab whose A buffer is PAR: MFMAs of (m block s / 2, k half s % 2) on fa[s % 8], sat[s % 8] against
-  // FB / SB[s % 2][0..7].  LGKM = LDS reads issued after those of step s - 4 (which filled fa and sat of this step).
+  // Step s of a slab whose A buffer is PAR: MFMAs of (m block s / 2, k half s % 2) on fa[s % 8] and byte s % 2 of
+  // sat[(s / 2) % 4] against FB[s % 2][0..7] and byte s % 2 of SB[0..7].  LGKM = LDS reads issued after those of step
+  // s - 4 (which filled fa of this step; the m block's scales came with the even step of the pair).
 #define MI355_SM_STEP(s, PAR, FB, FBN, SB, SBN, LGKM, FIRST)                                                               \
   do {                                                                                                                     \
-    constexpr int s4 = (s) + 4, nb = s4 >= 16 ? 1 - (PAR) : (PAR), ns = s4 & 15;                                           \
-    MI355_SM_ACCW(FIRST && !((s)&1), LGKM, acc[0][(s) >> 1], FB[(s)&1][0], SB[(s)&1][0], fa[(s)&7], sat[(s)&7]);            \
+    constexpr int s4 = (s) + 4, nb = s4 >= 16 ? 1 - (PAR) : (PAR), ns = s4 & 15, kh = (s)&1, mb = ((s) >> 1) & 3;          \
+    MI355_SM_ACCW(FIRST && !kh, kh, LGKM, acc[0][(s) >> 1], FB[kh][0], SB[0], fa[(s)&7], sat[mb]);                          \
     MI355_SM_READ(fa[s4 & 7], aaddr[nb][ns & 1], (ns >> 1) * 2048);                                                        \
     __builtin_amdgcn_sched_barrier(0);                                                                                     \
-    MI355_SM_ACC(FIRST && !((s)&1), acc[1][(s) >> 1], FB[(s)&1][1], SB[(s)&1][1], fa[(s)&7], sat[(s)&7]);                   \
-    if constexpr (s4 >= 16) MI355_SM_READ8(sat[s4 & 7], sa_rdn, (ns >> 1) * 256 + (ns & 1) * 4);                           \
-    else MI355_SM_READ8(sat[s4 & 7], sa_rd, (ns >> 1) * 256 + (ns & 1) * 4);                                               \
+    MI355_SM_ACC(FIRST && !kh, kh, acc[1][(s) >> 1], FB[kh][1], SB[1], fa[(s)&7], sat[mb]);                                 \
+    if constexpr (kh == 0) { /* both scale bytes of m block (s + 4) / 2, two steps before its first use */                \
+      if constexpr (s4 >= 16) MI355_SM_READ16(sat[(s4 >> 1) & 3], sa_rdn, (ns >> 1) * 256);                                \
+      else MI355_SM_READ16(sat[(s4 >> 1) & 3], sa_rd, (ns >> 1) * 256);                                                    \
+    }                                                                                                                      \
     __builtin_amdgcn_sched_barrier(0);                                                                                     \
-    MI355_SM_ACC(FIRST && !((s)&1), acc[2][(s) >> 1], FB[(s)&1][2], SB[(s)&1][2], fa[(s)&7], sat[(s)&7]);                   \
+    MI355_SM_ACC(FIRST && !kh, kh, acc[2][(s) >> 1], FB[kh][2], SB[2], fa[(s)&7], sat[mb]);                                 \
     if constexpr ((s) < 4) {                                                                                               \
       MI355_SM_READ(FBN[(s) >> 1][(4 * (s)) & 7], ((s)&1 ? bV : bU)[(s) >> 1], 0 * 2048);                                  \
       MI355_SM_READ(FBN[(s) >> 1][(4 * (s) + 1) & 7], ((s)&1 ? bV : bU)[(s) >> 1], 1 * 2048);                              \
     } else if constexpr ((s) < 12) {                                                                                       \
-      MI355_SM_READ8(SBN[((s)-4) >> 2][(2 * ((s)-4)) & 7], sb_rdn, ((2 * ((s)-4)) & 7) * 256 + (((s)-4) >> 2) * 4);        \
+      MI355_SM_READ16(SBN[(s)-4], sb_rdn, ((s)-4) * 256); /* the next slab's B scales, one row block per step */           \
     }                                                                                                                      \
     __builtin_amdgcn_sched_barrier(0);                                                                                     \
-    MI355_SM_ACC(FIRST && !((s)&1), acc[3][(s) >> 1], FB[(s)&1][3], SB[(s)&1][3], fa[(s)&7], sat[(s)&7]);                   \
+    MI355_SM_ACC(FIRST && !kh, kh, acc[3][(s) >> 1], FB[kh][3], SB[3], fa[(s)&7], sat[mb]);                                 \
     if constexpr ((s) < 4) {                                                                                               \
       MI355_SM_READ(FBN[(s) >> 1][(4 * (s) + 2) & 7], ((s)&1 ? bV : bU)[(s) >> 1], 2 * 2048);                              \
       MI355_SM_READ(FBN[(s) >> 1][(4 * (s) + 3) & 7], ((s)&1 ? bV : bU)[(s) >> 1], 3 * 2048);                              \
-    } else if constexpr ((s) < 12) {                                                                                       \
-      MI355_SM_READ8(SBN[((s)-4) >> 2][(2 * ((s)-4) + 1) & 7], sb_rdn, ((2 * ((s)-4) + 1) & 7) * 256 + (((s)-4) >> 2) * 4); \
     }                                                                                                                      \
     __builtin_amdgcn_sched_barrier(0);                                                                                     \
-    MI355_SM_ACC(FIRST && !((s)&1), acc[4][(s) >> 1], FB[(s)&1][4], SB[(s)&1][4], fa[(s)&7], sat[(s)&7]);                   \
-    MI355_SM_ACC(FIRST && !((s)&1), acc[5][(s) >> 1], FB[(s)&1][5], SB[(s)&1][5], fa[(s)&7], sat[(s)&7]);                   \
+    MI355_SM_ACC(FIRST && !kh, kh, acc[4][(s) >> 1], FB[kh][4], SB[4], fa[(s)&7], sat[mb]);                                 \
+    MI355_SM_ACC(FIRST && !kh, kh, acc[5][(s) >> 1], FB[kh][5], SB[5], fa[(s)&7], sat[mb]);                                 \
     {                                                                                                                      \
       constexpr int q = (s) >> 2, x = (s)&3;                                                                               \
       /* the scale group after this pair of slabs: A rows in step 0, B rows in step 1 of an even slab */                  \
@@ -1318,8 +1319,8 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_stream(const uint8_t* __restri
     if constexpr ((s) == 10) n_b3 = slab_at(kt + 4, b_cur, b_nxt);                                                         \
     if constexpr ((PAR) == 1 && (s) == 11) n_sa = grp_at(kt + 3, sa_cur, sa_nxt);                                          \
     if constexpr ((PAR) == 1 && (s) == 12) n_sb = grp_at(kt + 3, sb_cur, sb_nxt);                                          \
-    MI355_SM_ACC(FIRST && !((s)&1), acc[6][(s) >> 1], FB[(s)&1][6], SB[(s)&1][6], fa[(s)&7], sat[(s)&7]);                   \
-    MI355_SM_ACC(FIRST && !((s)&1), acc[7][(s) >> 1], FB[(s)&1][7], SB[(s)&1][7], fa[(s)&7], sat[(s)&7]);                   \
+    MI355_SM_ACC(FIRST && !kh, kh, acc[6][(s) >> 1], FB[kh][6], SB[6], fa[(s)&7], sat[mb]);                                 \
+    MI355_SM_ACC(FIRST && !kh, kh, acc[7][(s) >> 1], FB[kh][7], SB[7], fa[(s)&7], sat[mb]);                                 \
     __builtin_amdgcn_sched_barrier(0);                                                                                     \
   } while (0)
   // End of an interval: loads older than the newest VMC and LDS reads older than the interval are complete in every wave.
@@ -1329,40 +1330,42 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_stream(const uint8_t* __restri
     MI355_KLOOP_BARRIER();                                                               \
     __builtin_amdgcn_sched_barrier(0);                                                \
   } while (0)
-  // LDS reads per step: 2 (A fragment, A scale) + 4 B fragments in steps 0..3 or 2 B scales in steps 4..11.
+  // LDS reads per step: the A fragment, in even steps the m block's A scales, + 4 B fragments in steps 0..3 or one row
+  // block's B scales in steps 4..11: 6 5 6 5 | 3 2 3 2 | 3 2 3 2 | 2 1 2 1.  A step's count is the sum over the three
+  // steps before it (at most 15 can be counted); an interval's end waits for the reads older than the interval.
 #define MI355_SM_SLAB(PAR, FB, FBN, SB, SBN, FIRST, VMC)                                                         \
   do {                                                                                                          \
     {                                                                                                           \
       const int pu = pos + 2 >= 5 ? pos - 3 : pos + 2, pv = pos + 3 >= 5 ? pos - 2 : pos + 3; /* slab t + 1 */   \
       bU[0] = b_lane + (unsigned)(pu * HALF);                                                                   \
-      bU[1] = bU[0] ^ 64;                                                                                       \
+      bU[1] = bU[0] ^ 16;                                                                                       \
       bV[0] = b_lane + (unsigned)(pv * HALF);                                                                   \
-      bV[1] = bV[0] ^ 64;                                                                                       \
+      bV[1] = bV[0] ^ 16;                                                                                       \
     }                                                                                                           \
     /* slab t + 3: U half -> (2 t + 6) % 5 = pos + 1, V half -> (2 t + 7) % 5 = pos + 2 */                       \
     const int ld_u = (pos + 1 >= 5 ? pos - 4 : pos + 1) * HALF, ld_v = (pos + 2 >= 5 ? pos - 3 : pos + 2) * HALF; \
-    MI355_SM_STEP(0, PAR, FB, FBN, SB, SBN, MI355_SM_LG(6, 3), FIRST);                                          \
-    MI355_SM_STEP(1, PAR, FB, FBN, SB, SBN, MI355_SM_LG(10, 7), FIRST);                                         \
-    MI355_SM_STEP(2, PAR, FB, FBN, SB, SBN, MI355_SM_LG(14, 11), FIRST);                                        \
+    MI355_SM_STEP(0, PAR, FB, FBN, SB, SBN, MI355_SM_LG(4, 3), FIRST);                                          \
+    MI355_SM_STEP(1, PAR, FB, FBN, SB, SBN, MI355_SM_LG(9, 7), FIRST);                                         \
+    MI355_SM_STEP(2, PAR, FB, FBN, SB, SBN, MI355_SM_LG(12, 11), FIRST);                                        \
     MI355_SM_STEP(3, PAR, FB, FBN, SB, SBN, MI355_SM_LG(15, 15), FIRST);                                        \
     MI355_SM_SYNC(15, VMC);                                                                                     \
     MI355_SM_STEP(4, PAR, FB, FBN, SB, SBN, MI355_SM_LG(15, 15), FIRST);                                        \
-    MI355_SM_STEP(5, PAR, FB, FBN, SB, SBN, MI355_SM_LG(15, 15), FIRST);                                        \
-    MI355_SM_STEP(6, PAR, FB, FBN, SB, SBN, MI355_SM_LG(14, 11), FIRST);                                        \
-    MI355_SM_STEP(7, PAR, FB, FBN, SB, SBN, MI355_SM_LG(12, 7), FIRST);                                         \
-    MI355_SM_SYNC(15, VMC);                                                                                     \
-    MI355_SM_STEP(8, PAR, FB, FBN, SB, SBN, MI355_SM_LG(12, 3), FIRST);                                         \
-    MI355_SM_STEP(9, PAR, FB, FBN, SB, SBN, MI355_SM_LG(12, 3), FIRST);                                         \
-    MI355_SM_STEP(10, PAR, FB, FBN, SB, SBN, MI355_SM_LG(12, 3), FIRST);                                        \
-    MI355_SM_STEP(11, PAR, FB, FBN, SB, SBN, MI355_SM_LG(12, 3), FIRST);                                        \
-    MI355_SM_SYNC(15, VMC);                                                                                     \
-    MI355_SM_STEP(12, PAR, FB, FBN, SB, SBN, MI355_SM_LG(12, 3), FIRST);                                        \
-    MI355_SM_STEP(13, PAR, FB, FBN, SB, SBN, MI355_SM_LG(10, 3), FIRST);                                        \
-    MI355_SM_STEP(14, PAR, FB, FBN, SB, SBN, MI355_SM_LG(8, 3), FIRST);                                         \
-    MI355_SM_STEP(15, PAR, FB, FBN, SB, SBN, MI355_SM_LG(6, 3), FIRST);                                         \
+    MI355_SM_STEP(5, PAR, FB, FBN, SB, SBN, MI355_SM_LG(14, 15), FIRST);                                        \
+    MI355_SM_STEP(6, PAR, FB, FBN, SB, SBN, MI355_SM_LG(10, 11), FIRST);                                        \
+    MI355_SM_STEP(7, PAR, FB, FBN, SB, SBN, MI355_SM_LG(8, 7), FIRST);                                         \
+    MI355_SM_SYNC(MI355_SM_LG(10, 4), VMC);                                                                                     \
+    MI355_SM_STEP(8, PAR, FB, FBN, SB, SBN, MI355_SM_LG(7, 3), FIRST);                                         \
+    MI355_SM_STEP(9, PAR, FB, FBN, SB, SBN, MI355_SM_LG(8, 3), FIRST);                                         \
+    MI355_SM_STEP(10, PAR, FB, FBN, SB, SBN, MI355_SM_LG(7, 3), FIRST);                                        \
+    MI355_SM_STEP(11, PAR, FB, FBN, SB, SBN, MI355_SM_LG(8, 3), FIRST);                                        \
+    MI355_SM_SYNC(MI355_SM_LG(10, 4), VMC);                                                                                     \
+    MI355_SM_STEP(12, PAR, FB, FBN, SB, SBN, MI355_SM_LG(7, 3), FIRST);                                        \
+    MI355_SM_STEP(13, PAR, FB, FBN, SB, SBN, MI355_SM_LG(7, 3), FIRST);                                        \
+    MI355_SM_STEP(14, PAR, FB, FBN, SB, SBN, MI355_SM_LG(5, 3), FIRST);                                         \
+    MI355_SM_STEP(15, PAR, FB, FBN, SB, SBN, MI355_SM_LG(5, 3), FIRST);                                         \
     /* the next slab's B fragments and scales were requested in steps 0..11: they have landed; tie them here */ \
-    asm volatile("s_waitcnt vmcnt(%32) lgkmcnt(" MI355_SM_LG_END ")"                                                              \
-                 : MI355_SM_TIE8(FBN[0]), MI355_SM_TIE8(FBN[1]), MI355_SM_TIE8(SBN[0]), MI355_SM_TIE8(SBN[1])   \
+    asm volatile("s_waitcnt vmcnt(%24) lgkmcnt(" MI355_SM_LG_END ")"                                                              \
+                 : MI355_SM_TIE8(FBN[0]), MI355_SM_TIE8(FBN[1]), MI355_SM_TIE8(SBN)                             \
                  : "n"(MI355_KLOOP_VMCNT(VMC)) : "memory");                                                                        \
     MI355_KLOOP_BARRIER();                                                                                         \
     __builtin_amdgcn_sched_barrier(0);                                                                          \
@@ -1475,12 +1478,12 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_stream(const uint8_t* __restri
     __builtin_amdgcn_sched_barrier(0);
   }
   // the loads issued for a tile that does not exist still target LDS: let them land before the workgroup ends
-  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : MI355_SM_TIE8(fa), MI355_SM_TIE8(sat));
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : MI355_SM_TIE8(fa), "+v"(sat[0]), "+v"(sat[1]), "+v"(sat[2]), "+v"(sat[3]));
 #undef MI355_SM_SLAB
 #undef MI355_SM_SYNC
 #undef MI355_SM_STEP
 #undef MI355_SM_TIE8
-#undef MI355_SM_READ8
+#undef MI355_SM_READ16
 #undef MI355_SM_LG
 #undef MI355_SM_LG_END
 #undef MI355_SM_READ
