@@ -1,18 +1,21 @@
-// fp16 NT GEMM for gfx950:  C[M,N] = A[M,K] . B[N,K]^T with fp32 accumulation.
+// fp16 / bf16 NT GEMM for gfx950:  C[M,N] = A[M,K] . B[N,K]^T with fp32 accumulation.
 //
-// Main kernel (gemm_f16_nt_tiled): a BM x BN output tile per workgroup, K walked in slabs
-// of 64 halfs.  A slab row is 128 bytes = 8 chunks of 16 bytes; both operands are
-// K-contiguous, so the same row format serves A and B.  Slabs are copied global -> LDS with
-// direct-to-LDS loads (no VGPR staging) into a two-stage ring: while the MFMAs consume
-// stage s the loads for the next slab fill stage s^1, and one barrier per slab closes the
-// iteration.  LDS rows are XOR-swizzled at chunk granularity: chunk c of row r lives in slot
-// c ^ ((r >> 1) & 7).  LDS has 64 banks of 4 bytes, so two 128-byte rows span the banks once and a
+// Kernels in this file, all on the same LDS row format: gemm_f16_nt_stream (the current kernel for large shapes: whole-row
+// direct-to-LDS loads two slabs ahead, 16x16x32 MFMAs, a tile walk), gemm_f16_nt_persistent (8 waves, chosen for short
+// K), gemm_f16_nt_pipelined (128x128 tiles: few tiles, and the strip a sparse last round is cut into),
+// gemm_f16_nt_staged (the register-staged predecessor of the streamed kernel, kept as the independent comparator of
+// the bit-identity tests), gemm_f16_nt_skinny (M <= 64: weight streaming) and a bounds-checked kernel for any shape.
+//
+// LDS row format: K is walked in slabs of 64 halfs; a slab row is 128 bytes = 8 chunks of 16 bytes; both operands are
+// K-contiguous, so the same row format serves A and B.  Slabs are copied global -> LDS with direct-to-LDS loads (no VGPR
+// staging; the register-staged kernel excepted).  LDS rows are XOR-swizzled at chunk granularity: chunk c of row r lives
+// in slot c ^ ((r >> 1) & 7).  LDS has 64 banks of 4 bytes, so two 128-byte rows span the banks once and a
 // 16-lane phase of a ds_read_b128 (16 consecutive rows, one chunk each) is conflict-free exactly
 // when (r & 1, slot) is distinct over those rows; measured 247 B/clk/CU against 128 for the
 // c ^ (r & 7) swizzle and 32 unswizzled.  Because a direct-to-LDS load fixes the LDS slot by lane
 // id, the swizzle is applied on the global side (lane -> which chunk it fetches).
 //
-// The MFMA roles are swapped (B rows feed the "A" operand, A rows feed the "B" operand) so a
+// In the 32x32x16 kernels the MFMA roles are swapped (B rows feed the "A" operand, A rows feed the "B" operand) so a
 // lane ends up owning 4 consecutive n for one m, which turns the epilogue into 8/16-byte
 // row-contiguous stores.
 //
@@ -58,128 +61,8 @@ __device__ __forceinline__ void map_tile(int pid, int tiles_m, int tiles_n, int 
   tn = within / gsz;
 }
 
-template <int BM, int BN, int WM, int WN, typename OutT, bool BF>
-__global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_tiled(const half_t* __restrict__ A,
-                                                                 const half_t* __restrict__ B,
-                                                                 OutT* __restrict__ C, int M, int N, int K,
-                                                                 int tiles_m, int tiles_n, int group_m) {
-  constexpr int NW = WM * WN;
-  constexpr int WTM = BM / WM, WTN = BN / WN;
-  constexpr int TM = WTM / 32, TN = WTN / 32;
-  constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
-  constexpr int A_GROUPS = BM / 8, B_GROUPS = BN / 8;  // 8 rows = 1 KiB = one wave-wide load
-  static_assert(A_GROUPS % NW == 0 && B_GROUPS % NW == 0 && NW % 2 == 0, "loads must split evenly over an even number of waves");
-  constexpr int LA = A_GROUPS / NW, LB = B_GROUPS / NW;
-
-  extern __shared__ __attribute__((aligned(1024))) char lds[];
-
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int wm = wave / WN, wn = wave % WN;
-  int tile_m, tile_n;
-  map_tile(blockIdx.x, tiles_m, tiles_n, group_m, tile_m, tile_n);
-
-  // ---- global -> LDS: lane l of a wave-load covers row (l/8) of an 8-row group, slot l%8 ----
-  const int lrow = lane >> 3;
-  const int lchunk = (lane & 7) ^ (((wave & 1) << 2) | (lrow >> 1));  // the chunk that belongs in this lane's slot
-  const half_t* a_src = A + (size_t)(tile_m * BM + wave * 8 + lrow) * K + lchunk * 8;
-  const half_t* b_src = B + (size_t)(tile_n * BN + wave * 8 + lrow) * K + lchunk * 8;
-  const size_t row_step = (size_t)NW * 8 * K;  // halfs between this wave's consecutive groups
-
-  auto issue_loads = [&](int stage) {
-    char* dst = lds + stage * STAGE + wave * 1024;
-#pragma unroll
-    for (int i = 0; i < LA; i++) load_lds_16B(a_src + i * row_step, dst + i * NW * 1024);
-#pragma unroll
-    for (int i = 0; i < LB; i++) load_lds_16B(b_src + i * row_step, dst + A_BYTES + i * NW * 1024);
-    a_src += 64;
-    b_src += 64;
-  };
-
-  // ---- LDS -> MFMA fragments ----
-  const int r32 = lane & 31, h = lane >> 5;
-  const int sw = (h ^ ((r32 >> 1) & 7)) * 16;
-  const int a_base = (wm * WTM + r32) * 128 + sw;            // rows of A (m): feeds the MFMA "B" operand
-  const int b_base = A_BYTES + (wn * WTN + r32) * 128 + sw;  // rows of B (n): feeds the MFMA "A" operand
-
-  floatx16 acc[TN][TM];
-#pragma unroll
-  for (int i = 0; i < TN; i++)
-#pragma unroll
-    for (int j = 0; j < TM; j++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
-
-  const int KT = K / 64;
-  issue_loads(0);
-  wait_vmcnt0();
-  __syncthreads();
-
-  for (int kt = 0; kt < KT; kt++) {
-    if (kt + 1 < KT) issue_loads((kt + 1) & 1);
-    const char* st = lds + (kt & 1) * STAGE;
-#pragma unroll
-    for (int ks = 0; ks < 4; ks++) {
-      half8 fm[TM], fn[TN];
-#pragma unroll
-      for (int j = 0; j < TM; j++) fm[j] = *reinterpret_cast<const half8*>(st + ((a_base ^ (ks * 32)) + j * 4096));
-#pragma unroll
-      for (int i = 0; i < TN; i++) fn[i] = *reinterpret_cast<const half8*>(st + ((b_base ^ (ks * 32)) + i * 4096));
-#pragma unroll
-      for (int i = 0; i < TN; i++)
-#pragma unroll
-        for (int j = 0; j < TM; j++) acc[i][j] = mfma16<BF>(fn[i], fm[j], acc[i][j]);
-    }
-    wait_vmcnt0();
-    __syncthreads();
-  }
-
-  // ---- epilogue: lane owns m = r32 and, per register quad q, n = 8q + 4h .. +3 ----
-  if constexpr (sizeof(OutT) == 2) {
-    // fp16 epilogue through LDS (free after the last barrier): each wave transposes its own
-    // WTM x WTN tile in a private region (ds_write_b64 of 4 consecutive n, chunk slot c ^ ((m>>1)&7)),
-    // then reads whole rows back 16 bytes per lane and stores full 128-byte lines.
-    constexpr int ROW_B = WTN * 2, CH = WTN / 8;
-    char* ep = lds + wave * (WTM * ROW_B);
-#pragma unroll
-    for (int j = 0; j < TM; j++) {
-      const int ml = j * 32 + r32;
-#pragma unroll
-      for (int i = 0; i < TN; i++)
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-          const int c = i * 4 + q;
-          half4 v = {cvt16<BF>(acc[i][j][4 * q]), cvt16<BF>(acc[i][j][4 * q + 1]), cvt16<BF>(acc[i][j][4 * q + 2]),
-                     cvt16<BF>(acc[i][j][4 * q + 3])};
-          *reinterpret_cast<half4*>(ep + ml * ROW_B + ((c ^ ((ml >> 1) & 7)) * 16) + 8 * h) = v;
-        }
-    }
-    constexpr int ROWS_PER_IT = 64 / CH;
-    const int er = lane / CH, ec = lane % CH;
-    OutT* cbase = C + (size_t)(tile_m * BM + wm * WTM) * N + tile_n * BN + wn * WTN + ec * 8;
-#pragma unroll
-    for (int it = 0; it < WTM / ROWS_PER_IT; it++) {
-      const int row = it * ROWS_PER_IT + er;
-      half8 v = *reinterpret_cast<const half8*>(ep + row * ROW_B + ((ec ^ ((row >> 1) & 7)) * 16));
-      *reinterpret_cast<half8*>(cbase + (size_t)row * N) = v;
-    }
-  } else {
-    const int m0 = tile_m * BM + wm * WTM + r32;
-    const int n0 = tile_n * BN + wn * WTN + 4 * h;
-#pragma unroll
-    for (int j = 0; j < TM; j++) {
-      OutT* crow = C + (size_t)(m0 + j * 32) * N + n0;
-#pragma unroll
-      for (int i = 0; i < TN; i++)
-#pragma unroll
-        for (int q = 0; q < 4; q++)
-          OutPack<OutT, BF>::store4(crow + i * 32 + q * 8, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
-                                acc[i][j][4 * q + 3]);
-    }
-  }
-}
-
-// Software-pipelined form of the tiled kernel.  Same tiling, LDS format and swizzle; the k-loop is
+// Software-pipelined two-stage kernel: a BM x BN output tile per workgroup, slabs copied global -> LDS with
+// direct-to-LDS loads into a two-stage ring, 32x32x16 MFMAs.  The k-loop is
 // rotated so that (a) the fragments of k-step s+1 are requested from LDS before the MFMAs of
 // k-step s issue, (b) the barrier that retires a slab sits in front of the last k-step's MFMAs,
 // which then overlap the first fragment reads of the next slab, and (c) the global -> LDS loads
@@ -1399,21 +1282,16 @@ struct GemmVariant {
 };
 static const GemmVariant kGemmVariants[] = {
     {"persistent_256x256x64_w2x4", 256, 256, 512},
-    {"persistent_256x256x64_w2x2", 256, 256, 256},
-    {"pipelined_256x256x64_w2x4", 256, 256, 512},
-    {"pipelined_256x256x64_w2x2", 256, 256, 256},
     {"pipelined_128x128x64_w2x2", 128, 128, 256},
-    {"tiled_256x256x64_w2x4", 256, 256, 512},
-    {"tiled_128x128x64_w2x2", 128, 128, 256},
     {"staged_256x256x64_w2x2", 256, 256, 256},
-    {"staged_256x256_tail_128x128", 256, 256, 256},
     {"skinny_m32_n32_w8", 32, 32, 512},
-    {"staged_256x256x64_w2x2_walk", 256, 256, 256},
     {"stream_256x256x64_w2x2", 256, 256, 256},
     {"stream_256x256_tail_128x128", 256, 256, 256},
     {"stream_256x256x64_w2x2_walk", 256, 256, 256},
     {"generic_64x64x32", 64, 64, 256},
 };
+// indices of the table above
+enum { V_PERSISTENT = 0, V_PIPELINED_128 = 1, V_STAGED = 2, V_SKINNY = 3, V_STREAM = 4, V_STREAM_TAIL = 5, V_STREAM_WALK = 6 };
 constexpr int kNumGemmVariants = sizeof(kGemmVariants) / sizeof(kGemmVariants[0]);
 
 int gemm_variant_count() { return kNumGemmVariants; }
@@ -1432,33 +1310,24 @@ static int cu_count() {
   return cached[dev];
 }
 
-template <int BM, int BN, int WM, int WN, typename OutT, int KIND, bool BF>  // KIND: 0 tiled, 1 pipelined, 2 register-staged
-static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int K, int ldc, hipStream_t stream,
-                        bool one_per_cu = false) {
+template <int BM, int BN, int WM, int WN, typename OutT, int KIND, bool BF>  // KIND: 1 pipelined, 2 register-staged
+static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int K, int ldc, hipStream_t stream) {
   // the kernels use their N argument only as the row stride of C, so a column range of a wider C is the
   // same launch with ldc in its place
-  constexpr bool PIPELINED = KIND == 1;
+  static_assert(KIND == 1 || KIND == 2, "pipelined or register-staged");
   void (*kern)(const half_t*, const half_t*, OutT*, int, int, int, int, int, int);
   if constexpr (KIND == 2) kern = gemm_f16_nt_staged<BM, BN, WM, WN, OutT, BF>;
-  else if constexpr (PIPELINED) kern = gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT, BF>;
-  else kern = gemm_f16_nt_tiled<BM, BN, WM, WN, OutT, BF>;
+  else kern = gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT, BF>;
   // the register-staged kernel keeps its epilogue out of the stages: 32 rows x 128 bytes per wave
   constexpr int lds_bytes = 2 * (BM + BN) * 128 + (KIND == 2 ? WM * WN * 32 * 128 : 0);
   static std::atomic<uint64_t> lds_ok{0};
   if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt")) return rc;
   const int tiles_m = M / BM, tiles_n = N / BN;
   int group_m = 4;
-  int wgs = tiles_m * tiles_n;
-  if (KIND == 2 && one_per_cu) {
-    // one workgroup per CU walking tiles pid, pid + grid, ...; a multiple of 8 keeps a workgroup's tiles on its XCD
-    int g = cu_count() & ~7;
-    if (g < 8) g = 8;
-    if (wgs > g) wgs = g;
-  }
-  dim3 grid(wgs), block(WM * WN * 64);
+  dim3 grid(tiles_m * tiles_n), block(WM * WN * 64);
   hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, M, ldc, K, tiles_m,
                      tiles_n, group_m);
-  return check_launch(KIND == 2 ? "gemm_f16_nt_staged" : PIPELINED ? "gemm_f16_nt_pipelined" : "gemm_f16_nt_tiled", grid, block, lds_bytes);
+  return check_launch(KIND == 2 ? "gemm_f16_nt_staged" : "gemm_f16_nt_pipelined", grid, block, lds_bytes);
 }
 
 template <int BM, int BN, int WM, int WN, typename OutT, bool BF>
@@ -1519,12 +1388,9 @@ static bool tail_split(int M, int N, int& main_m, int& main_n) {
   return true;
 }
 
-template <typename OutT, bool BF, bool STREAMED>
+template <typename OutT, bool BF>
 static int launch_split(const void* a, const void* b, void* c, int M, int N, int K, hipStream_t stream) {
-  auto main_part = [&](int m, int n) {
-    if constexpr (STREAMED) return launch_stream<OutT, BF>(a, b, c, m, n, K, N, stream, true);  // one workgroup per CU
-    else return launch_tiled<256, 256, 2, 2, OutT, 2, BF>(a, b, c, m, n, K, N, stream);
-  };
+  auto main_part = [&](int m, int n) { return launch_stream<OutT, BF>(a, b, c, m, n, K, N, stream, true); };  // one workgroup per CU
   int mm, mn;
   if (!tail_split(M, N, mm, mn)) return main_part(M, N);
   int rc = main_part(mm, mn);
@@ -1539,16 +1405,10 @@ static int launch_split(const void* a, const void* b, void* c, int M, int N, int
 template <typename OutT, bool BF>
 static int launch_variant(int variant, const void* a, const void* b, void* c, int M, int N, int K, hipStream_t stream) {
   switch (variant) {
-    case 0: return launch_persistent<256, 256, 2, 4, OutT, BF>(a, b, c, M, N, K, stream);
-    case 1: return launch_persistent<256, 256, 2, 2, OutT, BF>(a, b, c, M, N, K, stream);
-    case 2: return launch_tiled<256, 256, 2, 4, OutT, 1, BF>(a, b, c, M, N, K, N, stream);
-    case 3: return launch_tiled<256, 256, 2, 2, OutT, 1, BF>(a, b, c, M, N, K, N, stream);
-    case 4: return launch_tiled<128, 128, 2, 2, OutT, 1, BF>(a, b, c, M, N, K, N, stream);
-    case 5: return launch_tiled<256, 256, 2, 4, OutT, 0, BF>(a, b, c, M, N, K, N, stream);
-    case 6: return launch_tiled<128, 128, 2, 2, OutT, 0, BF>(a, b, c, M, N, K, N, stream);
-    case 7: return launch_tiled<256, 256, 2, 2, OutT, 2, BF>(a, b, c, M, N, K, N, stream);
-    case 8: return launch_split<OutT, BF, false>(a, b, c, M, N, K, stream);
-    case 9: {
+    case V_PERSISTENT: return launch_persistent<256, 256, 2, 4, OutT, BF>(a, b, c, M, N, K, stream);
+    case V_PIPELINED_128: return launch_tiled<128, 128, 2, 2, OutT, 1, BF>(a, b, c, M, N, K, N, stream);
+    case V_STAGED: return launch_tiled<256, 256, 2, 2, OutT, 2, BF>(a, b, c, M, N, K, N, stream);
+    case V_SKINNY: {
       auto kern = gemm_f16_nt_skinny<OutT, BF>;
       constexpr int lds_bytes = 8 * 16384;
       static std::atomic<uint64_t> lds_ok{0};
@@ -1564,10 +1424,9 @@ static int launch_variant(int variant, const void* a, const void* b, void* c, in
       }
       return 0;
     }
-    case 10: return launch_tiled<256, 256, 2, 2, OutT, 2, BF>(a, b, c, M, N, K, N, stream, true);
-    case 11: return launch_stream<OutT, BF>(a, b, c, M, N, K, N, stream);
-    case 12: return launch_split<OutT, BF, true>(a, b, c, M, N, K, stream);
-    case 13: return launch_stream<OutT, BF>(a, b, c, M, N, K, N, stream, true);
+    case V_STREAM: return launch_stream<OutT, BF>(a, b, c, M, N, K, N, stream);
+    case V_STREAM_TAIL: return launch_split<OutT, BF>(a, b, c, M, N, K, stream);
+    case V_STREAM_WALK: return launch_stream<OutT, BF>(a, b, c, M, N, K, N, stream, true);
     default: {
       dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
       hipLaunchKernelGGL((gemm_f16_nt_generic<OutT, BF>), grid, block, 0, stream, (const half_t*)a, (const half_t*)b, (OutT*)c,
@@ -1593,13 +1452,14 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
   const bool al = aligned16(a) && aligned16(b) && aligned16(c);
   auto fits = [&](int v) {
     if (v == kNumGemmVariants - 1) return true;
-    if (v <= 1 && (K < 128 || K > (1 << 21))) return false;  // prefetches two slabs ahead; 32-bit byte offsets inside a 256-row panel
-    if ((v == 7 || v == 8 || v == 10) && N > (1 << 22)) return false;  // 32-bit byte offsets inside a wave's 128 rows of C
-    if ((v == 7 || v == 8 || v == 10) && (K < 256 || K % 128 != 0 || K > (1 << 21))) return false;  // slabs in pairs, three in flight
+    const bool streamed = v == V_STREAM || v == V_STREAM_TAIL || v == V_STREAM_WALK;
+    if (v == V_PERSISTENT && (K < 128 || K > (1 << 21))) return false;  // prefetches two slabs ahead; 32-bit byte offsets inside a 256-row panel
+    if (v == V_STAGED && N > (1 << 22)) return false;  // 32-bit byte offsets inside a wave's 128 rows of C
+    if (v == V_STAGED && (K < 256 || K % 128 != 0 || K > (1 << 21))) return false;  // slabs in pairs, three in flight
     // the streamed kernel addresses each operand through one buffer descriptor
-    if ((v == 11 || v == 12 || v == 13) && (M * K * 2 >= (1ll << 32) || N * K * 2 >= (1ll << 32))) return false;
-    if ((v == 11 || v == 12 || v == 13) && (K < 256 || K % 128 != 0 || K > (1 << 21))) return false;  // slabs in pairs; 32-bit byte offsets inside a 256-row panel
-    if (v == 9) return al && M <= 64 && N % 32 == 0 && K % 64 == 0;  // a tile is 32 rows of B; 64-half K segments
+    if (streamed && (M * K * 2 >= (1ll << 32) || N * K * 2 >= (1ll << 32))) return false;
+    if (streamed && (K < 256 || K % 128 != 0 || K > (1 << 21))) return false;  // slabs in pairs; 32-bit byte offsets inside a 256-row panel
+    if (v == V_SKINNY) return al && M <= 64 && N % 32 == 0 && K % 64 == 0;  // a tile is 32 rows of B; 64-half K segments
     return al && M % kGemmVariants[v].bm == 0 && N % kGemmVariants[v].bn == 0 && K % 64 == 0;
   };
   if (variant < 0) {
@@ -1607,20 +1467,19 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
     // 128x128 tile (4x the workgroups) wins; everything else goes to the bounds-checked kernel.
     const long long t256 = (M / 256) * (N / 256);
     const long long rounds = (t256 + 255) / 256;  // 256 CUs, one 256x256 workgroup each
-    // The streamed kernel with its sparse last round cut off (variant 12) from K = 1024 up: 8192^3 1460 against 1295
+    // The streamed kernel with its sparse last round cut off from K = 1024 up: 8192^3 1460 against 1295
     // TFLOP/s for the register-staged kernel and 1285 for the persistent one, 4096^3 1405 / 1240 / 1244,
     // 2048x10240x8192 1285 / 1180 / 1044, 8192x8192x1024 1174 / 1064 / 1167.  Shorter K: the persistent kernel, which
     // hides each tile's prologue and epilogue under its neighbours (8192x8192x512: 978 against 854), as long as its
     // last round is >= 85% busy.
     const bool full_rounds = t256 * 100 >= rounds * 256 * 85;
-    if (fits(9) && N >= 2048 && K >= 512) variant = 9;  // decode-shaped: stream the weights once
-    else
-    if (K < 1024 && t256 <= 2048 && fits(0) && t256 >= 128 && full_rounds) variant = 0;
-    else if (fits(12) && t256 >= 128) variant = 12;
-    else if (fits(0) && t256 >= 128 && full_rounds) variant = 0;
-    else if (fits(4)) variant = 4;
+    if (fits(V_SKINNY) && N >= 2048 && K >= 512) variant = V_SKINNY;  // decode-shaped: stream the weights once
+    else if (K < 1024 && t256 <= 2048 && fits(V_PERSISTENT) && t256 >= 128 && full_rounds) variant = V_PERSISTENT;
+    else if (fits(V_STREAM_TAIL) && t256 >= 128) variant = V_STREAM_TAIL;
+    else if (fits(V_PERSISTENT) && t256 >= 128 && full_rounds) variant = V_PERSISTENT;
+    else if (fits(V_PIPELINED_128)) variant = V_PIPELINED_128;
     else variant = kNumGemmVariants - 1;
-  } else if (!fits(variant) && variant == 9) {
+  } else if (!fits(variant) && variant == V_SKINNY) {
     return fail(-MI355_E_SHAPE, "gemm_f16_nt: variant %s needs M<=64, N%%32==0, K%%64==0 and 16-byte aligned pointers",
                 kGemmVariants[variant].name);
   } else if (!fits(variant)) {

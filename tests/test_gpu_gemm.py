@@ -22,7 +22,7 @@ def _run(dev, M, N, K, out_dtype, variant=-1, seed=10):
     return c.float().cpu(), ref
 
 
-@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 3, 4, 5, 6, 7, 8, 10, 11, 12, 13])
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 4, 5, 6])  # every tiled kernel (3 is the skinny-M kernel, 7 the any-shape one)
 def test_gemm_1024_f32_all_variants(dev, variant):
     c, ref = _run(dev, 1024, 1024, 1024, "float32", variant)
     torch.testing.assert_close(c, ref, rtol=RTOL, atol=ATOL)
@@ -149,14 +149,15 @@ def test_gemm_full_size_repeatable(dev, shape):
         if names[variant].startswith(("staged", "stream")):
             by_name[names[variant]] = first
         del first
-    # the tail split hands the last tile columns to a second kernel that adds K in the same order: the whole
-    # matrix equals the unsplit staged kernel's bit for bit
-    # and so does the same kernel launched with one workgroup per CU, walking its tiles as one slab sequence
-    staged = [v for k, v in sorted(by_name.items()) if k.startswith("staged")]
-    assert len(staged) == 3 and torch.equal(staged[0], staged[1]) and torch.equal(staged[0], staged[2])
-    # likewise the streamed kernel and its tail-split launch
+    # the tail split hands the last tile columns to a second kernel that adds K in the same order: the whole matrix
+    # equals the unsplit streamed kernel's bit for bit, and so does the same kernel launched with one workgroup per
+    # CU, walking its tiles as one slab sequence
     streamed = [v for k, v in sorted(by_name.items()) if k.startswith("stream")]
     assert len(streamed) == 3 and torch.equal(streamed[0], streamed[1]) and torch.equal(streamed[0], streamed[2])
+    # and the register-staged kernel, an independent implementation (other MFMA shape, other load path) that adds K
+    # in the same order per element
+    staged = [v for k, v in sorted(by_name.items()) if k.startswith("staged")]
+    assert len(staged) == 1 and torch.equal(staged[0], streamed[0])
 
 
 @pytest.mark.parametrize("shape", [(4096, 4608, 192), (4352, 4352, 128), (8192, 8704, 320), (512, 256, 4096)])
@@ -180,30 +181,6 @@ def test_gemm_persistent_tile_walk(dev, shape, out_dtype):
     rows = torch.tensor([0, 255, 256, M - 1])
     exact = a[rows.to(dev)].float() @ b.float().t()
     torch.testing.assert_close(got[rows.to(dev)].float(), exact, rtol=RTOL, atol=ATOL)
-
-
-@pytest.mark.parametrize("out_dtype", ["float16", "float32"])
-@pytest.mark.parametrize("shape", [(4096, 4608, 256), (4352, 4352, 384), (8192, 8704, 512), (8192, 16384, 1152), (512, 256, 4096)])
-def test_gemm_staged_tile_walk(dev, shape, out_dtype):
-    """The register-staged kernel launched with one workgroup per CU: every workgroup walks several tiles as one slab
-    sequence (the loads of a tile's last three slabs are the next tile's first three, the first two slabs of a
-    later tile run without load waits, the epilogue keeps off the stages).  More tiles than CUs with a ragged last
-    round, the minimum of four slabs, slab counts 2 and 0 mod 4, up to nine tiles per workgroup, fewer tiles than
-    CUs -- whole matrix bit-identical to the same kernel launched one workgroup per tile, and against the
-    independent generic kernel."""
-    import iree_turbine_amd as ita
-    from oracle import inputs
-
-    M, N, K = shape
-    announce(f"gemm staged walk {shape} {out_dtype}")
-    names = ita._lib.variants("gemm_f16_nt")
-    walk, plain = names.index("staged_256x256x64_w2x2_walk"), names.index("staged_256x256x64_w2x2")
-    a, b = [t.to(dev) for t in inputs.gemm_inputs(M, N, K)]
-    got = torch.ops.mi355.gemm_nt(a, b, out_dtype, walk)
-    assert torch.equal(got, torch.ops.mi355.gemm_nt(a, b, out_dtype, plain))
-    assert torch.equal(got, torch.ops.mi355.gemm_nt(a, b, out_dtype, walk))
-    ref = torch.ops.mi355.gemm_nt(a, b, out_dtype, len(names) - 1)
-    torch.testing.assert_close(got.float(), ref.float(), rtol=1e-3, atol=1e-3)
 
 
 @pytest.mark.parametrize("out_dtype", ["float16", "float32"])
@@ -289,9 +266,9 @@ def test_gemm_stream_contract(dev):
 
 @pytest.mark.parametrize("out_dtype", ["float16", "float32"])
 @pytest.mark.parametrize("shape", [(2048, 10240, 512), (10240, 2048, 256), (768, 23296, 256), (2048, 8448, 256)])
-@pytest.mark.parametrize("family", ["staged", "stream"])
+@pytest.mark.parametrize("family", ["stream"])
 def test_gemm_tail_split(dev, shape, out_dtype, family):
-    """The staged / streamed kernel with its sparse last round handed to the 128x128 kernel: a strip of tile columns
+    """The streamed kernel with its sparse last round handed to the 128x128 kernel: a strip of tile columns
     (2048 x 10240: 64 of 320 tiles), a strip of tile rows (10240 x 2048), a remainder that is neither (runs
     unsplit) and the smallest strip (one tile column after a full round of 8 x 32) -- bit-identical to the
     unsplit kernel (both accumulate K in the same order), whole matrix against the generic kernel."""
@@ -369,7 +346,7 @@ def test_gemm_output_beyond_4_gib(dev):
     rows = torch.tensor([0, 1000, 43690, 43691, M - 257, M - 1], device=dev)
     ref = a[rows].float() @ b.float().t()
     tails = [i for i, n in enumerate(names) if "tail" in n]
-    for variant in (-1, *tails, 0, 4, len(names) - 1):
+    for variant in (-1, *tails, 0, names.index("pipelined_128x128x64_w2x2"), len(names) - 1):
         announce(f"gemm {M}x{N}x{K} float16 variant={variant} (C beyond 4 GiB)")
         c = torch.ops.mi355.gemm_nt(a, b, "float16", variant)
         torch.testing.assert_close(c[rows].float(), ref, rtol=RTOL, atol=ATOL)
