@@ -32,6 +32,9 @@ _PROTOS = {
     "mi355_variant_name": (c_char_p, [c_char_p, c_int]),
     "mi355_gemm_f16_nt": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_void_p]),
     "mi355_gemm_bf16_nt": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_void_p]),
+    "mi355_gemm_nt_workspace_bytes": (c_int64, [c_int64, c_int64, c_int64]),
+    "mi355_gemm_f16_nt_ws": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_void_p, c_int64, c_void_p]),
+    "mi355_gemm_bf16_nt_ws": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_void_p, c_int64, c_void_p]),
     "mi355_flash_attn_fwd": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_float, c_int, c_int, c_void_p],

@@ -562,10 +562,14 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_staged(const half_t* 
 //                                B: part q + 1 of slab t + 3 (q = 3: part 0 of slab t + 4)
 // Reads and waits are inline assembly (with direct-to-LDS loads in flight the compiler would wait for all of them before
 // any LDS read it can see); every read's destination is tied to the wait that covers it.
+// K split (split_tiles_m > 0): the launch covers S = tiles_m / split_tiles_m partial products of K elements each, stacked
+// along M -- tile row tm belongs to split tm / split_tiles_m, reads rows (tm % split_tiles_m) * 256 .. of A and the K
+// range starting split * ksplit_bytes into every row of A and B, and writes rows tm * 256 .. of C, which the host
+// points at an [S * M, N] workspace.  ldk is the row length of A and B in elements (= K without a split).
 template <typename OutT, bool BF>
 __global__ __launch_bounds__(256) void gemm_f16_nt_stream(const half_t* __restrict__ A, const half_t* __restrict__ B,
-                                                          OutT* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n,
-                                                          int group_m) {
+                                                          OutT* __restrict__ C, int ldk, int N, int K, int tiles_m, int tiles_n,
+                                                          int group_m, int split_tiles_m, unsigned ksplit_bytes) {
   constexpr int BM = 256, BN = 256, WN = 2, WTM = 128, WTN = 128;
   constexpr int BUF = 256 * 128;                 // one operand, one slab
   constexpr int B_AT = 0, A_AT = 3 * BUF;        // three B buffers, then two A buffers
@@ -586,8 +590,9 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_stream(const half_t* __restri
   // has the parity of w
   // One descriptor per operand covers all of it (under 4 GiB, checked on the host); the tile, the slab and the row block
   // go into the scalar offset, so that moving on to the next tile changes one scalar.
-  const unsigned row_bytes = (unsigned)K * 2u;
-  const buffer_rsrc_t a_src = make_buffer(A, (unsigned)(tiles_m * BM) * row_bytes);
+  const unsigned row_bytes = (unsigned)ldk * 2u;
+  const int a_tiles = split_tiles_m > 0 ? split_tiles_m : tiles_m;  // tile rows of A itself
+  const buffer_rsrc_t a_src = make_buffer(A, (unsigned)(a_tiles * BM) * row_bytes);
   const buffer_rsrc_t b_src = make_buffer(B, (unsigned)(tiles_n * BN) * row_bytes);
   const int lrow = lane >> 3;
 #if defined(MI355_ABLATE_PLAIN_LOAD_ORDER)   // timing only: the lanes of a row fetch its chunks in ascending order (LDS then holds the wrong layout)
@@ -596,7 +601,18 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_stream(const half_t* __restri
   const unsigned g_off = (unsigned)(wave * 8 + lrow) * row_bytes + (unsigned)((lane & 7) ^ (((wave & 1) << 2) | (lrow >> 1))) * 16u;
 #endif
   const int KT = K / 64;  // even, >= 4 (checked on the host)
-  unsigned a_cur = (unsigned)(tile_m * BM) * row_bytes, b_cur = (unsigned)(tile_n * BN) * row_bytes;  // this tile's rows
+  // byte offsets of a tile's rows in A and B (with a K split: plus the split's K range)
+  auto tile_offsets = [&](int tm, int tn, unsigned& a_at, unsigned& b_at) {
+    unsigned k_at = 0;
+    while (tm >= a_tiles) {  // at most S - 1 turns, none without a split
+      tm -= a_tiles;
+      k_at += ksplit_bytes;
+    }
+    a_at = (unsigned)(tm * BM) * row_bytes + k_at;
+    b_at = (unsigned)(tn * BN) * row_bytes + k_at;
+  };
+  unsigned a_cur, b_cur;  // this tile's rows
+  tile_offsets(tile_m, tile_n, a_cur, b_cur);
   unsigned a_nxt = a_cur, b_nxt = b_cur;  // the next tile's (after the last tile: its own again; those loads are never used)
   // byte offset of slab kt + d of the walk: past this tile's end it is a slab of the next tile
   auto slab_at = [&](int s, unsigned cur, unsigned nxt) { return s < KT ? cur + (unsigned)s * 128u : nxt + (unsigned)(s - KT) * 128u; };
@@ -790,8 +806,7 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_stream(const half_t* __restri
   for (; pid < T; pid += G) {
     int nxt_m = tile_m, nxt_n = tile_n;
     if (pid + G < T) map_tile(pid + G, tiles_m, tiles_n, group_m, nxt_m, nxt_n);
-    a_nxt = (unsigned)(nxt_m * BM) * row_bytes;
-    b_nxt = (unsigned)(nxt_n * BN) * row_bytes;
+    tile_offsets(nxt_m, nxt_n, a_nxt, b_nxt);
     int kt = 0;
     MI355_SM_SLAB(0, fb0, fb1, false, true);  // everything its reads need landed before the tile began
     kt = 1;
@@ -1276,6 +1291,20 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_generic(const half_t* __restr
 
 // ---- host side ----------------------------------------------------------------------------
 
+// Sum of the S partial products of a K split (an [S * M, N] fp32 workspace, split s in rows s * M ..): four columns per
+// lane, the partials added in split order, the sum converted as the kernels' own epilogues convert theirs.
+template <typename OutT, bool BF>
+__global__ __launch_bounds__(256) void gemm_ksplit_merge(const float* __restrict__ ws, OutT* __restrict__ C, int M, int N, int ldc,
+                                                         int S) {
+  const size_t idx = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  const size_t plane = (size_t)M * N;
+  if (idx >= plane) return;
+  floatx4 acc = *reinterpret_cast<const floatx4*>(ws + idx);
+  for (int sp = 1; sp < S; sp++) acc += *reinterpret_cast<const floatx4*>(ws + sp * plane + idx);
+  const size_t r = idx / (size_t)N, c = idx - r * (size_t)N;
+  OutPack<OutT, BF>::store4(C + r * (size_t)ldc + c, acc[0], acc[1], acc[2], acc[3]);
+}
+
 struct GemmVariant {
   const char* name;
   int bm, bn, threads;
@@ -1348,25 +1377,26 @@ static int launch_persistent(const void* a, const void* b, void* c, int M, int N
   return check_launch("gemm_f16_nt_persistent", grid, block, lds_bytes);
 }
 
+// ksplit > 1: M, N, K describe the whole product; c is an [ksplit * M, N] workspace of OutT = float partial products.
 template <typename OutT, bool BF>
 static int launch_stream(const void* a, const void* b, void* c, int M, int N, int K, int ldc, hipStream_t stream,
-                         bool one_per_cu = false) {
+                         bool one_per_cu = false, int ksplit = 1) {
   auto kern = gemm_f16_nt_stream<OutT, BF>;
   constexpr int lds_bytes = 5 * 256 * 128;  // three B buffers and two A buffers of 32 KiB
   static std::atomic<uint64_t> lds_ok{0};
   if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt_stream")) return rc;
-  const int tiles_m = M / 256, tiles_n = N / 256;
+  const int tiles_m = (M / 256) * ksplit, tiles_n = N / 256, k_part = K / ksplit;
   int wgs = tiles_m * tiles_n;
   // The walk looks up to five slabs ahead and knows one tile ahead: a tile needs six slabs or more.
-  if (one_per_cu && K >= 384) {
+  if (one_per_cu && k_part >= 384) {
     // one workgroup per CU walking tiles pid, pid + grid, ...; a multiple of 8 keeps a workgroup's tiles on its XCD
     int g = cu_count() & ~7;
     if (g < 8) g = 8;
     if (wgs > g) wgs = g;
   }
   dim3 grid(wgs), block(256);
-  hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, M, ldc, K, tiles_m,
-                     tiles_n, 4);
+  hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, K, ldc, k_part, tiles_m,
+                     tiles_n, 4, ksplit > 1 ? M / 256 : 0, ksplit > 1 ? (unsigned)k_part * 2u : 0u);
   return check_launch("gemm_f16_nt_stream", grid, block, lds_bytes);
 }
 
@@ -1388,22 +1418,74 @@ static bool tail_split(int M, int N, int& main_m, int& main_n) {
   return true;
 }
 
-template <typename OutT, bool BF>
-static int launch_split(const void* a, const void* b, void* c, int M, int N, int K, hipStream_t stream) {
-  auto main_part = [&](int m, int n) { return launch_stream<OutT, BF>(a, b, c, m, n, K, N, stream, true); };  // one workgroup per CU
-  int mm, mn;
-  if (!tail_split(M, N, mm, mn)) return main_part(M, N);
-  int rc = main_part(mm, mn);
-  if (rc) return rc;
-  const half_t* ah = (const half_t*)a;
-  const half_t* bh = (const half_t*)b;
-  OutT* ch = (OutT*)c;
-  if (mn < N) return launch_tiled<128, 128, 2, 2, OutT, 1, BF>(ah, bh + (size_t)mn * K, ch + mn, M, N - mn, K, N, stream);
-  return launch_tiled<128, 128, 2, 2, OutT, 1, BF>(ah + (size_t)mm * K, bh, ch + (size_t)mm * N, M - mm, N, K, N, stream);
+// K split: a product with too few 256x256 tiles for the 256 CUs is cut into S K ranges, every (tile, range) pair a unit
+// of the streamed kernel's walk, fp32 partial products in a caller-provided workspace, one merge launch behind it.
+// S doubles while the units still fit one round of the chip and a range keeps 1024 or more of K in whole slab pairs.
+// The partial products cost a write and a read of 256 KiB per unit, so short K only splits when the units are few
+// (measured, one tile's time in us for K = 4096 / 8192 against the 128x128 kernel: 64 tiles 47.8 / 70.1 against
+// 45.5 / 82.7, 16 tiles 35.1 / 36.4 against 39.4 / 68.8, 128 tiles in two ranges 70.8 / 115.6 against 72.2 / 135.3).
+static int ksplit_factor(long long tiles, int K) {
+  if (K < 4096 || (K < 6144 && tiles > 32)) return 1;
+  int s = 1;
+  while (s < 8 && 2ll * s * tiles <= 256 && (K / (2 * s)) % 128 == 0 && K / (2 * s) >= 1024) s *= 2;
+  return s;
 }
 
 template <typename OutT, bool BF>
-static int launch_variant(int variant, const void* a, const void* b, void* c, int M, int N, int K, hipStream_t stream) {
+static int launch_ksplit(const half_t* a, const half_t* b, OutT* c, int M, int N, int K, int ldc, int S, float* ws, hipStream_t stream) {
+  if (int rc = launch_stream<float, BF>(a, b, ws, M, N, K, N, stream, true, S)) return rc;
+  const long long lanes = (long long)M * N / 4;
+  dim3 grid((unsigned)((lanes + 255) / 256)), block(256);
+  hipLaunchKernelGGL((gemm_ksplit_merge<OutT, BF>), grid, block, 0, stream, (const float*)ws, c, M, N, ldc, S);
+  return check_launch("gemm_ksplit_merge", grid, block, 0);
+}
+
+// The sub-problem that would take a K split under the automatic choice, if any: the strip a sparse last round is cut
+// into, or the whole product when it has fewer than 128 tiles.  Returns S (1: none) and the sub-problem's M and N.
+static int ksplit_plan(int M, int N, int K, int& sub_m, int& sub_n) {
+  sub_m = M;
+  sub_n = N;
+  if (M % 256 || N % 256) return 1;
+  const long long t256 = (long long)(M / 256) * (N / 256);
+  int mm, mn;
+  if (t256 > 128) {
+    if (!tail_split(M, N, mm, mn)) return 1;
+    if (mn < N) sub_n = N - mn;
+    else sub_m = M - mm;
+    return ksplit_factor((long long)(sub_m / 256) * (sub_n / 256), K);
+  }
+  return t256 >= 1 ? ksplit_factor(t256, K) : 1;
+}
+
+template <typename OutT, bool BF>
+static int launch_split(const void* a, const void* b, void* c, int M, int N, int K, hipStream_t stream, float* ws = nullptr,
+                        size_t ws_bytes = 0) {
+  auto main_part = [&](int m, int n) { return launch_stream<OutT, BF>(a, b, c, m, n, K, N, stream, true); };  // one workgroup per CU
+  const half_t* ah = (const half_t*)a;
+  const half_t* bh = (const half_t*)b;
+  OutT* ch = (OutT*)c;
+  int mm, mn;
+  if (!tail_split(M, N, mm, mn)) {
+    int sm, sn;
+    const int S = ws ? ksplit_plan(M, N, K, sm, sn) : 1;
+    if (S > 1 && ws_bytes >= (size_t)S * M * N * 4) return launch_ksplit<OutT, BF>(ah, bh, ch, M, N, K, N, S, ws, stream);
+    return main_part(M, N);
+  }
+  int rc = main_part(mm, mn);
+  if (rc) return rc;
+  // the strip: K split over 256x256 tiles when the caller brought a workspace, else the 128x128 kernel
+  const int sm = mn < N ? M : M - mm, sn = mn < N ? N - mn : N;
+  const half_t* sa = mn < N ? ah : ah + (size_t)mm * K;
+  const half_t* sb = mn < N ? bh + (size_t)mn * K : bh;
+  OutT* sc = mn < N ? ch + mn : ch + (size_t)mm * N;
+  const int S = ws ? ksplit_factor((long long)(sm / 256) * (sn / 256), K) : 1;
+  if (S > 1 && ws_bytes >= (size_t)S * sm * sn * 4) return launch_ksplit<OutT, BF>(sa, sb, sc, sm, sn, K, N, S, ws, stream);
+  return launch_tiled<128, 128, 2, 2, OutT, 1, BF>(sa, sb, sc, sm, sn, K, N, stream);
+}
+
+template <typename OutT, bool BF>
+static int launch_variant(int variant, const void* a, const void* b, void* c, int M, int N, int K, hipStream_t stream,
+                          float* ws = nullptr, size_t ws_bytes = 0) {
   switch (variant) {
     case V_PERSISTENT: return launch_persistent<256, 256, 2, 4, OutT, BF>(a, b, c, M, N, K, stream);
     case V_PIPELINED_128: return launch_tiled<128, 128, 2, 2, OutT, 1, BF>(a, b, c, M, N, K, N, stream);
@@ -1425,7 +1507,7 @@ static int launch_variant(int variant, const void* a, const void* b, void* c, in
       return 0;
     }
     case V_STREAM: return launch_stream<OutT, BF>(a, b, c, M, N, K, N, stream);
-    case V_STREAM_TAIL: return launch_split<OutT, BF>(a, b, c, M, N, K, stream);
+    case V_STREAM_TAIL: return launch_split<OutT, BF>(a, b, c, M, N, K, stream, ws, ws_bytes);
     case V_STREAM_WALK: return launch_stream<OutT, BF>(a, b, c, M, N, K, N, stream, true);
     default: {
       dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
@@ -1442,7 +1524,7 @@ using namespace mi355;
 
 // fp16 and bf16 share everything but the kernel instantiation; `bf` also names the 16-bit output format
 static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int out_dtype, int variant,
-                         void* stream) {
+                         void* stream, void* workspace = nullptr, int64_t workspace_bytes = 0) {
   if (!a || !b || !c) return fail(-MI355_E_NULL, "gemm_f16_nt: null pointer (a=%p b=%p c=%p)", a, b, c);
   if (M <= 0 || N <= 0 || K <= 0 || M > (1 << 30) || N > (1 << 30) || K > (1 << 27))
     return fail(-MI355_E_SHAPE, "gemm_f16_nt: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
@@ -1475,6 +1557,12 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
     const bool full_rounds = t256 * 100 >= rounds * 256 * 85;
     if (fits(V_SKINNY) && N >= 2048 && K >= 512) variant = V_SKINNY;  // decode-shaped: stream the weights once
     else if (K < 1024 && t256 <= 2048 && fits(V_PERSISTENT) && t256 >= 128 && full_rounds) variant = V_PERSISTENT;
+    else if (t256 <= 128 && fits(V_STREAM_TAIL) && workspace && [&] {  // too few tiles for the chip, and a workspace to split K into
+               int sm, sn;
+               const int S = ksplit_plan((int)M, (int)N, (int)K, sm, sn);
+               return S > 1 && workspace_bytes >= (int64_t)S * sm * sn * 4;
+             }())
+      variant = V_STREAM_TAIL;
     else if (fits(V_STREAM_TAIL) && t256 >= 128) variant = V_STREAM_TAIL;
     else if (fits(V_PERSISTENT) && t256 >= 128 && full_rounds) variant = V_PERSISTENT;
     else if (fits(V_PIPELINED_128)) variant = V_PIPELINED_128;
@@ -1490,12 +1578,25 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
     return fail(-MI355_E_ALIGN, "gemm_f16_nt: a and b must be 16-byte aligned when K %% 8 == 0");
   }
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  float* ws = static_cast<float*>(workspace);
+  const size_t wsb = workspace_bytes > 0 ? (size_t)workspace_bytes : 0;
+  if (ws && !aligned16(ws)) return fail(-MI355_E_ALIGN, "gemm_f16_nt: workspace must be 16-byte aligned");
   if (bf) {
-    if (out_dtype == MI355_F32) return launch_variant<float, true>(variant, a, b, c, (int)M, (int)N, (int)K, s);
-    return launch_variant<half_t, true>(variant, a, b, c, (int)M, (int)N, (int)K, s);
+    if (out_dtype == MI355_F32) return launch_variant<float, true>(variant, a, b, c, (int)M, (int)N, (int)K, s, ws, wsb);
+    return launch_variant<half_t, true>(variant, a, b, c, (int)M, (int)N, (int)K, s, ws, wsb);
   }
-  if (out_dtype == MI355_F32) return launch_variant<float, false>(variant, a, b, c, (int)M, (int)N, (int)K, s);
-  return launch_variant<half_t, false>(variant, a, b, c, (int)M, (int)N, (int)K, s);
+  if (out_dtype == MI355_F32) return launch_variant<float, false>(variant, a, b, c, (int)M, (int)N, (int)K, s, ws, wsb);
+  return launch_variant<half_t, false>(variant, a, b, c, (int)M, (int)N, (int)K, s, ws, wsb);
+}
+
+// Bytes of workspace with which the automatic choice would split K for this shape (0: it would not).
+static int64_t gemm_nt_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0 || M > (1 << 30) || N > (1 << 30) || K > (1 << 21) || K < 256 || K % 128 != 0) return 0;
+  if (M * K * 2 >= (1ll << 32) || N * K * 2 >= (1ll << 32)) return 0;  // the streamed kernel's one descriptor per operand
+  if (M <= 64 && N % 32 == 0 && N >= 2048 && K >= 512) return 0;        // the weight-streaming kernel's shapes
+  int sm, sn;
+  const int S = ksplit_plan((int)M, (int)N, (int)K, sm, sn);
+  return S > 1 ? (int64_t)S * sm * sn * 4 : 0;
 }
 
 extern "C" int mi355_gemm_f16_nt(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int out_dtype,
@@ -1506,4 +1607,16 @@ extern "C" int mi355_gemm_f16_nt(const void* a, const void* b, void* c, int64_t 
 extern "C" int mi355_gemm_bf16_nt(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int out_dtype,
                                   int variant, void* stream) {
   return gemm_nt_entry(true, a, b, c, M, N, K, out_dtype, variant, stream);
+}
+
+extern "C" int64_t mi355_gemm_nt_workspace_bytes(int64_t M, int64_t N, int64_t K) { return gemm_nt_workspace_bytes(M, N, K); }
+
+extern "C" int mi355_gemm_f16_nt_ws(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int out_dtype,
+                                    int variant, void* workspace, int64_t workspace_bytes, void* stream) {
+  return gemm_nt_entry(false, a, b, c, M, N, K, out_dtype, variant, stream, workspace, workspace_bytes);
+}
+
+extern "C" int mi355_gemm_bf16_nt_ws(const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int out_dtype,
+                                     int variant, void* workspace, int64_t workspace_bytes, void* stream) {
+  return gemm_nt_entry(true, a, b, c, M, N, K, out_dtype, variant, stream, workspace, workspace_bytes);
 }

@@ -75,9 +75,19 @@ def gemm_nt_out(a: Tensor, b: Tensor, c: Tensor, variant: int = -1) -> Tensor:
             b_k[:N, :K] = b
         if (Mp, Np) != (M, N):
             c_k = torch.empty((Mp, Np), dtype=c.dtype, device=dev)
+    # A shape with too few 256x256 tiles for the chip (or with a sparse last round of them) splits K when it gets a
+    # workspace for the fp32 partial products; the library says how large.  torch's caching allocator makes the
+    # allocation cheap and safe under graph capture.
+    ws_bytes = lib.mi355_gemm_nt_workspace_bytes(c_k.shape[0], c_k.shape[1], a_k.shape[1]) if variant < 0 else 0
     with torch.cuda.device(dev):
-        rc = entry(a_k.data_ptr(), b_k.data_ptr(), c_k.data_ptr(), c_k.shape[0], c_k.shape[1], a_k.shape[1],
-                   _lib.dtype_code(c.dtype), variant, _lib.current_stream_ptr(dev))
+        if ws_bytes > 0:
+            ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=dev)
+            entry_ws = lib.mi355_gemm_bf16_nt_ws if a.dtype == torch.bfloat16 else lib.mi355_gemm_f16_nt_ws
+            rc = entry_ws(a_k.data_ptr(), b_k.data_ptr(), c_k.data_ptr(), c_k.shape[0], c_k.shape[1], a_k.shape[1],
+                          _lib.dtype_code(c.dtype), variant, ws.data_ptr(), ws_bytes, _lib.current_stream_ptr(dev))
+        else:
+            rc = entry(a_k.data_ptr(), b_k.data_ptr(), c_k.data_ptr(), c_k.shape[0], c_k.shape[1], a_k.shape[1],
+                       _lib.dtype_code(c.dtype), variant, _lib.current_stream_ptr(dev))
     _lib.check(rc, f"gemm_nt M={M} N={N} K={K} in={a.dtype} out={c.dtype} variant={variant}")
     if c_k is not c:
         c.copy_(c_k[:M, :N])

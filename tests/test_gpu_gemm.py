@@ -479,3 +479,66 @@ def test_gemm_skinny_contract(dev):
         torch.ops.mi355.gemm_nt(a[:8], b[:48], "float32", sk)  # N = 48 is not whole 32-row tiles
     with pytest.raises(ValueError):
         torch.ops.mi355.gemm_nt(a[:8, :32].contiguous(), b[:, :32].contiguous(), "float32", sk)  # K = 32 < one segment
+
+
+@pytest.mark.parametrize("out_dtype", ["float16", "float32"])
+@pytest.mark.parametrize("shape", [(2048, 10240, 8192), (10240, 2048, 6144), (2048, 4096, 8192), (512, 2048, 8192), (1024, 1024, 4096), (256, 2048, 8192)])
+def test_gemm_k_split_with_workspace(dev, shape, out_dtype):
+    """The workspace entry point through the C ABI: a strip of tile columns (2048 x 10240: the last 64 of 320 tiles, four
+    K ranges), a strip of tile rows (four ranges of 1536), and whole products of 128, 16, 16 and 8 tiles (two, eight,
+    four and eight ranges) -- the whole matrix against the plain entry point (same products, other summation order), sampled rows
+    against an fp32 product; a workspace one byte short or absent runs exactly as the plain entry point does."""
+    from iree_turbine_amd import _lib
+    from oracle import inputs
+
+    M, N, K = shape
+    announce(f"gemm K split {shape} {out_dtype}")
+    lib = _lib.load()
+    a, b = [t.to(dev) for t in inputs.gemm_inputs(M, N, K)]
+    dt = getattr(torch, out_dtype)
+    need = lib.mi355_gemm_nt_workspace_bytes(M, N, K)
+    assert need > 0 and need % 1024 == 0
+    ws = torch.empty(need // 4, dtype=torch.float32, device=dev)
+    stream = _lib.current_stream_ptr(dev)
+
+    def run(ws_ptr, ws_bytes):
+        c = torch.full((M, N), float("nan"), dtype=dt, device=dev)
+        rc = lib.mi355_gemm_f16_nt_ws(a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K, _lib.dtype_code(dt), -1, ws_ptr, ws_bytes, stream)
+        _lib.check(rc, "gemm_f16_nt_ws")
+        return c
+
+    plain = torch.empty((M, N), dtype=dt, device=dev)
+    _lib.check(lib.mi355_gemm_f16_nt(a.data_ptr(), b.data_ptr(), plain.data_ptr(), M, N, K, _lib.dtype_code(dt), -1, stream), "gemm_f16_nt")
+    split = run(ws.data_ptr(), need)
+    assert torch.equal(split, run(ws.data_ptr(), need))  # launches repeat bit for bit (the workspace is scratch)
+    assert not torch.equal(split, plain) or out_dtype == "float16"  # another summation order: fp32 sums differ in the last bits
+    tol = dict(rtol=1e-4, atol=1e-4) if out_dtype == "float32" else dict(rtol=2e-3, atol=1e-3)
+    torch.testing.assert_close(split.float(), plain.float(), **tol)
+    rows = torch.tensor([0, 255, M - 256, M - 1], device=dev)
+    exact = a[rows].float() @ b.float().t()
+    torch.testing.assert_close(split[rows].float(), exact, rtol=RTOL, atol=ATOL)
+    assert torch.equal(run(ws.data_ptr(), need - 1), plain)
+    assert torch.equal(run(None, 0), plain)
+
+
+def test_gemm_k_split_through_the_op(dev):
+    """torch.ops.mi355.gemm_nt allocates the workspace the library asks for: a product of 16 tiles (bf16 operands) and
+    the benchmark shape with the sparse last round against the oracle's rows; shapes that take no split ask for none."""
+    from iree_turbine_amd import _lib
+    from oracle import inputs
+
+    lib = _lib.load()
+    assert lib.mi355_gemm_nt_workspace_bytes(8192, 8192, 8192) == 0
+    assert lib.mi355_gemm_nt_workspace_bytes(4096, 4096, 4096) == 0
+    assert lib.mi355_gemm_nt_workspace_bytes(16, 8192, 8192) == 0
+    assert lib.mi355_gemm_nt_workspace_bytes(2048, 10240, 4096) == 0  # K too short for 64 tiles' partial products to pay
+    assert lib.mi355_gemm_nt_workspace_bytes(2048, 4096, 8192) == 2 * 2048 * 4096 * 4
+    assert lib.mi355_gemm_nt_workspace_bytes(2048, 10240, 8192) == 4 * 2048 * 2048 * 4
+    for (M, N, K), dtype in (((512, 2048, 8192), torch.bfloat16), ((2048, 10240, 8192), torch.float16)):
+        announce(f"gemm K split through the op {(M, N, K)} {dtype}")
+        a, b = [t.to(dev) for t in inputs.gemm_inputs(M, N, K, dtype=dtype)]
+        c = torch.ops.mi355.gemm_nt(a, b, "float32", -1)
+        rows = torch.tensor([0, 300, M - 1], device=dev)
+        torch.testing.assert_close(c[rows], a[rows].float() @ b.float().t(), rtol=1e-3, atol=1e-3)
+        cols = torch.tensor([0, N - 2048, N - 1], device=dev)
+        torch.testing.assert_close(c[:, cols], a.float() @ b[cols].float().t(), rtol=1e-3, atol=1e-3)
