@@ -50,11 +50,12 @@ MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
     "gemm_8192": 1.754e9,              # 1545 MiB read + 128 MiB written: each of the 8 XCD L2s fetches its own copy of
                                        # the panels its 4x8 block of output tiles needs (12 panels x 4 MiB x 4 rounds x 8)
     "gemm_4096": 2.438e8,
-    "gemm_2048x10240x8192": 6.563e8,
+    "gemm_2048x10240x8192": 6.973e8,   # of which 128 MiB are the strip's fp32 partial products, written and read once
     "gemm_2048x57344x8192": 3.062e9,
     "gemm_1024_f32out": 1.684e7,
     "gemm_bf16_8192": 1.754e9,
     "gemm_16x8192x8192": 1.366e8,
+    "gemm_1024x8192x8192": 3.644e8,
     "fa_causal": 3.870e8,
     "fa_noncausal": 2.686e8,
     "decode": 1.177e9,
@@ -475,6 +476,8 @@ WORKLOADS = {
     "gemm_1024_f32out": wl_gemm(1024, 1024, 1024, "float32"),
     "gemm_bf16_8192": wl_gemm(8192, 8192, 8192, "bfloat16", torch.bfloat16),
     "gemm_16x8192x8192": wl_gemm(16, 8192, 8192),
+    "gemm_1024x8192x8192": wl_gemm(1024, 8192, 8192),  # 128 tiles: K split in two through the workspace entry point
+    "gemm_512x8192x8192": wl_gemm(512, 8192, 8192),    # 64 tiles: four K ranges
     "fa_causal": wl_attention(True),
     "fa_noncausal": wl_attention(False),
     "decode": wl_decode(),
@@ -507,6 +510,9 @@ def wl_library_gemm(M, N, K):
 
 CALIBRATION = {  # not part of the path: run only when named with --workload
     "library_gemm_8192": wl_library_gemm(8192, 8192, 8192),
+    "library_gemm_2048x10240x8192": wl_library_gemm(2048, 10240, 8192),
+    "library_gemm_1024x8192x8192": wl_library_gemm(1024, 8192, 8192),
+    "library_gemm_512x8192x8192": wl_library_gemm(512, 8192, 8192),
     "copy_1GiB": wl_copy(),
     "mfma_f16_regloop_zeros": wl_mfma_regloop("f16", "zeros"),
     "mfma_f16_regloop_benchmark": wl_mfma_regloop("f16", "benchmark"),
