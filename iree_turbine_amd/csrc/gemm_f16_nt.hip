@@ -26,6 +26,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "gemm_tiles.hpp"
 
 namespace mi355 {
 
@@ -47,19 +48,6 @@ template <bool BF> struct OutPack<half_t, BF> {
   }
   static __device__ __forceinline__ void store1(half_t* p, float a) { *p = cvt16<BF>(a); }
 };
-
-__device__ __forceinline__ void map_tile(int pid, int tiles_m, int tiles_n, int group_m, int& tm, int& tn) {
-  const int T = tiles_m * tiles_n;
-  const int xcd = pid & 7, loc = pid >> 3;
-  const int per = T >> 3, rem = T & 7;
-  const int id = xcd * per + (xcd < rem ? xcd : rem) + loc;
-  const int width = group_m * tiles_n;
-  const int grp = id / width, within = id - grp * width;
-  const int first_m = grp * group_m;
-  const int gsz = (tiles_m - first_m) < group_m ? (tiles_m - first_m) : group_m;
-  tm = first_m + within % gsz;
-  tn = within / gsz;
-}
 
 // Software-pipelined two-stage kernel: a BM x BN output tile per workgroup, slabs copied global -> LDS with
 // direct-to-LDS loads into a two-stage ring, 32x32x16 MFMAs.  The k-loop is

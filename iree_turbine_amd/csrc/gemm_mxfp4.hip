@@ -18,37 +18,9 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "gemm_tiles.hpp"
 
 namespace mi355 {
-
-__device__ __forceinline__ void map_tile_mx(int pid, int tiles_m, int tiles_n, int group_m, int& tm, int& tn) {
-  const int T = tiles_m * tiles_n;
-  const int xcd = pid & 7, loc = pid >> 3;
-  const int per = T >> 3, rem = T & 7;
-  const int id = xcd * per + (xcd < rem ? xcd : rem) + loc;
-  const int width = group_m * tiles_n;
-  const int grp = id / width, within = id - grp * width;
-  const int first_m = grp * group_m;
-  const int gsz = (tiles_m - first_m) < group_m ? (tiles_m - first_m) : group_m;
-  tm = first_m + within % gsz;
-  tn = within / gsz;
-}
-
-template <typename OutT> struct MxOut;
-template <> struct MxOut<float> {
-  static __device__ __forceinline__ void store4(float* p, float a, float b, float c, float d) {
-    floatx4 v = {a, b, c, d};
-    *reinterpret_cast<floatx4*>(p) = v;
-  }
-  static __device__ __forceinline__ void store1(float* p, float a) { *p = a; }
-};
-template <> struct MxOut<unsigned short> {  // bf16 bits
-  static __device__ __forceinline__ void store4(unsigned short* p, float a, float b, float c, float d) {
-    ushortx4 v = {f32_to_bf16_rne(a), f32_to_bf16_rne(b), f32_to_bf16_rne(c), f32_to_bf16_rne(d)};
-    *reinterpret_cast<ushortx4*>(p) = v;
-  }
-  static __device__ __forceinline__ void store1(unsigned short* p, float a) { *p = f32_to_bf16_rne(a); }
-};
 
 // byte SEL of sa / sb scales the lane's block of a / b
 template <int SEL>
@@ -79,7 +51,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm = wave / WN, wn = wave % WN;
   int tile_m, tile_n;
-  map_tile_mx(blockIdx.x, tiles_m, tiles_n, group_m, tile_m, tile_n);
+  map_tile(blockIdx.x, tiles_m, tiles_n, group_m, tile_m, tile_n);
 
   const int Kb = K >> 1;   // bytes per row of codes
   const int Ksc = K >> 5;  // scale bytes per row
@@ -365,7 +337,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_persistent(const uint8
   const unsigned sc_lane_off = (unsigned)lane * (unsigned)Ksc;
 
   auto tile_src = [&](int pid, buffer_rsrc_t& a_src, buffer_rsrc_t& b_src, buffer_rsrc_t& sc_src, int& tile_m, int& tile_n) {
-    map_tile_mx(pid, tiles_m, tiles_n, group_m, tile_m, tile_n);
+    map_tile(pid, tiles_m, tiles_n, group_m, tile_m, tile_n);
     a_src = make_buffer(A + (size_t)(tile_m * BM + wave * 8) * Kb, panel_a);
     b_src = make_buffer(B + (size_t)(tile_n * BN + wave * 8) * Kb, panel_b);
     const uint8_t* sp = sc_is_a ? As + (size_t)(tile_m * BM + wave * 64) * Ksc : Bs + (size_t)(tile_n * BN + wave * 64 - BM) * Ksc;
@@ -828,7 +800,7 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_staged(const uint8_t* __restri
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm = wave / WN, wn = wave % WN;
   int tile_m, tile_n;
-  map_tile_mx(blockIdx.x, tiles_m, tiles_n, group_m, tile_m, tile_n);
+  map_tile(blockIdx.x, tiles_m, tiles_n, group_m, tile_m, tile_n);
 
   const unsigned row_bytes = (unsigned)K >> 1;  // codes
   const unsigned sc_bytes = (unsigned)K >> 5;   // scale bytes per row
@@ -1113,7 +1085,7 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_stream(const uint8_t* __restri
   const int T = tiles_m * tiles_n, G = (int)gridDim.x;
   int pid = blockIdx.x;
   int tile_m, tile_n;
-  map_tile_mx(pid, tiles_m, tiles_n, group_m, tile_m, tile_n);
+  map_tile(pid, tiles_m, tiles_n, group_m, tile_m, tile_n);
 
   // One descriptor per array (each under 4 GiB, checked on the host); tile, slab and row block go into the scalar offset.
   const unsigned row_bytes = (unsigned)K / 2u, SK = (unsigned)K / 32u;
@@ -1390,7 +1362,7 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_stream(const uint8_t* __restri
 
   for (; pid < T; pid += G) {
     int nxt_m = tile_m, nxt_n = tile_n;
-    if (pid + G < T) map_tile_mx(pid + G, tiles_m, tiles_n, group_m, nxt_m, nxt_n);
+    if (pid + G < T) map_tile(pid + G, tiles_m, tiles_n, group_m, nxt_m, nxt_n);
     a_nxt = (unsigned)(nxt_m * BM) * row_bytes;
     b_nxt = (unsigned)(nxt_n * BN) * row_bytes;
     sa_nxt = (unsigned)(nxt_m * BM) * SK;
@@ -1408,65 +1380,11 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_stream(const uint8_t* __restri
       MI355_SM_SLAB(1, fb1, fb0, sb1, sb0, false, 15);
       kt--;
     }
-    // ---- epilogue ----
-    // The MFMAs are inline assembly, so the compiler does not know that the accumulators were written just now: the
-    // wait states an MFMA result needs before another instruction may read it are spelled out, and every accumulator is
-    // tied to a statement behind them so that no read of it can be scheduled earlier.
-    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-#pragma unroll
-    for (int i = 0; i < 8; i++)
-      asm volatile("" : "+a"(acc[i][0]), "+a"(acc[i][1]), "+a"(acc[i][2]), "+a"(acc[i][3]), "+a"(acc[i][4]), "+a"(acc[i][5]),
-                        "+a"(acc[i][6]), "+a"(acc[i][7]));
-    // lane holds, for m = 16 j + (l & 15): n = 16 i + 4 (l >> 4) + r, r < 4.  The addresses come from a lane id the
-    // compiler cannot see through, so that none of them is computed ahead of the K loop and kept across it.
-    const int le = opaque_lane_id();
-    const int r16e = le & 15, cqe = le >> 4;
-    if constexpr (sizeof(OutT) == 2) {
-      // bf16 results go through LDS, 16 rows x 64 columns (2 KiB) per pass in a wave-private region: 8-byte writes of 4
-      // consecutive n (chunk slot c ^ ((m >> 1) & 7) of the 128-byte row), whole rows read back 16 bytes per lane and
-      // stored as full cache lines.  LDS operations of a wave execute in order, so the passes need no waits between
-      // them.  The next tile's slabs are landing in LDS meanwhile; free at this point is block 3 of A buffer 1 (rows
-      // 96..127 of either half: twice 4 KiB), which the next loads reach only after the barrier below.  Inline
-      // assembly like the K loop's LDS accesses: direct-to-LDS loads are in flight.
-      const unsigned ep = lds0 + (unsigned)(A_AT + ABUF + (wave < 2 ? 12 * 1024 + wave * 2048 : 28 * 1024 + (wave - 2) * 2048));
-      const int er = le >> 3, ec = le & 7, sw = (r16e >> 1) & 7;
-      // write: row r16e, chunk (2 (i & 3) + (cqe >> 1)) ^ sw, 8-byte half cqe & 1; the i term is an XOR of the address
-      const unsigned wa = ep + (unsigned)(r16e * 128 + ((((cqe >> 1) ^ (sw & 1)) | (sw & 6)) * 16) + 8 * (cqe & 1));
-      // read: row 8 it + er, chunk ec ^ ((row >> 1) & 7) = (ec ^ (er >> 1)) ^ 4 it
-      const unsigned ra = ep + (unsigned)(er * 128 + ((ec ^ (er >> 1)) * 16));
-      OutT* cbase = C + (size_t)(tile_m * BM + wm * WTM + er) * N + tile_n * BN + wn * WTN + ec * 8;
-#pragma unroll
-      for (int j = 0; j < 8; j++) {
-#pragma unroll
-        for (int ih = 0; ih < 2; ih++) {
-#pragma unroll
-          for (int ii = 0; ii < 4; ii++) {
-            const int i = ih * 4 + ii;
-            ushortx4 v = {f32_to_bf16_rne(acc[i][j][0]), f32_to_bf16_rne(acc[i][j][1]), f32_to_bf16_rne(acc[i][j][2]),
-                          f32_to_bf16_rne(acc[i][j][3])};
-            asm volatile("ds_write_b64 %0, %1" ::"v"(wa ^ (unsigned)(32 * ii)), "v"(v) : "memory");
-          }
-          half8 rv[2];
-          asm volatile("ds_read_b128 %0, %1" : "=v"(rv[0]) : "v"(ra));
-          asm volatile("ds_read_b128 %0, %1 offset:1024" : "=v"(rv[1]) : "v"(ra ^ 64u));
-          asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(rv[0]), "+v"(rv[1]));
-#pragma unroll
-          for (int it = 0; it < 2; it++)  // one store instruction each: the next tile's first waits count past these 32
-            store_global_16B(cbase + (size_t)(j * 16 + it * 8) * N + ih * 64, rv[it]);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      }
-    } else {
-      OutT* crow = C + (size_t)(tile_m * BM + wm * WTM + r16e) * N + tile_n * BN + wn * WTN + 4 * cqe;
-#pragma unroll
-      for (int j = 0; j < 8; j++) {
-#pragma unroll
-        for (int i = 0; i < 8; i++)
-          MxOut<OutT>::store4(crow + (size_t)(j * 16) * N + i * 16, acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // 64 stores: more than a wait can count past
-    }
+    // ---- epilogue ---- (gemm_tiles.hpp).  16-bit results are staged through LDS in a wave-private 2 KiB region while
+    // the next tile's slabs are landing; free at this point is block 3 of A buffer 1 (rows 96..127 of either half: twice
+    // 4 KiB), which the next loads reach only after the barrier below.
+    mx_stream_epilogue<false>(acc, 1.f, C + (size_t)(tile_m * BM + wm * WTM) * N + tile_n * BN + wn * WTN, N,
+                              lds0 + (unsigned)(A_AT + ABUF + (wave < 2 ? 12 * 1024 + wave * 2048 : 28 * 1024 + (wave - 2) * 2048)));
     a_cur = a_nxt;
     b_cur = b_nxt;
     sa_cur = sa_nxt;

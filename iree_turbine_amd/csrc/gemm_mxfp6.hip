@@ -11,18 +11,11 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "gemm_tiles.hpp"
 
 namespace mi355 {
 
 namespace {
-
-template <typename OutT> struct Out6;
-template <> struct Out6<float> {
-  static __device__ __forceinline__ void store1(float* p, float a) { *p = a; }
-};
-template <> struct Out6<unsigned short> {  // bf16 bits
-  static __device__ __forceinline__ void store1(unsigned short* p, float a) { *p = f32_to_bf16_rne(a); }
-};
 
 // FMT: the instruction's format code, 2 = E2M3, 3 = E3M2
 template <int FMT>
@@ -34,21 +27,6 @@ __device__ __forceinline__ floatx16 mfma_fp6_32x32x64(intx8 a, int sa, intx8 b, 
 template <int FMT, int SEL>
 __device__ __forceinline__ floatx16 mfma_fp6_sel(intx8 a, int sa, intx8 b, int sb, floatx16 c) {
   return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, FMT, FMT, SEL, sa, SEL, sb);
-}
-
-// workgroup -> tile: eight consecutive ids run on eight XCDs, so each XCD gets a contiguous run of tiles, walked
-// in groups of group_m tile rows
-__device__ __forceinline__ void map_tile6(int pid, int tiles_m, int tiles_n, int group_m, int& tm, int& tn) {
-  const int T = tiles_m * tiles_n;
-  const int xcd = pid & 7, loc = pid >> 3;
-  const int per = T >> 3, rem = T & 7;
-  const int id = xcd * per + (xcd < rem ? xcd : rem) + loc;
-  const int width = group_m * tiles_n;
-  const int grp = id / width, within = id - grp * width;
-  const int first_m = grp * group_m;
-  const int gsz = (tiles_m - first_m) < group_m ? (tiles_m - first_m) : group_m;
-  tm = first_m + within % gsz;
-  tn = within / gsz;
 }
 
 // one 24-byte block (8-byte aligned) as an MFMA operand
@@ -96,7 +74,7 @@ __global__ __launch_bounds__(256) void gemm_mxfp6_generic(const uint8_t* __restr
 #pragma unroll
     for (int r = 0; r < 16; r++) {
       const int nn = nb + 8 * (r >> 2) + 4 * h + (r & 3);
-      if (nn < N) Out6<OutT>::store1(C + (size_t)m * N + nn, acc[r]);
+      if (nn < N) MxOut<OutT>::store1(C + (size_t)m * N + nn, acc[r]);
     }
   }
 }
@@ -136,7 +114,7 @@ __global__ __launch_bounds__(256) void gemm_mxfp6_staged(const uint8_t* __restri
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WN, wn = wave % WN;
   int tile_m, tile_n;
-  map_tile6(blockIdx.x, tiles_m, tiles_n, group_m, tile_m, tile_n);
+  map_tile(blockIdx.x, tiles_m, tiles_n, group_m, tile_m, tile_n);
 
   const unsigned row_bytes = ((unsigned)K >> 2) * 3u;
   const unsigned sc_bytes = (unsigned)K >> 5;
