@@ -1054,17 +1054,18 @@ __global__ __launch_bounds__(256) void gemm_mxfp4_staged(const uint8_t* __restri
 // bytes = 256 codes = 8 scale blocks).  Whole 128-byte rows go global -> LDS directly, about two slabs ahead; the B
 // fragments of a slab are held in registers (read from LDS during the first quarter of the slab before), the A rows
 // are streamed fragment by fragment, each feeding 8 MFMAs 16x16x128 (a lane's 16 bytes are one scale block: lane l
-// supplies row l & 15, block 4 kh + (l >> 4) of the slab).  One workgroup per CU walks its tiles as one slab sequence.
+// supplies row l & 15, block 2 (l >> 4) + kh of the slab in k half kh, so that its two scale bytes of a slab are
+// neighbours).  One workgroup per CU walks its tiles as one slab sequence.
 // LDS (160 KiB): B in a ring of five 16 KiB half buffers (U = rows 0..63, V = rows 64..127 of both 128-row halves; a
 // half is loaded over two intervals, read seven or six intervals later and free one interval after that), A in two 32
 // KiB buffers freed block by block, and 16 KiB for the scales.
 // Scales are staged through LDS in groups of two slabs: 16 bytes per row, one lane per row, 8 KiB per group (A rows,
 // then B rows), two buffers; a group is loaded in the first two steps of an even slab and first read 19 steps later.
-// A lane fetches its scale with a one-byte LDS read, which lands in bits 0..7 of a register as the MFMA wants it: the A
-// scale of a step four steps ahead, next to its fragment; the 16 B scales of the next slab in steps 4..11, into the
-// register set the current slab does not use.
-// One step = 8 MFMAs + LDS reads (A fragment and scale; steps 0..3: four B fragments; steps 4..11: two B scales) + one
-// data load (+ a scale group load); a barrier every 4 steps.  At a barrier every wave has waited for its loads older
+// A lane fetches the two scale bytes of a row block and slab with one two-byte LDS read and the MFMA's op_sel picks
+// the byte of its k half: the A scales of an m block four steps ahead, with the fragment of its first k half; the 8
+// B scale pairs of the next slab in steps 4..11, into the register set the current slab does not use.
+// One step = 8 MFMAs + LDS reads (A fragment, on even steps an A scale pair; steps 0..3: four B fragments; steps 4..11:
+// one B scale pair) + one data load (+ a scale group load); a barrier every 4 steps.  At a barrier every wave has waited for its loads older
 // than the newest 15 (about a slab's worth; the tightest case is B part 3, read 16 loads after its own) and for its LDS
 // reads older than the interval:
 //   interval q of slab t loads   A: block q - 1 of slab t + 2 (q = 0: block 3 of slab t + 1)
