@@ -43,6 +43,37 @@ def test_random_gemm(dev):
         torch.testing.assert_close(c.float().cpu(), og.gemm_nt_ref(a, b), rtol=1e-2, atol=1e-2)
 
 
+def test_random_gemm_few_tiles_long_k(dev):
+    """Tile-aligned products with few 256x256 tiles and long K: the shapes the op hands a K-split workspace to (and
+    their neighbours that take none), fp16 and bf16 operands, against an fp32 product of sampled rows and columns."""
+    import iree_turbine_amd  # noqa: F401
+    from iree_turbine_amd import _lib
+    from oracle import inputs
+
+    lib = _lib.load()
+    rng = random.Random(111)
+    split = 0
+    for case in range(24):
+        tm, tn = rng.randint(1, 12), rng.randint(1, 12)
+        if case % 6 == 5:
+            tm, tn = rng.choice([(8, 40), (40, 8), (16, 18), (9, 32)])  # a full round of tiles and a sparse one behind it
+        M, N = 256 * tm, 256 * tn
+        K = rng.choice([4096, 4224, 6144, 8192, 12288])
+        dtype = rng.choice([torch.float16, torch.bfloat16])
+        out_dtype = rng.choice(["float32", str(dtype).split(".")[1]])
+        need = lib.mi355_gemm_nt_workspace_bytes(M, N, K)
+        split += need > 0
+        announce(f"random few-tile gemm {case}: {M}x{N}x{K} {dtype} -> {out_dtype}, workspace {need >> 20} MiB")
+        a, b = [t.to(dev) for t in inputs.gemm_inputs(M, N, K, seed=200 + case, dtype=dtype)]
+        c = torch.ops.mi355.gemm_nt(a, b, out_dtype, -1)
+        tol = dict(rtol=1e-3, atol=1e-3) if out_dtype == "float32" else dict(rtol=1e-2, atol=1e-2)
+        rows = torch.tensor(sorted({0, M - 1, rng.randrange(M), rng.randrange(M)}), device=dev)
+        cols = torch.tensor(sorted({0, N - 1, rng.randrange(N), rng.randrange(N)}), device=dev)
+        torch.testing.assert_close(c[rows].float(), a[rows].float() @ b.float().t(), **tol)
+        torch.testing.assert_close(c[:, cols].float(), a.float() @ b[cols].float().t(), **tol)
+    assert split >= 8  # the draw does exercise the split
+
+
 def test_random_attention(dev):
     import iree_turbine_amd  # noqa: F401
     from oracle import attention as oa
