@@ -219,7 +219,7 @@ __global__ __launch_bounds__(256) void fa_fwd_d128(const half_t* __restrict__ Q,
   }
 }
 
-// Paged K/V (PAGED kernels): the keys and values of sequence b are the first seq_lens[b] token rows of the
+// Paged K/V (the PAGED form of fa_fwd_d128_m16): the keys and values of sequence b are the first seq_lens[b] token rows of the
 // pages block_table[b][0..], 16 << page_shift tokens per page, laid out [page][token][kv head][128].  The kernel
 // walks 16-token blocks; a page is 1 << page_shift consecutive blocks.
 struct FaPaged {
@@ -251,12 +251,12 @@ __device__ __forceinline__ void static_for(F&& body) {
 // NW = waves per workgroup: 4 (128 queries, two workgroups per CU) or 8 (256 queries, one workgroup per CU: the two
 // wave quartets of a CU then share ONE copy of every K / V tile instead of loading one each -- half the LDS writes
 // and half the L2 reads for the same fragment reads).
-template <bool CAUSAL, bool PAGED, bool BF, int NW = 4>
+template <bool CAUSAL, bool BF, int NW = 4>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void fa_fwd_d128_pipe(
     const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V, half_t* __restrict__ O, int BH,
-    int Sq, int Sk_arg, float scale_log2e, int q_blocks, FaLayout lay, FaPaged pg) {
+    int Sq, int Sk, float scale_log2e, int q_blocks, FaLayout lay) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
-  static_assert(NW == 4 || (NW == 8 && !PAGED), "the paged form maps one page to one wave-load of a 4-wave workgroup");
+  static_assert(NW == 4 || NW == 8, "four or eight waves");
   constexpr int BLOCK_M = NW * 32;          // queries per workgroup
   constexpr int NI = 16 / NW;               // wave-loads per wave and tile (a wave-load = 4 rows of 256 bytes)
   constexpr int TILE_B = FA_BLOCK_N * 256;  // bytes of one K or V tile
@@ -286,37 +286,12 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
       unit = pid % units;
     }
   }
-  int b_idx = bh / lay.H;
+  const int b_idx = bh / lay.H;
   const int h_idx = bh - b_idx * lay.H, hk_idx = h_idx / lay.group;
-  int Sk = Sk_arg;
-  if constexpr (PAGED) {
-    // Sequences differ in length and workgroups are dispatched in grid order: take the sequences longest first,
-    // so that the short ones make up the tail.  Thread t counts the sequences that come before sequence t.
-    const int num_seqs = BH / lay.H;
-    if (num_seqs > 1 && num_seqs <= 256) {
-      int* pick = reinterpret_cast<int*>(lds);
-      const int t = threadIdx.x;
-      if (t < num_seqs) {
-        const int mine = pg.seq_lens[t];
-        int rank = 0;
-        for (int j = 0; j < num_seqs; j++) {
-          const int other = pg.seq_lens[j];
-          rank += (other > mine) || (other == mine && j < t);
-        }
-        if (rank == b_idx) *pick = t;
-      }
-      __syncthreads();
-      b_idx = __builtin_amdgcn_readfirstlane(*pick);
-      __syncthreads();  // the slot is part of the K ring
-    }
-    Sk = __builtin_amdgcn_readfirstlane(pg.seq_lens[b_idx]);
-    const int cap = (pg.max_pages * 16) << pg.page_shift;
-    Sk = Sk < 0 ? 0 : (Sk > cap ? cap : Sk);
-  }
   const int causal_off = Sk - Sq;
   const half_t* Qb = Q + b_idx * lay.q_b + h_idx * lay.q_h;
-  const half_t* Kb = K + (PAGED ? 0 : b_idx * lay.k_b) + hk_idx * lay.k_h;
-  const half_t* Vb = V + (PAGED ? 0 : b_idx * lay.v_b) + hk_idx * lay.v_h;
+  const half_t* Kb = K + b_idx * lay.k_b + hk_idx * lay.k_h;
+  const half_t* Vb = V + b_idx * lay.v_b + hk_idx * lay.v_h;
   half_t* Ob = O + b_idx * lay.o_b + h_idx * lay.o_h;
 
   // LDS addresses of the eight K fragment reads of a 32-key half tile (ks = 0..7), formed once: left to the
@@ -386,44 +361,14 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
   const unsigned k_rb = lay.k_r * 2, v_rb = lay.v_r * 2;  // row strides in bytes
   const unsigned k_voff = (wave * 4 + lrow) * k_rb + k_chunk * 16;
   const unsigned v_voff = (wave * 4 + lrow) * v_rb + v_chunk * 16;
-  // page ids come through the scalar cache (constant address space: the table is not written while the kernel
-  // runs), one tile ahead of their use, so that no K/V load waits for a table read
-  typedef const int __attribute__((address_space(4)))* table_ptr_t;
-  const table_ptr_t table_row =
-      PAGED ? (table_ptr_t)(unsigned long long)(pg.block_table + (size_t)b_idx * pg.max_pages) : (table_ptr_t)0;
-  auto load_ids = [&](int tile, int* ids) {
-    if constexpr (PAGED) {
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const int blk = tile * 4 + i, page = blk >> pg.page_shift;  // 16-token block -> its page and place in it
-        const int e = page < pg.max_pages ? table_row[page] : -1;
-        ids[i] = (e >= 0 && e < pg.num_pages) ? (e << pg.page_shift) + (blk & ((1 << pg.page_shift) - 1)) : -1;
-      }
-    }
-  };
-  auto issue_kv = [&](const half_t* base, unsigned rb, unsigned voff, int tile, int lds_off, const int* ids) {
+  auto issue_kv = [&](const half_t* base, unsigned rb, unsigned voff, int tile, int lds_off) {
     char* dst = lds + lds_off + wave * 1024;
     const int row0 = tile * FA_BLOCK_N;
     int rem = Sk - row0;
     rem = rem > FA_BLOCK_N ? FA_BLOCK_N : rem;
-    if constexpr (PAGED) {
-      // wave-load i covers rows 16 i .. 16 i + 15 of the tile = page 4 tile + i of the sequence: one descriptor
-      // per page, sized to the page's valid rows (none for a page beyond the sequence or an id outside the cache)
+    const buffer_rsrc_t rs = make_buffer(reinterpret_cast<const char*>(base) + (size_t)row0 * rb, (unsigned)(rem - 1) * rb + 256u);
 #pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const int id = ids[i];
-        int rows = rem - 16 * i;
-        rows = rows > 16 ? 16 : rows;
-        const bool ok = rows > 0 && id >= 0;
-        const buffer_rsrc_t rs = make_buffer(reinterpret_cast<const char*>(base) + (size_t)(ok ? id : 0) * 16u * rb,
-                                             ok ? (unsigned)(rows - 1) * rb + 256u : 0u);
-        buffer_load_lds_16B(rs, voff, 0, dst + i * 4096);
-      }
-    } else {
-      const buffer_rsrc_t rs = make_buffer(reinterpret_cast<const char*>(base) + (size_t)row0 * rb, (unsigned)(rem - 1) * rb + 256u);
-#pragma unroll
-      for (int i = 0; i < NI; i++) buffer_load_lds_16B(rs, voff + (unsigned)(i * NW * 4) * rb, 0, dst + i * NW * 1024);
-    }
+    for (int i = 0; i < NI; i++) buffer_load_lds_16B(rs, voff + (unsigned)(i * NW * 4) * rb, 0, dst + i * NW * 1024);
   };
 
   floatx16 oacc[4];
@@ -507,74 +452,38 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
     }
     half8 pf[4];
     float psum = 0.f;
-    if constexpr (!PAGED) {
-      // Scores of the next tile and exponentials of this one in one straight-line block: a wave issues in
-      // order, so only VALU work placed between two MFMAs runs while the first occupies the matrix pipe.
-      // (Past the last tile the scores are computed from stale LDS bytes and never used.)
-      __builtin_amdgcn_sched_barrier(0);
-      scores(koff_next, s_next);
+    // Scores of the next tile and exponentials of this one in one straight-line block: a wave issues in
+    // order, so only VALU work placed between two MFMAs runs while the first occupies the matrix pipe.
+    // (Past the last tile the scores are computed from stale LDS bytes and never used.)
+    __builtin_amdgcn_sched_barrier(0);
+    scores(koff_next, s_next);
 #pragma unroll
-      for (int t = 0; t < 2; t++)
+    for (int t = 0; t < 2; t++)
 #pragma unroll
-        for (int r = 0; r < 16; r += 2) {
-          const half2v pp = cvt16x2<BF>(__builtin_amdgcn_exp2f(s[t][r]), __builtin_amdgcn_exp2f(s[t][r + 1]));
-          psum = dot2_ones<BF>(pp, psum);  // sums what the second MFMA multiplies
-          pf[t * 2 + (r >> 3)][r & 7] = pp[0];
-          pf[t * 2 + (r >> 3)][(r & 7) + 1] = pp[1];
-        }
-      // order: 3 K fragment reads up front, then per score MFMA one more read and the work of two scores
-      // (two exp, one cvt_pk, one dot2) -- a fragment is requested two MFMAs before its use
-      __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
-#pragma unroll
-      for (int i = 0; i < 13; i++) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+      for (int r = 0; r < 16; r += 2) {
+        const half2v pp = cvt16x2<BF>(__builtin_amdgcn_exp2f(s[t][r]), __builtin_amdgcn_exp2f(s[t][r + 1]));
+        psum = dot2_ones<BF>(pp, psum);  // sums what the second MFMA multiplies
+        pf[t * 2 + (r >> 3)][r & 7] = pp[0];
+        pf[t * 2 + (r >> 3)][(r & 7) + 1] = pp[1];
       }
+    // order: 3 K fragment reads up front, then per score MFMA one more read and the work of two scores
+    // (two exp, one cvt_pk, one dot2) -- a fragment is requested two MFMAs before its use
+    __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
 #pragma unroll
-      for (int i = 0; i < 3; i++) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    } else {
-      // The paged form's page-id bookkeeping keeps the group barriers above from being honoured (the block came out
-      // as sixteen MFMAs, each behind its own fragment read, and the exponentials after them); here the same order is
-      // written step by step.
-      // Scores of the next tile and the softmax of this one, step by step: score MFMA i, the K fragment of MFMA i + 3
-      // requested, and the work of score pair i (two exponentials, one packed conversion, one dot2) behind it.  A
-      // scheduling barrier after every step pins the order (a wave issues in order: only vector work placed between two
-      // MFMAs runs while the first occupies the matrix pipe).
-      __builtin_amdgcn_sched_barrier(0);
-      {
-        half8 kf[4];
-        half2v pp_prev = {(half_t)0, (half_t)0};
-        auto kread = [&](int i) { return *(lds_half8_t)(uintptr_t)(k_frag[i & 7] + (unsigned)(koff_next + (i >> 3) * 8192)); };
-        kf[0] = kread(0);
-        kf[1] = kread(1);
-        kf[2] = kread(2);
-  #pragma unroll
-        for (int i = 0; i < 16; i++) {
-          const int t = i >> 3, ks = i & 7, r = 2 * ks;
-          if (i + 3 < 16) kf[(i + 3) & 3] = kread(i + 3);
-          s_next[t] = mfma16<BF>(kf[i & 3], qf[ks], ks == 0 ? negm : s_next[t]);
-          // (the empty statement ties the pair's arithmetic to this step: without side effects of its own it is placed
-          // wherever instruction selection likes, scheduling barriers or not.  The dot2 of a pair runs one step behind its
-          // conversion, so that neither waits for the instruction in front of it.)
-          float e0 = __builtin_amdgcn_exp2f(s[t][r]), e1 = __builtin_amdgcn_exp2f(s[t][r + 1]);
-          if (i > 0) psum = dot2_ones<BF>(pp_prev, psum);  // sums what the second MFMA multiplies
-          half2v pp = cvt16x2<BF>(e0, e1);
-          asm volatile("" : "+v"(pp), "+v"(psum));
-          pf[t * 2 + (r >> 3)][r & 7] = pp[0];
-          pf[t * 2 + (r >> 3)][(r & 7) + 1] = pp[1];
-          pp_prev = pp;
-          __builtin_amdgcn_sched_barrier(0);
-        }
-        psum = dot2_ones<BF>(pp_prev, psum);
-      }
+    for (int i = 0; i < 13; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
     }
+#pragma unroll
+    for (int i = 0; i < 3; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  
     l_run += psum;
     // O^T += V^T P^T: 16 MFMAs, each V^T fragment (two transpose reads) requested two MFMAs ahead.
     // The reads and their waits are inline assembly: a transpose read the compiler can see makes it wait for
@@ -611,14 +520,10 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
   };
 
   floatx16 sa[2], sb[2];
-  int k_ids[4] = {-1, -1, -1, -1}, v_ids[4] = {-1, -1, -1, -1};  // page ids of the next K tile and the next V tile to fetch
   if (n_tiles > 0) {
-    load_ids(0, k_ids);
-    issue_kv(Kb, k_rb, k_voff, 0, 0, k_ids);
-    issue_kv(Vb, v_rb, v_voff, 0, VBUF, k_ids);
-    load_ids(1, v_ids);
-    if (n_tiles > 1) issue_kv(Kb, k_rb, k_voff, 1, TILE_B, v_ids);
-    load_ids(2, k_ids);  // what trip 0 issues: K(2) and V(1)
+    issue_kv(Kb, k_rb, k_voff, 0, 0);
+    issue_kv(Vb, v_rb, v_voff, 0, VBUF);
+    if (n_tiles > 1) issue_kv(Kb, k_rb, k_voff, 1, TILE_B);
     wait_vmcnt0();
     __syncthreads();
     if (wave_active(0)) scores(0, sa);
@@ -631,14 +536,8 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
   auto trip = [&](auto par_tag, int j, floatx16* s_cur, floatx16* s_next) {
     constexpr int PAR = decltype(par_tag)::value;
     constexpr int K_CUR = PAR * TILE_B, K_NEXT = (1 - PAR) * TILE_B, V_CUR = PAR * TILE_B, V_NEXT = VBUF + (1 - PAR) * TILE_B;
-    if (j + 2 < n_tiles) issue_kv(Kb, k_rb, k_voff, j + 2, K_CUR, k_ids);
-    if (j + 1 < n_tiles) issue_kv(Vb, v_rb, v_voff, j + 1, V_NEXT, v_ids);
-    if constexpr (PAGED) {
-      // the next trip fetches V(j+2) -- the tile whose ids K just used -- and K(j+3)
-#pragma unroll
-      for (int i = 0; i < 4; i++) v_ids[i] = k_ids[i];
-      load_ids(j + 3, k_ids);
-    }
+    if (j + 2 < n_tiles) issue_kv(Kb, k_rb, k_voff, j + 2, K_CUR);
+    if (j + 1 < n_tiles) issue_kv(Vb, v_rb, v_voff, j + 1, V_NEXT);
     if (wave_active(j)) softmax_pv(std::true_type{}, j, std::integral_constant<int, V_CUR>{}, s_cur, K_NEXT, s_next);  // idle from here on otherwise
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
@@ -700,11 +599,12 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 // the score MFMAs (vector work behind 48 of the trip's 64 MFMAs instead of 32).  Measured on 2 x 32 x 4096: ahead with
 // eight waves (unmasked 475 against 484 us), behind with four (causal 268 against 263); each form is built the way it
 // runs faster.
-template <bool CAUSAL, bool BF, int NW, bool SPREAD>
+template <bool CAUSAL, bool BF, int NW, bool SPREAD, bool PAGED = false>
 __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void fa_fwd_d128_m16(
     const half_t* __restrict__ Q, const half_t* __restrict__ K, const half_t* __restrict__ V, half_t* __restrict__ O, int BH,
-    int Sq, int Sk, float scale_log2e, int q_blocks, FaLayout lay) {
+    int Sq, int Sk_arg, float scale_log2e, int q_blocks, FaLayout lay, FaPaged pg) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];
+  static_assert(NW == 4 || !PAGED, "the paged form maps one page to one wave-load of a 4-wave workgroup");
   constexpr int BLOCK_M = NW * 32, NI = 16 / NW;
   constexpr int TILE_B = FA_BLOCK_N * 256, VBUF = 2 * TILE_B;
   const int lane = threadIdx.x & 63;
@@ -725,12 +625,37 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
       unit = pid % units;
     }
   }
-  const int b_idx = bh / lay.H;
+  int b_idx = bh / lay.H;
   const int h_idx = bh - b_idx * lay.H, hk_idx = h_idx / lay.group;
+  int Sk = Sk_arg;
+  if constexpr (PAGED) {
+    // Sequences differ in length and workgroups are dispatched in grid order: take the sequences longest first,
+    // so that the short ones make up the tail.  Thread t counts the sequences that come before sequence t.
+    const int num_seqs = BH / lay.H;
+    if (num_seqs > 1 && num_seqs <= 256) {
+      int* pick = reinterpret_cast<int*>(lds);
+      const int t = threadIdx.x;
+      if (t < num_seqs) {
+        const int mine = pg.seq_lens[t];
+        int rank = 0;
+        for (int j = 0; j < num_seqs; j++) {
+          const int other = pg.seq_lens[j];
+          rank += (other > mine) || (other == mine && j < t);
+        }
+        if (rank == b_idx) *pick = t;
+      }
+      __syncthreads();
+      b_idx = __builtin_amdgcn_readfirstlane(*pick);
+      __syncthreads();  // the slot is part of the K ring
+    }
+    Sk = __builtin_amdgcn_readfirstlane(pg.seq_lens[b_idx]);
+    const int cap = (pg.max_pages * 16) << pg.page_shift;
+    Sk = Sk < 0 ? 0 : (Sk > cap ? cap : Sk);
+  }
   const int causal_off = Sk - Sq;
   const half_t* Qb = Q + b_idx * lay.q_b + h_idx * lay.q_h;
-  const half_t* Kb = K + b_idx * lay.k_b + hk_idx * lay.k_h;
-  const half_t* Vb = V + b_idx * lay.v_b + hk_idx * lay.v_h;
+  const half_t* Kb = K + (PAGED ? 0 : b_idx * lay.k_b) + hk_idx * lay.k_h;
+  const half_t* Vb = V + (PAGED ? 0 : b_idx * lay.v_b) + hk_idx * lay.v_h;
   half_t* Ob = O + b_idx * lay.o_b + h_idx * lay.o_h;
 
   // fragment read addresses, opaque (see fa_fwd_d128_pipe): K by step over d, V by d group
@@ -791,17 +716,47 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
   const unsigned k_rb = lay.k_r * 2, v_rb = lay.v_r * 2;
   const unsigned k_voff = (wave * 4 + lrow) * k_rb + k_chunk * 16;
   const unsigned v_voff = (wave * 4 + lrow) * v_rb + v_chunk * 16;
-  auto issue_kv = [&](const half_t* base, unsigned rb, unsigned voff, int tile, int lds_off) {
+  // paged form: page ids come through the scalar cache (constant address space: the table is not written while the
+  // kernel runs), one tile ahead of their use, so that no K/V load waits for a table read
+  typedef const int __attribute__((address_space(4)))* table_ptr_t;
+  const table_ptr_t table_row =
+      PAGED ? (table_ptr_t)(unsigned long long)(pg.block_table + (size_t)b_idx * pg.max_pages) : (table_ptr_t)0;
+  auto load_ids = [&](int tile, int* ids) {
+    if constexpr (PAGED) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const int blk = tile * 4 + i, page = blk >> pg.page_shift;  // 16-token block -> its page and place in it
+        const int e = page < pg.max_pages ? table_row[page] : -1;
+        ids[i] = (e >= 0 && e < pg.num_pages) ? (e << pg.page_shift) + (blk & ((1 << pg.page_shift) - 1)) : -1;
+      }
+    }
+  };
+  auto issue_kv = [&](const half_t* base, unsigned rb, unsigned voff, int tile, int lds_off, const int* ids) {
     char* dst = lds + lds_off + wave * 1024;
     const int row0 = tile * FA_BLOCK_N;
     int rem = Sk - row0;
     rem = rem > FA_BLOCK_N ? FA_BLOCK_N : rem;
-    const buffer_rsrc_t rs = make_buffer(reinterpret_cast<const char*>(base) + (size_t)row0 * rb, (unsigned)(rem - 1) * rb + 256u);
+    if constexpr (PAGED) {
+      // wave-load i covers rows 16 i .. 16 i + 15 of the tile = 16-token block 4 tile + i of the sequence: one descriptor
+      // per block, sized to its valid rows (none for a block beyond the sequence or an id outside the cache)
 #pragma unroll
-    for (int i = 0; i < NI; i++) {
+      for (int i = 0; i < 4; i++) {
+        const int id = ids[i];
+        int rows = rem - 16 * i;
+        rows = rows > 16 ? 16 : rows;
+        const bool ok = rows > 0 && id >= 0;
+        const buffer_rsrc_t rs = make_buffer(reinterpret_cast<const char*>(base) + (size_t)(ok ? id : 0) * 16u * rb,
+                                             ok ? (unsigned)(rows - 1) * rb + 256u : 0u);
+        buffer_load_lds_16B(rs, voff, 0, dst + i * 4096);
+      }
+    } else {
+      const buffer_rsrc_t rs = make_buffer(reinterpret_cast<const char*>(base) + (size_t)row0 * rb, (unsigned)(rem - 1) * rb + 256u);
+#pragma unroll
+      for (int i = 0; i < NI; i++) {
 #if !defined(MI355_ABLATE_NO_LOADS)
-      buffer_load_lds_16B(rs, voff + (unsigned)(i * NW * 4) * rb, 0, dst + i * NW * 1024);
+        buffer_load_lds_16B(rs, voff + (unsigned)(i * NW * 4) * rb, 0, dst + i * NW * 1024);
 #endif
+      }
     }
   };
 
@@ -995,10 +950,14 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
   };
 
   floatx4 sa[4][2], sb[4][2];  // scores [key group][query group], two tiles
+  int k_ids[4] = {-1, -1, -1, -1}, v_ids[4] = {-1, -1, -1, -1};  // paged form: ids of the next K tile and the next V tile to fetch
   if (n_tiles > 0) {
-    issue_kv(Kb, k_rb, k_voff, 0, 0);
-    issue_kv(Vb, v_rb, v_voff, 0, VBUF);
-    if (n_tiles > 1) issue_kv(Kb, k_rb, k_voff, 1, TILE_B);
+    load_ids(0, k_ids);
+    issue_kv(Kb, k_rb, k_voff, 0, 0, k_ids);
+    issue_kv(Vb, v_rb, v_voff, 0, VBUF, k_ids);
+    load_ids(1, v_ids);
+    if (n_tiles > 1) issue_kv(Kb, k_rb, k_voff, 1, TILE_B, v_ids);
+    load_ids(2, k_ids);  // what trip 0 issues: K(2) and V(1)
     wait_vmcnt0();
     __syncthreads();
     if (wave_active(0)) scores(0, sa);
@@ -1008,8 +967,14 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
   auto trip = [&](auto par_tag, int j, floatx4 (*s_cur)[2], floatx4 (*s_next)[2]) {
     constexpr int PAR = decltype(par_tag)::value;
     constexpr int K_CUR = PAR * TILE_B, K_NEXT = (1 - PAR) * TILE_B, V_CUR = VBUF + PAR * TILE_B, V_NEXT = VBUF + (1 - PAR) * TILE_B;
-    if (j + 2 < n_tiles) issue_kv(Kb, k_rb, k_voff, j + 2, K_CUR);
-    if (j + 1 < n_tiles) issue_kv(Vb, v_rb, v_voff, j + 1, V_NEXT);
+    if (j + 2 < n_tiles) issue_kv(Kb, k_rb, k_voff, j + 2, K_CUR, k_ids);
+    if (j + 1 < n_tiles) issue_kv(Vb, v_rb, v_voff, j + 1, V_NEXT, v_ids);
+    if constexpr (PAGED) {
+      // the next trip fetches V(j+2) -- the tile whose ids K just used -- and K(j+3)
+#pragma unroll
+      for (int i = 0; i < 4; i++) v_ids[i] = k_ids[i];
+      load_ids(j + 3, k_ids);
+    }
     if (wave_active(j)) softmax_pv(j, std::integral_constant<int, V_CUR - VBUF>{}, s_cur, K_NEXT, s_next);
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
 #if !defined(MI355_ABLATE_NO_BARRIERS)
@@ -1478,8 +1443,8 @@ static int fa_launch(const void* q, const void* k, const void* v, void* o, int64
   const int lds_bytes = 2 * FA_STAGE;
   static std::atomic<uint64_t> lds_ok[4] = {};
   const void* kernels[4] = {reinterpret_cast<const void*>(fa_fwd_d128<true, BF>), reinterpret_cast<const void*>(fa_fwd_d128<false, BF>),
-                            reinterpret_cast<const void*>(fa_fwd_d128_pipe<true, false, BF>),
-                            reinterpret_cast<const void*>(fa_fwd_d128_pipe<false, false, BF>)};
+                            reinterpret_cast<const void*>(fa_fwd_d128_pipe<true, BF>),
+                            reinterpret_cast<const void*>(fa_fwd_d128_pipe<false, BF>)};
   for (int i = 0; i < 4; i++)
     if (int rc = allow_lds(kernels[i], lds_bytes, lds_ok[i], "fa_fwd_d128")) return rc;
   const float scale_log2e = scale * 1.4426950408889634f;
@@ -1504,7 +1469,8 @@ static int fa_launch(const void* q, const void* k, const void* v, void* o, int64
     int bh_i = BH, sq_i = (int)Sq, sk_i = (int)Sk, qb_i = qbm;
     FaLayout lay_v = lay;
     float sc = scale_log2e;
-    void* args[] = {&qp, &kp, &vp, &op, &bh_i, &sq_i, &sk_i, &sc, &qb_i, &lay_v};
+    FaPaged no_pages{nullptr, nullptr, 0, 0, 0};
+    void* args[] = {&qp, &kp, &vp, &op, &bh_i, &sq_i, &sk_i, &sc, &qb_i, &lay_v, &no_pages};
     hipError_t e = hipLaunchKernel(kern, grid, block, args, lds_bytes, reinterpret_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail((int)e, "%s: launch of fa_fwd_d128_m16 failed: %s", who, hipGetErrorString(e));
     return check_launch("fa_fwd_d128_m16", grid, block, lds_bytes);
@@ -1541,14 +1507,14 @@ static int fa_launch(const void* q, const void* k, const void* v, void* o, int64
   }
   if (variant == 2) {
     // eight waves: 256-query blocks, one workgroup per CU
-    auto kern = is_causal ? fa_fwd_d128_pipe<true, false, BF, 8> : fa_fwd_d128_pipe<false, false, BF, 8>;
+    auto kern = is_causal ? fa_fwd_d128_pipe<true, BF, 8> : fa_fwd_d128_pipe<false, BF, 8>;
     static std::atomic<uint64_t> ok8[2] = {};
     const int lds8 = lds_bytes;
     if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds8, ok8[is_causal ? 1 : 0], "fa_fwd_d128_pipe<8>")) return rc;
     const int qb8 = (int)((Sq + 255) / 256);
     dim3 grid(BH * (is_causal ? (qb8 + 1) / 2 : qb8)), block(512);
     hipLaunchKernelGGL(kern, grid, block, lds8, reinterpret_cast<hipStream_t>(stream), (const half_t*)q, (const half_t*)k,
-                       (const half_t*)v, (half_t*)o, BH, (int)Sq, (int)Sk, scale_log2e, qb8, lay, FaPaged{nullptr, nullptr, 0, 0, 0});
+                       (const half_t*)v, (half_t*)o, BH, (int)Sq, (int)Sk, scale_log2e, qb8, lay);
     return check_launch("fa_fwd_d128_pipe<8 waves>", grid, block, lds8);
   }
   // the pipelined causal kernel takes a pair of query blocks per workgroup
@@ -1560,9 +1526,9 @@ static int fa_launch(const void* q, const void* k, const void* v, void* o, int64
     hipLaunchKernelGGL(kern, grid, block, lds_bytes, s, (const half_t*)q, (const half_t*)k, (const half_t*)v, (half_t*)o, BH,
                        (int)Sq, (int)Sk, scale_log2e, q_blocks, lay);
   } else {
-    auto kern = is_causal ? fa_fwd_d128_pipe<true, false, BF> : fa_fwd_d128_pipe<false, false, BF>;
+    auto kern = is_causal ? fa_fwd_d128_pipe<true, BF> : fa_fwd_d128_pipe<false, BF>;
     hipLaunchKernelGGL(kern, grid, block, lds_bytes, s, (const half_t*)q, (const half_t*)k, (const half_t*)v, (half_t*)o, BH,
-                       (int)Sq, (int)Sk, scale_log2e, q_blocks, lay, FaPaged{nullptr, nullptr, 0, 0, 0});
+                       (int)Sq, (int)Sk, scale_log2e, q_blocks, lay);
   }
   return check_launch(variant == 1 ? "fa_fwd_d128" : "fa_fwd_d128_pipe", grid, block, lds_bytes);
 }
@@ -1659,15 +1625,15 @@ static int fa_paged_prefill(const void* q, const void* k_cache, const void* v_ca
   const int BH = (int)(num_seqs * num_q_heads);
   const int q_blocks = (int)((num_new + FA_BLOCK_M - 1) / FA_BLOCK_M);
   const int lds_bytes = 2 * FA_STAGE;
-  auto kern = fa_fwd_d128_pipe<true, true, BF>;
+  auto kern = fa_fwd_d128_m16<true, BF, 4, false, true>;
   static std::atomic<uint64_t> lds_ok{0};
-  if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "fa_fwd_d128_pipe")) return rc;
+  if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "fa_fwd_d128_m16<paged>")) return rc;
   dim3 grid(BH * ((q_blocks + 1) / 2)), block(256);
   const FaPaged pg{static_cast<const int*>(block_table), static_cast<const int*>(seq_lens), (int)max_pages_per_seq, (int)num_pages,
                    page_shift};
   hipLaunchKernelGGL(kern, grid, block, lds_bytes, reinterpret_cast<hipStream_t>(stream), (const half_t*)q, (const half_t*)k_cache,
                      (const half_t*)v_cache, (half_t*)out, BH, (int)num_new, 0, scale * 1.4426950408889634f, q_blocks, lay, pg);
-  return check_launch("fa_fwd_d128_pipe<paged>", grid, block, lds_bytes);
+  return check_launch("fa_fwd_d128_m16<paged>", grid, block, lds_bytes);
 }
 
 extern "C" int mi355_paged_prefill_attn(const void* q, const void* k_cache, const void* v_cache, const void* block_table,
