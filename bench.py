@@ -56,17 +56,17 @@ MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
     "gemm_bf16_8192": 1.754e9,
     "gemm_16x8192x8192": 1.366e8,
     "gemm_1024x8192x8192": 3.644e8,
-    "fa_causal": 3.870e8,
+    "fa_causal": 3.537e8,
     "fa_noncausal": 2.686e8,
     "decode": 1.177e9,
-    "fa_causal_bf16": 3.876e8,
+    "fa_causal_bf16": 3.531e8,
     "decode_bf16": 1.177e9,
     "mxfp4_4096x8192x8192": 2.958e8,
     "mxfp4_32x8192x8192": 3.739e7,
     "mxfp4_quantize_16384x16384": 6.796e8,
     "mxfp8_quantize_16384x16384": 8.138e8,
     "mxfp6_quantize_16384x16384": 7.466e8,
-    "paged_prefill": 7.207e8,
+    "paged_prefill": 6.832e8,
     "mxfp8_4096x8192x8192": 4.972e8,
     "mxfp6_4096x8192x8192": 3.819e8,
 }
