@@ -61,6 +61,7 @@ __device__ __forceinline__ int opaque_lane_id() {
 //   MI355_ABLATE_PLAIN_LOAD_ORDER  (fp16 GEMM) the lanes of a row fetch its 16-byte chunks in ascending order
 //   MI355_ABLATE_NO_BARRIERS    the K loop has no workgroup barriers
 //   MI355_ABLATE_NO_SCALE_READS / MI355_ABLATE_NO_SCALE_LOADS   (block-scaled GEMMs) no LDS reads / no loads of scales
+//   MI355_ABLATE_NO_A_LOADS     (skinny MXFP4 GEMM) no loads of the activation rows
 //   MI355_ABLATE_NO_EXP / MI355_ABLATE_NO_K_READS / MI355_ABLATE_NO_V_READS   (prefill) no exponentials / fragment reads
 #if defined(MI355_ABLATE_NO_BARRIERS)
 #define MI355_KLOOP_BARRIER() do {} while (0)

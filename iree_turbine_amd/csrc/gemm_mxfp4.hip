@@ -619,76 +619,135 @@ __global__ __launch_bounds__(512) void gemm_mxfp4_skinny(const uint8_t* __restri
   const bool m_ok = r32 < M;
   char* tr = lds + 8 * 16384 + wave * 4096;  // one A segment (32 rows x 128 bytes) per wave, for the transposition below
   const int m_cl = r32 < M ? r32 : M - 1;    // rows past M repeat the last one: their output columns are never stored
-  for (int seg0 = 0; seg0 < nseg; seg0 += 32) {  // a pass covers 32 segments (4 per wave)
+  // The MFMAs as inline assembly: with fp4 operands the instruction takes four registers per source, where the builtin
+  // wants eight (the upper four zeroed) and a pass's sixteen such tuples do not fit beside everything else.  ZERO: the
+  // first link of a chain takes a zero addend.  Scale byte of the operands' scale registers = LO + 2 HI.
+#define MI355_SK_MFMA(LO, HI, ZERO, c, x, sx, y, sy)                                                                      \
+  do {                                                                                                                   \
+    if (ZERO)                                                                                                            \
+      asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, 0, %3, %4 op_sel:[" #LO "," #LO ",0] op_sel_hi:[" #HI "," #HI \
+                   ",0] cbsz:4 blgp:4"                                                                                   \
+                   : "=v"(c) : "v"(x), "v"(y), "v"(sx), "v"(sy));                                                        \
+    else                                                                                                                 \
+      asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[" #LO "," #LO ",0] op_sel_hi:[" #HI "," #HI \
+                   ",0] cbsz:4 blgp:4"                                                                                   \
+                   : "+v"(c) : "v"(x), "v"(y), "v"(sx), "v"(sy));                                                        \
+  } while (0)
+  int seg0 = 0;
+  for (; seg0 + 32 <= nseg; seg0 += 32) {  // a full pass covers 32 segments (4 per wave), straight-line
+    // The wave takes four CONSECUTIVE segments (32 scale blocks per row), and lane half h the blocks 16 h .. 16 h + 15
+    // of them, one per MFMA: k-step t multiplies block t (lanes of half 0) and block 16 + t (half 1).  Any assignment
+    // of blocks to lanes and k-steps is valid as long as A, B and the scales agree; this one makes a lane's 16 scale
+    // bytes of either operand ONE aligned 16-byte load (op_sel picks the byte of a dword) where a dword per lane and
+    // segment took eight loads of 32 cache lines each.
+    // A is the same 128 KiB for every workgroup and comes out of L2 -- as many bytes per workgroup as its share of
+    // B.  It is fetched like B -- 8 rows x 128 bytes per instruction, lane = (row, chunk) -- FIRST, and while the B
+    // loads issued behind it are still in flight it is turned into the MFMA layout through a 4 KiB LDS region (same
+    // swizzle as B).
+    // The A loads, the wait for them and the LDS instructions of the transposition are inline assembly: the compiler
+    // waits for EVERY load in flight before the first use of a loaded register once direct-to-LDS loads are among
+    // them, and before any LDS access it can see.  Loads return in order, so "at most the 16 B loads outstanding"
+    // means A has landed.  LDS executes a wave's instructions in order, so the reads see the writes and the next
+    // pass's writes come after this one's reads.
+    // Workgroups start together and walk K in the same order: were wave w of every workgroup to take the same
+    // segments, every workgroup of an XCD would ask for the same A lines at the same time.  Ids 8 apart share an XCD,
+    // so the rotation is taken from the id's bits above those.
     intx4 fa[4][4];
-    int sa[4], sb[4];
-    int cnt = 0;
-    if (seg0 + 32 <= nseg) {
-      // Full pass, straight-line.  A is the same 128 KiB for every workgroup and comes out of L2 -- as many bytes
-      // per workgroup as its share of B, and what they cost is L2 bandwidth (32x8192x8192: 8.7 us without the A
-      // loads, 12.6 with them in the MFMA's own layout, where a lane = one row and every load instruction
-      // touches 32 cache lines).  A is fetched like B -- 8 rows x 128 bytes per instruction, lane = (row, chunk)
-      // -- FIRST, and while the B loads issued behind it are still in flight it is turned into the MFMA layout
-      // through a 4 KiB LDS region (same swizzle as B): 12.2 us; with the B loads first 12.4.
-      // The A loads, the wait for them and the LDS instructions of the transposition are inline assembly: the
-      // compiler waits for EVERY load in flight before the first use of a loaded register once direct-to-LDS
-      // loads are among them, and before any LDS access it can see.  Loads return in order, so "at most the 16 B
-      // loads outstanding" means A has landed; a scale load that the compiler places behind the A loads only
-      // makes that wait longer.  LDS executes a wave's instructions in order, so the reads see the writes and
-      // the next segment's writes come after this one's reads.
-      // Workgroups start together and walk K in the same order, and rows are a multiple of 4 KiB apart: without
-      // the rotation every workgroup of an XCD would ask for the same A lines at the same time (11.8 us with
-      // it).  Ids 8 apart share an XCD, so the step is taken from the id's bits above those.
-      const int rot = (blockIdx.x >> 3) & 3;
+    const int segw = seg0 + 4 * ((wave + (int)(blockIdx.x >> 3)) & 7);
+    intx4 sav, sbv;  // the lane's 16 scale bytes of A and of B
+#if defined(MI355_ABLATE_NO_SCALE_LOADS)
+    sav = sbv = intx4{0x7f7f7f7f, 0x7f7f7f7f + segw, 0x7f7f7f7f, 0x7f7f7f7f};
+#else
+    sav = *reinterpret_cast<const intx4*>(As + (size_t)m_cl * Ksc + segw * 8 + 16 * h);
+    sbv = *reinterpret_cast<const intx4*>(Bs + (size_t)(n0 + r32) * Ksc + segw * 8 + 16 * h);
+#endif
 #pragma unroll
-      for (int q = 0; q < 4; q++) {
-        const int seg = seg0 + wave + 8 * ((q + rot) & 3);
-        sa[q] = *reinterpret_cast<const int*>(As + (size_t)m_cl * Ksc + seg * 8 + 4 * h);
-        sb[q] = *reinterpret_cast<const int*>(Bs + (size_t)(n0 + r32) * Ksc + seg * 8 + 4 * h);
-      }
-#pragma unroll
-      for (int q = 0; q < 4; q++) {
-        const int seg = seg0 + wave + 8 * ((q + rot) & 3);
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-          const int row = i * 8 + lrow;
-          const uint8_t* ap = A + (size_t)(row < M ? row : M - 1) * Kb + seg * 128 + (lane & 7) * 16;
-          asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(fa[q][i]) : "v"(ap) : "memory");
-        }
-      }
-#pragma unroll
-      for (int q = 0; q < 4; q++) {
-        const int seg = seg0 + wave + 8 * ((q + rot) & 3);
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-          const int row = i * 8 + lrow;
-          const int chunk = (lane & 7) ^ ((row >> 1) & 7);
-          load_lds_16B(B + (size_t)(n0 + row) * Kb + seg * 128 + chunk * 16, my + q * 4096 + i * 1024);
-        }
-      }
-      cnt = 4;
-      __builtin_amdgcn_sched_barrier(0);
-      asm volatile("s_waitcnt vmcnt(16)"
-                   : "+v"(fa[0][0]), "+v"(fa[0][1]), "+v"(fa[0][2]), "+v"(fa[0][3]), "+v"(fa[1][0]), "+v"(fa[1][1]),
-                     "+v"(fa[1][2]), "+v"(fa[1][3]), "+v"(fa[2][0]), "+v"(fa[2][1]), "+v"(fa[2][2]), "+v"(fa[2][3]),
-                     "+v"(fa[3][0]), "+v"(fa[3][1]), "+v"(fa[3][2]), "+v"(fa[3][3]));
-      const unsigned tr_base = (unsigned)(uintptr_t)MI355_LDS(char, tr);
-      unsigned wa[4], ra[4];
+    for (int q = 0; q < 4; q++) {
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         const int row = i * 8 + lrow;
-        wa[i] = tr_base + row * 128 + (((lane & 7) ^ ((row >> 1) & 7)) * 16);
-        ra[i] = tr_base + r32 * 128 + (((4 * h + i) ^ ((r32 >> 1) & 7)) * 16);
+        const uint8_t* ap = A + (size_t)(row < M ? row : M - 1) * Kb + (segw + q) * 128 + (lane & 7) * 16;
+#if defined(MI355_ABLATE_NO_A_LOADS)
+        fa[q][i] = intx4{(int)(uintptr_t)ap, lane, q, i};
+#else
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(fa[q][i]) : "v"(ap) : "memory");
+#endif
       }
+    }
 #pragma unroll
-      for (int q = 0; q < 4; q++) {
+    for (int q = 0; q < 4; q++) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) asm volatile("ds_write_b128 %0, %1" ::"v"(wa[i]), "v"(fa[q][i]));
-#pragma unroll
-        for (int sp = 0; sp < 4; sp++) asm volatile("ds_read_b128 %0, %1" : "=v"(fa[q][sp]) : "v"(ra[sp]));
+      for (int i = 0; i < 4; i++) {
+        const int row = i * 8 + lrow;
+        const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+#if !defined(MI355_ABLATE_NO_LOADS)
+        load_lds_16B(B + (size_t)(n0 + row) * Kb + (segw + q) * 128 + chunk * 16, my + q * 4096 + i * 1024);
+#endif
       }
-      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    } else {
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt vmcnt(16)"
+                 : "+v"(fa[0][0]), "+v"(fa[0][1]), "+v"(fa[0][2]), "+v"(fa[0][3]), "+v"(fa[1][0]), "+v"(fa[1][1]),
+                   "+v"(fa[1][2]), "+v"(fa[1][3]), "+v"(fa[2][0]), "+v"(fa[2][1]), "+v"(fa[2][2]), "+v"(fa[2][3]),
+                   "+v"(fa[3][0]), "+v"(fa[3][1]), "+v"(fa[3][2]), "+v"(fa[3][3]));
+    const unsigned tr_base = (unsigned)(uintptr_t)MI355_LDS(char, tr);
+    const int sw = (r32 >> 1) & 7;
+    // The 4 KiB region takes, per pass, four chunks of a segment of lane half 0 (q01) in the first 64 bytes of a row's
+    // slots and the same four chunks of the segment of lane half 1 (2 + q01) in the second, so that every lane reads
+    // in every pass: written by the lanes that loaded those chunks, read as block t = 8 q01 + 4 ch + cc.
+    unsigned wa[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int row = i * 8 + lrow;
+      wa[i] = tr_base + row * 128 + (((lane & 3) ^ ((row >> 1) & 7)) * 16);  // slot (lane & 3) of half 0; half 1: ^ 64
+    }
+    const unsigned ra = tr_base + r32 * 128;
+    intx4 ga[16];  // A blocks in MFMA layout: ga[t] = block 16 h + t of the wave's 32
+#pragma unroll
+    for (int q01 = 0; q01 < 2; q01++) {
+#pragma unroll
+      for (int ch = 0; ch < 2; ch++) {
+        if (((lane >> 2) & 1) == ch) {
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            asm volatile("ds_write_b128 %0, %1" ::"v"(wa[i]), "v"(fa[q01][i]) : "memory");
+            asm volatile("ds_write_b128 %0, %1" ::"v"(wa[i] ^ 64u), "v"(fa[q01 + 2][i]) : "memory");
+          }
+        }
+#pragma unroll
+        for (int cc = 0; cc < 4; cc++)
+          asm volatile("ds_read_b128 %0, %1" : "=v"(ga[q01 * 8 + ch * 4 + cc]) : "v"(ra + (unsigned)(((h * 4 + cc) ^ sw) * 16)) : "memory");
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(ga[0]), "+v"(ga[1]), "+v"(ga[2]), "+v"(ga[3]), "+v"(ga[4]), "+v"(ga[5]), "+v"(ga[6]), "+v"(ga[7]),
+                   "+v"(ga[8]), "+v"(ga[9]), "+v"(ga[10]), "+v"(ga[11]), "+v"(ga[12]), "+v"(ga[13]), "+v"(ga[14]), "+v"(ga[15]));
+    wait_vmcnt0();
+    __builtin_amdgcn_sched_barrier(0);
+    const char* my_b = my + 2 * h * 4096 + r32 * 128;  // block 16 h + t: segment 2 h + t / 8, chunk t % 8
+    // Four chains (k-step t -> chain t % 4), so that no MFMA reads a sum written by one of the three before it.
+    // "A" operand = B rows (n), "B" operand = A rows (m): pacc[n][m].
+    floatx16 pacc[4];
+#pragma unroll
+    for (int t = 0; t < 16; t++) {
+      const intx4 fb = *reinterpret_cast<const intx4*>(my_b + (t >> 3) * 4096 + (((t & 7) ^ sw) * 16));
+      const int sbq = sbv[t >> 2], saq = sav[t >> 2];
+      if ((t & 3) == 0) MI355_SK_MFMA(0, 0, t < 4, pacc[0], fb, sbq, ga[t], saq);
+      if ((t & 3) == 1) MI355_SK_MFMA(1, 0, t < 4, pacc[1], fb, sbq, ga[t], saq);
+      if ((t & 3) == 2) MI355_SK_MFMA(0, 1, t < 4, pacc[2], fb, sbq, ga[t], saq);
+      if ((t & 3) == 3) MI355_SK_MFMA(1, 1, t < 4, pacc[3], fb, sbq, ga[t], saq);
+    }
+    // the compiler does not know that these registers were written by MFMAs just now: the wait states an MFMA result
+    // needs before a vector instruction may read it, and every sum tied to a statement behind them
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" : "+v"(pacc[0]), "+v"(pacc[1]), "+v"(pacc[2]), "+v"(pacc[3]));
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] += (pacc[0][r] + pacc[1][r]) + (pacc[2][r] + pacc[3][r]);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's LDS reads are done before the next pass overwrites
+  }
+  if (seg0 < nseg) {  // the last, partial pass: segments w, w + 8, ... of what is left, operands loaded in the MFMA's own layout
+    intx4 fa[4][4];
+    int sa[4], sb[4];
+    int cnt = 0;
 #pragma unroll
     for (int q = 0; q < 4; q++) {
       const int seg = seg0 + wave + 8 * q;
@@ -714,27 +773,31 @@ __global__ __launch_bounds__(512) void gemm_mxfp4_skinny(const uint8_t* __restri
         }
       }
     }
-    }
     wait_vmcnt0();
+    if (cnt > 0) {
+      floatx16 pacc[4];  // one chain per k-step of a segment; segment 0 starts them
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-      if (q < cnt) {
+      for (int q = 0; q < 4; q++) {
+        if (q < cnt) {
 #pragma unroll
-        for (int sp = 0; sp < 4; sp++) {
-          const int c = 4 * h + sp;
-          intx4 fb = *reinterpret_cast<const intx4*>(my + q * 4096 + r32 * 128 + ((c ^ ((r32 >> 1) & 7)) * 16));
-          intx8 av = {fb[0], fb[1], fb[2], fb[3], 0, 0, 0, 0};
-          intx8 bv = {fa[q][sp][0], fa[q][sp][1], fa[q][sp][2], fa[q][sp][3], 0, 0, 0, 0};
-          // MFMA "A" operand = B rows (n), "B" operand = A rows (m): acc[n][m]
-          if (sp == 0) acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc, 4, 4, 0, sb[q], 0, sa[q]);
-          if (sp == 1) acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc, 4, 4, 1, sb[q], 1, sa[q]);
-          if (sp == 2) acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc, 4, 4, 2, sb[q], 2, sa[q]);
-          if (sp == 3) acc = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc, 4, 4, 3, sb[q], 3, sa[q]);
+          for (int sp = 0; sp < 4; sp++) {
+            const int c = 4 * h + sp;
+            const intx4 fb = *reinterpret_cast<const intx4*>(my + q * 4096 + r32 * 128 + ((c ^ ((r32 >> 1) & 7)) * 16));
+            // MFMA "A" operand = B rows (n), "B" operand = A rows (m): pacc[n][m]
+            if (sp == 0) MI355_SK_MFMA(0, 0, q == 0, pacc[0], fb, sb[q], fa[q][sp], sa[q]);
+            if (sp == 1) MI355_SK_MFMA(1, 0, q == 0, pacc[1], fb, sb[q], fa[q][sp], sa[q]);
+            if (sp == 2) MI355_SK_MFMA(0, 1, q == 0, pacc[2], fb, sb[q], fa[q][sp], sa[q]);
+            if (sp == 3) MI355_SK_MFMA(1, 1, q == 0, pacc[3], fb, sb[q], fa[q][sp], sa[q]);
+          }
         }
       }
+      asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" : "+v"(pacc[0]), "+v"(pacc[1]), "+v"(pacc[2]), "+v"(pacc[3]));
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[r] += (pacc[0][r] + pacc[1][r]) + (pacc[2][r] + pacc[3][r]);
     }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's LDS reads are done before the next pass overwrites
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   }
+#undef MI355_SK_MFMA
 
   // reduce the 8 partial tiles: lane (m = r32, h) register r holds n = 8*(r/4) + 4h + r%4
   __syncthreads();
