@@ -675,7 +675,8 @@ __global__ __launch_bounds__(512) void gemm_mxfp4_skinny(const uint8_t* __restri
       }
     }
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
+    for (int qo = 0; qo < 4; qo++) {
+      const int q = ((qo & 1) << 1) | (qo >> 1);  // segments 0, 2, 1, 3: the first eight k-steps read segments 0 and 2
 #pragma unroll
       for (int i = 0; i < 4; i++) {
         const int row = i * 8 + lrow;
@@ -722,20 +723,31 @@ __global__ __launch_bounds__(512) void gemm_mxfp4_skinny(const uint8_t* __restri
     asm volatile("s_waitcnt lgkmcnt(0)"
                  : "+v"(ga[0]), "+v"(ga[1]), "+v"(ga[2]), "+v"(ga[3]), "+v"(ga[4]), "+v"(ga[5]), "+v"(ga[6]), "+v"(ga[7]),
                    "+v"(ga[8]), "+v"(ga[9]), "+v"(ga[10]), "+v"(ga[11]), "+v"(ga[12]), "+v"(ga[13]), "+v"(ga[14]), "+v"(ga[15]));
-    wait_vmcnt0();
-    __builtin_amdgcn_sched_barrier(0);
-    const char* my_b = my + 2 * h * 4096 + r32 * 128;  // block 16 h + t: segment 2 h + t / 8, chunk t % 8
+    // B lands in order: the first eight k-steps (segments 0 and 2) run while the other half is still in flight.  The
+    // fragment reads are assembly like the transposition's (the compiler would wait for every load in front of them).
     // Four chains (k-step t -> chain t % 4), so that no MFMA reads a sum written by one of the three before it.
     // "A" operand = B rows (n), "B" operand = A rows (m): pacc[n][m].
+    const unsigned my_b = (unsigned)(uintptr_t)MI355_LDS(char, my) + 2 * h * 4096 + r32 * 128;  // block 16 h + t: segment 2 h + t / 8, chunk t % 8
     floatx16 pacc[4];
 #pragma unroll
-    for (int t = 0; t < 16; t++) {
-      const intx4 fb = *reinterpret_cast<const intx4*>(my_b + (t >> 3) * 4096 + (((t & 7) ^ sw) * 16));
-      const int sbq = sbv[t >> 2], saq = sav[t >> 2];
-      if ((t & 3) == 0) MI355_SK_MFMA(0, 0, t < 4, pacc[0], fb, sbq, ga[t], saq);
-      if ((t & 3) == 1) MI355_SK_MFMA(1, 0, t < 4, pacc[1], fb, sbq, ga[t], saq);
-      if ((t & 3) == 2) MI355_SK_MFMA(0, 1, t < 4, pacc[2], fb, sbq, ga[t], saq);
-      if ((t & 3) == 3) MI355_SK_MFMA(1, 1, t < 4, pacc[3], fb, sbq, ga[t], saq);
+    for (int half = 0; half < 2; half++) {
+      if (half == 0) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      intx4 fb[8];
+#pragma unroll
+      for (int c = 0; c < 8; c++)
+        asm volatile("ds_read_b128 %0, %1" : "=v"(fb[c]) : "v"(my_b + (unsigned)(half * 4096 + ((c ^ sw) * 16))) : "memory");
+      asm volatile("s_waitcnt lgkmcnt(0)"
+                   : "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]), "+v"(fb[4]), "+v"(fb[5]), "+v"(fb[6]), "+v"(fb[7]));
+#pragma unroll
+      for (int c = 0; c < 8; c++) {
+        const int t = half * 8 + c;
+        const int sbq = sbv[t >> 2], saq = sav[t >> 2];
+        if ((t & 3) == 0) MI355_SK_MFMA(0, 0, t < 4, pacc[0], fb[c], sbq, ga[t], saq);
+        if ((t & 3) == 1) MI355_SK_MFMA(1, 0, t < 4, pacc[1], fb[c], sbq, ga[t], saq);
+        if ((t & 3) == 2) MI355_SK_MFMA(0, 1, t < 4, pacc[2], fb[c], sbq, ga[t], saq);
+        if ((t & 3) == 3) MI355_SK_MFMA(1, 1, t < 4, pacc[3], fb[c], sbq, ga[t], saq);
+      }
     }
     // the compiler does not know that these registers were written by MFMAs just now: the wait states an MFMA result
     // needs before a vector instruction may read it, and every sum tied to a statement behind them
