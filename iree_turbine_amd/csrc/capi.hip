@@ -75,6 +75,9 @@ extern "C" const char* mi355_build_flags(void) {
 #if defined(MI355_ABLATE_NO_A_LOADS)
          " NO_A_LOADS"
 #endif
+#if defined(MI355_ABLATE_NO_STORES)
+         " NO_STORES"
+#endif
 #if defined(MI355_ABLATE_NO_EXP)
          " NO_EXP"
 #endif

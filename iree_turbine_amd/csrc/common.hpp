@@ -62,6 +62,7 @@ __device__ __forceinline__ int opaque_lane_id() {
 //   MI355_ABLATE_NO_BARRIERS    the K loop has no workgroup barriers
 //   MI355_ABLATE_NO_SCALE_READS / MI355_ABLATE_NO_SCALE_LOADS   (block-scaled GEMMs) no LDS reads / no loads of scales
 //   MI355_ABLATE_NO_A_LOADS     (skinny MXFP4 GEMM) no loads of the activation rows
+//   MI355_ABLATE_NO_STORES      the streamed kernels' epilogues stage their results and store nothing
 //   MI355_ABLATE_NO_EXP / MI355_ABLATE_NO_K_READS / MI355_ABLATE_NO_V_READS   (prefill) no exponentials / fragment reads
 #if defined(MI355_ABLATE_NO_BARRIERS)
 #define MI355_KLOOP_BARRIER() do {} while (0)
@@ -88,7 +89,11 @@ __device__ __forceinline__ void wait_vmcnt0() { asm volatile("s_waitcnt vmcnt(0)
 template <typename T>
 __device__ __forceinline__ void store_global_16B(void* p, const T& v) {
   static_assert(sizeof(T) == 16, "store_global_16B stores exactly 16 bytes per lane");
+#if defined(MI355_ABLATE_NO_STORES)
+  asm volatile("" ::"v"(p), "v"(v) : "memory");
+#else
   asm volatile("global_store_dwordx4 %0, %1, off\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
+#endif
 }
 
 // D(32x32) += A(32x16) * B(16x32).  Lane l supplies A[l%32][8*(l/32) .. +7] and
