@@ -59,7 +59,11 @@ template <int BM, int BN, int WM, int WN, typename OutT, bool BF>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_t* __restrict__ A,
                                                                      const half_t* __restrict__ B,
                                                                      OutT* __restrict__ C, int M, int N, int K,
-                                                                     int tiles_m, int tiles_n, int group_m) {
+                                                                     int tiles_m, int tiles_n, int group_m, int ldk,
+                                                                     int split_tiles_m, int ksplit_halfs) {
+  // K: the length of the K range a workgroup adds up; ldk: the row pitch of A and B in halfs.  With a K split
+  // (split_tiles_m > 0) the tile grid is stacked S times along M: tile row t stands for tile row t % split_tiles_m of A
+  // and the K range t / split_tiles_m, ksplit_halfs apart, and C (the workspace) has S times the rows.
   constexpr int NW = WM * WN;
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -79,10 +83,17 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
   const int lrow = lane >> 3;
   const int lchunk = (lane & 7) ^ (((wave & 1) << 2) | (lrow >> 1));
   // wave-uniform base pointer + one 32-bit per-lane offset (in halfs) shared by every load of the wave
-  const half_t* a_src = A + (size_t)(tile_m * BM + wave * 8) * K;
-  const half_t* b_src = B + (size_t)(tile_n * BN + wave * 8) * K;
-  const unsigned lane_off = (unsigned)lrow * (unsigned)K + (unsigned)lchunk * 8u;
-  const size_t row_step = (size_t)NW * 8 * K;
+  int a_tile = tile_m;
+  size_t k_at = 0;
+  if (split_tiles_m > 0)
+    while (a_tile >= split_tiles_m) {  // at most S - 1 turns
+      a_tile -= split_tiles_m;
+      k_at += (size_t)ksplit_halfs;
+    }
+  const half_t* a_src = A + (size_t)(a_tile * BM + wave * 8) * ldk + k_at;
+  const half_t* b_src = B + (size_t)(tile_n * BN + wave * 8) * ldk + k_at;
+  const unsigned lane_off = (unsigned)lrow * (unsigned)ldk + (unsigned)lchunk * 8u;
+  const size_t row_step = (size_t)NW * 8 * ldk;
 
   auto issue_loads = [&](int stage, int slab) {
     char* dst = lds + stage * STAGE + wave * 1024;
@@ -1339,19 +1350,39 @@ static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int
   // the kernels use their N argument only as the row stride of C, so a column range of a wider C is the
   // same launch with ldc in its place
   static_assert(KIND == 1 || KIND == 2, "pipelined or register-staged");
-  void (*kern)(const half_t*, const half_t*, OutT*, int, int, int, int, int, int);
-  if constexpr (KIND == 2) kern = gemm_f16_nt_staged<BM, BN, WM, WN, OutT, BF>;
-  else kern = gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT, BF>;
   // the register-staged kernel keeps its epilogue out of the stages: 32 rows x 128 bytes per wave
   constexpr int lds_bytes = 2 * (BM + BN) * 128 + (KIND == 2 ? WM * WN * 32 * 128 : 0);
   static std::atomic<uint64_t> lds_ok{0};
-  if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt")) return rc;
   const int tiles_m = M / BM, tiles_n = N / BN;
   int group_m = 4;
   dim3 grid(tiles_m * tiles_n), block(WM * WN * 64);
-  hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, M, ldc, K, tiles_m,
-                     tiles_n, group_m);
+  if constexpr (KIND == 2) {
+    auto kern = gemm_f16_nt_staged<BM, BN, WM, WN, OutT, BF>;
+    if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt")) return rc;
+    hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, M, ldc, K, tiles_m,
+                       tiles_n, group_m);
+  } else {
+    auto kern = gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT, BF>;
+    if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt")) return rc;
+    hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, M, ldc, K, tiles_m,
+                       tiles_n, group_m, K, 0, 0);
+  }
   return check_launch(KIND == 2 ? "gemm_f16_nt_staged" : "gemm_f16_nt_pipelined", grid, block, lds_bytes);
+}
+
+// K split on the pipelined 128x128 kernel, for products too small for 256x256 tiles to spread over the chip: S K ranges
+// of k_part each, fp32 partial tiles stacked along M in the workspace (row pitch N).
+template <bool BF>
+static int launch_pipelined_ksplit(const half_t* a, const half_t* b, float* ws, int M, int N, int K, int S, hipStream_t stream) {
+  auto kern = gemm_f16_nt_pipelined<128, 128, 2, 2, float, BF>;
+  constexpr int lds_bytes = 2 * (128 + 128) * 128;
+  static std::atomic<uint64_t> lds_ok{0};
+  if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt")) return rc;
+  const int k_part = K / S;
+  const int tiles_m = (M / 128) * S, tiles_n = N / 128;
+  dim3 grid(tiles_m * tiles_n), block(256);
+  hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, a, b, ws, M * S, N, k_part, tiles_m, tiles_n, 4, K, M / 128, k_part);
+  return check_launch("gemm_f16_nt_pipelined (K split)", grid, block, lds_bytes);
 }
 
 template <int BM, int BN, int WM, int WN, typename OutT, bool BF>
@@ -1435,8 +1466,44 @@ static int launch_ksplit(const half_t* a, const half_t* b, OutT* c, int M, int N
   return check_launch("gemm_ksplit_merge", grid, block, 0);
 }
 
-// The sub-problem that would take a K split under the automatic choice, if any: the strip a sparse last round is cut
-// into, or the whole product when it has fewer than 128 tiles.  Returns S (1: none) and the sub-problem's M and N.
+template <typename OutT, bool BF>
+static int launch_ksplit128(const half_t* a, const half_t* b, OutT* c, int M, int N, int K, int ldc, int S, float* ws, hipStream_t stream) {
+  if (int rc = launch_pipelined_ksplit<BF>(a, b, ws, M, N, K, S, stream)) return rc;
+  const long long lanes = (long long)M * N / 4;
+  dim3 grid((unsigned)((lanes + 255) / 256)), block(256);
+  hipLaunchKernelGGL((gemm_ksplit_merge<OutT, BF>), grid, block, 0, stream, (const float*)ws, c, M, N, ldc, S);
+  return check_launch("gemm_ksplit_merge", grid, block, 0);
+}
+
+// K split on 128x128 tiles, for products that are small even for that: S doubles while the (tile, range) units still
+// number <= 256 and a range keeps 512 of K (1024 beyond 64 units).  Measured against the 256x256 split and the plain
+// kernels (us, graph-timed; best S in brackets): 256x256x8192 14.4 [16] against 30.3, 512x512x4096 15.2 [8] against 30.2,
+// 512x1024x8192 22.6 [8] against 33.5, 1024x1024x4096 22.6 [4] against 33.9, 384x640x8192 18.7 [8] against 73.6; no gain
+// from K = 1024, nor beyond 64 tiles except for 4096 <= K < 6144, where two ranges are level to ahead of the 256x256
+// split (1024x2048x4096: 31.9 against 36.0).
+static int ksplit128_factor(long long t128, int K) {
+  if (K < 2048 || K % 128 != 0) return 1;
+  if (t128 > 64) return (t128 <= 160 && K >= 4096 && K < 6144) ? 2 : 1;
+  if (t128 > 48 && K < 4096) return 1;
+  int s = 1;
+  while (s < 16) {
+    const int n = 2 * s;
+    const long long units = t128 * n;
+    if (units > 256 || K % (64 * n) != 0 || K / n < (units <= 64 ? 512 : 1024)) break;
+    s = n;
+  }
+  return s;
+}
+
+// S for a whole product on 128x128 tiles under the automatic choice (1: none)
+static int ksplit128_plan(int M, int N, int K) {
+  if (M % 128 || N % 128) return 1;
+  return ksplit128_factor((long long)(M / 128) * (N / 128), K);
+}
+
+// The sub-problem that would take a K split on 256x256 tiles under the automatic choice, if any: the strip a sparse
+// last round is cut into, or the whole product when it has at most 128 tiles (and the 128x128 split above does not
+// take it).  Returns S (1: none) and the sub-problem's M and N.
 static int ksplit_plan(int M, int N, int K, int& sub_m, int& sub_n) {
   sub_m = M;
   sub_n = N;
@@ -1449,6 +1516,7 @@ static int ksplit_plan(int M, int N, int K, int& sub_m, int& sub_n) {
     else sub_m = M - mm;
     return ksplit_factor((long long)(sub_m / 256) * (sub_n / 256), K);
   }
+  if (ksplit128_plan(M, N, K) > 1) return 1;
   return t256 >= 1 ? ksplit_factor(t256, K) : 1;
 }
 
@@ -1539,6 +1607,7 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
     if (v == V_SKINNY) return al && M <= 64 && N % 32 == 0 && K % 64 == 0;  // a tile is 32 rows of B; 64-half K segments
     return al && M % kGemmVariants[v].bm == 0 && N % kGemmVariants[v].bn == 0 && K % 64 == 0;
   };
+  int split128 = 1;  // K ranges of the 128x128 split, when the automatic choice takes it
   if (variant < 0) {
     // Large problems take the 256x256 tile; when that leaves most of the 256 CUs idle the
     // 128x128 tile (4x the workgroups) wins; everything else goes to the bounds-checked kernel.
@@ -1550,7 +1619,12 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
     // hides each tile's prologue and epilogue under its neighbours (8192x8192x512: 978 against 854), as long as its
     // last round is >= 85% busy.
     const bool full_rounds = t256 * 100 >= rounds * 256 * 85;
+    const int s128 = (workspace && fits(V_PIPELINED_128)) ? ksplit128_plan((int)M, (int)N, (int)K) : 1;
     if (fits(V_SKINNY) && N >= 2048 && K >= 512) variant = V_SKINNY;  // decode-shaped: stream the weights once
+    else if (s128 > 1 && workspace_bytes >= (int64_t)s128 * M * N * 4) {  // a small product: K split on 128x128 tiles
+      variant = V_PIPELINED_128;
+      split128 = s128;
+    }
     else if (K < 1024 && t256 <= 2048 && fits(V_PERSISTENT) && t256 >= 128 && full_rounds) variant = V_PERSISTENT;
     else if (t256 <= 128 && fits(V_STREAM_TAIL) && workspace && [&] {  // too few tiles for the chip, and a workspace to split K into
                int sm, sn;
@@ -1576,6 +1650,16 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
   float* ws = static_cast<float*>(workspace);
   const size_t wsb = workspace_bytes > 0 ? (size_t)workspace_bytes : 0;
   if (ws && !aligned16(ws)) return fail(-MI355_E_ALIGN, "gemm_f16_nt: workspace must be 16-byte aligned");
+  if (split128 > 1) {
+    const half_t *ah = (const half_t*)a, *bh = (const half_t*)b;
+    const int m = (int)M, n = (int)N, k = (int)K;
+    if (bf) {
+      if (out_dtype == MI355_F32) return launch_ksplit128<float, true>(ah, bh, (float*)c, m, n, k, n, split128, ws, s);
+      return launch_ksplit128<half_t, true>(ah, bh, (half_t*)c, m, n, k, n, split128, ws, s);
+    }
+    if (out_dtype == MI355_F32) return launch_ksplit128<float, false>(ah, bh, (float*)c, m, n, k, n, split128, ws, s);
+    return launch_ksplit128<half_t, false>(ah, bh, (half_t*)c, m, n, k, n, split128, ws, s);
+  }
   if (bf) {
     if (out_dtype == MI355_F32) return launch_variant<float, true>(variant, a, b, c, (int)M, (int)N, (int)K, s, ws, wsb);
     return launch_variant<half_t, true>(variant, a, b, c, (int)M, (int)N, (int)K, s, ws, wsb);
@@ -1589,6 +1673,8 @@ static int64_t gemm_nt_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (M <= 0 || N <= 0 || K <= 0 || M > (1 << 30) || N > (1 << 30) || K > (1 << 21) || K < 256 || K % 128 != 0) return 0;
   if (M * K * 2 >= (1ll << 32) || N * K * 2 >= (1ll << 32)) return 0;  // the streamed kernel's one descriptor per operand
   if (M <= 64 && N % 32 == 0 && N >= 2048 && K >= 512) return 0;        // the weight-streaming kernel's shapes
+  const int s128 = (K % 64 == 0) ? ksplit128_plan((int)M, (int)N, (int)K) : 1;
+  if (s128 > 1) return (int64_t)s128 * M * N * 4;
   int sm, sn;
   const int S = ksplit_plan((int)M, (int)N, (int)K, sm, sn);
   return S > 1 ? (int64_t)S * sm * sn * 4 : 0;

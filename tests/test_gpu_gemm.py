@@ -482,11 +482,12 @@ def test_gemm_skinny_contract(dev):
 
 
 @pytest.mark.parametrize("out_dtype", ["float16", "float32"])
-@pytest.mark.parametrize("shape", [(2048, 10240, 8192), (10240, 2048, 6144), (2048, 4096, 8192), (512, 2048, 8192), (1024, 1024, 4096), (256, 2048, 8192)])
+@pytest.mark.parametrize("shape", [(2048, 10240, 8192), (10240, 2048, 6144), (2048, 4096, 8192), (512, 2048, 8192), (1024, 1024, 4096), (256, 2048, 8192),
+                                   (384, 640, 8192), (256, 256, 8192), (128, 128, 2048), (1024, 2048, 4096)])
 def test_gemm_k_split_with_workspace(dev, shape, out_dtype):
     """The workspace entry point through the C ABI: a strip of tile columns (2048 x 10240: the last 64 of 320 tiles, four
-    K ranges), a strip of tile rows (four ranges of 1536), and whole products of 128, 16, 16 and 8 tiles (two, eight,
-    four and eight ranges) -- the whole matrix against the plain entry point (same products, other summation order), sampled rows
+    K ranges), a strip of tile rows (four ranges of 1536), a whole product of 128 tiles of 256x256 (two ranges) and
+    small products that split on 128x128 tiles (2 to 16 ranges; one of them not a multiple of 256) -- the whole matrix against the plain entry point (same products, other summation order), sampled rows
     against an fp32 product; a workspace one byte short or absent runs exactly as the plain entry point does."""
     from iree_turbine_amd import _lib
     from oracle import inputs
@@ -514,7 +515,7 @@ def test_gemm_k_split_with_workspace(dev, shape, out_dtype):
     assert not torch.equal(split, plain) or out_dtype == "float16"  # another summation order: fp32 sums differ in the last bits
     tol = dict(rtol=1e-4, atol=1e-4) if out_dtype == "float32" else dict(rtol=2e-3, atol=1e-3)
     torch.testing.assert_close(split.float(), plain.float(), **tol)
-    rows = torch.tensor([0, 255, M - 256, M - 1], device=dev)
+    rows = torch.tensor([0, min(255, M - 1), max(M - 256, 0), M - 1], device=dev)  # sampled rows, inside the matrix for the small shapes too
     exact = a[rows].float() @ b.float().t()
     torch.testing.assert_close(split[rows].float(), exact, rtol=RTOL, atol=ATOL)
     assert torch.equal(run(ws.data_ptr(), need - 1), plain)
