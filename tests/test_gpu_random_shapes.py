@@ -53,11 +53,13 @@ def test_random_gemm_few_tiles_long_k(dev):
     lib = _lib.load()
     rng = random.Random(111)
     split = 0
-    for case in range(24):
+    for case in range(30):
         tm, tn = rng.randint(1, 12), rng.randint(1, 12)
         if case % 6 == 5:
             tm, tn = rng.choice([(8, 40), (40, 8), (16, 18), (9, 32)])  # a full round of tiles and a sparse one behind it
         M, N = 256 * tm, 256 * tn
+        if case % 3 == 1:
+            M, N = 128 * rng.randint(1, 9), 128 * rng.randint(1, 9)  # small products, odd multiples of 128 among them
         K = rng.choice([4096, 4224, 6144, 8192, 12288])
         dtype = rng.choice([torch.float16, torch.bfloat16])
         out_dtype = rng.choice(["float32", str(dtype).split(".")[1]])
