@@ -49,13 +49,13 @@ template <bool BF> struct OutPack<half_t, BF> {
   static __device__ __forceinline__ void store1(half_t* p, float a) { *p = cvt16<BF>(a); }
 };
 
-// Software-pipelined two-stage kernel: a BM x BN output tile per workgroup, slabs copied global -> LDS with
-// direct-to-LDS loads into a two-stage ring, 32x32x16 MFMAs.  The k-loop is
+// Software-pipelined kernel: a BM x BN output tile per workgroup, slabs copied global -> LDS with
+// direct-to-LDS loads into a ring of STAGES slabs, 32x32x16 MFMAs.  The k-loop is
 // rotated so that (a) the fragments of k-step s+1 are requested from LDS before the MFMAs of
 // k-step s issue, (b) the barrier that retires a slab sits in front of the last k-step's MFMAs,
 // which then overlap the first fragment reads of the next slab, and (c) the global -> LDS loads
-// for slab k+2 are issued right after that barrier into the stage that was just retired.
-template <int BM, int BN, int WM, int WN, typename OutT, bool BF>
+// for slab k+STAGES are issued right after that barrier into the stage that was just retired.
+template <int BM, int BN, int WM, int WN, typename OutT, bool BF, int STAGES = 2>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_t* __restrict__ A,
                                                                      const half_t* __restrict__ B,
                                                                      OutT* __restrict__ C, int M, int N, int K,
@@ -71,6 +71,10 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
   constexpr int A_GROUPS = BM / 8, B_GROUPS = BN / 8;
   static_assert(A_GROUPS % NW == 0 && B_GROUPS % NW == 0 && NW % 2 == 0, "loads must split evenly over an even number of waves");
   constexpr int LA = A_GROUPS / NW, LB = B_GROUPS / NW;
+  // A ring of STAGES slabs: slab s+STAGES is requested when slab s retires, so a load has STAGES-1 slab times to land,
+  // and the wait that retires a slab leaves the loads of the STAGES-2 newest slabs in flight (loads return in order).
+  static_assert(STAGES >= 2 && (STAGES & (STAGES - 1)) == 0 && (STAGES - 2) * (LA + LB) < 64, "ring depth");
+  constexpr int IN_FLIGHT = (STAGES - 2) * (LA + LB);
 
   extern __shared__ __attribute__((aligned(1024))) char lds[];
 
@@ -134,10 +138,11 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
   const int KT = K / 64;
   half8 fm0[TM], fn0[TN], fm1[TM], fn1[TN];
 
-  issue_loads(0, 0);
-  wait_vmcnt0();
-  __syncthreads();
-  issue_loads(1, KT > 1 ? 1 : 0);
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; s++) issue_loads(s, s < KT ? s : KT - 1);
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(IN_FLIGHT) : "memory");
+  __builtin_amdgcn_s_barrier();  // not __syncthreads(): its fence would wait for every load in flight
+  issue_loads(STAGES - 1, STAGES - 1 < KT ? STAGES - 1 : KT - 1);
   read_frags(lds, 0, fm0, fn0);
 
   // One k-step region: the MFMAs of the current fragments with the LDS reads of the next fragments
@@ -153,7 +158,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
   };
 
   for (int kt = 0; kt < KT; kt++) {
-    const char* st = lds + (kt & 1) * STAGE;
+    const char* st = lds + (kt & (STAGES - 1)) * STAGE;
     __builtin_amdgcn_sched_barrier(0);
     read_frags(st, 1, fm1, fn1);
     mfmas(fm0, fn0);
@@ -168,14 +173,14 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
     interleave();
     __builtin_amdgcn_sched_barrier(0);
     // retire the slab: every wave's LDS reads of this stage have returned, next slab has landed
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-    __syncthreads();
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(IN_FLIGHT) : "memory");
+    __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    // The MFMAs of the last k-step need nothing new, so they lead; the loads for slab kt+2 (into the
+    // The MFMAs of the last k-step need nothing new, so they lead; the loads for slab kt+STAGES (into the
     // stage just retired) and the first fragment reads of slab kt+1 are slotted in between them.
     // Past the end the loads re-fetch the last slab and the reads see stale bytes; neither is used.
-    issue_loads(kt & 1, kt + 2 < KT ? kt + 2 : KT - 1);
-    read_frags(lds + ((kt + 1) & 1) * STAGE, 0, fm0, fn0);
+    issue_loads(kt & (STAGES - 1), kt + STAGES < KT ? kt + STAGES : KT - 1);
+    read_frags(lds + ((kt + 1) & (STAGES - 1)) * STAGE, 0, fm0, fn0);
     mfmas(fm1, fn1);
     {
       constexpr int NL = LA + LB, NR = TM + TN, NM = TM * TN;
@@ -1345,44 +1350,62 @@ static int cu_count() {
   return cached[dev];
 }
 
+// The pipelined kernel's ring is two slabs deep where workgroups share a CU (more than 256 tiles: 64 KiB each, two fit)
+// and four slabs deep where each has a CU to itself and K is long: a lone workgroup's loads then have three slab times
+// to land instead of one (128 tiles of K = 4096: 39.7 -> 32.3 us; 64 tiles of K = 8192: 68.8 -> 58.9 us), while at
+// K = 1024 the longer prologue costs 0.3 us, and with 320 tiles the lost co-residency costs 20 %.
+static bool pipelined_deep_ring(long long tiles, int k_range) {
+  return tiles <= 256 && (k_range >= 4096 || (k_range >= 2048 && tiles > 128));
+}
+
 template <int BM, int BN, int WM, int WN, typename OutT, int KIND, bool BF>  // KIND: 1 pipelined, 2 register-staged
 static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int K, int ldc, hipStream_t stream) {
   // the kernels use their N argument only as the row stride of C, so a column range of a wider C is the
   // same launch with ldc in its place
   static_assert(KIND == 1 || KIND == 2, "pipelined or register-staged");
-  // the register-staged kernel keeps its epilogue out of the stages: 32 rows x 128 bytes per wave
-  constexpr int lds_bytes = 2 * (BM + BN) * 128 + (KIND == 2 ? WM * WN * 32 * 128 : 0);
-  static std::atomic<uint64_t> lds_ok{0};
   const int tiles_m = M / BM, tiles_n = N / BN;
   int group_m = 4;
   dim3 grid(tiles_m * tiles_n), block(WM * WN * 64);
   if constexpr (KIND == 2) {
+    // the register-staged kernel keeps its epilogue out of the stages: 32 rows x 128 bytes per wave
+    constexpr int lds_bytes = 2 * (BM + BN) * 128 + WM * WN * 32 * 128;
+    static std::atomic<uint64_t> lds_ok{0};
     auto kern = gemm_f16_nt_staged<BM, BN, WM, WN, OutT, BF>;
     if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt")) return rc;
     hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, M, ldc, K, tiles_m,
                        tiles_n, group_m);
+    return check_launch("gemm_f16_nt_staged", grid, block, lds_bytes);
   } else {
-    auto kern = gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT, BF>;
-    if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt")) return rc;
-    hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, M, ldc, K, tiles_m,
-                       tiles_n, group_m, K, 0, 0);
+    auto go = [&](auto kern, int lds_bytes, std::atomic<uint64_t>& lds_ok) {
+      if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt")) return rc;
+      hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, M, ldc, K, tiles_m,
+                         tiles_n, group_m, K, 0, 0);
+      return check_launch("gemm_f16_nt_pipelined", grid, block, lds_bytes);
+    };
+    static std::atomic<uint64_t> lds_ok2{0}, lds_ok4{0};
+    if (4 * (BM + BN) * 128 <= 160 * 1024 && pipelined_deep_ring((long long)tiles_m * tiles_n, K))
+      return go(gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT, BF, 4>, 4 * (BM + BN) * 128, lds_ok4);
+    return go(gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT, BF, 2>, 2 * (BM + BN) * 128, lds_ok2);
   }
-  return check_launch(KIND == 2 ? "gemm_f16_nt_staged" : "gemm_f16_nt_pipelined", grid, block, lds_bytes);
 }
 
 // K split on the pipelined 128x128 kernel, for products too small for 256x256 tiles to spread over the chip: S K ranges
-// of k_part each, fp32 partial tiles stacked along M in the workspace (row pitch N).
+// of k_part each, fp32 partial tiles stacked along M in the workspace (row pitch N).  At most 256 workgroups, so the
+// ring is four slabs deep from k_part = 1024 up (64 tiles of K = 4096 in four ranges: 24.0 -> 23.0 us; 128 tiles in
+// two: 32.1 -> 29.9 us; ranges of 512 lose 0.3 us to the longer prologue).
 template <bool BF>
 static int launch_pipelined_ksplit(const half_t* a, const half_t* b, float* ws, int M, int N, int K, int S, hipStream_t stream) {
-  auto kern = gemm_f16_nt_pipelined<128, 128, 2, 2, float, BF>;
-  constexpr int lds_bytes = 2 * (128 + 128) * 128;
-  static std::atomic<uint64_t> lds_ok{0};
-  if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt")) return rc;
   const int k_part = K / S;
   const int tiles_m = (M / 128) * S, tiles_n = N / 128;
   dim3 grid(tiles_m * tiles_n), block(256);
-  hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, a, b, ws, M * S, N, k_part, tiles_m, tiles_n, 4, K, M / 128, k_part);
-  return check_launch("gemm_f16_nt_pipelined (K split)", grid, block, lds_bytes);
+  auto go = [&](auto kern, int lds_bytes, std::atomic<uint64_t>& lds_ok) {
+    if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt")) return rc;
+    hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, a, b, ws, M * S, N, k_part, tiles_m, tiles_n, 4, K, M / 128, k_part);
+    return check_launch("gemm_f16_nt_pipelined (K split)", grid, block, lds_bytes);
+  };
+  static std::atomic<uint64_t> lds_ok2{0}, lds_ok4{0};
+  if (k_part >= 1024 && grid.x <= 256) return go(gemm_f16_nt_pipelined<128, 128, 2, 2, float, BF, 4>, 4 * 256 * 128, lds_ok4);
+  return go(gemm_f16_nt_pipelined<128, 128, 2, 2, float, BF, 2>, 2 * 256 * 128, lds_ok2);
 }
 
 template <int BM, int BN, int WM, int WN, typename OutT, bool BF>

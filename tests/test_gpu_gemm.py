@@ -206,6 +206,35 @@ def test_gemm_staged_slab_rotation(dev, shape, out_dtype):
     assert torch.equal(got, torch.ops.mi355.gemm_nt(a, b, out_dtype, v))
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("out32", [False, True])
+@pytest.mark.parametrize("shape", [(128, 128, 4096), (256, 384, 4160), (1024, 1024, 4096), (2048, 1536, 2048), (2048, 1536, 2112),
+                                   (2048, 2048, 8192), (2048, 2176, 4096), (128, 256, 1984)])
+def test_gemm_pipelined_ring_depth(dev, shape, out32, dtype):
+    """The 128x128 kernel's ring is four slabs deep when every workgroup has a CU to itself and K is long, two deep
+    otherwise: one tile, slab counts that are 0, 1 and 3 mod 4 (64, 65, 33, 31 slabs), tile counts on both sides of the
+    128 and 256 limits (192 tiles at K = 2048 take the deep ring, 272 at K = 4096 and anything at K < 2048 the shallow
+    one) -- whole matrix against the independent generic kernel, rows against fp32, launches repeat bit for bit."""
+    import iree_turbine_amd as ita
+
+    M, N, K = shape
+    announce(f"gemm pipelined ring {shape} {dtype} out32={out32}")
+    names = ita._lib.variants("gemm_f16_nt")
+    v = next(i for i, n in enumerate(names) if n.startswith("pipelined"))
+    g = torch.Generator().manual_seed(M + 3 * N + 7 * K)
+    a = (torch.randn(M, K, generator=g) * 0.25).to(dtype).to(dev)
+    b = (torch.randn(N, K, generator=g) * 0.25).to(dtype).to(dev)
+    out_dtype = "float32" if out32 else str(dtype).replace("torch.", "")
+    got = torch.ops.mi355.gemm_nt(a, b, out_dtype, v)
+    ref = torch.ops.mi355.gemm_nt(a, b, out_dtype, len(names) - 1)
+    tol = 1e-3 if (out32 or dtype == torch.float16) else 8e-3
+    torch.testing.assert_close(got.float(), ref.float(), rtol=tol, atol=tol * 4)
+    rows = torch.tensor([0, 63, 64, M - 1])
+    exact = a[rows.to(dev)].float() @ b.float().t()
+    torch.testing.assert_close(got[rows.to(dev)].float(), exact, rtol=RTOL, atol=ATOL)
+    assert torch.equal(got, torch.ops.mi355.gemm_nt(a, b, out_dtype, v))
+
+
 @pytest.mark.parametrize("out_dtype", ["float16", "float32"])
 @pytest.mark.parametrize("shape", [(256, 256, 256), (512, 768, 384), (1024, 512, 1152), (2048, 10240, 512), (4352, 4352, 640)])
 def test_gemm_stream_slab_rotation(dev, shape, out_dtype):
