@@ -92,7 +92,7 @@ int mi355_gemm_bf16_nt(const void* a, const void* b, void* c,
 /*
  * The same two GEMMs with a caller-provided workspace, which lets the automatic choice (variant < 0) split K:
  * a product with too few 256x256 tiles for the 256 CUs -- the whole product when it has at most 128 such tiles
- * (on 128x128 tiles when it is smaller still), or the strip a sparse last round of tiles is cut into -- is computed
+ * (on 128x128, 128x64 or 64x64 tiles when it is smaller still), or the strip a sparse last round of tiles is cut into -- is computed
  * as S partial products over K ranges (fp32, in the workspace) and one merge launch.  mi355_gemm_nt_workspace_bytes returns the size with which a shape would
  * take that path (0: it would not; the plain entry points do the same work then).  A NULL or smaller workspace is
  * not an error: the call runs as mi355_gemm_f16_nt would.  The workspace is scratch: nothing in it is read before

@@ -148,13 +148,17 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
   // One k-step region: the MFMAs of the current fragments with the LDS reads of the next fragments
   // slotted in between them (first instruction is an MFMA, so the wait in front of it only covers
   // reads issued a whole k-step earlier).
+  // (Tiles with fewer MFMAs per k-step than fragment reads are left to the compiler's own order.)
+  constexpr bool HAND_ORDER = TM * TN >= TM + TN;
   auto interleave = [&]() {
+    if constexpr (HAND_ORDER) {
 #pragma unroll
-    for (int i = 0; i < TM + TN; i++) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
+      for (int i = 0; i < TM + TN; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // 1 MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // 1 DS read
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
     }
-    __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
   };
 
   for (int kt = 0; kt < KT; kt++) {
@@ -182,7 +186,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
     issue_loads(kt & (STAGES - 1), kt + STAGES < KT ? kt + STAGES : KT - 1);
     read_frags(lds + ((kt + 1) & (STAGES - 1)) * STAGE, 0, fm0, fn0);
     mfmas(fm1, fn1);
-    {
+    if constexpr (HAND_ORDER) {
       constexpr int NL = LA + LB, NR = TM + TN, NM = TM * TN;
       constexpr int M_FOR_LOADS = NM / 2, L_PER_M = (NL + M_FOR_LOADS - 1) / M_FOR_LOADS;
 #pragma unroll
@@ -220,7 +224,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
           const int c = i * 4 + q;
           half4 v = {cvt16<BF>(acc[i][j][4 * q]), cvt16<BF>(acc[i][j][4 * q + 1]), cvt16<BF>(acc[i][j][4 * q + 2]),
                      cvt16<BF>(acc[i][j][4 * q + 3])};
-          *reinterpret_cast<half4*>(ep + ml * ROW_B + ((c ^ ((ml >> 1) & 7)) * 16) + 8 * h) = v;
+          *reinterpret_cast<half4*>(ep + ml * ROW_B + ((c ^ ((ml >> 1) & (CH - 1))) * 16) + 8 * h) = v;
         }
     }
     constexpr int ROWS_PER_IT = 64 / CH;
@@ -229,7 +233,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
 #pragma unroll
     for (int it = 0; it < WTM / ROWS_PER_IT; it++) {
       const int row = it * ROWS_PER_IT + er;
-      half8 v = *reinterpret_cast<const half8*>(ep + row * ROW_B + ((ec ^ ((row >> 1) & 7)) * 16));
+      half8 v = *reinterpret_cast<const half8*>(ep + row * ROW_B + ((ec ^ ((row >> 1) & (CH - 1))) * 16));
       *reinterpret_cast<half8*>(cbase + (size_t)row * N) = v;
     }
   } else {
@@ -1328,10 +1332,13 @@ static const GemmVariant kGemmVariants[] = {
     {"stream_256x256x64_w2x2", 256, 256, 256},
     {"stream_256x256_tail_128x128", 256, 256, 256},
     {"stream_256x256x64_w2x2_walk", 256, 256, 256},
+    {"pipelined_64x64x64_w2x2", 64, 64, 256},
+    {"pipelined_128x64x64_w2x2", 128, 64, 256},
     {"generic_64x64x32", 64, 64, 256},
 };
 // indices of the table above
-enum { V_PERSISTENT = 0, V_PIPELINED_128 = 1, V_STAGED = 2, V_SKINNY = 3, V_STREAM = 4, V_STREAM_TAIL = 5, V_STREAM_WALK = 6 };
+enum { V_PERSISTENT = 0, V_PIPELINED_128 = 1, V_STAGED = 2, V_SKINNY = 3, V_STREAM = 4, V_STREAM_TAIL = 5, V_STREAM_WALK = 6,
+       V_PIPELINED_64 = 7, V_PIPELINED_128x64 = 8 };
 constexpr int kNumGemmVariants = sizeof(kGemmVariants) / sizeof(kGemmVariants[0]);
 
 int gemm_variant_count() { return kNumGemmVariants; }
@@ -1353,7 +1360,8 @@ static int cu_count() {
 // The pipelined kernel's ring is two slabs deep where workgroups share a CU (more than 256 tiles: 64 KiB each, two fit)
 // and four slabs deep where each has a CU to itself and K is long: a lone workgroup's loads then have three slab times
 // to land instead of one (128 tiles of K = 4096: 39.7 -> 32.3 us; 64 tiles of K = 8192: 68.8 -> 58.9 us), while at
-// K = 1024 the longer prologue costs 0.3 us, and with 320 tiles the lost co-residency costs 20 %.
+// K = 1024 the longer prologue costs 0.3 us, and with 320 tiles the lost co-residency costs 20 %.  The smaller tiles
+// need it as much once the operands outgrow an L2 (256 tiles of 64x64 at K = 4096, 16 MiB: 30.5 -> 17.8 us).
 static bool pipelined_deep_ring(long long tiles, int k_range) {
   return tiles <= 256 && (k_range >= 4096 || (k_range >= 2048 && tiles > 128));
 }
@@ -1383,7 +1391,8 @@ static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int
       return check_launch("gemm_f16_nt_pipelined", grid, block, lds_bytes);
     };
     static std::atomic<uint64_t> lds_ok2{0}, lds_ok4{0};
-    if (4 * (BM + BN) * 128 <= 160 * 1024 && pipelined_deep_ring((long long)tiles_m * tiles_n, K))
+    static_assert(4 * (BM + BN) * 128 <= 160 * 1024, "four slabs of the tile fit in LDS");
+    if (pipelined_deep_ring((long long)tiles_m * tiles_n, K))
       return go(gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT, BF, 4>, 4 * (BM + BN) * 128, lds_ok4);
     return go(gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT, BF, 2>, 2 * (BM + BN) * 128, lds_ok2);
   }
@@ -1393,19 +1402,20 @@ static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int
 // of k_part each, fp32 partial tiles stacked along M in the workspace (row pitch N).  At most 256 workgroups, so the
 // ring is four slabs deep from k_part = 1024 up (64 tiles of K = 4096 in four ranges: 24.0 -> 23.0 us; 128 tiles in
 // two: 32.1 -> 29.9 us; ranges of 512 lose 0.3 us to the longer prologue).
-template <bool BF>
+template <bool BF, int BM = 128, int BN = 128>
 static int launch_pipelined_ksplit(const half_t* a, const half_t* b, float* ws, int M, int N, int K, int S, hipStream_t stream) {
   const int k_part = K / S;
-  const int tiles_m = (M / 128) * S, tiles_n = N / 128;
+  const int tiles_m = (M / BM) * S, tiles_n = N / BN;
   dim3 grid(tiles_m * tiles_n), block(256);
   auto go = [&](auto kern, int lds_bytes, std::atomic<uint64_t>& lds_ok) {
     if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt")) return rc;
-    hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, a, b, ws, M * S, N, k_part, tiles_m, tiles_n, 4, K, M / 128, k_part);
+    hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, a, b, ws, M * S, N, k_part, tiles_m, tiles_n, 4, K, M / BM, k_part);
     return check_launch("gemm_f16_nt_pipelined (K split)", grid, block, lds_bytes);
   };
   static std::atomic<uint64_t> lds_ok2{0}, lds_ok4{0};
-  if (k_part >= 1024 && grid.x <= 256) return go(gemm_f16_nt_pipelined<128, 128, 2, 2, float, BF, 4>, 4 * 256 * 128, lds_ok4);
-  return go(gemm_f16_nt_pipelined<128, 128, 2, 2, float, BF, 2>, 2 * 256 * 128, lds_ok2);
+  if (k_part >= (BM + BN == 256 ? 1024 : 2048) && grid.x <= 256)
+    return go(gemm_f16_nt_pipelined<BM, BN, 2, 2, float, BF, 4>, 4 * (BM + BN) * 128, lds_ok4);
+  return go(gemm_f16_nt_pipelined<BM, BN, 2, 2, float, BF, 2>, 2 * (BM + BN) * 128, lds_ok2);
 }
 
 template <int BM, int BN, int WM, int WN, typename OutT, bool BF>
@@ -1489,9 +1499,9 @@ static int launch_ksplit(const half_t* a, const half_t* b, OutT* c, int M, int N
   return check_launch("gemm_ksplit_merge", grid, block, 0);
 }
 
-template <typename OutT, bool BF>
+template <typename OutT, bool BF, int BM = 128, int BN = 128>
 static int launch_ksplit128(const half_t* a, const half_t* b, OutT* c, int M, int N, int K, int ldc, int S, float* ws, hipStream_t stream) {
-  if (int rc = launch_pipelined_ksplit<BF>(a, b, ws, M, N, K, S, stream)) return rc;
+  if (int rc = launch_pipelined_ksplit<BF, BM, BN>(a, b, ws, M, N, K, S, stream)) return rc;
   const long long lanes = (long long)M * N / 4;
   dim3 grid((unsigned)((lanes + 255) / 256)), block(256);
   hipLaunchKernelGGL((gemm_ksplit_merge<OutT, BF>), grid, block, 0, stream, (const float*)ws, c, M, N, ldc, S);
@@ -1505,20 +1515,47 @@ static int launch_ksplit128(const half_t* a, const half_t* b, OutT* c, int M, in
 // from K = 1024, nor beyond 64 tiles except for 4096 <= K < 6144, where two ranges are level to ahead of the 256x256
 // split (1024x2048x4096: 31.9 against 36.0).
 static int ksplit128_factor(long long t128, int K) {
-  if (K < 2048 || K % 128 != 0) return 1;
-  if (t128 > 64) return (t128 <= 160 && K >= 4096 && K < 6144) ? 2 : 1;
-  if (t128 > 48 && K < 4096) return 1;
-  int s = 1;
-  while (s < 16) {
-    const int n = 2 * s;
-    const long long units = t128 * n;
-    if (units > 256 || K % (64 * n) != 0 || K / n < (units <= 64 ? 512 : 1024)) break;
-    s = n;
-  }
-  return s;
+  if (K % 128 != 0) return 1;
+  return (t128 > 128 && t128 <= 160 && K >= 4096 && K < 6144) ? 2 : 1;  // up to 128 tiles: small_plan below
 }
 
-// S for a whole product on 128x128 tiles under the automatic choice (1: none)
+// Products of at most 128 tiles of 128x128 (M * N <= 2 Mi): the tile shape and the K split that a cost model prices
+// lowest.  One workgroup per CU pulls its operands at about 75 GB/s whatever the tile shape (a 64x64 tile takes 0.22 us
+// per 64-wide slab, 128x64 0.31, 128x128 0.44 with the deep ring and 0.60 without), so the time of a launch is its fixed
+// part (3.0 us: launch, first loads, epilogue) plus the bytes the busiest CU pulls, and what shortens it is more CUs at
+// work: smaller tiles (more operand bytes in total, which the L2s serve) or K ranges (a merge launch: 2.8 us plus the
+// partial tiles written and read at about 4 TB/s).  Against a sweep of 25 shapes (256^2 to 1024x2048, K 512 to 8192,
+// three tile shapes, 1 to 16 ranges) the model's times are within 10 % and its choice within 2 % of the best measured
+// one, but for two shapes at K = 8192 (9 and 11 %).  1024^3: 10.4 -> 6.7 us (vendor library 8.0); 512x512x4096: 15.8 ->
+// 11.2 (10.3); 1024x2048x2048: 18.3 -> 13.6 (14.8); 1024x1024x4096: 21.1 -> 17.8 (17.7).
+struct SmallPlan {
+  int bm = 0, bn = 0, S = 1;  // bm == 0: not a small product
+};
+static SmallPlan small_plan(int64_t M, int64_t N, int64_t K, int64_t ws_bytes) {
+  SmallPlan best;
+  if (M % 64 || N % 64 || K % 64 || M * N > (1ll << 21) || K > (1 << 21)) return best;
+  double best_us = 0;
+  static const int kTiles[3][2] = {{64, 64}, {128, 64}, {128, 128}};
+  for (const auto& t : kTiles) {
+    const int bm = t[0], bn = t[1];
+    if (M % bm || N % bn) continue;
+    const int64_t tiles = (M / bm) * (N / bn);
+    for (int S = 1; S <= 8; S *= 2) {
+      const int64_t units = tiles * S, k_part = K / S;
+      if (units > 512 || K % (64 * S)) break;
+      if (S > 1 && (k_part < 512 || S * M * N * 4 > ws_bytes)) break;
+      const bool deep = bm + bn == 256 && (S > 1 ? k_part >= 1024 && units <= 256 : pipelined_deep_ring(units, (int)k_part));
+      const double per_cu_kib = (double)((units + 255) / 256) * (bm + bn) * 2 * k_part / 1024.0;
+      double us = 3.0 + per_cu_kib * ((bm + bn == 256 && !deep) ? 0.0188 : 0.0137);
+      if (S > 1) us += 2.8 + (double)S * M * N * 8 / 4e6;
+      if (best.bm == 0 || us < best_us) {
+        best_us = us;
+        best.bm = bm, best.bn = bn, best.S = S;
+      }
+    }
+  }
+  return best;
+}
 static int ksplit128_plan(int M, int N, int K) {
   if (M % 128 || N % 128) return 1;
   return ksplit128_factor((long long)(M / 128) * (N / 128), K);
@@ -1595,6 +1632,8 @@ static int launch_variant(int variant, const void* a, const void* b, void* c, in
     case V_STREAM: return launch_stream<OutT, BF>(a, b, c, M, N, K, N, stream);
     case V_STREAM_TAIL: return launch_split<OutT, BF>(a, b, c, M, N, K, stream, ws, ws_bytes);
     case V_STREAM_WALK: return launch_stream<OutT, BF>(a, b, c, M, N, K, N, stream, true);
+    case V_PIPELINED_64: return launch_tiled<64, 64, 2, 2, OutT, 1, BF>(a, b, c, M, N, K, N, stream);
+    case V_PIPELINED_128x64: return launch_tiled<128, 64, 2, 2, OutT, 1, BF>(a, b, c, M, N, K, N, stream);
     default: {
       dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
       hipLaunchKernelGGL((gemm_f16_nt_generic<OutT, BF>), grid, block, 0, stream, (const half_t*)a, (const half_t*)b, (OutT*)c,
@@ -1631,6 +1670,7 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
     return al && M % kGemmVariants[v].bm == 0 && N % kGemmVariants[v].bn == 0 && K % 64 == 0;
   };
   int split128 = 1;  // K ranges of the 128x128 split, when the automatic choice takes it
+  SmallPlan small;   // tile shape and K ranges of a small product, when the automatic choice takes it
   if (variant < 0) {
     // Large problems take the 256x256 tile; when that leaves most of the 256 CUs idle the
     // 128x128 tile (4x the workgroups) wins; everything else goes to the bounds-checked kernel.
@@ -1644,6 +1684,11 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
     const bool full_rounds = t256 * 100 >= rounds * 256 * 85;
     const int s128 = (workspace && fits(V_PIPELINED_128)) ? ksplit128_plan((int)M, (int)N, (int)K) : 1;
     if (fits(V_SKINNY) && N >= 2048 && K >= 512) variant = V_SKINNY;  // decode-shaped: stream the weights once
+    else if (al && (small = small_plan(M, N, K, INT64_MAX)).bm) {
+      // a workspace short of what the plan asks for is no workspace (not a plan with fewer ranges)
+      if (small.S > 1 && (!workspace || workspace_bytes < (int64_t)small.S * M * N * 4)) small = small_plan(M, N, K, 0);
+      variant = small.bm == 64 ? V_PIPELINED_64 : small.bn == 64 ? V_PIPELINED_128x64 : V_PIPELINED_128;
+    }
     else if (s128 > 1 && workspace_bytes >= (int64_t)s128 * M * N * 4) {  // a small product: K split on 128x128 tiles
       variant = V_PIPELINED_128;
       split128 = s128;
@@ -1673,6 +1718,19 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
   float* ws = static_cast<float*>(workspace);
   const size_t wsb = workspace_bytes > 0 ? (size_t)workspace_bytes : 0;
   if (ws && !aligned16(ws)) return fail(-MI355_E_ALIGN, "gemm_f16_nt: workspace must be 16-byte aligned");
+  if (small.S > 1) {
+    const half_t *ah = (const half_t*)a, *bh = (const half_t*)b;
+    const int m = (int)M, n = (int)N, k = (int)K, S = small.S;
+    auto tiled = [&](auto out, auto is_bf) {
+      using OutT = decltype(out);
+      constexpr bool BF = decltype(is_bf)::value;
+      if (small.bm == 64) return launch_ksplit128<OutT, BF, 64, 64>(ah, bh, (OutT*)c, m, n, k, n, S, ws, s);
+      if (small.bn == 64) return launch_ksplit128<OutT, BF, 128, 64>(ah, bh, (OutT*)c, m, n, k, n, S, ws, s);
+      return launch_ksplit128<OutT, BF, 128, 128>(ah, bh, (OutT*)c, m, n, k, n, S, ws, s);
+    };
+    if (bf) return out_dtype == MI355_F32 ? tiled(float{}, std::true_type{}) : tiled(half_t{}, std::true_type{});
+    return out_dtype == MI355_F32 ? tiled(float{}, std::false_type{}) : tiled(half_t{}, std::false_type{});
+  }
   if (split128 > 1) {
     const half_t *ah = (const half_t*)a, *bh = (const half_t*)b;
     const int m = (int)M, n = (int)N, k = (int)K;
@@ -1696,6 +1754,8 @@ static int64_t gemm_nt_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (M <= 0 || N <= 0 || K <= 0 || M > (1 << 30) || N > (1 << 30) || K > (1 << 21) || K < 256 || K % 128 != 0) return 0;
   if (M * K * 2 >= (1ll << 32) || N * K * 2 >= (1ll << 32)) return 0;  // the streamed kernel's one descriptor per operand
   if (M <= 64 && N % 32 == 0 && N >= 2048 && K >= 512) return 0;        // the weight-streaming kernel's shapes
+  const SmallPlan sp = small_plan(M, N, K, INT64_MAX);
+  if (sp.bm) return sp.S > 1 ? (int64_t)sp.S * M * N * 4 : 0;
   const int s128 = (K % 64 == 0) ? ksplit128_plan((int)M, (int)N, (int)K) : 1;
   if (s128 > 1) return (int64_t)s128 * M * N * 4;
   int sm, sn;

@@ -22,7 +22,7 @@ def _run(dev, M, N, K, out_dtype, variant=-1, seed=10):
     return c.float().cpu(), ref
 
 
-@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 4, 5, 6])  # every tiled kernel (3 is the skinny-M kernel, 7 the any-shape one)
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 4, 5, 6, 7, 8])  # every tiled kernel (3 is the skinny-M kernel, 9 the any-shape one)
 def test_gemm_1024_f32_all_variants(dev, variant):
     c, ref = _run(dev, 1024, 1024, 1024, "float32", variant)
     torch.testing.assert_close(c, ref, rtol=RTOL, atol=ATOL)
@@ -233,6 +233,36 @@ def test_gemm_pipelined_ring_depth(dev, shape, out32, dtype):
     exact = a[rows.to(dev)].float() @ b.float().t()
     torch.testing.assert_close(got[rows.to(dev)].float(), exact, rtol=RTOL, atol=ATOL)
     assert torch.equal(got, torch.ops.mi355.gemm_nt(a, b, out_dtype, v))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("out32", [False, True])
+@pytest.mark.parametrize("shape", [(64, 64, 64), (128, 64, 128), (192, 320, 1024), (1024, 1024, 1024), (512, 512, 4096), (1024, 2048, 2048),
+                                   (320, 448, 2560), (1024, 1024, 4096), (1024, 2048, 512), (64, 1024, 192), (1408, 1408, 1024)])
+def test_gemm_small_products(dev, shape, out32, dtype):
+    """Products of at most 128 tiles of 128x128 take 64x64, 128x64 or 128x128 tiles and one to eight K ranges by a cost
+    model: one tile and one slab, two and three slabs (shorter than the ring), shapes that are no multiple of 128, each
+    tile shape with and without a split, the largest size of the rule and the first beyond it (1408^2) -- the automatic
+    choice through the op (which brings the workspace) and the two small-tile kernels by index, whole matrix against the
+    independent generic kernel, rows against fp32, launches repeat bit for bit."""
+    import iree_turbine_amd as ita
+
+    M, N, K = shape
+    announce(f"gemm small product {shape} {dtype} out32={out32}")
+    names = ita._lib.variants("gemm_f16_nt")
+    g = torch.Generator().manual_seed(5 * M + 3 * N + K)
+    a = (torch.randn(M, K, generator=g) * 0.25).to(dtype).to(dev)
+    b = (torch.randn(N, K, generator=g) * 0.25).to(dtype).to(dev)
+    out_dtype = "float32" if out32 else str(dtype).replace("torch.", "")
+    ref = torch.ops.mi355.gemm_nt(a, b, out_dtype, len(names) - 1)
+    rows = torch.tensor([0, 63, M - 64, M - 1], device=dev)
+    exact = a[rows].float() @ b.float().t()
+    tol = 1e-3 if (out32 or dtype == torch.float16) else 8e-3
+    for v in [-1, names.index("pipelined_64x64x64_w2x2")] + ([names.index("pipelined_128x64x64_w2x2")] if M % 128 == 0 else []):
+        got = torch.ops.mi355.gemm_nt(a, b, out_dtype, v)
+        torch.testing.assert_close(got.float(), ref.float(), rtol=tol, atol=tol * 4)
+        torch.testing.assert_close(got[rows].float(), exact, rtol=RTOL, atol=ATOL)
+        assert torch.equal(got, torch.ops.mi355.gemm_nt(a, b, out_dtype, v))
 
 
 @pytest.mark.parametrize("out_dtype", ["float16", "float32"])
@@ -511,12 +541,15 @@ def test_gemm_skinny_contract(dev):
 
 
 @pytest.mark.parametrize("out_dtype", ["float16", "float32"])
-@pytest.mark.parametrize("shape", [(2048, 10240, 8192), (10240, 2048, 6144), (2048, 4096, 8192), (512, 2048, 8192), (1024, 1024, 4096), (256, 2048, 8192),
-                                   (384, 640, 8192), (256, 256, 8192), (128, 128, 2048), (1024, 2048, 4096)])
+@pytest.mark.parametrize("shape", [(2048, 10240, 8192), (10240, 2048, 6144), (2048, 4096, 8192), (512, 2048, 8192), (1024, 1024, 8192), (256, 2048, 8192),
+                                   (384, 640, 8192), (256, 256, 8192), (128, 128, 2048), (1024, 2048, 8192), (512, 1024, 4096), (64, 1024, 4096),
+                                   (2048, 1280, 4096)])
 def test_gemm_k_split_with_workspace(dev, shape, out_dtype):
     """The workspace entry point through the C ABI: a strip of tile columns (2048 x 10240: the last 64 of 320 tiles, four
-    K ranges), a strip of tile rows (four ranges of 1536), a whole product of 128 tiles of 256x256 (two ranges) and
-    small products that split on 128x128 tiles (2 to 16 ranges; one of them not a multiple of 256) -- the whole matrix against the plain entry point (same products, other summation order), sampled rows
+    K ranges), a strip of tile rows (four ranges of 1536), a whole product of 128 tiles of 256x256 (two ranges), small
+    products that split on 128x128 tiles (four and two ranges), on 128x64 tiles (256 x 2048: four ranges) and on 64x64
+    tiles (two, four and eight ranges; one shape no multiple of 128, one a single tile row) and 160 tiles of 128x128 in
+    two ranges -- the whole matrix against the plain entry point (same products, other summation order), sampled rows
     against an fp32 product; a workspace one byte short or absent runs exactly as the plain entry point does."""
     from iree_turbine_amd import _lib
     from oracle import inputs
