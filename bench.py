@@ -52,7 +52,7 @@ MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
     "gemm_4096": 2.438e8,
     "gemm_2048x10240x8192": 6.973e8,   # of which 128 MiB are the strip's fp32 partial products, written and read once
     "gemm_2048x57344x8192": 3.062e9,
-    "gemm_1024_f32out": 1.684e7,
+    "gemm_1024_f32out": 1.681e7,
     "gemm_bf16_8192": 1.754e9,
     "gemm_16x8192x8192": 1.366e8,
     "gemm_1024x8192x8192": 3.644e8,
