@@ -50,12 +50,19 @@ template <bool BF> struct OutPack<half_t, BF> {
 };
 
 // Software-pipelined kernel: a BM x BN output tile per workgroup, slabs copied global -> LDS with
-// direct-to-LDS loads into a ring of STAGES slabs, 32x32x16 MFMAs.  The k-loop is
-// rotated so that (a) the fragments of k-step s+1 are requested from LDS before the MFMAs of
-// k-step s issue, (b) the barrier that retires a slab sits in front of the last k-step's MFMAs,
-// which then overlap the first fragment reads of the next slab, and (c) the global -> LDS loads
-// for slab k+STAGES are issued right after that barrier into the stage that was just retired.
-template <int BM, int BN, int WM, int WN, typename OutT, bool BF, int STAGES = 2>
+// direct-to-LDS loads into a ring of slabs, 32x32x16 MFMAs.  Two forms of the k-loop:
+//  * k-step pipeline, two slabs (SLAB = false; more than 256 tiles of 128x128, where two workgroups of 64 KiB share a
+//    CU): the loop is rotated so that (a) the fragments of k-step s+1 are requested from LDS before the MFMAs of
+//    k-step s issue, (b) the barrier that retires a slab sits in front of the last k-step's MFMAs, which then overlap
+//    the first fragment reads of the next slab, and (c) the global -> LDS loads for slab k+2 are issued right after
+//    that barrier into the stage that was just retired.  A load has one slab time to land.
+//  * slab pipeline, four slabs (SLAB = true; a workgroup with a CU to itself, and the small tiles): the fragments of
+//    a whole slab sit in one of two register sets, so a trip has one wait, in front of its barrier; the reads of slab
+//    s+1 and the loads of slab s+4 are slotted between the MFMAs of slab s, and a load has three slab times to land.
+//    A lone workgroup's slab time in the k-step form is its load latency plus, on small tiles, the chain of LDS read
+//    latencies of four k-steps with one or two MFMAs each to cover them: 64x64 0.22 -> 0.15 us per slab, 128x128
+//    0.60 -> 0.42 (what LDS bandwidth allows); 1024^3 on 64x64 tiles 6.7 -> 5.4 us, 1024x1024x4096 19.4 -> 15.9 us.
+template <int BM, int BN, int WM, int WN, typename OutT, bool BF, bool SLAB = false>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_t* __restrict__ A,
                                                                      const half_t* __restrict__ B,
                                                                      OutT* __restrict__ C, int M, int N, int K,
@@ -73,7 +80,8 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
   constexpr int LA = A_GROUPS / NW, LB = B_GROUPS / NW;
   // A ring of STAGES slabs: slab s+STAGES is requested when slab s retires, so a load has STAGES-1 slab times to land,
   // and the wait that retires a slab leaves the loads of the STAGES-2 newest slabs in flight (loads return in order).
-  static_assert(STAGES >= 2 && (STAGES & (STAGES - 1)) == 0 && (STAGES - 2) * (LA + LB) < 64, "ring depth");
+  constexpr int STAGES = SLAB ? 4 : 2;
+  static_assert((STAGES - 2) * (LA + LB) < 64, "the load counter has six bits");
   constexpr int IN_FLIGHT = (STAGES - 2) * (LA + LB);
 
   extern __shared__ __attribute__((aligned(1024))) char lds[];
@@ -136,6 +144,49 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
   };
 
   const int KT = K / 64;
+  if constexpr (SLAB) {
+    // The stage slab s left is free at the start of trip s: every wave read it into registers a trip ago.
+    half8 am[2][4][TM], an[2][4][TN];
+    auto read_slab = [&](const char* st, half8(*fm)[TM], half8(*fn)[TN]) {
+#pragma unroll
+      for (int ks = 0; ks < 4; ks++) read_frags(st, ks, fm[ks], fn[ks]);
+    };
+    auto mfma_slab = [&](const half8(*fm)[TM], const half8(*fn)[TN]) {
+#pragma unroll
+      for (int ks = 0; ks < 4; ks++) mfmas(fm[ks], fn[ks]);
+    };
+    constexpr int NM = 4 * TM * TN, NR = 4 * (TM + TN), NL = LA + LB;
+    constexpr int R_PER_M = (NR + NM - 1) / NM, L_PER_M = (NL + NM - 1) / NM;
+    auto trip = [&](int kt, half8(*cm)[TM], half8(*cn)[TN], half8(*nm)[TM], half8(*nn)[TN]) {
+      __builtin_amdgcn_sched_barrier(0);
+      read_slab(lds + ((kt + 1) & (STAGES - 1)) * STAGE, nm, nn);
+      issue_loads(kt & (STAGES - 1), kt + STAGES < KT ? kt + STAGES : KT - 1);
+      mfma_slab(cm, cn);
+#pragma unroll
+      for (int i = 0; i < NM; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, R_PER_M, 0);
+        __builtin_amdgcn_sched_group_barrier(0x010, L_PER_M, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(IN_FLIGHT) : "memory");
+      __builtin_amdgcn_s_barrier();
+    };
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; s++) issue_loads(s, s < KT ? s : KT - 1);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(IN_FLIGHT) : "memory");
+    __builtin_amdgcn_s_barrier();
+    read_slab(lds, am[0], an[0]);
+    issue_loads(STAGES - 1, STAGES - 1 < KT ? STAGES - 1 : KT - 1);
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(IN_FLIGHT) : "memory");
+    __builtin_amdgcn_s_barrier();
+    int kt = 0;
+    for (; kt + 2 <= KT; kt += 2) {
+      trip(kt, am[0], an[0], am[1], an[1]);
+      trip(kt + 1, am[1], an[1], am[0], an[0]);
+    }
+    if (kt < KT) trip(kt, am[0], an[0], am[1], an[1]);
+  } else {
   half8 fm0[TM], fn0[TN], fm1[TM], fn1[TN];
 
 #pragma unroll
@@ -203,6 +254,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
+  }
   }
   // the speculative loads of the last iterations target LDS: drain them before the epilogue reuses it
   wait_vmcnt0();
@@ -1357,14 +1409,10 @@ static int cu_count() {
   return cached[dev];
 }
 
-// The pipelined kernel's ring is two slabs deep where workgroups share a CU (more than 256 tiles: 64 KiB each, two fit)
-// and four slabs deep where each has a CU to itself and K is long: a lone workgroup's loads then have three slab times
-// to land instead of one (128 tiles of K = 4096: 39.7 -> 32.3 us; 64 tiles of K = 8192: 68.8 -> 58.9 us), while at
-// K = 1024 the longer prologue costs 0.3 us, and with 320 tiles the lost co-residency costs 20 %.  The smaller tiles
-// need it as much once the operands outgrow an L2 (256 tiles of 64x64 at K = 4096, 16 MiB: 30.5 -> 17.8 us).
-static bool pipelined_deep_ring(long long tiles, int k_range) {
-  return tiles <= 256 && (k_range >= 4096 || (k_range >= 2048 && tiles > 128));
-}
+// The pipelined kernel's slab form needs 128 bytes of LDS per tile row and column four times over: the 128x128 tile
+// takes it when every workgroup has a CU to itself (with 320 tiles the lost co-residency costs 20 %), the smaller
+// tiles (64 and 96 KiB: two and one workgroup per CU) always.
+static bool pipelined_slab_form(long long tiles, int bm_plus_bn) { return bm_plus_bn < 256 || tiles <= 256; }
 
 template <int BM, int BN, int WM, int WN, typename OutT, int KIND, bool BF>  // KIND: 1 pipelined, 2 register-staged
 static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int K, int ldc, hipStream_t stream) {
@@ -1392,16 +1440,14 @@ static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int
     };
     static std::atomic<uint64_t> lds_ok2{0}, lds_ok4{0};
     static_assert(4 * (BM + BN) * 128 <= 160 * 1024, "four slabs of the tile fit in LDS");
-    if (pipelined_deep_ring((long long)tiles_m * tiles_n, K))
-      return go(gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT, BF, 4>, 4 * (BM + BN) * 128, lds_ok4);
-    return go(gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT, BF, 2>, 2 * (BM + BN) * 128, lds_ok2);
+    if (pipelined_slab_form((long long)tiles_m * tiles_n, BM + BN))
+      return go(gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT, BF, true>, 4 * (BM + BN) * 128, lds_ok4);
+    return go(gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT, BF, false>, 2 * (BM + BN) * 128, lds_ok2);
   }
 }
 
-// K split on the pipelined 128x128 kernel, for products too small for 256x256 tiles to spread over the chip: S K ranges
-// of k_part each, fp32 partial tiles stacked along M in the workspace (row pitch N).  At most 256 workgroups, so the
-// ring is four slabs deep from k_part = 1024 up (64 tiles of K = 4096 in four ranges: 24.0 -> 23.0 us; 128 tiles in
-// two: 32.1 -> 29.9 us; ranges of 512 lose 0.3 us to the longer prologue).
+// K split on the pipelined kernel, for products too small for 256x256 tiles to spread over the chip: S K ranges
+// of k_part each, fp32 partial tiles stacked along M in the workspace (row pitch N).
 template <bool BF, int BM = 128, int BN = 128>
 static int launch_pipelined_ksplit(const half_t* a, const half_t* b, float* ws, int M, int N, int K, int S, hipStream_t stream) {
   const int k_part = K / S;
@@ -1413,9 +1459,8 @@ static int launch_pipelined_ksplit(const half_t* a, const half_t* b, float* ws, 
     return check_launch("gemm_f16_nt_pipelined (K split)", grid, block, lds_bytes);
   };
   static std::atomic<uint64_t> lds_ok2{0}, lds_ok4{0};
-  if (k_part >= (BM + BN == 256 ? 1024 : 2048) && grid.x <= 256)
-    return go(gemm_f16_nt_pipelined<BM, BN, 2, 2, float, BF, 4>, 4 * (BM + BN) * 128, lds_ok4);
-  return go(gemm_f16_nt_pipelined<BM, BN, 2, 2, float, BF, 2>, 2 * (BM + BN) * 128, lds_ok2);
+  if (pipelined_slab_form(grid.x, BM + BN)) return go(gemm_f16_nt_pipelined<BM, BN, 2, 2, float, BF, true>, 4 * (BM + BN) * 128, lds_ok4);
+  return go(gemm_f16_nt_pipelined<BM, BN, 2, 2, float, BF, false>, 2 * (BM + BN) * 128, lds_ok2);
 }
 
 template <int BM, int BN, int WM, int WN, typename OutT, bool BF>
@@ -1520,14 +1565,16 @@ static int ksplit128_factor(long long t128, int K) {
 }
 
 // Products of at most 128 tiles of 128x128 (M * N <= 2 Mi): the tile shape and the K split that a cost model prices
-// lowest.  One workgroup per CU pulls its operands at about 75 GB/s whatever the tile shape (a 64x64 tile takes 0.22 us
-// per 64-wide slab, 128x64 0.31, 128x128 0.44 with the deep ring and 0.60 without), so the time of a launch is its fixed
-// part (3.0 us: launch, first loads, epilogue) plus the bytes the busiest CU pulls, and what shortens it is more CUs at
-// work: smaller tiles (more operand bytes in total, which the L2s serve) or K ranges (a merge launch: 2.8 us plus the
-// partial tiles written and read at about 4 TB/s).  Against a sweep of 25 shapes (256^2 to 1024x2048, K 512 to 8192,
-// three tile shapes, 1 to 16 ranges) the model's times are within 10 % and its choice within 2 % of the best measured
-// one, but for two shapes at K = 8192 (9 and 11 %).  1024^3: 10.4 -> 6.7 us (vendor library 8.0); 512x512x4096: 15.8 ->
-// 11.2 (10.3); 1024x2048x2048: 18.3 -> 13.6 (14.8); 1024x1024x4096: 21.1 -> 17.8 (17.7).
+// lowest.  These launches are bound by what their busiest CU moves through its LDS: per 64-wide slab a workgroup writes
+// (BM + BN) * 128 bytes into LDS and its four waves read twice that back, at 128 bytes per clock: 0.15 us on a 64x64
+// tile, 0.25 on 128x64, 0.42 on 128x128 (0.20 / 0.33 / 0.42 with all 256 CUs asking the L2s at once) against 0.05 /
+// 0.11 / 0.21 us of MFMA work.  So the time of a launch is its fixed part (2.5 us: launch, first loads, epilogue) plus
+// the operand bytes of its busiest CU at that rate, and what shortens it is more CUs at work: smaller tiles (more
+// operand bytes in total, which the L2s serve) or K ranges (a merge launch: 2.3 us plus the partial tiles written and
+// read at about 4.5 TB/s, half that beyond 8 MiB).  Against a sweep of 30 shapes (256^2 to 1408^2 and 1024x2048,
+// K 512 to 8192, three tile shapes, 1 to 8 ranges, every plan timed) the model's times are within 15 % (median 4 %)
+// and its choice within 4 % of the best measured plan.  1024^3: 10.4 -> 5.5 us (vendor library 7.8); 512x512x4096:
+// 15.8 -> 9.6 (10.1); 1024x2048x2048: 18.3 -> 13.1 (15.9); 1024x1024x4096: 21.1 -> 15.3 (18.6).
 struct SmallPlan {
   int bm = 0, bn = 0, S = 1;  // bm == 0: not a small product
 };
@@ -1544,10 +1591,15 @@ static SmallPlan small_plan(int64_t M, int64_t N, int64_t K, int64_t ws_bytes) {
       const int64_t units = tiles * S, k_part = K / S;
       if (units > 512 || K % (64 * S)) break;
       if (S > 1 && (k_part < 512 || S * M * N * 4 > ws_bytes)) break;
-      const bool deep = bm + bn == 256 && (S > 1 ? k_part >= 1024 && units <= 256 : pipelined_deep_ring(units, (int)k_part));
       const double per_cu_kib = (double)((units + 255) / 256) * (bm + bn) * 2 * k_part / 1024.0;
-      double us = 3.0 + per_cu_kib * ((bm + bn == 256 && !deep) ? 0.0188 : 0.0137);
-      if (S > 1) us += 2.8 + (double)S * M * N * 8 / 4e6;
+      double us_per_kib;
+      if (bm + bn == 256) us_per_kib = pipelined_slab_form(units, 256) ? 0.013 : 0.0188;
+      else us_per_kib = 0.0095 + 0.0035 * (units <= 128 ? 0.0 : units >= 256 ? 1.0 : (units - 128) / 128.0);
+      double us = 2.5 + per_cu_kib * us_per_kib;
+      if (S > 1) {
+        const double partial_bytes = (double)S * M * N * 8;
+        us += 2.3 + partial_bytes / 4.5e6 + (partial_bytes > (8 << 20) ? (partial_bytes - (8 << 20)) / 4.5e6 : 0.0);
+      }
       if (best.bm == 0 || us < best_us) {
         best_us = us;
         best.bm = bm, best.bn = bn, best.S = S;

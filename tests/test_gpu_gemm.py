@@ -211,10 +211,10 @@ def test_gemm_staged_slab_rotation(dev, shape, out_dtype):
 @pytest.mark.parametrize("shape", [(128, 128, 4096), (256, 384, 4160), (1024, 1024, 4096), (2048, 1536, 2048), (2048, 1536, 2112),
                                    (2048, 2048, 8192), (2048, 2176, 4096), (128, 256, 1984)])
 def test_gemm_pipelined_ring_depth(dev, shape, out32, dtype):
-    """The 128x128 kernel's ring is four slabs deep when every workgroup has a CU to itself and K is long, two deep
-    otherwise: one tile, slab counts that are 0, 1 and 3 mod 4 (64, 65, 33, 31 slabs), tile counts on both sides of the
-    128 and 256 limits (192 tiles at K = 2048 take the deep ring, 272 at K = 4096 and anything at K < 2048 the shallow
-    one) -- whole matrix against the independent generic kernel, rows against fp32, launches repeat bit for bit."""
+    """The 128x128 kernel takes its slab form (whole-slab fragment sets, four slabs in LDS) when every workgroup has a CU
+    to itself and its k-step form (two slabs) beyond 256 tiles: one tile, even and odd slab counts (64, 65, 33, 31: the
+    slab loop is unrolled by two), tile counts on both sides of the limit (192 and 256 against 272) -- whole matrix
+    against the independent generic kernel, rows against fp32, launches repeat bit for bit."""
     import iree_turbine_amd as ita
 
     M, N, K = shape
@@ -541,16 +541,16 @@ def test_gemm_skinny_contract(dev):
 
 
 @pytest.mark.parametrize("out_dtype", ["float16", "float32"])
-@pytest.mark.parametrize("shape", [(2048, 10240, 8192), (10240, 2048, 6144), (2048, 4096, 8192), (512, 2048, 8192), (1024, 1024, 8192), (256, 2048, 8192),
-                                   (384, 640, 8192), (256, 256, 8192), (128, 128, 2048), (1024, 2048, 8192), (512, 1024, 4096), (64, 1024, 4096),
-                                   (2048, 1280, 4096)])
+@pytest.mark.parametrize("shape", [(2048, 10240, 8192), (10240, 2048, 6144), (2048, 4096, 8192), (2048, 1280, 4096), (256, 2048, 8192),
+                                   (384, 640, 8192), (256, 256, 8192), (128, 128, 2048), (64, 1024, 4096), (512, 512, 4096),
+                                   (128, 2112, 4096), (128, 4160, 8192), (256, 4224, 32768), (128, 2432, 32768)])
 def test_gemm_k_split_with_workspace(dev, shape, out_dtype):
     """The workspace entry point through the C ABI: a strip of tile columns (2048 x 10240: the last 64 of 320 tiles, four
-    K ranges), a strip of tile rows (four ranges of 1536), a whole product of 128 tiles of 256x256 (two ranges), small
-    products that split on 128x128 tiles (four and two ranges), on 128x64 tiles (256 x 2048: four ranges) and on 64x64
-    tiles (two, four and eight ranges; one shape no multiple of 128, one a single tile row) and 160 tiles of 128x128 in
-    two ranges -- the whole matrix against the plain entry point (same products, other summation order), sampled rows
-    against an fp32 product; a workspace one byte short or absent runs exactly as the plain entry point does."""
+    K ranges), a strip of tile rows (four ranges of 1536), a whole product of 128 tiles of 256x256 (two ranges), 160 tiles
+    of 128x128 in two ranges, and small products that split on 64x64 tiles (two, four and eight ranges; one shape no
+    multiple of 128, one a single tile, one a single tile row), on 128x64 tiles (four and two ranges) and on 128x128
+    tiles (K = 32768: two and eight ranges) -- the whole matrix against the plain entry point (same products, other
+    summation order), sampled rows against an fp32 product; a workspace one byte short or absent runs exactly as the plain entry point does."""
     from iree_turbine_amd import _lib
     from oracle import inputs
 
@@ -585,7 +585,7 @@ def test_gemm_k_split_with_workspace(dev, shape, out_dtype):
 
 
 def test_gemm_k_split_through_the_op(dev):
-    """torch.ops.mi355.gemm_nt allocates the workspace the library asks for: a product of 16 tiles (bf16 operands) and
+    """torch.ops.mi355.gemm_nt allocates the workspace the library asks for: a small product (bf16 operands) and
     the benchmark shape with the sparse last round against the oracle's rows; shapes that take no split ask for none."""
     from iree_turbine_amd import _lib
     from oracle import inputs
