@@ -80,7 +80,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
   constexpr int LA = A_GROUPS / NW, LB = B_GROUPS / NW;
   // A ring of STAGES slabs: slab s+STAGES is requested when slab s retires, so a load has STAGES-1 slab times to land,
   // and the wait that retires a slab leaves the loads of the STAGES-2 newest slabs in flight (loads return in order).
-  constexpr int STAGES = SLAB ? 4 : 2;
+  constexpr int STAGES = !SLAB ? 2 : 4 * (BM + BN) * 128 <= 160 * 1024 ? 4 : 3;  // what 160 KiB of LDS hold
   static_assert((STAGES - 2) * (LA + LB) < 64, "the load counter has six bits");
   constexpr int IN_FLIGHT = (STAGES - 2) * (LA + LB);
 
@@ -151,24 +151,52 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
 #pragma unroll
       for (int ks = 0; ks < 4; ks++) read_frags(st, ks, fm[ks], fn[ks]);
     };
-    auto mfma_slab = [&](const half8(*fm)[TM], const half8(*fn)[TN]) {
-#pragma unroll
-      for (int ks = 0; ks < 4; ks++) mfmas(fm[ks], fn[ks]);
-    };
+    // A trip in source order, pinned by a scheduling fence behind every MFMA: the MFMA, then its share of the next
+    // slab's fragment reads and of the loads (left to itself the compiler issues the loads in one burst, and a wave's
+    // load is accepted only every 33 cycles: 1024x2048x4096 on 128x64 tiles 27.1 -> 24.7 us).  A trip of four MFMAs
+    // (the 64x64 tile) is too short to spread anything over and is left to the compiler, which puts the reads and the
+    // loads behind the first MFMA (pinned: 1024^3 5.4 -> 5.8 us).
     constexpr int NM = 4 * TM * TN, NR = 4 * (TM + TN), NL = LA + LB;
-    constexpr int R_PER_M = (NR + NM - 1) / NM, L_PER_M = (NL + NM - 1) / NM;
+    constexpr bool PINNED = NM > 4;
+    int stage = 0;  // kt % STAGES
     auto trip = [&](int kt, half8(*cm)[TM], half8(*cn)[TN], half8(*nm)[TM], half8(*nn)[TN]) {
+      const int next = stage + 1 == STAGES ? 0 : stage + 1;
+      const char* st = lds + next * STAGE;
+      const int slab = kt + STAGES < KT ? kt + STAGES : KT - 1;
       __builtin_amdgcn_sched_barrier(0);
-      read_slab(lds + ((kt + 1) & (STAGES - 1)) * STAGE, nm, nn);
-      issue_loads(kt & (STAGES - 1), kt + STAGES < KT ? kt + STAGES : KT - 1);
-      mfma_slab(cm, cn);
+      if constexpr (PINNED) {
+        char* dst = lds + stage * STAGE + wave * 1024;
+        const half_t* ap = a_src + slab * 64;
+        const half_t* bp = b_src + slab * 64;
 #pragma unroll
-      for (int i = 0; i < NM; i++) {
+        for (int m = 0; m < NM; m++) {
+          const int ks = m / (TM * TN), i = (m / TM) % TN, j = m % TM;
+          acc[i][j] = mfma16<BF>(cn[ks][i], cm[ks][j], acc[i][j]);
+#pragma unroll
+          for (int r = m * NR / NM; r < (m + 1) * NR / NM; r++) {
+            const int rk = r / (TM + TN), f = r % (TM + TN);
+            if (f < TM) nm[rk][f] = *reinterpret_cast<const half8*>(st + ((a_base ^ (rk * 32)) + f * 4096));
+            else nn[rk][f - TM] = *reinterpret_cast<const half8*>(st + ((b_base ^ (rk * 32)) + (f - TM) * 4096));
+          }
+#pragma unroll
+          for (int l = m * NL / NM; l < (m + 1) * NL / NM; l++) {
+            if (l < LA) load_lds_16B(ap + l * row_step + lane_off, dst + l * NW * 1024);
+            else load_lds_16B(bp + (l - LA) * row_step + lane_off, dst + A_BYTES + (l - LA) * NW * 1024);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
+        read_slab(st, nm, nn);
+        issue_loads(stage, slab);
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) mfmas(cm[ks], cn[ks]);
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, R_PER_M, 0);
-        __builtin_amdgcn_sched_group_barrier(0x010, L_PER_M, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, NR, 0);
+        __builtin_amdgcn_sched_group_barrier(0x010, NL, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, NM - 1, 0);
+        __builtin_amdgcn_sched_barrier(0);
       }
-      __builtin_amdgcn_sched_barrier(0);
+      stage = next;
       asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(IN_FLIGHT) : "memory");
       __builtin_amdgcn_s_barrier();
     };
@@ -1386,11 +1414,12 @@ static const GemmVariant kGemmVariants[] = {
     {"stream_256x256x64_w2x2_walk", 256, 256, 256},
     {"pipelined_64x64x64_w2x2", 64, 64, 256},
     {"pipelined_128x64x64_w2x2", 128, 64, 256},
+    {"pipelined_256x128x64_w2x2", 256, 128, 256},
     {"generic_64x64x32", 64, 64, 256},
 };
 // indices of the table above
 enum { V_PERSISTENT = 0, V_PIPELINED_128 = 1, V_STAGED = 2, V_SKINNY = 3, V_STREAM = 4, V_STREAM_TAIL = 5, V_STREAM_WALK = 6,
-       V_PIPELINED_64 = 7, V_PIPELINED_128x64 = 8 };
+       V_PIPELINED_64 = 7, V_PIPELINED_128x64 = 8, V_PIPELINED_256x128 = 9 };
 constexpr int kNumGemmVariants = sizeof(kGemmVariants) / sizeof(kGemmVariants[0]);
 
 int gemm_variant_count() { return kNumGemmVariants; }
@@ -1412,7 +1441,7 @@ static int cu_count() {
 // The pipelined kernel's slab form needs 128 bytes of LDS per tile row and column four times over: the 128x128 tile
 // takes it when every workgroup has a CU to itself (with 320 tiles the lost co-residency costs 20 %), the smaller
 // tiles (64 and 96 KiB: two and one workgroup per CU) always.
-static bool pipelined_slab_form(long long tiles, int bm_plus_bn) { return bm_plus_bn < 256 || tiles <= 256; }
+static bool pipelined_slab_form(long long tiles, int bm_plus_bn) { return bm_plus_bn != 256 || tiles <= 256; }
 
 template <int BM, int BN, int WM, int WN, typename OutT, int KIND, bool BF>  // KIND: 1 pipelined, 2 register-staged
 static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int K, int ldc, hipStream_t stream) {
@@ -1439,10 +1468,11 @@ static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int
       return check_launch("gemm_f16_nt_pipelined", grid, block, lds_bytes);
     };
     static std::atomic<uint64_t> lds_ok2{0}, lds_ok4{0};
-    static_assert(4 * (BM + BN) * 128 <= 160 * 1024, "four slabs of the tile fit in LDS");
+    constexpr int slab_stages = 4 * (BM + BN) * 128 <= 160 * 1024 ? 4 : 3;  // as the kernel picks them
     if (pipelined_slab_form((long long)tiles_m * tiles_n, BM + BN))
-      return go(gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT, BF, true>, 4 * (BM + BN) * 128, lds_ok4);
-    return go(gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT, BF, false>, 2 * (BM + BN) * 128, lds_ok2);
+      return go(gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT, BF, true>, slab_stages * (BM + BN) * 128, lds_ok4);
+    if constexpr (BM + BN == 256) return go(gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT, BF, false>, 2 * (BM + BN) * 128, lds_ok2);
+    return fail(-MI355_E_SHAPE, "gemm_f16_nt: no k-step form of this tile");  // not reached: pipelined_slab_form
   }
 }
 
@@ -1460,7 +1490,8 @@ static int launch_pipelined_ksplit(const half_t* a, const half_t* b, float* ws, 
   };
   static std::atomic<uint64_t> lds_ok2{0}, lds_ok4{0};
   if (pipelined_slab_form(grid.x, BM + BN)) return go(gemm_f16_nt_pipelined<BM, BN, 2, 2, float, BF, true>, 4 * (BM + BN) * 128, lds_ok4);
-  return go(gemm_f16_nt_pipelined<BM, BN, 2, 2, float, BF, false>, 2 * (BM + BN) * 128, lds_ok2);
+  if constexpr (BM + BN == 256) return go(gemm_f16_nt_pipelined<BM, BN, 2, 2, float, BF, false>, 2 * (BM + BN) * 128, lds_ok2);
+  return fail(-MI355_E_SHAPE, "gemm_f16_nt: no k-step form of this tile");  // not reached: pipelined_slab_form
 }
 
 template <int BM, int BN, int WM, int WN, typename OutT, bool BF>
@@ -1575,6 +1606,16 @@ static int ksplit128_factor(long long t128, int K) {
 // K 512 to 8192, three tile shapes, 1 to 8 ranges, every plan timed) the model's times are within 15 % (median 4 %)
 // and its choice within 4 % of the best measured plan.  1024^3: 10.4 -> 5.5 us (vendor library 7.8); 512x512x4096:
 // 15.8 -> 9.6 (10.1); 1024x2048x2048: 18.3 -> 13.1 (15.9); 1024x1024x4096: 21.1 -> 15.3 (18.6).
+// 129 to 256 tiles of 256x128 (257 to 512 of 128x128: more than one round of those, half a round of 256x256): one
+// round of the pipelined kernel's 256x128 tile.  2048x2560x4096 59.5 (128x128) / 72.1 (256x256) -> 54.1 us, 2048x4096x4096
+// 75.8 / 77.7 -> 67.2, 1024x8192x2048 40.7 / 44.6 -> 38.0 (vendor library 48.3, 66.4, 38.0); level with the K split on
+// 256x256 tiles at K = 8192 and behind the 128x128 tile at K = 1024 (27.1 against 24.1 us).
+static bool takes_256x128(int64_t M, int64_t N, int64_t K) {
+  if (M % 256 || N % 128 || K % 64 || K < 1536 || K >= 8192) return false;
+  const int64_t units = (M / 256) * (N / 128);
+  return units > 128 && units <= 256;
+}
+
 struct SmallPlan {
   int bm = 0, bn = 0, S = 1;  // bm == 0: not a small product
 };
@@ -1686,6 +1727,7 @@ static int launch_variant(int variant, const void* a, const void* b, void* c, in
     case V_STREAM_WALK: return launch_stream<OutT, BF>(a, b, c, M, N, K, N, stream, true);
     case V_PIPELINED_64: return launch_tiled<64, 64, 2, 2, OutT, 1, BF>(a, b, c, M, N, K, N, stream);
     case V_PIPELINED_128x64: return launch_tiled<128, 64, 2, 2, OutT, 1, BF>(a, b, c, M, N, K, N, stream);
+    case V_PIPELINED_256x128: return launch_tiled<256, 128, 2, 2, OutT, 1, BF>(a, b, c, M, N, K, N, stream);
     default: {
       dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
       hipLaunchKernelGGL((gemm_f16_nt_generic<OutT, BF>), grid, block, 0, stream, (const half_t*)a, (const half_t*)b, (OutT*)c,
@@ -1741,6 +1783,7 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
       if (small.S > 1 && (!workspace || workspace_bytes < (int64_t)small.S * M * N * 4)) small = small_plan(M, N, K, 0);
       variant = small.bm == 64 ? V_PIPELINED_64 : small.bn == 64 ? V_PIPELINED_128x64 : V_PIPELINED_128;
     }
+    else if (al && takes_256x128(M, N, K)) variant = V_PIPELINED_256x128;
     else if (s128 > 1 && workspace_bytes >= (int64_t)s128 * M * N * 4) {  // a small product: K split on 128x128 tiles
       variant = V_PIPELINED_128;
       split128 = s128;
@@ -1808,6 +1851,7 @@ static int64_t gemm_nt_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (M <= 64 && N % 32 == 0 && N >= 2048 && K >= 512) return 0;        // the weight-streaming kernel's shapes
   const SmallPlan sp = small_plan(M, N, K, INT64_MAX);
   if (sp.bm) return sp.S > 1 ? (int64_t)sp.S * M * N * 4 : 0;
+  if (takes_256x128(M, N, K)) return 0;
   const int s128 = (K % 64 == 0) ? ksplit128_plan((int)M, (int)N, (int)K) : 1;
   if (s128 > 1) return (int64_t)s128 * M * N * 4;
   int sm, sn;

@@ -22,7 +22,7 @@ def _run(dev, M, N, K, out_dtype, variant=-1, seed=10):
     return c.float().cpu(), ref
 
 
-@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 4, 5, 6, 7, 8])  # every tiled kernel (3 is the skinny-M kernel, 9 the any-shape one)
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 4, 5, 6, 7, 8, 9])  # every tiled kernel (3 is the skinny-M kernel, 10 the any-shape one)
 def test_gemm_1024_f32_all_variants(dev, variant):
     c, ref = _run(dev, 1024, 1024, 1024, "float32", variant)
     torch.testing.assert_close(c, ref, rtol=RTOL, atol=ATOL)
@@ -233,6 +233,35 @@ def test_gemm_pipelined_ring_depth(dev, shape, out32, dtype):
     exact = a[rows.to(dev)].float() @ b.float().t()
     torch.testing.assert_close(got[rows.to(dev)].float(), exact, rtol=RTOL, atol=ATOL)
     assert torch.equal(got, torch.ops.mi355.gemm_nt(a, b, out_dtype, v))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("out32", [False, True])
+@pytest.mark.parametrize("shape", [(256, 128, 64), (512, 256, 128), (256, 384, 192), (768, 640, 320), (2048, 2560, 2048), (2048, 4096, 1600),
+                                   (1024, 8192, 4096), (2304, 1792, 1536)])
+def test_gemm_pipelined_256x128(dev, shape, out32, dtype):
+    """The 256x128 tile of the pipelined kernel (slab form, three slabs in LDS): one tile and one slab, two, three and
+    five slabs (shorter than, equal to and just beyond the ring), an odd slab count (25), and the shapes the automatic
+    choice gives it (129 to 256 tiles, 1536 <= K < 8192; 126 tiles: not) -- by index and through the automatic choice,
+    whole matrix against the independent generic kernel, rows against fp32, launches repeat bit for bit."""
+    import iree_turbine_amd as ita
+
+    M, N, K = shape
+    announce(f"gemm pipelined 256x128 {shape} {dtype} out32={out32}")
+    names = ita._lib.variants("gemm_f16_nt")
+    g = torch.Generator().manual_seed(M + 5 * N + 11 * K)
+    a = (torch.randn(M, K, generator=g) * 0.25).to(dtype).to(dev)
+    b = (torch.randn(N, K, generator=g) * 0.25).to(dtype).to(dev)
+    out_dtype = "float32" if out32 else str(dtype).replace("torch.", "")
+    ref = torch.ops.mi355.gemm_nt(a, b, out_dtype, len(names) - 1)
+    rows = torch.tensor([0, 127, 128, M - 1], device=dev)
+    exact = a[rows].float() @ b.float().t()
+    tol = 1e-3 if (out32 or dtype == torch.float16) else 8e-3
+    for v in (names.index("pipelined_256x128x64_w2x2"), -1):
+        got = torch.ops.mi355.gemm_nt(a, b, out_dtype, v)
+        torch.testing.assert_close(got.float(), ref.float(), rtol=tol, atol=tol * 4)
+        torch.testing.assert_close(got[rows].float(), exact, rtol=RTOL, atol=ATOL)
+        assert torch.equal(got, torch.ops.mi355.gemm_nt(a, b, out_dtype, v))
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
