@@ -47,6 +47,32 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
         _lib.check(1, "x")
 
 
+def test_gemm_workspace_plan_without_a_gpu():
+    """mi355_gemm_nt_workspace_bytes is host arithmetic: what it asks for is a whole number (1, 2, 4 or 8 for the small
+    products) of fp32 copies of the output or of the strip of a sparse last round, nothing for shapes that take the
+    weight-streaming kernel, one round of 256x128 tiles or full rounds of 256x256 tiles, and nothing for bad shapes."""
+    lib = _lib.load()
+    need = lib.mi355_gemm_nt_workspace_bytes
+    for M in (64, 128, 256, 384, 512, 1024, 1408):
+        for N in (64, 128, 640, 1024, 1472, 2048):
+            for K in (64, 512, 1024, 2048, 4096, 8192, 32768):
+                if M * N > (1 << 21) or (M <= 64 and N >= 2048 and K >= 512):
+                    continue
+                b = need(M, N, K)
+                assert b % (M * N * 4) == 0 and b // (M * N * 4) in (0, 2, 4, 8), (M, N, K, b)
+                if K < 1024:
+                    assert b == 0, (M, N, K, b)  # ranges shorter than 512 do not pay for the merge launch
+    assert need(256, 256, 8192) == 8 * 256 * 256 * 4
+    assert need(1024, 1024, 1024) == 0 and need(1024, 2048, 4096) == 0  # enough tiles without a split
+    assert need(16, 8192, 8192) == 0 and need(64, 4096, 4096) == 0  # weight streaming
+    assert need(2048, 2560, 4096) == 0 and need(1024, 8192, 2048) == 0  # 256x128 tiles, one round
+    assert need(2048, 1280, 4096) == 2 * 2048 * 1280 * 4  # 160 tiles of 128x128
+    assert need(2048, 4096, 8192) == 2 * 2048 * 4096 * 4  # 128 tiles of 256x256
+    assert need(2048, 10240, 8192) == 4 * 2048 * 2048 * 4  # the strip of 64 tiles behind a full round
+    assert need(8192, 8192, 8192) == 0 and need(4096, 4096, 4096) == 0
+    assert need(0, 128, 128) == 0 and need(128, 128, -64) == 0 and need(128, 128, 1 << 22) == 0
+
+
 def test_ops_registered_with_meta_kernels():
     for name in ("gemm_nt", "flash_attn_fwd", "paged_decode_attn", "paged_decode_phase0", "paged_decode_phase1",
                  "mxfp4_gemm", "mxfp4_dequant"):
