@@ -317,17 +317,31 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
       *reinterpret_cast<half8*>(cbase + (size_t)row * N) = v;
     }
   } else {
-    const int m0 = tile_m * BM + wm * WTM + r32;
-    const int n0 = tile_n * BN + wn * WTN + 4 * h;
+    // fp32 epilogue, the same way (a lane's four consecutive n are one 16-byte chunk; chunk slot c ^ (m & (CH - 1))):
+    // stored straight from the accumulators a row would get 32 bytes per instruction, a quarter of a line.
+    constexpr int ROW_B = WTN * 4, CH = WTN / 4;
+    static_assert(NW * WTM * ROW_B <= STAGES * STAGE, "the waves' output tiles fit in the ring");
+    char* ep = lds + wave * (WTM * ROW_B);
 #pragma unroll
     for (int j = 0; j < TM; j++) {
-      OutT* crow = C + (size_t)(m0 + j * 32) * N + n0;
+      const int ml = j * 32 + r32;
 #pragma unroll
       for (int i = 0; i < TN; i++)
 #pragma unroll
-        for (int q = 0; q < 4; q++)
-          OutPack<OutT, BF>::store4(crow + i * 32 + q * 8, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
-                                acc[i][j][4 * q + 3]);
+        for (int q = 0; q < 4; q++) {
+          const int c = i * 8 + q * 2 + h;
+          floatx4 v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+          *reinterpret_cast<floatx4*>(ep + ml * ROW_B + ((c ^ (ml & (CH - 1))) * 16)) = v;
+        }
+    }
+    constexpr int ROWS_PER_IT = 64 / CH;
+    const int er = lane / CH, ec = lane % CH;
+    OutT* cbase = C + (size_t)(tile_m * BM + wm * WTM) * N + tile_n * BN + wn * WTN + ec * 4;
+#pragma unroll
+    for (int it = 0; it < WTM / ROWS_PER_IT; it++) {
+      const int row = it * ROWS_PER_IT + er;
+      floatx4 v = *reinterpret_cast<const floatx4*>(ep + row * ROW_B + ((ec ^ (row & (CH - 1))) * 16));
+      *reinterpret_cast<floatx4*>(cbase + (size_t)row * N) = v;
     }
   }
 }
