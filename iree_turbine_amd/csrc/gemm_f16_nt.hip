@@ -1623,9 +1623,10 @@ static int ksplit128_factor(long long t128, int K) {
 // 129 to 256 tiles of 256x128 (257 to 512 of 128x128: more than one round of those, half a round of 256x256): one
 // round of the pipelined kernel's 256x128 tile.  2048x2560x4096 59.5 (128x128) / 72.1 (256x256) -> 54.1 us, 2048x4096x4096
 // 75.8 / 77.7 -> 67.2, 1024x8192x2048 40.7 / 44.6 -> 38.0 (vendor library 48.3, 66.4, 38.0); level with the K split on
-// 256x256 tiles at K = 8192 and behind the 128x128 tile at K = 1024 (27.1 against 24.1 us).
+// 256x256 tiles at K = 8192.  Short K as well: 2048x4096x1024 22.9 (128x128) / 26.3 (256x256) -> 21.5 us, 1024x8192x512
+// 14.2 / 17.0 -> 14.1, 2048x2560x256 8.7 / 11.1 -> 8.5.
 static bool takes_256x128(int64_t M, int64_t N, int64_t K) {
-  if (M % 256 || N % 128 || K % 64 || K < 1536 || K >= 8192) return false;
+  if (M % 256 || N % 128 || K % 64 || K < 256 || K >= 8192) return false;
   const int64_t units = (M / 256) * (N / 128);
   return units > 128 && units <= 256;
 }

@@ -242,7 +242,7 @@ def test_gemm_pipelined_ring_depth(dev, shape, out32, dtype):
 def test_gemm_pipelined_256x128(dev, shape, out32, dtype):
     """The 256x128 tile of the pipelined kernel (slab form, three slabs in LDS): one tile and one slab, two, three and
     five slabs (shorter than, equal to and just beyond the ring), an odd slab count (25), and the shapes the automatic
-    choice gives it (129 to 256 tiles, 1536 <= K < 8192; 126 tiles: not) -- by index and through the automatic choice,
+    choice gives it (129 to 256 tiles, 256 <= K < 8192; 126 tiles: not) -- by index and through the automatic choice,
     whole matrix against the independent generic kernel, rows against fp32, launches repeat bit for bit."""
     import iree_turbine_amd as ita
 
