@@ -33,7 +33,10 @@ __device__ __forceinline__ floatx16 mfma_fp4_32x32x64(intx4 a, int sa, intx4 b, 
 // SCALES_LDS: scale bytes travel through LDS in groups of 4 slabs (32 bytes per row, two buffers behind
 // the data stages) instead of one strided 8-byte global load per lane, row tile and slab.  Needs
 // K % 1024 == 0.
-template <int BM, int BN, int WM, int WN, typename OutT, bool SCALES_LDS>
+// SLAB (with SCALES_LDS): the slab form of gemm_f16_nt_pipelined -- four data stages, the fragments and scale dwords
+// of a whole slab in one of two register sets, one wait per trip in front of its barrier -- for launches in which a
+// workgroup has its CU to itself: its slab time in the k-step form is its load latency.
+template <int BM, int BN, int WM, int WN, typename OutT, bool SCALES_LDS, bool SLAB = false>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* __restrict__ A, const uint8_t* __restrict__ As,
                                                                 const uint8_t* __restrict__ B, const uint8_t* __restrict__ Bs,
                                                                 OutT* __restrict__ C, int M, int N, int K, int tiles_m,
@@ -86,7 +89,9 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
   int sa[2][TM], sb[2][TN];
   // LDS scale buffers: [buffer][A rows then B rows][32 bytes = 4 slabs x 8 blocks]
   constexpr int SC_BUF = (BM + BN) * 32;
-  char* sc_lds = lds + 2 * STAGE;
+  constexpr int STAGES = SLAB ? 4 : 2;
+  static_assert(!SLAB || SCALES_LDS, "the slab form stages its scales through LDS");
+  char* sc_lds = lds + STAGES * STAGE;
   static_assert(((BM + BN) / 32) % NW == 0, "scale rows must split evenly over waves");
   constexpr int LS = (BM + BN) / 32 / NW;  // wave-loads (32 rows x 32 bytes) per wave per group
   const unsigned sc_lane_off = (unsigned)(lane >> 1) * (unsigned)Ksc + (unsigned)(lane & 1) * 16u;
@@ -147,8 +152,104 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
   };
 
   const int KT = K / 256;
-  intx4 fm0[TM], fn0[TN], fm1[TM], fn1[TN];
   const int KG = (KT + 3) >> 2;  // scale groups
+  using K0 = std::integral_constant<int, 0>;
+  using K1 = std::integral_constant<int, 1>;
+  using K2 = std::integral_constant<int, 2>;
+  using K3 = std::integral_constant<int, 3>;
+  if constexpr (SLAB) {
+    // Trip kt: MFMAs of slab kt from the current register set | fragment and scale reads of slab kt+1 into the other
+    // set | loads of slab kt+4 into the stage slab kt left (every wave read it a trip ago) and, on every fourth trip,
+    // of scale group kt/4 + 1 (its buffer's last reader was trip kt-2).  The wait in front of the barrier leaves the
+    // loads of the two newest trips in flight, so a load has three trips to land.
+    constexpr int NL = LA + LB, NM = 4 * TM * TN, NR = 5 * (TM + TN);
+    constexpr bool PINNED = NM > 4;  // a trip of four MFMAs is too short to spread anything over
+    intx4 am[2][4][TM], an[2][4][TN];
+    auto read_at = [&](const char* st, const char* scb, int r, intx4(*fm)[TM], intx4(*fn)[TN], int* da, int* db) __attribute__((always_inline)) {
+      // read r of a trip: first the scale dwords, then the fragments k-step by k-step
+      if (r < TM) da[r] = *reinterpret_cast<const int*>(scb + sa_off + r * 1024);
+      else if (r < TM + TN) db[r - TM] = *reinterpret_cast<const int*>(scb + sb_off + (r - TM) * 1024);
+      else {
+        const int q = r - (TM + TN), rk = q / (TM + TN), f = q % (TM + TN);
+        if (f < TM) fm[rk][f] = *reinterpret_cast<const intx4*>(st + ((a_base ^ (rk * 16)) + f * 4096));
+        else fn[rk][f - TM] = *reinterpret_cast<const intx4*>(st + ((b_base ^ (rk * 16)) + (f - TM) * 4096));
+      }
+    };
+    auto mfma_at = [&](int m, const intx4(*fm)[TM], const intx4(*fn)[TN], const int* ca, const int* cb) __attribute__((always_inline)) {
+      const int ks = m / (TM * TN), i = (m / TM) % TN, j = m % TM;
+      if (ks == 0) acc[i][j] = mfma_fp4_32x32x64<0>(fn[0][i], cb[i], fm[0][j], ca[j], acc[i][j]);
+      else if (ks == 1) acc[i][j] = mfma_fp4_32x32x64<1>(fn[1][i], cb[i], fm[1][j], ca[j], acc[i][j]);
+      else if (ks == 2) acc[i][j] = mfma_fp4_32x32x64<2>(fn[2][i], cb[i], fm[2][j], ca[j], acc[i][j]);
+      else acc[i][j] = mfma_fp4_32x32x64<3>(fn[3][i], cb[i], fm[3][j], ca[j], acc[i][j]);
+    };
+    auto trip = [&](auto kk_tag, int kt) __attribute__((always_inline)) {
+      constexpr int KK = decltype(kk_tag)::value;
+      constexpr int CUR = KK & 1, NXT = CUR ^ 1;
+      constexpr int NLT = NL + (KK == 0 ? LS : 0);  // loads of this trip
+      const int nslab = kt + 1;
+      const char* st = lds + (nslab & 3) * STAGE;
+      const char* scb = sc_lds + ((nslab >> 2) & 1) * SC_BUF + (nslab & 3) * 8;
+      const int lslab = kt + 4 < KT ? kt + 4 : KT - 1;
+      char* dst = lds + (kt & 3) * STAGE + wave * 1024;
+      const uint8_t* ap = a_src + lslab * 128;
+      const uint8_t* bp = b_src + lslab * 128;
+      const int g = (kt >> 2) + 1 < KG ? (kt >> 2) + 1 : KG - 1;
+      auto load_at = [&](int l) __attribute__((always_inline)) {
+        if (l < LA) load_lds_16B(ap + l * row_step + lane_off, dst + l * NW * 1024);
+        else if (l < NL) load_lds_16B(bp + (l - LA) * row_step + lane_off, dst + A_BYTES + (l - LA) * NW * 1024);
+        else {
+          const int r0 = (wave * LS + (l - NL)) * 32;
+          const uint8_t* src = r0 < BM ? As + (size_t)(tile_m * BM + r0) * Ksc : Bs + (size_t)(tile_n * BN + r0 - BM) * Ksc;
+          load_lds_16B(src + g * 32 + sc_lane_off, sc_lds + (g & 1) * SC_BUF + r0 * 32);
+        }
+      };
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (PINNED) {
+#pragma unroll
+        for (int m = 0; m < NM; m++) {
+          mfma_at(m, am[CUR], an[CUR], sa[CUR], sb[CUR]);
+#pragma unroll
+          for (int r = m * NR / NM; r < (m + 1) * NR / NM; r++) read_at(st, scb, r, am[NXT], an[NXT], sa[NXT], sb[NXT]);
+#pragma unroll
+          for (int l = m * NLT / NM; l < (m + 1) * NLT / NM; l++) load_at(l);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < NR; r++) read_at(st, scb, r, am[NXT], an[NXT], sa[NXT], sb[NXT]);
+#pragma unroll
+        for (int l = 0; l < NLT; l++) load_at(l);
+#pragma unroll
+        for (int m = 0; m < NM; m++) mfma_at(m, am[CUR], an[CUR], sa[CUR], sb[CUR]);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, NR, 0);
+        __builtin_amdgcn_sched_group_barrier(0x010, NLT, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, NM - 1, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // in flight behind the wait: the loads of this trip and of the one before (the scale group rides with trip 0 of
+      // a period, so trips 0 and 1 leave LS more)
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * NL + (KK <= 1 ? LS : 0)) : "memory");
+      __builtin_amdgcn_s_barrier();
+    };
+    issue_scale_loads(0);
+#pragma unroll
+    for (int t = 0; t < 3; t++) issue_loads(t, t < KT ? t : KT - 1);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NL) : "memory");
+    __builtin_amdgcn_s_barrier();  // not __syncthreads(): its fence would wait for every load in flight
+#pragma unroll
+    for (int r = 0; r < NR; r++) read_at(lds, sc_lds, r, am[0], an[0], sa[0], sb[0]);
+    issue_loads(3, 3 < KT ? 3 : KT - 1);
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * NL) : "memory");
+    __builtin_amdgcn_s_barrier();
+    for (int kt = 0; kt < KT; kt += 4) {  // K % 1024 == 0 on this path
+      trip(K0{}, kt);
+      trip(K1{}, kt + 1);
+      trip(K2{}, kt + 2);
+      trip(K3{}, kt + 3);
+    }
+  } else {
+  intx4 fm0[TM], fn0[TN], fm1[TM], fn1[TN];
   if constexpr (SCALES_LDS) issue_scale_loads(0);
   issue_loads(0, 0);
   wait_vmcnt0();
@@ -159,10 +260,6 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
   read_frags(lds, 0, fm0, fn0);
   if constexpr (!SCALES_LDS) wait_vmcnt0();
 
-  using K0 = std::integral_constant<int, 0>;
-  using K1 = std::integral_constant<int, 1>;
-  using K2 = std::integral_constant<int, 2>;
-  using K3 = std::integral_constant<int, 3>;
   // One slab (rotated k-loop, see gemm_f16_nt_pipelined): fragment reads for k-step s+1 ride between the
   // MFMAs of k-step s; the slab-retiring barrier sits in front of the last k-step's MFMAs, which overlap
   // the global -> LDS loads of slab kt+2 and the first fragment reads of slab kt+1.  With LDS-staged
@@ -243,6 +340,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
     }
     if (kt < KT) slab(K0{}, kt);
   }
+  }
   wait_vmcnt0();
   __syncthreads();
 
@@ -260,7 +358,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
           const int c = i * 4 + q;
           ushortx4 v = {f32_to_bf16_rne(acc[i][j][4 * q]), f32_to_bf16_rne(acc[i][j][4 * q + 1]),
                         f32_to_bf16_rne(acc[i][j][4 * q + 2]), f32_to_bf16_rne(acc[i][j][4 * q + 3])};
-          *reinterpret_cast<ushortx4*>(ep + ml * ROW_B + ((c ^ ((ml >> 1) & 7)) * 16) + 8 * h) = v;
+          *reinterpret_cast<ushortx4*>(ep + ml * ROW_B + ((c ^ ((ml >> 1) & (CH - 1))) * 16) + 8 * h) = v;
         }
     }
     constexpr int ROWS_PER_IT = 64 / CH;
@@ -269,7 +367,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
 #pragma unroll
     for (int it = 0; it < WTM / ROWS_PER_IT; it++) {
       const int row = it * ROWS_PER_IT + er;
-      intx4 v = *reinterpret_cast<const intx4*>(ep + row * ROW_B + ((ec ^ ((row >> 1) & 7)) * 16));
+      intx4 v = *reinterpret_cast<const intx4*>(ep + row * ROW_B + ((ec ^ ((row >> 1) & (CH - 1))) * 16));
       *reinterpret_cast<intx4*>(cbase + (size_t)row * N) = v;
     }
   } else {
@@ -1506,17 +1604,19 @@ static const MxVariant kMxVariants[] = {
     {"staged_256x256x256_w2x2", 256, 256},
     {"stream_256x256x256_w2x2", 256, 256},
     {"stream_256x256x256_w2x2_walk", 256, 256},
+    {"tiled_64x64x256_w2x2", 64, 64},
     {"generic_32x128", 32, 128},
 };
 constexpr int kNumMxVariants = sizeof(kMxVariants) / sizeof(kMxVariants[0]);
 int mxfp4_variant_count() { return kNumMxVariants; }
 const char* mxfp4_variant_name(int i) { return (i >= 0 && i < kNumMxVariants) ? kMxVariants[i].name : nullptr; }
 
-template <int BM, int BN, int WM, int WN, typename OutT, bool SCALES_LDS>
+template <int BM, int BN, int WM, int WN, typename OutT, bool SCALES_LDS, bool SLAB = false>
 static int launch_mx_tiled(const void* a, const void* as, const void* b, const void* bs, void* c, int M, int N, int K,
                            hipStream_t stream) {
-  auto kern = gemm_mxfp4_tiled<BM, BN, WM, WN, OutT, SCALES_LDS>;
-  constexpr int lds_bytes = 2 * (BM + BN) * 128 + (SCALES_LDS ? 2 * (BM + BN) * 32 : 0);
+  auto kern = gemm_mxfp4_tiled<BM, BN, WM, WN, OutT, SCALES_LDS, SLAB>;
+  constexpr int lds_bytes = (SLAB ? 4 : 2) * (BM + BN) * 128 + (SCALES_LDS ? 2 * (BM + BN) * 32 : 0);
+  static_assert(lds_bytes <= 160 * 1024, "the stages and the scale buffers fit in LDS");
   static std::atomic<uint64_t> lds_ok{0};
   if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_mxfp4_tiled")) return rc;
   const int tiles_m = M / BM, tiles_n = N / BN;
@@ -1599,6 +1699,8 @@ static int launch_mx(int variant, const void* a, const void* as, const void* b, 
       if (K % 1024 == 0) return launch_mx_tiled<256, 256, 2, 4, OutT, true>(a, as, b, bs, c, M, N, K, stream);
       return launch_mx_tiled<256, 256, 2, 4, OutT, false>(a, as, b, bs, c, M, N, K, stream);
     case 2:
+      if (K % 1024 == 0 && (long long)(M / 128) * (N / 128) <= 256)  // every workgroup has a CU to itself: the slab form
+        return launch_mx_tiled<128, 128, 2, 2, OutT, true, true>(a, as, b, bs, c, M, N, K, stream);
       if (K % 1024 == 0) return launch_mx_tiled<128, 128, 2, 2, OutT, true>(a, as, b, bs, c, M, N, K, stream);
       return launch_mx_tiled<128, 128, 2, 2, OutT, false>(a, as, b, bs, c, M, N, K, stream);
     case 3: {
@@ -1614,6 +1716,7 @@ static int launch_mx(int variant, const void* a, const void* as, const void* b, 
     case 4: return launch_mx_staged<OutT>(a, as, b, bs, c, M, N, K, stream);
     case 5: return launch_mx_stream<OutT>(a, as, b, bs, c, M, N, K, stream, false);
     case 6: return launch_mx_stream<OutT>(a, as, b, bs, c, M, N, K, stream, true);
+    case 7: return launch_mx_tiled<64, 64, 2, 2, OutT, true, true>(a, as, b, bs, c, M, N, K, stream);  // slab form only
     default: {
       dim3 grid((N + 127) / 128, (M + 31) / 32), block(256);
       hipLaunchKernelGGL(gemm_mxfp4_generic<OutT>, grid, block, 0, stream, (const uint8_t*)a, (const uint8_t*)as,
@@ -1644,6 +1747,7 @@ extern "C" int mi355_mxfp4_gemm(const void* a, const void* a_scale, const void* 
   auto fits = [&](int v) {
     if (v == kNumMxVariants - 1) return true;
     if (v == 3) return sc_al4 && M <= 32 && N % 32 == 0 && K % 256 == 0;  // skinny: whole 128-byte segments
+    if (v == 7 && K % 1024 != 0) return false;  // scale groups of four slabs
     if ((v == 0 || v == 4) && !(sc_al16 && K % 512 == 0 && K >= 1024 && K <= (1 << 22))) return false;  // 2-slab scale groups
     // streamed: slabs in pairs, four or more; each operand behind one buffer descriptor
     if ((v == 5 || v == 6) && !(sc_al16 && K % 512 == 0 && K >= 1024 && M * (K / 2) < (1ll << 32) && N * (K / 2) < (1ll << 32))) return false;
@@ -1661,6 +1765,10 @@ extern "C" int mi355_mxfp4_gemm(const void* a, const void* a_scale, const void* 
     else if (big && K >= 32768 && fits(4)) variant = 4;  // its epilogue is not overlapped: ahead only from 128 slabs per tile
     else if (big && fits(0)) variant = 0;
     else if (big && fits(1)) variant = 1;
+    // Few tiles: what counts is how many CUs pull operands (a lone workgroup moves about 75-100 GB/s through its CU
+    // whatever its tile), so up to 320 tiles of 64x64 take those (128x8192x8192: 16.7 us on 128x128 tiles, 10.8 on
+    // 64x64; 1024x1024x8192 15.3 -> 10.0; 256x8192x8192, 512 tiles of 64x64: 17.6 against 18.7).
+    else if (fits(7) && (M / 64) * (N / 64) <= 320) variant = 7;
     else if (fits(2)) variant = 2;
     else variant = kNumMxVariants - 1;
   } else if (!fits(variant)) {

@@ -43,7 +43,7 @@ def test_dequant_random_bit_exact(dev):
     assert np.array_equal(out.view(np.uint32), om.mxfp4_dequant_ref(a, asc).view(np.uint32))
 
 
-@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 4, 5, 6, 7])
+@pytest.mark.parametrize("variant", [-1, 0, 1, 2, 4, 5, 6, 7, 8])
 def test_mxfp4_gemm_variants(dev, variant):
     import iree_turbine_amd  # noqa: F401
     from oracle import inputs, mxfp4 as om
@@ -74,9 +74,9 @@ def test_mxfp4_gemm_ragged(dev, shape):
 
 
 @pytest.mark.parametrize("shape", [(32, 256, 512), (1, 64, 256), (7, 96, 2048), (32, 8192, 8192), (20, 160, 16384), (32, 64, 8192 + 256)])
-@pytest.mark.parametrize("variant", [3, 7])
+@pytest.mark.parametrize("variant", [3, 8])
 def test_mxfp4_skinny_vs_generic(dev, shape, variant):
-    """The weight-streaming kernel (variant 3) and the any-shape kernel (variant 7) on skinny shapes."""
+    """The weight-streaming kernel (variant 3) and the any-shape kernel (variant 8) on skinny shapes."""
     import iree_turbine_amd  # noqa: F401
     from oracle import inputs, mxfp4 as om
 
@@ -179,6 +179,35 @@ def test_mxfp4_full_size_repeatable(dev, shape):
             assert torch.equal(first, torch.ops.mi355.mxfp4_gemm(a, asc, b, bsc, "float32", variant)), names[variant]
         assert _rel_err(first, generic) < 1e-5, names[variant]
     assert ran >= 1
+
+
+@pytest.mark.parametrize("shape", [(128, 128, 1024), (64, 64, 1024), (256, 256, 2048), (192, 320, 3072), (384, 640, 5120), (1024, 1024, 8192),
+                                   (128, 8192, 8192), (2048, 2048, 2048), (2048, 2176, 1024), (1152, 1152, 4096)])
+@pytest.mark.parametrize("out_dtype", ["bfloat16", "float32"])
+def test_mxfp4_slab_form(dev, shape, out_dtype):
+    """The tiled kernel's slab form (four data stages, a whole slab's fragments and scale dwords in one of two register
+    sets, scale groups of four slabs riding with every fourth trip): one tile and one scale group (the minimum K), two,
+    three, five and eight groups, shapes that are no multiple of 128, 256 tiles of either shape, and 272 tiles of
+    128x128 (the k-step form) -- the 64x64 and 128x128 tiles by index and the automatic choice, whole matrix against
+    the independent generic kernel, launches repeat bit for bit."""
+    import iree_turbine_amd as ita
+    from oracle import inputs
+
+    M, N, K = shape
+    announce(f"mxfp4 slab form {shape} {out_dtype}")
+    names = ita._lib.variants("mxfp4_gemm")
+    a, asc, b, bsc = [t.to(dev) for t in inputs.mxfp4_inputs(M, N, K, seed=M + N + K)]
+    ref = torch.ops.mi355.mxfp4_gemm(a, asc, b, bsc, out_dtype, len(names) - 1)
+    todo = [-1, names.index("tiled_64x64x256_w2x2")] + ([names.index("tiled_128x128x256_w2x2")] if M % 128 == 0 and N % 128 == 0 else [])
+    for v in todo:
+        got = torch.ops.mi355.mxfp4_gemm(a, asc, b, bsc, out_dtype, v)
+        if out_dtype == "float32":
+            assert _rel_err(got, ref) < 1e-5, v
+        else:
+            g32, r32 = got.float(), ref.float()
+            assert _rel_err(g32, r32) < 1e-3, v
+            assert ((g32 - r32).abs() <= r32.abs() * 2 ** -7 + 1e-5 * r32.abs().max()).all(), v
+        assert torch.equal(got, torch.ops.mi355.mxfp4_gemm(a, asc, b, bsc, out_dtype, v)), v
 
 
 @pytest.mark.parametrize("shape", [(4352, 4352, 1024), (4096, 4608, 1536), (512, 256, 8192)])
