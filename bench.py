@@ -513,6 +513,7 @@ CALIBRATION = {  # not part of the path: run only when named with --workload
     "library_gemm_2048x10240x8192": wl_library_gemm(2048, 10240, 8192),
     "library_gemm_1024x8192x8192": wl_library_gemm(1024, 8192, 8192),
     "library_gemm_512x8192x8192": wl_library_gemm(512, 8192, 8192),
+    "library_gemm_1024": wl_library_gemm(1024, 1024, 1024),  # fp16 output: torch.mm has no fp32-output form
     "copy_1GiB": wl_copy(),
     "mfma_f16_regloop_zeros": wl_mfma_regloop("f16", "zeros"),
     "mfma_f16_regloop_benchmark": wl_mfma_regloop("f16", "benchmark"),
@@ -685,7 +686,7 @@ def measure(name: str, dev, steps: int, warmup: int, with_cpu: bool):
 # board's ceilings from the SAME box and session as the kernels' (boxes differ by a few per cent): hipBLASLt on the
 # headline shape, the register-only MFMA loops on benchmark-like operands (plain and with a GEMM's register structure),
 # the prefill tile's instruction mix out of registers.  They are not part of the path; `calibration: true` marks them.
-CALIBRATION_IN_DEFAULT_RUN = ("library_gemm_8192", "mfma_f16_regloop_benchmark", "mfma_f16x16walk_regloop_benchmark",
+CALIBRATION_IN_DEFAULT_RUN = ("library_gemm_8192", "library_gemm_1024", "mfma_f16_regloop_benchmark", "mfma_f16x16walk_regloop_benchmark",
                               "mfma_fp4_regloop_benchmark", "mfma_fp4x16walk_regloop_benchmark", "fa_issue_regloop_mix_w2",
                               "fa_issue_regloop_mfma_w2")
 
