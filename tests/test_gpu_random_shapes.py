@@ -76,6 +76,39 @@ def test_random_gemm_few_tiles_long_k(dev):
     assert split >= 8  # the draw does exercise the split
 
 
+def test_random_gemm_small_and_mid_products(dev):
+    """Products whose tile shape and K ranges the automatic choice picks by rule: multiples of 64 up to 128 tiles of
+    128x128 (64x64, 128x64 or 128x128 tiles, one to eight K ranges), and 129 to 256 tiles of 256x128 -- fp16 and bf16
+    operands, both output types, whole matrix against an fp32 product."""
+    import iree_turbine_amd  # noqa: F401
+    from iree_turbine_amd import _lib
+    from oracle import inputs
+
+    lib = _lib.load()
+    rng = random.Random(333)
+    split = 0
+    for case in range(48):
+        if case % 4 == 3:  # 129 to 256 tiles of 256x128
+            tm = rng.randint(2, 12)
+            tn = rng.randint(-(-129 // tm), 256 // tm)
+            M, N = 256 * tm, 128 * tn
+            K = 64 * rng.randint(4, 40)
+        else:
+            M = 64 * rng.randint(1, 32)
+            N = 64 * rng.randint(1, min(32, (1 << 21) // (64 * M)))
+            K = rng.choice([64, 128, 192, 320, 1024, 1088, 2048, 3072, 4096, 5120, 8192, 12288])
+        dtype = rng.choice([torch.float16, torch.bfloat16])
+        out_dtype = rng.choice(["float32", str(dtype).split(".")[1]])
+        need = lib.mi355_gemm_nt_workspace_bytes(M, N, K)
+        split += need > 0
+        announce(f"random small/mid gemm {case}: {M}x{N}x{K} {dtype} -> {out_dtype}, workspace {need >> 10} KiB")
+        a, b = [t.to(dev) for t in inputs.gemm_inputs(M, N, K, seed=400 + case, dtype=dtype)]
+        c = torch.ops.mi355.gemm_nt(a, b, out_dtype, -1)
+        tol = dict(rtol=1e-3, atol=1e-3) if out_dtype == "float32" else dict(rtol=1e-2, atol=1e-2)
+        torch.testing.assert_close(c.float(), a.float() @ b.float().t(), **tol)
+    assert split >= 6  # the draw does exercise the split
+
+
 def test_random_attention(dev):
     import iree_turbine_amd  # noqa: F401
     from oracle import attention as oa
