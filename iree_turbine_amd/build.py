@@ -128,7 +128,7 @@ def build_library(verbose: bool = True, save_temps: bool = False, defines: tuple
     return lib_path
 
 
-PROBES = ["lds_read_patterns.hip", "load_rate.hip", "mfma_load_bubble.hip"]
+PROBES = ["lds_read_patterns.hip", "load_rate.hip", "mfma_load_bubble.hip", "hbm_read_patterns.hip"]
 
 
 def build_probes(verbose: bool = True) -> list[Path]:
