@@ -1245,17 +1245,15 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_persistent(const half
 }
 
 // Skinny-M kernel (M <= 32, the decode-shaped product): weight streaming, HBM bound.  One workgroup of 8 waves per
-// 32 rows of B; wave w owns the 64-half K segments w, w + 8, ... of those rows.  Its B segments (32 rows x 128 bytes)
-// go global -> LDS directly, 8 rows per instruction, into a private ring of four 4 KiB stages; its A fragments
-// (row r32, 16 bytes per k-step: straight from L2 in the MFMA's layout) go into one of four register sets.  Both are
-// requested three segments ahead, so a CU keeps 96 KiB of weights in flight: what 8 TB/s over 256 CUs needs at a
-// latency of about 2 us is 62 KiB, and with one segment ahead (32 KiB; A staged through LDS beside B, two stages) the
-// kernel read at 4.5 TB/s where a plain read of the same 128 MiB runs at 6.3.  Rows of A past M repeat row M - 1
-// (same cache lines; their output columns are never stored).  The 8 partial 32 x 32 tiles are summed through LDS at
-// the end.
-// The loads of A, the waits and the LDS fragment reads are inline assembly: with direct-to-LDS loads in flight the
-// compiler waits for ALL of them before any LDS access it can see, which would serialise the ring.  Loads return in
-// order, so "at most the 8 loads each of the next three segments outstanding" means this one has landed.
+// 32 rows of B; wave w owns the 64-half K segments w, w + 8, ... of those rows and walks them through a private
+// double buffer in LDS (2 x (4 KiB of B + 4 KiB of A)): the direct-to-LDS loads of segment j + 1 -- 8 rows x 128
+// bytes per instruction for both operands -- are issued before segment j is consumed.  Rows of A past M repeat row
+// M - 1 (same cache lines; their output columns are never stored).  The 8 partial 32 x 32 tiles are summed through
+// LDS at the end.
+// Nothing loaded is carried in registers across iterations, and the waits and the LDS fragment reads are inline
+// assembly: with direct-to-LDS loads in flight the compiler waits for ALL of them before any LDS access it can
+// see, which would serialise the two segments.  Loads return in order, so "at most the 8 loads of the next segment
+// outstanding" means this one has landed.
 template <typename OutT, bool BF>
 __global__ __launch_bounds__(512) void gemm_f16_nt_skinny(const half_t* __restrict__ A, const half_t* __restrict__ B,
                                                           OutT* __restrict__ C, int M, int N, int K) {
@@ -1273,89 +1271,59 @@ __global__ __launch_bounds__(512) void gemm_f16_nt_skinny(const half_t* __restri
 #pragma unroll
   for (int r = 0; r < 16; r++) acc[r] = 0.f;
 
-  // global side of the B loads: instruction i covers rows 8i .. 8i + 7, lane = (row, slot); the chunk it fetches is
+  // global side of the loads: instruction i covers rows 8i .. 8i + 7, lane = (row, slot); the chunk it fetches is
   // slot ^ ((row >> 1) & 7), the swizzle of the tiled kernels
   const int lrow = lane >> 3;
   const half_t* b_src[4];
+  const half_t* a_src[4];
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     const int row = i * 8 + lrow;
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     b_src[i] = B + (size_t)(n0 + row) * K + chunk * 8;
+    a_src[i] = A + (size_t)(row < M ? row : M - 1) * K + chunk * 8;
   }
-  // A fragments: row r32 (clamped), halfs 16 ks + 8 h .. + 7 of the segment
-  const half_t* a_lane = A + (size_t)(r32 < M ? r32 : M - 1) * K + 8 * h + wave * 64;
-  // fragment reads of B: row r32, chunk 2 * ks + h
+  // fragment reads: row r32, chunk 2 * ks + h
   unsigned rd[4];
 #pragma unroll
   for (int ks = 0; ks < 4; ks++) rd[ks] = my_lds + r32 * 128 + (((2 * ks + h) ^ ((r32 >> 1) & 7)) * 16);
 
   // The workgroups of an XCD start their sweep over K at different places: rows are 2 K bytes apart, so 256 workgroups
   // that all read the same offset of their 32 rows at the same time crowd a few memory channels (a plain read of the
-  // same 128 MiB in this pattern: 27.9 us; with the start rotated by the workgroup's index within its XCD: 23.5 us).
+  // same 128 MiB in this order: 27.6 us whatever the prefetch depth; with the start rotated by the workgroup's index
+  // within its XCD: 23.2 us, as fast as a linear sweep; this kernel on 16 x 8192 x 8192: 31.2 -> 24.5 us).
   const int rot = mine > 0 ? (int)(blockIdx.x >> 3) % mine : 0;
-  half8 fa[4][4];  // [set][k-step]
-  auto issue = [&](auto set_tag, int j) __attribute__((always_inline)) {
-    constexpr int SET = decltype(set_tag)::value;
+  auto issue = [&](int j) {
     const int jr = j + rot < mine ? j + rot : j + rot - mine;
     const int seg = wave + 8 * jr;
-    char* dst = my + SET * 4096;
+    char* dst = my + (j & 1) * 8192;
 #pragma unroll
     for (int i = 0; i < 4; i++) load_lds_16B(b_src[i] + seg * 64, dst + i * 1024);
-    const half_t* ap = a_lane + (size_t)jr * 512;
-#if defined(MI355_ABLATE_NO_A_LOADS)
-    ap = a_lane;  // timing only: the same 128 bytes every time (an L1 hit)
-#endif
-    asm volatile("global_load_dwordx4 %0, %4, off\n\t"
-                 "global_load_dwordx4 %1, %4, off offset:32\n\t"
-                 "global_load_dwordx4 %2, %4, off offset:64\n\t"
-                 "global_load_dwordx4 %3, %4, off offset:96"
-                 : "=&v"(fa[SET][0]), "=&v"(fa[SET][1]), "=&v"(fa[SET][2]), "=&v"(fa[SET][3])
-                 : "v"(ap)
-                 : "memory");
+#pragma unroll
+    for (int i = 0; i < 4; i++) load_lds_16B(a_src[i] + seg * 64, dst + 4096 + i * 1024);
     __builtin_amdgcn_sched_barrier(0);
   };
-  auto step = [&](auto set_tag, auto ahead_tag, int j) __attribute__((always_inline)) {
-    constexpr int SET = decltype(set_tag)::value;
-    constexpr int AHEAD = (SET + 3) & 3;
-    if (j + 3 < mine) {
-      issue(std::integral_constant<int, AHEAD>{}, j + 3);
-      asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
-    } else if (j + 2 < mine) {
-      asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-    } else if (j + 1 < mine) {
-      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  if (mine > 0) issue(0);
+  for (int j = 0; j < mine; j++) {
+    if (j + 1 < mine) {
+      issue(j + 1);
+      asm volatile("s_waitcnt vmcnt(8)");
     } else {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      asm volatile("s_waitcnt vmcnt(0)");
     }
-    half8 fb[4];
+    const unsigned bo = (unsigned)(j & 1) << 13;
+    half8 fb[4], fa[4];
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) asm volatile("ds_read_b128 %0, %1" : "=v"(fb[ks]) : "v"(rd[ks] + SET * 4096));
+    for (int ks = 0; ks < 4; ks++) {
+      asm volatile("ds_read_b128 %0, %1" : "=v"(fb[ks]) : "v"(rd[ks] + bo));
+      asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(fa[ks]) : "v"(rd[ks] + bo));
+    }
     asm volatile("s_waitcnt lgkmcnt(0)"
-                 : "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]), "+v"(fa[SET][0]), "+v"(fa[SET][1]), "+v"(fa[SET][2]),
-                   "+v"(fa[SET][3]));
+                 : "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]), "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]));
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) acc = mfma16<BF>(fb[ks], fa[SET][ks], acc);  // acc[n][m]
+    for (int ks = 0; ks < 4; ks++) acc = mfma16<BF>(fb[ks], fa[ks], acc);  // acc[n][m]
     __builtin_amdgcn_sched_barrier(0);
-    (void)ahead_tag;
-  };
-  using S0 = std::integral_constant<int, 0>;
-  using S1 = std::integral_constant<int, 1>;
-  using S2 = std::integral_constant<int, 2>;
-  using S3 = std::integral_constant<int, 3>;
-  if (mine > 0) issue(S0{}, 0);
-  if (mine > 1) issue(S1{}, 1);
-  if (mine > 2) issue(S2{}, 2);
-  int j = 0;
-  for (; j + 4 <= mine; j += 4) {
-    step(S0{}, S3{}, j);
-    step(S1{}, S0{}, j + 1);
-    step(S2{}, S1{}, j + 2);
-    step(S3{}, S2{}, j + 3);
   }
-  if (j < mine) step(S0{}, S3{}, j);
-  if (j + 1 < mine) step(S1{}, S0{}, j + 1);
-  if (j + 2 < mine) step(S2{}, S1{}, j + 2);
 
   // reduce the 8 partial tiles: lane (m = r32, h) register r holds n = 8*(r/4) + 4h + r%4
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
