@@ -4,10 +4,16 @@
 //   columns: workgroup b of 256 owns 32 rows and sweeps them together, a 1 KiB window per row and step (wave w takes the
 //            128-byte segment w of the window, 8 rows per instruction): the skinny GEMM kernel's order
 //   columns, rotated: the same with the sweep started (b >> 3) steps in, i.e. at another place for every workgroup of an XCD
+// And the paged decode kernel's gather on its own: two pools of 18432 pages of 32 KiB (16 tokens x 8 kv heads x 256 B; 1.2 GB
+// in all), workgroup (list, kv head, split) reads slice `head` (16 rows of 256 B, 2 KiB apart) of each of the 96 pages of its
+// list from both pools, pages shuffled, in the kernel's grid order (split fastest) and with the head fastest.
 // Build and run: python -m iree_turbine_amd.build --probes && iree_turbine_amd/csrc/probes/bin/hbm_read_patterns
 #include <hip/hip_runtime.h>
+#include <algorithm>
 #include <cstdio>
 #include <cstdlib>
+#include <random>
+#include <vector>
 typedef int intx4 __attribute__((ext_vector_type(4)));
 #define CK(x) do { hipError_t e = (x); if (e != hipSuccess) { printf("err %s line %d\n", hipGetErrorString(e), __LINE__); exit(1);} } while (0)
 
@@ -47,6 +53,32 @@ __global__ __launch_bounds__(512) void read_columns(const char* __restrict__ src
     }
   }
   if (s == 0x12345) out[blockIdx.x * 512 + threadIdx.x] = s;
+}
+
+// grid: (split, head, list) for ORDER 0, (head, split, list) for ORDER 1; a wave takes pages w, w + 4, ..., two per step
+template <int ORDER>
+__global__ __launch_bounds__(256) void read_pages(const char* __restrict__ kp, const char* __restrict__ vp, const int* __restrict__ table, int pages,
+                                                  int* out) {
+  const int split = ORDER == 0 ? blockIdx.x : blockIdx.y, head = ORDER == 0 ? blockIdx.y : blockIdx.x, list = blockIdx.z;
+  const int nsplit = ORDER == 0 ? gridDim.x : gridDim.y;
+  const int* t = table + ((size_t)list * nsplit + split) * pages;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const size_t lo = (size_t)(lane >> 4) * 2048 + (lane & 15) * 16 + head * 256;  // 4 rows of 256 bytes per instruction
+  int s = 0;
+  for (int p = w; p < pages; p += 8) {
+    intx4 v[16];
+    const size_t b0 = (size_t)t[p] * 32768, b1 = (size_t)t[p + 4 < pages ? p + 4 : p] * 32768;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      v[i] = *(const intx4*)(kp + b0 + lo + i * 8192);
+      v[4 + i] = *(const intx4*)(vp + b0 + lo + i * 8192);
+      v[8 + i] = *(const intx4*)(kp + b1 + lo + i * 8192);
+      v[12 + i] = *(const intx4*)(vp + b1 + lo + i * 8192);
+    }
+#pragma unroll
+    for (int i = 0; i < 16; i++) s += v[i][0] ^ v[i][3];
+  }
+  if (s == 0x12345) out[threadIdx.x] = s;
 }
 
 static const size_t kBytes = (size_t)128 << 20;
@@ -94,6 +126,40 @@ int main() {
   });
   timed("columns, 4 steps ahead, rotated", [&](int s) { hipLaunchKernelGGL((read_columns<4, true>), dim3(256), dim3(512), 0, 0, set(s), out); });
   CK(hipFree(src));
+
+  const int lists = 64, nsplit = 3, pages = 96, P = lists * nsplit * pages;
+  char *kp, *vp;
+  int* table;
+  CK(hipMalloc(&kp, (size_t)P * 32768));
+  CK(hipMalloc(&vp, (size_t)P * 32768));
+  CK(hipMalloc(&table, P * 4));
+  CK(hipMemset(kp, 1, (size_t)P * 32768));
+  CK(hipMemset(vp, 1, (size_t)P * 32768));
+  std::vector<int> perm(P);
+  for (int i = 0; i < P; i++) perm[i] = i;
+  std::mt19937 gen(1);
+  std::shuffle(perm.begin(), perm.end(), gen);
+  CK(hipMemcpy(table, perm.data(), P * 4, hipMemcpyHostToDevice));
+  for (int order = 0; order < 2; order++) {
+    hipEvent_t e0, e1;
+    CK(hipEventCreate(&e0));
+    CK(hipEventCreate(&e1));
+    auto launch = [&]() {
+      if (order == 0) hipLaunchKernelGGL(read_pages<0>, dim3(nsplit, 8, lists), dim3(256), 0, 0, kp, vp, table, pages, out);
+      else hipLaunchKernelGGL(read_pages<1>, dim3(8, nsplit, lists), dim3(256), 0, 0, kp, vp, table, pages, out);
+    };
+    for (int r = 0; r < 5; r++) launch();
+    CK(hipEventRecord(e0, 0));
+    for (int r = 0; r < 20; r++) launch();
+    CK(hipEventRecord(e1, 0));
+    CK(hipEventSynchronize(e1));
+    float ms;
+    CK(hipEventElapsedTime(&ms, e0, e1));
+    const double bytes = 2.0 * P * 32768;
+    printf("%-72s %6.1f us per launch  %5.2f TB/s\n", order ? "decode's page gather (1.2 GB, shuffled pages), kv head fastest in the grid" : "decode's page gather (1.2 GB, shuffled pages), split fastest (the kernel's grid)",
+           ms * 1000 / 20, bytes / (ms / 20 * 1e-3) / 1e12);
+    fflush(stdout);
+  }
   CK(hipFree(out));
   return 0;
 }
