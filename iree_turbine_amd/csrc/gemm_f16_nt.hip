@@ -1348,6 +1348,122 @@ __global__ __launch_bounds__(512) void gemm_f16_nt_skinny(const half_t* __restri
   }
 }
 
+// The skinny kernel for 33 to 64 rows in one launch (two launches of the kernel above would read the weights twice): the
+// same decomposition and B path (segments through a private two-stage LDS ring), two 32-row blocks of A.  A wave's 16
+// KiB of LDS hold B's two stages and ONE 8 KiB stage of A (64 rows x 128 bytes; two would make 192 KiB for the
+// workgroup): the A segment j + 1 is requested as soon as the fragments of A segment j sit in registers, in front of the
+// step's MFMAs, and comes out of L2 while they run and while the wave waits for B, which comes from memory and was
+// requested a step earlier.  (A fragments loaded straight into registers, 32 lines per instruction instead of 8, made
+// the load path the bottleneck: 64 x 8192 x 8192 in 43.5 us.)  Loads return in order, and a step's B loads are issued
+// behind the A loads of the step before, so "at most the 4 newest loads outstanding" means B and A of this step have
+// landed.  Same rotation of the sweep's start.
+template <typename OutT, bool BF>
+__global__ __launch_bounds__(512) void gemm_f16_nt_skinny64(const half_t* __restrict__ A, const half_t* __restrict__ B,
+                                                            OutT* __restrict__ C, int M, int N, int K) {
+  extern __shared__ __attribute__((aligned(16384))) char lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r32 = lane & 31, h = lane >> 5;
+  const int n0 = blockIdx.x * 32;
+  const int nseg = K >> 6;
+  const int mine = wave < nseg ? (nseg - wave + 7) >> 3 : 0;  // segments of this wave
+  char* my = lds + wave * 16384;  // B stage 0 | B stage 1 | A (8 KiB)
+  const unsigned my_lds = (unsigned)(uintptr_t)MI355_LDS(char, my);
+
+  floatx16 acc[2];
+#pragma unroll
+  for (int b = 0; b < 2; b++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[b][r] = 0.f;
+
+  const int lrow = lane >> 3;
+  const half_t* b_src[4];
+  const half_t* a_src[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) {
+    const int row = i * 8 + lrow;
+    const int chunk = (lane & 7) ^ ((row >> 1) & 7);
+    if (i < 4) b_src[i] = B + (size_t)(n0 + row) * K + chunk * 8;
+    a_src[i] = A + (size_t)(row < M ? row : M - 1) * K + chunk * 8;
+  }
+  unsigned rd[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ks++) rd[ks] = my_lds + r32 * 128 + (((2 * ks + h) ^ ((r32 >> 1) & 7)) * 16);
+
+  const int rot = mine > 0 ? (int)(blockIdx.x >> 3) % mine : 0;
+  auto segment = [&](int j) {
+    const int jr = j + rot < mine ? j + rot : j + rot - mine;
+    return wave + 8 * jr;
+  };
+  auto issue_b = [&](int j) {
+    const int seg = segment(j);
+    char* dst = my + (j & 1) * 4096;
+#pragma unroll
+    for (int i = 0; i < 4; i++) load_lds_16B(b_src[i] + seg * 64, dst + i * 1024);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto issue_a = [&](int j) {
+    const int seg = segment(j);
+#pragma unroll
+    for (int i = 0; i < 8; i++) load_lds_16B(a_src[i] + seg * 64, my + 8192 + i * 1024);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  if (mine > 0) {
+    issue_b(0);
+    issue_a(0);
+  }
+  for (int j = 0; j < mine; j++) {
+    if (j + 1 < mine) {
+      issue_b(j + 1);
+      asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    const unsigned bo = (unsigned)(j & 1) << 12;
+    half8 fb[4], fa0[4], fa1[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+      asm volatile("ds_read_b128 %0, %1" : "=v"(fb[ks]) : "v"(rd[ks] + bo));
+      asm volatile("ds_read_b128 %0, %1 offset:8192" : "=v"(fa0[ks]) : "v"(rd[ks]));
+      asm volatile("ds_read_b128 %0, %1 offset:12288" : "=v"(fa1[ks]) : "v"(rd[ks]));
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]), "+v"(fa0[0]), "+v"(fa0[1]), "+v"(fa0[2]), "+v"(fa0[3]),
+                   "+v"(fa1[0]), "+v"(fa1[1]), "+v"(fa1[2]), "+v"(fa1[3])
+                 :
+                 : "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    if (j + 1 < mine) issue_a(j + 1);  // the A stage is free: its fragments sit in registers
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+      acc[0] = mfma16<BF>(fb[ks], fa0[ks], acc[0]);  // acc[n][m]
+      acc[1] = mfma16<BF>(fb[ks], fa1[ks], acc[1]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  // reduce the 8 partial tiles of each row block, as above
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+  __syncthreads();
+  constexpr int RED_PITCH = 36;
+  float* red = reinterpret_cast<float*>(lds);  // [wave][m 64][RED_PITCH]
+#pragma unroll
+  for (int b = 0; b < 2; b++)
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      const floatx4 v = {acc[b][4 * q], acc[b][4 * q + 1], acc[b][4 * q + 2], acc[b][4 * q + 3]};
+      *reinterpret_cast<floatx4*>(red + (wave * 64 + 32 * b + r32) * RED_PITCH + 8 * q + 4 * h) = v;
+    }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < 2048; idx += 512) {
+    const int m = idx >> 5, n = idx & 31;
+    float v = 0.f;
+#pragma unroll
+    for (int w = 0; w < 8; w++) v += red[(w * 64 + m) * RED_PITCH + n];
+    if (m < M) OutPack<OutT, BF>::store1(C + (size_t)m * N + n0 + n, v);
+  }
+}
+
 // Any-shape kernel: 64x64 tile, 4 waves, bounds-checked staging through registers.  Used for
 // shapes the tiled kernel does not divide (and as an independent implementation in tests).
 template <typename OutT, bool BF>
@@ -1733,8 +1849,13 @@ static int launch_variant(int variant, const void* a, const void* b, void* c, in
       static std::atomic<uint64_t> lds_ok{0};
       if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt_skinny")) return rc;
       dim3 grid(N / 32), block(512);
-      // 33 to 64 rows: two launches of up to 32 rows each (B streamed twice is still 1.8x faster than a 128x128
-      // tiling that leaves three quarters of the chip idle)
+      if (M > 32) {  // 33 to 64 rows: the kernel with two row blocks, which reads the weights once
+        auto kern64 = gemm_f16_nt_skinny64<OutT, BF>;
+        static std::atomic<uint64_t> lds_ok64{0};
+        if (int rc = allow_lds(reinterpret_cast<const void*>(kern64), lds_bytes, lds_ok64, "gemm_f16_nt_skinny64")) return rc;
+        hipLaunchKernelGGL(kern64, grid, block, lds_bytes, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, M, N, K);
+        return check_launch("gemm_f16_nt_skinny64", grid, block, lds_bytes);
+      }
       for (int m0 = 0; m0 < M; m0 += 32) {
         const int rows = M - m0 < 32 ? M - m0 : 32;
         hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)a + (size_t)m0 * K, (const half_t*)b,

@@ -528,10 +528,12 @@ def test_gemm_large_ragged_shapes_take_the_padded_path(dev, shape, dtype, out_dt
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("shape", [(16, 8192, 8192), (1, 4096, 4096), (32, 2048, 192), (7, 256, 64), (32, 32, 448), (5, 64, 1088),
-                                   (20, 4096, 14336), (31, 96, 8256), (64, 4096, 4096), (33, 2048, 1024), (50, 64, 320)])
+                                   (20, 4096, 14336), (31, 96, 8256), (64, 4096, 4096), (33, 2048, 1024), (50, 64, 320),
+                                   (64, 32, 64), (40, 96, 448), (48, 2048, 8256), (64, 8192, 8192), (57, 4096, 1088)])
 def test_gemm_skinny_m(dev, shape, dtype):
-    """The weight-streaming kernel for M <= 64 (33 rows and more take two launches): one to 64 rows, one K segment per wave and fewer segments than waves,
-    odd segment counts (the double buffer ends on either half), several segments per wave; fp32 result against the
+    """The weight-streaming kernels for M <= 64 (33 rows and more take the kernel with two row blocks): one to 64 rows, one K
+    segment per wave and fewer segments than waves, odd segment counts (the double buffer ends on either half), several
+    segments per wave, more workgroups per XCD than segments per wave (the rotated start wraps); fp32 result against the
     fp32 product of the same values, 16-bit result = the fp32 result rounded, launches repeat bit for bit, and
     decode-shaped products take this kernel by themselves."""
     import iree_turbine_amd as ita
