@@ -1940,6 +1940,8 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
     else if (fits(V_STREAM_TAIL) && t256 >= 128) variant = V_STREAM_TAIL;
     else if (fits(V_PERSISTENT) && t256 >= 128 && full_rounds) variant = V_PERSISTENT;
     else if (fits(V_PIPELINED_128)) variant = V_PIPELINED_128;
+    else if (fits(V_PIPELINED_128x64)) variant = V_PIPELINED_128x64;  // larger products that divide by 64 and not by 128
+    else if (fits(V_PIPELINED_64)) variant = V_PIPELINED_64;
     else variant = kNumGemmVariants - 1;
   } else if (!fits(variant) && variant == V_SKINNY) {
     return fail(-MI355_E_SHAPE, "gemm_f16_nt: variant %s needs M<=64, N%%32==0, K%%64==0 and 16-byte aligned pointers",

@@ -1768,7 +1768,7 @@ extern "C" int mi355_mxfp4_gemm(const void* a, const void* a_scale, const void* 
     // Few tiles: what counts is how many CUs pull operands (a lone workgroup moves about 75-100 GB/s through its CU
     // whatever its tile), so up to 320 tiles of 64x64 take those (128x8192x8192: 16.7 us on 128x128 tiles, 10.8 on
     // 64x64; 1024x1024x8192 15.3 -> 10.0; 256x8192x8192, 512 tiles of 64x64: 17.6 against 18.7).
-    else if (fits(7) && (M / 64) * (N / 64) <= 320) variant = 7;
+    else if (fits(7) && ((M / 64) * (N / 64) <= 320 || !fits(2))) variant = 7;  // also what divides by 64 and not by 128
     else if (fits(2)) variant = 2;
     else variant = kNumMxVariants - 1;
   } else if (!fits(variant)) {

@@ -294,6 +294,26 @@ def test_gemm_small_products(dev, shape, out32, dtype):
         assert torch.equal(got, torch.ops.mi355.gemm_nt(a, b, out_dtype, v))
 
 
+@pytest.mark.parametrize("shape", [(1088, 2112, 2048), (1152, 2112, 1024), (2112, 1152, 1024)])
+def test_gemm_multiples_of_64_beyond_the_small_rule(dev, shape):
+    """Products too large for the small-product rule that divide by 64 and not by 128 (and too small for the launcher to
+    pad them) take the 64x64 or the 128x64 tile rather than the bounds-checked kernel: whole matrix against that kernel
+    and against an fp32 product."""
+    import iree_turbine_amd as ita
+
+    M, N, K = shape
+    announce(f"gemm multiples of 64 {shape}")
+    names = ita._lib.variants("gemm_f16_nt")
+    g = torch.Generator().manual_seed(M + N + K)
+    a = (torch.randn(M, K, generator=g) * 0.25).half().to(dev)
+    b = (torch.randn(N, K, generator=g) * 0.25).half().to(dev)
+    got = torch.ops.mi355.gemm_nt(a, b, "float32", -1)
+    tile = "pipelined_128x64x64_w2x2" if M % 128 == 0 else "pipelined_64x64x64_w2x2"
+    assert torch.equal(got, torch.ops.mi355.gemm_nt(a, b, "float32", names.index(tile)))  # the automatic choice is that kernel
+    torch.testing.assert_close(got, torch.ops.mi355.gemm_nt(a, b, "float32", len(names) - 1), rtol=1e-3, atol=1e-3)
+    torch.testing.assert_close(got, a.float() @ b.float().t(), rtol=1e-3, atol=1e-3)
+
+
 @pytest.mark.parametrize("out_dtype", ["float16", "float32"])
 @pytest.mark.parametrize("shape", [(256, 256, 256), (512, 768, 384), (1024, 512, 1152), (2048, 10240, 512), (4352, 4352, 640)])
 def test_gemm_stream_slab_rotation(dev, shape, out_dtype):

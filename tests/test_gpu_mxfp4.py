@@ -182,7 +182,7 @@ def test_mxfp4_full_size_repeatable(dev, shape):
 
 
 @pytest.mark.parametrize("shape", [(128, 128, 1024), (64, 64, 1024), (256, 256, 2048), (192, 320, 3072), (384, 640, 5120), (1024, 1024, 8192),
-                                   (128, 8192, 8192), (2048, 2048, 2048), (2048, 2176, 1024), (1152, 1152, 4096)])
+                                   (128, 8192, 8192), (2048, 2048, 2048), (2048, 2176, 1024), (1152, 1152, 4096), (64, 28672, 1024)])
 @pytest.mark.parametrize("out_dtype", ["bfloat16", "float32"])
 def test_mxfp4_slab_form(dev, shape, out_dtype):
     """The tiled kernel's slab form (four data stages, a whole slab's fragments and scale dwords in one of two register
