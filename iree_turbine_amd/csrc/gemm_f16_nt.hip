@@ -67,7 +67,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
                                                                      const half_t* __restrict__ B,
                                                                      OutT* __restrict__ C, int M, int N, int K,
                                                                      int tiles_m, int tiles_n, int group_m, int ldk,
-                                                                     int split_tiles_m, int ksplit_halfs) {
+                                                                     int split_tiles_m, int ksplit_halfs, int krot_step) {
   // K: the length of the K range a workgroup adds up; ldk: the row pitch of A and B in halfs.  With a K split
   // (split_tiles_m > 0) the tile grid is stacked S times along M: tile row t stands for tile row t % split_tiles_m of A
   // and the K range t / split_tiles_m, ksplit_halfs apart, and C (the workspace) has S times the rows.
@@ -107,7 +107,19 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
   const unsigned lane_off = (unsigned)lrow * (unsigned)ldk + (unsigned)lchunk * 8u;
   const size_t row_step = (size_t)NW * 8 * ldk;
 
-  auto issue_loads = [&](int stage, int slab) {
+  // krot_step != 0 (a few rows of A against many rows of B, which then stream from memory): the workgroups of tile
+  // column n start their sweep over K n slabs in.  The rows of B are 2 K bytes apart, and workgroups that all read the
+  // same offset of their rows at the same time crowd a few memory channels (128 x 28672 x 8192 with the weights out of
+  // every cache: 122.5 -> 100.2 us); the workgroups of a column, which share those rows, still sweep together, and A is
+  // small enough to stay in the L2s whatever the order.  With both operands large the rotation loses (the row panels
+  // of A are shared by workgroups of different columns).
+  const int krot = krot_step ? tile_n % (K / 64) : 0;
+  auto rotated = [&](int slab) {
+    const int r = slab + krot;
+    return r < K / 64 ? r : r - K / 64;
+  };
+  auto issue_loads = [&](int stage, int slab0) {
+    const int slab = rotated(slab0);
     char* dst = lds + stage * STAGE + wave * 1024;
     const half_t* ap = a_src + slab * 64;
     const half_t* bp = b_src + slab * 64;
@@ -162,7 +174,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
     auto trip = [&](int kt, half8(*cm)[TM], half8(*cn)[TN], half8(*nm)[TM], half8(*nn)[TN]) {
       const int next = stage + 1 == STAGES ? 0 : stage + 1;
       const char* st = lds + next * STAGE;
-      const int slab = kt + STAGES < KT ? kt + STAGES : KT - 1;
+      const int slab = rotated(kt + STAGES < KT ? kt + STAGES : KT - 1);
       __builtin_amdgcn_sched_barrier(0);
       if constexpr (PINNED) {
         char* dst = lds + stage * STAGE + wave * 1024;
@@ -187,7 +199,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
         }
       } else {
         read_slab(st, nm, nn);
-        issue_loads(stage, slab);
+        issue_loads(stage, kt + STAGES < KT ? kt + STAGES : KT - 1);
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) mfmas(cm[ks], cn[ks]);
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -1579,6 +1591,10 @@ static int cu_count() {
 // tiles (64 and 96 KiB: two and one workgroup per CU) always.
 static bool pipelined_slab_form(long long tiles, int bm_plus_bn) { return bm_plus_bn != 256 || tiles <= 256; }
 
+// Whether the workgroups of a tile column start their K sweep at another place (the kernel's krot_step): A at most 4 MiB
+// (it stays in the L2s in any order), B at least 16 MiB (it streams).
+static int pipelined_krot(long long M, long long N, long long K) { return M * K * 2 <= (4 << 20) && N * K * 2 >= (16 << 20); }
+
 template <int BM, int BN, int WM, int WN, typename OutT, int KIND, bool BF>  // KIND: 1 pipelined, 2 register-staged
 static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int K, int ldc, hipStream_t stream) {
   // the kernels use their N argument only as the row stride of C, so a column range of a wider C is the
@@ -1600,7 +1616,7 @@ static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int
     auto go = [&](auto kern, int lds_bytes, std::atomic<uint64_t>& lds_ok) {
       if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt")) return rc;
       hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, M, ldc, K, tiles_m,
-                         tiles_n, group_m, K, 0, 0);
+                         tiles_n, group_m, K, 0, 0, pipelined_krot(M, N, K));
       return check_launch("gemm_f16_nt_pipelined", grid, block, lds_bytes);
     };
     static std::atomic<uint64_t> lds_ok2{0}, lds_ok4{0};
@@ -1621,7 +1637,8 @@ static int launch_pipelined_ksplit(const half_t* a, const half_t* b, float* ws, 
   dim3 grid(tiles_m * tiles_n), block(256);
   auto go = [&](auto kern, int lds_bytes, std::atomic<uint64_t>& lds_ok) {
     if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt")) return rc;
-    hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, a, b, ws, M * S, N, k_part, tiles_m, tiles_n, 4, K, M / BM, k_part);
+    hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, a, b, ws, M * S, N, k_part, tiles_m, tiles_n, 4, K, M / BM, k_part,
+                       pipelined_krot(M, N, K));
     return check_launch("gemm_f16_nt_pipelined (K split)", grid, block, lds_bytes);
   };
   static std::atomic<uint64_t> lds_ok2{0}, lds_ok4{0};
