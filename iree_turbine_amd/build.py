@@ -46,7 +46,7 @@ def _hipcc() -> str:
 # waves per SIMD (a spill there also costs the time their schedules were tuned for).
 NO_SPILL_KERNELS = ("staged", "skinny", "gemm_f16_nt_stream", "gemm_mxfp4_stream", "gemm_mxfp8_stream", "fa_fwd_d128_pipe",
                     "fa_fwd_d128_m16", "fa_fwd_d128_walk", "paged_decode_phase0", "gemm_f16_nt_pipelined", "gemm_mxfp4_tiled")
-EXPECTED_OCCUPANCY = {"staged": 1, "gemm_f16_nt_stream": 1, "gemm_mxfp4_stream": 1, "gemm_mxfp8_stream": 1, "gemm_f16_nt_skinny": 7, "gemm_f16_nt_skinny64": 4,
+EXPECTED_OCCUPANCY = {"staged": 1, "gemm_f16_nt_stream": 1, "gemm_mxfp4_stream": 1, "gemm_mxfp8_stream": 1, "gemm_f16_nt_skinnyI": 7,
                       "gemm_mxfp4_skinny": 2, "fa_fwd_d128_pipe": 2, "fa_fwd_d128_m16": 2, "fa_fwd_d128_walk": 2, "paged_decode_phase0": 2}
 _USAGE_FLAG = "-Rpass-analysis=kernel-resource-usage"
 

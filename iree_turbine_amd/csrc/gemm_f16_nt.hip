@@ -1360,39 +1360,43 @@ __global__ __launch_bounds__(512) void gemm_f16_nt_skinny(const half_t* __restri
   }
 }
 
-// The skinny kernel for 33 to 64 rows in one launch (two launches of the kernel above would read the weights twice): the
-// same decomposition and B path (segments through a private two-stage LDS ring), two 32-row blocks of A.  A wave's 16
-// KiB of LDS hold B's two stages and ONE 8 KiB stage of A (64 rows x 128 bytes; two would make 192 KiB for the
-// workgroup): the A segment j + 1 is requested as soon as the fragments of A segment j sit in registers, in front of the
-// step's MFMAs, and comes out of L2 while they run and while the wave waits for B, which comes from memory and was
+// The skinny kernel for more than 32 rows in one launch (launches of the kernel above for 32 rows each would read the
+// weights once each): the same decomposition and B path (segments through a private two-stage LDS ring), RB 32-row
+// blocks of A, NW waves that split K.  A wave's LDS holds B's two stages (8 KiB) and ONE stage of A (RB x 4 KiB: two
+// would not fit): the A segment j + 1 is requested as soon as the fragments of A segment j sit in registers, in front of
+// the step's MFMAs, and comes out of L2 while they run and while the wave waits for B, which comes from memory and was
 // requested a step earlier.  (A fragments loaded straight into registers, 32 lines per instruction instead of 8, made
-// the load path the bottleneck: 64 x 8192 x 8192 in 43.5 us.)  Loads return in order, and a step's B loads are issued
-// behind the A loads of the step before, so "at most the 4 newest loads outstanding" means B and A of this step have
-// landed.  Same rotation of the sweep's start.
-template <typename OutT, bool BF>
-__global__ __launch_bounds__(512) void gemm_f16_nt_skinny64(const half_t* __restrict__ A, const half_t* __restrict__ B,
-                                                            OutT* __restrict__ C, int M, int N, int K) {
+// the load path the bottleneck: 64 x 8192 x 8192 in 43.5 us against 35.7.)  RB = 2 with 8 waves (33 to 64 rows, 128 KiB
+// of LDS), RB = 4 with 4 waves (65 to 128 rows, 96 KiB).  Loads return in order, and a step's B loads are issued behind
+// the A loads of the step before, so "at most the 4 newest loads outstanding" means B and A of this step have landed.
+// Same rotation of the sweep's start.
+template <typename OutT, bool BF, int RB, int NW>
+__global__ __launch_bounds__(NW * 64) void gemm_f16_nt_skinny_rb(const half_t* __restrict__ A, const half_t* __restrict__ B,
+                                                                OutT* __restrict__ C, int M, int N, int K) {
+  constexpr int WAVE_LDS = 8192 + RB * 4096;  // B stage 0 | B stage 1 | A (RB x 4 KiB)
+  constexpr int RED_PITCH = 36;
+  static_assert(NW * WAVE_LDS <= 160 * 1024 && NW * 32 * RB * RED_PITCH * 4 <= NW * WAVE_LDS, "stages and the reduction fit");
   extern __shared__ __attribute__((aligned(16384))) char lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r32 = lane & 31, h = lane >> 5;
   const int n0 = blockIdx.x * 32;
   const int nseg = K >> 6;
-  const int mine = wave < nseg ? (nseg - wave + 7) >> 3 : 0;  // segments of this wave
-  char* my = lds + wave * 16384;  // B stage 0 | B stage 1 | A (8 KiB)
+  const int mine = wave < nseg ? (nseg - wave + NW - 1) / NW : 0;  // segments of this wave
+  char* my = lds + wave * WAVE_LDS;
   const unsigned my_lds = (unsigned)(uintptr_t)MI355_LDS(char, my);
 
-  floatx16 acc[2];
+  floatx16 acc[RB];
 #pragma unroll
-  for (int b = 0; b < 2; b++)
+  for (int b = 0; b < RB; b++)
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[b][r] = 0.f;
 
   const int lrow = lane >> 3;
   const half_t* b_src[4];
-  const half_t* a_src[8];
+  const half_t* a_src[4 * RB];
 #pragma unroll
-  for (int i = 0; i < 8; i++) {
+  for (int i = 0; i < 4 * RB; i++) {
     const int row = i * 8 + lrow;
     const int chunk = (lane & 7) ^ ((row >> 1) & 7);
     if (i < 4) b_src[i] = B + (size_t)(n0 + row) * K + chunk * 8;
@@ -1405,7 +1409,7 @@ __global__ __launch_bounds__(512) void gemm_f16_nt_skinny64(const half_t* __rest
   const int rot = mine > 0 ? (int)(blockIdx.x >> 3) % mine : 0;
   auto segment = [&](int j) {
     const int jr = j + rot < mine ? j + rot : j + rot - mine;
-    return wave + 8 * jr;
+    return wave + NW * jr;
   };
   auto issue_b = [&](int j) {
     const int seg = segment(j);
@@ -1417,7 +1421,7 @@ __global__ __launch_bounds__(512) void gemm_f16_nt_skinny64(const half_t* __rest
   auto issue_a = [&](int j) {
     const int seg = segment(j);
 #pragma unroll
-    for (int i = 0; i < 8; i++) load_lds_16B(a_src[i] + seg * 64, my + 8192 + i * 1024);
+    for (int i = 0; i < 4 * RB; i++) load_lds_16B(a_src[i] + seg * 64, my + 8192 + i * 1024);
     __builtin_amdgcn_sched_barrier(0);
   };
   if (mine > 0) {
@@ -1432,46 +1436,43 @@ __global__ __launch_bounds__(512) void gemm_f16_nt_skinny64(const half_t* __rest
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
     const unsigned bo = (unsigned)(j & 1) << 12;
-    half8 fb[4], fa0[4], fa1[4];
+    half8 fb[4], fa[RB][4];
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) {
       asm volatile("ds_read_b128 %0, %1" : "=v"(fb[ks]) : "v"(rd[ks] + bo));
-      asm volatile("ds_read_b128 %0, %1 offset:8192" : "=v"(fa0[ks]) : "v"(rd[ks]));
-      asm volatile("ds_read_b128 %0, %1 offset:12288" : "=v"(fa1[ks]) : "v"(rd[ks]));
+#pragma unroll
+      for (int b = 0; b < RB; b++) asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fa[b][ks]) : "v"(rd[ks]), "n"(8192 + 4096 * b));
     }
-    asm volatile("s_waitcnt lgkmcnt(0)"
-                 : "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3]), "+v"(fa0[0]), "+v"(fa0[1]), "+v"(fa0[2]), "+v"(fa0[3]),
-                   "+v"(fa1[0]), "+v"(fa1[1]), "+v"(fa1[2]), "+v"(fa1[3])
-                 :
-                 : "memory");
+    // one wait for all of them; the fragments are named so that no use moves above it
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fb[0]), "+v"(fb[1]), "+v"(fb[2]), "+v"(fb[3])::"memory");
+#pragma unroll
+    for (int b = 0; b < RB; b++) asm volatile("" : "+v"(fa[b][0]), "+v"(fa[b][1]), "+v"(fa[b][2]), "+v"(fa[b][3])::"memory");
     __builtin_amdgcn_sched_barrier(0);
     if (j + 1 < mine) issue_a(j + 1);  // the A stage is free: its fragments sit in registers
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) {
-      acc[0] = mfma16<BF>(fb[ks], fa0[ks], acc[0]);  // acc[n][m]
-      acc[1] = mfma16<BF>(fb[ks], fa1[ks], acc[1]);
-    }
+    for (int ks = 0; ks < 4; ks++)
+#pragma unroll
+      for (int b = 0; b < RB; b++) acc[b] = mfma16<BF>(fb[ks], fa[b][ks], acc[b]);  // acc[n][m]
     __builtin_amdgcn_sched_barrier(0);
   }
 
-  // reduce the 8 partial tiles of each row block, as above
+  // reduce the NW partial tiles of each row block, as above
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
   __syncthreads();
-  constexpr int RED_PITCH = 36;
-  float* red = reinterpret_cast<float*>(lds);  // [wave][m 64][RED_PITCH]
+  float* red = reinterpret_cast<float*>(lds);  // [wave][m 32 RB][RED_PITCH]
 #pragma unroll
-  for (int b = 0; b < 2; b++)
+  for (int b = 0; b < RB; b++)
 #pragma unroll
     for (int q = 0; q < 4; q++) {
       const floatx4 v = {acc[b][4 * q], acc[b][4 * q + 1], acc[b][4 * q + 2], acc[b][4 * q + 3]};
-      *reinterpret_cast<floatx4*>(red + (wave * 64 + 32 * b + r32) * RED_PITCH + 8 * q + 4 * h) = v;
+      *reinterpret_cast<floatx4*>(red + (wave * 32 * RB + 32 * b + r32) * RED_PITCH + 8 * q + 4 * h) = v;
     }
   __syncthreads();
-  for (int idx = threadIdx.x; idx < 2048; idx += 512) {
+  for (int idx = threadIdx.x; idx < 1024 * RB; idx += NW * 64) {
     const int m = idx >> 5, n = idx & 31;
     float v = 0.f;
 #pragma unroll
-    for (int w = 0; w < 8; w++) v += red[(w * 64 + m) * RED_PITCH + n];
+    for (int w = 0; w < NW; w++) v += red[(w * 32 * RB + m) * RED_PITCH + n];
     if (m < M) OutPack<OutT, BF>::store1(C + (size_t)m * N + n0 + n, v);
   }
 }
@@ -1866,12 +1867,20 @@ static int launch_variant(int variant, const void* a, const void* b, void* c, in
       static std::atomic<uint64_t> lds_ok{0};
       if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt_skinny")) return rc;
       dim3 grid(N / 32), block(512);
-      if (M > 32) {  // 33 to 64 rows: the kernel with two row blocks, which reads the weights once
-        auto kern64 = gemm_f16_nt_skinny64<OutT, BF>;
+      if (M > 64) {  // 65 to 128 rows: four row blocks, four waves
+        auto kern = gemm_f16_nt_skinny_rb<OutT, BF, 4, 4>;
+        constexpr int lds128 = 4 * (8192 + 4 * 4096);
+        static std::atomic<uint64_t> lds_ok128{0};
+        if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds128, lds_ok128, "gemm_f16_nt_skinny_rb")) return rc;
+        hipLaunchKernelGGL(kern, grid, dim3(256), lds128, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, M, N, K);
+        return check_launch("gemm_f16_nt_skinny_rb", grid, dim3(256), lds128);
+      }
+      if (M > 32) {  // 33 to 64 rows: two row blocks, eight waves; the weights are read once
+        auto kern64 = gemm_f16_nt_skinny_rb<OutT, BF, 2, 8>;
         static std::atomic<uint64_t> lds_ok64{0};
-        if (int rc = allow_lds(reinterpret_cast<const void*>(kern64), lds_bytes, lds_ok64, "gemm_f16_nt_skinny64")) return rc;
+        if (int rc = allow_lds(reinterpret_cast<const void*>(kern64), lds_bytes, lds_ok64, "gemm_f16_nt_skinny_rb")) return rc;
         hipLaunchKernelGGL(kern64, grid, block, lds_bytes, stream, (const half_t*)a, (const half_t*)b, (OutT*)c, M, N, K);
-        return check_launch("gemm_f16_nt_skinny64", grid, block, lds_bytes);
+        return check_launch("gemm_f16_nt_skinny_rb", grid, block, lds_bytes);
       }
       for (int m0 = 0; m0 < M; m0 += 32) {
         const int rows = M - m0 < 32 ? M - m0 : 32;
@@ -1919,7 +1928,7 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
     // the streamed kernel addresses each operand through one buffer descriptor
     if (streamed && (M * K * 2 >= (1ll << 32) || N * K * 2 >= (1ll << 32))) return false;
     if (streamed && (K < 256 || K % 128 != 0 || K > (1 << 21))) return false;  // slabs in pairs; 32-bit byte offsets inside a 256-row panel
-    if (v == V_SKINNY) return al && M <= 64 && N % 32 == 0 && K % 64 == 0;  // a tile is 32 rows of B; 64-half K segments
+    if (v == V_SKINNY) return al && M <= 128 && N % 32 == 0 && K % 64 == 0;  // a tile is 32 rows of B; 64-half K segments
     return al && M % kGemmVariants[v].bm == 0 && N % kGemmVariants[v].bn == 0 && K % 64 == 0;
   };
   int split128 = 1;  // K ranges of the 128x128 split, when the automatic choice takes it
@@ -1936,7 +1945,10 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
     // last round is >= 85% busy.
     const bool full_rounds = t256 * 100 >= rounds * 256 * 85;
     const int s128 = (workspace && fits(V_PIPELINED_128)) ? ksplit128_plan((int)M, (int)N, (int)K) : 1;
-    if (fits(V_SKINNY) && N >= 2048 && K >= 512) variant = V_SKINNY;  // decode-shaped: stream the weights once
+    // decode-shaped: stream the weights once.  Up to 64 rows always; 65 to 128 rows when M is no multiple of 64 (such
+    // products went to the bounds-checked kernel: 65 x 8192 x 8192 149 -> 36.5 us; at 128 rows the 64x64 tiles of the
+    // small-product rule are ahead, 43.9 against 47.9 us, and far ahead with many columns).
+    if (fits(V_SKINNY) && (M <= 64 || M % 64 != 0) && N >= 2048 && K >= 512) variant = V_SKINNY;
     else if (al && (small = small_plan(M, N, K, INT64_MAX)).bm) {
       // a workspace short of what the plan asks for is no workspace (not a plan with fewer ranges)
       if (small.S > 1 && (!workspace || workspace_bytes < (int64_t)small.S * M * N * 4)) small = small_plan(M, N, K, 0);
@@ -1961,7 +1973,7 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
     else if (fits(V_PIPELINED_64)) variant = V_PIPELINED_64;
     else variant = kNumGemmVariants - 1;
   } else if (!fits(variant) && variant == V_SKINNY) {
-    return fail(-MI355_E_SHAPE, "gemm_f16_nt: variant %s needs M<=64, N%%32==0, K%%64==0 and 16-byte aligned pointers",
+    return fail(-MI355_E_SHAPE, "gemm_f16_nt: variant %s needs M<=128, N%%32==0, K%%64==0 and 16-byte aligned pointers",
                 kGemmVariants[variant].name);
   } else if (!fits(variant)) {
     return fail(-MI355_E_SHAPE, "gemm_f16_nt: variant %s needs M%%%d==0, N%%%d==0, K%%64==0 and 16-byte aligned pointers",

@@ -549,9 +549,11 @@ def test_gemm_large_ragged_shapes_take_the_padded_path(dev, shape, dtype, out_dt
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("shape", [(16, 8192, 8192), (1, 4096, 4096), (32, 2048, 192), (7, 256, 64), (32, 32, 448), (5, 64, 1088),
                                    (20, 4096, 14336), (31, 96, 8256), (64, 4096, 4096), (33, 2048, 1024), (50, 64, 320),
-                                   (64, 32, 64), (40, 96, 448), (48, 2048, 8256), (64, 8192, 8192), (57, 4096, 1088)])
+                                   (64, 32, 64), (40, 96, 448), (48, 2048, 8256), (64, 8192, 8192), (57, 4096, 1088),
+                                   (65, 2048, 1024), (100, 4096, 2048), (128, 64, 320), (127, 2048, 8192), (96, 32, 64)])
 def test_gemm_skinny_m(dev, shape, dtype):
-    """The weight-streaming kernels for M <= 64 (33 rows and more take the kernel with two row blocks): one to 64 rows, one K
+    """The weight-streaming kernels for M <= 128 (33 to 64 rows take the kernel with two row blocks and eight waves, 65 to 128
+    rows four row blocks and four waves; the automatic choice takes them up to 64 rows and for ragged M beyond): one to 128 rows, one K
     segment per wave and fewer segments than waves, odd segment counts (the double buffer ends on either half), several
     segments per wave, more workgroups per XCD than segments per wave (the rotated start wraps); fp32 result against the
     fp32 product of the same values, 16-bit result = the fp32 result rounded, launches repeat bit for bit, and
@@ -572,7 +574,7 @@ def test_gemm_skinny_m(dev, shape, dtype):
     c16 = torch.ops.mi355.gemm_nt(a, b, own, sk)
     assert torch.equal(c16, c32.to(dtype))
     assert torch.equal(c32, torch.ops.mi355.gemm_nt(a, b, "float32", sk))
-    if N >= 2048 and K >= 512:
+    if N >= 2048 and K >= 512 and (M <= 64 or M % 64):
         assert torch.equal(c32, torch.ops.mi355.gemm_nt(a, b, "float32", -1))
 
 
@@ -581,10 +583,10 @@ def test_gemm_skinny_contract(dev):
 
     names = ita._lib.variants("gemm_f16_nt")
     sk = next(i for i, n in enumerate(names) if n.startswith("skinny"))
-    a = torch.zeros(65, 64, dtype=torch.float16, device=dev)
+    a = torch.zeros(129, 64, dtype=torch.float16, device=dev)
     b = torch.zeros(64, 64, dtype=torch.float16, device=dev)
     with pytest.raises(ValueError):
-        torch.ops.mi355.gemm_nt(a, b, "float32", sk)  # 65 rows
+        torch.ops.mi355.gemm_nt(a, b, "float32", sk)  # 129 rows
     with pytest.raises(ValueError):
         torch.ops.mi355.gemm_nt(a[:8], b[:48], "float32", sk)  # N = 48 is not whole 32-row tiles
     with pytest.raises(ValueError):
