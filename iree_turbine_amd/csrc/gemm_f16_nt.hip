@@ -62,7 +62,9 @@ template <bool BF> struct OutPack<half_t, BF> {
 //    A lone workgroup's slab time in the k-step form is its load latency plus, on small tiles, the chain of LDS read
 //    latencies of four k-steps with one or two MFMAs each to cover them: 64x64 0.22 -> 0.15 us per slab, 128x128
 //    0.60 -> 0.42 (what LDS bandwidth allows); 1024^3 on 64x64 tiles 6.7 -> 5.4 us, 1024x1024x4096 19.4 -> 15.9 us.
-template <int BM, int BN, int WM, int WN, typename OutT, bool BF, bool SLAB = false>
+//  * RAGGED_M: M is any number of rows (the last tile row is cut): its loads of A take row min(row, M - 1), so they
+//    stay inside A, and the epilogue stores the rows below M only.
+template <int BM, int BN, int WM, int WN, typename OutT, bool BF, bool SLAB = false, bool RAGGED_M = false>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_t* __restrict__ A,
                                                                      const half_t* __restrict__ B,
                                                                      OutT* __restrict__ C, int M, int N, int K,
@@ -102,10 +104,23 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
       a_tile -= split_tiles_m;
       k_at += (size_t)ksplit_halfs;
     }
-  const half_t* a_src = A + (size_t)(a_tile * BM + wave * 8) * ldk + k_at;
+  const half_t* a_src = A + (size_t)(a_tile * BM + (RAGGED_M ? 0 : wave * 8)) * ldk + k_at;
   const half_t* b_src = B + (size_t)(tile_n * BN + wave * 8) * ldk + k_at;
   const unsigned lane_off = (unsigned)lrow * (unsigned)ldk + (unsigned)lchunk * 8u;
   const size_t row_step = (size_t)NW * 8 * ldk;
+  // RAGGED_M: the offset (in halfs, from the tile's first row) of this lane's row in A load i, the row clamped to M - 1
+  unsigned a_off[RAGGED_M ? LA : 1];
+  if constexpr (RAGGED_M) {
+#pragma unroll
+    for (int i = 0; i < LA; i++) {
+      const int row = a_tile * BM + wave * 8 + i * NW * 8 + lrow;
+      a_off[i] = (unsigned)((row < M ? row : M - 1) - a_tile * BM) * (unsigned)ldk + (unsigned)lchunk * 8u;
+    }
+  }
+  auto load_a = [&](const half_t* ap, int i, char* dst) {  // ap: a_src at the slab
+    if constexpr (RAGGED_M) load_lds_16B(ap + a_off[i], dst);
+    else load_lds_16B(ap + i * row_step + lane_off, dst);
+  };
 
   // krot_step != 0 (a few rows of A against many rows of B, which then stream from memory): the workgroups of tile
   // column n start their sweep over K n slabs in.  The rows of B are 2 K bytes apart, and workgroups that all read the
@@ -124,7 +139,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
     const half_t* ap = a_src + slab * 64;
     const half_t* bp = b_src + slab * 64;
 #pragma unroll
-    for (int i = 0; i < LA; i++) load_lds_16B(ap + i * row_step + lane_off, dst + i * NW * 1024);
+    for (int i = 0; i < LA; i++) load_a(ap, i, dst + i * NW * 1024);
 #pragma unroll
     for (int i = 0; i < LB; i++) load_lds_16B(bp + i * row_step + lane_off, dst + A_BYTES + i * NW * 1024);
   };
@@ -192,7 +207,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
           }
 #pragma unroll
           for (int l = m * NL / NM; l < (m + 1) * NL / NM; l++) {
-            if (l < LA) load_lds_16B(ap + l * row_step + lane_off, dst + l * NW * 1024);
+            if (l < LA) load_a(ap, l, dst + l * NW * 1024);
             else load_lds_16B(bp + (l - LA) * row_step + lane_off, dst + A_BYTES + (l - LA) * NW * 1024);
           }
           __builtin_amdgcn_sched_barrier(0);
@@ -326,7 +341,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
     for (int it = 0; it < WTM / ROWS_PER_IT; it++) {
       const int row = it * ROWS_PER_IT + er;
       half8 v = *reinterpret_cast<const half8*>(ep + row * ROW_B + ((ec ^ ((row >> 1) & (CH - 1))) * 16));
-      *reinterpret_cast<half8*>(cbase + (size_t)row * N) = v;
+      if (!RAGGED_M || tile_m * BM + wm * WTM + row < M) *reinterpret_cast<half8*>(cbase + (size_t)row * N) = v;
     }
   } else {
     // fp32 epilogue, the same way (a lane's four consecutive n are one 16-byte chunk; chunk slot c ^ (m & (CH - 1))):
@@ -353,7 +368,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
     for (int it = 0; it < WTM / ROWS_PER_IT; it++) {
       const int row = it * ROWS_PER_IT + er;
       floatx4 v = *reinterpret_cast<const floatx4*>(ep + row * ROW_B + ((ec ^ (row & (CH - 1))) * 16));
-      *reinterpret_cast<floatx4*>(cbase + (size_t)row * N) = v;
+      if (!RAGGED_M || tile_m * BM + wm * WTM + row < M) *reinterpret_cast<floatx4*>(cbase + (size_t)row * N) = v;
     }
   }
 }
@@ -1596,12 +1611,14 @@ static bool pipelined_slab_form(long long tiles, int bm_plus_bn) { return bm_plu
 // (it stays in the L2s in any order), B at least 16 MiB (it streams).
 static int pipelined_krot(long long M, long long N, long long K) { return M * K * 2 <= (4 << 20) && N * K * 2 >= (16 << 20); }
 
-template <int BM, int BN, int WM, int WN, typename OutT, int KIND, bool BF>  // KIND: 1 pipelined, 2 register-staged
+// RAGGED: M is any number of rows (the pipelined kernel's slab form only: the caller has checked pipelined_slab_form)
+template <int BM, int BN, int WM, int WN, typename OutT, int KIND, bool BF, bool RAGGED = false>  // KIND: 1 pipelined, 2 register-staged
 static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int K, int ldc, hipStream_t stream) {
   // the kernels use their N argument only as the row stride of C, so a column range of a wider C is the
   // same launch with ldc in its place
   static_assert(KIND == 1 || KIND == 2, "pipelined or register-staged");
-  const int tiles_m = M / BM, tiles_n = N / BN;
+  static_assert(!RAGGED || KIND == 1, "only the pipelined kernel cuts its last tile row");
+  const int tiles_m = RAGGED ? (M + BM - 1) / BM : M / BM, tiles_n = N / BN;
   int group_m = 4;
   dim3 grid(tiles_m * tiles_n), block(WM * WN * 64);
   if constexpr (KIND == 2) {
@@ -1622,6 +1639,10 @@ static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int
     };
     static std::atomic<uint64_t> lds_ok2{0}, lds_ok4{0};
     constexpr int slab_stages = 4 * (BM + BN) * 128 <= 160 * 1024 ? 4 : 3;  // as the kernel picks them
+    if constexpr (RAGGED) {
+      static std::atomic<uint64_t> lds_okr{0};
+      return go(gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT, BF, true, true>, slab_stages * (BM + BN) * 128, lds_okr);
+    }
     if (pipelined_slab_form((long long)tiles_m * tiles_n, BM + BN))
       return go(gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT, BF, true>, slab_stages * (BM + BN) * 128, lds_ok4);
     if constexpr (BM + BN == 256) return go(gemm_f16_nt_pipelined<BM, BN, WM, WN, OutT, BF, false>, 2 * (BM + BN) * 128, lds_ok2);
@@ -1773,17 +1794,20 @@ static bool takes_256x128(int64_t M, int64_t N, int64_t K) {
 
 struct SmallPlan {
   int bm = 0, bn = 0, S = 1;  // bm == 0: not a small product
+  bool ragged = false;        // M is no multiple of bm: the last tile row is cut, and K is not split
 };
 static SmallPlan small_plan(int64_t M, int64_t N, int64_t K, int64_t ws_bytes) {
   SmallPlan best;
-  if (M % 64 || N % 64 || K % 64 || M * N > (1ll << 21) || K > (1 << 21)) return best;
+  // any number of rows (a cut last tile row costs what a whole one does, and nothing is padded or copied)
+  if (N % 64 || K % 64 || (M + 63) / 64 * 64 * N > (1ll << 21) || K > (1 << 21)) return best;
   double best_us = 0;
   static const int kTiles[3][2] = {{64, 64}, {128, 64}, {128, 128}};
   for (const auto& t : kTiles) {
     const int bm = t[0], bn = t[1];
-    if (M % bm || N % bn) continue;
-    const int64_t tiles = (M / bm) * (N / bn);
-    for (int S = 1; S <= 8; S *= 2) {
+    if (N % bn) continue;
+    const bool ragged = M % bm != 0;
+    const int64_t tiles = ((M + bm - 1) / bm) * (N / bn);
+    for (int S = 1; S <= (ragged ? 1 : 8); S *= 2) {
       const int64_t units = tiles * S, k_part = K / S;
       if (units > 512 || K % (64 * S)) break;
       if (S > 1 && (k_part < 512 || S * M * N * 4 > ws_bytes)) break;
@@ -1798,7 +1822,7 @@ static SmallPlan small_plan(int64_t M, int64_t N, int64_t K, int64_t ws_bytes) {
       }
       if (best.bm == 0 || us < best_us) {
         best_us = us;
-        best.bm = bm, best.bn = bn, best.S = S;
+        best.bm = bm, best.bn = bn, best.S = S, best.ragged = ragged;
       }
     }
   }
@@ -1986,6 +2010,18 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
   float* ws = static_cast<float*>(workspace);
   const size_t wsb = workspace_bytes > 0 ? (size_t)workspace_bytes : 0;
   if (ws && !aligned16(ws)) return fail(-MI355_E_ALIGN, "gemm_f16_nt: workspace must be 16-byte aligned");
+  if (small.ragged) {
+    const int m = (int)M, n = (int)N, k = (int)K;
+    auto tiled = [&](auto out, auto is_bf) {
+      using OutT = decltype(out);
+      constexpr bool BF = decltype(is_bf)::value;
+      if (small.bm == 64) return launch_tiled<64, 64, 2, 2, OutT, 1, BF, true>(a, b, c, m, n, k, n, s);
+      if (small.bn == 64) return launch_tiled<128, 64, 2, 2, OutT, 1, BF, true>(a, b, c, m, n, k, n, s);
+      return launch_tiled<128, 128, 2, 2, OutT, 1, BF, true>(a, b, c, m, n, k, n, s);
+    };
+    if (bf) return out_dtype == MI355_F32 ? tiled(float{}, std::true_type{}) : tiled(half_t{}, std::true_type{});
+    return out_dtype == MI355_F32 ? tiled(float{}, std::false_type{}) : tiled(half_t{}, std::false_type{});
+  }
   if (small.S > 1) {
     const half_t *ah = (const half_t*)a, *bh = (const half_t*)b;
     const int m = (int)M, n = (int)N, k = (int)K, S = small.S;

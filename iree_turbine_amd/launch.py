@@ -38,7 +38,12 @@ def _contig_out(t: Tensor, name: str) -> None:
         raise ValueError(f"{name}: output tensors must be contiguous")  # runtime/launch.py:246
 
 
-_PAD_MIN_FLOPS = 1.5e10  # below this the copies cost what the faster kernel gains (measured break-even 1-2e10)
+_PAD_MIN_FLOPS = 0.0  # the tiled kernels on padded copies beat the bounds-checked kernel at every size measured (from 2e7 flop)
+
+
+def _ragged_rows_fit(M: int, N: int, K: int) -> bool:
+    """Shapes whose ragged M the library handles itself (a cut last tile row): the small-product rule's range."""
+    return N % 64 == 0 and K % 64 == 0 and -(-M // 64) * 64 * N <= (1 << 21)
 
 
 def _skinny_fits(M: int, N: int, K: int) -> bool:
@@ -61,7 +66,8 @@ def gemm_nt_out(a: Tensor, b: Tensor, c: Tensor, variant: int = -1) -> Tensor:
     lib = _lib.load()
     entry = lib.mi355_gemm_bf16_nt if a.dtype == torch.bfloat16 else lib.mi355_gemm_f16_nt
     a_k, b_k, c_k = a, b, c
-    if variant < 0 and 2.0 * M * N * K >= _PAD_MIN_FLOPS and (M % 128 or N % 128 or K % 64) and not _skinny_fits(M, N, K):
+    if variant < 0 and 2.0 * M * N * K >= _PAD_MIN_FLOPS and (M % 128 or N % 128 or K % 64) and not _skinny_fits(M, N, K) \
+            and not _ragged_rows_fit(M, N, K):
         # Ragged sizes would go to the bounds-checked 64x64 kernel (about a fifth of the tiled kernels' rate).  Zero
         # padding changes no sum, so the ragged operands are copied into tile-aligned buffers and the result cut
         # out again: three extra passes over memory against a 4-5x faster product (3000x5000x4104: 508 -> 190 us).

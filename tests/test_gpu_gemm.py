@@ -294,6 +294,36 @@ def test_gemm_small_products(dev, shape, out32, dtype):
         assert torch.equal(got, torch.ops.mi355.gemm_nt(a, b, out_dtype, v))
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("out32", [False, True])
+@pytest.mark.parametrize("shape", [(1, 64, 64), (65, 64, 128), (127, 128, 192), (129, 1024, 1024), (200, 4096, 1024), (300, 2048, 2048),
+                                   (130, 8192, 1024), (1000, 2048, 512), (63, 1984, 4096), (1023, 1024, 64)])
+def test_gemm_ragged_rows(dev, shape, out32, dtype):
+    """Any number of rows in the small-product range (N and K multiples of 64): the last tile row is cut inside the
+    kernel -- its loads of A take row min(row, M - 1), its stores stop at M -- on 64x64, 128x64 and 128x128 tiles: one
+    row, one row more and one row fewer than a tile, one slab and many.  Whole matrix against an fp32 product, the
+    rows behind the result untouched, launches repeat bit for bit."""
+    import iree_turbine_amd as ita
+    from iree_turbine_amd import _lib
+
+    M, N, K = shape
+    announce(f"gemm ragged rows {shape} {dtype} out32={out32}")
+    assert _lib.load().mi355_gemm_nt_workspace_bytes(M, N, K) == 0  # a cut tile row takes no K split
+    g = torch.Generator().manual_seed(M + 2 * N + 3 * K)
+    a = (torch.randn(M, K, generator=g) * 0.25).to(dtype).to(dev)
+    b = (torch.randn(N, K, generator=g) * 0.25).to(dtype).to(dev)
+    odt = torch.float32 if out32 else dtype
+    full = torch.full((M + 130, N), float("nan"), dtype=odt, device=dev)
+    c = full[:M]
+    ita.launch.gemm_nt_out(a, b, c, -1)
+    tol = dict(rtol=1e-3, atol=1e-3) if out32 else dict(rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(c.float(), a.float() @ b.float().t(), **tol)
+    assert torch.isnan(full[M:]).all()  # nothing stored behind row M - 1
+    again = torch.empty_like(c)
+    ita.launch.gemm_nt_out(a, b, again, -1)
+    assert torch.equal(c, again)
+
+
 @pytest.mark.parametrize("shape", [(1088, 2112, 2048), (1152, 2112, 1024), (2112, 1152, 1024)])
 def test_gemm_multiples_of_64_beyond_the_small_rule(dev, shape):
     """Products too large for the small-product rule that divide by 64 and not by 128 (and too small for the launcher to
