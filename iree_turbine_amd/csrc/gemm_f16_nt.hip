@@ -1957,6 +1957,7 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
   };
   int split128 = 1;  // K ranges of the 128x128 split, when the automatic choice takes it
   SmallPlan small;   // tile shape and K ranges of a small product, when the automatic choice takes it
+  int cut_rows = 0;  // 1 / 2: a product beyond the small rule on 128x128 / 256x128 tiles with a cut last tile row
   if (variant < 0) {
     // Large problems take the 256x256 tile; when that leaves most of the 256 CUs idle the
     // 128x128 tile (4x the workgroups) wins; everything else goes to the bounds-checked kernel.
@@ -1982,6 +1983,16 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
     else if (s128 > 1 && workspace_bytes >= (int64_t)s128 * M * N * 4) {  // a small product: K split on 128x128 tiles
       variant = V_PIPELINED_128;
       split128 = s128;
+    }
+    // any number of rows beyond the small rule, as long as one round of workgroups covers the product: the last tile row
+    // of 128x128 tiles (up to 256 of them) or of 256x128 tiles (129 to 256) is cut inside the kernel
+    else if (al && N % 128 == 0 && K % 64 == 0 && M % 128 != 0 && ((M + 127) / 128) * (N / 128) <= 256) {
+      variant = V_PIPELINED_128;
+      cut_rows = 1;
+    } else if (al && N % 128 == 0 && K % 64 == 0 && M % 256 != 0 && K >= 256 && K < 8192 && ((M + 127) / 128) * (N / 128) > 256 &&
+               ((M + 255) / 256) * (N / 128) <= 256) {
+      variant = V_PIPELINED_256x128;
+      cut_rows = 2;
     }
     else if (K < 1024 && t256 <= 2048 && fits(V_PERSISTENT) && t256 >= 128 && full_rounds) variant = V_PERSISTENT;
     else if (t256 <= 128 && fits(V_STREAM_TAIL) && workspace && [&] {  // too few tiles for the chip, and a workspace to split K into
@@ -2010,11 +2021,13 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
   float* ws = static_cast<float*>(workspace);
   const size_t wsb = workspace_bytes > 0 ? (size_t)workspace_bytes : 0;
   if (ws && !aligned16(ws)) return fail(-MI355_E_ALIGN, "gemm_f16_nt: workspace must be 16-byte aligned");
-  if (small.ragged) {
+  if (small.ragged || cut_rows) {
     const int m = (int)M, n = (int)N, k = (int)K;
     auto tiled = [&](auto out, auto is_bf) {
       using OutT = decltype(out);
       constexpr bool BF = decltype(is_bf)::value;
+      if (cut_rows == 2) return launch_tiled<256, 128, 2, 2, OutT, 1, BF, true>(a, b, c, m, n, k, n, s);
+      if (cut_rows == 1) return launch_tiled<128, 128, 2, 2, OutT, 1, BF, true>(a, b, c, m, n, k, n, s);
       if (small.bm == 64) return launch_tiled<64, 64, 2, 2, OutT, 1, BF, true>(a, b, c, m, n, k, n, s);
       if (small.bn == 64) return launch_tiled<128, 64, 2, 2, OutT, 1, BF, true>(a, b, c, m, n, k, n, s);
       return launch_tiled<128, 128, 2, 2, OutT, 1, BF, true>(a, b, c, m, n, k, n, s);

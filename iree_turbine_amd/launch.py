@@ -42,8 +42,15 @@ _PAD_MIN_FLOPS = 0.0  # the tiled kernels on padded copies beat the bounds-check
 
 
 def _ragged_rows_fit(M: int, N: int, K: int) -> bool:
-    """Shapes whose ragged M the library handles itself (a cut last tile row): the small-product rule's range."""
-    return N % 64 == 0 and K % 64 == 0 and -(-M // 64) * 64 * N <= (1 << 21)
+    """Shapes whose ragged M the library handles itself (a cut last tile row): the small-product rule's range, and
+    beyond it what one round of 128x128 or 256x128 tiles covers."""
+    if N % 64 or K % 64:
+        return False
+    if -(-M // 64) * 64 * N <= (1 << 21):
+        return True
+    if N % 128:
+        return False
+    return -(-M // 128) * (N // 128) <= 256 or (256 <= K < 8192 and -(-M // 256) * (N // 128) <= 256)
 
 
 def _skinny_fits(M: int, N: int, K: int) -> bool:

@@ -297,11 +297,13 @@ def test_gemm_small_products(dev, shape, out32, dtype):
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("out32", [False, True])
 @pytest.mark.parametrize("shape", [(1, 64, 64), (65, 64, 128), (127, 128, 192), (129, 1024, 1024), (200, 4096, 1024), (300, 2048, 2048),
-                                   (130, 8192, 1024), (1000, 2048, 512), (63, 1984, 4096), (1023, 1024, 64)])
+                                   (130, 8192, 1024), (1000, 2048, 512), (63, 1984, 4096), (1023, 1024, 64),
+                                   (1500, 2048, 1024), (2000, 2048, 2048), (1100, 4096, 1024), (1793, 4096, 512), (1152, 4096, 1088)])
 def test_gemm_ragged_rows(dev, shape, out32, dtype):
-    """Any number of rows in the small-product range (N and K multiples of 64): the last tile row is cut inside the
-    kernel -- its loads of A take row min(row, M - 1), its stores stop at M -- on 64x64, 128x64 and 128x128 tiles: one
-    row, one row more and one row fewer than a tile, one slab and many.  Whole matrix against an fp32 product, the
+    """Any number of rows in the small-product range (N and K multiples of 64) and beyond it where one round of 128x128 or
+    256x128 tiles covers the product: the last tile row is cut inside the kernel -- its loads of A take row
+    min(row, M - 1), its stores stop at M -- on 64x64, 128x64, 128x128 and 256x128 tiles: one row, one row more and one
+    row fewer than a tile, one slab and many, 1152 rows on 256x128 tiles.  Whole matrix against an fp32 product, the
     rows behind the result untouched, launches repeat bit for bit."""
     import iree_turbine_amd as ita
     from iree_turbine_amd import _lib
