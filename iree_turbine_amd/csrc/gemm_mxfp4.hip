@@ -36,7 +36,9 @@ __device__ __forceinline__ floatx16 mfma_fp4_32x32x64(intx4 a, int sa, intx4 b, 
 // SLAB (with SCALES_LDS): the slab form of gemm_f16_nt_pipelined -- four data stages, the fragments and scale dwords
 // of a whole slab in one of two register sets, one wait per trip in front of its barrier -- for launches in which a
 // workgroup has its CU to itself: its slab time in the k-step form is its load latency.
-template <int BM, int BN, int WM, int WN, typename OutT, bool SCALES_LDS, bool SLAB = false>
+// RAGGED_M (slab form): M is any number of rows; the loads of A's codes and scales take row min(row, M - 1), the
+// epilogue stores the rows below M.
+template <int BM, int BN, int WM, int WN, typename OutT, bool SCALES_LDS, bool SLAB = false, bool RAGGED_M = false>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* __restrict__ A, const uint8_t* __restrict__ As,
                                                                 const uint8_t* __restrict__ B, const uint8_t* __restrict__ Bs,
                                                                 OutT* __restrict__ C, int M, int N, int K, int tiles_m,
@@ -62,17 +64,30 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
   // chunk c of row r lives in slot c ^ ((r >> 1) & 7): conflict-free fragment reads on 64 LDS banks
   const int lchunk = (lane & 7) ^ (((wave & 1) << 2) | (lrow >> 1));
   // wave-uniform base pointer + one 32-bit per-lane offset shared by every load of the wave
-  const uint8_t* a_src = A + (size_t)(tile_m * BM + wave * 8) * Kb;
+  const uint8_t* a_src = A + (size_t)(tile_m * BM + (RAGGED_M ? 0 : wave * 8)) * Kb;  // RAGGED_M: the tile's first row
   const uint8_t* b_src = B + (size_t)(tile_n * BN + wave * 8) * Kb;
   const unsigned lane_off = (unsigned)lrow * (unsigned)Kb + (unsigned)lchunk * 16u;
   const size_t row_step = (size_t)NW * 8 * Kb;
+  static_assert(!RAGGED_M || SLAB, "only the slab form cuts its last tile row");
+  // RAGGED_M: byte offset from the tile's first row of A (which exists) of this lane's clamped row in A load i
+  unsigned a_off[RAGGED_M ? LA : 1];
+  if constexpr (RAGGED_M) {
+#pragma unroll
+    for (int i = 0; i < LA; i++) {
+      const int row = tile_m * BM + wave * 8 + i * NW * 8 + lrow;
+      a_off[i] = (unsigned)((row < M ? row : M - 1) - tile_m * BM) * (unsigned)Kb + (unsigned)lchunk * 16u;  // from the tile's first row
+    }
+  }
 
   auto issue_loads = [&](int stage, int slab) {
     char* dst = lds + stage * STAGE + wave * 1024;
     const uint8_t* ap = a_src + slab * 128;
     const uint8_t* bp = b_src + slab * 128;
 #pragma unroll
-    for (int i = 0; i < LA; i++) load_lds_16B(ap + i * row_step + lane_off, dst + i * NW * 1024);
+    for (int i = 0; i < LA; i++) {
+      if constexpr (RAGGED_M) load_lds_16B(ap + a_off[i], dst + i * NW * 1024);
+      else load_lds_16B(ap + i * row_step + lane_off, dst + i * NW * 1024);
+    }
 #pragma unroll
     for (int i = 0; i < LB; i++) load_lds_16B(bp + i * row_step + lane_off, dst + A_BYTES + i * NW * 1024);
   };
@@ -101,6 +116,10 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
     for (int i = 0; i < LS; i++) {
       const int r0 = (wave * LS + i) * 32;  // first of 32 consecutive rows (all in A or all in B: BM % 32 == 0)
       const uint8_t* src = r0 < BM ? As + (size_t)(tile_m * BM + r0) * Ksc : Bs + (size_t)(tile_n * BN + r0 - BM) * Ksc;
+      if constexpr (RAGGED_M) {
+        const int row = tile_m * BM + r0 + (lane >> 1);
+        if (r0 < BM) src = As + (size_t)(row < M ? row : M - 1) * Ksc - (size_t)(lane >> 1) * Ksc;  // this lane's row, clamped
+      }
       load_lds_16B(src + group * 32 + sc_lane_off, dst + r0 * 32);
     }
   };
@@ -195,11 +214,17 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
       const uint8_t* bp = b_src + lslab * 128;
       const int g = (kt >> 2) + 1 < KG ? (kt >> 2) + 1 : KG - 1;
       auto load_at = [&](int l) __attribute__((always_inline)) {
-        if (l < LA) load_lds_16B(ap + l * row_step + lane_off, dst + l * NW * 1024);
-        else if (l < NL) load_lds_16B(bp + (l - LA) * row_step + lane_off, dst + A_BYTES + (l - LA) * NW * 1024);
+        if (l < LA) {
+          if constexpr (RAGGED_M) load_lds_16B(ap + a_off[l], dst + l * NW * 1024);
+          else load_lds_16B(ap + l * row_step + lane_off, dst + l * NW * 1024);
+        } else if (l < NL) load_lds_16B(bp + (l - LA) * row_step + lane_off, dst + A_BYTES + (l - LA) * NW * 1024);
         else {
           const int r0 = (wave * LS + (l - NL)) * 32;
           const uint8_t* src = r0 < BM ? As + (size_t)(tile_m * BM + r0) * Ksc : Bs + (size_t)(tile_n * BN + r0 - BM) * Ksc;
+          if constexpr (RAGGED_M) {
+            const int row = tile_m * BM + r0 + (lane >> 1);
+            if (r0 < BM) src = As + (size_t)(row < M ? row : M - 1) * Ksc - (size_t)(lane >> 1) * Ksc;  // this lane's row, clamped
+          }
           load_lds_16B(src + g * 32 + sc_lane_off, sc_lds + (g & 1) * SC_BUF + r0 * 32);
         }
       };
@@ -368,7 +393,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
     for (int it = 0; it < WTM / ROWS_PER_IT; it++) {
       const int row = it * ROWS_PER_IT + er;
       intx4 v = *reinterpret_cast<const intx4*>(ep + row * ROW_B + ((ec ^ ((row >> 1) & (CH - 1))) * 16));
-      *reinterpret_cast<intx4*>(cbase + (size_t)row * N) = v;
+      if (!RAGGED_M || tile_m * BM + wm * WTM + row < M) *reinterpret_cast<intx4*>(cbase + (size_t)row * N) = v;
     }
   } else {
     const int m0 = tile_m * BM + wm * WTM + r32;
@@ -376,6 +401,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_mxfp4_tiled(const uint8_t* _
 #pragma unroll
     for (int j = 0; j < TM; j++) {
       OutT* crow = C + (size_t)(m0 + j * 32) * N + n0;
+      if (RAGGED_M && m0 + j * 32 >= M) continue;
 #pragma unroll
       for (int i = 0; i < TN; i++)
 #pragma unroll
@@ -1611,15 +1637,15 @@ constexpr int kNumMxVariants = sizeof(kMxVariants) / sizeof(kMxVariants[0]);
 int mxfp4_variant_count() { return kNumMxVariants; }
 const char* mxfp4_variant_name(int i) { return (i >= 0 && i < kNumMxVariants) ? kMxVariants[i].name : nullptr; }
 
-template <int BM, int BN, int WM, int WN, typename OutT, bool SCALES_LDS, bool SLAB = false>
+template <int BM, int BN, int WM, int WN, typename OutT, bool SCALES_LDS, bool SLAB = false, bool RAGGED = false>
 static int launch_mx_tiled(const void* a, const void* as, const void* b, const void* bs, void* c, int M, int N, int K,
                            hipStream_t stream) {
-  auto kern = gemm_mxfp4_tiled<BM, BN, WM, WN, OutT, SCALES_LDS, SLAB>;
+  auto kern = gemm_mxfp4_tiled<BM, BN, WM, WN, OutT, SCALES_LDS, SLAB, RAGGED>;
   constexpr int lds_bytes = (SLAB ? 4 : 2) * (BM + BN) * 128 + (SCALES_LDS ? 2 * (BM + BN) * 32 : 0);
   static_assert(lds_bytes <= 160 * 1024, "the stages and the scale buffers fit in LDS");
   static std::atomic<uint64_t> lds_ok{0};
   if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_mxfp4_tiled")) return rc;
-  const int tiles_m = M / BM, tiles_n = N / BN;
+  const int tiles_m = RAGGED ? (M + BM - 1) / BM : M / BM, tiles_n = N / BN;
   dim3 grid(tiles_m * tiles_n), block(WM * WN * 64);
   hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, (const uint8_t*)a, (const uint8_t*)as, (const uint8_t*)b,
                      (const uint8_t*)bs, (OutT*)c, M, N, K, tiles_m, tiles_n, 4);
@@ -1753,6 +1779,7 @@ extern "C" int mi355_mxfp4_gemm(const void* a, const void* a_scale, const void* 
     if ((v == 5 || v == 6) && !(sc_al16 && K % 512 == 0 && K >= 1024 && M * (K / 2) < (1ll << 32) && N * (K / 2) < (1ll << 32))) return false;
     return sc_al && M % kMxVariants[v].bm == 0 && N % kMxVariants[v].bn == 0 && K % 256 == 0;
   };
+  bool cut_rows = false;  // the automatic choice took the 64x64 tile for a ragged M
   if (variant < 0) {
     // M <= 32 is weight streaming and has its own kernel.  The 256x256 tile halves the L2 -> LDS bytes per
     // flop; it is used when there are enough tiles to fill the 256 CUs and the last round of workgroups
@@ -1769,6 +1796,12 @@ extern "C" int mi355_mxfp4_gemm(const void* a, const void* a_scale, const void* 
     // whatever its tile), so up to 320 tiles of 64x64 take those (128x8192x8192: 16.7 us on 128x128 tiles, 10.8 on
     // 64x64; 1024x1024x8192 15.3 -> 10.0; 256x8192x8192, 512 tiles of 64x64: 17.6 against 18.7).
     else if (fits(7) && ((M / 64) * (N / 64) <= 320 || !fits(2))) variant = 7;  // also what divides by 64 and not by 128
+    // any number of rows against N % 64 == 0 and K % 1024 == 0 (activations against weights): the 64x64 tile with its
+    // last tile row cut, instead of the bounds-checked kernel (100 x 8192 x 8192: 61 -> 12 us)
+    else if (M % 64 != 0 && sc_al && N % 64 == 0 && K % 1024 == 0) {
+      variant = 7;
+      cut_rows = true;
+    }
     else if (fits(2)) variant = 2;
     else variant = kNumMxVariants - 1;
   } else if (!fits(variant)) {
@@ -1776,6 +1809,10 @@ extern "C" int mi355_mxfp4_gemm(const void* a, const void* a_scale, const void* 
                 kMxVariants[variant].name, (long long)M, (long long)N, (long long)K, kMxVariants[variant].bm, kMxVariants[variant].bn);
   }
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (cut_rows) {
+    if (out_dtype == MI355_F32) return launch_mx_tiled<64, 64, 2, 2, float, true, true, true>(a, a_scale, b, b_scale, c, (int)M, (int)N, (int)K, s);
+    return launch_mx_tiled<64, 64, 2, 2, unsigned short, true, true, true>(a, a_scale, b, b_scale, c, (int)M, (int)N, (int)K, s);
+  }
   if (out_dtype == MI355_F32) return launch_mx<float>(variant, a, a_scale, b, b_scale, c, (int)M, (int)N, (int)K, s);
   return launch_mx<unsigned short>(variant, a, a_scale, b, b_scale, c, (int)M, (int)N, (int)K, s);
 }

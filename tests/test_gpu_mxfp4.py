@@ -210,6 +210,37 @@ def test_mxfp4_slab_form(dev, shape, out_dtype):
         assert torch.equal(got, torch.ops.mi355.mxfp4_gemm(a, asc, b, bsc, out_dtype, v)), v
 
 
+@pytest.mark.parametrize("shape", [(33, 64, 1024), (65, 128, 2048), (100, 8192, 1024), (127, 64, 3072), (200, 2048, 4096), (1000, 1024, 1024),
+                                   (129, 4160, 1024)])
+@pytest.mark.parametrize("out_dtype", ["bfloat16", "float32"])
+def test_mxfp4_ragged_rows(dev, shape, out_dtype):
+    """Any number of rows beyond the weight-streaming kernel's 32 against N % 64 == 0 and K % 1024 == 0: the 64x64 tile
+    with its last tile row cut (codes and scales of A read from row min(row, M - 1), stores stop at M) -- whole matrix
+    against the bounds-checked kernel, the rows behind the result untouched, launches repeat bit for bit."""
+    import iree_turbine_amd as ita
+    from oracle import inputs
+
+    M, N, K = shape
+    announce(f"mxfp4 ragged rows {shape} {out_dtype}")
+    names = ita._lib.variants("mxfp4_gemm")
+    a, asc, b, bsc = [t.to(dev) for t in inputs.mxfp4_inputs(M, N, K, seed=M + N + K)]
+    ref = torch.ops.mi355.mxfp4_gemm(a, asc, b, bsc, out_dtype, len(names) - 1)
+    odt = getattr(torch, out_dtype)
+    full = torch.full((M + 70, N), float("nan"), dtype=odt, device=dev)
+    got = full[:M]
+    ita.launch.mxfp4_gemm_out(a, asc, b, bsc, got, -1)
+    if out_dtype == "float32":
+        assert _rel_err(got, ref) < 1e-5
+    else:
+        g32, r32 = got.float(), ref.float()
+        assert _rel_err(g32, r32) < 1e-3
+        assert ((g32 - r32).abs() <= r32.abs() * 2 ** -7 + 1e-5 * r32.abs().max()).all()
+    assert torch.isnan(full[M:]).all()
+    again = torch.empty_like(got)
+    ita.launch.mxfp4_gemm_out(a, asc, b, bsc, again, -1)
+    assert torch.equal(got, again)
+
+
 @pytest.mark.parametrize("shape", [(4352, 4352, 1024), (4096, 4608, 1536), (512, 256, 8192)])
 @pytest.mark.parametrize("out_dtype", ["bfloat16", "float32"])
 def test_mxfp4_persistent_tile_walk(dev, shape, out_dtype):
