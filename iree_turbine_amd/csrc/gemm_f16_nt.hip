@@ -2,9 +2,11 @@
 //
 // Kernels in this file, all on the same LDS row format: gemm_f16_nt_stream (the current kernel for large shapes: whole-row
 // direct-to-LDS loads two slabs ahead, 16x16x32 MFMAs, a tile walk), gemm_f16_nt_persistent (8 waves, chosen for short
-// K), gemm_f16_nt_pipelined (128x128 tiles: few tiles, and the strip a sparse last round is cut into),
-// gemm_f16_nt_staged (the register-staged predecessor of the streamed kernel, kept as the independent comparator of
-// the bit-identity tests), gemm_f16_nt_skinny (M <= 64: weight streaming) and a bounds-checked kernel for any shape.
+// K), gemm_f16_nt_pipelined (64x64, 128x64, 128x128 and 256x128 tiles: products of up to one round of tiles, any number
+// of rows, with or without a K split, and the strip a sparse last round is cut into), gemm_f16_nt_staged (the
+// register-staged predecessor of the streamed kernel, kept as the independent comparator of the bit-identity tests),
+// gemm_f16_nt_skinny and gemm_f16_nt_skinny_rb (M <= 32 and M <= 128: weight streaming) and a bounds-checked kernel for
+// any shape.
 //
 // LDS row format: K is walked in slabs of 64 halfs; a slab row is 128 bytes = 8 chunks of 16 bytes; both operands are
 // K-contiguous, so the same row format serves A and B.  Slabs are copied global -> LDS with direct-to-LDS loads (no VGPR
