@@ -1935,6 +1935,17 @@ static int launch_variant(int variant, const void* a, const void* b, void* c, in
 
 using namespace mi355;
 
+// Many rows that are no multiple of the 256-row tile (and more than one round of smaller tiles covers): the automatic
+// choice runs the multiple of 256 and the remainder as two products on row ranges of A and C.  Against padded copies
+// of A and of the result: 4100x4096x4096 162 -> 110 us, 9000x8192x2048 321 -> 243, 5000x8192x8192 598 -> 517.
+static bool splits_rows(int64_t M, int64_t N, int64_t K) {
+  if (M < 512 || M % 256 == 0 || N % 128 || K % 64) return false;
+  if ((M + 63) / 64 * 64 * N <= (1ll << 21)) return false;                                    // the small-product rule
+  if ((M + 127) / 128 * (N / 128) <= 256) return false;                                       // one round of 128x128 tiles
+  if (K >= 256 && K < 8192 && (M + 255) / 256 * (N / 128) <= 256) return false;               // one round of 256x128 tiles
+  return true;
+}
+
 // fp16 and bf16 share everything but the kernel instantiation; `bf` also names the 16-bit output format
 static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t M, int64_t N, int64_t K, int out_dtype, int variant,
                          void* stream, void* workspace = nullptr, int64_t workspace_bytes = 0) {
@@ -1957,6 +1968,13 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
     if (v == V_SKINNY) return al && M <= 128 && N % 32 == 0 && K % 64 == 0;  // a tile is 32 rows of B; 64-half K segments
     return al && M % kGemmVariants[v].bm == 0 && N % kGemmVariants[v].bn == 0 && K % 64 == 0;
   };
+  if (variant < 0 && al && splits_rows(M, N, K)) {
+    const int64_t m0 = M / 256 * 256;
+    const size_t out_bytes = out_dtype == MI355_F32 ? 4 : 2;
+    if (int rc = gemm_nt_entry(bf, a, b, c, m0, N, K, out_dtype, -1, stream, workspace, workspace_bytes)) return rc;
+    return gemm_nt_entry(bf, static_cast<const char*>(a) + (size_t)m0 * K * 2, b, static_cast<char*>(c) + (size_t)m0 * N * out_bytes,
+                         M - m0, N, K, out_dtype, -1, stream, workspace, workspace_bytes);
+  }
   int split128 = 1;  // K ranges of the 128x128 split, when the automatic choice takes it
   SmallPlan small;   // tile shape and K ranges of a small product, when the automatic choice takes it
   int cut_rows = 0;  // 1 / 2: a product beyond the small rule on 128x128 / 256x128 tiles with a cut last tile row
@@ -2070,6 +2088,10 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
 
 // Bytes of workspace with which the automatic choice would split K for this shape (0: it would not).
 static int64_t gemm_nt_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (M > 0 && N > 0 && K > 0 && splits_rows(M, N, K)) {  // two products, one after the other, on one workspace
+    const int64_t main = gemm_nt_workspace_bytes(M / 256 * 256, N, K), rest = gemm_nt_workspace_bytes(M % 256, N, K);
+    return main > rest ? main : rest;
+  }
   if (M <= 0 || N <= 0 || K <= 0 || M > (1 << 30) || N > (1 << 30) || K > (1 << 21) || K < 256 || K % 128 != 0) return 0;
   if (M * K * 2 >= (1ll << 32) || N * K * 2 >= (1ll << 32)) return 0;  // the streamed kernel's one descriptor per operand
   if (M <= 64 && N % 32 == 0 && N >= 2048 && K >= 512) return 0;        // the weight-streaming kernel's shapes

@@ -42,15 +42,17 @@ _PAD_MIN_FLOPS = 0.0  # the tiled kernels on padded copies beat the bounds-check
 
 
 def _ragged_rows_fit(M: int, N: int, K: int) -> bool:
-    """Shapes whose ragged M the library handles itself (a cut last tile row): the small-product rule's range, and
-    beyond it what one round of 128x128 or 256x128 tiles covers."""
+    """Shapes whose ragged M the library handles itself: a cut last tile row in the small-product rule's range and
+    where one round of 128x128 or 256x128 tiles covers the product, two products on row ranges beyond that."""
     if N % 64 or K % 64:
         return False
     if -(-M // 64) * 64 * N <= (1 << 21):
         return True
     if N % 128:
         return False
-    return -(-M // 128) * (N // 128) <= 256 or (256 <= K < 8192 and -(-M // 256) * (N // 128) <= 256)
+    if -(-M // 128) * (N // 128) <= 256 or (256 <= K < 8192 and -(-M // 256) * (N // 128) <= 256):
+        return True
+    return M >= 512  # many rows: the library runs the multiple of 256 and the remainder as two products
 
 
 def _skinny_fits(M: int, N: int, K: int) -> bool:
@@ -70,15 +72,6 @@ def gemm_nt_out(a: Tensor, b: Tensor, c: Tensor, variant: int = -1) -> Tensor:
         raise ValueError(f"gemm_nt: c is {tuple(c.shape)}, expected {(M, N)}")
     if c.dtype not in (torch.float32, a.dtype):
         raise ValueError(f"gemm_nt: c must be float32 or {a.dtype}, got {c.dtype}")
-    if variant < 0 and M >= 512 and M % 256 and N % 128 == 0 and K % 64 == 0 and not _ragged_rows_fit(M, N, K):
-        # Many rows that are no multiple of the 256-row tile: the multiple of 256 through the kernels for large shapes,
-        # the rest (fewer than 256 rows: a cut tile row, or the weight-streaming kernels) in a launch of its own, both on
-        # row ranges of the caller's tensors.  Against padded copies of A and of the result: 4100x4096x4096 162 -> 110
-        # us, 9000x8192x2048 321 -> 243, 5000x8192x8192 598 -> 517.
-        m0 = (M // 256) * 256
-        gemm_nt_out(a[:m0], b, c[:m0], variant)
-        gemm_nt_out(a[m0:], b, c[m0:], variant)
-        return c
     lib = _lib.load()
     entry = lib.mi355_gemm_bf16_nt if a.dtype == torch.bfloat16 else lib.mi355_gemm_f16_nt
     a_k, b_k, c_k = a, b, c

@@ -71,6 +71,7 @@ def test_gemm_workspace_plan_without_a_gpu():
     assert need(2048, 10240, 8192) == 4 * 2048 * 2048 * 4  # the strip of 64 tiles behind a full round
     assert need(8192, 8192, 8192) == 0 and need(4096, 4096, 4096) == 0
     assert need(200, 4096, 4096) == 0 and need(65, 64, 8192) == 0  # a cut last tile row takes no split
+    assert need(2100, 10240, 8192) == need(2048, 10240, 8192)  # 2048 rows and 52 rows, one after the other
     assert need(0, 128, 128) == 0 and need(128, 128, -64) == 0 and need(128, 128, 1 << 22) == 0
 
 
