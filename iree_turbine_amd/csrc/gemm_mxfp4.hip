@@ -1779,6 +1779,15 @@ extern "C" int mi355_mxfp4_gemm(const void* a, const void* a_scale, const void* 
     if ((v == 5 || v == 6) && !(sc_al16 && K % 512 == 0 && K >= 1024 && M * (K / 2) < (1ll << 32) && N * (K / 2) < (1ll << 32))) return false;
     return sc_al && M % kMxVariants[v].bm == 0 && N % kMxVariants[v].bn == 0 && K % 256 == 0;
   };
+  // Many rows that are no multiple of the 256-row tile against weights the large kernels take: the multiple of 256 and
+  // the remainder (the 64x64 tile with a cut last row, or the weight-streaming kernel) as two products on row ranges.
+  if (variant < 0 && M >= 512 && M % 256 != 0 && N % 256 == 0 && K % 1024 == 0 && sc_al16) {
+    const int64_t m0 = M / 256 * 256;
+    const size_t out_bytes = out_dtype == MI355_F32 ? 4 : 2;
+    if (int rc = mi355_mxfp4_gemm(a, a_scale, b, b_scale, c, m0, N, K, out_dtype, -1, stream)) return rc;
+    return mi355_mxfp4_gemm(static_cast<const char*>(a) + (size_t)m0 * (K / 2), static_cast<const char*>(a_scale) + (size_t)m0 * (K / 32), b,
+                            b_scale, static_cast<char*>(c) + (size_t)m0 * N * out_bytes, M - m0, N, K, out_dtype, -1, stream);
+  }
   bool cut_rows = false;  // the automatic choice took the 64x64 tile for a ragged M
   if (variant < 0) {
     // M <= 32 is weight streaming and has its own kernel.  The 256x256 tile halves the L2 -> LDS bytes per

@@ -211,11 +211,12 @@ def test_mxfp4_slab_form(dev, shape, out_dtype):
 
 
 @pytest.mark.parametrize("shape", [(33, 64, 1024), (65, 128, 2048), (100, 8192, 1024), (127, 64, 3072), (200, 2048, 4096), (1000, 1024, 1024),
-                                   (129, 4160, 1024)])
+                                   (129, 4160, 1024), (2100, 4096, 1024), (4100, 2048, 2048), (540, 8192, 1024)])
 @pytest.mark.parametrize("out_dtype", ["bfloat16", "float32"])
 def test_mxfp4_ragged_rows(dev, shape, out_dtype):
     """Any number of rows beyond the weight-streaming kernel's 32 against N % 64 == 0 and K % 1024 == 0: the 64x64 tile
-    with its last tile row cut (codes and scales of A read from row min(row, M - 1), stores stop at M) -- whole matrix
+    with its last tile row cut (codes and scales of A read from row min(row, M - 1), stores stop at M), and from 512
+    rows the multiple of 256 and the remainder as two products (2048 + 52, 4096 + 4, 512 + 28 rows) -- whole matrix
     against the bounds-checked kernel, the rows behind the result untouched, launches repeat bit for bit."""
     import iree_turbine_amd as ita
     from oracle import inputs
