@@ -1938,12 +1938,17 @@ using namespace mi355;
 // Many rows that are no multiple of the 256-row tile (and more than one round of smaller tiles covers): the automatic
 // choice runs the multiple of 256 and the remainder as two products on row ranges of A and C.  Against padded copies
 // of A and of the result: 4100x4096x4096 162 -> 110 us, 9000x8192x2048 321 -> 243, 5000x8192x8192 598 -> 517.
+// whether a product of M rows (any number) against N % 128 == 0, K % 64 == 0 is one the tiled or weight-streaming kernels
+// take whole: the small-product rule, one round of 128x128 or of 256x128 tiles, or up to 128 rows of a decode shape
+static bool one_round_of_rows(int64_t M, int64_t N, int64_t K) {
+  if ((M + 63) / 64 * 64 * N <= (1ll << 21)) return true;
+  if ((M + 127) / 128 * (N / 128) <= 256) return true;
+  if (K >= 256 && K < 8192 && (M + 255) / 256 * (N / 128) <= 256) return true;
+  return M <= 128 && N >= 2048 && K >= 512;
+}
 static bool splits_rows(int64_t M, int64_t N, int64_t K) {
   if (M < 512 || M % 256 == 0 || N % 128 || K % 64) return false;
-  if ((M + 63) / 64 * 64 * N <= (1ll << 21)) return false;                                    // the small-product rule
-  if ((M + 127) / 128 * (N / 128) <= 256) return false;                                       // one round of 128x128 tiles
-  if (K >= 256 && K < 8192 && (M + 255) / 256 * (N / 128) <= 256) return false;               // one round of 256x128 tiles
-  return true;
+  return !one_round_of_rows(M, N, K) && one_round_of_rows(M % 256, N, K);  // the remainder must have a fast kernel
 }
 
 // fp16 and bf16 share everything but the kernel instantiation; `bf` also names the 16-bit output format

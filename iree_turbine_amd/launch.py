@@ -41,6 +41,16 @@ def _contig_out(t: Tensor, name: str) -> None:
 _PAD_MIN_FLOPS = 0.0  # the tiled kernels on padded copies beat the bounds-checked kernel at every size measured (from 2e7 flop)
 
 
+def _one_round_of_rows(M: int, N: int, K: int) -> bool:
+    """A product of any M rows against N % 128 == 0, K % 64 == 0 that the library's tiled or weight-streaming kernels
+    take whole (the library's rule of the same name)."""
+    if -(-M // 64) * 64 * N <= (1 << 21) or -(-M // 128) * (N // 128) <= 256:
+        return True
+    if 256 <= K < 8192 and -(-M // 256) * (N // 128) <= 256:
+        return True
+    return M <= 128 and N >= 2048 and K >= 512
+
+
 def _ragged_rows_fit(M: int, N: int, K: int) -> bool:
     """Shapes whose ragged M the library handles itself: a cut last tile row in the small-product rule's range and
     where one round of 128x128 or 256x128 tiles covers the product, two products on row ranges beyond that."""
@@ -50,9 +60,7 @@ def _ragged_rows_fit(M: int, N: int, K: int) -> bool:
         return True
     if N % 128:
         return False
-    if -(-M // 128) * (N // 128) <= 256 or (256 <= K < 8192 and -(-M // 256) * (N // 128) <= 256):
-        return True
-    return M >= 512  # many rows: the library runs the multiple of 256 and the remainder as two products
+    return _one_round_of_rows(M, N, K) or (M >= 512 and M % 256 != 0 and _one_round_of_rows(M % 256, N, K))
 
 
 def _skinny_fits(M: int, N: int, K: int) -> bool:
