@@ -478,6 +478,8 @@ WORKLOADS = {
     "gemm_16x8192x8192": wl_gemm(16, 8192, 8192),
     "gemm_1024x8192x8192": wl_gemm(1024, 8192, 8192),  # 128 tiles: K split in two through the workspace entry point
     "gemm_512x8192x8192": wl_gemm(512, 8192, 8192),    # 64 tiles: four K ranges
+    "gemm_64x8192x8192": wl_gemm(64, 8192, 8192),      # weight streaming with two row blocks
+    "gemm_200x4096x4096": wl_gemm(200, 4096, 4096),    # a ragged number of rows: the last tile row cut inside the kernel
     "fa_causal": wl_attention(True),
     "fa_noncausal": wl_attention(False),
     "decode": wl_decode(),
