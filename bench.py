@@ -55,6 +55,8 @@ MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
     "gemm_1024_f32out": 1.681e7,
     "gemm_bf16_8192": 1.754e9,
     "gemm_16x8192x8192": 1.366e8,
+    "gemm_64x8192x8192": 1.439e8,
+    "gemm_200x4096x4096": 4.980e7,
     "gemm_1024x8192x8192": 3.644e8,
     "fa_causal": 3.537e8,
     "fa_noncausal": 2.686e8,
