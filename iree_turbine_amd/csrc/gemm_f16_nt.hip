@@ -64,8 +64,10 @@ template <bool BF> struct OutPack<half_t, BF> {
 //    A lone workgroup's slab time in the k-step form is its load latency plus, on small tiles, the chain of LDS read
 //    latencies of four k-steps with one or two MFMAs each to cover them: 64x64 0.22 -> 0.15 us per slab, 128x128
 //    0.60 -> 0.42 (what LDS bandwidth allows); 1024^3 on 64x64 tiles 6.7 -> 5.4 us, 1024x1024x4096 19.4 -> 15.9 us.
-//  * RAGGED_M: M is any number of rows (the last tile row is cut): its loads of A take row min(row, M - 1), so they
-//    stay inside A, and the epilogue stores the rows below M only.
+//  * RAGGED_M: M is any number of rows and N any multiple of 8 columns (the last tile row and the last tile column are
+//    cut): the loads of A take row min(row, M - 1) and those of B row min(row, N - 1), so they stay inside the operands,
+//    and the epilogue stores the rows below M and the 16-byte chunks left of column N only.  N is then both the row
+//    pitch of C and its number of columns.
 template <int BM, int BN, int WM, int WN, typename OutT, bool BF, bool SLAB = false, bool RAGGED_M = false>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_t* __restrict__ A,
                                                                      const half_t* __restrict__ B,
@@ -107,7 +109,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
       k_at += (size_t)ksplit_halfs;
     }
   const half_t* a_src = A + (size_t)(a_tile * BM + (RAGGED_M ? 0 : wave * 8)) * ldk + k_at;
-  const half_t* b_src = B + (size_t)(tile_n * BN + wave * 8) * ldk + k_at;
+  const half_t* b_src = B + (size_t)(tile_n * BN + (RAGGED_M ? 0 : wave * 8)) * ldk + k_at;
   const unsigned lane_off = (unsigned)lrow * (unsigned)ldk + (unsigned)lchunk * 8u;
   const size_t row_step = (size_t)NW * 8 * ldk;
   // RAGGED_M: the offset (in halfs, from the tile's first row) of this lane's row in A load i, the row clamped to M - 1
@@ -119,9 +121,21 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
       a_off[i] = (unsigned)((row < M ? row : M - 1) - a_tile * BM) * (unsigned)ldk + (unsigned)lchunk * 8u;
     }
   }
+  unsigned b_off[RAGGED_M ? LB : 1];  // the same for the rows of B, clamped to N - 1
+  if constexpr (RAGGED_M) {
+#pragma unroll
+    for (int i = 0; i < LB; i++) {
+      const int row = tile_n * BN + wave * 8 + i * NW * 8 + lrow;
+      b_off[i] = (unsigned)((row < N ? row : N - 1) - tile_n * BN) * (unsigned)ldk + (unsigned)lchunk * 8u;
+    }
+  }
   auto load_a = [&](const half_t* ap, int i, char* dst) {  // ap: a_src at the slab
     if constexpr (RAGGED_M) load_lds_16B(ap + a_off[i], dst);
     else load_lds_16B(ap + i * row_step + lane_off, dst);
+  };
+  auto load_b = [&](const half_t* bp, int i, char* dst) {
+    if constexpr (RAGGED_M) load_lds_16B(bp + b_off[i], dst);
+    else load_lds_16B(bp + i * row_step + lane_off, dst);
   };
 
   // krot_step != 0 (a few rows of A against many rows of B, which then stream from memory): the workgroups of tile
@@ -143,7 +157,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
 #pragma unroll
     for (int i = 0; i < LA; i++) load_a(ap, i, dst + i * NW * 1024);
 #pragma unroll
-    for (int i = 0; i < LB; i++) load_lds_16B(bp + i * row_step + lane_off, dst + A_BYTES + i * NW * 1024);
+    for (int i = 0; i < LB; i++) load_b(bp, i, dst + A_BYTES + i * NW * 1024);
   };
 
   const int r32 = lane & 31, h = lane >> 5;
@@ -210,7 +224,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
 #pragma unroll
           for (int l = m * NL / NM; l < (m + 1) * NL / NM; l++) {
             if (l < LA) load_a(ap, l, dst + l * NW * 1024);
-            else load_lds_16B(bp + (l - LA) * row_step + lane_off, dst + A_BYTES + (l - LA) * NW * 1024);
+            else load_b(bp, l - LA, dst + A_BYTES + (l - LA) * NW * 1024);
           }
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -343,7 +357,8 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
     for (int it = 0; it < WTM / ROWS_PER_IT; it++) {
       const int row = it * ROWS_PER_IT + er;
       half8 v = *reinterpret_cast<const half8*>(ep + row * ROW_B + ((ec ^ ((row >> 1) & (CH - 1))) * 16));
-      if (!RAGGED_M || tile_m * BM + wm * WTM + row < M) *reinterpret_cast<half8*>(cbase + (size_t)row * N) = v;
+      if (!RAGGED_M || (tile_m * BM + wm * WTM + row < M && tile_n * BN + wn * WTN + ec * 8 < N))
+        *reinterpret_cast<half8*>(cbase + (size_t)row * N) = v;
     }
   } else {
     // fp32 epilogue, the same way (a lane's four consecutive n are one 16-byte chunk; chunk slot c ^ (m & (CH - 1))):
@@ -370,7 +385,8 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
     for (int it = 0; it < WTM / ROWS_PER_IT; it++) {
       const int row = it * ROWS_PER_IT + er;
       floatx4 v = *reinterpret_cast<const floatx4*>(ep + row * ROW_B + ((ec ^ (row & (CH - 1))) * 16));
-      if (!RAGGED_M || tile_m * BM + wm * WTM + row < M) *reinterpret_cast<floatx4*>(cbase + (size_t)row * N) = v;
+      if (!RAGGED_M || (tile_m * BM + wm * WTM + row < M && tile_n * BN + wn * WTN + ec * 4 < N))
+        *reinterpret_cast<floatx4*>(cbase + (size_t)row * N) = v;
     }
   }
 }
@@ -1613,14 +1629,16 @@ static bool pipelined_slab_form(long long tiles, int bm_plus_bn) { return bm_plu
 // (it stays in the L2s in any order), B at least 16 MiB (it streams).
 static int pipelined_krot(long long M, long long N, long long K) { return M * K * 2 <= (4 << 20) && N * K * 2 >= (16 << 20); }
 
-// RAGGED: M is any number of rows (the pipelined kernel's slab form only: the caller has checked pipelined_slab_form)
+// RAGGED: M is any number of rows and N any multiple of 8 (the pipelined kernel's slab form only: the caller has
+// checked pipelined_slab_form); C is then N columns wide (ldc == N)
 template <int BM, int BN, int WM, int WN, typename OutT, int KIND, bool BF, bool RAGGED = false>  // KIND: 1 pipelined, 2 register-staged
 static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int K, int ldc, hipStream_t stream) {
   // the kernels use their N argument only as the row stride of C, so a column range of a wider C is the
   // same launch with ldc in its place
   static_assert(KIND == 1 || KIND == 2, "pipelined or register-staged");
   static_assert(!RAGGED || KIND == 1, "only the pipelined kernel cuts its last tile row");
-  const int tiles_m = RAGGED ? (M + BM - 1) / BM : M / BM, tiles_n = N / BN;
+  const int tiles_m = RAGGED ? (M + BM - 1) / BM : M / BM, tiles_n = RAGGED ? (N + BN - 1) / BN : N / BN;
+  if (RAGGED && (ldc != N || N % 8)) return fail(-MI355_E_SHAPE, "gemm_f16_nt: a cut tile column needs N %% 8 == 0 and a C of N columns");
   int group_m = 4;
   dim3 grid(tiles_m * tiles_n), block(WM * WN * 64);
   if constexpr (KIND == 2) {
@@ -1796,19 +1814,19 @@ static bool takes_256x128(int64_t M, int64_t N, int64_t K) {
 
 struct SmallPlan {
   int bm = 0, bn = 0, S = 1;  // bm == 0: not a small product
-  bool ragged = false;        // M is no multiple of bm: the last tile row is cut, and K is not split
+  bool ragged = false;        // M is no multiple of bm or N none of bn: the last tile row or column is cut, and K is not split
 };
 static SmallPlan small_plan(int64_t M, int64_t N, int64_t K, int64_t ws_bytes) {
   SmallPlan best;
-  // any number of rows (a cut last tile row costs what a whole one does, and nothing is padded or copied)
-  if (N % 64 || K % 64 || (M + 63) / 64 * 64 * N > (1ll << 21) || K > (1 << 21)) return best;
+  // any number of rows, any multiple of 8 columns (a cut last tile row or column costs what a whole one does, and
+  // nothing is padded or copied)
+  if (N % 8 || K % 64 || ((M + 63) / 64 * 64) * ((N + 63) / 64 * 64) > (1ll << 21) || K > (1 << 21)) return best;
   double best_us = 0;
   static const int kTiles[3][2] = {{64, 64}, {128, 64}, {128, 128}};
   for (const auto& t : kTiles) {
     const int bm = t[0], bn = t[1];
-    if (N % bn) continue;
-    const bool ragged = M % bm != 0;
-    const int64_t tiles = ((M + bm - 1) / bm) * (N / bn);
+    const bool ragged = M % bm != 0 || N % bn != 0;
+    const int64_t tiles = ((M + bm - 1) / bm) * ((N + bn - 1) / bn);
     for (int S = 1; S <= (ragged ? 1 : 8); S *= 2) {
       const int64_t units = tiles * S, k_part = K / S;
       if (units > 512 || K % (64 * S)) break;
@@ -1938,13 +1956,13 @@ using namespace mi355;
 // Many rows that are no multiple of the 256-row tile (and more than one round of smaller tiles covers): the automatic
 // choice runs the multiple of 256 and the remainder as two products on row ranges of A and C.  Against padded copies
 // of A and of the result: 4100x4096x4096 162 -> 110 us, 9000x8192x2048 321 -> 243, 5000x8192x8192 598 -> 517.
-// whether a product of M rows (any number) against N % 128 == 0, K % 64 == 0 is one the tiled or weight-streaming kernels
+// whether a product of M rows (any number) against N % 8 == 0, K % 64 == 0 is one the tiled or weight-streaming kernels
 // take whole: the small-product rule, one round of 128x128 or of 256x128 tiles, or up to 128 rows of a decode shape
 static bool one_round_of_rows(int64_t M, int64_t N, int64_t K) {
-  if ((M + 63) / 64 * 64 * N <= (1ll << 21)) return true;
-  if ((M + 127) / 128 * (N / 128) <= 256) return true;
-  if (K >= 256 && K < 8192 && (M + 255) / 256 * (N / 128) <= 256) return true;
-  return M <= 128 && N >= 2048 && K >= 512;
+  if (((M + 63) / 64 * 64) * ((N + 63) / 64 * 64) <= (1ll << 21)) return true;
+  if ((M + 127) / 128 * ((N + 127) / 128) <= 256) return true;
+  if (K >= 256 && K < 8192 && (M + 255) / 256 * ((N + 127) / 128) <= 256) return true;
+  return M <= 128 && N % 32 == 0 && N >= 2048 && K >= 512;
 }
 static bool splits_rows(int64_t M, int64_t N, int64_t K) {
   if (M < 512 || M % 256 == 0 || N % 128 || K % 64) return false;
@@ -1982,7 +2000,7 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
   }
   int split128 = 1;  // K ranges of the 128x128 split, when the automatic choice takes it
   SmallPlan small;   // tile shape and K ranges of a small product, when the automatic choice takes it
-  int cut_rows = 0;  // 1 / 2: a product beyond the small rule on 128x128 / 256x128 tiles with a cut last tile row
+  int cut_rows = 0;  // 1 / 2: a product beyond the small rule on 128x128 / 256x128 tiles with a cut last tile row or column
   if (variant < 0) {
     // Large problems take the 256x256 tile; when that leaves most of the 256 CUs idle the
     // 128x128 tile (4x the workgroups) wins; everything else goes to the bounds-checked kernel.
@@ -2009,13 +2027,14 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
       variant = V_PIPELINED_128;
       split128 = s128;
     }
-    // any number of rows beyond the small rule, as long as one round of workgroups covers the product: the last tile row
-    // of 128x128 tiles (up to 256 of them) or of 256x128 tiles (129 to 256) is cut inside the kernel
-    else if (al && N % 128 == 0 && K % 64 == 0 && M % 128 != 0 && ((M + 127) / 128) * (N / 128) <= 256) {
+    // any number of rows and any multiple of 8 columns beyond the small rule, as long as one round of workgroups covers
+    // the product: the last tile row and column of 128x128 tiles (up to 256 of them) or of 256x128 tiles (129 to 256)
+    // are cut inside the kernel
+    else if (al && N % 8 == 0 && K % 64 == 0 && (M % 128 != 0 || N % 128 != 0) && ((M + 127) / 128) * ((N + 127) / 128) <= 256) {
       variant = V_PIPELINED_128;
       cut_rows = 1;
-    } else if (al && N % 128 == 0 && K % 64 == 0 && M % 256 != 0 && K >= 256 && K < 8192 && ((M + 127) / 128) * (N / 128) > 256 &&
-               ((M + 255) / 256) * (N / 128) <= 256) {
+    } else if (al && N % 8 == 0 && K % 64 == 0 && (M % 256 != 0 || N % 128 != 0) && K >= 256 && K < 8192 &&
+               ((M + 127) / 128) * ((N + 127) / 128) > 256 && ((M + 255) / 256) * ((N + 127) / 128) <= 256) {
       variant = V_PIPELINED_256x128;
       cut_rows = 2;
     }

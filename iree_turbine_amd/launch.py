@@ -42,25 +42,24 @@ _PAD_MIN_FLOPS = 0.0  # the tiled kernels on padded copies beat the bounds-check
 
 
 def _one_round_of_rows(M: int, N: int, K: int) -> bool:
-    """A product of any M rows against N % 128 == 0, K % 64 == 0 that the library's tiled or weight-streaming kernels
+    """A product of any M rows against N % 8 == 0, K % 64 == 0 that the library's tiled or weight-streaming kernels
     take whole (the library's rule of the same name)."""
-    if -(-M // 64) * 64 * N <= (1 << 21) or -(-M // 128) * (N // 128) <= 256:
+    up = lambda x, t: -(-x // t)
+    if up(M, 64) * 64 * up(N, 64) * 64 <= (1 << 21) or up(M, 128) * up(N, 128) <= 256:
         return True
-    if 256 <= K < 8192 and -(-M // 256) * (N // 128) <= 256:
+    if 256 <= K < 8192 and up(M, 256) * up(N, 128) <= 256:
         return True
-    return M <= 128 and N >= 2048 and K >= 512
+    return M <= 128 and N % 32 == 0 and N >= 2048 and K >= 512
 
 
 def _ragged_rows_fit(M: int, N: int, K: int) -> bool:
-    """Shapes whose ragged M the library handles itself: a cut last tile row in the small-product rule's range and
-    where one round of 128x128 or 256x128 tiles covers the product, two products on row ranges beyond that."""
-    if N % 64 or K % 64:
+    """Shapes whose ragged M (and N, in multiples of 8) the library handles itself: a cut last tile row or column where
+    one round of tiles covers the product, two products on row ranges beyond that (N a multiple of 128 then)."""
+    if N % 8 or K % 64:
         return False
-    if -(-M // 64) * 64 * N <= (1 << 21):
+    if _one_round_of_rows(M, N, K):
         return True
-    if N % 128:
-        return False
-    return _one_round_of_rows(M, N, K) or (M >= 512 and M % 256 != 0 and _one_round_of_rows(M % 256, N, K))
+    return N % 128 == 0 and M >= 512 and M % 256 != 0 and _one_round_of_rows(M % 256, N, K)
 
 
 def _skinny_fits(M: int, N: int, K: int) -> bool:

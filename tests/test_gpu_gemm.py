@@ -326,6 +326,39 @@ def test_gemm_ragged_rows(dev, shape, out32, dtype):
     assert torch.equal(c, again)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("out32", [False, True])
+@pytest.mark.parametrize("shape", [(64, 8, 64), (64, 72, 128), (128, 136, 128), (100, 1000, 512), (512, 1000, 1024), (1024, 1016, 1024),
+                                   (256, 264, 2048), (1000, 1096, 4096), (200, 4104, 1024), (2048, 2056, 1024), (1793, 3976, 512),
+                                   (128, 24584, 256)])
+def test_gemm_ragged_columns(dev, shape, out32, dtype):
+    """Any multiple of 8 columns where one round of tiles covers the product: the last tile column is cut inside the kernel
+    -- its loads of B take row min(row, N - 1), its stores stop at column N -- alone and together with a cut tile row, on
+    64x64, 128x64, 128x128 and 256x128 tiles: fewer columns than a tile, one 16-byte chunk more and fewer than a tile, one
+    slab and many.  Whole matrix against an fp32 product (a store right of column N would land in the next row), the
+    rows behind the result untouched, launches repeat bit for bit; the launcher pads nothing."""
+    import iree_turbine_amd as ita
+    from iree_turbine_amd import _lib
+
+    M, N, K = shape
+    announce(f"gemm ragged columns {shape} {dtype} out32={out32}")
+    assert ita.launch._ragged_rows_fit(M, N, K)
+    assert _lib.load().mi355_gemm_nt_workspace_bytes(M, N, K) == 0  # a cut tile column takes no K split
+    g = torch.Generator().manual_seed(M + 2 * N + 3 * K)
+    a = (torch.randn(M, K, generator=g) * 0.25).to(dtype).to(dev)
+    b = (torch.randn(N, K, generator=g) * 0.25).to(dtype).to(dev)
+    odt = torch.float32 if out32 else dtype
+    full = torch.full((M + 130, N), float("nan"), dtype=odt, device=dev)
+    c = full[:M]
+    ita.launch.gemm_nt_out(a, b, c, -1)
+    tol = dict(rtol=1e-3, atol=1e-3) if out32 else dict(rtol=1e-2, atol=1e-2)
+    torch.testing.assert_close(c.float(), a.float() @ b.float().t(), **tol)
+    assert torch.isnan(full[M:]).all()  # nothing stored behind row M - 1
+    again = torch.empty_like(c)
+    ita.launch.gemm_nt_out(a, b, again, -1)
+    assert torch.equal(c, again)
+
+
 @pytest.mark.parametrize("shape", [(1088, 2112, 2048), (1152, 2112, 1024), (2112, 1152, 1024)])
 def test_gemm_multiples_of_64_beyond_the_small_rule(dev, shape):
     """Products too large for the small-product rule that divide by 64 and not by 128 (and too small for the launcher to
