@@ -67,7 +67,8 @@ template <bool BF> struct OutPack<half_t, BF> {
 //  * RAGGED_M: M is any number of rows and N any multiple of 8 columns (the last tile row and the last tile column are
 //    cut): the loads of A take row min(row, M - 1) and those of B row min(row, N - 1), so they stay inside the operands,
 //    and the epilogue stores the rows below M and the 16-byte chunks left of column N only.  N is then both the row
-//    pitch of C and its number of columns.
+//    pitch of C and its number of columns.  With a K split M is the number of rows of A, and every row of the stacked
+//    partial tiles is stored (the workspace holds whole tiles).
 template <int BM, int BN, int WM, int WN, typename OutT, bool BF, bool SLAB = false, bool RAGGED_M = false>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_t* __restrict__ A,
                                                                      const half_t* __restrict__ B,
@@ -357,7 +358,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
     for (int it = 0; it < WTM / ROWS_PER_IT; it++) {
       const int row = it * ROWS_PER_IT + er;
       half8 v = *reinterpret_cast<const half8*>(ep + row * ROW_B + ((ec ^ ((row >> 1) & (CH - 1))) * 16));
-      if (!RAGGED_M || (tile_m * BM + wm * WTM + row < M && tile_n * BN + wn * WTN + ec * 8 < N))
+      if (!RAGGED_M || ((split_tiles_m > 0 || tile_m * BM + wm * WTM + row < M) && tile_n * BN + wn * WTN + ec * 8 < N))
         *reinterpret_cast<half8*>(cbase + (size_t)row * N) = v;
     }
   } else {
@@ -385,7 +386,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_f16_nt_pipelined(const half_
     for (int it = 0; it < WTM / ROWS_PER_IT; it++) {
       const int row = it * ROWS_PER_IT + er;
       floatx4 v = *reinterpret_cast<const floatx4*>(ep + row * ROW_B + ((ec ^ (row & (CH - 1))) * 16));
-      if (!RAGGED_M || (tile_m * BM + wm * WTM + row < M && tile_n * BN + wn * WTN + ec * 4 < N))
+      if (!RAGGED_M || ((split_tiles_m > 0 || tile_m * BM + wm * WTM + row < M) && tile_n * BN + wn * WTN + ec * 4 < N))
         *reinterpret_cast<floatx4*>(cbase + (size_t)row * N) = v;
     }
   }
@@ -1568,14 +1569,15 @@ __global__ __launch_bounds__(256) void gemm_f16_nt_generic(const half_t* __restr
 
 // ---- host side ----------------------------------------------------------------------------
 
-// Sum of the S partial products of a K split (an [S * M, N] fp32 workspace, split s in rows s * M ..): four columns per
-// lane, the partials added in split order, the sum converted as the kernels' own epilogues convert theirs.
+// Sum of the S partial products of a K split (an [S * plane_rows, N] fp32 workspace, split s in rows s * plane_rows ..;
+// plane_rows >= M: with a cut last tile row the planes hold whole tiles): four columns per lane, the partials added in
+// split order, the sum converted as the kernels' own epilogues convert theirs.
 template <typename OutT, bool BF>
 __global__ __launch_bounds__(256) void gemm_ksplit_merge(const float* __restrict__ ws, OutT* __restrict__ C, int M, int N, int ldc,
-                                                         int S) {
+                                                         int S, int plane_rows) {
   const size_t idx = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
-  const size_t plane = (size_t)M * N;
-  if (idx >= plane) return;
+  const size_t plane = (size_t)plane_rows * N;
+  if (idx >= (size_t)M * N) return;
   floatx4 acc = *reinterpret_cast<const floatx4*>(ws + idx);
   for (int sp = 1; sp < S; sp++) acc += *reinterpret_cast<const floatx4*>(ws + sp * plane + idx);
   const size_t r = idx / (size_t)N, c = idx - r * (size_t)N;
@@ -1671,19 +1673,28 @@ static int launch_tiled(const void* a, const void* b, void* c, int M, int N, int
 }
 
 // K split on the pipelined kernel, for products too small for 256x256 tiles to spread over the chip: S K ranges
-// of k_part each, fp32 partial tiles stacked along M in the workspace (row pitch N).
+// of k_part each, fp32 partial tiles stacked along M in the workspace (row pitch N).  ragged: any M, N % 8 == 0 (the
+// slab form only); a range's partial products are then ceil(M / BM) whole tiles of rows, and the kernel takes M as the
+// number of rows of A.
 template <bool BF, int BM = 128, int BN = 128>
-static int launch_pipelined_ksplit(const half_t* a, const half_t* b, float* ws, int M, int N, int K, int S, hipStream_t stream) {
+static int launch_pipelined_ksplit(const half_t* a, const half_t* b, float* ws, int M, int N, int K, int S, hipStream_t stream,
+                                   bool ragged = false) {
   const int k_part = K / S;
-  const int tiles_m = (M / BM) * S, tiles_n = N / BN;
+  const int rows_of_tiles = ragged ? (M + BM - 1) / BM : M / BM;
+  const int tiles_m = rows_of_tiles * S, tiles_n = ragged ? (N + BN - 1) / BN : N / BN;
   dim3 grid(tiles_m * tiles_n), block(256);
   auto go = [&](auto kern, int lds_bytes, std::atomic<uint64_t>& lds_ok) {
     if (int rc = allow_lds(reinterpret_cast<const void*>(kern), lds_bytes, lds_ok, "gemm_f16_nt")) return rc;
-    hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, a, b, ws, M * S, N, k_part, tiles_m, tiles_n, 4, K, M / BM, k_part,
-                       pipelined_krot(M, N, K));
+    hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, a, b, ws, ragged ? M : M * S, N, k_part, tiles_m, tiles_n, 4, K,
+                       rows_of_tiles, k_part, pipelined_krot(M, N, K));
     return check_launch("gemm_f16_nt_pipelined (K split)", grid, block, lds_bytes);
   };
   static std::atomic<uint64_t> lds_ok2{0}, lds_ok4{0};
+  if (ragged) {
+    static std::atomic<uint64_t> lds_okr{0};
+    if (N % 8 || !pipelined_slab_form(grid.x, BM + BN)) return fail(-MI355_E_SHAPE, "gemm_f16_nt: no K split with cut tiles for this shape");
+    return go(gemm_f16_nt_pipelined<BM, BN, 2, 2, float, BF, true, true>, 4 * (BM + BN) * 128, lds_okr);
+  }
   if (pipelined_slab_form(grid.x, BM + BN)) return go(gemm_f16_nt_pipelined<BM, BN, 2, 2, float, BF, true>, 4 * (BM + BN) * 128, lds_ok4);
   if constexpr (BM + BN == 256) return go(gemm_f16_nt_pipelined<BM, BN, 2, 2, float, BF, false>, 2 * (BM + BN) * 128, lds_ok2);
   return fail(-MI355_E_SHAPE, "gemm_f16_nt: no k-step form of this tile");  // not reached: pipelined_slab_form
@@ -1766,16 +1777,18 @@ static int launch_ksplit(const half_t* a, const half_t* b, OutT* c, int M, int N
   if (int rc = launch_stream<float, BF>(a, b, ws, M, N, K, N, stream, true, S)) return rc;
   const long long lanes = (long long)M * N / 4;
   dim3 grid((unsigned)((lanes + 255) / 256)), block(256);
-  hipLaunchKernelGGL((gemm_ksplit_merge<OutT, BF>), grid, block, 0, stream, (const float*)ws, c, M, N, ldc, S);
+  hipLaunchKernelGGL((gemm_ksplit_merge<OutT, BF>), grid, block, 0, stream, (const float*)ws, c, M, N, ldc, S, M);
   return check_launch("gemm_ksplit_merge", grid, block, 0);
 }
 
 template <typename OutT, bool BF, int BM = 128, int BN = 128>
-static int launch_ksplit128(const half_t* a, const half_t* b, OutT* c, int M, int N, int K, int ldc, int S, float* ws, hipStream_t stream) {
-  if (int rc = launch_pipelined_ksplit<BF, BM, BN>(a, b, ws, M, N, K, S, stream)) return rc;
+static int launch_ksplit128(const half_t* a, const half_t* b, OutT* c, int M, int N, int K, int ldc, int S, float* ws, hipStream_t stream,
+                            bool ragged = false) {
+  if (int rc = launch_pipelined_ksplit<BF, BM, BN>(a, b, ws, M, N, K, S, stream, ragged)) return rc;
   const long long lanes = (long long)M * N / 4;
   dim3 grid((unsigned)((lanes + 255) / 256)), block(256);
-  hipLaunchKernelGGL((gemm_ksplit_merge<OutT, BF>), grid, block, 0, stream, (const float*)ws, c, M, N, ldc, S);
+  hipLaunchKernelGGL((gemm_ksplit_merge<OutT, BF>), grid, block, 0, stream, (const float*)ws, c, M, N, ldc, S,
+                     ragged ? (M + BM - 1) / BM * BM : M);
   return check_launch("gemm_ksplit_merge", grid, block, 0);
 }
 
@@ -1814,7 +1827,9 @@ static bool takes_256x128(int64_t M, int64_t N, int64_t K) {
 
 struct SmallPlan {
   int bm = 0, bn = 0, S = 1;  // bm == 0: not a small product
-  bool ragged = false;        // M is no multiple of bm or N none of bn: the last tile row or column is cut, and K is not split
+  bool ragged = false;        // M is no multiple of bm or N none of bn: the last tile row or column is cut
+  int64_t ws_bytes() const { return S > 1 ? (int64_t)S * plane_rows * cols * 4 : 0; }
+  int64_t plane_rows = 0, cols = 0;  // rows (whole tiles) and columns of one K range's partial products
 };
 static SmallPlan small_plan(int64_t M, int64_t N, int64_t K, int64_t ws_bytes) {
   SmallPlan best;
@@ -1827,22 +1842,24 @@ static SmallPlan small_plan(int64_t M, int64_t N, int64_t K, int64_t ws_bytes) {
     const int bm = t[0], bn = t[1];
     const bool ragged = M % bm != 0 || N % bn != 0;
     const int64_t tiles = ((M + bm - 1) / bm) * ((N + bn - 1) / bn);
-    for (int S = 1; S <= (ragged ? 1 : 8); S *= 2) {
+    const int64_t plane_rows = (M + bm - 1) / bm * bm;  // a cut tile row's partial products are whole tiles
+    for (int S = 1; S <= 8; S *= 2) {
       const int64_t units = tiles * S, k_part = K / S;
       if (units > 512 || K % (64 * S)) break;
-      if (S > 1 && (k_part < 512 || S * M * N * 4 > ws_bytes)) break;
+      if (ragged && !pipelined_slab_form(units, bm + bn)) break;  // cut tiles: the slab form only
+      if (S > 1 && (k_part < 512 || S * plane_rows * N * 4 > ws_bytes)) break;
       const double per_cu_kib = (double)((units + 255) / 256) * (bm + bn) * 2 * k_part / 1024.0;
       double us_per_kib;
       if (bm + bn == 256) us_per_kib = pipelined_slab_form(units, 256) ? 0.013 : 0.0188;
       else us_per_kib = 0.0095 + 0.0035 * (units <= 128 ? 0.0 : units >= 256 ? 1.0 : (units - 128) / 128.0);
       double us = 2.5 + per_cu_kib * us_per_kib;
       if (S > 1) {
-        const double partial_bytes = (double)S * M * N * 8;
+        const double partial_bytes = (double)S * plane_rows * N * 8;
         us += 2.3 + partial_bytes / 4.5e6 + (partial_bytes > (8 << 20) ? (partial_bytes - (8 << 20)) / 4.5e6 : 0.0);
       }
       if (best.bm == 0 || us < best_us) {
         best_us = us;
-        best.bm = bm, best.bn = bn, best.S = S, best.ragged = ragged;
+        best.bm = bm, best.bn = bn, best.S = S, best.ragged = ragged, best.plane_rows = plane_rows, best.cols = N;
       }
     }
   }
@@ -2019,7 +2036,7 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
     if (fits(V_SKINNY) && (M <= 64 || M % 64 != 0) && N >= 2048 && K >= 512) variant = V_SKINNY;
     else if (al && (small = small_plan(M, N, K, INT64_MAX)).bm) {
       // a workspace short of what the plan asks for is no workspace (not a plan with fewer ranges)
-      if (small.S > 1 && (!workspace || workspace_bytes < (int64_t)small.S * M * N * 4)) small = small_plan(M, N, K, 0);
+      if (small.S > 1 && (!workspace || workspace_bytes < small.ws_bytes())) small = small_plan(M, N, K, 0);
       variant = small.bm == 64 ? V_PIPELINED_64 : small.bn == 64 ? V_PIPELINED_128x64 : V_PIPELINED_128;
     }
     else if (al && takes_256x128(M, N, K)) variant = V_PIPELINED_256x128;
@@ -2065,7 +2082,7 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
   float* ws = static_cast<float*>(workspace);
   const size_t wsb = workspace_bytes > 0 ? (size_t)workspace_bytes : 0;
   if (ws && !aligned16(ws)) return fail(-MI355_E_ALIGN, "gemm_f16_nt: workspace must be 16-byte aligned");
-  if (small.ragged || cut_rows) {
+  if ((small.ragged && small.S == 1) || cut_rows) {
     const int m = (int)M, n = (int)N, k = (int)K;
     auto tiled = [&](auto out, auto is_bf) {
       using OutT = decltype(out);
@@ -2085,9 +2102,9 @@ static int gemm_nt_entry(bool bf, const void* a, const void* b, void* c, int64_t
     auto tiled = [&](auto out, auto is_bf) {
       using OutT = decltype(out);
       constexpr bool BF = decltype(is_bf)::value;
-      if (small.bm == 64) return launch_ksplit128<OutT, BF, 64, 64>(ah, bh, (OutT*)c, m, n, k, n, S, ws, s);
-      if (small.bn == 64) return launch_ksplit128<OutT, BF, 128, 64>(ah, bh, (OutT*)c, m, n, k, n, S, ws, s);
-      return launch_ksplit128<OutT, BF, 128, 128>(ah, bh, (OutT*)c, m, n, k, n, S, ws, s);
+      if (small.bm == 64) return launch_ksplit128<OutT, BF, 64, 64>(ah, bh, (OutT*)c, m, n, k, n, S, ws, s, small.ragged);
+      if (small.bn == 64) return launch_ksplit128<OutT, BF, 128, 64>(ah, bh, (OutT*)c, m, n, k, n, S, ws, s, small.ragged);
+      return launch_ksplit128<OutT, BF, 128, 128>(ah, bh, (OutT*)c, m, n, k, n, S, ws, s, small.ragged);
     };
     if (bf) return out_dtype == MI355_F32 ? tiled(float{}, std::true_type{}) : tiled(half_t{}, std::true_type{});
     return out_dtype == MI355_F32 ? tiled(float{}, std::false_type{}) : tiled(half_t{}, std::false_type{});
@@ -2120,7 +2137,7 @@ static int64_t gemm_nt_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (M * K * 2 >= (1ll << 32) || N * K * 2 >= (1ll << 32)) return 0;  // the streamed kernel's one descriptor per operand
   if (M <= 64 && N % 32 == 0 && N >= 2048 && K >= 512) return 0;        // the weight-streaming kernel's shapes
   const SmallPlan sp = small_plan(M, N, K, INT64_MAX);
-  if (sp.bm) return sp.S > 1 ? (int64_t)sp.S * M * N * 4 : 0;
+  if (sp.bm) return sp.ws_bytes();
   if (takes_256x128(M, N, K)) return 0;
   const int s128 = (K % 64 == 0) ? ksplit128_plan((int)M, (int)N, (int)K) : 1;
   if (s128 > 1) return (int64_t)s128 * M * N * 4;

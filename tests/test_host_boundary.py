@@ -70,7 +70,9 @@ def test_gemm_workspace_plan_without_a_gpu():
     assert need(2048, 4096, 8192) == 2 * 2048 * 4096 * 4  # 128 tiles of 256x256
     assert need(2048, 10240, 8192) == 4 * 2048 * 2048 * 4  # the strip of 64 tiles behind a full round
     assert need(8192, 8192, 8192) == 0 and need(4096, 4096, 4096) == 0
-    assert need(200, 4096, 4096) == 0 and need(65, 64, 8192) == 0  # a cut last tile row takes no split
+    assert need(200, 4096, 4096) == 0  # a cut last tile row, enough tiles without a split
+    assert need(65, 64, 8192) == 8 * 128 * 64 * 4  # a cut last tile row: the partial products are whole 64x64 tiles
+    assert need(256, 1000, 4096) == need(256, 1024, 4096) * 1000 // 1024  # a cut last tile column: N columns wide
     assert need(2100, 10240, 8192) == need(2048, 10240, 8192)  # 2048 rows and 52 rows, one after the other
     assert need(0, 128, 128) == 0 and need(128, 128, -64) == 0 and need(128, 128, 1 << 22) == 0
 
