@@ -109,6 +109,41 @@ def test_random_gemm_small_and_mid_products(dev):
     assert split >= 6  # the draw does exercise the split
 
 
+def test_random_gemm_cut_tiles(dev):
+    """Any number of rows against any multiple of 8 columns, within one round of tiles: the last tile row and column are
+    cut inside the kernels, with one to eight K ranges -- fp16 and bf16 operands, both output types, whole matrix against
+    an fp32 product; the launcher pads nothing."""
+    import iree_turbine_amd as ita
+    from iree_turbine_amd import _lib
+    from oracle import inputs
+
+    lib = _lib.load()
+    rng = random.Random(4242)
+    split = 0
+    for case in range(40):
+        if case % 4 == 3:  # beyond the small-product rule: one round of 128x128 or 256x128 tiles
+            M = rng.randint(1100, 3000)
+            N = 8 * rng.randint((1 << 21) // (-(-M // 64) * 64) // 8 + 1, 16 * (256 // -(-M // 256)))
+            K = 64 * rng.randint(4, 24)
+        elif case % 4 == 0:  # few tiles and a long K: K ranges with cut tiles
+            M, N, K = rng.randint(1, 300), 8 * rng.randint(1, 80), rng.choice([2048, 4096, 8192])
+        else:
+            M = rng.randint(1, 1400)
+            N = 8 * rng.randint(1, max(1, min(256, (1 << 21) // (-(-M // 64) * 64) // 8 - 8)))
+            K = rng.choice([64, 192, 1024, 1088, 2048, 4096, 8192])
+        dtype = rng.choice([torch.float16, torch.bfloat16])
+        out_dtype = rng.choice(["float32", str(dtype).split(".")[1]])
+        need = lib.mi355_gemm_nt_workspace_bytes(M, N, K)
+        split += need > 0
+        announce(f"random cut-tile gemm {case}: {M}x{N}x{K} {dtype} -> {out_dtype}, workspace {need >> 10} KiB")
+        assert ita.launch._ragged_rows_fit(M, N, K), (M, N, K)
+        a, b = [t.to(dev) for t in inputs.gemm_inputs(M, N, K, seed=900 + case, dtype=dtype)]
+        c = torch.ops.mi355.gemm_nt(a, b, out_dtype, -1)
+        tol = dict(rtol=1e-3, atol=1e-3) if out_dtype == "float32" else dict(rtol=1e-2, atol=1e-2)
+        torch.testing.assert_close(c.float(), a.float() @ b.float().t(), **tol)
+    assert split >= 8  # the draw does exercise the split
+
+
 def test_random_attention(dev):
     import iree_turbine_amd  # noqa: F401
     from oracle import attention as oa
