@@ -57,6 +57,7 @@ MEASURED_TRAFFIC_BYTES: dict[str, float | None] = {
     "gemm_16x8192x8192": 1.366e8,
     "gemm_64x8192x8192": 1.439e8,
     "gemm_200x4096x4096": 4.980e7,
+    "gemm_1000x1000x1024": 1.438e7,
     "gemm_1024x8192x8192": 3.644e8,
     "fa_causal": 3.537e8,
     "fa_noncausal": 2.686e8,
@@ -482,6 +483,7 @@ WORKLOADS = {
     "gemm_512x8192x8192": wl_gemm(512, 8192, 8192),    # 64 tiles: four K ranges
     "gemm_64x8192x8192": wl_gemm(64, 8192, 8192),      # weight streaming with two row blocks
     "gemm_200x4096x4096": wl_gemm(200, 4096, 4096),    # a ragged number of rows: the last tile row cut inside the kernel
+    "gemm_1000x1000x1024": wl_gemm(1000, 1000, 1024),  # ragged rows and columns: the last tile row and column cut inside the kernel
     "fa_causal": wl_attention(True),
     "fa_noncausal": wl_attention(False),
     "decode": wl_decode(),
